@@ -1,0 +1,121 @@
+"""Seeded synthetic inputs for the benchmark configurations.
+
+Every generator takes an explicit seed and returns plain numpy arrays, so the
+HIP path and the CPU checker consume byte-identical inputs.  The block layouts
+are GGML's: Q4_K 256 elems / 144 B, Q6_K 256 / 210 B, Q4_0 32 / 18 B
+(crates/ksearch_ir/src/lib.rs:52-74 in the ksearch tree).
+"""
+from __future__ import annotations
+
+import numpy as np
+
+Q4K_BYTES, Q6K_BYTES, Q40_BYTES = 144, 210, 18
+
+
+def _rng(seed: int) -> np.random.Generator:
+    return np.random.Generator(np.random.PCG64(seed))
+
+
+def _f16_uniform(rng, n, lo, hi) -> np.ndarray:
+    """n half-precision values ~U(lo, hi), as raw uint16 bit patterns."""
+    return rng.uniform(lo, hi, size=n).astype(np.float32).astype(np.float16).view(np.uint16)
+
+
+def q4k_blocks(n_blocks: int, seed: int) -> np.ndarray:
+    """Random Q4_K superblocks: d, dmin = f16(U(1e-3,1e-2)); 12 scale bytes and
+    128 quant bytes uniform over all byte values (every 6-bit field and every
+    nibble is then uniform)."""
+    rng = _rng(seed)
+    blk = np.empty((n_blocks, Q4K_BYTES), dtype=np.uint8)
+    blk[:, 0:2] = _f16_uniform(rng, n_blocks, 1e-3, 1e-2).view(np.uint8).reshape(n_blocks, 2)
+    blk[:, 2:4] = _f16_uniform(rng, n_blocks, 1e-3, 1e-2).view(np.uint8).reshape(n_blocks, 2)
+    blk[:, 4:] = rng.integers(0, 256, size=(n_blocks, Q4K_BYTES - 4), dtype=np.uint8)
+    return blk.reshape(-1)
+
+
+def q6k_blocks(n_blocks: int, seed: int) -> np.ndarray:
+    """Random Q6_K superblocks: ql/qh random bytes, 16 int8 scales ~U{-32..31},
+    d = f16(U(1e-3,1e-2))."""
+    rng = _rng(seed)
+    blk = np.empty((n_blocks, Q6K_BYTES), dtype=np.uint8)
+    blk[:, :192] = rng.integers(0, 256, size=(n_blocks, 192), dtype=np.uint8)
+    blk[:, 192:208] = rng.integers(-32, 32, size=(n_blocks, 16), dtype=np.int8).view(np.uint8)
+    blk[:, 208:210] = _f16_uniform(rng, n_blocks, 1e-3, 1e-2).view(np.uint8).reshape(n_blocks, 2)
+    return blk.reshape(-1)
+
+
+def q40_blocks(n_blocks: int, seed: int) -> np.ndarray:
+    """Random Q4_0 blocks: scale f16(U(0.01,0.1)) + 16 B of uniform nibbles."""
+    rng = _rng(seed)
+    blk = np.empty((n_blocks, Q40_BYTES), dtype=np.uint8)
+    blk[:, 0:2] = _f16_uniform(rng, n_blocks, 0.01, 0.1).view(np.uint8).reshape(n_blocks, 2)
+    blk[:, 2:] = rng.integers(0, 256, size=(n_blocks, 16), dtype=np.uint8)
+    return blk.reshape(-1)
+
+
+def normal_f32(n, seed: int, std: float = 1.0) -> np.ndarray:
+    return (_rng(seed).standard_normal(size=n) * std).astype(np.float32)
+
+
+def bf16_round(x: np.ndarray) -> np.ndarray:
+    """f32 -> nearest-even bf16, returned as f32 values and raw uint16 bits."""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    r = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+    return (r.astype(np.uint32) << 16).view(np.float32), r
+
+
+# -- the five benchmark configurations --------------------------------------
+
+def cfg0_q4k_matvec(rows=4096, cols=4096, seed=1000):
+    w = q4k_blocks(rows * cols // 256, seed)
+    x = normal_f32(cols, seed + 1)
+    return w, x
+
+
+def cfg1_q6k_lm_head(rows=262144, cols=2048, seed=1001):
+    w = q6k_blocks(rows * cols // 256, seed)
+    x = normal_f32(cols, seed + 1)
+    return w, x
+
+
+def cfg2_q4k_prefill(tokens=512, rows=8192, cols=2048, seed=1002):
+    w = q4k_blocks(rows * cols // 256, seed)
+    xf, xb = bf16_round(normal_f32(tokens * cols, seed + 1))
+    return w, xf.reshape(tokens, cols), xb.reshape(tokens, cols)
+
+
+def cfg3_q40_attention(n_slots=4, n_q=8, n_kv=1, hd=256, max_t=16384, lo=1024, seed=1003):
+    rng = _rng(seed)
+    lens = rng.integers(lo, max_t + 1, size=n_slots).astype(np.int32)
+    nblk = n_slots * max_t * n_kv * hd // 32
+    k = q40_blocks(nblk, seed + 1).reshape(n_slots, -1)
+    v = q40_blocks(nblk, seed + 2).reshape(n_slots, -1)
+    q = normal_f32(n_slots * n_q * hd, seed + 3).reshape(n_slots, n_q * hd)
+    return lens, k, v, q
+
+
+GEMMA_E2B_SYNTH = dict(n_layers=30, hidden=2048, ffn=8192, n_q=8, n_kv=1, hd=256,
+                       vocab=262144, max_seq=4096, eps=1e-6, softcap=30.0,
+                       rope_theta=10000.0, attn_scale=1.0 / 16.0)
+
+
+def gemma_weights(cfg: dict, seed: int, quantize_q4k, quantize_q6k, std: float = 0.02) -> dict:
+    """N(0, std) weights packed to Q4_K (attention/FFN) and Q6_K (tied
+    embedding / LM head); norm weights are 1.  The two quantizers are passed
+    in by the caller, so this module has no dependency on where they live."""
+    h, f, hd = cfg["hidden"], cfg["ffn"], cfg["hd"]
+    nq, nkv = cfg["n_q"] * hd, cfg["n_kv"] * hd
+    layers = []
+    s = seed
+    for _ in range(cfg["n_layers"]):
+        lw = {}
+        for name, (r, c) in (("wq", (nq, h)), ("wk", (nkv, h)), ("wv", (nkv, h)), ("wo", (h, nq)),
+                             ("wgate", (f, h)), ("wup", (f, h)), ("wdown", (h, f))):
+            s += 1
+            lw[name] = quantize_q4k(normal_f32(r * c, s, std))
+        for name, n in (("attn_norm", h), ("q_norm", hd), ("k_norm", hd),
+                        ("post_attn_norm", h), ("ffn_norm", h), ("post_ffw_norm", h)):
+            lw[name] = np.ones(n, dtype=np.float32)
+        layers.append(lw)
+    embd = quantize_q6k(normal_f32(cfg["vocab"] * h, s + 1, std))
+    return dict(layers=layers, token_embd=embd, output_norm=np.ones(h, dtype=np.float32))

@@ -1,0 +1,305 @@
+"""CPU checker for the HIP path (test infrastructure only).
+
+Thin ctypes/numpy wrappers over ``libksearch_oracle.so`` (built by
+``oracle/Makefile`` from ``ksearch_oracle.c``).  Only ``tests/``, the smoke
+check and the benchmark's ``cpu_baseline`` leg may import this package; the
+shipped library never does.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libksearch_oracle.so")
+
+F32, F16, Q4K, Q5K, Q6K, Q40, BF16 = range(7)
+BLOCK = {Q40: (32, 18), Q4K: (256, 144), Q5K: (256, 176), Q6K: (256, 210)}
+
+
+def build(force: bool = False) -> str:
+    """Compile the oracle with gcc (always when ``force``; else only if absent)."""
+    if force or not os.path.exists(LIB_PATH):
+        subprocess.check_call(["make", "-s", "-B", "-C", _HERE])
+    return LIB_PATH
+
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        build()
+        L = C.CDLL(LIB_PATH)
+        vp, sz, i32, u32, f32 = C.c_void_p, C.c_size_t, C.c_int, C.c_uint32, C.c_float
+        sig = {
+            "ko_bf16_to_f32": (f32, [C.c_uint16]),
+            "ko_f32_to_bf16": (C.c_uint16, [f32]),
+            "ko_f16_to_f32": (f32, [C.c_uint16]),
+            "ko_f32_to_f16": (C.c_uint16, [f32]),
+            "ko_f32_to_f16_rne": (C.c_uint16, [f32]),
+            "ko_get_scale_min_k4": (None, [i32, vp, vp, vp]),
+            "ko_row_bytes": (sz, [i32, sz]),
+            "ko_dequant": (i32, [i32, vp, sz, vp]),
+            "ko_quantize_q4k": (None, [vp, sz, vp]),
+            "ko_quantize_q6k": (None, [vp, sz, vp]),
+            "ko_pack_q40": (None, [vp, sz, vp, i32]),
+            "ko_matvec": (i32, [i32, vp, sz, sz, vp, vp, i32]),
+            "ko_matmul": (i32, [i32, vp, sz, sz, vp, sz, vp, i32]),
+            "ko_matvec_f64": (i32, [i32, vp, sz, sz, vp, vp, i32]),
+            "ko_max_threads": (i32, []),
+            "ko_sdpa_online": (None, [vp, vp, vp, i32, i32, i32, i32, i32, f32, vp]),
+            "ko_sdpa_mwg": (None, [vp, vp, vp, i32, i32, i32, i32, i32, f32, i32, vp]),
+            "ko_sdpa_f64": (None, [vp, vp, vp, i32, i32, i32, i32, i32, f32, vp]),
+            "ko_softcap_argmax": (u32, [vp, sz, f32]),
+            "ko_rmsnorm": (None, [vp, vp, vp, f32, f32, i32, sz, vp]),
+            "ko_rmsnorm_add_then_rmsnorm": (None, [vp, vp, vp, vp, f32, sz, vp, vp]),
+            "ko_rope_table": (None, [i32, i32, f32, i32, vp]),
+            "ko_rmsnorm_per_head_qkv_q40": (None, [vp, vp, vp, vp, vp, vp, i32, i32, i32, f32, vp, vp, vp]),
+            "ko_gelu_mul": (f32, [f32, f32]),
+            "ko_copy_scale_indexed": (i32, [i32, vp, u32, sz, f32, vp]),
+            "ko_gemma_create": (vp, [vp, vp, vp, vp]),
+            "ko_gemma_destroy": (None, [vp]),
+            "ko_gemma_reset": (None, [vp]),
+            "ko_gemma_forward": (u32, [vp, u32, i32, vp, i32]),
+            "ko_gemma_pos": (i32, [vp]),
+            "ko_gemma_kv": (vp, [vp, i32, i32]),
+            "ko_gemma_hidden": (vp, [vp]),
+        }
+        for name, (res, args) in sig.items():
+            fn = getattr(L, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = L
+    return _lib
+
+
+def _p(a: np.ndarray) -> int:
+    return a.ctypes.data
+
+
+def _f32(a) -> np.ndarray:
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _u8(a) -> np.ndarray:
+    return np.ascontiguousarray(a, dtype=np.uint8)
+
+
+def row_bytes(dtype: int, cols: int) -> int:
+    return lib().ko_row_bytes(dtype, cols)
+
+
+def f16_to_f32(bits) -> np.ndarray:
+    bits = np.asarray(bits, dtype=np.uint16).ravel()
+    L = lib()
+    return np.array([L.ko_f16_to_f32(int(b)) for b in bits], dtype=np.float32)
+
+
+def f32_to_f16(vals, rne: bool = False) -> np.ndarray:
+    fn = lib().ko_f32_to_f16_rne if rne else lib().ko_f32_to_f16
+    return np.array([fn(float(v)) for v in np.asarray(vals, dtype=np.float32).ravel()], dtype=np.uint16)
+
+
+def get_scale_min_k4(j: int, q12) -> tuple[int, int]:
+    q = _u8(q12)
+    d, m = C.c_uint8(), C.c_uint8()
+    lib().ko_get_scale_min_k4(j, _p(q), C.addressof(d), C.addressof(m))
+    return d.value, m.value
+
+
+def dequant(dtype: int, data, n_elems: int) -> np.ndarray:
+    data = _u8(data)
+    out = np.empty(n_elems, dtype=np.float32)
+    if lib().ko_dequant(dtype, _p(data), n_elems, _p(out)):
+        raise ValueError("unsupported dtype")
+    return out
+
+
+def quantize_q4k(x) -> np.ndarray:
+    x = _f32(x).ravel()
+    out = np.empty(x.size // 256 * 144, dtype=np.uint8)
+    lib().ko_quantize_q4k(_p(x), x.size, _p(out))
+    return out
+
+
+def quantize_q6k(x) -> np.ndarray:
+    x = _f32(x).ravel()
+    out = np.empty(x.size // 256 * 210, dtype=np.uint8)
+    lib().ko_quantize_q6k(_p(x), x.size, _p(out))
+    return out
+
+
+def pack_q40(x, half_roundtrip: bool = True) -> np.ndarray:
+    x = _f32(x).ravel()
+    out = np.empty(x.size // 32 * 18, dtype=np.uint8)
+    lib().ko_pack_q40(_p(x), x.size, _p(out), int(half_roundtrip))
+    return out
+
+
+def matvec(dtype: int, w, rows: int, cols: int, x, threads: int = 0) -> np.ndarray:
+    w, x = _u8(w), _f32(x)
+    y = np.empty(rows, dtype=np.float32)
+    if lib().ko_matvec(dtype, _p(w), rows, cols, _p(x), _p(y), threads):
+        raise ValueError("bad matvec shape/dtype")
+    return y
+
+
+def matvec_f64(dtype: int, w, rows: int, cols: int, x, threads: int = 0) -> np.ndarray:
+    w, x = _u8(w), _f32(x)
+    y = np.empty(rows, dtype=np.float64)
+    if lib().ko_matvec_f64(dtype, _p(w), rows, cols, _p(x), _p(y), threads):
+        raise ValueError("bad matvec shape/dtype")
+    return y
+
+
+def matmul(dtype: int, w, rows: int, cols: int, x, batch: int, threads: int = 0) -> np.ndarray:
+    w, x = _u8(w), _f32(x)
+    y = np.empty((batch, rows), dtype=np.float32)
+    if lib().ko_matmul(dtype, _p(w), rows, cols, _p(x), batch, _p(y), threads):
+        raise ValueError("bad matmul shape/dtype")
+    return y
+
+
+def max_threads() -> int:
+    return lib().ko_max_threads()
+
+
+def sdpa(q, k, v, n_q, n_kv, hd, tlen, start=0, scale=1.0, nwg: int | None = None, f64=False):
+    q, k, v = _f32(q), _u8(k), _u8(v)
+    L = lib()
+    if f64:
+        out = np.empty(n_q * hd, dtype=np.float64)
+        L.ko_sdpa_f64(_p(q), _p(k), _p(v), n_q, n_kv, hd, tlen, start, scale, _p(out))
+        return out
+    out = np.empty(n_q * hd, dtype=np.float32)
+    if nwg is None:
+        L.ko_sdpa_online(_p(q), _p(k), _p(v), n_q, n_kv, hd, tlen, start, scale, _p(out))
+    else:
+        L.ko_sdpa_mwg(_p(q), _p(k), _p(v), n_q, n_kv, hd, tlen, start, scale, nwg, _p(out))
+    return out
+
+
+def sdpa_hybrid(q, k, v, n_q, n_kv, hd, tlen, start=0, scale=1.0):
+    """sdpa_hybrid_kv: online below 128 rows, 16-way split from 128 on
+    (ksearch_kernels/src/lib.rs:1114-1178)."""
+    return sdpa(q, k, v, n_q, n_kv, hd, tlen, start, scale, nwg=16 if tlen >= 128 else None)
+
+
+def softcap_argmax(x, cap: float) -> int:
+    x = _f32(x)
+    return lib().ko_softcap_argmax(_p(x), x.size, cap)
+
+
+def rmsnorm(x, w, eps, res=None, scale=None) -> np.ndarray:
+    x, w = _f32(x), _f32(w)
+    out = np.empty_like(x)
+    r = _f32(res) if res is not None else None
+    lib().ko_rmsnorm(_p(x), _p(w), _p(r) if r is not None else None, eps,
+                     scale if scale is not None else 0.0, int(scale is not None), x.size, _p(out))
+    return out
+
+
+def rmsnorm_add_then_rmsnorm(y, w_post, res, w_ffn, eps):
+    y, w_post, res, w_ffn = _f32(y), _f32(w_post), _f32(res), _f32(w_ffn)
+    ox, ox2 = np.empty_like(y), np.empty_like(y)
+    lib().ko_rmsnorm_add_then_rmsnorm(_p(y), _p(w_post), _p(res), _p(w_ffn), eps, y.size, _p(ox), _p(ox2))
+    return ox, ox2
+
+
+def rope_table(max_seq, hd, theta, rope_angles=None) -> np.ndarray:
+    out = np.empty((max_seq, hd), dtype=np.float32)
+    lib().ko_rope_table(max_seq, hd, theta, hd // 2 if rope_angles is None else rope_angles, _p(out))
+    return out
+
+
+def rmsnorm_per_head_qkv_q40(q, qw, rope_row, k, kw, v, n_q, n_kv, hd, eps):
+    q, qw, rope_row, k, kw, v = map(_f32, (q, qw, rope_row, k, kw, v))
+    qo = np.empty(n_q * hd, dtype=np.float32)
+    ko = np.empty(n_kv * hd // 32 * 18, dtype=np.uint8)
+    vo = np.empty_like(ko)
+    lib().ko_rmsnorm_per_head_qkv_q40(_p(q), _p(qw), _p(rope_row), _p(k), _p(kw), _p(v),
+                                      n_q, n_kv, hd, eps, _p(qo), _p(ko), _p(vo))
+    return qo, ko, vo
+
+
+def gelu_mul(g, u) -> np.ndarray:
+    g, u = _f32(g).ravel(), _f32(u).ravel()
+    L = lib()
+    return np.array([L.ko_gelu_mul(float(a), float(b)) for a, b in zip(g, u)], dtype=np.float32)
+
+
+def copy_scale_indexed(dtype, src, idx, n, scale) -> np.ndarray:
+    src = _u8(src)
+    out = np.empty(n, dtype=np.float32)
+    if lib().ko_copy_scale_indexed(dtype, _p(src), idx, n, scale, _p(out)):
+        raise ValueError("bad dtype")
+    return out
+
+
+class GemmaCfg(C.Structure):
+    _fields_ = [(n, C.c_int) for n in ("n_layers", "hidden", "ffn", "n_q", "n_kv", "hd", "vocab", "max_seq")] + \
+               [(n, C.c_float) for n in ("eps", "softcap", "rope_theta", "attn_scale")]
+
+
+class GemmaLayer(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in (
+        "wq", "wk", "wv", "wo", "wgate", "wup", "wdown",
+        "attn_norm", "q_norm", "k_norm", "post_attn_norm", "ffn_norm", "post_ffw_norm")]
+
+
+class Gemma:
+    """CPU greedy decoder over the same packed weights the HIP path uses.
+
+    ``weights`` is the dict produced by ``ksearch_amd.synth.gemma_weights``:
+    per-layer arrays under ``layers[i][name]`` plus ``token_embd`` and
+    ``output_norm``.  Arrays are kept alive for the oracle's lifetime.
+    """
+
+    def __init__(self, cfg: dict, weights: dict):
+        self._keep = weights
+        self.cfg = GemmaCfg(**cfg)
+        n = cfg["n_layers"]
+        arr = (GemmaLayer * n)()
+        for i, lw in enumerate(weights["layers"]):
+            for name, _ in GemmaLayer._fields_:
+                setattr(arr[i], name, _p(lw[name]))
+        self._layers = arr
+        self.h = lib().ko_gemma_create(C.byref(self.cfg), arr, _p(weights["token_embd"]),
+                                       _p(weights["output_norm"]))
+        self.vocab = cfg["vocab"]
+
+    def reset(self):
+        lib().ko_gemma_reset(self.h)
+
+    @property
+    def pos(self) -> int:
+        return lib().ko_gemma_pos(self.h)
+
+    def forward(self, token: int, want_logits: bool = True, return_logits: bool = False, threads: int = 0):
+        logits = np.empty(self.vocab, dtype=np.float32) if return_logits else None
+        nxt = lib().ko_gemma_forward(self.h, int(token), int(want_logits),
+                                     _p(logits) if logits is not None else None, threads)
+        return (nxt, logits) if return_logits else nxt
+
+    def kv(self, layer: int, which: int, nbytes: int) -> np.ndarray:
+        ptr = lib().ko_gemma_kv(self.h, layer, which)
+        return np.ctypeslib.as_array(C.cast(ptr, C.POINTER(C.c_uint8)), shape=(nbytes,)).copy()
+
+    def hidden(self) -> np.ndarray:
+        ptr = lib().ko_gemma_hidden(self.h)
+        return np.ctypeslib.as_array(C.cast(ptr, C.POINTER(C.c_float)), shape=(self.cfg.hidden,)).copy()
+
+    def close(self):
+        if self.h:
+            lib().ko_gemma_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

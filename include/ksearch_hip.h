@@ -1,0 +1,257 @@
+/*
+ * ksearch_hip.h — C ABI of libksearch_hip.so, the MI355X (gfx950) backend for
+ * ksearch's quantized decode hot path.
+ *
+ * The library takes the place of two things in the ksearch tree:
+ *   - crates/ksearch_metal/src/lib.rs (MetalContext: device, buffers, one open
+ *     encoder, flush / wait / barrier / synchronize, timed run), and
+ *   - the kernel bodies crates/ksearch_codegen/src/{lower,render}.rs emit for
+ *     the Q4_K / Q6_K GEMVs, the Q4_K prefill GEMM, the Q4_0-KV attention and
+ *     the glue ops of a decode step.
+ * Kernels are prebuilt hand-written HIP selected by (kind, dims, dtypes,
+ * schedule); there is no run-time code generation.
+ *
+ * Conventions
+ *   - every function returns 0 on success, non-zero on failure; the message is
+ *     fetched with ksh_last_error() (thread-local, valid until the next call).
+ *     Count / size mismatches are errors, never aborts
+ *     (crates/ksearch_metal/src/lib.rs:280-307).
+ *   - a context is owned by one host thread (the reference context is !Sync).
+ *   - work is appended to one in-order HIP stream; program order is execution
+ *     order (the reference relies on Metal hazard tracking inside one encoder,
+ *     crates/ksearch_kernels/src/lib.rs:890).
+ *   - device memory is not host-visible: what the reference does through
+ *     `contents()` pointers goes through ksh_buffer_write / read / fill_zero.
+ */
+#ifndef KSEARCH_HIP_H
+#define KSEARCH_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct ksh_ctx ksh_ctx;
+typedef struct ksh_buf ksh_buf;
+typedef struct ksh_kernel ksh_kernel;
+typedef struct ksh_graph ksh_graph;
+
+/* DType, crates/ksearch_ir/src/lib.rs:17-27 (same order) */
+enum ksh_dtype {
+    KSH_F32 = 0, KSH_F16 = 1, KSH_Q4K = 2, KSH_Q5K = 3, KSH_Q6K = 4, KSH_Q40 = 5, KSH_BF16 = 6
+};
+
+/* The KernelKind variants on the hot path (crates/ksearch_ir/src/kernel.rs:399-744).
+ * Inputs/outputs are listed in binding order; "act" = activation dtype
+ * (dtypes[1], F32 unless stated). */
+enum ksh_kind {
+    /* Matvec{rows,cols,weight_dtype}: y = W x.  dims: rows, cols.
+     * dtypes[0] = Q4K | Q6K.  in: W, x   out: y[rows] */
+    KSH_MATVEC = 1,
+    /* MatvecBatch: Y[t,r] = sum_c W[r,c] X[t,c].  dims: rows, cols, batch.
+     * dtypes[0] = Q4K, dtypes[1] = BF16 (X), output F32 token-major.
+     * in: W, X   out: Y[batch, rows] */
+    KSH_MATVEC_BATCH = 2,
+    /* MatvecQkv: three GEMVs sharing x.  dims: q_rows, kv_rows, cols.
+     * in: Wq, Wk, Wv, x   out: q, k, v */
+    KSH_MATVEC_QKV = 3,
+    /* MatvecGateUpGelu: out[i] = gelu_tanh(clamp(Wg[i].x, +-20)) * (Wu[i].x).
+     * dims: rows, cols.  in: Wg, Wu, x   out: out[rows] */
+    KSH_MATVEC_GATE_UP_GELU = 4,
+    /* SdpaNaive: online-softmax attention over rows [start, start+tlen).
+     * dims: n_q, n_kv, hd, max_t.  params[0] = softmax scale (1.0 = reference).
+     * in: q[n_q*hd], K, V (Q4_0 [max_t,n_kv,hd]), meta f32[>=3] = tlen,start,window
+     * out: o[n_q*hd] */
+    KSH_SDPA_NAIVE = 5,
+    /* SdpaMwgPart: split-KV pass 1.  dims: n_q, n_kv, hd, max_t, nwg.
+     * in: q, K, V, meta   out: tmp f32[n_q*nwg*(hd+2)] = (m, l, O[hd]) */
+    KSH_SDPA_MWG_PART = 6,
+    /* SdpaMwgReduce: split-KV pass 2.  dims: n_q, hd, nwg.  in: tmp  out: o */
+    KSH_SDPA_MWG_REDUCE = 7,
+    /* Multi-slot decode attention in one launch (the reference runs slots
+     * serially, crates/ksearch_cli/src/scheduler.rs:163-187).
+     * dims: n_q, n_kv, hd, max_t, n_slots, nwg.  K/V pools are
+     * [n_slots][max_t,n_kv,hd] Q4_0; meta is f32[n_slots][4].
+     * in: q[n_slots,n_q*hd], Kpool, Vpool, meta   out: tmp, o[n_slots,n_q*hd] */
+    KSH_SDPA_SLOTS = 8,
+    /* QuantizeQ40: pack n f32 values (n%32==0) to Q4_0.  dims: n.  in: src  out: dst */
+    KSH_QUANTIZE_Q40 = 9,
+    /* RmsNorm / RmsNormAdd / RmsNormAddScale.  dims: n, has_residual, has_scale.
+     * params[0] = eps, params[1] = scale.  in: x, w, (residual)   out: y */
+    KSH_RMSNORM = 10,
+    /* RmsNormAddThenRmsNorm.  dims: n.  params[0] = eps.
+     * in: y, w_post, residual, w_ffn   out: x, x2 */
+    KSH_RMSNORM_ADD_THEN_RMSNORM = 11,
+    /* RmsNormPerHeadQkvQ40 (n_tok = 1).  dims: n_q, n_kv, hd.  params[0] = eps.
+     * in: q, qw, rope_row f32[hd], k, kw, v   out: q_out f32, K row Q4_0, V row Q4_0 */
+    KSH_RMSNORM_PER_HEAD_QKV_Q40 = 12,
+    /* CopyScaleIndexed: out[i] = scale * deq(src[id*n + i]); id is read from a
+     * device f32 (the reference keeps token ids as f32).  dims: n.
+     * dtypes[0] = source dtype.  params[0] = scale.  in: src, idx   out: out[n] */
+    KSH_COPY_SCALE_INDEXED = 13,
+    /* GeluMul: out[i] = gelu_tanh(clamp(g[i])) * u[i].  dims: n.  in: g, u  out: out */
+    KSH_GELU_MUL = 14,
+    /* CopySlice.  dims: n.  in: src   out: dst */
+    KSH_COPY_SLICE = 15,
+    /* SoftcapArgmax: argmax_i cap*tanh(x_i/cap), lowest index wins ties, index
+     * stored as f32.  dims: n.  params[0] = cap.  in: x   out: idx f32[1] */
+    KSH_SOFTCAP_ARGMAX = 16,
+    /* Dequantize packed blocks to f32 (the CPU-side dequant_type_to_f32,
+     * crates/ksearch_gguf/src/gguf_impl.rs:472-476, as a device kernel).
+     * dims: n_elems.  dtypes[0] = Q4K | Q6K | Q40.  in: src   out: dst f32 */
+    KSH_DEQUANT = 17,
+    /* quantize_f32_to_q4k (crates/ksearch_gguf/src/gguf_impl.rs:905-1016) and a
+     * Q6_K packer, as device kernels.  dims: n_elems.  dtypes[0] = Q4K | Q6K.
+     * in: src f32   out: packed */
+    KSH_QUANTIZE_K = 18,
+    KSH_KIND_COUNT
+};
+
+/* OptSchedule (crates/ksearch_ir/src/kernel.rs:11-18) retargeted to gfx950.
+ * All-zero means "library default, or the plan cache's entry if one exists". */
+typedef struct {
+    uint64_t tg;       /* threads per workgroup (64 * waves) */
+    uint32_t vec;      /* inner-product variant: 0/1 = cvt+fma, 2 = f16 mix-fma, 3 = int8 dot */
+    uint32_t unroll;   /* superblocks in flight per lane */
+    uint32_t nsg;      /* waves per workgroup */
+    uint32_t nr0;      /* rows per wave */
+    uint32_t k_split;  /* waves cooperating on one row along K */
+    uint32_t lds_tile; /* LDS tile: KV rows per tile (SDPA), K depth (GEMM) */
+} ksh_sched;
+
+typedef struct {
+    int32_t kind;          /* enum ksh_kind */
+    int32_t dtypes[4];
+    int64_t dims[8];
+    float params[4];
+    ksh_sched sched;
+} ksh_kernel_desc;
+
+/* LaunchHint / MetalKernelSource metadata (crates/ksearch_codegen/src/lib.rs:33-60) */
+typedef struct {
+    int32_t n_inputs, n_outputs;
+    uint32_t grid[3], block[3];
+    uint32_t lds_bytes;
+    ksh_sched sched;       /* the schedule actually bound */
+    char name[64];
+} ksh_kernel_info;
+
+const char *ksh_last_error(void);
+
+/* MetalContext::new / Drop, crates/ksearch_metal/src/lib.rs:25-41.  Device 0,
+ * one in-order stream.  Fails (never falls back) when no gfx950 GPU is usable. */
+int ksh_ctx_create(ksh_ctx **out);
+void ksh_ctx_destroy(ksh_ctx *ctx);
+/* device_name, :43.  KSEARCH_CHIP if set, otherwise the GCN arch name. */
+int ksh_device_name(ksh_ctx *ctx, char *dst, size_t n);
+/* the HIP stream work is appended to (hipStream_t), for event timing by callers */
+void *ksh_stream(ksh_ctx *ctx);
+
+/* buffer_bytes / buffer_empty_*, :63-91.  init may be NULL (zero-filled). */
+int ksh_buffer_alloc(ksh_ctx *ctx, size_t bytes, const void *init, ksh_buf **out);
+void ksh_buffer_retain(ksh_buf *buf);
+void ksh_buffer_release(ksh_buf *buf);
+size_t ksh_buffer_size(const ksh_buf *buf);
+void *ksh_buffer_device_ptr(const ksh_buf *buf);
+/* write_buffer / write_u16s (sync=1) and their *_nosync forms (sync=0), :110-135 */
+int ksh_buffer_write(ksh_ctx *ctx, ksh_buf *buf, size_t off, const void *src, size_t bytes, int sync);
+/* read_f32 / read_u16 (sync=1), read_f32_nosync (sync=0), :93-108 */
+int ksh_buffer_read(ksh_ctx *ctx, ksh_buf *buf, size_t off, void *dst, size_t bytes, int sync);
+/* the host memset of KvPool::clear_slot (crates/ksearch_gemma/src/kv_pool.rs:148-159) */
+int ksh_buffer_fill_zero(ksh_ctx *ctx, ksh_buf *buf);
+
+/* lower_to_metal_chip + MetalContext::compile
+ * (crates/ksearch_codegen/src/lib.rs:62-166, ksearch_metal/src/lib.rs:47-61):
+ * binds a prebuilt kernel to the descriptor, consulting the plan cache when the
+ * schedule is all-zero.  Handles are cached per context and owned by it. */
+int ksh_kernel_get(ksh_ctx *ctx, const ksh_kernel_desc *desc, ksh_kernel **out);
+int ksh_kernel_info_get(const ksh_kernel *k, ksh_kernel_info *info);
+
+/* encode_offsets_multi, crates/ksearch_metal/src/lib.rs:269-374 */
+int ksh_encode(ksh_ctx *ctx, ksh_kernel *k,
+               ksh_buf *const *inputs, const uint64_t *in_byte_off, int n_in,
+               ksh_buf *const *outputs, const uint64_t *out_byte_off, int n_out);
+/* run (:377-456): synchronize, then `iters` launches timed with HIP events on
+ * the context's stream; *ms is the average per launch. */
+int ksh_run_timed(ksh_ctx *ctx, ksh_kernel *k,
+                  ksh_buf *const *inputs, const uint64_t *in_byte_off, int n_in,
+                  ksh_buf *const *outputs, const uint64_t *out_byte_off, int n_out,
+                  int iters, double *ms);
+
+int ksh_flush_async(ksh_ctx *ctx);                        /* :162 */
+int ksh_wait_inflight_at_most(ksh_ctx *ctx, int n);       /* :173 */
+int ksh_barrier(ksh_ctx *ctx);                            /* encoder_barrier :196 */
+int ksh_synchronize(ksh_ctx *ctx);                        /* :205 */
+int ksh_has_gpu_work(ksh_ctx *ctx);                       /* :157 (1/0) */
+
+/* HIP-graph capture of everything encoded between begin and end; replay with
+ * ksh_graph_launch.  (The reference re-encodes every token into one Metal
+ * command buffer; a graph is the gfx950 equivalent of that single commit.) */
+int ksh_graph_begin(ksh_ctx *ctx);
+int ksh_graph_end(ksh_ctx *ctx, ksh_graph **out);
+int ksh_graph_launch(ksh_ctx *ctx, ksh_graph *g);
+void ksh_graph_destroy(ksh_graph *g);
+
+/* plan cache, crates/ksearch_codegen/src/{plan_cache.rs:9-44, beam.rs:67-139}:
+ * $KSEARCH_BEAM_CACHE or ~/.cache/ksearch/beam/{key}.txt holding key=value
+ * lines.  The key hash is FNV-1a 64 (the reference's DefaultHasher is not
+ * stable across Rust releases and is not reproduced). */
+int ksh_plan_key(const char *kind, const int64_t *dims, int n_dims, const char *chip,
+                 char *dst, size_t n);
+int ksh_plan_save(const char *kind, const int64_t *dims, int n_dims, const char *chip,
+                  const ksh_sched *sched, double ms);
+/* returns 0 and fills *sched / *ms when a plan exists, 1 when none does */
+int ksh_plan_load(const char *kind, const int64_t *dims, int n_dims, const char *chip,
+                  ksh_sched *sched, double *ms);
+/* plan kind string for a descriptor ("matvec_q4k", "matvec_q6k", "mul_mm_q4k",
+ * "sdpa_q40", ...; crates/ksearch_codegen/src/lib.rs:200-205) */
+const char *ksh_plan_kind(const ksh_kernel_desc *desc);
+/* BEAM: candidate schedules for a descriptor (beam.rs:26-65 retargeted) */
+int ksh_beam_candidates(const ksh_kernel_desc *desc, ksh_sched *out, int cap);
+/* beam_search_matvec / Eng::beam_matvec (crates/ksearch_codegen/src/lib.rs:178-246,
+ * ksearch_kernels/src/lib.rs:1985-2043): time every candidate (1 warm-up +
+ * `iters` timed), save the best plan, return it. force=1 ignores a cached plan. */
+int ksh_beam_search(ksh_ctx *ctx, const ksh_kernel_desc *desc,
+                    ksh_buf *const *inputs, int n_in, ksh_buf *const *outputs, int n_out,
+                    int iters, int force, ksh_sched *best, double *best_ms, int *from_cache);
+
+/* ---- decode loop: GemmaPrimModel for the synthetic Gemma-4-E2B shape
+ * (crates/ksearch_gemma/src/gemma_prim.rs:881-1275, 1658-1768), minus PLE,
+ * sliding window and shared KV, which that shape does not have. ---- */
+typedef struct {
+    int32_t n_layers, hidden, ffn, n_q, n_kv, hd, vocab, max_seq;
+    float eps, softcap, rope_theta, attn_scale;
+} ksh_gemma_cfg;
+
+typedef struct {
+    ksh_buf *wq, *wk, *wv, *wo, *wgate, *wup, *wdown;             /* Q4_K */
+    ksh_buf *attn_norm, *q_norm, *k_norm, *post_attn_norm, *ffn_norm, *post_ffw_norm; /* f32 */
+} ksh_gemma_layer;
+
+typedef struct ksh_gemma ksh_gemma;
+
+int ksh_gemma_create(ksh_ctx *ctx, const ksh_gemma_cfg *cfg, const ksh_gemma_layer *layers,
+                     ksh_buf *token_embd_q6k, ksh_buf *output_norm, ksh_gemma **out);
+void ksh_gemma_destroy(ksh_gemma *m);
+int ksh_gemma_reset(ksh_gemma *m);
+/* forward_token: one token at the model's current position.  use_graph=1
+ * replays a captured HIP graph.  next_id may be NULL (no host read-back). */
+int ksh_gemma_forward_token(ksh_gemma *m, uint32_t token, int use_graph, uint32_t *next_id);
+/* generate_timed: feeds the prompt token by token, then n_new greedy tokens
+ * whose ids never leave the device between steps.  decode_ms covers the n_new
+ * steps only. */
+int ksh_gemma_generate(ksh_gemma *m, const uint32_t *prompt, int n_prompt, int n_new,
+                       int use_graph, uint32_t *out_ids, double *prefill_ms, double *decode_ms);
+/* test hooks: device buffers of the last step */
+ksh_buf *ksh_gemma_logits(ksh_gemma *m);
+ksh_buf *ksh_gemma_hidden(ksh_gemma *m);
+ksh_buf *ksh_gemma_kv(ksh_gemma *m, int layer, int which);
+int ksh_gemma_pos(ksh_gemma *m);
+int ksh_gemma_launches_per_token(ksh_gemma *m);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,132 @@
+// Packed block -> f32 dequantization on the device, bit-exact with the CPU
+// loops of crates/ksearch_gguf/src/gguf_impl.rs:618-633 (Q4_0), :690-721
+// (Q4_K) and :761-791 (Q6_K).  Built with -ffp-contract=off: the reference
+// rounds `d1*q` and `- mn1` separately.
+//
+// One thread per 16-byte-aligned unit of packed input is not possible for
+// Q6_K / Q4_0 (blocks are 2-byte aligned), so the mapping is by OUTPUT: a
+// thread produces 4 consecutive f32 (one float4 store) and reads the few bytes
+// it needs with byte loads; the packed input is tiny next to the f32 output it
+// expands to (x7 for Q4_K), so the store stream is what bounds this kernel.
+#include "ksh_device.hpp"
+#include "ksh_internal.hpp"
+
+namespace ksh {
+namespace {
+
+__device__ __forceinline__ uint32_t ld16(const uint8_t *p) { return (uint32_t)p[0] | ((uint32_t)p[1] << 8); }
+
+// get_scale_min_k4, gguf_impl.rs:563-573
+__device__ __forceinline__ void scale_min_k4(int j, const uint8_t *q, uint32_t &d, uint32_t &m)
+{
+    if (j < 4) {
+        d = q[j] & 63u;
+        m = q[j + 4] & 63u;
+    } else {
+        d = (q[j + 4] & 0x0Fu) | ((uint32_t)(q[j - 4] >> 6) << 4);
+        m = (uint32_t)(q[j + 4] >> 4) | ((uint32_t)(q[j] >> 6) << 4);
+    }
+}
+
+__global__ void dequant_q4k_kernel(const uint8_t *__restrict__ src, float *__restrict__ dst, size_t n4)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n4) return;
+    const size_t e = i * 4, b = e >> 8;
+    const int j = (int)(e & 255);
+    const uint8_t *blk = src + b * 144;
+    const float d = half_bits_to_f32(ld16(blk)), dmin = half_bits_to_f32(ld16(blk + 2));
+    const int sub = j >> 5;                 // 32-wide sub-block
+    uint32_t sc, mn;
+    scale_min_k4(sub, blk + 4, sc, mn);
+    const float d1 = d * (float)sc, mn1 = dmin * (float)mn;
+    const uint8_t *qs = blk + 16 + (j >> 6) * 32 + (j & 31);
+    const bool hi = (j & 32) != 0;
+    float4 o;
+    o.x = d1 * (float)(hi ? (qs[0] >> 4) : (qs[0] & 0x0F)) - mn1;
+    o.y = d1 * (float)(hi ? (qs[1] >> 4) : (qs[1] & 0x0F)) - mn1;
+    o.z = d1 * (float)(hi ? (qs[2] >> 4) : (qs[2] & 0x0F)) - mn1;
+    o.w = d1 * (float)(hi ? (qs[3] >> 4) : (qs[3] & 0x0F)) - mn1;
+    reinterpret_cast<float4 *>(dst)[i] = o;
+}
+
+__global__ void dequant_q6k_kernel(const uint8_t *__restrict__ src, float *__restrict__ dst, size_t n4)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n4) return;
+    const size_t e = i * 4, b = e >> 8;
+    const int j = (int)(e & 255);
+    const uint8_t *blk = src + b * 210;
+    const int half = j >> 7, jl = j & 127, quad = jl >> 5, l = jl & 31;
+    const uint8_t *ql = blk + 64 * half + l + ((quad & 1) ? 32 : 0);
+    const uint8_t *qh = blk + 128 + 32 * half + l;
+    const int8_t sc = (int8_t)blk[192 + 8 * half + 2 * quad + (l >> 4)];
+    const float d = half_bits_to_f32(ld16(blk + 208));
+    const float ds = d * (float)sc;
+    float o[4];
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        const uint32_t lo = quad >= 2 ? (uint32_t)(ql[t] >> 4) : (uint32_t)(ql[t] & 0x0F);
+        const uint32_t hi2 = ((uint32_t)qh[t] >> (2 * quad)) & 3u;
+        const int q = (int)(lo | (hi2 << 4)) - 32;
+        o[t] = ds * (float)q;
+    }
+    reinterpret_cast<float4 *>(dst)[i] = make_float4(o[0], o[1], o[2], o[3]);
+}
+
+__global__ void dequant_q40_kernel(const uint8_t *__restrict__ src, float *__restrict__ dst, size_t n4)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n4) return;
+    const size_t e = i * 4, b = e >> 5;
+    const int j = (int)(e & 31);
+    const uint8_t *blk = src + b * 18;
+    const float d = half_bits_to_f32(ld16(blk));
+    const uint8_t *qs = blk + 2 + (j & 15);
+    const bool hi = j >= 16;
+    float o[4];
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        const int q = (int)(hi ? (qs[t] >> 4) : (qs[t] & 0x0F)) - 8;
+        o[t] = (float)q * d;
+    }
+    reinterpret_cast<float4 *>(dst)[i] = make_float4(o[0], o[1], o[2], o[3]);
+}
+
+int launch_dequant(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
+{
+    const size_t n4 = (size_t)k.desc.dims[0] / 4;
+    const unsigned grid = (unsigned)((n4 + 255) / 256);
+    const uint8_t *src = (const uint8_t *)a.in[0];
+    float *dst = (float *)a.out[0];
+    switch (k.desc.dtypes[0]) {
+    case KSH_Q4K: hipLaunchKernelGGL(dequant_q4k_kernel, dim3(grid), dim3(256), 0, st, src, dst, n4); break;
+    case KSH_Q6K: hipLaunchKernelGGL(dequant_q6k_kernel, dim3(grid), dim3(256), 0, st, src, dst, n4); break;
+    case KSH_Q40: hipLaunchKernelGGL(dequant_q40_kernel, dim3(grid), dim3(256), 0, st, src, dst, n4); break;
+    }
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : hip_fail(e, "dequant launch");
+}
+
+}  // namespace
+
+int bind_dequant(ksh_kernel &k)
+{
+    const int dt = k.desc.dtypes[0];
+    const int64_t n = k.desc.dims[0];
+    if (dt != KSH_Q4K && dt != KSH_Q6K && dt != KSH_Q40) return set_error("dequant: dtype %d is not built", dt);
+    const size_t pb = n > 0 ? packed_bytes(dt, (size_t)n) : 0;
+    if (!pb || (uint64_t)n / 4 / 256 > 0x7FFFFFFFull) return set_error("dequant: n=%lld is not a valid element count", (long long)n);
+    k.info.n_inputs = 1;
+    k.info.n_outputs = 1;
+    k.in_bytes[0] = pb;
+    k.out_bytes[0] = (size_t)n * 4;
+    k.in_align[0] = 2;
+    k.out_align[0] = 16;
+    set_launch(k, (uint32_t)(((size_t)n / 4 + 255) / 256), 1, 1, 256, 0);
+    set_name(k, "dequant_%s", dt == KSH_Q4K ? "q4k" : dt == KSH_Q6K ? "q6k" : "q40");
+    k.launch = launch_dequant;
+    return 0;
+}
+
+}  // namespace ksh

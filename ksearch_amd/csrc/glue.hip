@@ -1,0 +1,536 @@
+// Small ops between the GEMVs of a decode step: the RMSNorm family, per-head
+// RMS + RoPE + Q4_0 KV append, embedding row gather, GELU*up, slice copy,
+// Q4_0 packing, soft-capped argmax and a fill kernel.
+//
+// They take the place of lower_rmsnorm / lower_rmsnorm_add_then_rmsnorm
+// (crates/ksearch_codegen/src/lower.rs:4079-4162, 3926-4077),
+// lower_rmsnorm_per_head_qkv_q40 (:4619-4702), CopyScaleIndexed (:3899-3921),
+// gelu_mul (:4775-4838), copy_slice (:3831), lower_quantize_q40 (:4886-4895),
+// lower_softcap_argmax (:6090-6156) and ksearch_pack_q40_th
+// (crates/ksearch_codegen/src/render.rs:1040-1059).
+//
+// Built with -ffp-contract=off so that `u*cos - v*sin` and `(x*inv)*w + res`
+// round exactly like the unfused expressions they restate; the Q4_0 codes that
+// come out of the pack are integer functions of those values.
+#include "ksh_device.hpp"
+#include "ksh_internal.hpp"
+
+namespace ksh {
+namespace {
+
+constexpr int kNormThreads = 256;
+
+// block-wide sum for 256 threads (4 waves): DPP inside the wave, LDS across
+__device__ __forceinline__ float block_sum_256(float v, float *red)
+{
+    const float w = wave_sum(v);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    __syncthreads();   // `red` may still be read from a previous call
+    if (lane == 0) red[wave] = w;
+    __syncthreads();
+    return (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+__global__ void fill_zero_kernel(uint4 *p, size_t n16, uint8_t *tail, size_t ntail)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t j = i; j < n16; j += stride) p[j] = make_uint4(0, 0, 0, 0);
+    if (i < ntail) tail[i] = 0;
+}
+
+// y = (x * rsqrt(mean(x^2) + eps)) * w  (+ residual)  (* scale)
+__global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(const float *__restrict__ x,
+                                                               const float *__restrict__ w,
+                                                               const float *res, float *y, int n, float eps,
+                                                               int has_res, int has_scale, float scale)
+{
+    __shared__ float red[4];
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < n; i += kNormThreads) ss += x[i] * x[i];
+    ss = block_sum_256(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)n + eps);
+    for (int i = threadIdx.x; i < n; i += kNormThreads) {
+        float v = x[i] * inv * w[i];
+        if (has_res) v = v + res[i];
+        if (has_scale) v = scale * v;
+        y[i] = v;
+    }
+}
+
+// out_x = res + (y*inv)*w_post;  out_x2 = (out_x*inv2)*w_ffn   (n <= 8192)
+__global__ __launch_bounds__(kNormThreads) void rmsnorm_add_then_rmsnorm_kernel(
+    const float *__restrict__ y, const float *__restrict__ w_post, const float *res,
+    const float *__restrict__ w_ffn, float *out_x, float *out_x2, int n, float eps)
+{
+    __shared__ float red[4];
+    extern __shared__ float mid[];
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < n; i += kNormThreads) ss += y[i] * y[i];
+    ss = block_sum_256(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)n + eps);
+    float ss2 = 0.f;
+    for (int i = threadIdx.x; i < n; i += kNormThreads) {
+        const float v = res[i] + y[i] * inv * w_post[i];
+        mid[i] = v;
+        out_x[i] = v;
+        ss2 += v * v;
+    }
+    ss2 = block_sum_256(ss2, red);
+    const float inv2 = 1.0f / sqrtf(ss2 / (float)n + eps);
+    for (int i = threadIdx.x; i < n; i += kNormThreads) out_x2[i] = mid[i] * inv2 * w_ffn[i];
+}
+
+// ksearch_pack_q40_th for one 32-value block held by 32 consecutive lanes of
+// a wave (lane l of the group holds element l).  Values pass through a half
+// round trip first; scale = max|v|/7 (1 if all zero); code = clamp(round(v/scale)+8).
+// `group_base` is the first lane of the group.  Lanes 0..15 of the group store.
+__device__ __forceinline__ void pack_q40_group(float v, int l, uint8_t *blk, bool store)
+{
+    v = half_bits_to_f32(f32_to_half_bits(v));
+    float m = fabsf(v);
+    // max over the 32 lanes of the group: row of 16 via DPP, then the neighbour row
+    m = fmaxf(m, dpp_f32<0xB1>(m));
+    m = fmaxf(m, dpp_f32<0x4E>(m));
+    m = fmaxf(m, dpp_f32<0x141>(m));
+    m = fmaxf(m, dpp_f32<0x140>(m));
+    m = fmaxf(m, __shfl_xor(m, 16, 64));
+    const float scale = m > 0.0f ? m / 7.0f : 1.0f;
+    const float inv = 1.0f / scale;
+    int q = (int)roundf(v * inv) + 8;
+    q = min(15, max(0, q));
+    const int qhi = __shfl_down(q, 16, 64);    // element l+16's code, for l < 16
+    if (!store) return;
+    if (l == 0) {
+        const uint32_t h = f32_to_half_bits(scale);
+        blk[0] = (uint8_t)(h & 0xFF);
+        blk[1] = (uint8_t)(h >> 8);
+    }
+    if (l < 16) blk[2 + l] = (uint8_t)(q | (qhi << 4));
+}
+
+// QuantizeQ40: one 32-lane group per block of 32 source values
+__global__ __launch_bounds__(256) void quantize_q40_kernel(const float *__restrict__ src, uint8_t *dst, int nblk)
+{
+    const int gidx = (blockIdx.x * 256 + threadIdx.x) >> 5, l = threadIdx.x & 31;
+    const bool ok = gidx < nblk;
+    const float v = ok ? src[(size_t)gidx * 32 + l] : 0.f;
+    // every lane takes part in the cross-lane steps; only valid groups store
+    pack_q40_group(v, l, dst + (size_t)(ok ? gidx : 0) * 18, ok);
+}
+
+// RmsNormPerHeadQkvQ40, n_tok = 1.  One wave per head; blocks 0..n_q-1 do Q
+// (rms*w, RoPE, f32 out); blocks n_q..n_q+n_kv-1 do K (rms*w, RoPE, Q4_0) and
+// V (rms without weight, Q4_0) of one kv head.  RoPE pairs (i, i+hd/2) with
+// the row cos[0..hd/2) || sin[0..hd/2).  hd is 128, 256 or 512.
+template <int HD>
+__global__ __launch_bounds__(64) void per_head_qkv_q40_kernel(
+    const float *q, const float *__restrict__ qw, const float *__restrict__ rope,
+    const float *__restrict__ k, const float *__restrict__ kw, const float *__restrict__ v,
+    float *q_out, uint8_t *k_out, uint8_t *v_out, int n_q, float eps)
+{
+    constexpr int HALF = HD / 2, PER = HD / 64;   // elements per lane
+    const int lane = threadIdx.x;
+    const int head = blockIdx.x;
+    const bool is_q = head < n_q;
+    const int h = is_q ? head : head - n_q;
+    const float *x = (is_q ? q : k) + (size_t)h * HD;
+    const float *w = is_q ? qw : kw;
+
+    // lane owns elements lane + 64*j: consecutive lanes hold consecutive
+    // elements, so every 32-lane half of the wave holds one Q4_0 block per j
+    float xv[PER];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+        xv[j] = x[lane + 64 * j];
+        ss += xv[j] * xv[j];
+    }
+    ss = wave_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / (float)HD + eps);
+    float nv[PER];
+#pragma unroll
+    for (int j = 0; j < PER; j++) nv[j] = xv[j] * inv * w[lane + 64 * j];
+    // RoPE: element e < HALF pairs with e + HALF, i.e. register j with j + PER/2
+    float ro[PER];
+#pragma unroll
+    for (int j = 0; j < PER / 2; j++) {
+        const int e = lane + 64 * j;
+        const float c = rope[e], s = rope[HALF + e];
+        const float u = nv[j], vv = nv[j + PER / 2];
+        ro[j] = u * c - vv * s;
+        ro[j + PER / 2] = u * s + vv * c;
+    }
+    if (is_q) {
+#pragma unroll
+        for (int j = 0; j < PER; j++) q_out[(size_t)h * HD + lane + 64 * j] = ro[j];
+        return;
+    }
+    uint8_t *krow = k_out + (size_t)h * (HD / 32) * 18;
+    uint8_t *vrow = v_out + (size_t)h * (HD / 32) * 18;
+#pragma unroll
+    for (int j = 0; j < PER; j++) pack_q40_group(ro[j], lane & 31, krow + (size_t)(2 * j + (lane >> 5)) * 18, true);
+
+    const float *vx = v + (size_t)h * HD;
+    float vs = 0.f;
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+        xv[j] = vx[lane + 64 * j];
+        vs += xv[j] * xv[j];
+    }
+    vs = wave_sum(vs);
+    const float vinv = 1.0f / sqrtf(vs / (float)HD + eps);
+#pragma unroll
+    for (int j = 0; j < PER; j++)
+        pack_q40_group(xv[j] * vinv, lane & 31, vrow + (size_t)(2 * j + (lane >> 5)) * 18, true);
+}
+
+// ---- embedding gather: out[i] = scale * deq(src[id*n + i]) -------------------
+__device__ __forceinline__ float deq_q6k_at(const uint8_t *blk, int j)
+{
+    // ksearch_load_q6k, render.rs:729-756 / gguf_impl.rs:761-791: (d*sc)*q
+    const int half = j >> 7, jl = j & 127, quad = jl >> 5, l = jl & 31;
+    const uint8_t qlb = blk[64 * half + l + ((quad & 1) ? 32 : 0)];
+    const uint32_t lo = quad >= 2 ? (uint32_t)(qlb >> 4) : (uint32_t)(qlb & 0x0F);
+    const uint32_t hi = ((uint32_t)blk[128 + 32 * half + l] >> (2 * quad)) & 3u;
+    const int q = (int)(lo | (hi << 4)) - 32;
+    const float d = half_bits_to_f32((uint32_t)blk[208] | ((uint32_t)blk[209] << 8));
+    const float sc = (float)(int8_t)blk[192 + 8 * half + 2 * quad + (l >> 4)];
+    return d * sc * (float)q;
+}
+
+__device__ __forceinline__ float deq_q4k_at(const uint8_t *blk, int j)
+{
+    // ksearch_q4k_at, render.rs:12-26 / gguf_impl.rs:690-721
+    const float d = half_bits_to_f32((uint32_t)blk[0] | ((uint32_t)blk[1] << 8));
+    const float dmin = half_bits_to_f32((uint32_t)blk[2] | ((uint32_t)blk[3] << 8));
+    const uint8_t *sq = blk + 4;
+    const int sub = j >> 5;
+    uint32_t sc, mn;
+    if (sub < 4) {
+        sc = sq[sub] & 63u;
+        mn = sq[sub + 4] & 63u;
+    } else {
+        sc = (sq[sub + 4] & 0x0Fu) | ((uint32_t)(sq[sub - 4] >> 6) << 4);
+        mn = (uint32_t)(sq[sub + 4] >> 4) | ((uint32_t)(sq[sub] >> 6) << 4);
+    }
+    const uint8_t qb = blk[16 + (j >> 6) * 32 + (j & 31)];
+    const uint32_t n = (j & 32) ? (uint32_t)(qb >> 4) : (uint32_t)(qb & 0x0F);
+    return d * (float)sc * (float)n - dmin * (float)mn;
+}
+
+__global__ void copy_scale_indexed_kernel(const uint8_t *__restrict__ src, const float *__restrict__ idx,
+                                          float *out, int n, float scale, int dtype, int64_t n_rows)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    int64_t id = (int64_t)idx[0];
+    id = id < 0 ? 0 : (id >= n_rows ? n_rows - 1 : id);    // never read outside the table
+    float v;
+    if (dtype == KSH_Q6K) {
+        const uint8_t *row = src + (size_t)id * (size_t)(n / 256) * 210;
+        v = deq_q6k_at(row + (size_t)(i >> 8) * 210, i & 255);
+    } else if (dtype == KSH_Q4K) {
+        const uint8_t *row = src + (size_t)id * (size_t)(n / 256) * 144;
+        v = deq_q4k_at(row + (size_t)(i >> 8) * 144, i & 255);
+    } else {
+        v = reinterpret_cast<const float *>(src)[(size_t)id * n + i];
+    }
+    out[i] = scale * v;
+}
+
+__global__ void gelu_mul_kernel(const float *__restrict__ g, const float *__restrict__ u, float *out, int n)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    // lower.rs:4775-4838, same expression tree as the fused epilogue (:2926-2955)
+    const float ax = fminf(20.0f, fmaxf(-20.0f, g[i]));
+    const float t = 0.79788456f * (ax + 0.044715f * ((ax * ax) * ax));
+    out[i] = (0.5f * ax) * (1.0f + tanhf(t)) * u[i];
+}
+
+__global__ void copy_slice_kernel(const float *__restrict__ src, float *dst, int n)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) dst[i] = src[i];
+}
+
+// argmax_i cap*tanh(x_i/cap); lowest index wins ties.  Pass 1: one partial
+// (value, index) per workgroup; pass 2: one workgroup folds the partials.
+constexpr int kArgThreads = 256;
+
+__device__ __forceinline__ void argmax_fold(float &bv, uint32_t &bi, float v, uint32_t i)
+{
+    if (v > bv || (v == bv && i < bi)) { bv = v; bi = i; }
+}
+
+__device__ __forceinline__ void argmax_block(float &bv, uint32_t &bi, float *sv, uint32_t *si)
+{
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        const float ov = __shfl_xor(bv, off, 64);
+        const uint32_t oi = (uint32_t)__shfl_xor((int)bi, off, 64);
+        argmax_fold(bv, bi, ov, oi);
+    }
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane == 0) { sv[wave] = bv; si[wave] = bi; }
+    __syncthreads();
+    if (threadIdx.x == 0)
+        for (int w = 1; w < kArgThreads / 64; w++) argmax_fold(bv, bi, sv[w], si[w]);
+}
+
+__global__ __launch_bounds__(kArgThreads) void softcap_argmax_part_kernel(const float *__restrict__ x, int n,
+                                                                         float cap, float *pv, uint32_t *pi)
+{
+    __shared__ float sv[4];
+    __shared__ uint32_t si[4];
+    float bv = -INFINITY;
+    uint32_t bi = 0xFFFFFFFFu;
+    for (int i = blockIdx.x * kArgThreads + threadIdx.x; i < n; i += gridDim.x * kArgThreads) {
+        const float y = cap > 0.0f ? cap * tanhf(x[i] / cap) : x[i];
+        argmax_fold(bv, bi, y, (uint32_t)i);
+    }
+    argmax_block(bv, bi, sv, si);
+    if (threadIdx.x == 0) { pv[blockIdx.x] = bv; pi[blockIdx.x] = bi; }
+}
+
+__global__ __launch_bounds__(kArgThreads) void softcap_argmax_final_kernel(const float *pv, const uint32_t *pi,
+                                                                          int nparts, float *out)
+{
+    __shared__ float sv[4];
+    __shared__ uint32_t si[4];
+    float bv = -INFINITY;
+    uint32_t bi = 0xFFFFFFFFu;
+    for (int i = threadIdx.x; i < nparts; i += kArgThreads) argmax_fold(bv, bi, pv[i], pi[i]);
+    argmax_block(bv, bi, sv, si);
+    // the reference carries the index as f32 (exact below 2^24), lower.rs:6126
+    if (threadIdx.x == 0) out[0] = (float)(bi == 0xFFFFFFFFu ? 0u : bi);
+}
+
+int done(const char *what)
+{
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : hip_fail(e, what);
+}
+
+int launch_rmsnorm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
+{
+    const int n = (int)k.desc.dims[0], has_res = (int)k.desc.dims[1], has_scale = (int)k.desc.dims[2];
+    hipLaunchKernelGGL(rmsnorm_kernel, dim3(1), dim3(kNormThreads), 0, st, (const float *)a.in[0],
+                       (const float *)a.in[1], has_res ? (const float *)a.in[2] : nullptr, (float *)a.out[0], n,
+                       k.desc.params[0], has_res, has_scale, k.desc.params[1]);
+    return done("rmsnorm launch");
+}
+
+int launch_rmsnorm_add_then(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
+{
+    const int n = (int)k.desc.dims[0];
+    hipLaunchKernelGGL(rmsnorm_add_then_rmsnorm_kernel, dim3(1), dim3(kNormThreads), (size_t)n * 4, st,
+                       (const float *)a.in[0], (const float *)a.in[1], (const float *)a.in[2],
+                       (const float *)a.in[3], (float *)a.out[0], (float *)a.out[1], n, k.desc.params[0]);
+    return done("rmsnorm_add_then_rmsnorm launch");
+}
+
+int launch_per_head(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
+{
+    const int n_q = (int)k.desc.dims[0], n_kv = (int)k.desc.dims[1], hd = (int)k.desc.dims[2];
+    const dim3 grid(n_q + n_kv), block(64);
+#define KSH_PH(HD)                                                                                           \
+    hipLaunchKernelGGL((per_head_qkv_q40_kernel<HD>), grid, block, 0, st, (const float *)a.in[0],            \
+                       (const float *)a.in[1], (const float *)a.in[2], (const float *)a.in[3],               \
+                       (const float *)a.in[4], (const float *)a.in[5], (float *)a.out[0], (uint8_t *)a.out[1], \
+                       (uint8_t *)a.out[2], n_q, k.desc.params[0])
+    switch (hd) {
+    case 128: KSH_PH(128); break;
+    case 256: KSH_PH(256); break;
+    case 512: KSH_PH(512); break;
+    }
+#undef KSH_PH
+    return done("rmsnorm_per_head_qkv_q40 launch");
+}
+
+int launch_quantize_q40(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
+{
+    const int nblk = (int)(k.desc.dims[0] / 32);
+    hipLaunchKernelGGL(quantize_q40_kernel, dim3((nblk + 7) / 8), dim3(256), 0, st, (const float *)a.in[0],
+                       (uint8_t *)a.out[0], nblk);
+    return done("quantize_q40 launch");
+}
+
+int launch_copy_scale_indexed(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
+{
+    const int n = (int)k.desc.dims[0];
+    hipLaunchKernelGGL(copy_scale_indexed_kernel, dim3((n + 255) / 256), dim3(256), 0, st,
+                       (const uint8_t *)a.in[0], (const float *)a.in[1], (float *)a.out[0], n, k.desc.params[0],
+                       k.desc.dtypes[0], k.desc.dims[1]);
+    return done("copy_scale_indexed launch");
+}
+
+int launch_gelu_mul(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
+{
+    const int n = (int)k.desc.dims[0];
+    hipLaunchKernelGGL(gelu_mul_kernel, dim3((n + 255) / 256), dim3(256), 0, st, (const float *)a.in[0],
+                       (const float *)a.in[1], (float *)a.out[0], n);
+    return done("gelu_mul launch");
+}
+
+int launch_copy_slice(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
+{
+    const int n = (int)k.desc.dims[0];
+    hipLaunchKernelGGL(copy_slice_kernel, dim3((n + 255) / 256), dim3(256), 0, st, (const float *)a.in[0],
+                       (float *)a.out[0], n);
+    return done("copy_slice launch");
+}
+
+constexpr int kArgParts = 256;
+
+int launch_softcap_argmax(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
+{
+    // k.scratch holds kArgParts (value, index) pairs
+    const int n = (int)k.desc.dims[0];
+    const int parts = min(kArgParts, (n + kArgThreads - 1) / kArgThreads);
+    float *pv = (float *)k.scratch;
+    uint32_t *pi = (uint32_t *)(pv + kArgParts);
+    hipLaunchKernelGGL(softcap_argmax_part_kernel, dim3(parts), dim3(kArgThreads), 0, st, (const float *)a.in[0], n,
+                       k.desc.params[0], pv, pi);
+    hipLaunchKernelGGL(softcap_argmax_final_kernel, dim3(1), dim3(kArgThreads), 0, st, pv, pi, parts,
+                       (float *)a.out[0]);
+    return done("softcap_argmax launch");
+}
+
+}  // namespace
+
+int bind_rmsnorm(ksh_kernel &k)
+{
+    const int64_t n = k.desc.dims[0];
+    if (n <= 0 || n > (1 << 24)) return set_error("rmsnorm: n=%lld", (long long)n);
+    if (k.desc.kind == KSH_RMSNORM) {
+        const bool has_res = k.desc.dims[1] != 0;
+        k.info.n_inputs = has_res ? 3 : 2;
+        k.info.n_outputs = 1;
+        for (int i = 0; i < k.info.n_inputs; i++) { k.in_bytes[i] = (size_t)n * 4; k.in_align[i] = 4; }
+        k.out_bytes[0] = (size_t)n * 4;
+        k.out_align[0] = 4;
+        set_launch(k, 1, 1, 1, kNormThreads, 16);
+        set_name(k, "rmsnorm%s%s", has_res ? "_add" : "", k.desc.dims[2] ? "_scale" : "");
+        k.launch = launch_rmsnorm;
+        return 0;
+    }
+    // the reference stages the residual stream in threadgroup memory and
+    // refuses sizes that do not fit (lower.rs:3934-3938)
+    if (n > 8192) return set_error("rmsnorm_add_then_rmsnorm requires LOCAL staging of residual stream (n=%lld > 8192)", (long long)n);
+    k.info.n_inputs = 4;
+    k.info.n_outputs = 2;
+    for (int i = 0; i < 4; i++) { k.in_bytes[i] = (size_t)n * 4; k.in_align[i] = 4; }
+    for (int i = 0; i < 2; i++) { k.out_bytes[i] = (size_t)n * 4; k.out_align[i] = 4; }
+    set_launch(k, 1, 1, 1, kNormThreads, (uint32_t)n * 4 + 16);
+    set_name(k, "rmsnorm_add_then_rmsnorm");
+    k.launch = launch_rmsnorm_add_then;
+    return 0;
+}
+
+int bind_per_head_qkv_q40(ksh_kernel &k)
+{
+    const int64_t n_q = k.desc.dims[0], n_kv = k.desc.dims[1], hd = k.desc.dims[2];
+    if (n_q <= 0 || n_kv <= 0 || n_q > 4096 || n_kv > n_q) return set_error("rmsnorm_per_head_qkv_q40: n_q=%lld n_kv=%lld", (long long)n_q, (long long)n_kv);
+    if (hd != 128 && hd != 256 && hd != 512)
+        return set_error("rmsnorm_per_head_qkv_q40: hd=%lld is not built (128, 256, 512 are)", (long long)hd);
+    k.info.n_inputs = 6;
+    k.info.n_outputs = 3;
+    const size_t kvb = (size_t)n_kv * (hd / 32) * 18;
+    const size_t ib[6] = {(size_t)n_q * hd * 4, (size_t)hd * 4, (size_t)hd * 4, (size_t)n_kv * hd * 4, (size_t)hd * 4,
+                          (size_t)n_kv * hd * 4};
+    for (int i = 0; i < 6; i++) { k.in_bytes[i] = ib[i]; k.in_align[i] = 4; }
+    k.out_bytes[0] = (size_t)n_q * hd * 4; k.out_align[0] = 4;
+    k.out_bytes[1] = k.out_bytes[2] = kvb; k.out_align[1] = k.out_align[2] = 2;
+    set_launch(k, (uint32_t)(n_q + n_kv), 1, 1, 64, 0);
+    set_name(k, "rmsnorm_per_head_qkv_q40_hd%d", (int)hd);
+    k.launch = launch_per_head;
+    return 0;
+}
+
+int bind_quantize_q40(ksh_kernel &k)
+{
+    const int64_t n = k.desc.dims[0];
+    if (n <= 0 || n % 32 || n > (1ll << 31) - 64) return set_error("quantize_q40: n=%lld is not a positive multiple of 32", (long long)n);
+    k.info.n_inputs = 1;
+    k.info.n_outputs = 1;
+    k.in_bytes[0] = (size_t)n * 4; k.in_align[0] = 4;
+    k.out_bytes[0] = (size_t)n / 32 * 18; k.out_align[0] = 2;
+    set_launch(k, (uint32_t)((n / 32 + 7) / 8), 1, 1, 256, 0);
+    set_name(k, "quantize_q40");
+    k.launch = launch_quantize_q40;
+    return 0;
+}
+
+int bind_glue(ksh_kernel &k)
+{
+    const int64_t n = k.desc.dims[0];
+    if (n <= 0 || n > (1ll << 30)) return set_error("kernel kind %d: n=%lld", k.desc.kind, (long long)n);
+    set_launch(k, (uint32_t)((n + 255) / 256), 1, 1, 256, 0);
+    switch (k.desc.kind) {
+    case KSH_COPY_SCALE_INDEXED: {
+        const int dt = k.desc.dtypes[0];
+        const int64_t n_rows = k.desc.dims[1];
+        if (dt != KSH_Q6K && dt != KSH_Q4K && dt != KSH_F32) return set_error("copy_scale_indexed: source dtype %d is not built", dt);
+        if (n_rows <= 0) return set_error("copy_scale_indexed: dims[1] (rows in the table) must be positive");
+        const size_t rb = dt == KSH_F32 ? (size_t)n * 4 : packed_bytes(dt, (size_t)n);
+        if (!rb) return set_error("copy_scale_indexed: n=%lld is not a whole number of blocks", (long long)n);
+        k.info.n_inputs = 2;
+        k.info.n_outputs = 1;
+        k.in_bytes[0] = rb * (size_t)n_rows; k.in_align[0] = dt == KSH_F32 ? 4 : 2;
+        k.in_bytes[1] = 4; k.in_align[1] = 4;
+        k.out_bytes[0] = (size_t)n * 4; k.out_align[0] = 4;
+        set_name(k, "copy_scale_indexed_%d", dt);
+        k.launch = launch_copy_scale_indexed;
+        return 0;
+    }
+    case KSH_GELU_MUL:
+        k.info.n_inputs = 2;
+        k.info.n_outputs = 1;
+        k.in_bytes[0] = k.in_bytes[1] = k.out_bytes[0] = (size_t)n * 4;
+        k.in_align[0] = k.in_align[1] = k.out_align[0] = 4;
+        set_name(k, "gelu_mul");
+        k.launch = launch_gelu_mul;
+        return 0;
+    case KSH_COPY_SLICE:
+        k.info.n_inputs = 1;
+        k.info.n_outputs = 1;
+        k.in_bytes[0] = k.out_bytes[0] = (size_t)n * 4;
+        k.in_align[0] = k.out_align[0] = 4;
+        set_name(k, "copy_slice");
+        k.launch = launch_copy_slice;
+        return 0;
+    }
+    return set_error("bind_glue: kind %d", k.desc.kind);
+}
+
+int bind_softcap_argmax(ksh_kernel &k)
+{
+    const int64_t n = k.desc.dims[0];
+    if (n <= 0 || n >= (1 << 24)) return set_error("softcap_argmax: n=%lld (the f32 index is exact below 2^24 only)", (long long)n);
+    k.info.n_inputs = 1;
+    k.info.n_outputs = 1;
+    k.in_bytes[0] = (size_t)n * 4; k.in_align[0] = 4;
+    k.out_bytes[0] = 4; k.out_align[0] = 4;
+    k.scratch_bytes = (size_t)kArgParts * 8;
+    set_launch(k, (uint32_t)min((int64_t)kArgParts, (n + kArgThreads - 1) / kArgThreads), 1, 1, kArgThreads, 32);
+    set_name(k, "softcap_argmax");
+    k.launch = launch_softcap_argmax;
+    return 0;
+}
+
+}  // namespace ksh
+
+extern "C" int ksh_fill_zero_launch(void *ptr, size_t bytes, hipStream_t st)
+{
+    using namespace ksh;
+    const size_t n16 = bytes / 16, tail = bytes % 16;
+    size_t blocks = (n16 + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    if (blocks == 0) blocks = 1;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)blocks), dim3(256), 0, st, (uint4 *)ptr, n16,
+                       (uint8_t *)ptr + n16 * 16, tail);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : hip_fail(e, "fill_zero launch");
+}

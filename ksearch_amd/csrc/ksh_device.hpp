@@ -1,0 +1,120 @@
+// Device-side helpers shared by the gfx950 kernels: wave64 reductions over DPP,
+// half conversion, unaligned little-endian loads and Q4_K scale unpacking.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+
+#include <cstdint>
+
+namespace ksh {
+
+constexpr int kWave = 64;
+
+__device__ __forceinline__ float as_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t as_u32(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+// IEEE half bits -> f32 (exact, subnormals included)
+__device__ __forceinline__ float half_bits_to_f32(uint32_t h16)
+{
+    return __half2float(__ushort_as_half((unsigned short)h16));
+}
+
+// f32 -> half bits, round-to-nearest-even (what Metal's half() does)
+__device__ __forceinline__ uint32_t f32_to_half_bits(float f)
+{
+    return (uint32_t)__half_as_ushort(__float2half_rn(f));
+}
+
+// byte K of a dword as f32 in one instruction (v_cvt_f32_ubyteK).  Written as
+// inline asm because, given the C expression, the optimizer first folds the
+// caller's nibble mask into a per-element bit-field extract, which costs an
+// extra instruction per weight.
+template <int K>
+__device__ __forceinline__ float ubyte_f32(uint32_t w)
+{
+    float f;
+    if (K == 0) asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(f) : "v"(w));
+    if (K == 1) asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(f) : "v"(w));
+    if (K == 2) asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(f) : "v"(w));
+    if (K == 3) asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(f) : "v"(w));
+    return f;
+}
+
+// ---- DPP butterflies.  A DPP row is 16 lanes; quad_perm / row_half_mirror /
+// row_mirror combine lanes inside a row without touching LDS.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v)
+{
+    return as_f32((uint32_t)__builtin_amdgcn_update_dpp(0, (int)as_u32(v), CTRL, 0xF, 0xF, true));
+}
+
+// sum over each 16-lane row, result in every lane of the row
+__device__ __forceinline__ float row16_sum(float v)
+{
+    v += dpp_f32<0xB1>(v);   // quad_perm [1,0,3,2]
+    v += dpp_f32<0x4E>(v);   // quad_perm [2,3,0,1]
+    v += dpp_f32<0x141>(v);  // row_half_mirror
+    v += dpp_f32<0x140>(v);  // row_mirror
+    return v;
+}
+
+// sum over the whole wave64, result wave-uniform
+__device__ __forceinline__ float wave_sum(float v)
+{
+    v = row16_sum(v);
+    float a = as_f32((uint32_t)__builtin_amdgcn_readlane((int)as_u32(v), 0));
+    float b = as_f32((uint32_t)__builtin_amdgcn_readlane((int)as_u32(v), 16));
+    float c = as_f32((uint32_t)__builtin_amdgcn_readlane((int)as_u32(v), 32));
+    float d = as_f32((uint32_t)__builtin_amdgcn_readlane((int)as_u32(v), 48));
+    return (a + b) + (c + d);
+}
+
+// sums over lanes [0,32) and [32,64): lo half's total in .x, hi half's in .y
+__device__ __forceinline__ float2 wave_half_sums(float v)
+{
+    v = row16_sum(v);
+    float a = as_f32((uint32_t)__builtin_amdgcn_readlane((int)as_u32(v), 0));
+    float b = as_f32((uint32_t)__builtin_amdgcn_readlane((int)as_u32(v), 16));
+    float c = as_f32((uint32_t)__builtin_amdgcn_readlane((int)as_u32(v), 32));
+    float d = as_f32((uint32_t)__builtin_amdgcn_readlane((int)as_u32(v), 48));
+    return make_float2(a + b, c + d);
+}
+
+__device__ __forceinline__ float wave_max(float v)
+{
+    v = fmaxf(v, dpp_f32<0xB1>(v));
+    v = fmaxf(v, dpp_f32<0x4E>(v));
+    v = fmaxf(v, dpp_f32<0x141>(v));
+    v = fmaxf(v, dpp_f32<0x140>(v));
+    float a = as_f32((uint32_t)__builtin_amdgcn_readlane((int)as_u32(v), 0));
+    float b = as_f32((uint32_t)__builtin_amdgcn_readlane((int)as_u32(v), 16));
+    float c = as_f32((uint32_t)__builtin_amdgcn_readlane((int)as_u32(v), 32));
+    float d = as_f32((uint32_t)__builtin_amdgcn_readlane((int)as_u32(v), 48));
+    return fmaxf(fmaxf(a, b), fmaxf(c, d));
+}
+
+// ---- Q4_K scales.  `sy, sz, sw` are the three dwords holding the 12 scale
+// bytes (bytes 4..15 of the block).  Returns for 64-element group g (0..3) the
+// (scale, min) of its low-nibble sub-block 2g in .x/.y and of its high-nibble
+// sub-block 2g+1 in .z/.w, all as small integers.  Same bit algebra as
+// get_scale_min_k4 (crates/ksearch_gguf/src/gguf_impl.rs:563-573) in its
+// 16-bit-pair form (crates/ksearch_codegen/src/render.rs:486-489).
+__device__ __forceinline__ uint4 q4k_group_scales(uint32_t sy, uint32_t sz, uint32_t sw, int g)
+{
+    const int sh = (g & 1) * 16;
+    const uint32_t a = (sy >> sh) & 0xFFFFu;  // bytes 2iq, 2iq+1
+    const uint32_t b = (sz >> sh) & 0xFFFFu;  // bytes 4+2iq, 5+2iq
+    const uint32_t c = (sw >> sh) & 0xFFFFu;  // bytes 8+2iq, 9+2iq
+    uint32_t scp, mnp;
+    if (g < 2) {
+        scp = a & 0x3F3Fu;
+        mnp = b & 0x3F3Fu;
+    } else {
+        scp = (c & 0x0F0Fu) | ((a & 0xC0C0u) >> 2);
+        mnp = ((c >> 4) & 0x0F0Fu) | ((b & 0xC0C0u) >> 2);
+    }
+    return make_uint4(scp & 0xFFu, mnp & 0xFFu, scp >> 8, mnp >> 8);
+}
+
+}  // namespace ksh

@@ -1,0 +1,218 @@
+// BEAM schedule search and the on-disk plan cache, retargeted to gfx950 knobs.
+// File format and keying follow crates/ksearch_codegen/src/beam.rs:67-139 and
+// plan_cache.rs:9-44: one text file per (kind, dims, chip) under
+// $KSEARCH_BEAM_CACHE or ~/.cache/ksearch/beam, holding key=value lines
+// (tg, vec, unroll, nsg, nr0, ms; plus k_split and lds_tile, which a reader
+// that does not know them skips, beam.rs:112).
+#include <sys/stat.h>
+
+#include <cerrno>
+#include <cinttypes>
+#include <cstdlib>
+#include <string>
+#include <vector>
+
+#include "ksh_internal.hpp"
+
+namespace ksh {
+
+int matvec_q4k_candidates(const ksh_kernel_desc &d, ksh_sched *out, int cap);
+int matvec_q6k_candidates(const ksh_kernel_desc &d, ksh_sched *out, int cap);
+
+namespace {
+
+std::string cache_dir()
+{
+    // beam_cache_dir, beam.rs:67-79
+    if (const char *p = std::getenv("KSEARCH_BEAM_CACHE")) return p;
+    if (const char *h = std::getenv("HOME")) return std::string(h) + "/.cache/ksearch/beam";
+    return ".ksearch_beam_cache";
+}
+
+int mkdirs(const std::string &path)
+{
+    std::string cur;
+    for (size_t i = 0; i <= path.size(); i++) {
+        if (i == path.size() || path[i] == '/') {
+            if (!cur.empty() && mkdir(cur.c_str(), 0755) != 0 && errno != EEXIST) return -1;
+        }
+        if (i < path.size()) cur.push_back(path[i]);
+    }
+    return 0;
+}
+
+uint64_t fnv1a(uint64_t h, const void *data, size_t n)
+{
+    const unsigned char *p = (const unsigned char *)data;
+    for (size_t i = 0; i < n; i++) {
+        h ^= p[i];
+        h *= 0x100000001b3ull;
+    }
+    return h;
+}
+
+std::string make_key(const char *kind, const int64_t *dims, int n_dims, const char *chip)
+{
+    // plan_key, plan_cache.rs:9-22: "{kind}_{d0}x{d1}.._{hash:016x}"
+    uint64_t h = 0xcbf29ce484222325ull;
+    h = fnv1a(h, kind, strlen(kind));
+    for (int i = 0; i < n_dims; i++) {
+        const uint64_t d = (uint64_t)dims[i];
+        h = fnv1a(h, &d, sizeof(d));
+    }
+    h = fnv1a(h, chip, strlen(chip));
+    std::string s = kind;
+    s += "_";
+    for (int i = 0; i < n_dims; i++) {
+        if (i) s += "x";
+        s += std::to_string((long long)dims[i]);
+    }
+    char hex[32];
+    snprintf(hex, sizeof(hex), "_%016" PRIx64, h);
+    return s + hex;
+}
+
+}  // namespace
+}  // namespace ksh
+
+using namespace ksh;
+
+extern "C" {
+
+int ksh_plan_key(const char *kind, const int64_t *dims, int n_dims, const char *chip, char *dst, size_t n)
+{
+    if (!kind || !chip || !dst || n == 0 || n_dims < 0 || n_dims > 8 || (n_dims && !dims))
+        return set_error("ksh_plan_key: bad arguments");
+    snprintf(dst, n, "%s", make_key(kind, dims, n_dims, chip).c_str());
+    return 0;
+}
+
+int ksh_plan_save(const char *kind, const int64_t *dims, int n_dims, const char *chip, const ksh_sched *s, double ms)
+{
+    if (!kind || !chip || !s || n_dims < 0 || n_dims > 8 || (n_dims && !dims))
+        return set_error("ksh_plan_save: bad arguments");
+    const std::string dir = cache_dir();
+    if (mkdirs(dir)) return set_error("ksh_plan_save: cannot create %s", dir.c_str());
+    const std::string path = dir + "/" + make_key(kind, dims, n_dims, chip) + ".txt";
+    FILE *f = fopen(path.c_str(), "w");
+    if (!f) return set_error("ksh_plan_save: cannot write %s", path.c_str());
+    fprintf(f, "tg=%llu\nvec=%u\nunroll=%u\nnsg=%u\nnr0=%u\nms=%.6f\nk_split=%u\nlds_tile=%u\n",
+            (unsigned long long)s->tg, s->vec, s->unroll, s->nsg, s->nr0, ms, s->k_split, s->lds_tile);
+    fclose(f);
+    return 0;
+}
+
+int ksh_plan_load(const char *kind, const int64_t *dims, int n_dims, const char *chip, ksh_sched *s, double *ms)
+{
+    if (!kind || !chip || !s || n_dims < 0 || n_dims > 8 || (n_dims && !dims))
+        return set_error("ksh_plan_load: bad arguments");
+    const std::string path = cache_dir() + "/" + make_key(kind, dims, n_dims, chip) + ".txt";
+    FILE *f = fopen(path.c_str(), "r");
+    if (!f) return 1;
+    // load_beam_cache, beam.rs:90-123: tg, vec, unroll and ms are mandatory,
+    // nsg defaults to 2 and nr0 to 4, unknown keys are skipped
+    bool have_tg = false, have_vec = false, have_unroll = false, have_ms = false;
+    ksh_sched r{};
+    r.nsg = 2;
+    r.nr0 = 4;
+    double t = 0.0;
+    char line[256];
+    while (fgets(line, sizeof(line), f)) {
+        char *eq = strchr(line, '=');
+        if (!eq) continue;
+        *eq = 0;
+        const char *k = line, *v = eq + 1;
+        char *end = nullptr;
+        if (!strcmp(k, "ms")) {
+            t = strtod(v, &end);
+            have_ms = end != v;
+            continue;
+        }
+        const unsigned long long u = strtoull(v, &end, 10);
+        if (end == v) continue;
+        if (!strcmp(k, "tg")) { r.tg = u; have_tg = true; }
+        else if (!strcmp(k, "vec")) { r.vec = (uint32_t)u; have_vec = true; }
+        else if (!strcmp(k, "unroll")) { r.unroll = (uint32_t)u; have_unroll = true; }
+        else if (!strcmp(k, "nsg")) r.nsg = (uint32_t)u;
+        else if (!strcmp(k, "nr0")) r.nr0 = (uint32_t)u;
+        else if (!strcmp(k, "k_split")) r.k_split = (uint32_t)u;
+        else if (!strcmp(k, "lds_tile")) r.lds_tile = (uint32_t)u;
+    }
+    fclose(f);
+    if (!(have_tg && have_vec && have_unroll && have_ms)) return 1;
+    *s = r;
+    if (ms) *ms = t;
+    return 0;
+}
+
+const char *ksh_plan_kind(const ksh_kernel_desc *d)
+{
+    if (!d) return nullptr;
+    switch (d->kind) {
+    case KSH_MATVEC:
+        // crates/ksearch_codegen/src/lib.rs:200-205
+        return d->dtypes[0] == KSH_Q4K ? "matvec_q4k" : d->dtypes[0] == KSH_Q6K ? "matvec_q6k" : nullptr;
+    case KSH_MATVEC_QKV: return "matvec_qkv_q4k";
+    case KSH_MATVEC_GATE_UP_GELU: return "matvec_gate_up_q4k";
+    case KSH_MATVEC_BATCH: return "mul_mm_q4k";
+    case KSH_SDPA_SLOTS:
+    case KSH_SDPA_MWG_PART: return "sdpa_q40";
+    }
+    return nullptr;
+}
+
+int ksh_beam_candidates(const ksh_kernel_desc *d, ksh_sched *out, int cap)
+{
+    if (!d || !out || cap <= 0) return 0;
+    switch (d->kind) {
+    case KSH_MATVEC:
+        if (d->dtypes[0] == KSH_Q6K) return matvec_q6k_candidates(*d, out, cap);
+        return matvec_q4k_candidates(*d, out, cap);
+    case KSH_MATVEC_QKV:
+    case KSH_MATVEC_GATE_UP_GELU: return matvec_q4k_candidates(*d, out, cap);
+    }
+    return 0;
+}
+
+int ksh_beam_search(ksh_ctx *ctx, const ksh_kernel_desc *desc, ksh_buf *const *inputs, int n_in,
+                    ksh_buf *const *outputs, int n_out, int iters, int force, ksh_sched *best, double *best_ms,
+                    int *from_cache)
+{
+    if (!ctx || !desc || !best || !best_ms) return set_error("ksh_beam_search: bad arguments");
+    const char *pk = ksh_plan_kind(desc);
+    if (!pk) return set_error("ksh_beam_search: kind %d has no schedule space", desc->kind);
+    char chip[128];
+    if (ksh_device_name(ctx, chip, sizeof(chip))) return 1;
+    int nd = 0;
+    while (nd < 8 && desc->dims[nd] != 0) nd++;
+    if (from_cache) *from_cache = 0;
+    // KSEARCH_BEAM_FORCE, crates/ksearch_codegen/src/lib.rs:206
+    if (!force && !std::getenv("KSEARCH_BEAM_FORCE") && ksh_plan_load(pk, desc->dims, nd, chip, best, best_ms) == 0) {
+        if (from_cache) *from_cache = 1;
+        return 0;
+    }
+    std::vector<ksh_sched> cand(128);
+    const int n = ksh_beam_candidates(desc, cand.data(), (int)cand.size());
+    if (n <= 0) return set_error("ksh_beam_search: no candidates for kind %d", desc->kind);
+    if (iters < 1) iters = 3;
+    bool found = false;
+    for (int i = 0; i < n; i++) {
+        ksh_kernel_desc d = *desc;
+        d.sched = cand[i];
+        ksh_kernel *k = nullptr;
+        if (ksh_kernel_get(ctx, &d, &k)) continue;   // a candidate the kernel family refuses
+        double ms = 0.0;
+        // 1 warm-up + timed launches, crates/ksearch_kernels/src/lib.rs:2015-2031
+        if (ksh_run_timed(ctx, k, inputs, nullptr, n_in, outputs, nullptr, n_out, 1, &ms)) return 1;
+        if (ksh_run_timed(ctx, k, inputs, nullptr, n_in, outputs, nullptr, n_out, iters, &ms)) return 1;
+        if (!found || ms < *best_ms) {
+            found = true;
+            *best_ms = ms;
+            *best = cand[i];
+        }
+    }
+    if (!found) return set_error("ksh_beam_search: every candidate was refused");
+    return ksh_plan_save(pk, desc->dims, nd, chip, best, *best_ms);
+}
+
+}  // extern "C"

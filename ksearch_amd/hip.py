@@ -1,0 +1,537 @@
+"""ctypes binding of libksearch_hip.so (include/ksearch_hip.h).
+
+``Context`` carries the method names of ksearch's ``MetalContext``
+(crates/ksearch_metal/src/lib.rs) and ``Eng`` those of
+``ksearch_kernels::Eng`` (crates/ksearch_kernels/src/lib.rs), so code and
+tests written against the reference's runtime read the same here.  This
+module never computes anything itself: if the shared library is missing, or
+no gfx950 GPU is usable, it raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import enum
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libksearch_hip.so")
+
+
+class KshError(RuntimeError):
+    pass
+
+
+class DType(enum.IntEnum):          # crates/ksearch_ir/src/lib.rs:17-27
+    F32 = 0
+    F16 = 1
+    Q4K = 2
+    Q5K = 3
+    Q6K = 4
+    Q40 = 5
+    BF16 = 6
+
+
+class Kind(enum.IntEnum):           # enum ksh_kind
+    MATVEC = 1
+    MATVEC_BATCH = 2
+    MATVEC_QKV = 3
+    MATVEC_GATE_UP_GELU = 4
+    SDPA_NAIVE = 5
+    SDPA_MWG_PART = 6
+    SDPA_MWG_REDUCE = 7
+    SDPA_SLOTS = 8
+    QUANTIZE_Q40 = 9
+    RMSNORM = 10
+    RMSNORM_ADD_THEN_RMSNORM = 11
+    RMSNORM_PER_HEAD_QKV_Q40 = 12
+    COPY_SCALE_INDEXED = 13
+    GELU_MUL = 14
+    COPY_SLICE = 15
+    SOFTCAP_ARGMAX = 16
+    DEQUANT = 17
+    QUANTIZE_K = 18
+
+
+class Sched(C.Structure):           # ksh_sched: OptSchedule retargeted to gfx950
+    _fields_ = [("tg", C.c_uint64), ("vec", C.c_uint32), ("unroll", C.c_uint32), ("nsg", C.c_uint32),
+                ("nr0", C.c_uint32), ("k_split", C.c_uint32), ("lds_tile", C.c_uint32)]
+
+    def as_dict(self) -> dict:
+        return {n: int(getattr(self, n)) for n, _ in self._fields_}
+
+
+class KernelDesc(C.Structure):
+    _fields_ = [("kind", C.c_int32), ("dtypes", C.c_int32 * 4), ("dims", C.c_int64 * 8),
+                ("params", C.c_float * 4), ("sched", Sched)]
+
+
+class KernelInfo(C.Structure):
+    _fields_ = [("n_inputs", C.c_int32), ("n_outputs", C.c_int32), ("grid", C.c_uint32 * 3),
+                ("block", C.c_uint32 * 3), ("lds_bytes", C.c_uint32), ("sched", Sched), ("name", C.c_char * 64)]
+
+
+class GemmaCfg(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in ("n_layers", "hidden", "ffn", "n_q", "n_kv", "hd", "vocab", "max_seq")] + \
+               [(n, C.c_float) for n in ("eps", "softcap", "rope_theta", "attn_scale")]
+
+
+GEMMA_LAYER_FIELDS = ("wq", "wk", "wv", "wo", "wgate", "wup", "wdown",
+                      "attn_norm", "q_norm", "k_norm", "post_attn_norm", "ffn_norm", "post_ffw_norm")
+
+
+class GemmaLayer(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in GEMMA_LAYER_FIELDS]
+
+
+# every symbol include/ksearch_hip.h declares: name -> (restype, argtypes)
+_vp, _sz, _i, _u64p, _dp = C.c_void_p, C.c_size_t, C.c_int, C.POINTER(C.c_uint64), C.POINTER(C.c_double)
+_vpp = C.POINTER(C.c_void_p)
+_i64p = C.POINTER(C.c_int64)
+SYMBOLS = {
+    "ksh_last_error": (C.c_char_p, []),
+    "ksh_ctx_create": (_i, [_vpp]),
+    "ksh_ctx_destroy": (None, [_vp]),
+    "ksh_device_name": (_i, [_vp, C.c_char_p, _sz]),
+    "ksh_stream": (_vp, [_vp]),
+    "ksh_buffer_alloc": (_i, [_vp, _sz, _vp, _vpp]),
+    "ksh_buffer_retain": (None, [_vp]),
+    "ksh_buffer_release": (None, [_vp]),
+    "ksh_buffer_size": (_sz, [_vp]),
+    "ksh_buffer_device_ptr": (_vp, [_vp]),
+    "ksh_buffer_write": (_i, [_vp, _vp, _sz, _vp, _sz, _i]),
+    "ksh_buffer_read": (_i, [_vp, _vp, _sz, _vp, _sz, _i]),
+    "ksh_buffer_fill_zero": (_i, [_vp, _vp]),
+    "ksh_kernel_get": (_i, [_vp, C.POINTER(KernelDesc), _vpp]),
+    "ksh_kernel_info_get": (_i, [_vp, C.POINTER(KernelInfo)]),
+    "ksh_encode": (_i, [_vp, _vp, _vpp, _u64p, _i, _vpp, _u64p, _i]),
+    "ksh_run_timed": (_i, [_vp, _vp, _vpp, _u64p, _i, _vpp, _u64p, _i, _i, _dp]),
+    "ksh_flush_async": (_i, [_vp]),
+    "ksh_wait_inflight_at_most": (_i, [_vp, _i]),
+    "ksh_barrier": (_i, [_vp]),
+    "ksh_synchronize": (_i, [_vp]),
+    "ksh_has_gpu_work": (_i, [_vp]),
+    "ksh_graph_begin": (_i, [_vp]),
+    "ksh_graph_end": (_i, [_vp, _vpp]),
+    "ksh_graph_launch": (_i, [_vp, _vp]),
+    "ksh_graph_destroy": (None, [_vp]),
+    "ksh_plan_key": (_i, [C.c_char_p, _i64p, _i, C.c_char_p, C.c_char_p, _sz]),
+    "ksh_plan_save": (_i, [C.c_char_p, _i64p, _i, C.c_char_p, C.POINTER(Sched), C.c_double]),
+    "ksh_plan_load": (_i, [C.c_char_p, _i64p, _i, C.c_char_p, C.POINTER(Sched), _dp]),
+    "ksh_plan_kind": (C.c_char_p, [C.POINTER(KernelDesc)]),
+    "ksh_beam_candidates": (_i, [C.POINTER(KernelDesc), C.POINTER(Sched), _i]),
+    "ksh_beam_search": (_i, [_vp, C.POINTER(KernelDesc), _vpp, _i, _vpp, _i, _i, _i, C.POINTER(Sched), _dp,
+                             C.POINTER(C.c_int)]),
+    "ksh_gemma_create": (_i, [_vp, C.POINTER(GemmaCfg), C.POINTER(GemmaLayer), _vp, _vp, _vpp]),
+    "ksh_gemma_destroy": (None, [_vp]),
+    "ksh_gemma_reset": (_i, [_vp]),
+    "ksh_gemma_forward_token": (_i, [_vp, C.c_uint32, _i, C.POINTER(C.c_uint32)]),
+    "ksh_gemma_generate": (_i, [_vp, C.POINTER(C.c_uint32), _i, _i, _i, C.POINTER(C.c_uint32), _dp, _dp]),
+    "ksh_gemma_logits": (_vp, [_vp]),
+    "ksh_gemma_hidden": (_vp, [_vp]),
+    "ksh_gemma_kv": (_vp, [_vp, _i, _i]),
+    "ksh_gemma_pos": (_i, [_vp]),
+    "ksh_gemma_launches_per_token": (_i, [_vp]),
+}
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    """Loads the prebuilt library; never builds and never falls back."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise KshError(f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'`")
+        L = C.CDLL(LIB_PATH)
+        for name, (res, args) in SYMBOLS.items():
+            fn = getattr(L, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = L
+    return _lib
+
+
+def _check(rc: int) -> None:
+    if rc:
+        raise KshError(lib().ksh_last_error().decode())
+
+
+def make_desc(kind: int, dims=(), dtypes=(), params=(), sched: Sched | dict | None = None) -> KernelDesc:
+    d = KernelDesc()
+    d.kind = int(kind)
+    for i, v in enumerate(dims):
+        d.dims[i] = int(v)
+    for i, v in enumerate(dtypes):
+        d.dtypes[i] = int(v)
+    for i, v in enumerate(params):
+        d.params[i] = float(v)
+    if isinstance(sched, dict):
+        sched = Sched(**sched)
+    if sched is not None:
+        d.sched = sched
+    return d
+
+
+def plan_kind(desc: KernelDesc) -> str | None:
+    r = lib().ksh_plan_kind(C.byref(desc))
+    return r.decode() if r else None
+
+
+def plan_key(kind: str, dims, chip: str) -> str:
+    arr = (C.c_int64 * len(dims))(*dims)
+    buf = C.create_string_buffer(256)
+    _check(lib().ksh_plan_key(kind.encode(), arr, len(dims), chip.encode(), buf, 256))
+    return buf.value.decode()
+
+
+def plan_save(kind: str, dims, chip: str, sched: Sched, ms: float) -> None:
+    arr = (C.c_int64 * len(dims))(*dims)
+    _check(lib().ksh_plan_save(kind.encode(), arr, len(dims), chip.encode(), C.byref(sched), ms))
+
+
+def plan_load(kind: str, dims, chip: str):
+    arr = (C.c_int64 * len(dims))(*dims)
+    s, ms = Sched(), C.c_double()
+    rc = lib().ksh_plan_load(kind.encode(), arr, len(dims), chip.encode(), C.byref(s), C.byref(ms))
+    return (s, ms.value) if rc == 0 else None
+
+
+def beam_candidates(desc: KernelDesc, cap: int = 128) -> list[Sched]:
+    arr = (Sched * cap)()
+    n = lib().ksh_beam_candidates(C.byref(desc), arr, cap)
+    return [arr[i] for i in range(n)]
+
+
+class Buffer:
+    """A device allocation (the reference's metal::Buffer)."""
+
+    def __init__(self, ctx: "Context", handle: int, owned: bool = True):
+        self.ctx, self.h, self._owned = ctx, handle, owned
+
+    @property
+    def nbytes(self) -> int:
+        return lib().ksh_buffer_size(self.h)
+
+    @property
+    def device_ptr(self) -> int:
+        return lib().ksh_buffer_device_ptr(self.h)
+
+    def release(self) -> None:
+        if self.h and self._owned:
+            lib().ksh_buffer_release(self.h)
+        self.h = None
+
+    def __del__(self):
+        try:
+            self.release()
+        except Exception:
+            pass
+
+
+class Kernel:
+    def __init__(self, handle: int):
+        self.h = handle
+        info = KernelInfo()
+        _check(lib().ksh_kernel_info_get(handle, C.byref(info)))
+        self.info = info
+
+    @property
+    def name(self) -> str:
+        return self.info.name.decode()
+
+    @property
+    def grid(self):
+        return tuple(self.info.grid)
+
+    @property
+    def block(self):
+        return tuple(self.info.block)
+
+
+def _bufs(bufs):
+    arr = (C.c_void_p * max(1, len(bufs)))(*[b.h for b in bufs])
+    return arr
+
+
+def _offs(offs, n):
+    if offs is None:
+        return None
+    return (C.c_uint64 * max(1, n))(*[int(o) for o in offs])
+
+
+class Context:
+    """MetalContext for one MI355X: device 0, one in-order HIP stream."""
+
+    def __init__(self):
+        h = C.c_void_p()
+        _check(lib().ksh_ctx_create(C.byref(h)))
+        self.h = h
+
+    # -- lifetime -----------------------------------------------------------
+    def close(self) -> None:
+        if self.h:
+            lib().ksh_ctx_destroy(self.h)
+            self.h = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *a):
+        self.close()
+
+    def device_name(self) -> str:
+        buf = C.create_string_buffer(128)
+        _check(lib().ksh_device_name(self.h, buf, 128))
+        return buf.value.decode()
+
+    @property
+    def stream(self) -> int:
+        return lib().ksh_stream(self.h)
+
+    # -- buffers (crates/ksearch_metal/src/lib.rs:63-135) -------------------
+    def _alloc(self, nbytes: int, init) -> Buffer:
+        h = C.c_void_p()
+        _check(lib().ksh_buffer_alloc(self.h, nbytes, init, C.byref(h)))
+        return Buffer(self, h.value)
+
+    def buffer_bytes(self, data) -> Buffer:
+        a = np.ascontiguousarray(data)
+        return self._alloc(a.nbytes, a.ctypes.data)
+
+    def buffer_f32(self, data) -> Buffer:
+        return self.buffer_bytes(np.ascontiguousarray(data, dtype=np.float32))
+
+    def buffer_empty_bytes(self, n: int) -> Buffer:
+        return self._alloc(int(n), None)
+
+    def buffer_empty_f32(self, n: int) -> Buffer:
+        return self._alloc(int(n) * 4, None)
+
+    def buffer_empty_f16(self, n: int) -> Buffer:
+        return self._alloc(int(n) * 2, None)
+
+    def _read(self, buf: Buffer, dtype, n: int, off: int, sync: bool) -> np.ndarray:
+        out = np.empty(n, dtype=dtype)
+        _check(lib().ksh_buffer_read(self.h, buf.h, off, out.ctypes.data, out.nbytes, int(sync)))
+        return out
+
+    def read_f32(self, buf: Buffer, n: int, off: int = 0) -> np.ndarray:
+        return self._read(buf, np.float32, n, off, True)
+
+    def read_f32_nosync(self, buf: Buffer, n: int, off: int = 0) -> np.ndarray:
+        return self._read(buf, np.float32, n, off, False)
+
+    def read_u16(self, buf: Buffer, n: int, off: int = 0) -> np.ndarray:
+        return self._read(buf, np.uint16, n, off, True)
+
+    def read_bytes(self, buf: Buffer, n: int, off: int = 0) -> np.ndarray:
+        return self._read(buf, np.uint8, n, off, True)
+
+    def _write(self, buf: Buffer, data, off: int, sync: bool) -> None:
+        a = np.ascontiguousarray(data)
+        _check(lib().ksh_buffer_write(self.h, buf.h, off, a.ctypes.data, a.nbytes, int(sync)))
+
+    def write_buffer(self, buf: Buffer, data, off: int = 0) -> None:
+        self._write(buf, np.ascontiguousarray(data, dtype=np.float32), off, True)
+
+    def write_buffer_nosync(self, buf: Buffer, data, off: int = 0) -> None:
+        self._write(buf, np.ascontiguousarray(data, dtype=np.float32), off, False)
+
+    def write_u16s(self, buf: Buffer, data, off: int = 0) -> None:
+        self._write(buf, np.ascontiguousarray(data, dtype=np.uint16), off, True)
+
+    def write_bytes(self, buf: Buffer, data, off: int = 0, sync: bool = True) -> None:
+        self._write(buf, data, off, sync)
+
+    def fill_zero(self, buf: Buffer) -> None:
+        _check(lib().ksh_buffer_fill_zero(self.h, buf.h))
+
+    # -- kernels ------------------------------------------------------------
+    def compile(self, desc: KernelDesc) -> Kernel:
+        h = C.c_void_p()
+        _check(lib().ksh_kernel_get(self.h, C.byref(desc), C.byref(h)))
+        return Kernel(h.value)
+
+    def encode_offsets_multi(self, kernel: Kernel, inputs, in_offs, outputs, out_offs) -> None:
+        _check(lib().ksh_encode(self.h, kernel.h, _bufs(inputs), _offs(in_offs, len(inputs)), len(inputs),
+                                _bufs(outputs), _offs(out_offs, len(outputs)), len(outputs)))
+
+    def encode_multi(self, kernel: Kernel, inputs, outputs) -> None:
+        self.encode_offsets_multi(kernel, inputs, None, outputs, None)
+
+    def encode(self, kernel: Kernel, inputs, output) -> None:
+        self.encode_offsets_multi(kernel, inputs, None, [output], None)
+
+    def run(self, kernel: Kernel, inputs, outputs, iters: int = 1, in_offs=None, out_offs=None) -> float:
+        """Timed launches with HIP events on the context's stream; ms per launch."""
+        if isinstance(outputs, Buffer):
+            outputs = [outputs]
+        ms = C.c_double()
+        _check(lib().ksh_run_timed(self.h, kernel.h, _bufs(inputs), _offs(in_offs, len(inputs)), len(inputs),
+                                   _bufs(outputs), _offs(out_offs, len(outputs)), len(outputs), iters,
+                                   C.byref(ms)))
+        return ms.value
+
+    def flush_async(self) -> None:
+        _check(lib().ksh_flush_async(self.h))
+
+    def wait_inflight_at_most(self, n: int) -> None:
+        _check(lib().ksh_wait_inflight_at_most(self.h, n))
+
+    def encoder_barrier(self) -> None:
+        _check(lib().ksh_barrier(self.h))
+
+    def synchronize(self) -> None:
+        _check(lib().ksh_synchronize(self.h))
+
+    def has_gpu_work(self) -> bool:
+        return bool(lib().ksh_has_gpu_work(self.h))
+
+    # -- graphs -------------------------------------------------------------
+    def graph_begin(self) -> None:
+        _check(lib().ksh_graph_begin(self.h))
+
+    def graph_end(self) -> int:
+        g = C.c_void_p()
+        _check(lib().ksh_graph_end(self.h, C.byref(g)))
+        return g.value
+
+    def graph_launch(self, g: int) -> None:
+        _check(lib().ksh_graph_launch(self.h, g))
+
+    def graph_destroy(self, g: int) -> None:
+        lib().ksh_graph_destroy(g)
+
+    # -- BEAM ---------------------------------------------------------------
+    def beam_search(self, desc: KernelDesc, inputs, outputs, iters: int = 3, force: bool = False):
+        best, ms, cached = Sched(), C.c_double(), C.c_int()
+        _check(lib().ksh_beam_search(self.h, C.byref(desc), _bufs(inputs), len(inputs), _bufs(outputs),
+                                     len(outputs), iters, int(force), C.byref(best), C.byref(ms), C.byref(cached)))
+        return best, ms.value, bool(cached.value)
+
+
+class Eng:
+    """One method per op, named as in ksearch_kernels::Eng.  Each call looks up
+    (or binds) the kernel for its shape and appends one launch to the stream."""
+
+    SDPA_MWG_NWG = 16           # crates/ksearch_kernels/src/lib.rs:1114
+    SDPA_MWG_THRESHOLD = 128    # :1115
+
+    def __init__(self):
+        self.cache: dict = {}
+
+    def _k(self, ctx: Context, kind, dims=(), dtypes=(), params=(), sched=None) -> Kernel:
+        key = (int(kind), tuple(dims), tuple(int(d) for d in dtypes), tuple(params),
+               tuple(sorted(sched.items())) if isinstance(sched, dict) else None)
+        k = self.cache.get(key)
+        if k is None:
+            k = ctx.compile(make_desc(kind, dims, dtypes, params, sched))
+            self.cache[key] = k
+        return k
+
+    # :137-160
+    def matvec_wd(self, ctx, rows, cols, wdt, w, x, y, sched=None):
+        self.matvec_wd_at(ctx, rows, cols, wdt, w, x, 0, y, 0, sched)
+
+    def matvec_wd_at(self, ctx, rows, cols, wdt, w, x, x_off, y, y_off, sched=None):
+        k = self._k(ctx, Kind.MATVEC, (rows, cols), (wdt, DType.F32), (), sched)
+        ctx.encode_offsets_multi(k, [w, x], [0, x_off * 4], [y], [y_off * 4])
+
+    # :227-261
+    def matvec_qkv_wds(self, ctx, q_rows, kv_rows, cols, wdt, wq, wk, wv, x, q, k_out, v_out, sched=None):
+        k = self._k(ctx, Kind.MATVEC_QKV, (q_rows, kv_rows, cols), (wdt, DType.F32), (), sched)
+        ctx.encode_multi(k, [wq, wk, wv, x], [q, k_out, v_out])
+
+    # :953-975
+    def matvec_gate_up_gelu_wd(self, ctx, rows, cols, wdt, wg, wu, x, out, sched=None):
+        k = self._k(ctx, Kind.MATVEC_GATE_UP_GELU, (rows, cols), (wdt, DType.F32), (), sched)
+        ctx.encode_multi(k, [wg, wu, x], [out])
+
+    # :1414-1444
+    def matvec_batch(self, ctx, rows, cols, batch, wdt, w, x, y, sched=None):
+        k = self._k(ctx, Kind.MATVEC_BATCH, (rows, cols, batch), (wdt, DType.BF16, DType.F32), (), sched)
+        ctx.encode_multi(k, [w, x], [y])
+
+    # :468-490
+    def rmsnorm(self, ctx, n, eps, x, w, out):
+        k = self._k(ctx, Kind.RMSNORM, (n, 0, 0), (), (eps, 0.0))
+        ctx.encode_multi(k, [x, w], [out])
+
+    def rmsnorm_add(self, ctx, n, eps, x, w, res, out):
+        k = self._k(ctx, Kind.RMSNORM, (n, 1, 0), (), (eps, 0.0))
+        ctx.encode_multi(k, [x, w, res], [out])
+
+    def rmsnorm_add_scale(self, ctx, n, eps, scale, x, w, res, out):
+        k = self._k(ctx, Kind.RMSNORM, (n, 1, 1), (), (eps, scale))
+        ctx.encode_multi(k, [x, w, res], [out])
+
+    # :539-562
+    def rmsnorm_add_then_rmsnorm(self, ctx, n, eps, y, w_post, res, w_ffn, out_x, out_x2):
+        k = self._k(ctx, Kind.RMSNORM_ADD_THEN_RMSNORM, (n,), (), (eps,))
+        ctx.encode_multi(k, [y, w_post, res, w_ffn], [out_x, out_x2])
+
+    # :1257-1297
+    def rmsnorm_per_head_qkv_q40_off(self, ctx, n_q, n_kv, hd, eps, q, qw, rope, rope_off, k, kw, v,
+                                     q_out, k_out, v_out, kv_byte_off):
+        kk = self._k(ctx, Kind.RMSNORM_PER_HEAD_QKV_Q40, (n_q, n_kv, hd), (), (eps,))
+        ctx.encode_offsets_multi(kk, [q, qw, rope, k, kw, v], [0, 0, rope_off * 4, 0, 0, 0],
+                                 [q_out, k_out, v_out], [0, kv_byte_off, kv_byte_off])
+
+    # :1181-1197
+    def quantize_q40(self, ctx, n, src, dst, dst_byte_off=0):
+        k = self._k(ctx, Kind.QUANTIZE_Q40, (n,))
+        ctx.encode_offsets_multi(k, [src], [0], [dst], [dst_byte_off])
+
+    # :1086-1111
+    def sdpa_naive_kv(self, ctx, n_q, n_kv, hd, max_t, kv_dtype, q, k, v, meta, out, scale=1.0):
+        kk = self._k(ctx, Kind.SDPA_NAIVE, (n_q, n_kv, hd, max_t), (kv_dtype, DType.F32), (scale,))
+        ctx.encode_multi(kk, [q, k, v, meta], [out])
+
+    # :1118-1154
+    def sdpa_mwg_kv(self, ctx, n_q, n_kv, hd, max_t, kv_dtype, q, k, v, meta, tmp, out, scale=1.0, nwg=None):
+        nwg = nwg or self.SDPA_MWG_NWG
+        part = self._k(ctx, Kind.SDPA_MWG_PART, (n_q, n_kv, hd, max_t, nwg), (kv_dtype, DType.F32), (scale,))
+        red = self._k(ctx, Kind.SDPA_MWG_REDUCE, (n_q, hd, nwg))
+        ctx.encode_multi(part, [q, k, v, meta], [tmp])
+        ctx.encoder_barrier()
+        ctx.encode_multi(red, [tmp], [out])
+
+    # :1157-1178
+    def sdpa_hybrid_kv(self, ctx, n_q, n_kv, hd, max_t, attn_t, kv_dtype, q, k, v, meta, tmp, out, scale=1.0):
+        if attn_t >= self.SDPA_MWG_THRESHOLD:
+            self.sdpa_mwg_kv(ctx, n_q, n_kv, hd, max_t, kv_dtype, q, k, v, meta, tmp, out, scale)
+        else:
+            self.sdpa_naive_kv(ctx, n_q, n_kv, hd, max_t, kv_dtype, q, k, v, meta, out, scale)
+
+    def sdpa_slots(self, ctx, n_q, n_kv, hd, max_t, n_slots, q, k_pool, v_pool, meta, tmp, out, scale=1.0,
+                   nwg=0, sched=None):
+        kk = self._k(ctx, Kind.SDPA_SLOTS, (n_q, n_kv, hd, max_t, n_slots, nwg), (DType.Q40, DType.F32),
+                     (scale,), sched)
+        ctx.encode_multi(kk, [q, k_pool, v_pool, meta], [tmp, out])
+        return kk
+
+    # :1364-1384
+    def copy_scale_indexed_wd(self, ctx, n, scale, src_dtype, src, idx, out, n_rows):
+        k = self._k(ctx, Kind.COPY_SCALE_INDEXED, (n, n_rows), (src_dtype,), (scale,))
+        ctx.encode_multi(k, [src, idx], [out])
+
+    def gelu_mul(self, ctx, n, g, u, out):
+        ctx.encode_multi(self._k(ctx, Kind.GELU_MUL, (n,)), [g, u], [out])
+
+    def copy_slice(self, ctx, n, src, src_off, dst, dst_off):
+        ctx.encode_offsets_multi(self._k(ctx, Kind.COPY_SLICE, (n,)), [src], [src_off * 4], [dst], [dst_off * 4])
+
+    # :1966-1982
+    def softcap_argmax(self, ctx, n, cap, x, out):
+        ctx.encode_multi(self._k(ctx, Kind.SOFTCAP_ARGMAX, (n,), (), (cap,)), [x], [out])
+
+    def dequant(self, ctx, dtype, n, src, dst):
+        ctx.encode_multi(self._k(ctx, Kind.DEQUANT, (n,), (dtype,)), [src], [dst])
+
+    def quantize_k(self, ctx, dtype, n, src, dst):
+        ctx.encode_multi(self._k(ctx, Kind.QUANTIZE_K, (n,), (dtype,)), [src], [dst])
+
+    # :1985-2043
+    def beam_matvec(self, ctx, rows, cols, wdt, w, x, y, iters=3, force=False):
+        return ctx.beam_search(make_desc(Kind.MATVEC, (rows, cols), (wdt, DType.F32)), [w, x], [y], iters, force)

@@ -1,0 +1,18 @@
+"""Shared helpers for the GPU parity tests."""
+import numpy as np
+
+
+def rel_err(got, want):
+    """|got-want| relative to max(|want|, rms(want)): the 1e-3 bar of the GEMV /
+    attention parity tests is stated on this quantity.  The rms floor keeps
+    rows whose true value happens to cancel to ~0 from dominating."""
+    got = np.asarray(got, dtype=np.float64).ravel()
+    want = np.asarray(want, dtype=np.float64).ravel()
+    floor = np.sqrt(np.mean(want ** 2)) if want.size else 0.0
+    return np.abs(got - want) / np.maximum(np.abs(want), max(floor, 1e-30))
+
+
+def assert_close(got, want, tol, what=""):
+    e = rel_err(got, want)
+    i = int(np.argmax(e)) if e.size else 0
+    assert e.size == 0 or e[i] <= tol, f"{what}: max rel err {e[i]:.3e} at {i} (got {np.ravel(got)[i]}, want {np.ravel(want)[i]})"

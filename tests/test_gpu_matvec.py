@@ -1,0 +1,193 @@
+"""HIP GEMV family vs the CPU oracle, through the C ABI.  Bars: dequantized
+weights bit-exact; GEMV outputs within 1e-3 relative of the oracle's
+dequant + sequential-f32 dot (f32 accumulate on both sides)."""
+import numpy as np
+import pytest
+
+import oracle
+from ksearch_amd import hip, synth
+from ksearch_amd.hip import DType
+from tests.gpu_util import assert_close
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = hip.Context()
+    yield c
+    c.close()
+
+
+@pytest.fixture(scope="module")
+def eng():
+    return hip.Eng()
+
+
+def test_device_name(ctx, monkeypatch):
+    assert ctx.device_name() == "gfx950"
+    monkeypatch.setenv("KSEARCH_CHIP", "my-chip")
+    c2 = hip.Context()
+    assert c2.device_name() == "my-chip"
+    c2.close()
+
+
+@pytest.mark.parametrize("dtype,gen,n_blocks", [
+    (DType.Q4K, synth.q4k_blocks, 4099), (DType.Q6K, synth.q6k_blocks, 2051), (DType.Q40, synth.q40_blocks, 40003)])
+def test_dequant_bit_exact(ctx, eng, dtype, gen, n_blocks):
+    blocks = gen(n_blocks, seed=100 + int(dtype))
+    n = n_blocks * (32 if dtype == DType.Q40 else 256)
+    src, dst = ctx.buffer_bytes(blocks), ctx.buffer_empty_f32(n)
+    eng.dequant(ctx, dtype, n, src, dst)
+    got = ctx.read_f32(dst, n)
+    want = oracle.dequant(int(dtype), blocks, n)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_dequant_edge_blocks(ctx, eng):
+    # zero scales, saturated scales, subnormal and largest half d/dmin
+    blk = np.zeros((6, 144), dtype=np.uint8)
+    blk[1, 4:16] = 0xFF
+    blk[1, 16:] = 0xFF
+    blk[1, 0:4] = np.array([65504.0, 65504.0], dtype=np.float16).view(np.uint8)
+    blk[2, 0:4] = np.array([6e-8, 6e-8], dtype=np.float16).view(np.uint8)
+    blk[2, 4:] = 0xA5
+    blk[3, 0:4] = np.array([-1.5, 0.25], dtype=np.float16).view(np.uint8)
+    blk[3, 4:] = np.arange(140, dtype=np.uint8)
+    blk[4:] = synth.q4k_blocks(2, 5).reshape(2, 144)
+    src, dst = ctx.buffer_bytes(blk), ctx.buffer_empty_f32(6 * 256)
+    eng.dequant(ctx, DType.Q4K, 6 * 256, src, dst)
+    got, want = ctx.read_f32(dst, 6 * 256), oracle.dequant(oracle.Q4K, blk, 6 * 256)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+SCHEDS_Q4K = [None] + [dict(tg=64 * w, vec=v, unroll=1, nsg=w, nr0=r, k_split=1, lds_tile=0)
+                       for v in (0, 2) for w, r in ((4, 4), (4, 1), (2, 2), (8, 2), (1, 4))]
+
+
+@pytest.mark.parametrize("rows,cols", [(64, 256), (128, 256), (2048, 1536), (50, 2048), (37, 4096), (33, 8192), (512, 4096)])
+@pytest.mark.parametrize("sched", SCHEDS_Q4K[:5])
+def test_matvec_q4k_small(ctx, eng, rows, cols, sched):
+    w = synth.q4k_blocks(rows * cols // 256, seed=rows + cols)
+    x = synth.normal_f32(cols, seed=7)
+    bw, bx, by = ctx.buffer_bytes(w), ctx.buffer_f32(x), ctx.buffer_empty_f32(rows)
+    eng.matvec_wd(ctx, rows, cols, DType.Q4K, bw, bx, by, sched)
+    assert_close(ctx.read_f32(by, rows), oracle.matvec(oracle.Q4K, w, rows, cols, x), TOL, f"q4k {rows}x{cols} {sched}")
+
+
+@pytest.mark.parametrize("sched", SCHEDS_Q4K)
+def test_matvec_q4k_cfg0_full_size(ctx, eng, sched):
+    rows = cols = 4096
+    w, x = synth.cfg0_q4k_matvec()
+    bw, bx, by = ctx.buffer_bytes(w), ctx.buffer_f32(x), ctx.buffer_empty_f32(rows)
+    eng.matvec_wd(ctx, rows, cols, DType.Q4K, bw, bx, by, sched)
+    got = ctx.read_f32(by, rows)
+    want = oracle.matvec(oracle.Q4K, w, rows, cols, x)
+    assert_close(got, want, TOL, f"cfg0 {sched}")
+    # and it sits closer to the f64 truth than 1e-4, so the bar is not eaten by the GPU side alone
+    assert_close(got, oracle.matvec_f64(oracle.Q4K, w, rows, cols, x), 1e-4, "cfg0 vs f64")
+
+
+def test_matvec_q4k_unit_vectors_recover_weights(ctx, eng):
+    # y = W e_j is column j of the dequantized matrix: pins the lane -> element map
+    rows, cols = 8, 4096
+    w = synth.q4k_blocks(rows * cols // 256, seed=3)
+    wd = oracle.dequant(oracle.Q4K, w, rows * cols).reshape(rows, cols)
+    bw, by = ctx.buffer_bytes(w), ctx.buffer_empty_f32(rows)
+    for j in [0, 1, 15, 16, 31, 32, 63, 64, 255, 256, 1000, 2047, 2048, 4095]:
+        e = np.zeros(cols, dtype=np.float32)
+        e[j] = 1.0
+        eng.matvec_wd(ctx, rows, cols, DType.Q4K, bw, ctx.buffer_f32(e), by)
+        assert np.allclose(ctx.read_f32(by, rows), wd[:, j], rtol=1e-6, atol=1e-9), j
+
+
+def test_matvec_offsets_and_errors(ctx, eng):
+    rows, cols = 64, 512
+    w = synth.q4k_blocks(rows * cols // 256, seed=9)
+    xs = synth.normal_f32(3 * cols, seed=10)
+    bw, bx, by = ctx.buffer_bytes(w), ctx.buffer_f32(xs), ctx.buffer_empty_f32(3 * rows)
+    for t in range(3):
+        eng.matvec_wd_at(ctx, rows, cols, DType.Q4K, bw, bx, t * cols, by, t * rows)
+    got = ctx.read_f32(by, 3 * rows).reshape(3, rows)
+    for t in range(3):
+        assert_close(got[t], oracle.matvec(oracle.Q4K, w, rows, cols, xs[t * cols:(t + 1) * cols]), TOL)
+    k = ctx.compile(hip.make_desc(hip.Kind.MATVEC, (rows, cols), (DType.Q4K, DType.F32)))
+    with pytest.raises(hip.KshError, match="expected 2 inputs, got 1"):
+        ctx.encode_offsets_multi(k, [bw], None, [by], None)
+    with pytest.raises(hip.KshError, match="expected 1 outputs, got 2"):
+        ctx.encode_offsets_multi(k, [bw, bx], None, [by, by], None)
+    with pytest.raises(hip.KshError, match="needs"):
+        ctx.encode_offsets_multi(k, [bw, bx], [0, 3 * cols * 4 - 16], [by], [0])
+    with pytest.raises(hip.KshError, match="not built"):
+        ctx.compile(hip.make_desc(hip.Kind.MATVEC, (rows, cols), (DType.Q5K, DType.F32)))
+    with pytest.raises(hip.KshError, match="multiple of 256"):
+        ctx.compile(hip.make_desc(hip.Kind.MATVEC, (rows, 300), (DType.Q4K, DType.F32)))
+
+
+SCHEDS_Q6K = [None, dict(tg=256, vec=0, unroll=2, nsg=4, nr0=1, k_split=1, lds_tile=0),
+              dict(tg=512, vec=0, unroll=8, nsg=8, nr0=4, k_split=1, lds_tile=0),
+              dict(tg=128, vec=0, unroll=2, nsg=2, nr0=2, k_split=1, lds_tile=0)]
+
+
+@pytest.mark.parametrize("rows,cols", [(8, 2048), (1000, 2048), (4099, 2048), (300, 4096)])
+@pytest.mark.parametrize("sched", SCHEDS_Q6K)
+def test_matvec_q6k(ctx, eng, rows, cols, sched):
+    w = synth.q6k_blocks(rows * cols // 256, seed=rows)
+    x = synth.normal_f32(cols, seed=11)
+    bw, bx, by = ctx.buffer_bytes(w), ctx.buffer_f32(x), ctx.buffer_empty_f32(rows)
+    eng.matvec_wd(ctx, rows, cols, DType.Q6K, bw, bx, by, sched)
+    assert_close(ctx.read_f32(by, rows), oracle.matvec(oracle.Q6K, w, rows, cols, x), TOL, f"q6k {rows}x{cols} {sched}")
+
+
+def test_matvec_q6k_unit_vectors(ctx, eng):
+    rows, cols = 4, 2048
+    w = synth.q6k_blocks(rows * cols // 256, seed=4)
+    wd = oracle.dequant(oracle.Q6K, w, rows * cols).reshape(rows, cols)
+    bw, by = ctx.buffer_bytes(w), ctx.buffer_empty_f32(rows)
+    for j in [0, 7, 8, 15, 16, 31, 32, 64, 96, 127, 128, 255, 256, 2047]:
+        e = np.zeros(cols, dtype=np.float32)
+        e[j] = 1.0
+        eng.matvec_wd(ctx, rows, cols, DType.Q6K, bw, ctx.buffer_f32(e), by)
+        assert np.allclose(ctx.read_f32(by, rows), wd[:, j], rtol=1e-6, atol=1e-9), j
+
+
+def test_lm_head_cfg1_full_size_with_argmax(ctx, eng):
+    rows, cols = 262144, 2048
+    w, x = synth.cfg1_q6k_lm_head()
+    bw, bx, by = ctx.buffer_bytes(w), ctx.buffer_f32(x), ctx.buffer_empty_f32(rows)
+    bi = ctx.buffer_empty_f32(1)
+    eng.matvec_wd(ctx, rows, cols, DType.Q6K, bw, bx, by)
+    eng.softcap_argmax(ctx, rows, 30.0, by, bi)
+    got = ctx.read_f32(by, rows)
+    want = oracle.matvec(oracle.Q6K, w, rows, cols, x)
+    assert_close(got, want, TOL, "cfg1 logits")
+    # the GPU argmax of the GPU logits follows the oracle's rule on the same logits ...
+    assert int(ctx.read_f32(bi, 1)[0]) == oracle.softcap_argmax(got, 30.0)
+    # ... and equals the oracle's token whenever the oracle's top-2 margin exceeds the tolerance
+    top2 = np.sort(want)[-2:]
+    if top2[1] - top2[0] > 2 * TOL * abs(top2[1]):
+        assert int(ctx.read_f32(bi, 1)[0]) == oracle.softcap_argmax(want, 30.0)
+
+
+@pytest.mark.parametrize("q_rows,kv_rows,cols", [(2048, 256, 2048), (512, 256, 4096), (100, 36, 1024)])
+def test_matvec_qkv(ctx, eng, q_rows, kv_rows, cols):
+    ws = [synth.q4k_blocks(r * cols // 256, seed=20 + i) for i, r in enumerate((q_rows, kv_rows, kv_rows))]
+    x = synth.normal_f32(cols, seed=23)
+    bws = [ctx.buffer_bytes(w) for w in ws]
+    outs = [ctx.buffer_empty_f32(r) for r in (q_rows, kv_rows, kv_rows)]
+    eng.matvec_qkv_wds(ctx, q_rows, kv_rows, cols, DType.Q4K, *bws, ctx.buffer_f32(x), *outs)
+    for w, r, o in zip(ws, (q_rows, kv_rows, kv_rows), outs):
+        assert_close(ctx.read_f32(o, r), oracle.matvec(oracle.Q4K, w, r, cols, x), TOL, f"qkv {r}")
+
+
+@pytest.mark.parametrize("rows,cols", [(8192, 2048), (100, 4096), (64, 512)])
+def test_matvec_gate_up_gelu(ctx, eng, rows, cols):
+    wg = synth.q4k_blocks(rows * cols // 256, seed=30)
+    wu = synth.q4k_blocks(rows * cols // 256, seed=31)
+    x = synth.normal_f32(cols, seed=32, std=0.05)      # keeps gate values inside GELU's curved range
+    out = ctx.buffer_empty_f32(rows)
+    eng.matvec_gate_up_gelu_wd(ctx, rows, cols, DType.Q4K, ctx.buffer_bytes(wg), ctx.buffer_bytes(wu), ctx.buffer_f32(x), out)
+    g = oracle.matvec(oracle.Q4K, wg, rows, cols, x)
+    u = oracle.matvec(oracle.Q4K, wu, rows, cols, x)
+    assert_close(ctx.read_f32(out, rows), oracle.gelu_mul(g, u), TOL, "gate_up_gelu")

@@ -84,8 +84,11 @@ enum ksh_kind {
     /* RmsNormAddThenRmsNorm.  dims: n.  params[0] = eps.
      * in: y, w_post, residual, w_ffn   out: x, x2 */
     KSH_RMSNORM_ADD_THEN_RMSNORM = 11,
-    /* RmsNormPerHeadQkvQ40 (n_tok = 1).  dims: n_q, n_kv, hd.  params[0] = eps.
-     * in: q, qw, rope_row f32[hd], k, kw, v   out: q_out f32, K row Q4_0, V row Q4_0 */
+    /* RmsNormPerHeadQkvQ40 (n_tok = 1).  dims: n_q, n_kv, hd, max_seq.  params[0] = eps.
+     * max_seq = 0: in: q, qw, rope_row f32[hd], k, kw, v   out: q_out f32, K row Q4_0,
+     * V row Q4_0 (the caller applies the position as byte offsets, as the reference does).
+     * max_seq > 0: a 7th input meta f32[4] carries the position in [3]; rope is then the
+     * whole table f32[max_seq, hd] and the outputs are the cache bases. */
     KSH_RMSNORM_PER_HEAD_QKV_Q40 = 12,
     /* CopyScaleIndexed: out[i] = scale * deq(src[id*n + i]); id is read from a
      * device f32 (the reference keeps token ids as f32).  dims: n.

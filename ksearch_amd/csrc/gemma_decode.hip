@@ -1,0 +1,331 @@
+// Greedy decode loop for the synthetic Gemma-4-E2B shape, above the C ABI.
+//
+// Mirrors GemmaPrimModel::forward_token and generate_timed
+// (crates/ksearch_gemma/src/gemma_prim.rs:881-1275, 1658-1768) without the
+// parts that shape lacks (per-layer embeddings, sliding-window layers, shared
+// KV): per layer
+//   rmsnorm -> fused QKV GEMV -> per-head RMS + RoPE + Q4_0 KV append ->
+//   split-KV attention -> o-proj GEMV -> add-then-rmsnorm ->
+//   fused gate||up + GELU GEMV -> down GEMV -> rmsnorm_add
+// then the output norm, the Q6_K LM head and the soft-capped argmax.
+//
+// What differs from the reference's host loop, and why:
+//   - the position lives in a device buffer (meta = {tlen, start, window,
+//     pos}) that a one-thread kernel advances at the end of each token, so the
+//     whole token is one HIP graph that is replayed unchanged; the reference
+//     re-encodes every token with host-side offsets (:941, :976, :1017);
+//   - the next token id never leaves the device: argmax writes it where the
+//     embedding gather of the next step reads it (the reference ping-pongs two
+//     buffers for the same purpose, :1237-1241) and a history array keeps
+//     every id for one read-back at the end.
+#include <chrono>
+#include <cmath>
+#include <memory>
+#include <vector>
+
+#include "ksh_device.hpp"
+#include "ksh_internal.hpp"
+
+namespace {
+
+// end of token: remember the id, advance position and attended length
+__global__ void advance_kernel(float *meta, const float *tok, float *history, int max_hist)
+{
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        const int pos = (int)meta[3];
+        if (history && pos < max_hist) history[pos] = tok[0];
+        meta[3] = (float)(pos + 1);
+        meta[0] = (float)(pos + 2);   // the next token attends rows [0, pos+1]
+    }
+}
+
+// the id the next embedding gather reads; a kernel rather than a copy so that
+// it is ordered behind the previous token's work on the same stream
+__global__ void set_token_kernel(float *tok, float value)
+{
+    if (threadIdx.x == 0 && blockIdx.x == 0) tok[0] = value;
+}
+
+struct Bufs {
+    std::vector<ksh_buf *> owned;
+    ~Bufs()
+    {
+        for (ksh_buf *b : owned) ksh_buffer_release(b);
+    }
+};
+
+}  // namespace
+
+struct ksh_gemma {
+    ksh_ctx *ctx = nullptr;
+    ksh_gemma_cfg c{};
+    std::vector<ksh_gemma_layer> layers;
+    ksh_buf *embd = nullptr, *output_norm = nullptr;
+    Bufs bufs;
+    ksh_buf *x = nullptr, *x2 = nullptr, *tq = nullptr, *tk = nullptr, *tv = nullptr, *to = nullptr, *ff = nullptr,
+            *logits = nullptr, *tok = nullptr, *meta = nullptr, *rope = nullptr, *attn_tmp = nullptr,
+            *history = nullptr;
+    std::vector<ksh_buf *> kv_k, kv_v;
+    ksh_kernel *k_embed = nullptr, *k_rms = nullptr, *k_qkv = nullptr, *k_head = nullptr, *k_sdpa = nullptr,
+               *k_oproj = nullptr, *k_add_then = nullptr, *k_gate_up = nullptr, *k_down = nullptr,
+               *k_rms_add = nullptr, *k_lm_head = nullptr, *k_argmax = nullptr;
+    ksh_graph *g_body = nullptr, *g_full = nullptr;
+    int pos = 0;
+    int launches_full = 0;
+    int nwg = 16;
+};
+
+namespace {
+
+using namespace ksh;
+
+int alloc(ksh_gemma *m, size_t bytes, ksh_buf **out)
+{
+    if (ksh_buffer_alloc(m->ctx, bytes, nullptr, out)) return 1;
+    m->bufs.owned.push_back(*out);
+    return 0;
+}
+
+int get(ksh_gemma *m, int kind, std::initializer_list<int64_t> dims, std::initializer_list<int> dtypes,
+        std::initializer_list<float> params, ksh_kernel **out)
+{
+    ksh_kernel_desc d;
+    memset(&d, 0, sizeof(d));
+    d.kind = kind;
+    int i = 0;
+    for (int64_t v : dims) d.dims[i++] = v;
+    i = 0;
+    for (int v : dtypes) d.dtypes[i++] = v;
+    i = 0;
+    for (float v : params) d.params[i++] = v;
+    return ksh_kernel_get(m->ctx, &d, out);
+}
+
+int enc(ksh_gemma *m, ksh_kernel *k, std::initializer_list<ksh_buf *> in, std::initializer_list<ksh_buf *> out,
+        int &count)
+{
+    ksh_buf *ib[kMaxIn], *ob[kMaxOut];
+    int ni = 0, no = 0;
+    for (ksh_buf *b : in) ib[ni++] = b;
+    for (ksh_buf *b : out) ob[no++] = b;
+    count += 1;
+    return ksh_encode(m->ctx, k, ib, nullptr, ni, ob, nullptr, no);
+}
+
+// one token: embedding gather -> layers (-> logits -> argmax) -> advance
+int encode_token(ksh_gemma *m, bool want_logits, int &launches)
+{
+    const ksh_gemma_cfg &c = m->c;
+    launches = 0;
+    if (enc(m, m->k_embed, {m->embd, m->tok}, {m->x}, launches)) return 1;
+    for (int l = 0; l < c.n_layers; l++) {
+        const ksh_gemma_layer &L = m->layers[l];
+        if (enc(m, m->k_rms, {m->x, L.attn_norm}, {m->x2}, launches)) return 1;
+        if (enc(m, m->k_qkv, {L.wq, L.wk, L.wv, m->x2}, {m->tq, m->tk, m->tv}, launches)) return 1;
+        if (enc(m, m->k_head, {m->tq, L.q_norm, m->rope, m->tk, L.k_norm, m->tv, m->meta},
+                {m->tq, m->kv_k[l], m->kv_v[l]}, launches))
+            return 1;
+        if (enc(m, m->k_sdpa, {m->tq, m->kv_k[l], m->kv_v[l], m->meta}, {m->attn_tmp, m->to}, launches)) return 1;
+        launches += 1;   // the attention kind is two launches (partials, merge)
+        if (enc(m, m->k_oproj, {L.wo, m->to}, {m->x2}, launches)) return 1;
+        if (enc(m, m->k_add_then, {m->x2, L.post_attn_norm, m->x, L.ffn_norm}, {m->x, m->x2}, launches)) return 1;
+        if (enc(m, m->k_gate_up, {L.wgate, L.wup, m->x2}, {m->ff}, launches)) return 1;
+        if (enc(m, m->k_down, {L.wdown, m->ff}, {m->x2}, launches)) return 1;
+        if (enc(m, m->k_rms_add, {m->x2, L.post_ffw_norm, m->x}, {m->x}, launches)) return 1;
+    }
+    if (want_logits) {
+        if (enc(m, m->k_rms, {m->x, m->output_norm}, {m->x2}, launches)) return 1;
+        if (enc(m, m->k_lm_head, {m->embd, m->x2}, {m->logits}, launches)) return 1;
+        if (enc(m, m->k_argmax, {m->logits}, {m->tok}, launches)) return 1;
+        launches += 1;   // two passes
+    }
+    hipStream_t st = (hipStream_t)ksh_stream(m->ctx);
+    hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(64), 0, st, (float *)ksh_buffer_device_ptr(m->meta),
+                       (const float *)ksh_buffer_device_ptr(m->tok),
+                       want_logits ? (float *)ksh_buffer_device_ptr(m->history) : nullptr, c.max_seq);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return hip_fail(e, "advance launch");
+    launches += 1;
+    return 0;
+}
+
+int run_token(ksh_gemma *m, bool want_logits, bool use_graph)
+{
+    if (m->pos >= m->c.max_seq) return set_error("max_seq exceeded");   // gemma_prim.rs:882-884
+    int n = 0;
+    if (!use_graph) {
+        if (encode_token(m, want_logits, n)) return 1;
+    } else {
+        ksh_graph *&g = want_logits ? m->g_full : m->g_body;
+        if (!g) {
+            if (ksh_synchronize(m->ctx)) return 1;
+            if (ksh_graph_begin(m->ctx)) return 1;
+            if (encode_token(m, want_logits, n)) {
+                ksh_graph *dead = nullptr;
+                ksh_graph_end(m->ctx, &dead);
+                ksh_graph_destroy(dead);
+                return 1;
+            }
+            if (ksh_graph_end(m->ctx, &g)) return 1;
+            if (want_logits) m->launches_full = n;
+        }
+        if (ksh_graph_launch(m->ctx, g)) return 1;
+    }
+    if (want_logits && !use_graph) m->launches_full = n;
+    m->pos += 1;
+    return 0;
+}
+
+int write_token(ksh_gemma *m, uint32_t token)
+{
+    // ids are carried as f32 (exact below 2^24), gemma_prim.rs:893
+    hipLaunchKernelGGL(set_token_kernel, dim3(1), dim3(64), 0, (hipStream_t)ksh_stream(m->ctx),
+                       (float *)ksh_buffer_device_ptr(m->tok), (float)token);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : hip_fail(e, "set_token launch");
+}
+
+}  // namespace
+
+extern "C" {
+
+int ksh_gemma_create(ksh_ctx *ctx, const ksh_gemma_cfg *cfg, const ksh_gemma_layer *layers, ksh_buf *token_embd_q6k,
+                     ksh_buf *output_norm, ksh_gemma **out)
+{
+    if (!ctx || !cfg || !layers || !token_embd_q6k || !output_norm || !out) return set_error("ksh_gemma_create: bad arguments");
+    *out = nullptr;
+    const ksh_gemma_cfg &c = *cfg;
+    if (c.n_layers <= 0 || c.hidden <= 0 || c.hidden % 256 || c.ffn <= 0 || c.ffn % 256 || c.n_q <= 0 || c.n_kv <= 0 ||
+        c.n_q % c.n_kv || c.hd <= 0 || c.vocab <= 0 || c.max_seq <= 0 || c.vocab >= (1 << 24))
+        return set_error("ksh_gemma_create: invalid configuration");
+    auto m = std::make_unique<ksh_gemma>();
+    m->ctx = ctx;
+    m->c = c;
+    m->layers.assign(layers, layers + c.n_layers);
+    m->embd = token_embd_q6k;
+    m->output_norm = output_norm;
+    const int64_t qd = (int64_t)c.n_q * c.hd, kvd = (int64_t)c.n_kv * c.hd;
+    const size_t kv_bytes = (size_t)c.max_seq * c.n_kv * (c.hd / 32) * 18;   // kv_pool.rs:113-116
+    ksh_gemma *g = m.get();
+    if (alloc(g, (size_t)c.hidden * 4, &g->x) || alloc(g, (size_t)c.hidden * 4, &g->x2) ||
+        alloc(g, (size_t)qd * 4, &g->tq) || alloc(g, (size_t)kvd * 4, &g->tk) || alloc(g, (size_t)kvd * 4, &g->tv) ||
+        alloc(g, (size_t)qd * 4, &g->to) || alloc(g, (size_t)c.ffn * 4, &g->ff) ||
+        alloc(g, (size_t)c.vocab * 4, &g->logits) || alloc(g, 16, &g->tok) || alloc(g, 16, &g->meta) ||
+        alloc(g, (size_t)c.max_seq * 4, &g->history))
+        return 1;
+    g->kv_k.resize(c.n_layers);
+    g->kv_v.resize(c.n_layers);
+    for (int l = 0; l < c.n_layers; l++)
+        if (alloc(g, kv_bytes, &g->kv_k[l]) || alloc(g, kv_bytes, &g->kv_v[l])) return 1;
+    // RoPE table, gemma_prim.rs:33-56: per position cos[0..hd/2) || sin[0..hd/2),
+    // frequency in f64 then f32, angle = pos * freq in f32
+    {
+        const int half = c.hd / 2;
+        std::vector<float> tab((size_t)c.max_seq * c.hd);
+        for (int pos = 0; pos < c.max_seq; pos++)
+            for (int i = 0; i < half; i++) {
+                const float freq = (float)(1.0 / std::pow((double)c.rope_theta, (double)(2 * i) / (double)c.hd));
+                const float ang = (float)pos * freq;
+                tab[(size_t)pos * c.hd + i] = std::cos(ang);
+                tab[(size_t)pos * c.hd + half + i] = std::sin(ang);
+            }
+        if (ksh_buffer_alloc(ctx, tab.size() * 4, tab.data(), &g->rope)) return 1;
+        g->bufs.owned.push_back(g->rope);
+    }
+    if (alloc(g, (size_t)c.n_q * g->nwg * (c.hd + 2) * 4, &g->attn_tmp)) return 1;
+
+    const float embed_scale = std::sqrt((float)c.hidden);   // gemma_prim.rs:683
+    if (get(g, KSH_COPY_SCALE_INDEXED, {c.hidden, c.vocab}, {KSH_Q6K}, {embed_scale}, &g->k_embed) ||
+        get(g, KSH_RMSNORM, {c.hidden, 0, 0}, {}, {c.eps, 0.f}, &g->k_rms) ||
+        get(g, KSH_MATVEC_QKV, {qd, kvd, c.hidden}, {KSH_Q4K, KSH_F32}, {}, &g->k_qkv) ||
+        get(g, KSH_RMSNORM_PER_HEAD_QKV_Q40, {c.n_q, c.n_kv, c.hd, c.max_seq}, {}, {c.eps}, &g->k_head) ||
+        get(g, KSH_SDPA_SLOTS, {c.n_q, c.n_kv, c.hd, c.max_seq, 1, g->nwg}, {KSH_Q40, KSH_F32}, {c.attn_scale}, &g->k_sdpa) ||
+        get(g, KSH_MATVEC, {c.hidden, qd}, {KSH_Q4K, KSH_F32}, {}, &g->k_oproj) ||
+        get(g, KSH_RMSNORM_ADD_THEN_RMSNORM, {c.hidden}, {}, {c.eps}, &g->k_add_then) ||
+        get(g, KSH_MATVEC_GATE_UP_GELU, {c.ffn, c.hidden}, {KSH_Q4K, KSH_F32}, {}, &g->k_gate_up) ||
+        get(g, KSH_MATVEC, {c.hidden, c.ffn}, {KSH_Q4K, KSH_F32}, {}, &g->k_down) ||
+        get(g, KSH_RMSNORM, {c.hidden, 1, 0}, {}, {c.eps, 0.f}, &g->k_rms_add) ||
+        get(g, KSH_MATVEC, {c.vocab, c.hidden}, {KSH_Q6K, KSH_F32}, {}, &g->k_lm_head) ||
+        get(g, KSH_SOFTCAP_ARGMAX, {c.vocab}, {}, {c.softcap}, &g->k_argmax))
+        return 1;
+    if (ksh_gemma_reset(g)) return 1;
+    *out = m.release();
+    return 0;
+}
+
+void ksh_gemma_destroy(ksh_gemma *m)
+{
+    if (!m) return;
+    ksh_synchronize(m->ctx);
+    ksh_graph_destroy(m->g_body);
+    ksh_graph_destroy(m->g_full);
+    delete m;
+}
+
+int ksh_gemma_reset(ksh_gemma *m)
+{
+    if (!m) return set_error("ksh_gemma_reset: null model");
+    if (ksh_synchronize(m->ctx)) return 1;
+    const float meta[4] = {1.f, 0.f, 0.f, 0.f};   // tlen, start, window, pos
+    if (ksh_buffer_write(m->ctx, m->meta, 0, meta, 16, 1)) return 1;
+    m->pos = 0;
+    return 0;
+}
+
+int ksh_gemma_forward_token(ksh_gemma *m, uint32_t token, int use_graph, uint32_t *next_id)
+{
+    if (!m) return set_error("ksh_gemma_forward_token: null model");
+    if (token >= (uint32_t)m->c.vocab) return set_error("token id %u is outside the vocabulary", token);
+    if (write_token(m, token)) return 1;
+    if (run_token(m, true, use_graph != 0)) return 1;
+    if (next_id) {
+        float f = 0.f;
+        if (ksh_buffer_read(m->ctx, m->tok, 0, &f, 4, 1)) return 1;
+        *next_id = (uint32_t)f;
+    }
+    return 0;
+}
+
+int ksh_gemma_generate(ksh_gemma *m, const uint32_t *prompt, int n_prompt, int n_new, int use_graph, uint32_t *out_ids,
+                       double *prefill_ms, double *decode_ms)
+{
+    if (!m || !prompt || n_prompt < 1 || n_new < 0 || (n_new && !out_ids)) return set_error("ksh_gemma_generate: bad arguments");
+    if (m->pos + n_prompt - 1 + n_new > m->c.max_seq) return set_error("max_seq exceeded");
+    for (int i = 0; i < n_prompt; i++)
+        if (prompt[i] >= (uint32_t)m->c.vocab) return set_error("token id %u is outside the vocabulary", prompt[i]);
+    using clk = std::chrono::steady_clock;
+    const auto t0 = clk::now();
+    // all prompt tokens but the last go through without logits (gemma_prim.rs:1670-1675)
+    for (int i = 0; i + 1 < n_prompt; i++) {
+        if (write_token(m, prompt[i])) return 1;
+        if (run_token(m, false, use_graph != 0)) return 1;
+    }
+    if (write_token(m, prompt[n_prompt - 1])) return 1;
+    if (ksh_synchronize(m->ctx)) return 1;
+    const auto t1 = clk::now();
+    const int first = m->pos;
+    for (int i = 0; i < n_new; i++)
+        if (run_token(m, true, use_graph != 0)) return 1;
+    if (ksh_synchronize(m->ctx)) return 1;
+    const auto t2 = clk::now();
+    if (prefill_ms) *prefill_ms = std::chrono::duration<double, std::milli>(t1 - t0).count();
+    if (decode_ms) *decode_ms = std::chrono::duration<double, std::milli>(t2 - t1).count();
+    if (n_new) {
+        std::vector<float> ids((size_t)n_new);
+        if (ksh_buffer_read(m->ctx, m->history, (size_t)first * 4, ids.data(), (size_t)n_new * 4, 1)) return 1;
+        for (int i = 0; i < n_new; i++) out_ids[i] = (uint32_t)ids[i];
+    }
+    return 0;
+}
+
+ksh_buf *ksh_gemma_logits(ksh_gemma *m) { return m ? m->logits : nullptr; }
+ksh_buf *ksh_gemma_hidden(ksh_gemma *m) { return m ? m->x : nullptr; }
+ksh_buf *ksh_gemma_kv(ksh_gemma *m, int layer, int which)
+{
+    if (!m || layer < 0 || layer >= m->c.n_layers) return nullptr;
+    return which ? m->kv_v[layer] : m->kv_k[layer];
+}
+int ksh_gemma_pos(ksh_gemma *m) { return m ? m->pos : -1; }
+int ksh_gemma_launches_per_token(ksh_gemma *m) { return m ? m->launches_full : -1; }
+
+}  // extern "C"

@@ -127,10 +127,21 @@ template <int HD>
 __global__ __launch_bounds__(64) void per_head_qkv_q40_kernel(
     const float *q, const float *__restrict__ qw, const float *__restrict__ rope,
     const float *__restrict__ k, const float *__restrict__ kw, const float *__restrict__ v,
-    float *q_out, uint8_t *k_out, uint8_t *v_out, int n_q, float eps)
+    float *q_out, uint8_t *k_out, uint8_t *v_out, int n_q, int n_kv, float eps, const float *meta,
+    int max_seq)
 {
     constexpr int HALF = HD / 2, PER = HD / 64;   // elements per lane
     const int lane = threadIdx.x;
+    if (meta) {
+        // position kept on the device (meta[3]): the rope input is the whole
+        // table and the K/V outputs are the cache bases, so that one captured
+        // graph serves every token
+        // clamped: a position at or past max_seq must never write outside the cache
+        const size_t pos = (size_t)min(max((int)meta[3], 0), max_seq - 1);
+        rope += pos * HD;
+        k_out += pos * (size_t)n_kv * (HD / 32) * 18;
+        v_out += pos * (size_t)n_kv * (HD / 32) * 18;
+    }
     const int head = blockIdx.x;
     const bool is_q = head < n_q;
     const int h = is_q ? head : head - n_q;
@@ -339,7 +350,8 @@ int launch_per_head(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
     hipLaunchKernelGGL((per_head_qkv_q40_kernel<HD>), grid, block, 0, st, (const float *)a.in[0],            \
                        (const float *)a.in[1], (const float *)a.in[2], (const float *)a.in[3],               \
                        (const float *)a.in[4], (const float *)a.in[5], (float *)a.out[0], (uint8_t *)a.out[1], \
-                       (uint8_t *)a.out[2], n_q, k.desc.params[0])
+                       (uint8_t *)a.out[2], n_q, n_kv, k.desc.params[0],                                      \
+                       k.desc.dims[3] ? (const float *)a.in[6] : nullptr, (int)k.desc.dims[3])
     switch (hd) {
     case 128: KSH_PH(128); break;
     case 256: KSH_PH(256); break;
@@ -435,12 +447,17 @@ int bind_per_head_qkv_q40(ksh_kernel &k)
     if (n_q <= 0 || n_kv <= 0 || n_q > 4096 || n_kv > n_q) return set_error("rmsnorm_per_head_qkv_q40: n_q=%lld n_kv=%lld", (long long)n_q, (long long)n_kv);
     if (hd != 128 && hd != 256 && hd != 512)
         return set_error("rmsnorm_per_head_qkv_q40: hd=%lld is not built (128, 256, 512 are)", (long long)hd);
-    k.info.n_inputs = 6;
+    // dims[3] = max_seq when the position comes from a device-side meta buffer
+    // (7th input, f32[4] with the position in [3]); 0 for the host-offset form
+    const int64_t max_seq = k.desc.dims[3];
+    if (max_seq < 0 || max_seq > (1 << 24)) return set_error("rmsnorm_per_head_qkv_q40: max_seq=%lld", (long long)max_seq);
+    const size_t rows = max_seq ? (size_t)max_seq : 1;
+    k.info.n_inputs = max_seq ? 7 : 6;
     k.info.n_outputs = 3;
-    const size_t kvb = (size_t)n_kv * (hd / 32) * 18;
-    const size_t ib[6] = {(size_t)n_q * hd * 4, (size_t)hd * 4, (size_t)hd * 4, (size_t)n_kv * hd * 4, (size_t)hd * 4,
-                          (size_t)n_kv * hd * 4};
-    for (int i = 0; i < 6; i++) { k.in_bytes[i] = ib[i]; k.in_align[i] = 4; }
+    const size_t kvb = (size_t)n_kv * (hd / 32) * 18 * rows;
+    const size_t ib[7] = {(size_t)n_q * hd * 4, (size_t)hd * 4, (size_t)hd * 4 * rows, (size_t)n_kv * hd * 4, (size_t)hd * 4,
+                          (size_t)n_kv * hd * 4, 16};
+    for (int i = 0; i < k.info.n_inputs; i++) { k.in_bytes[i] = ib[i]; k.in_align[i] = 4; }
     k.out_bytes[0] = (size_t)n_q * hd * 4; k.out_align[0] = 4;
     k.out_bytes[1] = k.out_bytes[2] = kvb; k.out_align[1] = k.out_align[2] = 2;
     set_launch(k, (uint32_t)(n_q + n_kv), 1, 1, 64, 0);

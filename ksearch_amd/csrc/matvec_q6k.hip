@@ -107,7 +107,8 @@ struct Q6kParams {
     int rows, bpr, rows_per_wave;
 };
 
-// One step == 8 superblocks.  STEPS = bpr / 8 (cols = 2048 * STEPS).
+// One step == 8 superblocks.  STEPS = ceil(bpr / 8); lanes whose superblock lies
+// past the row's end re-read the last one against zeroed activations.
 template <int R, int NW, int STEPS>
 __global__ __launch_bounds__(NW * 64) void q6k_gemv_kernel(Q6kParams p)
 {
@@ -124,7 +125,8 @@ __global__ __launch_bounds__(NW * 64) void q6k_gemv_kernel(Q6kParams p)
         for (int r = 0; r < R; r++) {
             const uint8_t *rp = p.W + (size_t)min(row0 + r, p.rows - 1) * row_bytes;
 #pragma unroll
-            for (int s = 0; s < STEPS; s++) dst[s][r] = q6k_load(rp + (size_t)(s * 8 + bl) * kQ6kBytes, ip, il);
+            for (int s = 0; s < STEPS; s++)
+                dst[s][r] = q6k_load(rp + (size_t)min(s * 8 + bl, p.bpr - 1) * kQ6kBytes, ip, il);
         }
     };
     if (w0 < w1) load_rows(cur, w0);
@@ -142,12 +144,14 @@ __global__ __launch_bounds__(NW * 64) void q6k_gemv_kernel(Q6kParams p)
     float xr[STEPS][32], sx[STEPS][4];
 #pragma unroll
     for (int s = 0; s < STEPS; s++) {
-        const int e0 = (s * 8 + bl) * 256 + 128 * ip + 8 * il;
+        const bool valid = s * 8 + bl < p.bpr;
+        const int e0 = min(s * 8 + bl, p.bpr - 1) * 256 + 128 * ip + 8 * il;
+        const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
         for (int k = 0; k < 4; k++) {
             const float *src = &xs[xs6_index(e0 + 32 * k)];
-            const float4 a = *reinterpret_cast<const float4 *>(src);
-            const float4 b = *reinterpret_cast<const float4 *>(src + 4);
+            const float4 a = valid ? *reinterpret_cast<const float4 *>(src) : zero;
+            const float4 b = valid ? *reinterpret_cast<const float4 *>(src + 4) : zero;
             float *d = &xr[s][8 * k];
             d[0] = a.x; d[1] = a.y; d[2] = a.z; d[3] = a.w;
             d[4] = b.x; d[5] = b.y; d[6] = b.z; d[7] = b.w;
@@ -199,7 +203,9 @@ int launch_steps(int steps, const Q6kParams &p, unsigned grid, size_t lds, hipSt
     switch (steps) {
     case 1: hipLaunchKernelGGL((q6k_gemv_kernel<R, NW, 1>), dim3(grid), dim3(NW * 64), lds, st, p); break;
     case 2: hipLaunchKernelGGL((q6k_gemv_kernel<R, NW, 2>), dim3(grid), dim3(NW * 64), lds, st, p); break;
-    default: return set_error("matvec_q6k: cols=%d is not built (2048 and 4096 are)", steps * 2048);
+    case 3: hipLaunchKernelGGL((q6k_gemv_kernel<R, NW, 3>), dim3(grid), dim3(NW * 64), lds, st, p); break;
+    case 4: hipLaunchKernelGGL((q6k_gemv_kernel<R, NW, 4>), dim3(grid), dim3(NW * 64), lds, st, p); break;
+    default: return set_error("matvec_q6k: cols=%d is not built (up to 8192 are)", p.bpr * 256);
     }
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : hip_fail(e, "q6k_gemv launch");
@@ -217,7 +223,7 @@ int launch_matvec_q6k(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
     p.rows_per_wave = k.variant >> 16;
     const unsigned grid = k.info.grid[0];
     const size_t lds = k.info.lds_bytes;
-    const int steps = p.bpr / 8;
+    const int steps = (p.bpr + 7) / 8;
 #define KSH_CASE(r, w) \
     if (R == r && NW == w) return launch_steps<r, w>(steps, p, grid, lds, st);
     KSH_CASE(1, 4) KSH_CASE(2, 4) KSH_CASE(4, 4)
@@ -233,9 +239,10 @@ int bind_matvec_q6k(ksh_kernel &k)
 {
     const int64_t rows = k.desc.dims[0], cols = k.desc.dims[1];
     if (rows <= 0 || rows > (1 << 30)) return set_error("matvec: rows=%lld", (long long)rows);
-    if (cols != 2048 && cols != 4096)
-        return set_error("matvec_q6k: cols=%lld is not built (2048 and 4096 are)", (long long)cols);
-    const Q6kGeom G = pick_geom6(k.desc.sched, (int)rows);
+    if (cols <= 0 || cols % 256 || cols > 8192)
+        return set_error("matvec_q6k: cols=%lld is not a positive multiple of 256 up to 8192", (long long)cols);
+    Q6kGeom G = pick_geom6(k.desc.sched, (int)rows);
+    if (cols > 4096 && G.R > 2) { G.rpw = G.rpw / G.R * 2; G.R = 2; }   // keeps the double buffer in registers
     if (!((G.R == 1 || G.R == 2 || G.R == 4) && (G.NW == 2 || G.NW == 4 || G.NW == 8)) || G.rpw % G.R || G.rpw > 32767)
         return set_error("matvec_q6k: unsupported schedule nr0=%d nsg=%d unroll=%u", G.R, G.NW, k.desc.sched.unroll);
     const int bpr = (int)(cols / 256);

@@ -535,3 +535,74 @@ class Eng:
     # :1985-2043
     def beam_matvec(self, ctx, rows, cols, wdt, w, x, y, iters=3, force=False):
         return ctx.beam_search(make_desc(Kind.MATVEC, (rows, cols), (wdt, DType.F32)), [w, x], [y], iters, force)
+
+
+class Gemma:
+    """GemmaPrimModel for the synthetic Gemma-4-E2B shape
+    (crates/ksearch_gemma/src/gemma_prim.rs:76-132, 881-1275, 1658-1768):
+    weights packed on the host side are uploaded once; `generate` keeps token
+    ids on the device between steps."""
+
+    def __init__(self, ctx: Context, cfg: dict, weights: dict):
+        self.ctx, self.cfg = ctx, dict(cfg)
+        self._bufs = []
+
+        def up(a):
+            b = ctx.buffer_bytes(a)
+            self._bufs.append(b)
+            return b
+
+        n = cfg["n_layers"]
+        arr = (GemmaLayer * n)()
+        for i, lw in enumerate(weights["layers"]):
+            for name in GEMMA_LAYER_FIELDS:
+                setattr(arr[i], name, up(lw[name]).h)
+        self._layers = arr
+        self._embd, self._onorm = up(weights["token_embd"]), up(weights["output_norm"])
+        c = GemmaCfg(**cfg)
+        h = C.c_void_p()
+        _check(lib().ksh_gemma_create(ctx.h, C.byref(c), arr, self._embd.h, self._onorm.h, C.byref(h)))
+        self.h = h
+
+    def close(self):
+        if self.h:
+            lib().ksh_gemma_destroy(self.h)
+            self.h = None
+        for b in self._bufs:
+            b.release()
+        self._bufs = []
+
+    def reset(self):
+        _check(lib().ksh_gemma_reset(self.h))
+
+    @property
+    def pos(self) -> int:
+        return lib().ksh_gemma_pos(self.h)
+
+    @property
+    def launches_per_token(self) -> int:
+        return lib().ksh_gemma_launches_per_token(self.h)
+
+    def forward_token(self, token: int, use_graph: bool = False, read_next: bool = True):
+        nxt = C.c_uint32()
+        _check(lib().ksh_gemma_forward_token(self.h, int(token), int(use_graph), C.byref(nxt) if read_next else None))
+        return nxt.value if read_next else None
+
+    def generate(self, prompt, n_new: int, use_graph: bool = True):
+        p = (C.c_uint32 * len(prompt))(*[int(t) for t in prompt])
+        out = (C.c_uint32 * max(1, n_new))()
+        pre, dec = C.c_double(), C.c_double()
+        _check(lib().ksh_gemma_generate(self.h, p, len(prompt), n_new, int(use_graph), out, C.byref(pre), C.byref(dec)))
+        return list(out[:n_new]), pre.value, dec.value
+
+    def logits(self) -> np.ndarray:
+        b = Buffer(self.ctx, lib().ksh_gemma_logits(self.h), owned=False)
+        return self.ctx.read_f32(b, self.cfg["vocab"])
+
+    def hidden(self) -> np.ndarray:
+        b = Buffer(self.ctx, lib().ksh_gemma_hidden(self.h), owned=False)
+        return self.ctx.read_f32(b, self.cfg["hidden"])
+
+    def kv(self, layer: int, which: int, nbytes: int) -> np.ndarray:
+        b = Buffer(self.ctx, lib().ksh_gemma_kv(self.h, layer, which), owned=False)
+        return self.ctx.read_bytes(b, nbytes)

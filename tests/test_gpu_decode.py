@@ -1,0 +1,135 @@
+"""Device quantizers and the greedy decode loop vs the CPU oracle, on a
+scaled-down Gemma-shaped model (same op sequence as the full configuration)."""
+import numpy as np
+import pytest
+
+import oracle
+from ksearch_amd import hip, synth
+from ksearch_amd.hip import DType
+from tests.gpu_util import assert_close
+
+pytestmark = pytest.mark.gpu
+
+SMALL = dict(n_layers=3, hidden=512, ffn=1024, n_q=4, n_kv=1, hd=128, vocab=4096, max_seq=256,
+             eps=1e-6, softcap=30.0, rope_theta=10000.0, attn_scale=1.0 / np.sqrt(128.0))
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = hip.Context()
+    yield c
+    c.close()
+
+
+@pytest.fixture(scope="module")
+def eng():
+    return hip.Eng()
+
+
+def test_quantize_q4k_matches_host_routine_bytes(ctx, eng):
+    # weights-like signal, the reference unit test's signal, a zero and a constant block
+    i = np.arange(1024, dtype=np.float32)
+    sig = (np.sin(i * np.float32(0.017) + np.float32(0.3)) * np.float32(1.7)
+           + np.cos(i * np.float32(0.041)) * np.float32(0.4) - np.float32(0.15)).astype(np.float32)
+    sig[256:512] = 0.0
+    sig[512:768] = -0.25
+    x = np.concatenate([sig, synth.normal_f32(256 * 300, 400, std=0.02), synth.normal_f32(256 * 20, 401, std=3.0)])
+    dst = ctx.buffer_empty_bytes(x.size // 256 * 144)
+    eng.quantize_k(ctx, DType.Q4K, x.size, ctx.buffer_f32(x), dst)
+    got, want = ctx.read_bytes(dst, x.size // 256 * 144), oracle.quantize_q4k(x)
+    assert np.array_equal(got, want)
+    back = oracle.dequant(oracle.Q4K, got, x.size)
+    assert np.all(back[256:512] == 0.0) and np.abs(back[:1024] - sig).max() < 0.35
+
+
+def test_quantize_q6k_matches_host_routine_bytes(ctx, eng):
+    x = np.concatenate([synth.normal_f32(256 * 200, 402, std=0.02), np.zeros(256, np.float32),
+                        synth.normal_f32(256 * 10, 403, std=5.0)])
+    dst = ctx.buffer_empty_bytes(x.size // 256 * 210)
+    eng.quantize_k(ctx, DType.Q6K, x.size, ctx.buffer_f32(x), dst)
+    got, want = ctx.read_bytes(dst, x.size // 256 * 210), oracle.quantize_q6k(x)
+    assert np.array_equal(got, want)
+
+
+@pytest.fixture(scope="module")
+def small_model(ctx):
+    w = synth.gemma_weights(SMALL, 500, oracle.quantize_q4k, oracle.quantize_q6k, std=0.05)
+    # norm weights away from 1 so that a swapped or dropped norm shows
+    rng = np.random.default_rng(501)
+    for lw in w["layers"]:
+        for name in ("attn_norm", "q_norm", "k_norm", "post_attn_norm", "ffn_norm", "post_ffw_norm"):
+            lw[name] = (1.0 + 0.2 * rng.standard_normal(lw[name].size)).astype(np.float32)
+    w["output_norm"] = (1.0 + 0.2 * rng.standard_normal(SMALL["hidden"])).astype(np.float32)
+    gpu = hip.Gemma(ctx, SMALL, w)
+    cpu = oracle.Gemma(SMALL, w)
+    yield gpu, cpu, w
+    gpu.close()
+    cpu.close()
+
+
+def test_forward_token_matches_oracle_teacher_forced(small_model):
+    gpu, cpu, _ = small_model
+    gpu.reset()
+    cpu.reset()
+    rng = np.random.default_rng(502)
+    toks = rng.integers(0, SMALL["vocab"], 40)
+    row = SMALL["n_kv"] * SMALL["hd"] // 32 * 18
+    agree = 0
+    for i, t in enumerate(toks):
+        g_next = gpu.forward_token(int(t), use_graph=False)
+        c_next, c_logits = cpu.forward(int(t), return_logits=True)
+        g_logits = gpu.logits()
+        assert_close(g_logits, c_logits, 1e-3, f"logits at step {i}")
+        assert_close(gpu.hidden(), cpu.hidden(), 1e-3, f"hidden at step {i}")
+        # the device argmax follows the oracle's rule on the device's own logits
+        assert g_next == oracle.softcap_argmax(g_logits, SMALL["softcap"])
+        top2 = np.sort(c_logits)[-2:]
+        if top2[1] - top2[0] > 1e-3 * max(abs(top2[1]), float(np.sqrt(np.mean(c_logits ** 2)))):
+            assert g_next == c_next, f"step {i}: margin {top2[1] - top2[0]}"
+            agree += 1
+    assert agree >= 30 and gpu.pos == cpu.pos == len(toks)
+    # the KV cache rows written so far: codes equal up to rare one-step flips
+    for layer in (0, SMALL["n_layers"] - 1):
+        for which in (0, 1):
+            g, c = gpu.kv(layer, which, len(toks) * row), cpu.kv(layer, which, len(toks) * row)
+            assert (g != c).mean() < 0.02
+            dg, dc = oracle.dequant(oracle.Q40, g, len(toks) * SMALL["hd"]), oracle.dequant(oracle.Q40, c, len(toks) * SMALL["hd"])
+            assert np.abs(dg - dc).max() <= np.abs(dc).max() / 7 * 1.01
+    with pytest.raises(hip.KshError, match="outside the vocabulary"):
+        gpu.forward_token(SMALL["vocab"])
+
+
+def test_generate_graph_equals_eager_and_oracle(small_model):
+    gpu, cpu, _ = small_model
+    rng = np.random.default_rng(503)
+    prompt = [int(t) for t in rng.integers(0, SMALL["vocab"], 12)]
+    n_new = 48
+    gpu.reset()
+    eager, _, _ = gpu.generate(prompt, n_new, use_graph=False)
+    gpu.reset()
+    graph, _, ms = gpu.generate(prompt, n_new, use_graph=True)
+    assert graph == eager                     # same kernels, same order: bit-identical
+    gpu.reset()
+    assert gpu.generate(prompt, n_new, use_graph=True)[0] == graph      # replay after reset
+    assert gpu.launches_per_token > 0
+    # the oracle's greedy continuation
+    cpu.reset()
+    for t in prompt[:-1]:
+        cpu.forward(t, want_logits=False)
+    want, margins, t = [], [], prompt[-1]
+    for _ in range(n_new):
+        t, lg = cpu.forward(t, return_logits=True)
+        s = np.sort(lg)
+        margins.append(float((s[-1] - s[-2]) / max(abs(s[-1]), float(np.sqrt(np.mean(lg ** 2))))))
+        want.append(t)
+    # identical until (if ever) the oracle's own top-2 margin drops under the numeric tolerance
+    n_same = next((i for i, (a, b) in enumerate(zip(graph, want)) if a != b), n_new)
+    assert n_same == n_new or margins[n_same] < 1e-3, (n_same, margins[n_same] if n_same < n_new else None)
+    assert n_same >= 8
+
+
+def test_generate_refuses_past_max_seq(small_model):
+    gpu, _, _ = small_model
+    gpu.reset()
+    with pytest.raises(hip.KshError, match="max_seq exceeded"):
+        gpu.generate([1, 2, 3], SMALL["max_seq"], use_graph=False)

@@ -130,7 +130,7 @@ SCHEDS_Q6K = [None, dict(tg=256, vec=0, unroll=2, nsg=4, nr0=1, k_split=1, lds_t
               dict(tg=128, vec=0, unroll=2, nsg=2, nr0=2, k_split=1, lds_tile=0)]
 
 
-@pytest.mark.parametrize("rows,cols", [(8, 2048), (1000, 2048), (4099, 2048), (300, 4096)])
+@pytest.mark.parametrize("rows,cols", [(8, 2048), (1000, 2048), (4099, 2048), (300, 4096), (70, 256), (33, 512), (65, 1536), (40, 8192)])
 @pytest.mark.parametrize("sched", SCHEDS_Q6K)
 def test_matvec_q6k(ctx, eng, rows, cols, sched):
     w = synth.q6k_blocks(rows * cols // 256, seed=rows)

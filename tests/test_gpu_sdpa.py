@@ -1,0 +1,140 @@
+"""HIP decode attention over a Q4_0 KV cache vs the CPU oracle (1e-3 relative),
+plus the invariants the reference's own example checks: batch equals serial,
+partition-count independence, the needle."""
+import numpy as np
+import pytest
+
+import oracle
+from ksearch_amd import hip, synth
+from ksearch_amd.hip import DType
+from tests.gpu_util import assert_close
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = hip.Context()
+    yield c
+    c.close()
+
+
+@pytest.fixture(scope="module")
+def eng():
+    return hip.Eng()
+
+
+def kv(max_t, n_kv, hd, seed):
+    n = max_t * n_kv * hd // 32
+    return synth.q40_blocks(n, seed), synth.q40_blocks(n, seed + 1)
+
+
+@pytest.mark.parametrize("n_q,n_kv,hd,max_t,tlen,start,scale", [
+    (8, 1, 256, 64, 1, 0, 1.0 / 16),          # a single row
+    (8, 1, 256, 64, 33, 0, 1.0 / 16),         # one row past a tile
+    (8, 1, 256, 300, 127, 50, 1.0 / 16),      # largest online case, non-zero start (sliding window)
+    (8, 1, 256, 300, 128, 0, 1.0 / 16),       # first split-KV case
+    (8, 1, 256, 2048, 2048, 0, 1.0 / 16),
+    (8, 1, 256, 1000, 777, 200, 1.0),         # the reference's scale (none)
+    (4, 2, 128, 500, 300, 100, 0.09),         # GQA with two kv heads
+    (16, 1, 64, 200, 150, 3, 0.125),
+    (8, 1, 512, 400, 260, 7, 1.0 / 16),       # full-attention head size
+])
+def test_sdpa_hybrid_vs_oracle(ctx, eng, n_q, n_kv, hd, max_t, tlen, start, scale):
+    k, v = kv(max_t, n_kv, hd, 300 + hd)
+    q = synth.normal_f32(n_q * hd, 310)
+    bq, bk, bv = ctx.buffer_f32(q), ctx.buffer_bytes(k), ctx.buffer_bytes(v)
+    meta = ctx.buffer_f32([tlen, start, 0, 0])                   # write_meta_win, gemma_prim.rs:636-644
+    tmp = ctx.buffer_empty_f32(n_q * eng.SDPA_MWG_NWG * (hd + 2))
+    out = ctx.buffer_empty_f32(n_q * hd)
+    eng.sdpa_hybrid_kv(ctx, n_q, n_kv, hd, max_t, tlen, DType.Q40, bq, bk, bv, meta, tmp, out, scale)
+    got = ctx.read_f32(out, n_q * hd)
+    assert_close(got, oracle.sdpa_hybrid(q, k, v, n_q, n_kv, hd, tlen, start, scale), TOL, "vs oracle")
+    assert_close(got, oracle.sdpa(q, k, v, n_q, n_kv, hd, tlen, start, scale, f64=True), TOL, "vs f64")
+
+
+def test_sdpa_partition_count_independence(ctx, eng):
+    n_q, n_kv, hd, max_t, tlen = 8, 1, 256, 1024, 1000
+    k, v = kv(max_t, n_kv, hd, 320)
+    q = synth.normal_f32(n_q * hd, 321)
+    bq, bk, bv = ctx.buffer_f32(q), ctx.buffer_bytes(k), ctx.buffer_bytes(v)
+    meta = ctx.buffer_f32([tlen, 0, 0, 0])
+    out = ctx.buffer_empty_f32(n_q * hd)
+    want = oracle.sdpa(q, k, v, n_q, n_kv, hd, tlen, 0, 0.0625, f64=True)
+    for nwg in (1, 2, 16, 33, 1000, 1024):     # 1024 > tlen: trailing partitions are empty
+        tmp = ctx.buffer_empty_f32(n_q * nwg * (hd + 2))
+        eng.sdpa_mwg_kv(ctx, n_q, n_kv, hd, max_t, DType.Q40, bq, bk, bv, meta, tmp, out, 0.0625, nwg=nwg)
+        assert_close(ctx.read_f32(out, n_q * hd), want, TOL, f"nwg={nwg}")
+
+
+def test_sdpa_needle(ctx, eng):
+    # check_mul_mm.rs:250-294: Q = 1, K[0] = 1, V[0] = 1, other rows 0; the
+    # expectation comes from the brute-force oracle, not from "O ~ 1"
+    n_q, hd = 8, 256
+    for tlen in (64, 512):
+        kf = np.zeros((tlen, hd), dtype=np.float32)
+        vf = np.zeros((tlen, hd), dtype=np.float32)
+        kf[0] = vf[0] = 1.0
+        src = ctx.buffer_f32(kf)
+        bk, bv = ctx.buffer_empty_bytes(tlen * hd // 32 * 18), ctx.buffer_empty_bytes(tlen * hd // 32 * 18)
+        eng.quantize_q40(ctx, tlen * hd, src, bk)
+        eng.quantize_q40(ctx, tlen * hd, ctx.buffer_f32(vf), bv)
+        k, v = ctx.read_bytes(bk, tlen * hd // 32 * 18), ctx.read_bytes(bv, tlen * hd // 32 * 18)
+        assert np.array_equal(k, oracle.pack_q40(kf))
+        q = np.ones(n_q * hd, dtype=np.float32)
+        meta, out = ctx.buffer_f32([tlen, 0, tlen, 0]), ctx.buffer_empty_f32(n_q * hd)
+        tmp = ctx.buffer_empty_f32(n_q * eng.SDPA_MWG_NWG * (hd + 2))
+        for scale in (1.0, 1.0 / 256):
+            eng.sdpa_hybrid_kv(ctx, n_q, 1, hd, tlen, tlen, DType.Q40, ctx.buffer_f32(q), bk, bv, meta, tmp, out, scale)
+            assert_close(ctx.read_f32(out, n_q * hd), oracle.sdpa(q, k, v, n_q, 1, hd, tlen, 0, scale, f64=True), TOL,
+                         f"needle tlen={tlen} scale={scale}")
+
+
+@pytest.mark.parametrize("nwg", [0, 16, 64])
+def test_sdpa_slots_batch_equals_serial(ctx, eng, nwg):
+    # cfg3 at reduced context, then at full size below
+    n_slots, n_q, n_kv, hd, max_t = 4, 8, 1, 256, 2048
+    lens, k, v, q = synth.cfg3_q40_attention(n_slots, n_q, n_kv, hd, max_t, lo=100, seed=330)
+    lens[1] = 1           # one slot with a single row: every other partition of it is empty
+    bq, bk, bv = ctx.buffer_f32(q), ctx.buffer_bytes(k), ctx.buffer_bytes(v)
+    meta = np.zeros((n_slots, 4), dtype=np.float32)
+    meta[:, 0] = lens
+    bm = ctx.buffer_f32(meta)
+    kk = ctx.compile(hip.make_desc(hip.Kind.SDPA_SLOTS, (n_q, n_kv, hd, max_t, n_slots, nwg), (DType.Q40, DType.F32), (0.0625,)))
+    real_nwg = kk.info.sched.k_split
+    tmp = ctx.buffer_empty_f32(n_slots * n_q * real_nwg * (hd + 2))
+    out = ctx.buffer_empty_f32(n_slots * n_q * hd)
+    eng.sdpa_slots(ctx, n_q, n_kv, hd, max_t, n_slots, bq, bk, bv, bm, tmp, out, 0.0625, nwg)
+    got = ctx.read_f32(out, n_slots * n_q * hd).reshape(n_slots, -1)
+    for s in range(n_slots):
+        want = oracle.sdpa_hybrid(q[s], k[s], v[s], n_q, n_kv, hd, int(lens[s]), 0, 0.0625)
+        assert_close(got[s], want, TOL, f"slot {s} len {lens[s]}")
+
+
+def test_sdpa_cfg3_full_size(ctx, eng):
+    n_slots, n_q, n_kv, hd, max_t = 4, 8, 1, 256, 16384
+    lens, k, v, q = synth.cfg3_q40_attention()
+    bq, bk, bv = ctx.buffer_f32(q), ctx.buffer_bytes(k), ctx.buffer_bytes(v)
+    meta = np.zeros((n_slots, 4), dtype=np.float32)
+    meta[:, 0] = lens
+    kk = ctx.compile(hip.make_desc(hip.Kind.SDPA_SLOTS, (n_q, n_kv, hd, max_t, n_slots, 0), (DType.Q40, DType.F32), (0.0625,)))
+    tmp = ctx.buffer_empty_f32(n_slots * n_q * kk.info.sched.k_split * (hd + 2))
+    out = ctx.buffer_empty_f32(n_slots * n_q * hd)
+    eng.sdpa_slots(ctx, n_q, n_kv, hd, max_t, n_slots, bq, bk, bv, ctx.buffer_f32(meta), tmp, out, 0.0625, 0)
+    got = ctx.read_f32(out, n_slots * n_q * hd).reshape(n_slots, -1)
+    for s in range(n_slots):
+        assert_close(got[s], oracle.sdpa_hybrid(q[s], k[s], v[s], n_q, n_kv, hd, int(lens[s]), 0, 0.0625), TOL, f"slot {s}")
+    # softmax weights sum to one: with V == const c every output equals c (size-independent property)
+    vc = np.tile(np.concatenate([np.array([0.5], dtype=np.float16).view(np.uint8), np.full(16, 0xBB, np.uint8)]), k.size // 18)
+    eng.sdpa_slots(ctx, n_q, n_kv, hd, max_t, n_slots, bq, bk, ctx.buffer_bytes(vc), ctx.buffer_f32(meta), tmp, out, 0.0625, 0)
+    assert np.allclose(ctx.read_f32(out, n_slots * n_q * hd), 1.5, rtol=1e-5)
+
+
+def test_sdpa_errors(ctx):
+    with pytest.raises(hip.KshError, match="multiple of 32"):
+        ctx.compile(hip.make_desc(hip.Kind.SDPA_NAIVE, (8, 1, 100, 64), (DType.Q40, DType.F32), (1.0,)))
+    with pytest.raises(hip.KshError, match="not built"):
+        ctx.compile(hip.make_desc(hip.Kind.SDPA_NAIVE, (8, 1, 256, 64), (DType.F16, DType.F32), (1.0,)))
+    with pytest.raises(hip.KshError, match="divide evenly"):
+        ctx.compile(hip.make_desc(hip.Kind.SDPA_NAIVE, (8, 3, 256, 64), (DType.Q40, DType.F32), (1.0,)))

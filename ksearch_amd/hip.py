@@ -537,6 +537,35 @@ class Eng:
         return ctx.beam_search(make_desc(Kind.MATVEC, (rows, cols), (wdt, DType.F32)), [w, x], [y], iters, force)
 
 
+def device_quantizers(ctx: Context, eng: Eng):
+    """(quantize_q4k, quantize_q6k) for synth.gemma_weights: host f32 arrays go
+    up, are packed by the device kernels and stay on the device as Buffers.
+    The Q6_K one takes the embedding table as a list of row chunks."""
+
+    def q4k(x: np.ndarray) -> Buffer:
+        src = ctx.buffer_f32(x)
+        dst = ctx.buffer_empty_bytes(x.size // 256 * 144)
+        eng.quantize_k(ctx, DType.Q4K, x.size, src, dst)
+        ctx.synchronize()
+        src.release()
+        return dst
+
+    def q6k(parts) -> Buffer:
+        total = sum(p.size for p in parts)
+        dst = ctx.buffer_empty_bytes(total // 256 * 210)
+        off = 0
+        for p_ in parts:
+            src = ctx.buffer_f32(p_)
+            k = eng._k(ctx, Kind.QUANTIZE_K, (p_.size,), (DType.Q6K,))
+            ctx.encode_offsets_multi(k, [src], [0], [dst], [off])
+            ctx.synchronize()
+            src.release()
+            off += p_.size // 256 * 210
+        return dst
+
+    return q4k, q6k
+
+
 class Gemma:
     """GemmaPrimModel for the synthetic Gemma-4-E2B shape
     (crates/ksearch_gemma/src/gemma_prim.rs:76-132, 881-1275, 1658-1768):
@@ -548,7 +577,7 @@ class Gemma:
         self._bufs = []
 
         def up(a):
-            b = ctx.buffer_bytes(a)
+            b = a if isinstance(a, Buffer) else ctx.buffer_bytes(a)
             self._bufs.append(b)
             return b
 

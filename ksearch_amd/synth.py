@@ -99,23 +99,45 @@ GEMMA_E2B_SYNTH = dict(n_layers=30, hidden=2048, ffn=8192, n_q=8, n_kv=1, hd=256
                        rope_theta=10000.0, attn_scale=1.0 / 16.0)
 
 
-def gemma_weights(cfg: dict, seed: int, quantize_q4k, quantize_q6k, std: float = 0.02) -> dict:
+def chunked(quantize):
+    """Lifts a host quantizer (one f32 array -> packed bytes) to the list-of-row-
+    chunks form gemma_weights hands the embedding table over in."""
+    return lambda parts: np.concatenate([quantize(p) for p in parts])
+
+
+def gemma_weights(cfg: dict, seed: int, quantize_q4k, quantize_q6k, std: float = 0.02, threads: int = 0) -> dict:
     """N(0, std) weights packed to Q4_K (attention/FFN) and Q6_K (tied
     embedding / LM head); norm weights are 1.  The two quantizers are passed
-    in by the caller, so this module has no dependency on where they live."""
+    in by the caller (host arrays in, anything out: packed host arrays from a
+    CPU routine, device buffers from the device kernels), so this module does
+    not depend on where they live.  Every tensor has its own seed, so the
+    result does not depend on `threads` (float generation runs in a thread
+    pool; the quantizers are called from the calling thread, in order)."""
+    import concurrent.futures as cf
+    import os
+
     h, f, hd = cfg["hidden"], cfg["ffn"], cfg["hd"]
     nq, nkv = cfg["n_q"] * hd, cfg["n_kv"] * hd
+    shapes = (("wq", (nq, h)), ("wk", (nkv, h)), ("wv", (nkv, h)), ("wo", (h, nq)),
+              ("wgate", (f, h)), ("wup", (f, h)), ("wdown", (h, f)))
     layers = []
     s = seed
-    for _ in range(cfg["n_layers"]):
-        lw = {}
-        for name, (r, c) in (("wq", (nq, h)), ("wk", (nkv, h)), ("wv", (nkv, h)), ("wo", (h, nq)),
-                             ("wgate", (f, h)), ("wup", (f, h)), ("wdown", (h, f))):
+    with cf.ThreadPoolExecutor(max_workers=threads or min(16, os.cpu_count() or 1)) as ex:
+        for _ in range(cfg["n_layers"]):
+            futs = {}
+            for name, (r, c) in shapes:
+                s += 1
+                futs[name] = ex.submit(normal_f32, r * c, s, std)
+            lw = {name: quantize_q4k(futs[name].result()) for name, _ in shapes}
+            for name, n in (("attn_norm", h), ("q_norm", hd), ("k_norm", hd),
+                            ("post_attn_norm", h), ("ffn_norm", h), ("post_ffw_norm", h)):
+                lw[name] = np.ones(n, dtype=np.float32)
+            layers.append(lw)
+        # the embedding table in row chunks, so that no single float array exceeds ~0.5 GB
+        rows, chunk = cfg["vocab"], max(1, min(cfg["vocab"], (1 << 27) // h))
+        futs = []
+        for r0 in range(0, rows, chunk):
             s += 1
-            lw[name] = quantize_q4k(normal_f32(r * c, s, std))
-        for name, n in (("attn_norm", h), ("q_norm", hd), ("k_norm", hd),
-                        ("post_attn_norm", h), ("ffn_norm", h), ("post_ffw_norm", h)):
-            lw[name] = np.ones(n, dtype=np.float32)
-        layers.append(lw)
-    embd = quantize_q6k(normal_f32(cfg["vocab"] * h, s + 1, std))
+            futs.append(ex.submit(normal_f32, min(chunk, rows - r0) * h, s, std))
+        embd = quantize_q6k([fu.result() for fu in futs])
     return dict(layers=layers, token_embd=embd, output_norm=np.ones(h, dtype=np.float32))

@@ -53,7 +53,7 @@ def test_quantize_q6k_matches_host_routine_bytes(ctx, eng):
 
 @pytest.fixture(scope="module")
 def small_model(ctx):
-    w = synth.gemma_weights(SMALL, 500, oracle.quantize_q4k, oracle.quantize_q6k, std=0.05)
+    w = synth.gemma_weights(SMALL, 500, oracle.quantize_q4k, synth.chunked(oracle.quantize_q6k), std=0.05)
     # norm weights away from 1 so that a swapped or dropped norm shows
     rng = np.random.default_rng(501)
     for lw in w["layers"]:

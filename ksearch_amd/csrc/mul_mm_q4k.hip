@@ -1,0 +1,277 @@
+// Batched prefill GEMM over Q4_K weights on the gfx950 matrix cores:
+//   Y[t, r] = sum_c deq(W[r, c]) * X[t, c]      X bf16 [batch, cols], Y f32 [batch, rows]
+//
+// Takes the place of KirStmt::Q4kMulMm / ksearch_q4k_mul_mm
+// (crates/ksearch_codegen/src/lower.rs:404-424, 788-818,
+// crates/ksearch_codegen/src/render.rs:1073-1191), which dequantizes a 64x32
+// weight tile to half (rounding every weight) and runs 8x8 simdgroup MMAs.
+//
+// Here no weight is rounded.  With w = d*sc_j*n - dmin*m_j (n the 4-bit code,
+// j the 32-wide sub-block):
+//
+//   sum_c w*x = sum_sb [ d * sum_k (sc_j*n_k) x_k  -  sum_j dmin*m_j * Sx_j ],   Sx_j = sum_{k in j} x_k
+//
+// sc_j*n_k is an integer <= 945, exact in f16, and is produced two at a time
+// by one 24-bit multiply-add that also ORs it into the mantissa of half 1024.0:
+// (q & 0x000F000F) * sc + 0x64006400 = (1024 + sc*n_a, 1024 + sc*n_b).  The
+// matrix cores accumulate C' = sum_k (1024 + sc*n) x_k per superblock in f32;
+// the per-row f16 scale d is applied once per superblock (F += d * C'), and
+// the bias and the mins go through a second, short matrix product against the
+// per-sub-block sums of x:  F -= sum_j (dmin*m_j + 1024*d) * Sx_j, with both
+// factors split into f16 hi + lo parts so that this term keeps f32 accuracy.
+// X is bf16, which converts to f16 without loss for |x| >= 2^-17 (smaller
+// values lose at most 2^-25 absolutely).
+//
+// Tiling: a workgroup (4 waves) owns 128 tokens x 128 weight rows; a wave owns
+// 64 x 64 as 2 x 2 v_mfma_f32_32x32x16_f16 tiles.  M = tokens, N = weight
+// rows, so a lane's accumulator column is one weight row (one d per lane) and
+// stores are contiguous along Y's row index.  K advances 64 columns (one
+// 64-element group: 32 quant bytes per row) per step through LDS.
+#include "ksh_device.hpp"
+#include "ksh_internal.hpp"
+
+namespace ksh {
+namespace {
+
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef float f16v __attribute__((ext_vector_type(16)));
+
+constexpr int BM = 128, BN = 128, KS = 64;
+constexpr int PITCH = KS + 8;      // halves per LDS row of the main tiles (144 B: conflict-free 16 B reads)
+constexpr int PITCH2 = 32 + 8;     // halves per LDS row of the min-term tiles
+
+// within every 4 consecutive k the stored order is (0, 2, 1, 3): that is the
+// order the paired nibble extraction produces, applied to X as well
+__device__ __forceinline__ int kperm(int i) { return (i & ~3) | ((i & 1) << 1) | ((i >> 1) & 1); }
+
+// X bf16 -> f16 (permuted), plus the min-term operand per (token, superblock):
+// 32 halves = Sx_hi[8] | Sx_hi[8] | Sx_lo[8] | 0[8].  One thread per (token, sub-block).
+__global__ void mm_prep_x_kernel(const uint16_t *__restrict__ X, _Float16 *__restrict__ Xh,
+                                 _Float16 *__restrict__ SxA, int batch, int cols)
+{
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    const int spt = cols / 32;             // sub-blocks per token
+    if (idx >= batch * spt) return;
+    const int t = idx / spt, s = idx % spt;
+    const uint16_t *src = X + (size_t)t * cols + (size_t)s * 32;
+    _Float16 *dst = Xh + (size_t)t * cols + (size_t)s * 32;
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 32; i++) {
+        const float f = as_f32((uint32_t)src[i] << 16);
+        sum += f;
+        dst[kperm(i)] = (_Float16)f;
+    }
+    const _Float16 hi = (_Float16)sum;
+    const _Float16 lo = (_Float16)(sum - (float)hi);
+    _Float16 *a2 = SxA + ((size_t)t * (cols / 256) + s / 8) * 32;
+    const int j = s % 8;
+    a2[j] = hi;
+    a2[8 + j] = hi;
+    a2[16 + j] = lo;
+    a2[24 + j] = (_Float16)0.f;
+}
+
+struct MmParams {
+    const uint8_t *W;
+    const _Float16 *Xh, *SxA;
+    float *Y;
+    int rows, cols, batch;
+};
+
+__device__ __forceinline__ uint32_t pair_f16(uint32_t masked, uint32_t sc)
+{
+    return __umul24(masked, sc) + 0x64006400u;
+}
+
+__global__ __launch_bounds__(256) void q4k_mul_mm_kernel(MmParams p)
+{
+    __shared__ __attribute__((aligned(16))) _Float16 As[BM * PITCH];
+    __shared__ __attribute__((aligned(16))) _Float16 Bs[BN * PITCH];
+    __shared__ __attribute__((aligned(16))) _Float16 A2s[BM * PITCH2];
+    __shared__ __attribute__((aligned(16))) _Float16 B2s[BN * PITCH2];
+    __shared__ float dsc[BN];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int t0 = blockIdx.x * BM, r0 = blockIdx.y * BN;
+    const int nsb = p.cols / 256;
+    const size_t row_bytes = (size_t)nsb * 144;
+
+    // loader roles
+    const int lrow = tid >> 1, lhalf = tid & 1;
+    const uint8_t *wrow = p.W + (size_t)min(r0 + lrow, p.rows - 1) * row_bytes;
+    const _Float16 *xrow = p.Xh + (size_t)min(t0 + lrow, p.batch - 1) * p.cols;
+    const _Float16 *sxrow = p.SxA + (size_t)min(t0 + lrow, p.batch - 1) * nsb * 32;
+
+    f16v F[2][2], Cp[2][2];
+#pragma unroll
+    for (int a = 0; a < 2; a++)
+#pragma unroll
+        for (int b = 0; b < 2; b++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) { F[a][b][i] = 0.f; Cp[a][b][i] = 0.f; }
+
+    const int lm = lane & 31, lk = (lane >> 5) * 8;
+
+    for (int sb = 0; sb < nsb; sb++) {
+        const uint4 hdr = *reinterpret_cast<const uint4 *>(wrow + (size_t)sb * 144);
+        for (int g = 0; g < 4; g++) {
+            const uint4 q = *reinterpret_cast<const uint4 *>(wrow + (size_t)sb * 144 + 16 + 32 * g + 16 * lhalf);
+            const uint4 *xs = reinterpret_cast<const uint4 *>(xrow + sb * 256 + 64 * g + 32 * lhalf);
+            const uint4 x0 = xs[0], x1 = xs[1], x2 = xs[2], x3 = xs[3];
+            const uint4 s = q4k_group_scales(hdr.y, hdr.z, hdr.w, g);   // sc_lo, mn_lo, sc_hi, mn_hi
+            __syncthreads();   // the previous step's MFMA reads of As/Bs are done
+            {
+                uint4 *dst = reinterpret_cast<uint4 *>(&As[lrow * PITCH + 32 * lhalf]);
+                dst[0] = x0; dst[1] = x1; dst[2] = x2; dst[3] = x3;
+            }
+            {
+                const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+                uint32_t lo[8], hi[8];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const uint32_t t4 = w[i] >> 4;
+                    lo[2 * i] = pair_f16(w[i] & 0x000F000Fu, s.x);
+                    lo[2 * i + 1] = pair_f16((w[i] >> 8) & 0x000F000Fu, s.x);
+                    hi[2 * i] = pair_f16(t4 & 0x000F000Fu, s.z);
+                    hi[2 * i + 1] = pair_f16((t4 >> 8) & 0x000F000Fu, s.z);
+                }
+                uint4 *dlo = reinterpret_cast<uint4 *>(&Bs[lrow * PITCH + 16 * lhalf]);
+                uint4 *dhi = reinterpret_cast<uint4 *>(&Bs[lrow * PITCH + 32 + 16 * lhalf]);
+                dlo[0] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+                dlo[1] = make_uint4(lo[4], lo[5], lo[6], lo[7]);
+                dhi[0] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+                dhi[1] = make_uint4(hi[4], hi[5], hi[6], hi[7]);
+            }
+            __syncthreads();
+#pragma unroll
+            for (int ks = 0; ks < KS / 16; ks++) {
+                h8 a[2], b[2];
+#pragma unroll
+                for (int mt = 0; mt < 2; mt++)
+                    a[mt] = *reinterpret_cast<const h8 *>(&As[(wm * 64 + mt * 32 + lm) * PITCH + 16 * ks + lk]);
+#pragma unroll
+                for (int nt = 0; nt < 2; nt++)
+                    b[nt] = *reinterpret_cast<const h8 *>(&Bs[(wn * 64 + nt * 32 + lm) * PITCH + 16 * ks + lk]);
+#pragma unroll
+                for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+                    for (int nt = 0; nt < 2; nt++)
+                        Cp[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mt], b[nt], Cp[mt][nt], 0, 0, 0);
+            }
+        }
+        // ---- end of the superblock: bias + mins through a short second product, then the row scale
+        {
+            const float d = half_bits_to_f32(hdr.x & 0xFFFFu), dmin = half_bits_to_f32(hdr.x >> 16);
+            // this thread covers sub-blocks 4*lhalf .. 4*lhalf+3 of its row: groups 2*lhalf, 2*lhalf+1
+#pragma unroll
+            for (int gg = 0; gg < 2; gg++) {
+                const int g = 2 * lhalf + gg;
+                const uint4 s = q4k_group_scales(hdr.y, hdr.z, hdr.w, g);
+                const float c0 = -(dmin * (float)s.y + 1024.f * d), c1 = -(dmin * (float)s.w + 1024.f * d);
+                const _Float16 h0 = (_Float16)c0, h1 = (_Float16)c1;
+                const _Float16 l0 = (_Float16)(c0 - (float)h0), l1 = (_Float16)(c1 - (float)h1);
+                _Float16 *b2 = &B2s[lrow * PITCH2];
+                const int j = 2 * g;
+                b2[j] = h0; b2[j + 1] = h1;
+                b2[8 + j] = l0; b2[8 + j + 1] = l1;
+                b2[16 + j] = h0; b2[16 + j + 1] = h1;
+                b2[24 + j] = (_Float16)0.f; b2[24 + j + 1] = (_Float16)0.f;
+            }
+            if (lhalf == 0) dsc[lrow] = d;
+            const uint4 *sx = reinterpret_cast<const uint4 *>(sxrow + sb * 32 + 16 * lhalf);
+            uint4 *dst = reinterpret_cast<uint4 *>(&A2s[lrow * PITCH2 + 16 * lhalf]);
+            dst[0] = sx[0];
+            dst[1] = sx[1];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++) {
+            h8 a[2], b[2];
+#pragma unroll
+            for (int mt = 0; mt < 2; mt++)
+                a[mt] = *reinterpret_cast<const h8 *>(&A2s[(wm * 64 + mt * 32 + lm) * PITCH2 + 16 * ks + lk]);
+#pragma unroll
+            for (int nt = 0; nt < 2; nt++)
+                b[nt] = *reinterpret_cast<const h8 *>(&B2s[(wn * 64 + nt * 32 + lm) * PITCH2 + 16 * ks + lk]);
+#pragma unroll
+            for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+                for (int nt = 0; nt < 2; nt++)
+                    F[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mt], b[nt], F[mt][nt], 0, 0, 0);
+        }
+#pragma unroll
+        for (int nt = 0; nt < 2; nt++) {
+            const float dn = dsc[wn * 64 + nt * 32 + lm];
+#pragma unroll
+            for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    F[mt][nt][i] = fmaf(dn, Cp[mt][nt][i], F[mt][nt][i]);
+                    Cp[mt][nt][i] = 0.f;
+                }
+        }
+        // A2s/B2s/dsc are rewritten only after the next superblock's eight
+        // barriers, so no extra barrier is needed here
+    }
+
+    // accumulator layout of the 32x32 tile: column = lane % 32, row = 8*(i/4) + 4*(lane/32) + i%4
+#pragma unroll
+    for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+        for (int nt = 0; nt < 2; nt++) {
+            const int r = r0 + wn * 64 + nt * 32 + lm;
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int t = t0 + wm * 64 + mt * 32 + 8 * (i / 4) + 4 * (lane >> 5) + (i & 3);
+                if (t < p.batch && r < p.rows) p.Y[(size_t)t * p.rows + r] = F[mt][nt][i];
+            }
+        }
+}
+
+int launch_mul_mm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
+{
+    const int rows = (int)k.desc.dims[0], cols = (int)k.desc.dims[1], batch = (int)k.desc.dims[2];
+    _Float16 *Xh = (_Float16 *)k.scratch;
+    _Float16 *SxA = Xh + (size_t)batch * cols;
+    const int n = batch * (cols / 32);
+    hipLaunchKernelGGL(mm_prep_x_kernel, dim3((n + 255) / 256), dim3(256), 0, st, (const uint16_t *)a.in[1], Xh, SxA,
+                       batch, cols);
+    MmParams p;
+    p.W = (const uint8_t *)a.in[0];
+    p.Xh = Xh;
+    p.SxA = SxA;
+    p.Y = (float *)a.out[0];
+    p.rows = rows; p.cols = cols; p.batch = batch;
+    hipLaunchKernelGGL(q4k_mul_mm_kernel, dim3((batch + BM - 1) / BM, (rows + BN - 1) / BN), dim3(256), 0, st, p);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : hip_fail(e, "mul_mm launch");
+}
+
+}  // namespace
+
+int bind_matvec_batch(ksh_kernel &k)
+{
+    const int64_t rows = k.desc.dims[0], cols = k.desc.dims[1], batch = k.desc.dims[2];
+    if (k.desc.dtypes[0] != KSH_Q4K) return set_error("matvec_batch: weight dtype %d is not built (Q4_K is)", k.desc.dtypes[0]);
+    if (k.desc.dtypes[1] != KSH_BF16) return set_error("matvec_batch: activation dtype %d is not built (BF16 is)", k.desc.dtypes[1]);
+    if (rows <= 0 || batch <= 0 || rows > (1 << 24) || batch > (1 << 20)) return set_error("matvec_batch: rows=%lld batch=%lld", (long long)rows, (long long)batch);
+    if (cols <= 0 || cols % 256 || cols > (1 << 20)) return set_error("matvec_batch: cols=%lld is not a positive multiple of 256", (long long)cols);
+    k.info.n_inputs = 2;
+    k.info.n_outputs = 1;
+    k.in_bytes[0] = (size_t)rows * (cols / 256) * 144; k.in_align[0] = 16;
+    k.in_bytes[1] = (size_t)batch * cols * 2; k.in_align[1] = 16;
+    k.out_bytes[0] = (size_t)batch * rows * 4; k.out_align[0] = 4;
+    // f16 copy of X plus the min-term operand (32 halves per token and superblock)
+    k.scratch_bytes = (size_t)batch * cols * 2 + (size_t)batch * (cols / 256) * 64;
+    set_launch(k, (uint32_t)((batch + BM - 1) / BM), (uint32_t)((rows + BN - 1) / BN), 1, 256,
+               (uint32_t)((BM + BN) * (PITCH + PITCH2) * 2 + BN * 4));
+    k.info.sched = k.desc.sched;
+    k.info.sched.tg = 256; k.info.sched.nsg = 4; k.info.sched.lds_tile = KS;
+    set_name(k, "mul_mm_q4k_%dx%dx%d", BM, BN, KS);
+    k.launch = launch_mul_mm;
+    return 0;
+}
+
+}  // namespace ksh

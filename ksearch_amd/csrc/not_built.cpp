@@ -3,6 +3,5 @@
 #include "ksh_internal.hpp"
 
 namespace ksh {
-int bind_matvec_batch(ksh_kernel &) { return set_error("matvec_batch (Q4_K prefill GEMM) is not built yet"); }
 }  // namespace ksh
 

@@ -1,0 +1,90 @@
+"""Q4_K prefill GEMM on the matrix cores vs the CPU oracle (dequant, bf16->f32
+X, sequential f32 dot), 1e-3 relative; shapes and inputs of the reference's
+check_mul_mm example plus the full benchmark configuration."""
+import numpy as np
+import pytest
+
+import oracle
+from ksearch_amd import hip, synth
+from ksearch_amd.hip import DType
+from tests.gpu_util import assert_close
+from tests.test_oracle_ops import check_mul_mm_inputs
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = hip.Context()
+    yield c
+    c.close()
+
+
+@pytest.fixture(scope="module")
+def eng():
+    return hip.Eng()
+
+
+def run(ctx, eng, w, rows, cols, xf, xb, batch):
+    y = ctx.buffer_empty_f32(batch * rows)
+    eng.matvec_batch(ctx, rows, cols, batch, DType.Q4K, ctx.buffer_bytes(w), ctx.buffer_bytes(xb), y)
+    got = ctx.read_f32(y, batch * rows).reshape(batch, rows)
+    want = oracle.matmul(oracle.Q4K, w, rows, cols, xf, batch)
+    return got, want
+
+
+# crates/ksearch_kernels/examples/check_mul_mm.rs:296-304
+@pytest.mark.parametrize("rows,cols,batch", [(64, 256, 16), (128, 256, 9), (2048, 1536, 256), (4096, 1536, 55)])
+def test_mul_mm_check_mul_mm_shapes(ctx, eng, rows, cols, batch):
+    w, x = check_mul_mm_inputs(rows, cols, batch)
+    wq = oracle.quantize_q4k(w)
+    xf, xb = synth.bf16_round(x)
+    got, want = run(ctx, eng, wq, rows, cols, xf.reshape(batch, cols), xb.reshape(batch, cols), batch)
+    assert_close(got, want, 1e-3, f"mul_mm {rows}x{cols} b{batch}")
+    # mul_mm row t equals the GEMV on x[t] (the example's "mul_mm vs gemv" line)
+    by = ctx.buffer_empty_f32(rows)
+    bw = ctx.buffer_bytes(wq)
+    for t in (0, batch - 1):
+        eng.matvec_wd(ctx, rows, cols, DType.Q4K, bw, ctx.buffer_f32(xf.reshape(batch, cols)[t]), by)
+        assert_close(got[t], ctx.read_f32(by, rows), 1e-3, f"mul_mm vs gemv t={t}")
+
+
+@pytest.mark.parametrize("rows,cols,batch", [(1, 256, 1), (130, 512, 129), (257, 2048, 33)])
+def test_mul_mm_random_blocks_ragged(ctx, eng, rows, cols, batch):
+    w = synth.q4k_blocks(rows * cols // 256, seed=600 + rows)
+    xf, xb = synth.bf16_round(synth.normal_f32(batch * cols, 601))
+    got, want = run(ctx, eng, w, rows, cols, xf.reshape(batch, cols), xb.reshape(batch, cols), batch)
+    assert_close(got, want, 1e-3, f"mul_mm {rows}x{cols} b{batch}")
+
+
+def test_mul_mm_unit_columns_recover_weights(ctx, eng):
+    # X = one-hot rows: Y[t] is column k_t of the dequantized matrix (pins the K order end to end)
+    rows, cols = 64, 512
+    w = synth.q4k_blocks(rows * cols // 256, seed=610)
+    wd = oracle.dequant(oracle.Q4K, w, rows * cols).reshape(rows, cols)
+    ks = [0, 1, 2, 3, 15, 16, 31, 32, 33, 63, 64, 127, 255, 256, 300, 511]
+    x = np.zeros((len(ks), cols), dtype=np.float32)
+    for t, k in enumerate(ks):
+        x[t, k] = 1.0
+    xf, xb = synth.bf16_round(x.reshape(-1))
+    got, _ = run(ctx, eng, w, rows, cols, xf.reshape(len(ks), cols), xb.reshape(len(ks), cols), len(ks))
+    for t, k in enumerate(ks):
+        # the 1024-bias and the hi/lo split of the min term leave ~2^-22 of 1024*d
+        assert np.allclose(got[t], wd[:, k], rtol=1e-5, atol=1e-5 * np.abs(wd).max()), k
+
+
+def test_mul_mm_cfg2_full_size(ctx, eng):
+    tokens, rows, cols = 512, 8192, 2048
+    w, xf, xb = synth.cfg2_q4k_prefill()
+    got, want = run(ctx, eng, w, rows, cols, xf, xb, tokens)
+    assert_close(got, want, 1e-3, "cfg2")
+    # linearity in X (size-independent property): W(2x) = 2 W(x) exactly in binary floating point
+    got2, _ = run(ctx, eng, w, rows, cols, 2 * xf[:128], synth.bf16_round((2 * xf[:128]).reshape(-1))[1].reshape(128, cols), 128)
+    assert np.array_equal(got2, 2 * got[:128])
+
+
+def test_mul_mm_errors(ctx):
+    with pytest.raises(hip.KshError, match="not built"):
+        ctx.compile(hip.make_desc(hip.Kind.MATVEC_BATCH, (64, 256, 16), (DType.Q6K, DType.BF16, DType.F32)))
+    with pytest.raises(hip.KshError, match="multiple of 256"):
+        ctx.compile(hip.make_desc(hip.Kind.MATVEC_BATCH, (64, 100, 16), (DType.Q4K, DType.BF16, DType.F32)))

@@ -96,6 +96,69 @@ def bench_matvec(ctx, eng, ev, dtype, rows, cols, w_host, x_host, copies, steps,
                 alg_bytes=alg, ms=ms)
 
 
+def bench_prefill(ctx):
+    """cfg2: 512 bf16 tokens x Q4_K [8192 x 2048] -> f32, hipEvent average of 50 launches."""
+    from ksearch_amd import hip, synth
+
+    tokens, rows, cols = 512, 8192, 2048
+    w, _, xb = synth.cfg2_q4k_prefill()
+    bw, bx, by = ctx.buffer_bytes(w), ctx.buffer_bytes(xb), ctx.buffer_empty_f32(tokens * rows)
+    k = ctx.compile(hip.make_desc(hip.Kind.MATVEC_BATCH, (rows, cols, tokens),
+                                  (hip.DType.Q4K, hip.DType.BF16, hip.DType.F32)))
+    ctx.run(k, [bw, bx], [by], iters=5)
+    ms = ctx.run(k, [bw, bx], [by], iters=50)
+    tf = 2.0 * tokens * rows * cols / (ms * 1e-3) / 1e12
+    for b in (bw, bx, by):
+        b.release()
+    return dict(kernel=k.name, us_per_launch=round(ms * 1e3, 2), tflops=round(tf, 1), frac_mfma_f16=round(tf / 2500.0, 4))
+
+
+def bench_attention(ctx):
+    """cfg3: 4 slots, 8 q / 1 kv heads of 256, Q4_0 KV, lengths ~U{1024..16384}, one launch pair."""
+    from ksearch_amd import hip, synth
+
+    n_slots, n_q, n_kv, hd, max_t = 4, 8, 1, 256, 16384
+    lens, kk, vv, q = synth.cfg3_q40_attention()
+    meta = np.zeros((n_slots, 4), dtype=np.float32)
+    meta[:, 0] = lens
+    k = ctx.compile(hip.make_desc(hip.Kind.SDPA_SLOTS, (n_q, n_kv, hd, max_t, n_slots, 0),
+                                  (hip.DType.Q40, hip.DType.F32), (1.0 / 16.0,)))
+    nwg = k.info.sched.k_split
+    ins = [ctx.buffer_f32(q), ctx.buffer_bytes(kk), ctx.buffer_bytes(vv), ctx.buffer_f32(meta)]
+    outs = [ctx.buffer_empty_f32(n_slots * n_q * nwg * (hd + 2)), ctx.buffer_empty_f32(n_slots * n_q * hd)]
+    ctx.run(k, ins, outs, iters=5)
+    ms = ctx.run(k, ins, outs, iters=50)
+    alg = int(sum(288 * int(t) + 16384 for t in lens))
+    for b in ins + outs:
+        b.release()
+    return dict(kernel=k.name, lens=[int(t) for t in lens], us_per_launch=round(ms * 1e3, 2),
+                gbps=round(alg / (ms * 1e-3) / 1e9, 1), frac_hbm=round(alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                note="resident in cache between launches (7 MB working set)")
+
+
+def bench_decode(ctx, eng, use_graph=True):
+    """cfg4: synthetic Gemma-4-E2B-shaped greedy decode, 64-token prompt then 256 tokens, HIP-graph replay."""
+    from ksearch_amd import hip, synth
+
+    cfg = synth.GEMMA_E2B_SYNTH
+    q4k, q6k = hip.device_quantizers(ctx, eng)
+    w = synth.gemma_weights(cfg, 4000, q4k, q6k)
+    m = hip.Gemma(ctx, cfg, w)
+    prompt = [int(t) for t in np.random.default_rng(4001).integers(0, cfg["vocab"], 64)]
+    m.generate(prompt, 8, use_graph=use_graph)     # warm-up: binds kernels, captures the graphs
+    m.reset()
+    _, pre_ms, dec_ms = m.generate(prompt, 256, use_graph=use_graph)
+    h, f, hd = cfg["hidden"], cfg["ffn"], cfg["hd"]
+    layer = (cfg["n_q"] * hd * h + 2 * cfg["n_kv"] * hd * h + h * cfg["n_q"] * hd + 3 * f * h) // 256 * 144
+    per_tok = cfg["n_layers"] * layer + cfg["vocab"] * h // 256 * 210
+    out = dict(tok_per_s=round(256 / dec_ms * 1e3, 1), ms_per_token=round(dec_ms / 256, 4),
+               launches_per_token=m.launches_per_token, weight_gbps=round(per_tok * 256 / (dec_ms * 1e-3) / 1e9, 1),
+               frac_hbm=round(per_tok * 256 / (dec_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+               prompt_tokens=64, new_tokens=256, graph=bool(use_graph))
+    m.close()
+    return out
+
+
 def cpu_baseline_matvec(w, x, rows, cols, budget_s=1.5):
     """The CPU checker (oracle/) timed on this machine: all cores, then one."""
     import oracle
@@ -122,6 +185,9 @@ def main() -> int:
     ap.add_argument("--copies", type=int, default=64)
     ap.add_argument("--no-extras", action="store_true", help="headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--eager", action="store_true", help="cfg4 without HIP-graph replay (kernel-trace profiling)")
+    ap.add_argument("--only", choices=["cfg1", "cfg2", "cfg3", "cfg4"],
+                    help="run one secondary workload and print its record (for profiling runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (the hot path is a single-GPU kernel path); "
@@ -132,6 +198,16 @@ def main() -> int:
     from ksearch_amd.hip import DType
 
     ctx, eng, ev = hip.Context(), hip.Eng(), HipEvents()
+    if args.only:
+        if args.only == "cfg1":
+            w1, x1 = synth.cfg1_q6k_lm_head()
+            r = bench_matvec(ctx, eng, ev, DType.Q6K, 262144, 2048, w1, x1, 1, 50, 5)
+        else:
+            r = {"cfg2": lambda: bench_prefill(ctx), "cfg3": lambda: bench_attention(ctx),
+                 "cfg4": lambda: bench_decode(ctx, eng, not args.eager)}[args.only]()
+        ctx.close()
+        print(json.dumps({args.only: r}))
+        return 0
     rows = cols = 4096
     w, x = synth.cfg0_q4k_matvec()
     head = bench_matvec(ctx, eng, ev, DType.Q4K, rows, cols, w, x, args.copies, args.steps, args.warmup)
@@ -145,6 +221,9 @@ def main() -> int:
         also["cfg1_q6k_lm_head"] = dict(kernel=r1["kernel"], us_per_launch=round(r1["us_per_launch"], 2),
                                         gbps=round(r1["gbps"], 1), frac_hbm=round(r1["gbps"] / HBM_PEAK_GBPS, 4))
         del w1
+        also["cfg2_q4k_prefill_gemm"] = bench_prefill(ctx)
+        also["cfg3_q40_attention"] = bench_attention(ctx)
+        also["cfg4_gemma_decode"] = bench_decode(ctx, eng)
 
     cpu = None
     if not args.no_cpu:

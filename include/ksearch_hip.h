@@ -109,6 +109,18 @@ enum ksh_kind {
      * Q6_K packer, as device kernels.  dims: n_elems.  dtypes[0] = Q4K | Q6K.
      * in: src f32   out: packed */
     KSH_QUANTIZE_K = 18,
+    /* RmsNormMatvec / RmsNormMatvecQkv / RmsNormMatvecGateUpGelu
+     * (crates/ksearch_ir/src/kernel.rs:303-339): the GEMV's workgroups compute
+     * the RMSNorm of the vector themselves.  Same dims as the plain kinds plus a
+     * trailing has_residual flag; params[0] = eps.
+     *   has_residual = 0: in: W.., x, w_norm                 out: y..
+     *   has_residual = 1: in: W.., y, w_norm, w_post, res    out: y.., x_new
+     *     with x_new = res + rms(y)*w_post (RmsNormAdd, the new residual stream,
+     *     which must not alias res) and the GEMV input rms(x_new)*w_norm
+     *     (RmsNormAddThenRmsNorm, kernel.rs:474-481, folded into its consumer). */
+    KSH_RMSNORM_MATVEC = 19,
+    KSH_RMSNORM_MATVEC_QKV = 20,
+    KSH_RMSNORM_MATVEC_GATE_UP_GELU = 21,
     KSH_KIND_COUNT
 };
 
@@ -116,7 +128,7 @@ enum ksh_kind {
  * All-zero means "library default, or the plan cache's entry if one exists". */
 typedef struct {
     uint64_t tg;       /* threads per workgroup (64 * waves) */
-    uint32_t vec;      /* inner-product variant: 0/1 = cvt+fma, 2 = f16 mix-fma, 3 = int8 dot */
+    uint32_t vec;      /* inner-product variant: 1 = byte converts + f32 FMA, 3 = int8 dot over 3 digit planes */
     uint32_t unroll;   /* superblocks in flight per lane */
     uint32_t nsg;      /* waves per workgroup */
     uint32_t nr0;      /* rows per wave */

@@ -3,11 +3,20 @@
 // Mirrors GemmaPrimModel::forward_token and generate_timed
 // (crates/ksearch_gemma/src/gemma_prim.rs:881-1275, 1658-1768) without the
 // parts that shape lacks (per-layer embeddings, sliding-window layers, shared
-// KV): per layer
+// KV).  The reference's per-layer sequence is
 //   rmsnorm -> fused QKV GEMV -> per-head RMS + RoPE + Q4_0 KV append ->
 //   split-KV attention -> o-proj GEMV -> add-then-rmsnorm ->
 //   fused gate||up + GELU GEMV -> down GEMV -> rmsnorm_add
-// then the output norm, the Q6_K LM head and the soft-capped argmax.
+// then the output norm, the Q6_K LM head and the soft-capped argmax.  Here every
+// normalisation rides in the GEMV that consumes it (RmsNormMatvecQkv,
+// RmsNormMatvecGateUpGelu with the preceding residual add folded in), so a
+// layer is
+//   [add+]rmsnorm+QKV -> per-head RMS + RoPE + KV append -> attention ->
+//   o-proj -> add+rmsnorm+gate||up+GELU -> down
+// and the layer-closing rmsnorm_add becomes the prologue of the next layer's
+// QKV (or of the output norm).  The residual stream ping-pongs between two
+// buffers because the fused prologue may not overwrite the vector that other
+// workgroups of the same launch still read.
 //
 // What differs from the reference's host loop, and why:
 //   - the position lives in a device buffer (meta = {tlen, start, window,
@@ -62,13 +71,13 @@ struct ksh_gemma {
     std::vector<ksh_gemma_layer> layers;
     ksh_buf *embd = nullptr, *output_norm = nullptr;
     Bufs bufs;
-    ksh_buf *x = nullptr, *x2 = nullptr, *tq = nullptr, *tk = nullptr, *tv = nullptr, *to = nullptr, *ff = nullptr,
+    ksh_buf *x = nullptr, *xb = nullptr, *y = nullptr, *x2 = nullptr, *hidden = nullptr, *tq = nullptr, *tk = nullptr, *tv = nullptr, *to = nullptr, *ff = nullptr,
             *logits = nullptr, *tok = nullptr, *meta = nullptr, *rope = nullptr, *attn_tmp = nullptr,
             *history = nullptr;
     std::vector<ksh_buf *> kv_k, kv_v;
-    ksh_kernel *k_embed = nullptr, *k_rms = nullptr, *k_qkv = nullptr, *k_head = nullptr, *k_sdpa = nullptr,
+    ksh_kernel *k_embed = nullptr, *k_qkv_first = nullptr, *k_qkv = nullptr, *k_head = nullptr, *k_sdpa = nullptr,
                *k_oproj = nullptr, *k_add_then = nullptr, *k_gate_up = nullptr, *k_down = nullptr,
-               *k_rms_add = nullptr, *k_lm_head = nullptr, *k_argmax = nullptr;
+               *k_lm_head = nullptr, *k_argmax = nullptr;
     ksh_graph *g_body = nullptr, *g_full = nullptr;
     int pos = 0;
     int launches_full = 0;
@@ -117,24 +126,34 @@ int encode_token(ksh_gemma *m, bool want_logits, int &launches)
 {
     const ksh_gemma_cfg &c = m->c;
     launches = 0;
-    if (enc(m, m->k_embed, {m->embd, m->tok}, {m->x}, launches)) return 1;
+    ksh_buf *cur = m->x, *other = m->xb;   // the residual stream and its next home
+    if (enc(m, m->k_embed, {m->embd, m->tok}, {cur}, launches)) return 1;
     for (int l = 0; l < c.n_layers; l++) {
         const ksh_gemma_layer &L = m->layers[l];
-        if (enc(m, m->k_rms, {m->x, L.attn_norm}, {m->x2}, launches)) return 1;
-        if (enc(m, m->k_qkv, {L.wq, L.wk, L.wv, m->x2}, {m->tq, m->tk, m->tv}, launches)) return 1;
+        if (l == 0) {
+            if (enc(m, m->k_qkv_first, {L.wq, L.wk, L.wv, cur, L.attn_norm}, {m->tq, m->tk, m->tv}, launches)) return 1;
+        } else {
+            // closes layer l-1 (x += rmsnorm(down, post_ffw_norm), gemma_prim.rs:1150-1160) and opens layer l
+            if (enc(m, m->k_qkv, {L.wq, L.wk, L.wv, m->y, L.attn_norm, m->layers[l - 1].post_ffw_norm, cur},
+                    {m->tq, m->tk, m->tv, other}, launches))
+                return 1;
+            std::swap(cur, other);
+        }
         if (enc(m, m->k_head, {m->tq, L.q_norm, m->rope, m->tk, L.k_norm, m->tv, m->meta},
                 {m->tq, m->kv_k[l], m->kv_v[l]}, launches))
             return 1;
         if (enc(m, m->k_sdpa, {m->tq, m->kv_k[l], m->kv_v[l], m->meta}, {m->attn_tmp, m->to}, launches)) return 1;
         launches += 1;   // the attention kind is two launches (partials, merge)
-        if (enc(m, m->k_oproj, {L.wo, m->to}, {m->x2}, launches)) return 1;
-        if (enc(m, m->k_add_then, {m->x2, L.post_attn_norm, m->x, L.ffn_norm}, {m->x, m->x2}, launches)) return 1;
-        if (enc(m, m->k_gate_up, {L.wgate, L.wup, m->x2}, {m->ff}, launches)) return 1;
-        if (enc(m, m->k_down, {L.wdown, m->ff}, {m->x2}, launches)) return 1;
-        if (enc(m, m->k_rms_add, {m->x2, L.post_ffw_norm, m->x}, {m->x}, launches)) return 1;
+        if (enc(m, m->k_oproj, {L.wo, m->to}, {m->y}, launches)) return 1;
+        if (enc(m, m->k_gate_up, {L.wgate, L.wup, m->y, L.ffn_norm, L.post_attn_norm, cur}, {m->ff, other}, launches)) return 1;
+        std::swap(cur, other);
+        if (enc(m, m->k_down, {L.wdown, m->ff}, {m->y}, launches)) return 1;
     }
     if (want_logits) {
-        if (enc(m, m->k_rms, {m->x, m->output_norm}, {m->x2}, launches)) return 1;
+        // the last layer's rmsnorm_add and the output norm in one pass
+        if (enc(m, m->k_add_then, {m->y, m->layers[c.n_layers - 1].post_ffw_norm, cur, m->output_norm}, {other, m->x2}, launches))
+            return 1;
+        m->hidden = other;
         if (enc(m, m->k_lm_head, {m->embd, m->x2}, {m->logits}, launches)) return 1;
         if (enc(m, m->k_argmax, {m->logits}, {m->tok}, launches)) return 1;
         launches += 1;   // two passes
@@ -207,7 +226,8 @@ int ksh_gemma_create(ksh_ctx *ctx, const ksh_gemma_cfg *cfg, const ksh_gemma_lay
     const int64_t qd = (int64_t)c.n_q * c.hd, kvd = (int64_t)c.n_kv * c.hd;
     const size_t kv_bytes = (size_t)c.max_seq * c.n_kv * (c.hd / 32) * 18;   // kv_pool.rs:113-116
     ksh_gemma *g = m.get();
-    if (alloc(g, (size_t)c.hidden * 4, &g->x) || alloc(g, (size_t)c.hidden * 4, &g->x2) ||
+    if (alloc(g, (size_t)c.hidden * 4, &g->x) || alloc(g, (size_t)c.hidden * 4, &g->xb) ||
+        alloc(g, (size_t)c.hidden * 4, &g->y) || alloc(g, (size_t)c.hidden * 4, &g->x2) ||
         alloc(g, (size_t)qd * 4, &g->tq) || alloc(g, (size_t)kvd * 4, &g->tk) || alloc(g, (size_t)kvd * 4, &g->tv) ||
         alloc(g, (size_t)qd * 4, &g->to) || alloc(g, (size_t)c.ffn * 4, &g->ff) ||
         alloc(g, (size_t)c.vocab * 4, &g->logits) || alloc(g, 16, &g->tok) || alloc(g, 16, &g->meta) ||
@@ -236,15 +256,14 @@ int ksh_gemma_create(ksh_ctx *ctx, const ksh_gemma_cfg *cfg, const ksh_gemma_lay
 
     const float embed_scale = std::sqrt((float)c.hidden);   // gemma_prim.rs:683
     if (get(g, KSH_COPY_SCALE_INDEXED, {c.hidden, c.vocab}, {KSH_Q6K}, {embed_scale}, &g->k_embed) ||
-        get(g, KSH_RMSNORM, {c.hidden, 0, 0}, {}, {c.eps, 0.f}, &g->k_rms) ||
-        get(g, KSH_MATVEC_QKV, {qd, kvd, c.hidden}, {KSH_Q4K, KSH_F32}, {}, &g->k_qkv) ||
+        get(g, KSH_RMSNORM_MATVEC_QKV, {qd, kvd, c.hidden, 0}, {KSH_Q4K, KSH_F32}, {c.eps}, &g->k_qkv_first) ||
+        get(g, KSH_RMSNORM_MATVEC_QKV, {qd, kvd, c.hidden, 1}, {KSH_Q4K, KSH_F32}, {c.eps}, &g->k_qkv) ||
         get(g, KSH_RMSNORM_PER_HEAD_QKV_Q40, {c.n_q, c.n_kv, c.hd, c.max_seq}, {}, {c.eps}, &g->k_head) ||
         get(g, KSH_SDPA_SLOTS, {c.n_q, c.n_kv, c.hd, c.max_seq, 1, g->nwg}, {KSH_Q40, KSH_F32}, {c.attn_scale}, &g->k_sdpa) ||
         get(g, KSH_MATVEC, {c.hidden, qd}, {KSH_Q4K, KSH_F32}, {}, &g->k_oproj) ||
         get(g, KSH_RMSNORM_ADD_THEN_RMSNORM, {c.hidden}, {}, {c.eps}, &g->k_add_then) ||
-        get(g, KSH_MATVEC_GATE_UP_GELU, {c.ffn, c.hidden}, {KSH_Q4K, KSH_F32}, {}, &g->k_gate_up) ||
+        get(g, KSH_RMSNORM_MATVEC_GATE_UP_GELU, {c.ffn, c.hidden, 1}, {KSH_Q4K, KSH_F32}, {c.eps}, &g->k_gate_up) ||
         get(g, KSH_MATVEC, {c.hidden, c.ffn}, {KSH_Q4K, KSH_F32}, {}, &g->k_down) ||
-        get(g, KSH_RMSNORM, {c.hidden, 1, 0}, {}, {c.eps, 0.f}, &g->k_rms_add) ||
         get(g, KSH_MATVEC, {c.vocab, c.hidden}, {KSH_Q6K, KSH_F32}, {}, &g->k_lm_head) ||
         get(g, KSH_SOFTCAP_ARGMAX, {c.vocab}, {}, {c.softcap}, &g->k_argmax))
         return 1;
@@ -319,7 +338,7 @@ int ksh_gemma_generate(ksh_gemma *m, const uint32_t *prompt, int n_prompt, int n
 }
 
 ksh_buf *ksh_gemma_logits(ksh_gemma *m) { return m ? m->logits : nullptr; }
-ksh_buf *ksh_gemma_hidden(ksh_gemma *m) { return m ? m->x : nullptr; }
+ksh_buf *ksh_gemma_hidden(ksh_gemma *m) { return m ? (m->hidden ? m->hidden : m->x) : nullptr; }
 ksh_buf *ksh_gemma_kv(ksh_gemma *m, int layer, int which)
 {
     if (!m || layer < 0 || layer >= m->c.n_layers) return nullptr;

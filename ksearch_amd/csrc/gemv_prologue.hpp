@@ -1,0 +1,211 @@
+// What a GEMV workgroup does before it touches its weights' values: produce the
+// activation vector in LDS.  Three sources, selected at run time:
+//
+//   kPlain      x as given                                   (Matvec, MatvecQkv, MatvecGateUpGelu)
+//   kRms        (x * rsqrt(mean(x^2)+eps)) * w_norm          (RmsNormMatvec*, kernel.rs:303-339)
+//   kAddThenRms x_new = res + (y*inv)*w_post, written back by workgroup 0 as the
+//               residual stream, then (x_new*inv2)*w_norm     (RmsNormAddThenRmsNorm, lower.rs:3926-4077,
+//               folded into the consumer GEMV)
+//
+// and two LDS formats, selected at compile time:
+//
+//   F32   floats with 4 of padding per 64 (lane stride 68 dwords: conflict-free b128 reads)
+//   I8x3  per 32-element sub-block a scale s = amax/(2^20-1) and X = rint(x/s) as three
+//         balanced base-128 int8 digits (X = 16384 h + 128 m + l), laid out per 64
+//         elements as H[64] M[64] L[64] + 16 bytes of padding (lane stride 52 dwords),
+//         followed by s[] and the exact f32 sub-block sums Sx[].  |x - s X| <= s/2, i.e.
+//         2^-21 of the sub-block's largest magnitude: below f32 summation noise of a
+//         2048-term dot, so the integer dot products (exact) keep f32-class accuracy.
+#pragma once
+
+#include "ksh_device.hpp"
+
+namespace ksh {
+
+enum { kPlain = 0, kRms = 1, kAddThenRms = 2 };
+enum { kXF32 = 0, kXI8 = 3 };
+
+struct Prologue {
+    const float *x;        // kPlain/kRms: the vector; kAddThenRms: y
+    const float *w_norm;   // kRms / kAddThenRms
+    const float *w_post;   // kAddThenRms
+    const float *res;      // kAddThenRms
+    float *x_out;          // kAddThenRms: residual stream out
+    float eps;
+    int kind;
+};
+
+__host__ __device__ constexpr int xs_f32_floats(int cols) { return cols + (cols >> 6) * 4; }
+__host__ __device__ constexpr int xs_i8_bytes(int cols) { return (cols >> 6) * 208 + (cols >> 5) * 8; }
+__device__ __forceinline__ int xs_f32_index(int e) { return e + ((e >> 6) << 2); }
+
+template <int XF>
+__host__ __device__ constexpr size_t xs_bytes(int cols)
+{
+    return (XF == kXI8 ? (size_t)xs_i8_bytes(cols) : (size_t)xs_f32_floats(cols) * 4) + 64;   // + reduction scratch
+}
+
+// max / sum over 8 consecutive lanes (one 32-element sub-block at 4 elements per lane)
+__device__ __forceinline__ float oct_max(float v)
+{
+    v = fmaxf(v, dpp_f32<0xB1>(v));
+    v = fmaxf(v, dpp_f32<0x4E>(v));
+    return fmaxf(v, dpp_f32<0x141>(v));
+}
+__device__ __forceinline__ float oct_sum(float v)
+{
+    v += dpp_f32<0xB1>(v);
+    v += dpp_f32<0x4E>(v);
+    return v + dpp_f32<0x141>(v);
+}
+
+template <int NT>
+__device__ __forceinline__ float block_sum(float v, float *red)
+{
+    const float w = wave_sum(v);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    __syncthreads();
+    if (lane == 0) red[wave] = w;
+    __syncthreads();
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < NT / 64; i++) s += red[i];
+    return s;
+}
+
+__device__ __forceinline__ uint32_t pack4_i8(int a, int b, int c, int d)
+{
+    return ((uint32_t)a & 0xFFu) | (((uint32_t)b & 0xFFu) << 8) | (((uint32_t)c & 0xFFu) << 16) | ((uint32_t)d << 24);
+}
+
+// one float4 (elements 4i..4i+3) into the LDS image
+template <int XF>
+__device__ __forceinline__ void store_x4(uint8_t *lds, int cols, int i, float4 v)
+{
+    if (XF == kXF32) {
+        *reinterpret_cast<float4 *>(reinterpret_cast<float *>(lds) + xs_f32_index(i * 4)) = v;
+        return;
+    }
+    const float amax = oct_max(fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+    const float sum = oct_sum((v.x + v.y) + (v.z + v.w));
+    const float inv = amax > 0.f ? 1048575.0f / amax : 0.f;
+    const float s = amax * (1.0f / 1048575.0f);
+    const float xs4[4] = {v.x, v.y, v.z, v.w};
+    int h[4], m[4], l[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const int X = (int)rintf(xs4[k] * inv);
+        l[k] = (X << 25) >> 25;
+        const int X1 = (X - l[k]) >> 7;
+        m[k] = (X1 << 25) >> 25;
+        h[k] = (X1 - m[k]) >> 7;
+    }
+    uint8_t *chunk = lds + (i >> 4) * 208 + (i & 15) * 4;
+    *reinterpret_cast<uint32_t *>(chunk) = pack4_i8(h[0], h[1], h[2], h[3]);
+    *reinterpret_cast<uint32_t *>(chunk + 64) = pack4_i8(m[0], m[1], m[2], m[3]);
+    *reinterpret_cast<uint32_t *>(chunk + 128) = pack4_i8(l[0], l[1], l[2], l[3]);
+    if ((threadIdx.x & 7) == 0) {
+        float *sc = reinterpret_cast<float *>(lds + (cols >> 6) * 208);
+        sc[2 * (i >> 3)] = s;
+        sc[2 * (i >> 3) + 1] = sum;
+    }
+}
+
+// Staging is split in two so that a GEMV can put its weight loads between the
+// halves: vector memory loads return in issue order within a wave, so whatever
+// is fetched after the (HBM-cold) weights also waits for them.  stage_fetch
+// issues every load the prologue needs (the vector and the norm weights are
+// L2-resident after the first workgroup), the caller then issues its weight
+// loads, and stage_finish does the arithmetic and the LDS writes while the
+// weights are still in flight.
+constexpr int kStageX = 8;   // float4 per thread of x kept in registers (plain: longer vectors stream later)
+constexpr int kStageP = 4;   // float4 per thread of w_norm / w_post / res (normalising prologues; host-checked)
+
+struct StageRegs {
+    float4 x[kStageX];
+    float4 wn[kStageP], wp[kStageP], rs[kStageP];
+};
+
+template <int NT>
+__device__ __forceinline__ void stage_fetch(const Prologue &pr, int cols, StageRegs &s)
+{
+    // n4 is a multiple of 64, so "this float4 exists" is a per-wave fact: keep it
+    // in scalar registers and the loads stay unpredicated
+    const int wbase = __builtin_amdgcn_readfirstlane(threadIdx.x & ~63), tid = wbase + (threadIdx.x & 63), n4 = cols / 4;
+    if (n4 > NT * kStageX) return;
+#pragma unroll
+    for (int k = 0; k < kStageX; k++) {
+        const int i = tid + k * NT;
+        if (wbase + k * NT < n4) s.x[k] = ldg_f4(pr.x, i);
+    }
+    if (pr.kind == kPlain) return;
+#pragma unroll
+    for (int k = 0; k < kStageP; k++) {
+        const int i = tid + k * NT;
+        if (wbase + k * NT < n4) s.wn[k] = ldg_f4(pr.w_norm, i);
+    }
+    if (pr.kind != kAddThenRms) return;
+#pragma unroll
+    for (int k = 0; k < kStageP; k++) {
+        const int i = tid + k * NT;
+        if (wbase + k * NT < n4) { s.wp[k] = ldg_f4(pr.w_post, i); s.rs[k] = ldg_f4(pr.res, i); }
+    }
+}
+
+// Every thread must call this (it contains barriers); the LDS image is complete
+// after the caller's next __syncthreads().
+template <int XF, int NT>
+__device__ __forceinline__ void stage_finish(const Prologue &pr, uint8_t *lds, int cols, StageRegs &s)
+{
+    const int wbase = __builtin_amdgcn_readfirstlane(threadIdx.x & ~63), tid = wbase + (threadIdx.x & 63), n4 = cols / 4;
+    float *red = reinterpret_cast<float *>(lds + (XF == kXI8 ? (size_t)xs_i8_bytes(cols) : (size_t)xs_f32_floats(cols) * 4));
+    if (pr.kind == kPlain) {
+        if (n4 > NT * kStageX) {
+            for (int i = tid; i < n4; i += NT) store_x4<XF>(lds, cols, i, ldg_f4(pr.x, i));
+            return;
+        }
+#pragma unroll
+        for (int k = 0; k < kStageX; k++) {
+            const int i = tid + k * NT;
+            if (wbase + k * NT < n4) store_x4<XF>(lds, cols, i, s.x[k]);
+        }
+        return;
+    }
+    float4 *v = s.x;
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < kStageP; k++) {
+        const int i = tid + k * NT;
+        if (wbase + k * NT < n4) ss += (v[k].x * v[k].x + v[k].y * v[k].y) + (v[k].z * v[k].z + v[k].w * v[k].w);
+    }
+    ss = block_sum<NT>(ss, red);
+    float inv = 1.0f / sqrtf(ss / (float)cols + pr.eps);
+    if (pr.kind == kAddThenRms) {
+        float ss2 = 0.f;
+#pragma unroll
+        for (int k = 0; k < kStageP; k++) {
+            const int i = tid + k * NT;
+            if (wbase + k * NT < n4) {
+                const float4 r = s.rs[k], w = s.wp[k];
+                v[k].x = r.x + v[k].x * inv * w.x;
+                v[k].y = r.y + v[k].y * inv * w.y;
+                v[k].z = r.z + v[k].z * inv * w.z;
+                v[k].w = r.w + v[k].w * inv * w.w;
+                ss2 += (v[k].x * v[k].x + v[k].y * v[k].y) + (v[k].z * v[k].z + v[k].w * v[k].w);
+                if (blockIdx.x == 0) stg_f4(pr.x_out, i, v[k]);
+            }
+        }
+        ss2 = block_sum<NT>(ss2, red);
+        inv = 1.0f / sqrtf(ss2 / (float)cols + pr.eps);
+    }
+#pragma unroll
+    for (int k = 0; k < kStageP; k++) {
+        const int i = tid + k * NT;
+        if (wbase + k * NT < n4) {
+            const float4 w = s.wn[k];
+            store_x4<XF>(lds, cols, i, make_float4(v[k].x * inv * w.x, v[k].y * inv * w.y, v[k].z * inv * w.z, v[k].w * inv * w.w));
+        }
+    }
+}
+
+}  // namespace ksh

@@ -9,6 +9,32 @@
 
 namespace ksh {
 
+// Loads and stores that say "global memory" themselves.  A pointer that went
+// through an opaque statement (or a select the compiler cannot see through) is
+// otherwise accessed with flat instructions, which count against the LDS
+// counter as well and turn every later wait into a wait for everything.
+#define KSH_GLOBAL __attribute__((address_space(1)))
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ uint4 ldg_u4(const void *p, size_t i)
+{
+    const u32x4_t v = ((const KSH_GLOBAL u32x4_t *)p)[i];
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ float4 ldg_f4(const float *p, size_t i)
+{
+    const f32x4_t v = ((const KSH_GLOBAL f32x4_t *)p)[i];
+    return make_float4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void stg_f4(float *p, size_t i, float4 v)
+{
+    f32x4_t w;
+    w.x = v.x; w.y = v.y; w.z = v.z; w.w = v.w;
+    ((KSH_GLOBAL f32x4_t *)p)[i] = w;
+}
+__device__ __forceinline__ void stg_f32(float *p, size_t i, float v) { ((KSH_GLOBAL float *)p)[i] = v; }
+
 constexpr int kWave = 64;
 
 __device__ __forceinline__ float as_f32(uint32_t u) { return __builtin_bit_cast(float, u); }

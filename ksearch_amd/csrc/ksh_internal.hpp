@@ -91,6 +91,7 @@ inline bool sched_is_zero(const ksh_sched &s)
 int bind_matvec(ksh_kernel &k);
 int bind_matvec_q4k(ksh_kernel &k);
 int bind_matvec_q6k(ksh_kernel &k);
+int bind_matvec_q4k_family(ksh_kernel &k);
 int bind_matvec_qkv(ksh_kernel &k);
 int bind_matvec_gate_up_gelu(ksh_kernel &k);
 int bind_matvec_batch(ksh_kernel &k);

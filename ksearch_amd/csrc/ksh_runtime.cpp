@@ -49,6 +49,9 @@ static int bind(ksh_kernel &k)
     case KSH_MATVEC_BATCH: return bind_matvec_batch(k);
     case KSH_MATVEC_QKV: return bind_matvec_qkv(k);
     case KSH_MATVEC_GATE_UP_GELU: return bind_matvec_gate_up_gelu(k);
+    case KSH_RMSNORM_MATVEC: return bind_matvec(k);
+    case KSH_RMSNORM_MATVEC_QKV:
+    case KSH_RMSNORM_MATVEC_GATE_UP_GELU: return bind_matvec_q4k_family(k);
     case KSH_SDPA_NAIVE:
     case KSH_SDPA_MWG_PART:
     case KSH_SDPA_MWG_REDUCE:

@@ -14,31 +14,29 @@
 //   - a wave therefore sweeps 16 superblocks (4096 columns) per step, and keeps
 //     the matching 64 activations per lane in registers across R rows, so x is
 //     read once per R rows;
-//   - x is staged once per workgroup in LDS (stride-padded so that the
-//     256-byte lane stride is bank-conflict free);
+//   - the activation vector is staged once per workgroup in LDS, either as
+//     padded f32 or as three int8 digit planes (gemv_prologue.hpp), optionally
+//     after an RMSNorm / add-then-RMSNorm computed by the workgroup itself;
 //   - every row's loads are issued before the first use, so one workgroup
 //     keeps R * 192 B per lane in flight;
 //   - the 6-bit scales/mins are unpacked in registers, the mins are applied
-//     through per-sub-block sums of x, and rows are reduced with DPP.
+//     through per-sub-block sums of x, and rows are reduced with DPP;
+//   - inner product variant 0: nibble -> f32 byte converts + FMAs; variant 3:
+//     nibbles unpacked to bytes and v_dot4_i32_i8 against the digit planes
+//     (exact integer sums per 32-wide sub-block, one f32 scale per sub-block).
 //
 // Arithmetic per (row, superblock, group), all f32:
 //   acc += d*sc_lo * sum(n_lo*x) + d*sc_hi * sum(n_hi*x) - dmin*(m_lo*Sx_lo + m_hi*Sx_hi)
 // which is the reference's coop form (render.rs:506-511) and differs from the
 // CPU dequant-then-dot (gguf_impl.rs:690-721 + check_mul_mm.rs:60-71) by
 // reassociation only.
-#include "ksh_device.hpp"
+#include "gemv_prologue.hpp"
 #include "ksh_internal.hpp"
 
 namespace ksh {
 namespace {
 
 constexpr int kQ4kBytes = 144;
-
-// LDS layout of x: 4 floats of padding after every 64, so lanes that are 64
-// floats apart land 68 dwords apart and eight consecutive lanes cover all 32
-// banks with their 16-byte reads.
-__device__ __forceinline__ int xs_index(int e) { return e + ((e >> 6) << 2); }
-__host__ __device__ constexpr int xs_floats(int cols) { return cols + (cols >> 6) * 4; }
 
 struct Q4kLane {
     uint4 hdr;   // d | dmin<<16, then the 12 scale bytes
@@ -49,92 +47,102 @@ struct Q4kLane {
 __device__ __forceinline__ Q4kLane q4k_load(const uint8_t *blk, int g)
 {
     Q4kLane r;
-    const uint4 *p = reinterpret_cast<const uint4 *>(blk);
-    r.hdr = p[0];
-    r.qa = p[1 + 2 * g];
-    r.qb = p[2 + 2 * g];
+    r.hdr = ldg_u4(blk, 0);
+    r.qa = ldg_u4(blk, 1 + 2 * g);
+    r.qb = ldg_u4(blk, 2 + 2 * g);
     return r;
 }
 
-// VAR 0: byte->float converts (v_cvt_f32_ubyteN) feeding plain FMAs.  `lo` gets
-// sum(n_lo*x[l]), `hi` gets 16*sum(n_hi*x[32+l]) (the high nibbles are left in
-// place; the 1/16 is folded into the scale, exactly).
-__device__ __forceinline__ void dot_dword_cvt(uint32_t w, const float *xl, const float *xh,
-                                              float &lo, float &hi)
-{
-    const uint32_t t = w & 0x0F0F0F0Fu, u = w & 0xF0F0F0F0u;
-    lo = fmaf(ubyte_f32<0>(t), xl[0], lo);
-    hi = fmaf(ubyte_f32<0>(u), xh[0], hi);
-    lo = fmaf(ubyte_f32<1>(t), xl[1], lo);
-    hi = fmaf(ubyte_f32<1>(u), xh[1], hi);
-    lo = fmaf(ubyte_f32<2>(t), xl[2], lo);
-    hi = fmaf(ubyte_f32<2>(u), xh[2], hi);
-    lo = fmaf(ubyte_f32<3>(t), xl[3], lo);
-    hi = fmaf(ubyte_f32<3>(u), xh[3], hi);
-}
+// The activations of one lane's 64-element group, as registers, in the format
+// its inner product wants.
+template <int XF>
+struct XGroup;
 
-typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
-
-// VAR 2: nibbles are OR-ed into the mantissa of half 1024.0 (0x6400), two per
-// instruction, and consumed by mixed-precision FMAs (f16 * f32 + f32, exact
-// products).  `lo` gets sum((1024+n_lo)*x), `hi` gets sum((1024+16 n_hi)*x);
-// the 1024*Sx terms are removed in the epilogue.
-// (a & mask) | magic in one VOP3 instruction; the masks live in VGPRs and the
-// magic in an SGPR because gfx950's VOP3 encoding takes no 32-bit literals
-// (left to itself the compiler emits a v_and + v_or pair per use).
-__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t magic)
-{
-    uint32_t r;
-    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(mask), "s"(magic));
-    return r;
-}
-
-__device__ __forceinline__ void dot_dword_mix(uint32_t w, const float *xl, const float *xh,
-                                              float &lo, float &hi)
-{
-    const uint32_t w8 = w >> 8;
-    const uint32_t mlo = 0x000F000Fu, mhi = 0x00F000F0u, magic = 0x64006400u;
-    const half2_t p0 = __builtin_bit_cast(half2_t, and_or(w, mlo, magic));    // bytes 0,2 low
-    const half2_t p1 = __builtin_bit_cast(half2_t, and_or(w, mhi, magic));    // bytes 0,2 high
-    const half2_t p2 = __builtin_bit_cast(half2_t, and_or(w8, mlo, magic));   // bytes 1,3 low
-    const half2_t p3 = __builtin_bit_cast(half2_t, and_or(w8, mhi, magic));   // bytes 1,3 high
-    lo = fmaf((float)p0.x, xl[0], lo);
-    hi = fmaf((float)p1.x, xh[0], hi);
-    lo = fmaf((float)p2.x, xl[1], lo);
-    hi = fmaf((float)p3.x, xh[1], hi);
-    lo = fmaf((float)p0.y, xl[2], lo);
-    hi = fmaf((float)p1.y, xh[2], hi);
-    lo = fmaf((float)p2.y, xl[3], lo);
-    hi = fmaf((float)p3.y, xh[3], hi);
-}
-
-// one (row, superblock, group): returns the f32 contribution to y[row]
-template <int VAR>
-__device__ __forceinline__ float q4k_group_dot(const Q4kLane &L, int g, const float *xr, float sx_lo,
-                                               float sx_hi)
-{
-    float lo0 = 0.f, lo1 = 0.f, hi0 = 0.f, hi1 = 0.f;
-    const uint32_t q[8] = {L.qa.x, L.qa.y, L.qa.z, L.qa.w, L.qb.x, L.qb.y, L.qb.z, L.qb.w};
+template <>
+struct XGroup<kXF32> {
+    float xr[64], sx_lo, sx_hi;
+    __device__ __forceinline__ void load(const uint8_t *lds, int cols, int b, int g)
+    {
+        (void)cols;
+        const float *xg = reinterpret_cast<const float *>(lds) + xs_f32_index(b * 256 + g * 64);
 #pragma unroll
-    for (int k = 0; k < 8; k += 2) {
-        if (VAR == 2) {
-            dot_dword_mix(q[k], xr + 4 * k, xr + 32 + 4 * k, lo0, hi0);
-            dot_dword_mix(q[k + 1], xr + 4 * k + 4, xr + 32 + 4 * k + 4, lo1, hi1);
-        } else {
-            dot_dword_cvt(q[k], xr + 4 * k, xr + 32 + 4 * k, lo0, hi0);
-            dot_dword_cvt(q[k + 1], xr + 4 * k + 4, xr + 32 + 4 * k + 4, lo1, hi1);
+        for (int i = 0; i < 16; i++) {
+            const float4 v = *reinterpret_cast<const float4 *>(xg + 4 * i);
+            xr[4 * i] = v.x; xr[4 * i + 1] = v.y; xr[4 * i + 2] = v.z; xr[4 * i + 3] = v.w;
         }
+        float a0 = 0.f, a1 = 0.f, b0 = 0.f, b1 = 0.f;
+#pragma unroll
+        for (int i = 0; i < 32; i += 2) { a0 += xr[i]; a1 += xr[i + 1]; b0 += xr[32 + i]; b1 += xr[33 + i]; }
+        sx_lo = a0 + a1;
+        sx_hi = b0 + b1;
     }
-    float lo = lo0 + lo1, hi = hi0 + hi1;
+    // sum(n_lo*x) and 16*sum(n_hi*x): the high nibbles stay in place, the 1/16 is folded into the scale
+    __device__ __forceinline__ void dot(const Q4kLane &L, float &lo, float &hi) const
+    {
+        float lo0 = 0.f, lo1 = 0.f, hi0 = 0.f, hi1 = 0.f;
+        const uint32_t q[8] = {L.qa.x, L.qa.y, L.qa.z, L.qa.w, L.qb.x, L.qb.y, L.qb.z, L.qb.w};
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const uint32_t t = q[k] & 0x0F0F0F0Fu, u = q[k] & 0xF0F0F0F0u;
+            const float *xl = xr + 4 * k, *xh = xr + 32 + 4 * k;
+            float &a = (k & 1) ? lo1 : lo0, &c = (k & 1) ? hi1 : hi0;
+            a = fmaf(ubyte_f32<0>(t), xl[0], a); c = fmaf(ubyte_f32<0>(u), xh[0], c);
+            a = fmaf(ubyte_f32<1>(t), xl[1], a); c = fmaf(ubyte_f32<1>(u), xh[1], c);
+            a = fmaf(ubyte_f32<2>(t), xl[2], a); c = fmaf(ubyte_f32<2>(u), xh[2], c);
+            a = fmaf(ubyte_f32<3>(t), xl[3], a); c = fmaf(ubyte_f32<3>(u), xh[3], c);
+        }
+        lo = lo0 + lo1;
+        hi = (hi0 + hi1) * 0.0625f;
+    }
+};
+
+template <>
+struct XGroup<kXI8> {
+    uint32_t H[16], M[16], Lo[16];   // digit planes: dwords 0..7 low sub-block, 8..15 high sub-block
+    float s_lo, s_hi, sx_lo, sx_hi;
+    __device__ __forceinline__ void load(const uint8_t *lds, int cols, int b, int g)
+    {
+        const int c = b * 4 + g;
+        const uint4 *p = reinterpret_cast<const uint4 *>(lds + c * 208);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint4 h = p[i], m = p[4 + i], l = p[8 + i];
+            H[4 * i] = h.x; H[4 * i + 1] = h.y; H[4 * i + 2] = h.z; H[4 * i + 3] = h.w;
+            M[4 * i] = m.x; M[4 * i + 1] = m.y; M[4 * i + 2] = m.z; M[4 * i + 3] = m.w;
+            Lo[4 * i] = l.x; Lo[4 * i + 1] = l.y; Lo[4 * i + 2] = l.z; Lo[4 * i + 3] = l.w;
+        }
+        const float4 sc = *reinterpret_cast<const float4 *>(lds + (cols >> 6) * 208 + c * 16);
+        s_lo = sc.x; sx_lo = sc.y; s_hi = sc.z; sx_hi = sc.w;
+    }
+    __device__ __forceinline__ void dot(const Q4kLane &L, float &lo, float &hi) const
+    {
+        int hl = 0, ml = 0, ll = 0, hh = 0, mh = 0, lh = 0;
+        const uint32_t q[8] = {L.qa.x, L.qa.y, L.qa.z, L.qa.w, L.qb.x, L.qb.y, L.qb.z, L.qb.w};
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const int a = (int)(q[k] & 0x0F0F0F0Fu), c = (int)((q[k] >> 4) & 0x0F0F0F0Fu);
+            hl = __builtin_amdgcn_sdot4(a, (int)H[k], hl, false);
+            ml = __builtin_amdgcn_sdot4(a, (int)M[k], ml, false);
+            ll = __builtin_amdgcn_sdot4(a, (int)Lo[k], ll, false);
+            hh = __builtin_amdgcn_sdot4(c, (int)H[8 + k], hh, false);
+            mh = __builtin_amdgcn_sdot4(c, (int)M[8 + k], mh, false);
+            lh = __builtin_amdgcn_sdot4(c, (int)Lo[8 + k], lh, false);
+        }
+        lo = s_lo * (float)((hl << 14) + (ml << 7) + ll);
+        hi = s_hi * (float)((hh << 14) + (mh << 7) + lh);
+    }
+};
+
+// one (row, superblock, group): the f32 contribution to y[row]
+template <int XF>
+__device__ __forceinline__ float q4k_group_dot(const Q4kLane &L, int g, const XGroup<XF> &X)
+{
+    float lo, hi;
+    X.dot(L, lo, hi);
     const float d = half_bits_to_f32(L.hdr.x & 0xFFFFu), dmin = half_bits_to_f32(L.hdr.x >> 16);
     const uint4 s = q4k_group_scales(L.hdr.y, L.hdr.z, L.hdr.w, g);
-    const float sc_lo = (float)s.x, mn_lo = (float)s.y, sc_hi = (float)s.z, mn_hi = (float)s.w;
-    if (VAR == 2) {
-        lo = fmaf(-1024.f, sx_lo, lo);
-        hi = fmaf(-1024.f, sx_hi, hi);
-    }
-    const float pos = fmaf(sc_lo, lo, sc_hi * 0.0625f * hi);
-    const float neg = fmaf(mn_lo, sx_lo, mn_hi * sx_hi);
+    const float pos = fmaf((float)s.x, lo, (float)s.z * hi);
+    const float neg = fmaf((float)s.y, X.sx_lo, (float)s.w * X.sx_hi);
     return fmaf(d, pos, -(dmin * neg));
 }
 
@@ -146,20 +154,49 @@ __device__ __forceinline__ float gelu_mul_f32(float g, float u)
     return (0.5f * ax) * (1.0f + tanhf(t)) * u;
 }
 
-// One launch covers up to three weight matrices that share x.
+// One launch covers up to three weight matrices that share the input vector.
 //   mode 0: the matrices are independent row ranges (plain GEMV: one; QKV:
 //           three).  Every wave owns RPW consecutive rows of ONE matrix.
 //   mode 1: gate || up: every wave owns the same RPW rows of W[0] and W[1] and
 //           stores gelu(W0.x) * (W1.x).
+// (Named fields, not arrays: a run-time index into a by-value kernel argument
+// makes the compiler copy the whole struct to scratch memory.)
 struct MatvecParams {
-    const uint8_t *W[3];
-    float *y[3];
-    int rows[3];
-    int waves[3];      // waves assigned to each matrix (mode 0)
-    const float *x;
-    int bpr;           // superblocks per row (cols / 256)
+    const uint8_t *W0, *W1, *W2;
+    float *y0, *y1, *y2;
+    int rows0, rows1, rows2;
+    int waves0, waves1, waves2;   // waves assigned to each matrix (mode 0)
+    Prologue pro;
+    int bpr;                      // superblocks per row (cols / 256)
     int mode;
 };
+
+// Kernel arguments are fetched with scalar loads where they are first used;
+// left alone the compiler sinks each into the branch that needs it, and a wave
+// then pays one scalar-cache round trip after another before its first weight
+// load.  Copying the fields through two opaque statements at the top turns
+// that into a few wide loads and two waits.
+__device__ __forceinline__ MatvecParams fetch_params(const MatvecParams &p)
+{
+    const uint8_t *W0 = p.W0, *W1 = p.W1, *W2 = p.W2;
+    float *y0 = p.y0, *y1 = p.y1, *y2 = p.y2;
+    int rows0 = p.rows0, rows1 = p.rows1, rows2 = p.rows2, waves0 = p.waves0, waves1 = p.waves1, waves2 = p.waves2;
+    const float *x = p.pro.x, *w_norm = p.pro.w_norm, *w_post = p.pro.w_post, *res = p.pro.res;
+    float *x_out = p.pro.x_out;
+    int eps = __float_as_int(p.pro.eps), kind = p.pro.kind, bpr = p.bpr, mode = p.mode;
+    asm volatile("" : "+s"(W0), "+s"(W1), "+s"(W2), "+s"(y0), "+s"(y1), "+s"(y2), "+s"(rows0), "+s"(rows1), "+s"(rows2),
+                 "+s"(waves0), "+s"(waves1), "+s"(waves2));
+    asm volatile("" : "+s"(x), "+s"(w_norm), "+s"(w_post), "+s"(res), "+s"(x_out), "+s"(eps), "+s"(kind), "+s"(bpr), "+s"(mode));
+    MatvecParams q;
+    q.W0 = W0; q.W1 = W1; q.W2 = W2;
+    q.y0 = y0; q.y1 = y1; q.y2 = y2;
+    q.rows0 = rows0; q.rows1 = rows1; q.rows2 = rows2;
+    q.waves0 = waves0; q.waves1 = waves1; q.waves2 = waves2;
+    q.pro.x = x; q.pro.w_norm = w_norm; q.pro.w_post = w_post; q.pro.res = res; q.pro.x_out = x_out;
+    q.pro.eps = __int_as_float(eps); q.pro.kind = kind;
+    q.bpr = bpr; q.mode = mode;
+    return q;
+}
 
 struct WaveTask {
     const uint8_t *W0, *W1;
@@ -168,61 +205,53 @@ struct WaveTask {
     bool active;
 };
 
-// maps a global wave index onto (matrix, first row).  rpw = rows per wave.
+// (by-value arguments: all three are read before the choice, so nothing turns
+// this into a choice of address followed by a dependent load)
+template <class T>
+__device__ __forceinline__ T sel3(bool in1, bool in2, T a0, T a1, T a2)
+{
+    return in2 ? a2 : in1 ? a1 : a0;
+}
+
+// maps a global wave index onto (matrix, first row).  rpw = rows per wave.  The
+// index must live in scalar registers (readfirstlane): the matrix is then
+// picked with scalar loads of the kernel arguments instead of a per-lane
+// gather from them, which would put a memory round trip in front of every load.
 __device__ __forceinline__ WaveTask wave_task(const MatvecParams &p, int wv, int rpw)
 {
     WaveTask t;
-    int m = 0;
-    if (p.mode == 0) {
-        if (wv >= p.waves[0]) { wv -= p.waves[0]; m = 1; }
-        if (m == 1 && wv >= p.waves[1]) { wv -= p.waves[1]; m = 2; }
-    }
-    t.W0 = p.W[m];
-    t.W1 = p.W[1];
-    t.y = p.y[m];
-    t.rows = p.rows[m];
+    // selects between already-fetched arguments rather than indexing them
+    const bool in1 = p.mode == 0 && wv >= p.waves0;
+    const bool in2 = in1 && wv - p.waves0 >= p.waves1;
+    if (in1) wv -= p.waves0;
+    if (in2) wv -= p.waves1;
+    t.W0 = sel3(in1, in2, p.W0, p.W1, p.W2);
+    t.W1 = p.W1;
+    t.y = sel3(in1, in2, p.y0, p.y1, p.y2);
+    t.rows = sel3(in1, in2, p.rows0, p.rows1, p.rows2);
+    const int nw = sel3(in1, in2, p.waves0, p.waves1, p.waves2);
     t.row0 = wv * rpw;
-    t.active = t.row0 < t.rows && (p.mode == 1 || wv < p.waves[m]);
+    t.active = t.row0 < t.rows && (p.mode == 1 || wv < nw);
+    if (!t.active) {   // keeps its loads (so that every wave issues the same number) but points them at row 0
+        t.W0 = p.W0;
+        t.rows = p.rows0;
+        t.row0 = 0;
+    }
     return t;
-}
-
-template <int NW>
-__device__ __forceinline__ void stage_x(const float *x, float *xs, int n_float4, int tid)
-{
-    const float4 *x4 = reinterpret_cast<const float4 *>(x);
-    for (int i = tid; i < n_float4; i += NW * 64) {
-        const float4 v = x4[i];
-        *reinterpret_cast<float4 *>(&xs[xs_index(i * 4)]) = v;
-    }
-}
-
-__device__ __forceinline__ void load_x_group(const float *xs, int b, int g, float *xr, float &sx_lo,
-                                             float &sx_hi)
-{
-    const float *xg = &xs[xs_index(b * 256 + g * 64)];
-#pragma unroll
-    for (int i = 0; i < 16; i++) {
-        const float4 v = *reinterpret_cast<const float4 *>(xg + 4 * i);
-        xr[4 * i] = v.x; xr[4 * i + 1] = v.y; xr[4 * i + 2] = v.z; xr[4 * i + 3] = v.w;
-    }
-    float a0 = 0.f, a1 = 0.f, b0 = 0.f, b1 = 0.f;
-#pragma unroll
-    for (int i = 0; i < 32; i += 2) { a0 += xr[i]; a1 += xr[i + 1]; b0 += xr[32 + i]; b1 += xr[33 + i]; }
-    sx_lo = a0 + a1;
-    sx_hi = b0 + b1;
 }
 
 // Full-wave form: a wave owns R rows and sweeps 16 superblocks per step.
 // NM = 1 (mode 0) or 2 (mode 1).  The weight loads of step s+1 are issued
-// before step s is consumed, and step 0's before x is staged, so the first
-// HBM round trip overlaps the LDS fill.
-template <int R, int NW, int NM, int VAR, bool MULTI>
-__global__ __launch_bounds__(NW * 64) void q4k_gemv_kernel(MatvecParams p)
+// before step s is consumed, and step 0's before the input is staged, so the
+// first HBM round trip overlaps the prologue.
+template <int R, int NW, int NM, int XF, bool MULTI>
+__global__ __launch_bounds__(NW * 64) void q4k_gemv_kernel(MatvecParams p_in)
 {
-    extern __shared__ float xs[];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    extern __shared__ __attribute__((aligned(16))) uint8_t xs[];
+    const MatvecParams p = fetch_params(p_in);
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int g = lane & 3, bl = lane >> 2;
-    const int bpr = p.bpr;
+    const int bpr = p.bpr, cols = bpr * 256;
     const size_t row_bytes = (size_t)bpr * kQ4kBytes;
     const WaveTask t = wave_task(p, blockIdx.x * NW + wave, R);
 
@@ -235,15 +264,19 @@ __global__ __launch_bounds__(NW * 64) void q4k_gemv_kernel(MatvecParams p)
         if (NM == 2) rowp[NM - 1][r] = t.W1 + off;
     }
 
-    // MULTI: rows longer than 16 superblocks take several steps and double-buffer
+    // Every wave and lane issues the same loads, unconditionally (lanes past the
+    // row's end re-read its last superblock and drop the product): the wait for
+    // the staged vector can then be an exact count that leaves the weight loads
+    // in flight, where a conditional load would force a wait for everything.
+    // MULTI: rows longer than 16 superblocks take several steps and double-buffer.
     Q4kLane cur[NM][R], nxt[MULTI ? NM : 1][MULTI ? R : 1];
-    if (t.active && bl < bpr) {
+    StageRegs sr;
+    stage_fetch<NW * 64>(p.pro, cols, sr);
 #pragma unroll
-        for (int m = 0; m < NM; m++)
+    for (int m = 0; m < NM; m++)
 #pragma unroll
-            for (int r = 0; r < R; r++) cur[m][r] = q4k_load(rowp[m][r] + (size_t)bl * kQ4kBytes, g);
-    }
-    stage_x<NW>(p.x, xs, bpr * 64, tid);
+        for (int r = 0; r < R; r++) cur[m][r] = q4k_load(rowp[m][r] + (size_t)min(bl, bpr - 1) * kQ4kBytes, g);
+    stage_finish<XF, NW * 64>(p.pro, xs, cols, sr);
     __syncthreads();
     if (!t.active) return;
 
@@ -253,21 +286,26 @@ __global__ __launch_bounds__(NW * 64) void q4k_gemv_kernel(MatvecParams p)
 #pragma unroll
         for (int r = 0; r < R; r++) acc[m][r] = 0.f;
 
-    for (int b = bl; b < bpr; b += 16) {
-        const bool more = MULTI && b + 16 < bpr;
-        if (MULTI && more) {
+    for (int b0 = 0; b0 < bpr; b0 += 16) {
+        const int b = min(b0 + bl, bpr - 1);
+        const bool mine = b0 + bl < bpr;
+        if (MULTI) {
+            const int bn = min(b0 + 16 + bl, bpr - 1);
 #pragma unroll
             for (int m = 0; m < NM; m++)
 #pragma unroll
-                for (int r = 0; r < R; r++) nxt[m][r] = q4k_load(rowp[m][r] + (size_t)(b + 16) * kQ4kBytes, g);
+                for (int r = 0; r < R; r++) nxt[m][r] = q4k_load(rowp[m][r] + (size_t)bn * kQ4kBytes, g);
         }
-        float xr[64], sx_lo, sx_hi;
-        load_x_group(xs, b, g, xr, sx_lo, sx_hi);
+        XGroup<XF> X;
+        X.load(xs, cols, b, g);
 #pragma unroll
         for (int m = 0; m < NM; m++)
 #pragma unroll
-            for (int r = 0; r < R; r++) acc[m][r] += q4k_group_dot<VAR>(cur[m][r], g, xr, sx_lo, sx_hi);
-        if (MULTI && more) {
+            for (int r = 0; r < R; r++) {
+                const float v = q4k_group_dot<XF>(cur[m][r], g, X);
+                acc[m][r] += mine ? v : 0.f;
+            }
+        if (MULTI) {
 #pragma unroll
             for (int m = 0; m < NM; m++)
 #pragma unroll
@@ -281,18 +319,19 @@ __global__ __launch_bounds__(NW * 64) void q4k_gemv_kernel(MatvecParams p)
 #pragma unroll
         for (int m = 0; m < NM; m++) s[m] = wave_sum(acc[m][r]);
         const int row = t.row0 + r;
-        if (lane == 0 && row < t.rows) t.y[row] = (NM == 2) ? gelu_mul_f32(s[0], s[NM - 1]) : s[0];
+        if (lane == 0 && row < t.rows) stg_f32(t.y, row, (NM == 2) ? gelu_mul_f32(s[0], s[NM - 1]) : s[0]);
     }
 }
 
 // Half-wave form for rows of exactly 8 superblocks (2048 columns): lanes
 // 0..31 and 32..63 work on different rows, so a wave covers 2R rows in a single
 // step and no lane idles.
-template <int R, int NW, int NM, int VAR>
-__global__ __launch_bounds__(NW * 64) void q4k_gemv_half_kernel(MatvecParams p)
+template <int R, int NW, int NM, int XF>
+__global__ __launch_bounds__(NW * 64) void q4k_gemv_half_kernel(MatvecParams p_in)
 {
-    extern __shared__ float xs[];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    extern __shared__ __attribute__((aligned(16))) uint8_t xs[];
+    const MatvecParams p = fetch_params(p_in);
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int g = lane & 3, bl = (lane >> 2) & 7, hw = lane >> 5;
     constexpr int bpr = 8;
     constexpr size_t row_bytes = (size_t)bpr * kQ4kBytes;
@@ -300,31 +339,31 @@ __global__ __launch_bounds__(NW * 64) void q4k_gemv_half_kernel(MatvecParams p)
     const int row0 = t.row0 + hw * R;
 
     Q4kLane L[NM][R];
-    if (t.active) {
+    StageRegs sr;
+    stage_fetch<NW * 64>(p.pro, bpr * 256, sr);
 #pragma unroll
-        for (int r = 0; r < R; r++) {
-            const size_t off = (size_t)min(row0 + r, t.rows - 1) * row_bytes + (size_t)bl * kQ4kBytes;
-            L[0][r] = q4k_load(t.W0 + off, g);
-            if (NM == 2) L[NM - 1][r] = q4k_load(t.W1 + off, g);
-        }
+    for (int r = 0; r < R; r++) {
+        const size_t off = (size_t)min(row0 + r, t.rows - 1) * row_bytes + (size_t)bl * kQ4kBytes;
+        L[0][r] = q4k_load(t.W0 + off, g);
+        if (NM == 2) L[NM - 1][r] = q4k_load(t.W1 + off, g);
     }
-    stage_x<NW>(p.x, xs, bpr * 64, tid);
+    stage_finish<XF, NW * 64>(p.pro, xs, bpr * 256, sr);
     __syncthreads();
     if (!t.active) return;
 
-    float xr[64], sx_lo, sx_hi;
-    load_x_group(xs, bl, g, xr, sx_lo, sx_hi);
+    XGroup<XF> X;
+    X.load(xs, bpr * 256, bl, g);
 
 #pragma unroll
     for (int r = 0; r < R; r++) {
         float s[NM];
 #pragma unroll
         for (int m = 0; m < NM; m++) {
-            const float2 hs = wave_half_sums(q4k_group_dot<VAR>(L[m][r], g, xr, sx_lo, sx_hi));
+            const float2 hs = wave_half_sums(q4k_group_dot<XF>(L[m][r], g, X));
             s[m] = hw ? hs.y : hs.x;
         }
         const int row = row0 + r;
-        if ((lane & 31) == 0 && row < t.rows) t.y[row] = (NM == 2) ? gelu_mul_f32(s[0], s[NM - 1]) : s[0];
+        if ((lane & 31) == 0 && row < t.rows) stg_f32(t.y, row, (NM == 2) ? gelu_mul_f32(s[0], s[NM - 1]) : s[0]);
     }
 }
 
@@ -336,30 +375,30 @@ struct Q4kGeom {
 
 int waves_for(int rows, int rpw) { return (rows + rpw - 1) / rpw; }
 
-template <int R, int NW, int NM, int VAR>
+size_t lds_for(int var, int cols) { return var == kXI8 ? xs_bytes<kXI8>(cols) : xs_bytes<kXF32>(cols); }
+
+template <int R, int NW, int NM, int XF>
 int launch_inst(bool half, const MatvecParams &p, int total_waves, hipStream_t st)
 {
     const unsigned grid = (unsigned)((total_waves + NW - 1) / NW);
-    const size_t lds = (size_t)xs_floats(p.bpr * 256) * sizeof(float);
+    const size_t lds = xs_bytes<XF>(p.bpr * 256);
     if (half)
-        hipLaunchKernelGGL((q4k_gemv_half_kernel<R, NW, NM, VAR>), dim3(grid), dim3(NW * 64), lds, st, p);
+        hipLaunchKernelGGL((q4k_gemv_half_kernel<R, NW, NM, XF>), dim3(grid), dim3(NW * 64), lds, st, p);
     else if (p.bpr > 16)
-        hipLaunchKernelGGL((q4k_gemv_kernel<R, NW, NM, VAR, true>), dim3(grid), dim3(NW * 64), lds, st, p);
+        hipLaunchKernelGGL((q4k_gemv_kernel<R, NW, NM, XF, true>), dim3(grid), dim3(NW * 64), lds, st, p);
     else
-        hipLaunchKernelGGL((q4k_gemv_kernel<R, NW, NM, VAR, false>), dim3(grid), dim3(NW * 64), lds, st, p);
+        hipLaunchKernelGGL((q4k_gemv_kernel<R, NW, NM, XF, false>), dim3(grid), dim3(NW * 64), lds, st, p);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : hip_fail(e, "q4k_gemv launch");
 }
 
-template <int NM, int VAR>
+template <int NM, int XF>
 int launch_rn(const Q4kGeom &G, const MatvecParams &p, int total_waves, hipStream_t st)
 {
 #define KSH_CASE(r, w) \
-    if (G.R == r && G.NW == w) return launch_inst<r, w, NM, VAR>(G.half, p, total_waves, st);
+    if (G.R == r && G.NW == w) return launch_inst<r, w, NM, XF>(G.half, p, total_waves, st);
     KSH_CASE(1, 4) KSH_CASE(2, 4) KSH_CASE(4, 4)
-    KSH_CASE(1, 2) KSH_CASE(2, 2) KSH_CASE(4, 2)
     KSH_CASE(1, 8) KSH_CASE(2, 8) KSH_CASE(4, 8)
-    KSH_CASE(1, 1) KSH_CASE(2, 1) KSH_CASE(4, 1)
 #undef KSH_CASE
     return set_error("q4k gemv: no instance for nr0=%d nsg=%d", G.R, G.NW);
 }
@@ -367,35 +406,42 @@ int launch_rn(const Q4kGeom &G, const MatvecParams &p, int total_waves, hipStrea
 template <int NM>
 int launch_q4k(const Q4kGeom &G, const MatvecParams &p, int total_waves, hipStream_t st)
 {
-    return G.var == 2 ? launch_rn<NM, 2>(G, p, total_waves, st) : launch_rn<NM, 0>(G, p, total_waves, st);
+    return G.var == kXI8 ? launch_rn<NM, kXI8>(G, p, total_waves, st) : launch_rn<NM, kXF32>(G, p, total_waves, st);
 }
 
-// default schedule: rows per wave as high as still leaves >= 2 workgroups per
-// CU (x reuse vs. filling 256 CUs), 4 waves per workgroup.
+// default schedule: int8 dot, 8 waves per workgroup and 2 rows per wave if
+// that still gives every CU a workgroup (x staged once per 16 rows, and the
+// arithmetic that is left when the last weights arrive stays short), else
+// smaller workgroups.
 Q4kGeom pick_geom(const ksh_sched &s, int total_rows, int bpr)
 {
     Q4kGeom G;
     G.half = (bpr == 8);
-    G.var = s.vec == 2 ? 2 : 0;
-    G.NW = s.nsg ? (int)s.nsg : 4;
-    if (s.nr0) {
+    G.var = sched_is_zero(s) ? kXI8 : (s.vec == 3 ? kXI8 : kXF32);
+    if (s.nsg && s.nr0) {
+        G.NW = (int)s.nsg;
         G.R = (int)s.nr0;
-    } else {
-        G.R = 4;
-        while (G.R > 1 && total_rows / (G.NW * G.rpw()) < 512) G.R >>= 1;
+        return G;
     }
+    for (int nw : {8, 4})
+        for (int r : {2, 1}) {
+            if (s.nsg && (int)s.nsg != nw) continue;
+            if (s.nr0 && (int)s.nr0 != r) continue;
+            G.NW = nw;
+            G.R = r;
+            if (total_rows / (nw * G.rpw()) >= 256) return G;
+        }
+    G.NW = s.nsg ? (int)s.nsg : 4;
+    G.R = s.nr0 ? (int)s.nr0 : 1;
     return G;
 }
 
-bool geom_ok(const Q4kGeom &G)
-{
-    return (G.R == 1 || G.R == 2 || G.R == 4) && (G.NW == 1 || G.NW == 2 || G.NW == 4 || G.NW == 8);
-}
+bool geom_ok(const Q4kGeom &G) { return (G.R == 1 || G.R == 2 || G.R == 4) && (G.NW == 4 || G.NW == 8); }
 
 void fill_info(ksh_kernel &k, const Q4kGeom &G, int total_waves, int bpr, const char *base)
 {
     set_launch(k, (uint32_t)((total_waves + G.NW - 1) / G.NW), 1, 1, (uint32_t)G.NW * 64,
-               (uint32_t)(xs_floats(bpr * 256) * sizeof(float)));
+               (uint32_t)lds_for(G.var, bpr * 256));
     k.info.sched = k.desc.sched;
     k.info.sched.tg = (uint64_t)G.NW * 64;
     k.info.sched.nsg = (uint32_t)G.NW;
@@ -417,132 +463,131 @@ Q4kGeom geom_of(const ksh_kernel &k)
     return G;
 }
 
-int launch_matvec_q4k(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
+// The three shapes (plain / QKV / gate-up), each with an optional normalising
+// prologue.  Binding order of inputs: weight matrices, the vector, then for a
+// prologue w_norm, and with a residual w_post, res; outputs: the GEMV results,
+// then with a residual the new residual stream.
+struct Shape {
+    int n_mat;        // weight matrices bound
+    int nm;           // matrices per wave (2 for gate||up)
+    int64_t rows[3];
+    int64_t cols;
+    int prologue;     // kPlain / kRms / kAddThenRms
+    float eps;
+};
+
+Shape shape_of(const ksh_kernel_desc &d)
 {
-    const Q4kGeom G = geom_of(k);
-    MatvecParams p{};
-    p.W[0] = (const uint8_t *)a.in[0];
-    p.x = (const float *)a.in[1];
-    p.y[0] = (float *)a.out[0];
-    p.rows[0] = (int)k.desc.dims[0];
-    p.waves[0] = waves_for(p.rows[0], G.rpw());
-    p.bpr = (int)(k.desc.dims[1] / 256);
-    return launch_q4k<1>(G, p, p.waves[0], st);
+    Shape s{};
+    const int64_t *D = d.dims;
+    switch (d.kind) {
+    case KSH_MATVEC: s.n_mat = 1; s.nm = 1; s.rows[0] = D[0]; s.cols = D[1]; break;
+    case KSH_RMSNORM_MATVEC: s.n_mat = 1; s.nm = 1; s.rows[0] = D[0]; s.cols = D[1]; s.prologue = D[2] ? kAddThenRms : kRms; break;
+    case KSH_MATVEC_QKV: s.n_mat = 3; s.nm = 1; s.rows[0] = D[0]; s.rows[1] = s.rows[2] = D[1]; s.cols = D[2]; break;
+    case KSH_RMSNORM_MATVEC_QKV:
+        s.n_mat = 3; s.nm = 1; s.rows[0] = D[0]; s.rows[1] = s.rows[2] = D[1]; s.cols = D[2];
+        s.prologue = D[3] ? kAddThenRms : kRms;
+        break;
+    case KSH_MATVEC_GATE_UP_GELU: s.n_mat = 2; s.nm = 2; s.rows[0] = s.rows[1] = D[0]; s.cols = D[1]; break;
+    case KSH_RMSNORM_MATVEC_GATE_UP_GELU:
+        s.n_mat = 2; s.nm = 2; s.rows[0] = s.rows[1] = D[0]; s.cols = D[1];
+        s.prologue = D[2] ? kAddThenRms : kRms;
+        break;
+    }
+    s.eps = d.params[0];
+    return s;
 }
 
-int launch_qkv_q4k(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
+int launch_any(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
 {
     const Q4kGeom G = geom_of(k);
+    const Shape s = shape_of(k.desc);
     MatvecParams p{};
     int total = 0;
-    for (int m = 0; m < 3; m++) {
-        p.W[m] = (const uint8_t *)a.in[m];
-        p.y[m] = (float *)a.out[m];
-        p.rows[m] = (int)k.desc.dims[m == 0 ? 0 : 1];
-        p.waves[m] = waves_for(p.rows[m], G.rpw());
-        total += p.waves[m];
+    const int n_y = s.nm == 2 ? 1 : s.n_mat;
+    const uint8_t **W[3] = {&p.W0, &p.W1, &p.W2};
+    float **y[3] = {&p.y0, &p.y1, &p.y2};
+    int *rows[3] = {&p.rows0, &p.rows1, &p.rows2}, *waves[3] = {&p.waves0, &p.waves1, &p.waves2};
+    for (int m = 0; m < s.n_mat; m++) {
+        *W[m] = (const uint8_t *)a.in[m];
+        *rows[m] = (int)s.rows[m];
+        *waves[m] = waves_for(*rows[m], G.rpw());
+        if (s.nm == 1) total += *waves[m];
     }
-    p.x = (const float *)a.in[3];
-    p.bpr = (int)(k.desc.dims[2] / 256);
-    return launch_q4k<1>(G, p, total, st);
-}
-
-int launch_gate_up_q4k(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
-{
-    const Q4kGeom G = geom_of(k);
-    MatvecParams p{};
-    p.W[0] = (const uint8_t *)a.in[0];
-    p.W[1] = (const uint8_t *)a.in[1];
-    p.x = (const float *)a.in[2];
-    p.y[0] = (float *)a.out[0];
-    p.rows[0] = p.rows[1] = (int)k.desc.dims[0];
-    p.waves[0] = waves_for(p.rows[0], G.rpw());
-    p.bpr = (int)(k.desc.dims[1] / 256);
-    p.mode = 1;
-    return launch_q4k<2>(G, p, p.waves[0], st);
-}
-
-int check_cols(int64_t cols)
-{
-    if (cols <= 0 || cols % 256)
-        return set_error("Q4_K matvec: cols=%lld is not a positive multiple of 256", (long long)cols);
-    if (cols > 32768)
-        return set_error("Q4_K matvec: cols=%lld does not fit the LDS staging buffer", (long long)cols);
-    return 0;
+    for (int m = 0; m < n_y; m++) *y[m] = (float *)a.out[m];
+    if (s.nm == 2) total = p.waves0;
+    p.mode = s.nm == 2 ? 1 : 0;
+    p.bpr = (int)(s.cols / 256);
+    p.pro.kind = s.prologue;
+    p.pro.eps = s.eps;
+    p.pro.x = (const float *)a.in[s.n_mat];
+    if (s.prologue != kPlain) p.pro.w_norm = (const float *)a.in[s.n_mat + 1];
+    if (s.prologue == kAddThenRms) {
+        p.pro.w_post = (const float *)a.in[s.n_mat + 2];
+        p.pro.res = (const float *)a.in[s.n_mat + 3];
+        p.pro.x_out = (float *)a.out[n_y];
+    }
+    return s.nm == 2 ? launch_q4k<2>(G, p, total, st) : launch_q4k<1>(G, p, total, st);
 }
 
 }  // namespace
 
-int bind_matvec_q4k(ksh_kernel &k)
+int bind_matvec_q4k_family(ksh_kernel &k)
 {
-    const int64_t rows = k.desc.dims[0], cols = k.desc.dims[1];
-    if (rows <= 0 || rows > (1 << 30)) return set_error("matvec: rows=%lld", (long long)rows);
-    if (check_cols(cols)) return 1;
-    const int bpr = (int)(cols / 256);
-    const Q4kGeom G = pick_geom(k.desc.sched, (int)rows, bpr);
-    if (!geom_ok(G)) return set_error("matvec_q4k: unsupported schedule nr0=%d nsg=%d", G.R, G.NW);
-    k.info.n_inputs = 2;
-    k.info.n_outputs = 1;
-    k.in_bytes[0] = (size_t)rows * bpr * kQ4kBytes;
-    k.in_bytes[1] = (size_t)cols * 4;
-    k.out_bytes[0] = (size_t)rows * 4;
-    k.in_align[0] = 16; k.in_align[1] = 16; k.out_align[0] = 4;
-    fill_info(k, G, waves_for((int)rows, G.rpw()), bpr, "matvec");
-    k.launch = launch_matvec_q4k;
+    const Shape s = shape_of(k.desc);
+    if (!s.n_mat) return set_error("q4k gemv: kind %d", k.desc.kind);
+    if (k.desc.dtypes[0] != KSH_Q4K) return set_error("%d: only Q4_K weights are built for this kind", k.desc.kind);
+    if (k.desc.dtypes[1] != KSH_F32 && k.desc.dtypes[1] != 0)
+        return set_error("matvec: activation dtype %d is not built (f32 only)", k.desc.dtypes[1]);
+    int64_t total_rows = 0;
+    for (int m = 0; m < s.n_mat; m++) {
+        if (s.rows[m] <= 0 || s.rows[m] > (1 << 30)) return set_error("matvec: rows=%lld", (long long)s.rows[m]);
+        total_rows += s.rows[m];
+    }
+    if (s.cols <= 0 || s.cols % 256) return set_error("Q4_K matvec: cols=%lld is not a positive multiple of 256", (long long)s.cols);
+    if (s.cols > 32768) return set_error("Q4_K matvec: cols=%lld does not fit the LDS staging buffer", (long long)s.cols);
+    const int bpr = (int)(s.cols / 256);
+    const Q4kGeom G = pick_geom(k.desc.sched, (int)(s.nm == 2 ? s.rows[0] : total_rows), bpr);
+    if (lds_for(G.var, (int)s.cols) > 65536)
+        return set_error("Q4_K matvec: cols=%lld does not fit the LDS staging buffer", (long long)s.cols);
+    if (!geom_ok(G)) return set_error("matvec_q4k: unsupported schedule nr0=%d nsg=%d (nr0 in 1,2,4; nsg in 4,8)", G.R, G.NW);
+    if (s.prologue != kPlain && s.cols > (int64_t)4 * G.NW * 64 * kStageP)
+        return set_error("rmsnorm_matvec requires LOCAL staging of the vector (cols=%lld too large)", (long long)s.cols);
+    const size_t rb = (size_t)bpr * kQ4kBytes, vb = (size_t)s.cols * 4;
+    const int n_y = s.nm == 2 ? 1 : s.n_mat;
+    int ni = 0, no = 0;
+    for (int m = 0; m < s.n_mat; m++) { k.in_bytes[ni] = (size_t)s.rows[m] * rb; k.in_align[ni++] = 16; }
+    k.in_bytes[ni] = vb; k.in_align[ni++] = 16;
+    if (s.prologue != kPlain) { k.in_bytes[ni] = vb; k.in_align[ni++] = 16; }
+    if (s.prologue == kAddThenRms) {
+        k.in_bytes[ni] = vb; k.in_align[ni++] = 16;
+        k.in_bytes[ni] = vb; k.in_align[ni++] = 16;
+    }
+    for (int m = 0; m < n_y; m++) { k.out_bytes[no] = (size_t)s.rows[m] * 4; k.out_align[no++] = 4; }
+    if (s.prologue == kAddThenRms) { k.out_bytes[no] = vb; k.out_align[no++] = 16; }
+    k.info.n_inputs = ni;
+    k.info.n_outputs = no;
+    int waves = 0;
+    if (s.nm == 2) waves = waves_for((int)s.rows[0], G.rpw());
+    else for (int m = 0; m < s.n_mat; m++) waves += waves_for((int)s.rows[m], G.rpw());
+    static const char *pre[] = {"", "rms_", "addrms_"};
+    char base[48];
+    snprintf(base, sizeof(base), "%smatvec%s", pre[s.prologue], s.n_mat == 3 ? "_qkv" : s.nm == 2 ? "_gate_up_gelu" : "");
+    fill_info(k, G, waves, bpr, base);
+    k.launch = launch_any;
     return 0;
 }
 
-int bind_matvec_qkv(ksh_kernel &k)
-{
-    const int64_t qr = k.desc.dims[0], kvr = k.desc.dims[1], cols = k.desc.dims[2];
-    if (k.desc.dtypes[0] != KSH_Q4K) return set_error("matvec_qkv: only Q4_K weights are built");
-    if (qr <= 0 || kvr <= 0 || qr > (1 << 30) || kvr > (1 << 30))
-        return set_error("matvec_qkv: q_rows=%lld kv_rows=%lld", (long long)qr, (long long)kvr);
-    if (check_cols(cols)) return 1;
-    const int bpr = (int)(cols / 256);
-    const Q4kGeom G = pick_geom(k.desc.sched, (int)(qr + 2 * kvr), bpr);
-    if (!geom_ok(G)) return set_error("matvec_qkv: unsupported schedule nr0=%d nsg=%d", G.R, G.NW);
-    k.info.n_inputs = 4;
-    k.info.n_outputs = 3;
-    const size_t rb = (size_t)bpr * kQ4kBytes;
-    k.in_bytes[0] = (size_t)qr * rb; k.in_bytes[1] = k.in_bytes[2] = (size_t)kvr * rb;
-    k.in_bytes[3] = (size_t)cols * 4;
-    k.out_bytes[0] = (size_t)qr * 4; k.out_bytes[1] = k.out_bytes[2] = (size_t)kvr * 4;
-    for (int i = 0; i < 4; i++) k.in_align[i] = 16;
-    for (int i = 0; i < 3; i++) k.out_align[i] = 4;
-    fill_info(k, G, waves_for((int)qr, G.rpw()) + 2 * waves_for((int)kvr, G.rpw()), bpr, "matvec_qkv");
-    k.launch = launch_qkv_q4k;
-    return 0;
-}
-
-int bind_matvec_gate_up_gelu(ksh_kernel &k)
-{
-    const int64_t rows = k.desc.dims[0], cols = k.desc.dims[1];
-    if (k.desc.dtypes[0] != KSH_Q4K) return set_error("matvec_gate_up_gelu: only Q4_K weights are built");
-    if (rows <= 0 || rows > (1 << 30)) return set_error("matvec_gate_up_gelu: rows=%lld", (long long)rows);
-    if (check_cols(cols)) return 1;
-    const int bpr = (int)(cols / 256);
-    Q4kGeom G = pick_geom(k.desc.sched, (int)rows * 2, bpr);
-    if (!geom_ok(G)) return set_error("matvec_gate_up_gelu: unsupported schedule nr0=%d nsg=%d", G.R, G.NW);
-    k.info.n_inputs = 3;
-    k.info.n_outputs = 1;
-    const size_t rb = (size_t)bpr * kQ4kBytes;
-    k.in_bytes[0] = k.in_bytes[1] = (size_t)rows * rb;
-    k.in_bytes[2] = (size_t)cols * 4;
-    k.out_bytes[0] = (size_t)rows * 4;
-    for (int i = 0; i < 3; i++) k.in_align[i] = 16;
-    k.out_align[0] = 4;
-    fill_info(k, G, waves_for((int)rows, G.rpw()), bpr, "matvec_gate_up_gelu");
-    k.launch = launch_gate_up_q4k;
-    return 0;
-}
+int bind_matvec_q4k(ksh_kernel &k) { return bind_matvec_q4k_family(k); }
+int bind_matvec_qkv(ksh_kernel &k) { return bind_matvec_q4k_family(k); }
+int bind_matvec_gate_up_gelu(ksh_kernel &k) { return bind_matvec_q4k_family(k); }
 
 int matvec_q4k_candidates(const ksh_kernel_desc &d, ksh_sched *out, int cap)
 {
     (void)d;
     int n = 0;
-    for (uint32_t var : {0u, 2u})
-        for (uint32_t nsg : {1u, 2u, 4u, 8u})
+    for (uint32_t var : {3u, 1u})
+        for (uint32_t nsg : {4u, 8u})
             for (uint32_t nr0 : {1u, 2u, 4u}) {
                 if (n >= cap) return n;
                 ksh_sched s{};

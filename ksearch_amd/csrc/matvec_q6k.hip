@@ -238,6 +238,7 @@ int launch_matvec_q6k(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
 int bind_matvec_q6k(ksh_kernel &k)
 {
     const int64_t rows = k.desc.dims[0], cols = k.desc.dims[1];
+    if (k.desc.kind != KSH_MATVEC) return set_error("rmsnorm_matvec: Q6_K weights are not built for this kind");
     if (rows <= 0 || rows > (1 << 30)) return set_error("matvec: rows=%lld", (long long)rows);
     if (cols <= 0 || cols % 256 || cols > 8192)
         return set_error("matvec_q6k: cols=%lld is not a positive multiple of 256 up to 8192", (long long)cols);

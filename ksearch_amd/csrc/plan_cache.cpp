@@ -152,8 +152,11 @@ const char *ksh_plan_kind(const ksh_kernel_desc *d)
     case KSH_MATVEC:
         // crates/ksearch_codegen/src/lib.rs:200-205
         return d->dtypes[0] == KSH_Q4K ? "matvec_q4k" : d->dtypes[0] == KSH_Q6K ? "matvec_q6k" : nullptr;
+    case KSH_RMSNORM_MATVEC: return d->dtypes[0] == KSH_Q4K ? "rms_matvec_q4k" : d->dtypes[0] == KSH_Q6K ? "rms_matvec_q6k" : nullptr;
     case KSH_MATVEC_QKV: return "matvec_qkv_q4k";
+    case KSH_RMSNORM_MATVEC_QKV: return "rms_matvec_qkv_q4k";
     case KSH_MATVEC_GATE_UP_GELU: return "matvec_gate_up_q4k";
+    case KSH_RMSNORM_MATVEC_GATE_UP_GELU: return "rms_matvec_gate_up_q4k";
     case KSH_MATVEC_BATCH: return "mul_mm_q4k";
     case KSH_SDPA_SLOTS:
     case KSH_SDPA_MWG_PART: return "sdpa_q40";
@@ -168,8 +171,13 @@ int ksh_beam_candidates(const ksh_kernel_desc *d, ksh_sched *out, int cap)
     case KSH_MATVEC:
         if (d->dtypes[0] == KSH_Q6K) return matvec_q6k_candidates(*d, out, cap);
         return matvec_q4k_candidates(*d, out, cap);
+    case KSH_RMSNORM_MATVEC:
+        if (d->dtypes[0] == KSH_Q6K) return matvec_q6k_candidates(*d, out, cap);
+        return matvec_q4k_candidates(*d, out, cap);
     case KSH_MATVEC_QKV:
-    case KSH_MATVEC_GATE_UP_GELU: return matvec_q4k_candidates(*d, out, cap);
+    case KSH_MATVEC_GATE_UP_GELU:
+    case KSH_RMSNORM_MATVEC_QKV:
+    case KSH_RMSNORM_MATVEC_GATE_UP_GELU: return matvec_q4k_candidates(*d, out, cap);
     }
     return 0;
 }

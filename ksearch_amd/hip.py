@@ -52,6 +52,9 @@ class Kind(enum.IntEnum):           # enum ksh_kind
     SOFTCAP_ARGMAX = 16
     DEQUANT = 17
     QUANTIZE_K = 18
+    RMSNORM_MATVEC = 19
+    RMSNORM_MATVEC_QKV = 20
+    RMSNORM_MATVEC_GATE_UP_GELU = 21
 
 
 class Sched(C.Structure):           # ksh_sched: OptSchedule retargeted to gfx950
@@ -447,6 +450,27 @@ class Eng:
     def matvec_gate_up_gelu_wd(self, ctx, rows, cols, wdt, wg, wu, x, out, sched=None):
         k = self._k(ctx, Kind.MATVEC_GATE_UP_GELU, (rows, cols), (wdt, DType.F32), (), sched)
         ctx.encode_multi(k, [wg, wu, x], [out])
+
+    # rmsnorm_matvec_wd / rmsnorm_matvec_qkv_w / rmsnorm_matvec_gate_up_gelu_w (:1233-1236, gemma_prim.rs:948-961,
+    # 1121-1130).  With res/w_post given, the residual add of the previous block is folded in as well
+    # and the new residual stream comes back in x_new (which must not alias res).
+    def rmsnorm_matvec_wd(self, ctx, rows, cols, eps, wdt, x, w_norm, w, y, w_post=None, res=None, x_new=None, sched=None):
+        has_res = res is not None
+        k = self._k(ctx, Kind.RMSNORM_MATVEC, (rows, cols, int(has_res)), (wdt, DType.F32), (eps,), sched)
+        ctx.encode_multi(k, [w, x, w_norm] + ([w_post, res] if has_res else []), [y] + ([x_new] if has_res else []))
+
+    def rmsnorm_matvec_qkv_w(self, ctx, q_rows, kv_rows, cols, eps, wdt, x, w_norm, wq, wk, wv, q, k_out, v_out,
+                             w_post=None, res=None, x_new=None, sched=None):
+        has_res = res is not None
+        k = self._k(ctx, Kind.RMSNORM_MATVEC_QKV, (q_rows, kv_rows, cols, int(has_res)), (wdt, DType.F32), (eps,), sched)
+        ctx.encode_multi(k, [wq, wk, wv, x, w_norm] + ([w_post, res] if has_res else []),
+                         [q, k_out, v_out] + ([x_new] if has_res else []))
+
+    def rmsnorm_matvec_gate_up_gelu_w(self, ctx, rows, cols, eps, wdt, x, w_norm, wg, wu, out,
+                                      w_post=None, res=None, x_new=None, sched=None):
+        has_res = res is not None
+        k = self._k(ctx, Kind.RMSNORM_MATVEC_GATE_UP_GELU, (rows, cols, int(has_res)), (wdt, DType.F32), (eps,), sched)
+        ctx.encode_multi(k, [wg, wu, x, w_norm] + ([w_post, res] if has_res else []), [out] + ([x_new] if has_res else []))
 
     # :1414-1444
     def matvec_batch(self, ctx, rows, cols, batch, wdt, w, x, y, sched=None):

@@ -63,11 +63,11 @@ def test_dequant_edge_blocks(ctx, eng):
 
 
 SCHEDS_Q4K = [None] + [dict(tg=64 * w, vec=v, unroll=1, nsg=w, nr0=r, k_split=1, lds_tile=0)
-                       for v in (0, 2) for w, r in ((4, 4), (4, 1), (2, 2), (8, 2), (1, 4))]
+                       for v in (3, 1) for w, r in ((4, 4), (4, 1), (8, 2))]
 
 
 @pytest.mark.parametrize("rows,cols", [(64, 256), (128, 256), (2048, 1536), (50, 2048), (37, 4096), (33, 8192), (512, 4096)])
-@pytest.mark.parametrize("sched", SCHEDS_Q4K[:5])
+@pytest.mark.parametrize("sched", SCHEDS_Q4K)
 def test_matvec_q4k_small(ctx, eng, rows, cols, sched):
     w = synth.q4k_blocks(rows * cols // 256, seed=rows + cols)
     x = synth.normal_f32(cols, seed=7)
@@ -85,8 +85,9 @@ def test_matvec_q4k_cfg0_full_size(ctx, eng, sched):
     got = ctx.read_f32(by, rows)
     want = oracle.matvec(oracle.Q4K, w, rows, cols, x)
     assert_close(got, want, TOL, f"cfg0 {sched}")
-    # and it sits closer to the f64 truth than 1e-4, so the bar is not eaten by the GPU side alone
-    assert_close(got, oracle.matvec_f64(oracle.Q4K, w, rows, cols, x), 1e-4, "cfg0 vs f64")
+    # and it sits within 1e-5 of the f64 truth (closer than the sequential-f32 oracle itself does),
+    # for the int8-digit inner product as much as for the f32 one
+    assert_close(got, oracle.matvec_f64(oracle.Q4K, w, rows, cols, x), 1e-5, "cfg0 vs f64")
 
 
 def test_matvec_q4k_unit_vectors_recover_weights(ctx, eng):
@@ -191,3 +192,51 @@ def test_matvec_gate_up_gelu(ctx, eng, rows, cols):
     g = oracle.matvec(oracle.Q4K, wg, rows, cols, x)
     u = oracle.matvec(oracle.Q4K, wu, rows, cols, x)
     assert_close(ctx.read_f32(out, rows), oracle.gelu_mul(g, u), TOL, "gate_up_gelu")
+
+
+@pytest.mark.parametrize("sched", [None, dict(tg=256, vec=1, unroll=1, nsg=4, nr0=2, k_split=1, lds_tile=0)])
+@pytest.mark.parametrize("has_res", [False, True])
+def test_rmsnorm_matvec_prologues(ctx, eng, has_res, sched):
+    """RmsNormMatvec / RmsNormMatvecQkv / RmsNormMatvecGateUpGelu, alone and with the previous block's
+    residual add folded in, against the unfused oracle ops."""
+    n, eps = 2048, 1e-6
+    x, w_norm, w_post, res = (synth.normal_f32(n, 700 + i) for i in range(4))
+    w_norm, w_post = 1.0 + 0.1 * w_norm, 1.0 + 0.1 * w_post
+    if has_res:
+        x_new, vec = oracle.rmsnorm_add_then_rmsnorm(x, w_post, res, w_norm, eps)
+    else:
+        x_new, vec = None, oracle.rmsnorm(x, w_norm, eps)
+    bx, bwn, bwp, br = (ctx.buffer_f32(a) for a in (x, w_norm, w_post, res))
+    extra = dict(w_post=bwp, res=br) if has_res else {}
+
+    def check_xnew(b):
+        if has_res:
+            assert_close(ctx.read_f32(b, n), x_new, 1e-5, "x_new")
+            assert np.array_equal(ctx.read_f32(br, n), res)          # the old residual stream is left alone
+
+    # plain
+    rows = 2048
+    w = synth.q4k_blocks(rows * n // 256, seed=710)
+    y, xn = ctx.buffer_empty_f32(rows), ctx.buffer_empty_f32(n)
+    eng.rmsnorm_matvec_wd(ctx, rows, n, eps, DType.Q4K, bx, bwn, ctx.buffer_bytes(w), y, x_new=xn if has_res else None, sched=sched, **extra)
+    assert_close(ctx.read_f32(y, rows), oracle.matvec(oracle.Q4K, w, rows, n, vec), TOL, "rms_matvec")
+    check_xnew(xn)
+    # qkv
+    ws = [synth.q4k_blocks(r * n // 256, seed=711 + i) for i, r in enumerate((2048, 256, 256))]
+    outs = [ctx.buffer_empty_f32(r) for r in (2048, 256, 256)]
+    xn = ctx.buffer_empty_f32(n)
+    eng.rmsnorm_matvec_qkv_w(ctx, 2048, 256, n, eps, DType.Q4K, bx, bwn, *[ctx.buffer_bytes(a) for a in ws], *outs,
+                             x_new=xn if has_res else None, sched=sched, **extra)
+    for a, r, o in zip(ws, (2048, 256, 256), outs):
+        assert_close(ctx.read_f32(o, r), oracle.matvec(oracle.Q4K, a, r, n, vec), TOL, "rms_qkv")
+    check_xnew(xn)
+    # gate-up
+    rows = 8192
+    wg, wu = synth.q4k_blocks(rows * n // 256, seed=720), synth.q4k_blocks(rows * n // 256, seed=721)
+    out, xn = ctx.buffer_empty_f32(rows), ctx.buffer_empty_f32(n)
+    eng.rmsnorm_matvec_gate_up_gelu_w(ctx, rows, n, eps, DType.Q4K, bx, bwn, ctx.buffer_bytes(wg), ctx.buffer_bytes(wu), out,
+                                      x_new=xn if has_res else None, sched=sched, **extra)
+    v2 = vec * np.float32(0.05)
+    g, u = oracle.matvec(oracle.Q4K, wg, rows, n, vec), oracle.matvec(oracle.Q4K, wu, rows, n, vec)
+    assert_close(ctx.read_f32(out, rows), oracle.gelu_mul(g, u), TOL, "rms_gate_up")
+    check_xnew(xn)

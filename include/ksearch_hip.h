@@ -121,6 +121,18 @@ enum ksh_kind {
     KSH_RMSNORM_MATVEC = 19,
     KSH_RMSNORM_MATVEC_QKV = 20,
     KSH_RMSNORM_MATVEC_GATE_UP_GELU = 21,
+    /* AttendDecode: one decode step's attention in one launch.  It is the
+     * composition RmsNormPerHeadQkvQ40 (n_tok = 1, position on the device)
+     * -> SdpaMwgPart -> SdpaMwgReduce of the reference's forward_token
+     * (crates/ksearch_gemma/src/gemma_prim.rs:984-1060); the reference has no
+     * single op for it.  dims: n_q, n_kv, hd, max_seq, nwg (0 = default).
+     * params[0] = eps, params[1] = softmax scale.
+     * in: q f32[n_q*hd] (raw, before the per-head norm), q_norm f32[hd],
+     *     rope f32[max_seq, hd], k f32[n_kv*hd], k_norm f32[hd], v f32[n_kv*hd],
+     *     meta f32[4] = {tlen, start, window, pos} with start + tlen - 1 == pos
+     * out: K cache, V cache (row pos is written), tmp f32[n_q, nwg, hd+2],
+     *      out f32[n_q*hd].  Built for hd 128 / 256, up to 8 q heads per kv head. */
+    KSH_ATTEND_DECODE = 22,
     KSH_KIND_COUNT
 };
 

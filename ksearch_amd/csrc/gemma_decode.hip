@@ -11,8 +11,8 @@
 // normalisation rides in the GEMV that consumes it (RmsNormMatvecQkv,
 // RmsNormMatvecGateUpGelu with the preceding residual add folded in), so a
 // layer is
-//   [add+]rmsnorm+QKV -> per-head RMS + RoPE + KV append -> attention ->
-//   o-proj -> add+rmsnorm+gate||up+GELU -> down
+//   [add+]rmsnorm+QKV -> per-head RMS + RoPE + KV append + attention + merge
+//   (AttendDecode) -> o-proj -> add+rmsnorm+gate||up+GELU -> down
 // and the layer-closing rmsnorm_add becomes the prologue of the next layer's
 // QKV (or of the output norm).  The residual stream ping-pongs between two
 // buffers because the fused prologue may not overwrite the vector that other
@@ -75,13 +75,14 @@ struct ksh_gemma {
             *logits = nullptr, *tok = nullptr, *meta = nullptr, *rope = nullptr, *attn_tmp = nullptr,
             *history = nullptr;
     std::vector<ksh_buf *> kv_k, kv_v;
-    ksh_kernel *k_embed = nullptr, *k_qkv_first = nullptr, *k_qkv = nullptr, *k_head = nullptr, *k_sdpa = nullptr,
+    ksh_kernel *k_embed = nullptr, *k_qkv_first = nullptr, *k_qkv = nullptr, *k_head = nullptr, *k_sdpa = nullptr, *k_attend = nullptr,
                *k_oproj = nullptr, *k_add_then = nullptr, *k_gate_up = nullptr, *k_down = nullptr,
                *k_lm_head = nullptr, *k_argmax = nullptr;
     ksh_graph *g_body = nullptr, *g_full = nullptr;
     int pos = 0;
     int launches_full = 0;
     int nwg = 16;
+    int sdpa_launches = 2;
 };
 
 namespace {
@@ -139,11 +140,17 @@ int encode_token(ksh_gemma *m, bool want_logits, int &launches)
                 return 1;
             std::swap(cur, other);
         }
-        if (enc(m, m->k_head, {m->tq, L.q_norm, m->rope, m->tk, L.k_norm, m->tv, m->meta},
-                {m->tq, m->kv_k[l], m->kv_v[l]}, launches))
-            return 1;
-        if (enc(m, m->k_sdpa, {m->tq, m->kv_k[l], m->kv_v[l], m->meta}, {m->attn_tmp, m->to}, launches)) return 1;
-        launches += 1;   // the attention kind is two launches (partials, merge)
+        if (m->k_attend) {
+            if (enc(m, m->k_attend, {m->tq, L.q_norm, m->rope, m->tk, L.k_norm, m->tv, m->meta},
+                    {m->kv_k[l], m->kv_v[l], m->attn_tmp, m->to}, launches))
+                return 1;
+        } else {
+            if (enc(m, m->k_head, {m->tq, L.q_norm, m->rope, m->tk, L.k_norm, m->tv, m->meta},
+                    {m->tq, m->kv_k[l], m->kv_v[l]}, launches))
+                return 1;
+            if (enc(m, m->k_sdpa, {m->tq, m->kv_k[l], m->kv_v[l], m->meta}, {m->attn_tmp, m->to}, launches)) return 1;
+            if (m->sdpa_launches == 2) launches += 1;   // partials, then the merge
+        }
         if (enc(m, m->k_oproj, {L.wo, m->to}, {m->y}, launches)) return 1;
         if (enc(m, m->k_gate_up, {L.wgate, L.wup, m->y, L.ffn_norm, L.post_attn_norm, cur}, {m->ff, other}, launches)) return 1;
         std::swap(cur, other);
@@ -258,8 +265,6 @@ int ksh_gemma_create(ksh_ctx *ctx, const ksh_gemma_cfg *cfg, const ksh_gemma_lay
     if (get(g, KSH_COPY_SCALE_INDEXED, {c.hidden, c.vocab}, {KSH_Q6K}, {embed_scale}, &g->k_embed) ||
         get(g, KSH_RMSNORM_MATVEC_QKV, {qd, kvd, c.hidden, 0}, {KSH_Q4K, KSH_F32}, {c.eps}, &g->k_qkv_first) ||
         get(g, KSH_RMSNORM_MATVEC_QKV, {qd, kvd, c.hidden, 1}, {KSH_Q4K, KSH_F32}, {c.eps}, &g->k_qkv) ||
-        get(g, KSH_RMSNORM_PER_HEAD_QKV_Q40, {c.n_q, c.n_kv, c.hd, c.max_seq}, {}, {c.eps}, &g->k_head) ||
-        get(g, KSH_SDPA_SLOTS, {c.n_q, c.n_kv, c.hd, c.max_seq, 1, g->nwg}, {KSH_Q40, KSH_F32}, {c.attn_scale}, &g->k_sdpa) ||
         get(g, KSH_MATVEC, {c.hidden, qd}, {KSH_Q4K, KSH_F32}, {}, &g->k_oproj) ||
         get(g, KSH_RMSNORM_ADD_THEN_RMSNORM, {c.hidden}, {}, {c.eps}, &g->k_add_then) ||
         get(g, KSH_RMSNORM_MATVEC_GATE_UP_GELU, {c.ffn, c.hidden, 1}, {KSH_Q4K, KSH_F32}, {c.eps}, &g->k_gate_up) ||
@@ -267,6 +272,17 @@ int ksh_gemma_create(ksh_ctx *ctx, const ksh_gemma_cfg *cfg, const ksh_gemma_lay
         get(g, KSH_MATVEC, {c.vocab, c.hidden}, {KSH_Q6K, KSH_F32}, {}, &g->k_lm_head) ||
         get(g, KSH_SOFTCAP_ARGMAX, {c.vocab}, {}, {c.softcap}, &g->k_argmax))
         return 1;
+    // per-head norm + RoPE + KV append + attention + merge: one launch where the fused kind is built for the
+    // shape, the three reference ops otherwise
+    if (sdpa_lanes_supports(c.n_q, c.n_kv, c.hd)) {
+        if (get(g, KSH_ATTEND_DECODE, {c.n_q, c.n_kv, c.hd, c.max_seq, g->nwg}, {KSH_Q40, KSH_F32}, {c.eps, c.attn_scale},
+                &g->k_attend))
+            return 1;
+    } else {
+        if (get(g, KSH_RMSNORM_PER_HEAD_QKV_Q40, {c.n_q, c.n_kv, c.hd, c.max_seq}, {}, {c.eps}, &g->k_head) ||
+            get(g, KSH_SDPA_SLOTS, {c.n_q, c.n_kv, c.hd, c.max_seq, 1, g->nwg}, {KSH_Q40, KSH_F32}, {c.attn_scale}, &g->k_sdpa))
+            return 1;
+    }
     if (ksh_gemma_reset(g)) return 1;
     *out = m.release();
     return 0;

@@ -13,6 +13,7 @@
 // round exactly like the unfused expressions they restate; the Q4_0 codes that
 // come out of the pack are integer functions of those values.
 #include "ksh_device.hpp"
+#include "q40_pack.hpp"
 #include "ksh_internal.hpp"
 
 namespace ksh {
@@ -79,34 +80,6 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_add_then_rmsnorm_kernel(
     ss2 = block_sum_256(ss2, red);
     const float inv2 = 1.0f / sqrtf(ss2 / (float)n + eps);
     for (int i = threadIdx.x; i < n; i += kNormThreads) out_x2[i] = mid[i] * inv2 * w_ffn[i];
-}
-
-// ksearch_pack_q40_th for one 32-value block held by 32 consecutive lanes of
-// a wave (lane l of the group holds element l).  Values pass through a half
-// round trip first; scale = max|v|/7 (1 if all zero); code = clamp(round(v/scale)+8).
-// `group_base` is the first lane of the group.  Lanes 0..15 of the group store.
-__device__ __forceinline__ void pack_q40_group(float v, int l, uint8_t *blk, bool store)
-{
-    v = half_bits_to_f32(f32_to_half_bits(v));
-    float m = fabsf(v);
-    // max over the 32 lanes of the group: row of 16 via DPP, then the neighbour row
-    m = fmaxf(m, dpp_f32<0xB1>(m));
-    m = fmaxf(m, dpp_f32<0x4E>(m));
-    m = fmaxf(m, dpp_f32<0x141>(m));
-    m = fmaxf(m, dpp_f32<0x140>(m));
-    m = fmaxf(m, __shfl_xor(m, 16, 64));
-    const float scale = m > 0.0f ? m / 7.0f : 1.0f;
-    const float inv = 1.0f / scale;
-    int q = (int)roundf(v * inv) + 8;
-    q = min(15, max(0, q));
-    const int qhi = __shfl_down(q, 16, 64);    // element l+16's code, for l < 16
-    if (!store) return;
-    if (l == 0) {
-        const uint32_t h = f32_to_half_bits(scale);
-        blk[0] = (uint8_t)(h & 0xFF);
-        blk[1] = (uint8_t)(h >> 8);
-    }
-    if (l < 16) blk[2 + l] = (uint8_t)(q | (qhi << 4));
 }
 
 // QuantizeQ40: one 32-lane group per block of 32 source values

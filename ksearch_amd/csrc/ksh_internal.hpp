@@ -98,7 +98,10 @@ int bind_matvec_batch(ksh_kernel &k);
 int bind_dequant(ksh_kernel &k);
 int bind_quantize_k(ksh_kernel &k);
 int bind_quantize_q40(ksh_kernel &k);
-int bind_sdpa(ksh_kernel &k);          // NAIVE, MWG_PART, MWG_REDUCE, SLOTS
+int bind_sdpa(ksh_kernel &k);
+bool sdpa_lanes_supports(int64_t n_q, int64_t n_kv, int64_t hd);
+int bind_sdpa_lanes(ksh_kernel &k, int nwg, int n_slots);
+int bind_attend_decode(ksh_kernel &k);          // NAIVE, MWG_PART, MWG_REDUCE, SLOTS
 int bind_rmsnorm(ksh_kernel &k);       // RMSNORM, RMSNORM_ADD_THEN_RMSNORM
 int bind_per_head_qkv_q40(ksh_kernel &k);
 int bind_glue(ksh_kernel &k);          // COPY_SCALE_INDEXED, GELU_MUL, COPY_SLICE

@@ -160,6 +160,7 @@ const char *ksh_plan_kind(const ksh_kernel_desc *d)
     case KSH_MATVEC_BATCH: return "mul_mm_q4k";
     case KSH_SDPA_SLOTS:
     case KSH_SDPA_MWG_PART: return "sdpa_q40";
+    case KSH_ATTEND_DECODE: return "attend_decode_q40";
     }
     return nullptr;
 }

@@ -317,6 +317,9 @@ int bind_sdpa(ksh_kernel &k)
     if (check_shape("sdpa", n_q, n_kv, hd, max_t)) return 1;
     const size_t kvb = (size_t)max_t * n_kv * (hd / 32) * 18;
     const uint32_t lds = (uint32_t)part_lds_bytes((int)(n_q / n_kv), (int)hd);
+    // the register form takes the shapes it is built for; sched.vec = 1 asks for the tile form
+    const bool lanes = sdpa_lanes_supports(n_q, n_kv, hd) && k.desc.sched.vec != 1;
+    int lanes_nwg = 1, lanes_slots = 1;
     switch (k.desc.kind) {
     case KSH_SDPA_NAIVE:
         k.info.n_inputs = 4;
@@ -337,12 +340,21 @@ int bind_sdpa(ksh_kernel &k)
         set_launch(k, (uint32_t)nwg, (uint32_t)n_kv, 1, kThreads, lds);
         set_name(k, "sdpa_mwg_part_hd%d_nwg%d", (int)hd, (int)nwg);
         k.launch = launch_mwg_part;
+        lanes_nwg = (int)nwg;
         break;
     }
     case KSH_SDPA_SLOTS: {
         const int64_t n_slots = d[4];
         int64_t nwg = d[5];
         if (n_slots <= 0 || n_slots > 65535) return set_error("sdpa_slots: n_slots=%lld", (long long)n_slots);
+        if (nwg == 0 && lanes) {
+            // two workgroups per CU, at least 64 rows each, and few enough partials for one workgroup to fold
+            nwg = (512 + n_slots * n_kv - 1) / (n_slots * n_kv);
+            const int64_t cap = (max_t + 63) / 64;
+            if (nwg > cap) nwg = cap;
+            if (nwg > 64) nwg = 64;
+            if (nwg < 1) nwg = 1;
+        }
         if (nwg == 0) {
             // enough partitions to put ~4 workgroups on each of the 256 CUs, rows permitting
             nwg = (1024 + n_slots * n_kv - 1) / (n_slots * n_kv);
@@ -365,11 +377,20 @@ int bind_sdpa(ksh_kernel &k)
         k.info.sched.k_split = (uint32_t)nwg;
         k.info.sched.lds_tile = kTile;
         k.launch = launch_slots;
+        lanes_nwg = (int)nwg;
+        lanes_slots = (int)n_slots;
         break;
     }
     default: return set_error("bind_sdpa: kind %d", k.desc.kind);
     }
     k.in_align[0] = 4; k.in_align[1] = k.in_align[2] = 2; k.in_align[3] = 4; k.out_align[0] = 4;
+    if (lanes) {
+        k.in_align[0] = 16;
+        if (bind_sdpa_lanes(k, lanes_nwg, lanes_slots)) return 1;
+        char name[64];
+        snprintf(name, sizeof(name), "%s", k.info.name);
+        set_name(k, "%s_regs_w%d", name, (int)k.info.sched.nsg);
+    }
     return 0;
 }
 

@@ -1,0 +1,713 @@
+// Decode attention over a Q4_0 KV cache, register form, for head sizes 128 and
+// 256 with up to 8 q heads per kv head; optionally with the per-head RMSNorm +
+// RoPE + Q4_0 KV append in front of it and always with the split-KV merge
+// behind it, so that a decode step's attention is one launch.
+//
+// Same semantics as the tile form next door (which stays for the other
+// shapes): lower_sdpa_online / lower_sdpa_mwg_part / lower_sdpa_mwg_reduce
+// (crates/ksearch_codegen/src/lower.rs:4897-5359, 5367-5894, 5897-6087) and,
+// for the fused prologue, RmsNormPerHeadQkvQ40 (lower.rs:4080-4440,
+// gemma_prim.rs:984-1008).
+//
+// Layout of the work:
+//   - a KV row of hd elements is hd/8 dwords of nibbles; hd/8 consecutive
+//     lanes take one row, lane j owning dword j: Q4_0 block b = j/4, bytes
+//     4w..4w+3 (w = j%4), i.e. elements 32b+4w+{0..3} (low nibbles) and
+//     32b+16+4w+{0..3} (high nibbles).  A wave therefore works on 64/(hd/8)
+//     rows at once, and the four lanes of a DPP quad share a block and its
+//     scale;
+//   - every lane keeps the matching 8 elements of q for all heads in registers
+//     (pre-multiplied by the softmax scale) and its 8 elements of the output
+//     accumulator for all heads;
+//   - scores: 8 FMAs per head on the lane's nibbles, times the block scale,
+//     then a transposing butterfly (two quad steps that halve the number of
+//     heads a lane carries, then row rotations and one row swap) leaves every
+//     lane with the finished scores of GP/4 heads of its row;
+//   - softmax bookkeeping is lane-local: rows are taken four at a time, their
+//     maximum and the rescale factor are per lane, and the probabilities are
+//     handed to the other three lanes of the quad with quad broadcasts;
+//   - P.V: p*scale per head, then 8 FMAs per head; the -8 offset of the codes
+//     is applied once at the end through the running sum of p*scale;
+//   - every row group ends with its own (m, l, O); the workgroup folds them
+//     through LDS, writes one partial per partition, and the last partition
+//     to arrive (a device-scope counter) folds the partials into the output.
+#include "ksh_device.hpp"
+#include "q40_pack.hpp"
+#include "ksh_internal.hpp"
+
+namespace ksh {
+namespace {
+
+// phase timestamps for a timing probe that includes this file; nothing in the library build
+#ifdef KSH_TRACE
+__device__ unsigned long long ksh_trace_buf[64 * 16];
+#define KSH_MARK(n) do { if ((threadIdx.x & 63) == 0 && threadIdx.x < 64) ksh_trace_buf[blockIdx.x * 16 + (n)] = wall_clock64(); } while (0)
+#else
+#define KSH_MARK(n) do { } while (0)
+#endif
+
+enum { kModeDirect = 0, kModePart = 1, kModeMerge = 2 };
+constexpr int kRT = 4;   // row steps per softmax update
+
+struct LaneParams {
+    const float *q;          // [n_slots][n_q*hd]; fused: the raw q of the QKV GEMV
+    const uint8_t *k, *v;    // [n_slots][max_t*n_kv*row_bytes]
+    const float *meta;       // [n_slots][meta_stride]: tlen, start, window(, pos)
+    float *tmp;              // [n_slots][n_q][nwg][hd+2]
+    float *out;              // [n_slots][n_q*hd]
+    uint32_t *counters;      // [n_slots*n_kv], zero between launches
+    const float *qw, *kw, *rope, *k_raw, *v_raw;   // fused prologue
+    uint8_t *k_w, *v_w;                            // the caches again, writable
+    float eps, scale;
+    int n_q, n_kv, max_t, nwg, meta_stride, groups, mode, fused;
+};
+
+__device__ __forceinline__ uint32_t ld32_a2(const uint8_t *p)
+{
+    uint32_t v;
+    __builtin_memcpy(&v, p, 4);
+    return v;
+}
+__device__ __forceinline__ uint32_t ld16_a2(const uint8_t *p)
+{
+    uint16_t v;
+    __builtin_memcpy(&v, p, 2);
+    return v;
+}
+
+__device__ __forceinline__ float xor16_sum(float x)
+{
+    // rows 1 and 3 of the first copy trade places with rows 0 and 2 of the second
+    const auto r = __builtin_amdgcn_permlane16_swap(as_u32(x), as_u32(x), false, false);
+    return as_f32(r[0]) + as_f32(r[1]);
+}
+
+struct RowRegs {
+    uint32_t kd, ks, vd, vs;
+};
+
+template <int GP>
+struct State {
+    float m[GP / 4], l[GP / 4];
+    float O[GP][8], S[GP];
+};
+
+// the head whose finished score ends up in slot i of the lane at quad position c
+template <int GP>
+__device__ __forceinline__ int head_of(int c, int i)
+{
+    return (c & 1) * (GP / 2) + ((c >> 1) & 1) * (GP / 4) + i;
+}
+
+// per-lane partial dots of GP heads -> finished dots of GP/4 heads, in every lane of the row group
+template <int HD, int GP>
+__device__ __forceinline__ void reduce_heads(const float (&v)[GP], int c, float (&out)[GP / 4])
+{
+    const bool b0 = c & 1, b1 = c & 2;
+    float a[GP / 2];
+#pragma unroll
+    for (int i = 0; i < GP / 2; i++) {
+        const float keep = b0 ? v[i + GP / 2] : v[i], send = b0 ? v[i] : v[i + GP / 2];
+        a[i] = keep + dpp_f32<0xB1>(send);   // quad_perm [1,0,3,2]
+    }
+#pragma unroll
+    for (int i = 0; i < GP / 4; i++) {
+        const float keep = b1 ? a[i + GP / 4] : a[i], send = b1 ? a[i] : a[i + GP / 4];
+        float x = keep + dpp_f32<0x4E>(send);   // quad_perm [2,3,0,1]
+        x += dpp_f32<0x124>(x);                 // row_ror:4
+        x += dpp_f32<0x128>(x);                 // row_ror:8
+        if (HD == 256) x = xor16_sum(x);
+        out[i] = x;
+    }
+}
+
+// one lane's GP/4 values -> all GP, through the quad
+template <int GP>
+__device__ __forceinline__ void quad_gather(const float (&x)[GP / 4], float (&all)[GP])
+{
+#pragma unroll
+    for (int i = 0; i < GP / 4; i++) {
+        all[i] = dpp_f32<0x00>(x[i]);
+        all[GP / 2 + i] = dpp_f32<0x55>(x[i]);
+        all[GP / 4 + i] = dpp_f32<0xAA>(x[i]);
+        all[GP / 2 + GP / 4 + i] = dpp_f32<0xFF>(x[i]);
+    }
+}
+
+__device__ __forceinline__ void unpack8(uint32_t d, float (&n)[8])
+{
+    const uint32_t lo = d & 0x0F0F0F0Fu, hi = (d >> 4) & 0x0F0F0F0Fu;
+    n[0] = ubyte_f32<0>(lo); n[1] = ubyte_f32<1>(lo); n[2] = ubyte_f32<2>(lo); n[3] = ubyte_f32<3>(lo);
+    n[4] = ubyte_f32<0>(hi); n[5] = ubyte_f32<1>(hi); n[6] = ubyte_f32<2>(hi); n[7] = ubyte_f32<3>(hi);
+}
+
+// NR row steps: scores, one online-softmax update, P.V
+template <int HD, int GP, int NR>
+__device__ __forceinline__ void process_rows(const RowRegs (&r)[NR], const bool (&valid)[NR], const bool (&live)[NR],
+                                             const float (&qv)[GP][8], const float (&Sq)[GP], State<GP> &st, int c)
+{
+    // valid: this lane's row exists; live: some row of this wave's step exists (wave-uniform: dead steps are skipped)
+    constexpr int HPL = GP / 4;
+    float s[NR][HPL];
+#pragma unroll
+    for (int t = 0; t < NR; t++) {
+#pragma unroll
+        for (int i = 0; i < HPL; i++) s[t][i] = -INFINITY;
+        if (!live[t]) continue;
+        float n[8], part[GP];
+        unpack8(r[t].kd, n);
+        const float ks = half_bits_to_f32(r[t].ks);
+#pragma unroll
+        for (int h = 0; h < GP; h++) {
+            float acc = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) acc = fmaf(n[e], qv[h][e], acc);
+            part[h] = ks * fmaf(-8.f, Sq[h], acc);
+        }
+        float fin[HPL];
+        reduce_heads<HD, GP>(part, c, fin);
+#pragma unroll
+        for (int i = 0; i < HPL; i++) s[t][i] = valid[t] ? fin[i] : -INFINITY;
+    }
+    float alpha[HPL], pr[NR][HPL];
+#pragma unroll
+    for (int i = 0; i < HPL; i++) {
+        float mt = s[0][i];
+#pragma unroll
+        for (int t = 1; t < NR; t++) mt = fmaxf(mt, s[t][i]);
+        const float m2 = fmaxf(st.m[i], mt);
+        alpha[i] = __expf(st.m[i] - m2);
+        float ls = 0.f;
+#pragma unroll
+        for (int t = 0; t < NR; t++) {
+            pr[t][i] = __expf(s[t][i] - m2);
+            ls += pr[t][i];
+        }
+        st.l[i] = fmaf(st.l[i], alpha[i], ls);
+        st.m[i] = m2;
+    }
+    float aall[GP];
+    quad_gather<GP>(alpha, aall);
+#pragma unroll
+    for (int h = 0; h < GP; h++) {
+        st.S[h] *= aall[h];
+#pragma unroll
+        for (int e = 0; e < 8; e++) st.O[h][e] *= aall[h];
+    }
+#pragma unroll
+    for (int t = 0; t < NR; t++) {
+        if (!live[t]) continue;
+        float n[8], pall[GP];
+        unpack8(r[t].vd, n);
+        const float vs = half_bits_to_f32(r[t].vs);
+        quad_gather<GP>(pr[t], pall);
+#pragma unroll
+        for (int h = 0; h < GP; h++) {
+            const float pd = pall[h] * vs;
+            st.S[h] += pd;
+#pragma unroll
+            for (int e = 0; e < 8; e++) st.O[h][e] = fmaf(pd, n[e], st.O[h][e]);
+        }
+    }
+}
+
+// Device-scope traffic between workgroups that may sit on different XCDs (each
+// with its own L2): the partials are written and read with agent-scope atomic
+// accesses, which go through to the memory side instead of staying in the
+// writer's L2, so that the hand-over needs no L2 write-back / invalidate
+// (a full __threadfence() costs about a microsecond per workgroup here, and
+// they serialise).
+__device__ __forceinline__ void st_agent(float *p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ float ld_agent(const float *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+
+// One wave computes, for one head, the log-sum-exp weights of n partial states
+// whose (m, l) pairs sit `stride` floats apart: w[i] = exp(m_i - M), and
+// (M, L = sum w_i l_i) into ML.  Lane-parallel, so no chain of LDS round trips.
+__device__ __forceinline__ void merge_weights(const float *ml, int stride, int n, float *w, float *ML, int lane)
+{
+    float m = -1.0e30f;
+    for (int i = lane; i < n; i += 64) m = fmaxf(m, ml[i * stride]);
+    const float M = wave_max(m);
+    float ls = 0.f;
+    for (int i = lane; i < n; i += 64) {
+        const float wt = __expf(ml[i * stride] - M);
+        w[i] = wt;
+        ls = fmaf(wt, ml[i * stride + 1], ls);
+    }
+    const float L = wave_sum(ls);
+    if (lane == 0) { ML[0] = M; ML[1] = L; }
+}
+
+// RMSNorm (optionally weighted), optional RoPE, of one head already in
+// registers as element lane + 64*j
+template <int HD>
+__device__ __forceinline__ void norm_rope_regs(const float (&xv)[HD / 64], const float *wv, const float *cs, const float *sn,
+                                               float eps, float (&ro)[HD / 64])
+{
+    constexpr int PER = HD / 64;
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < PER; j++) ss += xv[j] * xv[j];
+    ss = wave_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / (float)HD + eps);
+    float nv[PER];
+#pragma unroll
+    for (int j = 0; j < PER; j++) nv[j] = wv ? xv[j] * inv * wv[j] : xv[j] * inv;
+    if (!cs) {
+#pragma unroll
+        for (int j = 0; j < PER; j++) ro[j] = nv[j];
+        return;
+    }
+#pragma unroll
+    for (int j = 0; j < PER / 2; j++) {
+        const float u = nv[j], vv = nv[j + PER / 2];
+        ro[j] = u * cs[j] - vv * sn[j];
+        ro[j + PER / 2] = u * sn[j] + vv * cs[j];
+    }
+}
+
+// grid = (nwg, n_kv, n_slots)
+template <int HD, int GP, int NW>
+__global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
+{
+    constexpr int LPR = HD / 8, RPS = 64 / LPR, HPL = GP / 4, NSLOT = NW * RPS, NT = NW * 64;
+    constexpr int SLOTF = GP * HD + 2 * GP;   // floats of one row group's state
+    constexpr int ROWB = HD / 32 * 18;
+    extern __shared__ __attribute__((aligned(16))) float smem[];
+    float *qs = smem;                            // [GP][HD]            fused prologue only
+    float *slots = qs + GP * HD;                 // [NSLOT][SLOTF]      later [groups][nwg] merge weights
+    float *wts = slots + NSLOT * SLOTF;          // [GP][NSLOT]
+    float *mlh = wts + GP * NSLOT;               // [GP][2]
+    uint8_t *newrow = reinterpret_cast<uint8_t *>(mlh + 2 * GP);   // K row, V row of the appended position
+    __shared__ int last_flag;
+
+    KSH_MARK(0);
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int j = lane % LPR, sub = lane / LPR, b = j >> 2, w = j & 3, c = w;
+    const int part = blockIdx.x, kvh = blockIdx.y, slot = blockIdx.z;
+    const int groups = p.groups;
+
+    const float *meta = p.meta + (size_t)slot * p.meta_stride;
+    const int tlen = (int)meta[0], start = (int)meta[1];
+    const int chunk = (tlen + p.nwg - 1) / p.nwg;
+    const int p0 = part * chunk;
+    int p1 = min(p0 + chunk, tlen);
+
+    const size_t slot_bytes = (size_t)p.max_t * p.n_kv * ROWB;
+    const uint8_t *kbase = p.k + (size_t)slot * slot_bytes + (size_t)kvh * ROWB + 18 * b;
+    const uint8_t *vbase = p.v + (size_t)slot * slot_bytes + (size_t)kvh * ROWB + 18 * b;
+    const size_t row_stride = (size_t)p.n_kv * ROWB;
+    const float *qg = p.q + ((size_t)slot * p.n_q + (size_t)kvh * groups) * HD;
+
+    auto load_row = [&](int t) {
+        RowRegs r;
+        const size_t off = (size_t)(start + t) * row_stride;
+        r.kd = ld32_a2(kbase + off + 2 + 4 * w);
+        r.ks = ld16_a2(kbase + off);
+        r.vd = ld32_a2(vbase + off + 2 + 4 * w);
+        r.vs = ld16_a2(vbase + off);
+        return r;
+    };
+
+    // the partition's first rows are requested before anything else is worked on
+    const bool owner = p.fused && part == (tlen - 1) / chunk;
+    if (owner) p1 = min(p1, tlen - 1);   // the row this step appends is attended from LDS, at the end
+    constexpr int TILE = NW * RPS * kRT;
+    RowRegs cur[kRT], nxt[kRT];
+    {
+        const int last = max(p1 - 1, p0 < tlen ? p0 : 0);   // an empty partition still loads (a valid row) and drops it
+#pragma unroll
+        for (int t = 0; t < kRT; t++) cur[t] = load_row(min(p0 + (t * NW + wave) * RPS + sub, last));
+    }
+
+    KSH_MARK(1);
+    // ---- q into registers (and, fused, the new K/V row into the cache) -------
+    float qv[GP][8], Sq[GP];
+    if (p.fused) {
+        const int pos = min(max((int)meta[3], 0), p.max_t - 1);
+        const float *rope = p.rope + (size_t)pos * HD;
+        // head tasks: q heads 0..groups-1, then (owner only) K and V; a wave takes
+        // tasks wave, wave+NW, ... and issues all their loads before the first sum
+        constexpr int PER = HD / 64, MAXT = GP / NW + 1;
+        const int ntask = groups + (owner ? 2 : 0);
+        float xv[MAXT][PER], wq[PER], wk[PER], cs[PER / 2], sn[PER / 2];
+#pragma unroll
+        for (int t = 0; t < MAXT; t++) {
+            const int task = wave + t * NW;
+            const float *src = task < groups ? qg + (size_t)task * HD
+                                             : (task == groups ? p.k_raw : p.v_raw) + (size_t)kvh * HD;
+#pragma unroll
+            for (int jj = 0; jj < PER; jj++) xv[t][jj] = task < ntask ? src[lane + 64 * jj] : 0.f;
+        }
+#pragma unroll
+        for (int jj = 0; jj < PER; jj++) {
+            wq[jj] = p.qw[lane + 64 * jj];
+            wk[jj] = p.kw[lane + 64 * jj];
+        }
+#pragma unroll
+        for (int jj = 0; jj < PER / 2; jj++) {
+            cs[jj] = rope[lane + 64 * jj];
+            sn[jj] = rope[HD / 2 + lane + 64 * jj];
+        }
+#pragma unroll
+        for (int t = 0; t < MAXT; t++) {
+            const int task = wave + t * NW;
+            if (task >= ntask) continue;
+            float ro[PER];
+            if (task < groups) {
+                norm_rope_regs<HD>(xv[t], wq, cs, sn, p.eps, ro);
+#pragma unroll
+                for (int jj = 0; jj < PER; jj++) qs[task * HD + lane + 64 * jj] = ro[jj] * p.scale;
+            } else {
+                const bool is_k = task == groups;
+                if (is_k) norm_rope_regs<HD>(xv[t], wk, cs, sn, p.eps, ro);
+                else norm_rope_regs<HD>(xv[t], nullptr, nullptr, nullptr, p.eps, ro);
+                uint8_t *dst = newrow + (is_k ? 0 : ROWB);
+#pragma unroll
+                for (int jj = 0; jj < PER; jj++) pack_q40_group(ro[jj], lane & 31, dst + (2 * jj + (lane >> 5)) * 18, true);
+            }
+        }
+        __syncthreads();
+        if (owner) {
+            // the appended row goes to the cache; this workgroup attends it from LDS
+            const size_t off = (size_t)slot * slot_bytes + ((size_t)pos * p.n_kv + kvh) * ROWB;
+            if (tid < ROWB / 2)
+                reinterpret_cast<uint16_t *>(p.k_w + off)[tid] = reinterpret_cast<const uint16_t *>(newrow)[tid];
+            else if (tid < ROWB)
+                reinterpret_cast<uint16_t *>(p.v_w + off)[tid - ROWB / 2] =
+                    reinterpret_cast<const uint16_t *>(newrow + ROWB)[tid - ROWB / 2];
+        }
+#pragma unroll
+        for (int h = 0; h < GP; h++) {
+            const float4 a = h < groups ? *reinterpret_cast<const float4 *>(qs + h * HD + 32 * b + 4 * w) : make_float4(0.f, 0.f, 0.f, 0.f);
+            const float4 d = h < groups ? *reinterpret_cast<const float4 *>(qs + h * HD + 32 * b + 16 + 4 * w) : make_float4(0.f, 0.f, 0.f, 0.f);
+            qv[h][0] = a.x; qv[h][1] = a.y; qv[h][2] = a.z; qv[h][3] = a.w;
+            qv[h][4] = d.x; qv[h][5] = d.y; qv[h][6] = d.z; qv[h][7] = d.w;
+        }
+    } else {
+#pragma unroll
+        for (int h = 0; h < GP; h++) {
+            const float *qh = qg + (size_t)min(h, groups - 1) * HD + 32 * b + 4 * w;
+            const float4 a = *reinterpret_cast<const float4 *>(qh), d = *reinterpret_cast<const float4 *>(qh + 16);
+            const float sc = h < groups ? p.scale : 0.f;
+            qv[h][0] = a.x * sc; qv[h][1] = a.y * sc; qv[h][2] = a.z * sc; qv[h][3] = a.w * sc;
+            qv[h][4] = d.x * sc; qv[h][5] = d.y * sc; qv[h][6] = d.z * sc; qv[h][7] = d.w * sc;
+        }
+    }
+#pragma unroll
+    for (int h = 0; h < GP; h++)
+        Sq[h] = ((qv[h][0] + qv[h][1]) + (qv[h][2] + qv[h][3])) + ((qv[h][4] + qv[h][5]) + (qv[h][6] + qv[h][7]));
+
+    State<GP> st;
+#pragma unroll
+    for (int i = 0; i < HPL; i++) { st.m[i] = -1.0e30f; st.l[i] = 0.f; }
+#pragma unroll
+    for (int h = 0; h < GP; h++) {
+        st.S[h] = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; e++) st.O[h][e] = 0.f;
+    }
+
+    KSH_MARK(2);
+    // ---- the partition's rows: kRT steps of RPS rows per wave at a time -----
+    if (p0 < p1) {
+        for (int base = p0; base < p1; base += TILE) {
+            bool valid[kRT], live[kRT];
+#pragma unroll
+            for (int t = 0; t < kRT; t++) {
+                const int row = base + (t * NW + wave) * RPS + sub;
+                valid[t] = row < p1;
+                live[t] = base + (t * NW + wave) * RPS < p1;
+                nxt[t] = load_row(min(row + TILE, p1 - 1));   // unconditional: keeps the wait counts exact
+            }
+            process_rows<HD, GP, kRT>(cur, valid, live, qv, Sq, st, c);
+#pragma unroll
+            for (int t = 0; t < kRT; t++) cur[t] = nxt[t];
+        }
+    }
+    if (p.fused && owner) {
+        RowRegs r[1];
+        const uint16_t *kr = reinterpret_cast<const uint16_t *>(newrow + 18 * b);
+        const uint16_t *vr = reinterpret_cast<const uint16_t *>(newrow + ROWB + 18 * b);
+        r[0].ks = kr[0];
+        r[0].kd = (uint32_t)kr[1 + 2 * w] | ((uint32_t)kr[2 + 2 * w] << 16);
+        r[0].vs = vr[0];
+        r[0].vd = (uint32_t)vr[1 + 2 * w] | ((uint32_t)vr[2 + 2 * w] << 16);
+        const bool valid[1] = {wave == 0 && sub == 0}, live[1] = {wave == 0};
+        process_rows<HD, GP, 1>(r, valid, live, qv, Sq, st, c);
+    }
+
+    KSH_MARK(3);
+    // ---- fold the row groups of this workgroup ------------------------------
+    {
+        float *my = slots + (wave * RPS + sub) * SLOTF;
+        if (j < 4) {
+#pragma unroll
+            for (int i = 0; i < HPL; i++) {
+                const int h = head_of<GP>(c, i);
+                my[2 * h] = st.m[i];
+                my[2 * h + 1] = st.l[i];
+            }
+        }
+#pragma unroll
+        for (int h = 0; h < GP; h++) {
+            const float o8 = 8.f * st.S[h];
+            float *o = my + 2 * GP + h * HD + 32 * b + 4 * w;
+            *reinterpret_cast<float4 *>(o) = make_float4(st.O[h][0] - o8, st.O[h][1] - o8, st.O[h][2] - o8, st.O[h][3] - o8);
+            *reinterpret_cast<float4 *>(o + 16) = make_float4(st.O[h][4] - o8, st.O[h][5] - o8, st.O[h][6] - o8, st.O[h][7] - o8);
+        }
+    }
+    __syncthreads();
+    KSH_MARK(4);
+    for (int h = wave; h < groups; h += NW) merge_weights(slots + 2 * h, SLOTF, NSLOT, wts + h * NSLOT, mlh + 2 * h, lane);
+    __syncthreads();
+    {
+        // fully unrolled: one wave per SIMD has nothing to hide an LDS round trip behind, so all reads go out first
+        constexpr int OBW = GP * HD / NT;
+        float accw[OBW];
+#pragma unroll
+        for (int ob = 0; ob < OBW; ob++) {
+            const int o = min(tid + ob * NT, groups * HD - 1), h = o / HD, d = o % HD;
+            accw[ob] = 0.f;
+#pragma unroll
+            for (int s = 0; s < NSLOT; s++) accw[ob] = fmaf(wts[h * NSLOT + s], slots[s * SLOTF + 2 * GP + h * HD + d], accw[ob]);
+        }
+#pragma unroll
+        for (int ob = 0; ob < OBW; ob++) {
+            const int o = tid + ob * NT;
+            if (o >= groups * HD) continue;
+            const int h = o / HD, d = o % HD, head = kvh * groups + h;
+            if (p.mode == kModeDirect) {
+                p.out[((size_t)slot * p.n_q + head) * HD + d] = accw[ob] / mlh[2 * h + 1];
+            } else {
+                float *rec = p.tmp + (((size_t)slot * p.n_q + head) * p.nwg + part) * (size_t)(HD + 2);
+                st_agent(rec + 2 + d, accw[ob]);
+                if (d == 0) { st_agent(rec, mlh[2 * h]); st_agent(rec + 1, mlh[2 * h + 1]); }
+            }
+        }
+    }
+    KSH_MARK(5);
+    if (p.mode != kModeMerge) return;
+
+    // ---- the last partition to arrive folds the partials (lower.rs:5897-6087) -
+    // every thread's record stores have completed (they are write-through) before the barrier lets thread 0 count
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    KSH_MARK(6);
+    if (tid == 0) {
+        const uint32_t arrived = __hip_atomic_fetch_add(&p.counters[slot * p.n_kv + kvh], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        last_flag = arrived == (uint32_t)p.nwg - 1u;
+    }
+    __syncthreads();
+    KSH_MARK(7);
+    if (!last_flag) return;
+    // The records come from the memory side (about a microsecond away), so all of
+    // a thread's loads -- its output elements' values from up to QB partitions,
+    // then its share of the (m, l) pairs -- are issued before anything is used.
+    constexpr int QB = 16, OB = GP * HD / NT;   // partitions in flight x output elements per thread
+    float *w2 = slots;                          // [groups][nwg] weights
+    float *mq = slots + groups * p.nwg;         // [groups][nwg][2]
+    const float *recs = p.tmp + ((size_t)slot * p.n_q + (size_t)kvh * groups) * p.nwg * (size_t)(HD + 2);
+    float acc[OB], val[OB][QB];
+#pragma unroll
+    for (int ob = 0; ob < OB; ob++) {
+        acc[ob] = 0.f;
+        const int o = min(tid + ob * NT, groups * HD - 1), h = o / HD, d = o % HD;
+        const float *rh = recs + (size_t)h * p.nwg * (HD + 2) + 2 + d;
+#pragma unroll
+        for (int u = 0; u < QB; u++) val[ob][u] = ld_agent(rh + (size_t)min(u, p.nwg - 1) * (HD + 2));
+    }
+    for (int i = tid; i < groups * p.nwg; i += NT) {
+        const float *rec = recs + (size_t)i * (HD + 2);   // (head, partition) records are contiguous in that order
+        mq[2 * i] = ld_agent(rec);
+        mq[2 * i + 1] = ld_agent(rec + 1);
+    }
+    __syncthreads();
+    KSH_MARK(8);
+    for (int h = wave; h < groups; h += NW) merge_weights(mq + 2 * h * p.nwg, 2, p.nwg, w2 + h * p.nwg, mlh + 2 * h, lane);
+    __syncthreads();
+    KSH_MARK(9);
+    for (int q0 = 0; q0 < p.nwg; q0 += QB) {
+#pragma unroll
+        for (int ob = 0; ob < OB; ob++) {
+            const int o = min(tid + ob * NT, groups * HD - 1), h = o / HD, d = o % HD;
+            if (q0) {
+                const float *rh = recs + (size_t)h * p.nwg * (HD + 2) + 2 + d;
+#pragma unroll
+                for (int u = 0; u < QB; u++) val[ob][u] = ld_agent(rh + (size_t)min(q0 + u, p.nwg - 1) * (HD + 2));
+            }
+#pragma unroll
+            for (int u = 0; u < QB; u++) acc[ob] = fmaf(q0 + u < p.nwg ? w2[h * p.nwg + q0 + u] : 0.f, val[ob][u], acc[ob]);
+        }
+    }
+#pragma unroll
+    for (int ob = 0; ob < OB; ob++) {
+        const int o = tid + ob * NT;
+        if (o < groups * HD) {
+            const int h = o / HD, d = o % HD;
+            p.out[((size_t)slot * p.n_q + kvh * groups + h) * HD + d] = acc[ob] / mlh[2 * h + 1];
+        }
+    }
+    KSH_MARK(10);
+    if (tid == 0) __hip_atomic_store(&p.counters[slot * p.n_kv + kvh], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next launch
+}
+
+template <int HD, int GP, int NW>
+constexpr size_t lanes_lds_bytes()
+{
+    constexpr int NSLOT = NW * (64 / (HD / 8));
+    return ((size_t)GP * HD + (size_t)NSLOT * (GP * HD + 2 * GP) + (size_t)GP * NSLOT + 2 * GP) * 4 + 2 * (HD / 32 * 18) + 16;
+}
+
+template <int HD, int GP, int NW>
+int launch_inst(const LaneParams &p, int n_slots, hipStream_t st)
+{
+    const size_t lds = lanes_lds_bytes<HD, GP, NW>();
+    hipLaunchKernelGGL((sdpa_lanes_kernel<HD, GP, NW>), dim3(p.nwg, p.n_kv, n_slots), dim3(NW * 64), lds, st, p);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : hip_fail(e, "sdpa (register form) launch");
+}
+
+int launch_lanes(const LaneParams &p, int hd, int nw, int n_slots, hipStream_t st)
+{
+    const int gp = p.groups <= 4 ? 4 : 8;
+#define KSH_CASE(H, G, W) \
+    if (hd == H && gp == G && nw == W) return launch_inst<H, G, W>(p, n_slots, st);
+    KSH_CASE(128, 4, 4) KSH_CASE(128, 8, 4) KSH_CASE(256, 4, 4) KSH_CASE(256, 8, 4)
+    KSH_CASE(128, 4, 8) KSH_CASE(128, 8, 8) KSH_CASE(256, 4, 8) KSH_CASE(256, 8, 8)
+#undef KSH_CASE
+    return set_error("sdpa (register form): no instance for hd=%d groups=%d nsg=%d", hd, p.groups, nw);
+}
+
+size_t lanes_lds(int hd, int groups, int nw)
+{
+    const int gp = groups <= 4 ? 4 : 8;
+    const int nslot = nw * (64 / (hd / 8));
+    return ((size_t)gp * hd + (size_t)nslot * (gp * hd + 2 * gp) + (size_t)gp * nslot + 2 * gp) * 4 + 2 * (hd / 32 * 18) + 16;
+}
+
+LaneParams base_params(const ksh_kernel &k)
+{
+    LaneParams p{};
+    p.n_q = (int)k.desc.dims[0];
+    p.n_kv = (int)k.desc.dims[1];
+    p.max_t = (int)k.desc.dims[3];
+    p.groups = p.n_q / p.n_kv;
+    p.counters = (uint32_t *)k.scratch;
+    return p;
+}
+
+// variant: nwg | NW << 16
+int launch_bound(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
+{
+    LaneParams p = base_params(k);
+    const int hd = (int)k.desc.dims[2], nw = (k.variant >> 16) & 0xFF;
+    p.nwg = k.variant & 0xFFFF;
+    int n_slots = 1;
+    switch (k.desc.kind) {
+    case KSH_SDPA_NAIVE:
+        p.q = (const float *)a.in[0]; p.k = (const uint8_t *)a.in[1]; p.v = (const uint8_t *)a.in[2];
+        p.meta = (const float *)a.in[3];
+        p.out = (float *)a.out[0];
+        p.scale = k.desc.params[0];
+        p.mode = kModeDirect;
+        break;
+    case KSH_SDPA_MWG_PART:
+        p.q = (const float *)a.in[0]; p.k = (const uint8_t *)a.in[1]; p.v = (const uint8_t *)a.in[2];
+        p.meta = (const float *)a.in[3];
+        p.tmp = (float *)a.out[0];
+        p.scale = k.desc.params[0];
+        p.mode = kModePart;
+        break;
+    case KSH_SDPA_SLOTS:
+        n_slots = (int)k.desc.dims[4];
+        p.q = (const float *)a.in[0]; p.k = (const uint8_t *)a.in[1]; p.v = (const uint8_t *)a.in[2];
+        p.meta = (const float *)a.in[3];
+        p.meta_stride = 4;
+        p.tmp = (float *)a.out[0];
+        p.out = (float *)a.out[1];
+        p.scale = k.desc.params[0];
+        p.mode = kModeMerge;
+        break;
+    case KSH_ATTEND_DECODE:
+        p.q = (const float *)a.in[0]; p.qw = (const float *)a.in[1]; p.rope = (const float *)a.in[2];
+        p.k_raw = (const float *)a.in[3]; p.kw = (const float *)a.in[4]; p.v_raw = (const float *)a.in[5];
+        p.meta = (const float *)a.in[6];
+        p.meta_stride = 4;
+        p.k_w = (uint8_t *)a.out[0]; p.v_w = (uint8_t *)a.out[1];
+        p.k = p.k_w; p.v = p.v_w;
+        p.tmp = (float *)a.out[2];
+        p.out = (float *)a.out[3];
+        p.eps = k.desc.params[0];
+        p.scale = k.desc.params[1];
+        p.mode = kModeMerge;
+        p.fused = 1;
+        break;
+    default: return set_error("sdpa (register form): kind %d", k.desc.kind);
+    }
+    return launch_lanes(p, hd, nw, n_slots, st);
+}
+
+}  // namespace
+
+bool sdpa_lanes_supports(int64_t n_q, int64_t n_kv, int64_t hd)
+{
+    return n_kv > 0 && n_q % n_kv == 0 && n_q / n_kv <= 8 && (hd == 128 || hd == 256);
+}
+
+// Fills in the launch for a shape sdpa_lanes_supports(); the caller has
+// validated the shape and set the buffer sizes of the SDPA kinds.
+int bind_sdpa_lanes(ksh_kernel &k, int nwg, int n_slots)
+{
+    const int64_t *d = k.desc.dims;
+    const int n_q = (int)d[0], n_kv = (int)d[1], hd = (int)d[2];
+    int nw = k.desc.sched.nsg ? (int)k.desc.sched.nsg : 0;
+    if (!nw) nw = (d[3] / nwg >= 256) ? 8 : 4;   // long partitions: more waves per workgroup
+    if (nw != 4 && nw != 8) return set_error("sdpa: unsupported schedule nsg=%d (4 or 8)", nw);
+    if (nwg < 1 || nwg > 4096) return set_error("sdpa: nwg=%d", nwg);
+    const size_t lds = lanes_lds(hd, n_q / n_kv, nw);
+    const bool merges = k.desc.kind == KSH_SDPA_SLOTS || k.desc.kind == KSH_ATTEND_DECODE;
+    if (merges && (size_t)(n_q / n_kv) * nwg * 3 * 4 > (size_t)nw * (64 / (hd / 8)) * ((n_q / n_kv <= 4 ? 4 : 8) * hd) * 4)
+        return set_error("sdpa: nwg=%d is too many partitions for the merge", nwg);
+    k.scratch_bytes = (size_t)n_slots * n_kv * 4;
+    set_launch(k, (uint32_t)nwg, (uint32_t)n_kv, (uint32_t)n_slots, (uint32_t)nw * 64, (uint32_t)lds);
+    k.info.sched = k.desc.sched;
+    k.info.sched.tg = (uint64_t)nw * 64;
+    k.info.sched.nsg = (uint32_t)nw;
+    k.info.sched.k_split = (uint32_t)nwg;
+    k.info.sched.lds_tile = 0;
+    k.variant = nwg | (nw << 16);
+    k.launch = launch_bound;
+    return 0;
+}
+
+// AttendDecode: RmsNormPerHeadQkvQ40 + split-KV attention + merge, one launch.
+int bind_attend_decode(ksh_kernel &k)
+{
+    const int64_t *d = k.desc.dims;
+    const int64_t n_q = d[0], n_kv = d[1], hd = d[2], max_t = d[3];
+    int64_t nwg = d[4];
+    if (n_q <= 0 || n_kv <= 0 || n_q % n_kv) return set_error("attend_decode: n_q=%lld n_kv=%lld", (long long)n_q, (long long)n_kv);
+    if (!sdpa_lanes_supports(n_q, n_kv, hd))
+        return set_error("attend_decode: built for hd 128 or 256 and up to 8 q heads per kv head (got hd=%lld, %lld)",
+                         (long long)hd, (long long)(n_q / n_kv));
+    if (max_t <= 0 || max_t > (1 << 24)) return set_error("attend_decode: max_seq=%lld", (long long)max_t);
+    if (nwg == 0) nwg = max_t >= 2048 ? 16 : (max_t + 127) / 128;
+    const size_t kvb = (size_t)max_t * n_kv * (hd / 32) * 18, qb = (size_t)n_q * hd * 4, kb = (size_t)n_kv * hd * 4;
+    k.info.n_inputs = 7;
+    k.info.n_outputs = 4;
+    k.in_bytes[0] = qb; k.in_bytes[1] = (size_t)hd * 4; k.in_bytes[2] = (size_t)max_t * hd * 4; k.in_bytes[3] = kb;
+    k.in_bytes[4] = (size_t)hd * 4; k.in_bytes[5] = kb; k.in_bytes[6] = 16;
+    for (int i = 0; i < 7; i++) k.in_align[i] = 4;
+    k.in_align[0] = 16;
+    k.out_bytes[0] = k.out_bytes[1] = kvb;
+    k.out_bytes[2] = (size_t)n_q * nwg * (hd + 2) * 4;
+    k.out_bytes[3] = qb;
+    k.out_align[0] = k.out_align[1] = 2; k.out_align[2] = k.out_align[3] = 4;
+    if (bind_sdpa_lanes(k, (int)nwg, 1)) return 1;
+    set_name(k, "attend_decode_hd%d_nwg%d_w%d", (int)hd, (int)nwg, (int)k.info.sched.nsg);
+    return 0;
+}
+
+}  // namespace ksh

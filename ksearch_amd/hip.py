@@ -55,6 +55,7 @@ class Kind(enum.IntEnum):           # enum ksh_kind
     RMSNORM_MATVEC = 19
     RMSNORM_MATVEC_QKV = 20
     RMSNORM_MATVEC_GATE_UP_GELU = 21
+    ATTEND_DECODE = 22
 
 
 class Sched(C.Structure):           # ksh_sched: OptSchedule retargeted to gfx950
@@ -471,6 +472,13 @@ class Eng:
         has_res = res is not None
         k = self._k(ctx, Kind.RMSNORM_MATVEC_GATE_UP_GELU, (rows, cols, int(has_res)), (wdt, DType.F32), (eps,), sched)
         ctx.encode_multi(k, [wg, wu, x, w_norm] + ([w_post, res] if has_res else []), [out] + ([x_new] if has_res else []))
+
+    # the decode step's RmsNormPerHeadQkvQ40 -> SdpaMwgPart -> SdpaMwgReduce (gemma_prim.rs:984-1060) as one launch
+    def attend_decode(self, ctx, n_q, n_kv, hd, max_seq, eps, scale, q, q_norm, rope, k, k_norm, v, meta, k_cache, v_cache,
+                      tmp, out, nwg=0, sched=None):
+        kk = self._k(ctx, Kind.ATTEND_DECODE, (n_q, n_kv, hd, max_seq, nwg), (DType.Q40, DType.F32), (eps, scale), sched)
+        ctx.encode_multi(kk, [q, q_norm, rope, k, k_norm, v, meta], [k_cache, v_cache, tmp, out])
+        return kk
 
     # :1414-1444
     def matvec_batch(self, ctx, rows, cols, batch, wdt, w, x, y, sched=None):

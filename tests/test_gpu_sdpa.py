@@ -138,3 +138,46 @@ def test_sdpa_errors(ctx):
         ctx.compile(hip.make_desc(hip.Kind.SDPA_NAIVE, (8, 1, 256, 64), (DType.F16, DType.F32), (1.0,)))
     with pytest.raises(hip.KshError, match="divide evenly"):
         ctx.compile(hip.make_desc(hip.Kind.SDPA_NAIVE, (8, 3, 256, 64), (DType.Q40, DType.F32), (1.0,)))
+
+
+@pytest.mark.parametrize("n_q,n_kv,hd,max_seq,pos,nwg", [
+    (8, 1, 256, 512, 0, 0),        # the first token attends only itself
+    (8, 1, 256, 512, 1, 4),
+    (8, 1, 256, 512, 200, 16),     # partitions of 13 rows, the last one short
+    (8, 1, 256, 4096, 319, 0),     # the decode loop's shape and default split
+    (4, 1, 128, 256, 77, 3),       # the small decode model
+    (4, 2, 128, 300, 150, 5),      # two kv heads
+])
+def test_attend_decode_vs_unfused_oracle(ctx, eng, n_q, n_kv, hd, max_seq, pos, nwg):
+    """AttendDecode = RmsNormPerHeadQkvQ40 at `pos` + attention over rows [0, pos] + merge.  The oracle runs the
+    three reference ops one after the other; the cache rows the kernel appends are compared as codes (they may
+    differ by one step where a value sits on a rounding boundary) and the attention output against the oracle's
+    attention over the DEVICE's cache, so that such a step does not leak into the comparison."""
+    eps, scale = 1e-6, 1.0 / float(np.sqrt(hd))
+    row = n_kv * hd // 32 * 18
+    k, v = kv(max_seq, n_kv, hd, 340 + pos)
+    k[pos * row:] = 0
+    v[pos * row:] = 0
+    q, kr, vr = (synth.normal_f32(r * hd, 350 + i) for i, r in enumerate((n_q, n_kv, n_kv)))
+    qw, kw = 1.0 + 0.2 * synth.normal_f32(hd, 353), 1.0 + 0.2 * synth.normal_f32(hd, 354)
+    rope = oracle.rope_table(max_seq, hd, 10000.0)
+    kc, vc = ctx.buffer_bytes(k), ctx.buffer_bytes(v)
+    out = ctx.buffer_empty_f32(n_q * hd)
+    meta = ctx.buffer_f32([pos + 1, 0, 0, pos])
+    kk = ctx.compile(hip.make_desc(hip.Kind.ATTEND_DECODE, (n_q, n_kv, hd, max_seq, nwg), (DType.Q40, DType.F32), (eps, scale)))
+    tmp = ctx.buffer_empty_f32(n_q * kk.grid[0] * (hd + 2))
+    for rep in range(2):                     # twice: the arrival counter must come back to zero
+        ctx.encode_multi(kk, [ctx.buffer_f32(q), ctx.buffer_f32(qw), ctx.buffer_f32(rope), ctx.buffer_f32(kr), ctx.buffer_f32(kw),
+                              ctx.buffer_f32(vr), meta], [kc, vc, tmp, out])
+        got = ctx.read_f32(out, n_q * hd)
+        wq, wk, wv = oracle.rmsnorm_per_head_qkv_q40(q, qw, rope[pos], kr, kw, vr, n_q, n_kv, hd, eps)
+        gk, gv = ctx.read_bytes(kc, (pos + 1) * row), ctx.read_bytes(vc, (pos + 1) * row)
+        assert np.array_equal(gk[:pos * row], k[:pos * row]) and np.array_equal(gv[:pos * row], v[:pos * row])
+        for g, w_ in ((gk[pos * row:], wk), (gv[pos * row:], wv)):
+            dg, dw = oracle.dequant(oracle.Q40, g, n_kv * hd), oracle.dequant(oracle.Q40, w_, n_kv * hd)
+            assert np.abs(dg - dw).max() <= np.abs(dw).max() / 7.0 * 1.01
+            assert (g != w_).mean() < 0.02
+        want = oracle.sdpa(wq, gk, gv, n_q, n_kv, hd, pos + 1, 0, scale, f64=True)
+        assert_close(got, want, TOL, f"rep {rep}")
+    if pos + 1 < max_seq:
+        assert not ctx.read_bytes(kc, row, (pos + 1) * row).any()

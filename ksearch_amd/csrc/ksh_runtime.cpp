@@ -166,6 +166,9 @@ int ksh_buffer_alloc(ksh_ctx *ctx, size_t bytes, const void *init, ksh_buf **out
     KSH_HIP(hipMalloc(&b->ptr, bytes ? bytes : 16));
     hipError_t e = init ? hipMemcpy(b->ptr, init, bytes, hipMemcpyHostToDevice)
                         : hipMemset(b->ptr, 0, bytes ? bytes : 16);
+    // hipMemset of device memory may return before the fill has run, and the fill is on the null stream, which the
+    // context's non-blocking streams do not wait for: finish it here, or a kernel's output can be zeroed after the fact
+    if (e == hipSuccess && !init) e = hipStreamSynchronize(nullptr);
     if (e != hipSuccess) {
         (void)hipFree(b->ptr);
         return hip_fail(e, "buffer init");
@@ -283,6 +286,7 @@ int ksh_kernel_get(ksh_ctx *ctx, const ksh_kernel_desc *desc, ksh_kernel **out)
     if (k->scratch_bytes) {
         KSH_HIP(hipMalloc(&k->scratch, k->scratch_bytes));
         KSH_HIP(hipMemset(k->scratch, 0, k->scratch_bytes));
+        KSH_HIP(hipStreamSynchronize(nullptr));   // see ksh_buffer_alloc
     }
     *out = k.get();
     ctx->kernels[key] = std::move(k);

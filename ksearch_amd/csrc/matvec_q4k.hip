@@ -409,15 +409,16 @@ int launch_q4k(const Q4kGeom &G, const MatvecParams &p, int total_waves, hipStre
     return G.var == kXI8 ? launch_rn<NM, kXI8>(G, p, total_waves, st) : launch_rn<NM, kXF32>(G, p, total_waves, st);
 }
 
-// default schedule: int8 dot, 8 waves per workgroup and 2 rows per wave if
-// that still gives every CU a workgroup (x staged once per 16 rows, and the
-// arithmetic that is left when the last weights arrive stays short), else
-// smaller workgroups.
+// default schedule, from cold-cache timings of the candidate set on the decode
+// shapes and the 4096 x 4096 case: 8 waves per workgroup and 2 rows per wave
+// where that still leaves ~150 workgroups, else fewer rows, else smaller
+// workgroups; int8 dot, except for rows longer than one 16-superblock step,
+// where the f32 form is the faster one.
 Q4kGeom pick_geom(const ksh_sched &s, int total_rows, int bpr)
 {
     Q4kGeom G;
     G.half = (bpr == 8);
-    G.var = sched_is_zero(s) ? kXI8 : (s.vec == 3 ? kXI8 : kXF32);
+    G.var = sched_is_zero(s) ? (bpr > 16 ? kXF32 : kXI8) : (s.vec == 3 ? kXI8 : kXF32);
     if (s.nsg && s.nr0) {
         G.NW = (int)s.nsg;
         G.R = (int)s.nr0;
@@ -429,7 +430,7 @@ Q4kGeom pick_geom(const ksh_sched &s, int total_rows, int bpr)
             if (s.nr0 && (int)s.nr0 != r) continue;
             G.NW = nw;
             G.R = r;
-            if (total_rows / (nw * G.rpw()) >= 256) return G;
+            if (total_rows / (nw * G.rpw()) >= 144) return G;
         }
     G.NW = s.nsg ? (int)s.nsg : 4;
     G.R = s.nr0 ? (int)s.nr0 : 1;

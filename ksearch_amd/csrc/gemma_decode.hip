@@ -157,11 +157,11 @@ int encode_token(ksh_gemma *m, bool want_logits, int &launches)
         if (enc(m, m->k_down, {L.wdown, m->ff}, {m->y}, launches)) return 1;
     }
     if (want_logits) {
-        // the last layer's rmsnorm_add and the output norm in one pass
-        if (enc(m, m->k_add_then, {m->y, m->layers[c.n_layers - 1].post_ffw_norm, cur, m->output_norm}, {other, m->x2}, launches))
+        // the last layer's rmsnorm_add and the output norm ride in the LM head's prologue
+        if (enc(m, m->k_lm_head, {m->embd, m->y, m->output_norm, m->layers[c.n_layers - 1].post_ffw_norm, cur},
+                {m->logits, other}, launches))
             return 1;
         m->hidden = other;
-        if (enc(m, m->k_lm_head, {m->embd, m->x2}, {m->logits}, launches)) return 1;
         if (enc(m, m->k_argmax, {m->logits}, {m->tok}, launches)) return 1;
         launches += 1;   // two passes
     }
@@ -266,10 +266,9 @@ int ksh_gemma_create(ksh_ctx *ctx, const ksh_gemma_cfg *cfg, const ksh_gemma_lay
         get(g, KSH_RMSNORM_MATVEC_QKV, {qd, kvd, c.hidden, 0}, {KSH_Q4K, KSH_F32}, {c.eps}, &g->k_qkv_first) ||
         get(g, KSH_RMSNORM_MATVEC_QKV, {qd, kvd, c.hidden, 1}, {KSH_Q4K, KSH_F32}, {c.eps}, &g->k_qkv) ||
         get(g, KSH_MATVEC, {c.hidden, qd}, {KSH_Q4K, KSH_F32}, {}, &g->k_oproj) ||
-        get(g, KSH_RMSNORM_ADD_THEN_RMSNORM, {c.hidden}, {}, {c.eps}, &g->k_add_then) ||
         get(g, KSH_RMSNORM_MATVEC_GATE_UP_GELU, {c.ffn, c.hidden, 1}, {KSH_Q4K, KSH_F32}, {c.eps}, &g->k_gate_up) ||
         get(g, KSH_MATVEC, {c.hidden, c.ffn}, {KSH_Q4K, KSH_F32}, {}, &g->k_down) ||
-        get(g, KSH_MATVEC, {c.vocab, c.hidden}, {KSH_Q6K, KSH_F32}, {}, &g->k_lm_head) ||
+        get(g, KSH_RMSNORM_MATVEC, {c.vocab, c.hidden, 1}, {KSH_Q6K, KSH_F32}, {c.eps}, &g->k_lm_head) ||
         get(g, KSH_SOFTCAP_ARGMAX, {c.vocab}, {}, {c.softcap}, &g->k_argmax))
         return 1;
     // per-head norm + RoPE + KV append + attention + merge: one launch where the fused kind is built for the

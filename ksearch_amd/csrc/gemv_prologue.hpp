@@ -23,7 +23,7 @@
 namespace ksh {
 
 enum { kPlain = 0, kRms = 1, kAddThenRms = 2 };
-enum { kXF32 = 0, kXI8 = 3 };
+enum { kXF32 = 0, kXI8 = 3, kXQ6 = 6 };
 
 struct Prologue {
     const float *x;        // kPlain/kRms: the vector; kAddThenRms: y
@@ -39,10 +39,20 @@ __host__ __device__ constexpr int xs_f32_floats(int cols) { return cols + (cols 
 __host__ __device__ constexpr int xs_i8_bytes(int cols) { return (cols >> 6) * 208 + (cols >> 5) * 8; }
 __device__ __forceinline__ int xs_f32_index(int e) { return e + ((e >> 6) << 2); }
 
+// Q6 planes: per 128 elements H[128] M[128] L[128], then for each run of 8
+// elements minus the sum of its X (int32 x 16), then the scale (one per 128).
+constexpr int kQ6HalfBytes = 464;
+__host__ __device__ constexpr int xs_q6_bytes(int cols) { return (cols >> 7) * kQ6HalfBytes; }
+
+template <int XF>
+__host__ __device__ constexpr size_t xs_image_bytes(int cols)
+{
+    return XF == kXI8 ? (size_t)xs_i8_bytes(cols) : XF == kXQ6 ? (size_t)xs_q6_bytes(cols) : (size_t)xs_f32_floats(cols) * 4;
+}
 template <int XF>
 __host__ __device__ constexpr size_t xs_bytes(int cols)
 {
-    return (XF == kXI8 ? (size_t)xs_i8_bytes(cols) : (size_t)xs_f32_floats(cols) * 4) + 64;   // + reduction scratch
+    return xs_image_bytes<XF>(cols) + 64;   // + reduction scratch
 }
 
 // max / sum over 8 consecutive lanes (one 32-element sub-block at 4 elements per lane)
@@ -84,6 +94,33 @@ __device__ __forceinline__ void store_x4(uint8_t *lds, int cols, int i, float4 v
 {
     if (XF == kXF32) {
         *reinterpret_cast<float4 *>(reinterpret_cast<float *>(lds) + xs_f32_index(i * 4)) = v;
+        return;
+    }
+    if (XF == kXQ6) {
+        // 32 consecutive lanes hold one run of 128 elements: one scale for the run
+        float amax = oct_max(fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+        amax = fmaxf(amax, dpp_f32<0x140>(amax));                 // row_mirror: the other 8 of the 16-lane row
+        amax = fmaxf(amax, __shfl_xor(amax, 16, 64));             // the other row of the 32
+        const float inv = amax > 0.f ? 1048575.0f / amax : 0.f;
+        const float xs4[4] = {v.x, v.y, v.z, v.w};
+        int h[4], m[4], l[4], sx = 0;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int X = (int)rintf(xs4[k] * inv);
+            sx += X;
+            l[k] = (X << 25) >> 25;
+            const int X1 = (X - l[k]) >> 7;
+            m[k] = (X1 << 25) >> 25;
+            h[k] = (X1 - m[k]) >> 7;
+        }
+        sx += __builtin_amdgcn_update_dpp(0, sx, 0xB1, 0xF, 0xF, true);   // the neighbour's four: a run of 8
+        uint8_t *half = lds + (i >> 5) * kQ6HalfBytes;
+        const int o = (i & 31) * 4;
+        *reinterpret_cast<uint32_t *>(half + o) = pack4_i8(h[0], h[1], h[2], h[3]);
+        *reinterpret_cast<uint32_t *>(half + 128 + o) = pack4_i8(m[0], m[1], m[2], m[3]);
+        *reinterpret_cast<uint32_t *>(half + 256 + o) = pack4_i8(l[0], l[1], l[2], l[3]);
+        if ((i & 1) == 0) reinterpret_cast<int *>(half + 384)[(i & 31) >> 1] = -sx;
+        if ((i & 31) == 0) *reinterpret_cast<float *>(half + 448) = amax * (1.0f / 1048575.0f);
         return;
     }
     const float amax = oct_max(fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
@@ -158,7 +195,7 @@ template <int XF, int NT>
 __device__ __forceinline__ void stage_finish(const Prologue &pr, uint8_t *lds, int cols, StageRegs &s)
 {
     const int wbase = __builtin_amdgcn_readfirstlane(threadIdx.x & ~63), tid = wbase + (threadIdx.x & 63), n4 = cols / 4;
-    float *red = reinterpret_cast<float *>(lds + (XF == kXI8 ? (size_t)xs_i8_bytes(cols) : (size_t)xs_f32_floats(cols) * 4));
+    float *red = reinterpret_cast<float *>(lds + xs_image_bytes<XF>(cols));
     if (pr.kind == kPlain) {
         if (n4 > NT * kStageX) {
             for (int i = tid; i < n4; i += NT) store_x4<XF>(lds, cols, i, ldg_f4(pr.x, i));

@@ -240,3 +240,24 @@ def test_rmsnorm_matvec_prologues(ctx, eng, has_res, sched):
     g, u = oracle.matvec(oracle.Q4K, wg, rows, n, vec), oracle.matvec(oracle.Q4K, wu, rows, n, vec)
     assert_close(ctx.read_f32(out, rows), oracle.gelu_mul(g, u), TOL, "rms_gate_up")
     check_xnew(xn)
+
+
+@pytest.mark.parametrize("has_res", [False, True])
+def test_rmsnorm_matvec_q6k_lm_head_prologue(ctx, eng, has_res):
+    """The LM head with the output norm (and the last layer's residual add) in its prologue."""
+    n, rows, eps = 2048, 3000, 1e-6
+    x, w_norm, w_post, res = (synth.normal_f32(n, 800 + i) for i in range(4))
+    w_norm, w_post = 1.0 + 0.1 * w_norm, 1.0 + 0.1 * w_post
+    if has_res:
+        x_new, vec = oracle.rmsnorm_add_then_rmsnorm(x, w_post, res, w_norm, eps)
+    else:
+        x_new, vec = None, oracle.rmsnorm(x, w_norm, eps)
+    w = synth.q6k_blocks(rows * n // 256, seed=810)
+    bx, bwn, bwp, br = (ctx.buffer_f32(a) for a in (x, w_norm, w_post, res))
+    y, xn = ctx.buffer_empty_f32(rows), ctx.buffer_empty_f32(n)
+    extra = dict(w_post=bwp, res=br, x_new=xn) if has_res else {}
+    eng.rmsnorm_matvec_wd(ctx, rows, n, eps, DType.Q6K, bx, bwn, ctx.buffer_bytes(w), y, **extra)
+    assert_close(ctx.read_f32(y, rows), oracle.matvec(oracle.Q6K, w, rows, n, vec), TOL, "rms_matvec_q6k")
+    assert_close(ctx.read_f32(y, rows), oracle.matvec_f64(oracle.Q6K, w, rows, n, vec), 1e-5, "rms_matvec_q6k vs f64")
+    if has_res:
+        assert_close(ctx.read_f32(xn, n), x_new, 1e-5, "x_new")

@@ -177,6 +177,12 @@ def cpu_baseline_matvec(w, x, rows, cols, budget_s=1.5):
     return out, oracle.max_threads()
 
 
+# HBM bytes per launch of the headline kernel, from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
+# profiles/q4k_gemv_cfg0_cold.txt (2.00 x 4760.1 KiB fetched + 16.0 KiB written).  Counters cannot be read from
+# inside this script, so the figure is carried here for the kernel it was taken on and is null for any other.
+MEASURED_TRAFFIC_BYTES = {"matvec_q4k_r2_w8_v3": 9765069}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -186,8 +192,9 @@ def main() -> int:
     ap.add_argument("--no-extras", action="store_true", help="headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--eager", action="store_true", help="cfg4 without HIP-graph replay (kernel-trace profiling)")
-    ap.add_argument("--only", choices=["cfg1", "cfg2", "cfg3", "cfg4"],
-                    help="run one secondary workload and print its record (for profiling runs)")
+    ap.add_argument("--only", choices=["cfg1", "cfg2", "cfg3", "cfg4", "copy"],
+                    help="run one secondary workload and print its record (for profiling runs); 'copy' is a plain "
+                         "64 MiB device copy, the known-size kernel that calibrates the FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (the hot path is a single-GPU kernel path); "
@@ -198,6 +205,14 @@ def main() -> int:
     from ksearch_amd.hip import DType
 
     ctx, eng, ev = hip.Context(), hip.Eng(), HipEvents()
+    if args.only == "copy":
+        n = 16 << 20
+        src, dst = ctx.buffer_f32(np.ones(n, dtype=np.float32)), ctx.buffer_empty_f32(n)
+        k = ctx.compile(hip.make_desc(hip.Kind.COPY_SLICE, (n,)))
+        ms = ctx.run(k, [src], [dst], iters=8)
+        ctx.close()
+        print(json.dumps({"copy": {"bytes_read": n * 4, "bytes_written": n * 4, "us_per_launch": round(ms * 1e3, 2)}}))
+        return 0
     if args.only:
         if args.only == "cfg1":
             w1, x1 = synth.cfg1_q6k_lm_head()
@@ -236,11 +251,12 @@ def main() -> int:
     line = {
         "metric": "q4k_matvec_GBps", "value": round(head["gbps"], 1), "unit": "GB/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["ms"] / args.steps,
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "i8+f32", "data": "synthetic",
         "config": {"workload": "cfg0: Q4_K GEMV rows=4096 cols=4096 batch=1, f32 x/y, weights streamed from HBM "
                                f"({args.copies} rotating copies)", "kernel": head["kernel"]},
         "roofline": {"bound": "hbm", "achieved": round(head["gbps"], 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(head["gbps"] / HBM_PEAK_GBPS, 4), "traffic": None},
+                     "frac": round(head["gbps"] / HBM_PEAK_GBPS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(head["kernel"])},
         "cpu_baseline": cpu,
         "also": also,
     }

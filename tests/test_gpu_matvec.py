@@ -261,3 +261,25 @@ def test_rmsnorm_matvec_q6k_lm_head_prologue(ctx, eng, has_res):
     assert_close(ctx.read_f32(y, rows), oracle.matvec_f64(oracle.Q6K, w, rows, n, vec), 1e-5, "rms_matvec_q6k vs f64")
     if has_res:
         assert_close(ctx.read_f32(xn, n), x_new, 1e-5, "x_new")
+
+
+def test_beam_search_on_device(ctx, eng, tmp_path, monkeypatch):
+    """Eng::beam_matvec (ksearch_kernels/src/lib.rs:1985-2043): every candidate is timed on the device, the best one
+    is saved as a plan under KSEARCH_BEAM_CACHE, a second search is served from the file, and a kernel compiled
+    with an all-zero schedule then picks the plan up."""
+    monkeypatch.setenv("KSEARCH_BEAM_CACHE", str(tmp_path / "beam"))
+    monkeypatch.setenv("KSEARCH_CHIP", "gfx950-test")
+    rows, cols = 1024, 2048
+    w = synth.q4k_blocks(rows * cols // 256, seed=900)
+    x = synth.normal_f32(cols, seed=901)
+    bw, bx, by = ctx.buffer_bytes(w), ctx.buffer_f32(x), ctx.buffer_empty_f32(rows)
+    best, ms, cached = eng.beam_matvec(ctx, rows, cols, DType.Q4K, bw, bx, by, iters=5, force=True)
+    cands = [c.as_dict() for c in hip.beam_candidates(hip.make_desc(hip.Kind.MATVEC, (rows, cols), (DType.Q4K, DType.F32)))]
+    assert not cached and 0 < ms < 1.0
+    assert any(all(best.as_dict()[k] == c[k] for k in ("nsg", "nr0", "vec")) for c in cands)
+    # the search leaves a correct result behind, whichever candidate ran last
+    assert_close(ctx.read_f32(by, rows), oracle.matvec(oracle.Q4K, w, rows, cols, x), TOL, "after beam")
+    files = list((tmp_path / "beam").glob("*.txt"))
+    assert len(files) == 1 and files[0].name.startswith("matvec_q4k_1024x2048_")     # the chip name is in the hash
+    best2, ms2, cached2 = eng.beam_matvec(ctx, rows, cols, DType.Q4K, bw, bx, by, iters=5)
+    assert cached2 and best2.as_dict() == best.as_dict()

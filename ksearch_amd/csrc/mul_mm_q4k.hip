@@ -26,7 +26,8 @@
 // 64 x 64 as 2 x 2 v_mfma_f32_32x32x16_f16 tiles.  M = tokens, N = weight
 // rows, so a lane's accumulator column is one weight row (one d per lane) and
 // stores are contiguous along Y's row index.  K advances 64 columns (one
-// 64-element group: 32 quant bytes per row) per step through LDS.
+// 64-element group: 32 quant bytes per row) per step through a double-buffered
+// LDS stage, with the next step's global loads in flight under the MFMAs.
 #include "ksh_device.hpp"
 #include "ksh_internal.hpp"
 
@@ -84,18 +85,34 @@ __device__ __forceinline__ uint32_t pair_f16(uint32_t masked, uint32_t sc)
     return __umul24(masked, sc) + 0x64006400u;
 }
 
+// what a loader thread holds for one K step (64 columns) of its row: 16 quant
+// bytes, 32 activations, and -- for the first step of a superblock -- the
+// superblock header and the token's sums of x
+struct StepRegs {
+    uint4 q, x0, x1, x2, x3;
+    uint4 hdr, sx0, sx1;
+};
+
+constexpr int kLdsMain = (BM + BN) * PITCH;      // halves per main stage (A tile, then B tile)
+constexpr int kLdsMin = (BM + BN) * PITCH2;      // halves per min-term stage
+constexpr size_t kLdsBytes = 2 * (size_t)(kLdsMain + kLdsMin) * 2 + 2 * BN * 4;
+
+// Software pipeline, one barrier per K step: the global loads of step s+1 are
+// issued, the matrix cores work on LDS stage s&1, then the loaded registers
+// are converted and written to stage (s+1)&1.  The min-term operands of a
+// superblock are written together with its first step into their own double
+// buffer and consumed after its fourth.
 __global__ __launch_bounds__(256) void q4k_mul_mm_kernel(MmParams p)
 {
-    __shared__ __attribute__((aligned(16))) _Float16 As[BM * PITCH];
-    __shared__ __attribute__((aligned(16))) _Float16 Bs[BN * PITCH];
-    __shared__ __attribute__((aligned(16))) _Float16 A2s[BM * PITCH2];
-    __shared__ __attribute__((aligned(16))) _Float16 B2s[BN * PITCH2];
-    __shared__ float dsc[BN];
+    extern __shared__ __attribute__((aligned(16))) _Float16 lds[];
+    auto main_stage = [&](int i) { return lds + (i & 1) * kLdsMain; };
+    auto min_stage = [&](int i) { return lds + 2 * kLdsMain + (i & 1) * kLdsMin; };
+    auto dsc_stage = [&](int i) { return reinterpret_cast<float *>(lds + 2 * kLdsMain + 2 * kLdsMin) + (i & 1) * BN; };
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int t0 = blockIdx.x * BM, r0 = blockIdx.y * BN;
-    const int nsb = p.cols / 256;
+    const int nsb = p.cols / 256, nsteps = nsb * 4;
     const size_t row_bytes = (size_t)nsb * 144;
 
     // loader roles
@@ -103,6 +120,72 @@ __global__ __launch_bounds__(256) void q4k_mul_mm_kernel(MmParams p)
     const uint8_t *wrow = p.W + (size_t)min(r0 + lrow, p.rows - 1) * row_bytes;
     const _Float16 *xrow = p.Xh + (size_t)min(t0 + lrow, p.batch - 1) * p.cols;
     const _Float16 *sxrow = p.SxA + (size_t)min(t0 + lrow, p.batch - 1) * nsb * 32;
+
+    auto fetch = [&](int step, StepRegs &r) {
+        const int sb = step >> 2, g = step & 3;
+        r.q = *reinterpret_cast<const uint4 *>(wrow + (size_t)sb * 144 + 16 + 32 * g + 16 * lhalf);
+        const uint4 *xs = reinterpret_cast<const uint4 *>(xrow + sb * 256 + 64 * g + 32 * lhalf);
+        r.x0 = xs[0]; r.x1 = xs[1]; r.x2 = xs[2]; r.x3 = xs[3];
+        if (g == 0) {
+            r.hdr = *reinterpret_cast<const uint4 *>(wrow + (size_t)sb * 144);
+            const uint4 *sx = reinterpret_cast<const uint4 *>(sxrow + sb * 32 + 16 * lhalf);
+            r.sx0 = sx[0]; r.sx1 = sx[1];
+        }
+    };
+    // r.hdr is the header of the step's superblock (carried over from its first step)
+    auto stage = [&](int step, const StepRegs &r) {
+        const int sb = step >> 2, g = step & 3;
+        _Float16 *As = main_stage(step), *Bs = As + BM * PITCH;
+        {
+            uint4 *dst = reinterpret_cast<uint4 *>(&As[lrow * PITCH + 32 * lhalf]);
+            dst[0] = r.x0; dst[1] = r.x1; dst[2] = r.x2; dst[3] = r.x3;
+        }
+        {
+            const uint4 s = q4k_group_scales(r.hdr.y, r.hdr.z, r.hdr.w, g);   // sc_lo, mn_lo, sc_hi, mn_hi
+            const uint32_t w[4] = {r.q.x, r.q.y, r.q.z, r.q.w};
+            uint32_t lo[8], hi[8];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const uint32_t t4 = w[i] >> 4;
+                lo[2 * i] = pair_f16(w[i] & 0x000F000Fu, s.x);
+                lo[2 * i + 1] = pair_f16((w[i] >> 8) & 0x000F000Fu, s.x);
+                hi[2 * i] = pair_f16(t4 & 0x000F000Fu, s.z);
+                hi[2 * i + 1] = pair_f16((t4 >> 8) & 0x000F000Fu, s.z);
+            }
+            uint4 *dlo = reinterpret_cast<uint4 *>(&Bs[lrow * PITCH + 16 * lhalf]);
+            uint4 *dhi = reinterpret_cast<uint4 *>(&Bs[lrow * PITCH + 32 + 16 * lhalf]);
+            dlo[0] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+            dlo[1] = make_uint4(lo[4], lo[5], lo[6], lo[7]);
+            dhi[0] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+            dhi[1] = make_uint4(hi[4], hi[5], hi[6], hi[7]);
+        }
+        if (g == 0) {
+            // bias + mins of this superblock, for the short second product after its fourth step
+            _Float16 *A2s = min_stage(sb), *B2s = A2s + BM * PITCH2;
+            const float d = half_bits_to_f32(r.hdr.x & 0xFFFFu), dmin = half_bits_to_f32(r.hdr.x >> 16);
+            // this thread covers sub-blocks 4*lhalf .. 4*lhalf+3 of its row: groups 2*lhalf, 2*lhalf+1
+            uint32_t hi2[2], lo2[2];
+#pragma unroll
+            for (int gg = 0; gg < 2; gg++) {
+                const uint4 s = q4k_group_scales(r.hdr.y, r.hdr.z, r.hdr.w, 2 * lhalf + gg);
+                const float c0 = -(dmin * (float)s.y + 1024.f * d), c1 = -(dmin * (float)s.w + 1024.f * d);
+                const _Float16 h0 = (_Float16)c0, h1 = (_Float16)c1;
+                const _Float16 l0 = (_Float16)(c0 - (float)h0), l1 = (_Float16)(c1 - (float)h1);
+                hi2[gg] = (uint32_t)__builtin_bit_cast(uint16_t, h0) | ((uint32_t)__builtin_bit_cast(uint16_t, h1) << 16);
+                lo2[gg] = (uint32_t)__builtin_bit_cast(uint16_t, l0) | ((uint32_t)__builtin_bit_cast(uint16_t, l1) << 16);
+            }
+            // row layout (32 halves): hi[8] | lo[8] | hi[8] | 0[8]; this thread owns halves 4*lhalf .. +3 of each octet
+            uint2 *b2 = reinterpret_cast<uint2 *>(&B2s[lrow * PITCH2 + 4 * lhalf]);
+            b2[0] = make_uint2(hi2[0], hi2[1]);
+            b2[2] = make_uint2(lo2[0], lo2[1]);
+            b2[4] = make_uint2(hi2[0], hi2[1]);
+            b2[6] = make_uint2(0u, 0u);
+            if (lhalf == 0) dsc_stage(sb)[lrow] = d;
+            uint4 *dst = reinterpret_cast<uint4 *>(&A2s[lrow * PITCH2 + 16 * lhalf]);
+            dst[0] = r.sx0;
+            dst[1] = r.sx1;
+        }
+    };
 
     f16v F[2][2], Cp[2][2];
 #pragma unroll
@@ -114,106 +197,69 @@ __global__ __launch_bounds__(256) void q4k_mul_mm_kernel(MmParams p)
 
     const int lm = lane & 31, lk = (lane >> 5) * 8;
 
+    StepRegs regs;
+    fetch(0, regs);
+    stage(0, regs);
+    __syncthreads();
+
+    // (superblock, group) as two loops with the inner one unrolled, so that "is this the superblock's first /
+    // last step" is a compile-time fact and the accumulators stay where the matrix cores want them in between
     for (int sb = 0; sb < nsb; sb++) {
-        const uint4 hdr = *reinterpret_cast<const uint4 *>(wrow + (size_t)sb * 144);
-        for (int g = 0; g < 4; g++) {
-            const uint4 q = *reinterpret_cast<const uint4 *>(wrow + (size_t)sb * 144 + 16 + 32 * g + 16 * lhalf);
-            const uint4 *xs = reinterpret_cast<const uint4 *>(xrow + sb * 256 + 64 * g + 32 * lhalf);
-            const uint4 x0 = xs[0], x1 = xs[1], x2 = xs[2], x3 = xs[3];
-            const uint4 s = q4k_group_scales(hdr.y, hdr.z, hdr.w, g);   // sc_lo, mn_lo, sc_hi, mn_hi
-            __syncthreads();   // the previous step's MFMA reads of As/Bs are done
-            {
-                uint4 *dst = reinterpret_cast<uint4 *>(&As[lrow * PITCH + 32 * lhalf]);
-                dst[0] = x0; dst[1] = x1; dst[2] = x2; dst[3] = x3;
-            }
-            {
-                const uint32_t w[4] = {q.x, q.y, q.z, q.w};
-                uint32_t lo[8], hi[8];
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const uint32_t t4 = w[i] >> 4;
-                    lo[2 * i] = pair_f16(w[i] & 0x000F000Fu, s.x);
-                    lo[2 * i + 1] = pair_f16((w[i] >> 8) & 0x000F000Fu, s.x);
-                    hi[2 * i] = pair_f16(t4 & 0x000F000Fu, s.z);
-                    hi[2 * i + 1] = pair_f16((t4 >> 8) & 0x000F000Fu, s.z);
-                }
-                uint4 *dlo = reinterpret_cast<uint4 *>(&Bs[lrow * PITCH + 16 * lhalf]);
-                uint4 *dhi = reinterpret_cast<uint4 *>(&Bs[lrow * PITCH + 32 + 16 * lhalf]);
-                dlo[0] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
-                dlo[1] = make_uint4(lo[4], lo[5], lo[6], lo[7]);
-                dhi[0] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
-                dhi[1] = make_uint4(hi[4], hi[5], hi[6], hi[7]);
-            }
-            __syncthreads();
+      for (int g = 0; g < 4; g++) {
+        const int step = 4 * sb + g;
+        const bool more = step + 1 < nsteps;
+        if (more) fetch(step + 1, regs);   // hdr/sx are overwritten only when step+1 opens a superblock
+        const _Float16 *As = main_stage(step), *Bs = As + BM * PITCH;
 #pragma unroll
-            for (int ks = 0; ks < KS / 16; ks++) {
+        for (int ks = 0; ks < KS / 16; ks++) {
+            h8 a[2], b[2];
+#pragma unroll
+            for (int mt = 0; mt < 2; mt++)
+                a[mt] = *reinterpret_cast<const h8 *>(&As[(wm * 64 + mt * 32 + lm) * PITCH + 16 * ks + lk]);
+#pragma unroll
+            for (int nt = 0; nt < 2; nt++)
+                b[nt] = *reinterpret_cast<const h8 *>(&Bs[(wn * 64 + nt * 32 + lm) * PITCH + 16 * ks + lk]);
+#pragma unroll
+            for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+                for (int nt = 0; nt < 2; nt++)
+                    Cp[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mt], b[nt], Cp[mt][nt], 0, 0, 0);
+        }
+        if (g == 3) {
+            // ---- end of the superblock: bias + mins through the short second product, then the row scale
+            const _Float16 *A2s = min_stage(sb), *B2s = A2s + BM * PITCH2;
+            const float *dsc = dsc_stage(sb);
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++) {
                 h8 a[2], b[2];
 #pragma unroll
                 for (int mt = 0; mt < 2; mt++)
-                    a[mt] = *reinterpret_cast<const h8 *>(&As[(wm * 64 + mt * 32 + lm) * PITCH + 16 * ks + lk]);
+                    a[mt] = *reinterpret_cast<const h8 *>(&A2s[(wm * 64 + mt * 32 + lm) * PITCH2 + 16 * ks + lk]);
 #pragma unroll
                 for (int nt = 0; nt < 2; nt++)
-                    b[nt] = *reinterpret_cast<const h8 *>(&Bs[(wn * 64 + nt * 32 + lm) * PITCH + 16 * ks + lk]);
+                    b[nt] = *reinterpret_cast<const h8 *>(&B2s[(wn * 64 + nt * 32 + lm) * PITCH2 + 16 * ks + lk]);
 #pragma unroll
                 for (int mt = 0; mt < 2; mt++)
 #pragma unroll
                     for (int nt = 0; nt < 2; nt++)
-                        Cp[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mt], b[nt], Cp[mt][nt], 0, 0, 0);
+                        F[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mt], b[nt], F[mt][nt], 0, 0, 0);
             }
-        }
-        // ---- end of the superblock: bias + mins through a short second product, then the row scale
-        {
-            const float d = half_bits_to_f32(hdr.x & 0xFFFFu), dmin = half_bits_to_f32(hdr.x >> 16);
-            // this thread covers sub-blocks 4*lhalf .. 4*lhalf+3 of its row: groups 2*lhalf, 2*lhalf+1
 #pragma unroll
-            for (int gg = 0; gg < 2; gg++) {
-                const int g = 2 * lhalf + gg;
-                const uint4 s = q4k_group_scales(hdr.y, hdr.z, hdr.w, g);
-                const float c0 = -(dmin * (float)s.y + 1024.f * d), c1 = -(dmin * (float)s.w + 1024.f * d);
-                const _Float16 h0 = (_Float16)c0, h1 = (_Float16)c1;
-                const _Float16 l0 = (_Float16)(c0 - (float)h0), l1 = (_Float16)(c1 - (float)h1);
-                _Float16 *b2 = &B2s[lrow * PITCH2];
-                const int j = 2 * g;
-                b2[j] = h0; b2[j + 1] = h1;
-                b2[8 + j] = l0; b2[8 + j + 1] = l1;
-                b2[16 + j] = h0; b2[16 + j + 1] = h1;
-                b2[24 + j] = (_Float16)0.f; b2[24 + j + 1] = (_Float16)0.f;
+            for (int nt = 0; nt < 2; nt++) {
+                const float dn = dsc[wn * 64 + nt * 32 + lm];
+#pragma unroll
+                for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++) {
+                        F[mt][nt][i] = fmaf(dn, Cp[mt][nt][i], F[mt][nt][i]);
+                        Cp[mt][nt][i] = 0.f;
+                    }
             }
-            if (lhalf == 0) dsc[lrow] = d;
-            const uint4 *sx = reinterpret_cast<const uint4 *>(sxrow + sb * 32 + 16 * lhalf);
-            uint4 *dst = reinterpret_cast<uint4 *>(&A2s[lrow * PITCH2 + 16 * lhalf]);
-            dst[0] = sx[0];
-            dst[1] = sx[1];
         }
+        if (more) stage(step + 1, regs);
         __syncthreads();
-#pragma unroll
-        for (int ks = 0; ks < 2; ks++) {
-            h8 a[2], b[2];
-#pragma unroll
-            for (int mt = 0; mt < 2; mt++)
-                a[mt] = *reinterpret_cast<const h8 *>(&A2s[(wm * 64 + mt * 32 + lm) * PITCH2 + 16 * ks + lk]);
-#pragma unroll
-            for (int nt = 0; nt < 2; nt++)
-                b[nt] = *reinterpret_cast<const h8 *>(&B2s[(wn * 64 + nt * 32 + lm) * PITCH2 + 16 * ks + lk]);
-#pragma unroll
-            for (int mt = 0; mt < 2; mt++)
-#pragma unroll
-                for (int nt = 0; nt < 2; nt++)
-                    F[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mt], b[nt], F[mt][nt], 0, 0, 0);
-        }
-#pragma unroll
-        for (int nt = 0; nt < 2; nt++) {
-            const float dn = dsc[wn * 64 + nt * 32 + lm];
-#pragma unroll
-            for (int mt = 0; mt < 2; mt++)
-#pragma unroll
-                for (int i = 0; i < 16; i++) {
-                    F[mt][nt][i] = fmaf(dn, Cp[mt][nt][i], F[mt][nt][i]);
-                    Cp[mt][nt][i] = 0.f;
-                }
-        }
-        // A2s/B2s/dsc are rewritten only after the next superblock's eight
-        // barriers, so no extra barrier is needed here
+      }
     }
 
     // accumulator layout of the 32x32 tile: column = lane % 32, row = 8*(i/4) + 4*(lane/32) + i%4
@@ -244,7 +290,7 @@ int launch_mul_mm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
     p.SxA = SxA;
     p.Y = (float *)a.out[0];
     p.rows = rows; p.cols = cols; p.batch = batch;
-    hipLaunchKernelGGL(q4k_mul_mm_kernel, dim3((batch + BM - 1) / BM, (rows + BN - 1) / BN), dim3(256), 0, st, p);
+    hipLaunchKernelGGL(q4k_mul_mm_kernel, dim3((batch + BM - 1) / BM, (rows + BN - 1) / BN), dim3(256), kLdsBytes, st, p);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : hip_fail(e, "mul_mm launch");
 }
@@ -266,7 +312,7 @@ int bind_matvec_batch(ksh_kernel &k)
     // f16 copy of X plus the min-term operand (32 halves per token and superblock)
     k.scratch_bytes = (size_t)batch * cols * 2 + (size_t)batch * (cols / 256) * 64;
     set_launch(k, (uint32_t)((batch + BM - 1) / BM), (uint32_t)((rows + BN - 1) / BN), 1, 256,
-               (uint32_t)((BM + BN) * (PITCH + PITCH2) * 2 + BN * 4));
+               (uint32_t)kLdsBytes);
     k.info.sched = k.desc.sched;
     k.info.sched.tg = 256; k.info.sched.nsg = 4; k.info.sched.lds_tile = KS;
     set_name(k, "mul_mm_q4k_%dx%dx%d", BM, BN, KS);

@@ -22,8 +22,9 @@
 // X is bf16, which converts to f16 without loss for |x| >= 2^-17 (smaller
 // values lose at most 2^-25 absolutely).
 //
-// Tiling: a workgroup (8 waves) owns 128 tokens x 128 weight rows; a wave owns
-// 64 x 32 as 2 x 1 v_mfma_f32_32x32x16_f16 tiles.  M = tokens, N = weight
+// Tiling: a workgroup owns 128 tokens x 128 weight rows; each of its four
+// multiplying waves owns 64 x 64 as 2 x 2 v_mfma_f32_32x32x16_f16 tiles (four
+// more waves load and convert).  M = tokens, N = weight
 // rows, so a lane's accumulator column is one weight row (one d per lane) and
 // stores are contiguous along Y's row index.  K advances 64 columns (one
 // 64-element group: 32 quant bytes per row) per step through a double-buffered
@@ -87,17 +88,17 @@ __device__ __forceinline__ uint32_t pair_f16(uint32_t masked, uint32_t sc)
     return __umul24(masked, sc) + 0x64006400u;
 }
 
-// what a loader thread (four per tile row) holds: per K step 16 activations;
-// per superblock the 32 quant bytes of ONE of its four 64-column groups (so
+// what a loader thread (two per tile row) holds: per K step 32 activations;
+// per superblock the 64 quant bytes of TWO of its four 64-column groups (so
 // that a weight row's cache lines are fetched once, not once per step), the
-// header and a quarter of the token's sums of x
+// header and half of the token's sums of x
 // (native vector types: with HIP's uint4 class the copies become memcpys that keep these sets in scratch memory)
 struct XRegs {
-    u32x4_t x0, x1;
+    u32x4_t x[4];
 };
 struct SbRegs {
-    u32x4_t qa, qb;    // quant bytes 0..15, 16..31 of group lq
-    u32x4_t hdr, sx;
+    u32x4_t q[4];      // quant bytes of groups 2*lh and 2*lh+1, 32 each
+    u32x4_t hdr, sx0, sx1;
 };
 
 constexpr int kThreadsMM = 512;
@@ -105,13 +106,16 @@ constexpr int kLdsMain = (BM + BN) * PITCH;      // halves per main stage (A til
 constexpr int kLdsMin = (BM + BN) * PITCH2;      // halves per min-term stage
 constexpr size_t kLdsBytes = 2 * (size_t)(kLdsMain + kLdsMin) * 2 + 2 * BN * 4;
 
-// Software pipeline, one barrier per K step: the global loads of step s+4 are
-// issued, the matrix cores work on LDS stage s&1, then the registers loaded for
-// step s+1 are converted and written to stage (s+1)&1.  The min-term operands of a
-// superblock are written together with its first step into their own double
-// buffer and consumed after its fourth.  Eight waves (two per SIMD, each a
-// 64 x 32 piece of the 128 x 128 tile), so that one wave's conversions and LDS
-// traffic run while the other's matrix instructions execute.
+// Eight waves in two roles, one of each per SIMD.  Waves 0..3 only multiply:
+// each owns a 64 x 64 piece of the tile (2 x 2 MFMA tiles, one LDS operand
+// read per matrix instruction) and works on LDS stage s&1.  Waves 4..7 only
+// load and convert: during the same step they request the activations of step
+// s+4 (and, when a superblock opens, the next superblock's weights) and write
+// step s+1 into stage (s+1)&1.  One barrier per K step joins them, so the
+// conversions and the LDS writes of one role run in the shadow of the other
+// role's matrix instructions.  The min-term operands of a superblock are
+// written together with its first step into their own double buffer and
+// consumed after its fourth.
 __global__ __launch_bounds__(kThreadsMM) void q4k_mul_mm_kernel(MmParams p)
 {
     extern __shared__ __attribute__((aligned(16))) _Float16 lds[];
@@ -119,169 +123,214 @@ __global__ __launch_bounds__(kThreadsMM) void q4k_mul_mm_kernel(MmParams p)
     auto min_stage = [&](int i) { return lds + 2 * kLdsMain + (i & 1) * kLdsMin; };
     auto dsc_stage = [&](int i) { return reinterpret_cast<float *>(lds + 2 * kLdsMain + 2 * kLdsMin) + (i & 1) * BN; };
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 2, wn = wave & 3;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int t0 = blockIdx.x * BM, r0 = blockIdx.y * BN;
     const int nsb = p.cols / 256, nsteps = nsb * 4;
-    const size_t row_bytes = (size_t)nsb * 144;
 
-    // loader roles: four threads per tile row
-    const int lrow = tid >> 2, lq = tid & 3;
-    const uint8_t *wrow = p.W + (size_t)min(r0 + lrow, p.rows - 1) * row_bytes;
-    const _Float16 *xrow = p.Xh + (size_t)min(t0 + lrow, p.batch - 1) * p.cols;
-    const _Float16 *sxrow = p.SxA + (size_t)min(t0 + lrow, p.batch - 1) * nsb * 32;
+    if (wave >= 4) {
+        // ------------------------------------------------------------------ loaders
+        const int lt = tid - 256, lrow = lt >> 1, lh = lt & 1;   // two threads per tile row
+        const size_t row_bytes = (size_t)nsb * 144;
+        const uint8_t *wrow = p.W + (size_t)min(r0 + lrow, p.rows - 1) * row_bytes;
+        const _Float16 *xrow = p.Xh + (size_t)min(t0 + lrow, p.batch - 1) * p.cols;
+        const _Float16 *sxrow = p.SxA + (size_t)min(t0 + lrow, p.batch - 1) * nsb * 32;
 
-    auto fetch_x = [&](int step, XRegs &r) __attribute__((always_inline)) {
-        const int sb = step >> 2, g = step & 3;
-        const u32x4_t *xs = reinterpret_cast<const u32x4_t *>(xrow + sb * 256 + 64 * g + 16 * lq);
-        r.x0 = xs[0]; r.x1 = xs[1];
-    };
-    auto fetch_sb = [&](int sb, SbRegs &r) __attribute__((always_inline)) {
-        const u32x4_t *w = reinterpret_cast<const u32x4_t *>(wrow + (size_t)sb * 144);
-        r.hdr = w[0];
-        r.qa = w[1 + 2 * lq];
-        r.qb = w[2 + 2 * lq];
-        r.sx = *reinterpret_cast<const u32x4_t *>(sxrow + sb * 32 + 8 * lq);
-    };
-    // G = the step's group: its 32 quant bytes sit in lane G of every quad; this thread converts bytes
-    // 8*lq .. 8*lq+7 of them (dwords 2*lq, 2*lq+1), fetched with quad broadcasts and a per-lane pick
-    auto stage = [&](int step, auto gtag, const XRegs &xr, const SbRegs &w) __attribute__((always_inline)) {
-        constexpr int G = decltype(gtag)::value;
-        const int sb = step >> 2;
-        _Float16 *As = main_stage(step), *Bs = As + BM * PITCH;
-        {
-            u32x4_t *dst = reinterpret_cast<u32x4_t *>(&As[lrow * PITCH + 16 * lq]);
-            dst[0] = xr.x0; dst[1] = xr.x1;
-        }
-        {
-            const uint32_t own[8] = {w.qa.x, w.qa.y, w.qa.z, w.qa.w, w.qb.x, w.qb.y, w.qb.z, w.qb.w};
-            uint32_t bc[8];
+        auto fetch_x = [&](int step, XRegs &r) __attribute__((always_inline)) {
+            const int sb = step >> 2, g = step & 3;
+            const u32x4_t *xs = reinterpret_cast<const u32x4_t *>(xrow + sb * 256 + 64 * g + 32 * lh);
 #pragma unroll
-            for (int j = 0; j < 8; j++) bc[j] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)own[j], G * 0x55, 0xF, 0xF, true);
-            const uint32_t q[2] = {lq & 2 ? (lq & 1 ? bc[6] : bc[4]) : (lq & 1 ? bc[2] : bc[0]),
-                                   lq & 2 ? (lq & 1 ? bc[7] : bc[5]) : (lq & 1 ? bc[3] : bc[1])};
-            const uint4 s = q4k_group_scales(w.hdr.y, w.hdr.z, w.hdr.w, G);   // sc_lo, mn_lo, sc_hi, mn_hi
-            uint32_t lo[4], hi[4];
+            for (int i = 0; i < 4; i++) r.x[i] = xs[i];
+        };
+        auto fetch_sb = [&](int sb, SbRegs &r) __attribute__((always_inline)) {
+            const u32x4_t *w = reinterpret_cast<const u32x4_t *>(wrow + (size_t)sb * 144);
+            r.hdr = w[0];
 #pragma unroll
-            for (int i = 0; i < 2; i++) {
-                const uint32_t t4 = q[i] >> 4;
-                lo[2 * i] = pair_f16(q[i] & 0x000F000Fu, s.x);
-                lo[2 * i + 1] = pair_f16((q[i] >> 8) & 0x000F000Fu, s.x);
-                hi[2 * i] = pair_f16(t4 & 0x000F000Fu, s.z);
-                hi[2 * i + 1] = pair_f16((t4 >> 8) & 0x000F000Fu, s.z);
+            for (int i = 0; i < 4; i++) r.q[i] = w[1 + 4 * lh + i];
+            const u32x4_t *sx = reinterpret_cast<const u32x4_t *>(sxrow + sb * 32 + 16 * lh);
+            r.sx0 = sx[0];
+            r.sx1 = sx[1];
+        };
+        // G = the step's group: its 32 quant bytes sit in lane G/2 of every pair, registers q[2*(G%2)] and
+        // q[2*(G%2)+1]; this thread converts bytes 16*lh .. 16*lh+15 of them
+        auto stage = [&](int step, auto gtag, const XRegs &xr, const SbRegs &w) __attribute__((always_inline)) {
+            constexpr int G = decltype(gtag)::value;
+            const int sb = step >> 2;
+            _Float16 *As = main_stage(step), *Bs = As + BM * PITCH;
+            {
+                u32x4_t *dst = reinterpret_cast<u32x4_t *>(&As[lrow * PITCH + 32 * lh]);
+#pragma unroll
+                for (int i = 0; i < 4; i++) dst[i] = xr.x[i];
             }
-            *reinterpret_cast<uint4 *>(&Bs[lrow * PITCH + 8 * lq]) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
-            *reinterpret_cast<uint4 *>(&Bs[lrow * PITCH + 32 + 8 * lq]) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
-        }
-        if (G == 0) {
-            // bias + mins of this superblock, for the short second product after its fourth step
-            _Float16 *A2s = min_stage(sb), *B2s = A2s + BM * PITCH2;
-            const float d = half_bits_to_f32(w.hdr.x & 0xFFFFu), dmin = half_bits_to_f32(w.hdr.x >> 16);
-            // this thread covers group lq of its row: sub-blocks 2*lq and 2*lq+1
-            const uint4 s = q4k_group_scales(w.hdr.y, w.hdr.z, w.hdr.w, lq);
-            const float c0 = -(dmin * (float)s.y + 1024.f * d), c1 = -(dmin * (float)s.w + 1024.f * d);
-            const _Float16 h0 = (_Float16)c0, h1 = (_Float16)c1;
-            const _Float16 l0 = (_Float16)(c0 - (float)h0), l1 = (_Float16)(c1 - (float)h1);
-            const uint32_t hi2 = (uint32_t)__builtin_bit_cast(uint16_t, h0) | ((uint32_t)__builtin_bit_cast(uint16_t, h1) << 16);
-            const uint32_t lo2 = (uint32_t)__builtin_bit_cast(uint16_t, l0) | ((uint32_t)__builtin_bit_cast(uint16_t, l1) << 16);
-            // row layout (32 halves): hi[8] | lo[8] | hi[8] | 0[8]; this thread owns halves 2*lq, 2*lq+1 of each octet
-            uint32_t *b2 = reinterpret_cast<uint32_t *>(&B2s[lrow * PITCH2 + 2 * lq]);
-            b2[0] = hi2;
-            b2[4] = lo2;
-            b2[8] = hi2;
-            b2[12] = 0u;
-            if (lq == 0) dsc_stage(sb)[lrow] = d;
-            *reinterpret_cast<u32x4_t *>(&A2s[lrow * PITCH2 + 8 * lq]) = w.sx;
-        }
-    };
+            {
+                constexpr int kSrc = (G >> 1) ? 0xF5 : 0xA0;   // quad_perm [1,1,3,3] : [0,0,2,2]
+                const u32x4_t c0 = w.q[2 * (G & 1)], c1 = w.q[2 * (G & 1) + 1];
+                uint32_t q[4];
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const uint32_t b0 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)c0[j], kSrc, 0xF, 0xF, true);
+                    const uint32_t b1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)c1[j], kSrc, 0xF, 0xF, true);
+                    q[j] = lh ? b1 : b0;
+                }
+                const uint4 s = q4k_group_scales(w.hdr.y, w.hdr.z, w.hdr.w, G);   // sc_lo, mn_lo, sc_hi, mn_hi
+                uint32_t lo[8], hi[8];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const uint32_t t4 = q[i] >> 4;
+                    lo[2 * i] = pair_f16(q[i] & 0x000F000Fu, s.x);
+                    lo[2 * i + 1] = pair_f16((q[i] >> 8) & 0x000F000Fu, s.x);
+                    hi[2 * i] = pair_f16(t4 & 0x000F000Fu, s.z);
+                    hi[2 * i + 1] = pair_f16((t4 >> 8) & 0x000F000Fu, s.z);
+                }
+                uint4 *dlo = reinterpret_cast<uint4 *>(&Bs[lrow * PITCH + 16 * lh]);
+                uint4 *dhi = reinterpret_cast<uint4 *>(&Bs[lrow * PITCH + 32 + 16 * lh]);
+                dlo[0] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+                dlo[1] = make_uint4(lo[4], lo[5], lo[6], lo[7]);
+                dhi[0] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+                dhi[1] = make_uint4(hi[4], hi[5], hi[6], hi[7]);
+            }
+            if (G == 0) {
+                // bias + mins of this superblock, for the short second product after its fourth step
+                _Float16 *A2s = min_stage(sb), *B2s = A2s + BM * PITCH2;
+                const float d = half_bits_to_f32(w.hdr.x & 0xFFFFu), dmin = half_bits_to_f32(w.hdr.x >> 16);
+                // this thread covers sub-blocks 4*lh .. 4*lh+3 of its row: groups 2*lh, 2*lh+1
+                uint32_t hi2[2], lo2[2];
+#pragma unroll
+                for (int gg = 0; gg < 2; gg++) {
+                    const uint4 s = q4k_group_scales(w.hdr.y, w.hdr.z, w.hdr.w, 2 * lh + gg);
+                    const float c0 = -(dmin * (float)s.y + 1024.f * d), c1 = -(dmin * (float)s.w + 1024.f * d);
+                    const _Float16 h0 = (_Float16)c0, h1 = (_Float16)c1;
+                    const _Float16 l0 = (_Float16)(c0 - (float)h0), l1 = (_Float16)(c1 - (float)h1);
+                    hi2[gg] = (uint32_t)__builtin_bit_cast(uint16_t, h0) | ((uint32_t)__builtin_bit_cast(uint16_t, h1) << 16);
+                    lo2[gg] = (uint32_t)__builtin_bit_cast(uint16_t, l0) | ((uint32_t)__builtin_bit_cast(uint16_t, l1) << 16);
+                }
+                // row layout (32 halves): hi[8] | lo[8] | hi[8] | 0[8]; this thread owns halves 4*lh .. +3 of each octet
+                uint2 *b2 = reinterpret_cast<uint2 *>(&B2s[lrow * PITCH2 + 4 * lh]);
+                b2[0] = make_uint2(hi2[0], hi2[1]);
+                b2[2] = make_uint2(lo2[0], lo2[1]);
+                b2[4] = make_uint2(hi2[0], hi2[1]);
+                b2[6] = make_uint2(0u, 0u);
+                if (lh == 0) dsc_stage(sb)[lrow] = d;
+                u32x4_t *dst = reinterpret_cast<u32x4_t *>(&A2s[lrow * PITCH2 + 16 * lh]);
+                dst[0] = w.sx0;
+                dst[1] = w.sx1;
+            }
+        };
 
-    f16v F[2], Cp[2];
+        // Named register sets (an array, even with constant indices, ends up in scratch here): set g serves the
+        // steps 4*sb + g and is refilled for step s+4 right after step s+... its own step was staged, so a load
+        // has three whole steps to arrive.  Loads past the end re-read the last step / superblock, unused.
+        XRegs xr0, xr1, xr2, xr3;
+        SbRegs wcur, wnext;
+        fetch_x(0, xr0);   // nsteps is a multiple of 4
+        fetch_x(1, xr1);
+        fetch_x(2, xr2);
+        fetch_x(3, xr3);
+        fetch_sb(0, wcur);
+        stage(0, std::integral_constant<int, 0>{}, xr0, wcur);
+        __syncthreads();
+        auto step_body = [&](int sb, auto gtag, XRegs &mine, const XRegs &next) __attribute__((always_inline)) {
+            constexpr int g = decltype(gtag)::value;
+            const int step = 4 * sb + g;
+            fetch_x(min(step + 4, nsteps - 1), mine);   // this set's own step was staged one iteration ago
+            if (g == 0) fetch_sb(min(sb + 1, nsb - 1), wnext);
+            if (step + 1 < nsteps) {
+                if (g == 3) wcur = wnext;
+                stage(step + 1, std::integral_constant<int, (g + 1) & 3>{}, next, wcur);
+            }
+            __syncthreads();
+        };
+        for (int sb = 0; sb < nsb; sb++) {
+            step_body(sb, std::integral_constant<int, 0>{}, xr0, xr1);
+            step_body(sb, std::integral_constant<int, 1>{}, xr1, xr2);
+            step_body(sb, std::integral_constant<int, 2>{}, xr2, xr3);
+            step_body(sb, std::integral_constant<int, 3>{}, xr3, xr0);
+        }
+        return;
+    }
+
+    // ---------------------------------------------------------------------- multipliers
+    const int wm = wave >> 1, wn = wave & 1;
+    f16v F[2][2], Cp[2][2];
 #pragma unroll
     for (int a = 0; a < 2; a++)
 #pragma unroll
-        for (int i = 0; i < 16; i++) { F[a][i] = 0.f; Cp[a][i] = 0.f; }
-
+        for (int b = 0; b < 2; b++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) { F[a][b][i] = 0.f; Cp[a][b][i] = 0.f; }
     const int lm = lane & 31, lk = (lane >> 5) * 8;
+    __syncthreads();   // stage 0 is written
 
-    // The activations of step s+4 and, at a superblock's first step, the weights of the next superblock are
-    // requested while step s is multiplied and step s+1 is staged: a load has three whole steps to arrive.  Set g
-    // of xr serves the steps 4*sb + g, which keeps every register index a compile-time constant.
-    XRegs xr0, xr1, xr2, xr3;   // named, not an array: an array, even with constant indices, ends up in scratch here
-    SbRegs wcur, wnext;
-    fetch_x(0, xr0);   // nsteps is a multiple of 4
-    fetch_x(1, xr1);
-    fetch_x(2, xr2);
-    fetch_x(3, xr3);
-    fetch_sb(0, wcur);
-    stage(0, std::integral_constant<int, 0>{}, xr0, wcur);
-    __syncthreads();
-
-    // the four steps of a superblock are written out, so that "is this the superblock's first / last step" and
-    // every register-set index are compile-time facts and the accumulators stay where the matrix cores want them
-    auto step_body = [&](int sb, auto gtag, XRegs &mine, const XRegs &next) __attribute__((always_inline)) {
+    auto mul_step = [&](int sb, auto gtag) __attribute__((always_inline)) {
         constexpr int g = decltype(gtag)::value;
         const int step = 4 * sb + g;
-        const bool more = step + 1 < nsteps;
-        // unconditional (past the end they re-read the last step / superblock and nothing uses the result): a
-        // conditional update would push the register sets into scratch memory
-        fetch_x(min(step + 4, nsteps - 1), mine);   // this set's own step was staged one iteration ago
-        if (g == 0) fetch_sb(min(sb + 1, nsb - 1), wnext);
         const _Float16 *As = main_stage(step), *Bs = As + BM * PITCH;
 #pragma unroll
         for (int ks = 0; ks < KS / 16; ks++) {
-            h8 a[2], b;
+            h8 a[2], b[2];
 #pragma unroll
             for (int mt = 0; mt < 2; mt++)
                 a[mt] = *reinterpret_cast<const h8 *>(&As[(wm * 64 + mt * 32 + lm) * PITCH + 16 * ks + lk]);
-            b = *reinterpret_cast<const h8 *>(&Bs[(wn * 32 + lm) * PITCH + 16 * ks + lk]);
 #pragma unroll
-            for (int mt = 0; mt < 2; mt++) Cp[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mt], b, Cp[mt], 0, 0, 0);
+            for (int nt = 0; nt < 2; nt++)
+                b[nt] = *reinterpret_cast<const h8 *>(&Bs[(wn * 64 + nt * 32 + lm) * PITCH + 16 * ks + lk]);
+#pragma unroll
+            for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+                for (int nt = 0; nt < 2; nt++)
+                    Cp[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mt], b[nt], Cp[mt][nt], 0, 0, 0);
         }
         if (g == 3) {
             // ---- end of the superblock: bias + mins through the short second product, then the row scale
             const _Float16 *A2s = min_stage(sb), *B2s = A2s + BM * PITCH2;
+            const float *dsc = dsc_stage(sb);
 #pragma unroll
             for (int ks = 0; ks < 2; ks++) {
-                h8 a[2], b;
+                h8 a[2], b[2];
 #pragma unroll
                 for (int mt = 0; mt < 2; mt++)
                     a[mt] = *reinterpret_cast<const h8 *>(&A2s[(wm * 64 + mt * 32 + lm) * PITCH2 + 16 * ks + lk]);
-                b = *reinterpret_cast<const h8 *>(&B2s[(wn * 32 + lm) * PITCH2 + 16 * ks + lk]);
 #pragma unroll
-                for (int mt = 0; mt < 2; mt++) F[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mt], b, F[mt], 0, 0, 0);
+                for (int nt = 0; nt < 2; nt++)
+                    b[nt] = *reinterpret_cast<const h8 *>(&B2s[(wn * 64 + nt * 32 + lm) * PITCH2 + 16 * ks + lk]);
+#pragma unroll
+                for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+                    for (int nt = 0; nt < 2; nt++)
+                        F[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mt], b[nt], F[mt][nt], 0, 0, 0);
             }
-            const float dn = dsc_stage(sb)[wn * 32 + lm];
 #pragma unroll
-            for (int mt = 0; mt < 2; mt++)
+            for (int nt = 0; nt < 2; nt++) {
+                const float dn = dsc[wn * 64 + nt * 32 + lm];
 #pragma unroll
-                for (int i = 0; i < 16; i++) {
-                    F[mt][i] = fmaf(dn, Cp[mt][i], F[mt][i]);
-                    Cp[mt][i] = 0.f;
-                }
-        }
-        if (more) {
-            if (g == 3) wcur = wnext;
-            stage(step + 1, std::integral_constant<int, (g + 1) & 3>{}, next, wcur);
+                for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++) {
+                        F[mt][nt][i] = fmaf(dn, Cp[mt][nt][i], F[mt][nt][i]);
+                        Cp[mt][nt][i] = 0.f;
+                    }
+            }
         }
         __syncthreads();
     };
     for (int sb = 0; sb < nsb; sb++) {
-        step_body(sb, std::integral_constant<int, 0>{}, xr0, xr1);
-        step_body(sb, std::integral_constant<int, 1>{}, xr1, xr2);
-        step_body(sb, std::integral_constant<int, 2>{}, xr2, xr3);
-        step_body(sb, std::integral_constant<int, 3>{}, xr3, xr0);
+        mul_step(sb, std::integral_constant<int, 0>{});
+        mul_step(sb, std::integral_constant<int, 1>{});
+        mul_step(sb, std::integral_constant<int, 2>{});
+        mul_step(sb, std::integral_constant<int, 3>{});
     }
 
     // accumulator layout of the 32x32 tile: column = lane % 32, row = 8*(i/4) + 4*(lane/32) + i%4
 #pragma unroll
-    for (int mt = 0; mt < 2; mt++) {
-        const int r = r0 + wn * 32 + lm;
+    for (int mt = 0; mt < 2; mt++)
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-            const int t = t0 + wm * 64 + mt * 32 + 8 * (i / 4) + 4 * (lane >> 5) + (i & 3);
-            if (t < p.batch && r < p.rows) p.Y[(size_t)t * p.rows + r] = F[mt][i];
+        for (int nt = 0; nt < 2; nt++) {
+            const int r = r0 + wn * 64 + nt * 32 + lm;
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int t = t0 + wm * 64 + mt * 32 + 8 * (i / 4) + 4 * (lane >> 5) + (i & 3);
+                if (t < p.batch && r < p.rows) p.Y[(size_t)t * p.rows + r] = F[mt][nt][i];
+            }
         }
-    }
 }
 
 int launch_mul_mm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)

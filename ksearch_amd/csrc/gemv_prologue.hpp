@@ -52,7 +52,7 @@ __host__ __device__ constexpr size_t xs_image_bytes(int cols)
 template <int XF>
 __host__ __device__ constexpr size_t xs_bytes(int cols)
 {
-    return xs_image_bytes<XF>(cols) + 64;   // + reduction scratch
+    return xs_image_bytes<XF>(cols) + 128;   // + reduction scratch (4 sums x up to 8 waves)
 }
 
 // max / sum over 8 consecutive lanes (one 32-element sub-block at 4 elements per lane)
@@ -208,17 +208,51 @@ __device__ __forceinline__ void stage_finish(const Prologue &pr, uint8_t *lds, i
         }
         return;
     }
+    // One pass, one reduction: with a = rsqrt(mean(y^2) + eps) the second norm's sum of squares is
+    //   sum (res + a*y*wp)^2 = sum res^2 + 2a sum res*(y*wp) + a^2 sum (y*wp)^2,
+    // so all four sums are taken together and cross the workgroup behind a single barrier.
     float4 *v = s.x;
-    float ss = 0.f;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    const bool add = pr.kind == kAddThenRms;
 #pragma unroll
     for (int k = 0; k < kStageP; k++) {
-        const int i = tid + k * NT;
-        if (wbase + k * NT < n4) ss += (v[k].x * v[k].x + v[k].y * v[k].y) + (v[k].z * v[k].z + v[k].w * v[k].w);
+        if (wbase + k * NT < n4) {
+            const float y4[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
+            const float r4[4] = {s.rs[k].x, s.rs[k].y, s.rs[k].z, s.rs[k].w};
+            const float w4[4] = {s.wp[k].x, s.wp[k].y, s.wp[k].z, s.wp[k].w};
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                acc[0] = fmaf(y4[e], y4[e], acc[0]);
+                if (add) {
+                    const float yw = y4[e] * w4[e];
+                    acc[1] = fmaf(r4[e], r4[e], acc[1]);
+                    acc[2] = fmaf(r4[e], yw, acc[2]);
+                    acc[3] = fmaf(yw, yw, acc[3]);
+                }
+            }
+        }
     }
-    ss = block_sum<NT>(ss, red);
-    float inv = 1.0f / sqrtf(ss / (float)cols + pr.eps);
-    if (pr.kind == kAddThenRms) {
-        float ss2 = 0.f;
+    {
+        const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            if (j == 0 || add) {
+                const float wsum = wave_sum(acc[j]);
+                if (lane == 0) red[wave * 4 + j] = wsum;
+            }
+        }
+        __syncthreads();   // `red` has no earlier use in the kernel, so one barrier is enough
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            acc[j] = 0.f;
+            if (j == 0 || add) {
+#pragma unroll
+                for (int w = 0; w < NT / 64; w++) acc[j] += red[w * 4 + j];
+            }
+        }
+    }
+    float inv = 1.0f / sqrtf(acc[0] / (float)cols + pr.eps);
+    if (add) {
 #pragma unroll
         for (int k = 0; k < kStageP; k++) {
             const int i = tid + k * NT;
@@ -228,11 +262,10 @@ __device__ __forceinline__ void stage_finish(const Prologue &pr, uint8_t *lds, i
                 v[k].y = r.y + v[k].y * inv * w.y;
                 v[k].z = r.z + v[k].z * inv * w.z;
                 v[k].w = r.w + v[k].w * inv * w.w;
-                ss2 += (v[k].x * v[k].x + v[k].y * v[k].y) + (v[k].z * v[k].z + v[k].w * v[k].w);
                 if (blockIdx.x == 0) stg_f4(pr.x_out, i, v[k]);
             }
         }
-        ss2 = block_sum<NT>(ss2, red);
+        const float ss2 = fmaf(inv * inv, acc[3], fmaf(2.0f * inv, acc[2], acc[1]));
         inv = 1.0f / sqrtf(ss2 / (float)cols + pr.eps);
     }
 #pragma unroll

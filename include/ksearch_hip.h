@@ -131,8 +131,19 @@ enum ksh_kind {
      *     rope f32[max_seq, hd], k f32[n_kv*hd], k_norm f32[hd], v f32[n_kv*hd],
      *     meta f32[4] = {tlen, start, window, pos} with start + tlen - 1 == pos
      * out: K cache, V cache (row pos is written), tmp f32[n_q, nwg, hd+2],
-     *      out f32[n_q*hd].  Built for hd 128 / 256, up to 8 q heads per kv head. */
+     *      out f32[n_q*hd].  Built for hd 128 / 256, up to 8 q heads per kv head.
+     * With dims[5] = 1 the partitions are not merged: the outputs are K cache,
+     * V cache and parts = { o f32[n_q, nwg, hd] (unnormalised), ml f32[n_q, nwg, 2]
+     * (running max, sum) } in one buffer, for KSH_ATTN_MERGE_MATVEC. */
     KSH_ATTEND_DECODE = 22,
+    /* SdpaMwgReduce (crates/ksearch_metal/src/lower.rs:5897-6087) folded into the
+     * GEMV that consumes the attention output: every workgroup merges the
+     * partitions' states itself while its weights are in flight, which takes
+     * the cross-workgroup hand-over out of the attention launch.
+     * dims: rows, n_q, hd, nwg (<= 8; n_q*hd <= 2048, hd a power of two).
+     * in: W Q4_K[rows, n_q*hd], parts (as written by KSH_ATTEND_DECODE with dims[5] = 1)
+     * out: y f32[rows] */
+    KSH_ATTN_MERGE_MATVEC = 23,
     KSH_KIND_COUNT
 };
 

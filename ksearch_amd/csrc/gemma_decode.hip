@@ -29,6 +29,8 @@
 //     every id for one read-back at the end.
 #include <chrono>
 #include <cmath>
+#include <cstdlib>
+#include <algorithm>
 #include <memory>
 #include <vector>
 
@@ -76,13 +78,15 @@ struct ksh_gemma {
             *history = nullptr;
     std::vector<ksh_buf *> kv_k, kv_v;
     ksh_kernel *k_embed = nullptr, *k_qkv_first = nullptr, *k_qkv = nullptr, *k_head = nullptr, *k_sdpa = nullptr, *k_attend = nullptr,
+               *k_attend_parts = nullptr, *k_oproj_merge = nullptr,   // short contexts: the o-projection merges the partitions
                *k_oproj = nullptr, *k_add_then = nullptr, *k_gate_up = nullptr, *k_down = nullptr,
                *k_lm_head = nullptr, *k_argmax = nullptr;
-    ksh_graph *g_body = nullptr, *g_full = nullptr;
+    ksh_graph *g_body[2] = {nullptr, nullptr}, *g_full[2] = {nullptr, nullptr};   // [1]: the short-context form
     int pos = 0;
     int launches_full = 0;
     int nwg = 16;
     int sdpa_launches = 2;
+    int short_context = 0;   // positions below this use the short-context graph
 };
 
 namespace {
@@ -122,8 +126,15 @@ int enc(ksh_gemma *m, ksh_kernel *k, std::initializer_list<ksh_buf *> in, std::i
     return ksh_encode(m->ctx, k, ib, nullptr, ni, ob, nullptr, no);
 }
 
+// Up to this many cached positions the attention launch leaves its (then 8) partitions unmerged and the
+// o-projection folds them in its prologue: 0.8 us per layer less at 320 positions, 1.5 us more at 1500,
+// where 16 partitions and the merge inside the attention launch win.
+// (KSEARCH_SHORT_CONTEXT overrides the limit when the model is built; 0 switches the short form off.)
+constexpr int kShortContext = 640;
+constexpr int kShortPartitions = 8;
+
 // one token: embedding gather -> layers (-> logits -> argmax) -> advance
-int encode_token(ksh_gemma *m, bool want_logits, int &launches)
+int encode_token(ksh_gemma *m, bool want_logits, bool short_ctx, int &launches)
 {
     const ksh_gemma_cfg &c = m->c;
     launches = 0;
@@ -140,7 +151,11 @@ int encode_token(ksh_gemma *m, bool want_logits, int &launches)
                 return 1;
             std::swap(cur, other);
         }
-        if (m->k_attend) {
+        if (short_ctx) {
+            if (enc(m, m->k_attend_parts, {m->tq, L.q_norm, m->rope, m->tk, L.k_norm, m->tv, m->meta},
+                    {m->kv_k[l], m->kv_v[l], m->attn_tmp}, launches))
+                return 1;
+        } else if (m->k_attend) {
             if (enc(m, m->k_attend, {m->tq, L.q_norm, m->rope, m->tk, L.k_norm, m->tv, m->meta},
                     {m->kv_k[l], m->kv_v[l], m->attn_tmp, m->to}, launches))
                 return 1;
@@ -151,7 +166,8 @@ int encode_token(ksh_gemma *m, bool want_logits, int &launches)
             if (enc(m, m->k_sdpa, {m->tq, m->kv_k[l], m->kv_v[l], m->meta}, {m->attn_tmp, m->to}, launches)) return 1;
             if (m->sdpa_launches == 2) launches += 1;   // partials, then the merge
         }
-        if (enc(m, m->k_oproj, {L.wo, m->to}, {m->y}, launches)) return 1;
+        if (short_ctx ? enc(m, m->k_oproj_merge, {L.wo, m->attn_tmp}, {m->y}, launches) : enc(m, m->k_oproj, {L.wo, m->to}, {m->y}, launches))
+            return 1;
         if (enc(m, m->k_gate_up, {L.wgate, L.wup, m->y, L.ffn_norm, L.post_attn_norm, cur}, {m->ff, other}, launches)) return 1;
         std::swap(cur, other);
         if (enc(m, m->k_down, {L.wdown, m->ff}, {m->y}, launches)) return 1;
@@ -179,14 +195,15 @@ int run_token(ksh_gemma *m, bool want_logits, bool use_graph)
 {
     if (m->pos >= m->c.max_seq) return set_error("max_seq exceeded");   // gemma_prim.rs:882-884
     int n = 0;
+    const bool short_ctx = m->k_attend_parts && m->pos < m->short_context;
     if (!use_graph) {
-        if (encode_token(m, want_logits, n)) return 1;
+        if (encode_token(m, want_logits, short_ctx, n)) return 1;
     } else {
-        ksh_graph *&g = want_logits ? m->g_full : m->g_body;
+        ksh_graph *&g = want_logits ? m->g_full[short_ctx] : m->g_body[short_ctx];
         if (!g) {
             if (ksh_synchronize(m->ctx)) return 1;
             if (ksh_graph_begin(m->ctx)) return 1;
-            if (encode_token(m, want_logits, n)) {
+            if (encode_token(m, want_logits, short_ctx, n)) {
                 ksh_graph *dead = nullptr;
                 ksh_graph_end(m->ctx, &dead);
                 ksh_graph_destroy(dead);
@@ -259,7 +276,7 @@ int ksh_gemma_create(ksh_ctx *ctx, const ksh_gemma_cfg *cfg, const ksh_gemma_lay
         if (ksh_buffer_alloc(ctx, tab.size() * 4, tab.data(), &g->rope)) return 1;
         g->bufs.owned.push_back(g->rope);
     }
-    if (alloc(g, (size_t)c.n_q * g->nwg * (c.hd + 2) * 4, &g->attn_tmp)) return 1;
+    if (alloc(g, (size_t)c.n_q * std::max(g->nwg, kShortPartitions) * (c.hd + 2) * 4, &g->attn_tmp)) return 1;
 
     const float embed_scale = std::sqrt((float)c.hidden);   // gemma_prim.rs:683
     if (get(g, KSH_COPY_SCALE_INDEXED, {c.hidden, c.vocab}, {KSH_Q6K}, {embed_scale}, &g->k_embed) ||
@@ -277,6 +294,13 @@ int ksh_gemma_create(ksh_ctx *ctx, const ksh_gemma_cfg *cfg, const ksh_gemma_lay
         if (get(g, KSH_ATTEND_DECODE, {c.n_q, c.n_kv, c.hd, c.max_seq, g->nwg}, {KSH_Q40, KSH_F32}, {c.eps, c.attn_scale},
                 &g->k_attend))
             return 1;
+        g->short_context = kShortContext;
+        if (const char *e = getenv("KSEARCH_SHORT_CONTEXT")) g->short_context = atoi(e);
+        if (g->short_context > 0 && qd <= 2048 && (c.hd & (c.hd - 1)) == 0 &&
+            (get(g, KSH_ATTEND_DECODE, {c.n_q, c.n_kv, c.hd, c.max_seq, kShortPartitions, 1}, {KSH_Q40, KSH_F32},
+                 {c.eps, c.attn_scale}, &g->k_attend_parts) ||
+             get(g, KSH_ATTN_MERGE_MATVEC, {c.hidden, c.n_q, c.hd, kShortPartitions}, {KSH_Q4K, KSH_F32}, {}, &g->k_oproj_merge)))
+            return 1;
     } else {
         if (get(g, KSH_RMSNORM_PER_HEAD_QKV_Q40, {c.n_q, c.n_kv, c.hd, c.max_seq}, {}, {c.eps}, &g->k_head) ||
             get(g, KSH_SDPA_SLOTS, {c.n_q, c.n_kv, c.hd, c.max_seq, 1, g->nwg}, {KSH_Q40, KSH_F32}, {c.attn_scale}, &g->k_sdpa))
@@ -291,8 +315,10 @@ void ksh_gemma_destroy(ksh_gemma *m)
 {
     if (!m) return;
     ksh_synchronize(m->ctx);
-    ksh_graph_destroy(m->g_body);
-    ksh_graph_destroy(m->g_full);
+    for (int i = 0; i < 2; i++) {
+        ksh_graph_destroy(m->g_body[i]);
+        ksh_graph_destroy(m->g_full[i]);
+    }
     delete m;
 }
 

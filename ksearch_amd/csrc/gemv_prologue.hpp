@@ -6,6 +6,9 @@
 //   kAddThenRms x_new = res + (y*inv)*w_post, written back by workgroup 0 as the
 //               residual stream, then (x_new*inv2)*w_norm     (RmsNormAddThenRmsNorm, lower.rs:3926-4077,
 //               folded into the consumer GEMV)
+//   kMergeParts the merge of a split-KV attention's partitions (SdpaMwgReduce,
+//               lower.rs:5897-6087): x = sum_p w_p o_p / sum_p w_p l_p with
+//               w_p = exp(m_p - max m); one float4 per thread, no reduction
 //
 // and two LDS formats, selected at compile time:
 //
@@ -22,17 +25,19 @@
 
 namespace ksh {
 
-enum { kPlain = 0, kRms = 1, kAddThenRms = 2 };
+enum { kPlain = 0, kRms = 1, kAddThenRms = 2, kMergeParts = 3 };
+constexpr int kMergeMaxParts = 8;
 enum { kXF32 = 0, kXI8 = 3, kXQ6 = 6 };
 
 struct Prologue {
-    const float *x;        // kPlain/kRms: the vector; kAddThenRms: y
-    const float *w_norm;   // kRms / kAddThenRms
+    const float *x;        // kPlain/kRms: the vector; kAddThenRms: y; kMergeParts: o[heads][nwg][hd]
+    const float *w_norm;   // kRms / kAddThenRms; kMergeParts: (m, l)[heads][nwg]
     const float *w_post;   // kAddThenRms
     const float *res;      // kAddThenRms
     float *x_out;          // kAddThenRms: residual stream out
     float eps;
     int kind;
+    int nwg, hd_log2;      // kMergeParts
 };
 
 __host__ __device__ constexpr int xs_f32_floats(int cols) { return cols + (cols >> 6) * 4; }
@@ -169,6 +174,24 @@ __device__ __forceinline__ void stage_fetch(const Prologue &pr, int cols, StageR
     // n4 is a multiple of 64, so "this float4 exists" is a per-wave fact: keep it
     // in scalar registers and the loads stay unpredicated
     const int wbase = __builtin_amdgcn_readfirstlane(threadIdx.x & ~63), tid = wbase + (threadIdx.x & 63), n4 = cols / 4;
+    if (pr.kind == kMergeParts) {
+        // one float4 of the output per thread (host-checked: n4 <= NT, nwg <= 8): its
+        // eight partitions' values and (m, l) pairs; partitions past nwg re-read the
+        // last one, so that the number of loads is fixed
+        if (wbase < n4) {
+            const int e = tid * 4, h = e >> pr.hd_log2, d = e - (h << pr.hd_log2);
+            const float *o = pr.x + (((size_t)h * pr.nwg) << pr.hd_log2) + d;
+            const float *ml = pr.w_norm + (size_t)h * pr.nwg * 2;
+#pragma unroll
+            for (int q = 0; q < kMergeMaxParts; q++) s.x[q] = ldg_f4(o + ((size_t)min(q, pr.nwg - 1) << pr.hd_log2), 0);
+#pragma unroll
+            for (int q = 0; q < kMergeMaxParts / 2; q++) {
+                const float2 a = ldg_f2(ml, min(2 * q, pr.nwg - 1)), b = ldg_f2(ml, min(2 * q + 1, pr.nwg - 1));
+                s.wn[q] = make_float4(a.x, a.y, b.x, b.y);
+            }
+        }
+        return;
+    }
     if (n4 > NT * kStageX) return;
 #pragma unroll
     for (int k = 0; k < kStageX; k++) {
@@ -196,6 +219,33 @@ __device__ __forceinline__ void stage_finish(const Prologue &pr, uint8_t *lds, i
 {
     const int wbase = __builtin_amdgcn_readfirstlane(threadIdx.x & ~63), tid = wbase + (threadIdx.x & 63), n4 = cols / 4;
     float *red = reinterpret_cast<float *>(lds + xs_image_bytes<XF>(cols));
+    if (pr.kind == kMergeParts) {
+        if (wbase < n4) {
+            float m[kMergeMaxParts], l[kMergeMaxParts];
+#pragma unroll
+            for (int q = 0; q < kMergeMaxParts / 2; q++) {
+                m[2 * q] = s.wn[q].x; l[2 * q] = s.wn[q].y;
+                m[2 * q + 1] = s.wn[q].z; l[2 * q + 1] = s.wn[q].w;
+            }
+            float M = m[0];
+#pragma unroll
+            for (int q = 1; q < kMergeMaxParts; q++) M = fmaxf(M, m[q]);
+            float L = 0.f;
+            float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+            for (int q = 0; q < kMergeMaxParts; q++) {
+                const float w = q < pr.nwg ? __expf(m[q] - M) : 0.f;
+                L = fmaf(w, l[q], L);
+                a.x = fmaf(w, s.x[q].x, a.x);
+                a.y = fmaf(w, s.x[q].y, a.y);
+                a.z = fmaf(w, s.x[q].z, a.z);
+                a.w = fmaf(w, s.x[q].w, a.w);
+            }
+            const float rl = 1.0f / L;   // (the merging attention launch divides; the two differ by an ulp)
+            store_x4<XF>(lds, cols, tid, make_float4(a.x * rl, a.y * rl, a.z * rl, a.w * rl));
+        }
+        return;
+    }
     if (pr.kind == kPlain) {
         if (n4 > NT * kStageX) {
             for (int i = tid; i < n4; i += NT) store_x4<XF>(lds, cols, i, ldg_f4(pr.x, i));

@@ -27,6 +27,12 @@ __device__ __forceinline__ float4 ldg_f4(const float *p, size_t i)
     const f32x4_t v = ((const KSH_GLOBAL f32x4_t *)p)[i];
     return make_float4(v.x, v.y, v.z, v.w);
 }
+__device__ __forceinline__ float2 ldg_f2(const float *p, size_t i)
+{
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    const f32x2_t v = ((const KSH_GLOBAL f32x2_t *)p)[i];
+    return make_float2(v.x, v.y);
+}
 __device__ __forceinline__ void stg_f4(float *p, size_t i, float4 v)
 {
     f32x4_t w;

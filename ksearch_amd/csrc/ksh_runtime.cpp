@@ -51,7 +51,8 @@ static int bind(ksh_kernel &k)
     case KSH_MATVEC_GATE_UP_GELU: return bind_matvec_gate_up_gelu(k);
     case KSH_RMSNORM_MATVEC: return bind_matvec(k);
     case KSH_RMSNORM_MATVEC_QKV:
-    case KSH_RMSNORM_MATVEC_GATE_UP_GELU: return bind_matvec_q4k_family(k);
+    case KSH_RMSNORM_MATVEC_GATE_UP_GELU:
+    case KSH_ATTN_MERGE_MATVEC: return bind_matvec_q4k_family(k);
     case KSH_SDPA_NAIVE:
     case KSH_SDPA_MWG_PART:
     case KSH_SDPA_MWG_REDUCE:

@@ -183,17 +183,18 @@ __device__ __forceinline__ MatvecParams fetch_params(const MatvecParams &p)
     int rows0 = p.rows0, rows1 = p.rows1, rows2 = p.rows2, waves0 = p.waves0, waves1 = p.waves1, waves2 = p.waves2;
     const float *x = p.pro.x, *w_norm = p.pro.w_norm, *w_post = p.pro.w_post, *res = p.pro.res;
     float *x_out = p.pro.x_out;
-    int eps = __float_as_int(p.pro.eps), kind = p.pro.kind, bpr = p.bpr, mode = p.mode;
+    int eps = __float_as_int(p.pro.eps), kind = p.pro.kind, bpr = p.bpr, mode = p.mode, nwg = p.pro.nwg, hd_log2 = p.pro.hd_log2;
     asm volatile("" : "+s"(W0), "+s"(W1), "+s"(W2), "+s"(y0), "+s"(y1), "+s"(y2), "+s"(rows0), "+s"(rows1), "+s"(rows2),
                  "+s"(waves0), "+s"(waves1), "+s"(waves2));
-    asm volatile("" : "+s"(x), "+s"(w_norm), "+s"(w_post), "+s"(res), "+s"(x_out), "+s"(eps), "+s"(kind), "+s"(bpr), "+s"(mode));
+    asm volatile("" : "+s"(x), "+s"(w_norm), "+s"(w_post), "+s"(res), "+s"(x_out), "+s"(eps), "+s"(kind), "+s"(bpr), "+s"(mode),
+                 "+s"(nwg), "+s"(hd_log2));
     MatvecParams q;
     q.W0 = W0; q.W1 = W1; q.W2 = W2;
     q.y0 = y0; q.y1 = y1; q.y2 = y2;
     q.rows0 = rows0; q.rows1 = rows1; q.rows2 = rows2;
     q.waves0 = waves0; q.waves1 = waves1; q.waves2 = waves2;
     q.pro.x = x; q.pro.w_norm = w_norm; q.pro.w_post = w_post; q.pro.res = res; q.pro.x_out = x_out;
-    q.pro.eps = __int_as_float(eps); q.pro.kind = kind;
+    q.pro.eps = __int_as_float(eps); q.pro.kind = kind; q.pro.nwg = nwg; q.pro.hd_log2 = hd_log2;
     q.bpr = bpr; q.mode = mode;
     return q;
 }
@@ -486,8 +487,9 @@ struct Shape {
     int nm;           // matrices per wave (2 for gate||up)
     int64_t rows[3];
     int64_t cols;
-    int prologue;     // kPlain / kRms / kAddThenRms
+    int prologue;     // kPlain / kRms / kAddThenRms / kMergeParts
     float eps;
+    int nwg, hd;      // kMergeParts
 };
 
 Shape shape_of(const ksh_kernel_desc &d)
@@ -506,6 +508,10 @@ Shape shape_of(const ksh_kernel_desc &d)
     case KSH_RMSNORM_MATVEC_GATE_UP_GELU:
         s.n_mat = 2; s.nm = 2; s.rows[0] = s.rows[1] = D[0]; s.cols = D[1];
         s.prologue = D[2] ? kAddThenRms : kRms;
+        break;
+    case KSH_ATTN_MERGE_MATVEC:
+        s.n_mat = 1; s.nm = 1; s.rows[0] = D[0]; s.cols = D[1] * D[2]; s.prologue = kMergeParts;
+        s.hd = (int)D[2]; s.nwg = (int)D[3];
         break;
     }
     s.eps = d.params[0];
@@ -535,6 +541,12 @@ int launch_any(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
     p.pro.kind = s.prologue;
     p.pro.eps = s.eps;
     p.pro.x = (const float *)a.in[s.n_mat];
+    if (s.prologue == kMergeParts) {
+        p.pro.w_norm = p.pro.x + (size_t)s.cols * s.nwg;   // the (m, l) pairs follow the values
+        p.pro.nwg = s.nwg;
+        p.pro.hd_log2 = __builtin_ctz((unsigned)s.hd);
+        return launch_q4k<1>(G, p, total, st);
+    }
     if (s.prologue != kPlain) p.pro.w_norm = (const float *)a.in[s.n_mat + 1];
     if (s.prologue == kAddThenRms) {
         p.pro.w_post = (const float *)a.in[s.n_mat + 2];
@@ -561,18 +573,25 @@ int bind_matvec_q4k_family(ksh_kernel &k)
     if (s.cols <= 0 || s.cols % 256) return set_error("Q4_K matvec: cols=%lld is not a positive multiple of 256", (long long)s.cols);
     if (s.cols > 32768) return set_error("Q4_K matvec: cols=%lld does not fit the LDS staging buffer", (long long)s.cols);
     const int bpr = (int)(s.cols / 256);
-    const Q4kGeom G = pick_geom(k.desc.sched, (int)(s.nm == 2 ? s.rows[0] : total_rows), bpr);
+    Q4kGeom G = pick_geom(k.desc.sched, (int)(s.nm == 2 ? s.rows[0] : total_rows), bpr);
+    if (s.prologue == kMergeParts) {
+        if (s.hd < 4 || (s.hd & (s.hd - 1)) || s.nwg < 1 || s.nwg > kMergeMaxParts)
+            return set_error("attn_merge_matvec: hd=%d must be a power of two, nwg=%d at most %d", s.hd, s.nwg, kMergeMaxParts);
+        if (!k.desc.sched.nsg) { G.NW = 8; if (!k.desc.sched.nr0) G.R = 1; }   // one float4 of the merged vector per thread
+        if (s.cols > (int64_t)4 * G.NW * 64)
+            return set_error("attn_merge_matvec: n_q*hd=%lld exceeds one float4 per thread (%d)", (long long)s.cols, 4 * G.NW * 64);
+    }
     if (lds_for(G.var, (int)s.cols) > 65536)
         return set_error("Q4_K matvec: cols=%lld does not fit the LDS staging buffer", (long long)s.cols);
     if (!geom_ok(G)) return set_error("matvec_q4k: unsupported schedule nr0=%d nsg=%d (nr0 in 1,2,4; nsg in 4,8)", G.R, G.NW);
-    if (s.prologue != kPlain && s.cols > (int64_t)4 * G.NW * 64 * kStageP)
+    if (s.prologue != kPlain && s.prologue != kMergeParts && s.cols > (int64_t)4 * G.NW * 64 * kStageP)
         return set_error("rmsnorm_matvec requires LOCAL staging of the vector (cols=%lld too large)", (long long)s.cols);
     const size_t rb = (size_t)bpr * kQ4kBytes, vb = (size_t)s.cols * 4;
     const int n_y = s.nm == 2 ? 1 : s.n_mat;
     int ni = 0, no = 0;
     for (int m = 0; m < s.n_mat; m++) { k.in_bytes[ni] = (size_t)s.rows[m] * rb; k.in_align[ni++] = 16; }
-    k.in_bytes[ni] = vb; k.in_align[ni++] = 16;
-    if (s.prologue != kPlain) { k.in_bytes[ni] = vb; k.in_align[ni++] = 16; }
+    k.in_bytes[ni] = s.prologue == kMergeParts ? (size_t)s.nwg * (s.cols + 2 * (s.cols / s.hd)) * 4 : vb; k.in_align[ni++] = 16;
+    if (s.prologue == kRms || s.prologue == kAddThenRms) { k.in_bytes[ni] = vb; k.in_align[ni++] = 16; }
     if (s.prologue == kAddThenRms) {
         k.in_bytes[ni] = vb; k.in_align[ni++] = 16;
         k.in_bytes[ni] = vb; k.in_align[ni++] = 16;
@@ -584,7 +603,7 @@ int bind_matvec_q4k_family(ksh_kernel &k)
     int waves = 0;
     if (s.nm == 2) waves = waves_for((int)s.rows[0], G.rpw());
     else for (int m = 0; m < s.n_mat; m++) waves += waves_for((int)s.rows[m], G.rpw());
-    static const char *pre[] = {"", "rms_", "addrms_"};
+    static const char *pre[] = {"", "rms_", "addrms_", "attn_merge_"};
     char base[48];
     snprintf(base, sizeof(base), "%smatvec%s", pre[s.prologue], s.n_mat == 3 ? "_qkv" : s.nm == 2 ? "_gate_up_gelu" : "");
     fill_info(k, G, waves, bpr, base);

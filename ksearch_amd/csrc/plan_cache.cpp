@@ -161,6 +161,7 @@ const char *ksh_plan_kind(const ksh_kernel_desc *d)
     case KSH_SDPA_SLOTS:
     case KSH_SDPA_MWG_PART: return "sdpa_q40";
     case KSH_ATTEND_DECODE: return "attend_decode_q40";
+    case KSH_ATTN_MERGE_MATVEC: return "attn_merge_matvec_q4k";
     }
     return nullptr;
 }

@@ -46,7 +46,7 @@ __device__ unsigned long long ksh_trace_buf[64 * 16];
 #define KSH_MARK(n) do { } while (0)
 #endif
 
-enum { kModeDirect = 0, kModePart = 1, kModeMerge = 2 };
+enum { kModeDirect = 0, kModePart = 1, kModeMerge = 2, kModeSplitPart = 3 };   // SplitPart: values and (m, l) pairs in separate arrays, no merge
 constexpr int kRT = 4;   // row steps per softmax update
 
 struct LaneParams {
@@ -484,6 +484,11 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
             const int h = o / HD, d = o % HD, head = head0 + h;
             if (p.mode == kModeDirect) {
                 p.out[((size_t)slot * p.n_q + head) * HD + d] = accw[ob] / mlh[2 * h + 1];
+            } else if (p.mode == kModeSplitPart) {
+                const size_t r = ((size_t)slot * p.n_q + head) * p.nwg + part;
+                float *ml = p.tmp + (size_t)gridDim.z * p.n_q * p.nwg * HD;
+                p.tmp[r * HD + d] = accw[ob];
+                if (d == 0) { ml[2 * r] = mlh[2 * h]; ml[2 * r + 1] = mlh[2 * h + 1]; }
             } else {
                 float *rec = p.tmp + (((size_t)slot * p.n_q + head) * p.nwg + part) * (size_t)(HD + 2);
                 st_agent(rec + 2 + d, accw[ob]);
@@ -645,10 +650,14 @@ int launch_bound(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
         p.k_w = (uint8_t *)a.out[0]; p.v_w = (uint8_t *)a.out[1];
         p.k = p.k_w; p.v = p.v_w;
         p.tmp = (float *)a.out[2];
-        p.out = (float *)a.out[3];
         p.eps = k.desc.params[0];
         p.scale = k.desc.params[1];
-        p.mode = kModeMerge;
+        if (k.desc.dims[5]) {
+            p.mode = kModeSplitPart;
+        } else {
+            p.out = (float *)a.out[3];
+            p.mode = kModeMerge;
+        }
         p.fused = 1;
         break;
     default: return set_error("sdpa (register form): kind %d", k.desc.kind);
@@ -680,7 +689,7 @@ int bind_sdpa_lanes(ksh_kernel &k, int nwg, int n_slots)
     if (hsplit < 1 || hsplit > 255 || total_groups % hsplit) return set_error("sdpa: unsupported schedule unroll=%d (must divide %d)", hsplit, total_groups);
     const int wg_groups = total_groups / hsplit;
     const size_t lds = lanes_lds(hd, wg_groups, nw);
-    const bool merges = k.desc.kind == KSH_SDPA_SLOTS || k.desc.kind == KSH_ATTEND_DECODE;
+    const bool merges = k.desc.kind == KSH_SDPA_SLOTS || (k.desc.kind == KSH_ATTEND_DECODE && !k.desc.dims[5]);
     if (merges && (size_t)wg_groups * (nwg + 16) * 3 * 4 > (size_t)nw * (64 / (hd / 8)) * ((wg_groups <= 4 ? 4 : 8) * hd) * 4)
         return set_error("sdpa: nwg=%d is too many partitions for the merge", nwg);
     k.scratch_bytes = (size_t)n_slots * n_kv * hsplit * 4;
@@ -719,8 +728,10 @@ int bind_attend_decode(ksh_kernel &k)
     k.out_bytes[2] = (size_t)n_q * nwg * (hd + 2) * 4;
     k.out_bytes[3] = qb;
     k.out_align[0] = k.out_align[1] = 2; k.out_align[2] = k.out_align[3] = 4;
+    const bool parts_only = d[5] != 0;
+    if (parts_only) { k.info.n_outputs = 3; k.out_align[2] = 16; }
     if (bind_sdpa_lanes(k, (int)nwg, 1)) return 1;
-    set_name(k, "attend_decode_hd%d_nwg%d_w%d_h%d", (int)hd, (int)nwg, (int)k.info.sched.nsg, (int)k.info.sched.unroll);
+    set_name(k, "attend_decode%s_hd%d_nwg%d_w%d_h%d", parts_only ? "_parts" : "", (int)hd, (int)nwg, (int)k.info.sched.nsg, (int)k.info.sched.unroll);
     return 0;
 }
 

@@ -56,6 +56,7 @@ class Kind(enum.IntEnum):           # enum ksh_kind
     RMSNORM_MATVEC_QKV = 20
     RMSNORM_MATVEC_GATE_UP_GELU = 21
     ATTEND_DECODE = 22
+    ATTN_MERGE_MATVEC = 23
 
 
 class Sched(C.Structure):           # ksh_sched: OptSchedule retargeted to gfx950
@@ -479,6 +480,19 @@ class Eng:
         kk = self._k(ctx, Kind.ATTEND_DECODE, (n_q, n_kv, hd, max_seq, nwg), (DType.Q40, DType.F32), (eps, scale), sched)
         ctx.encode_multi(kk, [q, q_norm, rope, k, k_norm, v, meta], [k_cache, v_cache, tmp, out])
         return kk
+
+    # the same without the merge: `parts` = o f32[n_q, nwg, hd] then (m, l) f32[n_q, nwg, 2], for attn_merge_matvec_wd
+    def attend_decode_parts(self, ctx, n_q, n_kv, hd, max_seq, eps, scale, q, q_norm, rope, k, k_norm, v, meta, k_cache,
+                            v_cache, parts, nwg, sched=None):
+        kk = self._k(ctx, Kind.ATTEND_DECODE, (n_q, n_kv, hd, max_seq, nwg, 1), (DType.Q40, DType.F32), (eps, scale), sched)
+        ctx.encode_multi(kk, [q, q_norm, rope, k, k_norm, v, meta], [k_cache, v_cache, parts])
+        return kk
+
+    # SdpaMwgReduce (lower.rs:5897-6087) folded into the GEMV that consumes the attention output
+    def attn_merge_matvec_wd(self, ctx, rows, n_q, hd, nwg, wdt, w, parts, y, sched=None):
+        k = self._k(ctx, Kind.ATTN_MERGE_MATVEC, (rows, n_q, hd, nwg), (wdt, DType.F32), (), sched)
+        ctx.encode_multi(k, [w, parts], [y])
+        return k
 
     # :1414-1444
     def matvec_batch(self, ctx, rows, cols, batch, wdt, w, x, y, sched=None):

@@ -51,8 +51,14 @@ def test_quantize_q6k_matches_host_routine_bytes(ctx, eng):
     assert np.array_equal(got, want)
 
 
-@pytest.fixture(scope="module")
-def small_model(ctx):
+@pytest.fixture(scope="module", params=["short_context_form", "crosses_to_long_form_at_20"])
+def small_model(ctx, request):
+    """The decode loop has two forms of the attention / o-projection pair and switches between them by position
+    (KSEARCH_SHORT_CONTEXT, read when the model is built): once with every position on the short form, once with
+    the switch inside the test sequences."""
+    import os
+    if request.param != "short_context_form":
+        os.environ["KSEARCH_SHORT_CONTEXT"] = "20"
     w = synth.gemma_weights(SMALL, 500, oracle.quantize_q4k, synth.chunked(oracle.quantize_q6k), std=0.05)
     # norm weights away from 1 so that a swapped or dropped norm shows
     rng = np.random.default_rng(501)
@@ -60,7 +66,10 @@ def small_model(ctx):
         for name in ("attn_norm", "q_norm", "k_norm", "post_attn_norm", "ffn_norm", "post_ffw_norm"):
             lw[name] = (1.0 + 0.2 * rng.standard_normal(lw[name].size)).astype(np.float32)
     w["output_norm"] = (1.0 + 0.2 * rng.standard_normal(SMALL["hidden"])).astype(np.float32)
-    gpu = hip.Gemma(ctx, SMALL, w)
+    try:
+        gpu = hip.Gemma(ctx, SMALL, w)
+    finally:
+        os.environ.pop("KSEARCH_SHORT_CONTEXT", None)
     cpu = oracle.Gemma(SMALL, w)
     yield gpu, cpu, w
     gpu.close()

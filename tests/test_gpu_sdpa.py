@@ -181,3 +181,60 @@ def test_attend_decode_vs_unfused_oracle(ctx, eng, n_q, n_kv, hd, max_seq, pos, 
         assert_close(got, want, TOL, f"rep {rep}")
     if pos + 1 < max_seq:
         assert not ctx.read_bytes(kc, row, (pos + 1) * row).any()
+
+
+@pytest.mark.parametrize("n_q,n_kv,hd,max_seq,pos,nwg,rows", [
+    (8, 1, 256, 4096, 0, 8, 2048),      # one row: seven partitions are empty
+    (8, 1, 256, 4096, 5, 8, 2048),      # fewer rows than partitions
+    (8, 1, 256, 4096, 319, 8, 2048),    # the decode loop's shape
+    (8, 1, 256, 512, 200, 3, 512),      # fewer partitions than the prologue holds
+    (4, 1, 128, 256, 77, 4, 512),       # the small decode model: half of the threads hold no element
+    (4, 2, 128, 300, 150, 1, 300),      # a single partition
+])
+def test_attn_merge_matvec_vs_merged_attention(ctx, eng, n_q, n_kv, hd, max_seq, pos, nwg, rows):
+    """AttendDecode without its merge, then the o-projection that merges the partitions in its prologue, against
+    (a) the oracle's attention over the device's cache followed by the oracle's Q4_K GEMV and (b) the merging
+    AttendDecode followed by the plain GEMV."""
+    eps, scale = 1e-6, 1.0 / float(np.sqrt(hd))
+    row = n_kv * hd // 32 * 18
+    k, v = kv(max_seq, n_kv, hd, 440 + pos)
+    k[pos * row:] = 0
+    v[pos * row:] = 0
+    q, kr, vr = (synth.normal_f32(r * hd, 450 + i) for i, r in enumerate((n_q, n_kv, n_kv)))
+    qw, kw = 1.0 + 0.2 * synth.normal_f32(hd, 453), 1.0 + 0.2 * synth.normal_f32(hd, 454)
+    rope = oracle.rope_table(max_seq, hd, 10000.0)
+    cols = n_q * hd
+    w = synth.q4k_blocks(rows * cols // 256, seed=455)
+    bw = ctx.buffer_bytes(w)
+    ins = [ctx.buffer_f32(a) for a in (q, qw, rope, kr, kw, vr)] + [ctx.buffer_f32([pos + 1, 0, 0, pos])]
+    # (b) merge inside the attention launch, plain GEMV
+    kc, vc = ctx.buffer_bytes(k), ctx.buffer_bytes(v)
+    out, y_ref = ctx.buffer_empty_f32(cols), ctx.buffer_empty_f32(rows)
+    tmp = ctx.buffer_empty_f32(n_q * nwg * (hd + 2))
+    eng.attend_decode(ctx, n_q, n_kv, hd, max_seq, eps, scale, *ins, kc, vc, tmp, out, nwg=nwg)
+    eng.matvec_wd(ctx, rows, cols, DType.Q4K, bw, out, y_ref)
+    want_b = ctx.read_f32(y_ref, rows)
+    # the path under test, twice (nothing may depend on what the last call left in `parts`)
+    kc2, vc2 = ctx.buffer_bytes(k), ctx.buffer_bytes(v)
+    parts, y = ctx.buffer_f32(np.full(n_q * nwg * (hd + 2), np.nan, np.float32)), ctx.buffer_empty_f32(rows)
+    for rep in range(2):
+        eng.attend_decode_parts(ctx, n_q, n_kv, hd, max_seq, eps, scale, *ins, kc2, vc2, parts, nwg)
+        kk = eng.attn_merge_matvec_wd(ctx, rows, n_q, hd, nwg, DType.Q4K, bw, parts, y)
+        got = ctx.read_f32(y, rows)
+        assert np.array_equal(ctx.read_bytes(kc2, (pos + 1) * row), ctx.read_bytes(kc, (pos + 1) * row))
+        wq = oracle.rmsnorm_per_head_qkv_q40(q, qw, rope[pos], kr, kw, vr, n_q, n_kv, hd, eps)[0]
+        att = oracle.sdpa(wq, ctx.read_bytes(kc2, (pos + 1) * row), ctx.read_bytes(vc2, (pos + 1) * row), n_q, n_kv, hd,
+                          pos + 1, 0, scale, f64=True)
+        want_a = oracle.matvec(oracle.Q4K, w, rows, cols, att.astype(np.float32))
+        assert_close(got, want_a, TOL, f"vs oracle, rep {rep}")
+        assert_close(got, want_b, 1e-4, f"vs merging launch, rep {rep}")
+    assert "attn_merge" in kk.name
+
+
+def test_attn_merge_matvec_errors(ctx):
+    with pytest.raises(hip.KshError, match="at most 8"):
+        ctx.compile(hip.make_desc(hip.Kind.ATTN_MERGE_MATVEC, (2048, 8, 256, 16), (DType.Q4K, DType.F32), ()))
+    with pytest.raises(hip.KshError, match="power of two"):
+        ctx.compile(hip.make_desc(hip.Kind.ATTN_MERGE_MATVEC, (2048, 8, 96, 4), (DType.Q4K, DType.F32), ()))
+    with pytest.raises(hip.KshError, match="one float4 per thread"):
+        ctx.compile(hip.make_desc(hip.Kind.ATTN_MERGE_MATVEC, (2048, 16, 256, 4), (DType.Q4K, DType.F32), ()))

@@ -62,6 +62,7 @@ struct LaneParams {
     int n_q, n_kv, max_t, nwg, meta_stride, mode, fused;
     int groups;   // q heads this workgroup handles: (n_q / n_kv) / hsplit
     int hsplit;   // workgroups that share a kv head's rows, each with its own q heads
+    int balance;  // the launch's nwg * n_slots partitions are dealt to the slots by length (kModeMerge, several slots)
 };
 
 __device__ __forceinline__ uint32_t ld32_a2(const uint8_t *p)
@@ -270,6 +271,94 @@ __device__ __forceinline__ void norm_rope_regs(const float (&xv)[HD / 64], const
     }
 }
 
+// Slots of unequal length share a launch's P = nwg * n_slots workgroups by length: ceil(tlen / c) to a slot (at
+// least one), with c = ceil(T / (P - n_slots)) rows, so that they sum to at most P; what is left over exits.
+// Every workgroup derives the same table from the slots' lengths.  Slot s's partitions are the consecutive
+// flat indices from the sum of its predecessors' counts, and its records sit in that order.
+__device__ __forceinline__ int dealt_rows(const float *meta, int stride, int n_slots, int nwg)
+{
+    int T = 0;
+    for (int s = 0; s < n_slots; s++) T += (int)meta[(size_t)s * stride];
+    const int spare = nwg * n_slots - n_slots;   // host-checked: nwg >= 2
+    return max(1, (T + spare - 1) / spare);
+}
+__device__ __forceinline__ int dealt_parts(const float *meta, int stride, int s, int c)
+{
+    return max(1, ((int)meta[(size_t)s * stride] + c - 1) / c);
+}
+
+// The merge of a balanced launch's partials, as a second launch: with a hundred partitions to a long slot a
+// single (last-arriving) workgroup would pull them all through one compute unit.  A workgroup takes 64
+// dimensions of one (slot, head): thread (g, j) = (tid / 16, tid % 16) holds a float4 of them for the partitions
+// g, g + 16, ..., so that a slot's whole set of records is requested in one go, while the weights
+// exp(m_i - M) are still being worked out.  grid = (n_q * HD / 64, n_slots), 256 threads.
+// Records of a balanced launch: values [flat][n_q][HD], then (m, l) [flat][n_q][2].
+template <int HD>
+__global__ __launch_bounds__(256) void sdpa_dealt_merge_kernel(const float *tmp, const float *meta, int meta_stride, int nwg,
+                                                                int n_q, float *out)
+{
+    constexpr int kMaxParts = 16 * 64;   // host-checked: nwg * n_slots
+    constexpr int QB = 8;                // partitions per thread in flight
+    __shared__ float w[kMaxParts];
+    __shared__ float red[8];
+    __shared__ __attribute__((aligned(16))) float part4[16][64];
+    const int head = blockIdx.x / (HD / 64), dq = blockIdx.x % (HD / 64), slot = blockIdx.y, S = gridDim.y;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = tid >> 4, j = tid & 15;
+    const int c = dealt_rows(meta, meta_stride, S, nwg);
+    int first = 0;
+    for (int s = 0; s < slot; s++) first += dealt_parts(meta, meta_stride, s, c);
+    const int n = dealt_parts(meta, meta_stride, slot, c);
+    const size_t P = (size_t)nwg * S;
+    const float *ov = tmp + ((size_t)first * n_q + head) * HD + dq * 64 + 4 * j;   // + i * n_q * HD
+    const float *ml = tmp + P * n_q * HD + ((size_t)first * n_q + head) * 2;      // + i * n_q * 2
+    const size_t ops = (size_t)n_q * HD, mps = (size_t)n_q * 2;
+    // first batch of values, requested before the weights exist
+    float4 v[QB];
+#pragma unroll
+    for (int u = 0; u < QB; u++) v[u] = ldg_f4(ov + (size_t)min(g + 16 * u, n - 1) * ops, 0);
+    float m = -1.0e30f;
+    for (int i = tid; i < n; i += 256) m = fmaxf(m, ml[i * mps]);
+    m = wave_max(m);
+    if (lane == 0) red[wave] = m;
+    __syncthreads();
+    const float M = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    float ls = 0.f;
+    for (int i = tid; i < n; i += 256) {
+        const float2 p2 = ldg_f2(ml + i * mps, 0);
+        const float wt = __expf(p2.x - M);
+        w[i] = wt;
+        ls = fmaf(wt, p2.y, ls);
+    }
+    ls = wave_sum(ls);
+    if (lane == 0) red[4 + wave] = ls;
+    __syncthreads();
+    const float L = (red[4] + red[5]) + (red[6] + red[7]);
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int i0 = 0; i0 < n; i0 += 16 * QB) {
+        if (i0) {
+#pragma unroll
+            for (int u = 0; u < QB; u++) v[u] = ldg_f4(ov + (size_t)min(i0 + g + 16 * u, n - 1) * ops, 0);
+        }
+#pragma unroll
+        for (int u = 0; u < QB; u++) {
+            const int i = i0 + g + 16 * u;
+            const float wt = i < n ? w[i] : 0.f;
+            acc.x = fmaf(wt, v[u].x, acc.x);
+            acc.y = fmaf(wt, v[u].y, acc.y);
+            acc.z = fmaf(wt, v[u].z, acc.z);
+            acc.w = fmaf(wt, v[u].w, acc.w);
+        }
+    }
+    *reinterpret_cast<float4 *>(&part4[g][4 * j]) = acc;
+    __syncthreads();
+    if (tid < 64) {
+        float sum = 0.f;
+#pragma unroll
+        for (int q = 0; q < 16; q++) sum += part4[q][tid];
+        out[((size_t)slot * n_q + head) * HD + dq * 64 + tid] = sum / L;
+    }
+}
+
 // grid = (nwg, n_kv, n_slots)
 template <int HD, int GP, int NW>
 __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
@@ -288,13 +377,29 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
     KSH_MARK(0);
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int j = lane % LPR, sub = lane / LPR, b = j >> 2, w = j & 3, c = w;
-    const int part = blockIdx.x, kvh = blockIdx.y / p.hsplit, hg = blockIdx.y % p.hsplit, slot = blockIdx.z;
+    int part = blockIdx.x, slot = blockIdx.z, nparts = p.nwg;
+    const int kvh = blockIdx.y / p.hsplit, hg = blockIdx.y % p.hsplit;
     const int groups = p.groups;
     const int head0 = (kvh * p.hsplit + hg) * groups;   // first q head of this workgroup
+    // partial records: rec(head, part) = tmp + rec_base + head * rec_hs + part * rec_ps
+    size_t rec_base = (size_t)slot * p.n_q * p.nwg * (HD + 2), rec_hs = (size_t)p.nwg * (HD + 2), rec_ps = HD + 2;
+    if (p.balance) {
+        const int S = gridDim.z, f = blockIdx.z * p.nwg + blockIdx.x;
+        const int c = dealt_rows(p.meta, p.meta_stride, S, p.nwg);
+        int first = 0;
+        slot = -1;
+        for (int s = 0; s < S; s++) {
+            const int n = dealt_parts(p.meta, p.meta_stride, s, c);
+            if (f < first + n) { slot = s; part = f - first; nparts = n; break; }
+            first += n;
+        }
+        if (slot < 0) return;   // left over
+        rec_base = (size_t)first + part;   // flat partition index: values [flat][n_q][HD], then (m, l) [flat][n_q][2]
+    }
 
     const float *meta = p.meta + (size_t)slot * p.meta_stride;
     const int tlen = (int)meta[0], start = (int)meta[1];
-    const int chunk = (tlen + p.nwg - 1) / p.nwg;
+    const int chunk = (tlen + nparts - 1) / nparts;
     const int p0 = part * chunk;
     int p1 = min(p0 + chunk, tlen);
 
@@ -484,13 +589,18 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
             const int h = o / HD, d = o % HD, head = head0 + h;
             if (p.mode == kModeDirect) {
                 p.out[((size_t)slot * p.n_q + head) * HD + d] = accw[ob] / mlh[2 * h + 1];
+            } else if (p.balance) {
+                const size_t r = rec_base * p.n_q + head;
+                float *ml = p.tmp + (size_t)gridDim.z * p.nwg * p.n_q * HD;
+                p.tmp[r * HD + d] = accw[ob];
+                if (d == 0) { ml[2 * r] = mlh[2 * h]; ml[2 * r + 1] = mlh[2 * h + 1]; }
             } else if (p.mode == kModeSplitPart) {
                 const size_t r = ((size_t)slot * p.n_q + head) * p.nwg + part;
                 float *ml = p.tmp + (size_t)gridDim.z * p.n_q * p.nwg * HD;
                 p.tmp[r * HD + d] = accw[ob];
                 if (d == 0) { ml[2 * r] = mlh[2 * h]; ml[2 * r + 1] = mlh[2 * h + 1]; }
             } else {
-                float *rec = p.tmp + (((size_t)slot * p.n_q + head) * p.nwg + part) * (size_t)(HD + 2);
+                float *rec = p.tmp + rec_base + head * rec_hs + part * rec_ps;
                 st_agent(rec + 2 + d, accw[ob]);
                 if (d == 0) { st_agent(rec, mlh[2 * h]); st_agent(rec + 1, mlh[2 * h + 1]); }
             }
@@ -507,7 +617,7 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
     KSH_MARK(6);
     if (tid == 0) {
         const uint32_t arrived = __hip_atomic_fetch_add(&p.counters[slot * gridDim.y + blockIdx.y], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        last_flag = arrived == (uint32_t)p.nwg - 1u;
+        last_flag = arrived == (uint32_t)nparts - 1u;
     }
     __syncthreads();
     KSH_MARK(7);
@@ -516,37 +626,38 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
     // a thread's loads -- its output elements' values from up to QB partitions,
     // then its share of the (m, l) pairs -- are issued before anything is used.
     constexpr int QB = 16, OB = GP * HD / NT;   // partitions in flight x output elements per thread
-    const int nwgp = (p.nwg + QB - 1) / QB * QB;
-    float *w2 = slots;                          // [groups][nwgp] weights, zero past nwg
-    float *mq = slots + groups * nwgp;          // [groups][nwg][2]
-    const float *recs = p.tmp + ((size_t)slot * p.n_q + head0) * p.nwg * (size_t)(HD + 2);
+    const int nwgp = (nparts + QB - 1) / QB * QB;
+    float *w2 = slots;                          // [groups][nwgp] weights, zero past nparts
+    float *mq = slots + groups * nwgp;          // [groups][nparts][2]
+    const float *recs = p.tmp + rec_base + head0 * rec_hs;
     float acc[OB], val[OB][QB];
 #pragma unroll
     for (int ob = 0; ob < OB; ob++) {
         acc[ob] = 0.f;
         const int o = min(tid + ob * NT, groups * HD - 1), h = o / HD, d = o % HD;
-        const float *rh = recs + (size_t)h * p.nwg * (HD + 2) + 2 + d;
+        const float *rh = recs + h * rec_hs + 2 + d;
 #pragma unroll
-        for (int u = 0; u < QB; u++) val[ob][u] = ld_agent(rh + (size_t)min(u, p.nwg - 1) * (HD + 2));
+        for (int u = 0; u < QB; u++) val[ob][u] = ld_agent(rh + (size_t)min(u, nparts - 1) * rec_ps);
     }
-    for (int i = tid; i < groups * p.nwg; i += NT) {
-        const float *rec = recs + (size_t)i * (HD + 2);   // (head, partition) records are contiguous in that order
+    for (int i = tid; i < groups * nparts; i += NT) {
+        const int h = i / nparts, q = i - h * nparts;
+        const float *rec = recs + h * rec_hs + q * rec_ps;
         mq[2 * i] = ld_agent(rec);
         mq[2 * i + 1] = ld_agent(rec + 1);
     }
     __syncthreads();
     KSH_MARK(8);
-    for (int h = wave; h < groups; h += NW) merge_weights(mq + 2 * h * p.nwg, 2, p.nwg, nwgp, w2 + h * nwgp, mlh + 2 * h, lane);
+    for (int h = wave; h < groups; h += NW) merge_weights(mq + 2 * h * nparts, 2, nparts, nwgp, w2 + h * nwgp, mlh + 2 * h, lane);
     __syncthreads();
     KSH_MARK(9);
-    for (int q0 = 0; q0 < p.nwg; q0 += QB) {
+    for (int q0 = 0; q0 < nparts; q0 += QB) {
 #pragma unroll
         for (int ob = 0; ob < OB; ob++) {
             const int o = min(tid + ob * NT, groups * HD - 1), h = o / HD, d = o % HD;
             if (q0) {
-                const float *rh = recs + (size_t)h * p.nwg * (HD + 2) + 2 + d;
+                const float *rh = recs + h * rec_hs + 2 + d;
 #pragma unroll
-                for (int u = 0; u < QB; u++) val[ob][u] = ld_agent(rh + (size_t)min(q0 + u, p.nwg - 1) * (HD + 2));
+                for (int u = 0; u < QB; u++) val[ob][u] = ld_agent(rh + (size_t)min(q0 + u, nparts - 1) * rec_ps);
             }
 #pragma unroll
             for (int u = 0; u < QB; u++) acc[ob] = fmaf(w2[h * nwgp + q0 + u], val[ob][u], acc[ob]);
@@ -610,6 +721,10 @@ LaneParams base_params(const ksh_kernel &k)
     return p;
 }
 
+// Several slots share one launch's partitions by length when there are few enough of them for every workgroup
+// to derive the table itself.
+bool balanced_slots(int n_slots, int nwg) { return n_slots > 1 && n_slots <= 16 && nwg >= 2 && nwg <= 64; }
+
 // variant: nwg | NW << 16 | hsplit << 24
 int launch_bound(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
 {
@@ -641,6 +756,17 @@ int launch_bound(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
         p.out = (float *)a.out[1];
         p.scale = k.desc.params[0];
         p.mode = kModeMerge;
+        if (balanced_slots(n_slots, p.nwg)) {
+            p.balance = 1;
+            p.mode = kModePart;
+            if (launch_lanes(p, hd, nw, n_slots, st)) return 1;
+            if (hd == 256)
+                hipLaunchKernelGGL(sdpa_dealt_merge_kernel<256>, dim3(p.n_q * 4, n_slots), dim3(256), 0, st, p.tmp, p.meta, p.meta_stride, p.nwg, p.n_q, p.out);
+            else
+                hipLaunchKernelGGL(sdpa_dealt_merge_kernel<128>, dim3(p.n_q * 2, n_slots), dim3(256), 0, st, p.tmp, p.meta, p.meta_stride, p.nwg, p.n_q, p.out);
+            const hipError_t e = hipGetLastError();
+            return e == hipSuccess ? 0 : hip_fail(e, "sdpa merge launch");
+        }
         break;
     case KSH_ATTEND_DECODE:
         p.q = (const float *)a.in[0]; p.qw = (const float *)a.in[1]; p.rope = (const float *)a.in[2];
@@ -690,7 +816,8 @@ int bind_sdpa_lanes(ksh_kernel &k, int nwg, int n_slots)
     const int wg_groups = total_groups / hsplit;
     const size_t lds = lanes_lds(hd, wg_groups, nw);
     const bool merges = k.desc.kind == KSH_SDPA_SLOTS || (k.desc.kind == KSH_ATTEND_DECODE && !k.desc.dims[5]);
-    if (merges && (size_t)wg_groups * (nwg + 16) * 3 * 4 > (size_t)nw * (64 / (hd / 8)) * ((wg_groups <= 4 ? 4 : 8) * hd) * 4)
+    if (merges && !(k.desc.kind == KSH_SDPA_SLOTS && balanced_slots(n_slots, nwg)) &&   // (those merge in a launch of their own)
+        (size_t)wg_groups * (nwg + 16) * 3 * 4 > (size_t)nw * (64 / (hd / 8)) * ((wg_groups <= 4 ? 4 : 8) * hd) * 4)
         return set_error("sdpa: nwg=%d is too many partitions for the merge", nwg);
     k.scratch_bytes = (size_t)n_slots * n_kv * hsplit * 4;
     set_launch(k, (uint32_t)nwg, (uint32_t)(n_kv * hsplit), (uint32_t)n_slots, (uint32_t)nw * 64, (uint32_t)lds);

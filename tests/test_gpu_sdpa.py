@@ -131,6 +131,32 @@ def test_sdpa_cfg3_full_size(ctx, eng):
     assert np.allclose(ctx.read_f32(out, n_slots * n_q * hd), 1.5, rtol=1e-5)
 
 
+@pytest.mark.parametrize("n_slots,nwg,lens", [
+    (4, 2, [2048, 1, 1, 1]),            # nearly every partition goes to one slot
+    (3, 8, [7, 5, 2048]),               # fewer rows than partitions in two slots
+    (16, 4, None),                      # the most slots that share partitions by length
+    (17, 4, None),                      # one more: every slot keeps its own nwg partitions
+    (2, 16, [2048, 2048]),              # equal lengths
+])
+def test_sdpa_slots_partitions_dealt_by_length(ctx, eng, n_slots, nwg, lens):
+    """A launch's nwg * n_slots partitions are shared out by slot length (up to 16 slots); every slot's result is
+    still the oracle's attention over its own rows, on two launches in a row (the arrival counters return to zero)."""
+    n_q, n_kv, hd, max_t = 8, 1, 256, 2048
+    rnd, k, v, q = synth.cfg3_q40_attention(n_slots, n_q, n_kv, hd, max_t, lo=1, seed=360 + n_slots)
+    lens = [int(t) for t in (rnd if lens is None else lens)]
+    meta = np.zeros((n_slots, 4), dtype=np.float32)
+    meta[:, 0] = lens
+    bq, bk, bv, bm = ctx.buffer_f32(q), ctx.buffer_bytes(k), ctx.buffer_bytes(v), ctx.buffer_f32(meta)
+    tmp = ctx.buffer_empty_f32(n_slots * n_q * nwg * (hd + 2))
+    out = ctx.buffer_empty_f32(n_slots * n_q * hd)
+    for rep in range(2):
+        eng.sdpa_slots(ctx, n_q, n_kv, hd, max_t, n_slots, bq, bk, bv, bm, tmp, out, 0.0625, nwg)
+        got = ctx.read_f32(out, n_slots * n_q * hd).reshape(n_slots, -1)
+        for s in range(n_slots):
+            want = oracle.sdpa(q[s], k[s], v[s], n_q, n_kv, hd, lens[s], 0, 0.0625, f64=True)
+            assert_close(got[s], want, TOL, f"rep {rep} slot {s} len {lens[s]}")
+
+
 def test_sdpa_errors(ctx):
     with pytest.raises(hip.KshError, match="multiple of 32"):
         ctx.compile(hip.make_desc(hip.Kind.SDPA_NAIVE, (8, 1, 100, 64), (DType.Q40, DType.F32), (1.0,)))

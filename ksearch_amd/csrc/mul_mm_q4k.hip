@@ -48,37 +48,49 @@ constexpr int PITCH2 = 32 + 8;     // halves per LDS row of the min-term tiles
 // order the paired nibble extraction produces, applied to X as well
 __device__ __forceinline__ int kperm(int i) { return (i & ~3) | ((i & 1) << 1) | ((i >> 1) & 1); }
 
-// X bf16 -> f16 (permuted), plus the min-term operand per (token, superblock):
-// 32 halves = Sx_hi[8] | Sx_hi[8] | Sx_lo[8] | 0[8].  One thread per (token, sub-block).
-__global__ void mm_prep_x_kernel(const uint16_t *__restrict__ X, _Float16 *__restrict__ Xh,
-                                 _Float16 *__restrict__ SxA, int batch, int cols)
+// X bf16 -> f16 (permuted) in the order the matrix instruction wants its A operand, plus the min-term
+// operand per (token, superblock): 32 halves = Sx_hi[8] | Sx_hi[8] | Sx_lo[8] | 0[8].
+// Xf[token / 32][k / 16][lane][8] with lane = token % 32 + 32 * ((k / 8) % 2): one 32 x 16 fragment is 1 KB,
+// lane after lane, so that a multiplying wave fetches it with a single 128-bit load per lane and the
+// activations never pass through LDS.  One thread per 8 elements; the four threads of a sub-block add their
+// sums up over the quad.
+__global__ __launch_bounds__(256) void mm_prep_x_kernel(const uint16_t *__restrict__ X, _Float16 *__restrict__ Xf,
+                                                        _Float16 *__restrict__ SxA, int batch, int cols)
 {
-    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
-    const int spt = cols / 32;             // sub-blocks per token
-    if (idx >= batch * spt) return;
-    const int t = idx / spt, s = idx % spt;
-    const uint16_t *src = X + (size_t)t * cols + (size_t)s * 32;
-    _Float16 *dst = Xh + (size_t)t * cols + (size_t)s * 32;
-    float sum = 0.f;
+    const int idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= batch * (cols / 8)) return;   // (whole quads: cols is a multiple of 32)
+    const u32x4_t in = reinterpret_cast<const u32x4_t *>(X)[idx];
+    const uint32_t w[4] = {in.x, in.y, in.z, in.w};
+    float f[8];
 #pragma unroll
-    for (int i = 0; i < 32; i++) {
-        const float f = as_f32((uint32_t)src[i] << 16);
-        sum += f;
-        dst[kperm(i)] = (_Float16)f;
+    for (int i = 0; i < 4; i++) {
+        f[2 * i] = as_f32(w[i] << 16);
+        f[2 * i + 1] = as_f32(w[i] & 0xFFFF0000u);
     }
-    const _Float16 hi = (_Float16)sum;
-    const _Float16 lo = (_Float16)(sum - (float)hi);
-    _Float16 *a2 = SxA + ((size_t)t * (cols / 256) + s / 8) * 32;
-    const int j = s % 8;
-    a2[j] = hi;
-    a2[8 + j] = hi;
-    a2[16 + j] = lo;
-    a2[24 + j] = (_Float16)0.f;
+    float sum = ((f[0] + f[1]) + (f[2] + f[3])) + ((f[4] + f[5]) + (f[6] + f[7]));
+    sum += dpp_f32<0xB1>(sum);   // quad neighbours: 1 0 3 2, then 2 3 0 1
+    sum += dpp_f32<0x4E>(sum);
+    h8 o;
+#pragma unroll
+    for (int i = 0; i < 8; i++) o[kperm(i)] = (_Float16)f[i];
+    const int k8 = cols / 8, t = idx / k8, j = idx - t * k8;
+    reinterpret_cast<h8 *>(Xf)[((size_t)(t >> 5) * (cols / 16) + (j >> 1)) * 64 + (t & 31) + 32 * (j & 1)] = o;
+    if ((threadIdx.x & 3) == 0) {
+        const int s = j / 4;
+        const _Float16 hi = (_Float16)sum;
+        const _Float16 lo = (_Float16)(sum - (float)hi);
+        _Float16 *a2 = SxA + ((size_t)t * (cols / 256) + s / 8) * 32;
+        const int jj = s % 8;
+        a2[jj] = hi;
+        a2[8 + jj] = hi;
+        a2[16 + jj] = lo;
+        a2[24 + jj] = (_Float16)0.f;
+    }
 }
 
 struct MmParams {
     const uint8_t *W;
-    const _Float16 *Xh, *SxA;
+    const _Float16 *Xf, *SxA;   // fragment-ordered f16 activations (mm_prep_x_kernel), sums of x
     float *Y;
     int rows, cols, batch;
 };
@@ -88,21 +100,17 @@ __device__ __forceinline__ uint32_t pair_f16(uint32_t masked, uint32_t sc)
     return __umul24(masked, sc) + 0x64006400u;
 }
 
-// what a loader thread (two per tile row) holds: per K step 32 activations;
-// per superblock the 64 quant bytes of TWO of its four 64-column groups (so
-// that a weight row's cache lines are fetched once, not once per step), the
-// header and half of the token's sums of x
+// what a loader thread (two per tile row) holds per superblock: the 64 quant bytes of TWO of its four
+// 64-column groups (so that a weight row's cache lines are fetched once, not once per step), the header and
+// half of the token's sums of x
 // (native vector types: with HIP's uint4 class the copies become memcpys that keep these sets in scratch memory)
-struct XRegs {
-    u32x4_t x[4];
-};
 struct SbRegs {
     u32x4_t q[4];      // quant bytes of groups 2*lh and 2*lh+1, 32 each
     u32x4_t hdr, sx0, sx1;
 };
 
 constexpr int kThreadsMM = 512;
-constexpr int kLdsMain = (BM + BN) * PITCH;      // halves per main stage (A tile, then B tile)
+constexpr int kLdsMain = BN * PITCH;             // halves per main stage (the dequantized weight tile)
 constexpr int kLdsMin = (BM + BN) * PITCH2;      // halves per min-term stage
 constexpr size_t kLdsBytes = 2 * (size_t)(kLdsMain + kLdsMin) * 2 + 2 * BN * 4;
 
@@ -132,15 +140,8 @@ __global__ __launch_bounds__(kThreadsMM) void q4k_mul_mm_kernel(MmParams p)
         const int lt = tid - 256, lrow = lt >> 1, lh = lt & 1;   // two threads per tile row
         const size_t row_bytes = (size_t)nsb * 144;
         const uint8_t *wrow = p.W + (size_t)min(r0 + lrow, p.rows - 1) * row_bytes;
-        const _Float16 *xrow = p.Xh + (size_t)min(t0 + lrow, p.batch - 1) * p.cols;
         const _Float16 *sxrow = p.SxA + (size_t)min(t0 + lrow, p.batch - 1) * nsb * 32;
 
-        auto fetch_x = [&](int step, XRegs &r) __attribute__((always_inline)) {
-            const int sb = step >> 2, g = step & 3;
-            const u32x4_t *xs = reinterpret_cast<const u32x4_t *>(xrow + sb * 256 + 64 * g + 32 * lh);
-#pragma unroll
-            for (int i = 0; i < 4; i++) r.x[i] = xs[i];
-        };
         auto fetch_sb = [&](int sb, SbRegs &r) __attribute__((always_inline)) {
             const u32x4_t *w = reinterpret_cast<const u32x4_t *>(wrow + (size_t)sb * 144);
             r.hdr = w[0];
@@ -152,15 +153,10 @@ __global__ __launch_bounds__(kThreadsMM) void q4k_mul_mm_kernel(MmParams p)
         };
         // G = the step's group: its 32 quant bytes sit in lane G/2 of every pair, registers q[2*(G%2)] and
         // q[2*(G%2)+1]; this thread converts bytes 16*lh .. 16*lh+15 of them
-        auto stage = [&](int step, auto gtag, const XRegs &xr, const SbRegs &w) __attribute__((always_inline)) {
+        auto stage = [&](int step, auto gtag, const SbRegs &w) __attribute__((always_inline)) {
             constexpr int G = decltype(gtag)::value;
             const int sb = step >> 2;
-            _Float16 *As = main_stage(step), *Bs = As + BM * PITCH;
-            {
-                u32x4_t *dst = reinterpret_cast<u32x4_t *>(&As[lrow * PITCH + 32 * lh]);
-#pragma unroll
-                for (int i = 0; i < 4; i++) dst[i] = xr.x[i];
-            }
+            _Float16 *Bs = main_stage(step);
             {
                 constexpr int kSrc = (G >> 1) ? 0xF5 : 0xA0;   // quad_perm [1,1,3,3] : [0,0,2,2]
                 const u32x4_t c0 = w.q[2 * (G & 1)], c1 = w.q[2 * (G & 1) + 1];
@@ -216,34 +212,26 @@ __global__ __launch_bounds__(kThreadsMM) void q4k_mul_mm_kernel(MmParams p)
             }
         };
 
-        // Named register sets (an array, even with constant indices, ends up in scratch here): set g serves the
-        // steps 4*sb + g and is refilled for step s+4 right after step s+... its own step was staged, so a load
-        // has three whole steps to arrive.  Loads past the end re-read the last step / superblock, unused.
-        XRegs xr0, xr1, xr2, xr3;
+        // the next superblock's weights are requested when a superblock opens: four steps to arrive
         SbRegs wcur, wnext;
-        fetch_x(0, xr0);   // nsteps is a multiple of 4
-        fetch_x(1, xr1);
-        fetch_x(2, xr2);
-        fetch_x(3, xr3);
         fetch_sb(0, wcur);
-        stage(0, std::integral_constant<int, 0>{}, xr0, wcur);
+        stage(0, std::integral_constant<int, 0>{}, wcur);
         __syncthreads();
-        auto step_body = [&](int sb, auto gtag, XRegs &mine, const XRegs &next) __attribute__((always_inline)) {
+        auto step_body = [&](int sb, auto gtag) __attribute__((always_inline)) {
             constexpr int g = decltype(gtag)::value;
             const int step = 4 * sb + g;
-            fetch_x(min(step + 4, nsteps - 1), mine);   // this set's own step was staged one iteration ago
             if (g == 0) fetch_sb(min(sb + 1, nsb - 1), wnext);
             if (step + 1 < nsteps) {
                 if (g == 3) wcur = wnext;
-                stage(step + 1, std::integral_constant<int, (g + 1) & 3>{}, next, wcur);
+                stage(step + 1, std::integral_constant<int, (g + 1) & 3>{}, wcur);
             }
             __syncthreads();
         };
         for (int sb = 0; sb < nsb; sb++) {
-            step_body(sb, std::integral_constant<int, 0>{}, xr0, xr1);
-            step_body(sb, std::integral_constant<int, 1>{}, xr1, xr2);
-            step_body(sb, std::integral_constant<int, 2>{}, xr2, xr3);
-            step_body(sb, std::integral_constant<int, 3>{}, xr3, xr0);
+            step_body(sb, std::integral_constant<int, 0>{});
+            step_body(sb, std::integral_constant<int, 1>{});
+            step_body(sb, std::integral_constant<int, 2>{});
+            step_body(sb, std::integral_constant<int, 3>{});
         }
         return;
     }
@@ -258,18 +246,32 @@ __global__ __launch_bounds__(kThreadsMM) void q4k_mul_mm_kernel(MmParams p)
 #pragma unroll
             for (int i = 0; i < 16; i++) { F[a][b][i] = 0.f; Cp[a][b][i] = 0.f; }
     const int lm = lane & 31, lk = (lane >> 5) * 8;
+    // A operands straight from memory: fragment (token tile, k / 16) is 64 lanes x 16 bytes, 1 KB apart along k.
+    // Two register sets, each refilled for two steps ahead as soon as its own step's instructions are issued.
+    const int ntt = (p.batch + 31) / 32;
+    const h8 *xa[2];
+#pragma unroll
+    for (int mt = 0; mt < 2; mt++)
+        xa[mt] = reinterpret_cast<const h8 *>(p.Xf) + (size_t)min((t0 + wm * 64 + mt * 32) / 32, ntt - 1) * (p.cols / 16) * 64 + lane;
+    struct ARegs { h8 a[2][KS / 16]; };
+    auto fetch_a = [&](int step, ARegs &r) __attribute__((always_inline)) {
+#pragma unroll
+        for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+            for (int ks = 0; ks < KS / 16; ks++) r.a[mt][ks] = xa[mt][(size_t)(step * (KS / 16) + ks) * 64];
+    };
+    ARegs a0, a1;
+    fetch_a(0, a0);
+    fetch_a(min(1, nsteps - 1), a1);
     __syncthreads();   // stage 0 is written
 
-    auto mul_step = [&](int sb, auto gtag) __attribute__((always_inline)) {
+    auto mul_step = [&](int sb, auto gtag, ARegs &A) __attribute__((always_inline)) {
         constexpr int g = decltype(gtag)::value;
         const int step = 4 * sb + g;
-        const _Float16 *As = main_stage(step), *Bs = As + BM * PITCH;
+        const _Float16 *Bs = main_stage(step);
 #pragma unroll
         for (int ks = 0; ks < KS / 16; ks++) {
-            h8 a[2], b[2];
-#pragma unroll
-            for (int mt = 0; mt < 2; mt++)
-                a[mt] = *reinterpret_cast<const h8 *>(&As[(wm * 64 + mt * 32 + lm) * PITCH + 16 * ks + lk]);
+            h8 b[2];
 #pragma unroll
             for (int nt = 0; nt < 2; nt++)
                 b[nt] = *reinterpret_cast<const h8 *>(&Bs[(wn * 64 + nt * 32 + lm) * PITCH + 16 * ks + lk]);
@@ -277,8 +279,9 @@ __global__ __launch_bounds__(kThreadsMM) void q4k_mul_mm_kernel(MmParams p)
             for (int mt = 0; mt < 2; mt++)
 #pragma unroll
                 for (int nt = 0; nt < 2; nt++)
-                    Cp[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mt], b[nt], Cp[mt][nt], 0, 0, 0);
+                    Cp[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A.a[mt][ks], b[nt], Cp[mt][nt], 0, 0, 0);
         }
+        fetch_a(min(step + 2, nsteps - 1), A);
         if (g == 3) {
             // ---- end of the superblock: bias + mins through the short second product, then the row scale
             const _Float16 *A2s = min_stage(sb), *B2s = A2s + BM * PITCH2;
@@ -313,10 +316,10 @@ __global__ __launch_bounds__(kThreadsMM) void q4k_mul_mm_kernel(MmParams p)
         __syncthreads();
     };
     for (int sb = 0; sb < nsb; sb++) {
-        mul_step(sb, std::integral_constant<int, 0>{});
-        mul_step(sb, std::integral_constant<int, 1>{});
-        mul_step(sb, std::integral_constant<int, 2>{});
-        mul_step(sb, std::integral_constant<int, 3>{});
+        mul_step(sb, std::integral_constant<int, 0>{}, a0);
+        mul_step(sb, std::integral_constant<int, 1>{}, a1);
+        mul_step(sb, std::integral_constant<int, 2>{}, a0);
+        mul_step(sb, std::integral_constant<int, 3>{}, a1);
     }
 
     // accumulator layout of the 32x32 tile: column = lane % 32, row = 8*(i/4) + 4*(lane/32) + i%4
@@ -336,14 +339,13 @@ __global__ __launch_bounds__(kThreadsMM) void q4k_mul_mm_kernel(MmParams p)
 int launch_mul_mm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
 {
     const int rows = (int)k.desc.dims[0], cols = (int)k.desc.dims[1], batch = (int)k.desc.dims[2];
-    _Float16 *Xh = (_Float16 *)k.scratch;
-    _Float16 *SxA = Xh + (size_t)batch * cols;
-    const int n = batch * (cols / 32);
-    hipLaunchKernelGGL(mm_prep_x_kernel, dim3((n + 255) / 256), dim3(256), 0, st, (const uint16_t *)a.in[1], Xh, SxA,
-                       batch, cols);
+    _Float16 *Xf = (_Float16 *)k.scratch;
+    _Float16 *SxA = Xf + (size_t)((batch + 31) / 32 * 32) * cols;
+    const int n = batch * (cols / 8);
+    hipLaunchKernelGGL(mm_prep_x_kernel, dim3((n + 255) / 256), dim3(256), 0, st, (const uint16_t *)a.in[1], Xf, SxA, batch, cols);
     MmParams p;
     p.W = (const uint8_t *)a.in[0];
-    p.Xh = Xh;
+    p.Xf = Xf;
     p.SxA = SxA;
     p.Y = (float *)a.out[0];
     p.rows = rows; p.cols = cols; p.batch = batch;
@@ -367,7 +369,7 @@ int bind_matvec_batch(ksh_kernel &k)
     k.in_bytes[1] = (size_t)batch * cols * 2; k.in_align[1] = 16;
     k.out_bytes[0] = (size_t)batch * rows * 4; k.out_align[0] = 4;
     // f16 copy of X plus the min-term operand (32 halves per token and superblock)
-    k.scratch_bytes = (size_t)batch * cols * 2 + (size_t)batch * (cols / 256) * 64;
+    k.scratch_bytes = (size_t)((batch + 31) / 32 * 32) * cols * 2 + (size_t)batch * (cols / 256) * 64;
     set_launch(k, (uint32_t)((batch + BM - 1) / BM), (uint32_t)((rows + BN - 1) / BN), 1, kThreadsMM,
                (uint32_t)kLdsBytes);
     k.info.sched = k.desc.sched;

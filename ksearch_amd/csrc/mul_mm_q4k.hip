@@ -246,6 +246,7 @@ __global__ __launch_bounds__(kThreadsMM) void q4k_mul_mm_kernel(MmParams p)
 #pragma unroll
             for (int i = 0; i < 16; i++) { F[a][b][i] = 0.f; Cp[a][b][i] = 0.f; }
     const int lm = lane & 31, lk = (lane >> 5) * 8;
+    const f16v kZero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     // A operands straight from memory: fragment (token tile, k / 16) is 64 lanes x 16 bytes, 1 KB apart along k.
     // Two register sets, each refilled for two steps ahead as soon as its own step's instructions are issued.
     const int ntt = (p.batch + 31) / 32;
@@ -279,9 +280,12 @@ __global__ __launch_bounds__(kThreadsMM) void q4k_mul_mm_kernel(MmParams p)
             for (int mt = 0; mt < 2; mt++)
 #pragma unroll
                 for (int nt = 0; nt < 2; nt++)
-                    Cp[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A.a[mt][ks], b[nt], Cp[mt][nt], 0, 0, 0);
+                    // a superblock's first product starts from the constant zero: no pass over the accumulators to clear them
+                    Cp[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A.a[mt][ks], b[nt], (g == 0 && ks == 0) ? kZero16 : Cp[mt][nt], 0, 0, 0);
+            // this k slice's fragments are spent: ask for the ones of two steps ahead right away
+#pragma unroll
+            for (int mt = 0; mt < 2; mt++) A.a[mt][ks] = xa[mt][(size_t)(min(step + 2, nsteps - 1) * (KS / 16) + ks) * 64];
         }
-        fetch_a(min(step + 2, nsteps - 1), A);
         if (g == 3) {
             // ---- end of the superblock: bias + mins through the short second product, then the row scale
             const _Float16 *A2s = min_stage(sb), *B2s = A2s + BM * PITCH2;
@@ -307,10 +311,8 @@ __global__ __launch_bounds__(kThreadsMM) void q4k_mul_mm_kernel(MmParams p)
 #pragma unroll
                 for (int mt = 0; mt < 2; mt++)
 #pragma unroll
-                    for (int i = 0; i < 16; i++) {
+                    for (int i = 0; i < 16; i++)
                         F[mt][nt][i] = fmaf(dn, Cp[mt][nt][i], F[mt][nt][i]);
-                        Cp[mt][nt][i] = 0.f;
-                    }
             }
         }
         __syncthreads();

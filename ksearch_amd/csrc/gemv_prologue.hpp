@@ -168,13 +168,14 @@ struct StageRegs {
     float4 wn[kStageP], wp[kStageP], rs[kStageP];
 };
 
-template <int NT>
+// kMerge: whether the kernel is built with the kMergeParts source at all (the Q4_K kernels' prologue instances are)
+template <int NT, bool kMerge = false>
 __device__ __forceinline__ void stage_fetch(const Prologue &pr, int cols, StageRegs &s)
 {
     // n4 is a multiple of 64, so "this float4 exists" is a per-wave fact: keep it
     // in scalar registers and the loads stay unpredicated
     const int wbase = __builtin_amdgcn_readfirstlane(threadIdx.x & ~63), tid = wbase + (threadIdx.x & 63), n4 = cols / 4;
-    if (pr.kind == kMergeParts) {
+    if (kMerge && pr.kind == kMergeParts) {
         // one float4 of the output per thread (host-checked: n4 <= NT, nwg <= 8): its
         // eight partitions' values and (m, l) pairs; partitions past nwg re-read the
         // last one, so that the number of loads is fixed
@@ -214,12 +215,12 @@ __device__ __forceinline__ void stage_fetch(const Prologue &pr, int cols, StageR
 
 // Every thread must call this (it contains barriers); the LDS image is complete
 // after the caller's next __syncthreads().
-template <int XF, int NT>
+template <int XF, int NT, bool kMerge = false>
 __device__ __forceinline__ void stage_finish(const Prologue &pr, uint8_t *lds, int cols, StageRegs &s)
 {
     const int wbase = __builtin_amdgcn_readfirstlane(threadIdx.x & ~63), tid = wbase + (threadIdx.x & 63), n4 = cols / 4;
     float *red = reinterpret_cast<float *>(lds + xs_image_bytes<XF>(cols));
-    if (pr.kind == kMergeParts) {
+    if (kMerge && pr.kind == kMergeParts) {
         if (wbase < n4) {
             float m[kMergeMaxParts], l[kMergeMaxParts];
 #pragma unroll

@@ -245,7 +245,9 @@ __device__ __forceinline__ WaveTask wave_task(const MatvecParams &p, int wv, int
 // NM = 1 (mode 0) or 2 (mode 1).  The weight loads of step s+1 are issued
 // before step s is consumed, and step 0's before the input is staged, so the
 // first HBM round trip overlaps the prologue.
-template <int R, int NW, int NM, int XF, bool MULTI>
+// MERGE: built with the partition-merging prologue (kept out of every other instance: a longer program in front
+// of the first weight load costs 0.1 us at 4096 x 4096)
+template <int R, int NW, int NM, int XF, bool MULTI, bool MERGE>
 __global__ __launch_bounds__(NW * 64) void q4k_gemv_kernel(MatvecParams p_in)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t xs[];
@@ -273,12 +275,12 @@ __global__ __launch_bounds__(NW * 64) void q4k_gemv_kernel(MatvecParams p_in)
     Q4kLane cur[NM][R], nxt[MULTI ? NM : 1][MULTI ? R : 1];
     StageRegs sr;
     constexpr int RPRE = R;   // (splitting the issue as the half-wave form does costs 0.5 us at 4096 x 4096)
-    stage_fetch<NW * 64>(p.pro, cols, sr);
+    stage_fetch<NW * 64, MERGE>(p.pro, cols, sr);
 #pragma unroll
     for (int m = 0; m < NM; m++)
 #pragma unroll
         for (int r = 0; r < RPRE; r++) cur[m][r] = q4k_load(rowp[m][r] + (size_t)min(bl, bpr - 1) * kQ4kBytes, g);
-    stage_finish<XF, NW * 64>(p.pro, xs, cols, sr);
+    stage_finish<XF, NW * 64, MERGE>(p.pro, xs, cols, sr);
     __syncthreads();
     if (!t.active) return;
 #pragma unroll
@@ -332,7 +334,7 @@ __global__ __launch_bounds__(NW * 64) void q4k_gemv_kernel(MatvecParams p_in)
 // Half-wave form for rows of exactly 8 superblocks (2048 columns): lanes
 // 0..31 and 32..63 work on different rows, so a wave covers 2R rows in a single
 // step and no lane idles.
-template <int R, int NW, int NM, int XF>
+template <int R, int NW, int NM, int XF, bool MERGE>
 __global__ __launch_bounds__(NW * 64) void q4k_gemv_half_kernel(MatvecParams p_in)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t xs[];
@@ -346,7 +348,7 @@ __global__ __launch_bounds__(NW * 64) void q4k_gemv_half_kernel(MatvecParams p_i
 
     Q4kLane L[NM][R];
     StageRegs sr;
-    stage_fetch<NW * 64>(p.pro, bpr * 256, sr);
+    stage_fetch<NW * 64, MERGE>(p.pro, bpr * 256, sr);
     auto load_r = [&](int r) {
         const size_t off = (size_t)min(row0 + r, t.rows - 1) * row_bytes + (size_t)bl * kQ4kBytes;
         L[0][r] = q4k_load(t.W0 + off, g);
@@ -359,7 +361,7 @@ __global__ __launch_bounds__(NW * 64) void q4k_gemv_half_kernel(MatvecParams p_i
     // and stream in while the first is being multiplied (gate || up, 2048 ->
     // 8192 with the add-then-norm prologue: 8.1 -> 7.1 us).
     load_r(0);
-    stage_finish<XF, NW * 64>(p.pro, xs, bpr * 256, sr);
+    stage_finish<XF, NW * 64, MERGE>(p.pro, xs, bpr * 256, sr);
     __syncthreads();
     if (!t.active) return;
 #pragma unroll
@@ -391,17 +393,24 @@ int waves_for(int rows, int rpw) { return (rows + rpw - 1) / rpw; }
 
 size_t lds_for(int var, int cols) { return var == kXI8 ? xs_bytes<kXI8>(cols) : xs_bytes<kXF32>(cols); }
 
+template <int R, int NW, int NM, int XF, bool MERGE>
+void launch_pro(bool half, const MatvecParams &p, unsigned grid, size_t lds, hipStream_t st)
+{
+    if (half)
+        hipLaunchKernelGGL((q4k_gemv_half_kernel<R, NW, NM, XF, MERGE>), dim3(grid), dim3(NW * 64), lds, st, p);
+    else if (p.bpr > 16)
+        hipLaunchKernelGGL((q4k_gemv_kernel<R, NW, NM, XF, true, MERGE>), dim3(grid), dim3(NW * 64), lds, st, p);
+    else
+        hipLaunchKernelGGL((q4k_gemv_kernel<R, NW, NM, XF, false, MERGE>), dim3(grid), dim3(NW * 64), lds, st, p);
+}
+
 template <int R, int NW, int NM, int XF>
 int launch_inst(bool half, const MatvecParams &p, int total_waves, hipStream_t st)
 {
     const unsigned grid = (unsigned)((total_waves + NW - 1) / NW);
     const size_t lds = xs_bytes<XF>(p.bpr * 256);
-    if (half)
-        hipLaunchKernelGGL((q4k_gemv_half_kernel<R, NW, NM, XF>), dim3(grid), dim3(NW * 64), lds, st, p);
-    else if (p.bpr > 16)
-        hipLaunchKernelGGL((q4k_gemv_kernel<R, NW, NM, XF, true>), dim3(grid), dim3(NW * 64), lds, st, p);
-    else
-        hipLaunchKernelGGL((q4k_gemv_kernel<R, NW, NM, XF, false>), dim3(grid), dim3(NW * 64), lds, st, p);
+    if (NM == 1 && p.pro.kind == kMergeParts) launch_pro<R, NW, 1, XF, true>(half, p, grid, lds, st);
+    else launch_pro<R, NW, NM, XF, false>(half, p, grid, lds, st);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : hip_fail(e, "q4k_gemv launch");
 }

@@ -38,9 +38,13 @@ typedef struct ksh_buf ksh_buf;
 typedef struct ksh_kernel ksh_kernel;
 typedef struct ksh_graph ksh_graph;
 
-/* DType, crates/ksearch_ir/src/lib.rs:17-27 (same order) */
+/* DType, crates/ksearch_ir/src/lib.rs:17-27 (same order).
+ * KSH_Q6K_ROWS has no counterpart there: it is Q6_K with the bytes of every weight row regrouped by field
+ * (all ql of the row's superblocks, then all qh, all scales, all d: the same 210 B per 256 weights, every
+ * field 16-byte aligned), which is how the LM head is kept in HBM so that a wave fetches a row with whole
+ * 128-bit loads.  KSH_REPACK_ROWS makes it from Q6_K; rows must be a multiple of 2048 columns long. */
 enum ksh_dtype {
-    KSH_F32 = 0, KSH_F16 = 1, KSH_Q4K = 2, KSH_Q5K = 3, KSH_Q6K = 4, KSH_Q40 = 5, KSH_BF16 = 6
+    KSH_F32 = 0, KSH_F16 = 1, KSH_Q4K = 2, KSH_Q5K = 3, KSH_Q6K = 4, KSH_Q40 = 5, KSH_BF16 = 6, KSH_Q6K_ROWS = 7
 };
 
 /* The KernelKind variants on the hot path (crates/ksearch_ir/src/kernel.rs:399-744).
@@ -144,6 +148,9 @@ enum ksh_kind {
      * in: W Q4_K[rows, n_q*hd], parts (as written by KSH_ATTEND_DECODE with dims[5] = 1)
      * out: y f32[rows] */
     KSH_ATTN_MERGE_MATVEC = 23,
+    /* Q6_K [rows, cols] -> KSH_Q6K_ROWS, a byte permutation inside every row (done once, when weights are
+     * loaded).  dims: rows, cols (a multiple of 2048).  in: src Q6_K   out: dst (same size, 16-byte aligned) */
+    KSH_REPACK_ROWS = 24,
     KSH_KIND_COUNT
 };
 

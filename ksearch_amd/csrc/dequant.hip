@@ -108,7 +108,51 @@ int launch_dequant(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
     return e == hipSuccess ? 0 : hip_fail(e, "dequant launch");
 }
 
+// Q6_K -> Q6K_ROWS: one workgroup per weight row, one thread per output dword.  Row of bpr superblocks:
+// ql [bpr][128] | qh [bpr][64] | sc [bpr][16] | d [bpr][2].
+__global__ __launch_bounds__(256) void repack_q6k_rows_kernel(const uint8_t *src, uint8_t *dst, int bpr)
+{
+    const size_t row = blockIdx.x, rb = (size_t)bpr * 210;
+    const uint16_t *s = reinterpret_cast<const uint16_t *>(src + row * rb);   // blocks are 2-byte aligned
+    uint16_t *d = reinterpret_cast<uint16_t *>(dst + row * rb);
+    const int nql = bpr * 64, nqh = bpr * 32, nsc = bpr * 8;                   // in 16-bit units
+    for (int o = threadIdx.x; o < (int)(rb / 2); o += 256) {
+        int b, i;
+        if (o < nql) { b = o / 64; i = o % 64; }
+        else if (o < nql + nqh) { b = (o - nql) / 32; i = 64 + (o - nql) % 32; }
+        else if (o < nql + nqh + nsc) { b = (o - nql - nqh) / 8; i = 96 + (o - nql - nqh) % 8; }
+        else { b = o - nql - nqh - nsc; i = 104; }
+        d[o] = s[b * 105 + i];
+    }
+}
+
+int launch_repack_rows(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
+{
+    hipLaunchKernelGGL(repack_q6k_rows_kernel, dim3((unsigned)k.desc.dims[0]), dim3(256), 0, st, (const uint8_t *)a.in[0],
+                       (uint8_t *)a.out[0], (int)(k.desc.dims[1] / 256));
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : hip_fail(e, "repack launch");
+}
+
 }  // namespace
+
+int bind_repack_rows(ksh_kernel &k)
+{
+    const int64_t rows = k.desc.dims[0], cols = k.desc.dims[1];
+    if (k.desc.dtypes[0] != KSH_Q6K || k.desc.dtypes[1] != KSH_Q6K_ROWS)
+        return set_error("repack_rows: only Q6_K -> Q6K_ROWS is built (got %d -> %d)", k.desc.dtypes[0], k.desc.dtypes[1]);
+    if (rows <= 0 || rows > 0x7FFFFFFF || cols <= 0 || cols % 2048 || cols > (1 << 20))
+        return set_error("repack_rows: rows=%lld cols=%lld (cols must be a positive multiple of 2048)", (long long)rows, (long long)cols);
+    k.info.n_inputs = 1;
+    k.info.n_outputs = 1;
+    k.in_bytes[0] = k.out_bytes[0] = (size_t)rows * (cols / 256) * 210;
+    k.in_align[0] = 2;
+    k.out_align[0] = 16;
+    set_launch(k, (uint32_t)rows, 1, 1, 256, 0);
+    set_name(k, "repack_q6k_rows");
+    k.launch = launch_repack_rows;
+    return 0;
+}
 
 int bind_dequant(ksh_kernel &k)
 {

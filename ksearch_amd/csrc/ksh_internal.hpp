@@ -68,7 +68,7 @@ inline bool block_spec(int dtype, size_t &elems, size_t &bytes)
     case KSH_Q40: elems = 32; bytes = 18; return true;
     case KSH_Q4K: elems = 256; bytes = 144; return true;
     case KSH_Q5K: elems = 256; bytes = 176; return true;
-    case KSH_Q6K: elems = 256; bytes = 210; return true;
+    case KSH_Q6K: case KSH_Q6K_ROWS: elems = 256; bytes = 210; return true;
     }
     return false;
 }
@@ -96,6 +96,7 @@ int bind_matvec_qkv(ksh_kernel &k);
 int bind_matvec_gate_up_gelu(ksh_kernel &k);
 int bind_matvec_batch(ksh_kernel &k);
 int bind_dequant(ksh_kernel &k);
+int bind_repack_rows(ksh_kernel &k);
 int bind_quantize_k(ksh_kernel &k);
 int bind_quantize_q40(ksh_kernel &k);
 int bind_sdpa(ksh_kernel &k);

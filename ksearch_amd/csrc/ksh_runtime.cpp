@@ -36,7 +36,8 @@ int bind_matvec(ksh_kernel &k)
         return set_error("matvec: activation dtype %d is not built (f32 only)", k.desc.dtypes[1]);
     switch (k.desc.dtypes[0]) {
     case KSH_Q4K: return bind_matvec_q4k(k);
-    case KSH_Q6K: return bind_matvec_q6k(k);
+    case KSH_Q6K:
+    case KSH_Q6K_ROWS: return bind_matvec_q6k(k);
     }
     // unsupported dtype in lowering is an error, crates/ksearch_codegen/src/lower.rs:44-48
     return set_error("matvec: weight dtype %d is not built (Q4_K and Q6_K are)", k.desc.dtypes[0]);
@@ -67,6 +68,7 @@ static int bind(ksh_kernel &k)
     case KSH_COPY_SLICE: return bind_glue(k);
     case KSH_SOFTCAP_ARGMAX: return bind_softcap_argmax(k);
     case KSH_DEQUANT: return bind_dequant(k);
+    case KSH_REPACK_ROWS: return bind_repack_rows(k);
     case KSH_QUANTIZE_K: return bind_quantize_k(k);
     }
     return set_error("unknown kernel kind %d", k.desc.kind);

@@ -192,6 +192,130 @@ __global__ __launch_bounds__(NW * 64) void q6k_gemv_kernel(Q6kParams p)
     }
 }
 
+// ---- Q6K_ROWS: the same weights with every row regrouped by field ------------
+// Row of bpr superblocks (bpr a multiple of 8): ql [bpr][128] | qh [bpr][64] | sc [bpr][16] | d [bpr][2], each
+// section 16-byte aligned.  A step covers 8 superblocks with ONE 128-bit load per lane over 1 KB of ql, lane
+// after lane: lane j = lane % 8 of superblock b = lane / 8 holds ql bytes 16j .. 16j+15, i.e. in half ip = j / 4
+// the positions l0 = 16 * (j % 2) .. +15 of the quadrants k = part (low nibbles) and part + 2 (high nibbles),
+// part = (j / 2) % 2.  It fetches the 16 qh bytes of those positions (lanes j and j ^ 2 the same ones), the
+// half's 8 scale bytes and d.  A row is then fetched through the fewest cache lines it spans (14) instead of
+// the ~80 that the per-field loads of the 210-byte superblocks touch.
+struct Q6rLane {
+    u32x4_t ql, qh;
+    u32x2 sc;
+    uint32_t d;
+};
+
+__device__ __forceinline__ Q6rLane q6r_load(const uint8_t *row, int bpr, int blk, int lane)
+{
+    const int j = lane & 7, ip = j >> 2;
+    Q6rLane r;
+    r.ql = *(const KSH_GLOBAL u32x4_t *)(row + (size_t)blk * 128 + 16 * j);
+    r.qh = *(const KSH_GLOBAL u32x4_t *)(row + (size_t)bpr * 128 + (size_t)blk * 64 + 32 * ip + 16 * (j & 1));
+    r.sc = *(const KSH_GLOBAL u32x2 *)(row + (size_t)bpr * 192 + (size_t)blk * 16 + 8 * ip);
+    r.d = *(const KSH_GLOBAL uint16_t *)(row + (size_t)bpr * 208 + (size_t)blk * 2);
+    return r;
+}
+
+// the lane's share of the staged vector: digit planes of its 16 positions in its two quadrants, minus 32 times
+// the sum of X over each 16, and the scale of its 128-element half
+struct XQ6r {
+    u32x4_t H[2], M[2], L[2];
+    int nsx5[2];
+    float s;
+    __device__ __forceinline__ void load(const uint8_t *lds, int blk, int lane, bool valid)
+    {
+        const int j = lane & 7, ip = j >> 2, part = (j >> 1) & 1, l0 = 16 * (j & 1);
+        const uint8_t *half = lds + (blk * 2 + ip) * kQ6HalfBytes;
+#pragma unroll
+        for (int q = 0; q < 2; q++) {
+            const int k = part + 2 * q, o = 32 * k + l0;
+            H[q] = *reinterpret_cast<const u32x4_t *>(half + o);
+            M[q] = *reinterpret_cast<const u32x4_t *>(half + 128 + o);
+            L[q] = *reinterpret_cast<const u32x4_t *>(half + 256 + o);
+            const int *nsx = reinterpret_cast<const int *>(half + 384) + 4 * k + 2 * (j & 1);   // runs of 8
+            nsx5[q] = (nsx[0] + nsx[1]) * 32;
+        }
+        s = valid ? *reinterpret_cast<const float *>(half + 448) : 0.f;
+    }
+};
+
+__device__ __forceinline__ float q6r_lane_dot(const Q6rLane &B, int lane, const XQ6r &X)
+{
+    const int j = lane & 7, part = (j >> 1) & 1;
+    int hs[2], ms[2], ls[2];
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+        const uint32_t t = B.qh[w] >> (2 * part);
+        const uint32_t a[2] = {(B.ql[w] & 0x0F0F0F0Fu) | ((t << 4) & 0x30303030u), ((B.ql[w] >> 4) & 0x0F0F0F0Fu) | (t & 0x30303030u)};
+#pragma unroll
+        for (int q = 0; q < 2; q++) {
+            if (w == 0) {
+                hs[q] = dot4_start((int)a[q], (int)X.H[q][0]);
+                ms[q] = dot4_start((int)a[q], (int)X.M[q][0]);
+                ls[q] = __builtin_amdgcn_sdot4((int)a[q], (int)X.L[q][0], X.nsx5[q], false);   // starts at -32*sum(X)
+            } else {
+                hs[q] = __builtin_amdgcn_sdot4((int)a[q], (int)X.H[q][w], hs[q], false);
+                ms[q] = __builtin_amdgcn_sdot4((int)a[q], (int)X.M[q][w], ms[q], false);
+                ls[q] = __builtin_amdgcn_sdot4((int)a[q], (int)X.L[q][w], ls[q], false);
+            }
+        }
+    }
+    // scales of the half: index 2k + l0/16 for k = part and part + 2: byte 2*part + (j&1) of each dword
+    const int sh = 8 * (2 * part + (j & 1));
+    const float c0 = (float)(int8_t)(B.sc.x >> sh), c1 = (float)(int8_t)(B.sc.y >> sh);
+    const int x0 = (((hs[0] << 7) + ms[0]) << 7) + ls[0], x1 = (((hs[1] << 7) + ms[1]) << 7) + ls[1];
+    return (half_bits_to_f32(B.d) * X.s) * fmaf(c1, (float)x1, c0 * (float)x0);
+}
+
+template <int R, int NW, int STEPS>
+__global__ __launch_bounds__(NW * 64) void q6r_gemv_kernel(Q6kParams p)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t xs[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int bl = lane >> 3;
+    const int cols = p.bpr * 256;
+    const size_t row_bytes = (size_t)p.bpr * kQ6kBytes;
+    const int w0 = (blockIdx.x * NW + wave) * p.rows_per_wave;
+    const int w1 = min(w0 + p.rows_per_wave, p.rows);
+
+    Q6rLane cur[STEPS][R], nxt[STEPS][R];
+    auto load_rows = [&](Q6rLane (&dst)[STEPS][R], int row0) {
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const uint8_t *rp = p.W + (size_t)min(row0 + r, p.rows - 1) * row_bytes;
+#pragma unroll
+            for (int s = 0; s < STEPS; s++) dst[s][r] = q6r_load(rp, p.bpr, s * 8 + bl, lane);   // bpr is a multiple of 8: every lane's superblock exists
+        }
+    };
+    StageRegs sr;
+    stage_fetch<NW * 64>(p.pro, cols, sr);
+    load_rows(cur, min(w0, p.rows - 1));
+    stage_finish<kXQ6, NW * 64>(p.pro, xs, cols, sr);
+    __syncthreads();
+    if (w0 >= w1) return;
+
+    XQ6r X[STEPS];
+#pragma unroll
+    for (int s = 0; s < STEPS; s++) X[s].load(xs, s * 8 + bl, lane, true);
+
+    for (int row0 = w0; row0 < w1; row0 += R) {
+        load_rows(nxt, min(row0 + R, p.rows - 1));
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            float acc = 0.f;
+#pragma unroll
+            for (int s = 0; s < STEPS; s++) acc += q6r_lane_dot(cur[s][r], lane, X[s]);
+            acc = wave_sum(acc);
+            if (lane == 0 && row0 + r < w1) p.y[row0 + r] = acc;
+        }
+#pragma unroll
+        for (int s = 0; s < STEPS; s++)
+#pragma unroll
+            for (int r = 0; r < R; r++) cur[s][r] = nxt[s][r];
+    }
+}
+
 struct Q6kGeom {
     int R, NW, rpw;
 };
@@ -211,8 +335,17 @@ Q6kGeom pick_geom6(const ksh_sched &s, int rows)
 }
 
 template <int R, int NW>
-int launch_steps(int steps, const Q6kParams &p, unsigned grid, size_t lds, hipStream_t st)
+int launch_steps(int steps, bool by_rows, const Q6kParams &p, unsigned grid, size_t lds, hipStream_t st)
 {
+    if (by_rows) {
+        switch (steps) {
+        case 1: hipLaunchKernelGGL((q6r_gemv_kernel<R, NW, 1>), dim3(grid), dim3(NW * 64), lds, st, p); break;
+        case 2: hipLaunchKernelGGL((q6r_gemv_kernel<(R > 2 ? 2 : R), NW, 2>), dim3(grid), dim3(NW * 64), lds, st, p); break;
+        default: return set_error("matvec_q6k: cols=%d is not built for row-grouped weights (2048 and 4096 are)", p.bpr * 256);
+        }
+        const hipError_t e = hipGetLastError();
+        return e == hipSuccess ? 0 : hip_fail(e, "q6k_gemv launch");
+    }
     switch (steps) {
     case 1: hipLaunchKernelGGL((q6k_gemv_kernel<R, NW, 1>), dim3(grid), dim3(NW * 64), lds, st, p); break;
     case 2: hipLaunchKernelGGL((q6k_gemv_kernel<(R > 2 ? 2 : R), NW, 2>), dim3(grid), dim3(NW * 64), lds, st, p); break;
@@ -246,7 +379,7 @@ int launch_matvec_q6k(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
     const size_t lds = k.info.lds_bytes;
     const int steps = (p.bpr + 7) / 8;
 #define KSH_CASE(r, w) \
-    if (R == r && NW == w) return launch_steps<r, w>(steps, p, grid, lds, st);
+    if (R == r && NW == w) return launch_steps<r, w>(steps, k.desc.dtypes[0] == KSH_Q6K_ROWS, p, grid, lds, st);
     KSH_CASE(1, 4) KSH_CASE(2, 4) KSH_CASE(4, 4)
     KSH_CASE(1, 2) KSH_CASE(2, 2) KSH_CASE(4, 2)
     KSH_CASE(1, 8) KSH_CASE(2, 8) KSH_CASE(4, 8)
@@ -264,7 +397,16 @@ int bind_matvec_q6k(ksh_kernel &k)
     if (rows <= 0 || rows > (1 << 30)) return set_error("matvec: rows=%lld", (long long)rows);
     if (cols <= 0 || cols % 256 || cols > 8192)
         return set_error("matvec_q6k: cols=%lld is not a positive multiple of 256 up to 8192", (long long)cols);
+    const bool by_rows = k.desc.dtypes[0] == KSH_Q6K_ROWS;
+    if (by_rows && cols != 2048 && cols != 4096)
+        return set_error("matvec_q6k: row-grouped weights are built for 2048 and 4096 columns (got %lld)", (long long)cols);
     Q6kGeom G = pick_geom6(k.desc.sched, (int)rows);
+    if (k.desc.dtypes[0] == KSH_Q6K_ROWS && sched_is_zero(k.desc.sched)) {   // measured best on 262144 x 2048
+        G.NW = 8;
+        G.R = 1;
+        G.rpw = 16;
+        while (G.rpw > 1 && rows / (G.rpw * G.NW) < 2048) G.rpw >>= 1;
+    }
     // keeps the double buffer and the digit planes in registers
     if (cols > 4096) { G.rpw = G.rpw / G.R; G.R = 1; }
     else if (cols > 2048 && G.R > 2) { G.rpw = G.rpw / G.R * 2; G.R = 2; }
@@ -276,7 +418,7 @@ int bind_matvec_q6k(ksh_kernel &k)
     k.info.n_inputs = pro ? (has_res ? 5 : 3) : 2;
     k.info.n_outputs = has_res ? 2 : 1;
     k.in_bytes[0] = (size_t)rows * bpr * kQ6kBytes;
-    k.in_align[0] = 2;
+    k.in_align[0] = by_rows ? 16 : 2;
     for (int i = 1; i < k.info.n_inputs; i++) { k.in_bytes[i] = (size_t)cols * 4; k.in_align[i] = 16; }
     k.out_bytes[0] = (size_t)rows * 4;
     k.out_align[0] = 4;
@@ -291,7 +433,7 @@ int bind_matvec_q6k(ksh_kernel &k)
     k.info.sched.unroll = (uint32_t)(G.rpw / G.R);
     k.info.sched.vec = 3;
     k.info.sched.k_split = 1;
-    set_name(k, "%smatvec_q6k_r%d_w%d_u%d", pro ? (has_res ? "addrms_" : "rms_") : "", G.R, G.NW, G.rpw / G.R);
+    set_name(k, "%smatvec_q6k%s_r%d_w%d_u%d", pro ? (has_res ? "addrms_" : "rms_") : "", by_rows ? "rows" : "", G.R, G.NW, G.rpw / G.R);
     k.variant = G.R | (G.NW << 8) | (G.rpw << 16);
     k.launch = launch_matvec_q6k;
     return 0;

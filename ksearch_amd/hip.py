@@ -31,6 +31,7 @@ class DType(enum.IntEnum):          # crates/ksearch_ir/src/lib.rs:17-27
     Q6K = 4
     Q40 = 5
     BF16 = 6
+    Q6K_ROWS = 7                    # Q6_K regrouped by field inside every row (ksearch_hip.h)
 
 
 class Kind(enum.IntEnum):           # enum ksh_kind
@@ -57,6 +58,7 @@ class Kind(enum.IntEnum):           # enum ksh_kind
     RMSNORM_MATVEC_GATE_UP_GELU = 21
     ATTEND_DECODE = 22
     ATTN_MERGE_MATVEC = 23
+    REPACK_ROWS = 24
 
 
 class Sched(C.Structure):           # ksh_sched: OptSchedule retargeted to gfx950
@@ -487,6 +489,11 @@ class Eng:
         kk = self._k(ctx, Kind.ATTEND_DECODE, (n_q, n_kv, hd, max_seq, nwg, 1), (DType.Q40, DType.F32), (eps, scale), sched)
         ctx.encode_multi(kk, [q, q_norm, rope, k, k_norm, v, meta], [k_cache, v_cache, parts])
         return kk
+
+    # Q6_K -> Q6K_ROWS (a byte permutation inside every row)
+    def repack_rows(self, ctx, rows, cols, src, dst):
+        k = self._k(ctx, Kind.REPACK_ROWS, (rows, cols), (DType.Q6K, DType.Q6K_ROWS), ())
+        ctx.encode_multi(k, [src], [dst])
 
     # SdpaMwgReduce (lower.rs:5897-6087) folded into the GEMV that consumes the attention output
     def attn_merge_matvec_wd(self, ctx, rows, n_q, hd, nwg, wdt, w, parts, y, sched=None):

@@ -16,3 +16,11 @@ def assert_close(got, want, tol, what=""):
     e = rel_err(got, want)
     i = int(np.argmax(e)) if e.size else 0
     assert e.size == 0 or e[i] <= tol, f"{what}: max rel err {e[i]:.3e} at {i} (got {np.ravel(got)[i]}, want {np.ravel(want)[i]})"
+
+
+def q6k_rows(w, rows, cols):
+    """Q6_K bytes [rows, cols/256, 210] -> the library's row-grouped form (KSH_Q6K_ROWS): per row all ql, then all
+    qh, all scales, all d.  The definition the device repacker is checked against."""
+    b = np.asarray(w, dtype=np.uint8).reshape(rows, cols // 256, 210)
+    return np.concatenate([b[:, :, :128].reshape(rows, -1), b[:, :, 128:192].reshape(rows, -1),
+                           b[:, :, 192:208].reshape(rows, -1), b[:, :, 208:].reshape(rows, -1)], axis=1).reshape(-1)

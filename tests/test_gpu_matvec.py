@@ -7,7 +7,7 @@ import pytest
 import oracle
 from ksearch_amd import hip, synth
 from ksearch_amd.hip import DType
-from tests.gpu_util import assert_close
+from tests.gpu_util import assert_close, q6k_rows
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-3
@@ -141,6 +141,40 @@ def test_matvec_q6k(ctx, eng, rows, cols, sched):
     assert_close(ctx.read_f32(by, rows), oracle.matvec(oracle.Q6K, w, rows, cols, x), TOL, f"q6k {rows}x{cols} {sched}")
 
 
+@pytest.mark.parametrize("rows,cols", [(8, 2048), (1000, 2048), (4099, 2048), (300, 4096), (1, 2048)])
+@pytest.mark.parametrize("sched", SCHEDS_Q6K)
+def test_matvec_q6k_row_grouped(ctx, eng, rows, cols, sched):
+    """The LM head's storage form: the device repack is the stated byte permutation, and the GEMV over it gives
+    what the oracle gives for the original Q6_K bytes."""
+    w = synth.q6k_blocks(rows * cols // 256, seed=rows + 1)
+    x = synth.normal_f32(cols, seed=12)
+    bw, br = ctx.buffer_bytes(w), ctx.buffer_empty_bytes(w.size)
+    eng.repack_rows(ctx, rows, cols, bw, br)
+    assert np.array_equal(ctx.read_bytes(br, w.size), q6k_rows(w, rows, cols))
+    by = ctx.buffer_empty_f32(rows)
+    eng.matvec_wd(ctx, rows, cols, DType.Q6K_ROWS, br, ctx.buffer_f32(x), by, sched)
+    assert_close(ctx.read_f32(by, rows), oracle.matvec(oracle.Q6K, w, rows, cols, x), TOL, f"q6k rows {rows}x{cols} {sched}")
+    assert_close(ctx.read_f32(by, rows), oracle.matvec_f64(oracle.Q6K, w, rows, cols, x), 1e-5, "vs f64")
+
+
+def test_matvec_q6k_row_grouped_unit_vectors_and_errors(ctx, eng):
+    rows, cols = 4, 2048
+    w = synth.q6k_blocks(rows * cols // 256, seed=5)
+    wd = oracle.dequant(oracle.Q6K, w, rows * cols).reshape(rows, cols)
+    br, by = ctx.buffer_bytes(q6k_rows(w, rows, cols)), ctx.buffer_empty_f32(rows)
+    for j in [0, 7, 8, 15, 16, 31, 32, 64, 96, 127, 128, 255, 256, 2047]:   # pins the position of every field
+        e = np.zeros(cols, dtype=np.float32)
+        e[j] = 1.0
+        eng.matvec_wd(ctx, rows, cols, DType.Q6K_ROWS, br, ctx.buffer_f32(e), by)
+        assert np.allclose(ctx.read_f32(by, rows), wd[:, j], rtol=1e-6, atol=1e-9), j
+    with pytest.raises(hip.KshError, match="2048 and 4096"):
+        ctx.compile(hip.make_desc(hip.Kind.MATVEC, (64, 1024), (DType.Q6K_ROWS, DType.F32)))
+    with pytest.raises(hip.KshError, match="multiple of 2048"):
+        ctx.compile(hip.make_desc(hip.Kind.REPACK_ROWS, (64, 1024), (DType.Q6K, DType.Q6K_ROWS)))
+    with pytest.raises(hip.KshError, match="only Q6_K"):
+        ctx.compile(hip.make_desc(hip.Kind.REPACK_ROWS, (64, 2048), (DType.Q4K, DType.Q6K_ROWS)))
+
+
 def test_matvec_q6k_unit_vectors(ctx, eng):
     rows, cols = 4, 2048
     w = synth.q6k_blocks(rows * cols // 256, seed=4)
@@ -256,11 +290,12 @@ def test_rmsnorm_matvec_q6k_lm_head_prologue(ctx, eng, has_res):
     bx, bwn, bwp, br = (ctx.buffer_f32(a) for a in (x, w_norm, w_post, res))
     y, xn = ctx.buffer_empty_f32(rows), ctx.buffer_empty_f32(n)
     extra = dict(w_post=bwp, res=br, x_new=xn) if has_res else {}
-    eng.rmsnorm_matvec_wd(ctx, rows, n, eps, DType.Q6K, bx, bwn, ctx.buffer_bytes(w), y, **extra)
-    assert_close(ctx.read_f32(y, rows), oracle.matvec(oracle.Q6K, w, rows, n, vec), TOL, "rms_matvec_q6k")
-    assert_close(ctx.read_f32(y, rows), oracle.matvec_f64(oracle.Q6K, w, rows, n, vec), 1e-5, "rms_matvec_q6k vs f64")
-    if has_res:
-        assert_close(ctx.read_f32(xn, n), x_new, 1e-5, "x_new")
+    for dt, wb in ((DType.Q6K, w), (DType.Q6K_ROWS, q6k_rows(w, rows, n))):
+        eng.rmsnorm_matvec_wd(ctx, rows, n, eps, dt, bx, bwn, ctx.buffer_bytes(wb), y, **extra)
+        assert_close(ctx.read_f32(y, rows), oracle.matvec(oracle.Q6K, w, rows, n, vec), TOL, f"rms_matvec_q6k {dt}")
+        assert_close(ctx.read_f32(y, rows), oracle.matvec_f64(oracle.Q6K, w, rows, n, vec), 1e-5, f"rms_matvec_q6k vs f64 {dt}")
+        if has_res:
+            assert_close(ctx.read_f32(xn, n), x_new, 1e-5, "x_new")
 
 
 def test_beam_search_on_device(ctx, eng, tmp_path, monkeypatch):

@@ -202,7 +202,7 @@ def cpu_baseline_matvec(w, x, rows, cols, budget_s=1.5):
 # HBM bytes per launch of the headline kernel, from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
 # profiles/q4k_gemv_cfg0_cold.txt (2.00 x 4760.1 KiB fetched + 16.0 KiB written).  Counters cannot be read from
 # inside this script, so the figure is carried here for the kernel it was taken on and is null for any other.
-MEASURED_TRAFFIC_BYTES = {"matvec_q4k_r2_w8_v3": 9765069}
+MEASURED_TRAFFIC_BYTES = {"matvec_q4k_r2_w8_v3": 9753805}
 
 
 def main() -> int:
@@ -253,7 +253,6 @@ def main() -> int:
         hot = bench_matvec(ctx, eng, ev, DType.Q4K, rows, cols, w, x, 1, args.steps, args.warmup)
         also["cfg0_hot_cache"] = dict(us_per_launch=round(hot["us_per_launch"], 3), gbps=round(hot["gbps"], 1))
         also["cfg1_q6k_lm_head"] = bench_lm_head(ctx, eng, ev)
-        del w1
         also["cfg2_q4k_prefill_gemm"] = bench_prefill(ctx)
         also["cfg3_q40_attention"] = bench_attention(ctx)
         also["cfg4_gemma_decode"] = bench_decode(ctx, eng)

@@ -561,6 +561,7 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
         }
 #pragma unroll
         for (int h = 0; h < GP; h++) {
+            if (h >= groups) break;   // heads past the workgroup's share carry nothing
             const float o8 = 8.f * st.S[h];
             float *o = my + 2 * GP + h * HD + 32 * b + 4 * w;
             *reinterpret_cast<float4 *>(o) = make_float4(st.O[h][0] - o8, st.O[h][1] - o8, st.O[h][2] - o8, st.O[h][3] - o8);
@@ -569,18 +570,42 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
     }
     __syncthreads();
     KSH_MARK(4);
-    for (int h = wave; h < groups; h += NW) merge_weights(slots + 2 * h, SLOTF, NSLOT, NSLOT, wts + h * NSLOT, mlh + 2 * h, lane);
-    __syncthreads();
     {
-        // fully unrolled: one wave per SIMD has nothing to hide an LDS round trip behind, so all reads go out first
+        // One barrier: every thread works out its head's weights exp(m_s - M) itself (NSLOT broadcast reads and
+        // exponentials) instead of waiting for a wave per head to publish them behind a second barrier.
+        // Fully unrolled: one wave per SIMD has nothing to hide an LDS round trip behind, so all reads go out first.
+        // (With four outputs per thread -- eight heads -- that is four times the exponentials: there a wave per head
+        // publishes the weights and a second barrier follows, 1 us less at 4 slots x 64 partitions.)
         constexpr int OBW = GP * HD / NT;
-        float accw[OBW];
+        constexpr bool kOwnWeights = OBW <= 2;
+        float accw[OBW], Mh[OBW], Lh[OBW];
+        if (!kOwnWeights) {
+            for (int h = wave; h < groups; h += NW) merge_weights(slots + 2 * h, SLOTF, NSLOT, NSLOT, wts + h * NSLOT, mlh + 2 * h, lane);
+            __syncthreads();
+        }
 #pragma unroll
         for (int ob = 0; ob < OBW; ob++) {
+            accw[ob] = 0.f; Mh[ob] = 0.f; Lh[ob] = 1.f;
+            if (ob * NT >= groups * HD) continue;   // (the same for the whole workgroup)
             const int o = min(tid + ob * NT, groups * HD - 1), h = o / HD, d = o % HD;
-            accw[ob] = 0.f;
+            float M = -1.0e30f, L = 0.f, a = 0.f;
+            if (kOwnWeights) {
+                float mv[NSLOT];
 #pragma unroll
-            for (int s = 0; s < NSLOT; s++) accw[ob] = fmaf(wts[h * NSLOT + s], slots[s * SLOTF + 2 * GP + h * HD + d], accw[ob]);
+                for (int s = 0; s < NSLOT; s++) { mv[s] = slots[s * SLOTF + 2 * h]; M = fmaxf(M, mv[s]); }
+#pragma unroll
+                for (int s = 0; s < NSLOT; s++) {
+                    const float wt = __expf(mv[s] - M);
+                    L = fmaf(wt, slots[s * SLOTF + 2 * h + 1], L);
+                    a = fmaf(wt, slots[s * SLOTF + 2 * GP + h * HD + d], a);
+                }
+            } else {
+#pragma unroll
+                for (int s = 0; s < NSLOT; s++) a = fmaf(wts[h * NSLOT + s], slots[s * SLOTF + 2 * GP + h * HD + d], a);
+                M = mlh[2 * h];
+                L = mlh[2 * h + 1];
+            }
+            accw[ob] = a; Mh[ob] = M; Lh[ob] = L;
         }
 #pragma unroll
         for (int ob = 0; ob < OBW; ob++) {
@@ -588,21 +613,21 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
             if (o >= groups * HD) continue;
             const int h = o / HD, d = o % HD, head = head0 + h;
             if (p.mode == kModeDirect) {
-                p.out[((size_t)slot * p.n_q + head) * HD + d] = accw[ob] / mlh[2 * h + 1];
+                p.out[((size_t)slot * p.n_q + head) * HD + d] = accw[ob] / Lh[ob];
             } else if (p.balance) {
                 const size_t r = rec_base * p.n_q + head;
                 float *ml = p.tmp + (size_t)gridDim.z * p.nwg * p.n_q * HD;
                 p.tmp[r * HD + d] = accw[ob];
-                if (d == 0) { ml[2 * r] = mlh[2 * h]; ml[2 * r + 1] = mlh[2 * h + 1]; }
+                if (d == 0) { ml[2 * r] = Mh[ob]; ml[2 * r + 1] = Lh[ob]; }
             } else if (p.mode == kModeSplitPart) {
                 const size_t r = ((size_t)slot * p.n_q + head) * p.nwg + part;
                 float *ml = p.tmp + (size_t)gridDim.z * p.n_q * p.nwg * HD;
                 p.tmp[r * HD + d] = accw[ob];
-                if (d == 0) { ml[2 * r] = mlh[2 * h]; ml[2 * r + 1] = mlh[2 * h + 1]; }
+                if (d == 0) { ml[2 * r] = Mh[ob]; ml[2 * r + 1] = Lh[ob]; }
             } else {
                 float *rec = p.tmp + rec_base + head * rec_hs + part * rec_ps;
                 st_agent(rec + 2 + d, accw[ob]);
-                if (d == 0) { st_agent(rec, mlh[2 * h]); st_agent(rec + 1, mlh[2 * h + 1]); }
+                if (d == 0) { st_agent(rec, Mh[ob]); st_agent(rec + 1, Lh[ob]); }
             }
         }
     }

@@ -138,7 +138,9 @@ enum ksh_kind {
      *      out f32[n_q*hd].  Built for hd 128 / 256, up to 8 q heads per kv head.
      * With dims[5] = 1 the partitions are not merged: the outputs are K cache,
      * V cache and parts = { o f32[n_q, nwg, hd] (unnormalised), ml f32[n_q, nwg, 2]
-     * (running max, sum) } in one buffer, for KSH_ATTN_MERGE_MATVEC. */
+     * (running max, sum) } in one buffer, for KSH_ATTN_MERGE_MATVEC.
+     * With dims[6] = 1 the rope input is the row of the table for meta's pos, f32[hd], kept current by the
+     * caller: the launch then has nothing to wait for between reading pos and fetching its rope values. */
     KSH_ATTEND_DECODE = 22,
     /* SdpaMwgReduce (crates/ksearch_metal/src/lower.rs:5897-6087) folded into the
      * GEMV that consumes the attention output: every workgroup merges the

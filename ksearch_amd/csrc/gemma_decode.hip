@@ -39,11 +39,16 @@
 
 namespace {
 
-// end of token: remember the id, advance position and attended length
-__global__ void advance_kernel(float *meta, const float *tok, float *history, int max_hist)
+// end of token: remember the id, advance position and attended length, and put the next position's row of the
+// rope table where the attention launches read it (they then fetch it without first waiting for the position)
+__global__ void advance_kernel(float *meta, const float *tok, float *history, int max_hist, const float *rope,
+                               float *rope_cur, int hd)
 {
-    if (threadIdx.x == 0 && blockIdx.x == 0) {
-        const int pos = (int)meta[3];
+    const int pos = (int)meta[3];
+    __syncthreads();   // every thread has read the position before thread 0 moves it
+    if (pos + 1 < max_hist)
+        for (int i = threadIdx.x; i < hd; i += blockDim.x) rope_cur[i] = rope[(size_t)(pos + 1) * hd + i];
+    if (threadIdx.x == 0) {
         if (history && pos < max_hist) history[pos] = tok[0];
         meta[3] = (float)(pos + 1);
         meta[0] = (float)(pos + 2);   // the next token attends rows [0, pos+1]
@@ -75,7 +80,7 @@ struct ksh_gemma {
     ksh_buf *embd_rows = nullptr;   // the LM head's copy of the embedding table, rows regrouped by field (KSH_Q6K_ROWS)
     Bufs bufs;
     ksh_buf *x = nullptr, *xb = nullptr, *y = nullptr, *x2 = nullptr, *hidden = nullptr, *tq = nullptr, *tk = nullptr, *tv = nullptr, *to = nullptr, *ff = nullptr,
-            *logits = nullptr, *tok = nullptr, *meta = nullptr, *rope = nullptr, *attn_tmp = nullptr,
+            *logits = nullptr, *tok = nullptr, *meta = nullptr, *rope = nullptr, *rope_cur = nullptr, *attn_tmp = nullptr,
             *history = nullptr;
     std::vector<ksh_buf *> kv_k, kv_v;
     ksh_kernel *k_embed = nullptr, *k_qkv_first = nullptr, *k_qkv = nullptr, *k_head = nullptr, *k_sdpa = nullptr, *k_attend = nullptr,
@@ -88,6 +93,7 @@ struct ksh_gemma {
     int nwg = 16;
     int sdpa_launches = 2;
     int short_context = 0;   // positions below this use the short-context graph
+    std::vector<float> rope0;   // row 0 of the rope table, for reset
 };
 
 namespace {
@@ -153,11 +159,11 @@ int encode_token(ksh_gemma *m, bool want_logits, bool short_ctx, int &launches)
             std::swap(cur, other);
         }
         if (short_ctx) {
-            if (enc(m, m->k_attend_parts, {m->tq, L.q_norm, m->rope, m->tk, L.k_norm, m->tv, m->meta},
+            if (enc(m, m->k_attend_parts, {m->tq, L.q_norm, m->rope_cur, m->tk, L.k_norm, m->tv, m->meta},
                     {m->kv_k[l], m->kv_v[l], m->attn_tmp}, launches))
                 return 1;
         } else if (m->k_attend) {
-            if (enc(m, m->k_attend, {m->tq, L.q_norm, m->rope, m->tk, L.k_norm, m->tv, m->meta},
+            if (enc(m, m->k_attend, {m->tq, L.q_norm, m->rope_cur, m->tk, L.k_norm, m->tv, m->meta},
                     {m->kv_k[l], m->kv_v[l], m->attn_tmp, m->to}, launches))
                 return 1;
         } else {
@@ -185,7 +191,8 @@ int encode_token(ksh_gemma *m, bool want_logits, bool short_ctx, int &launches)
     hipStream_t st = (hipStream_t)ksh_stream(m->ctx);
     hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(64), 0, st, (float *)ksh_buffer_device_ptr(m->meta),
                        (const float *)ksh_buffer_device_ptr(m->tok),
-                       want_logits ? (float *)ksh_buffer_device_ptr(m->history) : nullptr, c.max_seq);
+                       want_logits ? (float *)ksh_buffer_device_ptr(m->history) : nullptr, c.max_seq,
+                       (const float *)ksh_buffer_device_ptr(m->rope), (float *)ksh_buffer_device_ptr(m->rope_cur), c.hd);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return hip_fail(e, "advance launch");
     launches += 1;
@@ -276,6 +283,8 @@ int ksh_gemma_create(ksh_ctx *ctx, const ksh_gemma_cfg *cfg, const ksh_gemma_lay
             }
         if (ksh_buffer_alloc(ctx, tab.size() * 4, tab.data(), &g->rope)) return 1;
         g->bufs.owned.push_back(g->rope);
+        g->rope0.assign(tab.begin(), tab.begin() + c.hd);
+        if (alloc(g, (size_t)c.hd * 4, &g->rope_cur)) return 1;   // the current position's row (advance_kernel keeps it so)
     }
     if (alloc(g, (size_t)c.n_q * std::max(g->nwg, kShortPartitions) * (c.hd + 2) * 4, &g->attn_tmp)) return 1;
 
@@ -303,13 +312,13 @@ int ksh_gemma_create(ksh_ctx *ctx, const ksh_gemma_cfg *cfg, const ksh_gemma_lay
     // per-head norm + RoPE + KV append + attention + merge: one launch where the fused kind is built for the
     // shape, the three reference ops otherwise
     if (sdpa_lanes_supports(c.n_q, c.n_kv, c.hd)) {
-        if (get(g, KSH_ATTEND_DECODE, {c.n_q, c.n_kv, c.hd, c.max_seq, g->nwg}, {KSH_Q40, KSH_F32}, {c.eps, c.attn_scale},
+        if (get(g, KSH_ATTEND_DECODE, {c.n_q, c.n_kv, c.hd, c.max_seq, g->nwg, 0, 1}, {KSH_Q40, KSH_F32}, {c.eps, c.attn_scale},
                 &g->k_attend))
             return 1;
         g->short_context = kShortContext;
         if (const char *e = getenv("KSEARCH_SHORT_CONTEXT")) g->short_context = atoi(e);
         if (g->short_context > 0 && qd <= 2048 && (c.hd & (c.hd - 1)) == 0 &&
-            (get(g, KSH_ATTEND_DECODE, {c.n_q, c.n_kv, c.hd, c.max_seq, kShortPartitions, 1}, {KSH_Q40, KSH_F32},
+            (get(g, KSH_ATTEND_DECODE, {c.n_q, c.n_kv, c.hd, c.max_seq, kShortPartitions, 1, 1}, {KSH_Q40, KSH_F32},
                  {c.eps, c.attn_scale}, &g->k_attend_parts) ||
              get(g, KSH_ATTN_MERGE_MATVEC, {c.hidden, c.n_q, c.hd, kShortPartitions}, {KSH_Q4K, KSH_F32}, {}, &g->k_oproj_merge)))
             return 1;
@@ -340,6 +349,7 @@ int ksh_gemma_reset(ksh_gemma *m)
     if (ksh_synchronize(m->ctx)) return 1;
     const float meta[4] = {1.f, 0.f, 0.f, 0.f};   // tlen, start, window, pos
     if (ksh_buffer_write(m->ctx, m->meta, 0, meta, 16, 1)) return 1;
+    if (ksh_buffer_write(m->ctx, m->rope_cur, 0, m->rope0.data(), m->rope0.size() * 4, 1)) return 1;
     m->pos = 0;
     return 0;
 }

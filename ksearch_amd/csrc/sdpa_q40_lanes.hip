@@ -63,6 +63,7 @@ struct LaneParams {
     int groups;   // q heads this workgroup handles: (n_q / n_kv) / hsplit
     int hsplit;   // workgroups that share a kv head's rows, each with its own q heads
     int balance;  // the launch's nwg * n_slots partitions are dealt to the slots by length (kModeMerge, several slots)
+    int rope_row; // fused: `rope` is the current position's row of the table, not the table
 };
 
 __device__ __forceinline__ uint32_t ld32_a2(const uint8_t *p)
@@ -397,21 +398,15 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
         rec_base = (size_t)first + part;   // flat partition index: values [flat][n_q][HD], then (m, l) [flat][n_q][2]
     }
 
-    const float *meta = p.meta + (size_t)slot * p.meta_stride;
-    const int tlen = (int)meta[0], start = (int)meta[1];
-    const int chunk = (tlen + nparts - 1) / nparts;
-    const int p0 = part * chunk;
-    int p1 = min(p0 + chunk, tlen);
-
     const size_t slot_bytes = (size_t)p.max_t * p.n_kv * ROWB;
     const uint8_t *kbase = p.k + (size_t)slot * slot_bytes + (size_t)kvh * ROWB + 18 * b;
     const uint8_t *vbase = p.v + (size_t)slot * slot_bytes + (size_t)kvh * ROWB + 18 * b;
     const size_t row_stride = (size_t)p.n_kv * ROWB;
     const float *qg = p.q + ((size_t)slot * p.n_q + head0) * HD;
 
-    auto load_row = [&](int t) {
+    auto load_row_at = [&](int first, int t) {
         RowRegs r;
-        const size_t off = (size_t)(start + t) * row_stride;
+        const size_t off = (size_t)(first + t) * row_stride;
         r.kd = ld32_a2(kbase + off + 2 + 4 * w);
         r.ks = ld16_a2(kbase + off);
         r.vd = ld32_a2(vbase + off + 2 + 4 * w);
@@ -419,12 +414,63 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
         return r;
     };
 
-    // the partition's first rows are requested before anything else is worked on
-    const bool owner = p.fused && part == (tlen - 1) / chunk;
-    if (owner) p1 = min(p1, tlen - 1);   // the row this step appends is attended from LDS, at the end
-    constexpr int TILE = NW * RPS * kRT;
+    // The fused decode step deals rows to the partitions in groups of GRP (one step of the workgroup), round
+    // robin: which rows a workgroup starts with then does not depend on the attended length, and its first
+    // loads go out before the length has come back from memory (rows past the end are read -- the cache is
+    // max_t rows long -- and dropped).  The other kinds give every partition one contiguous range.
+    constexpr int GRP = NW * RPS, TILE = GRP * kRT;
+    const bool dealt = p.fused != 0;
+    auto dealt_row = [&](int it, int t) { return ((it * kRT + t) * p.nwg + part) * GRP + wave * RPS + sub; };   // relative to start
     RowRegs cur[kRT], nxt[kRT];
-    {
+
+    // Vector loads return in the order they were issued: the length and position first, then what the fused
+    // prologue needs (raw q / k / v of this workgroup's head tasks, the norm weights, the position's rope row
+    // when it is given directly), then the rows.
+    const float *meta = p.meta + (size_t)slot * p.meta_stride;
+    const float meta_tlen = meta[0], meta_start = meta[1], meta_pos = dealt ? meta[3] : 0.f;
+    // head tasks: q heads 0..groups-1, then K and V (used by the owner only); a wave takes tasks wave, wave+NW, ...
+    constexpr int PER = HD / 64, MAXT = GP / NW + 1;
+    float xv[MAXT][PER], wq[PER], wk[PER], cs[PER / 2], sn[PER / 2];
+    if (dealt) {
+#pragma unroll
+        for (int t = 0; t < MAXT; t++) {
+            const int task = min(wave + t * NW, groups + 1);
+            const float *src = task < groups ? qg + (size_t)task * HD
+                                             : (task == groups ? p.k_raw : p.v_raw) + (size_t)kvh * HD;
+#pragma unroll
+            for (int jj = 0; jj < PER; jj++) xv[t][jj] = src[lane + 64 * jj];
+        }
+#pragma unroll
+        for (int jj = 0; jj < PER; jj++) {
+            wq[jj] = p.qw[lane + 64 * jj];
+            wk[jj] = p.kw[lane + 64 * jj];
+        }
+        if (p.rope_row) {
+#pragma unroll
+            for (int jj = 0; jj < PER / 2; jj++) {
+                cs[jj] = p.rope[lane + 64 * jj];
+                sn[jj] = p.rope[HD / 2 + lane + 64 * jj];
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < kRT; t++) cur[t] = load_row_at(0, min(dealt_row(0, t), p.max_t - 1));   // as if start == 0
+    }
+    const int tlen = (int)meta_tlen, start = (int)meta_start;
+    const int chunk = (tlen + nparts - 1) / nparts;
+    const int p0 = part * chunk;
+    int p1 = min(p0 + chunk, tlen);
+    auto load_row = [&](int t) { return load_row_at(start, t); };
+
+    // the row this step appends is attended from LDS, at the end, by the partition it falls to
+    const bool owner = p.fused && part == (dealt ? ((tlen - 1) / GRP) % p.nwg : (tlen - 1) / chunk);
+    const int tend = tlen - 1;           // dealt: rows [0, tend) come from the cache
+    if (dealt) {
+        if (start != 0) {                // a window that has begun to slide: ask again
+#pragma unroll
+            for (int t = 0; t < kRT; t++) cur[t] = load_row(min(dealt_row(0, t), p.max_t - 1 - start));
+        }
+    } else {
+        if (owner) p1 = min(p1, tlen - 1);
         const int last = max(p1 - 1, p0 < tlen ? p0 : 0);   // an empty partition still loads (a valid row) and drops it
 #pragma unroll
         for (int t = 0; t < kRT; t++) cur[t] = load_row(min(p0 + (t * NW + wave) * RPS + sub, last));
@@ -434,30 +480,15 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
     // ---- q into registers (and, fused, the new K/V row into the cache) -------
     float qv[GP][8], Sq[GP];
     if (p.fused) {
-        const int pos = min(max((int)meta[3], 0), p.max_t - 1);
-        const float *rope = p.rope + (size_t)pos * HD;
-        // head tasks: q heads 0..groups-1, then (owner only) K and V; a wave takes
-        // tasks wave, wave+NW, ... and issues all their loads before the first sum
-        constexpr int PER = HD / 64, MAXT = GP / NW + 1;
+        const int pos = min(max((int)meta_pos, 0), p.max_t - 1);
         const int ntask = groups + (owner ? 2 : 0);
-        float xv[MAXT][PER], wq[PER], wk[PER], cs[PER / 2], sn[PER / 2];
+        if (!p.rope_row) {
+            const float *rope = p.rope + (size_t)pos * HD;
 #pragma unroll
-        for (int t = 0; t < MAXT; t++) {
-            const int task = wave + t * NW;
-            const float *src = task < groups ? qg + (size_t)task * HD
-                                             : (task == groups ? p.k_raw : p.v_raw) + (size_t)kvh * HD;
-#pragma unroll
-            for (int jj = 0; jj < PER; jj++) xv[t][jj] = task < ntask ? src[lane + 64 * jj] : 0.f;
-        }
-#pragma unroll
-        for (int jj = 0; jj < PER; jj++) {
-            wq[jj] = p.qw[lane + 64 * jj];
-            wk[jj] = p.kw[lane + 64 * jj];
-        }
-#pragma unroll
-        for (int jj = 0; jj < PER / 2; jj++) {
-            cs[jj] = rope[lane + 64 * jj];
-            sn[jj] = rope[HD / 2 + lane + 64 * jj];
+            for (int jj = 0; jj < PER / 2; jj++) {
+                cs[jj] = rope[lane + 64 * jj];
+                sn[jj] = rope[HD / 2 + lane + 64 * jj];
+            }
         }
 #pragma unroll
         for (int t = 0; t < MAXT; t++) {
@@ -520,7 +551,20 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
 
     KSH_MARK(2);
     // ---- the partition's rows: kRT steps of RPS rows per wave at a time -----
-    if (p0 < p1) {
+    if (dealt) {
+        for (int it = 0; (it * kRT * p.nwg + part) * GRP < tend; it++) {
+            bool valid[kRT], live[kRT];
+#pragma unroll
+            for (int t = 0; t < kRT; t++) {
+                valid[t] = dealt_row(it, t) < tend;
+                live[t] = ((it * kRT + t) * p.nwg + part) * GRP + wave * RPS < tend;
+                nxt[t] = load_row(min(dealt_row(it + 1, t), p.max_t - 1 - start));   // unconditional: keeps the wait counts exact
+            }
+            process_rows<HD, GP, kRT>(cur, valid, live, qv, Sq, st, c);
+#pragma unroll
+            for (int t = 0; t < kRT; t++) cur[t] = nxt[t];
+        }
+    } else if (p0 < p1) {
         for (int base = p0; base < p1; base += TILE) {
             bool valid[kRT], live[kRT];
 #pragma unroll
@@ -803,6 +847,7 @@ int launch_bound(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
         p.tmp = (float *)a.out[2];
         p.eps = k.desc.params[0];
         p.scale = k.desc.params[1];
+        p.rope_row = k.desc.dims[6] != 0;
         if (k.desc.dims[5]) {
             p.mode = kModeSplitPart;
         } else {
@@ -872,7 +917,7 @@ int bind_attend_decode(ksh_kernel &k)
     const size_t kvb = (size_t)max_t * n_kv * (hd / 32) * 18, qb = (size_t)n_q * hd * 4, kb = (size_t)n_kv * hd * 4;
     k.info.n_inputs = 7;
     k.info.n_outputs = 4;
-    k.in_bytes[0] = qb; k.in_bytes[1] = (size_t)hd * 4; k.in_bytes[2] = (size_t)max_t * hd * 4; k.in_bytes[3] = kb;
+    k.in_bytes[0] = qb; k.in_bytes[1] = (size_t)hd * 4; k.in_bytes[2] = (d[6] ? 1 : (size_t)max_t) * hd * 4; k.in_bytes[3] = kb;
     k.in_bytes[4] = (size_t)hd * 4; k.in_bytes[5] = kb; k.in_bytes[6] = 16;
     for (int i = 0; i < 7; i++) k.in_align[i] = 4;
     k.in_align[0] = 16;

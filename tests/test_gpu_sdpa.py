@@ -166,15 +166,18 @@ def test_sdpa_errors(ctx):
         ctx.compile(hip.make_desc(hip.Kind.SDPA_NAIVE, (8, 3, 256, 64), (DType.Q40, DType.F32), (1.0,)))
 
 
-@pytest.mark.parametrize("n_q,n_kv,hd,max_seq,pos,nwg", [
-    (8, 1, 256, 512, 0, 0),        # the first token attends only itself
-    (8, 1, 256, 512, 1, 4),
-    (8, 1, 256, 512, 200, 16),     # partitions of 13 rows, the last one short
-    (8, 1, 256, 4096, 319, 0),     # the decode loop's shape and default split
-    (4, 1, 128, 256, 77, 3),       # the small decode model
-    (4, 2, 128, 300, 150, 5),      # two kv heads
+@pytest.mark.parametrize("n_q,n_kv,hd,max_seq,pos,nwg,start", [
+    (8, 1, 256, 512, 0, 0, 0),        # the first token attends only itself
+    (8, 1, 256, 512, 1, 4, 0),
+    (8, 1, 256, 512, 200, 16, 0),     # row groups dealt round robin: some partitions get one more than others
+    (8, 1, 256, 4096, 319, 0, 0),     # the decode loop's shape and default split
+    (8, 1, 256, 4096, 1500, 16, 0),   # several rounds of row groups per partition
+    (4, 1, 128, 256, 77, 3, 0),       # the small decode model
+    (4, 2, 128, 300, 150, 5, 0),      # two kv heads
+    (8, 1, 256, 512, 300, 4, 173),    # a window that has begun to slide: rows [173, 300]
+    (4, 1, 128, 256, 255, 2, 250),    # ... ending at the last row of the cache
 ])
-def test_attend_decode_vs_unfused_oracle(ctx, eng, n_q, n_kv, hd, max_seq, pos, nwg):
+def test_attend_decode_vs_unfused_oracle(ctx, eng, n_q, n_kv, hd, max_seq, pos, nwg, start):
     """AttendDecode = RmsNormPerHeadQkvQ40 at `pos` + attention over rows [0, pos] + merge.  The oracle runs the
     three reference ops one after the other; the cache rows the kernel appends are compared as codes (they may
     differ by one step where a value sits on a rounding boundary) and the attention output against the oracle's
@@ -189,7 +192,8 @@ def test_attend_decode_vs_unfused_oracle(ctx, eng, n_q, n_kv, hd, max_seq, pos, 
     rope = oracle.rope_table(max_seq, hd, 10000.0)
     kc, vc = ctx.buffer_bytes(k), ctx.buffer_bytes(v)
     out = ctx.buffer_empty_f32(n_q * hd)
-    meta = ctx.buffer_f32([pos + 1, 0, 0, pos])
+    tlen = pos + 1 - start
+    meta = ctx.buffer_f32([tlen, start, tlen if start else 0, pos])
     kk = ctx.compile(hip.make_desc(hip.Kind.ATTEND_DECODE, (n_q, n_kv, hd, max_seq, nwg), (DType.Q40, DType.F32), (eps, scale)))
     tmp = ctx.buffer_empty_f32(n_q * kk.grid[0] * (hd + 2))
     for rep in range(2):                     # twice: the arrival counter must come back to zero
@@ -203,8 +207,15 @@ def test_attend_decode_vs_unfused_oracle(ctx, eng, n_q, n_kv, hd, max_seq, pos, 
             dg, dw = oracle.dequant(oracle.Q40, g, n_kv * hd), oracle.dequant(oracle.Q40, w_, n_kv * hd)
             assert np.abs(dg - dw).max() <= np.abs(dw).max() / 7.0 * 1.01
             assert (g != w_).mean() < 0.02
-        want = oracle.sdpa(wq, gk, gv, n_q, n_kv, hd, pos + 1, 0, scale, f64=True)
+        want = oracle.sdpa(wq, gk, gv, n_q, n_kv, hd, tlen, start, scale, f64=True)
         assert_close(got, want, TOL, f"rep {rep}")
+    # the same launch given the position's rope row instead of the table (dims[6] = 1): identical bits
+    k2 = ctx.compile(hip.make_desc(hip.Kind.ATTEND_DECODE, (n_q, n_kv, hd, max_seq, nwg, 0, 1), (DType.Q40, DType.F32), (eps, scale)))
+    kc2, vc2, out2 = ctx.buffer_bytes(k), ctx.buffer_bytes(v), ctx.buffer_empty_f32(n_q * hd)
+    ctx.encode_multi(k2, [ctx.buffer_f32(q), ctx.buffer_f32(qw), ctx.buffer_f32(rope[pos]), ctx.buffer_f32(kr), ctx.buffer_f32(kw),
+                          ctx.buffer_f32(vr), meta], [kc2, vc2, tmp, out2])
+    assert np.array_equal(ctx.read_f32(out2, n_q * hd), got)
+    assert np.array_equal(ctx.read_bytes(kc2, (pos + 1) * row), gk) and np.array_equal(ctx.read_bytes(vc2, (pos + 1) * row), gv)
     if pos + 1 < max_seq:
         assert not ctx.read_bytes(kc, row, (pos + 1) * row).any()
 

@@ -420,7 +420,11 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
     // max_t rows long -- and dropped).  The other kinds give every partition one contiguous range.
     constexpr int GRP = NW * RPS, TILE = GRP * kRT;
     const bool dealt = p.fused != 0;
-    auto dealt_row = [&](int it, int t) { return ((it * kRT + t) * p.nwg + part) * GRP + wave * RPS + sub; };   // relative to start
+    // The last partition of a fused step takes no cached rows: it norms, ropes and packs the new K / V row,
+    // stores it and attends it.  That work (0.7 us) would otherwise sit in front of one row partition's rows.
+    const int rparts = p.nwg > 1 ? p.nwg - 1 : 1;              // partitions that share the cached rows
+    const bool has_rows = p.nwg == 1 || part < p.nwg - 1;
+    auto dealt_row = [&](int it, int t) { return ((it * kRT + t) * rparts + part) * GRP + wave * RPS + sub; };   // relative to start
     RowRegs cur[kRT], nxt[kRT];
 
     // Vector loads return in the order they were issued: the length and position first, then what the fused
@@ -461,8 +465,8 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
     int p1 = min(p0 + chunk, tlen);
     auto load_row = [&](int t) { return load_row_at(start, t); };
 
-    // the row this step appends is attended from LDS, at the end, by the partition it falls to
-    const bool owner = p.fused && part == (dealt ? ((tlen - 1) / GRP) % p.nwg : (tlen - 1) / chunk);
+    // the row this step appends is attended from LDS by the last partition (other kinds: by the one whose range holds it)
+    const bool owner = p.fused && (p.nwg == 1 || part == p.nwg - 1);   // (p.fused kinds are always dealt)
     const int tend = tlen - 1;           // dealt: rows [0, tend) come from the cache
     if (dealt) {
         if (start != 0) {                // a window that has begun to slide: ask again
@@ -552,12 +556,12 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
     KSH_MARK(2);
     // ---- the partition's rows: kRT steps of RPS rows per wave at a time -----
     if (dealt) {
-        for (int it = 0; (it * kRT * p.nwg + part) * GRP < tend; it++) {
+        for (int it = 0; has_rows && (it * kRT * rparts + part) * GRP < tend; it++) {
             bool valid[kRT], live[kRT];
 #pragma unroll
             for (int t = 0; t < kRT; t++) {
                 valid[t] = dealt_row(it, t) < tend;
-                live[t] = ((it * kRT + t) * p.nwg + part) * GRP + wave * RPS < tend;
+                live[t] = ((it * kRT + t) * rparts + part) * GRP + wave * RPS < tend;
                 nxt[t] = load_row(min(dealt_row(it + 1, t), p.max_t - 1 - start));   // unconditional: keeps the wait counts exact
             }
             process_rows<HD, GP, kRT>(cur, valid, live, qv, Sq, st, c);

@@ -169,9 +169,12 @@ struct StageRegs {
 };
 
 // kMerge: whether the kernel is built with the kMergeParts source at all (the Q4_K kernels' prologue instances are)
-template <int NT, bool kMerge = false>
+// KMAX: a compile-time bound on the float4 per thread (kernels built for a fixed row length): what lies past it
+// takes no registers, which is what decides the occupancy of the long-running LM head.
+template <int NT, bool kMerge = false, int KMAX = kStageX>
 __device__ __forceinline__ void stage_fetch(const Prologue &pr, int cols, StageRegs &s)
 {
+    constexpr int KX = KMAX < kStageX ? KMAX : kStageX, KP = KMAX < kStageP ? KMAX : kStageP;
     // n4 is a multiple of 64, so "this float4 exists" is a per-wave fact: keep it
     // in scalar registers and the loads stay unpredicated
     const int wbase = __builtin_amdgcn_readfirstlane(threadIdx.x & ~63), tid = wbase + (threadIdx.x & 63), n4 = cols / 4;
@@ -193,21 +196,21 @@ __device__ __forceinline__ void stage_fetch(const Prologue &pr, int cols, StageR
         }
         return;
     }
-    if (n4 > NT * kStageX) return;
+    if (KMAX >= kStageX && n4 > NT * kStageX) return;
 #pragma unroll
-    for (int k = 0; k < kStageX; k++) {
+    for (int k = 0; k < KX; k++) {
         const int i = tid + k * NT;
         if (wbase + k * NT < n4) s.x[k] = ldg_f4(pr.x, i);
     }
     if (pr.kind == kPlain) return;
 #pragma unroll
-    for (int k = 0; k < kStageP; k++) {
+    for (int k = 0; k < KP; k++) {
         const int i = tid + k * NT;
         if (wbase + k * NT < n4) s.wn[k] = ldg_f4(pr.w_norm, i);
     }
     if (pr.kind != kAddThenRms) return;
 #pragma unroll
-    for (int k = 0; k < kStageP; k++) {
+    for (int k = 0; k < KP; k++) {
         const int i = tid + k * NT;
         if (wbase + k * NT < n4) { s.wp[k] = ldg_f4(pr.w_post, i); s.rs[k] = ldg_f4(pr.res, i); }
     }
@@ -215,9 +218,10 @@ __device__ __forceinline__ void stage_fetch(const Prologue &pr, int cols, StageR
 
 // Every thread must call this (it contains barriers); the LDS image is complete
 // after the caller's next __syncthreads().
-template <int XF, int NT, bool kMerge = false>
+template <int XF, int NT, bool kMerge = false, int KMAX = kStageX>
 __device__ __forceinline__ void stage_finish(const Prologue &pr, uint8_t *lds, int cols, StageRegs &s)
 {
+    constexpr int KX = KMAX < kStageX ? KMAX : kStageX, KP = KMAX < kStageP ? KMAX : kStageP;
     const int wbase = __builtin_amdgcn_readfirstlane(threadIdx.x & ~63), tid = wbase + (threadIdx.x & 63), n4 = cols / 4;
     float *red = reinterpret_cast<float *>(lds + xs_image_bytes<XF>(cols));
     if (kMerge && pr.kind == kMergeParts) {
@@ -248,12 +252,12 @@ __device__ __forceinline__ void stage_finish(const Prologue &pr, uint8_t *lds, i
         return;
     }
     if (pr.kind == kPlain) {
-        if (n4 > NT * kStageX) {
+        if (KMAX >= kStageX && n4 > NT * kStageX) {
             for (int i = tid; i < n4; i += NT) store_x4<XF>(lds, cols, i, ldg_f4(pr.x, i));
             return;
         }
 #pragma unroll
-        for (int k = 0; k < kStageX; k++) {
+        for (int k = 0; k < KX; k++) {
             const int i = tid + k * NT;
             if (wbase + k * NT < n4) store_x4<XF>(lds, cols, i, s.x[k]);
         }
@@ -266,7 +270,7 @@ __device__ __forceinline__ void stage_finish(const Prologue &pr, uint8_t *lds, i
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
     const bool add = pr.kind == kAddThenRms;
 #pragma unroll
-    for (int k = 0; k < kStageP; k++) {
+    for (int k = 0; k < KP; k++) {
         if (wbase + k * NT < n4) {
             const float y4[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
             const float r4[4] = {s.rs[k].x, s.rs[k].y, s.rs[k].z, s.rs[k].w};
@@ -305,7 +309,7 @@ __device__ __forceinline__ void stage_finish(const Prologue &pr, uint8_t *lds, i
     float inv = 1.0f / sqrtf(acc[0] / (float)cols + pr.eps);
     if (add) {
 #pragma unroll
-        for (int k = 0; k < kStageP; k++) {
+        for (int k = 0; k < KP; k++) {
             const int i = tid + k * NT;
             if (wbase + k * NT < n4) {
                 const float4 r = s.rs[k], w = s.wp[k];
@@ -320,7 +324,7 @@ __device__ __forceinline__ void stage_finish(const Prologue &pr, uint8_t *lds, i
         inv = 1.0f / sqrtf(ss2 / (float)cols + pr.eps);
     }
 #pragma unroll
-    for (int k = 0; k < kStageP; k++) {
+    for (int k = 0; k < KP; k++) {
         const int i = tid + k * NT;
         if (wbase + k * NT < n4) {
             const float4 w = s.wn[k];

@@ -164,10 +164,11 @@ __global__ __launch_bounds__(NW * 64) void q6k_gemv_kernel(Q6kParams p)
                 dst[s][r] = q6k_load(rp + (size_t)min(s * 8 + bl, p.bpr - 1) * kQ6kBytes, ip, il);
         }
     };
+    constexpr int KMAX = (STEPS * 512 + NW * 64 - 1) / (NW * 64);   // float4 of the vector per thread: cols <= STEPS * 2048
     StageRegs sr;
-    stage_fetch<NW * 64>(p.pro, cols, sr);
+    stage_fetch<NW * 64, false, KMAX>(p.pro, cols, sr);
     load_rows(cur, min(w0, p.rows - 1));   // unconditional (clamped): the staging wait can then leave these in flight
-    stage_finish<kXQ6, NW * 64>(p.pro, xs, cols, sr);
+    stage_finish<kXQ6, NW * 64, false, KMAX>(p.pro, xs, cols, sr);
     __syncthreads();
     if (w0 >= w1) return;
 
@@ -288,10 +289,11 @@ __global__ __launch_bounds__(NW * 64) void q6r_gemv_kernel(Q6kParams p)
             for (int s = 0; s < STEPS; s++) dst[s][r] = q6r_load(rp, p.bpr, s * 8 + bl, lane);   // bpr is a multiple of 8: every lane's superblock exists
         }
     };
+    constexpr int KMAX = (STEPS * 512 + NW * 64 - 1) / (NW * 64);   // float4 of the vector per thread: cols == STEPS * 2048
     StageRegs sr;
-    stage_fetch<NW * 64>(p.pro, cols, sr);
+    stage_fetch<NW * 64, false, KMAX>(p.pro, cols, sr);
     load_rows(cur, min(w0, p.rows - 1));
-    stage_finish<kXQ6, NW * 64>(p.pro, xs, cols, sr);
+    stage_finish<kXQ6, NW * 64, false, KMAX>(p.pro, xs, cols, sr);
     __syncthreads();
     if (w0 >= w1) return;
 

@@ -349,6 +349,10 @@ __global__ __launch_bounds__(NW * 64) void q4k_gemv_half_kernel(MatvecParams p_i
     Q4kLane L[NM][R];
     StageRegs sr;
     stage_fetch<NW * 64, MERGE>(p.pro, bpr * 256, sr);
+    // With a normalising prologue every wave's vector loads are queued before any wave's weight loads: behind
+    // another wave's HBM-cold weights in the compute unit's memory pipeline they came back up to 1.3 us late, and
+    // the prologue's reduction waits for the slowest wave.
+    if (p.pro.kind != kPlain) __syncthreads();
     auto load_r = [&](int r) {
         const size_t off = (size_t)min(row0 + r, t.rows - 1) * row_bytes + (size_t)bl * kQ4kBytes;
         L[0][r] = q4k_load(t.W0 + off, g);

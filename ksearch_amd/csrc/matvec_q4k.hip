@@ -587,6 +587,8 @@ int bind_matvec_q4k_family(ksh_kernel &k)
     if (s.cols > 32768) return set_error("Q4_K matvec: cols=%lld does not fit the LDS staging buffer", (long long)s.cols);
     const int bpr = (int)(s.cols / 256);
     Q4kGeom G = pick_geom(k.desc.sched, (int)(s.nm == 2 ? s.rows[0] : total_rows), bpr);
+    // QKV at one row per half-wave: one dot per lane does not pay for turning the vector into digit planes (3.86 vs 4.08 us)
+    if (sched_is_zero(k.desc.sched) && s.n_mat == 3 && G.half && G.R == 1) G.var = kXF32;
     if (s.prologue == kMergeParts) {
         if (s.hd < 4 || (s.hd & (s.hd - 1)) || s.nwg < 1 || s.nwg > kMergeMaxParts)
             return set_error("attn_merge_matvec: hd=%d must be a power of two, nwg=%d at most %d", s.hd, s.nwg, kMergeMaxParts);

@@ -885,7 +885,10 @@ int bind_sdpa_lanes(ksh_kernel &k, int nwg, int n_slots)
     // sched.unroll: workgroups per kv head, each with a share of its q heads (rows are then unpacked once per
     // share, but a decode step's latency is in the per-row work and the merge, both of which shrink with it)
     const int total_groups = n_q / n_kv;
-    int hsplit = k.desc.sched.unroll ? (int)k.desc.sched.unroll : (k.desc.kind == KSH_ATTEND_DECODE && total_groups >= 4 && total_groups % 2 == 0 ? total_groups / 2 : 1);
+    // (defaults from timing the decode shape: two heads per workgroup where the launch merges, one where it does not)
+    int hsplit = k.desc.sched.unroll ? (int)k.desc.sched.unroll
+                 : k.desc.kind != KSH_ATTEND_DECODE || total_groups < 4 ? 1
+                 : k.desc.dims[5] ? total_groups : (total_groups % 2 == 0 ? total_groups / 2 : 1);
     if (hsplit < 1 || hsplit > 255 || total_groups % hsplit) return set_error("sdpa: unsupported schedule unroll=%d (must divide %d)", hsplit, total_groups);
     const int wg_groups = total_groups / hsplit;
     const size_t lds = lanes_lds(hd, wg_groups, nw);

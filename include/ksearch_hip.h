@@ -95,8 +95,8 @@ enum ksh_kind {
      * whole table f32[max_seq, hd] and the outputs are the cache bases. */
     KSH_RMSNORM_PER_HEAD_QKV_Q40 = 12,
     /* CopyScaleIndexed: out[i] = scale * deq(src[id*n + i]); id is read from a
-     * device f32 (the reference keeps token ids as f32).  dims: n.
-     * dtypes[0] = source dtype.  params[0] = scale.  in: src, idx   out: out[n] */
+     * device f32 (the reference keeps token ids as f32).  dims: n, rows in the table.
+     * dtypes[0] = source dtype (Q4K | Q5K | Q6K | F16 | F32).  params[0] = scale.  in: src, idx   out: out[n] */
     KSH_COPY_SCALE_INDEXED = 13,
     /* GeluMul: out[i] = gelu_tanh(clamp(g[i])) * u[i].  dims: n.  in: g, u  out: out */
     KSH_GELU_MUL = 14,
@@ -107,7 +107,7 @@ enum ksh_kind {
     KSH_SOFTCAP_ARGMAX = 16,
     /* Dequantize packed blocks to f32 (the CPU-side dequant_type_to_f32,
      * crates/ksearch_gguf/src/gguf_impl.rs:472-476, as a device kernel).
-     * dims: n_elems.  dtypes[0] = Q4K | Q6K | Q40.  in: src   out: dst f32 */
+     * dims: n_elems.  dtypes[0] = Q4K | Q5K | Q6K | Q40.  in: src   out: dst f32 */
     KSH_DEQUANT = 17,
     /* quantize_f32_to_q4k (crates/ksearch_gguf/src/gguf_impl.rs:905-1016) and a
      * Q6_K packer, as device kernels.  dims: n_elems.  dtypes[0] = Q4K | Q6K.
@@ -153,6 +153,21 @@ enum ksh_kind {
     /* Q6_K [rows, cols] -> KSH_Q6K_ROWS, a byte permutation inside every row (done once, when weights are
      * loaded).  dims: rows, cols (a multiple of 2048).  in: src Q6_K   out: dst (same size, 16-byte aligned) */
     KSH_REPACK_ROWS = 24,
+    /* Eng::rmsnorm_per_head and rmsnorm_per_head_rope_off (crates/ksearch_kernels/src/lib.rs:564-625):
+     * y[h,i] = x[h,i] * rsqrt(mean_h(x^2) + eps) * w[i], then RoPE with pairs (i, i + hd/2) of the row
+     * cos[0..hd/2) || sin[0..hd/2).  The query heads of layers that reuse another layer's KV cache, and the
+     * per-layer-embedding prepass.  y may be x.
+     * dims: n_heads, hd (64 | 128 | 256 | 512), rope (0 none; 1 the row, placed with a byte offset; 2 the whole
+     *       table, row = position in meta[3]), max_seq (rope = 2)
+     * params: eps.   in: x, w f32[hd] [, rope [, meta f32[4]]]   out: y */
+    KSH_RMSNORM_PER_HEAD = 25,
+    /* Eng::add_scale (crates/ksearch_kernels/src/lib.rs:918-937): y = scale * (a + b).
+     * dims: n.  params: scale.  in: a, b   out: y */
+    KSH_ADD_SCALE = 26,
+    /* Eng::matvec_gelu_mul_at (crates/ksearch_kernels/src/lib.rs:791-822): y[r] = gelu(W[r].x) * ctx[r], the
+     * per-layer-embedding gate; the context slice is placed with a byte offset.
+     * dims: rows, cols.  dtypes: Q4K, F32.  in: W, x, ctx f32[rows]   out: y */
+    KSH_MATVEC_GELU_MUL = 27,
     KSH_KIND_COUNT
 };
 
@@ -297,6 +312,58 @@ ksh_buf *ksh_gemma_hidden(ksh_gemma *m);
 ksh_buf *ksh_gemma_kv(ksh_gemma *m, int layer, int which);
 int ksh_gemma_pos(ksh_gemma *m);
 int ksh_gemma_launches_per_token(ksh_gemma *m);
+
+/* ---- decode loop with the layer features of the real Gemma-4 checkpoints: GemmaPrimModel::forward_token
+ * (crates/ksearch_gemma/src/gemma_prim.rs:881-1275) under GemmaConfig's rules (crates/ksearch_gemma/src/lib.rs:
+ * 39-167).  A layer is a sliding-window layer (head dim hd_swa, rope base rope_theta_swa, attends the last
+ * sliding_window rows) or a full-attention layer (hd_full, rope_theta_full over the first hd_full*partial_rotary/2
+ * pairs, attends everything); the last shared_kv_layers layers append nothing and read the cache of the nearest
+ * earlier owning layer of their kind; with ple_dim > 0 every layer ends with the per-layer-embedding block.
+ * Weight tensors are Q4_K or Q6_K each (what the reference keeps on the device, gemma_prim.rs:414-450; other GGUF
+ * types are requantized by the loader).  The reference's attention is unscaled: attn_scale = 1. ---- */
+typedef struct {
+    int32_t n_layers, hidden, n_q, n_kv, vocab, max_seq;
+    int32_t hd_swa, hd_full, sliding_window, shared_kv_layers, ple_dim;   /* ple_dim 0: no per-layer embeddings */
+    float eps, softcap, rope_theta_swa, rope_theta_full, partial_rotary, attn_scale;
+} ksh_gemma4_cfg;
+
+typedef struct {
+    int32_t is_swa, ffn;
+    int32_t dt_q, dt_k, dt_v, dt_o, dt_gate, dt_up, dt_down, dt_inp_gate, dt_proj;   /* KSH_Q4K | KSH_Q6K */
+    ksh_buf *wq, *wk, *wv, *wo, *wgate, *wup, *wdown;   /* wk, wv unused by layers that reuse a cache */
+    ksh_buf *inp_gate, *proj;                           /* [ple_dim, hidden], [hidden, ple_dim] */
+    ksh_buf *attn_norm, *q_norm, *k_norm, *post_attn_norm, *ffn_norm, *post_ffw_norm, *post_norm;   /* f32 */
+    float layer_scale;                                  /* layer_output_scale (gemma_prim.rs:185) */
+} ksh_gemma4_layer;
+
+typedef struct {
+    ksh_buf *token_embd;       /* [vocab, hidden], also the LM head */
+    int32_t dt_embd;           /* KSH_Q4K | KSH_Q6K */
+    ksh_buf *output_norm;      /* f32[hidden] */
+    ksh_buf *ple_embd;         /* [vocab, n_layers*ple_dim] */
+    int32_t dt_ple;            /* KSH_Q4K | KSH_Q5K | KSH_Q6K | KSH_F16 | KSH_F32 */
+    ksh_buf *ple_model_proj;   /* [n_layers*ple_dim, hidden] */
+    int32_t dt_ple_proj;       /* KSH_Q4K | KSH_Q6K */
+    ksh_buf *ple_proj_norm;    /* f32[ple_dim] */
+} ksh_gemma4_globals;
+
+typedef struct ksh_gemma4 ksh_gemma4;
+
+int ksh_gemma4_create(ksh_ctx *ctx, const ksh_gemma4_cfg *cfg, const ksh_gemma4_layer *layers,
+                      const ksh_gemma4_globals *globals, ksh_gemma4 **out);
+void ksh_gemma4_destroy(ksh_gemma4 *m);
+int ksh_gemma4_reset(ksh_gemma4 *m);
+/* forward_token(token, want_logits): want_logits = 0 stops after the layers (prompt tokens but the last) */
+int ksh_gemma4_forward_token(ksh_gemma4 *m, uint32_t token, int want_logits, int use_graph, uint32_t *next_id);
+int ksh_gemma4_generate(ksh_gemma4 *m, const uint32_t *prompt, int n_prompt, int n_new,
+                        int use_graph, uint32_t *out_ids, double *prefill_ms, double *decode_ms);
+ksh_buf *ksh_gemma4_logits(ksh_gemma4 *m);
+ksh_buf *ksh_gemma4_hidden(ksh_gemma4 *m);
+/* kv_source(layer) (crates/ksearch_gemma/src/lib.rs:151-162) and that layer's cache */
+int ksh_gemma4_kv_source(ksh_gemma4 *m, int layer);
+ksh_buf *ksh_gemma4_kv(ksh_gemma4 *m, int layer, int which);
+int ksh_gemma4_pos(ksh_gemma4 *m);
+int ksh_gemma4_launches_per_token(ksh_gemma4 *m);
 
 #ifdef __cplusplus
 }

@@ -1,6 +1,6 @@
 // Packed block -> f32 dequantization on the device, bit-exact with the CPU
 // loops of crates/ksearch_gguf/src/gguf_impl.rs:618-633 (Q4_0), :690-721
-// (Q4_K) and :761-791 (Q6_K).  Built with -ffp-contract=off: the reference
+// (Q4_K), :722-760 (Q5_K) and :761-791 (Q6_K).  Built with -ffp-contract=off: the reference
 // rounds `d1*q` and `- mn1` separately.
 //
 // One thread per 16-byte-aligned unit of packed input is not possible for
@@ -48,6 +48,33 @@ __global__ void dequant_q4k_kernel(const uint8_t *__restrict__ src, float *__res
     o.z = d1 * (float)(hi ? (qs[2] >> 4) : (qs[2] & 0x0F)) - mn1;
     o.w = d1 * (float)(hi ? (qs[3] >> 4) : (qs[3] & 0x0F)) - mn1;
     reinterpret_cast<float4 *>(dst)[i] = o;
+}
+
+// Q5_K: the Q4_K layout with a fifth bit per weight (qh[l] bit 2g for the low nibbles of group g, bit 2g+1 for
+// the high ones): d1*(nibble + 16*bit) - mn1
+__global__ void dequant_q5k_kernel(const uint8_t *__restrict__ src, float *__restrict__ dst, size_t n4)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n4) return;
+    const size_t e = i * 4, b = e >> 8;
+    const int j = (int)(e & 255);
+    const uint8_t *blk = src + b * 176;
+    const float d = half_bits_to_f32(ld16(blk)), dmin = half_bits_to_f32(ld16(blk + 2));
+    const int sub = j >> 5;
+    uint32_t sc, mn;
+    scale_min_k4(sub, blk + 4, sc, mn);
+    const float d1 = d * (float)sc, mn1 = dmin * (float)mn;
+    const uint8_t *qh = blk + 16 + (j & 31);
+    const uint8_t *qs = blk + 48 + (j >> 6) * 32 + (j & 31);
+    const bool hi = (j & 32) != 0;
+    float o[4];
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        const float nib = (float)(hi ? (qs[t] >> 4) : (qs[t] & 0x0F));
+        const float bit = ((qh[t] >> sub) & 1) ? 16.0f : 0.0f;
+        o[t] = d1 * (nib + bit) - mn1;
+    }
+    reinterpret_cast<float4 *>(dst)[i] = make_float4(o[0], o[1], o[2], o[3]);
 }
 
 __global__ void dequant_q6k_kernel(const uint8_t *__restrict__ src, float *__restrict__ dst, size_t n4)
@@ -101,6 +128,7 @@ int launch_dequant(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
     float *dst = (float *)a.out[0];
     switch (k.desc.dtypes[0]) {
     case KSH_Q4K: hipLaunchKernelGGL(dequant_q4k_kernel, dim3(grid), dim3(256), 0, st, src, dst, n4); break;
+    case KSH_Q5K: hipLaunchKernelGGL(dequant_q5k_kernel, dim3(grid), dim3(256), 0, st, src, dst, n4); break;
     case KSH_Q6K: hipLaunchKernelGGL(dequant_q6k_kernel, dim3(grid), dim3(256), 0, st, src, dst, n4); break;
     case KSH_Q40: hipLaunchKernelGGL(dequant_q40_kernel, dim3(grid), dim3(256), 0, st, src, dst, n4); break;
     }
@@ -158,7 +186,7 @@ int bind_dequant(ksh_kernel &k)
 {
     const int dt = k.desc.dtypes[0];
     const int64_t n = k.desc.dims[0];
-    if (dt != KSH_Q4K && dt != KSH_Q6K && dt != KSH_Q40) return set_error("dequant: dtype %d is not built", dt);
+    if (dt != KSH_Q4K && dt != KSH_Q5K && dt != KSH_Q6K && dt != KSH_Q40) return set_error("dequant: dtype %d is not built", dt);
     const size_t pb = n > 0 ? packed_bytes(dt, (size_t)n) : 0;
     if (!pb || (uint64_t)n / 4 / 256 > 0x7FFFFFFFull) return set_error("dequant: n=%lld is not a valid element count", (long long)n);
     k.info.n_inputs = 1;
@@ -168,7 +196,7 @@ int bind_dequant(ksh_kernel &k)
     k.in_align[0] = 2;
     k.out_align[0] = 16;
     set_launch(k, (uint32_t)(((size_t)n / 4 + 255) / 256), 1, 1, 256, 0);
-    set_name(k, "dequant_%s", dt == KSH_Q4K ? "q4k" : dt == KSH_Q6K ? "q6k" : "q40");
+    set_name(k, "dequant_%s", dt == KSH_Q4K ? "q4k" : dt == KSH_Q5K ? "q5k" : dt == KSH_Q6K ? "q6k" : "q40");
     k.launch = launch_dequant;
     return 0;
 }

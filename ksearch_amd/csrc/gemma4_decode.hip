@@ -1,0 +1,579 @@
+// Greedy decode loop with the layer features of the real Gemma-4 checkpoints,
+// above the C ABI: sliding-window and full-attention layers with their own head
+// dims, rope tables and windows, layers that reuse an earlier layer's KV cache,
+// per-layer embeddings, Q4_K or Q6_K per weight tensor.
+//
+// Mirrors GemmaPrimModel::forward_token (crates/ksearch_gemma/src/gemma_prim.rs:
+// 881-1275) with GemmaConfig's layer rules (crates/ksearch_gemma/src/lib.rs:
+// 136-167).  As in the loop for the synthetic shape, norms ride in the GEMV that
+// consumes them wherever a fused kind is built for the weight types at hand, the
+// position lives on the device and a token is one HIP graph.  The layer-closing
+// residual add stays "pending" (y, norm weight) until its consumer folds it in;
+// where no fused consumer exists (per-layer embeddings scale the stream) it is
+// materialised with the RmsNorm kind.
+#include <chrono>
+#include <cmath>
+#include <cstdlib>
+#include <algorithm>
+#include <memory>
+#include <vector>
+
+#include "ksh_device.hpp"
+#include "ksh_internal.hpp"
+
+namespace {
+
+// end of token: remember the id, advance the position and both attended ranges
+// (full attention: rows [0, pos]; sliding window: the last `window` of them,
+// gemma_prim.rs:1010-1017), and put the next position's rows of the two rope
+// tables where the attention launches read them
+__global__ void advance4_kernel(float *meta_full, float *meta_swa, const float *tok, float *history, int max_hist,
+                                const float *rope_full, float *cur_full, int hd_full, const float *rope_swa,
+                                float *cur_swa, int hd_swa, int window)
+{
+    const int pos = (int)meta_full[3];
+    __syncthreads();   // every thread has read the position before thread 0 moves it
+    if (pos + 1 < max_hist) {
+        for (int i = threadIdx.x; i < hd_full; i += blockDim.x) cur_full[i] = rope_full[(size_t)(pos + 1) * hd_full + i];
+        for (int i = threadIdx.x; i < hd_swa; i += blockDim.x) cur_swa[i] = rope_swa[(size_t)(pos + 1) * hd_swa + i];
+    }
+    if (threadIdx.x == 0) {
+        if (history && pos < max_hist) history[pos] = tok[0];
+        const int kv_len = pos + 2;   // the next token attends up to and including its own row
+        const int start = kv_len > window ? kv_len - window : 0;
+        meta_full[3] = meta_swa[3] = (float)(pos + 1);
+        meta_full[0] = (float)kv_len;
+        meta_swa[0] = (float)(kv_len - start);
+        meta_swa[1] = (float)start;
+    }
+}
+
+__global__ void set_token4_kernel(float *tok, float value)
+{
+    if (threadIdx.x == 0 && blockIdx.x == 0) tok[0] = value;
+}
+
+struct Bufs {
+    std::vector<ksh_buf *> owned;
+    ~Bufs()
+    {
+        for (ksh_buf *b : owned) ksh_buffer_release(b);
+    }
+};
+
+// the kernels of one layer, bound when the model is built
+struct LayerPlan {
+    int hd = 0, qd = 0, kvd = 0, src = 0;
+    bool swa = false, owns = false;
+    bool fused_qkv = false, fused_gate_up = false, attend = false, attend_parts = false;
+    ksh_kernel *qkv[2] = {nullptr, nullptr};       // [pending add folded in?]; fused QKV, or q alone
+    ksh_kernel *kmat[2] = {nullptr, nullptr};      // k and v one by one (mixed weight types), on the materialised stream
+    ksh_kernel *head = nullptr, *sdpa = nullptr, *k_attend = nullptr;
+    ksh_kernel *oproj = nullptr;
+    ksh_kernel *gate_up = nullptr, *gate = nullptr, *up = nullptr, *gelu = nullptr;
+    ksh_kernel *down = nullptr;
+    ksh_kernel *ple_gate = nullptr, *ple_proj = nullptr, *ple_close = nullptr;
+};
+
+}  // namespace
+
+struct ksh_gemma4 {
+    ksh_ctx *ctx = nullptr;
+    ksh_gemma4_cfg c{};
+    ksh_gemma4_globals g{};
+    std::vector<ksh_gemma4_layer> layers;
+    std::vector<LayerPlan> plan;
+    Bufs bufs;
+    ksh_buf *embd_rows = nullptr;
+    ksh_buf *x = nullptr, *xb = nullptr, *y = nullptr, *hidden = nullptr, *tq = nullptr, *tk = nullptr, *tv = nullptr, *to = nullptr,
+            *ff = nullptr, *ff2 = nullptr, *logits = nullptr, *tok = nullptr, *meta_full = nullptr, *meta_swa = nullptr,
+            *rope_full = nullptr, *rope_swa = nullptr, *cur_full = nullptr, *cur_swa = nullptr, *attn_tmp = nullptr,
+            *history = nullptr, *ple_tok = nullptr, *ple_tmp = nullptr, *ple_ctx = nullptr, *ple_u = nullptr;
+    std::vector<ksh_buf *> kv_k, kv_v;   // per layer; null where the layer reads another layer's cache
+    ksh_kernel *k_embed = nullptr, *k_ple_gather = nullptr, *k_ple_proj = nullptr, *k_ple_norm = nullptr, *k_ple_mix = nullptr,
+               *k_close = nullptr, *k_lm_head[2] = {nullptr, nullptr}, *k_argmax = nullptr;
+    ksh_graph *g_body = nullptr, *g_full = nullptr;
+    std::vector<float> rope0_full, rope0_swa;
+    int pos = 0, launches_full = 0;
+};
+
+namespace {
+
+using namespace ksh;
+
+constexpr int kAttendPartitions = 16;
+constexpr int kShortPartitions = 8;     // sliding-window layers: the o-projection merges the partitions
+constexpr int kShortWindow = 640;
+
+int alloc(ksh_gemma4 *m, size_t bytes, ksh_buf **out)
+{
+    if (ksh_buffer_alloc(m->ctx, bytes ? bytes : 16, nullptr, out)) return 1;
+    m->bufs.owned.push_back(*out);
+    return 0;
+}
+
+int get(ksh_gemma4 *m, int kind, std::initializer_list<int64_t> dims, std::initializer_list<int> dtypes,
+        std::initializer_list<float> params, ksh_kernel **out)
+{
+    ksh_kernel_desc d;
+    memset(&d, 0, sizeof(d));
+    d.kind = kind;
+    int i = 0;
+    for (int64_t v : dims) d.dims[i++] = v;
+    i = 0;
+    for (int v : dtypes) d.dtypes[i++] = v;
+    i = 0;
+    for (float v : params) d.params[i++] = v;
+    return ksh_kernel_get(m->ctx, &d, out);
+}
+
+int enc(ksh_gemma4 *m, ksh_kernel *k, std::initializer_list<ksh_buf *> in, std::initializer_list<ksh_buf *> out, int &count)
+{
+    ksh_buf *ib[kMaxIn], *ob[kMaxOut];
+    int ni = 0, no = 0;
+    for (ksh_buf *b : in) ib[ni++] = b;
+    for (ksh_buf *b : out) ob[no++] = b;
+    count += 1;
+    return ksh_encode(m->ctx, k, ib, nullptr, ni, ob, nullptr, no);
+}
+
+int enc_off(ksh_gemma4 *m, ksh_kernel *k, std::initializer_list<ksh_buf *> in, std::initializer_list<size_t> in_off,
+            std::initializer_list<ksh_buf *> out, int &count)
+{
+    ksh_buf *ib[kMaxIn], *ob[kMaxOut];
+    size_t io[kMaxIn];
+    int ni = 0, no = 0, nf = 0;
+    for (ksh_buf *b : in) ib[ni++] = b;
+    for (size_t o : in_off) io[nf++] = o;
+    for (ksh_buf *b : out) ob[no++] = b;
+    count += 1;
+    return ksh_encode(m->ctx, k, ib, io, ni, ob, nullptr, no);
+}
+
+bool packed_ok(int dt) { return dt == KSH_Q4K || dt == KSH_Q6K; }
+
+// the residual stream while a token is encoded: `cur` holds x; if `y` is set, the
+// stream is really cur + rms(y)*w and the add has not been written anywhere yet
+struct Stream {
+    ksh_buf *cur, *other;
+    ksh_buf *y = nullptr, *w = nullptr;
+};
+
+// norm(x)*w_norm -> GEMV, folding a pending add in (the fused kinds write the new stream themselves)
+int enc_norm_gemv(ksh_gemma4 *m, ksh_kernel *const k[2], std::initializer_list<ksh_buf *> weights, ksh_buf *w_norm, Stream &s,
+                  std::initializer_list<ksh_buf *> outs, int &n)
+{
+    ksh_buf *ib[kMaxIn], *ob[kMaxOut];
+    int ni = 0, no = 0;
+    for (ksh_buf *b : weights) ib[ni++] = b;
+    for (ksh_buf *b : outs) ob[no++] = b;
+    if (s.y) {
+        ib[ni++] = s.y; ib[ni++] = w_norm; ib[ni++] = s.w; ib[ni++] = s.cur;
+        ob[no++] = s.other;
+        n += 1;
+        if (ksh_encode(m->ctx, k[1], ib, nullptr, ni, ob, nullptr, no)) return 1;
+        std::swap(s.cur, s.other);
+        s.y = s.w = nullptr;
+        return 0;
+    }
+    ib[ni++] = s.cur; ib[ni++] = w_norm;
+    n += 1;
+    return ksh_encode(m->ctx, k[0], ib, nullptr, ni, ob, nullptr, no);
+}
+
+// writes a pending add out: cur <- (cur + rms(y)*w) [* scale]
+int materialise(ksh_gemma4 *m, Stream &s, ksh_kernel *k, int &n)
+{
+    if (!s.y) return 0;
+    if (enc(m, k, {s.y, s.w, s.cur}, {s.other}, n)) return 1;
+    std::swap(s.cur, s.other);
+    s.y = s.w = nullptr;
+    return 0;
+}
+
+int encode_token(ksh_gemma4 *m, bool want_logits, int &launches)
+{
+    const ksh_gemma4_cfg &c = m->c;
+    launches = 0;
+    Stream s{m->x, m->xb};
+    if (enc(m, m->k_embed, {m->g.token_embd, m->tok}, {s.cur}, launches)) return 1;
+    if (c.ple_dim > 0) {
+        // ple_from_idx + ple_prepass (gemma_prim.rs:712-728, 845-878)
+        if (enc(m, m->k_ple_gather, {m->g.ple_embd, m->tok}, {m->ple_tok}, launches) ||
+            enc(m, m->k_ple_proj, {m->g.ple_model_proj, s.cur}, {m->ple_tmp}, launches) ||
+            enc(m, m->k_ple_norm, {m->ple_tmp, m->g.ple_proj_norm}, {m->ple_ctx}, launches) ||
+            enc(m, m->k_ple_mix, {m->ple_ctx, m->ple_tok}, {m->ple_ctx}, launches))
+            return 1;
+    }
+    for (int l = 0; l < c.n_layers; l++) {
+        const ksh_gemma4_layer &L = m->layers[l];
+        const LayerPlan &P = m->plan[l];
+        ksh_buf *meta = P.swa ? m->meta_swa : m->meta_full;
+        ksh_buf *rope_cur = P.swa ? m->cur_swa : m->cur_full, *rope_tab = P.swa ? m->rope_swa : m->rope_full;
+        ksh_buf *kc = m->kv_k[P.src], *vc = m->kv_v[P.src];
+        // -- q, k, v of the normalised stream
+        if (P.owns && P.fused_qkv) {
+            if (enc_norm_gemv(m, P.qkv, {L.wq, L.wk, L.wv}, L.attn_norm, s, {m->tq, m->tk, m->tv}, launches)) return 1;
+        } else {
+            if (enc_norm_gemv(m, P.qkv, {L.wq}, L.attn_norm, s, {m->tq}, launches)) return 1;
+            if (P.owns &&
+                (enc(m, P.kmat[0], {L.wk, s.cur, L.attn_norm}, {m->tk}, launches) ||
+                 enc(m, P.kmat[1], {L.wv, s.cur, L.attn_norm}, {m->tv}, launches)))
+                return 1;
+        }
+        // -- per-head norm, RoPE, cache append, attention
+        bool parts = false;
+        if (P.attend) {
+            parts = P.attend_parts;
+            if (parts ? enc(m, P.k_attend, {m->tq, L.q_norm, rope_cur, m->tk, L.k_norm, m->tv, meta}, {kc, vc, m->attn_tmp}, launches)
+                      : enc(m, P.k_attend, {m->tq, L.q_norm, rope_cur, m->tk, L.k_norm, m->tv, meta}, {kc, vc, m->attn_tmp, m->to}, launches))
+                return 1;
+        } else {
+            if (P.owns ? enc(m, P.head, {m->tq, L.q_norm, rope_tab, m->tk, L.k_norm, m->tv, meta}, {m->tq, kc, vc}, launches)
+                       : enc(m, P.head, {m->tq, L.q_norm, rope_tab, meta}, {m->tq}, launches))   // gemma_prim.rs:989-1008
+                return 1;
+            if (enc(m, P.sdpa, {m->tq, kc, vc, meta}, {m->attn_tmp, m->to}, launches)) return 1;
+        }
+        if (enc(m, P.oproj, {L.wo, parts ? m->attn_tmp : m->to}, {m->y}, launches)) return 1;
+        // -- feed-forward on norm(x + rms(o)*post_attn_norm)
+        s.y = m->y;
+        s.w = L.post_attn_norm;
+        if (P.fused_gate_up) {
+            ksh_kernel *const k2[2] = {nullptr, P.gate_up};
+            if (enc_norm_gemv(m, k2, {L.wgate, L.wup}, L.ffn_norm, s, {m->ff}, launches)) return 1;
+        } else {
+            ksh_kernel *const k2[2] = {nullptr, P.gate};
+            if (enc_norm_gemv(m, k2, {L.wgate}, L.ffn_norm, s, {m->ff}, launches) ||
+                enc(m, P.up, {L.wup, s.cur, L.ffn_norm}, {m->ff2}, launches) ||
+                enc(m, P.gelu, {m->ff, m->ff2}, {m->ff}, launches))
+                return 1;
+        }
+        if (enc(m, P.down, {L.wdown, m->ff}, {m->y}, launches)) return 1;
+        s.y = m->y;
+        s.w = L.post_ffw_norm;
+        if (c.ple_dim > 0) {
+            // gemma_prim.rs:1166-1200: x += rms(down)*post_ffw_norm; u = gelu(Wg x) * ctx_l; x = (x + rms(Wp u)*post_norm) * scale
+            if (materialise(m, s, m->k_close, launches)) return 1;
+            if (enc_off(m, P.ple_gate, {L.inp_gate, s.cur, m->ple_ctx}, {0, 0, (size_t)l * c.ple_dim * 4}, {m->ple_u}, launches) ||
+                enc(m, P.ple_proj, {L.proj, m->ple_u}, {m->y}, launches) ||
+                enc(m, P.ple_close, {m->y, L.post_norm, s.cur}, {s.other}, launches))
+                return 1;
+            std::swap(s.cur, s.other);
+        }
+    }
+    if (want_logits) {
+        if (enc_norm_gemv(m, m->k_lm_head, {m->embd_rows ? m->embd_rows : m->g.token_embd}, m->g.output_norm, s, {m->logits}, launches))
+            return 1;
+        if (enc(m, m->k_argmax, {m->logits}, {m->tok}, launches)) return 1;
+        launches += 1;   // two passes
+    }
+    m->hidden = s.cur;   // (a pending add of the last layer of a logits-free token is never needed)
+    hipStream_t st = (hipStream_t)ksh_stream(m->ctx);
+    hipLaunchKernelGGL(advance4_kernel, dim3(1), dim3(64), 0, st, (float *)ksh_buffer_device_ptr(m->meta_full),
+                       (float *)ksh_buffer_device_ptr(m->meta_swa), (const float *)ksh_buffer_device_ptr(m->tok),
+                       want_logits ? (float *)ksh_buffer_device_ptr(m->history) : nullptr, c.max_seq,
+                       (const float *)ksh_buffer_device_ptr(m->rope_full), (float *)ksh_buffer_device_ptr(m->cur_full), c.hd_full,
+                       (const float *)ksh_buffer_device_ptr(m->rope_swa), (float *)ksh_buffer_device_ptr(m->cur_swa), c.hd_swa,
+                       c.sliding_window);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return hip_fail(e, "advance launch");
+    launches += 1;
+    return 0;
+}
+
+int run_token(ksh_gemma4 *m, bool want_logits, bool use_graph)
+{
+    if (m->pos >= m->c.max_seq) return set_error("max_seq exceeded");   // gemma_prim.rs:882-884
+    int n = 0;
+    if (!use_graph) {
+        if (encode_token(m, want_logits, n)) return 1;
+    } else {
+        ksh_graph *&g = want_logits ? m->g_full : m->g_body;
+        if (!g) {
+            if (ksh_synchronize(m->ctx)) return 1;
+            if (ksh_graph_begin(m->ctx)) return 1;
+            if (encode_token(m, want_logits, n)) {
+                ksh_graph *dead = nullptr;
+                ksh_graph_end(m->ctx, &dead);
+                ksh_graph_destroy(dead);
+                return 1;
+            }
+            if (ksh_graph_end(m->ctx, &g)) return 1;
+            if (want_logits) m->launches_full = n;
+        }
+        if (ksh_graph_launch(m->ctx, g)) return 1;
+    }
+    if (want_logits && !use_graph) m->launches_full = n;
+    m->pos += 1;
+    return 0;
+}
+
+int write_token(ksh_gemma4 *m, uint32_t token)
+{
+    hipLaunchKernelGGL(set_token4_kernel, dim3(1), dim3(64), 0, (hipStream_t)ksh_stream(m->ctx),
+                       (float *)ksh_buffer_device_ptr(m->tok), (float)token);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : hip_fail(e, "set_token launch");
+}
+
+// gemma_prim.rs:33-56: per position cos[0..hd/2) || sin[0..hd/2); pairs past `angles` are the identity
+int make_rope(ksh_gemma4 *m, int hd, float theta, int angles, ksh_buf **table, ksh_buf **cur, std::vector<float> &row0)
+{
+    const int half = hd / 2, max_seq = m->c.max_seq;
+    angles = std::min(angles, half);
+    std::vector<float> tab((size_t)max_seq * hd);
+    for (int pos = 0; pos < max_seq; pos++)
+        for (int i = 0; i < half; i++) {
+            float cs = 1.0f, sn = 0.0f;
+            if (i < angles) {
+                const float freq = (float)(1.0 / std::pow((double)theta, (double)(2 * i) / (double)hd));
+                const float ang = (float)pos * freq;
+                cs = std::cos(ang);
+                sn = std::sin(ang);
+            }
+            tab[(size_t)pos * hd + i] = cs;
+            tab[(size_t)pos * hd + half + i] = sn;
+        }
+    if (ksh_buffer_alloc(m->ctx, tab.size() * 4, tab.data(), table)) return 1;
+    m->bufs.owned.push_back(*table);
+    row0.assign(tab.begin(), tab.begin() + hd);
+    return alloc(m, (size_t)hd * 4, cur);
+}
+
+int plan_layer(ksh_gemma4 *m, int l)
+{
+    const ksh_gemma4_cfg &c = m->c;
+    const ksh_gemma4_layer &L = m->layers[l];
+    LayerPlan &P = m->plan[l];
+    const int64_t h = c.hidden;
+    P.swa = L.is_swa != 0;
+    P.hd = P.swa ? c.hd_swa : c.hd_full;
+    P.qd = c.n_q * P.hd;
+    P.kvd = c.n_kv * P.hd;
+    P.owns = l < c.n_layers - c.shared_kv_layers;
+    P.src = l;
+    if (!P.owns) {
+        // kv_source, crates/ksearch_gemma/src/lib.rs:151-162
+        P.src = 0;
+        for (int i = l - 1; i >= 0; i--)
+            if (i < c.n_layers - c.shared_kv_layers && (m->layers[i].is_swa != 0) == P.swa) { P.src = i; break; }
+        if ((m->layers[P.src].is_swa != 0) != P.swa)
+            return set_error("layer %d reuses the cache of layer %d, which has another head dim", l, P.src);
+    }
+    const int dts[] = {L.dt_q, L.dt_o, L.dt_gate, L.dt_up, L.dt_down};
+    for (int dt : dts)
+        if (!packed_ok(dt)) return set_error("layer %d: weight dtype %d is not built (Q4_K and Q6_K are)", l, dt);
+    if (P.owns && (!packed_ok(L.dt_k) || !packed_ok(L.dt_v))) return set_error("layer %d: k/v weight dtype is not built", l);
+    if (L.ffn <= 0 || L.ffn % 256) return set_error("layer %d: ffn=%d is not a positive multiple of 256", l, L.ffn);
+
+    P.fused_qkv = P.owns && L.dt_q == KSH_Q4K && L.dt_k == KSH_Q4K && L.dt_v == KSH_Q4K;
+    if (P.fused_qkv) {
+        for (int r = 0; r < 2; r++)
+            if (get(m, KSH_RMSNORM_MATVEC_QKV, {P.qd, P.kvd, h, r}, {KSH_Q4K, KSH_F32}, {c.eps}, &P.qkv[r])) return 1;
+    } else {
+        for (int r = 0; r < 2; r++)
+            if (get(m, KSH_RMSNORM_MATVEC, {P.qd, h, r}, {L.dt_q, KSH_F32}, {c.eps}, &P.qkv[r])) return 1;
+        if (P.owns && (get(m, KSH_RMSNORM_MATVEC, {P.kvd, h, 0}, {L.dt_k, KSH_F32}, {c.eps}, &P.kmat[0]) ||
+                       get(m, KSH_RMSNORM_MATVEC, {P.kvd, h, 0}, {L.dt_v, KSH_F32}, {c.eps}, &P.kmat[1])))
+            return 1;
+    }
+    // attention: one launch where the fused kind is built for the shape and the layer appends to its own cache
+    const bool short_form = P.swa && c.sliding_window <= kShortWindow && L.dt_o == KSH_Q4K && P.qd <= 2048 && (P.hd & (P.hd - 1)) == 0;
+    P.attend = P.owns && sdpa_lanes_supports(c.n_q, c.n_kv, P.hd);
+    P.attend_parts = P.attend && short_form;
+    if (P.attend) {
+        if (get(m, KSH_ATTEND_DECODE, {c.n_q, c.n_kv, P.hd, c.max_seq, P.attend_parts ? kShortPartitions : kAttendPartitions, P.attend_parts ? 1 : 0, 1},
+                {KSH_Q40, KSH_F32}, {c.eps, c.attn_scale}, &P.k_attend))
+            return 1;
+    } else {
+        if (P.owns ? get(m, KSH_RMSNORM_PER_HEAD_QKV_Q40, {c.n_q, c.n_kv, P.hd, c.max_seq}, {}, {c.eps}, &P.head)
+                   : get(m, KSH_RMSNORM_PER_HEAD, {c.n_q, P.hd, 2, c.max_seq}, {}, {c.eps}, &P.head))
+            return 1;
+        if (get(m, KSH_SDPA_SLOTS, {c.n_q, c.n_kv, P.hd, c.max_seq, 1, kAttendPartitions}, {KSH_Q40, KSH_F32}, {c.attn_scale}, &P.sdpa)) return 1;
+    }
+    if (P.attend_parts ? get(m, KSH_ATTN_MERGE_MATVEC, {h, c.n_q, P.hd, kShortPartitions}, {KSH_Q4K, KSH_F32}, {}, &P.oproj)
+                       : get(m, KSH_MATVEC, {h, P.qd}, {L.dt_o, KSH_F32}, {}, &P.oproj))
+        return 1;
+    P.fused_gate_up = L.dt_gate == KSH_Q4K && L.dt_up == KSH_Q4K;
+    if (P.fused_gate_up) {
+        if (get(m, KSH_RMSNORM_MATVEC_GATE_UP_GELU, {L.ffn, h, 1}, {KSH_Q4K, KSH_F32}, {c.eps}, &P.gate_up)) return 1;
+    } else {
+        if (get(m, KSH_RMSNORM_MATVEC, {L.ffn, h, 1}, {L.dt_gate, KSH_F32}, {c.eps}, &P.gate) ||
+            get(m, KSH_RMSNORM_MATVEC, {L.ffn, h, 0}, {L.dt_up, KSH_F32}, {c.eps}, &P.up) ||
+            get(m, KSH_GELU_MUL, {L.ffn}, {}, {}, &P.gelu))
+            return 1;
+    }
+    if (get(m, KSH_MATVEC, {h, L.ffn}, {L.dt_down, KSH_F32}, {}, &P.down)) return 1;
+    if (c.ple_dim > 0) {
+        if (L.dt_inp_gate != KSH_Q4K || !packed_ok(L.dt_proj))
+            return set_error("layer %d: per-layer-embedding weights must be Q4_K (gate) and Q4_K or Q6_K (projection)", l);
+        if (get(m, KSH_MATVEC_GELU_MUL, {c.ple_dim, h}, {KSH_Q4K, KSH_F32}, {}, &P.ple_gate) ||
+            get(m, KSH_MATVEC, {h, c.ple_dim}, {L.dt_proj, KSH_F32}, {}, &P.ple_proj) ||
+            get(m, KSH_RMSNORM, {h, 1, 1}, {}, {c.eps, L.layer_scale}, &P.ple_close))
+            return 1;
+    }
+    return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int ksh_gemma4_create(ksh_ctx *ctx, const ksh_gemma4_cfg *cfg, const ksh_gemma4_layer *layers, const ksh_gemma4_globals *globals,
+                      ksh_gemma4 **out)
+{
+    if (!ctx || !cfg || !layers || !globals || !out || !globals->token_embd || !globals->output_norm)
+        return set_error("ksh_gemma4_create: bad arguments");
+    *out = nullptr;
+    const ksh_gemma4_cfg &c = *cfg;
+    if (c.n_layers <= 0 || c.hidden <= 0 || c.hidden % 256 || c.n_q <= 0 || c.n_kv <= 0 || c.n_q % c.n_kv || c.hd_swa <= 0 ||
+        c.hd_full <= 0 || c.vocab <= 0 || c.vocab >= (1 << 24) || c.max_seq <= 0 || c.sliding_window <= 0 ||
+        c.shared_kv_layers < 0 || c.shared_kv_layers >= c.n_layers || c.ple_dim < 0 || c.ple_dim % 256)
+        return set_error("ksh_gemma4_create: invalid configuration");
+    if (c.ple_dim > 0 && (!globals->ple_embd || !globals->ple_model_proj || !globals->ple_proj_norm))
+        return set_error("ksh_gemma4_create: per-layer embeddings need their table, projection and norm");
+    auto mp = std::make_unique<ksh_gemma4>();
+    ksh_gemma4 *m = mp.get();
+    m->ctx = ctx;
+    m->c = c;
+    m->g = *globals;
+    m->layers.assign(layers, layers + c.n_layers);
+    m->plan.resize(c.n_layers);
+    const int max_hd = std::max(c.hd_swa, c.hd_full);
+    int max_ff = 0;
+    for (const ksh_gemma4_layer &L : m->layers) max_ff = std::max(max_ff, (int)L.ffn);
+    const size_t h4 = (size_t)c.hidden * 4, pt = (size_t)c.n_layers * c.ple_dim;
+    if (alloc(m, h4, &m->x) || alloc(m, h4, &m->xb) || alloc(m, h4, &m->y) || alloc(m, (size_t)c.n_q * max_hd * 4, &m->tq) ||
+        alloc(m, (size_t)c.n_kv * max_hd * 4, &m->tk) || alloc(m, (size_t)c.n_kv * max_hd * 4, &m->tv) ||
+        alloc(m, (size_t)c.n_q * max_hd * 4, &m->to) || alloc(m, (size_t)max_ff * 4, &m->ff) || alloc(m, (size_t)max_ff * 4, &m->ff2) ||
+        alloc(m, (size_t)c.vocab * 4, &m->logits) || alloc(m, 16, &m->tok) || alloc(m, 16, &m->meta_full) || alloc(m, 16, &m->meta_swa) ||
+        alloc(m, (size_t)c.max_seq * 4, &m->history) || alloc(m, pt * 4, &m->ple_tok) || alloc(m, pt * 4, &m->ple_tmp) ||
+        alloc(m, pt * 4, &m->ple_ctx) || alloc(m, (size_t)c.ple_dim * 4, &m->ple_u) ||
+        alloc(m, (size_t)c.n_q * kAttendPartitions * (max_hd + 2) * 4, &m->attn_tmp))
+        return 1;
+    if (make_rope(m, c.hd_swa, c.rope_theta_swa, c.hd_swa / 2, &m->rope_swa, &m->cur_swa, m->rope0_swa) ||
+        make_rope(m, c.hd_full, c.rope_theta_full, (int)((float)c.hd_full * c.partial_rotary) / 2, &m->rope_full, &m->cur_full,
+                  m->rope0_full))
+        return 1;
+    m->kv_k.assign(c.n_layers, nullptr);
+    m->kv_v.assign(c.n_layers, nullptr);
+    for (int l = 0; l < c.n_layers; l++) {
+        if (plan_layer(m, l)) return 1;
+        if (!m->plan[l].owns) continue;
+        const size_t kvb = (size_t)c.max_seq * c.n_kv * (m->plan[l].hd / 32) * 18;   // gemma_prim.rs:199-207
+        if (alloc(m, kvb, &m->kv_k[l]) || alloc(m, kvb, &m->kv_v[l])) return 1;
+    }
+    const int de = globals->dt_embd;
+    if (!packed_ok(de)) return set_error("ksh_gemma4_create: embedding dtype %d is not built (Q4_K and Q6_K are)", de);
+    int lm_dt = de;
+    if (de == KSH_Q6K && (c.hidden == 2048 || c.hidden == 4096)) {
+        // the LM head streams the whole table every token: it gets a copy with each row's fields grouped
+        ksh_kernel *rp = nullptr;
+        if (alloc(m, (size_t)c.vocab * (c.hidden / 256) * 210, &m->embd_rows) ||
+            get(m, KSH_REPACK_ROWS, {c.vocab, c.hidden}, {KSH_Q6K, KSH_Q6K_ROWS}, {}, &rp))
+            return 1;
+        int n = 0;
+        if (enc(m, rp, {m->g.token_embd}, {m->embd_rows}, n) || ksh_synchronize(ctx)) return 1;
+        lm_dt = KSH_Q6K_ROWS;
+    }
+    if (get(m, KSH_COPY_SCALE_INDEXED, {c.hidden, c.vocab}, {de}, {std::sqrt((float)c.hidden)}, &m->k_embed) ||
+        get(m, KSH_RMSNORM, {c.hidden, 1, 0}, {}, {c.eps, 0.f}, &m->k_close) ||
+        get(m, KSH_RMSNORM_MATVEC, {c.vocab, c.hidden, 0}, {lm_dt, KSH_F32}, {c.eps}, &m->k_lm_head[0]) ||
+        get(m, KSH_RMSNORM_MATVEC, {c.vocab, c.hidden, 1}, {lm_dt, KSH_F32}, {c.eps}, &m->k_lm_head[1]) ||
+        get(m, KSH_SOFTCAP_ARGMAX, {c.vocab}, {}, {c.softcap}, &m->k_argmax))
+        return 1;
+    if (c.ple_dim > 0) {
+        if (!packed_ok(globals->dt_ple_proj)) return set_error("ksh_gemma4_create: per-layer projection dtype %d is not built", globals->dt_ple_proj);
+        if (get(m, KSH_COPY_SCALE_INDEXED, {(int64_t)pt, c.vocab}, {globals->dt_ple}, {std::sqrt((float)c.ple_dim)}, &m->k_ple_gather) ||
+            get(m, KSH_MATVEC, {(int64_t)pt, c.hidden}, {globals->dt_ple_proj, KSH_F32}, {}, &m->k_ple_proj) ||
+            get(m, KSH_RMSNORM_PER_HEAD, {c.n_layers, c.ple_dim, 0}, {}, {c.eps}, &m->k_ple_norm) ||
+            get(m, KSH_ADD_SCALE, {(int64_t)pt}, {}, {0.70710678118654752440f}, &m->k_ple_mix))
+            return 1;
+    }
+    if (ksh_gemma4_reset(m)) return 1;
+    *out = mp.release();
+    return 0;
+}
+
+void ksh_gemma4_destroy(ksh_gemma4 *m)
+{
+    if (!m) return;
+    ksh_synchronize(m->ctx);
+    ksh_graph_destroy(m->g_body);
+    ksh_graph_destroy(m->g_full);
+    delete m;
+}
+
+int ksh_gemma4_reset(ksh_gemma4 *m)
+{
+    if (!m) return set_error("ksh_gemma4_reset: null model");
+    if (ksh_synchronize(m->ctx)) return 1;
+    const float full[4] = {1.f, 0.f, 0.f, 0.f};                              // tlen, start, window, pos
+    const float swa[4] = {1.f, 0.f, (float)m->c.sliding_window, 0.f};
+    if (ksh_buffer_write(m->ctx, m->meta_full, 0, full, 16, 1) || ksh_buffer_write(m->ctx, m->meta_swa, 0, swa, 16, 1) ||
+        ksh_buffer_write(m->ctx, m->cur_full, 0, m->rope0_full.data(), m->rope0_full.size() * 4, 1) ||
+        ksh_buffer_write(m->ctx, m->cur_swa, 0, m->rope0_swa.data(), m->rope0_swa.size() * 4, 1))
+        return 1;
+    m->pos = 0;
+    return 0;
+}
+
+int ksh_gemma4_forward_token(ksh_gemma4 *m, uint32_t token, int want_logits, int use_graph, uint32_t *next_id)
+{
+    if (!m) return set_error("ksh_gemma4_forward_token: null model");
+    if (token >= (uint32_t)m->c.vocab) return set_error("token id %u is outside the vocabulary", token);
+    if (write_token(m, token)) return 1;
+    if (run_token(m, want_logits != 0, use_graph != 0)) return 1;
+    if (next_id && want_logits) {
+        float f = 0.f;
+        if (ksh_buffer_read(m->ctx, m->tok, 0, &f, 4, 1)) return 1;
+        *next_id = (uint32_t)f;
+    }
+    return 0;
+}
+
+int ksh_gemma4_generate(ksh_gemma4 *m, const uint32_t *prompt, int n_prompt, int n_new, int use_graph, uint32_t *out_ids,
+                        double *prefill_ms, double *decode_ms)
+{
+    if (!m || !prompt || n_prompt < 1 || n_new < 0 || (n_new && !out_ids)) return set_error("ksh_gemma4_generate: bad arguments");
+    if (m->pos + n_prompt - 1 + n_new > m->c.max_seq) return set_error("max_seq exceeded");
+    for (int i = 0; i < n_prompt; i++)
+        if (prompt[i] >= (uint32_t)m->c.vocab) return set_error("token id %u is outside the vocabulary", prompt[i]);
+    using clk = std::chrono::steady_clock;
+    const auto t0 = clk::now();
+    // all prompt tokens but the last go through without logits (gemma_prim.rs:1670-1675)
+    for (int i = 0; i + 1 < n_prompt; i++) {
+        if (write_token(m, prompt[i])) return 1;
+        if (run_token(m, false, use_graph != 0)) return 1;
+    }
+    if (write_token(m, prompt[n_prompt - 1])) return 1;
+    if (ksh_synchronize(m->ctx)) return 1;
+    const auto t1 = clk::now();
+    const int first = m->pos;
+    for (int i = 0; i < n_new; i++)
+        if (run_token(m, true, use_graph != 0)) return 1;
+    if (ksh_synchronize(m->ctx)) return 1;
+    const auto t2 = clk::now();
+    if (prefill_ms) *prefill_ms = std::chrono::duration<double, std::milli>(t1 - t0).count();
+    if (decode_ms) *decode_ms = std::chrono::duration<double, std::milli>(t2 - t1).count();
+    if (n_new) {
+        std::vector<float> ids((size_t)n_new);
+        if (ksh_buffer_read(m->ctx, m->history, (size_t)first * 4, ids.data(), (size_t)n_new * 4, 1)) return 1;
+        for (int i = 0; i < n_new; i++) out_ids[i] = (uint32_t)ids[i];
+    }
+    return 0;
+}
+
+ksh_buf *ksh_gemma4_logits(ksh_gemma4 *m) { return m ? m->logits : nullptr; }
+ksh_buf *ksh_gemma4_hidden(ksh_gemma4 *m) { return m ? (m->hidden ? m->hidden : m->x) : nullptr; }
+int ksh_gemma4_kv_source(ksh_gemma4 *m, int layer) { return (!m || layer < 0 || layer >= m->c.n_layers) ? -1 : m->plan[layer].src; }
+ksh_buf *ksh_gemma4_kv(ksh_gemma4 *m, int layer, int which)
+{
+    if (!m || layer < 0 || layer >= m->c.n_layers) return nullptr;
+    const int src = m->plan[layer].src;
+    return which ? m->kv_v[src] : m->kv_k[src];
+}
+int ksh_gemma4_pos(ksh_gemma4 *m) { return m ? m->pos : -1; }
+int ksh_gemma4_launches_per_token(ksh_gemma4 *m) { return m ? m->launches_full : -1; }
+
+}  // extern "C"

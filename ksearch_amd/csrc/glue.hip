@@ -203,6 +203,27 @@ __device__ __forceinline__ float deq_q4k_at(const uint8_t *blk, int j)
     return d * (float)sc * (float)n - dmin * (float)mn;
 }
 
+__device__ __forceinline__ float deq_q5k_at(const uint8_t *blk, int j)
+{
+    // ksearch_load_q5k, render.rs:695-724 / gguf_impl.rs:722-760
+    const float d = half_bits_to_f32((uint32_t)blk[0] | ((uint32_t)blk[1] << 8));
+    const float dmin = half_bits_to_f32((uint32_t)blk[2] | ((uint32_t)blk[3] << 8));
+    const uint8_t *sq = blk + 4;
+    const int sub = j >> 5;
+    uint32_t sc, mn;
+    if (sub < 4) {
+        sc = sq[sub] & 63u;
+        mn = sq[sub + 4] & 63u;
+    } else {
+        sc = (sq[sub + 4] & 0x0Fu) | ((uint32_t)(sq[sub - 4] >> 6) << 4);
+        mn = (uint32_t)(sq[sub + 4] >> 4) | ((uint32_t)(sq[sub] >> 6) << 4);
+    }
+    const uint8_t qb = blk[48 + (j >> 6) * 32 + (j & 31)];
+    const float n = (float)((j & 32) ? (uint32_t)(qb >> 4) : (uint32_t)(qb & 0x0F));
+    const float hi = ((blk[16 + (j & 31)] >> sub) & 1) ? 16.0f : 0.0f;
+    return d * (float)sc * (n + hi) - dmin * (float)mn;
+}
+
 __global__ void copy_scale_indexed_kernel(const uint8_t *__restrict__ src, const float *__restrict__ idx,
                                           float *out, int n, float scale, int dtype, int64_t n_rows)
 {
@@ -217,6 +238,11 @@ __global__ void copy_scale_indexed_kernel(const uint8_t *__restrict__ src, const
     } else if (dtype == KSH_Q4K) {
         const uint8_t *row = src + (size_t)id * (size_t)(n / 256) * 144;
         v = deq_q4k_at(row + (size_t)(i >> 8) * 144, i & 255);
+    } else if (dtype == KSH_Q5K) {
+        const uint8_t *row = src + (size_t)id * (size_t)(n / 256) * 176;
+        v = deq_q5k_at(row + (size_t)(i >> 8) * 176, i & 255);
+    } else if (dtype == KSH_F16) {
+        v = half_bits_to_f32(reinterpret_cast<const uint16_t *>(src)[(size_t)id * n + i]);
     } else {
         v = reinterpret_cast<const float *>(src)[(size_t)id * n + i];
     }
@@ -462,7 +488,8 @@ int bind_glue(ksh_kernel &k)
     case KSH_COPY_SCALE_INDEXED: {
         const int dt = k.desc.dtypes[0];
         const int64_t n_rows = k.desc.dims[1];
-        if (dt != KSH_Q6K && dt != KSH_Q4K && dt != KSH_F32) return set_error("copy_scale_indexed: source dtype %d is not built", dt);
+        if (dt != KSH_Q6K && dt != KSH_Q5K && dt != KSH_Q4K && dt != KSH_F16 && dt != KSH_F32)
+            return set_error("copy_scale_indexed: source dtype %d is not built", dt);
         if (n_rows <= 0) return set_error("copy_scale_indexed: dims[1] (rows in the table) must be positive");
         const size_t rb = dt == KSH_F32 ? (size_t)n * 4 : packed_bytes(dt, (size_t)n);
         if (!rb) return set_error("copy_scale_indexed: n=%lld is not a whole number of blocks", (long long)n);

@@ -70,6 +70,9 @@ static int bind(ksh_kernel &k)
     case KSH_DEQUANT: return bind_dequant(k);
     case KSH_REPACK_ROWS: return bind_repack_rows(k);
     case KSH_QUANTIZE_K: return bind_quantize_k(k);
+    case KSH_RMSNORM_PER_HEAD:
+    case KSH_ADD_SCALE:
+    case KSH_MATVEC_GELU_MUL: return bind_ple_ops(k);
     }
     return set_error("unknown kernel kind %d", k.desc.kind);
 }

@@ -59,6 +59,9 @@ class Kind(enum.IntEnum):           # enum ksh_kind
     ATTEND_DECODE = 22
     ATTN_MERGE_MATVEC = 23
     REPACK_ROWS = 24
+    RMSNORM_PER_HEAD = 25
+    ADD_SCALE = 26
+    MATVEC_GELU_MUL = 27
 
 
 class Sched(C.Structure):           # ksh_sched: OptSchedule retargeted to gfx950
@@ -90,6 +93,29 @@ GEMMA_LAYER_FIELDS = ("wq", "wk", "wv", "wo", "wgate", "wup", "wdown",
 
 class GemmaLayer(C.Structure):
     _fields_ = [(n, C.c_void_p) for n in GEMMA_LAYER_FIELDS]
+
+
+GEMMA4_CFG_INTS = ("n_layers", "hidden", "n_q", "n_kv", "vocab", "max_seq", "hd_swa", "hd_full", "sliding_window",
+                   "shared_kv_layers", "ple_dim")
+GEMMA4_CFG_FLOATS = ("eps", "softcap", "rope_theta_swa", "rope_theta_full", "partial_rotary", "attn_scale")
+GEMMA4_WEIGHTS = ("wq", "wk", "wv", "wo", "wgate", "wup", "wdown", "inp_gate", "proj")
+GEMMA4_NORMS = ("attn_norm", "q_norm", "k_norm", "post_attn_norm", "ffn_norm", "post_ffw_norm", "post_norm")
+GEMMA4_DTYPES = ("dt_q", "dt_k", "dt_v", "dt_o", "dt_gate", "dt_up", "dt_down", "dt_inp_gate", "dt_proj")
+
+
+class Gemma4Cfg(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in GEMMA4_CFG_INTS] + [(n, C.c_float) for n in GEMMA4_CFG_FLOATS]
+
+
+class Gemma4Layer(C.Structure):
+    _fields_ = [("is_swa", C.c_int32), ("ffn", C.c_int32)] + [(n, C.c_int32) for n in GEMMA4_DTYPES] + \
+               [(n, C.c_void_p) for n in GEMMA4_WEIGHTS + GEMMA4_NORMS] + [("layer_scale", C.c_float)]
+
+
+class Gemma4Globals(C.Structure):
+    _fields_ = [("token_embd", C.c_void_p), ("dt_embd", C.c_int32), ("output_norm", C.c_void_p),
+                ("ple_embd", C.c_void_p), ("dt_ple", C.c_int32), ("ple_model_proj", C.c_void_p),
+                ("dt_ple_proj", C.c_int32), ("ple_proj_norm", C.c_void_p)]
 
 
 # every symbol include/ksearch_hip.h declares: name -> (restype, argtypes)
@@ -140,6 +166,17 @@ SYMBOLS = {
     "ksh_gemma_kv": (_vp, [_vp, _i, _i]),
     "ksh_gemma_pos": (_i, [_vp]),
     "ksh_gemma_launches_per_token": (_i, [_vp]),
+    "ksh_gemma4_create": (_i, [_vp, C.POINTER(Gemma4Cfg), C.POINTER(Gemma4Layer), C.POINTER(Gemma4Globals), _vpp]),
+    "ksh_gemma4_destroy": (None, [_vp]),
+    "ksh_gemma4_reset": (_i, [_vp]),
+    "ksh_gemma4_forward_token": (_i, [_vp, C.c_uint32, _i, _i, C.POINTER(C.c_uint32)]),
+    "ksh_gemma4_generate": (_i, [_vp, C.POINTER(C.c_uint32), _i, _i, _i, C.POINTER(C.c_uint32), _dp, _dp]),
+    "ksh_gemma4_logits": (_vp, [_vp]),
+    "ksh_gemma4_hidden": (_vp, [_vp]),
+    "ksh_gemma4_kv_source": (_i, [_vp, _i]),
+    "ksh_gemma4_kv": (_vp, [_vp, _i, _i]),
+    "ksh_gemma4_pos": (_i, [_vp]),
+    "ksh_gemma4_launches_per_token": (_i, [_vp]),
 }
 
 _lib = None
@@ -531,6 +568,31 @@ class Eng:
         ctx.encode_offsets_multi(kk, [q, qw, rope, k, kw, v], [0, 0, rope_off * 4, 0, 0, 0],
                                  [q_out, k_out, v_out], [0, kv_byte_off, kv_byte_off])
 
+    # :564-583
+    def rmsnorm_per_head(self, ctx, n_heads, hd, eps, x, w, y):
+        k = self._k(ctx, Kind.RMSNORM_PER_HEAD, (n_heads, hd, 0), (), (eps,))
+        ctx.encode_multi(k, [x, w], [y])
+
+    # :601-632 (offsets in f32 elements)
+    def rmsnorm_per_head_rope_off(self, ctx, n_heads, hd, eps, x, w, cos_sin, cos_sin_off, y, y_off=0):
+        k = self._k(ctx, Kind.RMSNORM_PER_HEAD, (n_heads, hd, 1), (), (eps,))
+        ctx.encode_offsets_multi(k, [x, w, cos_sin], [0, 0, cos_sin_off * 4], [y], [y_off * 4])
+
+    # :918-937
+    def add_scale(self, ctx, n, scale, a, b, y):
+        k = self._k(ctx, Kind.ADD_SCALE, (n,), (), (scale,))
+        ctx.encode_multi(k, [a, b], [y])
+
+    # :791-822
+    def matvec_gelu_mul_at(self, ctx, rows, cols, wdt, w, x, ctx_buf, ctx_off, y):
+        k = self._k(ctx, Kind.MATVEC_GELU_MUL, (rows, cols), (wdt, DType.F32), ())
+        ctx.encode_offsets_multi(k, [w, x, ctx_buf], [0, 0, ctx_off * 4], [y], [0])
+
+    # :897-916: the projection, then rmsnorm_add_scale, as two launches like the reference's
+    def matvec_rmsnorm_add_scale(self, ctx, rows, cols, eps, scale, wdt, w, x, w_norm, residual, y, scratch):
+        self.matvec_wd(ctx, rows, cols, wdt, w, x, scratch)
+        self.rmsnorm_add_scale(ctx, rows, eps, scale, scratch, w_norm, residual, y)
+
     # :1181-1197
     def quantize_q40(self, ctx, n, src, dst, dst_byte_off=0):
         k = self._k(ctx, Kind.QUANTIZE_Q40, (n,))
@@ -687,4 +749,95 @@ class Gemma:
 
     def kv(self, layer: int, which: int, nbytes: int) -> np.ndarray:
         b = Buffer(self.ctx, lib().ksh_gemma_kv(self.h, layer, which), owned=False)
+        return self.ctx.read_bytes(b, nbytes)
+
+
+class Gemma4:
+    """GemmaPrimModel with the layer features of the real Gemma-4 checkpoints
+    (crates/ksearch_gemma/src/gemma_prim.rs:881-1275; crates/ksearch_gemma/src/lib.rs:39-167).
+
+    ``cfg``: the fields of ksh_gemma4_cfg.  ``weights``: ``layers`` (one dict per
+    layer: ``is_swa``, ``ffn``, ``layer_scale``, the weight tensors with their
+    ``dt_*`` codes, the f32 norm vectors) and ``globals`` (``token_embd``,
+    ``dt_embd``, ``output_norm`` and, with per-layer embeddings, ``ple_embd``,
+    ``dt_ple``, ``ple_model_proj``, ``dt_ple_proj``, ``ple_proj_norm``).
+    Tensors are host arrays (uploaded here) or device Buffers."""
+
+    def __init__(self, ctx: Context, cfg: dict, weights: dict):
+        self.ctx, self.cfg = ctx, dict(cfg)
+        self._bufs = []
+
+        def up(a):
+            if a is None:
+                return None
+            b = a if isinstance(a, Buffer) else ctx.buffer_bytes(a)
+            self._bufs.append(b)
+            return b.h
+
+        n = cfg["n_layers"]
+        arr = (Gemma4Layer * n)()
+        for i, lw in enumerate(weights["layers"]):
+            arr[i].is_swa, arr[i].ffn = int(lw["is_swa"]), int(lw["ffn"])
+            arr[i].layer_scale = float(lw.get("layer_scale", 1.0))
+            for name in GEMMA4_DTYPES:
+                setattr(arr[i], name, int(lw.get(name, DType.Q4K)))
+            for name in GEMMA4_WEIGHTS + GEMMA4_NORMS:
+                setattr(arr[i], name, up(lw.get(name)))
+        self._layers = arr
+        g, gw = Gemma4Globals(), weights["globals"]
+        for name in ("token_embd", "output_norm", "ple_embd", "ple_model_proj", "ple_proj_norm"):
+            setattr(g, name, up(gw.get(name)))
+        for name in ("dt_embd", "dt_ple", "dt_ple_proj"):
+            setattr(g, name, int(gw.get(name, DType.Q4K)))
+        self._globals = g
+        c = Gemma4Cfg(**{k: cfg[k] for k in GEMMA4_CFG_INTS + GEMMA4_CFG_FLOATS})
+        h = C.c_void_p()
+        _check(lib().ksh_gemma4_create(ctx.h, C.byref(c), arr, C.byref(g), C.byref(h)))
+        self.h = h
+
+    def close(self):
+        if self.h:
+            lib().ksh_gemma4_destroy(self.h)
+            self.h = None
+        for b in self._bufs:
+            b.release()
+        self._bufs = []
+
+    def reset(self):
+        _check(lib().ksh_gemma4_reset(self.h))
+
+    @property
+    def pos(self) -> int:
+        return lib().ksh_gemma4_pos(self.h)
+
+    @property
+    def launches_per_token(self) -> int:
+        return lib().ksh_gemma4_launches_per_token(self.h)
+
+    def kv_source(self, layer: int) -> int:
+        return lib().ksh_gemma4_kv_source(self.h, layer)
+
+    def forward_token(self, token: int, want_logits: bool = True, use_graph: bool = False, read_next: bool = True):
+        nxt = C.c_uint32()
+        _check(lib().ksh_gemma4_forward_token(self.h, int(token), int(want_logits), int(use_graph),
+                                              C.byref(nxt) if read_next and want_logits else None))
+        return nxt.value if read_next and want_logits else None
+
+    def generate(self, prompt, n_new: int, use_graph: bool = True):
+        p = (C.c_uint32 * len(prompt))(*[int(t) for t in prompt])
+        out = (C.c_uint32 * max(1, n_new))()
+        pre, dec = C.c_double(), C.c_double()
+        _check(lib().ksh_gemma4_generate(self.h, p, len(prompt), n_new, int(use_graph), out, C.byref(pre), C.byref(dec)))
+        return list(out[:n_new]), pre.value, dec.value
+
+    def logits(self) -> np.ndarray:
+        b = Buffer(self.ctx, lib().ksh_gemma4_logits(self.h), owned=False)
+        return self.ctx.read_f32(b, self.cfg["vocab"])
+
+    def hidden(self) -> np.ndarray:
+        b = Buffer(self.ctx, lib().ksh_gemma4_hidden(self.h), owned=False)
+        return self.ctx.read_f32(b, self.cfg["hidden"])
+
+    def kv(self, layer: int, which: int, nbytes: int) -> np.ndarray:
+        b = Buffer(self.ctx, lib().ksh_gemma4_kv(self.h, layer, which), owned=False)
         return self.ctx.read_bytes(b, nbytes)

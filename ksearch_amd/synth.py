@@ -141,3 +141,68 @@ def gemma_weights(cfg: dict, seed: int, quantize_q4k, quantize_q6k, std: float =
             futs.append(ex.submit(normal_f32, min(chunk, rows - r0) * h, s, std))
         embd = quantize_q6k([fu.result() for fu in futs])
     return dict(layers=layers, token_embd=embd, output_norm=np.ones(h, dtype=np.float32))
+
+
+def q5k_blocks(n_blocks: int, seed: int, d_lo: float = 1e-4, d_hi: float = 1e-3) -> np.ndarray:
+    """Random Q5_K superblocks (176 B): d, dmin = f16(U(d_lo, d_hi)); scales, high bits and nibbles uniform."""
+    rng = _rng(seed)
+    blk = np.empty((n_blocks, 176), dtype=np.uint8)
+    blk[:, 0:2] = _f16_uniform(rng, n_blocks, d_lo, d_hi).view(np.uint8).reshape(n_blocks, 2)
+    blk[:, 2:4] = _f16_uniform(rng, n_blocks, d_lo, d_hi).view(np.uint8).reshape(n_blocks, 2)
+    blk[:, 4:] = rng.integers(0, 256, size=(n_blocks, 172), dtype=np.uint8)
+    return blk.reshape(-1)
+
+
+# dtype codes shared by the C ABI and the CPU checker
+_Q4K, _Q5K, _Q6K = 2, 3, 4
+
+# a small model with every layer feature of the real checkpoints: five sliding-window layers per full-attention
+# layer, the last three layers reusing earlier caches, per-layer embeddings, a window shorter than the test runs
+GEMMA4_TINY = dict(n_layers=8, hidden=512, n_q=4, n_kv=1, vocab=1024, max_seq=64, hd_swa=128, hd_full=256,
+                   sliding_window=8, shared_kv_layers=3, ple_dim=256, eps=1e-6, softcap=30.0,
+                   rope_theta_swa=10000.0, rope_theta_full=1000000.0, partial_rotary=0.25, attn_scale=1.0)
+
+
+def gemma4_weights(cfg: dict, seed: int, quantize_q4k, quantize_q6k, ffn=None, swa_pattern=None, q6k_tensors=(),
+                   std: float = 0.02) -> dict:
+    """Weights for the Gemma-4 decode loop: N(0, std) matrices packed to Q4_K (or Q6_K for the (layer, name)
+    pairs in `q6k_tensors`), the tied embedding / LM head in Q6_K, a random Q5_K per-layer-embedding table, norm
+    vectors 1 + 0.1 N(0,1), layer scales in [0.5, 1.5].  `ffn` is one width or a list per layer; `swa_pattern`
+    defaults to the reference's (every sixth layer attends everything, crates/ksearch_gemma/src/lib.rs:93-96)."""
+    n, h, pd = cfg["n_layers"], cfg["hidden"], cfg["ple_dim"]
+    ffn = [ffn or 4 * h] * n if not isinstance(ffn, (list, tuple)) else list(ffn)
+    swa = list(swa_pattern) if swa_pattern is not None else [(i + 1) % 6 != 0 for i in range(n)]
+    owners = n - cfg["shared_kv_layers"]
+    rng = _rng(seed)
+    s = seed * 1000
+
+    def norm(k):
+        return (1.0 + 0.1 * rng.standard_normal(k)).astype(np.float32)
+
+    layers = []
+    for i in range(n):
+        hd = cfg["hd_swa"] if swa[i] else cfg["hd_full"]
+        qd, kvd = cfg["n_q"] * hd, cfg["n_kv"] * hd
+        shapes = [("wq", "dt_q", qd, h), ("wo", "dt_o", h, qd), ("wgate", "dt_gate", ffn[i], h),
+                  ("wup", "dt_up", ffn[i], h), ("wdown", "dt_down", h, ffn[i])]
+        if i < owners:
+            shapes += [("wk", "dt_k", kvd, h), ("wv", "dt_v", kvd, h)]
+        if pd:
+            shapes += [("inp_gate", "dt_inp_gate", pd, h), ("proj", "dt_proj", h, pd)]
+        lw = dict(is_swa=int(swa[i]), ffn=ffn[i], layer_scale=float(rng.uniform(0.5, 1.5)))
+        for name, dt, r, c in shapes:
+            s += 1
+            x = normal_f32(r * c, s, std)
+            six = (i, name) in q6k_tensors
+            lw[name] = quantize_q6k(x) if six else quantize_q4k(x)
+            lw[dt] = _Q6K if six else _Q4K
+        for name, k in (("attn_norm", h), ("q_norm", hd), ("k_norm", hd), ("post_attn_norm", h), ("ffn_norm", h),
+                        ("post_ffw_norm", h), ("post_norm", h)):
+            lw[name] = norm(k)
+        layers.append(lw)
+    g = dict(token_embd=quantize_q6k(normal_f32(cfg["vocab"] * h, s + 1, std)), dt_embd=_Q6K, output_norm=norm(h))
+    if pd:
+        pt = n * pd
+        g.update(ple_embd=q5k_blocks(cfg["vocab"] * pt // 256, s + 2), dt_ple=_Q5K,
+                 ple_model_proj=quantize_q4k(normal_f32(pt * h, s + 3, std)), dt_ple_proj=_Q4K, ple_proj_norm=norm(pd))
+    return dict(layers=layers, globals=g)

@@ -69,6 +69,17 @@ def lib() -> C.CDLL:
             "ko_gemma_pos": (i32, [vp]),
             "ko_gemma_kv": (vp, [vp, i32, i32]),
             "ko_gemma_hidden": (vp, [vp]),
+            "ko_rmsnorm_per_head": (None, [vp, vp, vp, i32, i32, f32, vp]),
+            "ko_add_scale": (None, [vp, vp, f32, sz, vp]),
+            "ko_matvec_gelu_mul": (i32, [i32, vp, sz, sz, vp, vp, vp, i32]),
+            "ko_gemma4_create": (vp, [vp, vp, vp]),
+            "ko_gemma4_destroy": (None, [vp]),
+            "ko_gemma4_reset": (None, [vp]),
+            "ko_gemma4_forward": (u32, [vp, u32, i32, vp, i32]),
+            "ko_gemma4_pos": (i32, [vp]),
+            "ko_gemma4_kv_source": (i32, [vp, i32]),
+            "ko_gemma4_kv": (vp, [vp, i32, i32]),
+            "ko_gemma4_hidden": (vp, [vp]),
         }
         for name, (res, args) in sig.items():
             fn = getattr(L, name)
@@ -296,6 +307,117 @@ class Gemma:
     def close(self):
         if self.h:
             lib().ko_gemma_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def rmsnorm_per_head(x, w, n_heads, hd, eps, rope_row=None) -> np.ndarray:
+    x, w = _f32(x), _f32(w)
+    r = _f32(rope_row) if rope_row is not None else None
+    out = np.empty(n_heads * hd, dtype=np.float32)
+    lib().ko_rmsnorm_per_head(_p(x), _p(w), _p(r) if r is not None else None, n_heads, hd, eps, _p(out))
+    return out
+
+
+def add_scale(a, b, scale) -> np.ndarray:
+    a, b = _f32(a), _f32(b)
+    out = np.empty_like(a)
+    lib().ko_add_scale(_p(a), _p(b), scale, a.size, _p(out))
+    return out
+
+
+def matvec_gelu_mul(dtype, w, rows, cols, x, ctx, threads=0) -> np.ndarray:
+    w, x, ctx = _u8(w), _f32(x), _f32(ctx)
+    y = np.empty(rows, dtype=np.float32)
+    if lib().ko_matvec_gelu_mul(dtype, _p(w), rows, cols, _p(x), _p(ctx), _p(y), threads):
+        raise ValueError("bad dtype/shape")
+    return y
+
+
+G4_CFG_INTS = ("n_layers", "hidden", "n_q", "n_kv", "vocab", "max_seq", "hd_swa", "hd_full", "sliding_window",
+               "shared_kv_layers", "ple_dim")
+G4_CFG_FLOATS = ("eps", "softcap", "rope_theta_swa", "rope_theta_full", "partial_rotary", "attn_scale")
+G4_DTYPES = ("dt_q", "dt_k", "dt_v", "dt_o", "dt_gate", "dt_up", "dt_down", "dt_inp_gate", "dt_proj")
+G4_WEIGHTS = ("wq", "wk", "wv", "wo", "wgate", "wup", "wdown", "inp_gate", "proj")
+G4_NORMS = ("attn_norm", "q_norm", "k_norm", "post_attn_norm", "ffn_norm", "post_ffw_norm", "post_norm")
+
+
+class Gemma4Cfg(C.Structure):
+    _fields_ = [(n, C.c_int) for n in G4_CFG_INTS] + [(n, C.c_float) for n in G4_CFG_FLOATS]
+
+
+class Gemma4Layer(C.Structure):
+    _fields_ = [("is_swa", C.c_int), ("ffn", C.c_int)] + [(n, C.c_int) for n in G4_DTYPES] + \
+               [(n, C.c_void_p) for n in G4_WEIGHTS + G4_NORMS] + [("layer_scale", C.c_float)]
+
+
+class Gemma4Globals(C.Structure):
+    _fields_ = [("token_embd", C.c_void_p), ("dt_embd", C.c_int), ("output_norm", C.c_void_p),
+                ("ple_embd", C.c_void_p), ("dt_ple", C.c_int), ("ple_model_proj", C.c_void_p),
+                ("dt_ple_proj", C.c_int), ("ple_proj_norm", C.c_void_p)]
+
+
+class Gemma4:
+    """CPU greedy decoder with the real checkpoints' layer features, over the
+    same packed host arrays the HIP path uploads (``cfg`` / ``weights`` as for
+    ``ksearch_amd.hip.Gemma4``; dtype codes are the shared 0..6 numbering)."""
+
+    def __init__(self, cfg: dict, weights: dict):
+        self._keep = weights
+        self.cfg = Gemma4Cfg(**{k: cfg[k] for k in G4_CFG_INTS + G4_CFG_FLOATS})
+        n = cfg["n_layers"]
+        arr = (Gemma4Layer * n)()
+        for i, lw in enumerate(weights["layers"]):
+            arr[i].is_swa, arr[i].ffn = int(lw["is_swa"]), int(lw["ffn"])
+            arr[i].layer_scale = float(lw.get("layer_scale", 1.0))
+            for name in G4_DTYPES:
+                setattr(arr[i], name, int(lw.get(name, Q4K)))
+            for name in G4_WEIGHTS + G4_NORMS:
+                a = lw.get(name)
+                setattr(arr[i], name, _p(a) if a is not None else None)
+        self._layers = arr
+        g, gw = Gemma4Globals(), weights["globals"]
+        for name in ("token_embd", "output_norm", "ple_embd", "ple_model_proj", "ple_proj_norm"):
+            a = gw.get(name)
+            setattr(g, name, _p(a) if a is not None else None)
+        for name in ("dt_embd", "dt_ple", "dt_ple_proj"):
+            setattr(g, name, int(gw.get(name, Q4K)))
+        self._globals = g
+        self.h = lib().ko_gemma4_create(C.byref(self.cfg), arr, C.byref(g))
+        self.vocab = cfg["vocab"]
+
+    def reset(self):
+        lib().ko_gemma4_reset(self.h)
+
+    @property
+    def pos(self) -> int:
+        return lib().ko_gemma4_pos(self.h)
+
+    def kv_source(self, layer: int) -> int:
+        return lib().ko_gemma4_kv_source(self.h, layer)
+
+    def forward(self, token: int, want_logits: bool = True, return_logits: bool = False, threads: int = 0):
+        logits = np.empty(self.vocab, dtype=np.float32) if return_logits else None
+        nxt = lib().ko_gemma4_forward(self.h, int(token), int(want_logits),
+                                      _p(logits) if logits is not None else None, threads)
+        return (nxt, logits) if return_logits else nxt
+
+    def kv(self, layer: int, which: int, nbytes: int) -> np.ndarray:
+        ptr = lib().ko_gemma4_kv(self.h, layer, which)
+        return np.ctypeslib.as_array(C.cast(ptr, C.POINTER(C.c_uint8)), shape=(nbytes,)).copy()
+
+    def hidden(self) -> np.ndarray:
+        ptr = lib().ko_gemma4_hidden(self.h)
+        return np.ctypeslib.as_array(C.cast(ptr, C.POINTER(C.c_float)), shape=(self.cfg.hidden,)).copy()
+
+    def close(self):
+        if self.h:
+            lib().ko_gemma4_destroy(self.h)
             self.h = None
 
     def __del__(self):

@@ -900,3 +900,189 @@ uint32_t ko_gemma_forward(ko_gemma *m, uint32_t token, int want_logits, float *l
     if (logits_out) memcpy(logits_out, m->logits, sizeof(float) * (size_t)c->vocab);
     return ko_softcap_argmax(m->logits, (size_t)c->vocab, c->softcap);
 }
+
+/* ------------------------------------------------------------------ Gemma-4 extras */
+
+void ko_rmsnorm_per_head(const float *x, const float *w, const float *rope_row, int n_heads, int hd,
+                         float eps, float *out)
+{
+    for (int h = 0; h < n_heads; h++) {
+        const float *xh = x + (size_t)h * hd;
+        float *oh = out + (size_t)h * hd;
+        if (rope_row) {
+            float *tmp = (float *)malloc(sizeof(float) * (size_t)hd);
+            head_rms_rope(xh, w, rope_row, hd, eps, tmp);
+            memcpy(oh, tmp, sizeof(float) * (size_t)hd);
+            free(tmp);
+        } else {
+            float inv = head_rms_inv(xh, hd, eps);
+            for (int i = 0; i < hd; i++) oh[i] = xh[i] * inv * w[i];
+        }
+    }
+}
+
+void ko_add_scale(const float *a, const float *b, float scale, size_t n, float *out)
+{
+    for (size_t i = 0; i < n; i++) out[i] = scale * (a[i] + b[i]);
+}
+
+int ko_matvec_gelu_mul(int dtype, const uint8_t *w, size_t rows, size_t cols, const float *x,
+                       const float *ctx, float *y, int threads)
+{
+    int rc = ko_matvec(dtype, w, rows, cols, x, y, threads);
+    if (rc) return rc;
+    for (size_t r = 0; r < rows; r++) y[r] = ko_gelu_mul(y[r], ctx[r]);
+    return 0;
+}
+
+struct ko_gemma4 {
+    ko_gemma4_cfg c;
+    ko_gemma4_layer *layers;
+    ko_gemma4_globals g;
+    uint8_t **kv_k, **kv_v;      /* per owning layer */
+    float *rope_swa, *rope_full;
+    float *x, *x2, *tq, *tk, *tv, *to, *ff, *ff2, *logits;
+    float *ple_tok, *ple_tmp, *ple_ctx, *ple_u;
+    int pos;
+};
+
+static int g4_hd(const ko_gemma4_cfg *c, const ko_gemma4_layer *L) { return L->is_swa ? c->hd_swa : c->hd_full; }
+static int g4_owns(const ko_gemma4_cfg *c, int l)
+{
+    int owners = c->n_layers - c->shared_kv_layers;
+    return l < (owners > 0 ? owners : 0);
+}
+
+int ko_gemma4_kv_source(const ko_gemma4 *m, int layer)
+{
+    if (g4_owns(&m->c, layer)) return layer;
+    for (int i = layer - 1; i >= 0; i--)
+        if (g4_owns(&m->c, i) && m->layers[i].is_swa == m->layers[layer].is_swa) return i;
+    return 0;
+}
+
+ko_gemma4 *ko_gemma4_create(const ko_gemma4_cfg *cfg, const ko_gemma4_layer *layers,
+                            const ko_gemma4_globals *g)
+{
+    ko_gemma4 *m = (ko_gemma4 *)calloc(1, sizeof(*m));
+    m->c = *cfg;
+    m->g = *g;
+    m->layers = (ko_gemma4_layer *)malloc(sizeof(ko_gemma4_layer) * (size_t)cfg->n_layers);
+    memcpy(m->layers, layers, sizeof(ko_gemma4_layer) * (size_t)cfg->n_layers);
+    m->kv_k = (uint8_t **)calloc((size_t)cfg->n_layers, sizeof(uint8_t *));
+    m->kv_v = (uint8_t **)calloc((size_t)cfg->n_layers, sizeof(uint8_t *));
+    int max_hd = cfg->hd_swa > cfg->hd_full ? cfg->hd_swa : cfg->hd_full, max_ff = 0;
+    for (int l = 0; l < cfg->n_layers; l++) {
+        if (layers[l].ffn > max_ff) max_ff = layers[l].ffn;
+        if (!g4_owns(cfg, l)) continue;
+        int hd = g4_hd(cfg, &layers[l]);
+        size_t kvb = (size_t)cfg->max_seq * cfg->n_kv * (hd / 32) * 18; /* gemma_prim.rs:199-207 */
+        m->kv_k[l] = (uint8_t *)calloc(kvb, 1);
+        m->kv_v[l] = (uint8_t *)calloc(kvb, 1);
+    }
+    /* gemma_prim.rs:217-228: the sliding-window table rotates every pair, the full-attention table the
+     * first hd*partial_rotary/2 of them */
+    m->rope_swa = (float *)malloc(sizeof(float) * (size_t)cfg->max_seq * cfg->hd_swa);
+    ko_rope_table(cfg->max_seq, cfg->hd_swa, cfg->rope_theta_swa, cfg->hd_swa / 2, m->rope_swa);
+    m->rope_full = (float *)malloc(sizeof(float) * (size_t)cfg->max_seq * cfg->hd_full);
+    ko_rope_table(cfg->max_seq, cfg->hd_full, cfg->rope_theta_full,
+                  (int)((float)cfg->hd_full * cfg->partial_rotary) / 2, m->rope_full);
+    size_t h = (size_t)cfg->hidden, pt = (size_t)cfg->n_layers * cfg->ple_dim;
+    m->x = (float *)calloc(h, 4);
+    m->x2 = (float *)calloc(h, 4);
+    m->tq = (float *)calloc((size_t)cfg->n_q * max_hd, 4);
+    m->tk = (float *)calloc((size_t)cfg->n_kv * max_hd, 4);
+    m->tv = (float *)calloc((size_t)cfg->n_kv * max_hd, 4);
+    m->to = (float *)calloc((size_t)cfg->n_q * max_hd, 4);
+    m->ff = (float *)calloc((size_t)max_ff, 4);
+    m->ff2 = (float *)calloc((size_t)max_ff, 4);
+    m->logits = (float *)calloc((size_t)cfg->vocab, 4);
+    m->ple_tok = (float *)calloc(pt + 1, 4);
+    m->ple_tmp = (float *)calloc(pt + 1, 4);
+    m->ple_ctx = (float *)calloc(pt + 1, 4);
+    m->ple_u = (float *)calloc((size_t)cfg->ple_dim + 1, 4);
+    return m;
+}
+
+void ko_gemma4_destroy(ko_gemma4 *m)
+{
+    if (!m) return;
+    for (int l = 0; l < m->c.n_layers; l++) { free(m->kv_k[l]); free(m->kv_v[l]); }
+    free(m->kv_k); free(m->kv_v); free(m->layers); free(m->rope_swa); free(m->rope_full);
+    free(m->x); free(m->x2); free(m->tq); free(m->tk); free(m->tv); free(m->to); free(m->ff); free(m->ff2);
+    free(m->logits); free(m->ple_tok); free(m->ple_tmp); free(m->ple_ctx); free(m->ple_u); free(m);
+}
+
+void ko_gemma4_reset(ko_gemma4 *m) { m->pos = 0; }
+int ko_gemma4_pos(const ko_gemma4 *m) { return m->pos; }
+const uint8_t *ko_gemma4_kv(const ko_gemma4 *m, int layer, int which)
+{
+    return which ? m->kv_v[layer] : m->kv_k[layer];
+}
+const float *ko_gemma4_hidden(const ko_gemma4 *m) { return m->x; }
+
+uint32_t ko_gemma4_forward(ko_gemma4 *m, uint32_t token, int want_logits, float *logits_out, int threads)
+{
+    const ko_gemma4_cfg *c = &m->c;
+    const int h = c->hidden, pd = c->ple_dim;
+    const size_t pt = (size_t)c->n_layers * pd;
+    /* embed (gemma_prim.rs:681-710) */
+    ko_copy_scale_indexed(m->g.dt_embd, m->g.token_embd, token, (size_t)h, sqrtf((float)h), m->x);
+    if (pd > 0) {
+        /* ple_from_idx (:712-728): row of the per-layer table times sqrt(ple_dim);
+         * ple_prepass (:845-878): model projection, per-layer norm, (ctx + tok)/sqrt(2) */
+        ko_copy_scale_indexed(m->g.dt_ple, m->g.ple_embd, token, pt, sqrtf((float)pd), m->ple_tok);
+        ko_matvec(m->g.dt_ple_proj, m->g.ple_model_proj, pt, (size_t)h, m->x, m->ple_tmp, threads);
+        ko_rmsnorm_per_head(m->ple_tmp, m->g.ple_proj_norm, NULL, c->n_layers, pd, c->eps, m->ple_ctx);
+        ko_add_scale(m->ple_ctx, m->ple_tok, 0.70710678118654752440f, pt, m->ple_ctx);
+    }
+    for (int l = 0; l < c->n_layers; l++) {
+        const ko_gemma4_layer *L = &m->layers[l];
+        const int hd = g4_hd(c, L), owns = g4_owns(c, l), src = ko_gemma4_kv_source(m, l);
+        const float *rope = (L->is_swa ? m->rope_swa : m->rope_full) + (size_t)m->pos * hd;
+        const size_t krow = (size_t)c->n_kv * (hd / 32) * 18;
+        const size_t qd = (size_t)c->n_q * hd, kvd = (size_t)c->n_kv * hd;
+        ko_rmsnorm(m->x, L->attn_norm, NULL, c->eps, 0, 0, (size_t)h, m->x2);
+        ko_matvec(L->dt_q, L->wq, qd, (size_t)h, m->x2, m->tq, threads);
+        if (owns) {
+            ko_matvec(L->dt_k, L->wk, kvd, (size_t)h, m->x2, m->tk, threads);
+            ko_matvec(L->dt_v, L->wv, kvd, (size_t)h, m->x2, m->tv, threads);
+            ko_rmsnorm_per_head_qkv_q40(m->tq, L->q_norm, rope, m->tk, L->k_norm, m->tv, c->n_q, c->n_kv,
+                                        hd, c->eps, m->tq, m->kv_k[src] + (size_t)m->pos * krow,
+                                        m->kv_v[src] + (size_t)m->pos * krow);
+        } else {
+            ko_rmsnorm_per_head(m->tq, L->q_norm, rope, c->n_q, hd, c->eps, m->tq);   /* :989-1008 */
+        }
+        /* :1010-1017 */
+        int kv_len = m->pos + 1, start = 0;
+        if (L->is_swa) start = kv_len > c->sliding_window ? kv_len - c->sliding_window : 0;
+        int tlen = kv_len - start;
+        if (tlen >= 128)
+            ko_sdpa_mwg(m->tq, m->kv_k[src], m->kv_v[src], c->n_q, c->n_kv, hd, tlen, start,
+                        c->attn_scale, 16, m->to);
+        else
+            ko_sdpa_online(m->tq, m->kv_k[src], m->kv_v[src], c->n_q, c->n_kv, hd, tlen, start,
+                           c->attn_scale, m->to);
+        ko_matvec(L->dt_o, L->wo, (size_t)h, qd, m->to, m->x2, threads);
+        ko_rmsnorm_add_then_rmsnorm(m->x2, L->post_attn_norm, m->x, L->ffn_norm, c->eps, (size_t)h,
+                                    m->x, m->x2);
+        ko_matvec(L->dt_gate, L->wgate, (size_t)L->ffn, (size_t)h, m->x2, m->ff, threads);
+        ko_matvec(L->dt_up, L->wup, (size_t)L->ffn, (size_t)h, m->x2, m->ff2, threads);
+        for (int i = 0; i < L->ffn; i++) m->ff[i] = ko_gelu_mul(m->ff[i], m->ff2[i]);
+        ko_matvec(L->dt_down, L->wdown, (size_t)h, (size_t)L->ffn, m->ff, m->x2, threads);
+        ko_rmsnorm(m->x2, L->post_ffw_norm, m->x, c->eps, 0, 0, (size_t)h, m->x);
+        if (pd > 0) {
+            /* :1166-1200: gate GEMV with gelu*ctx, projection, rmsnorm_add_scale */
+            ko_matvec_gelu_mul(L->dt_inp_gate, L->inp_gate, (size_t)pd, (size_t)h, m->x,
+                               m->ple_ctx + (size_t)l * pd, m->ple_u, threads);
+            ko_matvec(L->dt_proj, L->proj, (size_t)h, (size_t)pd, m->ple_u, m->x2, threads);
+            ko_rmsnorm(m->x2, L->post_norm, m->x, c->eps, L->layer_scale, 1, (size_t)h, m->x);
+        }
+    }
+    m->pos += 1;
+    if (!want_logits) return 0;
+    ko_rmsnorm(m->x, m->g.output_norm, NULL, c->eps, 0, 0, (size_t)h, m->x2);
+    ko_matvec(m->g.dt_embd, m->g.token_embd, (size_t)c->vocab, (size_t)h, m->x2, m->logits, threads);
+    if (logits_out) memcpy(logits_out, m->logits, sizeof(float) * (size_t)c->vocab);
+    return ko_softcap_argmax(m->logits, (size_t)c->vocab, c->softcap);
+}

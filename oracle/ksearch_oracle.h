@@ -142,6 +142,61 @@ const uint8_t *ko_gemma_kv(const ko_gemma *m, int layer, int which);
 /* last token's hidden state after the final layer (before output norm) */
 const float *ko_gemma_hidden(const ko_gemma *m);
 
+/* ---- ops the real Gemma-4 checkpoints add to the decode step ---- */
+/* Eng::rmsnorm_per_head / rmsnorm_per_head_rope_off (crates/ksearch_kernels/src/lib.rs:564-625;
+ * crates/ksearch_codegen/src/lower.rs:4164-4228, 4356-4435): y[h,i] = x[h,i]*inv_h*w[i], then RoPE with
+ * `rope_row` (cos[0..hd/2) || sin[0..hd/2)) unless it is NULL */
+void ko_rmsnorm_per_head(const float *x, const float *w, const float *rope_row, int n_heads, int hd,
+                         float eps, float *out);
+/* Eng::add_scale (crates/ksearch_kernels/src/lib.rs:918-937): y = scale*(a+b) */
+void ko_add_scale(const float *a, const float *b, float scale, size_t n, float *out);
+/* Eng::matvec_gelu_mul_at (crates/ksearch_kernels/src/lib.rs:791-822; epilogue GeluMulCtx,
+ * crates/ksearch_codegen/src/lower.rs:622-643): y[r] = gelu(W[r].x) * ctx[r] */
+int ko_matvec_gelu_mul(int dtype, const uint8_t *w, size_t rows, size_t cols, const float *x,
+                       const float *ctx, float *y, int threads);
+
+/* ---- whole-model greedy decode with those extras, following forward_token
+ * (crates/ksearch_gemma/src/gemma_prim.rs:881-1275) and GemmaConfig (crates/ksearch_gemma/src/lib.rs:39-167):
+ * sliding-window and full-attention layers with their own head dims, rope tables and windows; layers past
+ * n_layers - shared_kv_layers reuse the cache of the last owning layer of their kind; per-layer embeddings
+ * (ple_dim > 0).  Activations stay f32 (the reference keeps them in f16). ---- */
+typedef struct {
+    int n_layers, hidden, n_q, n_kv, vocab, max_seq;
+    int hd_swa, hd_full, sliding_window, shared_kv_layers, ple_dim;
+    float eps, softcap, rope_theta_swa, rope_theta_full, partial_rotary, attn_scale;
+} ko_gemma4_cfg;
+
+typedef struct {
+    int is_swa, ffn;
+    int dt_q, dt_k, dt_v, dt_o, dt_gate, dt_up, dt_down, dt_inp_gate, dt_proj;   /* KO_Q4K or KO_Q6K */
+    const uint8_t *wq, *wk, *wv, *wo, *wgate, *wup, *wdown, *inp_gate, *proj;
+    const float *attn_norm, *q_norm, *k_norm, *post_attn_norm, *ffn_norm, *post_ffw_norm, *post_norm;
+    float layer_scale;
+} ko_gemma4_layer;
+
+typedef struct {
+    const uint8_t *token_embd;      /* [vocab, hidden], also the LM head */
+    int dt_embd;
+    const float *output_norm;
+    const uint8_t *ple_embd;        /* [vocab, n_layers*ple_dim] */
+    int dt_ple;
+    const uint8_t *ple_model_proj;  /* [n_layers*ple_dim, hidden] */
+    int dt_ple_proj;
+    const float *ple_proj_norm;     /* [ple_dim] */
+} ko_gemma4_globals;
+
+typedef struct ko_gemma4 ko_gemma4;
+ko_gemma4 *ko_gemma4_create(const ko_gemma4_cfg *cfg, const ko_gemma4_layer *layers,
+                            const ko_gemma4_globals *g);
+void ko_gemma4_destroy(ko_gemma4 *m);
+void ko_gemma4_reset(ko_gemma4 *m);
+uint32_t ko_gemma4_forward(ko_gemma4 *m, uint32_t token, int want_logits, float *logits_out, int threads);
+int ko_gemma4_pos(const ko_gemma4 *m);
+/* which layer's cache layer `l` reads (crates/ksearch_gemma/src/lib.rs:151-162) */
+int ko_gemma4_kv_source(const ko_gemma4 *m, int layer);
+const uint8_t *ko_gemma4_kv(const ko_gemma4 *m, int layer, int which);
+const float *ko_gemma4_hidden(const ko_gemma4 *m);
+
 #ifdef __cplusplus
 }
 #endif

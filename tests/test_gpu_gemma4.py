@@ -1,0 +1,197 @@
+"""The ops and the decode loop for the real Gemma-4 checkpoints' layer features (sliding-window and full-attention
+layers, shared KV caches, per-layer embeddings, mixed Q4_K / Q6_K tensors) vs the CPU oracle."""
+import numpy as np
+import pytest
+
+import oracle
+from ksearch_amd import hip, synth
+from ksearch_amd.hip import DType, Kind
+from tests.gpu_util import assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = hip.Context()
+    yield c
+    c.close()
+
+
+@pytest.fixture(scope="module")
+def eng():
+    return hip.Eng()
+
+
+def test_dequant_q5k_bit_exact(ctx, eng):
+    n = 256 * 300
+    blocks = synth.q5k_blocks(n // 256, 600, 1e-3, 1e-2)
+    dst = ctx.buffer_empty_f32(n)
+    eng.dequant(ctx, DType.Q5K, n, ctx.buffer_bytes(blocks), dst)
+    assert np.array_equal(ctx.read_f32(dst, n), oracle.dequant(oracle.Q5K, blocks, n))
+
+
+@pytest.mark.parametrize("dt,rb", [(DType.Q5K, 176), (DType.Q4K, 144), (DType.Q6K, 210), (DType.F16, 512)])
+def test_copy_scale_indexed_row_gather(ctx, eng, dt, rb):
+    n, rows = 1024, 37
+    if dt == DType.F16:
+        table = synth.normal_f32(rows * n, 601).astype(np.float16)
+        raw, odt = table.view(np.uint8), oracle.F16
+    else:
+        gen = {DType.Q5K: synth.q5k_blocks, DType.Q4K: synth.q4k_blocks, DType.Q6K: synth.q6k_blocks}[dt]
+        raw, odt = gen(rows * n // 256, 601), int(dt)
+    src, out, idx = ctx.buffer_bytes(raw), ctx.buffer_empty_f32(n), ctx.buffer_f32(np.array([0], np.float32))
+    for rid in (0, 17, rows - 1):
+        ctx.write_buffer(idx, np.array([rid], np.float32))
+        k = eng._k(ctx, Kind.COPY_SCALE_INDEXED, (n, rows), (dt,), (16.0,))
+        ctx.encode_multi(k, [src, idx], [out])
+        assert np.array_equal(ctx.read_f32(out, n), oracle.copy_scale_indexed(odt, raw, rid, n, 16.0)), rid
+
+
+@pytest.mark.parametrize("n_heads,hd", [(5, 64), (4, 128), (30, 256), (8, 512)])
+def test_rmsnorm_per_head_and_rope(ctx, eng, n_heads, hd):
+    rng = np.random.default_rng(602 + hd)
+    x = (rng.standard_normal(n_heads * hd) * 2).astype(np.float32)
+    w = (1 + 0.2 * rng.standard_normal(hd)).astype(np.float32)
+    tab = oracle.rope_table(9, hd, 10000.0, hd // 4)
+    bx, bw, bt, y = ctx.buffer_f32(x), ctx.buffer_f32(w), ctx.buffer_f32(tab), ctx.buffer_empty_f32(n_heads * hd)
+    eng.rmsnorm_per_head(ctx, n_heads, hd, 1e-6, bx, bw, y)
+    assert_close(ctx.read_f32(y, n_heads * hd), oracle.rmsnorm_per_head(x, w, n_heads, hd, 1e-6), 1e-5, "norm")
+    for pos in (0, 6):
+        eng.rmsnorm_per_head_rope_off(ctx, n_heads, hd, 1e-6, bx, bw, bt, pos * hd, y)
+        want = oracle.rmsnorm_per_head(x, w, n_heads, hd, 1e-6, tab[pos])
+        assert_close(ctx.read_f32(y, n_heads * hd), want, 1e-5, f"rope row {pos}")
+    # the position on the device, the whole table as input, in place
+    meta = ctx.buffer_f32(np.array([7, 0, 0, 6], np.float32))
+    k = eng._k(ctx, Kind.RMSNORM_PER_HEAD, (n_heads, hd, 2, 9), (), (1e-6,))
+    ctx.encode_multi(k, [bx, bw, bt, meta], [bx])
+    assert_close(ctx.read_f32(bx, n_heads * hd), want, 1e-5, "meta form, in place")
+    with pytest.raises(hip.KshError, match="hd=96"):
+        ctx.compile(hip.make_desc(Kind.RMSNORM_PER_HEAD, (2, 96, 0), (), (1e-6,)))
+
+
+def test_add_scale_and_matvec_gelu_mul(ctx, eng):
+    rng = np.random.default_rng(603)
+    n = 7680
+    a, b = rng.standard_normal(n).astype(np.float32), rng.standard_normal(n).astype(np.float32)
+    ba, out = ctx.buffer_f32(a), ctx.buffer_empty_f32(n)
+    eng.add_scale(ctx, n, 0.70710678, ba, ctx.buffer_f32(b), out)
+    assert np.array_equal(ctx.read_f32(out, n), oracle.add_scale(a, b, 0.70710678))
+    for rows, cols in ((256, 1536), (256, 2048), (10, 256), (64, 4608)):
+        w = synth.q4k_blocks(rows * cols // 256, 604)
+        x = rng.standard_normal(cols).astype(np.float32)
+        cvec = rng.standard_normal(3 * rows).astype(np.float32)
+        y = ctx.buffer_empty_f32(rows)
+        eng.matvec_gelu_mul_at(ctx, rows, cols, DType.Q4K, ctx.buffer_bytes(w), ctx.buffer_f32(x), ctx.buffer_f32(cvec), 2 * rows, y)
+        want = oracle.matvec_gelu_mul(oracle.Q4K, w, rows, cols, x, cvec[2 * rows:])
+        assert_close(ctx.read_f32(y, rows), want, 1e-3, f"{rows}x{cols}")
+    with pytest.raises(hip.KshError, match="Q4_K"):
+        ctx.compile(hip.make_desc(Kind.MATVEC_GELU_MUL, (256, 2048), (DType.Q6K, DType.F32)))
+
+
+PATTERN = [1, 1, 0, 1, 1, 1, 0, 1]
+FFN = [1024, 1024, 2048, 1024, 1024, 1024, 2048, 1024]
+
+
+@pytest.fixture(scope="module", params=["all_q4k", "mixed_q6k", "no_ple"])
+def tiny(ctx, request):
+    cfg = dict(synth.GEMMA4_TINY)
+    q6 = ()
+    if request.param == "mixed_q6k":
+        q6 = {(1, "wv"), (2, "wdown"), (3, "wq"), (4, "wgate"), (5, "wo"), (6, "wup"), (7, "proj")}
+    if request.param == "no_ple":
+        cfg["ple_dim"] = 0
+    w = synth.gemma4_weights(cfg, 610, oracle.quantize_q4k, oracle.quantize_q6k, ffn=FFN, swa_pattern=PATTERN, q6k_tensors=q6, std=0.05)
+    gpu, cpu = hip.Gemma4(ctx, cfg, w), oracle.Gemma4(cfg, w)
+    yield gpu, cpu, cfg
+    gpu.close()
+    cpu.close()
+
+
+def test_gemma4_forward_token_matches_oracle_teacher_forced(tiny):
+    """Teacher-forced and cache-synchronised, as for the synthetic shape: a K/V value on a Q4_0 rounding boundary
+    may take the neighbouring code; such a step is counted, its rows are overwritten with the oracle's, and its
+    logits are not compared.  24 positions: three times the sliding window."""
+    gpu, cpu, cfg = tiny
+    ctx = gpu.ctx
+    gpu.reset()
+    cpu.reset()
+    n_layers = cfg["n_layers"]
+    assert [gpu.kv_source(l) for l in range(n_layers)] == [cpu.kv_source(l) for l in range(n_layers)] == [0, 1, 2, 3, 4, 4, 2, 4]
+    owners = [l for l in range(n_layers) if gpu.kv_source(l) == l]
+    hd = {l: cfg["hd_swa"] if PATTERN[l] else cfg["hd_full"] for l in owners}
+    bufs = {l: [hip.Buffer(ctx, hip.lib().ksh_gemma4_kv(gpu.h, l, w), owned=False) for w in (0, 1)] for l in owners}
+    toks = np.random.default_rng(611).integers(0, cfg["vocab"], 24)
+    agree = clean = 0
+    for i, t in enumerate(toks):
+        g_next = gpu.forward_token(int(t), use_graph=False)
+        c_next, c_logits = cpu.forward(int(t), return_logits=True)
+        g_logits = gpu.logits()
+        flips = 0
+        for l in owners:
+            row = cfg["n_kv"] * hd[l] // 32 * 18
+            for w in (0, 1):
+                got, want = ctx.read_bytes(bufs[l][w], row, i * row), cpu.kv(l, w, (i + 1) * row)[i * row:]
+                if not np.array_equal(got, want):
+                    flips += int((got != want).sum())
+                    dg, dc = oracle.dequant(oracle.Q40, got, row // 18 * 32), oracle.dequant(oracle.Q40, want, row // 18 * 32)
+                    assert np.abs(dg - dc).max() <= np.abs(dc).max() / 7 * 1.01
+                    ctx.write_bytes(bufs[l][w], want, i * row)
+        assert g_next == oracle.softcap_argmax(g_logits, cfg["softcap"])
+        if flips:
+            continue
+        clean += 1
+        assert_close(g_logits, c_logits, 1e-3, f"logits at step {i}")
+        assert_close(gpu.hidden(), cpu.hidden(), 1e-3, f"hidden at step {i}")
+        top2 = np.sort(c_logits)[-2:]
+        if top2[1] - top2[0] > 1e-3 * max(abs(top2[1]), float(np.sqrt(np.mean(c_logits ** 2)))):
+            assert g_next == c_next, f"step {i}: margin {top2[1] - top2[0]}"
+            agree += 1
+    assert clean >= 18 and agree >= 14 and gpu.pos == cpu.pos == len(toks)
+    with pytest.raises(hip.KshError, match="outside the vocabulary"):
+        gpu.forward_token(cfg["vocab"])
+
+
+def test_gemma4_generate_graph_equals_eager_and_oracle(tiny):
+    gpu, cpu, cfg = tiny
+    prompt = [int(t) for t in np.random.default_rng(612).integers(0, cfg["vocab"], 6)]
+    n_new = 30
+    gpu.reset()
+    eager, _, _ = gpu.generate(prompt, n_new, use_graph=False)
+    gpu.reset()
+    graph, _, _ = gpu.generate(prompt, n_new, use_graph=True)
+    assert graph == eager
+    gpu.reset()
+    assert gpu.generate(prompt, n_new, use_graph=True)[0] == graph      # replay after reset
+    assert gpu.launches_per_token > 0
+    cpu.reset()
+    for t in prompt[:-1]:
+        cpu.forward(t, want_logits=False)
+    want, tok = [], prompt[-1]
+    margins = []
+    for _ in range(n_new):
+        tok, logits = cpu.forward(tok, return_logits=True)
+        want.append(tok)
+        top2 = np.sort(logits)[-2:]
+        margins.append((top2[1] - top2[0]) / max(abs(top2[1]), 1e-6))
+    # identical up to the first step whose top-2 margin is inside f32 reassociation noise
+    first_close = next((i for i, mg in enumerate(margins) if mg < 1e-3), n_new)
+    assert graph[:first_close] == want[:first_close]
+    assert first_close >= 8
+    with pytest.raises(hip.KshError, match="max_seq"):
+        gpu.generate(prompt, cfg["max_seq"], use_graph=True)
+
+
+def test_gemma4_create_errors(ctx):
+    cfg = dict(synth.GEMMA4_TINY, vocab=256)
+    w = synth.gemma4_weights(cfg, 613, oracle.quantize_q4k, oracle.quantize_q6k, ffn=512, swa_pattern=PATTERN)
+    with pytest.raises(hip.KshError, match="invalid configuration"):
+        hip.Gemma4(ctx, dict(cfg, shared_kv_layers=8), w)
+    # the reference's default pattern has no owning full-attention layer among the first five: the sixth layer
+    # would read a cache of another head dim
+    w_bad = synth.gemma4_weights(cfg, 613, oracle.quantize_q4k, oracle.quantize_q6k, ffn=512)
+    with pytest.raises(hip.KshError, match="another head dim"):
+        hip.Gemma4(ctx, cfg, w_bad)
+    bad = dict(w, layers=[dict(w["layers"][0], dt_q=int(DType.Q5K))] + w["layers"][1:])
+    with pytest.raises(hip.KshError, match="weight dtype"):
+        hip.Gemma4(ctx, cfg, bad)

@@ -364,6 +364,44 @@ int ksh_gemma4_kv_source(ksh_gemma4 *m, int layer);
 ksh_buf *ksh_gemma4_kv(ksh_gemma4 *m, int layer, int which);
 int ksh_gemma4_pos(ksh_gemma4 *m);
 int ksh_gemma4_launches_per_token(ksh_gemma4 *m);
+int ksh_gemma4_config(ksh_gemma4 *m, ksh_gemma4_cfg *cfg);
+
+/* ---- GGUF files: Gguf::open and its accessors (crates/ksearch_gguf/src/gguf_impl.rs:217-420).  The file is
+ * memory-mapped; tensor data pointers stay valid until ksh_gguf_close.  A malformed file is an error here where
+ * the reference panics. ---- */
+enum ksh_ggml_type {   /* gguf_impl.rs:19-31 */
+    KSH_GGML_F32 = 0, KSH_GGML_F16 = 1, KSH_GGML_Q4_0 = 2, KSH_GGML_Q4_1 = 3, KSH_GGML_Q5_1 = 7, KSH_GGML_Q8_0 = 8,
+    KSH_GGML_Q4_K = 12, KSH_GGML_Q5_K = 13, KSH_GGML_Q6_K = 14, KSH_GGML_BF16 = 30
+};
+typedef struct ksh_gguf ksh_gguf;
+int ksh_gguf_open(const char *path, ksh_gguf **out);
+void ksh_gguf_close(ksh_gguf *g);
+int ksh_gguf_version(const ksh_gguf *g);
+int64_t ksh_gguf_n_tensors(const ksh_gguf *g);
+int ksh_gguf_tensor_name(const ksh_gguf *g, int64_t index, char *dst, size_t n);
+int ksh_gguf_has_tensor(const ksh_gguf *g, const char *name);
+/* TensorInfo + tensor_raw: dims[0] is the contiguous dimension (columns), the rest multiply to the row count;
+ * any out pointer may be NULL */
+int ksh_gguf_tensor(const ksh_gguf *g, const char *name, int32_t *ggml_type, int64_t *dims /*[4]*/, int32_t *n_dims,
+                    const void **data, size_t *bytes);
+/* metadata accessors: 0 when the key exists with a fitting type, 1 otherwise (the reference's None) */
+int ksh_gguf_get_u32(const ksh_gguf *g, const char *key, uint32_t *out);
+int ksh_gguf_get_f32(const ksh_gguf *g, const char *key, float *out);
+int ksh_gguf_get_str(const ksh_gguf *g, const char *key, char *dst, size_t n);
+/* u32 / i32 / bool arrays (bools as 0/1); an integer scalar reads as a list of one (get_usize_list) */
+int ksh_gguf_get_arr_u32(const ksh_gguf *g, const char *key, uint32_t *dst, int cap, int *n);
+int ksh_gguf_arr_is_bool(const ksh_gguf *g, const char *key);
+/* dequant_blocks for F32 / F16 / BF16 / Q4_0 / Q4_1 / Q5_1 / Q8_0 on the host (gguf_impl.rs:577-689); the
+ * K-quants are dequantized by KSH_DEQUANT on the device */
+int ksh_gguf_dequant_host(int32_t ggml_type, const void *src, size_t n_elems, float *out);
+
+/* GemmaConfig::from_gguf (crates/ksearch_gemma/src/lib.rs:39-122).  ffn / is_swa (room for `cap` layers) may be
+ * NULL.  ple_dim is 0 when the file has no per-layer tables. */
+int ksh_gemma4_config_from_gguf(const ksh_gguf *g, int max_seq, ksh_gemma4_cfg *cfg, int32_t *ffn, int32_t *is_swa, int cap);
+/* GemmaPrimModel's load path (crates/ksearch_gemma/src/gemma_prim.rs:146-450): uploads Q4_K (and Q6_K) tensors as
+ * they are, converts the rest, builds the model, which then owns the buffers. */
+enum { KSH_LOAD_KEEP_Q6K = 1 };   /* do not requantize Q6_K ffn_down / attn_v to Q4_K (the reference does, :418-433) */
+int ksh_gemma4_load_gguf(ksh_ctx *ctx, const ksh_gguf *g, int max_seq, int flags, ksh_gemma4 **out);
 
 #ifdef __cplusplus
 }

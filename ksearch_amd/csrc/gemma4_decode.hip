@@ -575,5 +575,15 @@ ksh_buf *ksh_gemma4_kv(ksh_gemma4 *m, int layer, int which)
 }
 int ksh_gemma4_pos(ksh_gemma4 *m) { return m ? m->pos : -1; }
 int ksh_gemma4_launches_per_token(ksh_gemma4 *m) { return m ? m->launches_full : -1; }
+int ksh_gemma4_config(ksh_gemma4 *m, ksh_gemma4_cfg *cfg)
+{
+    if (!m || !cfg) return set_error("ksh_gemma4_config: bad arguments");
+    *cfg = m->c;
+    return 0;
+}
+void ksh_gemma4_adopt(ksh_gemma4 *m, ksh_buf *b)
+{
+    if (m && b) m->bufs.owned.push_back(b);
+}
 
 }  // extern "C"

@@ -57,6 +57,9 @@ struct ksh_kernel {
     int (*launch)(const ksh_kernel &, const ksh::LaunchArgs &, hipStream_t) = nullptr;
 };
 
+// hands a buffer's reference over to a model, which releases it when it is destroyed (the GGUF loader's uploads)
+extern "C" void ksh_gemma4_adopt(ksh_gemma4 *m, ksh_buf *b);
+
 namespace ksh {
 
 // block geometry: crates/ksearch_ir/src/lib.rs:52-74, gguf_impl.rs:50-64

@@ -177,6 +177,22 @@ SYMBOLS = {
     "ksh_gemma4_kv": (_vp, [_vp, _i, _i]),
     "ksh_gemma4_pos": (_i, [_vp]),
     "ksh_gemma4_launches_per_token": (_i, [_vp]),
+    "ksh_gemma4_config": (_i, [_vp, C.POINTER(Gemma4Cfg)]),
+    "ksh_gguf_open": (_i, [C.c_char_p, _vpp]),
+    "ksh_gguf_close": (None, [_vp]),
+    "ksh_gguf_version": (_i, [_vp]),
+    "ksh_gguf_n_tensors": (C.c_int64, [_vp]),
+    "ksh_gguf_tensor_name": (_i, [_vp, C.c_int64, C.c_char_p, _sz]),
+    "ksh_gguf_has_tensor": (_i, [_vp, C.c_char_p]),
+    "ksh_gguf_tensor": (_i, [_vp, C.c_char_p, C.POINTER(C.c_int32), _i64p, C.POINTER(C.c_int32), _vpp, C.POINTER(_sz)]),
+    "ksh_gguf_get_u32": (_i, [_vp, C.c_char_p, C.POINTER(C.c_uint32)]),
+    "ksh_gguf_get_f32": (_i, [_vp, C.c_char_p, C.POINTER(C.c_float)]),
+    "ksh_gguf_get_str": (_i, [_vp, C.c_char_p, C.c_char_p, _sz]),
+    "ksh_gguf_get_arr_u32": (_i, [_vp, C.c_char_p, C.POINTER(C.c_uint32), _i, C.POINTER(C.c_int)]),
+    "ksh_gguf_arr_is_bool": (_i, [_vp, C.c_char_p]),
+    "ksh_gguf_dequant_host": (_i, [C.c_int32, _vp, _sz, _vp]),
+    "ksh_gemma4_config_from_gguf": (_i, [_vp, _i, C.POINTER(Gemma4Cfg), C.POINTER(C.c_int32), C.POINTER(C.c_int32), _i]),
+    "ksh_gemma4_load_gguf": (_i, [_vp, _vp, _i, _i, _vpp]),
 }
 
 _lib = None
@@ -752,6 +768,101 @@ class Gemma:
         return self.ctx.read_bytes(b, nbytes)
 
 
+class GgmlType(enum.IntEnum):
+    F32 = 0
+    F16 = 1
+    Q4_0 = 2
+    Q4_1 = 3
+    Q5_1 = 7
+    Q8_0 = 8
+    Q4_K = 12
+    Q5_K = 13
+    Q6_K = 14
+    BF16 = 30
+
+
+LOAD_KEEP_Q6K = 1
+
+
+class Gguf:
+    """A memory-mapped GGUF file (Gguf::open, crates/ksearch_gguf/src/gguf_impl.rs:217-420).  Needs no GPU."""
+
+    def __init__(self, path: str):
+        h = C.c_void_p()
+        _check(lib().ksh_gguf_open(os.fsencode(path), C.byref(h)))
+        self.h = h
+
+    def close(self):
+        if self.h:
+            lib().ksh_gguf_close(self.h)
+            self.h = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    @property
+    def version(self) -> int:
+        return lib().ksh_gguf_version(self.h)
+
+    def tensor_names(self) -> list:
+        buf = C.create_string_buffer(512)
+        out = []
+        for i in range(lib().ksh_gguf_n_tensors(self.h)):
+            _check(lib().ksh_gguf_tensor_name(self.h, i, buf, 512))
+            out.append(buf.value.decode())
+        return out
+
+    def has_tensor(self, name: str) -> bool:
+        return bool(lib().ksh_gguf_has_tensor(self.h, name.encode()))
+
+    def tensor(self, name: str):
+        """(ggml type, dims as stored (dims[0] = columns), raw bytes as a numpy view into the mapping)."""
+        ty, nd, dims = C.c_int32(), C.c_int32(), (C.c_int64 * 4)()
+        data, nbytes = C.c_void_p(), C.c_size_t()
+        _check(lib().ksh_gguf_tensor(self.h, name.encode(), C.byref(ty), dims, C.byref(nd), C.byref(data), C.byref(nbytes)))
+        raw = np.ctypeslib.as_array(C.cast(data, C.POINTER(C.c_uint8)), shape=(nbytes.value,)) if nbytes.value else np.empty(0, np.uint8)
+        return ty.value, tuple(dims[i] for i in range(nd.value)), raw
+
+    def get_u32(self, key: str):
+        v = C.c_uint32()
+        return None if lib().ksh_gguf_get_u32(self.h, key.encode(), C.byref(v)) else v.value
+
+    def get_f32(self, key: str):
+        v = C.c_float()
+        return None if lib().ksh_gguf_get_f32(self.h, key.encode(), C.byref(v)) else v.value
+
+    def get_str(self, key: str):
+        buf = C.create_string_buffer(4096)
+        return None if lib().ksh_gguf_get_str(self.h, key.encode(), buf, 4096) else buf.value.decode()
+
+    def get_list(self, key: str):
+        n = C.c_int()
+        if lib().ksh_gguf_get_arr_u32(self.h, key.encode(), None, 0, C.byref(n)):
+            return None
+        arr = (C.c_uint32 * max(1, n.value))()
+        lib().ksh_gguf_get_arr_u32(self.h, key.encode(), arr, n.value, C.byref(n))
+        vals = list(arr[:n.value])
+        return [bool(v) for v in vals] if lib().ksh_gguf_arr_is_bool(self.h, key.encode()) else vals
+
+    def gemma4_config(self, max_seq: int):
+        """GemmaConfig::from_gguf: (cfg dict, ffn per layer, is_swa per layer)."""
+        c = Gemma4Cfg()
+        ffn, swa = (C.c_int32 * 4096)(), (C.c_int32 * 4096)()
+        _check(lib().ksh_gemma4_config_from_gguf(self.h, max_seq, C.byref(c), ffn, swa, 4096))
+        cfg = {k: getattr(c, k) for k in GEMMA4_CFG_INTS + GEMMA4_CFG_FLOATS}
+        return cfg, list(ffn[:c.n_layers]), [bool(v) for v in swa[:c.n_layers]]
+
+
+def gguf_dequant_host(ggml_type: int, raw: np.ndarray, n: int) -> np.ndarray:
+    raw = np.ascontiguousarray(raw, dtype=np.uint8)
+    out = np.empty(n, dtype=np.float32)
+    _check(lib().ksh_gguf_dequant_host(int(ggml_type), raw.ctypes.data, n, out.ctypes.data))
+    return out
+
+
 class Gemma4:
     """GemmaPrimModel with the layer features of the real Gemma-4 checkpoints
     (crates/ksearch_gemma/src/gemma_prim.rs:881-1275; crates/ksearch_gemma/src/lib.rs:39-167).
@@ -794,6 +905,19 @@ class Gemma4:
         h = C.c_void_p()
         _check(lib().ksh_gemma4_create(ctx.h, C.byref(c), arr, C.byref(g), C.byref(h)))
         self.h = h
+
+    @classmethod
+    def from_gguf(cls, ctx: Context, gguf: "Gguf", max_seq: int, keep_q6k: bool = False) -> "Gemma4":
+        """GemmaPrimModel's load path: every tensor of the file onto the device, in the forms the loop takes."""
+        self = cls.__new__(cls)
+        self.ctx, self._bufs = ctx, []
+        h = C.c_void_p()
+        _check(lib().ksh_gemma4_load_gguf(ctx.h, gguf.h, max_seq, LOAD_KEEP_Q6K if keep_q6k else 0, C.byref(h)))
+        self.h = h
+        c = Gemma4Cfg()
+        _check(lib().ksh_gemma4_config(h, C.byref(c)))
+        self.cfg = {k: getattr(c, k) for k in GEMMA4_CFG_INTS + GEMMA4_CFG_FLOATS}
+        return self
 
     def close(self):
         if self.h:

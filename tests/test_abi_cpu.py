@@ -36,6 +36,10 @@ def test_enums_match_header():
             assert hip.DType[name] == val
         elif name in hip.Kind.__members__:
             assert hip.Kind[name] == val
+        elif name.startswith("GGML_"):
+            assert hip.GgmlType[name[5:]] == val
+        elif name == "LOAD_KEEP_Q6K":
+            assert hip.LOAD_KEEP_Q6K == val
         else:
             raise AssertionError(f"KSH_{name} has no Python counterpart")
 
@@ -45,6 +49,9 @@ def test_struct_sizes():
     assert C.sizeof(hip.KernelDesc) == 4 + 16 + 4 + 64 + 16 + 32     # kind, dtypes, pad, dims, params, sched
     assert C.sizeof(hip.GemmaCfg) == 48
     assert C.sizeof(hip.GemmaLayer) == 13 * 8
+    assert C.sizeof(hip.Gemma4Cfg) == 11 * 4 + 6 * 4
+    assert C.sizeof(hip.Gemma4Layer) == 11 * 4 + 4 + 16 * 8 + 8          # ints, pad, pointers, scale + tail pad
+    assert C.sizeof(hip.Gemma4Globals) == 8 * 8
 
 
 def test_context_fails_loudly_without_gpu():

@@ -195,3 +195,92 @@ def test_gemma4_create_errors(ctx):
     bad = dict(w, layers=[dict(w["layers"][0], dt_q=int(DType.Q5K))] + w["layers"][1:])
     with pytest.raises(hip.KshError, match="weight dtype"):
         hip.Gemma4(ctx, cfg, bad)
+
+
+def test_gemma4_from_gguf_matches_oracle(ctx, tmp_path):
+    """A GGUF file with the tensor names, types and metadata keys of the real checkpoints: Q4_K and Q6_K
+    matrices, f32 norms, an f32 per-layer model projection (scaled by 1/sqrt(hidden) and packed at load), an f16
+    per-layer gate and a bf16 projection (packed at load), a Q5_K per-layer table, a Q6_K ffn_down (requantized
+    to Q4_K like the reference does) beside a Q6_K attn_q (kept).  The oracle gets the same tensors converted by
+    the host routines."""
+    from tests import gguf_writer as gw
+    from ksearch_amd.hip import GgmlType
+    cfg = dict(synth.GEMMA4_TINY)
+    n, h, pd = cfg["n_layers"], cfg["hidden"], cfg["ple_dim"]
+    w = synth.gemma4_weights(cfg, 620, oracle.quantize_q4k, oracle.quantize_q6k, ffn=FFN, swa_pattern=PATTERN,
+                             q6k_tensors={(2, "wdown"), (3, "wq")}, std=0.05)
+    rng = np.random.default_rng(621)
+    names = dict(wq="attn_q", wk="attn_k", wv="attn_v", wo="attn_output", wgate="ffn_gate", wup="ffn_up", wdown="ffn_down",
+                 attn_norm="attn_norm", q_norm="attn_q_norm", k_norm="attn_k_norm", post_attn_norm="post_attention_norm", ffn_norm="ffn_norm",
+                 post_ffw_norm="post_ffw_norm", post_norm="post_norm")
+    dt2ggml = {oracle.Q4K: GgmlType.Q4_K, oracle.Q6K: GgmlType.Q6_K}
+    tensors = []
+    for i, lw in enumerate(w["layers"]):
+        hd = cfg["hd_swa"] if lw["is_swa"] else cfg["hd_full"]
+        cols = dict(wq=h, wk=h, wv=h, wo=cfg["n_q"] * hd, wgate=h, wup=h, wdown=lw["ffn"])
+        for key, dtk in (("wq", "dt_q"), ("wk", "dt_k"), ("wv", "dt_v"), ("wo", "dt_o"), ("wgate", "dt_gate"), ("wup", "dt_up"), ("wdown", "dt_down")):
+            if key not in lw:
+                continue
+            blk = 144 if lw[dtk] == oracle.Q4K else 210
+            rows = lw[key].size // blk * 256 // cols[key]
+            tensors.append((f"blk.{i}.{names[key]}.weight", dt2ggml[lw[dtk]], (cols[key], rows), lw[key]))
+        for key in ("attn_norm", "q_norm", "k_norm", "post_attn_norm", "ffn_norm", "post_ffw_norm", "post_norm"):
+            tensors.append((f"blk.{i}.{names[key]}.weight", GgmlType.F32, (lw[key].size,), lw[key]))
+        tensors.append((f"blk.{i}.layer_output_scale.weight", GgmlType.F32, (1,), np.array([lw["layer_scale"]], np.float32)))
+        # per-layer gate in f16, projection in bf16: both are packed to Q4_K by the loader
+        gate = (rng.standard_normal(pd * h) * 0.05).astype(np.float16)
+        proj32 = (rng.standard_normal(h * pd) * 0.05).astype(np.float32)
+        proj = (proj32.view(np.uint32) >> 16).astype(np.uint16)
+        tensors.append((f"blk.{i}.inp_gate.weight", GgmlType.F16, (h, pd), gate))
+        tensors.append((f"blk.{i}.proj.weight", GgmlType.BF16, (pd, h), proj))
+        lw["inp_gate"], lw["dt_inp_gate"] = oracle.quantize_q4k(gate.astype(np.float32)), oracle.Q4K
+        lw["proj"], lw["dt_proj"] = oracle.quantize_q4k((proj.astype(np.uint32) << 16).view(np.float32)), oracle.Q4K
+        if lw["dt_down"] == oracle.Q6K:      # gemma_prim.rs:418-433
+            lw["wdown"], lw["dt_down"] = oracle.quantize_q4k(oracle.dequant(oracle.Q6K, lw["wdown"], h * lw["ffn"])), oracle.Q4K
+    g = w["globals"]
+    pt = n * pd
+    model_proj = (rng.standard_normal(pt * h) * 0.05).astype(np.float32)
+    tensors += [("token_embd.weight", GgmlType.Q6_K, (h, cfg["vocab"]), g["token_embd"]), ("output_norm.weight", GgmlType.F32, (h,), g["output_norm"]),
+                ("per_layer_token_embd.weight", GgmlType.Q5_K, (pt, cfg["vocab"]), g["ple_embd"]),
+                ("per_layer_model_proj.weight", GgmlType.F32, (h, pt), model_proj),
+                ("per_layer_proj_norm.weight", GgmlType.F32, (pd,), g["ple_proj_norm"])]
+    g["ple_model_proj"] = oracle.quantize_q4k(model_proj * np.float32(1.0 / np.sqrt(np.float32(h))))      # :341-352
+    meta = [("general.architecture", gw.STR, "gemma4"), ("gemma4.block_count", gw.U32, n), ("gemma4.embedding_length", gw.U32, h),
+            ("gemma4.attention.head_count", gw.U32, cfg["n_q"]), ("gemma4.attention.head_count_kv", gw.U32, cfg["n_kv"]),
+            ("gemma4.attention.key_length", gw.U32, cfg["hd_full"]), ("gemma4.attention.key_length_swa", gw.U32, cfg["hd_swa"]),
+            ("gemma4.attention.sliding_window", gw.U32, cfg["sliding_window"]), ("gemma4.attention.shared_kv_layers", gw.U32, cfg["shared_kv_layers"]),
+            ("gemma4.embedding_length_per_layer_input", gw.U32, pd), ("gemma4.feed_forward_length", gw.ARR, (gw.U32, FFN)),
+            ("gemma4.attention.sliding_window_pattern", gw.ARR, (gw.BOOL, PATTERN))]
+    path = str(tmp_path / "tiny.gguf")
+    gw.write(path, meta, tensors)
+    with hip.Gguf(path) as f:
+        gpu = hip.Gemma4.from_gguf(ctx, f, cfg["max_seq"])
+    for k in ("n_layers", "hidden", "vocab", "hd_swa", "hd_full", "sliding_window", "shared_kv_layers", "ple_dim", "attn_scale"):
+        assert gpu.cfg[k] == cfg[k], k
+    cpu = oracle.Gemma4(cfg, w)
+    prompt = [int(t) for t in np.random.default_rng(622).integers(0, cfg["vocab"], 5)]
+    got, _, _ = gpu.generate(prompt, 24, use_graph=True)
+    for t in prompt[:-1]:
+        cpu.forward(t, want_logits=False)
+    want, tok, margins = [], prompt[-1], []
+    for _ in range(24):
+        tok, logits = cpu.forward(tok, return_logits=True)
+        want.append(tok)
+        top2 = np.sort(logits)[-2:]
+        margins.append((top2[1] - top2[0]) / max(abs(top2[1]), 1e-6))
+    first_close = next((i for i, mg in enumerate(margins) if mg < 1e-3), 24)
+    assert got[:first_close] == want[:first_close] and first_close >= 8
+    gpu.close()
+    cpu.close()
+    # the same file with the Q6_K ffn_down kept: a different (closer) model, so not the reference's tokens in general,
+    # but the loader must take it
+    with hip.Gguf(path) as f:
+        kept = hip.Gemma4.from_gguf(ctx, f, cfg["max_seq"], keep_q6k=True)
+    assert len(kept.generate(prompt, 4, use_graph=False)[0]) == 4
+    kept.close()
+    # a tensor whose shape contradicts the metadata
+    bad = [(nm, ty, ((dims[0], dims[1] - 1) if nm == "blk.0.attn_q.weight" else dims), (raw[:-(h // 256 * 144)] if nm == "blk.0.attn_q.weight" else raw))
+           for nm, ty, dims, raw in tensors]
+    gw.write(path, meta, bad)
+    with hip.Gguf(path) as f, pytest.raises(hip.KshError, match="blk.0.attn_q.weight is"):
+        hip.Gemma4.from_gguf(ctx, f, cfg["max_seq"])

@@ -121,7 +121,9 @@ enum ksh_kind {
      *   has_residual = 1: in: W.., y, w_norm, w_post, res    out: y.., x_new
      *     with x_new = res + rms(y)*w_post (RmsNormAdd, the new residual stream,
      *     which must not alias res) and the GEMV input rms(x_new)*w_norm
-     *     (RmsNormAddThenRmsNorm, kernel.rs:474-481, folded into its consumer). */
+     *     (RmsNormAddThenRmsNorm, kernel.rs:474-481, folded into its consumer).
+     *     params[1] != 0: x_new = params[1] * (res + rms(y)*w_post) (RmsNormAddScale: the
+     *     per-layer-embedding block's closing op, folded in the same way). */
     KSH_RMSNORM_MATVEC = 19,
     KSH_RMSNORM_MATVEC_QKV = 20,
     KSH_RMSNORM_MATVEC_GATE_UP_GELU = 21,
@@ -166,7 +168,11 @@ enum ksh_kind {
     KSH_ADD_SCALE = 26,
     /* Eng::matvec_gelu_mul_at (crates/ksearch_kernels/src/lib.rs:791-822): y[r] = gelu(W[r].x) * ctx[r], the
      * per-layer-embedding gate; the context slice is placed with a byte offset.
-     * dims: rows, cols.  dtypes: Q4K, F32.  in: W, x, ctx f32[rows]   out: y */
+     * dims: rows, cols (<= 8192), has_residual.  dtypes: Q4K, F32.  params: eps (has_residual).
+     *   has_residual = 0: in: W, x, ctx f32[rows]                 out: y
+     *   has_residual = 1: in: W, y_prev, ctx, w_post, res         out: y, x_new
+     *     with x_new = res + rms(y_prev)*w_post (the RmsNormAdd that closes the feed-forward block, folded in;
+     *     x_new must not alias res) and the GEMV input x_new */
     KSH_MATVEC_GELU_MUL = 27,
     KSH_KIND_COUNT
 };

@@ -6,11 +6,11 @@
 // Mirrors GemmaPrimModel::forward_token (crates/ksearch_gemma/src/gemma_prim.rs:
 // 881-1275) with GemmaConfig's layer rules (crates/ksearch_gemma/src/lib.rs:
 // 136-167).  As in the loop for the synthetic shape, norms ride in the GEMV that
-// consumes them wherever a fused kind is built for the weight types at hand, the
-// position lives on the device and a token is one HIP graph.  The layer-closing
-// residual add stays "pending" (y, norm weight) until its consumer folds it in;
-// where no fused consumer exists (per-layer embeddings scale the stream) it is
-// materialised with the RmsNorm kind.
+// consumes them, the position lives on the device and a token is one HIP graph.
+// A residual add stays "pending" (y, norm weight) until the next GEMV folds it
+// into its prologue: the feed-forward block's into the per-layer-embedding gate,
+// the layer-closing one (with the layer's output scale) into the next layer's
+// QKV or the LM head.
 #include <chrono>
 #include <cmath>
 #include <cstdlib>
@@ -72,7 +72,7 @@ struct LayerPlan {
     ksh_kernel *oproj = nullptr;
     ksh_kernel *gate_up = nullptr, *gate = nullptr, *up = nullptr, *gelu = nullptr;
     ksh_kernel *down = nullptr;
-    ksh_kernel *ple_gate = nullptr, *ple_proj = nullptr, *ple_close = nullptr;
+    ksh_kernel *ple_gate = nullptr, *ple_proj = nullptr;
 };
 
 }  // namespace
@@ -91,7 +91,7 @@ struct ksh_gemma4 {
             *history = nullptr, *ple_tok = nullptr, *ple_tmp = nullptr, *ple_ctx = nullptr, *ple_u = nullptr;
     std::vector<ksh_buf *> kv_k, kv_v;   // per layer; null where the layer reads another layer's cache
     ksh_kernel *k_embed = nullptr, *k_ple_gather = nullptr, *k_ple_proj = nullptr, *k_ple_norm = nullptr, *k_ple_mix = nullptr,
-               *k_close = nullptr, *k_lm_head[2] = {nullptr, nullptr}, *k_argmax = nullptr;
+               *k_lm_head[2] = {nullptr, nullptr}, *k_argmax = nullptr;
     ksh_graph *g_body = nullptr, *g_full = nullptr;
     std::vector<float> rope0_full, rope0_swa;
     int pos = 0, launches_full = 0;
@@ -181,16 +181,6 @@ int enc_norm_gemv(ksh_gemma4 *m, ksh_kernel *const k[2], std::initializer_list<k
     return ksh_encode(m->ctx, k[0], ib, nullptr, ni, ob, nullptr, no);
 }
 
-// writes a pending add out: cur <- (cur + rms(y)*w) [* scale]
-int materialise(ksh_gemma4 *m, Stream &s, ksh_kernel *k, int &n)
-{
-    if (!s.y) return 0;
-    if (enc(m, k, {s.y, s.w, s.cur}, {s.other}, n)) return 1;
-    std::swap(s.cur, s.other);
-    s.y = s.w = nullptr;
-    return 0;
-}
-
 int encode_token(ksh_gemma4 *m, bool want_logits, int &launches)
 {
     const ksh_gemma4_cfg &c = m->c;
@@ -252,13 +242,16 @@ int encode_token(ksh_gemma4 *m, bool want_logits, int &launches)
         s.y = m->y;
         s.w = L.post_ffw_norm;
         if (c.ple_dim > 0) {
-            // gemma_prim.rs:1166-1200: x += rms(down)*post_ffw_norm; u = gelu(Wg x) * ctx_l; x = (x + rms(Wp u)*post_norm) * scale
-            if (materialise(m, s, m->k_close, launches)) return 1;
-            if (enc_off(m, P.ple_gate, {L.inp_gate, s.cur, m->ple_ctx}, {0, 0, (size_t)l * c.ple_dim * 4}, {m->ple_u}, launches) ||
-                enc(m, P.ple_proj, {L.proj, m->ple_u}, {m->y}, launches) ||
-                enc(m, P.ple_close, {m->y, L.post_norm, s.cur}, {s.other}, launches))
+            // gemma_prim.rs:1150-1200: x += rms(down)*post_ffw_norm; u = gelu(Wg x) * ctx_l; x = (x + rms(Wp u)*post_norm) * scale.
+            // The first add rides in the gate GEMV; the last one stays pending, with the scale, for the next layer's
+            // QKV (or the LM head).
+            if (enc_off(m, P.ple_gate, {L.inp_gate, s.y, m->ple_ctx, s.w, s.cur}, {0, 0, (size_t)l * c.ple_dim * 4, 0, 0}, {m->ple_u, s.other},
+                        launches))
                 return 1;
             std::swap(s.cur, s.other);
+            if (enc(m, P.ple_proj, {L.proj, m->ple_u}, {m->y}, launches)) return 1;
+            s.y = m->y;
+            s.w = L.post_norm;
         }
     }
     if (want_logits) {
@@ -367,12 +360,15 @@ int plan_layer(ksh_gemma4 *m, int l)
     if (L.ffn <= 0 || L.ffn % 256) return set_error("layer %d: ffn=%d is not a positive multiple of 256", l, L.ffn);
 
     P.fused_qkv = P.owns && L.dt_q == KSH_Q4K && L.dt_k == KSH_Q4K && L.dt_v == KSH_Q4K;
+    // the add that this layer's first GEMV folds in closes the previous layer: with per-layer embeddings it carries
+    // that layer's output scale
+    const float prev_scale = c.ple_dim > 0 && l > 0 ? m->layers[l - 1].layer_scale : 0.f;
     if (P.fused_qkv) {
         for (int r = 0; r < 2; r++)
-            if (get(m, KSH_RMSNORM_MATVEC_QKV, {P.qd, P.kvd, h, r}, {KSH_Q4K, KSH_F32}, {c.eps}, &P.qkv[r])) return 1;
+            if (get(m, KSH_RMSNORM_MATVEC_QKV, {P.qd, P.kvd, h, r}, {KSH_Q4K, KSH_F32}, {c.eps, r ? prev_scale : 0.f}, &P.qkv[r])) return 1;
     } else {
         for (int r = 0; r < 2; r++)
-            if (get(m, KSH_RMSNORM_MATVEC, {P.qd, h, r}, {L.dt_q, KSH_F32}, {c.eps}, &P.qkv[r])) return 1;
+            if (get(m, KSH_RMSNORM_MATVEC, {P.qd, h, r}, {L.dt_q, KSH_F32}, {c.eps, r ? prev_scale : 0.f}, &P.qkv[r])) return 1;
         if (P.owns && (get(m, KSH_RMSNORM_MATVEC, {P.kvd, h, 0}, {L.dt_k, KSH_F32}, {c.eps}, &P.kmat[0]) ||
                        get(m, KSH_RMSNORM_MATVEC, {P.kvd, h, 0}, {L.dt_v, KSH_F32}, {c.eps}, &P.kmat[1])))
             return 1;
@@ -407,9 +403,8 @@ int plan_layer(ksh_gemma4 *m, int l)
     if (c.ple_dim > 0) {
         if (L.dt_inp_gate != KSH_Q4K || !packed_ok(L.dt_proj))
             return set_error("layer %d: per-layer-embedding weights must be Q4_K (gate) and Q4_K or Q6_K (projection)", l);
-        if (get(m, KSH_MATVEC_GELU_MUL, {c.ple_dim, h}, {KSH_Q4K, KSH_F32}, {}, &P.ple_gate) ||
-            get(m, KSH_MATVEC, {h, c.ple_dim}, {L.dt_proj, KSH_F32}, {}, &P.ple_proj) ||
-            get(m, KSH_RMSNORM, {h, 1, 1}, {}, {c.eps, L.layer_scale}, &P.ple_close))
+        if (get(m, KSH_MATVEC_GELU_MUL, {c.ple_dim, h, 1}, {KSH_Q4K, KSH_F32}, {c.eps}, &P.ple_gate) ||
+            get(m, KSH_MATVEC, {h, c.ple_dim}, {L.dt_proj, KSH_F32}, {}, &P.ple_proj))
             return 1;
     }
     return 0;
@@ -477,9 +472,9 @@ int ksh_gemma4_create(ksh_ctx *ctx, const ksh_gemma4_cfg *cfg, const ksh_gemma4_
         lm_dt = KSH_Q6K_ROWS;
     }
     if (get(m, KSH_COPY_SCALE_INDEXED, {c.hidden, c.vocab}, {de}, {std::sqrt((float)c.hidden)}, &m->k_embed) ||
-        get(m, KSH_RMSNORM, {c.hidden, 1, 0}, {}, {c.eps, 0.f}, &m->k_close) ||
         get(m, KSH_RMSNORM_MATVEC, {c.vocab, c.hidden, 0}, {lm_dt, KSH_F32}, {c.eps}, &m->k_lm_head[0]) ||
-        get(m, KSH_RMSNORM_MATVEC, {c.vocab, c.hidden, 1}, {lm_dt, KSH_F32}, {c.eps}, &m->k_lm_head[1]) ||
+        get(m, KSH_RMSNORM_MATVEC, {c.vocab, c.hidden, 1}, {lm_dt, KSH_F32}, {c.eps, c.ple_dim > 0 ? m->layers[c.n_layers - 1].layer_scale : 0.f},
+            &m->k_lm_head[1]) ||
         get(m, KSH_SOFTCAP_ARGMAX, {c.vocab}, {}, {c.softcap}, &m->k_argmax))
         return 1;
     if (c.ple_dim > 0) {

@@ -37,7 +37,7 @@ struct Prologue {
     float *x_out;          // kAddThenRms: residual stream out
     float eps;
     int kind;
-    int nwg, hd_log2;      // kMergeParts
+    int nwg, hd_log2;      // kMergeParts.  kAddThenRms: nwg carries the bits of the stream scale s, x_out = s * (res + rms(y) * w_post)
 };
 
 __host__ __device__ constexpr int xs_f32_floats(int cols) { return cols + (cols >> 6) * 4; }
@@ -308,19 +308,20 @@ __device__ __forceinline__ void stage_finish(const Prologue &pr, uint8_t *lds, i
     }
     float inv = 1.0f / sqrtf(acc[0] / (float)cols + pr.eps);
     if (add) {
+        const float sc = __int_as_float(pr.nwg);   // 1 except where per-layer embeddings scale the stream
 #pragma unroll
         for (int k = 0; k < KP; k++) {
             const int i = tid + k * NT;
             if (wbase + k * NT < n4) {
                 const float4 r = s.rs[k], w = s.wp[k];
-                v[k].x = r.x + v[k].x * inv * w.x;
-                v[k].y = r.y + v[k].y * inv * w.y;
-                v[k].z = r.z + v[k].z * inv * w.z;
-                v[k].w = r.w + v[k].w * inv * w.w;
+                v[k].x = (r.x + v[k].x * inv * w.x) * sc;
+                v[k].y = (r.y + v[k].y * inv * w.y) * sc;
+                v[k].z = (r.z + v[k].z * inv * w.z) * sc;
+                v[k].w = (r.w + v[k].w * inv * w.w) * sc;
                 if (blockIdx.x == 0) stg_f4(pr.x_out, i, v[k]);
             }
         }
-        const float ss2 = fmaf(inv * inv, acc[3], fmaf(2.0f * inv, acc[2], acc[1]));
+        const float ss2 = (sc * sc) * fmaf(inv * inv, acc[3], fmaf(2.0f * inv, acc[2], acc[1]));
         inv = 1.0f / sqrtf(ss2 / (float)cols + pr.eps);
     }
 #pragma unroll

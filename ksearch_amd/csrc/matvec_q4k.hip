@@ -331,17 +331,19 @@ __global__ __launch_bounds__(NW * 64) void q4k_gemv_kernel(MatvecParams p_in)
     }
 }
 
-// Half-wave form for rows of exactly 8 superblocks (2048 columns): lanes
-// 0..31 and 32..63 work on different rows, so a wave covers 2R rows in a single
-// step and no lane idles.
-template <int R, int NW, int NM, int XF, bool MERGE>
+// Half-wave form for rows of at most 8 superblocks (BPR = 8: 2048 columns, no lane idles; BPR = 6: 1536 columns,
+// a quarter of the lanes re-read the row's last superblock and drop the product): lanes 0..31 and 32..63 work
+// on different rows, so a wave covers 2R rows in a single step.
+template <int R, int NW, int NM, int XF, bool MERGE, int BPR>
 __global__ __launch_bounds__(NW * 64) void q4k_gemv_half_kernel(MatvecParams p_in)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t xs[];
     const MatvecParams p = fetch_params(p_in);
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int g = lane & 3, bl = (lane >> 2) & 7, hw = lane >> 5;
-    constexpr int bpr = 8;
+    const int g = lane & 3, slot = (lane >> 2) & 7, hw = lane >> 5;
+    constexpr int bpr = BPR;
+    const int bl = BPR == 8 ? slot : min(slot, BPR - 1);
+    const bool mine = BPR == 8 || slot < BPR;
     constexpr size_t row_bytes = (size_t)bpr * kQ4kBytes;
     WaveTask t = wave_task(p, blockIdx.x * NW + wave, 2 * R);
     const int row0 = t.row0 + hw * R;
@@ -379,7 +381,8 @@ __global__ __launch_bounds__(NW * 64) void q4k_gemv_half_kernel(MatvecParams p_i
         float s[NM];
 #pragma unroll
         for (int m = 0; m < NM; m++) {
-            const float2 hs = wave_half_sums(q4k_group_dot<XF>(L[m][r], g, X));
+            const float v = q4k_group_dot<XF>(L[m][r], g, X);
+            const float2 hs = wave_half_sums(mine ? v : 0.f);
             s[m] = hw ? hs.y : hs.x;
         }
         const int row = row0 + r;
@@ -400,8 +403,10 @@ size_t lds_for(int var, int cols) { return var == kXI8 ? xs_bytes<kXI8>(cols) : 
 template <int R, int NW, int NM, int XF, bool MERGE>
 void launch_pro(bool half, const MatvecParams &p, unsigned grid, size_t lds, hipStream_t st)
 {
-    if (half)
-        hipLaunchKernelGGL((q4k_gemv_half_kernel<R, NW, NM, XF, MERGE>), dim3(grid), dim3(NW * 64), lds, st, p);
+    if (half && p.bpr == 8)
+        hipLaunchKernelGGL((q4k_gemv_half_kernel<R, NW, NM, XF, MERGE, 8>), dim3(grid), dim3(NW * 64), lds, st, p);
+    else if (half)
+        hipLaunchKernelGGL((q4k_gemv_half_kernel<R, NW, NM, XF, MERGE, 6>), dim3(grid), dim3(NW * 64), lds, st, p);
     else if (p.bpr > 16)
         hipLaunchKernelGGL((q4k_gemv_kernel<R, NW, NM, XF, true, MERGE>), dim3(grid), dim3(NW * 64), lds, st, p);
     else
@@ -444,7 +449,7 @@ int launch_q4k(const Q4kGeom &G, const MatvecParams &p, int total_waves, hipStre
 Q4kGeom pick_geom(const ksh_sched &s, int total_rows, int bpr)
 {
     Q4kGeom G;
-    G.half = (bpr == 8);
+    G.half = (bpr == 8 || bpr == 6);
     G.var = sched_is_zero(s) ? (bpr > 16 ? kXF32 : kXI8) : (s.vec == 3 ? kXI8 : kXF32);
     if (s.nsg && s.nr0) {
         G.NW = (int)s.nsg;
@@ -562,6 +567,7 @@ int launch_any(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
     }
     if (s.prologue != kPlain) p.pro.w_norm = (const float *)a.in[s.n_mat + 1];
     if (s.prologue == kAddThenRms) {
+        p.pro.nwg = __builtin_bit_cast(int, k.desc.params[1] != 0.f ? k.desc.params[1] : 1.0f);   // the stream scale
         p.pro.w_post = (const float *)a.in[s.n_mat + 2];
         p.pro.res = (const float *)a.in[s.n_mat + 3];
         p.pro.x_out = (float *)a.out[n_y];

@@ -369,6 +369,7 @@ int launch_matvec_q6k(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
     p.pro.kind = k.desc.kind == KSH_MATVEC ? kPlain : (k.desc.dims[2] ? kAddThenRms : kRms);
     if (p.pro.kind != kPlain) p.pro.w_norm = (const float *)a.in[2];
     if (p.pro.kind == kAddThenRms) {
+        p.pro.nwg = __builtin_bit_cast(int, k.desc.params[1] != 0.f ? k.desc.params[1] : 1.0f);   // the stream scale
         p.pro.w_post = (const float *)a.in[3];
         p.pro.res = (const float *)a.in[4];
         p.pro.x_out = (float *)a.out[1];

@@ -86,30 +86,65 @@ __device__ __forceinline__ float gelu_mul_f32(float g, float u)
 
 // y[r] = gelu(W[r].x) * ctx[r], W Q4_K.  A few hundred rows of a few thousand
 // columns: one wave per row, four lanes per superblock (one 64-element group
-// each), the vector read straight from the cache.
+// each).  The vector is staged in LDS once per workgroup; with HAS_RES the
+// workgroup first closes the feed-forward block itself,
+//   x = res + rms(y) * w_post      (RmsNormAdd, gemma_prim.rs:1150-1160)
+// and workgroup 0 writes the new residual stream out.  The first superblock's
+// weight loads are issued ahead of the staging.
 constexpr int kGmWaves = 4;
 
+template <bool HAS_RES>
 __global__ __launch_bounds__(kGmWaves * 64) void q4k_gemv_gelu_mul_kernel(const uint8_t *__restrict__ W,
                                                                          const float *__restrict__ x,
                                                                          const float *__restrict__ ctx, float *y,
-                                                                         int rows, int bpr)
+                                                                         int rows, int bpr, const float *__restrict__ w_post,
+                                                                         const float *__restrict__ res, float *x_out, float eps)
 {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int row = blockIdx.x * kGmWaves + wave;
-    if (row >= rows) return;
-    const int g = lane & 3;
+    extern __shared__ __attribute__((aligned(16))) float xs[];
+    __shared__ float red[kGmWaves];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int row = min(blockIdx.x * kGmWaves + wave, rows - 1);   // (a wave past the end repeats the last row: same barriers)
+    const int g = lane & 3, cols = bpr * 256;
     const uint8_t *wr = W + (size_t)row * bpr * 144;
+    const int b0 = min(lane >> 2, bpr - 1);
+    const uint8_t *blk0 = wr + (size_t)b0 * 144;
+    uint4 hdr = ldg_u4(blk0, 0), q0 = ldg_u4(blk0 + 16 + 32 * g, 0), q1 = ldg_u4(blk0 + 16 + 32 * g, 1);
+
+    if (HAS_RES) {
+        float ss = 0.f;
+        for (int i = tid; i < cols / 4; i += kGmWaves * 64) {
+            const float4 v = ldg_f4(x, i);
+            ss += (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w);
+        }
+        ss = wave_sum(ss);
+        if (lane == 0) red[wave] = ss;
+        __syncthreads();
+        const float inv = 1.0f / sqrtf(((red[0] + red[1]) + (red[2] + red[3])) / (float)cols + eps);
+        for (int i = tid; i < cols / 4; i += kGmWaves * 64) {
+            const float4 v = ldg_f4(x, i), w = ldg_f4(w_post, i), r = ldg_f4(res, i);
+            const float4 o = make_float4(r.x + v.x * inv * w.x, r.y + v.y * inv * w.y, r.z + v.z * inv * w.z, r.w + v.w * inv * w.w);
+            *reinterpret_cast<float4 *>(xs + 4 * i + (i >> 4) * 4) = o;   // four floats of padding per 64: the groups of a wave land on distinct banks
+            if (blockIdx.x == 0) stg_f4(x_out, i, o);
+        }
+    } else {
+        for (int i = tid; i < cols / 4; i += kGmWaves * 64) *reinterpret_cast<float4 *>(xs + 4 * i + (i >> 4) * 4) = ldg_f4(x, i);
+    }
+    __syncthreads();
+
     float acc = 0.f;
     for (int b = lane >> 2; b < bpr; b += 16) {
-        const uint8_t *blk = wr + (size_t)b * 144;
-        const uint4 hdr = ldg_u4(blk, 0);
-        const uint4 q0 = ldg_u4(blk + 16 + 32 * g, 0), q1 = ldg_u4(blk + 16 + 32 * g, 1);
+        if (b != b0) {
+            const uint8_t *blk = wr + (size_t)b * 144;
+            hdr = ldg_u4(blk, 0);
+            q0 = ldg_u4(blk + 16 + 32 * g, 0);
+            q1 = ldg_u4(blk + 16 + 32 * g, 1);
+        }
         const uint32_t qw[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
-        const float *xg = x + (size_t)b * 256 + 64 * g;
+        const float4 *xg = reinterpret_cast<const float4 *>(xs + (size_t)b * 256 + 64 * g + (4 * b + g) * 4);
         float lo = 0.f, hi = 0.f, sl = 0.f, sh = 0.f;
 #pragma unroll
         for (int k = 0; k < 8; k++) {
-            const float4 a = ldg_f4(xg, k), c = ldg_f4(xg + 32, k);
+            const float4 a = xg[k], c = xg[8 + k];
             const uint32_t v = qw[k];
             lo += (float)(v & 15u) * a.x + (float)((v >> 8) & 15u) * a.y + (float)((v >> 16) & 15u) * a.z +
                   (float)((v >> 24) & 15u) * a.w;
@@ -123,7 +158,7 @@ __global__ __launch_bounds__(kGmWaves * 64) void q4k_gemv_gelu_mul_kernel(const 
         acc += d * ((float)s.x * lo + (float)s.z * hi) - dmin * ((float)s.y * sl + (float)s.w * sh);
     }
     acc = wave_sum(acc);
-    if (lane == 0) y[row] = gelu_mul_f32(acc, ctx[row]);
+    if (lane == 0 && blockIdx.x * kGmWaves + wave < rows) y[row] = gelu_mul_f32(acc, ctx[row]);
 }
 
 int launch_per_head(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
@@ -155,8 +190,15 @@ int launch_add_scale(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
 int launch_gelu_mul_gemv(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
 {
     const int rows = (int)k.desc.dims[0], bpr = (int)(k.desc.dims[1] / 256);
-    hipLaunchKernelGGL(q4k_gemv_gelu_mul_kernel, dim3((rows + kGmWaves - 1) / kGmWaves), dim3(kGmWaves * 64), 0, st,
-                       (const uint8_t *)a.in[0], (const float *)a.in[1], (const float *)a.in[2], (float *)a.out[0], rows, bpr);
+    const dim3 grid((rows + kGmWaves - 1) / kGmWaves), block(kGmWaves * 64);
+    const size_t lds = (size_t)(k.desc.dims[1] + k.desc.dims[1] / 64 * 4) * 4;
+    if (k.desc.dims[2])
+        hipLaunchKernelGGL(q4k_gemv_gelu_mul_kernel<true>, grid, block, lds, st, (const uint8_t *)a.in[0], (const float *)a.in[1],
+                           (const float *)a.in[2], (float *)a.out[0], rows, bpr, (const float *)a.in[3], (const float *)a.in[4],
+                           (float *)a.out[1], k.desc.params[0]);
+    else
+        hipLaunchKernelGGL(q4k_gemv_gelu_mul_kernel<false>, grid, block, lds, st, (const uint8_t *)a.in[0], (const float *)a.in[1],
+                           (const float *)a.in[2], (float *)a.out[0], rows, bpr, nullptr, nullptr, nullptr, 0.f);
     return done("matvec_gelu_mul launch");
 }
 
@@ -204,15 +246,18 @@ int bind_ple_ops(ksh_kernel &k)
         if (k.desc.dtypes[1] != KSH_F32 && k.desc.dtypes[1] != 0)
             return set_error("matvec_gelu_mul: activation dtype %d is not built (f32 only)", k.desc.dtypes[1]);
         if (rows <= 0 || rows > (1 << 24)) return set_error("matvec_gelu_mul: rows=%lld", (long long)rows);
-        if (cols <= 0 || cols % 256 || cols > (1 << 20)) return set_error("matvec_gelu_mul: cols=%lld is not a positive multiple of 256", (long long)cols);
-        k.info.n_inputs = 3;
-        k.info.n_outputs = 1;
+        if (cols <= 0 || cols % 256 || cols > 8192) return set_error("matvec_gelu_mul: cols=%lld is not a positive multiple of 256 up to 8192", (long long)cols);
+        const bool has_res = d[2] != 0;
+        k.info.n_inputs = has_res ? 5 : 3;
+        k.info.n_outputs = has_res ? 2 : 1;
+        k.in_bytes[3] = k.in_bytes[4] = k.out_bytes[1] = (size_t)cols * 4;
+        k.in_align[3] = k.in_align[4] = k.out_align[1] = 16;
         k.in_bytes[0] = (size_t)rows * (cols / 256) * 144; k.in_align[0] = 16;
         k.in_bytes[1] = (size_t)cols * 4; k.in_align[1] = 16;
         k.in_bytes[2] = (size_t)rows * 4; k.in_align[2] = 4;
         k.out_bytes[0] = (size_t)rows * 4; k.out_align[0] = 4;
-        set_launch(k, (uint32_t)((rows + kGmWaves - 1) / kGmWaves), 1, 1, kGmWaves * 64, 0);
-        set_name(k, "matvec_gelu_mul_q4k");
+        set_launch(k, (uint32_t)((rows + kGmWaves - 1) / kGmWaves), 1, 1, kGmWaves * 64, (uint32_t)(cols + cols / 64 * 4) * 4);
+        set_name(k, "%smatvec_gelu_mul_q4k", has_res ? "addrms_" : "");
         k.launch = launch_gelu_mul_gemv;
         return 0;
     }

@@ -89,6 +89,39 @@ def test_add_scale_and_matvec_gelu_mul(ctx, eng):
         ctx.compile(hip.make_desc(Kind.MATVEC_GELU_MUL, (256, 2048), (DType.Q6K, DType.F32)))
 
 
+def test_matvec_gelu_mul_closes_the_feed_forward_block(ctx, eng):
+    """has_residual = 1: the gate GEMV computes x = res + rms(y)*w_post itself, multiplies against it and writes it."""
+    rng = np.random.default_rng(605)
+    for rows, cols in ((256, 1536), (256, 2048), (12, 512)):
+        w = synth.q4k_blocks(rows * cols // 256, 606)
+        y, res = (rng.standard_normal(cols) * 3).astype(np.float32), rng.standard_normal(cols).astype(np.float32)
+        w_post = (1 + 0.2 * rng.standard_normal(cols)).astype(np.float32)
+        cvec = rng.standard_normal(rows).astype(np.float32)
+        u, x_new = ctx.buffer_empty_f32(rows), ctx.buffer_empty_f32(cols)
+        k = eng._k(ctx, Kind.MATVEC_GELU_MUL, (rows, cols, 1), (DType.Q4K, DType.F32), (1e-6,))
+        ctx.encode_multi(k, [ctx.buffer_bytes(w), ctx.buffer_f32(y), ctx.buffer_f32(cvec), ctx.buffer_f32(w_post), ctx.buffer_f32(res)], [u, x_new])
+        want_x = oracle.rmsnorm(y, w_post, 1e-6, res=res)
+        assert_close(ctx.read_f32(x_new, cols), want_x, 1e-5, "x_new")
+        assert_close(ctx.read_f32(u, rows), oracle.matvec_gelu_mul(oracle.Q4K, w, rows, cols, want_x, cvec), 1e-3, f"{rows}x{cols}")
+
+
+@pytest.mark.parametrize("wdt", [DType.Q4K, DType.Q6K])
+def test_rmsnorm_matvec_stream_scale(ctx, eng, wdt):
+    """params[1]: the folded-in add is RmsNormAddScale, x_new = scale * (res + rms(y)*w_post)."""
+    rng = np.random.default_rng(607)
+    rows, cols, scale = 512, 1536, 0.625
+    w = (synth.q4k_blocks if wdt == DType.Q4K else synth.q6k_blocks)(rows * cols // 256, 608)
+    y, res = (rng.standard_normal(cols) * 2).astype(np.float32), rng.standard_normal(cols).astype(np.float32)
+    w_norm, w_post = ((1 + 0.2 * rng.standard_normal(cols)).astype(np.float32) for _ in range(2))
+    out, x_new = ctx.buffer_empty_f32(rows), ctx.buffer_empty_f32(cols)
+    k = eng._k(ctx, Kind.RMSNORM_MATVEC, (rows, cols, 1), (wdt, DType.F32), (1e-6, scale))
+    ctx.encode_multi(k, [ctx.buffer_bytes(w), ctx.buffer_f32(y), ctx.buffer_f32(w_norm), ctx.buffer_f32(w_post), ctx.buffer_f32(res)], [out, x_new])
+    want_x = oracle.rmsnorm(y, w_post, 1e-6, res=res, scale=scale)
+    assert_close(ctx.read_f32(x_new, cols), want_x, 1e-5, "x_new")
+    want = oracle.matvec(int(wdt), w, rows, cols, oracle.rmsnorm(want_x, w_norm, 1e-6))
+    assert_close(ctx.read_f32(out, rows), want, 1e-3, "y")
+
+
 PATTERN = [1, 1, 0, 1, 1, 1, 0, 1]
 FFN = [1024, 1024, 2048, 1024, 1024, 1024, 2048, 1024]
 

@@ -103,6 +103,19 @@ def test_matvec_q4k_unit_vectors_recover_weights(ctx, eng):
         assert np.allclose(ctx.read_f32(by, rows), wd[:, j], rtol=1e-6, atol=1e-9), j
 
 
+def test_matvec_q4k_1536_columns_unit_vectors(ctx, eng):
+    # rows of six superblocks go through the half-wave form with a quarter of the lanes masked
+    rows, cols = 9, 1536
+    w = synth.q4k_blocks(rows * cols // 256, seed=4)
+    wd = oracle.dequant(oracle.Q4K, w, rows * cols).reshape(rows, cols)
+    bw, by = ctx.buffer_bytes(w), ctx.buffer_empty_f32(rows)
+    for j in [0, 31, 32, 63, 64, 255, 256, 1279, 1280, 1535]:
+        e = np.zeros(cols, dtype=np.float32)
+        e[j] = 1.0
+        eng.matvec_wd(ctx, rows, cols, DType.Q4K, bw, ctx.buffer_f32(e), by)
+        assert np.allclose(ctx.read_f32(by, rows), wd[:, j], rtol=1e-6, atol=1e-9), j
+
+
 def test_matvec_offsets_and_errors(ctx, eng):
     rows, cols = 64, 512
     w = synth.q4k_blocks(rows * cols // 256, seed=9)
@@ -205,7 +218,7 @@ def test_lm_head_cfg1_full_size_with_argmax(ctx, eng):
         assert int(ctx.read_f32(bi, 1)[0]) == oracle.softcap_argmax(want, 30.0)
 
 
-@pytest.mark.parametrize("q_rows,kv_rows,cols", [(2048, 256, 2048), (512, 256, 4096), (100, 36, 1024)])
+@pytest.mark.parametrize("q_rows,kv_rows,cols", [(2048, 256, 2048), (512, 256, 4096), (100, 36, 1024), (2048, 256, 1536), (77, 19, 1536)])
 def test_matvec_qkv(ctx, eng, q_rows, kv_rows, cols):
     ws = [synth.q4k_blocks(r * cols // 256, seed=20 + i) for i, r in enumerate((q_rows, kv_rows, kv_rows))]
     x = synth.normal_f32(cols, seed=23)
@@ -216,7 +229,7 @@ def test_matvec_qkv(ctx, eng, q_rows, kv_rows, cols):
         assert_close(ctx.read_f32(o, r), oracle.matvec(oracle.Q4K, w, r, cols, x), TOL, f"qkv {r}")
 
 
-@pytest.mark.parametrize("rows,cols", [(8192, 2048), (100, 4096), (64, 512)])
+@pytest.mark.parametrize("rows,cols", [(8192, 2048), (100, 4096), (64, 512), (6144, 1536), (45, 1536)])
 def test_matvec_gate_up_gelu(ctx, eng, rows, cols):
     wg = synth.q4k_blocks(rows * cols // 256, seed=30)
     wu = synth.q4k_blocks(rows * cols // 256, seed=31)

@@ -260,7 +260,9 @@ int encode_token(ksh_gemma4 *m, bool want_logits, int &launches)
         if (enc(m, m->k_argmax, {m->logits}, {m->tok}, launches)) return 1;
         launches += 1;   // two passes
     }
-    m->hidden = s.cur;   // (a pending add of the last layer of a logits-free token is never needed)
+    // (a pending add of the last layer of a logits-free token is never needed, and the test hook follows the
+    // tokens that produce logits: the two captured graphs end in different buffers)
+    if (want_logits) m->hidden = s.cur;
     hipStream_t st = (hipStream_t)ksh_stream(m->ctx);
     hipLaunchKernelGGL(advance4_kernel, dim3(1), dim3(64), 0, st, (float *)ksh_buffer_device_ptr(m->meta_full),
                        (float *)ksh_buffer_device_ptr(m->meta_swa), (const float *)ksh_buffer_device_ptr(m->tok),

@@ -141,25 +141,20 @@ def tiny(ctx, request):
     cpu.close()
 
 
-def test_gemma4_forward_token_matches_oracle_teacher_forced(tiny):
-    """Teacher-forced and cache-synchronised, as for the synthetic shape: a K/V value on a Q4_0 rounding boundary
-    may take the neighbouring code; such a step is counted, its rows are overwritten with the oracle's, and its
-    logits are not compared.  24 positions: three times the sliding window."""
-    gpu, cpu, cfg = tiny
+def teacher_forced(gpu, cpu, cfg, pattern, toks, check=None, use_graph=False, tol=1e-3):
+    """Feeds both models the same tokens and keeps their caches identical: a K/V value on a Q4_0 rounding boundary
+    may take the neighbouring code on two correct f32 implementations; such a step is counted, its rows are
+    overwritten with the oracle's, and its logits (which see the other code through every later layer) are not
+    compared.  Returns (steps compared, steps whose greedy token was checked and agreed)."""
     ctx = gpu.ctx
-    gpu.reset()
-    cpu.reset()
-    n_layers = cfg["n_layers"]
-    assert [gpu.kv_source(l) for l in range(n_layers)] == [cpu.kv_source(l) for l in range(n_layers)] == [0, 1, 2, 3, 4, 4, 2, 4]
-    owners = [l for l in range(n_layers) if gpu.kv_source(l) == l]
-    hd = {l: cfg["hd_swa"] if PATTERN[l] else cfg["hd_full"] for l in owners}
+    owners = [l for l in range(cfg["n_layers"]) if gpu.kv_source(l) == l]
+    hd = {l: cfg["hd_swa"] if pattern[l] else cfg["hd_full"] for l in owners}
     bufs = {l: [hip.Buffer(ctx, hip.lib().ksh_gemma4_kv(gpu.h, l, w), owned=False) for w in (0, 1)] for l in owners}
-    toks = np.random.default_rng(611).integers(0, cfg["vocab"], 24)
     agree = clean = 0
     for i, t in enumerate(toks):
-        g_next = gpu.forward_token(int(t), use_graph=False)
-        c_next, c_logits = cpu.forward(int(t), return_logits=True)
-        g_logits = gpu.logits()
+        compare = check is None or i in check
+        g_next = gpu.forward_token(int(t), want_logits=compare, use_graph=use_graph)
+        c_next, c_logits = cpu.forward(int(t), want_logits=compare, return_logits=True)
         flips = 0
         for l in owners:
             row = cfg["n_kv"] * hd[l] // 32 * 18
@@ -168,18 +163,33 @@ def test_gemma4_forward_token_matches_oracle_teacher_forced(tiny):
                 if not np.array_equal(got, want):
                     flips += int((got != want).sum())
                     dg, dc = oracle.dequant(oracle.Q40, got, row // 18 * 32), oracle.dequant(oracle.Q40, want, row // 18 * 32)
-                    assert np.abs(dg - dc).max() <= np.abs(dc).max() / 7 * 1.01
+                    assert np.abs(dg - dc).max() <= np.abs(dc).max() / 7 * 1.01      # a flip is one code step, never more
                     ctx.write_bytes(bufs[l][w], want, i * row)
-        assert g_next == oracle.softcap_argmax(g_logits, cfg["softcap"])
+        if not compare:
+            continue
+        g_logits = gpu.logits()
+        assert g_next == oracle.softcap_argmax(g_logits, cfg["softcap"])       # the device argmax follows the oracle's rule
         if flips:
             continue
         clean += 1
-        assert_close(g_logits, c_logits, 1e-3, f"logits at step {i}")
-        assert_close(gpu.hidden(), cpu.hidden(), 1e-3, f"hidden at step {i}")
+        assert_close(g_logits, c_logits, tol, f"logits at step {i}")
+        assert_close(gpu.hidden(), cpu.hidden(), tol, f"hidden at step {i}")
         top2 = np.sort(c_logits)[-2:]
-        if top2[1] - top2[0] > 1e-3 * max(abs(top2[1]), float(np.sqrt(np.mean(c_logits ** 2)))):
+        if top2[1] - top2[0] > tol * max(abs(top2[1]), float(np.sqrt(np.mean(c_logits ** 2)))):
             assert g_next == c_next, f"step {i}: margin {top2[1] - top2[0]}"
             agree += 1
+    return clean, agree
+
+
+def test_gemma4_forward_token_matches_oracle_teacher_forced(tiny):
+    """24 positions: three times the sliding window."""
+    gpu, cpu, cfg = tiny
+    gpu.reset()
+    cpu.reset()
+    n_layers = cfg["n_layers"]
+    assert [gpu.kv_source(l) for l in range(n_layers)] == [cpu.kv_source(l) for l in range(n_layers)] == [0, 1, 2, 3, 4, 4, 2, 4]
+    toks = np.random.default_rng(611).integers(0, cfg["vocab"], 24)
+    clean, agree = teacher_forced(gpu, cpu, cfg, PATTERN, toks)
     assert clean >= 18 and agree >= 14 and gpu.pos == cpu.pos == len(toks)
     with pytest.raises(hip.KshError, match="outside the vocabulary"):
         gpu.forward_token(cfg["vocab"])
@@ -317,3 +327,35 @@ def test_gemma4_from_gguf_matches_oracle(ctx, tmp_path):
     gw.write(path, meta, bad)
     with hip.Gguf(path) as f, pytest.raises(hip.KshError, match="blk.0.attn_q.weight is"):
         hip.Gemma4.from_gguf(ctx, f, cfg["max_seq"])
+
+
+def test_gemma4_real_widths_long_run_matches_oracle(ctx, eng):
+    """The real checkpoints' widths (hidden 1536, head dims 256 / 512, window 512, double-wide feed-forward on the
+    layers that reuse a cache, unscaled attention) on a shortened stack, teacher-forced past the window through
+    the captured graph, against the oracle on the very same packed bytes (quantized on the device, read back for
+    the CPU).  Logits are compared where the run changes regime: the first positions, the oracle's switch to
+    split-KV attention at 128 rows, the window's edge at 512.  The bar is 5e-3 on whole-model logits here: with
+    unscaled scores over hundreds of rows of random weights the softmax is close to one-hot, and an f32
+    reassociation difference in a score moves the output by more than it does at the tiny model's 24 rows (1e-3
+    there; the single ops stay at 1e-3 in their own tests)."""
+    n, shared = 9, 4
+    cfg = dict(n_layers=n, hidden=1536, n_q=8, n_kv=1, vocab=8192, max_seq=576, hd_swa=256, hd_full=512, sliding_window=512,
+               shared_kv_layers=shared, ple_dim=256, eps=1e-6, softcap=30.0, rope_theta_swa=1e4, rope_theta_full=1e6,
+               partial_rotary=0.25, attn_scale=1.0)
+    pattern = [1, 1, 0, 1, 1, 1, 1, 0, 1]          # owners 0..4 (full: 2); 5, 6, 8 read layer 4's cache, 7 reads layer 2's
+    ffn = [6144 if i < n - shared else 12288 for i in range(n)]
+    dq4, dq6 = hip.device_quantizers(ctx, eng)
+    dev = synth.gemma4_weights(cfg, 630, dq4, lambda x: dq6([x]), ffn=ffn, swa_pattern=pattern, std=0.05)
+
+    def host(v):
+        return ctx.read_bytes(v, v.nbytes) if isinstance(v, hip.Buffer) else v
+
+    w = dict(layers=[{k: host(v) for k, v in lw.items()} for lw in dev["layers"]], globals={k: host(v) for k, v in dev["globals"].items()})
+    gpu, cpu = hip.Gemma4(ctx, cfg, dev), oracle.Gemma4(cfg, w)
+    assert [gpu.kv_source(l) for l in range(n)] == [0, 1, 2, 3, 4, 4, 4, 2, 4]
+    toks = np.random.default_rng(631).integers(0, cfg["vocab"], 540)
+    check = set(range(12)) | set(range(124, 134)) | set(range(506, 520)) | {300, 539}
+    clean, agree = teacher_forced(gpu, cpu, cfg, pattern, toks, check=check, use_graph=True, tol=5e-3)
+    assert clean >= 24 and agree >= 12, (clean, agree)
+    gpu.close()
+    cpu.close()

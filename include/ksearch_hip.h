@@ -137,12 +137,15 @@ enum ksh_kind {
      *     rope f32[max_seq, hd], k f32[n_kv*hd], k_norm f32[hd], v f32[n_kv*hd],
      *     meta f32[4] = {tlen, start, window, pos} with start + tlen - 1 == pos
      * out: K cache, V cache (row pos is written), tmp f32[n_q, nwg, hd+2],
-     *      out f32[n_q*hd].  Built for hd 128 / 256, up to 8 q heads per kv head.
+     *      out f32[n_q*hd].  Built for hd 128 / 256 / 512, up to 8 q heads per kv head.
      * With dims[5] = 1 the partitions are not merged: the outputs are K cache,
      * V cache and parts = { o f32[n_q, nwg, hd] (unnormalised), ml f32[n_q, nwg, 2]
      * (running max, sum) } in one buffer, for KSH_ATTN_MERGE_MATVEC.
      * With dims[6] = 1 the rope input is the row of the table for meta's pos, f32[hd], kept current by the
-     * caller: the launch then has nothing to wait for between reading pos and fetching its rope values. */
+     * caller: the launch then has nothing to wait for between reading pos and fetching its rope values.
+     * With dims[7] = 1 nothing is appended (a layer that reuses another layer's cache, whose row pos that layer
+     * has written in this step; RmsNormPerHeadRope -> SdpaMwg*, gemma_prim.rs:989-1034):
+     *   in: q, q_norm, rope, K cache, V cache, meta    out: tmp, out (or parts alone with dims[5] = 1) */
     KSH_ATTEND_DECODE = 22,
     /* SdpaMwgReduce (crates/ksearch_metal/src/lower.rs:5897-6087) folded into the
      * GEMV that consumes the attention output: every workgroup merges the

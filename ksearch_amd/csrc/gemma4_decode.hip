@@ -213,7 +213,12 @@ int encode_token(ksh_gemma4 *m, bool want_logits, int &launches)
         }
         // -- per-head norm, RoPE, cache append, attention
         bool parts = false;
-        if (P.attend) {
+        if (P.attend && !P.owns) {
+            parts = P.attend_parts;
+            if (parts ? enc(m, P.k_attend, {m->tq, L.q_norm, rope_cur, kc, vc, meta}, {m->attn_tmp}, launches)
+                      : enc(m, P.k_attend, {m->tq, L.q_norm, rope_cur, kc, vc, meta}, {m->attn_tmp, m->to}, launches))
+                return 1;
+        } else if (P.attend) {
             parts = P.attend_parts;
             if (parts ? enc(m, P.k_attend, {m->tq, L.q_norm, rope_cur, m->tk, L.k_norm, m->tv, meta}, {kc, vc, m->attn_tmp}, launches)
                       : enc(m, P.k_attend, {m->tq, L.q_norm, rope_cur, m->tk, L.k_norm, m->tv, meta}, {kc, vc, m->attn_tmp, m->to}, launches))
@@ -375,12 +380,13 @@ int plan_layer(ksh_gemma4 *m, int l)
                        get(m, KSH_RMSNORM_MATVEC, {P.kvd, h, 0}, {L.dt_v, KSH_F32}, {c.eps}, &P.kmat[1])))
             return 1;
     }
-    // attention: one launch where the fused kind is built for the shape and the layer appends to its own cache
+    // attention: one launch where the fused kind is built for the shape (appending, or reading another layer's cache)
     const bool short_form = P.swa && c.sliding_window <= kShortWindow && L.dt_o == KSH_Q4K && P.qd <= 2048 && (P.hd & (P.hd - 1)) == 0;
-    P.attend = P.owns && sdpa_lanes_supports(c.n_q, c.n_kv, P.hd);
+    P.attend = sdpa_lanes_supports(c.n_q, c.n_kv, P.hd);
     P.attend_parts = P.attend && short_form;
     if (P.attend) {
-        if (get(m, KSH_ATTEND_DECODE, {c.n_q, c.n_kv, P.hd, c.max_seq, P.attend_parts ? kShortPartitions : kAttendPartitions, P.attend_parts ? 1 : 0, 1},
+        if (get(m, KSH_ATTEND_DECODE,
+                {c.n_q, c.n_kv, P.hd, c.max_seq, P.attend_parts ? kShortPartitions : kAttendPartitions, P.attend_parts ? 1 : 0, 1, P.owns ? 0 : 1},
                 {KSH_Q40, KSH_F32}, {c.eps, c.attn_scale}, &P.k_attend))
             return 1;
     } else {

@@ -1,5 +1,5 @@
-// Decode attention over a Q4_0 KV cache, register form, for head sizes 128 and
-// 256 with up to 8 q heads per kv head; optionally with the per-head RMSNorm +
+// Decode attention over a Q4_0 KV cache, register form, for head sizes 128, 256
+// and 512 with up to 8 q heads per kv head; optionally with the per-head RMSNorm +
 // RoPE + Q4_0 KV append in front of it and always with the split-KV merge
 // behind it, so that a decode step's attention is one launch.
 //
@@ -64,6 +64,8 @@ struct LaneParams {
     int hsplit;   // workgroups that share a kv head's rows, each with its own q heads
     int balance;  // the launch's nwg * n_slots partitions are dealt to the slots by length (kModeMerge, several slots)
     int rope_row; // fused: `rope` is the current position's row of the table, not the table
+    int no_append; // fused: the step's K / V row is in the cache already (a layer that reuses another layer's cache): q is normed and
+                   // roped as usual, nothing is appended, every attended row comes from the cache
 };
 
 __device__ __forceinline__ uint32_t ld32_a2(const uint8_t *p)
@@ -83,6 +85,13 @@ __device__ __forceinline__ float xor16_sum(float x)
 {
     // rows 1 and 3 of the first copy trade places with rows 0 and 2 of the second
     const auto r = __builtin_amdgcn_permlane16_swap(as_u32(x), as_u32(x), false, false);
+    return as_f32(r[0]) + as_f32(r[1]);
+}
+
+__device__ __forceinline__ float xor32_sum(float x)
+{
+    // the two halves of the wave trade places
+    const auto r = __builtin_amdgcn_permlane32_swap(as_u32(x), as_u32(x), false, false);
     return as_f32(r[0]) + as_f32(r[1]);
 }
 
@@ -120,7 +129,8 @@ __device__ __forceinline__ void reduce_heads(const float (&v)[GP], int c, float 
         float x = keep + dpp_f32<0x4E>(send);   // quad_perm [2,3,0,1]
         x += dpp_f32<0x124>(x);                 // row_ror:4
         x += dpp_f32<0x128>(x);                 // row_ror:8
-        if (HD == 256) x = xor16_sum(x);
+        if (HD >= 256) x = xor16_sum(x);
+        if (HD == 512) x = xor32_sum(x);
         out[i] = x;
     }
 }
@@ -422,8 +432,9 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
     const bool dealt = p.fused != 0;
     // The last partition of a fused step takes no cached rows: it norms, ropes and packs the new K / V row,
     // stores it and attends it.  That work (0.7 us) would otherwise sit in front of one row partition's rows.
-    const int rparts = p.nwg > 1 ? p.nwg - 1 : 1;              // partitions that share the cached rows
-    const bool has_rows = p.nwg == 1 || part < p.nwg - 1;
+    const bool appender = p.nwg > 1 && !p.no_append;          // (nothing to append: every partition takes rows)
+    const int rparts = appender ? p.nwg - 1 : p.nwg;          // partitions that share the cached rows
+    const bool has_rows = !appender || part < p.nwg - 1;
     auto dealt_row = [&](int it, int t) { return ((it * kRT + t) * rparts + part) * GRP + wave * RPS + sub; };   // relative to start
     RowRegs cur[kRT], nxt[kRT];
 
@@ -466,8 +477,8 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
     auto load_row = [&](int t) { return load_row_at(start, t); };
 
     // the row this step appends is attended from LDS by the last partition (other kinds: by the one whose range holds it)
-    const bool owner = p.fused && (p.nwg == 1 || part == p.nwg - 1);   // (p.fused kinds are always dealt)
-    const int tend = tlen - 1;           // dealt: rows [0, tend) come from the cache
+    const bool owner = p.fused && !p.no_append && (p.nwg == 1 || part == p.nwg - 1);   // (p.fused kinds are always dealt)
+    const int tend = p.no_append ? tlen : tlen - 1;   // dealt: rows [0, tend) come from the cache
     if (dealt) {
         if (start != 0) {                // a window that has begun to slide: ask again
 #pragma unroll
@@ -516,11 +527,12 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
         if (owner && hg == 0) {
             // the appended row goes to the cache; the owners attend it from LDS
             const size_t off = (size_t)slot * slot_bytes + ((size_t)pos * p.n_kv + kvh) * ROWB;
-            if (tid < ROWB / 2)
-                reinterpret_cast<uint16_t *>(p.k_w + off)[tid] = reinterpret_cast<const uint16_t *>(newrow)[tid];
-            else if (tid < ROWB)
-                reinterpret_cast<uint16_t *>(p.v_w + off)[tid - ROWB / 2] =
-                    reinterpret_cast<const uint16_t *>(newrow + ROWB)[tid - ROWB / 2];
+            for (int i = tid; i < ROWB; i += NT) {   // (one pass, except 512-wide heads on four waves)
+                if (i < ROWB / 2)
+                    reinterpret_cast<uint16_t *>(p.k_w + off)[i] = reinterpret_cast<const uint16_t *>(newrow)[i];
+                else
+                    reinterpret_cast<uint16_t *>(p.v_w + off)[i - ROWB / 2] = reinterpret_cast<const uint16_t *>(newrow + ROWB)[i - ROWB / 2];
+            }
         }
 #pragma unroll
         for (int h = 0; h < GP; h++) {
@@ -771,6 +783,7 @@ int launch_lanes(const LaneParams &p, int hd, int nw, int n_slots, hipStream_t s
     if (hd == H && gp == G && nw == W) return launch_inst<H, G, W>(p, n_slots, st);
     KSH_CASE(128, 4, 4) KSH_CASE(128, 8, 4) KSH_CASE(256, 4, 4) KSH_CASE(256, 8, 4)
     KSH_CASE(128, 4, 8) KSH_CASE(128, 8, 8) KSH_CASE(256, 4, 8) KSH_CASE(256, 8, 8)
+    KSH_CASE(512, 4, 4) KSH_CASE(512, 4, 8)     // (eight heads of 512 do not fit the fold's LDS: such shapes split the heads)
 #undef KSH_CASE
     return set_error("sdpa (register form): no instance for hd=%d groups=%d nsg=%d", hd, p.groups, nw);
 }
@@ -833,7 +846,9 @@ int launch_bound(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
             p.balance = 1;
             p.mode = kModePart;
             if (launch_lanes(p, hd, nw, n_slots, st)) return 1;
-            if (hd == 256)
+            if (hd == 512)
+                hipLaunchKernelGGL(sdpa_dealt_merge_kernel<512>, dim3(p.n_q * 8, n_slots), dim3(256), 0, st, p.tmp, p.meta, p.meta_stride, p.nwg, p.n_q, p.out);
+            else if (hd == 256)
                 hipLaunchKernelGGL(sdpa_dealt_merge_kernel<256>, dim3(p.n_q * 4, n_slots), dim3(256), 0, st, p.tmp, p.meta, p.meta_stride, p.nwg, p.n_q, p.out);
             else
                 hipLaunchKernelGGL(sdpa_dealt_merge_kernel<128>, dim3(p.n_q * 2, n_slots), dim3(256), 0, st, p.tmp, p.meta, p.meta_stride, p.nwg, p.n_q, p.out);
@@ -841,25 +856,38 @@ int launch_bound(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
             return e == hipSuccess ? 0 : hip_fail(e, "sdpa merge launch");
         }
         break;
-    case KSH_ATTEND_DECODE:
+    case KSH_ATTEND_DECODE: {
+        const bool reader = k.desc.dims[7] != 0;
         p.q = (const float *)a.in[0]; p.qw = (const float *)a.in[1]; p.rope = (const float *)a.in[2];
-        p.k_raw = (const float *)a.in[3]; p.kw = (const float *)a.in[4]; p.v_raw = (const float *)a.in[5];
-        p.meta = (const float *)a.in[6];
+        int no = 0;
+        if (reader) {
+            // in: q, q_norm, rope, K cache, V cache, meta.  The loads of the raw k / v and of the key norm are issued
+            // unconditionally: they read q and the query norm again and nothing uses them.
+            p.k_raw = p.v_raw = p.q; p.kw = p.qw;
+            p.k = (const uint8_t *)a.in[3]; p.v = (const uint8_t *)a.in[4];
+            p.meta = (const float *)a.in[5];
+            p.no_append = 1;
+        } else {
+            p.k_raw = (const float *)a.in[3]; p.kw = (const float *)a.in[4]; p.v_raw = (const float *)a.in[5];
+            p.meta = (const float *)a.in[6];
+            p.k_w = (uint8_t *)a.out[0]; p.v_w = (uint8_t *)a.out[1];
+            p.k = p.k_w; p.v = p.v_w;
+            no = 2;
+        }
         p.meta_stride = 4;
-        p.k_w = (uint8_t *)a.out[0]; p.v_w = (uint8_t *)a.out[1];
-        p.k = p.k_w; p.v = p.v_w;
-        p.tmp = (float *)a.out[2];
+        p.tmp = (float *)a.out[no];
         p.eps = k.desc.params[0];
         p.scale = k.desc.params[1];
         p.rope_row = k.desc.dims[6] != 0;
         if (k.desc.dims[5]) {
             p.mode = kModeSplitPart;
         } else {
-            p.out = (float *)a.out[3];
+            p.out = (float *)a.out[no + 1];
             p.mode = kModeMerge;
         }
         p.fused = 1;
         break;
+    }
     default: return set_error("sdpa (register form): kind %d", k.desc.kind);
     }
     return launch_lanes(p, hd, nw, n_slots, st);
@@ -869,7 +897,7 @@ int launch_bound(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
 
 bool sdpa_lanes_supports(int64_t n_q, int64_t n_kv, int64_t hd)
 {
-    return n_kv > 0 && n_q % n_kv == 0 && n_q / n_kv <= 8 && (hd == 128 || hd == 256);
+    return n_kv > 0 && n_q % n_kv == 0 && n_q / n_kv <= 8 && (hd == 128 || hd == 256 || hd == 512);
 }
 
 // Fills in the launch for a shape sdpa_lanes_supports(); the caller has
@@ -889,7 +917,10 @@ int bind_sdpa_lanes(ksh_kernel &k, int nwg, int n_slots)
     int hsplit = k.desc.sched.unroll ? (int)k.desc.sched.unroll
                  : k.desc.kind != KSH_ATTEND_DECODE || total_groups < 4 ? 1
                  : k.desc.dims[5] ? total_groups : (total_groups % 2 == 0 ? total_groups / 2 : 1);
+    // heads of 512: at most four per workgroup (the fold's LDS)
+    if (hd == 512 && !k.desc.sched.unroll && total_groups / hsplit > 4 && total_groups % 4 == 0) hsplit = total_groups / 4;
     if (hsplit < 1 || hsplit > 255 || total_groups % hsplit) return set_error("sdpa: unsupported schedule unroll=%d (must divide %d)", hsplit, total_groups);
+    if (hd == 512 && total_groups / hsplit > 4) return set_error("sdpa: heads of 512 take at most four q heads per workgroup (unroll=%d leaves %d)", hsplit, total_groups / hsplit);
     const int wg_groups = total_groups / hsplit;
     const size_t lds = lanes_lds(hd, wg_groups, nw);
     const bool merges = k.desc.kind == KSH_SDPA_SLOTS || (k.desc.kind == KSH_ATTEND_DECODE && !k.desc.dims[5]);
@@ -917,25 +948,36 @@ int bind_attend_decode(ksh_kernel &k)
     int64_t nwg = d[4];
     if (n_q <= 0 || n_kv <= 0 || n_q % n_kv) return set_error("attend_decode: n_q=%lld n_kv=%lld", (long long)n_q, (long long)n_kv);
     if (!sdpa_lanes_supports(n_q, n_kv, hd))
-        return set_error("attend_decode: built for hd 128 or 256 and up to 8 q heads per kv head (got hd=%lld, %lld)",
+        return set_error("attend_decode: built for hd 128, 256 or 512 and up to 8 q heads per kv head (got hd=%lld, %lld)",
                          (long long)hd, (long long)(n_q / n_kv));
     if (max_t <= 0 || max_t > (1 << 24)) return set_error("attend_decode: max_seq=%lld", (long long)max_t);
     if (nwg == 0) nwg = max_t >= 2048 ? 16 : (max_t + 127) / 128;
     const size_t kvb = (size_t)max_t * n_kv * (hd / 32) * 18, qb = (size_t)n_q * hd * 4, kb = (size_t)n_kv * hd * 4;
-    k.info.n_inputs = 7;
-    k.info.n_outputs = 4;
-    k.in_bytes[0] = qb; k.in_bytes[1] = (size_t)hd * 4; k.in_bytes[2] = (d[6] ? 1 : (size_t)max_t) * hd * 4; k.in_bytes[3] = kb;
-    k.in_bytes[4] = (size_t)hd * 4; k.in_bytes[5] = kb; k.in_bytes[6] = 16;
+    const bool parts_only = d[5] != 0, reader = d[7] != 0;
+    const size_t partb = (size_t)n_q * nwg * (hd + 2) * 4;
     for (int i = 0; i < 7; i++) k.in_align[i] = 4;
     k.in_align[0] = 16;
-    k.out_bytes[0] = k.out_bytes[1] = kvb;
-    k.out_bytes[2] = (size_t)n_q * nwg * (hd + 2) * 4;
-    k.out_bytes[3] = qb;
-    k.out_align[0] = k.out_align[1] = 2; k.out_align[2] = k.out_align[3] = 4;
-    const bool parts_only = d[5] != 0;
-    if (parts_only) { k.info.n_outputs = 3; k.out_align[2] = 16; }
+    k.in_bytes[0] = qb; k.in_bytes[1] = (size_t)hd * 4; k.in_bytes[2] = (d[6] ? 1 : (size_t)max_t) * hd * 4;
+    if (reader) {
+        // nothing to append: in: q, q_norm, rope, K cache, V cache, meta   out: parts | tmp, o
+        k.info.n_inputs = 6;
+        k.info.n_outputs = parts_only ? 1 : 2;
+        k.in_bytes[3] = k.in_bytes[4] = kvb; k.in_bytes[5] = 16;
+        k.in_align[3] = k.in_align[4] = 2;
+        k.out_bytes[0] = partb; k.out_bytes[1] = qb;
+        k.out_align[0] = parts_only ? 16 : 4; k.out_align[1] = 4;
+    } else {
+        k.info.n_inputs = 7;
+        k.info.n_outputs = parts_only ? 3 : 4;
+        k.in_bytes[3] = kb; k.in_bytes[4] = (size_t)hd * 4; k.in_bytes[5] = kb; k.in_bytes[6] = 16;
+        k.out_bytes[0] = k.out_bytes[1] = kvb;
+        k.out_bytes[2] = partb;
+        k.out_bytes[3] = qb;
+        k.out_align[0] = k.out_align[1] = 2; k.out_align[2] = parts_only ? 16 : 4; k.out_align[3] = 4;
+    }
     if (bind_sdpa_lanes(k, (int)nwg, 1)) return 1;
-    set_name(k, "attend_decode%s_hd%d_nwg%d_w%d_h%d", parts_only ? "_parts" : "", (int)hd, (int)nwg, (int)k.info.sched.nsg, (int)k.info.sched.unroll);
+    set_name(k, "attend_decode%s%s_hd%d_nwg%d_w%d_h%d", reader ? "_reader" : "", parts_only ? "_parts" : "", (int)hd, (int)nwg, (int)k.info.sched.nsg,
+             (int)k.info.sched.unroll);
     return 0;
 }
 

@@ -176,6 +176,9 @@ def test_sdpa_errors(ctx):
     (4, 2, 128, 300, 150, 5, 0),      # two kv heads
     (8, 1, 256, 512, 300, 4, 173),    # a window that has begun to slide: rows [173, 300]
     (4, 1, 128, 256, 255, 2, 250),    # ... ending at the last row of the cache
+    (8, 1, 512, 512, 0, 0, 0),        # 512-wide heads (the full-attention layers of the real checkpoints): a row per wave
+    (8, 1, 512, 1024, 700, 16, 0),
+    (4, 2, 512, 300, 150, 5, 40),
 ])
 def test_attend_decode_vs_unfused_oracle(ctx, eng, n_q, n_kv, hd, max_seq, pos, nwg, start):
     """AttendDecode = RmsNormPerHeadQkvQ40 at `pos` + attention over rows [0, pos] + merge.  The oracle runs the
@@ -218,6 +221,46 @@ def test_attend_decode_vs_unfused_oracle(ctx, eng, n_q, n_kv, hd, max_seq, pos, 
     assert np.array_equal(ctx.read_bytes(kc2, (pos + 1) * row), gk) and np.array_equal(ctx.read_bytes(vc2, (pos + 1) * row), gv)
     if pos + 1 < max_seq:
         assert not ctx.read_bytes(kc, row, (pos + 1) * row).any()
+
+
+@pytest.mark.parametrize("n_q,n_kv,hd,max_seq,pos,nwg,start,parts", [
+    (8, 1, 256, 1024, 0, 8, 0, True),       # one row, every partition but one empty
+    (8, 1, 256, 1024, 600, 8, 89, True),    # the sliding-window layers that reuse a cache: 512 rows, unmerged
+    (8, 1, 256, 1024, 300, 16, 0, False),
+    (8, 1, 512, 1024, 700, 16, 0, False),   # the full-attention ones
+    (8, 1, 512, 512, 3, 16, 0, False),      # fewer rows than partitions
+    (4, 2, 128, 300, 150, 5, 40, False),
+    (4, 1, 128, 256, 77, 1, 0, False),      # a single partition
+])
+def test_attend_decode_reading_another_layers_cache(ctx, eng, n_q, n_kv, hd, max_seq, pos, nwg, start, parts):
+    """dims[7] = 1: q is normed and roped, nothing is appended, rows [start, pos] all come from the cache (which
+    must come back untouched).  Against the oracle's per-head norm + RoPE and attention, merged or through the
+    unmerged partitions."""
+    eps, scale = 1e-6, 1.0 / float(np.sqrt(hd))
+    row = n_kv * hd // 32 * 18
+    k, v = kv(max_seq, n_kv, hd, 540 + pos)
+    q = synth.normal_f32(n_q * hd, 550)
+    qw = 1.0 + 0.2 * synth.normal_f32(hd, 553)
+    rope = oracle.rope_table(max_seq, hd, 10000.0, hd // 4 if hd == 512 else None)
+    kc, vc = ctx.buffer_bytes(k), ctx.buffer_bytes(v)
+    tlen = pos + 1 - start
+    meta = ctx.buffer_f32([tlen, start, tlen if start else 0, pos])
+    kk = ctx.compile(hip.make_desc(hip.Kind.ATTEND_DECODE, (n_q, n_kv, hd, max_seq, nwg, int(parts), 1, 1), (DType.Q40, DType.F32), (eps, scale)))
+    assert "reader" in kk.name and kk.info.n_inputs == 6 and kk.info.n_outputs == (1 if parts else 2)
+    tmp, out = ctx.buffer_empty_f32(n_q * nwg * (hd + 2)), ctx.buffer_empty_f32(n_q * hd)
+    ins = [ctx.buffer_f32(q), ctx.buffer_f32(qw), ctx.buffer_f32(rope[pos]), kc, vc, meta]
+    want = oracle.sdpa(oracle.rmsnorm_per_head(q, qw, n_q, hd, eps, rope[pos]), k, v, n_q, n_kv, hd, tlen, start, scale, f64=True)
+    for rep in range(2):
+        ctx.encode_multi(kk, ins, [tmp] if parts else [tmp, out])
+        if parts:
+            t = ctx.read_f32(tmp, n_q * nwg * (hd + 2))
+            o, ml = t[:n_q * nwg * hd].reshape(n_q, nwg, hd).astype(np.float64), t[n_q * nwg * hd:].reshape(n_q, nwg, 2).astype(np.float64)
+            wt = np.exp(ml[:, :, 0] - ml[:, :, 0].max(1, keepdims=True))
+            got = (wt[:, :, None] * o).sum(1) / (wt * ml[:, :, 1]).sum(1)[:, None]
+        else:
+            got = ctx.read_f32(out, n_q * hd)
+        assert_close(got, want, TOL, f"rep {rep}")
+    assert np.array_equal(ctx.read_bytes(kc, max_seq * row), k) and np.array_equal(ctx.read_bytes(vc, max_seq * row), v)
 
 
 @pytest.mark.parametrize("n_q,n_kv,hd,max_seq,pos,nwg,rows", [

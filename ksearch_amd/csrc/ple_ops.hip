@@ -110,24 +110,37 @@ __global__ __launch_bounds__(kGmWaves * 64) void q4k_gemv_gelu_mul_kernel(const 
     const uint8_t *blk0 = wr + (size_t)b0 * 144;
     uint4 hdr = ldg_u4(blk0, 0), q0 = ldg_u4(blk0 + 16 + 32 * g, 0), q1 = ldg_u4(blk0 + 16 + 32 * g, 1);
 
+    // all of the vector's loads go out before anything is used (cols <= 8192: at most 8 float4 per thread and array)
+    constexpr int KMAX = 8192 / 4 / (kGmWaves * 64);
+    const int n4 = cols / 4;
+    float4 xv[KMAX], wv[HAS_RES ? KMAX : 1], rv[HAS_RES ? KMAX : 1];
+#pragma unroll
+    for (int k = 0; k < KMAX; k++) {
+        const int i = min(tid + k * kGmWaves * 64, n4 - 1);
+        xv[k] = ldg_f4(x, i);
+        if (HAS_RES) { wv[k] = ldg_f4(w_post, i); rv[k] = ldg_f4(res, i); }
+    }
+    float inv = 0.f;
     if (HAS_RES) {
         float ss = 0.f;
-        for (int i = tid; i < cols / 4; i += kGmWaves * 64) {
-            const float4 v = ldg_f4(x, i);
-            ss += (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w);
-        }
+#pragma unroll
+        for (int k = 0; k < KMAX; k++)
+            if (tid + k * kGmWaves * 64 < n4) ss += (xv[k].x * xv[k].x + xv[k].y * xv[k].y) + (xv[k].z * xv[k].z + xv[k].w * xv[k].w);
         ss = wave_sum(ss);
         if (lane == 0) red[wave] = ss;
         __syncthreads();
-        const float inv = 1.0f / sqrtf(((red[0] + red[1]) + (red[2] + red[3])) / (float)cols + eps);
-        for (int i = tid; i < cols / 4; i += kGmWaves * 64) {
-            const float4 v = ldg_f4(x, i), w = ldg_f4(w_post, i), r = ldg_f4(res, i);
-            const float4 o = make_float4(r.x + v.x * inv * w.x, r.y + v.y * inv * w.y, r.z + v.z * inv * w.z, r.w + v.w * inv * w.w);
-            *reinterpret_cast<float4 *>(xs + 4 * i + (i >> 4) * 4) = o;   // four floats of padding per 64: the groups of a wave land on distinct banks
+        inv = 1.0f / sqrtf(((red[0] + red[1]) + (red[2] + red[3])) / (float)cols + eps);
+    }
+#pragma unroll
+    for (int k = 0; k < KMAX; k++) {
+        const int i = tid + k * kGmWaves * 64;
+        if (i >= n4) continue;
+        float4 o = xv[k];
+        if (HAS_RES) {
+            o = make_float4(rv[k].x + o.x * inv * wv[k].x, rv[k].y + o.y * inv * wv[k].y, rv[k].z + o.z * inv * wv[k].z, rv[k].w + o.w * inv * wv[k].w);
             if (blockIdx.x == 0) stg_f4(x_out, i, o);
         }
-    } else {
-        for (int i = tid; i < cols / 4; i += kGmWaves * 64) *reinterpret_cast<float4 *>(xs + 4 * i + (i >> 4) * 4) = ldg_f4(x, i);
+        *reinterpret_cast<float4 *>(xs + 4 * i + (i >> 4) * 4) = o;   // four floats of padding per 64: the groups of a wave land on distinct banks
     }
     __syncthreads();
 

@@ -181,6 +181,38 @@ def bench_decode(ctx, eng, use_graph=True):
     return out
 
 
+def bench_decode_gemma4_layout(ctx, eng, use_graph=True):
+    """Greedy decode at the layer layout of the real Gemma-4 E2B checkpoints (synthetic weights): 35 layers of
+    hidden 1536, four sliding-window layers (head dim 256, window 512) per full-attention layer (head dim 512),
+    the last 20 layers reading earlier layers' KV caches with a double-wide feed-forward, per-layer embeddings
+    (a Q5_K table of 35 x 256 per token), Q6_K tied LM head.  Not the headline configuration (that one has none
+    of these features): a second point, for the loop that takes GGUF files."""
+    from ksearch_amd import hip, synth
+
+    n, shared = 35, 20
+    cfg = dict(n_layers=n, hidden=1536, n_q=8, n_kv=1, vocab=262144, max_seq=4096, hd_swa=256, hd_full=512, sliding_window=512,
+               shared_kv_layers=shared, ple_dim=256, eps=1e-6, softcap=30.0, rope_theta_swa=1e4, rope_theta_full=1e6, partial_rotary=0.25,
+               attn_scale=1.0)
+    ffn = [6144 if i < n - shared else 12288 for i in range(n)]
+    q4k, q6k = hip.device_quantizers(ctx, eng)
+    w = synth.gemma4_weights(cfg, 1005, q4k, lambda x: q6k([x]), ffn=ffn)
+    model = hip.Gemma4(ctx, cfg, w)
+    prompt = [int(t) for t in np.random.default_rng(1005).integers(0, cfg["vocab"], 64)]
+    ms = []
+    for _ in range(3):
+        model.reset()
+        ids, _, decode_ms = model.generate(prompt, 256, use_graph=use_graph)
+        ms.append(decode_ms)
+    # bytes a token streams: every packed matrix once (the per-layer table contributes one row)
+    wbytes = sum(b.nbytes for lw in w["layers"] for b in lw.values() if isinstance(b, hip.Buffer))
+    wbytes += w["globals"]["token_embd"].nbytes + w["globals"]["ple_model_proj"].nbytes
+    r = {"tok_s": round(256 / min(ms) * 1e3, 1), "ms_per_token": round(min(ms) / 256, 4), "launches_per_token": model.launches_per_token,
+         "weight_GB_per_token": round(wbytes / 1e9, 3), "GB_s": round(wbytes / (min(ms) / 256 * 1e-3) / 1e9, 1),
+         "layout": "35 layers, hidden 1536, 4 SWA(256, window 512) : 1 full(512), 20 shared-KV layers, PLE 256, ffn 6144/12288"}
+    model.close()
+    return r
+
+
 def cpu_baseline_matvec(w, x, rows, cols, budget_s=1.5):
     """The CPU checker (oracle/) timed on this machine: all cores, then one."""
     import oracle
@@ -214,7 +246,7 @@ def main() -> int:
     ap.add_argument("--no-extras", action="store_true", help="headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--eager", action="store_true", help="cfg4 without HIP-graph replay (kernel-trace profiling)")
-    ap.add_argument("--only", choices=["cfg1", "cfg2", "cfg3", "cfg4", "copy"],
+    ap.add_argument("--only", choices=["cfg1", "cfg2", "cfg3", "cfg4", "gemma4", "copy"],
                     help="run one secondary workload and print its record (for profiling runs); 'copy' is a plain "
                          "64 MiB device copy, the known-size kernel that calibrates the FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
@@ -240,7 +272,8 @@ def main() -> int:
             r = bench_lm_head(ctx, eng, ev)
         else:
             r = {"cfg2": lambda: bench_prefill(ctx), "cfg3": lambda: bench_attention(ctx),
-                 "cfg4": lambda: bench_decode(ctx, eng, not args.eager)}[args.only]()
+                 "cfg4": lambda: bench_decode(ctx, eng, not args.eager),
+                 "gemma4": lambda: bench_decode_gemma4_layout(ctx, eng, not args.eager)}[args.only]()
         ctx.close()
         print(json.dumps({args.only: r}))
         return 0
@@ -256,6 +289,7 @@ def main() -> int:
         also["cfg2_q4k_prefill_gemm"] = bench_prefill(ctx)
         also["cfg3_q40_attention"] = bench_attention(ctx)
         also["cfg4_gemma_decode"] = bench_decode(ctx, eng)
+        also["gemma4_e2b_layer_layout_decode"] = bench_decode_gemma4_layout(ctx, eng)
 
     cpu = None
     if not args.no_cpu:

@@ -28,6 +28,17 @@
  *                            independence, needle case
  *   ko_softcap_argmax        reference unit test ([1,9,3] -> 1), tie rule
  *   ko_rmsnorm*, rope, gelu  closed forms, pos=0 identity
+ *   ko_dequant (Q5_K)        the block loop vs an independent per-element
+ *                            restatement of the GPU helper, reduction to Q4_K
+ *                            with every fifth bit clear, +16*d*sc with all set
+ *   ko_rmsnorm_per_head      f64 closed form, rope row 0 = identity, rotation
+ *                            keeps the norm, equals the pinned QKV op's q half
+ *   ko_add_scale,
+ *   ko_matvec_gelu_mul       closed forms (f64 GELU-tanh on the f64 dot)
+ *   ko_gemma4_*              bit-identical to the pinned ko_gemma_* loop when
+ *                            the extras are off; kv_source vs the rule restated;
+ *                            the window: equal to a wide-window run for exactly
+ *                            `window` positions
  *   ko_quantize_q4k          reference round-trip test only (output bytes of
  *                            the iterative search are PARITY UNPINNED; they
  *                            never enter a GPU-vs-oracle comparison because

@@ -41,8 +41,9 @@ typedef struct ksh_graph ksh_graph;
 /* DType, crates/ksearch_ir/src/lib.rs:17-27 (same order).
  * KSH_Q6K_ROWS has no counterpart there: it is Q6_K with the bytes of every weight row regrouped by field
  * (all ql of the row's superblocks, then all qh, all scales, all d: the same 210 B per 256 weights, every
- * field 16-byte aligned), which is how the LM head is kept in HBM so that a wave fetches a row with whole
- * 128-bit loads.  KSH_REPACK_ROWS makes it from Q6_K; rows must be a multiple of 2048 columns long. */
+ * field 16-byte aligned, the row padded to a multiple of 16 bytes), which is how the LM head is kept in HBM
+ * so that a wave fetches a row with whole 128-bit loads.  KSH_REPACK_ROWS makes it from Q6_K; the GEMV takes
+ * rows of 1536, 2048 or 4096 columns (1264, 1680, 3360 bytes). */
 enum ksh_dtype {
     KSH_F32 = 0, KSH_F16 = 1, KSH_Q4K = 2, KSH_Q5K = 3, KSH_Q6K = 4, KSH_Q40 = 5, KSH_BF16 = 6, KSH_Q6K_ROWS = 7
 };
@@ -156,7 +157,7 @@ enum ksh_kind {
      * out: y f32[rows] */
     KSH_ATTN_MERGE_MATVEC = 23,
     /* Q6_K [rows, cols] -> KSH_Q6K_ROWS, a byte permutation inside every row (done once, when weights are
-     * loaded).  dims: rows, cols (a multiple of 2048).  in: src Q6_K   out: dst (same size, 16-byte aligned) */
+     * loaded).  dims: rows, cols.  in: src Q6_K   out: dst, rows * round_up(cols/256*210, 16) bytes, 16-byte aligned */
     KSH_REPACK_ROWS = 24,
     /* Eng::rmsnorm_per_head and rmsnorm_per_head_rope_off (crates/ksearch_kernels/src/lib.rs:564-625):
      * y[h,i] = x[h,i] * rsqrt(mean_h(x^2) + eps) * w[i], then RoPE with pairs (i, i + hd/2) of the row

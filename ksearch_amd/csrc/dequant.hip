@@ -137,12 +137,13 @@ int launch_dequant(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
 }
 
 // Q6_K -> Q6K_ROWS: one workgroup per weight row, one thread per output dword.  Row of bpr superblocks:
-// ql [bpr][128] | qh [bpr][64] | sc [bpr][16] | d [bpr][2].
+// ql [bpr][128] | qh [bpr][64] | sc [bpr][16] | d [bpr][2], then zero padding to a multiple of 16 bytes.
 __global__ __launch_bounds__(256) void repack_q6k_rows_kernel(const uint8_t *src, uint8_t *dst, int bpr)
 {
-    const size_t row = blockIdx.x, rb = (size_t)bpr * 210;
+    const size_t row = blockIdx.x, rb = (size_t)bpr * 210, stride = (rb + 15) / 16 * 16;
     const uint16_t *s = reinterpret_cast<const uint16_t *>(src + row * rb);   // blocks are 2-byte aligned
-    uint16_t *d = reinterpret_cast<uint16_t *>(dst + row * rb);
+    uint16_t *d = reinterpret_cast<uint16_t *>(dst + row * stride);
+    for (int o = (int)(rb / 2) + threadIdx.x; o < (int)(stride / 2); o += 256) d[o] = 0;
     const int nql = bpr * 64, nqh = bpr * 32, nsc = bpr * 8;                   // in 16-bit units
     for (int o = threadIdx.x; o < (int)(rb / 2); o += 256) {
         int b, i;
@@ -169,11 +170,12 @@ int bind_repack_rows(ksh_kernel &k)
     const int64_t rows = k.desc.dims[0], cols = k.desc.dims[1];
     if (k.desc.dtypes[0] != KSH_Q6K || k.desc.dtypes[1] != KSH_Q6K_ROWS)
         return set_error("repack_rows: only Q6_K -> Q6K_ROWS is built (got %d -> %d)", k.desc.dtypes[0], k.desc.dtypes[1]);
-    if (rows <= 0 || rows > 0x7FFFFFFF || cols <= 0 || cols % 2048 || cols > (1 << 20))
-        return set_error("repack_rows: rows=%lld cols=%lld (cols must be a positive multiple of 2048)", (long long)rows, (long long)cols);
+    if (rows <= 0 || rows > 0x7FFFFFFF || cols <= 0 || cols % 256 || cols > (1 << 20))
+        return set_error("repack_rows: rows=%lld cols=%lld (cols must be a positive multiple of 256)", (long long)rows, (long long)cols);
     k.info.n_inputs = 1;
     k.info.n_outputs = 1;
-    k.in_bytes[0] = k.out_bytes[0] = (size_t)rows * (cols / 256) * 210;
+    k.in_bytes[0] = (size_t)rows * (cols / 256) * 210;
+    k.out_bytes[0] = (size_t)rows * (((size_t)(cols / 256) * 210 + 15) / 16 * 16);   // rows padded to 16 bytes
     k.in_align[0] = 2;
     k.out_align[0] = 16;
     set_launch(k, (uint32_t)rows, 1, 1, 256, 0);

@@ -360,6 +360,14 @@ int plan_layer(ksh_gemma4 *m, int l)
         if ((m->layers[P.src].is_swa != 0) != P.swa)
             return set_error("layer %d reuses the cache of layer %d, which has another head dim", l, P.src);
     }
+    {
+        // every buffer the layer's launches will bind
+        const ksh_buf *need[] = {L.wq, L.wo, L.wgate, L.wup, L.wdown, L.attn_norm, L.q_norm, L.post_attn_norm, L.ffn_norm, L.post_ffw_norm};
+        for (const ksh_buf *b : need)
+            if (!b) return set_error("layer %d: a weight or norm buffer is missing", l);
+        if (P.owns && (!L.wk || !L.wv || !L.k_norm)) return set_error("layer %d owns its KV cache and needs k / v weights and the key norm", l);
+        if (c.ple_dim > 0 && (!L.inp_gate || !L.proj || !L.post_norm)) return set_error("layer %d: per-layer-embedding weights are missing", l);
+    }
     const int dts[] = {L.dt_q, L.dt_o, L.dt_gate, L.dt_up, L.dt_down};
     for (int dt : dts)
         if (!packed_ok(dt)) return set_error("layer %d: weight dtype %d is not built (Q4_K and Q6_K are)", l, dt);
@@ -469,10 +477,10 @@ int ksh_gemma4_create(ksh_ctx *ctx, const ksh_gemma4_cfg *cfg, const ksh_gemma4_
     const int de = globals->dt_embd;
     if (!packed_ok(de)) return set_error("ksh_gemma4_create: embedding dtype %d is not built (Q4_K and Q6_K are)", de);
     int lm_dt = de;
-    if (de == KSH_Q6K && (c.hidden == 2048 || c.hidden == 4096)) {
+    if (de == KSH_Q6K && (c.hidden == 1536 || c.hidden == 2048 || c.hidden == 4096)) {
         // the LM head streams the whole table every token: it gets a copy with each row's fields grouped
         ksh_kernel *rp = nullptr;
-        if (alloc(m, (size_t)c.vocab * (c.hidden / 256) * 210, &m->embd_rows) ||
+        if (alloc(m, (size_t)c.vocab * (((size_t)(c.hidden / 256) * 210 + 15) / 16 * 16), &m->embd_rows) ||
             get(m, KSH_REPACK_ROWS, {c.vocab, c.hidden}, {KSH_Q6K, KSH_Q6K_ROWS}, {}, &rp))
             return 1;
         int n = 0;

@@ -194,13 +194,16 @@ __global__ __launch_bounds__(NW * 64) void q6k_gemv_kernel(Q6kParams p)
 }
 
 // ---- Q6K_ROWS: the same weights with every row regrouped by field ------------
-// Row of bpr superblocks (bpr a multiple of 8): ql [bpr][128] | qh [bpr][64] | sc [bpr][16] | d [bpr][2], each
-// section 16-byte aligned.  A step covers 8 superblocks with ONE 128-bit load per lane over 1 KB of ql, lane
+// Row of bpr superblocks: ql [bpr][128] | qh [bpr][64] | sc [bpr][16] | d [bpr][2], each section 16-byte
+// aligned, the row padded to a multiple of 16 bytes (q6r_row_bytes: 1264 for the 1260 bytes of a 1536-column
+// row; nothing for 2048 or 4096 columns).  A step covers 8 superblocks with ONE 128-bit load per lane over 1 KB of ql, lane
 // after lane: lane j = lane % 8 of superblock b = lane / 8 holds ql bytes 16j .. 16j+15, i.e. in half ip = j / 4
 // the positions l0 = 16 * (j % 2) .. +15 of the quadrants k = part (low nibbles) and part + 2 (high nibbles),
 // part = (j / 2) % 2.  It fetches the 16 qh bytes of those positions (lanes j and j ^ 2 the same ones), the
 // half's 8 scale bytes and d.  A row is then fetched through the fewest cache lines it spans (14) instead of
 // the ~80 that the per-field loads of the 210-byte superblocks touch.
+__host__ __device__ constexpr size_t q6r_row_bytes(int bpr) { return ((size_t)bpr * 210 + 15) / 16 * 16; }
+
 struct Q6rLane {
     u32x4_t ql, qh;
     u32x2 sc;
@@ -276,7 +279,7 @@ __global__ __launch_bounds__(NW * 64) void q6r_gemv_kernel(Q6kParams p)
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int bl = lane >> 3;
     const int cols = p.bpr * 256;
-    const size_t row_bytes = (size_t)p.bpr * kQ6kBytes;
+    const size_t row_bytes = q6r_row_bytes(p.bpr);
     const int w0 = (blockIdx.x * NW + wave) * p.rows_per_wave;
     const int w1 = min(w0 + p.rows_per_wave, p.rows);
 
@@ -286,7 +289,7 @@ __global__ __launch_bounds__(NW * 64) void q6r_gemv_kernel(Q6kParams p)
         for (int r = 0; r < R; r++) {
             const uint8_t *rp = p.W + (size_t)min(row0 + r, p.rows - 1) * row_bytes;
 #pragma unroll
-            for (int s = 0; s < STEPS; s++) dst[s][r] = q6r_load(rp, p.bpr, s * 8 + bl, lane);   // bpr is a multiple of 8: every lane's superblock exists
+            for (int s = 0; s < STEPS; s++) dst[s][r] = q6r_load(rp, p.bpr, min(s * 8 + bl, p.bpr - 1), lane);   // past the row's end: the last superblock again, against a zero scale
         }
     };
     constexpr int KMAX = (STEPS * 512 + NW * 64 - 1) / (NW * 64);   // float4 of the vector per thread: cols == STEPS * 2048
@@ -299,7 +302,7 @@ __global__ __launch_bounds__(NW * 64) void q6r_gemv_kernel(Q6kParams p)
 
     XQ6r X[STEPS];
 #pragma unroll
-    for (int s = 0; s < STEPS; s++) X[s].load(xs, s * 8 + bl, lane, true);
+    for (int s = 0; s < STEPS; s++) X[s].load(xs, min(s * 8 + bl, p.bpr - 1), lane, s * 8 + bl < p.bpr);
 
     for (int row0 = w0; row0 < w1; row0 += R) {
         load_rows(nxt, min(row0 + R, p.rows - 1));
@@ -401,8 +404,8 @@ int bind_matvec_q6k(ksh_kernel &k)
     if (cols <= 0 || cols % 256 || cols > 8192)
         return set_error("matvec_q6k: cols=%lld is not a positive multiple of 256 up to 8192", (long long)cols);
     const bool by_rows = k.desc.dtypes[0] == KSH_Q6K_ROWS;
-    if (by_rows && cols != 2048 && cols != 4096)
-        return set_error("matvec_q6k: row-grouped weights are built for 2048 and 4096 columns (got %lld)", (long long)cols);
+    if (by_rows && cols != 1536 && cols != 2048 && cols != 4096)
+        return set_error("matvec_q6k: row-grouped weights are built for 1536, 2048 and 4096 columns (got %lld)", (long long)cols);
     Q6kGeom G = pick_geom6(k.desc.sched, (int)rows);
     if (k.desc.dtypes[0] == KSH_Q6K_ROWS && sched_is_zero(k.desc.sched)) {   // measured best on 262144 x 2048
         G.NW = 8;
@@ -420,7 +423,7 @@ int bind_matvec_q6k(ksh_kernel &k)
         return set_error("rmsnorm_matvec requires LOCAL staging of the vector (cols=%lld too large)", (long long)cols);
     k.info.n_inputs = pro ? (has_res ? 5 : 3) : 2;
     k.info.n_outputs = has_res ? 2 : 1;
-    k.in_bytes[0] = (size_t)rows * bpr * kQ6kBytes;
+    k.in_bytes[0] = by_rows ? (size_t)rows * q6r_row_bytes(bpr) : (size_t)rows * bpr * kQ6kBytes;
     k.in_align[0] = by_rows ? 16 : 2;
     for (int i = 1; i < k.info.n_inputs; i++) { k.in_bytes[i] = (size_t)cols * 4; k.in_align[i] = 16; }
     k.out_bytes[0] = (size_t)rows * 4;

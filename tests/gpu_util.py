@@ -20,7 +20,9 @@ def assert_close(got, want, tol, what=""):
 
 def q6k_rows(w, rows, cols):
     """Q6_K bytes [rows, cols/256, 210] -> the library's row-grouped form (KSH_Q6K_ROWS): per row all ql, then all
-    qh, all scales, all d.  The definition the device repacker is checked against."""
+    qh, all scales, all d, zero padding to 16 bytes.  The definition the device repacker is checked against."""
     b = np.asarray(w, dtype=np.uint8).reshape(rows, cols // 256, 210)
+    pad = -(cols // 256 * 210) % 16                 # rows are padded to 16 bytes (1536 columns: 1260 -> 1264)
     return np.concatenate([b[:, :, :128].reshape(rows, -1), b[:, :, 128:192].reshape(rows, -1),
-                           b[:, :, 192:208].reshape(rows, -1), b[:, :, 208:].reshape(rows, -1)], axis=1).reshape(-1)
+                           b[:, :, 192:208].reshape(rows, -1), b[:, :, 208:].reshape(rows, -1),
+                           np.zeros((rows, pad), np.uint8)], axis=1).reshape(-1)

@@ -235,6 +235,9 @@ def test_gemma4_create_errors(ctx):
     w_bad = synth.gemma4_weights(cfg, 613, oracle.quantize_q4k, oracle.quantize_q6k, ffn=512)
     with pytest.raises(hip.KshError, match="another head dim"):
         hip.Gemma4(ctx, cfg, w_bad)
+    gone = dict(w, layers=[{k: v for k, v in w["layers"][0].items() if k != "post_norm"}] + w["layers"][1:])
+    with pytest.raises(hip.KshError, match="per-layer-embedding weights are missing"):
+        hip.Gemma4(ctx, cfg, gone)
     bad = dict(w, layers=[dict(w["layers"][0], dt_q=int(DType.Q5K))] + w["layers"][1:])
     with pytest.raises(hip.KshError, match="weight dtype"):
         hip.Gemma4(ctx, cfg, bad)

@@ -154,16 +154,17 @@ def test_matvec_q6k(ctx, eng, rows, cols, sched):
     assert_close(ctx.read_f32(by, rows), oracle.matvec(oracle.Q6K, w, rows, cols, x), TOL, f"q6k {rows}x{cols} {sched}")
 
 
-@pytest.mark.parametrize("rows,cols", [(8, 2048), (1000, 2048), (4099, 2048), (300, 4096), (1, 2048)])
+@pytest.mark.parametrize("rows,cols", [(8, 2048), (1000, 2048), (4099, 2048), (300, 4096), (1, 2048), (1000, 1536), (7, 1536)])
 @pytest.mark.parametrize("sched", SCHEDS_Q6K)
 def test_matvec_q6k_row_grouped(ctx, eng, rows, cols, sched):
     """The LM head's storage form: the device repack is the stated byte permutation, and the GEMV over it gives
     what the oracle gives for the original Q6_K bytes."""
     w = synth.q6k_blocks(rows * cols // 256, seed=rows + 1)
     x = synth.normal_f32(cols, seed=12)
-    bw, br = ctx.buffer_bytes(w), ctx.buffer_empty_bytes(w.size)
+    want_rows = q6k_rows(w, rows, cols)           # (1536-column rows are padded from 1260 to 1264 bytes)
+    bw, br = ctx.buffer_bytes(w), ctx.buffer_empty_bytes(want_rows.size)
     eng.repack_rows(ctx, rows, cols, bw, br)
-    assert np.array_equal(ctx.read_bytes(br, w.size), q6k_rows(w, rows, cols))
+    assert np.array_equal(ctx.read_bytes(br, want_rows.size), want_rows)
     by = ctx.buffer_empty_f32(rows)
     eng.matvec_wd(ctx, rows, cols, DType.Q6K_ROWS, br, ctx.buffer_f32(x), by, sched)
     assert_close(ctx.read_f32(by, rows), oracle.matvec(oracle.Q6K, w, rows, cols, x), TOL, f"q6k rows {rows}x{cols} {sched}")
@@ -180,10 +181,20 @@ def test_matvec_q6k_row_grouped_unit_vectors_and_errors(ctx, eng):
         e[j] = 1.0
         eng.matvec_wd(ctx, rows, cols, DType.Q6K_ROWS, br, ctx.buffer_f32(e), by)
         assert np.allclose(ctx.read_f32(by, rows), wd[:, j], rtol=1e-6, atol=1e-9), j
-    with pytest.raises(hip.KshError, match="2048 and 4096"):
+    with pytest.raises(hip.KshError, match="1536, 2048 and 4096"):
         ctx.compile(hip.make_desc(hip.Kind.MATVEC, (64, 1024), (DType.Q6K_ROWS, DType.F32)))
-    with pytest.raises(hip.KshError, match="multiple of 2048"):
-        ctx.compile(hip.make_desc(hip.Kind.REPACK_ROWS, (64, 1024), (DType.Q6K, DType.Q6K_ROWS)))
+    with pytest.raises(hip.KshError, match="multiple of 256"):
+        ctx.compile(hip.make_desc(hip.Kind.REPACK_ROWS, (64, 1000), (DType.Q6K, DType.Q6K_ROWS)))
+    # 1536 columns: six of a step's eight superblock slots hold weights
+    rows, cols = 3, 1536
+    w = synth.q6k_blocks(rows * cols // 256, seed=6)
+    wd = oracle.dequant(oracle.Q6K, w, rows * cols).reshape(rows, cols)
+    br, by = ctx.buffer_bytes(q6k_rows(w, rows, cols)), ctx.buffer_empty_f32(rows)
+    for j in [0, 127, 128, 255, 256, 1279, 1280, 1535]:
+        e = np.zeros(cols, dtype=np.float32)
+        e[j] = 1.0
+        eng.matvec_wd(ctx, rows, cols, DType.Q6K_ROWS, br, ctx.buffer_f32(e), by)
+        assert np.allclose(ctx.read_f32(by, rows), wd[:, j], rtol=1e-6, atol=1e-9), j
     with pytest.raises(hip.KshError, match="only Q6_K"):
         ctx.compile(hip.make_desc(hip.Kind.REPACK_ROWS, (64, 2048), (DType.Q4K, DType.Q6K_ROWS)))
 

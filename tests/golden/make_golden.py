@@ -3,6 +3,7 @@
 
     python tests/golden/make_golden.py            # small.npz (seconds)
     python tests/golden/make_golden.py --cfg4     # + cfg4_tokens.json (minutes: full-size CPU decode)
+    python tests/golden/make_golden.py --gemma4   # gemma4_small.npz only (seconds)
 
 The reference ships no golden vectors for this path (its kernel checks only
 print statistics), so these are the oracle's outputs on seeded inputs, kept as
@@ -57,6 +58,47 @@ def small():
     print("wrote small.npz", {k_: v_.shape for k_, v_ in out.items()})
 
 
+G4_PATTERN = [1, 1, 0, 1, 1, 1, 0, 1]
+G4_FFN = [1024, 1024, 2048, 1024, 1024, 1024, 2048, 1024]
+G4_Q6K = ((1, "wv"), (2, "wdown"), (4, "wgate"))
+
+
+def gemma4_tiny_weights():
+    return synth.gemma4_weights(dict(synth.GEMMA4_TINY), 9100, oracle.quantize_q4k, oracle.quantize_q6k, ffn=G4_FFN,
+                                swa_pattern=G4_PATTERN, q6k_tensors=set(G4_Q6K), std=0.05)
+
+
+def gemma4():
+    """gemma4_small.npz: the ops and the loop that the real checkpoints add (Q5_K, per-head norm + RoPE,
+    gelu(Wx)*ctx, the tiny 8-layer model with both layer kinds, shared caches and per-layer embeddings)."""
+    out = {}
+    q5 = synth.q5k_blocks(6, 9101, 1e-3, 1e-2)
+    out["q5k_blocks"], out["q5k_deq"] = q5, oracle.dequant(oracle.Q5K, q5, 6 * 256)
+    x, w = synth.normal_f32(3 * 128, 9102), 1.0 + 0.2 * synth.normal_f32(128, 9103)
+    rope = oracle.rope_table(6, 128, 10000.0, 16)[5]
+    out["ph_x"], out["ph_w"], out["ph_rope"] = x, w, rope
+    out["ph_norm"], out["ph_rope_out"] = oracle.rmsnorm_per_head(x, w, 3, 128, 1e-6), oracle.rmsnorm_per_head(x, w, 3, 128, 1e-6, rope)
+    wg, xg, cg = synth.q4k_blocks(16 * 2, 9104), synth.normal_f32(512, 9105), synth.normal_f32(16, 9106)
+    out["gm_w"], out["gm_x"], out["gm_ctx"], out["gm_y"] = wg, xg, cg, oracle.matvec_gelu_mul(oracle.Q4K, wg, 16, 512, xg, cg)
+    cfg = dict(synth.GEMMA4_TINY)
+    m = oracle.Gemma4(cfg, gemma4_tiny_weights())
+    # teacher-forced on random ids (the free-running model settles on one token): 20 positions, past the window of 8
+    prompt = [int(t) for t in np.random.default_rng(9107).integers(0, cfg["vocab"], 20)]
+    toks, top, margin = [], [], []
+    for t in prompt:
+        tok, lg = m.forward(t, return_logits=True)
+        s2 = np.sort(lg)[-2:]
+        toks.append(tok)
+        top.append(float(s2[1]))
+        margin.append(float((s2[1] - s2[0]) / max(abs(s2[1]), 1e-6)))
+    out["g4_prompt"], out["g4_tokens"] = np.array(prompt, np.int64), np.array(toks, np.int64)
+    out["g4_top_logit"], out["g4_margin"] = np.array(top, np.float32), np.array(margin, np.float32)
+    out["g4_hidden"] = m.hidden()
+    out["g4_kv_source"] = np.array([m.kv_source(l) for l in range(cfg["n_layers"])], np.int64)
+    np.savez_compressed(os.path.join(HERE, "gemma4_small.npz"), **out)
+    print("wrote gemma4_small.npz", {k_: v_.shape for k_, v_ in out.items()})
+
+
 CFG4_SEED, PROMPT_SEED, N_PROMPT, N_NEW, KV_STEPS = 4000, 4001, 64, 256, 40
 
 
@@ -109,8 +151,12 @@ def cfg4(n_new=N_NEW):
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--cfg4", action="store_true")
+    ap.add_argument("--gemma4", action="store_true")
     ap.add_argument("--n-new", type=int, default=N_NEW)
     a = ap.parse_args()
-    small()
-    if a.cfg4:
-        cfg4(a.n_new)
+    if a.gemma4:
+        gemma4()
+    else:
+        small()
+        if a.cfg4:
+            cfg4(a.n_new)

@@ -109,6 +109,7 @@ __global__ __launch_bounds__(kGmWaves * 64) void q4k_gemv_gelu_mul_kernel(const 
     const int b0 = min(lane >> 2, bpr - 1);
     const uint8_t *blk0 = wr + (size_t)b0 * 144;
     uint4 hdr = ldg_u4(blk0, 0), q0 = ldg_u4(blk0 + 16 + 32 * g, 0), q1 = ldg_u4(blk0 + 16 + 32 * g, 1);
+    const float cr = ctx[row];   // fetched now: at the end it would be a cold round trip on the critical path
 
     // all of the vector's loads go out before anything is used (cols <= 8192: at most 8 float4 per thread and array)
     constexpr int KMAX = 8192 / 4 / (kGmWaves * 64);
@@ -171,7 +172,7 @@ __global__ __launch_bounds__(kGmWaves * 64) void q4k_gemv_gelu_mul_kernel(const 
         acc += d * ((float)s.x * lo + (float)s.z * hi) - dmin * ((float)s.y * sl + (float)s.w * sh);
     }
     acc = wave_sum(acc);
-    if (lane == 0 && blockIdx.x * kGmWaves + wave < rows) y[row] = gelu_mul_f32(acc, ctx[row]);
+    if (lane == 0 && blockIdx.x * kGmWaves + wave < rows) y[row] = gelu_mul_f32(acc, cr);
 }
 
 int launch_per_head(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)

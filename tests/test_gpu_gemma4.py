@@ -126,7 +126,7 @@ PATTERN = [1, 1, 0, 1, 1, 1, 0, 1]
 FFN = [1024, 1024, 2048, 1024, 1024, 1024, 2048, 1024]
 
 
-@pytest.fixture(scope="module", params=["all_q4k", "mixed_q6k", "no_ple"])
+@pytest.fixture(scope="module", params=["all_q4k", "mixed_q6k", "no_ple", "two_kv_heads", "wide_window"])
 def tiny(ctx, request):
     cfg = dict(synth.GEMMA4_TINY)
     q6 = ()
@@ -134,6 +134,11 @@ def tiny(ctx, request):
         q6 = {(1, "wv"), (2, "wdown"), (3, "wq"), (4, "wgate"), (5, "wo"), (6, "wup"), (7, "proj")}
     if request.param == "no_ple":
         cfg["ple_dim"] = 0
+    if request.param == "two_kv_heads":
+        cfg["n_kv"] = 2                     # grouped-query attention: two q heads per kv head
+    if request.param == "wide_window":
+        cfg["sliding_window"] = 700         # longer than the short-context form takes: the merging attention on every layer
+        cfg["max_seq"] = 800
     w = synth.gemma4_weights(cfg, 610, oracle.quantize_q4k, oracle.quantize_q6k, ffn=FFN, swa_pattern=PATTERN, q6k_tensors=q6, std=0.05)
     gpu, cpu = hip.Gemma4(ctx, cfg, w), oracle.Gemma4(cfg, w)
     yield gpu, cpu, cfg

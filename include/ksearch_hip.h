@@ -367,6 +367,11 @@ int ksh_gemma4_reset(ksh_gemma4 *m);
 int ksh_gemma4_forward_token(ksh_gemma4 *m, uint32_t token, int want_logits, int use_graph, uint32_t *next_id);
 int ksh_gemma4_generate(ksh_gemma4 *m, const uint32_t *prompt, int n_prompt, int n_new,
                         int use_graph, uint32_t *out_ids, double *prefill_ms, double *decode_ms);
+/* generate_timed with its stop rule (gemma_prim.rs:1683-1710; the reference stops at ids 1 and 106): ids are
+ * read one step behind the device, an id from `eos` ends the run and is the last of the *n_out ids written. */
+int ksh_gemma4_generate_until(ksh_gemma4 *m, const uint32_t *prompt, int n_prompt, int n_new,
+                              const uint32_t *eos, int n_eos, int use_graph, uint32_t *out_ids, int *n_out,
+                              double *prefill_ms, double *decode_ms);
 ksh_buf *ksh_gemma4_logits(ksh_gemma4 *m);
 ksh_buf *ksh_gemma4_hidden(ksh_gemma4 *m);
 /* kv_source(layer) (crates/ksearch_gemma/src/lib.rs:151-162) and that layer's cache */

@@ -575,6 +575,57 @@ int ksh_gemma4_generate(ksh_gemma4 *m, const uint32_t *prompt, int n_prompt, int
     return 0;
 }
 
+// generate_timed's stop rule (gemma_prim.rs:1683-1710): the id of step i-1 is read while step i runs, and an id
+// from `eos` ends the run with that id as the last output (the step already in flight is discarded; the model's
+// position has moved past it, as the reference's has).
+int ksh_gemma4_generate_until(ksh_gemma4 *m, const uint32_t *prompt, int n_prompt, int n_new, const uint32_t *eos, int n_eos,
+                              int use_graph, uint32_t *out_ids, int *n_out, double *prefill_ms, double *decode_ms)
+{
+    if (!m || !prompt || n_prompt < 1 || n_new < 0 || (n_new && !out_ids) || !n_out || n_eos < 0 || (n_eos && !eos))
+        return set_error("ksh_gemma4_generate_until: bad arguments");
+    *n_out = 0;
+    if (m->pos + n_prompt - 1 + n_new > m->c.max_seq) return set_error("max_seq exceeded");
+    for (int i = 0; i < n_prompt; i++)
+        if (prompt[i] >= (uint32_t)m->c.vocab) return set_error("token id %u is outside the vocabulary", prompt[i]);
+    using clk = std::chrono::steady_clock;
+    const auto t0 = clk::now();
+    for (int i = 0; i + 1 < n_prompt; i++) {
+        if (write_token(m, prompt[i])) return 1;
+        if (run_token(m, false, use_graph != 0)) return 1;
+    }
+    if (write_token(m, prompt[n_prompt - 1])) return 1;
+    if (ksh_synchronize(m->ctx)) return 1;
+    const auto t1 = clk::now();
+    const int first = m->pos;
+    auto is_eos = [&](uint32_t id) {
+        for (int e = 0; e < n_eos; e++)
+            if (eos[e] == id) return true;
+        return false;
+    };
+    auto take = [&](int step) -> int {   // the id step `step` produced (that step has completed)
+        float f = 0.f;
+        if (ksh_buffer_read(m->ctx, m->history, (size_t)(first + step) * 4, &f, 4, 0)) return -1;
+        out_ids[(*n_out)++] = (uint32_t)f;
+        return is_eos((uint32_t)f) ? 1 : 0;
+    };
+    bool stopped = false;
+    for (int i = 0; i < n_new && !stopped; i++) {
+        if (run_token(m, true, use_graph != 0) || ksh_flush_async(m->ctx)) return 1;
+        if (i > 0) {
+            if (ksh_wait_inflight_at_most(m->ctx, 1)) return 1;
+            const int r = take(i - 1);
+            if (r < 0) return 1;
+            stopped = r == 1;
+        }
+    }
+    if (ksh_synchronize(m->ctx)) return 1;
+    if (!stopped && n_new > 0 && take(n_new - 1) < 0) return 1;
+    const auto t2 = clk::now();
+    if (prefill_ms) *prefill_ms = std::chrono::duration<double, std::milli>(t1 - t0).count();
+    if (decode_ms) *decode_ms = std::chrono::duration<double, std::milli>(t2 - t1).count();
+    return 0;
+}
+
 ksh_buf *ksh_gemma4_logits(ksh_gemma4 *m) { return m ? m->logits : nullptr; }
 ksh_buf *ksh_gemma4_hidden(ksh_gemma4 *m) { return m ? (m->hidden ? m->hidden : m->x) : nullptr; }
 int ksh_gemma4_kv_source(ksh_gemma4 *m, int layer) { return (!m || layer < 0 || layer >= m->c.n_layers) ? -1 : m->plan[layer].src; }

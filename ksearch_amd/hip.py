@@ -171,6 +171,8 @@ SYMBOLS = {
     "ksh_gemma4_reset": (_i, [_vp]),
     "ksh_gemma4_forward_token": (_i, [_vp, C.c_uint32, _i, _i, C.POINTER(C.c_uint32)]),
     "ksh_gemma4_generate": (_i, [_vp, C.POINTER(C.c_uint32), _i, _i, _i, C.POINTER(C.c_uint32), _dp, _dp]),
+    "ksh_gemma4_generate_until": (_i, [_vp, C.POINTER(C.c_uint32), _i, _i, C.POINTER(C.c_uint32), _i, _i, C.POINTER(C.c_uint32),
+                                       C.POINTER(C.c_int), _dp, _dp]),
     "ksh_gemma4_logits": (_vp, [_vp]),
     "ksh_gemma4_hidden": (_vp, [_vp]),
     "ksh_gemma4_kv_source": (_i, [_vp, _i]),
@@ -953,6 +955,16 @@ class Gemma4:
         pre, dec = C.c_double(), C.c_double()
         _check(lib().ksh_gemma4_generate(self.h, p, len(prompt), n_new, int(use_graph), out, C.byref(pre), C.byref(dec)))
         return list(out[:n_new]), pre.value, dec.value
+
+    def generate_until(self, prompt, n_new: int, eos=(1, 106), use_graph: bool = True):
+        """generate_timed with its stop rule: ends after the first id from `eos` (which is the last one returned)."""
+        p = (C.c_uint32 * len(prompt))(*[int(t) for t in prompt])
+        e = (C.c_uint32 * max(1, len(eos)))(*[int(t) for t in eos])
+        out = (C.c_uint32 * max(1, n_new))()
+        n, pre, dec = C.c_int(), C.c_double(), C.c_double()
+        _check(lib().ksh_gemma4_generate_until(self.h, p, len(prompt), n_new, e, len(eos), int(use_graph), out, C.byref(n),
+                                               C.byref(pre), C.byref(dec)))
+        return list(out[:n.value]), pre.value, dec.value
 
     def logits(self) -> np.ndarray:
         b = Buffer(self.ctx, lib().ksh_gemma4_logits(self.h), owned=False)

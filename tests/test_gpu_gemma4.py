@@ -228,6 +228,15 @@ def test_gemma4_generate_graph_equals_eager_and_oracle(tiny):
     assert first_close >= 8
     with pytest.raises(hip.KshError, match="max_seq"):
         gpu.generate(prompt, cfg["max_seq"], use_graph=True)
+    # the stop rule: the run ends with the first id from the list, which is the last id returned
+    for stop_at in (0, 3, n_new - 1):
+        eos = [graph[stop_at], cfg["vocab"] - 1]
+        first = next(i for i, t in enumerate(graph) if t in eos)
+        gpu.reset()
+        got, _, _ = gpu.generate_until(prompt, n_new, eos=eos, use_graph=True)
+        assert got == graph[:first + 1], stop_at
+    gpu.reset()
+    assert gpu.generate_until(prompt, n_new, eos=(), use_graph=False)[0] == graph     # nothing to stop at: the whole run
 
 
 def test_gemma4_create_errors(ctx):

@@ -381,6 +381,12 @@ int ksh_gemma4_pos(ksh_gemma4 *m);
 int ksh_gemma4_launches_per_token(ksh_gemma4 *m);
 int ksh_gemma4_config(ksh_gemma4 *m, ksh_gemma4_cfg *cfg);
 
+/* sample_softcap_min_p (crates/ksearch_gemma/src/sample.rs:9-77), the host-side sampler of forward_token's
+ * non-greedy branch, on f32 logits read back from ksh_gemma4_logits: cap*tanh(x/cap), softmax at `temperature`,
+ * ids below min_p * p_max dropped, one splitmix32 draw from `seed`.  temperature < 1e-6 is the greedy argmax. */
+int ksh_sample_softcap_min_p(const float *logits, size_t n, float cap, float temperature, float min_p,
+                             uint32_t seed, uint32_t *out);
+
 /* ---- GGUF files: Gguf::open and its accessors (crates/ksearch_gguf/src/gguf_impl.rs:217-420).  The file is
  * memory-mapped; tensor data pointers stay valid until ksh_gguf_close.  A malformed file is an error here where
  * the reference panics. ---- */

@@ -180,6 +180,7 @@ SYMBOLS = {
     "ksh_gemma4_pos": (_i, [_vp]),
     "ksh_gemma4_launches_per_token": (_i, [_vp]),
     "ksh_gemma4_config": (_i, [_vp, C.POINTER(Gemma4Cfg)]),
+    "ksh_sample_softcap_min_p": (_i, [_vp, _sz, C.c_float, C.c_float, C.c_float, C.c_uint32, C.POINTER(C.c_uint32)]),
     "ksh_gguf_open": (_i, [C.c_char_p, _vpp]),
     "ksh_gguf_close": (None, [_vp]),
     "ksh_gguf_version": (_i, [_vp]),
@@ -856,6 +857,14 @@ class Gguf:
         _check(lib().ksh_gemma4_config_from_gguf(self.h, max_seq, C.byref(c), ffn, swa, 4096))
         cfg = {k: getattr(c, k) for k in GEMMA4_CFG_INTS + GEMMA4_CFG_FLOATS}
         return cfg, list(ffn[:c.n_layers]), [bool(v) for v in swa[:c.n_layers]]
+
+
+def sample_softcap_min_p(logits: np.ndarray, cap: float, temperature: float, min_p: float = 0.05, seed: int = 1) -> int:
+    """crates/ksearch_gemma/src/sample.rs:9-77 on f32 logits (host)."""
+    x = np.ascontiguousarray(logits, dtype=np.float32)
+    out = C.c_uint32()
+    _check(lib().ksh_sample_softcap_min_p(x.ctypes.data, x.size, cap, temperature, min_p, seed, C.byref(out)))
+    return out.value
 
 
 def gguf_dequant_host(ggml_type: int, raw: np.ndarray, n: int) -> np.ndarray:

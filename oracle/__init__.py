@@ -69,6 +69,7 @@ def lib() -> C.CDLL:
             "ko_gemma_pos": (i32, [vp]),
             "ko_gemma_kv": (vp, [vp, i32, i32]),
             "ko_gemma_hidden": (vp, [vp]),
+            "ko_sample_softcap_min_p": (u32, [vp, sz, f32, f32, f32, u32]),
             "ko_rmsnorm_per_head": (None, [vp, vp, vp, i32, i32, f32, vp]),
             "ko_add_scale": (None, [vp, vp, f32, sz, vp]),
             "ko_matvec_gelu_mul": (i32, [i32, vp, sz, sz, vp, vp, vp, i32]),
@@ -425,3 +426,8 @@ class Gemma4:
             self.close()
         except Exception:
             pass
+
+
+def sample_softcap_min_p(logits, cap, temperature, min_p=0.05, seed=1) -> int:
+    x = _f32(logits)
+    return lib().ko_sample_softcap_min_p(_p(x), x.size, cap, temperature, min_p, seed)

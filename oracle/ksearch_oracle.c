@@ -1086,3 +1086,61 @@ uint32_t ko_gemma4_forward(ko_gemma4 *m, uint32_t token, int want_logits, float 
     if (logits_out) memcpy(logits_out, m->logits, sizeof(float) * (size_t)c->vocab);
     return ko_softcap_argmax(m->logits, (size_t)c->vocab, c->softcap);
 }
+
+/* ------------------------------------------------------------------ sampler */
+
+/* sample.rs:79-85 */
+static uint32_t splitmix32(uint32_t *state)
+{
+    *state += 0x9E3779B9u;
+    uint32_t z = *state;
+    z = (z ^ (z >> 16)) * 0x7feb352du;
+    z = (z ^ (z >> 15)) * 0x846ca68bu;
+    return z ^ (z >> 16);
+}
+
+/* sample.rs:9-77 */
+uint32_t ko_sample_softcap_min_p(const float *logits, size_t n, float cap, float temperature,
+                                 float min_p, uint32_t seed)
+{
+    uint32_t best_i = 0;
+    float best_v = -INFINITY;
+    float *xs = (float *)malloc(sizeof(float) * n);
+    for (size_t i = 0; i < n; i++) {
+        float x = logits[i];
+        float y = cap > 0.0f ? cap * tanhf(x / cap) : x;
+        xs[i] = y;
+        if (y > best_v) { best_v = y; best_i = (uint32_t)i; }
+    }
+    if (temperature < 1e-6f) { free(xs); return best_i; }
+    float sum = 0.0f;
+    for (size_t i = 0; i < n; i++) {
+        xs[i] = expf((xs[i] - best_v) / temperature);
+        sum += xs[i];
+    }
+    float inv = 1.0f / fmaxf(sum, 1e-30f);
+    float p_max = 0.0f;
+    for (size_t i = 0; i < n; i++) {
+        xs[i] *= inv;
+        if (xs[i] > p_max) p_max = xs[i];
+    }
+    float threshold = p_max * fmaxf(min_p, 0.0f);
+    float filtered = 0.0f;
+    for (size_t i = 0; i < n; i++) {
+        if (xs[i] < threshold) xs[i] = 0.0f;
+        else filtered += xs[i];
+    }
+    uint32_t pick = best_i;
+    if (filtered > 1e-9f) {
+        uint32_t rng = seed | 1u;
+        float r = ((float)splitmix32(&rng) / 4294967296.0f) * filtered;
+        float cdf = 0.0f;
+        pick = (uint32_t)(n - 1);
+        for (size_t i = 0; i < n; i++) {
+            cdf += xs[i];
+            if (r < cdf) { pick = (uint32_t)i; break; }
+        }
+    }
+    free(xs);
+    return pick;
+}

@@ -39,6 +39,8 @@
  *                            the extras are off; kv_source vs the rule restated;
  *                            the window: equal to a wide-window run for exactly
  *                            `window` positions
+ *   ko_sample_softcap_min_p  the reference's three unit tests restated (sample.rs:87-117),
+ *                            the draw's distribution against the closed-form softmax
  *   ko_quantize_q4k          reference round-trip test only (output bytes of
  *                            the iterative search are PARITY UNPINNED; they
  *                            never enter a GPU-vs-oracle comparison because
@@ -152,6 +154,10 @@ int ko_gemma_pos(const ko_gemma *m);
 const uint8_t *ko_gemma_kv(const ko_gemma *m, int layer, int which);
 /* last token's hidden state after the final layer (before output norm) */
 const float *ko_gemma_hidden(const ko_gemma *m);
+
+/* crates/ksearch_gemma/src/sample.rs:9-77 on f32 logits: soft cap, temperature, min-p, one splitmix32 draw */
+uint32_t ko_sample_softcap_min_p(const float *logits, size_t n, float cap, float temperature,
+                                 float min_p, uint32_t seed);
 
 /* ---- ops the real Gemma-4 checkpoints add to the decode step ---- */
 /* Eng::rmsnorm_per_head / rmsnorm_per_head_rope_off (crates/ksearch_kernels/src/lib.rs:564-625;

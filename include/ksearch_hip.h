@@ -381,6 +381,29 @@ int ksh_gemma4_pos(ksh_gemma4 *m);
 int ksh_gemma4_launches_per_token(ksh_gemma4 *m);
 int ksh_gemma4_config(ksh_gemma4 *m, ksh_gemma4_cfg *cfg);
 
+/* ---- KV slots for serving several sequences from one set of weights: KvPool, Q4_0 form
+ * (crates/ksearch_gemma/src/kv_pool.rs:24-228).  max_batch slots x n_kv_layers x (K, V), each
+ * max_seq * n_kv * (hd/32) * 18 bytes; the first free slot is handed out, freed slots are reused, the caller bumps
+ * a slot's sequence length after the tokens it has run (kv_pool.rs:196-228), as the reference's scheduler does. ---- */
+typedef struct ksh_kvpool ksh_kvpool;
+int ksh_kvpool_create(ksh_ctx *ctx, int max_batch, int max_seq, int n_kv_layers, int hd, int n_kv, ksh_kvpool **out);
+void ksh_kvpool_destroy(ksh_kvpool *p);
+int ksh_kvpool_alloc(ksh_kvpool *p, int *slot);          /* error "KvPool full (max_batch=N)" */
+int ksh_kvpool_free(ksh_kvpool *p, int slot);
+int ksh_kvpool_clear_slot(ksh_kvpool *p, int slot);      /* zero the slot's caches (a fill kernel on the stream) */
+int ksh_kvpool_seq_len(const ksh_kvpool *p, int slot);   /* -1: bad slot */
+int ksh_kvpool_occupied(const ksh_kvpool *p, int slot);
+int ksh_kvpool_bump_len_by(ksh_kvpool *p, int slot, int n, int *new_len);
+int ksh_kvpool_active_batch(const ksh_kvpool *p, int *slots, int cap);   /* returns the count */
+ksh_buf *ksh_kvpool_k(const ksh_kvpool *p, int slot, int layer);
+ksh_buf *ksh_kvpool_v(const ksh_kvpool *p, int slot, int layer);
+int ksh_kvpool_dims(const ksh_kvpool *p, int *max_batch, int *max_seq, int *n_kv_layers, int *hd, int *n_kv);
+/* GemmaPrimModel::bind_slot (gemma_prim.rs:1277-1292): the model's caches become the slot's (the pool needs one
+ * layer per cache-owning layer and hd >= the larger head dim) and its position the slot's sequence length; the
+ * device-side position follows on the stream.  Graphs are captured once per slot.  pool = NULL: back to the
+ * model's own caches, at position `slot`. */
+int ksh_gemma4_bind_slot(ksh_gemma4 *m, ksh_kvpool *pool, int slot);
+
 /* sample_softcap_min_p (crates/ksearch_gemma/src/sample.rs:9-77), the host-side sampler of forward_token's
  * non-greedy branch, on f32 logits read back from ksh_gemma4_logits: cap*tanh(x/cap), softmax at `temperature`,
  * ids below min_p * p_max dropped, one splitmix32 draw from `seed`.  temperature < 1e-6 is the greedy argmax. */

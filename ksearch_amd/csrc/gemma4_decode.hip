@@ -48,6 +48,19 @@ __global__ void advance4_kernel(float *meta_full, float *meta_swa, const float *
     }
 }
 
+// points the device-side state at position `pos` (a model that is bound to another sequence's KV slot)
+__global__ void seek4_kernel(float *meta_full, float *meta_swa, int pos, const float *rope_full, float *cur_full, int hd_full,
+                             const float *rope_swa, float *cur_swa, int hd_swa, int window)
+{
+    for (int i = threadIdx.x; i < hd_full; i += blockDim.x) cur_full[i] = rope_full[(size_t)pos * hd_full + i];
+    for (int i = threadIdx.x; i < hd_swa; i += blockDim.x) cur_swa[i] = rope_swa[(size_t)pos * hd_swa + i];
+    if (threadIdx.x == 0) {
+        const int kv_len = pos + 1, start = kv_len > window ? kv_len - window : 0;
+        meta_full[0] = (float)kv_len; meta_full[1] = 0.f; meta_full[2] = 0.f; meta_full[3] = (float)pos;
+        meta_swa[0] = (float)(kv_len - start); meta_swa[1] = (float)start; meta_swa[2] = (float)window; meta_swa[3] = (float)pos;
+    }
+}
+
 __global__ void set_token4_kernel(float *tok, float value)
 {
     if (threadIdx.x == 0 && blockIdx.x == 0) tok[0] = value;
@@ -92,9 +105,16 @@ struct ksh_gemma4 {
     std::vector<ksh_buf *> kv_k, kv_v;   // per layer; null where the layer reads another layer's cache
     ksh_kernel *k_embed = nullptr, *k_ple_gather = nullptr, *k_ple_proj = nullptr, *k_ple_norm = nullptr, *k_ple_mix = nullptr,
                *k_lm_head[2] = {nullptr, nullptr}, *k_argmax = nullptr;
-    ksh_graph *g_body = nullptr, *g_full = nullptr;
+    ksh_graph *g_body = nullptr, *g_full = nullptr;   // the graphs of the caches in use (own or a pool slot's)
     std::vector<float> rope0_full, rope0_swa;
     int pos = 0, launches_full = 0;
+    // serving: the model's own caches, and the graphs captured for each slot of the pool it was last bound to
+    std::vector<ksh_buf *> own_k, own_v;
+    struct SlotGraphs { ksh_graph *body = nullptr, *full = nullptr; };
+    ksh_kvpool *pool = nullptr;
+    std::vector<SlotGraphs> slot_graphs;
+    SlotGraphs own_graphs;
+    int bound_slot = -1;
 };
 
 namespace {
@@ -426,6 +446,15 @@ int plan_layer(ksh_gemma4 *m, int l)
     return 0;
 }
 
+// puts the graphs in use back where they belong (they are tied to the cache buffers they were captured with)
+void stash_graphs(ksh_gemma4 *m)
+{
+    ksh_gemma4::SlotGraphs &g = m->bound_slot >= 0 ? m->slot_graphs[(size_t)m->bound_slot] : m->own_graphs;
+    g.body = m->g_body;
+    g.full = m->g_full;
+    m->g_body = m->g_full = nullptr;
+}
+
 }  // namespace
 
 extern "C" {
@@ -510,8 +539,10 @@ void ksh_gemma4_destroy(ksh_gemma4 *m)
 {
     if (!m) return;
     ksh_synchronize(m->ctx);
-    ksh_graph_destroy(m->g_body);
-    ksh_graph_destroy(m->g_full);
+    stash_graphs(m);
+    ksh_graph_destroy(m->own_graphs.body);
+    ksh_graph_destroy(m->own_graphs.full);
+    for (auto &g : m->slot_graphs) { ksh_graph_destroy(g.body); ksh_graph_destroy(g.full); }
     delete m;
 }
 
@@ -624,6 +655,55 @@ int ksh_gemma4_generate_until(ksh_gemma4 *m, const uint32_t *prompt, int n_promp
     if (prefill_ms) *prefill_ms = std::chrono::duration<double, std::milli>(t1 - t0).count();
     if (decode_ms) *decode_ms = std::chrono::duration<double, std::milli>(t2 - t1).count();
     return 0;
+}
+
+// GemmaPrimModel::bind_slot (gemma_prim.rs:1277-1292): the model's K / V caches become the slot's and its position the
+// slot's sequence length.  pool == NULL goes back to the model's own caches at position `slot` (0 after a reset).
+int ksh_gemma4_bind_slot(ksh_gemma4 *m, ksh_kvpool *pool, int slot)
+{
+    if (!m) return set_error("ksh_gemma4_bind_slot: null model");
+    const ksh_gemma4_cfg &c = m->c;
+    const int owners = c.n_layers - c.shared_kv_layers;
+    int pos = slot;
+    if (pool) {
+        int max_batch, max_seq, n_kv_layers, hd, n_kv;
+        if (ksh_kvpool_dims(pool, &max_batch, &max_seq, &n_kv_layers, &hd, &n_kv)) return 1;
+        if (n_kv_layers != owners) return set_error("kv layer mismatch: model=%d pool=%d", owners, n_kv_layers);
+        if (max_seq != c.max_seq || n_kv != c.n_kv || hd < std::max(c.hd_swa, c.hd_full))
+            return set_error("KvPool(max_seq=%d, n_kv=%d, hd=%d) does not fit the model (max_seq=%d, n_kv=%d, hd=%d)", max_seq, n_kv, hd,
+                             c.max_seq, c.n_kv, std::max(c.hd_swa, c.hd_full));
+        if (slot < 0 || slot >= max_batch) return set_error("bad SlotId");
+        pos = ksh_kvpool_seq_len(pool, slot);
+    }
+    if (pos < 0 || pos > c.max_seq) return set_error("ksh_gemma4_bind_slot: position %d", pos);
+    stash_graphs(m);
+    if (pool && pool != m->pool) {
+        // graphs captured over another pool's buffers are of no use any more
+        if (ksh_synchronize(m->ctx)) return 1;
+        for (auto &g : m->slot_graphs) { ksh_graph_destroy(g.body); ksh_graph_destroy(g.full); }
+        int max_batch = 0;
+        ksh_kvpool_dims(pool, &max_batch, nullptr, nullptr, nullptr, nullptr);
+        m->slot_graphs.assign((size_t)max_batch, ksh_gemma4::SlotGraphs{});
+        m->pool = pool;
+    }
+    if (m->own_k.empty()) { m->own_k = m->kv_k; m->own_v = m->kv_v; }
+    for (int l = 0; l < owners; l++) {
+        m->kv_k[l] = pool ? ksh_kvpool_k(pool, slot, l) : m->own_k[l];
+        m->kv_v[l] = pool ? ksh_kvpool_v(pool, slot, l) : m->own_v[l];
+    }
+    m->bound_slot = pool ? slot : -1;
+    const ksh_gemma4::SlotGraphs &g = pool ? m->slot_graphs[(size_t)slot] : m->own_graphs;
+    m->g_body = g.body;
+    m->g_full = g.full;
+    m->pos = pos;
+    // the device-side position, attended ranges and rope rows, ordered behind whatever is still running
+    const int at = std::min(pos, c.max_seq - 1);
+    hipLaunchKernelGGL(seek4_kernel, dim3(1), dim3(64), 0, (hipStream_t)ksh_stream(m->ctx), (float *)ksh_buffer_device_ptr(m->meta_full),
+                       (float *)ksh_buffer_device_ptr(m->meta_swa), at, (const float *)ksh_buffer_device_ptr(m->rope_full),
+                       (float *)ksh_buffer_device_ptr(m->cur_full), c.hd_full, (const float *)ksh_buffer_device_ptr(m->rope_swa),
+                       (float *)ksh_buffer_device_ptr(m->cur_swa), c.hd_swa, c.sliding_window);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : hip_fail(e, "seek launch");
 }
 
 ksh_buf *ksh_gemma4_logits(ksh_gemma4 *m) { return m ? m->logits : nullptr; }

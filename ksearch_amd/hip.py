@@ -180,6 +180,19 @@ SYMBOLS = {
     "ksh_gemma4_pos": (_i, [_vp]),
     "ksh_gemma4_launches_per_token": (_i, [_vp]),
     "ksh_gemma4_config": (_i, [_vp, C.POINTER(Gemma4Cfg)]),
+    "ksh_kvpool_create": (_i, [_vp, _i, _i, _i, _i, _i, _vpp]),
+    "ksh_kvpool_destroy": (None, [_vp]),
+    "ksh_kvpool_alloc": (_i, [_vp, C.POINTER(C.c_int)]),
+    "ksh_kvpool_free": (_i, [_vp, _i]),
+    "ksh_kvpool_clear_slot": (_i, [_vp, _i]),
+    "ksh_kvpool_seq_len": (_i, [_vp, _i]),
+    "ksh_kvpool_occupied": (_i, [_vp, _i]),
+    "ksh_kvpool_bump_len_by": (_i, [_vp, _i, _i, C.POINTER(C.c_int)]),
+    "ksh_kvpool_active_batch": (_i, [_vp, C.POINTER(C.c_int), _i]),
+    "ksh_kvpool_k": (_vp, [_vp, _i, _i]),
+    "ksh_kvpool_v": (_vp, [_vp, _i, _i]),
+    "ksh_kvpool_dims": (_i, [_vp] + [C.POINTER(C.c_int)] * 5),
+    "ksh_gemma4_bind_slot": (_i, [_vp, _vp, _i]),
     "ksh_sample_softcap_min_p": (_i, [_vp, _sz, C.c_float, C.c_float, C.c_float, C.c_uint32, C.POINTER(C.c_uint32)]),
     "ksh_gguf_open": (_i, [C.c_char_p, _vpp]),
     "ksh_gguf_close": (None, [_vp]),
@@ -874,6 +887,51 @@ def gguf_dequant_host(ggml_type: int, raw: np.ndarray, n: int) -> np.ndarray:
     return out
 
 
+class KvPool:
+    """KvPool, Q4_0 form (crates/ksearch_gemma/src/kv_pool.rs)."""
+
+    def __init__(self, ctx: Context, max_batch: int, max_seq: int, n_kv_layers: int, hd: int, n_kv: int):
+        self.ctx = ctx
+        h = C.c_void_p()
+        _check(lib().ksh_kvpool_create(ctx.h, max_batch, max_seq, n_kv_layers, hd, n_kv, C.byref(h)))
+        self.h, self.max_batch = h, max_batch
+
+    def close(self):
+        if self.h:
+            lib().ksh_kvpool_destroy(self.h)
+            self.h = None
+
+    def alloc(self) -> int:
+        s = C.c_int()
+        _check(lib().ksh_kvpool_alloc(self.h, C.byref(s)))
+        return s.value
+
+    def free(self, slot: int):
+        _check(lib().ksh_kvpool_free(self.h, slot))
+
+    def clear_slot(self, slot: int):
+        _check(lib().ksh_kvpool_clear_slot(self.h, slot))
+
+    def seq_len(self, slot: int) -> int:
+        return lib().ksh_kvpool_seq_len(self.h, slot)
+
+    def bump_len(self, slot: int, n: int = 1) -> int:
+        out = C.c_int()
+        _check(lib().ksh_kvpool_bump_len_by(self.h, slot, n, C.byref(out)))
+        return out.value
+
+    def active_batch(self) -> list:
+        arr = (C.c_int * self.max_batch)()
+        n = lib().ksh_kvpool_active_batch(self.h, arr, self.max_batch)
+        return list(arr[:n])
+
+    def k_buf(self, slot: int, layer: int) -> Buffer:
+        return Buffer(self.ctx, lib().ksh_kvpool_k(self.h, slot, layer), owned=False)
+
+    def v_buf(self, slot: int, layer: int) -> Buffer:
+        return Buffer(self.ctx, lib().ksh_kvpool_v(self.h, slot, layer), owned=False)
+
+
 class Gemma4:
     """GemmaPrimModel with the layer features of the real Gemma-4 checkpoints
     (crates/ksearch_gemma/src/gemma_prim.rs:881-1275; crates/ksearch_gemma/src/lib.rs:39-167).
@@ -964,6 +1022,10 @@ class Gemma4:
         pre, dec = C.c_double(), C.c_double()
         _check(lib().ksh_gemma4_generate(self.h, p, len(prompt), n_new, int(use_graph), out, C.byref(pre), C.byref(dec)))
         return list(out[:n_new]), pre.value, dec.value
+
+    def bind_slot(self, pool, slot: int):
+        """GemmaPrimModel::bind_slot; pool=None goes back to the model's own caches at position `slot`."""
+        _check(lib().ksh_gemma4_bind_slot(self.h, pool.h if pool is not None else None, slot))
 
     def generate_until(self, prompt, n_new: int, eos=(1, 106), use_graph: bool = True):
         """generate_timed with its stop rule: ends after the first id from `eos` (which is the last one returned)."""

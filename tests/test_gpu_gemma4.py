@@ -376,3 +376,80 @@ def test_gemma4_real_widths_long_run_matches_oracle(ctx, eng):
     assert clean >= 24 and agree >= 12, (clean, agree)
     gpu.close()
     cpu.close()
+
+
+def test_kvpool_slot_rules(ctx):
+    """kv_pool.rs:232-248 restated (first free slot, a freed slot is reused), the bump and bounds rules, clear_slot."""
+    pool = hip.KvPool(ctx, 4, 64, 2, 256, 1)
+    a, b = pool.alloc(), pool.alloc()
+    assert a != b and len(pool.active_batch()) == 2
+    pool.free(a)
+    assert pool.active_batch() == [b]
+    assert pool.alloc() == a
+    assert pool.bump_len(a, 5) == 5 and pool.bump_len(a) == 6 and pool.seq_len(a) == 6 and pool.seq_len(b) == 0
+    with pytest.raises(hip.KshError, match="slot seq full"):
+        pool.bump_len(a, 59)
+    pool.alloc(), pool.alloc()
+    with pytest.raises(hip.KshError, match=r"KvPool full \(max_batch=4\)"):
+        pool.alloc()
+    pool.free(b)
+    with pytest.raises(hip.KshError, match="slot not occupied"):
+        pool.bump_len(b)
+    with pytest.raises(hip.KshError, match="bad SlotId"):
+        pool.free(9)
+    assert pool.seq_len(9) == -1
+    nbytes = 64 * 1 * 8 * 18
+    ctx.write_bytes(pool.k_buf(a, 1), np.full(nbytes, 0xAB, np.uint8))
+    pool.clear_slot(a)
+    assert not ctx.read_bytes(pool.k_buf(a, 1), nbytes).any() and pool.k_buf(a, 1).nbytes == nbytes
+    pool.close()
+    with pytest.raises(hip.KshError, match="non-zero"):
+        hip.KvPool(ctx, 0, 64, 2, 256, 1)
+
+
+def test_gemma4_two_sequences_interleaved_through_pool_slots(tiny):
+    """One model, two sequences in two pool slots, advanced in turn (bind_slot, one token, bump): each produces the
+    tokens it produces alone, through the captured per-slot graphs and eagerly; then the model goes back to its own
+    caches."""
+    gpu, _, cfg = tiny
+    ctx = gpu.ctx
+    rng = np.random.default_rng(640)
+    prompts = [[int(t) for t in rng.integers(0, cfg["vocab"], n)] for n in (5, 9)]
+    n_new = 14
+    alone = []
+    for p in prompts:
+        gpu.bind_slot(None, 0)
+        gpu.reset()
+        alone.append(gpu.generate(p, n_new, use_graph=True)[0])
+    owners = cfg["n_layers"] - cfg["shared_kv_layers"]
+    pool = hip.KvPool(ctx, 3, cfg["max_seq"], owners, max(cfg["hd_swa"], cfg["hd_full"]), cfg["n_kv"])
+    for use_graph in (True, False):
+        slots = [pool.alloc(), pool.alloc()]
+        for s_ in slots:
+            pool.clear_slot(s_)
+        feed = [list(p) for p in prompts]           # tokens still to be fed; the last fed token's successor is appended
+        outs = [[], []]
+        while any(len(o) < n_new for o in outs):
+            for i, s_ in enumerate(slots):
+                if len(outs[i]) >= n_new:
+                    continue
+                gpu.bind_slot(pool, s_)
+                assert gpu.pos == pool.seq_len(s_)
+                tok = feed[i].pop(0)
+                last_of_prompt = not feed[i]
+                nxt = gpu.forward_token(tok, want_logits=last_of_prompt, use_graph=use_graph)
+                pool.bump_len(s_)
+                if last_of_prompt:
+                    outs[i].append(nxt)
+                    feed[i].append(nxt)
+        assert outs == alone, use_graph
+        for s_ in slots:
+            pool.free(s_)
+    with pytest.raises(hip.KshError, match="kv layer mismatch"):
+        gpu.bind_slot(hip.KvPool(ctx, 1, cfg["max_seq"], owners + 1, 256, cfg["n_kv"]), 0)
+    with pytest.raises(hip.KshError, match="bad SlotId"):
+        gpu.bind_slot(pool, 7)
+    gpu.bind_slot(None, 0)
+    gpu.reset()
+    assert gpu.generate(prompts[0], n_new, use_graph=True)[0] == alone[0]
+    pool.close()

@@ -401,7 +401,8 @@ int ksh_kvpool_dims(const ksh_kvpool *p, int *max_batch, int *max_seq, int *n_kv
 /* GemmaPrimModel::bind_slot (gemma_prim.rs:1277-1292): the model's caches become the slot's (the pool needs one
  * layer per cache-owning layer and hd >= the larger head dim) and its position the slot's sequence length; the
  * device-side position follows on the stream.  Graphs are captured once per slot.  pool = NULL: back to the
- * model's own caches, at position `slot`. */
+ * model's own caches, at position `slot`.  The pool must outlive the binding (and the model's graphs over it:
+ * bind to another pool or to NULL before destroying it). */
 int ksh_gemma4_bind_slot(ksh_gemma4 *m, ksh_kvpool *pool, int slot);
 
 /* sample_softcap_min_p (crates/ksearch_gemma/src/sample.rs:9-77), the host-side sampler of forward_token's

@@ -199,7 +199,11 @@ int ksh_gguf_open(const char *path, ksh_gguf **out)
         size_t e, b;
         if (!ggml_block(t.type, e, b)) continue;   // unknown types are refused when asked for
         uint64_t n = 1;
-        for (uint64_t d : t.dims) n *= d;
+        for (uint64_t d : t.dims) {
+            // (a product that does not fit 64 bits cannot be a tensor of this file)
+            if (d && n > (uint64_t)g->size * 256 / d) return set_error("tensor %s lies outside the file", t.name.c_str());
+            n *= d;
+        }
         if (n % e) return set_error("tensor %s elems %llu not divisible by block %zu", t.name.c_str(), (unsigned long long)n, e);
         const uint64_t bytes = n / e * b;
         if (g->data_offset > g->size || t.offset > g->size - g->data_offset || bytes > g->size - g->data_offset - t.offset)

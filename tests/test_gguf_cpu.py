@@ -60,6 +60,10 @@ def test_reader_rejects_malformed_files(tmp_path):
     gw.write(p, [], [("t", GgmlType.Q4_K, (100,), np.zeros(144, np.uint8))])
     with pytest.raises(hip.KshError, match="not divisible by block"):
         hip.Gguf(p)
+    # dims whose product overflows 64 bits
+    gw.write(p, [], [("huge", GgmlType.F32, (2 ** 40, 2 ** 40), np.zeros(8, np.float32))])
+    with pytest.raises(hip.KshError, match="outside the file"):
+        hip.Gguf(p)
     with pytest.raises(hip.KshError, match="failed to open"):
         hip.Gguf(str(tmp_path / "missing.gguf"))
     # a type this reader does not know is refused when the tensor is asked for, not at open

@@ -119,20 +119,27 @@ def bench_lm_head(ctx, eng, ev):
 
 
 def bench_prefill(ctx):
-    """cfg2: 512 bf16 tokens x Q4_K [8192 x 2048] -> f32, hipEvent average of 50 launches."""
+    """cfg2: 512 bf16 tokens x Q4_K [8192 x 2048] -> f32, hipEvent average of 50 launches; the same shape over
+    Q6_K weights beside it."""
     from ksearch_amd import hip, synth
 
     tokens, rows, cols = 512, 8192, 2048
     w, _, xb = synth.cfg2_q4k_prefill()
-    bw, bx, by = ctx.buffer_bytes(w), ctx.buffer_bytes(xb), ctx.buffer_empty_f32(tokens * rows)
-    k = ctx.compile(hip.make_desc(hip.Kind.MATVEC_BATCH, (rows, cols, tokens),
-                                  (hip.DType.Q4K, hip.DType.BF16, hip.DType.F32)))
-    ctx.run(k, [bw, bx], [by], iters=5)
-    ms = ctx.run(k, [bw, bx], [by], iters=50)
-    tf = 2.0 * tokens * rows * cols / (ms * 1e-3) / 1e12
-    for b in (bw, bx, by):
-        b.release()
-    return dict(kernel=k.name, us_per_launch=round(ms * 1e3, 2), tflops=round(tf, 1), frac_mfma_f16=round(tf / 2500.0, 4))
+    out = {}
+    for dt, wq in ((hip.DType.Q4K, w), (hip.DType.Q6K, synth.q6k_blocks(rows * cols // 256, seed=1012))):
+        bw, bx, by = ctx.buffer_bytes(wq), ctx.buffer_bytes(xb), ctx.buffer_empty_f32(tokens * rows)
+        k = ctx.compile(hip.make_desc(hip.Kind.MATVEC_BATCH, (rows, cols, tokens), (dt, hip.DType.BF16, hip.DType.F32)))
+        ctx.run(k, [bw, bx], [by], iters=5)
+        ms = ctx.run(k, [bw, bx], [by], iters=50)
+        tf = 2.0 * tokens * rows * cols / (ms * 1e-3) / 1e12
+        for b in (bw, bx, by):
+            b.release()
+        r = dict(kernel=k.name, us_per_launch=round(ms * 1e3, 2), tflops=round(tf, 1), frac_mfma_f16=round(tf / 2500.0, 4))
+        if dt == hip.DType.Q4K:
+            out = r
+        else:
+            out["q6k_weights"] = r
+    return out
 
 
 def bench_attention(ctx):

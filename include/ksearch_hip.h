@@ -56,7 +56,8 @@ enum ksh_kind {
      * dtypes[0] = Q4K | Q6K.  in: W, x   out: y[rows] */
     KSH_MATVEC = 1,
     /* MatvecBatch: Y[t,r] = sum_c W[r,c] X[t,c].  dims: rows, cols, batch.
-     * dtypes[0] = Q4K, dtypes[1] = BF16 (X), output F32 token-major.
+     * dtypes[0] = Q4K | Q6K (GGUF byte order, blocks at 2-byte alignment),
+     * dtypes[1] = BF16 (X), output F32 token-major.
      * in: W, X   out: Y[batch, rows] */
     KSH_MATVEC_BATCH = 2,
     /* MatvecQkv: three GEMVs sharing x.  dims: q_rows, kv_rows, cols.

@@ -39,6 +39,8 @@ namespace {
 
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef float f16v __attribute__((ext_vector_type(16)));
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 
 constexpr int BM = 128, BN = 128, KS = 64;
 constexpr int PITCH = KS + 8;      // halves per LDS row of the main tiles (144 B: conflict-free 16 B reads)
@@ -124,7 +126,15 @@ constexpr size_t kLdsBytes = 2 * (size_t)(kLdsMain + kLdsMin) * 2 + 2 * BN * 4;
 // role's matrix instructions.  The min-term operands of a superblock are
 // written together with its first step into their own double buffer and
 // consumed after its fourth.
-__global__ __launch_bounds__(kThreadsMM) void q4k_mul_mm_kernel(MmParams p)
+//
+// Q6 = true: the same tile and roles over Q6_K weights (K3b of the reference's plan: Q6_K tensors in prefill).
+// w = d * sc_j * q with q = code - 32 in [-32, 31] and sc_j an int8 per 16 columns; the loaders build the f16
+// pair (1024 + code) by an OR into the mantissa, subtract 1056 and multiply by sc_j, both as packed f16.
+// sc_j * q is exact in f16 up to 2048; beyond that (needs |sc_j| > 64) it rounds to the nearest even integer, a
+// relative 2^-11 at most and on those weights only (the reference's tile rounds every weight to half, the same
+// bound).  There is no min term, so the short second product is skipped; d is applied per superblock as for Q4_K.
+template <bool Q6>
+__global__ __launch_bounds__(kThreadsMM) void q_mul_mm_kernel(MmParams p)
 {
     extern __shared__ __attribute__((aligned(16))) _Float16 lds[];
     auto main_stage = [&](int i) { return lds + (i & 1) * kLdsMain; };
@@ -135,7 +145,90 @@ __global__ __launch_bounds__(kThreadsMM) void q4k_mul_mm_kernel(MmParams p)
     const int t0 = blockIdx.x * BM, r0 = blockIdx.y * BN;
     const int nsb = p.cols / 256, nsteps = nsb * 4;
 
-    if (wave >= 4) {
+    if (Q6 && wave >= 4) {
+        // ------------------------------------------------------------------ loaders, Q6_K
+        // thread lh of a row's pair converts columns 32*lh .. 32*lh+31 of every 64-column step: step (h, part)
+        // of a superblock = ql bytes 64h + 32lh .. +31 (nibble `part`), qh bytes 32h .. +31 (bit pair
+        // 4*part + 2*lh), scales 8h + 4*part + 2*lh and the next one.  Blocks are 2-byte aligned.
+        const int lt = tid - 256, lrow = lt >> 1, lh = lt & 1;
+        const size_t row_bytes = (size_t)nsb * 210;
+        const uint8_t *wrow = p.W + (size_t)min(r0 + lrow, p.rows - 1) * row_bytes;
+        struct Sb6Regs {
+            u32x2_t ql[8];    // [4h + i]: ql bytes 64h + 32lh + 8i .. +7
+            u32x2_t qh[8];    // all 64 qh bytes
+            u32x2_t sc[2];    // the 16 int8 scales
+            uint32_t d;
+        };
+        auto ld64 = [](const uint8_t *a) __attribute__((always_inline)) {
+            u32x2_t v;
+            __builtin_memcpy(&v, a, 8);
+            return v;
+        };
+        auto fetch_sb = [&](int sb, Sb6Regs &r) __attribute__((always_inline)) {
+            const uint8_t *blk = wrow + (size_t)sb * 210;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                r.ql[i] = ld64(blk + 32 * lh + 8 * i);
+                r.ql[4 + i] = ld64(blk + 64 + 32 * lh + 8 * i);
+            }
+#pragma unroll
+            for (int i = 0; i < 8; i++) r.qh[i] = ld64(blk + 128 + 8 * i);
+            r.sc[0] = ld64(blk + 192);
+            r.sc[1] = ld64(blk + 200);
+            uint16_t d;
+            __builtin_memcpy(&d, blk + 208, 2);
+            r.d = d;
+        };
+        auto stage = [&](int step, auto gtag, const Sb6Regs &w) __attribute__((always_inline)) {
+            constexpr int G = decltype(gtag)::value, H = G >> 1, P = G & 1;
+            _Float16 *Bs = main_stage(step);
+            const uint32_t s16 = (w.sc[H][P] >> (16 * lh)) & 0xFFFFu;
+            const _Float16 sa = (_Float16)(int)(int8_t)(s16 & 0xFFu), sb_ = (_Float16)(int)(int8_t)(s16 >> 8);
+            const h2 sc2[2] = {h2{sa, sa}, h2{sb_, sb_}};
+            const h2 bias = {(_Float16)1056.f, (_Float16)1056.f};
+            const int hsh = 4 * P + 2 * lh;
+            uint32_t o[16];
+#pragma unroll
+            for (int j = 0; j < 8; j++) {   // 4 columns per dword; dwords 0..3 take the first scale, 4..7 the second
+                const uint32_t L = w.ql[4 * H + (j >> 1)][j & 1], Q = w.qh[4 * H + (j >> 1)][j & 1];
+                const uint32_t nib = (P ? (L >> 4) : L) & 0x0F0F0F0Fu;
+                const uint32_t c = nib | (((Q >> hsh) & 0x03030303u) << 4);   // four 6-bit codes
+                const uint32_t pa = (c & 0x00FF00FFu) | 0x64006400u;          // columns (0, 2) as 1024 + code
+                const uint32_t pb = ((c >> 8) & 0x00FF00FFu) | 0x64006400u;   // columns (1, 3)
+                const h2 va = (__builtin_bit_cast(h2, pa) - bias) * sc2[j >> 2];
+                const h2 vb = (__builtin_bit_cast(h2, pb) - bias) * sc2[j >> 2];
+                o[2 * j] = __builtin_bit_cast(uint32_t, va);
+                o[2 * j + 1] = __builtin_bit_cast(uint32_t, vb);
+            }
+            uint4 *dst = reinterpret_cast<uint4 *>(&Bs[lrow * PITCH + 32 * lh]);
+#pragma unroll
+            for (int i = 0; i < 4; i++) dst[i] = make_uint4(o[4 * i], o[4 * i + 1], o[4 * i + 2], o[4 * i + 3]);
+            if (G == 0 && lh == 0) dsc_stage(step >> 2)[lrow] = half_bits_to_f32(w.d);
+        };
+        Sb6Regs wcur, wnext;
+        fetch_sb(0, wcur);
+        stage(0, std::integral_constant<int, 0>{}, wcur);
+        __syncthreads();
+        auto step_body = [&](int sb, auto gtag) __attribute__((always_inline)) {
+            constexpr int g = decltype(gtag)::value;
+            const int step = 4 * sb + g;
+            if (g == 0) fetch_sb(min(sb + 1, nsb - 1), wnext);
+            if (step + 1 < nsteps) {
+                if (g == 3) wcur = wnext;
+                stage(step + 1, std::integral_constant<int, (g + 1) & 3>{}, wcur);
+            }
+            __syncthreads();
+        };
+        for (int sb = 0; sb < nsb; sb++) {
+            step_body(sb, std::integral_constant<int, 0>{});
+            step_body(sb, std::integral_constant<int, 1>{});
+            step_body(sb, std::integral_constant<int, 2>{});
+            step_body(sb, std::integral_constant<int, 3>{});
+        }
+        return;
+    }
+
+    if (!Q6 && wave >= 4) {
         // ------------------------------------------------------------------ loaders
         const int lt = tid - 256, lrow = lt >> 1, lh = lt & 1;   // two threads per tile row
         const size_t row_bytes = (size_t)nsb * 144;
@@ -291,7 +384,7 @@ __global__ __launch_bounds__(kThreadsMM) void q4k_mul_mm_kernel(MmParams p)
             const _Float16 *A2s = min_stage(sb), *B2s = A2s + BM * PITCH2;
             const float *dsc = dsc_stage(sb);
 #pragma unroll
-            for (int ks = 0; ks < 2; ks++) {
+            for (int ks = 0; ks < (Q6 ? 0 : 2); ks++) {
                 h8 a[2], b[2];
 #pragma unroll
                 for (int mt = 0; mt < 2; mt++)
@@ -351,7 +444,9 @@ int launch_mul_mm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
     p.SxA = SxA;
     p.Y = (float *)a.out[0];
     p.rows = rows; p.cols = cols; p.batch = batch;
-    hipLaunchKernelGGL(q4k_mul_mm_kernel, dim3((batch + BM - 1) / BM, (rows + BN - 1) / BN), dim3(kThreadsMM), kLdsBytes, st, p);
+    const dim3 grid((batch + BM - 1) / BM, (rows + BN - 1) / BN);
+    if (k.desc.dtypes[0] == KSH_Q6K) hipLaunchKernelGGL(q_mul_mm_kernel<true>, grid, dim3(kThreadsMM), kLdsBytes, st, p);
+    else hipLaunchKernelGGL(q_mul_mm_kernel<false>, grid, dim3(kThreadsMM), kLdsBytes, st, p);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : hip_fail(e, "mul_mm launch");
 }
@@ -361,13 +456,14 @@ int launch_mul_mm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
 int bind_matvec_batch(ksh_kernel &k)
 {
     const int64_t rows = k.desc.dims[0], cols = k.desc.dims[1], batch = k.desc.dims[2];
-    if (k.desc.dtypes[0] != KSH_Q4K) return set_error("matvec_batch: weight dtype %d is not built (Q4_K is)", k.desc.dtypes[0]);
+    const bool q6 = k.desc.dtypes[0] == KSH_Q6K;
+    if (k.desc.dtypes[0] != KSH_Q4K && !q6) return set_error("matvec_batch: weight dtype %d is not built (Q4_K and Q6_K are)", k.desc.dtypes[0]);
     if (k.desc.dtypes[1] != KSH_BF16) return set_error("matvec_batch: activation dtype %d is not built (BF16 is)", k.desc.dtypes[1]);
     if (rows <= 0 || batch <= 0 || rows > (1 << 24) || batch > (1 << 20)) return set_error("matvec_batch: rows=%lld batch=%lld", (long long)rows, (long long)batch);
     if (cols <= 0 || cols % 256 || cols > (1 << 20)) return set_error("matvec_batch: cols=%lld is not a positive multiple of 256", (long long)cols);
     k.info.n_inputs = 2;
     k.info.n_outputs = 1;
-    k.in_bytes[0] = (size_t)rows * (cols / 256) * 144; k.in_align[0] = 16;
+    k.in_bytes[0] = (size_t)rows * (cols / 256) * (q6 ? 210 : 144); k.in_align[0] = q6 ? 2 : 16;
     k.in_bytes[1] = (size_t)batch * cols * 2; k.in_align[1] = 16;
     k.out_bytes[0] = (size_t)batch * rows * 4; k.out_align[0] = 4;
     // f16 copy of X plus the min-term operand (32 halves per token and superblock)
@@ -376,7 +472,7 @@ int bind_matvec_batch(ksh_kernel &k)
                (uint32_t)kLdsBytes);
     k.info.sched = k.desc.sched;
     k.info.sched.tg = kThreadsMM; k.info.sched.nsg = kThreadsMM / 64; k.info.sched.lds_tile = KS;
-    set_name(k, "mul_mm_q4k_%dx%dx%d", BM, BN, KS);
+    set_name(k, "mul_mm_%s_%dx%dx%d", q6 ? "q6k" : "q4k", BM, BN, KS);
     k.launch = launch_mul_mm;
     return 0;
 }

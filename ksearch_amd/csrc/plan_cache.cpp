@@ -157,7 +157,7 @@ const char *ksh_plan_kind(const ksh_kernel_desc *d)
     case KSH_RMSNORM_MATVEC_QKV: return "rms_matvec_qkv_q4k";
     case KSH_MATVEC_GATE_UP_GELU: return "matvec_gate_up_q4k";
     case KSH_RMSNORM_MATVEC_GATE_UP_GELU: return "rms_matvec_gate_up_q4k";
-    case KSH_MATVEC_BATCH: return "mul_mm_q4k";
+    case KSH_MATVEC_BATCH: return d->dtypes[0] == KSH_Q6K ? "mul_mm_q6k" : "mul_mm_q4k";
     case KSH_SDPA_SLOTS:
     case KSH_SDPA_MWG_PART: return "sdpa_q40";
     case KSH_ATTEND_DECODE: return "attend_decode_q40";

@@ -100,6 +100,7 @@ def test_plan_kinds_and_candidates():
     assert hip.plan_kind(d) == "matvec_q4k"
     assert hip.plan_kind(hip.make_desc(hip.Kind.MATVEC, (8, 2048), (hip.DType.Q6K,))) == "matvec_q6k"
     assert hip.plan_kind(hip.make_desc(hip.Kind.MATVEC_BATCH, (8, 2048, 16), (hip.DType.Q4K,))) == "mul_mm_q4k"
+    assert hip.plan_kind(hip.make_desc(hip.Kind.MATVEC_BATCH, (8, 2048, 16), (hip.DType.Q6K,))) == "mul_mm_q6k"
     assert hip.plan_kind(hip.make_desc(hip.Kind.RMSNORM, (2048,))) is None
     c = hip.beam_candidates(d)
     assert len(c) >= 12

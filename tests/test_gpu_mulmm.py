@@ -1,6 +1,6 @@
-"""Q4_K prefill GEMM on the matrix cores vs the CPU oracle (dequant, bf16->f32
-X, sequential f32 dot), 1e-3 relative; shapes and inputs of the reference's
-check_mul_mm example plus the full benchmark configuration."""
+"""Q4_K / Q6_K prefill GEMM on the matrix cores vs the CPU oracle (dequant,
+bf16->f32 X, sequential f32 dot), 1e-3 relative; shapes and inputs of the
+reference's check_mul_mm example plus the full benchmark configuration."""
 import numpy as np
 import pytest
 
@@ -25,11 +25,11 @@ def eng():
     return hip.Eng()
 
 
-def run(ctx, eng, w, rows, cols, xf, xb, batch):
+def run(ctx, eng, w, rows, cols, xf, xb, batch, q6=False):
     y = ctx.buffer_empty_f32(batch * rows)
-    eng.matvec_batch(ctx, rows, cols, batch, DType.Q4K, ctx.buffer_bytes(w), ctx.buffer_bytes(xb), y)
+    eng.matvec_batch(ctx, rows, cols, batch, DType.Q6K if q6 else DType.Q4K, ctx.buffer_bytes(w), ctx.buffer_bytes(xb), y)
     got = ctx.read_f32(y, batch * rows).reshape(batch, rows)
-    want = oracle.matmul(oracle.Q4K, w, rows, cols, xf, batch)
+    want = oracle.matmul(oracle.Q6K if q6 else oracle.Q4K, w, rows, cols, xf, batch)
     return got, want
 
 
@@ -73,6 +73,69 @@ def test_mul_mm_unit_columns_recover_weights(ctx, eng):
         assert np.allclose(got[t], wd[:, k], rtol=1e-5, atol=1e-5 * np.abs(wd).max()), k
 
 
+def q6k_blocks_full_scales(n_blocks, seed):
+    """Random Q6_K superblocks whose int8 scales span -128..127 (the synthetic set's stay within -32..31)."""
+    blk = synth.q6k_blocks(n_blocks, seed).reshape(n_blocks, 210).copy()
+    blk[:, 192:208] = np.random.default_rng(seed + 1).integers(-128, 128, size=(n_blocks, 16), dtype=np.int16).astype(np.int8).view(np.uint8)
+    return blk.reshape(-1)
+
+
+# Q6_K tensors in prefill: same shapes (1536 columns: rows of 1260 bytes, blocks at 2-byte alignment)
+@pytest.mark.parametrize("rows,cols,batch", [(64, 256, 16), (128, 256, 9), (2048, 1536, 256), (4096, 1536, 55)])
+def test_mul_mm_q6k_check_mul_mm_shapes(ctx, eng, rows, cols, batch):
+    w, x = check_mul_mm_inputs(rows, cols, batch)
+    wq = oracle.quantize_q6k(w)
+    xf, xb = synth.bf16_round(x)
+    got, want = run(ctx, eng, wq, rows, cols, xf.reshape(batch, cols), xb.reshape(batch, cols), batch, q6=True)
+    assert_close(got, want, 1e-3, f"mul_mm q6k {rows}x{cols} b{batch}")
+    by = ctx.buffer_empty_f32(rows)
+    bw = ctx.buffer_bytes(wq)
+    for t in (0, batch - 1):
+        eng.matvec_wd(ctx, rows, cols, DType.Q6K, bw, ctx.buffer_f32(xf.reshape(batch, cols)[t]), by)
+        assert_close(got[t], ctx.read_f32(by, rows), 1e-3, f"mul_mm q6k vs gemv t={t}")
+
+
+@pytest.mark.parametrize("rows,cols,batch", [(1, 256, 1), (130, 512, 129), (257, 2048, 33), (300, 1280, 140)])
+def test_mul_mm_q6k_random_blocks_ragged(ctx, eng, rows, cols, batch):
+    # scales over the whole int8 range, so products beyond 2048 (rounded to even) occur
+    w = q6k_blocks_full_scales(rows * cols // 256, seed=620 + rows)
+    xf, xb = synth.bf16_round(synth.normal_f32(batch * cols, 621))
+    got, want = run(ctx, eng, w, rows, cols, xf.reshape(batch, cols), xb.reshape(batch, cols), batch, q6=True)
+    assert_close(got, want, 1e-3, f"mul_mm q6k {rows}x{cols} b{batch}")
+
+
+@pytest.mark.parametrize("full_scales", [False, True])
+def test_mul_mm_q6k_unit_columns_recover_weights(ctx, eng, full_scales):
+    # one-hot rows of X return columns of the dequantized matrix: pins the ql / qh / scale indexing of every
+    # position class.  Scales within -32..31: every scale * code is exact in f16 and the columns come back
+    # bit-exact; over the whole int8 range a product beyond 2048 is rounded to an even integer (2^-11).
+    rows, cols = 64, 512
+    w = (q6k_blocks_full_scales if full_scales else synth.q6k_blocks)(rows * cols // 256, seed=630)
+    wd = oracle.dequant(oracle.Q6K, w, rows * cols).reshape(rows, cols)
+    ks = [0, 1, 2, 3, 15, 16, 17, 31, 32, 33, 47, 48, 63, 64, 65, 95, 96, 127, 128, 129, 191, 192, 255, 256, 300, 511]
+    x = np.zeros((len(ks), cols), dtype=np.float32)
+    for t, k in enumerate(ks):
+        x[t, k] = 1.0
+    xf, xb = synth.bf16_round(x.reshape(-1))
+    got, _ = run(ctx, eng, w, rows, cols, xf.reshape(len(ks), cols), xb.reshape(len(ks), cols), len(ks), q6=True)
+    for t, k in enumerate(ks):
+        if full_scales:
+            assert np.allclose(got[t], wd[:, k], rtol=2.0 ** -11, atol=0), k
+        else:
+            assert np.array_equal(got[t], wd[:, k]), k
+
+
+def test_mul_mm_q6k_cfg2_shape(ctx, eng):
+    tokens, rows, cols = 512, 8192, 2048
+    w = q6k_blocks_full_scales(rows * cols // 256, seed=640)
+    xf, xb = synth.bf16_round(synth.normal_f32(tokens * cols, 641))
+    xf, xb = xf.reshape(tokens, cols), xb.reshape(tokens, cols)
+    got, want = run(ctx, eng, w, rows, cols, xf, xb, tokens, q6=True)
+    assert_close(got, want, 1e-3, "q6k 512x8192x2048")
+    got2, _ = run(ctx, eng, w, rows, cols, 2 * xf[:128], synth.bf16_round((2 * xf[:128]).reshape(-1))[1].reshape(128, cols), 128, q6=True)
+    assert np.array_equal(got2, 2 * got[:128])
+
+
 def test_mul_mm_cfg2_full_size(ctx, eng):
     tokens, rows, cols = 512, 8192, 2048
     w, xf, xb = synth.cfg2_q4k_prefill()
@@ -85,6 +148,6 @@ def test_mul_mm_cfg2_full_size(ctx, eng):
 
 def test_mul_mm_errors(ctx):
     with pytest.raises(hip.KshError, match="not built"):
-        ctx.compile(hip.make_desc(hip.Kind.MATVEC_BATCH, (64, 256, 16), (DType.Q6K, DType.BF16, DType.F32)))
+        ctx.compile(hip.make_desc(hip.Kind.MATVEC_BATCH, (64, 256, 16), (DType.Q40, DType.BF16, DType.F32)))
     with pytest.raises(hip.KshError, match="multiple of 256"):
         ctx.compile(hip.make_desc(hip.Kind.MATVEC_BATCH, (64, 100, 16), (DType.Q4K, DType.BF16, DType.F32)))

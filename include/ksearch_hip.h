@@ -412,6 +412,58 @@ int ksh_gemma4_bind_slot(ksh_gemma4 *m, ksh_kvpool *pool, int slot);
 int ksh_sample_softcap_min_p(const float *logits, size_t n, float cap, float temperature, float min_p,
                              uint32_t seed, uint32_t *out);
 
+/* GemmaPrimModel::decode_token_sampled (gemma_prim.rs:1614-1635): one token with logits at the model's position;
+ * temperature < 1e-6: the device argmax; else the logits are read back and ksh_sample_softcap_min_p draws. */
+int ksh_gemma4_decode_token_sampled(ksh_gemma4 *m, uint32_t token, float temperature, float min_p, uint32_t seed,
+                                    int use_graph, uint32_t *next_id);
+/* GemmaPrimModel::prefill_chunk (gemma_prim.rs:1305-1315): n tokens without logits, then one synchronisation
+ * (token by token here: the layer stack has no batched prefill). */
+int ksh_gemma4_prefill_chunk(ksh_gemma4 *m, const uint32_t *tokens, int n, int use_graph);
+
+/* ---- decode-before-prefill slot scheduler: spawn_scheduler and its rounds (crates/ksearch_cli/src/scheduler.rs:
+ * 78-349) as a tick the host drives.  One tick = admit waiting requests into free slots (alloc + clear), one
+ * decode token for every decoding request, chunked prefill for the prefilling ones (prefill_chunk tokens each
+ * while anything decodes, else up to prefill_tokens_per_tick), then finished requests free their slots.  GPU
+ * work is serial, as in the reference.  Requests are token ids; where the reference matches stop strings on the
+ * decoded text (scheduler.rs:207-217), `stop` is asked instead (non-zero: finish with reason "stop", the token is
+ * not emitted).  What the reference sends over channels is queued as events and drained with ksh_serve_poll. ---- */
+typedef struct ksh_serve ksh_serve;
+typedef int (*ksh_serve_stop_fn)(void *user, uint64_t request, uint32_t token);
+typedef struct {
+    int32_t slots;                     /* requests admitted at once (SchedulerConfig, scheduler.rs:60-76: 4) */
+    int32_t prefill_chunk;             /* 256 */
+    int32_t prefill_tokens_per_tick;   /* 2048 */
+    uint32_t eos[2];                   /* EOS_IDS (scheduler.rs:14): 1, 106 */
+    int32_t use_graph;                 /* replay the model's HIP graphs (1) or launch eagerly (0) */
+    ksh_serve_stop_fn stop;            /* may be NULL */
+    void *stop_user;
+} ksh_serve_cfg;
+enum ksh_serve_event_kind { KSH_SERVE_TOKEN = 0, KSH_SERVE_DONE = 1, KSH_SERVE_ERROR = 2 };
+/* finish_reason of StreamEvent::Done: "stop", "length", "cancelled"; "error" accompanies an error event */
+enum ksh_finish_reason { KSH_FINISH_STOP = 0, KSH_FINISH_LENGTH = 1, KSH_FINISH_CANCELLED = 2, KSH_FINISH_ERROR = 3 };
+typedef struct {
+    uint64_t request;
+    int32_t kind;                 /* ksh_serve_event_kind */
+    uint32_t token;               /* KSH_SERVE_TOKEN */
+    int32_t reason;               /* KSH_SERVE_DONE: ksh_finish_reason */
+    uint32_t prompt_tokens, completion_tokens;   /* KSH_SERVE_DONE */
+} ksh_serve_event;
+int ksh_serve_default_cfg(ksh_serve_cfg *cfg);
+/* the model and the pool must outlive the scheduler; the model is bound to the pool's slots from here on */
+int ksh_serve_create(ksh_gemma4 *model, ksh_kvpool *pool, const ksh_serve_cfg *cfg, ksh_serve **out);
+void ksh_serve_destroy(ksh_serve *s);
+/* InferenceRequest (scheduler.rs:28-36).  An empty prompt is accepted here and answered with an error event at
+ * admission, as the reference does.  max_tokens 0 counts as 1; the sampler's state starts at seed | 1. */
+int ksh_serve_submit(ksh_serve *s, const uint32_t *prompt, size_t n_prompt, size_t max_tokens, float temperature,
+                     float min_p, uint32_t seed, uint64_t *request);
+/* the reference notices a dropped receiver when it sends the next token: the request then finishes "cancelled" */
+int ksh_serve_cancel(ksh_serve *s, uint64_t request);
+int ksh_serve_tick(ksh_serve *s);
+size_t ksh_serve_poll(ksh_serve *s, ksh_serve_event *out, size_t cap);   /* returns the number written */
+/* text of the oldest error event not yet asked for (one per KSH_SERVE_ERROR event, in their order); NULL: none */
+const char *ksh_serve_error_text(ksh_serve *s);
+int ksh_serve_pending(const ksh_serve *s, int *waiting, int *active);
+
 /* ---- GGUF files: Gguf::open and its accessors (crates/ksearch_gguf/src/gguf_impl.rs:217-420).  The file is
  * memory-mapped; tensor data pointers stay valid until ksh_gguf_close.  A malformed file is an error here where
  * the reference panics. ---- */

@@ -657,6 +657,34 @@ int ksh_gemma4_generate_until(ksh_gemma4 *m, const uint32_t *prompt, int n_promp
     return 0;
 }
 
+// GemmaPrimModel::decode_token_sampled (gemma_prim.rs:1614-1635): one token with logits; below a temperature of 1e-6
+// the device argmax decides, else the logits are read back and the host sampler draws (gemma_prim.rs:1239-1261).
+int ksh_gemma4_decode_token_sampled(ksh_gemma4 *m, uint32_t token, float temperature, float min_p, uint32_t seed, int use_graph,
+                                    uint32_t *next_id)
+{
+    if (!m || !next_id) return set_error("ksh_gemma4_decode_token_sampled: bad arguments");
+    if (temperature < 1e-6f) return ksh_gemma4_forward_token(m, token, 1, use_graph, next_id);
+    if (ksh_gemma4_forward_token(m, token, 1, use_graph, nullptr)) return 1;
+    std::vector<float> logits((size_t)m->c.vocab);
+    if (ksh_buffer_read(m->ctx, m->logits, 0, logits.data(), logits.size() * 4, 1)) return 1;
+    return ksh_sample_softcap_min_p(logits.data(), logits.size(), m->c.softcap, temperature, min_p, seed, next_id);
+}
+
+// GemmaPrimModel::prefill_chunk (gemma_prim.rs:1305-1315): the tokens go through without logits, then one
+// synchronisation.  (Token by token: this build has no batched prefill of the layer stack.)
+int ksh_gemma4_prefill_chunk(ksh_gemma4 *m, const uint32_t *tokens, int n, int use_graph)
+{
+    if (!m || (n > 0 && !tokens) || n < 0) return set_error("ksh_gemma4_prefill_chunk: bad arguments");
+    if (m->pos + n > m->c.max_seq) return set_error("max_seq exceeded");
+    for (int i = 0; i < n; i++)
+        if (tokens[i] >= (uint32_t)m->c.vocab) return set_error("token id %u is outside the vocabulary", tokens[i]);
+    for (int i = 0; i < n; i++) {
+        if (write_token(m, tokens[i])) return 1;
+        if (run_token(m, false, use_graph != 0)) return 1;
+    }
+    return ksh_synchronize(m->ctx);
+}
+
 // GemmaPrimModel::bind_slot (gemma_prim.rs:1277-1292): the model's K / V caches become the slot's and its position the
 // slot's sequence length.  pool == NULL goes back to the model's own caches at position `slot` (0 after a reset).
 int ksh_gemma4_bind_slot(ksh_gemma4 *m, ksh_kvpool *pool, int slot)

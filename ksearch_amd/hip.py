@@ -118,6 +118,19 @@ class Gemma4Globals(C.Structure):
                 ("dt_ple_proj", C.c_int32), ("ple_proj_norm", C.c_void_p)]
 
 
+SERVE_STOP_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_uint64, C.c_uint32)
+
+
+class ServeCfg(C.Structure):
+    _fields_ = [("slots", C.c_int32), ("prefill_chunk", C.c_int32), ("prefill_tokens_per_tick", C.c_int32),
+                ("eos", C.c_uint32 * 2), ("use_graph", C.c_int32), ("stop", SERVE_STOP_FN), ("stop_user", C.c_void_p)]
+
+
+class ServeEvent(C.Structure):
+    _fields_ = [("request", C.c_uint64), ("kind", C.c_int32), ("token", C.c_uint32), ("reason", C.c_int32),
+                ("prompt_tokens", C.c_uint32), ("completion_tokens", C.c_uint32)]
+
+
 # every symbol include/ksearch_hip.h declares: name -> (restype, argtypes)
 _vp, _sz, _i, _u64p, _dp = C.c_void_p, C.c_size_t, C.c_int, C.POINTER(C.c_uint64), C.POINTER(C.c_double)
 _vpp = C.POINTER(C.c_void_p)
@@ -193,6 +206,17 @@ SYMBOLS = {
     "ksh_kvpool_v": (_vp, [_vp, _i, _i]),
     "ksh_kvpool_dims": (_i, [_vp] + [C.POINTER(C.c_int)] * 5),
     "ksh_gemma4_bind_slot": (_i, [_vp, _vp, _i]),
+    "ksh_gemma4_decode_token_sampled": (_i, [_vp, C.c_uint32, C.c_float, C.c_float, C.c_uint32, _i, C.POINTER(C.c_uint32)]),
+    "ksh_gemma4_prefill_chunk": (_i, [_vp, C.POINTER(C.c_uint32), _i, _i]),
+    "ksh_serve_default_cfg": (_i, [C.POINTER(ServeCfg)]),
+    "ksh_serve_create": (_i, [_vp, _vp, C.POINTER(ServeCfg), _vpp]),
+    "ksh_serve_destroy": (None, [_vp]),
+    "ksh_serve_submit": (_i, [_vp, C.POINTER(C.c_uint32), _sz, _sz, C.c_float, C.c_float, C.c_uint32, _u64p]),
+    "ksh_serve_cancel": (_i, [_vp, C.c_uint64]),
+    "ksh_serve_tick": (_i, [_vp]),
+    "ksh_serve_poll": (_sz, [_vp, C.POINTER(ServeEvent), _sz]),
+    "ksh_serve_error_text": (C.c_char_p, [_vp]),
+    "ksh_serve_pending": (_i, [_vp, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "ksh_sample_softcap_min_p": (_i, [_vp, _sz, C.c_float, C.c_float, C.c_float, C.c_uint32, C.POINTER(C.c_uint32)]),
     "ksh_gguf_open": (_i, [C.c_char_p, _vpp]),
     "ksh_gguf_close": (None, [_vp]),
@@ -932,6 +956,76 @@ class KvPool:
         return Buffer(self.ctx, lib().ksh_kvpool_v(self.h, slot, layer), owned=False)
 
 
+FINISH_REASONS = ("stop", "length", "cancelled", "error")
+
+
+class Serve:
+    """The decode-before-prefill slot scheduler (crates/ksearch_cli/src/scheduler.rs:78-349) as a tick the caller
+    drives.  Events come back as tuples: ("token", request, id), ("done", request, reason, prompt_tokens,
+    completion_tokens), ("error", request, text)."""
+
+    def __init__(self, model, pool, slots: int = 4, prefill_chunk: int = 256, prefill_tokens_per_tick: int = 2048,
+                 eos=(1, 106), use_graph: bool = True, stop=None):
+        cfg = ServeCfg()
+        _check(lib().ksh_serve_default_cfg(C.byref(cfg)))
+        cfg.slots, cfg.prefill_chunk, cfg.prefill_tokens_per_tick = slots, prefill_chunk, prefill_tokens_per_tick
+        cfg.eos[0], cfg.eos[1] = int(eos[0]), int(eos[1])
+        cfg.use_graph = int(use_graph)
+        # the callback object must live as long as the scheduler
+        self._stop = SERVE_STOP_FN(lambda user, req, tok: int(bool(stop(req, tok)))) if stop else SERVE_STOP_FN()
+        cfg.stop = self._stop
+        self.model, self.pool = model, pool
+        h = C.c_void_p()
+        _check(lib().ksh_serve_create(model.h, pool.h, C.byref(cfg), C.byref(h)))
+        self.h = h
+
+    def close(self):
+        if self.h:
+            lib().ksh_serve_destroy(self.h)
+            self.h = None
+
+    def submit(self, prompt, max_tokens: int, temperature: float = 0.0, min_p: float = 0.0, seed: int = 1) -> int:
+        p = (C.c_uint32 * max(1, len(prompt)))(*[int(t) for t in prompt])
+        rid = C.c_uint64()
+        _check(lib().ksh_serve_submit(self.h, p, len(prompt), max_tokens, temperature, min_p, seed & 0xFFFFFFFF, C.byref(rid)))
+        return rid.value
+
+    def cancel(self, request: int):
+        _check(lib().ksh_serve_cancel(self.h, request))
+
+    def tick(self) -> list:
+        _check(lib().ksh_serve_tick(self.h))
+        return self.poll()
+
+    def poll(self) -> list:
+        out, buf = [], (ServeEvent * 64)()
+        while True:
+            n = lib().ksh_serve_poll(self.h, buf, 64)
+            for e in buf[:n]:
+                if e.kind == 0:
+                    out.append(("token", e.request, e.token))
+                elif e.kind == 1:
+                    out.append(("done", e.request, FINISH_REASONS[e.reason], e.prompt_tokens, e.completion_tokens))
+                else:
+                    out.append(("error", e.request, (lib().ksh_serve_error_text(self.h) or b"").decode()))
+            if n < 64:
+                return out
+
+    def pending(self):
+        w, a = C.c_int(), C.c_int()
+        _check(lib().ksh_serve_pending(self.h, C.byref(w), C.byref(a)))
+        return w.value, a.value
+
+    def run(self, max_ticks: int = 100000) -> list:
+        """Ticks until nothing is waiting or running."""
+        out = []
+        for _ in range(max_ticks):
+            out += self.tick()
+            if self.pending() == (0, 0):
+                return out
+        raise KshError("Serve.run: still busy after max_ticks")
+
+
 class Gemma4:
     """GemmaPrimModel with the layer features of the real Gemma-4 checkpoints
     (crates/ksearch_gemma/src/gemma_prim.rs:881-1275; crates/ksearch_gemma/src/lib.rs:39-167).
@@ -1022,6 +1116,18 @@ class Gemma4:
         pre, dec = C.c_double(), C.c_double()
         _check(lib().ksh_gemma4_generate(self.h, p, len(prompt), n_new, int(use_graph), out, C.byref(pre), C.byref(dec)))
         return list(out[:n_new]), pre.value, dec.value
+
+    def decode_token_sampled(self, token: int, temperature: float, min_p: float, seed: int, use_graph: bool = False) -> int:
+        """GemmaPrimModel::decode_token_sampled (gemma_prim.rs:1614-1635)."""
+        nxt = C.c_uint32()
+        _check(lib().ksh_gemma4_decode_token_sampled(self.h, int(token), temperature, min_p, seed & 0xFFFFFFFF, int(use_graph),
+                                                     C.byref(nxt)))
+        return nxt.value
+
+    def prefill_chunk(self, tokens, use_graph: bool = False):
+        """GemmaPrimModel::prefill_chunk (gemma_prim.rs:1305-1315), token by token."""
+        t = (C.c_uint32 * max(1, len(tokens)))(*[int(x) for x in tokens])
+        _check(lib().ksh_gemma4_prefill_chunk(self.h, t, len(tokens), int(use_graph)))
 
     def bind_slot(self, pool, slot: int):
         """GemmaPrimModel::bind_slot; pool=None goes back to the model's own caches at position `slot`."""

@@ -40,6 +40,10 @@ def test_enums_match_header():
             assert hip.GgmlType[name[5:]] == val
         elif name == "LOAD_KEEP_Q6K":
             assert hip.LOAD_KEEP_Q6K == val
+        elif name.startswith("SERVE_"):
+            assert ("token", "done", "error")[val] == name[6:].lower()   # the kinds Serve.poll maps
+        elif name.startswith("FINISH_"):
+            assert hip.FINISH_REASONS[val] == name[7:].lower()
         else:
             raise AssertionError(f"KSH_{name} has no Python counterpart")
 
@@ -52,6 +56,8 @@ def test_struct_sizes():
     assert C.sizeof(hip.Gemma4Cfg) == 11 * 4 + 6 * 4
     assert C.sizeof(hip.Gemma4Layer) == 11 * 4 + 4 + 16 * 8 + 8          # ints, pad, pointers, scale + tail pad
     assert C.sizeof(hip.Gemma4Globals) == 8 * 8
+    assert C.sizeof(hip.ServeCfg) == 3 * 4 + 8 + 4 + 2 * 8
+    assert C.sizeof(hip.ServeEvent) == 8 + 5 * 4 + 4
 
 
 def test_context_fails_loudly_without_gpu():

@@ -216,6 +216,23 @@ def bench_decode_gemma4_layout(ctx, eng, use_graph=True):
     r = {"tok_s": round(256 / min(ms) * 1e3, 1), "ms_per_token": round(min(ms) / 256, 4), "launches_per_token": model.launches_per_token,
          "weight_GB_per_token": round(wbytes / 1e9, 3), "GB_s": round(wbytes / (min(ms) / 256 * 1e-3) / 1e9, 1),
          "layout": "35 layers, hidden 1536, 4 SWA(256, window 512) : 1 full(512), 20 shared-KV layers, PLE 256, ffn 6144/12288"}
+    # the same model under the slot scheduler: two requests of 64 + 128 tokens decoded in turn from two KV slots
+    # (serial GPU work, one host read-back per token, as the reference's serving loop does it)
+    pool = hip.KvPool(ctx, 2, cfg["max_seq"], n - shared, 512, 1)
+    sv = hip.Serve(model, pool, slots=2, eos=(0xFFFFFFFF, 0xFFFFFFFE), use_graph=use_graph)
+    best = 1e9
+    for rep in range(2):
+        for i in range(2):
+            sv.submit(prompt[i:] + prompt[:i], 128)
+        sv.tick()                                   # admission + prefill of both prompts
+        ctx.synchronize()
+        t0 = time.perf_counter()
+        n_tok = sum(1 for e in sv.run() if e[0] == "token")
+        best = min(best, (time.perf_counter() - t0) / n_tok)
+    r["served_two_slots_tok_s"] = round(1.0 / best, 1)
+    sv.close()
+    model.bind_slot(None, 0)
+    pool.close()
     model.close()
     return r
 

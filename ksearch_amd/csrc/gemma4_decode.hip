@@ -704,6 +704,9 @@ int ksh_gemma4_bind_slot(ksh_gemma4 *m, ksh_kvpool *pool, int slot)
         pos = ksh_kvpool_seq_len(pool, slot);
     }
     if (pos < 0 || pos > c.max_seq) return set_error("ksh_gemma4_bind_slot: position %d", pos);
+    // the slot it is bound to already, at the position the model has reached by itself: the device-side state is
+    // in place (a scheduler with one decoding request asks for this before every token)
+    if (pool && pool == m->pool && slot == m->bound_slot && pos == m->pos) return 0;
     stash_graphs(m);
     if (pool && pool != m->pool) {
         // graphs captured over another pool's buffers are of no use any more

@@ -91,6 +91,7 @@ struct LayerPlan {
 }  // namespace
 
 struct ksh_gemma4 {
+    std::vector<float> host_logits;   // decode_token_sampled's read-back
     ksh_ctx *ctx = nullptr;
     ksh_gemma4_cfg c{};
     ksh_gemma4_globals g{};
@@ -665,7 +666,8 @@ int ksh_gemma4_decode_token_sampled(ksh_gemma4 *m, uint32_t token, float tempera
     if (!m || !next_id) return set_error("ksh_gemma4_decode_token_sampled: bad arguments");
     if (temperature < 1e-6f) return ksh_gemma4_forward_token(m, token, 1, use_graph, next_id);
     if (ksh_gemma4_forward_token(m, token, 1, use_graph, nullptr)) return 1;
-    std::vector<float> logits((size_t)m->c.vocab);
+    std::vector<float> &logits = m->host_logits;   // (kept: a megabyte at the real vocabulary, every token)
+    logits.resize((size_t)m->c.vocab);
     if (ksh_buffer_read(m->ctx, m->logits, 0, logits.data(), logits.size() * 4, 1)) return 1;
     return ksh_sample_softcap_min_p(logits.data(), logits.size(), m->c.softcap, temperature, min_p, seed, next_id);
 }

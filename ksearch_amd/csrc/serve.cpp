@@ -231,7 +231,13 @@ int ksh_serve_create(ksh_gemma4 *model, ksh_kvpool *pool, const ksh_serve_cfg *c
     return 0;
 }
 
-void ksh_serve_destroy(ksh_serve *s) { delete s; }
+void ksh_serve_destroy(ksh_serve *s)
+{
+    if (!s) return;
+    // requests still running give their slots back: the pool outlives the scheduler
+    for (const Active &a : s->active) ksh_kvpool_free(s->pool, a.slot);
+    delete s;
+}
 
 int ksh_serve_submit(ksh_serve *s, const uint32_t *prompt, size_t n_prompt, size_t max_tokens, float temperature, float min_p,
                      uint32_t seed, uint64_t *request)

@@ -243,3 +243,17 @@ def test_a_token_repeated_24_times_ends_the_request(ctx):
     sv.close()
     pool.close()
     m.close()
+
+
+def test_destroying_a_busy_scheduler_frees_its_slots(ctx, model):
+    m, cfg = model
+    pool = make_pool(ctx, cfg, 2)
+    sv = hip.Serve(m, pool, slots=2, eos=NO_EOS)
+    (p,) = prompts_of(cfg, (5,), 705)
+    sv.submit(p, 30), sv.submit(p, 30), sv.submit(p, 30)
+    sv.tick(), sv.tick()
+    assert len(pool.active_batch()) == 2 and sv.pending() == (1, 2)
+    sv.close()
+    assert pool.active_batch() == []
+    m.bind_slot(None, 0)
+    pool.close()

@@ -254,7 +254,7 @@ def lib() -> C.CDLL:
 
 def _check(rc: int) -> None:
     if rc:
-        raise KshError(lib().ksh_last_error().decode())
+        raise KshError(lib().ksh_last_error().decode(errors="replace"))
 
 
 def make_desc(kind: int, dims=(), dtypes=(), params=(), sched: Sched | dict | None = None) -> KernelDesc:
@@ -852,7 +852,7 @@ class Gguf:
         out = []
         for i in range(lib().ksh_gguf_n_tensors(self.h)):
             _check(lib().ksh_gguf_tensor_name(self.h, i, buf, 512))
-            out.append(buf.value.decode())
+            out.append(buf.value.decode(errors="replace"))   # (gguf_impl.rs:170-173 reads strings lossily)
         return out
 
     def has_tensor(self, name: str) -> bool:
@@ -876,7 +876,7 @@ class Gguf:
 
     def get_str(self, key: str):
         buf = C.create_string_buffer(4096)
-        return None if lib().ksh_gguf_get_str(self.h, key.encode(), buf, 4096) else buf.value.decode()
+        return None if lib().ksh_gguf_get_str(self.h, key.encode(), buf, 4096) else buf.value.decode(errors="replace")
 
     def get_list(self, key: str):
         n = C.c_int()

@@ -161,3 +161,46 @@ def test_config_from_gguf_errors(tmp_path):
     gw.write(p, [("general.architecture", gw.STR, "gemma4")], t)
     with hip.Gguf(p) as g, pytest.raises(hip.KshError, match="block_count"):
         g.gemma4_config(64)
+
+
+def test_reader_survives_every_truncation_and_header_mutation(tmp_path):
+    """A damaged file is either refused with an error or opened with every tensor inside the mapping: each
+    prefix of a small file, bytes of its header overwritten at random, and 8-byte fields blown up."""
+    rng = np.random.default_rng(11)
+    meta = [("x", gw.U32, 7), ("s", gw.STR, "hello"), ("arr", gw.ARR, (gw.U32, [1, 2, 3])), ("n", gw.ARR, (gw.STR, ["a", "bc"]))]
+    tensors = [("t.f32", GgmlType.F32, (8, 4), rng.normal(size=32).astype(np.float32)),
+               ("t.q4k", GgmlType.Q4_K, (256, 2), rng.integers(0, 256, 288, dtype=np.uint8)),
+               ("t.q8_0", GgmlType.Q8_0, (32, 2), rng.integers(0, 256, 68, dtype=np.uint8))]
+    base = tmp_path / "base.gguf"
+    data_off = gw.write(str(base), meta, tensors)
+    raw = base.read_bytes()
+    variants = [raw[:cut] for cut in range(len(raw))]
+    for _ in range(400):
+        b = bytearray(raw)
+        for _ in range(int(rng.integers(1, 4))):
+            b[int(rng.integers(0, data_off))] = int(rng.integers(0, 256))
+        variants.append(bytes(b))
+    for _ in range(200):
+        b = bytearray(raw)
+        p = int(rng.integers(0, data_off - 8))
+        b[p:p + 8] = [2**63, 2**64 - 1, 2**40, 2**32, 2**31][int(rng.integers(0, 5))].to_bytes(8, "little")
+        variants.append(bytes(b))
+    path = tmp_path / "v.gguf"
+    opened = refused = 0
+    for v in variants:
+        path.write_bytes(v)
+        try:
+            g = hip.Gguf(str(path))
+        except hip.KshError:
+            refused += 1
+            continue
+        opened += 1
+        for name in g.tensor_names():
+            try:
+                _, dims, view = g.tensor(name)
+            except hip.KshError:                 # a name that is no longer valid UTF-8 cannot be asked for from here
+                continue
+            int(view.sum())                      # every byte the reader hands out is readable
+        g.get_u32("x"), g.get_str("s"), g.get_list("arr"), g.get_list("n")
+        g.close()
+    assert refused >= len(raw) - 64 and opened >= 1     # prefixes short of the data section are all refused

@@ -426,7 +426,9 @@ int ksh_gemma4_prefill_chunk(ksh_gemma4 *m, const uint32_t *tokens, int n, int u
  * while anything decodes, else up to prefill_tokens_per_tick), then finished requests free their slots.  GPU
  * work is serial, as in the reference.  Requests are token ids; where the reference matches stop strings on the
  * decoded text (scheduler.rs:207-217), `stop` is asked instead (non-zero: finish with reason "stop", the token is
- * not emitted).  What the reference sends over channels is queued as events and drained with ksh_serve_poll. ---- */
+ * not emitted).  What the reference sends over channels is queued as events and drained with ksh_serve_poll.
+ * One thread drives a scheduler (submit, cancel, tick and poll are not synchronised with one another): the
+ * reference's job channel from its HTTP handlers is the embedding host's to keep. ---- */
 typedef struct ksh_serve ksh_serve;
 typedef int (*ksh_serve_stop_fn)(void *user, uint64_t request, uint32_t token);
 typedef struct {

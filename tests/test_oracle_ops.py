@@ -34,6 +34,21 @@ def test_matmul_check_mul_mm_shapes(rows, cols, batch):
         assert np.array_equal(oracle.matvec(oracle.Q4K, wq, rows, cols, x[t]), got[t])
 
 
+@pytest.mark.parametrize("rows,cols,batch", [(64, 256, 16), (33, 1536, 5)])
+def test_matmul_q6k_brute_force(rows, cols, batch):
+    # the checker of the Q6_K prefill GEMM: float64 brute force on the dequantized matrix, batch row = GEMV
+    w, x = check_mul_mm_inputs(rows, cols, batch)
+    wq = oracle.quantize_q6k(w)
+    wd = oracle.dequant(oracle.Q6K, wq, rows * cols).reshape(rows, cols)
+    assert np.abs(wd - w).max() < 0.05
+    got = oracle.matmul(oracle.Q6K, wq, rows, cols, x, batch)
+    want = x.astype(np.float64) @ wd.astype(np.float64).T
+    mag = np.abs(x.astype(np.float64)) @ np.abs(wd.astype(np.float64)).T
+    assert np.all(np.abs(got - want) <= 3e-6 * mag + 1e-12)
+    for t in (0, batch - 1):
+        assert np.array_equal(oracle.matvec(oracle.Q6K, wq, rows, cols, x[t]), got[t])
+
+
 @pytest.mark.parametrize("dtype,gen,bpb", [(oracle.Q4K, synth.q4k_blocks, 144), (oracle.Q6K, synth.q6k_blocks, 210)])
 def test_matvec_sequential_f32_order(dtype, gen, bpb):
     rows, cols = 6, 512

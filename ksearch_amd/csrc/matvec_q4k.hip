@@ -456,6 +456,13 @@ Q4kGeom pick_geom(const ksh_sched &s, int total_rows, int bpr)
         G.R = (int)s.nr0;
         return G;
     }
+    // 1536-column matrices of 12288 rows and more (the wide feed-forward of the cache-reading layers): 4-wave
+    // workgroups, twice as many of them (in the decode loop 1.398 against 1.410 ms per token)
+    if (bpr == 6 && total_rows >= 12288 && !s.nsg && !s.nr0) {
+        G.NW = 4;
+        G.R = 2;
+        return G;
+    }
     for (int nw : {8, 4})
         for (int r : {2, 1}) {
             if (s.nsg && (int)s.nsg != nw) continue;

@@ -240,7 +240,7 @@ def test_matvec_qkv(ctx, eng, q_rows, kv_rows, cols):
         assert_close(ctx.read_f32(o, r), oracle.matvec(oracle.Q4K, w, r, cols, x), TOL, f"qkv {r}")
 
 
-@pytest.mark.parametrize("rows,cols", [(8192, 2048), (100, 4096), (64, 512), (6144, 1536), (45, 1536)])
+@pytest.mark.parametrize("rows,cols", [(8192, 2048), (100, 4096), (64, 512), (6144, 1536), (12288, 1536), (45, 1536)])
 def test_matvec_gate_up_gelu(ctx, eng, rows, cols):
     wg = synth.q4k_blocks(rows * cols // 256, seed=30)
     wu = synth.q4k_blocks(rows * cols // 256, seed=31)

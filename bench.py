@@ -35,6 +35,12 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0
 
+# kernels are chosen by the library's defaults, never by a plan file an earlier search left in the user's cache
+if "KSEARCH_BEAM_CACHE" not in os.environ:
+    import tempfile
+
+    os.environ["KSEARCH_BEAM_CACHE"] = tempfile.mkdtemp(prefix="ksearch_bench_plans_")
+
 
 class HipEvents:
     """hipEvent timing on a given stream (torch's events only see torch's stream)."""

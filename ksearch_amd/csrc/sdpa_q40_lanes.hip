@@ -38,14 +38,6 @@
 namespace ksh {
 namespace {
 
-// phase timestamps for a timing probe that includes this file; nothing in the library build
-#ifdef KSH_TRACE
-__device__ unsigned long long ksh_trace_buf[64 * 16];
-#define KSH_MARK(n) do { if ((threadIdx.x & 63) == 0 && threadIdx.x < 64) ksh_trace_buf[blockIdx.x * 16 + (n)] = wall_clock64(); } while (0)
-#else
-#define KSH_MARK(n) do { } while (0)
-#endif
-
 enum { kModeDirect = 0, kModePart = 1, kModeMerge = 2, kModeSplitPart = 3 };   // SplitPart: values and (m, l) pairs in separate arrays, no merge
 constexpr int kRT = 4;   // row steps per softmax update
 
@@ -385,7 +377,6 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
     uint8_t *newrow = reinterpret_cast<uint8_t *>(mlh + 2 * GP);   // K row, V row of the appended position
     __shared__ int last_flag;
 
-    KSH_MARK(0);
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int j = lane % LPR, sub = lane / LPR, b = j >> 2, w = j & 3, c = w;
     int part = blockIdx.x, slot = blockIdx.z, nparts = p.nwg;
@@ -491,7 +482,6 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
         for (int t = 0; t < kRT; t++) cur[t] = load_row(min(p0 + (t * NW + wave) * RPS + sub, last));
     }
 
-    KSH_MARK(1);
     // ---- q into registers (and, fused, the new K/V row into the cache) -------
     float qv[GP][8], Sq[GP];
     if (p.fused) {
@@ -565,7 +555,6 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
         for (int e = 0; e < 8; e++) st.O[h][e] = 0.f;
     }
 
-    KSH_MARK(2);
     // ---- the partition's rows: kRT steps of RPS rows per wave at a time -----
     if (dealt) {
         for (int it = 0; has_rows && (it * kRT * rparts + part) * GRP < tend; it++) {
@@ -607,7 +596,6 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
         process_rows<HD, GP, 1>(r, valid, live, qv, Sq, st, c);
     }
 
-    KSH_MARK(3);
     // ---- fold the row groups of this workgroup ------------------------------
     {
         float *my = slots + (wave * RPS + sub) * SLOTF;
@@ -629,7 +617,6 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
         }
     }
     __syncthreads();
-    KSH_MARK(4);
     {
         // One barrier: every thread works out its head's weights exp(m_s - M) itself (NSLOT broadcast reads and
         // exponentials) instead of waiting for a wave per head to publish them behind a second barrier.
@@ -691,7 +678,6 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
             }
         }
     }
-    KSH_MARK(5);
     if (p.mode != kModeMerge) return;
 
     // ---- the last partition to arrive folds the partials (lower.rs:5897-6087) -
@@ -699,13 +685,11 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
-    KSH_MARK(6);
     if (tid == 0) {
         const uint32_t arrived = __hip_atomic_fetch_add(&p.counters[slot * gridDim.y + blockIdx.y], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         last_flag = arrived == (uint32_t)nparts - 1u;
     }
     __syncthreads();
-    KSH_MARK(7);
     if (!last_flag) return;
     // The records come from the memory side (about a microsecond away), so all of
     // a thread's loads -- its output elements' values from up to QB partitions,
@@ -731,10 +715,8 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
         mq[2 * i + 1] = ld_agent(rec + 1);
     }
     __syncthreads();
-    KSH_MARK(8);
     for (int h = wave; h < groups; h += NW) merge_weights(mq + 2 * h * nparts, 2, nparts, nwgp, w2 + h * nwgp, mlh + 2 * h, lane);
     __syncthreads();
-    KSH_MARK(9);
     for (int q0 = 0; q0 < nparts; q0 += QB) {
 #pragma unroll
         for (int ob = 0; ob < OB; ob++) {
@@ -756,7 +738,6 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
             p.out[((size_t)slot * p.n_q + head0 + h) * HD + d] = acc[ob] / mlh[2 * h + 1];
         }
     }
-    KSH_MARK(10);
     if (tid == 0) __hip_atomic_store(&p.counters[slot * gridDim.y + blockIdx.y], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next launch
 }
 

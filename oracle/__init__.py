@@ -69,6 +69,8 @@ def lib() -> C.CDLL:
             "ko_gemma_pos": (i32, [vp]),
             "ko_gemma_kv": (vp, [vp, i32, i32]),
             "ko_gemma_hidden": (vp, [vp]),
+            "ko_gemma_set_row_sync": (None, [vp, vp]),
+            "ko_gemma4_set_row_sync": (None, [vp, vp]),
             "ko_sample_softcap_min_p": (u32, [vp, sz, f32, f32, f32, u32]),
             "ko_rmsnorm_per_head": (None, [vp, vp, vp, i32, i32, f32, vp]),
             "ko_add_scale": (None, [vp, vp, f32, sz, vp]),
@@ -252,6 +254,33 @@ def copy_scale_indexed(dtype, src, idx, n, scale) -> np.ndarray:
     return out
 
 
+class RowSync(C.Structure):
+    _fields_ = [("rows", C.c_void_p), ("row_stride", C.c_size_t), ("diff_bytes", C.c_void_p), ("max_step", C.c_void_p)]
+
+
+class _RowAdoption:
+    """Shared by the two decode loops: `forward(..., adopt_rows=a)` makes every cache-appending layer pack its
+    own Q4_0 K / V rows, measure how the rows in `a` ([n_layers, 2, row_bytes] uint8, another implementation's
+    rows for this position) differ from them, and continue with those.  Afterwards `row_diff_bytes` and
+    `row_max_step` ([n_layers, 2]; a step of 1.0 is one code of the own block) describe the differences."""
+
+    _set_sync = None
+
+    def _forward_adopting(self, fwd, n_layers, adopt_rows):
+        if adopt_rows is None:
+            return fwd()
+        rows = np.ascontiguousarray(adopt_rows, dtype=np.uint8)
+        assert rows.ndim == 3 and rows.shape[:2] == (n_layers, 2), rows.shape
+        self.row_diff_bytes = np.zeros((n_layers, 2), dtype=np.int32)
+        self.row_max_step = np.zeros((n_layers, 2), dtype=np.float32)
+        s = RowSync(_p(rows), rows.shape[2], _p(self.row_diff_bytes), _p(self.row_max_step))
+        getattr(lib(), self._set_sync)(self.h, C.byref(s))
+        try:
+            return fwd()
+        finally:
+            getattr(lib(), self._set_sync)(self.h, None)
+
+
 class GemmaCfg(C.Structure):
     _fields_ = [(n, C.c_int) for n in ("n_layers", "hidden", "ffn", "n_q", "n_kv", "hd", "vocab", "max_seq")] + \
                [(n, C.c_float) for n in ("eps", "softcap", "rope_theta", "attn_scale")]
@@ -263,7 +292,7 @@ class GemmaLayer(C.Structure):
         "attn_norm", "q_norm", "k_norm", "post_attn_norm", "ffn_norm", "post_ffw_norm")]
 
 
-class Gemma:
+class Gemma(_RowAdoption):
     """CPU greedy decoder over the same packed weights the HIP path uses.
 
     ``weights`` is the dict produced by ``ksearch_amd.synth.gemma_weights``:
@@ -291,10 +320,15 @@ class Gemma:
     def pos(self) -> int:
         return lib().ko_gemma_pos(self.h)
 
-    def forward(self, token: int, want_logits: bool = True, return_logits: bool = False, threads: int = 0):
+    _set_sync = "ko_gemma_set_row_sync"
+
+    def forward(self, token: int, want_logits: bool = True, return_logits: bool = False, threads: int = 0,
+                adopt_rows=None):
         logits = np.empty(self.vocab, dtype=np.float32) if return_logits else None
-        nxt = lib().ko_gemma_forward(self.h, int(token), int(want_logits),
-                                     _p(logits) if logits is not None else None, threads)
+        nxt = self._forward_adopting(
+            lambda: lib().ko_gemma_forward(self.h, int(token), int(want_logits),
+                                           _p(logits) if logits is not None else None, threads),
+            self.cfg.n_layers, adopt_rows)
         return (nxt, logits) if return_logits else nxt
 
     def kv(self, layer: int, which: int, nbytes: int) -> np.ndarray:
@@ -363,7 +397,7 @@ class Gemma4Globals(C.Structure):
                 ("dt_ple_proj", C.c_int), ("ple_proj_norm", C.c_void_p)]
 
 
-class Gemma4:
+class Gemma4(_RowAdoption):
     """CPU greedy decoder with the real checkpoints' layer features, over the
     same packed host arrays the HIP path uploads (``cfg`` / ``weights`` as for
     ``ksearch_amd.hip.Gemma4``; dtype codes are the shared 0..6 numbering)."""
@@ -402,10 +436,15 @@ class Gemma4:
     def kv_source(self, layer: int) -> int:
         return lib().ko_gemma4_kv_source(self.h, layer)
 
-    def forward(self, token: int, want_logits: bool = True, return_logits: bool = False, threads: int = 0):
+    _set_sync = "ko_gemma4_set_row_sync"
+
+    def forward(self, token: int, want_logits: bool = True, return_logits: bool = False, threads: int = 0,
+                adopt_rows=None):
         logits = np.empty(self.vocab, dtype=np.float32) if return_logits else None
-        nxt = lib().ko_gemma4_forward(self.h, int(token), int(want_logits),
-                                      _p(logits) if logits is not None else None, threads)
+        nxt = self._forward_adopting(
+            lambda: lib().ko_gemma4_forward(self.h, int(token), int(want_logits),
+                                            _p(logits) if logits is not None else None, threads),
+            self.cfg.n_layers, adopt_rows)
         return (nxt, logits) if return_logits else nxt
 
     def kv(self, layer: int, which: int, nbytes: int) -> np.ndarray:

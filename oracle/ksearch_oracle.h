@@ -141,7 +141,21 @@ typedef struct {
     const float *attn_norm, *q_norm, *k_norm, *post_attn_norm, *ffn_norm, *post_ffw_norm;
 } ko_gemma_layer;
 
+/* Row adoption for whole-step comparisons with another implementation (no counterpart in the reference; it
+ * removes Q4_0 rounding-boundary flips from the comparison).  When `rows` is set, every layer that appends
+ * to a cache packs its own K and V rows, records how the other implementation's rows differ from them
+ * (`diff_bytes[2*layer + which]`: differing bytes; `max_step[2*layer + which]`: largest difference of
+ * dequantized values in units of the own block's scale, 1.0 = one code step) and then continues with the
+ * other rows.  `rows` is [n_layers][2][row_stride] bytes (K then V); `diff_bytes` / `max_step` may be NULL. */
+typedef struct {
+    const uint8_t *rows;
+    size_t row_stride;
+    int *diff_bytes;
+    float *max_step;
+} ko_row_sync;
+
 typedef struct ko_gemma ko_gemma;
+void ko_gemma_set_row_sync(ko_gemma *m, const ko_row_sync *s);   /* NULL switches it off */
 ko_gemma *ko_gemma_create(const ko_gemma_cfg *cfg, const ko_gemma_layer *layers,
                           const uint8_t *token_embd_q6k, const float *output_norm);
 void ko_gemma_destroy(ko_gemma *m);
@@ -203,6 +217,7 @@ typedef struct {
 } ko_gemma4_globals;
 
 typedef struct ko_gemma4 ko_gemma4;
+void ko_gemma4_set_row_sync(ko_gemma4 *m, const ko_row_sync *s);   /* layers that append nothing are skipped */
 ko_gemma4 *ko_gemma4_create(const ko_gemma4_cfg *cfg, const ko_gemma4_layer *layers,
                             const ko_gemma4_globals *g);
 void ko_gemma4_destroy(ko_gemma4 *m);

@@ -8,6 +8,19 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 
+@pytest.fixture(autouse=True, scope="session")
+def _isolated_plan_cache(tmp_path_factory):
+    """Kernels requested with a zero schedule consult the plan cache; point it at an empty directory so that a plan
+    left by an earlier search cannot change which kernel variant a test exercises (tests of the cache set their own)."""
+    old = os.environ.get("KSEARCH_BEAM_CACHE")
+    os.environ["KSEARCH_BEAM_CACHE"] = str(tmp_path_factory.mktemp("plans"))
+    yield
+    if old is None:
+        os.environ.pop("KSEARCH_BEAM_CACHE", None)
+    else:
+        os.environ["KSEARCH_BEAM_CACHE"] = old
+
+
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 

@@ -77,10 +77,9 @@ def small_model(ctx, request):
 
 
 def test_forward_token_matches_oracle_teacher_forced(small_model):
-    """Teacher-forced and cache-synchronised: a K/V value that sits on a Q4_0 rounding boundary
-    may take the neighbouring code on two correct f32 implementations; such a step is counted,
-    its rows are overwritten with the oracle's, and its logits (which see the other code through
-    every later layer) are not compared."""
+    """Teacher-forced with the oracle in lockstep: a K/V value that sits on a Q4_0 rounding boundary may take the
+    neighbouring code on two correct f32 implementations, so the oracle packs its own row per layer, checks that
+    the device's is within one code step and continues with the device's (`adopt_rows`): every step is compared."""
     gpu, cpu, _ = small_model
     ctx = gpu.ctx
     gpu.reset()
@@ -90,33 +89,23 @@ def test_forward_token_matches_oracle_teacher_forced(small_model):
     row = SMALL["n_kv"] * SMALL["hd"] // 32 * 18
     bufs = [[hip.Buffer(ctx, hip.lib().ksh_gemma_kv(gpu.h, l, w), owned=False) for w in (0, 1)]
             for l in range(SMALL["n_layers"])]
-    agree, clean = 0, 0
+    agree, flipped = 0, 0
     for i, t in enumerate(toks):
         g_next = gpu.forward_token(int(t), use_graph=False)
-        c_next, c_logits = cpu.forward(int(t), return_logits=True)
+        rows = np.stack([np.stack([ctx.read_bytes(bufs[l][w], row, i * row) for w in (0, 1)]) for l in range(SMALL["n_layers"])])
+        c_next, c_logits = cpu.forward(int(t), return_logits=True, adopt_rows=rows)
+        assert cpu.row_max_step.max() <= 1.0 + 1e-3, (i, cpu.row_max_step)      # a flip is one code step, never more
+        flipped += int(cpu.row_diff_bytes.sum())
         g_logits = gpu.logits()
-        flips = 0
-        for l in range(SMALL["n_layers"]):
-            for w in (0, 1):
-                got, want = ctx.read_bytes(bufs[l][w], row, i * row), cpu.kv(l, w, (i + 1) * row)[i * row:]
-                if not np.array_equal(got, want):
-                    flips += int((got != want).sum())
-                    # a flip is one code step, never more
-                    dg, dc = oracle.dequant(oracle.Q40, got, row // 18 * 32), oracle.dequant(oracle.Q40, want, row // 18 * 32)
-                    assert np.abs(dg - dc).max() <= np.abs(dc).max() / 7 * 1.01
-                    ctx.write_bytes(bufs[l][w], want, i * row)
         # the device argmax follows the oracle's rule on the device's own logits
         assert g_next == oracle.softcap_argmax(g_logits, SMALL["softcap"])
-        if flips:
-            continue
-        clean += 1
         assert_close(g_logits, c_logits, 1e-3, f"logits at step {i}")
         assert_close(gpu.hidden(), cpu.hidden(), 1e-3, f"hidden at step {i}")
         top2 = np.sort(c_logits)[-2:]
-        if top2[1] - top2[0] > 1e-3 * max(abs(top2[1]), float(np.sqrt(np.mean(c_logits ** 2)))):
+        if top2[1] - top2[0] > 2e-3 * max(abs(top2[1]), float(np.sqrt(np.mean(c_logits ** 2)))):
             assert g_next == c_next, f"step {i}: margin {top2[1] - top2[0]}"
             agree += 1
-    assert clean >= 32 and agree >= 24 and gpu.pos == cpu.pos == len(toks)
+    assert agree >= 30 and flipped <= 0.02 * 40 * SMALL["n_layers"] * 2 * row and gpu.pos == cpu.pos == len(toks)
     with pytest.raises(hip.KshError, match="outside the vocabulary"):
         gpu.forward_token(SMALL["vocab"])
 

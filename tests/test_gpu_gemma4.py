@@ -147,43 +147,42 @@ def tiny(ctx, request):
 
 
 def teacher_forced(gpu, cpu, cfg, pattern, toks, check=None, use_graph=False, tol=1e-3):
-    """Feeds both models the same tokens and keeps their caches identical: a K/V value on a Q4_0 rounding boundary
-    may take the neighbouring code on two correct f32 implementations; such a step is counted, its rows are
-    overwritten with the oracle's, and its logits (which see the other code through every later layer) are not
-    compared.  Returns (steps compared, steps whose greedy token was checked and agreed)."""
+    """Feeds both models the same tokens with the oracle in lockstep: a K/V value on a Q4_0 rounding boundary may
+    take the neighbouring code on two correct f32 implementations, so the oracle packs its own row in every
+    cache-owning layer, checks that the device's row is within one code step of it and continues with the device's
+    row (`adopt_rows`).  Both sides attend over identical caches in every layer, so every step is compared.
+    Returns (steps compared, steps whose greedy token was checked and agreed)."""
     ctx = gpu.ctx
-    owners = [l for l in range(cfg["n_layers"]) if gpu.kv_source(l) == l]
+    n = cfg["n_layers"]
+    owners = [l for l in range(n) if gpu.kv_source(l) == l]
     hd = {l: cfg["hd_swa"] if pattern[l] else cfg["hd_full"] for l in owners}
     bufs = {l: [hip.Buffer(ctx, hip.lib().ksh_gemma4_kv(gpu.h, l, w), owned=False) for w in (0, 1)] for l in owners}
-    agree = clean = 0
+    stride = max(cfg["n_kv"] * h // 32 * 18 for h in hd.values())
+    agree = compared = flipped = 0
     for i, t in enumerate(toks):
         compare = check is None or i in check
         g_next = gpu.forward_token(int(t), want_logits=compare, use_graph=use_graph)
-        c_next, c_logits = cpu.forward(int(t), want_logits=compare, return_logits=True)
-        flips = 0
+        rows = np.zeros((n, 2, stride), np.uint8)
         for l in owners:
             row = cfg["n_kv"] * hd[l] // 32 * 18
             for w in (0, 1):
-                got, want = ctx.read_bytes(bufs[l][w], row, i * row), cpu.kv(l, w, (i + 1) * row)[i * row:]
-                if not np.array_equal(got, want):
-                    flips += int((got != want).sum())
-                    dg, dc = oracle.dequant(oracle.Q40, got, row // 18 * 32), oracle.dequant(oracle.Q40, want, row // 18 * 32)
-                    assert np.abs(dg - dc).max() <= np.abs(dc).max() / 7 * 1.01      # a flip is one code step, never more
-                    ctx.write_bytes(bufs[l][w], want, i * row)
+                rows[l, w, :row] = ctx.read_bytes(bufs[l][w], row, i * row)
+        c_next, c_logits = cpu.forward(int(t), want_logits=compare, return_logits=True, adopt_rows=rows)
+        assert cpu.row_max_step.max() <= 1.0 + 1e-3, (i, cpu.row_max_step.max(1))      # a flip is one code step, never more
+        flipped += int(cpu.row_diff_bytes.sum())
         if not compare:
             continue
         g_logits = gpu.logits()
         assert g_next == oracle.softcap_argmax(g_logits, cfg["softcap"])       # the device argmax follows the oracle's rule
-        if flips:
-            continue
-        clean += 1
+        compared += 1
         assert_close(g_logits, c_logits, tol, f"logits at step {i}")
         assert_close(gpu.hidden(), cpu.hidden(), tol, f"hidden at step {i}")
         top2 = np.sort(c_logits)[-2:]
-        if top2[1] - top2[0] > tol * max(abs(top2[1]), float(np.sqrt(np.mean(c_logits ** 2)))):
+        if top2[1] - top2[0] > 2 * tol * max(abs(top2[1]), float(np.sqrt(np.mean(c_logits ** 2)))):
             assert g_next == c_next, f"step {i}: margin {top2[1] - top2[0]}"
             agree += 1
-    return clean, agree
+    assert flipped <= 0.02 * len(toks) * len(owners) * 2 * stride, flipped
+    return compared, agree
 
 
 def test_gemma4_forward_token_matches_oracle_teacher_forced(tiny):
@@ -195,7 +194,7 @@ def test_gemma4_forward_token_matches_oracle_teacher_forced(tiny):
     assert [gpu.kv_source(l) for l in range(n_layers)] == [cpu.kv_source(l) for l in range(n_layers)] == [0, 1, 2, 3, 4, 4, 2, 4]
     toks = np.random.default_rng(611).integers(0, cfg["vocab"], 24)
     clean, agree = teacher_forced(gpu, cpu, cfg, PATTERN, toks)
-    assert clean >= 18 and agree >= 14 and gpu.pos == cpu.pos == len(toks)
+    assert clean == len(toks) and agree >= 16 and gpu.pos == cpu.pos == len(toks), (clean, agree)
     with pytest.raises(hip.KshError, match="outside the vocabulary"):
         gpu.forward_token(cfg["vocab"])
 
@@ -373,7 +372,7 @@ def test_gemma4_real_widths_long_run_matches_oracle(ctx, eng):
     toks = np.random.default_rng(631).integers(0, cfg["vocab"], 540)
     check = set(range(12)) | set(range(124, 134)) | set(range(506, 520)) | {300, 539}
     clean, agree = teacher_forced(gpu, cpu, cfg, pattern, toks, check=check, use_graph=True, tol=5e-3)
-    assert clean >= 24 and agree >= 12, (clean, agree)
+    assert clean == len(check) and agree >= 0.5 * len(check), (clean, agree)
     gpu.close()
     cpu.close()
 

@@ -246,6 +246,20 @@ int ksh_kernel_info_get(const ksh_kernel *k, ksh_kernel_info *info);
 int ksh_encode(ksh_ctx *ctx, ksh_kernel *k,
                ksh_buf *const *inputs, const uint64_t *in_byte_off, int n_in,
                ksh_buf *const *outputs, const uint64_t *out_byte_off, int n_out);
+/* Soft-capped argmax without any allocation.  No counterpart in the reference: it is for callers that cannot
+ * allocate device memory (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
+ * Same result as ksh_kernel_get(KSH_SOFTCAP_ARGMAX, dims = {n}, params = {cap}) + ksh_encode, on the context's
+ * stream: out f32[1] at `out_byte_off` = argmax_i cap*tanh(x_i/cap) over the n floats at `x_byte_off` (cap <= 0:
+ * plain argmax), lowest index wins ties.  The per-workgroup partial results (256 value/index pairs, 2 KB) live in a
+ * fixed array inside the library's device image instead of a buffer allocated per kernel handle, and the call
+ * creates no kernel handle: it calls no hipMalloc / hipFree and allocates no host memory.  n must be in
+ * [1, 2^24 - 1] (KSH_ARGMAX_STATIC_MAX_N: the f32 index is exact below 2^24); anything else is refused.  Every
+ * call on a GPU shares that GPU's array: calls that overlap on one GPU (two contexts, two streams) race, calls
+ * on one context are ordered by its stream.  Nothing needs clearing between calls: a launch writes every partial
+ * it later reads. */
+#define KSH_ARGMAX_STATIC_MAX_N ((1 << 24) - 1)
+int ksh_softcap_argmax_static(ksh_ctx *ctx, ksh_buf *x, uint64_t x_byte_off, int64_t n, float cap,
+                              ksh_buf *out, uint64_t out_byte_off);
 /* run (:377-456): synchronize, then `iters` launches timed with HIP events on
  * the context's stream; *ms is the average per launch. */
 int ksh_run_timed(ksh_ctx *ctx, ksh_kernel *k,

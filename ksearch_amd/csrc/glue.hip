@@ -409,7 +409,62 @@ int launch_softcap_argmax(const ksh_kernel &k, const LaunchArgs &a, hipStream_t 
     return done("softcap_argmax launch");
 }
 
+// ---- ksh_softcap_argmax_static: the same two kernels over a fixed array in the device image ----
+// kArgParts (value, index) pairs.  In host code the array's name is only a handle for hipGetSymbolAddress; the
+// kernels get the per-device address that call returns.
+static __device__ __align__(256) unsigned char scratch[kArgParts * 8];
+constexpr int kMaxDevices = 64;
+void *g_scratch_ptr[kMaxDevices];      // per device: every GPU holds its own copy of the array
+
 }  // namespace
+
+int argmax_static_setup()
+{
+    int dev = -1;
+    KSH_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return set_error("softcap_argmax_static: device ordinal %d", dev);
+    if (g_scratch_ptr[dev]) return 0;
+    void *p = nullptr;
+    KSH_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) return set_error("softcap_argmax_static: the partial-result array has no device address");
+    g_scratch_ptr[dev] = p;
+    return 0;
+}
+
+}  // namespace ksh
+
+extern "C" int ksh_softcap_argmax_static(ksh_ctx *ctx, ksh_buf *x, uint64_t x_off, int64_t n, float cap, ksh_buf *out,
+                                         uint64_t out_off)
+{
+    using namespace ksh;
+    if (!ctx || !x || !out) return set_error("ksh_softcap_argmax_static: bad arguments");
+    if (n < 1 || n > KSH_ARGMAX_STATIC_MAX_N)
+        return set_error("ksh_softcap_argmax_static: n=%lld is outside [1, %d] (the f32 index is exact below 2^24 only)",
+                         (long long)n, KSH_ARGMAX_STATIC_MAX_N);
+    if (x_off % 4 || x_off > x->bytes || (uint64_t)n * 4 > x->bytes - x_off)
+        return set_error("ksh_softcap_argmax_static: x needs %lld bytes from 4-byte-aligned offset %llu, buffer has %zu",
+                         (long long)n * 4, (unsigned long long)x_off, x->bytes);
+    if (out_off % 4 || out_off > out->bytes || 4 > out->bytes - out_off)
+        return set_error("ksh_softcap_argmax_static: out needs 4 bytes from 4-byte-aligned offset %llu, buffer has %zu",
+                         (unsigned long long)out_off, out->bytes);
+    int dev = -1;
+    KSH_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return set_error("ksh_softcap_argmax_static: device ordinal %d", dev);
+    if (!g_scratch_ptr[dev] && argmax_static_setup()) return 1;
+    float *pv = (float *)g_scratch_ptr[dev];
+    uint32_t *pi = (uint32_t *)(pv + kArgParts);
+    const int parts = (int)min((int64_t)kArgParts, (n + kArgThreads - 1) / kArgThreads);
+    hipStream_t st = ctx_stream(ctx);
+    hipLaunchKernelGGL(softcap_argmax_part_kernel, dim3(parts), dim3(kArgThreads), 0, st,
+                       (const float *)((const char *)x->ptr + x_off), (int)n, cap, pv, pi);
+    hipLaunchKernelGGL(softcap_argmax_final_kernel, dim3(1), dim3(kArgThreads), 0, st, pv, pi, parts,
+                       (float *)((char *)out->ptr + out_off));
+    if (done("softcap_argmax_static launch")) return 1;
+    ctx_mark_pending(ctx);
+    return 0;
+}
+
+namespace ksh {
 
 int bind_rmsnorm(ksh_kernel &k)
 {

@@ -57,6 +57,15 @@ struct ksh_kernel {
     int (*launch)(const ksh_kernel &, const ksh::LaunchArgs &, hipStream_t) = nullptr;
 };
 
+namespace ksh {
+// what entry points outside the runtime's translation unit need of a context
+hipStream_t ctx_stream(ksh_ctx *ctx);
+void ctx_mark_pending(ksh_ctx *ctx);
+// resolves the device address of the static partial-result array of ksh_softcap_argmax_static for the current
+// device (called when a context is created; the entry point does it itself for a device it has not seen)
+int argmax_static_setup();
+}  // namespace ksh
+
 // hands a buffer's reference over to a model, which releases it when it is destroyed (the GGUF loader's uploads)
 extern "C" void ksh_gemma4_adopt(ksh_gemma4 *m, ksh_buf *b);
 

@@ -105,6 +105,11 @@ struct ksh_ctx {
     hipEvent_t t0 = nullptr, t1 = nullptr;
 };
 
+namespace ksh {
+hipStream_t ctx_stream(ksh_ctx *ctx) { return ctx->stream; }
+void ctx_mark_pending(ksh_ctx *ctx) { ctx->pending = true; }
+}  // namespace ksh
+
 using namespace ksh;
 
 extern "C" {
@@ -134,6 +139,7 @@ int ksh_ctx_create(ksh_ctx **out)
     KSH_HIP(hipEventCreateWithFlags(&ctx->copy_done, hipEventDisableTiming));
     KSH_HIP(hipEventCreate(&ctx->t0));
     KSH_HIP(hipEventCreate(&ctx->t1));
+    if (argmax_static_setup()) return 1;
     *out = ctx.release();
     return 0;
 }

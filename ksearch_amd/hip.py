@@ -152,6 +152,7 @@ SYMBOLS = {
     "ksh_kernel_get": (_i, [_vp, C.POINTER(KernelDesc), _vpp]),
     "ksh_kernel_info_get": (_i, [_vp, C.POINTER(KernelInfo)]),
     "ksh_encode": (_i, [_vp, _vp, _vpp, _u64p, _i, _vpp, _u64p, _i]),
+    "ksh_softcap_argmax_static": (_i, [_vp, _vp, C.c_uint64, C.c_int64, C.c_float, _vp, C.c_uint64]),
     "ksh_run_timed": (_i, [_vp, _vp, _vpp, _u64p, _i, _vpp, _u64p, _i, _i, _dp]),
     "ksh_flush_async": (_i, [_vp]),
     "ksh_wait_inflight_at_most": (_i, [_vp, _i]),
@@ -696,6 +697,11 @@ class Eng:
     # :1966-1982
     def softcap_argmax(self, ctx, n, cap, x, out):
         ctx.encode_multi(self._k(ctx, Kind.SOFTCAP_ARGMAX, (n,), (), (cap,)), [x], [out])
+
+    def softcap_argmax_static(self, ctx, n, cap, x, out, x_off=0, out_off=0):
+        """The same op through the entry point that allocates nothing (no kernel handle, partial results in a fixed
+        array of the device image); no counterpart in the reference."""
+        _check(lib().ksh_softcap_argmax_static(ctx.h, x.h, x_off, n, cap, out.h, out_off))
 
     def dequant(self, ctx, dtype, n, src, dst):
         ctx.encode_multi(self._k(ctx, Kind.DEQUANT, (n,), (dtype,)), [src], [dst])

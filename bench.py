@@ -67,7 +67,8 @@ class HipEvents:
 
 def timed_graph(ctx, ev, encode_one, n_launches: int, warmup: int) -> float:
     """Captures `n_launches` calls of encode_one(i) into a graph, runs `warmup`
-    launches eagerly first, then times one replay.  Returns ms for the replay."""
+    launches eagerly first and (when there is a warm-up at all) one untimed replay,
+    then times one replay.  Returns ms for that replay."""
     for i in range(warmup):
         encode_one(i)
     ctx.synchronize()
@@ -75,6 +76,8 @@ def timed_graph(ctx, ev, encode_one, n_launches: int, warmup: int) -> float:
     for i in range(n_launches):
         encode_one(i)
     g = ctx.graph_end()
+    if warmup:
+        ctx.graph_launch(g)      # the first replay of a new executable graph also uploads it: part of the warm-up
     ctx.synchronize()
     ev.start(ctx.stream)
     ctx.graph_launch(g)
@@ -100,6 +103,33 @@ def bench_matvec(ctx, eng, ev, dtype, rows, cols, w_host, x_host, copies, steps,
     big.release()
     return dict(kernel=k.name, us_per_launch=ms * 1e3 / steps, gbps=alg * steps / (ms * 1e-3) / 1e9,
                 alg_bytes=alg, ms=ms)
+
+
+def bench_floor(ctx, eng, ev, copies, steps, warmup):
+    """The memory-only floors of the headline launch, under the headline's protocol (one HIP graph of `steps`
+    dependent launches over `copies` rotating weight copies, HIP events on the stream): the same grid / workgroup /
+    LDS doing nothing, issuing only the GEMV's weight loads, and reading the same bytes with flat 128-bit loads;
+    then the GEMV itself for comparison."""
+    from ksearch_amd import hip, synth
+
+    rows = cols = 4096
+    w, x = synth.cfg0_q4k_matvec()
+    wbytes = w.size
+    big, sink = ctx.buffer_bytes(np.tile(w, copies)), ctx.buffer_empty_f32(1)
+    out = {"protocol": f"graph of {steps} launches, {copies} rotating copies of the 9.4 MB matrix, hipEvents; best of 5 replays"}
+    for mode, name in ((0, "empty_launch"), (1, "gemv_load_pattern_only"), (2, "flat_128bit_loads_only")):
+        k = ctx.compile(hip.make_desc(hip.Kind.READ_FLOOR, (rows, cols, mode), (hip.DType.Q4K,)))
+
+        def one(i, k=k):
+            ctx.encode_offsets_multi(k, [big], [(i % copies) * wbytes], [sink], [0])
+
+        us = min(timed_graph(ctx, ev, one, steps, warmup) for _ in range(5)) * 1e3 / steps
+        out[name] = dict(kernel=k.name, us_per_launch=round(us, 3), tbps=round(wbytes / us / 1e6, 2) if mode else None)
+    big.release()
+    g = min((bench_matvec(ctx, eng, ev, hip.DType.Q4K, rows, cols, w, x, copies, steps, warmup) for _ in range(5)),
+            key=lambda r: r["us_per_launch"])
+    out["gemv"] = dict(kernel=g["kernel"], us_per_launch=round(g["us_per_launch"], 3), tbps=round(g["gbps"] / 1e3, 2))
+    return out
 
 
 def bench_lm_head(ctx, eng, ev):
@@ -148,8 +178,10 @@ def bench_prefill(ctx):
     return out
 
 
-def bench_attention(ctx):
-    """cfg3: 4 slots, 8 q / 1 kv heads of 256, Q4_0 KV, lengths ~U{1024..16384}, one launch pair."""
+def bench_attention(ctx, ev, copies=16):
+    """cfg3: 4 slots, 8 q / 1 kv heads of 256, Q4_0 KV, lengths ~U{1024..16384}, one launch pair.  Timed twice: with
+    the 7 MB of rows resident in cache between launches, and cold, cycling through `copies` copies of the K / V
+    pools (16 x 18.9 MB = 302 MB, more than the 256 MB last-level cache) inside one HIP graph."""
     from ksearch_amd import hip, synth
 
     n_slots, n_q, n_kv, hd, max_t = 4, 8, 1, 256, 16384
@@ -164,11 +196,23 @@ def bench_attention(ctx):
     ctx.run(k, ins, outs, iters=5)
     ms = ctx.run(k, ins, outs, iters=50)
     alg = int(sum(288 * int(t) + 16384 for t in lens))
-    for b in ins + outs:
+    bk, bv = ctx.buffer_bytes(np.tile(kk.reshape(-1), copies)), ctx.buffer_bytes(np.tile(vv.reshape(-1), copies))
+
+    def one(i):
+        c = i % copies
+        ctx.encode_offsets_multi(k, [ins[0], bk, bv, ins[3]], [0, c * kk.size, c * vv.size, 0], outs, [0, 0])
+
+    cold_ms = min(timed_graph(ctx, ev, one, 64, 8) for _ in range(3)) / 64
+    for b in ins + outs + [bk, bv]:
         b.release()
-    return dict(kernel=k.name, lens=[int(t) for t in lens], us_per_launch=round(ms * 1e3, 2),
-                gbps=round(alg / (ms * 1e-3) / 1e9, 1), frac_hbm=round(alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
-                note="resident in cache between launches (7 MB working set)")
+
+    def rec(t_ms):
+        return dict(us_per_launch=round(t_ms * 1e3, 2), gbps=round(alg / (t_ms * 1e-3) / 1e9, 1),
+                    frac_hbm=round(alg / (t_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4))
+
+    return dict(kernel=k.name, lens=[int(t) for t in lens], alg_bytes=alg, **rec(cold_ms),
+                protocol=f"cold: graph of 64 launch pairs over {copies} rotating copies of the K / V pools ({copies * (kk.size + vv.size) >> 20} MiB)",
+                hot_cache=rec(ms))
 
 
 def bench_decode(ctx, eng, use_graph=True):
@@ -276,7 +320,7 @@ def main() -> int:
     ap.add_argument("--no-extras", action="store_true", help="headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--eager", action="store_true", help="cfg4 without HIP-graph replay (kernel-trace profiling)")
-    ap.add_argument("--only", choices=["cfg1", "cfg2", "cfg3", "cfg4", "gemma4", "copy"],
+    ap.add_argument("--only", choices=["cfg1", "cfg2", "cfg3", "cfg4", "gemma4", "copy", "floor"],
                     help="run one secondary workload and print its record (for profiling runs); 'copy' is a plain "
                          "64 MiB device copy, the known-size kernel that calibrates the FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
@@ -300,8 +344,10 @@ def main() -> int:
     if args.only:
         if args.only == "cfg1":
             r = bench_lm_head(ctx, eng, ev)
+        elif args.only == "floor":
+            r = bench_floor(ctx, eng, ev, args.copies, args.steps, args.warmup)
         else:
-            r = {"cfg2": lambda: bench_prefill(ctx), "cfg3": lambda: bench_attention(ctx),
+            r = {"cfg2": lambda: bench_prefill(ctx), "cfg3": lambda: bench_attention(ctx, ev),
                  "cfg4": lambda: bench_decode(ctx, eng, not args.eager),
                  "gemma4": lambda: bench_decode_gemma4_layout(ctx, eng, not args.eager)}[args.only]()
         ctx.close()
@@ -317,7 +363,7 @@ def main() -> int:
         also["cfg0_hot_cache"] = dict(us_per_launch=round(hot["us_per_launch"], 3), gbps=round(hot["gbps"], 1))
         also["cfg1_q6k_lm_head"] = bench_lm_head(ctx, eng, ev)
         also["cfg2_q4k_prefill_gemm"] = bench_prefill(ctx)
-        also["cfg3_q40_attention"] = bench_attention(ctx)
+        also["cfg3_q40_attention"] = bench_attention(ctx, ev)
         also["cfg4_gemma_decode"] = bench_decode(ctx, eng)
         also["gemma4_e2b_layer_layout_decode"] = bench_decode_gemma4_layout(ctx, eng)
 

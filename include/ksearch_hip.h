@@ -179,6 +179,12 @@ enum ksh_kind {
      *     with x_new = res + rms(y_prev)*w_post (the RmsNormAdd that closes the feed-forward block, folded in;
      *     x_new must not alias res) and the GEMV input x_new */
     KSH_MATVEC_GELU_MUL = 27,
+    /* Measurement aid, no counterpart in the reference: the memory-only floor of a Q4_K GEMV launch.  The grid,
+     * workgroup size and LDS reservation of the default GEMV schedule (2 rows per wave, 8 waves), doing nothing
+     * (mode 0), issuing exactly the GEMV's weight loads and nothing else (mode 1), or reading the same bytes with
+     * flat 128-bit loads (mode 2).  dims: rows, cols (<= 4096), mode.  dtypes: Q4K.  in: W   out: sink f32[1]
+     * (never written for real weights) */
+    KSH_READ_FLOOR = 28,
     KSH_KIND_COUNT
 };
 

@@ -120,6 +120,7 @@ int bind_per_head_qkv_q40(ksh_kernel &k);
 int bind_glue(ksh_kernel &k);          // COPY_SCALE_INDEXED, GELU_MUL, COPY_SLICE
 int bind_softcap_argmax(ksh_kernel &k);
 int bind_ple_ops(ksh_kernel &k);       // RMSNORM_PER_HEAD, ADD_SCALE, MATVEC_GELU_MUL
+int bind_read_floor(ksh_kernel &k);
 
 // candidate schedules per kind (BEAM)
 int matvec_candidates(const ksh_kernel_desc &d, ksh_sched *out, int cap);

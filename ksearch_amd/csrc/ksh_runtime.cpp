@@ -73,6 +73,7 @@ static int bind(ksh_kernel &k)
     case KSH_RMSNORM_PER_HEAD:
     case KSH_ADD_SCALE:
     case KSH_MATVEC_GELU_MUL: return bind_ple_ops(k);
+    case KSH_READ_FLOOR: return bind_read_floor(k);
     }
     return set_error("unknown kernel kind %d", k.desc.kind);
 }

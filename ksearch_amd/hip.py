@@ -62,6 +62,7 @@ class Kind(enum.IntEnum):           # enum ksh_kind
     RMSNORM_PER_HEAD = 25
     ADD_SCALE = 26
     MATVEC_GELU_MUL = 27
+    READ_FLOOR = 28
 
 
 class Sched(C.Structure):           # ksh_sched: OptSchedule retargeted to gfx950

@@ -57,7 +57,8 @@ enum ksh_kind {
     KSH_MATVEC = 1,
     /* MatvecBatch: Y[t,r] = sum_c W[r,c] X[t,c].  dims: rows, cols, batch.
      * dtypes[0] = Q4K | Q6K (GGUF byte order, blocks at 2-byte alignment),
-     * dtypes[1] = BF16 (X), output F32 token-major.
+     * dtypes[1] = BF16 (X) or F32 (X is then taken as hi + lo f16 parts, 22 bits, in two passes: the form the
+     * decode loops' prompt chunks use), output F32 token-major.
      * in: W, X   out: Y[batch, rows] */
     KSH_MATVEC_BATCH = 2,
     /* MatvecQkv: three GEMVs sharing x.  dims: q_rows, kv_rows, cols.
@@ -84,20 +85,25 @@ enum ksh_kind {
     KSH_SDPA_SLOTS = 8,
     /* QuantizeQ40: pack n f32 values (n%32==0) to Q4_0.  dims: n.  in: src  out: dst */
     KSH_QUANTIZE_Q40 = 9,
-    /* RmsNorm / RmsNormAdd / RmsNormAddScale.  dims: n, has_residual, has_scale.
-     * params[0] = eps, params[1] = scale.  in: x, w, (residual)   out: y */
+    /* RmsNorm / RmsNormAdd / RmsNormAddScale.  dims: n, has_residual, has_scale, rows.
+     * params[0] = eps, params[1] = scale.  in: x, w, (residual)   out: y
+     * rows > 1: rmsnorm_rows / rmsnorm_add_rows / rmsnorm_add_scale_rows (crates/ksearch_kernels/src/lib.rs:
+     * 1478-1560): x, residual and y are [rows, n], the weight is shared. */
     KSH_RMSNORM = 10,
-    /* RmsNormAddThenRmsNorm.  dims: n.  params[0] = eps.
-     * in: y, w_post, residual, w_ffn   out: x, x2 */
+    /* RmsNormAddThenRmsNorm.  dims: n, rows.  params[0] = eps.
+     * in: y, w_post, residual, w_ffn   out: x, x2   (rows > 1: rmsnorm_add_then_rmsnorm_rows, matrices [rows, n]) */
     KSH_RMSNORM_ADD_THEN_RMSNORM = 11,
-    /* RmsNormPerHeadQkvQ40 (n_tok = 1).  dims: n_q, n_kv, hd, max_seq.  params[0] = eps.
+    /* RmsNormPerHeadQkvQ40.  dims: n_q, n_kv, hd, max_seq, n_tok.  params[0] = eps.
+     * n_tok > 1 (rmsnorm_per_head_qkv_q40_batch, crates/ksearch_kernels/src/lib.rs:1750): q, k, v and q_out hold
+     * n_tok rows for consecutive positions; token i uses rope row / cache row (first position + i).
      * max_seq = 0: in: q, qw, rope_row f32[hd], k, kw, v   out: q_out f32, K row Q4_0,
      * V row Q4_0 (the caller applies the position as byte offsets, as the reference does).
      * max_seq > 0: a 7th input meta f32[4] carries the position in [3]; rope is then the
      * whole table f32[max_seq, hd] and the outputs are the cache bases. */
     KSH_RMSNORM_PER_HEAD_QKV_Q40 = 12,
     /* CopyScaleIndexed: out[i] = scale * deq(src[id*n + i]); id is read from a
-     * device f32 (the reference keeps token ids as f32).  dims: n, rows in the table.
+     * device f32 (the reference keeps token ids as f32).  dims: n, rows in the table, n_tok (> 1:
+     * copy_scale_indexed_batch_wd, idx f32[n_tok], out [n_tok, n]).
      * dtypes[0] = source dtype (Q4K | Q5K | Q6K | F16 | F32).  params[0] = scale.  in: src, idx   out: out[n] */
     KSH_COPY_SCALE_INDEXED = 13,
     /* GeluMul: out[i] = gelu_tanh(clamp(g[i])) * u[i].  dims: n.  in: g, u  out: out */
@@ -185,6 +191,12 @@ enum ksh_kind {
      * flat 128-bit loads (mode 2).  dims: rows, cols (<= 4096), mode.  dtypes: Q4K.  in: W   out: sink f32[1]
      * (never written for real weights) */
     KSH_READ_FLOOR = 28,
+    /* sdpa_hybrid_kv_batch (crates/ksearch_kernels/src/lib.rs:1592-1623, lower.rs:4961-4983): causal attention of
+     * n_tok consecutive prompt tokens over one Q4_0 cache that already holds their rows.  meta = f32{tlen of token
+     * 0, -, window}: token i attends tlen_i = min(tlen0 + i, window) rows from start_i = tlen0 + i - tlen_i.
+     * dims: n_q, n_kv, hd, max_t, n_tok, nwg (0 = default; sched.k_split sets it too).
+     * in: q[n_tok, n_q*hd], K, V, meta   out: tmp f32[n_tok*n_q*nwg*(hd+2)], o[n_tok, n_q*hd] */
+    KSH_SDPA_BATCH = 29,
     KSH_KIND_COUNT
 };
 
@@ -332,9 +344,13 @@ int ksh_gemma_reset(ksh_gemma *m);
 /* forward_token: one token at the model's current position.  use_graph=1
  * replays a captured HIP graph.  next_id may be NULL (no host read-back). */
 int ksh_gemma_forward_token(ksh_gemma *m, uint32_t token, int use_graph, uint32_t *next_id);
-/* generate_timed: feeds the prompt token by token, then n_new greedy tokens
- * whose ids never leave the device between steps.  decode_ms covers the n_new
- * steps only. */
+/* prefill_chunk (crates/ksearch_gemma/src/gemma_prim.rs:1305-1607): n tokens at the model's current position, no
+ * logits; chunks of up to 256 tokens run as one batched pass per layer (row norms, MFMA GEMMs over f32 activations,
+ * batched per-head norm + RoPE + Q4_0 append, causal attention over the cache), a single token as a decode step. */
+int ksh_gemma_prefill_chunk(ksh_gemma *m, const uint32_t *tokens, int n);
+/* generate_timed (:1658-1768): all prompt tokens but the last through prefill_chunk (use_graph & 2: token by token
+ * through the decode step instead), then n_new greedy tokens whose ids never leave the device between steps
+ * (use_graph & 1: replayed from a captured HIP graph).  decode_ms covers the n_new steps only. */
 int ksh_gemma_generate(ksh_gemma *m, const uint32_t *prompt, int n_prompt, int n_new,
                        int use_graph, uint32_t *out_ids, double *prefill_ms, double *decode_ms);
 /* test hooks: device buffers of the last step */

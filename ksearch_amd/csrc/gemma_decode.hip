@@ -62,6 +62,32 @@ __global__ void set_token_kernel(float *tok, float value)
     if (threadIdx.x == 0 && blockIdx.x == 0) tok[0] = value;
 }
 
+// start of a prompt chunk: the record the batched attention reads ({rows the first token attends, -, window}),
+// derived on the stream from the device-side position
+__global__ void chunk_begin_kernel(const float *meta, float *bmeta, int max_seq)
+{
+    if (threadIdx.x == 0) {
+        bmeta[0] = meta[3] + 1.0f;
+        bmeta[1] = 0.f;
+        bmeta[2] = (float)max_seq;
+        bmeta[3] = 0.f;
+    }
+}
+
+// end of a prompt chunk: position and attended length move on by n tokens, and the new position's rope row is put
+// where the decode step's attention reads it
+__global__ void chunk_end_kernel(float *meta, int n, int max_seq, const float *rope, float *rope_cur, int hd)
+{
+    const int pos = (int)meta[3] + n;
+    __syncthreads();
+    if (pos < max_seq)
+        for (int i = threadIdx.x; i < hd; i += blockDim.x) rope_cur[i] = rope[(size_t)pos * hd + i];
+    if (threadIdx.x == 0) {
+        meta[3] = (float)pos;
+        meta[0] = (float)(pos + 1);
+    }
+}
+
 struct Bufs {
     std::vector<ksh_buf *> owned;
     ~Bufs()
@@ -94,6 +120,10 @@ struct ksh_gemma {
     int sdpa_launches = 2;
     int short_context = 0;   // positions below this use the short-context graph
     std::vector<float> rope0;   // row 0 of the rope table, for reset
+    // prompt chunks (allocated at the first chunk): [kChunk, .] activations of the batched layer pass
+    ksh_buf *c_tok = nullptr, *c_x = nullptr, *c_x2 = nullptr, *c_y = nullptr, *c_q = nullptr, *c_k = nullptr, *c_v = nullptr, *c_o = nullptr,
+            *c_g = nullptr, *c_u = nullptr, *c_ff = nullptr, *c_tmp = nullptr, *c_meta = nullptr;
+    int c_nwg = 0;
 };
 
 namespace {
@@ -224,6 +254,77 @@ int run_token(ksh_gemma *m, bool want_logits, bool use_graph)
     }
     if (want_logits && !use_graph) m->launches_full = n;
     m->pos += 1;
+    return 0;
+}
+
+// prefill_chunk's chunk length (gemma_prim.rs:16)
+constexpr int kChunk = 256;
+constexpr int kChunkPartitions = 8;   // partitions per token of the batched attention (its tmp buffer is sized for this)
+
+int chunk_buffers(ksh_gemma *m)
+{
+    if (m->c_tok) return 0;
+    const ksh_gemma_cfg &c = m->c;
+    const size_t T = kChunk, qd = (size_t)c.n_q * c.hd, kvd = (size_t)c.n_kv * c.hd;
+    m->c_nwg = kChunkPartitions;
+    return alloc(m, T * 4, &m->c_tok) || alloc(m, T * c.hidden * 4, &m->c_x) || alloc(m, T * c.hidden * 4, &m->c_x2) ||
+           alloc(m, T * c.hidden * 4, &m->c_y) || alloc(m, T * qd * 4, &m->c_q) || alloc(m, T * kvd * 4, &m->c_k) ||
+           alloc(m, T * kvd * 4, &m->c_v) || alloc(m, T * qd * 4, &m->c_o) || alloc(m, T * c.ffn * 4, &m->c_g) ||
+           alloc(m, T * c.ffn * 4, &m->c_u) || alloc(m, T * c.ffn * 4, &m->c_ff) ||
+           alloc(m, T * c.n_q * m->c_nwg * (c.hd + 2) * 4, &m->c_tmp) || alloc(m, 16, &m->c_meta);
+}
+
+// forward_prefill_chunk (gemma_prim.rs:1317-1607) for 2 <= t <= kChunk tokens already validated: the layer as
+// matrices of t rows.  The GEMMs run on the batch rounded up to 32 rows (one kernel handle per 32 instead of
+// one per length; the rows past t are stale and nothing reads their results).
+int forward_prefill_chunk(ksh_gemma *m, const uint32_t *tokens, int t)
+{
+    const ksh_gemma_cfg &c = m->c;
+    if (chunk_buffers(m)) return 1;
+    const int64_t qd = (int64_t)c.n_q * c.hd, kvd = (int64_t)c.n_kv * c.hd, tp = (t + 31) / 32 * 32;
+    float ids[kChunk];
+    for (int i = 0; i < t; i++) ids[i] = (float)tokens[i];
+    if (ksh_synchronize(m->ctx)) return 1;                                   // c_tok may still be read by the previous chunk
+    if (ksh_buffer_write(m->ctx, m->c_tok, 0, ids, (size_t)t * 4, 1)) return 1;
+    ksh_kernel *k_embed, *k_norm, *k_mm_q, *k_mm_kv, *k_head, *k_sdpa, *k_mm_o, *k_add_then, *k_mm_ff, *k_gelu, *k_mm_down, *k_add;
+    const float embed_scale = std::sqrt((float)c.hidden);
+    if (get(m, KSH_COPY_SCALE_INDEXED, {c.hidden, c.vocab, t}, {KSH_Q6K}, {embed_scale}, &k_embed) ||
+        get(m, KSH_RMSNORM, {c.hidden, 0, 0, t}, {}, {c.eps}, &k_norm) ||
+        get(m, KSH_MATVEC_BATCH, {qd, c.hidden, tp}, {KSH_Q4K, KSH_F32, KSH_F32}, {}, &k_mm_q) ||
+        get(m, KSH_MATVEC_BATCH, {kvd, c.hidden, tp}, {KSH_Q4K, KSH_F32, KSH_F32}, {}, &k_mm_kv) ||
+        get(m, KSH_RMSNORM_PER_HEAD_QKV_Q40, {c.n_q, c.n_kv, c.hd, c.max_seq, t}, {}, {c.eps}, &k_head) ||
+        get(m, KSH_SDPA_BATCH, {c.n_q, c.n_kv, c.hd, c.max_seq, t, m->c_nwg}, {KSH_Q40, KSH_F32}, {c.attn_scale}, &k_sdpa) ||
+        get(m, KSH_MATVEC_BATCH, {c.hidden, qd, tp}, {KSH_Q4K, KSH_F32, KSH_F32}, {}, &k_mm_o) ||
+        get(m, KSH_RMSNORM_ADD_THEN_RMSNORM, {c.hidden, t}, {}, {c.eps}, &k_add_then) ||
+        get(m, KSH_MATVEC_BATCH, {c.ffn, c.hidden, tp}, {KSH_Q4K, KSH_F32, KSH_F32}, {}, &k_mm_ff) ||
+        get(m, KSH_GELU_MUL, {(int64_t)t * c.ffn}, {}, {}, &k_gelu) ||
+        get(m, KSH_MATVEC_BATCH, {c.hidden, c.ffn, tp}, {KSH_Q4K, KSH_F32, KSH_F32}, {}, &k_mm_down) ||
+        get(m, KSH_RMSNORM, {c.hidden, 1, 0, t}, {}, {c.eps}, &k_add))
+        return 1;
+    hipStream_t st = (hipStream_t)ksh_stream(m->ctx);
+    hipLaunchKernelGGL(chunk_begin_kernel, dim3(1), dim3(64), 0, st, (const float *)ksh_buffer_device_ptr(m->meta),
+                       (float *)ksh_buffer_device_ptr(m->c_meta), c.max_seq);
+    if (hipGetLastError() != hipSuccess) return set_error("chunk_begin launch failed");
+    int n = 0;
+    if (enc(m, k_embed, {m->embd, m->c_tok}, {m->c_x}, n)) return 1;
+    for (int l = 0; l < c.n_layers; l++) {
+        const ksh_gemma_layer &L = m->layers[l];
+        if (enc(m, k_norm, {m->c_x, L.attn_norm}, {m->c_x2}, n) ||
+            enc(m, k_mm_q, {L.wq, m->c_x2}, {m->c_q}, n) || enc(m, k_mm_kv, {L.wk, m->c_x2}, {m->c_k}, n) ||
+            enc(m, k_mm_kv, {L.wv, m->c_x2}, {m->c_v}, n) ||
+            enc(m, k_head, {m->c_q, L.q_norm, m->rope, m->c_k, L.k_norm, m->c_v, m->meta}, {m->c_q, m->kv_k[l], m->kv_v[l]}, n) ||
+            enc(m, k_sdpa, {m->c_q, m->kv_k[l], m->kv_v[l], m->c_meta}, {m->c_tmp, m->c_o}, n) ||
+            enc(m, k_mm_o, {L.wo, m->c_o}, {m->c_y}, n) ||
+            enc(m, k_add_then, {m->c_y, L.post_attn_norm, m->c_x, L.ffn_norm}, {m->c_x, m->c_x2}, n) ||
+            enc(m, k_mm_ff, {L.wgate, m->c_x2}, {m->c_g}, n) || enc(m, k_mm_ff, {L.wup, m->c_x2}, {m->c_u}, n) ||
+            enc(m, k_gelu, {m->c_g, m->c_u}, {m->c_ff}, n) || enc(m, k_mm_down, {L.wdown, m->c_ff}, {m->c_y}, n) ||
+            enc(m, k_add, {m->c_y, L.post_ffw_norm, m->c_x}, {m->c_x}, n))
+            return 1;
+    }
+    hipLaunchKernelGGL(chunk_end_kernel, dim3(1), dim3(64), 0, st, (float *)ksh_buffer_device_ptr(m->meta), t, c.max_seq,
+                       (const float *)ksh_buffer_device_ptr(m->rope), (float *)ksh_buffer_device_ptr(m->rope_cur), c.hd);
+    if (hipGetLastError() != hipSuccess) return set_error("chunk_end launch failed");
+    m->pos += t;
     return 0;
 }
 
@@ -368,6 +469,24 @@ int ksh_gemma_forward_token(ksh_gemma *m, uint32_t token, int use_graph, uint32_
     return 0;
 }
 
+int ksh_gemma_prefill_chunk(ksh_gemma *m, const uint32_t *tokens, int n)
+{
+    if (!m || (n && !tokens) || n < 0) return set_error("ksh_gemma_prefill_chunk: bad arguments");
+    if (m->pos + n > m->c.max_seq) return set_error("max_seq exceeded");
+    for (int i = 0; i < n; i++)
+        if (tokens[i] >= (uint32_t)m->c.vocab) return set_error("token id %u is outside the vocabulary", tokens[i]);
+    // gemma_prim.rs:1305-1315: chunks of PREFILL_CHUNK, a remainder of one token through the decode step
+    for (int i = 0; i < n; i += kChunk) {
+        const int t = std::min(kChunk, n - i);
+        if (t == 1) {
+            if (write_token(m, tokens[i]) || run_token(m, false, false)) return 1;
+        } else if (forward_prefill_chunk(m, tokens + i, t)) {
+            return 1;
+        }
+    }
+    return ksh_synchronize(m->ctx);
+}
+
 int ksh_gemma_generate(ksh_gemma *m, const uint32_t *prompt, int n_prompt, int n_new, int use_graph, uint32_t *out_ids,
                        double *prefill_ms, double *decode_ms)
 {
@@ -378,16 +497,21 @@ int ksh_gemma_generate(ksh_gemma *m, const uint32_t *prompt, int n_prompt, int n
     using clk = std::chrono::steady_clock;
     const auto t0 = clk::now();
     // all prompt tokens but the last go through without logits (gemma_prim.rs:1670-1675)
-    for (int i = 0; i + 1 < n_prompt; i++) {
-        if (write_token(m, prompt[i])) return 1;
-        if (run_token(m, false, use_graph != 0)) return 1;
+    const bool graph = (use_graph & 1) != 0;
+    if (use_graph & 2) {
+        for (int i = 0; i + 1 < n_prompt; i++) {
+            if (write_token(m, prompt[i])) return 1;
+            if (run_token(m, false, graph)) return 1;
+        }
+    } else if (ksh_gemma_prefill_chunk(m, prompt, n_prompt - 1)) {
+        return 1;
     }
     if (write_token(m, prompt[n_prompt - 1])) return 1;
     if (ksh_synchronize(m->ctx)) return 1;
     const auto t1 = clk::now();
     const int first = m->pos;
     for (int i = 0; i < n_new; i++)
-        if (run_token(m, true, use_graph != 0)) return 1;
+        if (run_token(m, true, graph)) return 1;
     if (ksh_synchronize(m->ctx)) return 1;
     const auto t2 = clk::now();
     if (prefill_ms) *prefill_ms = std::chrono::duration<double, std::milli>(t1 - t0).count();

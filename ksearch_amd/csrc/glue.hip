@@ -47,6 +47,11 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(const float *__re
                                                                int has_res, int has_scale, float scale)
 {
     __shared__ float red[4];
+    // rows form (rmsnorm_rows / rmsnorm_add_rows / rmsnorm_add_scale_rows, crates/ksearch_kernels/src/lib.rs:1478-1560):
+    // one workgroup per row of a [rows, n] matrix, the weight shared
+    x += (size_t)blockIdx.x * n;
+    y += (size_t)blockIdx.x * n;
+    if (has_res) res += (size_t)blockIdx.x * n;
     float ss = 0.f;
     for (int i = threadIdx.x; i < n; i += kNormThreads) ss += x[i] * x[i];
     ss = block_sum_256(ss, red);
@@ -66,6 +71,11 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_add_then_rmsnorm_kernel(
 {
     __shared__ float red[4];
     extern __shared__ float mid[];
+    // rows form (rmsnorm_add_then_rmsnorm_rows): one workgroup per row
+    y += (size_t)blockIdx.x * n;
+    res += (size_t)blockIdx.x * n;
+    out_x += (size_t)blockIdx.x * n;
+    out_x2 += (size_t)blockIdx.x * n;
     float ss = 0.f;
     for (int i = threadIdx.x; i < n; i += kNormThreads) ss += y[i] * y[i];
     ss = block_sum_256(ss, red);
@@ -105,15 +115,26 @@ __global__ __launch_bounds__(64) void per_head_qkv_q40_kernel(
 {
     constexpr int HALF = HD / 2, PER = HD / 64;   // elements per lane
     const int lane = threadIdx.x;
+    // batch form (rmsnorm_per_head_qkv_q40_batch, crates/ksearch_kernels/src/lib.rs:1750): blockIdx.y is the token
+    // of a chunk of consecutive positions; its q / k / v rows, rope row and cache rows follow the first token's
+    const int tok = blockIdx.y;
+    q += (size_t)tok * n_q * HD;
+    k += (size_t)tok * n_kv * HD;
+    v += (size_t)tok * n_kv * HD;
+    q_out += (size_t)tok * n_q * HD;
     if (meta) {
         // position kept on the device (meta[3]): the rope input is the whole
         // table and the K/V outputs are the cache bases, so that one captured
         // graph serves every token
         // clamped: a position at or past max_seq must never write outside the cache
-        const size_t pos = (size_t)min(max((int)meta[3], 0), max_seq - 1);
+        const size_t pos = (size_t)min(max((int)meta[3] + tok, 0), max_seq - 1);
         rope += pos * HD;
         k_out += pos * (size_t)n_kv * (HD / 32) * 18;
         v_out += pos * (size_t)n_kv * (HD / 32) * 18;
+    } else {
+        rope += (size_t)tok * HD;
+        k_out += (size_t)tok * n_kv * (HD / 32) * 18;
+        v_out += (size_t)tok * n_kv * (HD / 32) * 18;
     }
     const int head = blockIdx.x;
     const bool is_q = head < n_q;
@@ -229,7 +250,9 @@ __global__ void copy_scale_indexed_kernel(const uint8_t *__restrict__ src, const
 {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
-    int64_t id = (int64_t)idx[0];
+    // batch form (copy_scale_indexed_batch_wd): blockIdx.y is the token, its id at idx[token], its row of `out`
+    out += (size_t)blockIdx.y * n;
+    int64_t id = (int64_t)idx[blockIdx.y];
     id = id < 0 ? 0 : (id >= n_rows ? n_rows - 1 : id);    // never read outside the table
     float v;
     if (dtype == KSH_Q6K) {
@@ -326,7 +349,7 @@ int done(const char *what)
 int launch_rmsnorm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
 {
     const int n = (int)k.desc.dims[0], has_res = (int)k.desc.dims[1], has_scale = (int)k.desc.dims[2];
-    hipLaunchKernelGGL(rmsnorm_kernel, dim3(1), dim3(kNormThreads), 0, st, (const float *)a.in[0],
+    hipLaunchKernelGGL(rmsnorm_kernel, dim3((unsigned)max((int64_t)1, k.desc.dims[3])), dim3(kNormThreads), 0, st, (const float *)a.in[0],
                        (const float *)a.in[1], has_res ? (const float *)a.in[2] : nullptr, (float *)a.out[0], n,
                        k.desc.params[0], has_res, has_scale, k.desc.params[1]);
     return done("rmsnorm launch");
@@ -335,7 +358,7 @@ int launch_rmsnorm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
 int launch_rmsnorm_add_then(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
 {
     const int n = (int)k.desc.dims[0];
-    hipLaunchKernelGGL(rmsnorm_add_then_rmsnorm_kernel, dim3(1), dim3(kNormThreads), (size_t)n * 4, st,
+    hipLaunchKernelGGL(rmsnorm_add_then_rmsnorm_kernel, dim3((unsigned)max((int64_t)1, k.desc.dims[1])), dim3(kNormThreads), (size_t)n * 4, st,
                        (const float *)a.in[0], (const float *)a.in[1], (const float *)a.in[2],
                        (const float *)a.in[3], (float *)a.out[0], (float *)a.out[1], n, k.desc.params[0]);
     return done("rmsnorm_add_then_rmsnorm launch");
@@ -344,7 +367,7 @@ int launch_rmsnorm_add_then(const ksh_kernel &k, const LaunchArgs &a, hipStream_
 int launch_per_head(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
 {
     const int n_q = (int)k.desc.dims[0], n_kv = (int)k.desc.dims[1], hd = (int)k.desc.dims[2];
-    const dim3 grid(n_q + n_kv), block(64);
+    const dim3 grid(n_q + n_kv, (unsigned)max((int64_t)1, k.desc.dims[4])), block(64);
 #define KSH_PH(HD)                                                                                           \
     hipLaunchKernelGGL((per_head_qkv_q40_kernel<HD>), grid, block, 0, st, (const float *)a.in[0],            \
                        (const float *)a.in[1], (const float *)a.in[2], (const float *)a.in[3],               \
@@ -371,7 +394,7 @@ int launch_quantize_q40(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st
 int launch_copy_scale_indexed(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
 {
     const int n = (int)k.desc.dims[0];
-    hipLaunchKernelGGL(copy_scale_indexed_kernel, dim3((n + 255) / 256), dim3(256), 0, st,
+    hipLaunchKernelGGL(copy_scale_indexed_kernel, dim3((n + 255) / 256, (unsigned)max((int64_t)1, k.desc.dims[2])), dim3(256), 0, st,
                        (const uint8_t *)a.in[0], (const float *)a.in[1], (float *)a.out[0], n, k.desc.params[0],
                        k.desc.dtypes[0], k.desc.dims[1]);
     return done("copy_scale_indexed launch");
@@ -472,25 +495,29 @@ int bind_rmsnorm(ksh_kernel &k)
     if (n <= 0 || n > (1 << 24)) return set_error("rmsnorm: n=%lld", (long long)n);
     if (k.desc.kind == KSH_RMSNORM) {
         const bool has_res = k.desc.dims[1] != 0;
+        const int64_t rows = k.desc.dims[3] ? k.desc.dims[3] : 1;
+        if (rows < 0 || rows > 65535) return set_error("rmsnorm: rows=%lld", (long long)rows);
         k.info.n_inputs = has_res ? 3 : 2;
         k.info.n_outputs = 1;
-        for (int i = 0; i < k.info.n_inputs; i++) { k.in_bytes[i] = (size_t)n * 4; k.in_align[i] = 4; }
-        k.out_bytes[0] = (size_t)n * 4;
+        for (int i = 0; i < k.info.n_inputs; i++) { k.in_bytes[i] = (size_t)n * 4 * (i == 1 ? 1 : rows); k.in_align[i] = 4; }
+        k.out_bytes[0] = (size_t)n * 4 * rows;
         k.out_align[0] = 4;
-        set_launch(k, 1, 1, 1, kNormThreads, 16);
-        set_name(k, "rmsnorm%s%s", has_res ? "_add" : "", k.desc.dims[2] ? "_scale" : "");
+        set_launch(k, (uint32_t)rows, 1, 1, kNormThreads, 16);
+        set_name(k, "rmsnorm%s%s%s", has_res ? "_add" : "", k.desc.dims[2] ? "_scale" : "", rows > 1 ? "_rows" : "");
         k.launch = launch_rmsnorm;
         return 0;
     }
     // the reference stages the residual stream in threadgroup memory and
     // refuses sizes that do not fit (lower.rs:3934-3938)
     if (n > 8192) return set_error("rmsnorm_add_then_rmsnorm requires LOCAL staging of residual stream (n=%lld > 8192)", (long long)n);
+    const int64_t rows = k.desc.dims[1] ? k.desc.dims[1] : 1;
+    if (rows < 0 || rows > 65535) return set_error("rmsnorm_add_then_rmsnorm: rows=%lld", (long long)rows);
     k.info.n_inputs = 4;
     k.info.n_outputs = 2;
-    for (int i = 0; i < 4; i++) { k.in_bytes[i] = (size_t)n * 4; k.in_align[i] = 4; }
-    for (int i = 0; i < 2; i++) { k.out_bytes[i] = (size_t)n * 4; k.out_align[i] = 4; }
-    set_launch(k, 1, 1, 1, kNormThreads, (uint32_t)n * 4 + 16);
-    set_name(k, "rmsnorm_add_then_rmsnorm");
+    for (int i = 0; i < 4; i++) { k.in_bytes[i] = (size_t)n * 4 * ((i & 1) ? 1 : rows); k.in_align[i] = 4; }   // y, w_post, res, w_ffn
+    for (int i = 0; i < 2; i++) { k.out_bytes[i] = (size_t)n * 4 * rows; k.out_align[i] = 4; }
+    set_launch(k, (uint32_t)rows, 1, 1, kNormThreads, (uint32_t)n * 4 + 16);
+    set_name(k, "rmsnorm_add_then_rmsnorm%s", rows > 1 ? "_rows" : "");
     k.launch = launch_rmsnorm_add_then;
     return 0;
 }
@@ -505,17 +532,20 @@ int bind_per_head_qkv_q40(ksh_kernel &k)
     // (7th input, f32[4] with the position in [3]); 0 for the host-offset form
     const int64_t max_seq = k.desc.dims[3];
     if (max_seq < 0 || max_seq > (1 << 24)) return set_error("rmsnorm_per_head_qkv_q40: max_seq=%lld", (long long)max_seq);
-    const size_t rows = max_seq ? (size_t)max_seq : 1;
+    // dims[4] = tokens of a chunk of consecutive positions (0 or 1: a single token)
+    const int64_t n_tok = k.desc.dims[4] ? k.desc.dims[4] : 1;
+    if (n_tok < 0 || n_tok > 65535) return set_error("rmsnorm_per_head_qkv_q40: n_tok=%lld", (long long)n_tok);
+    const size_t rows = max_seq ? (size_t)max_seq : (size_t)n_tok;
     k.info.n_inputs = max_seq ? 7 : 6;
     k.info.n_outputs = 3;
     const size_t kvb = (size_t)n_kv * (hd / 32) * 18 * rows;
-    const size_t ib[7] = {(size_t)n_q * hd * 4, (size_t)hd * 4, (size_t)hd * 4 * rows, (size_t)n_kv * hd * 4, (size_t)hd * 4,
-                          (size_t)n_kv * hd * 4, 16};
+    const size_t ib[7] = {(size_t)n_q * hd * 4 * n_tok, (size_t)hd * 4, (size_t)hd * 4 * rows, (size_t)n_kv * hd * 4 * n_tok, (size_t)hd * 4,
+                          (size_t)n_kv * hd * 4 * n_tok, 16};
     for (int i = 0; i < k.info.n_inputs; i++) { k.in_bytes[i] = ib[i]; k.in_align[i] = 4; }
-    k.out_bytes[0] = (size_t)n_q * hd * 4; k.out_align[0] = 4;
+    k.out_bytes[0] = (size_t)n_q * hd * 4 * n_tok; k.out_align[0] = 4;
     k.out_bytes[1] = k.out_bytes[2] = kvb; k.out_align[1] = k.out_align[2] = 2;
-    set_launch(k, (uint32_t)(n_q + n_kv), 1, 1, 64, 0);
-    set_name(k, "rmsnorm_per_head_qkv_q40_hd%d", (int)hd);
+    set_launch(k, (uint32_t)(n_q + n_kv), (uint32_t)n_tok, 1, 64, 0);
+    set_name(k, "rmsnorm_per_head_qkv_q40_hd%d%s", (int)hd, n_tok > 1 ? "_batch" : "");
     k.launch = launch_per_head;
     return 0;
 }
@@ -551,9 +581,13 @@ int bind_glue(ksh_kernel &k)
         k.info.n_inputs = 2;
         k.info.n_outputs = 1;
         k.in_bytes[0] = rb * (size_t)n_rows; k.in_align[0] = dt == KSH_F32 ? 4 : 2;
-        k.in_bytes[1] = 4; k.in_align[1] = 4;
-        k.out_bytes[0] = (size_t)n * 4; k.out_align[0] = 4;
-        set_name(k, "copy_scale_indexed_%d", dt);
+        // dims[2] = tokens (0 or 1: a single id)
+        const int64_t n_tok = k.desc.dims[2] ? k.desc.dims[2] : 1;
+        if (n_tok < 0 || n_tok > 65535) return set_error("copy_scale_indexed: n_tok=%lld", (long long)n_tok);
+        k.in_bytes[1] = 4 * (size_t)n_tok; k.in_align[1] = 4;
+        k.out_bytes[0] = (size_t)n * 4 * n_tok; k.out_align[0] = 4;
+        k.info.grid[1] = (uint32_t)n_tok;
+        set_name(k, "copy_scale_indexed_%d%s", dt, n_tok > 1 ? "_batch" : "");
         k.launch = launch_copy_scale_indexed;
         return 0;
     }

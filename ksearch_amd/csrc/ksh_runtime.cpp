@@ -57,7 +57,8 @@ static int bind(ksh_kernel &k)
     case KSH_SDPA_NAIVE:
     case KSH_SDPA_MWG_PART:
     case KSH_SDPA_MWG_REDUCE:
-    case KSH_SDPA_SLOTS: return bind_sdpa(k);
+    case KSH_SDPA_SLOTS:
+    case KSH_SDPA_BATCH: return bind_sdpa(k);
     case KSH_ATTEND_DECODE: return bind_attend_decode(k);
     case KSH_QUANTIZE_Q40: return bind_quantize_q40(k);
     case KSH_RMSNORM:

@@ -90,11 +90,61 @@ __global__ __launch_bounds__(256) void mm_prep_x_kernel(const uint16_t *__restri
     }
 }
 
+// The same for f32 activations (the decode loops' prompt chunks): x = hi + 2^-11 lo with hi = f16(x) and
+// lo = f16(2^11 (x - hi)), 22 bits of x, each part with its own fragments and its own sums.  The product then runs
+// twice, the second pass adding 2^-11 times its result to the first.
+__global__ __launch_bounds__(256) void mm_prep_x_f32_kernel(const float *__restrict__ X, _Float16 *__restrict__ Xf_hi,
+                                                            _Float16 *__restrict__ Xf_lo, _Float16 *__restrict__ SxA_hi,
+                                                            _Float16 *__restrict__ SxA_lo, int batch, int cols)
+{
+    const int idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= batch * (cols / 8)) return;   // (whole quads: cols is a multiple of 32)
+    const f32x4_t in0 = reinterpret_cast<const f32x4_t *>(X)[2 * (size_t)idx], in1 = reinterpret_cast<const f32x4_t *>(X)[2 * (size_t)idx + 1];
+    const float f[8] = {in0.x, in0.y, in0.z, in0.w, in1.x, in1.y, in1.z, in1.w};
+    h8 oh, ol;
+    float fh[8], fl[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const _Float16 hi = (_Float16)f[i];
+        const _Float16 lo = (_Float16)((f[i] - (float)hi) * 2048.0f);   // kept 2^11 up, in the normal range wherever hi is
+        oh[kperm(i)] = hi;
+        ol[kperm(i)] = lo;
+        fh[i] = (float)hi;
+        fl[i] = (float)lo;
+    }
+    float sh = ((fh[0] + fh[1]) + (fh[2] + fh[3])) + ((fh[4] + fh[5]) + (fh[6] + fh[7]));
+    float sl = ((fl[0] + fl[1]) + (fl[2] + fl[3])) + ((fl[4] + fl[5]) + (fl[6] + fl[7]));
+    sh += dpp_f32<0xB1>(sh);
+    sh += dpp_f32<0x4E>(sh);
+    sl += dpp_f32<0xB1>(sl);
+    sl += dpp_f32<0x4E>(sl);
+    const int k8 = cols / 8, t = idx / k8, j = idx - t * k8;
+    const size_t frag = ((size_t)(t >> 5) * (cols / 16) + (j >> 1)) * 64 + (t & 31) + 32 * (j & 1);
+    reinterpret_cast<h8 *>(Xf_hi)[frag] = oh;
+    reinterpret_cast<h8 *>(Xf_lo)[frag] = ol;
+    if ((threadIdx.x & 3) == 0) {
+        const int s = j / 4, jj = s % 8;
+        const size_t o = ((size_t)t * (cols / 256) + s / 8) * 32;
+        const float sums[2] = {sh, sl};
+        _Float16 *dst[2] = {SxA_hi + o, SxA_lo + o};
+#pragma unroll
+        for (int part = 0; part < 2; part++) {
+            const _Float16 hi = (_Float16)sums[part];
+            const _Float16 lo = (_Float16)(sums[part] - (float)hi);
+            dst[part][jj] = hi;
+            dst[part][8 + jj] = hi;
+            dst[part][16 + jj] = lo;
+            dst[part][24 + jj] = (_Float16)0.f;
+        }
+    }
+}
+
 struct MmParams {
     const uint8_t *W;
     const _Float16 *Xf, *SxA;   // fragment-ordered f16 activations (mm_prep_x_kernel), sums of x
     float *Y;
     int rows, cols, batch;
+    float accum;                // 0: store; else add `accum` times the result to Y (the second pass of f32 activations)
 };
 
 __device__ __forceinline__ uint32_t pair_f16(uint32_t masked, uint32_t sc)
@@ -426,7 +476,10 @@ __global__ __launch_bounds__(kThreadsMM) void q_mul_mm_kernel(MmParams p)
 #pragma unroll
             for (int i = 0; i < 16; i++) {
                 const int t = t0 + wm * 64 + mt * 32 + 8 * (i / 4) + 4 * (lane >> 5) + (i & 3);
-                if (t < p.batch && r < p.rows) p.Y[(size_t)t * p.rows + r] = F[mt][nt][i];
+                if (t < p.batch && r < p.rows) {
+                    float *y = &p.Y[(size_t)t * p.rows + r];
+                    *y = p.accum != 0.f ? fmaf(p.accum, F[mt][nt][i], *y) : F[mt][nt][i];
+                }
             }
         }
 }
@@ -434,19 +487,26 @@ __global__ __launch_bounds__(kThreadsMM) void q_mul_mm_kernel(MmParams p)
 int launch_mul_mm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
 {
     const int rows = (int)k.desc.dims[0], cols = (int)k.desc.dims[1], batch = (int)k.desc.dims[2];
+    const bool f32x = k.desc.dtypes[1] == KSH_F32;
+    const size_t xf_halves = (size_t)((batch + 31) / 32 * 32) * cols, sx_halves = (size_t)batch * (cols / 256) * 32;
     _Float16 *Xf = (_Float16 *)k.scratch;
-    _Float16 *SxA = Xf + (size_t)((batch + 31) / 32 * 32) * cols;
+    _Float16 *SxA = Xf + xf_halves;
+    _Float16 *Xf_lo = SxA + sx_halves, *SxA_lo = Xf_lo + xf_halves;     // f32 activations only
     const int n = batch * (cols / 8);
-    hipLaunchKernelGGL(mm_prep_x_kernel, dim3((n + 255) / 256), dim3(256), 0, st, (const uint16_t *)a.in[1], Xf, SxA, batch, cols);
+    if (f32x) hipLaunchKernelGGL(mm_prep_x_f32_kernel, dim3((n + 255) / 256), dim3(256), 0, st, (const float *)a.in[1], Xf, Xf_lo, SxA, SxA_lo, batch, cols);
+    else hipLaunchKernelGGL(mm_prep_x_kernel, dim3((n + 255) / 256), dim3(256), 0, st, (const uint16_t *)a.in[1], Xf, SxA, batch, cols);
     MmParams p;
     p.W = (const uint8_t *)a.in[0];
-    p.Xf = Xf;
-    p.SxA = SxA;
     p.Y = (float *)a.out[0];
     p.rows = rows; p.cols = cols; p.batch = batch;
     const dim3 grid((batch + BM - 1) / BM, (rows + BN - 1) / BN);
-    if (k.desc.dtypes[0] == KSH_Q6K) hipLaunchKernelGGL(q_mul_mm_kernel<true>, grid, dim3(kThreadsMM), kLdsBytes, st, p);
-    else hipLaunchKernelGGL(q_mul_mm_kernel<false>, grid, dim3(kThreadsMM), kLdsBytes, st, p);
+    for (int pass = 0; pass < (f32x ? 2 : 1); pass++) {
+        p.Xf = pass ? Xf_lo : Xf;
+        p.SxA = pass ? SxA_lo : SxA;
+        p.accum = pass ? 1.0f / 2048.0f : 0.f;
+        if (k.desc.dtypes[0] == KSH_Q6K) hipLaunchKernelGGL(q_mul_mm_kernel<true>, grid, dim3(kThreadsMM), kLdsBytes, st, p);
+        else hipLaunchKernelGGL(q_mul_mm_kernel<false>, grid, dim3(kThreadsMM), kLdsBytes, st, p);
+    }
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : hip_fail(e, "mul_mm launch");
 }
@@ -458,21 +518,22 @@ int bind_matvec_batch(ksh_kernel &k)
     const int64_t rows = k.desc.dims[0], cols = k.desc.dims[1], batch = k.desc.dims[2];
     const bool q6 = k.desc.dtypes[0] == KSH_Q6K;
     if (k.desc.dtypes[0] != KSH_Q4K && !q6) return set_error("matvec_batch: weight dtype %d is not built (Q4_K and Q6_K are)", k.desc.dtypes[0]);
-    if (k.desc.dtypes[1] != KSH_BF16) return set_error("matvec_batch: activation dtype %d is not built (BF16 is)", k.desc.dtypes[1]);
+    const bool f32x = k.desc.dtypes[1] == KSH_F32;
+    if (k.desc.dtypes[1] != KSH_BF16 && !f32x) return set_error("matvec_batch: activation dtype %d is not built (BF16 and F32 are)", k.desc.dtypes[1]);
     if (rows <= 0 || batch <= 0 || rows > (1 << 24) || batch > (1 << 20)) return set_error("matvec_batch: rows=%lld batch=%lld", (long long)rows, (long long)batch);
     if (cols <= 0 || cols % 256 || cols > (1 << 20)) return set_error("matvec_batch: cols=%lld is not a positive multiple of 256", (long long)cols);
     k.info.n_inputs = 2;
     k.info.n_outputs = 1;
     k.in_bytes[0] = (size_t)rows * (cols / 256) * (q6 ? 210 : 144); k.in_align[0] = q6 ? 2 : 16;
-    k.in_bytes[1] = (size_t)batch * cols * 2; k.in_align[1] = 16;
+    k.in_bytes[1] = (size_t)batch * cols * (f32x ? 4 : 2); k.in_align[1] = 16;
     k.out_bytes[0] = (size_t)batch * rows * 4; k.out_align[0] = 4;
     // f16 copy of X plus the min-term operand (32 halves per token and superblock)
-    k.scratch_bytes = (size_t)((batch + 31) / 32 * 32) * cols * 2 + (size_t)batch * (cols / 256) * 64;
+    k.scratch_bytes = ((size_t)((batch + 31) / 32 * 32) * cols * 2 + (size_t)batch * (cols / 256) * 64) * (f32x ? 2 : 1);
     set_launch(k, (uint32_t)((batch + BM - 1) / BM), (uint32_t)((rows + BN - 1) / BN), 1, kThreadsMM,
                (uint32_t)kLdsBytes);
     k.info.sched = k.desc.sched;
     k.info.sched.tg = kThreadsMM; k.info.sched.nsg = kThreadsMM / 64; k.info.sched.lds_tile = KS;
-    set_name(k, "mul_mm_%s_%dx%dx%d", q6 ? "q6k" : "q4k", BM, BN, KS);
+    set_name(k, "mul_mm_%s_%dx%dx%d%s", q6 ? "q6k" : "q4k", BM, BN, KS, f32x ? "_f32x" : "");
     k.launch = launch_mul_mm;
     return 0;
 }

@@ -42,6 +42,7 @@ struct SdpaParams {
     int n_q, n_kv, hd, max_t, nwg, meta_stride;
     float scale;
     int direct;             // 1: single partition, write normalised output, no tmp
+    int kv_shared;          // every slot attends the same cache (a chunk of prompt tokens)
 };
 
 __device__ __forceinline__ int pad_stride(int hd) { return hd + 4; }
@@ -65,7 +66,7 @@ __global__ __launch_bounds__(kThreads) void sdpa_part_kernel(SdpaParams p)
     const int p0 = part * chunk, p1 = min(p0 + chunk, tlen);
 
     const size_t row_bytes = (size_t)nblk * 18;
-    const size_t slot_bytes = (size_t)p.max_t * p.n_kv * row_bytes;
+    const size_t slot_bytes = p.kv_shared ? 0 : (size_t)p.max_t * p.n_kv * row_bytes;
     const uint8_t *kbase = p.k + (size_t)slot * slot_bytes;
     const uint8_t *vbase = p.v + (size_t)slot * slot_bytes;
     const float *qg = p.q + ((size_t)slot * p.n_q + (size_t)kvh * groups) * hd;
@@ -283,6 +284,38 @@ int launch_slots(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
     return done("sdpa_slots reduce launch");
 }
 
+// same per-token records as the register form writes (lower.rs:4961-4983)
+__global__ void sdpa_batch_meta_tile_kernel(const float *meta, float *tok_meta, int n_tok)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n_tok) return;
+    const int abs_t = (int)meta[0] + i, win = (int)meta[2];
+    const int tlen = min(abs_t, win);
+    tok_meta[4 * i] = (float)tlen;
+    tok_meta[4 * i + 1] = (float)(abs_t - tlen);
+    tok_meta[4 * i + 2] = (float)win;
+    tok_meta[4 * i + 3] = 0.f;
+}
+
+int launch_batch(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
+{
+    SdpaParams p = base_params(k);
+    const int n_tok = (int)k.desc.dims[4];
+    float *tok_meta = (float *)k.scratch;
+    hipLaunchKernelGGL(sdpa_batch_meta_tile_kernel, dim3((n_tok + 255) / 256), dim3(256), 0, st, (const float *)a.in[3], tok_meta, n_tok);
+    p.q = (const float *)a.in[0]; p.k = (const uint8_t *)a.in[1]; p.v = (const uint8_t *)a.in[2];
+    p.meta = tok_meta;
+    p.meta_stride = 4;
+    p.tmp = (float *)a.out[0];
+    p.out = (float *)a.out[1];
+    p.nwg = k.variant;
+    p.kv_shared = 1;
+    launch_part(p, n_tok, st);
+    if (done("sdpa_batch part launch")) return 1;
+    hipLaunchKernelGGL(sdpa_reduce_kernel, dim3(p.n_q, n_tok), dim3(kThreads), 0, st, p.tmp, p.out, p.n_q, p.hd, p.nwg);
+    return done("sdpa_batch reduce launch");
+}
+
 int check_shape(const char *what, int64_t n_q, int64_t n_kv, int64_t hd, int64_t max_t)
 {
     if (n_q <= 0 || n_kv <= 0 || n_q % n_kv || n_q / n_kv > kMaxGroups || n_q > 4096)
@@ -379,6 +412,40 @@ int bind_sdpa(ksh_kernel &k)
         k.launch = launch_slots;
         lanes_nwg = (int)nwg;
         lanes_slots = (int)n_slots;
+        break;
+    }
+    case KSH_SDPA_BATCH: {
+        // sdpa_hybrid_kv_batch (crates/ksearch_kernels/src/lib.rs:1592-1623): n_tok consecutive prompt tokens over one cache
+        const int64_t n_tok = d[4];
+        int64_t nwg = d[5];
+        if (n_tok <= 0 || n_tok > 4096) return set_error("sdpa_batch: n_tok=%lld", (long long)n_tok);
+        if (nwg == 0 && k.desc.sched.k_split) nwg = k.desc.sched.k_split;
+        if (nwg == 0) {
+            // ~4 workgroups per compute unit over all tokens, at least 64 rows per partition, at most 16 partitions
+            nwg = (1024 + n_tok * n_kv - 1) / (n_tok * n_kv);
+            const int64_t cap = (max_t + 63) / 64;
+            if (nwg > cap) nwg = cap;
+            if (nwg > 16) nwg = 16;
+            if (nwg < 1) nwg = 1;
+        }
+        if (nwg < 0 || nwg > 64) return set_error("sdpa_batch: nwg=%lld", (long long)nwg);
+        k.info.n_inputs = 4;
+        k.info.n_outputs = 2;
+        k.in_bytes[0] = (size_t)n_tok * n_q * hd * 4;
+        k.in_bytes[1] = k.in_bytes[2] = kvb;
+        k.in_bytes[3] = 12;
+        k.out_bytes[0] = (size_t)n_tok * n_q * nwg * (hd + 2) * 4;
+        k.out_bytes[1] = (size_t)n_tok * n_q * hd * 4;
+        k.out_align[1] = 4;
+        set_launch(k, (uint32_t)nwg, (uint32_t)n_kv, (uint32_t)n_tok, kThreads, lds);
+        set_name(k, "sdpa_batch_hd%d_t%d_nwg%d", (int)hd, (int)n_tok, (int)nwg);
+        k.variant = (int)nwg;
+        k.info.sched.k_split = (uint32_t)nwg;
+        k.info.sched.lds_tile = kTile;
+        k.scratch_bytes = (size_t)n_tok * 16;
+        k.launch = launch_batch;
+        lanes_nwg = (int)nwg;
+        lanes_slots = (int)n_tok;
         break;
     }
     default: return set_error("bind_sdpa: kind %d", k.desc.kind);

@@ -56,6 +56,7 @@ struct LaneParams {
     int hsplit;   // workgroups that share a kv head's rows, each with its own q heads
     int balance;  // the launch's nwg * n_slots partitions are dealt to the slots by length (kModeMerge, several slots)
     int rope_row; // fused: `rope` is the current position's row of the table, not the table
+    int kv_shared; // every slot attends the same cache (a chunk of prompt tokens, one meta record and one q per token)
     int no_append; // fused: the step's K / V row is in the cache already (a layer that reuses another layer's cache): q is normed and
                    // roped as usual, nothing is appended, every attended row comes from the cache
 };
@@ -362,6 +363,20 @@ __global__ __launch_bounds__(256) void sdpa_dealt_merge_kernel(const float *tmp,
     }
 }
 
+// Per-token records of a chunk of consecutive prompt tokens (crates/ksearch_codegen/src/lower.rs:4961-4983): token i
+// attends tlen_i = min(tlen0 + i, window) rows from start_i = tlen0 + i - tlen_i; in: {tlen0, -, window}.
+__global__ void sdpa_batch_meta_kernel(const float *meta, float *tok_meta, int n_tok)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n_tok) return;
+    const int abs_t = (int)meta[0] + i, win = (int)meta[2];
+    const int tlen = min(abs_t, win);
+    tok_meta[4 * i] = (float)tlen;
+    tok_meta[4 * i + 1] = (float)(abs_t - tlen);
+    tok_meta[4 * i + 2] = (float)win;
+    tok_meta[4 * i + 3] = 0.f;
+}
+
 // grid = (nwg, n_kv, n_slots)
 template <int HD, int GP, int NW>
 __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
@@ -399,7 +414,7 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
         rec_base = (size_t)first + part;   // flat partition index: values [flat][n_q][HD], then (m, l) [flat][n_q][2]
     }
 
-    const size_t slot_bytes = (size_t)p.max_t * p.n_kv * ROWB;
+    const size_t slot_bytes = p.kv_shared ? 0 : (size_t)p.max_t * p.n_kv * ROWB;
     const uint8_t *kbase = p.k + (size_t)slot * slot_bytes + (size_t)kvh * ROWB + 18 * b;
     const uint8_t *vbase = p.v + (size_t)slot * slot_bytes + (size_t)kvh * ROWB + 18 * b;
     const size_t row_stride = (size_t)p.n_kv * ROWB;
@@ -837,6 +852,22 @@ int launch_bound(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
             return e == hipSuccess ? 0 : hip_fail(e, "sdpa merge launch");
         }
         break;
+    case KSH_SDPA_BATCH: {
+        // in: q, K, V, meta{tlen of token 0, -, window}   out: tmp, o.  The per-token records are written by a small
+        // kernel into the handle's scratch (behind the counters); K and V are shared by all tokens.
+        n_slots = (int)k.desc.dims[4];
+        float *tok_meta = (float *)((uint8_t *)k.scratch + (((size_t)n_slots * p.n_kv * p.hsplit * 4 + 15) & ~(size_t)15));
+        hipLaunchKernelGGL(sdpa_batch_meta_kernel, dim3((n_slots + 255) / 256), dim3(256), 0, st, (const float *)a.in[3], tok_meta, n_slots);
+        p.q = (const float *)a.in[0]; p.k = (const uint8_t *)a.in[1]; p.v = (const uint8_t *)a.in[2];
+        p.meta = tok_meta;
+        p.meta_stride = 4;
+        p.tmp = (float *)a.out[0];
+        p.out = (float *)a.out[1];
+        p.scale = k.desc.params[0];
+        p.mode = kModeMerge;
+        p.kv_shared = 1;
+        break;
+    }
     case KSH_ATTEND_DECODE: {
         const bool reader = k.desc.dims[7] != 0;
         p.q = (const float *)a.in[0]; p.qw = (const float *)a.in[1]; p.rope = (const float *)a.in[2];
@@ -904,11 +935,12 @@ int bind_sdpa_lanes(ksh_kernel &k, int nwg, int n_slots)
     if (hd == 512 && total_groups / hsplit > 4) return set_error("sdpa: heads of 512 take at most four q heads per workgroup (unroll=%d leaves %d)", hsplit, total_groups / hsplit);
     const int wg_groups = total_groups / hsplit;
     const size_t lds = lanes_lds(hd, wg_groups, nw);
-    const bool merges = k.desc.kind == KSH_SDPA_SLOTS || (k.desc.kind == KSH_ATTEND_DECODE && !k.desc.dims[5]);
+    const bool merges = k.desc.kind == KSH_SDPA_SLOTS || k.desc.kind == KSH_SDPA_BATCH || (k.desc.kind == KSH_ATTEND_DECODE && !k.desc.dims[5]);
     if (merges && !(k.desc.kind == KSH_SDPA_SLOTS && balanced_slots(n_slots, nwg)) &&   // (those merge in a launch of their own)
         (size_t)wg_groups * (nwg + 16) * 3 * 4 > (size_t)nw * (64 / (hd / 8)) * ((wg_groups <= 4 ? 4 : 8) * hd) * 4)
         return set_error("sdpa: nwg=%d is too many partitions for the merge", nwg);
     k.scratch_bytes = (size_t)n_slots * n_kv * hsplit * 4;
+    if (k.desc.kind == KSH_SDPA_BATCH) k.scratch_bytes = ((k.scratch_bytes + 15) & ~(size_t)15) + (size_t)n_slots * 16;   // + per-token records
     set_launch(k, (uint32_t)nwg, (uint32_t)(n_kv * hsplit), (uint32_t)n_slots, (uint32_t)nw * 64, (uint32_t)lds);
     k.info.sched = k.desc.sched;
     k.info.sched.tg = (uint64_t)nw * 64;

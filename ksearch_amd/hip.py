@@ -63,6 +63,7 @@ class Kind(enum.IntEnum):           # enum ksh_kind
     ADD_SCALE = 26
     MATVEC_GELU_MUL = 27
     READ_FLOOR = 28
+    SDPA_BATCH = 29
 
 
 class Sched(C.Structure):           # ksh_sched: OptSchedule retargeted to gfx950
@@ -175,6 +176,7 @@ SYMBOLS = {
     "ksh_gemma_destroy": (None, [_vp]),
     "ksh_gemma_reset": (_i, [_vp]),
     "ksh_gemma_forward_token": (_i, [_vp, C.c_uint32, _i, C.POINTER(C.c_uint32)]),
+    "ksh_gemma_prefill_chunk": (_i, [_vp, C.POINTER(C.c_uint32), _i]),
     "ksh_gemma_generate": (_i, [_vp, C.POINTER(C.c_uint32), _i, _i, _i, C.POINTER(C.c_uint32), _dp, _dp]),
     "ksh_gemma_logits": (_vp, [_vp]),
     "ksh_gemma_hidden": (_vp, [_vp]),
@@ -795,11 +797,17 @@ class Gemma:
         _check(lib().ksh_gemma_forward_token(self.h, int(token), int(use_graph), C.byref(nxt) if read_next else None))
         return nxt.value if read_next else None
 
-    def generate(self, prompt, n_new: int, use_graph: bool = True):
+    def prefill_chunk(self, tokens) -> None:
+        """prefill_chunk: the tokens at the current position, no logits; batched per layer in chunks of 256."""
+        p = (C.c_uint32 * max(1, len(tokens)))(*[int(t) for t in tokens])
+        _check(lib().ksh_gemma_prefill_chunk(self.h, p, len(tokens)))
+
+    def generate(self, prompt, n_new: int, use_graph: bool = True, serial_prefill: bool = False):
         p = (C.c_uint32 * len(prompt))(*[int(t) for t in prompt])
         out = (C.c_uint32 * max(1, n_new))()
         pre, dec = C.c_double(), C.c_double()
-        _check(lib().ksh_gemma_generate(self.h, p, len(prompt), n_new, int(use_graph), out, C.byref(pre), C.byref(dec)))
+        flags = int(bool(use_graph)) | (2 if serial_prefill else 0)
+        _check(lib().ksh_gemma_generate(self.h, p, len(prompt), n_new, flags, out, C.byref(pre), C.byref(dec)))
         return list(out[:n_new]), pre.value, dec.value
 
     def logits(self) -> np.ndarray:

@@ -226,6 +226,8 @@ def bench_decode(ctx, eng, use_graph=True):
     prompt = [int(t) for t in np.random.default_rng(4001).integers(0, cfg["vocab"], 64)]
     m.generate(prompt, 8, use_graph=use_graph)     # warm-up: binds kernels, captures the graphs
     m.reset()
+    _, serial_pre_ms, _ = m.generate(prompt, 1, use_graph=use_graph, serial_prefill=True)
+    m.reset()
     _, pre_ms, dec_ms = m.generate(prompt, 256, use_graph=use_graph)
     h, f, hd = cfg["hidden"], cfg["ffn"], cfg["hd"]
     layer = (cfg["n_q"] * hd * h + 2 * cfg["n_kv"] * hd * h + h * cfg["n_q"] * hd + 3 * f * h) // 256 * 144
@@ -233,7 +235,9 @@ def bench_decode(ctx, eng, use_graph=True):
     out = dict(tok_per_s=round(256 / dec_ms * 1e3, 1), ms_per_token=round(dec_ms / 256, 4),
                launches_per_token=m.launches_per_token, weight_gbps=round(per_tok * 256 / (dec_ms * 1e-3) / 1e9, 1),
                frac_hbm=round(per_tok * 256 / (dec_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
-               prompt_tokens=64, new_tokens=256, graph=bool(use_graph))
+               prompt_tokens=64, new_tokens=256, graph=bool(use_graph),
+               prefill_ms=round(pre_ms, 3), prefill_tok_per_s=round(63 / pre_ms * 1e3, 1),
+               prefill_ms_token_by_token=round(serial_pre_ms, 3))
     m.close()
     return out
 

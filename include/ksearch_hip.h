@@ -201,7 +201,8 @@ enum ksh_kind {
 };
 
 /* OptSchedule (crates/ksearch_ir/src/kernel.rs:11-18) retargeted to gfx950.
- * All-zero means "library default, or the plan cache's entry if one exists". */
+ * All-zero means "library default, or the plan cache's entry if one exists"; tg = all ones (the other fields zero)
+ * means "library default, whatever the plan cache holds". */
 typedef struct {
     uint64_t tg;       /* threads per workgroup (64 * waves) */
     uint32_t vec;      /* inner-product variant: 1 = byte converts + f32 FMA, 3 = int8 dot over 3 digit planes */

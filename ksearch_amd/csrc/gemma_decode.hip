@@ -163,6 +163,32 @@ int enc(ksh_gemma *m, ksh_kernel *k, std::initializer_list<ksh_buf *> in, std::i
     return ksh_encode(m->ctx, k, ib, nullptr, ni, ob, nullptr, no);
 }
 
+// Schedule search at load (Eng::warm_matvec_plans + beam_matvec, gemma_prim.rs:254-290, ksearch_kernels/src/lib.rs:
+// 1985-2080): the kind is timed on the model's own buffers over its candidate schedules and the winner saved in the
+// plan cache, where the kernel lookups that follow find it; a plan that is there already is taken as it is.  A kind
+// without a schedule space, or whose search fails, keeps the library default.
+void warm_plan(ksh_gemma *m, int kind, std::initializer_list<int64_t> dims, std::initializer_list<int> dtypes,
+               std::initializer_list<float> params, std::initializer_list<ksh_buf *> in, std::initializer_list<ksh_buf *> out)
+{
+    ksh_kernel_desc d;
+    memset(&d, 0, sizeof(d));
+    d.kind = kind;
+    int i = 0;
+    for (int64_t v : dims) d.dims[i++] = v;
+    i = 0;
+    for (int v : dtypes) d.dtypes[i++] = v;
+    i = 0;
+    for (float v : params) d.params[i++] = v;
+    ksh_buf *ib[kMaxIn], *ob[kMaxOut];
+    int ni = 0, no = 0;
+    for (ksh_buf *b : in) ib[ni++] = b;
+    for (ksh_buf *b : out) ob[no++] = b;
+    ksh_sched best;
+    double ms = 0.0;
+    int cached = 0;
+    (void)ksh_beam_search(m->ctx, &d, ib, ni, ob, no, 8, 0, &best, &ms, &cached);
+}
+
 // Up to this many cached positions the attention launch leaves its (then 8) partitions unmerged and the
 // o-projection folds them in its prologue: 0.8 us per layer less at 320 positions, 1.5 us more at 1500,
 // where 16 partitions and the merge inside the attention launch win.
@@ -387,7 +413,8 @@ int ksh_gemma_create(ksh_ctx *ctx, const ksh_gemma_cfg *cfg, const ksh_gemma_lay
         g->rope0.assign(tab.begin(), tab.begin() + c.hd);
         if (alloc(g, (size_t)c.hd * 4, &g->rope_cur)) return 1;   // the current position's row (advance_kernel keeps it so)
     }
-    if (alloc(g, (size_t)c.n_q * std::max(g->nwg, kShortPartitions) * (c.hd + 2) * 4, &g->attn_tmp)) return 1;
+    constexpr int kMaxPartitions = 64;   // the partials buffer holds the largest K-split a schedule may choose
+    if (alloc(g, (size_t)c.n_q * kMaxPartitions * (c.hd + 2) * 4, &g->attn_tmp)) return 1;
 
     // The LM head streams the whole table every token: it gets a copy with each row's fields grouped (whole
     // 128-bit loads, 84 instead of 101 us at 262144 x 2048); the embedding gather keeps reading the Q6_K original.
@@ -399,6 +426,27 @@ int ksh_gemma_create(ksh_ctx *ctx, const ksh_gemma_cfg *cfg, const ksh_gemma_lay
             return 1;
         int n = 0;
         if (enc(g, rp, {g->embd}, {g->embd_rows}, n) || ksh_synchronize(ctx)) return 1;
+    }
+    const bool fused_attend = sdpa_lanes_supports(c.n_q, c.n_kv, c.hd);
+    if (!getenv("KSEARCH_SKIP_BEAM")) {   // gemma_prim.rs:271-286
+        const ksh_gemma_layer &L = g->layers[0];
+        const float T = (float)std::min(c.max_seq, 1024);
+        const float meta[4] = {T, 0.f, 0.f, T - 1.f};
+        if (ksh_buffer_write(ctx, g->meta, 0, meta, 16, 1)) return 1;
+        ksh_buf *lm_w = g->embd_rows ? g->embd_rows : g->embd;
+        warm_plan(g, KSH_RMSNORM_MATVEC_QKV, {qd, kvd, c.hidden, 0}, {KSH_Q4K, KSH_F32}, {c.eps}, {L.wq, L.wk, L.wv, g->x, L.attn_norm}, {g->tq, g->tk, g->tv});
+        warm_plan(g, KSH_RMSNORM_MATVEC_QKV, {qd, kvd, c.hidden, 1}, {KSH_Q4K, KSH_F32}, {c.eps},
+                  {L.wq, L.wk, L.wv, g->y, L.attn_norm, L.post_ffw_norm, g->x}, {g->tq, g->tk, g->tv, g->xb});
+        warm_plan(g, KSH_MATVEC, {c.hidden, qd}, {KSH_Q4K, KSH_F32}, {}, {L.wo, g->to}, {g->y});
+        warm_plan(g, KSH_RMSNORM_MATVEC_GATE_UP_GELU, {c.ffn, c.hidden, 1}, {KSH_Q4K, KSH_F32}, {c.eps},
+                  {L.wgate, L.wup, g->y, L.ffn_norm, L.post_attn_norm, g->x}, {g->ff, g->xb});
+        warm_plan(g, KSH_MATVEC, {c.hidden, c.ffn}, {KSH_Q4K, KSH_F32}, {}, {L.wdown, g->ff}, {g->y});
+        warm_plan(g, KSH_RMSNORM_MATVEC, {c.vocab, c.hidden, 1}, {lm_rows ? KSH_Q6K_ROWS : KSH_Q6K, KSH_F32}, {c.eps},
+                  {lm_w, g->y, g->output_norm, L.post_ffw_norm, g->x}, {g->logits, g->xb});
+        if (fused_attend)
+            warm_plan(g, KSH_ATTEND_DECODE, {c.n_q, c.n_kv, c.hd, c.max_seq, 0, 0, 1}, {KSH_Q40, KSH_F32}, {c.eps, c.attn_scale},
+                      {g->tq, L.q_norm, g->rope_cur, g->tk, L.k_norm, g->tv, g->meta}, {g->kv_k[0], g->kv_v[0], g->attn_tmp, g->to});
+        if (ksh_synchronize(ctx)) return 1;
     }
     const float embed_scale = std::sqrt((float)c.hidden);   // gemma_prim.rs:683
     if (get(g, KSH_COPY_SCALE_INDEXED, {c.hidden, c.vocab}, {KSH_Q6K}, {embed_scale}, &g->k_embed) ||
@@ -412,10 +460,15 @@ int ksh_gemma_create(ksh_ctx *ctx, const ksh_gemma_cfg *cfg, const ksh_gemma_lay
         return 1;
     // per-head norm + RoPE + KV append + attention + merge: one launch where the fused kind is built for the
     // shape, the three reference ops otherwise
-    if (sdpa_lanes_supports(c.n_q, c.n_kv, c.hd)) {
-        if (get(g, KSH_ATTEND_DECODE, {c.n_q, c.n_kv, c.hd, c.max_seq, g->nwg, 0, 1}, {KSH_Q40, KSH_F32}, {c.eps, c.attn_scale},
+    if (fused_attend) {
+        // the partition count (K-split) is the schedule's: the plan cache's, or the kind's default
+        if (get(g, KSH_ATTEND_DECODE, {c.n_q, c.n_kv, c.hd, c.max_seq, 0, 0, 1}, {KSH_Q40, KSH_F32}, {c.eps, c.attn_scale},
                 &g->k_attend))
             return 1;
+        ksh_kernel_info info;
+        if (ksh_kernel_info_get(g->k_attend, &info)) return 1;
+        g->nwg = (int)info.sched.k_split;
+        if (g->nwg < 1 || g->nwg > kMaxPartitions) return set_error("attend_decode: schedule with %d partitions", g->nwg);
         g->short_context = kShortContext;
         if (const char *e = getenv("KSEARCH_SHORT_CONTEXT")) g->short_context = atoi(e);
         if (g->short_context > 0 && qd <= 2048 && (c.hd & (c.hd - 1)) == 0 &&

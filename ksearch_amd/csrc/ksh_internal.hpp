@@ -122,6 +122,7 @@ int bind_softcap_argmax(ksh_kernel &k);
 int bind_ple_ops(ksh_kernel &k);       // RMSNORM_PER_HEAD, ADD_SCALE, MATVEC_GELU_MUL
 int bind_read_floor(ksh_kernel &k);
 
+int plan_dims(const ksh_kernel_desc &d);   // how many leading dims take part in a plan's key
 // candidate schedules per kind (BEAM)
 int matvec_candidates(const ksh_kernel_desc &d, ksh_sched *out, int cap);
 

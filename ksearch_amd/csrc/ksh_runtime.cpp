@@ -276,22 +276,25 @@ int ksh_kernel_get(ksh_ctx *ctx, const ksh_kernel_desc *desc, ksh_kernel **out)
     }
     ksh_sched planned{};
     bool have_plan = false;
+    // tg = all ones asks for the library's default schedule whatever the plan cache holds (the schedule search times
+    // it as the incumbent); such a handle has its own cache entry
+    const bool library_default = key.sched.tg == ~0ull;
     if (sched_is_zero(key.sched)) {
         // plan lookup by (kind, dims, chip), crates/ksearch_codegen/src/lib.rs:80-90
         const char *pk = ksh_plan_kind(&key);
         if (pk) {
-            int nd = 0;
-            while (nd < 8 && key.dims[nd] != 0) nd++;
             double ms;
-            have_plan = ksh_plan_load(pk, key.dims, nd, ctx->chip.c_str(), &planned, &ms) == 0;
+            have_plan = ksh_plan_load(pk, key.dims, plan_dims(key), ctx->chip.c_str(), &planned, &ms) == 0;
         }
     }
     auto k = std::make_unique<ksh_kernel>();
     k->desc = key;
     if (have_plan) k->desc.sched = planned;
+    if (library_default) memset(&k->desc.sched, 0, sizeof(k->desc.sched));
     if (bind(*k)) {
         // a stale or foreign plan must not make a kernel unusable
         if (!have_plan) return 1;
+        fprintf(stderr, "[ksearch_hip] plan for kind %d refused (%s); using the default schedule\n", key.kind, ksh_last_error());
         k = std::make_unique<ksh_kernel>();
         k->desc = key;
         if (bind(*k)) return 1;

@@ -538,4 +538,15 @@ int bind_matvec_batch(ksh_kernel &k)
     return 0;
 }
 
+// schedules of the prefill GEMM: the 128 x 128 tile with K depth 64 (the only tile built so far)
+int mul_mm_candidates(const ksh_kernel_desc &d, ksh_sched *out, int cap)
+{
+    (void)d;
+    if (cap < 1) return 0;
+    ksh_sched s{};
+    s.tg = kThreadsMM; s.nsg = kThreadsMM / 64; s.nr0 = BN; s.lds_tile = KS; s.unroll = 1; s.vec = 0; s.k_split = 1;
+    out[0] = s;
+    return 1;
+}
+
 }  // namespace ksh

@@ -18,6 +18,42 @@ namespace ksh {
 
 int matvec_q4k_candidates(const ksh_kernel_desc &d, ksh_sched *out, int cap);
 int matvec_q6k_candidates(const ksh_kernel_desc &d, ksh_sched *out, int cap);
+int mul_mm_candidates(const ksh_kernel_desc &d, ksh_sched *out, int cap);
+
+// dims that take part in a plan's key: everything up to the last non-zero entry (a zero in the middle -- a flag
+// that is off, a partition count left to the schedule -- is part of the shape)
+int plan_dims(const ksh_kernel_desc &d)
+{
+    int nd = 0;
+    for (int i = 0; i < 8; i++)
+        if (d.dims[i] != 0) nd = i + 1;
+    return nd;
+}
+
+// Split-KV attention (sdpa_q40: KSH_SDPA_SLOTS / KSH_SDPA_BATCH with the partition count left open, and
+// attend_decode_q40): K-split = partitions per sequence, waves per workgroup, and for the fused decode step the
+// number of workgroups that share a kv head's rows (each with its share of the q heads).
+static int sdpa_candidates(const ksh_kernel_desc &d, ksh_sched *out, int cap)
+{
+    const bool attend = d.kind == KSH_ATTEND_DECODE;
+    const int64_t nwg_dim = attend ? d.dims[4] : d.dims[5];
+    const int64_t max_t = d.dims[3], groups = d.dims[1] > 0 ? d.dims[0] / d.dims[1] : 1;
+    int n = 0;
+    for (uint32_t ks : {0u, 4u, 8u, 16u, 32u, 64u}) {
+        if ((ks == 0) != (nwg_dim != 0)) continue;            // a fixed partition count leaves only the other knobs
+        if (ks && (int64_t)ks * 32 > max_t && ks > 4) continue;   // fewer than 32 rows per partition
+        for (uint32_t nsg : {4u, 8u})
+            for (uint32_t hs : {1u, 2u, 4u, 8u}) {
+                if (!attend && hs != 1) continue;
+                if (hs > groups || groups % hs) continue;
+                if (n >= cap) return n;
+                ksh_sched s{};
+                s.tg = 64ull * nsg; s.vec = 0; s.unroll = attend ? hs : 0; s.nsg = nsg; s.nr0 = 0; s.k_split = ks;
+                out[n++] = s;
+            }
+    }
+    return n;
+}
 
 namespace {
 
@@ -151,8 +187,9 @@ const char *ksh_plan_kind(const ksh_kernel_desc *d)
     switch (d->kind) {
     case KSH_MATVEC:
         // crates/ksearch_codegen/src/lib.rs:200-205
-        return d->dtypes[0] == KSH_Q4K ? "matvec_q4k" : d->dtypes[0] == KSH_Q6K ? "matvec_q6k" : nullptr;
-    case KSH_RMSNORM_MATVEC: return d->dtypes[0] == KSH_Q4K ? "rms_matvec_q4k" : d->dtypes[0] == KSH_Q6K ? "rms_matvec_q6k" : nullptr;
+        return d->dtypes[0] == KSH_Q4K ? "matvec_q4k" : d->dtypes[0] == KSH_Q6K ? "matvec_q6k" : d->dtypes[0] == KSH_Q6K_ROWS ? "matvec_q6krows" : nullptr;
+    case KSH_RMSNORM_MATVEC:
+        return d->dtypes[0] == KSH_Q4K ? "rms_matvec_q4k" : d->dtypes[0] == KSH_Q6K ? "rms_matvec_q6k" : d->dtypes[0] == KSH_Q6K_ROWS ? "rms_matvec_q6krows" : nullptr;
     case KSH_MATVEC_QKV: return "matvec_qkv_q4k";
     case KSH_RMSNORM_MATVEC_QKV: return "rms_matvec_qkv_q4k";
     case KSH_MATVEC_GATE_UP_GELU: return "matvec_gate_up_q4k";
@@ -160,6 +197,7 @@ const char *ksh_plan_kind(const ksh_kernel_desc *d)
     case KSH_MATVEC_BATCH: return d->dtypes[0] == KSH_Q6K ? "mul_mm_q6k" : "mul_mm_q4k";
     case KSH_SDPA_SLOTS:
     case KSH_SDPA_MWG_PART: return "sdpa_q40";
+    case KSH_SDPA_BATCH: return "sdpa_q40_batch";
     case KSH_ATTEND_DECODE: return "attend_decode_q40";
     case KSH_ATTN_MERGE_MATVEC: return "attn_merge_matvec_q4k";
     }
@@ -171,15 +209,19 @@ int ksh_beam_candidates(const ksh_kernel_desc *d, ksh_sched *out, int cap)
     if (!d || !out || cap <= 0) return 0;
     switch (d->kind) {
     case KSH_MATVEC:
-        if (d->dtypes[0] == KSH_Q6K) return matvec_q6k_candidates(*d, out, cap);
+        if (d->dtypes[0] == KSH_Q6K || d->dtypes[0] == KSH_Q6K_ROWS) return matvec_q6k_candidates(*d, out, cap);
         return matvec_q4k_candidates(*d, out, cap);
     case KSH_RMSNORM_MATVEC:
-        if (d->dtypes[0] == KSH_Q6K) return matvec_q6k_candidates(*d, out, cap);
+        if (d->dtypes[0] == KSH_Q6K || d->dtypes[0] == KSH_Q6K_ROWS) return matvec_q6k_candidates(*d, out, cap);
         return matvec_q4k_candidates(*d, out, cap);
     case KSH_MATVEC_QKV:
     case KSH_MATVEC_GATE_UP_GELU:
     case KSH_RMSNORM_MATVEC_QKV:
     case KSH_RMSNORM_MATVEC_GATE_UP_GELU: return matvec_q4k_candidates(*d, out, cap);
+    case KSH_MATVEC_BATCH: return mul_mm_candidates(*d, out, cap);
+    case KSH_SDPA_SLOTS:
+    case KSH_SDPA_BATCH:
+    case KSH_ATTEND_DECODE: return sdpa_candidates(*d, out, cap);
     }
     return 0;
 }
@@ -193,8 +235,7 @@ int ksh_beam_search(ksh_ctx *ctx, const ksh_kernel_desc *desc, ksh_buf *const *i
     if (!pk) return set_error("ksh_beam_search: kind %d has no schedule space", desc->kind);
     char chip[128];
     if (ksh_device_name(ctx, chip, sizeof(chip))) return 1;
-    int nd = 0;
-    while (nd < 8 && desc->dims[nd] != 0) nd++;
+    const int nd = plan_dims(*desc);
     if (from_cache) *from_cache = 0;
     // KSEARCH_BEAM_FORCE, crates/ksearch_codegen/src/lib.rs:206
     if (!force && !std::getenv("KSEARCH_BEAM_FORCE") && ksh_plan_load(pk, desc->dims, nd, chip, best, best_ms) == 0) {
@@ -206,22 +247,48 @@ int ksh_beam_search(ksh_ctx *ctx, const ksh_kernel_desc *desc, ksh_buf *const *i
     if (n <= 0) return set_error("ksh_beam_search: no candidates for kind %d", desc->kind);
     if (iters < 1) iters = 3;
     bool found = false;
+    std::string refusal;
+    // The library's own default goes first (no plan file exists at this point, or the search is forced): a candidate
+    // replaces it only when it is at least 3 % faster, so that timing noise between near-equal schedules does not
+    // move a shape off the schedule its default was chosen for.
+    double default_ms = 0.0;
+    {
+        ksh_kernel_desc d = *desc;
+        memset(&d.sched, 0, sizeof(d.sched));
+        d.sched.tg = ~0ull;   // the library default, whatever the plan cache holds
+        ksh_kernel *k = nullptr;
+        double ms = 0.0;
+        if (ksh_kernel_get(ctx, &d, &k) == 0 &&
+            ksh_run_timed(ctx, k, inputs, nullptr, n_in, outputs, nullptr, n_out, 1, &ms) == 0 &&
+            ksh_run_timed(ctx, k, inputs, nullptr, n_in, outputs, nullptr, n_out, iters, &ms) == 0) {
+            ksh_kernel_info info;
+            ksh_kernel_info_get(k, &info);
+            found = true;
+            default_ms = ms;
+            *best_ms = ms;
+            *best = info.sched;
+        }
+    }
     for (int i = 0; i < n; i++) {
         ksh_kernel_desc d = *desc;
         d.sched = cand[i];
         ksh_kernel *k = nullptr;
         if (ksh_kernel_get(ctx, &d, &k)) continue;   // a candidate the kernel family refuses
         double ms = 0.0;
-        // 1 warm-up + timed launches, crates/ksearch_kernels/src/lib.rs:2015-2031
-        if (ksh_run_timed(ctx, k, inputs, nullptr, n_in, outputs, nullptr, n_out, 1, &ms)) return 1;
+        // 1 warm-up + timed launches, crates/ksearch_kernels/src/lib.rs:2015-2031.  A candidate whose bindings do
+        // not fit (a partition count the caller's scratch buffer was not sized for) is passed over like a refused one.
+        if (ksh_run_timed(ctx, k, inputs, nullptr, n_in, outputs, nullptr, n_out, 1, &ms)) {
+            refusal = ksh_last_error();
+            continue;
+        }
         if (ksh_run_timed(ctx, k, inputs, nullptr, n_in, outputs, nullptr, n_out, iters, &ms)) return 1;
-        if (!found || ms < *best_ms) {
+        if (!found || (ms < *best_ms && (default_ms == 0.0 || ms < 0.97 * default_ms))) {
             found = true;
             *best_ms = ms;
             *best = cand[i];
         }
     }
-    if (!found) return set_error("ksh_beam_search: every candidate was refused");
+    if (!found) return set_error("ksh_beam_search: every candidate was refused (%s)", refusal.c_str());
     return ksh_plan_save(pk, desc->dims, nd, chip, best, *best_ms);
 }
 

@@ -380,6 +380,7 @@ int bind_sdpa(ksh_kernel &k)
         const int64_t n_slots = d[4];
         int64_t nwg = d[5];
         if (n_slots <= 0 || n_slots > 65535) return set_error("sdpa_slots: n_slots=%lld", (long long)n_slots);
+        if (nwg == 0 && k.desc.sched.k_split) nwg = k.desc.sched.k_split;   // K-split from the schedule
         if (nwg == 0 && lanes) {
             // two workgroups per CU, at least 64 rows each, and few enough partials for one workgroup to fold
             nwg = (512 + n_slots * n_kv - 1) / (n_slots * n_kv);

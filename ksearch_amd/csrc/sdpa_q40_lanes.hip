@@ -964,6 +964,7 @@ int bind_attend_decode(ksh_kernel &k)
         return set_error("attend_decode: built for hd 128, 256 or 512 and up to 8 q heads per kv head (got hd=%lld, %lld)",
                          (long long)hd, (long long)(n_q / n_kv));
     if (max_t <= 0 || max_t > (1 << 24)) return set_error("attend_decode: max_seq=%lld", (long long)max_t);
+    if (nwg == 0 && k.desc.sched.k_split) nwg = k.desc.sched.k_split;   // K-split from the schedule
     if (nwg == 0) nwg = max_t >= 2048 ? 16 : (max_t + 127) / 128;
     const size_t kvb = (size_t)max_t * n_kv * (hd / 32) * 18, qb = (size_t)n_q * hd * 4, kb = (size_t)n_kv * hd * 4;
     const bool parts_only = d[5] != 0, reader = d[7] != 0;

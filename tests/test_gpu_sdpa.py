@@ -318,3 +318,61 @@ def test_attn_merge_matvec_errors(ctx):
         ctx.compile(hip.make_desc(hip.Kind.ATTN_MERGE_MATVEC, (2048, 8, 96, 4), (DType.Q4K, DType.F32), ()))
     with pytest.raises(hip.KshError, match="one float4 per thread"):
         ctx.compile(hip.make_desc(hip.Kind.ATTN_MERGE_MATVEC, (2048, 16, 256, 4), (DType.Q4K, DType.F32), ()))
+
+
+def test_beam_search_attention_kinds(ctx, tmp_path, monkeypatch):
+    """The schedule search over the attention kinds' knobs (K-split = partitions per sequence, waves per workgroup,
+    workgroups per kv head for the fused decode step): every candidate is timed on the device, the winner is saved
+    under KSEARCH_BEAM_CACHE keyed by kind, dims and chip, a second search is served from the file, a kernel
+    requested with an all-zero schedule in a fresh context picks the plan up, and the result stays the oracle's."""
+    monkeypatch.setenv("KSEARCH_BEAM_CACHE", str(tmp_path / "beam"))
+    n_slots, n_q, n_kv, hd, max_t = 2, 8, 1, 256, 2048
+    lens, kk, vv, q = synth.cfg3_q40_attention(n_slots=n_slots, max_t=max_t, lo=700, seed=1203)
+    meta = np.zeros((n_slots, 4), np.float32)
+    meta[:, 0] = lens
+    desc = hip.make_desc(hip.Kind.SDPA_SLOTS, (n_q, n_kv, hd, max_t, n_slots, 0), (hip.DType.Q40, hip.DType.F32), (1.0 / 16.0,))
+    cands = [c.as_dict() for c in hip.beam_candidates(desc)]
+    assert len(cands) >= 6 and {c["k_split"] for c in cands} >= {8, 16, 32} and {c["nsg"] for c in cands} == {4, 8}
+    ins = [ctx.buffer_f32(q), ctx.buffer_bytes(kk), ctx.buffer_bytes(vv), ctx.buffer_f32(meta)]
+    outs = [ctx.buffer_empty_f32(n_slots * n_q * 64 * (hd + 2)), ctx.buffer_empty_f32(n_slots * n_q * hd)]
+    best, ms, cached = ctx.beam_search(desc, ins, outs, iters=5, force=True)
+    assert not cached and 0 < ms < 1.0 and best.k_split >= 1
+    files = list((tmp_path / "beam").glob("sdpa_q40_*.txt"))
+    assert len(files) == 1
+    best2, _, cached2 = ctx.beam_search(desc, ins, outs, iters=5)
+    assert cached2 and best2.as_dict() == best.as_dict()
+    ctx2 = hip.Context()
+    try:
+        k = ctx2.compile(desc)
+        assert k.info.sched.k_split == best.k_split and k.info.sched.nsg == best.nsg
+        ins2 = [ctx2.buffer_f32(q), ctx2.buffer_bytes(kk), ctx2.buffer_bytes(vv), ctx2.buffer_f32(meta)]
+        outs2 = [ctx2.buffer_empty_f32(n_slots * n_q * k.info.sched.k_split * (hd + 2)), ctx2.buffer_empty_f32(n_slots * n_q * hd)]
+        ctx2.encode_multi(k, ins2, outs2)
+        ctx2.synchronize()
+        got = ctx2.read_f32(outs2[1], n_slots * n_q * hd).reshape(n_slots, -1)
+        for s in range(n_slots):
+            want = oracle.sdpa(q[s], kk[s], vv[s], n_q, n_kv, hd, int(lens[s]), 0, 1.0 / 16.0)
+            assert_close(got[s], want, 1e-3, f"slot {s} under the planned schedule")
+    finally:
+        ctx2.close()
+    # the fused decode step: K-split, waves and the head split are all open
+    d2 = hip.make_desc(hip.Kind.ATTEND_DECODE, (n_q, n_kv, hd, max_t, 0, 0, 0), (hip.DType.Q40, hip.DType.F32), (1e-6, 1.0 / 16.0))
+    c2 = [c.as_dict() for c in hip.beam_candidates(d2)]
+    assert {c["unroll"] for c in c2} == {1, 2, 4, 8} and {c["k_split"] for c in c2} >= {8, 16, 32}
+    rope = oracle.rope_table(max_t, hd, 10000.0)
+    raw_q, raw_k, raw_v = synth.normal_f32(n_q * hd, 1210), synth.normal_f32(hd, 1211), synth.normal_f32(hd, 1212)
+    m2 = np.array([601, 0, 0, 600], np.float32)
+    ones = np.ones(hd, np.float32)
+    ins3 = [ctx.buffer_f32(raw_q), ctx.buffer_f32(ones), ctx.buffer_f32(rope), ctx.buffer_f32(raw_k), ctx.buffer_f32(ones),
+            ctx.buffer_f32(raw_v), ctx.buffer_f32(m2)]
+    kc, vc = ctx.buffer_bytes(kk[0]), ctx.buffer_bytes(vv[0])
+    outs3 = [kc, vc, ctx.buffer_empty_f32(n_q * 64 * (hd + 2)), ctx.buffer_empty_f32(n_q * hd)]
+    best3, ms3, cached3 = ctx.beam_search(d2, ins3, outs3, iters=5, force=True)
+    assert not cached3 and 0 < ms3 < 1.0
+    assert len(list((tmp_path / "beam").glob("attend_decode_q40_*.txt"))) == 1
+    # whichever candidate ran last left the oracle's result for that step
+    q_o, k_row, v_row = oracle.rmsnorm_per_head_qkv_q40(raw_q, ones, rope[600], raw_k, ones, raw_v, n_q, n_kv, hd, 1e-6)
+    kh, vh = kk[0].copy(), vv[0].copy()
+    kh[600 * 144:601 * 144], vh[600 * 144:601 * 144] = k_row, v_row
+    want = oracle.sdpa(q_o, kh, vh, n_q, n_kv, hd, 601, 0, 1.0 / 16.0)
+    assert_close(ctx.read_f32(outs3[3], n_q * hd), want, 1e-3, "attend_decode after the search")

@@ -484,6 +484,142 @@ __global__ __launch_bounds__(kThreadsMM) void q_mul_mm_kernel(MmParams p)
         }
 }
 
+// ---- small batches (up to 64 tokens): a GEMV-shaped launch on the matrix cores ---------------------------------
+// A prompt remainder or a round of decoding slots is a few dozen tokens: the 128 x 128 tile then leaves most of the
+// chip idle (rows / 128 workgroups) and half of every tile empty.  Here a workgroup owns 32 weight rows and all
+// tokens; its 8 waves split the row's superblocks between them (K-split inside the workgroup, folded through LDS at
+// the end, so the sum order is fixed) and every wave reads its weights straight from memory in the order the matrix
+// instruction wants its B operand: lane (n, h) = (lane % 32, lane / 32) owns row n and, in every 16-column slice,
+// columns 8h .. 8h+7 -- per 64-column group the low and the high nibbles of bytes 8h .. 8h+7 and 16+8h .. 16+8h+7,
+// two 8-byte loads.  Conversion (sc*n as exact f16, biased by 1024), the per-superblock scale and the bias / min
+// product are those of the big tile; the activations come as the same fragments, hi and lo part in the same pass
+// (each converted weight is used for both), so f32 activations cost one launch.
+template <int MT, bool HAS_LO>
+__global__ __launch_bounds__(512) void q4k_mm_skinny_kernel(MmParams p, const _Float16 *__restrict__ Xf_lo, const _Float16 *__restrict__ SxA_lo,
+                                                             float lo_scale)
+{
+    extern __shared__ __attribute__((aligned(16))) float red[];   // [8][MT][16][64]
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 31, h = lane >> 5;
+    const int r0 = blockIdx.x * 32, nsb = p.cols / 256;
+    const size_t row_bytes = (size_t)nsb * 144;
+    const uint8_t *wrow = p.W + (size_t)min(r0 + n, p.rows - 1) * row_bytes;
+    const int ntt = (p.batch + 31) / 32;
+    const h8 *xa[MT], *xl[MT];
+    const _Float16 *sxa[MT], *sxl[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++) {
+        const size_t frag0 = (size_t)min(mt, ntt - 1) * (p.cols / 16) * 64 + lane;
+        xa[mt] = reinterpret_cast<const h8 *>(p.Xf) + frag0;
+        xl[mt] = reinterpret_cast<const h8 *>(HAS_LO ? Xf_lo : p.Xf) + frag0;
+        const size_t so = (size_t)min(mt * 32 + n, p.batch - 1) * nsb * 32 + 8 * h;   // + sb * 32 + 16 * ks
+        sxa[mt] = p.SxA + so;
+        sxl[mt] = (HAS_LO ? SxA_lo : p.SxA) + so;
+    }
+    f16v F[MT], Fl[MT];
+    const f16v kZero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++) { F[mt] = kZero16; Fl[mt] = kZero16; }
+
+    for (int sb = wave; sb < nsb; sb += 8) {
+        const uint8_t *blk = wrow + (size_t)sb * 144;
+        const u32x4_t hdr = *reinterpret_cast<const u32x4_t *>(blk);
+        u32x2_t q[4][2];
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            q[g][0] = *reinterpret_cast<const u32x2_t *>(blk + 16 + 32 * g + 8 * h);
+            q[g][1] = *reinterpret_cast<const u32x2_t *>(blk + 16 + 32 * g + 16 + 8 * h);
+        }
+        f16v C[MT], Cl[MT];
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            // this group's activation fragments: slices 4g .. 4g+3 of the superblock
+            h8 a[MT][4], al[MT][4];
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const size_t o = (size_t)(sb * 16 + 4 * g + j) * 64;
+                    a[mt][j] = xa[mt][o];
+                    if (HAS_LO) al[mt][j] = xl[mt][o];
+                }
+            const uint4 s = q4k_group_scales(hdr.y, hdr.z, hdr.w, g);   // sc_lo, mn_lo, sc_hi, mn_hi
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                // slice j: bytes (j & 1 ? 16 + 8h : 8h) .. +7, low nibbles for j < 2, high nibbles after
+                const u32x2_t qq = q[g][j & 1];
+                const uint32_t sc = j < 2 ? s.x : s.z;
+                uint32_t o[4];
+#pragma unroll
+                for (int i = 0; i < 2; i++) {
+                    const uint32_t d = j < 2 ? qq[i] : qq[i] >> 4;
+                    o[2 * i] = pair_f16(d & 0x000F000Fu, sc);
+                    o[2 * i + 1] = pair_f16((d >> 8) & 0x000F000Fu, sc);
+                }
+                const u32x4_t ov = {o[0], o[1], o[2], o[3]};
+                const h8 b = __builtin_bit_cast(h8, ov);
+#pragma unroll
+                for (int mt = 0; mt < MT; mt++) {
+                    C[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mt][j], b, (g == 0 && j == 0) ? kZero16 : C[mt], 0, 0, 0);
+                    if (HAS_LO) Cl[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al[mt][j], b, (g == 0 && j == 0) ? kZero16 : Cl[mt], 0, 0, 0);
+                }
+            }
+        }
+        // bias + mins of the superblock: the row's eight coefficients -(dmin*m_j + 1024*d) as f16 hi | lo, against the
+        // tokens' sums of x (hi[8] hi[8] lo[8] 0[8] per token and superblock): hi*hi + hi*lo + lo*hi
+        const float d = half_bits_to_f32(hdr.x & 0xFFFFu), dmin = half_bits_to_f32(hdr.x >> 16);
+        _Float16 chi[8], clo[8];
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const uint4 s = q4k_group_scales(hdr.y, hdr.z, hdr.w, g);
+            const float c0 = -(dmin * (float)s.y + 1024.f * d), c1 = -(dmin * (float)s.w + 1024.f * d);
+            chi[2 * g] = (_Float16)c0; chi[2 * g + 1] = (_Float16)c1;
+            clo[2 * g] = (_Float16)(c0 - (float)chi[2 * g]); clo[2 * g + 1] = (_Float16)(c1 - (float)chi[2 * g + 1]);
+        }
+        h8 b2[2];
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            b2[0][i] = h ? clo[i] : chi[i];                 // columns 0..7: hi, 8..15: lo
+            b2[1][i] = h ? (_Float16)0.f : chi[i];          // columns 16..23: hi, 24..31: zero
+        }
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) {
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++) {
+                const h8 a2 = *reinterpret_cast<const h8 *>(sxa[mt] + (size_t)sb * 32 + 16 * ks);
+                F[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a2, b2[ks], F[mt], 0, 0, 0);
+                if (HAS_LO) {
+                    const h8 a2l = *reinterpret_cast<const h8 *>(sxl[mt] + (size_t)sb * 32 + 16 * ks);
+                    Fl[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a2l, b2[ks], Fl[mt], 0, 0, 0);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                F[mt][i] = fmaf(d, C[mt][i], F[mt][i]);
+                if (HAS_LO) Fl[mt][i] = fmaf(d, Cl[mt][i], Fl[mt][i]);
+            }
+        }
+    }
+    // fold the eight waves' shares (fixed order), then store: accumulator i of lane (n, h) is token
+    // 8*(i/4) + 4*h + i%4 of the tile, weight row n
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+        for (int i = 0; i < 16; i++)
+            red[((wave * MT + mt) * 16 + i) * 64 + lane] = HAS_LO ? fmaf(lo_scale, Fl[mt][i], F[mt][i]) : F[mt][i];
+    __syncthreads();
+    for (int o = tid; o < MT * 16 * 64; o += 512) {
+        float sum = 0.f;
+#pragma unroll
+        for (int w = 0; w < 8; w++) sum += red[w * MT * 16 * 64 + o];
+        const int mt = o / (16 * 64), i = (o / 64) & 15, l = o & 63;
+        const int t = mt * 32 + 8 * (i / 4) + 4 * (l >> 5) + (i & 3), r = r0 + (l & 31);
+        if (t < p.batch && r < p.rows) p.Y[(size_t)t * p.rows + r] = sum;
+    }
+}
+
+constexpr int kSkinnyMaxBatch = 64;
+
 int launch_mul_mm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
 {
     const int rows = (int)k.desc.dims[0], cols = (int)k.desc.dims[1], batch = (int)k.desc.dims[2];
@@ -499,6 +635,19 @@ int launch_mul_mm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
     p.W = (const uint8_t *)a.in[0];
     p.Y = (float *)a.out[0];
     p.rows = rows; p.cols = cols; p.batch = batch;
+    if (k.variant == 1) {
+        // the small-batch form: one launch, the low parts riding along
+        p.Xf = Xf; p.SxA = SxA; p.accum = 0.f;
+        const dim3 sg((rows + 31) / 32);
+        const int mt = batch <= 32 ? 1 : 2;
+        const size_t lds = (size_t)8 * mt * 16 * 64 * 4;
+        if (f32x && mt == 1) hipLaunchKernelGGL((q4k_mm_skinny_kernel<1, true>), sg, dim3(512), lds, st, p, Xf_lo, SxA_lo, 1.0f / 2048.0f);
+        else if (f32x) hipLaunchKernelGGL((q4k_mm_skinny_kernel<2, true>), sg, dim3(512), lds, st, p, Xf_lo, SxA_lo, 1.0f / 2048.0f);
+        else if (mt == 1) hipLaunchKernelGGL((q4k_mm_skinny_kernel<1, false>), sg, dim3(512), lds, st, p, Xf, SxA, 0.f);
+        else hipLaunchKernelGGL((q4k_mm_skinny_kernel<2, false>), sg, dim3(512), lds, st, p, Xf, SxA, 0.f);
+        const hipError_t e2 = hipGetLastError();
+        return e2 == hipSuccess ? 0 : hip_fail(e2, "mul_mm (small batch) launch");
+    }
     const dim3 grid((batch + BM - 1) / BM, (rows + BN - 1) / BN);
     for (int pass = 0; pass < (f32x ? 2 : 1); pass++) {
         p.Xf = pass ? Xf_lo : Xf;
@@ -529,24 +678,45 @@ int bind_matvec_batch(ksh_kernel &k)
     k.out_bytes[0] = (size_t)batch * rows * 4; k.out_align[0] = 4;
     // f16 copy of X plus the min-term operand (32 halves per token and superblock)
     k.scratch_bytes = ((size_t)((batch + 31) / 32 * 32) * cols * 2 + (size_t)batch * (cols / 256) * 64) * (f32x ? 2 : 1);
+    // schedule: nr0 = weight rows per workgroup.  32 = the small-batch form (Q4_K, up to 64 tokens: the default
+    // there), 128 = the 128 x 128 tile.
+    const uint32_t want = k.desc.sched.nr0;
+    if (want && want != 32 && want != BN) return set_error("matvec_batch: unsupported schedule nr0=%u (32 or %d)", want, BN);
+    const bool can_skinny = !q6 && batch <= kSkinnyMaxBatch;
+    if (want == 32 && !can_skinny) return set_error("matvec_batch: the small-batch form takes Q4_K weights and up to %d tokens", kSkinnyMaxBatch);
+    k.variant = (want == 32 || (want == 0 && can_skinny)) ? 1 : 0;
+    k.info.sched = k.desc.sched;
+    if (k.variant == 1) {
+        set_launch(k, (uint32_t)((rows + 31) / 32), 1, 1, 512, (uint32_t)(8 * (batch <= 32 ? 1 : 2) * 16 * 64 * 4));
+        k.info.sched.tg = 512; k.info.sched.nsg = 8; k.info.sched.nr0 = 32; k.info.sched.k_split = 8; k.info.sched.lds_tile = 16;
+        set_name(k, "mul_mm_q4k_skinny_32xT%d%s", batch <= 32 ? 32 : 64, f32x ? "_f32x" : "");
+        k.launch = launch_mul_mm;
+        return 0;
+    }
     set_launch(k, (uint32_t)((batch + BM - 1) / BM), (uint32_t)((rows + BN - 1) / BN), 1, kThreadsMM,
                (uint32_t)kLdsBytes);
-    k.info.sched = k.desc.sched;
-    k.info.sched.tg = kThreadsMM; k.info.sched.nsg = kThreadsMM / 64; k.info.sched.lds_tile = KS;
+    k.info.sched.tg = kThreadsMM; k.info.sched.nsg = kThreadsMM / 64; k.info.sched.nr0 = BN; k.info.sched.k_split = 1; k.info.sched.lds_tile = KS;
     set_name(k, "mul_mm_%s_%dx%dx%d%s", q6 ? "q6k" : "q4k", BM, BN, KS, f32x ? "_f32x" : "");
     k.launch = launch_mul_mm;
     return 0;
 }
 
-// schedules of the prefill GEMM: the 128 x 128 tile with K depth 64 (the only tile built so far)
+// schedules of the prefill GEMM: the 128 x 128 tile with K depth 64 (LDS-staged, one K range per workgroup) and, for
+// Q4_K weights and up to 64 tokens, 32 weight rows per workgroup with the K range split over its 8 waves
 int mul_mm_candidates(const ksh_kernel_desc &d, ksh_sched *out, int cap)
 {
-    (void)d;
-    if (cap < 1) return 0;
-    ksh_sched s{};
-    s.tg = kThreadsMM; s.nsg = kThreadsMM / 64; s.nr0 = BN; s.lds_tile = KS; s.unroll = 1; s.vec = 0; s.k_split = 1;
-    out[0] = s;
-    return 1;
+    int n = 0;
+    if (n < cap) {
+        ksh_sched s{};
+        s.tg = kThreadsMM; s.nsg = kThreadsMM / 64; s.nr0 = BN; s.lds_tile = KS; s.unroll = 1; s.vec = 0; s.k_split = 1;
+        out[n++] = s;
+    }
+    if (n < cap && d.dtypes[0] == KSH_Q4K && d.dims[2] <= kSkinnyMaxBatch) {
+        ksh_sched s{};
+        s.tg = 512; s.nsg = 8; s.nr0 = 32; s.lds_tile = 16; s.unroll = 1; s.vec = 0; s.k_split = 8;
+        out[n++] = s;
+    }
+    return n;
 }
 
 }  // namespace ksh

@@ -124,16 +124,20 @@ def test_sdpa_batch_equals_the_serial_oracle(ctx, hd, n_q, n_kv, sched, t, pos0,
     del row
 
 
-@pytest.mark.parametrize("wdt", [DType.Q4K, DType.Q6K])
-def test_mul_mm_f32_activations(ctx, wdt):
+@pytest.mark.parametrize("wdt,batch,sched", [(DType.Q4K, 45, None), (DType.Q6K, 45, None), (DType.Q4K, 5, None), (DType.Q4K, 32, None),
+                                             (DType.Q4K, 64, None), (DType.Q4K, 45, dict(nr0=128)), (DType.Q4K, 100, None)])
+def test_mul_mm_f32_activations(ctx, wdt, batch, sched):
     """f32 activations go through as hi + lo f16 parts: the result keeps the GEMV's accuracy (1e-5 of the float64
-    product), where a single f16 rounding of x would leave 3e-4."""
-    rows, cols, batch = 384, 2048, 45
+    product), where a single f16 rounding of x would leave 3e-4.  Up to 64 tokens over Q4_K weights take the
+    small-batch form (32 weight rows per workgroup, K split over its waves) unless the schedule asks for the
+    128 x 128 tile; both forms, one and two token tiles, a ragged last row tile."""
+    rows, cols = 400, 2048
     w = synth.q4k_blocks(rows * cols // 256, 720) if wdt == DType.Q4K else synth.q6k_blocks(rows * cols // 256, 720)
     x = synth.normal_f32(batch * cols, 721).reshape(batch, cols)
     x[3] *= 1e-3           # small rows: the low part is kept 2^11 up, so it stays a normal f16
     x[4] *= 300.0
-    k = ctx.compile(hip.make_desc(Kind.MATVEC_BATCH, (rows, cols, batch), (wdt, DType.F32, DType.F32)))
+    k = ctx.compile(hip.make_desc(Kind.MATVEC_BATCH, (rows, cols, batch), (wdt, DType.F32, DType.F32), (), sched))
+    assert ("skinny" in k.name) == (wdt == DType.Q4K and batch <= 64 and sched is None), k.name
     by = ctx.buffer_empty_f32(batch * rows)
     ctx.encode_multi(k, [ctx.buffer_bytes(w), ctx.buffer_f32(x)], [by])
     ctx.synchronize()

@@ -259,16 +259,18 @@ def bench_decode_gemma4_layout(ctx, eng, use_graph=True):
     w = synth.gemma4_weights(cfg, 1005, q4k, lambda x: q6k([x]), ffn=ffn)
     model = hip.Gemma4(ctx, cfg, w)
     prompt = [int(t) for t in np.random.default_rng(1005).integers(0, cfg["vocab"], 64)]
-    ms = []
+    ms, pre = [], []
     for _ in range(3):
         model.reset()
-        ids, _, decode_ms = model.generate(prompt, 256, use_graph=use_graph)
+        ids, prefill_ms, decode_ms = model.generate(prompt, 256, use_graph=use_graph)
         ms.append(decode_ms)
+        pre.append(prefill_ms)
     # bytes a token streams: every packed matrix once (the per-layer table contributes one row)
     wbytes = sum(b.nbytes for lw in w["layers"] for b in lw.values() if isinstance(b, hip.Buffer))
     wbytes += w["globals"]["token_embd"].nbytes + w["globals"]["ple_model_proj"].nbytes
     r = {"tok_s": round(256 / min(ms) * 1e3, 1), "ms_per_token": round(min(ms) / 256, 4), "launches_per_token": model.launches_per_token,
          "weight_GB_per_token": round(wbytes / 1e9, 3), "GB_s": round(wbytes / (min(ms) / 256 * 1e-3) / 1e9, 1),
+         "prefill_ms": round(min(pre), 3), "prefill_tok_per_s": round(63 / min(pre) * 1e3, 1),
          "layout": "35 layers, hidden 1536, 4 SWA(256, window 512) : 1 full(512), 20 shared-KV layers, PLE 256, ffn 6144/12288"}
     # the same model under the slot scheduler: two requests of 64 + 128 tokens decoded in turn from two KV slots
     # (serial GPU work, one host read-back per token, as the reference's serving loop does it)

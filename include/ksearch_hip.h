@@ -453,8 +453,10 @@ int ksh_sample_softcap_min_p(const float *logits, size_t n, float cap, float tem
  * temperature < 1e-6: the device argmax; else the logits are read back and ksh_sample_softcap_min_p draws. */
 int ksh_gemma4_decode_token_sampled(ksh_gemma4 *m, uint32_t token, float temperature, float min_p, uint32_t seed,
                                     int use_graph, uint32_t *next_id);
-/* GemmaPrimModel::prefill_chunk (gemma_prim.rs:1305-1315): n tokens without logits, then one synchronisation
- * (token by token here: the layer stack has no batched prefill). */
+/* GemmaPrimModel::prefill_chunk (gemma_prim.rs:1305-1607): n tokens without logits, then one synchronisation.
+ * Chunks of up to 256 tokens run as one batched pass per layer (forward_prefill_chunk), a chunk of one token as a
+ * decode step.  use_graph & 1: decode steps replay the captured graph; use_graph & 2: every token goes through the
+ * decode step (no batching).  ksh_gemma4_generate / _generate_until feed the prompt through this with the same flags. */
 int ksh_gemma4_prefill_chunk(ksh_gemma4 *m, const uint32_t *tokens, int n, int use_graph);
 
 /* ---- decode-before-prefill slot scheduler: spawn_scheduler and its rounds (crates/ksearch_cli/src/scheduler.rs:

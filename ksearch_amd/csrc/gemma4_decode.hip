@@ -61,6 +61,18 @@ __global__ void seek4_kernel(float *meta_full, float *meta_swa, int pos, const f
     }
 }
 
+// start of a prompt chunk: the records the batched attention reads ({rows the first token attends, -, window}), from
+// the device-side position; full-attention layers see everything up to the token, sliding-window layers the last
+// `window` rows (gemma_prim.rs:1426-1436)
+__global__ void chunk_begin4_kernel(const float *meta_full, float *bmeta_full, float *bmeta_swa, int max_seq, int window)
+{
+    if (threadIdx.x == 0) {
+        const float tlen0 = meta_full[3] + 1.0f;
+        bmeta_full[0] = tlen0; bmeta_full[1] = 0.f; bmeta_full[2] = (float)max_seq; bmeta_full[3] = 0.f;
+        bmeta_swa[0] = tlen0; bmeta_swa[1] = 0.f; bmeta_swa[2] = (float)window; bmeta_swa[3] = 0.f;
+    }
+}
+
 __global__ void set_token4_kernel(float *tok, float value)
 {
     if (threadIdx.x == 0 && blockIdx.x == 0) tok[0] = value;
@@ -116,6 +128,10 @@ struct ksh_gemma4 {
     std::vector<SlotGraphs> slot_graphs;
     SlotGraphs own_graphs;
     int bound_slot = -1;
+    // prompt chunks (allocated at the first chunk): [kChunk, .] activations of the batched layer pass
+    ksh_buf *c_tok = nullptr, *c_x = nullptr, *c_x2 = nullptr, *c_y = nullptr, *c_q = nullptr, *c_k = nullptr, *c_v = nullptr, *c_o = nullptr,
+            *c_g = nullptr, *c_u = nullptr, *c_ff = nullptr, *c_tmp = nullptr, *c_meta_full = nullptr, *c_meta_swa = nullptr,
+            *c_ple_tok = nullptr, *c_ple_tmp = nullptr, *c_ple_ctx = nullptr, *c_ple_u = nullptr;
 };
 
 namespace {
@@ -338,6 +354,116 @@ int write_token(ksh_gemma4 *m, uint32_t token)
 }
 
 // gemma_prim.rs:33-56: per position cos[0..hd/2) || sin[0..hd/2); pairs past `angles` are the identity
+// prefill_chunk's chunk length (gemma_prim.rs:16)
+constexpr int kChunk4 = 256;
+constexpr int kChunkPartitions4 = 8;
+
+int chunk_buffers4(ksh_gemma4 *m)
+{
+    if (m->c_tok) return 0;
+    const ksh_gemma4_cfg &c = m->c;
+    const size_t T = kChunk4, max_hd = (size_t)std::max(c.hd_swa, c.hd_full), qd = c.n_q * max_hd, kvd = c.n_kv * max_hd;
+    size_t max_ff = 0;
+    for (const ksh_gemma4_layer &L : m->layers) max_ff = std::max(max_ff, (size_t)L.ffn);
+    const size_t pt = (size_t)c.n_layers * c.ple_dim;
+    if (alloc(m, T * 4, &m->c_tok) || alloc(m, T * c.hidden * 4, &m->c_x) || alloc(m, T * c.hidden * 4, &m->c_x2) ||
+        alloc(m, T * c.hidden * 4, &m->c_y) || alloc(m, T * qd * 4, &m->c_q) || alloc(m, T * kvd * 4, &m->c_k) ||
+        alloc(m, T * kvd * 4, &m->c_v) || alloc(m, T * qd * 4, &m->c_o) || alloc(m, T * max_ff * 4, &m->c_g) ||
+        alloc(m, T * max_ff * 4, &m->c_u) || alloc(m, T * max_ff * 4, &m->c_ff) ||
+        alloc(m, T * c.n_q * kChunkPartitions4 * (max_hd + 2) * 4, &m->c_tmp) || alloc(m, 16, &m->c_meta_full) || alloc(m, 16, &m->c_meta_swa))
+        return 1;
+    if (c.ple_dim > 0 && (alloc(m, T * pt * 4, &m->c_ple_tok) || alloc(m, T * pt * 4, &m->c_ple_tmp) || alloc(m, T * pt * 4, &m->c_ple_ctx) ||
+                          alloc(m, T * c.ple_dim * 4, &m->c_ple_u)))
+        return 1;
+    return 0;
+}
+
+// forward_prefill_chunk (gemma_prim.rs:1317-1607) for 2 <= t <= kChunk4 validated tokens: every layer as matrices
+// of t rows, with the layer kinds' own head sizes, rope tables and windows, cache-reading layers attending over their
+// source layer's rows, and the per-layer-embedding block.  The GEMMs run on the batch rounded up to 32 rows.
+int forward_prefill_chunk4(ksh_gemma4 *m, const uint32_t *tokens, int t)
+{
+    const ksh_gemma4_cfg &c = m->c;
+    if (chunk_buffers4(m)) return 1;
+    const int64_t h = c.hidden, tp = (t + 31) / 32 * 32, pt = (int64_t)c.n_layers * c.ple_dim;
+    float ids[kChunk4];
+    for (int i = 0; i < t; i++) ids[i] = (float)tokens[i];
+    if (ksh_synchronize(m->ctx)) return 1;                                   // c_tok may still be read by the previous chunk
+    if (ksh_buffer_write(m->ctx, m->c_tok, 0, ids, (size_t)t * 4, 1)) return 1;
+    hipStream_t st = (hipStream_t)ksh_stream(m->ctx);
+    hipLaunchKernelGGL(chunk_begin4_kernel, dim3(1), dim3(64), 0, st, (const float *)ksh_buffer_device_ptr(m->meta_full),
+                       (float *)ksh_buffer_device_ptr(m->c_meta_full), (float *)ksh_buffer_device_ptr(m->c_meta_swa), c.max_seq, c.sliding_window);
+    if (hipGetLastError() != hipSuccess) return set_error("chunk_begin launch failed");
+    int n = 0;
+    ksh_kernel *k = nullptr, *k_norm = nullptr, *k_add = nullptr, *k_add_then = nullptr;
+    auto mm = [&](int dt, int64_t rows, int64_t cols, ksh_buf *w, ksh_buf *x, ksh_buf *y) {
+        ksh_kernel *kk = nullptr;
+        return get(m, KSH_MATVEC_BATCH, {rows, cols, tp}, {dt, KSH_F32, KSH_F32}, {}, &kk) || enc(m, kk, {w, x}, {y}, n);
+    };
+    if (get(m, KSH_COPY_SCALE_INDEXED, {h, c.vocab, t}, {m->g.dt_embd}, {std::sqrt((float)c.hidden)}, &k) ||
+        enc(m, k, {m->g.token_embd, m->c_tok}, {m->c_x}, n))
+        return 1;
+    if (c.ple_dim > 0) {
+        // ple_from_idx_batch + ple_prepass_batch (gemma_prim.rs:1333-1358)
+        ksh_kernel *kg = nullptr, *kn = nullptr, *kmix = nullptr;
+        if (get(m, KSH_COPY_SCALE_INDEXED, {pt, c.vocab, t}, {m->g.dt_ple}, {std::sqrt((float)c.ple_dim)}, &kg) ||
+            enc(m, kg, {m->g.ple_embd, m->c_tok}, {m->c_ple_tok}, n) ||
+            mm(m->g.dt_ple_proj, pt, h, m->g.ple_model_proj, m->c_x, m->c_ple_tmp) ||
+            get(m, KSH_RMSNORM_PER_HEAD, {(int64_t)t * c.n_layers, c.ple_dim, 0}, {}, {c.eps}, &kn) ||
+            enc(m, kn, {m->c_ple_tmp, m->g.ple_proj_norm}, {m->c_ple_ctx}, n) ||
+            get(m, KSH_ADD_SCALE, {(int64_t)t * pt}, {}, {0.70710678118654752440f}, &kmix) ||
+            enc(m, kmix, {m->c_ple_ctx, m->c_ple_tok}, {m->c_ple_ctx}, n))
+            return 1;
+    }
+    if (get(m, KSH_RMSNORM, {h, 0, 0, t}, {}, {c.eps}, &k_norm) || get(m, KSH_RMSNORM, {h, 1, 0, t}, {}, {c.eps}, &k_add) ||
+        get(m, KSH_RMSNORM_ADD_THEN_RMSNORM, {h, t}, {}, {c.eps}, &k_add_then))
+        return 1;
+    for (int l = 0; l < c.n_layers; l++) {
+        const ksh_gemma4_layer &L = m->layers[l];
+        const LayerPlan &P = m->plan[l];
+        ksh_buf *rope_tab = P.swa ? m->rope_swa : m->rope_full;
+        ksh_buf *kc = m->kv_k[P.src], *vc = m->kv_v[P.src];
+        ksh_kernel *k_head = nullptr, *k_sdpa = nullptr, *k_gelu = nullptr;
+        if (enc(m, k_norm, {m->c_x, L.attn_norm}, {m->c_x2}, n) || mm(L.dt_q, P.qd, h, L.wq, m->c_x2, m->c_q)) return 1;
+        if (P.owns) {
+            if (mm(L.dt_k, P.kvd, h, L.wk, m->c_x2, m->c_k) || mm(L.dt_v, P.kvd, h, L.wv, m->c_x2, m->c_v) ||
+                get(m, KSH_RMSNORM_PER_HEAD_QKV_Q40, {c.n_q, c.n_kv, P.hd, c.max_seq, t}, {}, {c.eps}, &k_head) ||
+                enc(m, k_head, {m->c_q, L.q_norm, rope_tab, m->c_k, L.k_norm, m->c_v, m->meta_full}, {m->c_q, kc, vc}, n))
+                return 1;
+        } else {
+            if (get(m, KSH_RMSNORM_PER_HEAD, {(int64_t)t * c.n_q, P.hd, 2, c.max_seq, c.n_q}, {}, {c.eps}, &k_head) ||
+                enc(m, k_head, {m->c_q, L.q_norm, rope_tab, m->meta_full}, {m->c_q}, n))
+                return 1;
+        }
+        if (get(m, KSH_SDPA_BATCH, {c.n_q, c.n_kv, P.hd, c.max_seq, t, kChunkPartitions4}, {KSH_Q40, KSH_F32}, {c.attn_scale}, &k_sdpa) ||
+            enc(m, k_sdpa, {m->c_q, kc, vc, P.swa ? m->c_meta_swa : m->c_meta_full}, {m->c_tmp, m->c_o}, n) ||
+            mm(L.dt_o, h, P.qd, L.wo, m->c_o, m->c_y) ||
+            enc(m, k_add_then, {m->c_y, L.post_attn_norm, m->c_x, L.ffn_norm}, {m->c_x, m->c_x2}, n) ||
+            mm(L.dt_gate, L.ffn, h, L.wgate, m->c_x2, m->c_g) || mm(L.dt_up, L.ffn, h, L.wup, m->c_x2, m->c_u) ||
+            get(m, KSH_GELU_MUL, {(int64_t)t * L.ffn}, {}, {}, &k_gelu) || enc(m, k_gelu, {m->c_g, m->c_u}, {m->c_ff}, n) ||
+            mm(L.dt_down, h, L.ffn, L.wdown, m->c_ff, m->c_y) || enc(m, k_add, {m->c_y, L.post_ffw_norm, m->c_x}, {m->c_x}, n))
+            return 1;
+        if (c.ple_dim > 0) {
+            // gemma_prim.rs:1558-1600: u = gelu(Wg x) * ctx_l; x = (x + rms(Wp u) * post_norm) * layer_scale
+            ksh_kernel *k_gs = nullptr, *k_as = nullptr;
+            if (mm(L.dt_inp_gate, c.ple_dim, h, L.inp_gate, m->c_x, m->c_ple_u) ||
+                get(m, KSH_GELU_MUL, {(int64_t)t * c.ple_dim, c.ple_dim, pt}, {}, {}, &k_gs) ||
+                enc_off(m, k_gs, {m->c_ple_u, m->c_ple_ctx}, {0, (size_t)l * c.ple_dim * 4}, {m->c_ple_u}, n) ||
+                mm(L.dt_proj, h, c.ple_dim, L.proj, m->c_ple_u, m->c_y) ||
+                get(m, KSH_RMSNORM, {h, 1, 1, t}, {}, {c.eps, L.layer_scale}, &k_as) ||
+                enc(m, k_as, {m->c_y, L.post_norm, m->c_x}, {m->c_x}, n))
+                return 1;
+        }
+    }
+    m->pos += t;
+    const int at = std::min(m->pos, c.max_seq - 1);
+    hipLaunchKernelGGL(seek4_kernel, dim3(1), dim3(64), 0, st, (float *)ksh_buffer_device_ptr(m->meta_full),
+                       (float *)ksh_buffer_device_ptr(m->meta_swa), at, (const float *)ksh_buffer_device_ptr(m->rope_full),
+                       (float *)ksh_buffer_device_ptr(m->cur_full), c.hd_full, (const float *)ksh_buffer_device_ptr(m->rope_swa),
+                       (float *)ksh_buffer_device_ptr(m->cur_swa), c.hd_swa, c.sliding_window);
+    return hipGetLastError() == hipSuccess ? 0 : set_error("seek launch failed");
+}
+
 int make_rope(ksh_gemma4 *m, int hd, float theta, int angles, ksh_buf **table, ksh_buf **cur, std::vector<float> &row0)
 {
     const int half = hd / 2, max_seq = m->c.max_seq;
@@ -585,16 +711,13 @@ int ksh_gemma4_generate(ksh_gemma4 *m, const uint32_t *prompt, int n_prompt, int
     using clk = std::chrono::steady_clock;
     const auto t0 = clk::now();
     // all prompt tokens but the last go through without logits (gemma_prim.rs:1670-1675)
-    for (int i = 0; i + 1 < n_prompt; i++) {
-        if (write_token(m, prompt[i])) return 1;
-        if (run_token(m, false, use_graph != 0)) return 1;
-    }
+    if (ksh_gemma4_prefill_chunk(m, prompt, n_prompt - 1, use_graph)) return 1;   // (use_graph & 2: token by token)
     if (write_token(m, prompt[n_prompt - 1])) return 1;
     if (ksh_synchronize(m->ctx)) return 1;
     const auto t1 = clk::now();
     const int first = m->pos;
     for (int i = 0; i < n_new; i++)
-        if (run_token(m, true, use_graph != 0)) return 1;
+        if (run_token(m, true, (use_graph & 1) != 0)) return 1;
     if (ksh_synchronize(m->ctx)) return 1;
     const auto t2 = clk::now();
     if (prefill_ms) *prefill_ms = std::chrono::duration<double, std::milli>(t1 - t0).count();
@@ -621,10 +744,7 @@ int ksh_gemma4_generate_until(ksh_gemma4 *m, const uint32_t *prompt, int n_promp
         if (prompt[i] >= (uint32_t)m->c.vocab) return set_error("token id %u is outside the vocabulary", prompt[i]);
     using clk = std::chrono::steady_clock;
     const auto t0 = clk::now();
-    for (int i = 0; i + 1 < n_prompt; i++) {
-        if (write_token(m, prompt[i])) return 1;
-        if (run_token(m, false, use_graph != 0)) return 1;
-    }
+    if (ksh_gemma4_prefill_chunk(m, prompt, n_prompt - 1, use_graph)) return 1;   // (use_graph & 2: token by token)
     if (write_token(m, prompt[n_prompt - 1])) return 1;
     if (ksh_synchronize(m->ctx)) return 1;
     const auto t1 = clk::now();
@@ -642,7 +762,7 @@ int ksh_gemma4_generate_until(ksh_gemma4 *m, const uint32_t *prompt, int n_promp
     };
     bool stopped = false;
     for (int i = 0; i < n_new && !stopped; i++) {
-        if (run_token(m, true, use_graph != 0) || ksh_flush_async(m->ctx)) return 1;
+        if (run_token(m, true, (use_graph & 1) != 0) || ksh_flush_async(m->ctx)) return 1;
         if (i > 0) {
             if (ksh_wait_inflight_at_most(m->ctx, 1)) return 1;
             const int r = take(i - 1);
@@ -673,16 +793,24 @@ int ksh_gemma4_decode_token_sampled(ksh_gemma4 *m, uint32_t token, float tempera
 }
 
 // GemmaPrimModel::prefill_chunk (gemma_prim.rs:1305-1315): the tokens go through without logits, then one
-// synchronisation.  (Token by token: this build has no batched prefill of the layer stack.)
+// synchronisation.  Chunks of up to 256 tokens go through the batched layer pass (forward_prefill_chunk,
+// gemma_prim.rs:1317-1607), a chunk of one token through the decode step; use_graph & 2 feeds every token through
+// the decode step instead (use_graph & 1: from its captured graph).
 int ksh_gemma4_prefill_chunk(ksh_gemma4 *m, const uint32_t *tokens, int n, int use_graph)
 {
     if (!m || (n > 0 && !tokens) || n < 0) return set_error("ksh_gemma4_prefill_chunk: bad arguments");
     if (m->pos + n > m->c.max_seq) return set_error("max_seq exceeded");
     for (int i = 0; i < n; i++)
         if (tokens[i] >= (uint32_t)m->c.vocab) return set_error("token id %u is outside the vocabulary", tokens[i]);
-    for (int i = 0; i < n; i++) {
-        if (write_token(m, tokens[i])) return 1;
-        if (run_token(m, false, use_graph != 0)) return 1;
+    for (int i = 0; i < n;) {
+        const int t = (use_graph & 2) ? 1 : std::min(kChunk4, n - i);
+        if (t == 1) {
+            if (write_token(m, tokens[i])) return 1;
+            if (run_token(m, false, (use_graph & 1) != 0)) return 1;
+        } else if (forward_prefill_chunk4(m, tokens + i, t)) {
+            return 1;
+        }
+        i += t;
     }
     return ksh_synchronize(m->ctx);
 }

@@ -272,10 +272,13 @@ __global__ void copy_scale_indexed_kernel(const uint8_t *__restrict__ src, const
     out[i] = scale * v;
 }
 
-__global__ void gelu_mul_kernel(const float *__restrict__ g, const float *__restrict__ u, float *out, int n)
+// inner > 0 (gelu_mul_strided, gemma_prim.rs:1566-1576): g and out are [n / inner, inner], row r of u starts at
+// r * stride (one layer's slice of every token's per-layer context)
+__global__ void gelu_mul_kernel(const float *__restrict__ g, const float *__restrict__ u, float *out, int n, int inner, int stride)
 {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
+    if (inner > 0) u += (size_t)(i / inner) * stride - (size_t)(i / inner) * inner;
     // lower.rs:4775-4838, same expression tree as the fused epilogue (:2926-2955)
     const float ax = fminf(20.0f, fmaxf(-20.0f, g[i]));
     const float t = 0.79788456f * (ax + 0.044715f * ((ax * ax) * ax));
@@ -404,7 +407,7 @@ int launch_gelu_mul(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
 {
     const int n = (int)k.desc.dims[0];
     hipLaunchKernelGGL(gelu_mul_kernel, dim3((n + 255) / 256), dim3(256), 0, st, (const float *)a.in[0],
-                       (const float *)a.in[1], (float *)a.out[0], n);
+                       (const float *)a.in[1], (float *)a.out[0], n, (int)k.desc.dims[1], (int)k.desc.dims[2]);
     return done("gelu_mul launch");
 }
 
@@ -591,14 +594,19 @@ int bind_glue(ksh_kernel &k)
         k.launch = launch_copy_scale_indexed;
         return 0;
     }
-    case KSH_GELU_MUL:
+    case KSH_GELU_MUL: {
+        // dims[1] = inner, dims[2] = stride: the second operand's rows of `inner` values are `stride` floats apart
+        const int64_t inner = k.desc.dims[1], stride = k.desc.dims[2];
+        if (inner < 0 || stride < 0 || (inner && (n % inner || stride < inner))) return set_error("gelu_mul: inner=%lld stride=%lld", (long long)inner, (long long)stride);
         k.info.n_inputs = 2;
         k.info.n_outputs = 1;
         k.in_bytes[0] = k.in_bytes[1] = k.out_bytes[0] = (size_t)n * 4;
+        if (inner) k.in_bytes[1] = ((size_t)(n / inner - 1) * stride + inner) * 4;
         k.in_align[0] = k.in_align[1] = k.out_align[0] = 4;
-        set_name(k, "gelu_mul");
+        set_name(k, "gelu_mul%s", inner ? "_strided" : "");
         k.launch = launch_gelu_mul;
         return 0;
+    }
     case KSH_COPY_SLICE:
         k.info.n_inputs = 1;
         k.info.n_outputs = 1;

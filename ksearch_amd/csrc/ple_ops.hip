@@ -29,12 +29,15 @@ int done(const char *what)
 template <int HD>
 __global__ __launch_bounds__(64) void per_head_kernel(const float *x, const float *__restrict__ w,
                                                       const float *__restrict__ rope, const float *__restrict__ meta,
-                                                      float *y, float eps, int max_seq)
+                                                      float *y, float eps, int max_seq, int heads_per_token)
 {
     constexpr int HALF = HD / 2, PER = HD / 64;
     const int lane = threadIdx.x;
     const size_t base = (size_t)blockIdx.x * HD;
-    if (meta) rope += (size_t)min(max((int)meta[3], 0), max_seq - 1) * HD;
+    // heads_per_token > 0 (rmsnorm_per_head_rope_batch, gemma_prim.rs:1411-1424): the heads of a chunk of consecutive
+    // positions, token after token; token i takes the rope row of (first position + i)
+    const int tok = heads_per_token > 0 ? blockIdx.x / heads_per_token : 0;
+    if (meta) rope += (size_t)min(max((int)meta[3] + tok, 0), max_seq - 1) * HD;
     float xv[PER], nv[PER];
     float ss = 0.f;
 #pragma unroll
@@ -182,7 +185,7 @@ int launch_per_head(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
     const float *meta = mode == 2 ? (const float *)a.in[3] : nullptr;
 #define KSH_PH(HD)                                                                                                  \
     hipLaunchKernelGGL((per_head_kernel<HD>), dim3(n_heads), dim3(64), 0, st, (const float *)a.in[0],               \
-                       (const float *)a.in[1], rope, meta, (float *)a.out[0], k.desc.params[0], (int)k.desc.dims[3])
+                       (const float *)a.in[1], rope, meta, (float *)a.out[0], k.desc.params[0], (int)k.desc.dims[3], (int)k.desc.dims[4])
     switch (hd) {
     case 64: KSH_PH(64); break;
     case 128: KSH_PH(128); break;
@@ -229,6 +232,8 @@ int bind_ple_ops(ksh_kernel &k)
             return set_error("rmsnorm_per_head: hd=%lld is not built (64, 128, 256, 512 are)", (long long)hd);
         if (mode < 0 || mode > 2) return set_error("rmsnorm_per_head: dims[2]=%lld (0 norm only, 1 rope row, 2 rope table + meta)", (long long)mode);
         if (mode == 2 && (max_seq <= 0 || max_seq > (1 << 24))) return set_error("rmsnorm_per_head: max_seq=%lld", (long long)max_seq);
+        // dims[4] = heads per token when the heads belong to a chunk of consecutive positions (rope = 2 only)
+        if (d[4] < 0 || (d[4] && (mode != 2 || n_heads % d[4]))) return set_error("rmsnorm_per_head: heads per token %lld", (long long)d[4]);
         k.info.n_inputs = 2 + (int)mode;
         k.info.n_outputs = 1;
         k.in_bytes[0] = k.out_bytes[0] = (size_t)n_heads * hd * 4;

@@ -1125,11 +1125,12 @@ class Gemma4:
                                               C.byref(nxt) if read_next and want_logits else None))
         return nxt.value if read_next and want_logits else None
 
-    def generate(self, prompt, n_new: int, use_graph: bool = True):
+    def generate(self, prompt, n_new: int, use_graph: bool = True, serial_prefill: bool = False):
         p = (C.c_uint32 * len(prompt))(*[int(t) for t in prompt])
         out = (C.c_uint32 * max(1, n_new))()
         pre, dec = C.c_double(), C.c_double()
-        _check(lib().ksh_gemma4_generate(self.h, p, len(prompt), n_new, int(use_graph), out, C.byref(pre), C.byref(dec)))
+        flags = int(bool(use_graph)) | (2 if serial_prefill else 0)
+        _check(lib().ksh_gemma4_generate(self.h, p, len(prompt), n_new, flags, out, C.byref(pre), C.byref(dec)))
         return list(out[:n_new]), pre.value, dec.value
 
     def decode_token_sampled(self, token: int, temperature: float, min_p: float, seed: int, use_graph: bool = False) -> int:
@@ -1139,10 +1140,11 @@ class Gemma4:
                                                      C.byref(nxt)))
         return nxt.value
 
-    def prefill_chunk(self, tokens, use_graph: bool = False):
-        """GemmaPrimModel::prefill_chunk (gemma_prim.rs:1305-1315), token by token."""
+    def prefill_chunk(self, tokens, use_graph: bool = False, serial: bool = False):
+        """GemmaPrimModel::prefill_chunk (gemma_prim.rs:1305-1315): chunks of up to 256 tokens as one batched pass
+        per layer; `serial` feeds every token through the decode step instead."""
         t = (C.c_uint32 * max(1, len(tokens)))(*[int(x) for x in tokens])
-        _check(lib().ksh_gemma4_prefill_chunk(self.h, t, len(tokens), int(use_graph)))
+        _check(lib().ksh_gemma4_prefill_chunk(self.h, t, len(tokens), int(bool(use_graph)) | (2 if serial else 0)))
 
     def bind_slot(self, pool, slot: int):
         """GemmaPrimModel::bind_slot; pool=None goes back to the model's own caches at position `slot`."""

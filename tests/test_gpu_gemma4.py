@@ -199,6 +199,63 @@ def test_gemma4_forward_token_matches_oracle_teacher_forced(tiny):
         gpu.forward_token(cfg["vocab"])
 
 
+def prefilled_in_lockstep(gpu, cpu, cfg, pattern, toks, then=4, tol=1e-3):
+    """prefill_chunk(toks) as batched chunks, then the oracle walks the same positions adopting the rows the chunk
+    left (one code step at most from its own), then `then` decode steps with logits compared."""
+    ctx, n = gpu.ctx, cfg["n_layers"]
+    owners = [l for l in range(n) if gpu.kv_source(l) == l]
+    hd = {l: cfg["hd_swa"] if pattern[l] else cfg["hd_full"] for l in owners}
+    stride = max(cfg["n_kv"] * h // 32 * 18 for h in hd.values())
+    n_pre = len(toks) - then
+    gpu.reset()
+    cpu.reset()
+    gpu.prefill_chunk(toks[:n_pre])
+    assert gpu.pos == n_pre
+    cache = {l: [gpu.kv(l, w, n_pre * (cfg["n_kv"] * hd[l] // 32 * 18)) for w in (0, 1)] for l in owners}
+    flipped = 0
+    for i in range(n_pre):
+        rows = np.zeros((n, 2, stride), np.uint8)
+        for l in owners:
+            row = cfg["n_kv"] * hd[l] // 32 * 18
+            for w in (0, 1):
+                rows[l, w, :row] = cache[l][w][i * row:(i + 1) * row]
+        cpu.forward(int(toks[i]), want_logits=False, adopt_rows=rows)
+        assert cpu.row_max_step.max() <= 1.0 + 1e-3, (i, cpu.row_max_step.max(1))
+        flipped += int(cpu.row_diff_bytes.sum())
+    assert flipped <= 0.02 * n_pre * len(owners) * 2 * stride, flipped
+    bufs = {l: [hip.Buffer(ctx, hip.lib().ksh_gemma4_kv(gpu.h, l, w), owned=False) for w in (0, 1)] for l in owners}
+    for i in range(n_pre, len(toks)):
+        g_next = gpu.forward_token(int(toks[i]), use_graph=bool(i & 1))
+        rows = np.zeros((n, 2, stride), np.uint8)
+        for l in owners:
+            row = cfg["n_kv"] * hd[l] // 32 * 18
+            for w in (0, 1):
+                rows[l, w, :row] = ctx.read_bytes(bufs[l][w], row, i * row)
+        c_next, c_logits = cpu.forward(int(toks[i]), return_logits=True, adopt_rows=rows)
+        assert cpu.row_max_step.max() <= 1.0 + 1e-3
+        assert_close(gpu.logits(), c_logits, tol, f"logits at position {i}")
+        top2 = np.sort(c_logits)[-2:]
+        if top2[1] - top2[0] > 2 * tol * max(abs(top2[1]), float(np.sqrt(np.mean(c_logits ** 2)))):
+            assert g_next == c_next
+
+
+@pytest.mark.parametrize("n_pre", [2, 7, 20, 37])
+def test_gemma4_prefill_chunk_batched(tiny, n_pre):
+    """The batched layer pass over a prompt chunk (both layer kinds, a window of 8 that the chunk outgrows, layers
+    reading earlier caches, per-layer embeddings, Q4_K and Q6_K tensors): the KV rows of the serial run up to
+    one-code flips, and the oracle's logits on the decode steps behind it."""
+    gpu, cpu, cfg = tiny
+    toks = np.random.default_rng(640 + n_pre).integers(0, cfg["vocab"], n_pre + 4)
+    prefilled_in_lockstep(gpu, cpu, cfg, PATTERN, toks)
+    # the same prompt through the decode step leaves the same position and (up to flips) the same cache
+    batched = {l: gpu.kv(l, 0, 64) for l in range(cfg["n_layers"]) if gpu.kv_source(l) == l}
+    gpu.reset()
+    gpu.prefill_chunk(toks[:n_pre], serial=True)
+    assert gpu.pos == n_pre
+    for l, b in batched.items():
+        assert (gpu.kv(l, 0, 64) != b).mean() <= 0.1
+
+
 def test_gemma4_generate_graph_equals_eager_and_oracle(tiny):
     gpu, cpu, cfg = tiny
     prompt = [int(t) for t in np.random.default_rng(612).integers(0, cfg["vocab"], 6)]
@@ -345,15 +402,10 @@ def test_gemma4_from_gguf_matches_oracle(ctx, tmp_path):
         hip.Gemma4.from_gguf(ctx, f, cfg["max_seq"])
 
 
-def test_gemma4_real_widths_long_run_matches_oracle(ctx, eng):
+def real_widths_models(ctx, eng):
     """The real checkpoints' widths (hidden 1536, head dims 256 / 512, window 512, double-wide feed-forward on the
-    layers that reuse a cache, unscaled attention) on a shortened stack, teacher-forced past the window through
-    the captured graph, against the oracle on the very same packed bytes (quantized on the device, read back for
-    the CPU).  Logits are compared where the run changes regime: the first positions, the oracle's switch to
-    split-KV attention at 128 rows, the window's edge at 512.  The bar is 5e-3 on whole-model logits here: with
-    unscaled scores over hundreds of rows of random weights the softmax is close to one-hot, and an f32
-    reassociation difference in a score moves the output by more than it does at the tiny model's 24 rows (1e-3
-    there; the single ops stay at 1e-3 in their own tests)."""
+    layers that reuse a cache, unscaled attention) on a shortened stack; the oracle on the very same packed bytes
+    (quantized on the device, read back for the CPU)."""
     n, shared = 9, 4
     cfg = dict(n_layers=n, hidden=1536, n_q=8, n_kv=1, vocab=8192, max_seq=576, hd_swa=256, hd_full=512, sliding_window=512,
                shared_kv_layers=shared, ple_dim=256, eps=1e-6, softcap=30.0, rope_theta_swa=1e4, rope_theta_full=1e6,
@@ -369,6 +421,29 @@ def test_gemma4_real_widths_long_run_matches_oracle(ctx, eng):
     w = dict(layers=[{k: host(v) for k, v in lw.items()} for lw in dev["layers"]], globals={k: host(v) for k, v in dev["globals"].items()})
     gpu, cpu = hip.Gemma4(ctx, cfg, dev), oracle.Gemma4(cfg, w)
     assert [gpu.kv_source(l) for l in range(n)] == [0, 1, 2, 3, 4, 4, 4, 2, 4]
+    return gpu, cpu, cfg, pattern
+
+
+def test_gemma4_real_widths_batched_prefill(ctx, eng):
+    """300 prompt tokens at the real widths as a chunk of 256 and one of 44 (512-wide heads, 12288-wide feed-forward,
+    1536-column GEMMs, the per-layer table), then decode steps against the oracle (bar 5e-3, as for the long run)."""
+    gpu, cpu, cfg, pattern = real_widths_models(ctx, eng)
+    toks = np.random.default_rng(632).integers(0, cfg["vocab"], 304)
+    prefilled_in_lockstep(gpu, cpu, cfg, pattern, toks, then=4, tol=5e-3)
+    gpu.close()
+    cpu.close()
+
+
+def test_gemma4_real_widths_long_run_matches_oracle(ctx, eng):
+    """The real checkpoints' widths (hidden 1536, head dims 256 / 512, window 512, double-wide feed-forward on the
+    layers that reuse a cache, unscaled attention) on a shortened stack, teacher-forced past the window through
+    the captured graph, against the oracle on the very same packed bytes (quantized on the device, read back for
+    the CPU).  Logits are compared where the run changes regime: the first positions, the oracle's switch to
+    split-KV attention at 128 rows, the window's edge at 512.  The bar is 5e-3 on whole-model logits here: with
+    unscaled scores over hundreds of rows of random weights the softmax is close to one-hot, and an f32
+    reassociation difference in a score moves the output by more than it does at the tiny model's 24 rows (1e-3
+    there; the single ops stay at 1e-3 in their own tests)."""
+    gpu, cpu, cfg, pattern = real_widths_models(ctx, eng)
     toks = np.random.default_rng(631).integers(0, cfg["vocab"], 540)
     check = set(range(12)) | set(range(124, 134)) | set(range(506, 520)) | {300, 539}
     clean, agree = teacher_forced(gpu, cpu, cfg, pattern, toks, check=check, use_graph=True, tol=5e-3)

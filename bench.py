@@ -178,7 +178,7 @@ def bench_prefill(ctx):
     return out
 
 
-def bench_attention(ctx, ev, copies=16):
+def bench_attention(ctx, ev, copies=16, sched=None):
     """cfg3: 4 slots, 8 q / 1 kv heads of 256, Q4_0 KV, lengths ~U{1024..16384}, one launch pair.  Timed twice: with
     the 7 MB of rows resident in cache between launches, and cold, cycling through `copies` copies of the K / V
     pools (16 x 18.9 MB = 302 MB, more than the 256 MB last-level cache) inside one HIP graph."""
@@ -189,7 +189,7 @@ def bench_attention(ctx, ev, copies=16):
     meta = np.zeros((n_slots, 4), dtype=np.float32)
     meta[:, 0] = lens
     k = ctx.compile(hip.make_desc(hip.Kind.SDPA_SLOTS, (n_q, n_kv, hd, max_t, n_slots, 0),
-                                  (hip.DType.Q40, hip.DType.F32), (1.0 / 16.0,)))
+                                  (hip.DType.Q40, hip.DType.F32), (1.0 / 16.0,), sched))
     nwg = k.info.sched.k_split
     ins = [ctx.buffer_f32(q), ctx.buffer_bytes(kk), ctx.buffer_bytes(vv), ctx.buffer_f32(meta)]
     outs = [ctx.buffer_empty_f32(n_slots * n_q * nwg * (hd + 2)), ctx.buffer_empty_f32(n_slots * n_q * hd)]

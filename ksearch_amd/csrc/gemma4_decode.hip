@@ -125,6 +125,7 @@ struct ksh_gemma4 {
     std::vector<ksh_buf *> own_k, own_v;
     struct SlotGraphs { ksh_graph *body = nullptr, *full = nullptr; };
     ksh_kvpool *pool = nullptr;
+    uint64_t pool_uid = 0;   // (a new pool can be allocated where a destroyed one lay: the address alone does not identify it)
     std::vector<SlotGraphs> slot_graphs;
     SlotGraphs own_graphs;
     int bound_slot = -1;
@@ -836,9 +837,10 @@ int ksh_gemma4_bind_slot(ksh_gemma4 *m, ksh_kvpool *pool, int slot)
     if (pos < 0 || pos > c.max_seq) return set_error("ksh_gemma4_bind_slot: position %d", pos);
     // the slot it is bound to already, at the position the model has reached by itself: the device-side state is
     // in place (a scheduler with one decoding request asks for this before every token)
-    if (pool && pool == m->pool && slot == m->bound_slot && pos == m->pos) return 0;
+    const bool same_pool = pool && pool == m->pool && ksh_kvpool_uid(pool) == m->pool_uid;
+    if (same_pool && slot == m->bound_slot && pos == m->pos) return 0;
     stash_graphs(m);
-    if (pool && pool != m->pool) {
+    if (pool && !same_pool) {
         // graphs captured over another pool's buffers are of no use any more
         if (ksh_synchronize(m->ctx)) return 1;
         for (auto &g : m->slot_graphs) { ksh_graph_destroy(g.body); ksh_graph_destroy(g.full); }
@@ -846,6 +848,7 @@ int ksh_gemma4_bind_slot(ksh_gemma4 *m, ksh_kvpool *pool, int slot)
         ksh_kvpool_dims(pool, &max_batch, nullptr, nullptr, nullptr, nullptr);
         m->slot_graphs.assign((size_t)max_batch, ksh_gemma4::SlotGraphs{});
         m->pool = pool;
+        m->pool_uid = ksh_kvpool_uid(pool);
     }
     if (m->own_k.empty()) { m->own_k = m->kv_k; m->own_v = m->kv_v; }
     for (int l = 0; l < owners; l++) {

@@ -66,6 +66,10 @@ void ctx_mark_pending(ksh_ctx *ctx);
 int argmax_static_setup();
 }  // namespace ksh
 
+// a pool's identity for whoever caches things per pool (HIP graphs captured over its buffers): unlike its address,
+// never handed out twice
+extern "C" uint64_t ksh_kvpool_uid(const ksh_kvpool *p);
+
 // hands a buffer's reference over to a model, which releases it when it is destroyed (the GGUF loader's uploads)
 extern "C" void ksh_gemma4_adopt(ksh_gemma4 *m, ksh_buf *b);
 

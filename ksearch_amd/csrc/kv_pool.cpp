@@ -13,6 +13,7 @@
 
 struct ksh_kvpool {
     ksh_ctx *ctx = nullptr;
+    uint64_t uid = 0;   // never reused: a pool created where a destroyed one lay is still another pool
     int max_batch = 0, max_seq = 0, n_kv_layers = 0, hd = 0, n_kv = 0;
     std::vector<char> occupied;
     std::vector<int> seq_len;
@@ -39,6 +40,8 @@ int ksh_kvpool_create(ksh_ctx *ctx, int max_batch, int max_seq, int n_kv_layers,
     if (max_batch <= 0 || max_seq <= 0 || n_kv_layers <= 0 || hd <= 0 || n_kv <= 0) return set_error("KvPool dims must be non-zero");
     if (hd % 32) return set_error("KvPool: hd=%d is not a multiple of the Q4_0 block (32)", hd);
     auto p = std::make_unique<ksh_kvpool>();
+    static std::atomic<uint64_t> next_uid{1};
+    p->uid = next_uid.fetch_add(1);
     p->ctx = ctx;
     p->max_batch = max_batch; p->max_seq = max_seq; p->n_kv_layers = n_kv_layers; p->hd = hd; p->n_kv = n_kv;
     p->occupied.assign((size_t)max_batch, 0);
@@ -54,6 +57,8 @@ int ksh_kvpool_create(ksh_ctx *ctx, int max_batch, int max_seq, int n_kv_layers,
     *out = p.release();
     return 0;
 }
+
+uint64_t ksh_kvpool_uid(const ksh_kvpool *p) { return p ? p->uid : 0; }
 
 void ksh_kvpool_destroy(ksh_kvpool *p)
 {

@@ -48,9 +48,15 @@ static int sdpa_candidates(const ksh_kernel_desc &d, ksh_sched *out, int cap)
                 if (hs > groups || groups % hs) continue;
                 if (n >= cap) return n;
                 ksh_sched s{};
-                s.tg = 64ull * nsg; s.vec = 0; s.unroll = attend ? hs : 0; s.nsg = nsg; s.nr0 = 0; s.k_split = ks;
+                s.tg = 64ull * nsg; s.vec = 3; s.unroll = attend ? hs : 0; s.nsg = nsg; s.nr0 = 0; s.k_split = ks;   // vector-ALU form
                 out[n++] = s;
             }
+        // the matrix-core form of the row phase (several slots, heads of 256)
+        if (d.kind == KSH_SDPA_SLOTS && d.dims[2] == 256 && groups <= 8 && d.dims[4] <= 16 && n < cap) {
+            ksh_sched s{};
+            s.tg = 256; s.vec = 2; s.unroll = 1; s.nsg = 4; s.k_split = ks; s.lds_tile = 32;
+            out[n++] = s;
+        }
     }
     return n;
 }

@@ -457,7 +457,7 @@ int bind_sdpa(ksh_kernel &k)
         if (bind_sdpa_lanes(k, lanes_nwg, lanes_slots)) return 1;
         char name[64];
         snprintf(name, sizeof(name), "%s", k.info.name);
-        set_name(k, "%s_regs_w%d", name, (int)k.info.sched.nsg);
+        set_name(k, k.info.sched.vec == 2 ? "%s_mfma_w%d" : "%s_regs_w%d", name, (int)k.info.sched.nsg);
     }
     return 0;
 }

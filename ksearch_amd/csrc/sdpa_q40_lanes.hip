@@ -279,12 +279,14 @@ __device__ __forceinline__ void norm_rope_regs(const float (&xv)[HD / 64], const
 // least one), with c = ceil(T / (P - n_slots)) rows, so that they sum to at most P; what is left over exits.
 // Every workgroup derives the same table from the slots' lengths.  Slot s's partitions are the consecutive
 // flat indices from the sum of its predecessors' counts, and its records sit in that order.
-__device__ __forceinline__ int dealt_rows(const float *meta, int stride, int n_slots, int nwg)
+// round > 1: the rows per partition are rounded up to a multiple of it (the matrix-core form works in tiles of rows).
+__device__ __forceinline__ int dealt_rows(const float *meta, int stride, int n_slots, int nwg, int round = 1)
 {
     int T = 0;
     for (int s = 0; s < n_slots; s++) T += (int)meta[(size_t)s * stride];
-    const int spare = nwg * n_slots - n_slots;   // host-checked: nwg >= 2
-    return max(1, (T + spare - 1) / spare);
+    const int spare = max(1, nwg * n_slots - n_slots);   // host-checked: nwg >= 2
+    const int c = max(1, (T + spare - 1) / spare);
+    return (c + round - 1) / round * round;
 }
 __device__ __forceinline__ int dealt_parts(const float *meta, int stride, int s, int c)
 {
@@ -299,7 +301,7 @@ __device__ __forceinline__ int dealt_parts(const float *meta, int stride, int s,
 // Records of a balanced launch: values [flat][n_q][HD], then (m, l) [flat][n_q][2].
 template <int HD>
 __global__ __launch_bounds__(256) void sdpa_dealt_merge_kernel(const float *tmp, const float *meta, int meta_stride, int nwg,
-                                                                int n_q, float *out)
+                                                                int n_q, float *out, int round)
 {
     constexpr int kMaxParts = 16 * 64;   // host-checked: nwg * n_slots
     constexpr int QB = 8;                // partitions per thread in flight
@@ -308,7 +310,7 @@ __global__ __launch_bounds__(256) void sdpa_dealt_merge_kernel(const float *tmp,
     __shared__ __attribute__((aligned(16))) float part4[16][64];
     const int head = blockIdx.x / (HD / 64), dq = blockIdx.x % (HD / 64), slot = blockIdx.y, S = gridDim.y;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = tid >> 4, j = tid & 15;
-    const int c = dealt_rows(meta, meta_stride, S, nwg);
+    const int c = dealt_rows(meta, meta_stride, S, nwg, round);
     int first = 0;
     for (int s = 0; s < slot; s++) first += dealt_parts(meta, meta_stride, s, c);
     const int n = dealt_parts(meta, meta_stride, slot, c);
@@ -756,6 +758,361 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
     if (tid == 0) __hip_atomic_store(&p.counters[slot * gridDim.y + blockIdx.y], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next launch
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// Matrix-core form of the row phase (split-KV partials), for head size 256 and up to 8 q heads per kv head.
+//
+// The vector-ALU form above spends ~200 instructions per KV row and wave (8 FMAs per head and dword for the scores,
+// as many for P.V, the butterflies between them).  Here both products run on v_mfma_f32_16x16x32_f16 with exact
+// operands and the vector ALU only converts and scales:
+//   - a wave takes tiles of 32 rows.  The tile's K and V bytes are copied to the wave's LDS strip with whole 128-bit
+//     loads (a row is 9 of them), and its 2 x 256 block scales are converted once into two f32 tables.
+//   - scores: per 16 rows and Q4_0 block b, A = the block's codes as f16 (16 + n: the nibble ORed into the mantissa
+//     of 16.0, two ops per pair), B = the 8 heads' q of that block as f16 hi parts in columns 0..7 and lo parts in
+//     columns 8..15 (22 bits of q; fixed for the whole launch).  The 16 x 16 result is exact up to f32 summation;
+//     S += d[row, b] * (C - 24 * sum_b(q)) applies the block scale and takes the 16 + 8 offset out again.
+//   - softmax bookkeeping on the accumulator layout (a lane holds 8 rows of one column); hi and lo columns are
+//     added across lanes, the running maximum is shared across the wave.
+//   - P.V: A = P' = p * dv[row, b] per block b, again split hi | lo over the 16 output rows, which needs no data
+//     movement because the accumulator layout of the scores is the A-operand layout of this product when k runs
+//     over a lane's own rows; B = the V codes of 8 rows and one element per lane, gathered bytewise from the LDS
+//     strip (the one transposition of the kernel).  A third product against ones keeps sum(P') per block for the
+//     code offset.
+// A workgroup folds its waves' states through LDS and writes one partial record per head, in the layout of the
+// vector-ALU form, so the same merge kernels follow.
+typedef _Float16 h8v __attribute__((ext_vector_type(8)));
+typedef float f4v __attribute__((ext_vector_type(4)));
+constexpr int kMfmaWaves = 4, kMfmaTile = 32, kMfmaRound = kMfmaWaves * kMfmaTile;
+
+__device__ __forceinline__ float xor16_max(float x)
+{
+    const auto r = __builtin_amdgcn_permlane16_swap(as_u32(x), as_u32(x), false, false);
+    return fmaxf(as_f32(r[0]), as_f32(r[1]));
+}
+__device__ __forceinline__ float xor32_max(float x)
+{
+    const auto r = __builtin_amdgcn_permlane32_swap(as_u32(x), as_u32(x), false, false);
+    return fmaxf(as_f32(r[0]), as_f32(r[1]));
+}
+
+// 8 nibbles of a dword as f16 (16 + n), in the order (n0, n4), (n1, n5), (n2, n6), (n3, n7)
+__device__ __forceinline__ h8v nibbles_f16(uint32_t d)
+{
+    constexpr uint32_t M = 0x03C003C0u, G = 0x4C004C00u;
+    const u32x4_t o = {((d << 6) & M) | G, ((d << 2) & M) | G, ((d >> 2) & M) | G, ((d >> 6) & M) | G};
+    return __builtin_bit_cast(h8v, o);
+}
+
+// the element of a 32-wide Q4_0 block that slot s of lane group kq holds in the score products (see nibbles_f16:
+// byte i of the lane's dword carries elements 4kq + i (low nibble) and 16 + 4kq + i (high nibble))
+__device__ __forceinline__ int mfma_k_elem(int s, int kq)
+{
+    const int byte = ((s >> 2) & 1) + 2 * (s & 1);   // s: 0 1 2 3 4 5 6 7 -> byte 0 2 0 2 1 3 1 3
+    return 4 * kq + byte + ((s >> 1) & 1) * 16;      //    nibble: lo lo hi hi lo lo hi hi
+}
+
+template <int HD>
+__global__ __launch_bounds__(kMfmaWaves * 64, 2) void sdpa_mfma_kernel(LaneParams p)
+{
+    constexpr int NW = kMfmaWaves, NT = NW * 64, NB = HD / 32, ROWB = NB * 18, TR = kMfmaTile, TILEB = TR * ROWB;
+    constexpr int STRIP = 2 * TILEB + 2 * TR * NB * 4;           // K bytes, V bytes, K scales, V scales
+    constexpr int PIECES = TR * ROWB / 16;                       // 128-bit pieces of a tile
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int col = lane & 15, q4 = lane >> 4, head = col & 7, is_lo = col >> 3;
+    uint8_t *strip = lds_raw + (size_t)wave * STRIP;
+    uint8_t *kraw = strip, *vraw = strip + TILEB;
+    float *ksc = reinterpret_cast<float *>(strip + 2 * TILEB), *vsc = ksc + TR * NB;
+
+    int part = blockIdx.x, slot = blockIdx.z, nparts = p.nwg;
+    const int kvh = blockIdx.y, groups = p.groups, head0 = kvh * groups;
+    size_t rec_base = 0;
+    int p0, p1, start;
+    if (p.balance) {
+        const int S = gridDim.z, f = blockIdx.z * p.nwg + blockIdx.x;
+        const int c = dealt_rows(p.meta, p.meta_stride, S, p.nwg, kMfmaRound);
+        int first = 0;
+        slot = -1;
+        for (int s = 0; s < S; s++) {
+            const int n = dealt_parts(p.meta, p.meta_stride, s, c);
+            if (f < first + n) { slot = s; part = f - first; nparts = n; break; }
+            first += n;
+        }
+        if (slot < 0) return;   // left over
+        rec_base = (size_t)first + part;
+        const int tlen = (int)p.meta[(size_t)slot * p.meta_stride];
+        p0 = part * c;
+        p1 = min(p0 + c, tlen);
+    } else {
+        const int tlen = (int)p.meta[(size_t)slot * p.meta_stride];
+        const int chunk = ((tlen + nparts - 1) / nparts + TR - 1) / TR * TR;
+        p0 = min(part * chunk, tlen);
+        p1 = min(p0 + chunk, tlen);
+    }
+    start = (int)p.meta[(size_t)slot * p.meta_stride + 1];
+    const size_t slot_bytes = p.kv_shared ? 0 : (size_t)p.max_t * p.n_kv * ROWB;
+    const size_t row_stride = (size_t)p.n_kv * ROWB;
+    const uint8_t *kbase = p.k + (size_t)slot * slot_bytes + (size_t)kvh * ROWB;
+    const uint8_t *vbase = p.v + (size_t)slot * slot_bytes + (size_t)kvh * ROWB;
+
+    // ---- the first tile's bytes are requested before anything else (they have the longest way to come)
+    constexpr int NPC = (PIECES + 63) / 64;
+    u32x4_t kpre[NPC], vpre[NPC];
+    auto fetch_tile = [&](int it) __attribute__((always_inline)) {
+        const int row0 = p0 + (it * NW + wave) * TR;
+        const int nvalid = max(0, min(TR, p1 - row0));
+#pragma unroll
+        for (int u = 0; u < NPC; u++) {
+            const int idx = lane + 64 * u, row = idx / (ROWB / 16), pc = idx % (ROWB / 16);
+            kpre[u] = u32x4_t{0u, 0u, 0u, 0u};
+            vpre[u] = u32x4_t{0u, 0u, 0u, 0u};
+            if (idx < PIECES && row < nvalid) {
+                const size_t off = (size_t)(start + row0 + row) * row_stride + (size_t)pc * 16;
+                kpre[u] = *reinterpret_cast<const u32x4_t *>(kbase + off);
+                vpre[u] = *reinterpret_cast<const u32x4_t *>(vbase + off);
+            }
+        }
+    };
+    fetch_tile(0);
+
+    // ---- q: the B operands of the score products and 24 * sum_b(q), fixed for the launch.  Wave w prepares blocks
+    // w, w + NW, ... and the workgroup shares them through LDS (behind the strips).
+    h8v qop[NB];
+    float qs24[NB];
+    {
+        h8v *qshare = reinterpret_cast<h8v *>(lds_raw + (size_t)NW * STRIP);       // [NB][64] operands
+        float *qsum_share = reinterpret_cast<float *>(qshare + NB * 64);            // [NB][64]
+        const float *qh = p.q + ((size_t)slot * p.n_q + head0 + min(head, groups - 1)) * HD;
+        const bool have = head < groups;
+        for (int b = wave; b < NB; b += NW) {
+            const float4 lo4 = *reinterpret_cast<const float4 *>(qh + 32 * b + 4 * q4);        // elements 4kq .. 4kq+3
+            const float4 hi4 = *reinterpret_cast<const float4 *>(qh + 32 * b + 16 + 4 * q4);   // 16+4kq .. 16+4kq+3
+            const float x[8] = {lo4.x, lo4.z, hi4.x, hi4.z, lo4.y, lo4.w, hi4.y, hi4.w};       // slot order (mfma_k_elem)
+            h8v op;
+            float sum = 0.f;
+#pragma unroll
+            for (int s2 = 0; s2 < 8; s2++) {
+                const float xs = have ? x[s2] * p.scale : 0.f;
+                const _Float16 hi = (_Float16)xs;
+                const _Float16 lo = (_Float16)(xs - (float)hi);
+                const _Float16 v = is_lo ? lo : hi;
+                op[s2] = v;
+                sum += (float)v;
+            }
+            sum = xor32_sum(xor16_sum(sum));      // the column's four lane groups hold the block's 32 elements
+            qshare[b * 64 + lane] = op;
+            qsum_share[b * 64 + lane] = 24.f * sum;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            qop[b] = qshare[b * 64 + lane];
+            qs24[b] = qsum_share[b * 64 + lane];
+        }
+    }
+
+    f4v O[2 * NB];
+    float Tl[NB];
+#pragma unroll
+    for (int c = 0; c < 2 * NB; c++) O[c] = f4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int b = 0; b < NB; b++) Tl[b] = 0.f;
+    float m_run = -1.0e30f, l_run = 0.f;
+
+    const int ntiles = (p1 - p0 + TR - 1) / TR;
+    const int nsteps = (ntiles + NW - 1) / NW;               // the same for every wave: the barriers below are uniform
+    for (int it = 0; it < nsteps; it++) {
+        const int row0 = p0 + (it * NW + wave) * TR;
+        const int nvalid = max(0, min(TR, p1 - row0));         // wave-uniform
+        // The strip belongs to this wave alone, and a wave's LDS operations complete in the order they were issued:
+        // no workgroup barrier in this loop, only fences that keep the compiler from moving accesses across them.
+        // (Later tiles are requested here, not a tile ahead: forty registers less make room for a second wave per
+        // SIMD, which covers the wait better than the look-ahead did.)
+        if (it > 0) fetch_tile(it);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+#pragma unroll
+        for (int u = 0; u < NPC; u++) {
+            const int idx = lane + 64 * u;
+            if (idx < PIECES) {
+                *reinterpret_cast<u32x4_t *>(kraw + idx * 16) = kpre[u];
+                *reinterpret_cast<u32x4_t *>(vraw + idx * 16) = vpre[u];
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        // ---- block scales as f32 tables [row][block]; rows past the end get 0 (their codes are zeros too)
+#pragma unroll
+        for (int u = 0; u < TR * NB / 64; u++) {
+            const int idx = lane + 64 * u, b = idx / TR, row = idx % TR;      // tables are [block][row]
+            const uint32_t kb = *reinterpret_cast<const uint16_t *>(kraw + row * ROWB + 18 * b);
+            const uint32_t vb = *reinterpret_cast<const uint16_t *>(vraw + row * ROWB + 18 * b);
+            ksc[idx] = row < nvalid ? half_bits_to_f32(kb) : 0.f;
+            vsc[idx] = row < nvalid ? half_bits_to_f32(vb) : 0.f;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        if (nvalid > 0) {
+            // ---- scores of the tile's two 16-row halves: lane (col, q4) ends up with rows 4*q4 + r of each
+            float sv[8];
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+                float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int b = 0; b < NB; b++) {
+                    const float4 dk4 = *reinterpret_cast<const float4 *>(ksc + b * TR + 16 * t + 4 * q4);   // rows 4*q4 .. +3
+                    const float dk[4] = {dk4.x, dk4.y, dk4.z, dk4.w};
+                    // A operand: row (16t + lane % 16), bytes 4*q4 .. 4*q4+3 of block b (2-byte aligned)
+                    const uint8_t *src = kraw + (16 * t + col) * ROWB + 18 * b + 2 + 4 * q4;
+                    const uint32_t d = (uint32_t)*reinterpret_cast<const uint16_t *>(src) |
+                                       ((uint32_t)*reinterpret_cast<const uint16_t *>(src + 2) << 16);
+                    const f4v c = __builtin_amdgcn_mfma_f32_16x16x32_f16(nibbles_f16(d), qop[b], f4v{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+#pragma unroll
+                    for (int r = 0; r < 4; r++) acc[r] = fmaf(dk[r], c[r] - qs24[b], acc[r]);
+                }
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const float tot = acc[r] + dpp_f32<0x128>(acc[r]);        // hi + lo column (row_ror:8)
+                    sv[4 * t + r] = (16 * t + 4 * q4 + r) < nvalid ? tot : -1.0e30f;
+                }
+            }
+            // ---- online softmax over the tile (per column; the maximum across the wave's four lane groups)
+            float mt = sv[0];
+#pragma unroll
+            for (int i = 1; i < 8; i++) mt = fmaxf(mt, sv[i]);
+            mt = xor32_max(xor16_max(mt));
+            const float m_new = fmaxf(m_run, mt);
+            const float alpha = __expf(m_run - m_new);
+            float pr[8], ls = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const int row = 16 * (i >> 2) + 4 * q4 + (i & 3);
+                pr[i] = row < nvalid ? __expf(sv[i] - m_new) : 0.f;
+                ls += pr[i];
+            }
+            l_run = fmaf(l_run, alpha, ls);
+            m_run = m_new;
+            // the accumulators of P.V hold output rows 4*q4 + r = columns of the scores: heads 4*(q4 & 1) + r
+            float ah[8];
+#pragma unroll
+            for (int h = 0; h < 8; h++) ah[h] = as_f32((uint32_t)__builtin_amdgcn_readlane((int)as_u32(alpha), h));
+            bool rescale = false;
+#pragma unroll
+            for (int h = 0; h < 8; h++) rescale = rescale || ah[h] != 1.0f;
+            if (rescale) {
+                float ar[4];
+#pragma unroll
+                for (int r = 0; r < 4; r++) ar[r] = (q4 & 1) ? ah[4 + r] : ah[r];
+#pragma unroll
+                for (int c = 0; c < 2 * NB; c++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) O[c][r] *= ar[r];
+            }
+#pragma unroll
+            for (int b = 0; b < NB; b++) Tl[b] *= alpha;       // (a lane's own column: its own factor)
+            // ---- P.V per block: P' = p * dv (hi | lo), V codes gathered bytewise: slot s of the lane <-> row
+            // 16*(s/4) + 4*q4 + s%4, the rows its own scores belong to
+#pragma unroll
+            for (int b = 0; b < NB; b++) {
+                h8v pa;
+                uint32_t vlo[4], vhi[4];
+                const float4 d0 = *reinterpret_cast<const float4 *>(vsc + b * TR + 4 * q4);        // rows 4*q4 .. +3
+                const float4 d1 = *reinterpret_cast<const float4 *>(vsc + b * TR + 16 + 4 * q4);   // rows 16 + 4*q4 .. +3
+                const float dv[8] = {d0.x, d0.y, d0.z, d0.w, d1.x, d1.y, d1.z, d1.w};
+                float tsum = 0.f;
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    const float x = pr[i] * dv[i];
+                    const _Float16 hi = (_Float16)x;
+                    const _Float16 lo = (_Float16)(x - (float)hi);
+                    pa[i] = is_lo ? lo : hi;
+                    tsum += x;
+                }
+                Tl[b] += tsum;                                  // sum(P') of the lane's own rows and column, for the code offset
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int ra = 16 * ((2 * i) >> 2) + 4 * q4 + ((2 * i) & 3), rb = ra + 1;
+                    const uint32_t t2 = (uint32_t)vraw[ra * ROWB + 18 * b + 2 + col] | ((uint32_t)vraw[rb * ROWB + 18 * b + 2 + col] << 16);
+                    vlo[i] = ((t2 << 6) & 0x03C003C0u) | 0x4C004C00u;
+                    vhi[i] = ((t2 << 2) & 0x03C003C0u) | 0x4C004C00u;
+                }
+                const u32x4_t lo4 = {vlo[0], vlo[1], vlo[2], vlo[3]}, hi4 = {vhi[0], vhi[1], vhi[2], vhi[3]};
+                O[2 * b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, __builtin_bit_cast(h8v, lo4), O[2 * b], 0, 0, 0);
+                O[2 * b + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, __builtin_bit_cast(h8v, hi4), O[2 * b + 1], 0, 0, 0);
+            }
+        }
+    }
+
+    // ---- fold: every wave's state to LDS (hi rows first, lo rows added), then one record per head
+    __syncthreads();
+    float *ow = reinterpret_cast<float *>(lds_raw);            // [NW][8][HD]
+    float *mlw = ow + NW * 8 * HD;                             // [NW][8][2]
+    float *tw = mlw + NW * 8 * 2;                              // [NW][8 heads][NB]: 24 * sum(P') per head and block
+    const float l_tot = xor32_sum(xor16_sum(l_run));
+    {
+        // the lanes of a column (four lane groups) and its hi / lo twin (their P' were the two parts of one value)
+        // together hold sum(P'): to a table the accumulator layout can be read from
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            const float tcol = xor32_sum(xor16_sum(Tl[b]));
+            if (lane < 8) tw[((size_t)wave * 8 + lane) * NB + b] = 24.f * tcol;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    }
+    {
+        // hi rows are stored, lo rows added on top: the same wave's LDS operations, in order
+        float *dst[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) dst[r] = ow + ((size_t)wave * 8 + 4 * (q4 & 1) + r) * HD + col;
+        // (the offset 24 * sum(P') of the whole value -- hi and lo part -- is taken off the hi rows)
+        if (q4 < 2) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const float *t24 = tw + ((size_t)wave * 8 + 4 * (q4 & 1) + r) * NB;
+#pragma unroll
+                for (int c = 0; c < 2 * NB; c++) dst[r][16 * c] = O[c][r] - t24[c >> 1];
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        if (q4 >= 2) {
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+#pragma unroll
+                for (int c = 0; c < 2 * NB; c++) dst[r][16 * c] += O[c][r];
+        }
+    }
+    if (lane < 8) { mlw[(wave * 8 + lane) * 2] = m_run; mlw[(wave * 8 + lane) * 2 + 1] = l_tot; }
+    __syncthreads();
+    for (int o = tid; o < groups * HD; o += NT) {
+        const int h = o / HD, d = o % HD, hq = head0 + h;
+        float M = -1.0e30f;
+#pragma unroll
+        for (int w = 0; w < NW; w++) M = fmaxf(M, mlw[(w * 8 + h) * 2]);
+        float L = 0.f, a = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; w++) {
+            const float wt = __expf(mlw[(w * 8 + h) * 2] - M);
+            L = fmaf(wt, mlw[(w * 8 + h) * 2 + 1], L);
+            a = fmaf(wt, ow[((size_t)w * 8 + h) * HD + d], a);
+        }
+        if (p.balance) {
+            const size_t r = rec_base * p.n_q + hq;
+            float *ml = p.tmp + (size_t)gridDim.z * p.nwg * p.n_q * HD;
+            p.tmp[r * HD + d] = a;
+            if (d == 0) { ml[2 * r] = M; ml[2 * r + 1] = L; }
+        } else {
+            float *rec = p.tmp + (size_t)slot * p.n_q * p.nwg * (HD + 2) + (size_t)hq * p.nwg * (HD + 2) + (size_t)part * (HD + 2);
+            rec[2 + d] = a;
+            if (d == 0) { rec[0] = M; rec[1] = L; }
+        }
+    }
+}
+
+template <int HD>
+constexpr size_t mfma_lds_bytes()
+{
+    constexpr size_t strip = 2 * (size_t)kMfmaTile * (HD / 32 * 18) + 2 * (size_t)kMfmaTile * (HD / 32) * 4;
+    constexpr size_t qshare = (size_t)(HD / 32) * 64 * (16 + 4);                 // the shared q operands and sums
+    constexpr size_t fold = (size_t)kMfmaWaves * 8 * HD * 4 + (size_t)kMfmaWaves * 8 * 2 * 4 + (size_t)kMfmaWaves * 8 * (HD / 32) * 4;
+    return strip * kMfmaWaves + qshare > fold ? strip * kMfmaWaves + qshare : fold;
+}
+
 template <int HD, int GP, int NW>
 constexpr size_t lanes_lds_bytes()
 {
@@ -813,6 +1170,8 @@ int launch_bound(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
     LaneParams p = base_params(k);
     const int hd = (int)k.desc.dims[2], nw = (k.variant >> 16) & 0xFF;
     p.nwg = k.variant & 0xFFFF;
+    const bool mfma = nw == 0xFF;          // the matrix-core form of the row phase (bind_sdpa_lanes)
+    if (mfma) { p.hsplit = 1; p.groups = p.n_q / p.n_kv; }
     int n_slots = 1;
     switch (k.desc.kind) {
     case KSH_SDPA_NAIVE:
@@ -838,16 +1197,22 @@ int launch_bound(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
         p.out = (float *)a.out[1];
         p.scale = k.desc.params[0];
         p.mode = kModeMerge;
-        if (balanced_slots(n_slots, p.nwg)) {
+        if (balanced_slots(n_slots, p.nwg) || mfma) {
             p.balance = 1;
             p.mode = kModePart;
-            if (launch_lanes(p, hd, nw, n_slots, st)) return 1;
+            if (mfma) {
+                hipLaunchKernelGGL(sdpa_mfma_kernel<256>, dim3(p.nwg, p.n_kv, n_slots), dim3(kMfmaWaves * 64), mfma_lds_bytes<256>(), st, p);
+                const hipError_t e0 = hipGetLastError();
+                if (e0 != hipSuccess) return hip_fail(e0, "sdpa (matrix-core form) launch");
+            } else if (launch_lanes(p, hd, nw, n_slots, st)) {
+                return 1;
+            }
             if (hd == 512)
-                hipLaunchKernelGGL(sdpa_dealt_merge_kernel<512>, dim3(p.n_q * 8, n_slots), dim3(256), 0, st, p.tmp, p.meta, p.meta_stride, p.nwg, p.n_q, p.out);
+                hipLaunchKernelGGL(sdpa_dealt_merge_kernel<512>, dim3(p.n_q * 8, n_slots), dim3(256), 0, st, p.tmp, p.meta, p.meta_stride, p.nwg, p.n_q, p.out, mfma ? kMfmaRound : 1);
             else if (hd == 256)
-                hipLaunchKernelGGL(sdpa_dealt_merge_kernel<256>, dim3(p.n_q * 4, n_slots), dim3(256), 0, st, p.tmp, p.meta, p.meta_stride, p.nwg, p.n_q, p.out);
+                hipLaunchKernelGGL(sdpa_dealt_merge_kernel<256>, dim3(p.n_q * 4, n_slots), dim3(256), 0, st, p.tmp, p.meta, p.meta_stride, p.nwg, p.n_q, p.out, mfma ? kMfmaRound : 1);
             else
-                hipLaunchKernelGGL(sdpa_dealt_merge_kernel<128>, dim3(p.n_q * 2, n_slots), dim3(256), 0, st, p.tmp, p.meta, p.meta_stride, p.nwg, p.n_q, p.out);
+                hipLaunchKernelGGL(sdpa_dealt_merge_kernel<128>, dim3(p.n_q * 2, n_slots), dim3(256), 0, st, p.tmp, p.meta, p.meta_stride, p.nwg, p.n_q, p.out, mfma ? kMfmaRound : 1);
             const hipError_t e = hipGetLastError();
             return e == hipSuccess ? 0 : hip_fail(e, "sdpa merge launch");
         }
@@ -918,6 +1283,28 @@ int bind_sdpa_lanes(ksh_kernel &k, int nwg, int n_slots)
 {
     const int64_t *d = k.desc.dims;
     const int n_q = (int)d[0], n_kv = (int)d[1], hd = (int)d[2];
+    // sched.vec = 2: the matrix-core form of the row phase -- several slots' (or one slot's) split-KV partials for
+    // heads of 256 and up to 8 q heads per kv head, merged by a second launch
+    // It is the default where the launch can hold 2^17 rows or more (several long sequences: there it runs at 1.7x
+    // the vector form's rate); below that the two forms tie and the vector form stays (vec = 3 asks for it by name).
+    const bool mfma_fits = k.desc.kind == KSH_SDPA_SLOTS && hd == 256 && n_q / n_kv <= 8 && n_slots <= 16 && nwg >= 2 && nwg <= 64;
+    if (k.desc.sched.vec == 2 || (k.desc.sched.vec == 0 && mfma_fits && (int64_t)n_slots * d[3] >= (1 << 17))) {
+        if (!mfma_fits)
+            return set_error("sdpa: the matrix-core form (vec=2) takes KSH_SDPA_SLOTS with hd 256, up to 8 q heads per kv head, "
+                             "up to 16 slots and 2..64 partitions");
+        k.scratch_bytes = 16;
+        set_launch(k, (uint32_t)nwg, (uint32_t)n_kv, (uint32_t)n_slots, kMfmaWaves * 64, (uint32_t)mfma_lds_bytes<256>());
+        k.info.sched = k.desc.sched;
+        k.info.sched.vec = 2;
+        k.info.sched.tg = kMfmaWaves * 64;
+        k.info.sched.nsg = kMfmaWaves;
+        k.info.sched.k_split = (uint32_t)nwg;
+        k.info.sched.lds_tile = kMfmaTile;
+        k.info.sched.unroll = 1;
+        k.variant = nwg | (0xFF << 16) | (1 << 24);
+        k.launch = launch_bound;
+        return 0;
+    }
     int nw = k.desc.sched.nsg ? (int)k.desc.sched.nsg : 0;
     if (!nw) nw = (d[3] / nwg >= 256) ? 8 : 4;   // long partitions: more waves per workgroup
     if (nw != 4 && nw != 8) return set_error("sdpa: unsupported schedule nsg=%d (4 or 8)", nw);

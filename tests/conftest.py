@@ -12,13 +12,18 @@ if ROOT not in sys.path:
 def _isolated_plan_cache(tmp_path_factory):
     """Kernels requested with a zero schedule consult the plan cache; point it at an empty directory so that a plan
     left by an earlier search cannot change which kernel variant a test exercises (tests of the cache set their own)."""
-    old = os.environ.get("KSEARCH_BEAM_CACHE")
+    old = {k: os.environ.get(k) for k in ("KSEARCH_BEAM_CACHE", "KSEARCH_SKIP_BEAM")}
     os.environ["KSEARCH_BEAM_CACHE"] = str(tmp_path_factory.mktemp("plans"))
+    # models search their schedules when they are loaded and keep the winners as plans: timing decides between
+    # near-equal candidates, so the kernel variants (and with them the f32 summation order) would change from run to
+    # run and leak from one test's model to the next.  The tests of the search and of the warm-up switch it on.
+    os.environ["KSEARCH_SKIP_BEAM"] = "1"
     yield
-    if old is None:
-        os.environ.pop("KSEARCH_BEAM_CACHE", None)
-    else:
-        os.environ["KSEARCH_BEAM_CACHE"] = old
+    for k, v in old.items():
+        if v is None:
+            os.environ.pop(k, None)
+        else:
+            os.environ[k] = v
 
 
 def pytest_configure(config):

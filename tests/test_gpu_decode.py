@@ -144,3 +144,33 @@ def test_generate_refuses_past_max_seq(small_model):
     gpu.reset()
     with pytest.raises(hip.KshError, match="max_seq exceeded"):
         gpu.generate([1, 2, 3], SMALL["max_seq"], use_graph=False)
+
+
+def test_plans_are_warmed_at_load_and_picked_up(ctx, tmp_path, monkeypatch):
+    """GemmaPrimModel's load warms the schedule search for its GEMV shapes (gemma_prim.rs:254-290) unless
+    KSEARCH_SKIP_BEAM is set: the model's kinds leave plan files, a second model is served from them, and the
+    decode step under the planned schedules still matches the oracle."""
+    monkeypatch.setenv("KSEARCH_BEAM_CACHE", str(tmp_path / "beam"))
+    monkeypatch.delenv("KSEARCH_SKIP_BEAM", raising=False)
+    w = synth.gemma_weights(SMALL, 500, oracle.quantize_q4k, synth.chunked(oracle.quantize_q6k), std=0.05)
+    gpu = hip.Gemma(ctx, SMALL, w)
+    names = sorted(f.name.split("_0")[0].rsplit("_", 1)[0] for f in (tmp_path / "beam").glob("*.txt"))
+    kinds = {n.split("_" + str(SMALL["hidden"]))[0] for n in names}
+    assert any(n.startswith("rms_matvec_qkv_q4k") for n in names) and any(n.startswith("rms_matvec_gate_up_q4k") for n in names)
+    assert any(n.startswith("matvec_q4k") for n in names) and any(n.startswith("attend_decode_q40") for n in names), names
+    stamp = {f.name: f.stat().st_mtime_ns for f in (tmp_path / "beam").glob("*.txt")}
+    cpu = oracle.Gemma(SMALL, w)
+    row = SMALL["n_kv"] * SMALL["hd"] // 32 * 18
+    bufs = [[hip.Buffer(ctx, hip.lib().ksh_gemma_kv(gpu.h, l, x), owned=False) for x in (0, 1)] for l in range(SMALL["n_layers"])]
+    for i, t in enumerate(np.random.default_rng(504).integers(0, SMALL["vocab"], 6)):
+        gpu.forward_token(int(t), use_graph=bool(i & 1))
+        rows = np.stack([np.stack([ctx.read_bytes(bufs[l][x], row, i * row) for x in (0, 1)]) for l in range(SMALL["n_layers"])])
+        _, c_logits = cpu.forward(int(t), return_logits=True, adopt_rows=rows)
+        assert cpu.row_max_step.max() <= 1.0 + 1e-3
+        assert_close(gpu.logits(), c_logits, 1e-3, f"logits at step {i} under planned schedules")
+    gpu.close()
+    again = hip.Gemma(ctx, SMALL, w)                       # every search is served from its file: none is rewritten
+    assert {f.name: f.stat().st_mtime_ns for f in (tmp_path / "beam").glob("*.txt")} == stamp
+    again.close()
+    cpu.close()
+    del kinds

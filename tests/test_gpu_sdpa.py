@@ -376,3 +376,45 @@ def test_beam_search_attention_kinds(ctx, tmp_path, monkeypatch):
     kh[600 * 144:601 * 144], vh[600 * 144:601 * 144] = k_row, v_row
     want = oracle.sdpa(q_o, kh, vh, n_q, n_kv, hd, 601, 0, 1.0 / 16.0)
     assert_close(ctx.read_f32(outs3[3], n_q * hd), want, 1e-3, "attend_decode after the search")
+
+
+@pytest.mark.parametrize("n_q,n_kv,lens,max_t,nwg,start", [
+    (8, 1, [5583, 3908, 9979, 4967], 16384, 0, 0),     # BASELINE config 3
+    (8, 1, [1, 33, 127, 128, 129, 700], 1024, 8, 0),   # a single row, tile edges, the wave-tile boundary
+    (8, 1, [2048], 2048, 16, 0),                       # one slot
+    (8, 2, [300, 1500, 31], 2048, 8, 0),               # two kv heads of four q heads each
+    (4, 1, [900, 64], 1024, 4, 100),                   # four q heads, a window that starts at row 100
+    (8, 1, [16384, 1024], 16384, 64, 0),               # the longest sequence beside a short one
+])
+def test_sdpa_slots_matrix_core_form(ctx, n_q, n_kv, lens, max_t, nwg, start):
+    """The matrix-core form of the row phase (schedule vec = 2: f16 MFMA on exact integer codes, q and p*dv split
+    hi | lo) against the serial oracle per slot, 1e-3 relative; and against the float64 brute force, where it is
+    held to 1e-4 (the products are exact, only f32 accumulation and exp remain)."""
+    hd, n_slots = 256, len(lens)
+    _, kk, vv, q = synth.cfg3_q40_attention(n_slots=n_slots, n_q=n_q, n_kv=n_kv, hd=hd, max_t=max_t, lo=1, seed=1303)
+    meta = np.zeros((n_slots, 4), np.float32)
+    meta[:, 0] = lens
+    meta[:, 1] = start
+    lens = [min(t, max_t - start) for t in lens]
+    meta[:, 0] = lens
+    scale = 1.0 / 16.0
+    k = ctx.compile(hip.make_desc(hip.Kind.SDPA_SLOTS, (n_q, n_kv, hd, max_t, n_slots, nwg), (DType.Q40, DType.F32), (scale,), dict(vec=2)))
+    assert "mfma" in k.name
+    parts = k.info.sched.k_split
+    tmp, out = ctx.buffer_empty_f32(n_slots * n_q * parts * (hd + 2)), ctx.buffer_empty_f32(n_slots * n_q * hd)
+    ins = [ctx.buffer_f32(q), ctx.buffer_bytes(kk.reshape(-1)), ctx.buffer_bytes(vv.reshape(-1)), ctx.buffer_f32(meta)]
+    ctx.encode_multi(k, ins, [tmp, out])
+    ctx.synchronize()
+    got = ctx.read_f32(out, n_slots * n_q * hd).reshape(n_slots, -1)
+    worst64 = 0.0
+    for s in range(n_slots):
+        want = oracle.sdpa(q[s], kk[s], vv[s], n_q, n_kv, hd, lens[s], start, scale)
+        assert_close(got[s], want, TOL, f"{k.name} slot {s} ({lens[s]} rows)")
+        if lens[s] <= 4096:
+            w64 = oracle.sdpa(q[s], kk[s], vv[s], n_q, n_kv, hd, lens[s], start, scale, f64=True)
+            worst64 = max(worst64, float(np.max(np.abs(got[s] - w64) / np.maximum(np.abs(w64), np.sqrt(np.mean(w64 ** 2))))))
+    assert worst64 <= 1e-4, worst64
+    # a second launch on the same buffers gives the same bits (fixed summation order)
+    ctx.encode_multi(k, ins, [tmp, out])
+    ctx.synchronize()
+    assert np.array_equal(ctx.read_f32(out, n_slots * n_q * hd).reshape(n_slots, -1), got)

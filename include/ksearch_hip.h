@@ -320,10 +320,21 @@ const char *ksh_plan_kind(const ksh_kernel_desc *desc);
 int ksh_beam_candidates(const ksh_kernel_desc *desc, ksh_sched *out, int cap);
 /* beam_search_matvec / Eng::beam_matvec (crates/ksearch_codegen/src/lib.rs:178-246,
  * ksearch_kernels/src/lib.rs:1985-2043): time every candidate (1 warm-up +
- * `iters` timed), save the best plan, return it. force=1 ignores a cached plan. */
+ * `iters` timed), save the best plan, return it.  The library's own default schedule is timed first and a
+ * candidate replaces it only when it is clearly faster (3 %; 10 % for cold timing, whose single launches are noisier).  force & 1 ignores a cached plan;
+ * force & 2 times cold: one launch at a time, the caches evicted in between (what the model loaders use: a decode
+ * step streams its weights from HBM), where the plain form launches `iters` times back to back. */
 int ksh_beam_search(ksh_ctx *ctx, const ksh_kernel_desc *desc,
                     ksh_buf *const *inputs, int n_in, ksh_buf *const *outputs, int n_out,
                     int iters, int force, ksh_sched *best, double *best_ms, int *from_cache);
+/* The same search with every candidate timed the way a decode loop runs it (Eng::warm_matvec_plans at model load,
+ * crates/ksearch_kernels/src/lib.rs:2057-2080, gemma_prim.rs:254-290): one HIP graph of n_sets dependent launches,
+ * launch i over set i (input_sets[i * n_in ..], output_sets[i * n_out ..]: another layer's weights of the same shape,
+ * so that every launch streams its weights from HBM), replayed `iters` times, best replay / n_sets.  Isolated launches rank
+ * schedules differently from the loop (measured: plans from them cost the decode loop 2 - 4 %). */
+int ksh_beam_search_chain(ksh_ctx *ctx, const ksh_kernel_desc *desc, int n_sets,
+                          ksh_buf *const *input_sets, int n_in, ksh_buf *const *output_sets, int n_out,
+                          int iters, int force, ksh_sched *best, double *best_ms, int *from_cache);
 
 /* ---- decode loop: GemmaPrimModel for the synthetic Gemma-4-E2B shape
  * (crates/ksearch_gemma/src/gemma_prim.rs:881-1275, 1658-1768), minus PLE,

@@ -15,6 +15,7 @@
 #include <cmath>
 #include <cstdlib>
 #include <algorithm>
+#include <map>
 #include <memory>
 #include <vector>
 
@@ -574,6 +575,66 @@ int plan_layer(ksh_gemma4 *m, int l)
     return 0;
 }
 
+// Schedule searches at model load (Eng::warm_matvec_plans, gemma_prim.rs:254-290), one per distinct GEMV shape of the
+// layers: the candidates run as the decode step runs them, a graph of one launch per layer of that shape over the
+// layer's own weights.  Kinds whose partition count the loop fixes (attention) keep their defaults.
+void warm_plans(ksh_gemma4 *m)
+{
+    const ksh_gemma4_cfg &c = m->c;
+    struct Group {
+        ksh_kernel_desc d;
+        std::vector<ksh_buf *> in, out;
+        int n_in = 0, n_out = 0, n_sets = 0;
+    };
+    std::map<std::vector<int64_t>, Group> groups;
+    auto add = [&](int kind, std::initializer_list<int64_t> dims, int wdt, std::initializer_list<ksh_buf *> in, std::initializer_list<ksh_buf *> out) {
+        std::vector<int64_t> key{kind, wdt};
+        key.insert(key.end(), dims.begin(), dims.end());
+        Group &g = groups[key];
+        if (!g.n_sets) {
+            memset(&g.d, 0, sizeof(g.d));
+            g.d.kind = kind;
+            int i = 0;
+            for (int64_t v : dims) g.d.dims[i++] = v;
+            g.d.dtypes[0] = wdt;
+            g.d.dtypes[1] = KSH_F32;
+            g.d.params[0] = c.eps;
+            g.n_in = (int)in.size();
+            g.n_out = (int)out.size();
+        }
+        g.in.insert(g.in.end(), in.begin(), in.end());
+        g.out.insert(g.out.end(), out.begin(), out.end());
+        g.n_sets++;
+    };
+    const int64_t h = c.hidden;
+    for (int l = 0; l < c.n_layers; l++) {
+        const ksh_gemma4_layer &L = m->layers[l];
+        const int hd = L.is_swa ? c.hd_swa : c.hd_full;
+        const int64_t qd = (int64_t)c.n_q * hd, kvd = (int64_t)c.n_kv * hd;
+        const bool owns = l < c.n_layers - c.shared_kv_layers;
+        // (a layer that plan_layer is about to refuse takes no part)
+        if (!L.wq || !L.wo || !L.wgate || !L.wup || !L.wdown || !L.attn_norm || !L.post_attn_norm || !L.ffn_norm || !L.post_ffw_norm ||
+            L.ffn <= 0 || L.ffn % 256 || (owns && (!L.wk || !L.wv)))
+            continue;
+        if (owns && L.dt_q == KSH_Q4K && L.dt_k == KSH_Q4K && L.dt_v == KSH_Q4K)
+            add(KSH_RMSNORM_MATVEC_QKV, {qd, kvd, h, 1}, KSH_Q4K, {L.wq, L.wk, L.wv, m->y, L.attn_norm, L.post_ffw_norm, m->x}, {m->tq, m->tk, m->tv, m->xb});
+        else
+            add(KSH_RMSNORM_MATVEC, {qd, h, 1}, L.dt_q, {L.wq, m->y, L.attn_norm, L.post_ffw_norm, m->x}, {m->tq, m->xb});
+        add(KSH_MATVEC, {h, qd}, L.dt_o, {L.wo, m->to}, {m->y});
+        if (L.dt_gate == KSH_Q4K && L.dt_up == KSH_Q4K)
+            add(KSH_RMSNORM_MATVEC_GATE_UP_GELU, {L.ffn, h, 1}, KSH_Q4K, {L.wgate, L.wup, m->y, L.ffn_norm, L.post_attn_norm, m->x}, {m->ff, m->xb});
+        add(KSH_MATVEC, {h, L.ffn}, L.dt_down, {L.wdown, m->ff}, {m->y});
+    }
+    for (auto &kv : groups) {
+        Group &g = kv.second;
+        ksh_sched best;
+        double ms = 0.0;
+        int cached = 0;
+        (void)ksh_beam_search_chain(m->ctx, &g.d, g.n_sets, g.in.data(), g.n_in, g.out.data(), g.n_out, 4, 0, &best, &ms, &cached);
+    }
+    (void)ksh_synchronize(m->ctx);
+}
+
 // puts the graphs in use back where they belong (they are tied to the cache buffers they were captured with)
 void stash_graphs(ksh_gemma4 *m)
 {
@@ -625,6 +686,7 @@ int ksh_gemma4_create(ksh_ctx *ctx, const ksh_gemma4_cfg *cfg, const ksh_gemma4_
         return 1;
     m->kv_k.assign(c.n_layers, nullptr);
     m->kv_v.assign(c.n_layers, nullptr);
+    if (!getenv("KSEARCH_SKIP_BEAM")) warm_plans(m);
     for (int l = 0; l < c.n_layers; l++) {
         if (plan_layer(m, l)) return 1;
         if (!m->plan[l].owns) continue;

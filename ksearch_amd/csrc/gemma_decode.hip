@@ -32,6 +32,7 @@
 #include <cstdlib>
 #include <algorithm>
 #include <memory>
+#include <functional>
 #include <vector>
 
 #include "ksh_device.hpp"
@@ -167,8 +168,10 @@ int enc(ksh_gemma *m, ksh_kernel *k, std::initializer_list<ksh_buf *> in, std::i
 // 1985-2080): the kind is timed on the model's own buffers over its candidate schedules and the winner saved in the
 // plan cache, where the kernel lookups that follow find it; a plan that is there already is taken as it is.  A kind
 // without a schedule space, or whose search fails, keeps the library default.
+// One schedule search at model load: the candidate kernels run as the decode step runs them, a graph of one launch
+// per layer over that layer's own weights (Eng::warm_matvec_plans, gemma_prim.rs:254-290).
 void warm_plan(ksh_gemma *m, int kind, std::initializer_list<int64_t> dims, std::initializer_list<int> dtypes,
-               std::initializer_list<float> params, std::initializer_list<ksh_buf *> in, std::initializer_list<ksh_buf *> out)
+               std::initializer_list<float> params, int n_sets, const std::function<void(int, std::vector<ksh_buf *> &, std::vector<ksh_buf *> &)> &set)
 {
     ksh_kernel_desc d;
     memset(&d, 0, sizeof(d));
@@ -179,14 +182,18 @@ void warm_plan(ksh_gemma *m, int kind, std::initializer_list<int64_t> dims, std:
     for (int v : dtypes) d.dtypes[i++] = v;
     i = 0;
     for (float v : params) d.params[i++] = v;
-    ksh_buf *ib[kMaxIn], *ob[kMaxOut];
-    int ni = 0, no = 0;
-    for (ksh_buf *b : in) ib[ni++] = b;
-    for (ksh_buf *b : out) ob[no++] = b;
+    std::vector<ksh_buf *> in, out, one_in, one_out;
+    for (int l = 0; l < n_sets; l++) {
+        one_in.clear();
+        one_out.clear();
+        set(l, one_in, one_out);
+        in.insert(in.end(), one_in.begin(), one_in.end());
+        out.insert(out.end(), one_out.begin(), one_out.end());
+    }
     ksh_sched best;
     double ms = 0.0;
     int cached = 0;
-    (void)ksh_beam_search(m->ctx, &d, ib, ni, ob, no, 8, 0, &best, &ms, &cached);
+    (void)ksh_beam_search_chain(m->ctx, &d, n_sets, in.data(), (int)one_in.size(), out.data(), (int)one_out.size(), 4, 0, &best, &ms, &cached);
 }
 
 // Up to this many cached positions the attention launch leaves its (then 8) partitions unmerged and the
@@ -434,18 +441,40 @@ int ksh_gemma_create(ksh_ctx *ctx, const ksh_gemma_cfg *cfg, const ksh_gemma_lay
         const float meta[4] = {T, 0.f, 0.f, T - 1.f};
         if (ksh_buffer_write(ctx, g->meta, 0, meta, 16, 1)) return 1;
         ksh_buf *lm_w = g->embd_rows ? g->embd_rows : g->embd;
-        warm_plan(g, KSH_RMSNORM_MATVEC_QKV, {qd, kvd, c.hidden, 0}, {KSH_Q4K, KSH_F32}, {c.eps}, {L.wq, L.wk, L.wv, g->x, L.attn_norm}, {g->tq, g->tk, g->tv});
-        warm_plan(g, KSH_RMSNORM_MATVEC_QKV, {qd, kvd, c.hidden, 1}, {KSH_Q4K, KSH_F32}, {c.eps},
-                  {L.wq, L.wk, L.wv, g->y, L.attn_norm, L.post_ffw_norm, g->x}, {g->tq, g->tk, g->tv, g->xb});
-        warm_plan(g, KSH_MATVEC, {c.hidden, qd}, {KSH_Q4K, KSH_F32}, {}, {L.wo, g->to}, {g->y});
-        warm_plan(g, KSH_RMSNORM_MATVEC_GATE_UP_GELU, {c.ffn, c.hidden, 1}, {KSH_Q4K, KSH_F32}, {c.eps},
-                  {L.wgate, L.wup, g->y, L.ffn_norm, L.post_attn_norm, g->x}, {g->ff, g->xb});
-        warm_plan(g, KSH_MATVEC, {c.hidden, c.ffn}, {KSH_Q4K, KSH_F32}, {}, {L.wdown, g->ff}, {g->y});
-        warm_plan(g, KSH_RMSNORM_MATVEC, {c.vocab, c.hidden, 1}, {lm_rows ? KSH_Q6K_ROWS : KSH_Q6K, KSH_F32}, {c.eps},
-                  {lm_w, g->y, g->output_norm, L.post_ffw_norm, g->x}, {g->logits, g->xb});
+        using Bufs = std::vector<ksh_buf *>;
+        const int nl = c.n_layers;
+        auto Lw = [&](int l) -> const ksh_gemma_layer & { return g->layers[l]; };
+        warm_plan(g, KSH_RMSNORM_MATVEC_QKV, {qd, kvd, c.hidden, 0}, {KSH_Q4K, KSH_F32}, {c.eps}, nl, [&](int l, Bufs &in, Bufs &out) {
+            in = {Lw(l).wq, Lw(l).wk, Lw(l).wv, g->x, Lw(l).attn_norm};
+            out = {g->tq, g->tk, g->tv};
+        });
+        warm_plan(g, KSH_RMSNORM_MATVEC_QKV, {qd, kvd, c.hidden, 1}, {KSH_Q4K, KSH_F32}, {c.eps}, nl, [&](int l, Bufs &in, Bufs &out) {
+            in = {Lw(l).wq, Lw(l).wk, Lw(l).wv, g->y, Lw(l).attn_norm, Lw(l).post_ffw_norm, g->x};
+            out = {g->tq, g->tk, g->tv, g->xb};
+        });
+        warm_plan(g, KSH_MATVEC, {c.hidden, qd}, {KSH_Q4K, KSH_F32}, {}, nl, [&](int l, Bufs &in, Bufs &out) {
+            in = {Lw(l).wo, g->to};
+            out = {g->y};
+        });
+        warm_plan(g, KSH_RMSNORM_MATVEC_GATE_UP_GELU, {c.ffn, c.hidden, 1}, {KSH_Q4K, KSH_F32}, {c.eps}, nl, [&](int l, Bufs &in, Bufs &out) {
+            in = {Lw(l).wgate, Lw(l).wup, g->y, Lw(l).ffn_norm, Lw(l).post_attn_norm, g->x};
+            out = {g->ff, g->xb};
+        });
+        warm_plan(g, KSH_MATVEC, {c.hidden, c.ffn}, {KSH_Q4K, KSH_F32}, {}, nl, [&](int l, Bufs &in, Bufs &out) {
+            in = {Lw(l).wdown, g->ff};
+            out = {g->y};
+        });
+        // the table is larger than the last-level cache: two launches over it are two cold ones
+        warm_plan(g, KSH_RMSNORM_MATVEC, {c.vocab, c.hidden, 1}, {lm_rows ? KSH_Q6K_ROWS : KSH_Q6K, KSH_F32}, {c.eps}, 2, [&](int, Bufs &in, Bufs &out) {
+            in = {lm_w, g->y, g->output_norm, L.post_ffw_norm, g->x};
+            out = {g->logits, g->xb};
+        });
         if (fused_attend)
-            warm_plan(g, KSH_ATTEND_DECODE, {c.n_q, c.n_kv, c.hd, c.max_seq, 0, 0, 1}, {KSH_Q40, KSH_F32}, {c.eps, c.attn_scale},
-                      {g->tq, L.q_norm, g->rope_cur, g->tk, L.k_norm, g->tv, g->meta}, {g->kv_k[0], g->kv_v[0], g->attn_tmp, g->to});
+            warm_plan(g, KSH_ATTEND_DECODE, {c.n_q, c.n_kv, c.hd, c.max_seq, 0, 0, 1}, {KSH_Q40, KSH_F32}, {c.eps, c.attn_scale}, nl,
+                      [&](int l, Bufs &in, Bufs &out) {
+                          in = {g->tq, Lw(l).q_norm, g->rope_cur, g->tk, Lw(l).k_norm, g->tv, g->meta};
+                          out = {g->kv_k[l], g->kv_v[l], g->attn_tmp, g->to};
+                      });
         if (ksh_synchronize(ctx)) return 1;
     }
     const float embed_scale = std::sqrt((float)c.hidden);   // gemma_prim.rs:683

@@ -9,6 +9,7 @@
 #include <cerrno>
 #include <cinttypes>
 #include <cstdlib>
+#include <functional>
 #include <string>
 #include <vector>
 
@@ -118,6 +119,28 @@ std::string make_key(const char *kind, const int64_t *dims, int n_dims, const ch
 }  // namespace ksh
 
 using namespace ksh;
+
+namespace {
+
+// One candidate's time: `iters` launches timed together (weights stay in cache between them), or -- cold -- one
+// launch at a time with the caches evicted in between by zero-filling `flush` (larger than the last-level cache),
+// which is how a decode step meets its weights; the minimum of the single launches is taken.
+int time_candidate(ksh_ctx *ctx, ksh_kernel *k, ksh_buf *const *inputs, int n_in, ksh_buf *const *outputs, int n_out, int iters,
+                   ksh_buf *flush, double *ms)
+{
+    if (ksh_run_timed(ctx, k, inputs, nullptr, n_in, outputs, nullptr, n_out, 1, ms)) return 2;   // warm-up; a refusal shows here
+    if (!flush) return ksh_run_timed(ctx, k, inputs, nullptr, n_in, outputs, nullptr, n_out, iters, ms) ? 1 : 0;
+    double best = 0.0;
+    for (int i = 0; i < iters; i++) {
+        double t = 0.0;
+        if (ksh_buffer_fill_zero(ctx, flush) || ksh_run_timed(ctx, k, inputs, nullptr, n_in, outputs, nullptr, n_out, 1, &t)) return 1;
+        if (i == 0 || t < best) best = t;
+    }
+    *ms = best;
+    return 0;
+}
+
+}  // namespace
 
 extern "C" {
 
@@ -232,11 +255,10 @@ int ksh_beam_candidates(const ksh_kernel_desc *d, ksh_sched *out, int cap)
     return 0;
 }
 
-int ksh_beam_search(ksh_ctx *ctx, const ksh_kernel_desc *desc, ksh_buf *const *inputs, int n_in,
-                    ksh_buf *const *outputs, int n_out, int iters, int force, ksh_sched *best, double *best_ms,
-                    int *from_cache)
+// the search proper: `time_one(kernel, &ms)` returns 0, 1 (error) or 2 (this candidate cannot run: pass it over)
+static int beam_search_with(ksh_ctx *ctx, const ksh_kernel_desc *desc, const std::function<int(ksh_kernel *, double *)> &time_one,
+                            int force, double margin, ksh_sched *best, double *best_ms, int *from_cache)
 {
-    if (!ctx || !desc || !best || !best_ms) return set_error("ksh_beam_search: bad arguments");
     const char *pk = ksh_plan_kind(desc);
     if (!pk) return set_error("ksh_beam_search: kind %d has no schedule space", desc->kind);
     char chip[128];
@@ -244,19 +266,17 @@ int ksh_beam_search(ksh_ctx *ctx, const ksh_kernel_desc *desc, ksh_buf *const *i
     const int nd = plan_dims(*desc);
     if (from_cache) *from_cache = 0;
     // KSEARCH_BEAM_FORCE, crates/ksearch_codegen/src/lib.rs:206
-    if (!force && !std::getenv("KSEARCH_BEAM_FORCE") && ksh_plan_load(pk, desc->dims, nd, chip, best, best_ms) == 0) {
+    if (!(force & 1) && !std::getenv("KSEARCH_BEAM_FORCE") && ksh_plan_load(pk, desc->dims, nd, chip, best, best_ms) == 0) {
         if (from_cache) *from_cache = 1;
         return 0;
     }
     std::vector<ksh_sched> cand(128);
     const int n = ksh_beam_candidates(desc, cand.data(), (int)cand.size());
     if (n <= 0) return set_error("ksh_beam_search: no candidates for kind %d", desc->kind);
-    if (iters < 1) iters = 3;
     bool found = false;
     std::string refusal;
-    // The library's own default goes first (no plan file exists at this point, or the search is forced): a candidate
-    // replaces it only when it is at least 3 % faster, so that timing noise between near-equal schedules does not
-    // move a shape off the schedule its default was chosen for.
+    // The library's own default goes first: a candidate replaces it only when it is faster by the margin, so that
+    // timing noise between near-equal schedules does not move a shape off the schedule its default was chosen for.
     double default_ms = 0.0;
     {
         ksh_kernel_desc d = *desc;
@@ -264,9 +284,7 @@ int ksh_beam_search(ksh_ctx *ctx, const ksh_kernel_desc *desc, ksh_buf *const *i
         d.sched.tg = ~0ull;   // the library default, whatever the plan cache holds
         ksh_kernel *k = nullptr;
         double ms = 0.0;
-        if (ksh_kernel_get(ctx, &d, &k) == 0 &&
-            ksh_run_timed(ctx, k, inputs, nullptr, n_in, outputs, nullptr, n_out, 1, &ms) == 0 &&
-            ksh_run_timed(ctx, k, inputs, nullptr, n_in, outputs, nullptr, n_out, iters, &ms) == 0) {
+        if (ksh_kernel_get(ctx, &d, &k) == 0 && time_one(k, &ms) == 0) {
             ksh_kernel_info info;
             ksh_kernel_info_get(k, &info);
             found = true;
@@ -281,14 +299,15 @@ int ksh_beam_search(ksh_ctx *ctx, const ksh_kernel_desc *desc, ksh_buf *const *i
         ksh_kernel *k = nullptr;
         if (ksh_kernel_get(ctx, &d, &k)) continue;   // a candidate the kernel family refuses
         double ms = 0.0;
-        // 1 warm-up + timed launches, crates/ksearch_kernels/src/lib.rs:2015-2031.  A candidate whose bindings do
-        // not fit (a partition count the caller's scratch buffer was not sized for) is passed over like a refused one.
-        if (ksh_run_timed(ctx, k, inputs, nullptr, n_in, outputs, nullptr, n_out, 1, &ms)) {
+        // A candidate whose bindings do not fit (a partition count the caller's scratch buffer was not sized for) is
+        // passed over like a refused one.
+        const int rc = time_one(k, &ms);
+        if (rc == 2) {
             refusal = ksh_last_error();
             continue;
         }
-        if (ksh_run_timed(ctx, k, inputs, nullptr, n_in, outputs, nullptr, n_out, iters, &ms)) return 1;
-        if (!found || (ms < *best_ms && (default_ms == 0.0 || ms < 0.97 * default_ms))) {
+        if (rc) return 1;
+        if (!found || (ms < *best_ms && (default_ms == 0.0 || ms < margin * default_ms))) {
             found = true;
             *best_ms = ms;
             *best = cand[i];
@@ -296,6 +315,64 @@ int ksh_beam_search(ksh_ctx *ctx, const ksh_kernel_desc *desc, ksh_buf *const *i
     }
     if (!found) return set_error("ksh_beam_search: every candidate was refused (%s)", refusal.c_str());
     return ksh_plan_save(pk, desc->dims, nd, chip, best, *best_ms);
+}
+
+int ksh_beam_search(ksh_ctx *ctx, const ksh_kernel_desc *desc, ksh_buf *const *inputs, int n_in,
+                    ksh_buf *const *outputs, int n_out, int iters, int force, ksh_sched *best, double *best_ms,
+                    int *from_cache)
+{
+    if (!ctx || !desc || !best || !best_ms) return set_error("ksh_beam_search: bad arguments");
+    if (iters < 1) iters = 3;
+    // force & 2: cold timing
+    ksh_buf *flush = nullptr;
+    if ((force & 2) && ksh_buffer_alloc(ctx, (size_t)384 << 20, nullptr, &flush)) return 1;
+    struct Release {
+        ksh_buf *b;
+        ~Release() { if (b) ksh_buffer_release(b); }
+    } release{flush};
+    // 1 warm-up + timed launches, crates/ksearch_kernels/src/lib.rs:2015-2031
+    auto time_one = [&](ksh_kernel *k, double *ms) { return time_candidate(ctx, k, inputs, n_in, outputs, n_out, iters, flush, ms); };
+    return beam_search_with(ctx, desc, time_one, force, flush ? 0.90 : 0.97, best, best_ms, from_cache);
+}
+
+int ksh_beam_search_chain(ksh_ctx *ctx, const ksh_kernel_desc *desc, int n_sets, ksh_buf *const *input_sets, int n_in,
+                          ksh_buf *const *output_sets, int n_out, int iters, int force, ksh_sched *best, double *best_ms,
+                          int *from_cache)
+{
+    if (!ctx || !desc || !best || !best_ms || !input_sets || !output_sets || n_sets < 1 || n_in < 1 || n_out < 1) return set_error("ksh_beam_search_chain: bad arguments");
+    if (iters < 1) iters = 3;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    KSH_HIP(hipEventCreate(&e0));
+    KSH_HIP(hipEventCreate(&e1));
+    struct Events {
+        hipEvent_t a, b;
+        ~Events() { (void)hipEventDestroy(a); (void)hipEventDestroy(b); }
+    } events{e0, e1};
+    hipStream_t st = (hipStream_t)ksh_stream(ctx);
+    auto time_one = [&](ksh_kernel *k, double *ms) -> int {
+        // the candidate as the decode loop runs it: one HIP graph of n_sets dependent launches, each over another
+        // set of inputs (another layer's weights: cold), replayed a few times; the best replay counts
+        if (ksh_synchronize(ctx) || ksh_graph_begin(ctx)) return 1;
+        int rc = 0;
+        for (int s2 = 0; s2 < n_sets && !rc; s2++)
+            if (ksh_encode(ctx, k, input_sets + (size_t)s2 * n_in, nullptr, n_in, output_sets + (size_t)s2 * n_out, nullptr, n_out)) rc = 2;
+        ksh_graph *g = nullptr;
+        if (ksh_graph_end(ctx, &g)) return 1;
+        double best_t = 0.0;
+        if (!rc && ksh_graph_launch(ctx, g)) rc = 1;
+        for (int i = 0; i < iters && !rc; i++) {
+            float t = 0.f;
+            if (hipEventRecord(e0, st) != hipSuccess || ksh_graph_launch(ctx, g) || hipEventRecord(e1, st) != hipSuccess ||
+                hipEventSynchronize(e1) != hipSuccess || hipEventElapsedTime(&t, e0, e1) != hipSuccess)
+                rc = 1;
+            if (i == 0 || t < best_t) best_t = t;
+        }
+        if (ksh_synchronize(ctx)) rc = rc ? rc : 1;
+        ksh_graph_destroy(g);
+        *ms = best_t / n_sets;
+        return rc;
+    };
+    return beam_search_with(ctx, desc, time_one, force, 0.97, best, best_ms, from_cache);
 }
 
 }  // extern "C"

@@ -156,6 +156,7 @@ SYMBOLS = {
     "ksh_encode": (_i, [_vp, _vp, _vpp, _u64p, _i, _vpp, _u64p, _i]),
     "ksh_softcap_argmax_static": (_i, [_vp, _vp, C.c_uint64, C.c_int64, C.c_float, _vp, C.c_uint64]),
     "ksh_run_timed": (_i, [_vp, _vp, _vpp, _u64p, _i, _vpp, _u64p, _i, _i, _dp]),
+    "ksh_beam_search_chain": (_i, [_vp, C.POINTER(KernelDesc), _i, _vpp, _i, _vpp, _i, _i, _i, C.POINTER(Sched), _dp, C.POINTER(C.c_int)]),
     "ksh_flush_async": (_i, [_vp]),
     "ksh_wait_inflight_at_most": (_i, [_vp, _i]),
     "ksh_barrier": (_i, [_vp]),
@@ -512,6 +513,16 @@ class Context:
         best, ms, cached = Sched(), C.c_double(), C.c_int()
         _check(lib().ksh_beam_search(self.h, C.byref(desc), _bufs(inputs), len(inputs), _bufs(outputs),
                                      len(outputs), iters, int(force), C.byref(best), C.byref(ms), C.byref(cached)))
+        return best, ms.value, bool(cached.value)
+
+    def beam_search_chain(self, desc: KernelDesc, input_sets, output_sets, iters: int = 3, force: bool = False):
+        """Every candidate timed as one graph of len(input_sets) dependent launches, launch i over set i."""
+        n_sets, n_in, n_out = len(input_sets), len(input_sets[0]), len(output_sets[0])
+        assert len(output_sets) == n_sets and all(len(s) == n_in for s in input_sets) and all(len(s) == n_out for s in output_sets)
+        best, ms, cached = Sched(), C.c_double(), C.c_int()
+        _check(lib().ksh_beam_search_chain(self.h, C.byref(desc), n_sets, _bufs([b for s in input_sets for b in s]), n_in,
+                                           _bufs([b for s in output_sets for b in s]), n_out, iters, int(force),
+                                           C.byref(best), C.byref(ms), C.byref(cached)))
         return best, ms.value, bool(cached.value)
 
 

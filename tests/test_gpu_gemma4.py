@@ -295,6 +295,29 @@ def test_gemma4_generate_graph_equals_eager_and_oracle(tiny):
     assert gpu.generate_until(prompt, n_new, eos=(), use_graph=False)[0] == graph     # nothing to stop at: the whole run
 
 
+def test_gemma4_plans_are_warmed_at_load(ctx, tmp_path, monkeypatch):
+    """The load warms one schedule search per distinct GEMV shape of the layers (gemma_prim.rs:254-290) unless
+    KSEARCH_SKIP_BEAM is set: two feed-forward widths leave two plans each for the gate/up and the down kinds, a
+    second load is served from the files, and the decode step under the planned schedules matches the oracle."""
+    monkeypatch.setenv("KSEARCH_BEAM_CACHE", str(tmp_path / "beam"))
+    monkeypatch.delenv("KSEARCH_SKIP_BEAM", raising=False)
+    cfg = dict(synth.GEMMA4_TINY)
+    w = synth.gemma4_weights(cfg, 612, oracle.quantize_q4k, oracle.quantize_q6k, ffn=FFN, swa_pattern=PATTERN, std=0.05)
+    gpu, cpu = hip.Gemma4(ctx, cfg, w), oracle.Gemma4(cfg, w)
+    names = sorted(f.name for f in (tmp_path / "beam").glob("*.txt"))
+    assert sum(n.startswith("rms_matvec_gate_up_q4k") for n in names) == 2, names
+    assert sum(n.startswith("rms_matvec_qkv_q4k") for n in names) >= 1 and sum(n.startswith("matvec_q4k") for n in names) >= 3, names
+    stamp = {f.name: f.stat().st_mtime_ns for f in (tmp_path / "beam").glob("*.txt")}
+    toks = np.random.default_rng(613).integers(0, cfg["vocab"], 6)
+    compared, _ = teacher_forced(gpu, cpu, cfg, PATTERN, toks, use_graph=True)
+    assert compared == 6
+    gpu.close()
+    again = hip.Gemma4(ctx, cfg, w)
+    assert {f.name: f.stat().st_mtime_ns for f in (tmp_path / "beam").glob("*.txt")} == stamp
+    again.close()
+    cpu.close()
+
+
 def test_gemma4_create_errors(ctx):
     cfg = dict(synth.GEMMA4_TINY, vocab=256)
     w = synth.gemma4_weights(cfg, 613, oracle.quantize_q4k, oracle.quantize_q6k, ffn=512, swa_pattern=PATTERN)

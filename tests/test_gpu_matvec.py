@@ -342,3 +342,28 @@ def test_beam_search_on_device(ctx, eng, tmp_path, monkeypatch):
     assert len(files) == 1 and files[0].name.startswith("matvec_q4k_1024x2048_")     # the chip name is in the hash
     best2, ms2, cached2 = eng.beam_matvec(ctx, rows, cols, DType.Q4K, bw, bx, by, iters=5)
     assert cached2 and best2.as_dict() == best.as_dict()
+
+
+def test_beam_search_over_a_chain_of_layers(ctx, tmp_path, monkeypatch):
+    """The search as a model load runs it (Eng::warm_matvec_plans, ksearch_kernels/src/lib.rs:2057-2080): each
+    candidate is one graph of dependent launches, one per layer over that layer's weights; the winner is a member of
+    the candidate list (or the library's default), it is saved, and the last set's output is that set's product."""
+    monkeypatch.setenv("KSEARCH_BEAM_CACHE", str(tmp_path / "beam"))
+    rows, cols, n_sets = 512, 1024, 5
+    ws = [synth.q4k_blocks(rows * cols // 256, seed=910 + i) for i in range(n_sets)]
+    x = synth.normal_f32(cols, seed=920)
+    bx = ctx.buffer_f32(x)
+    bws = [ctx.buffer_bytes(w) for w in ws]
+    bys = [ctx.buffer_empty_f32(rows) for _ in range(n_sets)]
+    desc = hip.make_desc(hip.Kind.MATVEC, (rows, cols), (DType.Q4K, DType.F32))
+    best, ms, cached = ctx.beam_search_chain(desc, [[w, bx] for w in bws], [[y] for y in bys], iters=3, force=True)
+    assert not cached and 0 < ms < 1.0
+    for w, y in zip(ws, bys):
+        assert_close(ctx.read_f32(y, rows), oracle.matvec(oracle.Q4K, w, rows, cols, x), TOL, "after chain search")
+    files = list((tmp_path / "beam").glob("*.txt"))
+    assert len(files) == 1 and files[0].name.startswith("matvec_q4k_512x1024_")
+    best2, _, cached2 = ctx.beam_search_chain(desc, [[w, bx] for w in bws], [[y] for y in bys])
+    assert cached2 and best2.as_dict() == best.as_dict()
+    # bad arguments are errors, not crashes
+    with pytest.raises(hip.KshError):
+        ctx.beam_search_chain(hip.make_desc(hip.Kind.RMSNORM_ADD_THEN_RMSNORM, (64,), (), (1e-6,)), [[bx]], [[bys[0]]], force=True)

@@ -312,9 +312,17 @@ def cpu_baseline_matvec(w, x, rows, cols, budget_s=1.5):
 
 
 # HBM bytes per launch of the headline kernel, from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
-# profiles/q4k_gemv_cfg0_cold.txt (2.00 x 4760.1 KiB fetched + 16.0 KiB written).  Counters cannot be read from
-# inside this script, so the figure is carried here for the kernel it was taken on and is null for any other.
-MEASURED_TRAFFIC_BYTES = {"matvec_q4k_r2_w8_v3": 9753805}
+# profiles/q4k_gemv_cfg0_cold.txt (2.00 x 4765.1 KiB fetched + 16.0 KiB written).  Counters cannot be read from
+# inside this script, so the figure is carried here for the kernel it was taken on; a headline kernel that is not in
+# the table is an error (the counters have to be taken again for it), never a silent null.
+MEASURED_TRAFFIC_BYTES = {"matvec_q4k_r2_w8_v3": 9775309}
+
+
+def measured_traffic(kernel: str) -> int:
+    if kernel not in MEASURED_TRAFFIC_BYTES:
+        raise SystemExit(f"bench.py: no FETCH_SIZE / WRITE_SIZE figures for the headline kernel {kernel!r}: take the two "
+                         f"counter runs on it (profiles/q4k_gemv_cfg0_cold.txt holds the commands) and add it to MEASURED_TRAFFIC_BYTES")
+    return MEASURED_TRAFFIC_BYTES[kernel]
 
 
 def main() -> int:
@@ -326,6 +334,9 @@ def main() -> int:
     ap.add_argument("--no-extras", action="store_true", help="headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--eager", action="store_true", help="cfg4 without HIP-graph replay (kernel-trace profiling)")
+    ap.add_argument("--attn-form", choices=["default", "lanes", "mfma"], default="default",
+                    help="cfg3: the split-KV row phase as the register (lanes) or the matrix-core (mfma) kernel instead of "
+                         "the library's choice for the shape")
     ap.add_argument("--only", choices=["cfg1", "cfg2", "cfg3", "cfg4", "gemma4", "copy", "floor"],
                     help="run one secondary workload and print its record (for profiling runs); 'copy' is a plain "
                          "64 MiB device copy, the known-size kernel that calibrates the FETCH_SIZE / WRITE_SIZE counters")
@@ -353,7 +364,7 @@ def main() -> int:
         elif args.only == "floor":
             r = bench_floor(ctx, eng, ev, args.copies, args.steps, args.warmup)
         else:
-            r = {"cfg2": lambda: bench_prefill(ctx), "cfg3": lambda: bench_attention(ctx, ev),
+            r = {"cfg2": lambda: bench_prefill(ctx), "cfg3": lambda: bench_attention(ctx, ev, sched={"lanes": dict(vec=3), "mfma": dict(vec=2)}.get(args.attn_form)),
                  "cfg4": lambda: bench_decode(ctx, eng, not args.eager),
                  "gemma4": lambda: bench_decode_gemma4_layout(ctx, eng, not args.eager)}[args.only]()
         ctx.close()
@@ -362,6 +373,7 @@ def main() -> int:
     rows = cols = 4096
     w, x = synth.cfg0_q4k_matvec()
     head = bench_matvec(ctx, eng, ev, DType.Q4K, rows, cols, w, x, args.copies, args.steps, args.warmup)
+    traffic = measured_traffic(head["kernel"])      # before the minutes of secondary workloads, not after
 
     also = {}
     if not args.no_extras:
@@ -389,7 +401,7 @@ def main() -> int:
                                f"({args.copies} rotating copies)", "kernel": head["kernel"]},
         "roofline": {"bound": "hbm", "achieved": round(head["gbps"], 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(head["gbps"] / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(head["kernel"])},
+                     "traffic": traffic},
         "cpu_baseline": cpu,
         "also": also,
     }

@@ -272,21 +272,25 @@ def bench_decode_gemma4_layout(ctx, eng, use_graph=True):
          "weight_GB_per_token": round(wbytes / 1e9, 3), "GB_s": round(wbytes / (min(ms) / 256 * 1e-3) / 1e9, 1),
          "prefill_ms": round(min(pre), 3), "prefill_tok_per_s": round(63 / min(pre) * 1e3, 1),
          "layout": "35 layers, hidden 1536, 4 SWA(256, window 512) : 1 full(512), 20 shared-KV layers, PLE 256, ffn 6144/12288"}
-    # the same model under the slot scheduler: two requests of 64 + 128 tokens decoded in turn from two KV slots
-    # (serial GPU work, one host read-back per token, as the reference's serving loop does it)
-    pool = hip.KvPool(ctx, 2, cfg["max_seq"], n - shared, 512, 1)
-    sv = hip.Serve(model, pool, slots=2, eos=(0xFFFFFFFF, 0xFFFFFFFE), use_graph=use_graph)
-    best = 1e9
-    for rep in range(2):
-        for i in range(2):
-            sv.submit(prompt[i:] + prompt[:i], 128)
-        sv.tick()                                   # admission + prefill of both prompts
-        ctx.synchronize()
-        t0 = time.perf_counter()
-        n_tok = sum(1 for e in sv.run() if e[0] == "token")
-        best = min(best, (time.perf_counter() - t0) / n_tok)
-    r["served_two_slots_tok_s"] = round(1.0 / best, 1)
-    sv.close()
+    # the same model under the slot scheduler: requests of 64 + 128 tokens from as many KV slots, the decoding ones
+    # taking each step together as one pass over the weights (one by one, as the reference's serving loop does it,
+    # for comparison); one host read-back per round
+    pool = hip.KvPool(ctx, 16, cfg["max_seq"], n - shared, 512, 1)
+    served = {}
+    for n_req, batched in ((2, 0), (2, 2), (4, 0), (4, 2), (8, 2), (16, 2)):
+        sv = hip.Serve(model, pool, slots=n_req, eos=(0xFFFFFFFF, 0xFFFFFFFE), use_graph=use_graph, batched_decode=batched)
+        best = 1e9
+        for rep in range(2):
+            for i in range(n_req):
+                sv.submit(prompt[i:] + prompt[:i], 128)
+            sv.tick()                                   # admission + prefill of the prompts
+            ctx.synchronize()
+            t0 = time.perf_counter()
+            n_tok = sum(1 for e in sv.run() if e[0] == "token")
+            best = min(best, (time.perf_counter() - t0) / n_tok)
+        served[f"{n_req}_slots" + ("" if batched else "_one_by_one")] = round(1.0 / best, 1)
+        sv.close()
+    r["served_tok_s"] = served
     model.bind_slot(None, 0)
     pool.close()
     model.close()

@@ -81,7 +81,10 @@ enum ksh_kind {
      * serially, crates/ksearch_cli/src/scheduler.rs:163-187).
      * dims: n_q, n_kv, hd, max_t, n_slots, nwg.  K/V pools are
      * [n_slots][max_t,n_kv,hd] Q4_0; meta is f32[n_slots][4].
-     * in: q[n_slots,n_q*hd], Kpool, Vpool, meta   out: tmp, o[n_slots,n_q*hd] */
+     * in: q[n_slots,n_q*hd], Kpool, Vpool, meta   out: tmp, o[n_slots,n_q*hd]
+     * dims[6] = pool slots > 0: the launch's n_slots entries are a subset, in any order, of pools that hold dims[6]
+     * slots (one decode step for several sequences); a 5th input f32[n_slots] names each entry's pool slot, and
+     * dims[7] is the byte distance between slots of the pools (0: max_t rows). */
     KSH_SDPA_SLOTS = 8,
     /* QuantizeQ40: pack n f32 values (n%32==0) to Q4_0.  dims: n.  in: src  out: dst */
     KSH_QUANTIZE_Q40 = 9,
@@ -99,7 +102,10 @@ enum ksh_kind {
      * max_seq = 0: in: q, qw, rope_row f32[hd], k, kw, v   out: q_out f32, K row Q4_0,
      * V row Q4_0 (the caller applies the position as byte offsets, as the reference does).
      * max_seq > 0: a 7th input meta f32[4] carries the position in [3]; rope is then the
-     * whole table f32[max_seq, hd] and the outputs are the cache bases. */
+     * whole table f32[max_seq, hd] and the outputs are the cache bases.
+     * dims[5] = slots > 0 (tokens of different sequences): meta is f32[n_tok][4] with token i's position in
+     * [4 i + 3], an 8th input f32[n_tok] names token i's slot, the outputs are caches of dims[5] slots
+     * ([slot][max_seq, n_kv, hd]; dims[6] = byte distance between slots, 0: max_seq rows). */
     KSH_RMSNORM_PER_HEAD_QKV_Q40 = 12,
     /* CopyScaleIndexed: out[i] = scale * deq(src[id*n + i]); id is read from a
      * device f32 (the reference keeps token ids as f32).  dims: n, rows in the table, n_tok (> 1:
@@ -171,7 +177,9 @@ enum ksh_kind {
      * cos[0..hd/2) || sin[0..hd/2).  The query heads of layers that reuse another layer's KV cache, and the
      * per-layer-embedding prepass.  y may be x.
      * dims: n_heads, hd (64 | 128 | 256 | 512), rope (0 none; 1 the row, placed with a byte offset; 2 the whole
-     *       table, row = position in meta[3]), max_seq (rope = 2)
+     *       table, row = position in meta[3]), max_seq (rope = 2), heads per token (rope = 2, > 0: the heads of
+     *       several tokens, token after token; token i is at position meta[3] + i), per-token records (1: tokens of
+     *       different sequences, meta is f32[n_tok][4] with token i's position in [4 i + 3])
      * params: eps.   in: x, w f32[hd] [, rope [, meta f32[4]]]   out: y */
     KSH_RMSNORM_PER_HEAD = 25,
     /* Eng::add_scale (crates/ksearch_kernels/src/lib.rs:918-937): y = scale * (a + b).
@@ -448,6 +456,12 @@ int ksh_kvpool_bump_len_by(ksh_kvpool *p, int slot, int n, int *new_len);
 int ksh_kvpool_active_batch(const ksh_kvpool *p, int *slots, int cap);   /* returns the count */
 ksh_buf *ksh_kvpool_k(const ksh_kvpool *p, int slot, int layer);
 ksh_buf *ksh_kvpool_v(const ksh_kvpool *p, int slot, int layer);
+/* A layer's K (V) caches of all slots are one allocation, [max_batch][max_seq * n_kv * (hd/32) * 18]; the per-slot
+ * buffers above are views into it.  These return the whole allocation, which a pass over several slots' tokens
+ * addresses by slot index (KSH_SDPA_SLOTS with dims[6], KSH_RMSNORM_PER_HEAD_QKV_Q40 with dims[5]).  No counterpart
+ * in kv_pool.rs, whose slots are separate buffers (its decode rounds are serial). */
+ksh_buf *ksh_kvpool_layer_k(const ksh_kvpool *p, int layer);
+ksh_buf *ksh_kvpool_layer_v(const ksh_kvpool *p, int layer);
 int ksh_kvpool_dims(const ksh_kvpool *p, int *max_batch, int *max_seq, int *n_kv_layers, int *hd, int *n_kv);
 /* GemmaPrimModel::bind_slot (gemma_prim.rs:1277-1292): the model's caches become the slot's (the pool needs one
  * layer per cache-owning layer and hd >= the larger head dim) and its position the slot's sequence length; the
@@ -471,6 +485,18 @@ int ksh_gemma4_decode_token_sampled(ksh_gemma4 *m, uint32_t token, float tempera
  * decode step.  use_graph & 1: decode steps replay the captured graph; use_graph & 2: every token goes through the
  * decode step (no batching).  ksh_gemma4_generate / _generate_until feed the prompt through this with the same flags. */
 int ksh_gemma4_prefill_chunk(ksh_gemma4 *m, const uint32_t *tokens, int n, int use_graph);
+/* One decode step for n (1 to 16) sequences at once: the scheduler's decode round (crates/ksearch_cli/src/scheduler.rs:
+ * 163-231, there one decode_token_sampled per request) as ONE pass over the weights.  Row i feeds tokens[i] to the
+ * sequence in pool slot slots[i] at that slot's sequence length: its K / V row is appended there and it attends that
+ * slot's rows.  next_ids[i] is the greedy id, or, where temperature (may be NULL: all greedy) gives
+ * temperature[i] >= 1e-6, the draw of ksh_sample_softcap_min_p on row i's logits with min_p[i] and seed[i].  The
+ * caller bumps the slots' lengths afterwards (ksh_kvpool_bump_len_by), as after a serial step.  The model's own
+ * position and binding are not touched; ksh_gemma4_bind_slot re-seeks a bound slot whose length has moved.
+ * Slots must be occupied and distinct. */
+int ksh_gemma4_decode_round(ksh_gemma4 *m, ksh_kvpool *pool, const int32_t *slots, const uint32_t *tokens, int n,
+                            const float *temperature, const float *min_p, const uint32_t *seed, uint32_t *next_ids);
+/* f32 [n][vocab]: the logits of the last round's rows */
+ksh_buf *ksh_gemma4_round_logits(ksh_gemma4 *m);
 
 /* ---- decode-before-prefill slot scheduler: spawn_scheduler and its rounds (crates/ksearch_cli/src/scheduler.rs:
  * 78-349) as a tick the host drives.  One tick = admit waiting requests into free slots (alloc + clear), one
@@ -489,6 +515,9 @@ typedef struct {
     int32_t prefill_tokens_per_tick;   /* 2048 */
     uint32_t eos[2];                   /* EOS_IDS (scheduler.rs:14): 1, 106 */
     int32_t use_graph;                 /* replay the model's HIP graphs (1) or launch eagerly (0) */
+    int32_t batched_decode;            /* from this many decoding requests on (>= 2; default 4) they take their step as one
+                                        * ksh_gemma4_decode_round (the weights are read once per round); 0: always one
+                                        * by one, as the reference does */
     ksh_serve_stop_fn stop;            /* may be NULL */
     void *stop_user;
 } ksh_serve_cfg;

@@ -134,6 +134,10 @@ struct ksh_gemma4 {
     ksh_buf *c_tok = nullptr, *c_x = nullptr, *c_x2 = nullptr, *c_y = nullptr, *c_q = nullptr, *c_k = nullptr, *c_v = nullptr, *c_o = nullptr,
             *c_g = nullptr, *c_u = nullptr, *c_ff = nullptr, *c_tmp = nullptr, *c_meta_full = nullptr, *c_meta_swa = nullptr,
             *c_ple_tok = nullptr, *c_ple_tmp = nullptr, *c_ple_ctx = nullptr, *c_ple_u = nullptr;
+    // decode rounds over several KV slots (allocated at the first round): the per-token table (ids, slots, attended
+    // ranges of the two layer kinds), the logits of every token of the round, the greedy ids
+    ksh_buf *r_tab = nullptr, *r_logits = nullptr, *r_next = nullptr;
+    int r_count = 0;
 };
 
 namespace {
@@ -877,6 +881,191 @@ int ksh_gemma4_prefill_chunk(ksh_gemma4 *m, const uint32_t *tokens, int n, int u
     }
     return ksh_synchronize(m->ctx);
 }
+
+}  // extern "C"
+
+// One decode step for several sequences at once: the reference's decode round (crates/ksearch_cli/src/scheduler.rs:
+// 163-231) runs decode_token_sampled once per decoding request, each a full pass over the weights; here the round's
+// tokens go through the layers together as a matrix of n rows (the batched layer pass of forward_prefill_chunk,
+// gemma_prim.rs:1317-1607, with one position, one attended range and one KV slot per row), so the weights are read
+// once per round.  Row i appends to and attends the caches of pool slot slots[i] at that slot's sequence length.
+namespace {
+constexpr int kRoundMax = 16;         // the attention launch shares its partitions among up to 16 entries by length
+constexpr int kRoundPartitions = 16;
+constexpr int kRoundStride = 16;      // floats per field of the table: ids | slots | full-attention records | sliding-window records
+
+int pool_fits(const ksh_gemma4 *m, const ksh_kvpool *pool, int *max_batch, int *pool_hd)
+{
+    const ksh_gemma4_cfg &c = m->c;
+    int max_seq, n_kv_layers, n_kv;
+    if (ksh_kvpool_dims(pool, max_batch, &max_seq, &n_kv_layers, pool_hd, &n_kv)) return 1;
+    const int owners = c.n_layers - c.shared_kv_layers;
+    if (n_kv_layers != owners) return set_error("kv layer mismatch: model=%d pool=%d", owners, n_kv_layers);
+    if (max_seq != c.max_seq || n_kv != c.n_kv || *pool_hd < std::max(c.hd_swa, c.hd_full))
+        return set_error("KvPool(max_seq=%d, n_kv=%d, hd=%d) does not fit the model (max_seq=%d, n_kv=%d, hd=%d)", max_seq, n_kv, *pool_hd,
+                         c.max_seq, c.n_kv, std::max(c.hd_swa, c.hd_full));
+    return 0;
+}
+
+int forward_decode_round4(ksh_gemma4 *m, ksh_kvpool *pool, const int32_t *slots, const uint32_t *tokens, int t)
+{
+    const ksh_gemma4_cfg &c = m->c;
+    int max_batch = 0, pool_hd = 0;
+    if (pool_fits(m, pool, &max_batch, &pool_hd)) return 1;
+    if (chunk_buffers4(m)) return 1;
+    if (!m->r_tab && (alloc(m, (size_t)kRoundStride * 10 * 4, &m->r_tab) || alloc(m, (size_t)kRoundMax * c.vocab * 4, &m->r_logits) ||
+                      alloc(m, (size_t)kRoundMax * 4, &m->r_next)))
+        return 1;
+    float tab[kRoundStride * 10] = {};
+    for (int i = 0; i < t; i++) {
+        const int pos = ksh_kvpool_seq_len(pool, slots[i]);
+        const int kv_len = pos + 1, start = kv_len > c.sliding_window ? kv_len - c.sliding_window : 0;
+        tab[i] = (float)tokens[i];
+        tab[kRoundStride + i] = (float)slots[i];
+        float *full = tab + 2 * kRoundStride + 4 * i, *swa = tab + 6 * kRoundStride + 4 * i;
+        full[0] = (float)kv_len; full[3] = (float)pos;
+        swa[0] = (float)(kv_len - start); swa[1] = (float)start; swa[2] = (float)c.sliding_window; swa[3] = (float)pos;
+    }
+    if (ksh_synchronize(m->ctx)) return 1;   // the table may still be read by the previous round
+    if (ksh_buffer_write(m->ctx, m->r_tab, 0, tab, sizeof(tab), 1)) return 1;
+    const size_t o_ids = 0, o_slots = (size_t)kRoundStride * 4, o_full = (size_t)2 * kRoundStride * 4, o_swa = (size_t)6 * kRoundStride * 4;
+    const int64_t h = c.hidden, tp = 32, pt = (int64_t)c.n_layers * c.ple_dim;
+    const size_t slot_stride = (size_t)c.max_seq * c.n_kv * (pool_hd / 32) * 18;
+    int n = 0;
+    ksh_kernel *k = nullptr, *k_norm = nullptr, *k_add = nullptr, *k_add_then = nullptr;
+    auto run = [&](ksh_kernel *kk, std::initializer_list<ksh_buf *> in, std::initializer_list<size_t> in_off, std::initializer_list<ksh_buf *> out,
+                   std::initializer_list<size_t> out_off) {
+        ksh_buf *ib[kMaxIn], *ob[kMaxOut];
+        uint64_t io[kMaxIn] = {}, oo[kMaxOut] = {};
+        int ni = 0, no = 0, j = 0;
+        for (ksh_buf *b : in) ib[ni++] = b;
+        for (size_t o : in_off) io[j++] = o;
+        j = 0;
+        for (ksh_buf *b : out) ob[no++] = b;
+        for (size_t o : out_off) oo[j++] = o;
+        n += 1;
+        return ksh_encode(m->ctx, kk, ib, io, ni, ob, oo, no);
+    };
+    // Q4_K matrices: the small-batch GEMM on exact integer codes (the GEMV's accuracy).  Q6_K matrices (files loaded
+    // with their Q6_K tensors kept): the GEMM's f16 operand rounds sc * q above 2048 to even integers, 2^-11 on those
+    // weights, which a step that must equal the serial one to 1e-3 through every layer cannot afford: row by row
+    // through the GEMV instead.
+    auto mm = [&](int dt, int64_t rows, int64_t cols, ksh_buf *w, ksh_buf *x, ksh_buf *y) -> int {
+        ksh_kernel *kk = nullptr;
+        if (dt != KSH_Q6K) return get(m, KSH_MATVEC_BATCH, {rows, cols, tp}, {dt, KSH_F32, KSH_F32}, {}, &kk) || enc(m, kk, {w, x}, {y}, n);
+        if (get(m, KSH_MATVEC, {rows, cols}, {dt, KSH_F32}, {}, &kk)) return 1;
+        for (int i = 0; i < t; i++)
+            if (run(kk, {w, x}, {0, (size_t)i * cols * 4}, {y}, {(size_t)i * rows * 4})) return 1;
+        return 0;
+    };
+    if (get(m, KSH_COPY_SCALE_INDEXED, {h, c.vocab, t}, {m->g.dt_embd}, {std::sqrt((float)c.hidden)}, &k) ||
+        run(k, {m->g.token_embd, m->r_tab}, {0, o_ids}, {m->c_x}, {0}))
+        return 1;
+    if (c.ple_dim > 0) {
+        ksh_kernel *kg = nullptr, *kn = nullptr, *kmix = nullptr;
+        if (get(m, KSH_COPY_SCALE_INDEXED, {pt, c.vocab, t}, {m->g.dt_ple}, {std::sqrt((float)c.ple_dim)}, &kg) ||
+            run(kg, {m->g.ple_embd, m->r_tab}, {0, o_ids}, {m->c_ple_tok}, {0}) ||
+            mm(m->g.dt_ple_proj, pt, h, m->g.ple_model_proj, m->c_x, m->c_ple_tmp) ||
+            get(m, KSH_RMSNORM_PER_HEAD, {(int64_t)t * c.n_layers, c.ple_dim, 0}, {}, {c.eps}, &kn) ||
+            enc(m, kn, {m->c_ple_tmp, m->g.ple_proj_norm}, {m->c_ple_ctx}, n) ||
+            get(m, KSH_ADD_SCALE, {(int64_t)t * pt}, {}, {0.70710678118654752440f}, &kmix) ||
+            enc(m, kmix, {m->c_ple_ctx, m->c_ple_tok}, {m->c_ple_ctx}, n))
+            return 1;
+    }
+    if (get(m, KSH_RMSNORM, {h, 0, 0, t}, {}, {c.eps}, &k_norm) || get(m, KSH_RMSNORM, {h, 1, 0, t}, {}, {c.eps}, &k_add) ||
+        get(m, KSH_RMSNORM_ADD_THEN_RMSNORM, {h, t}, {}, {c.eps}, &k_add_then))
+        return 1;
+    for (int l = 0; l < c.n_layers; l++) {
+        const ksh_gemma4_layer &L = m->layers[l];
+        const LayerPlan &P = m->plan[l];
+        ksh_buf *rope_tab = P.swa ? m->rope_swa : m->rope_full;
+        ksh_buf *kc = ksh_kvpool_layer_k(pool, P.src), *vc = ksh_kvpool_layer_v(pool, P.src);
+        const size_t o_meta = P.swa ? o_swa : o_full;
+        ksh_kernel *k_head = nullptr, *k_sdpa = nullptr, *k_gelu = nullptr;
+        if (!sdpa_lanes_supports(c.n_q, c.n_kv, P.hd))
+            return set_error("ksh_gemma4_decode_round: attention over several slots is built for heads of 128 / 256 / 512 with up to 8 q heads per kv head");
+        if (enc(m, k_norm, {m->c_x, L.attn_norm}, {m->c_x2}, n) || mm(L.dt_q, P.qd, h, L.wq, m->c_x2, m->c_q)) return 1;
+        if (P.owns) {
+            if (mm(L.dt_k, P.kvd, h, L.wk, m->c_x2, m->c_k) || mm(L.dt_v, P.kvd, h, L.wv, m->c_x2, m->c_v) ||
+                get(m, KSH_RMSNORM_PER_HEAD_QKV_Q40, {c.n_q, c.n_kv, P.hd, c.max_seq, t, max_batch, (int64_t)slot_stride}, {}, {c.eps}, &k_head) ||
+                run(k_head, {m->c_q, L.q_norm, rope_tab, m->c_k, L.k_norm, m->c_v, m->r_tab, m->r_tab}, {0, 0, 0, 0, 0, 0, o_meta, o_slots},
+                    {m->c_q, kc, vc}, {0, 0, 0}))
+                return 1;
+        } else {
+            if (get(m, KSH_RMSNORM_PER_HEAD, {(int64_t)t * c.n_q, P.hd, 2, c.max_seq, c.n_q, 1}, {}, {c.eps}, &k_head) ||
+                run(k_head, {m->c_q, L.q_norm, rope_tab, m->r_tab}, {0, 0, 0, o_meta}, {m->c_q}, {0}))
+                return 1;
+        }
+        if (get(m, KSH_SDPA_SLOTS, {c.n_q, c.n_kv, P.hd, c.max_seq, t, kRoundPartitions, max_batch, (int64_t)slot_stride}, {KSH_Q40, KSH_F32},
+                {c.attn_scale}, &k_sdpa) ||
+            run(k_sdpa, {m->c_q, kc, vc, m->r_tab, m->r_tab}, {0, 0, 0, o_meta, o_slots}, {m->c_tmp, m->c_o}, {0, 0}) ||
+            mm(L.dt_o, h, P.qd, L.wo, m->c_o, m->c_y) ||
+            enc(m, k_add_then, {m->c_y, L.post_attn_norm, m->c_x, L.ffn_norm}, {m->c_x, m->c_x2}, n) ||
+            mm(L.dt_gate, L.ffn, h, L.wgate, m->c_x2, m->c_g) || mm(L.dt_up, L.ffn, h, L.wup, m->c_x2, m->c_u) ||
+            get(m, KSH_GELU_MUL, {(int64_t)t * L.ffn}, {}, {}, &k_gelu) || enc(m, k_gelu, {m->c_g, m->c_u}, {m->c_ff}, n) ||
+            mm(L.dt_down, h, L.ffn, L.wdown, m->c_ff, m->c_y) || enc(m, k_add, {m->c_y, L.post_ffw_norm, m->c_x}, {m->c_x}, n))
+            return 1;
+        if (c.ple_dim > 0) {
+            ksh_kernel *k_gs = nullptr, *k_as = nullptr;
+            if (mm(L.dt_inp_gate, c.ple_dim, h, L.inp_gate, m->c_x, m->c_ple_u) ||
+                get(m, KSH_GELU_MUL, {(int64_t)t * c.ple_dim, c.ple_dim, pt}, {}, {}, &k_gs) ||
+                enc_off(m, k_gs, {m->c_ple_u, m->c_ple_ctx}, {0, (size_t)l * c.ple_dim * 4}, {m->c_ple_u}, n) ||
+                mm(L.dt_proj, h, c.ple_dim, L.proj, m->c_ple_u, m->c_y) ||
+                get(m, KSH_RMSNORM, {h, 1, 1, t}, {}, {c.eps, L.layer_scale}, &k_as) ||
+                enc(m, k_as, {m->c_y, L.post_norm, m->c_x}, {m->c_x}, n))
+                return 1;
+        }
+    }
+    // logits and the greedy id of every row: the output norm rides in the LM head's prologue, as in the decode step
+    ksh_buf *lm_w = m->embd_rows ? m->embd_rows : m->g.token_embd;
+    for (int i = 0; i < t; i++)
+        if (run(m->k_lm_head[0], {lm_w, m->c_x, m->g.output_norm}, {0, (size_t)i * h * 4, 0}, {m->r_logits}, {(size_t)i * c.vocab * 4}) ||
+            run(m->k_argmax, {m->r_logits}, {(size_t)i * c.vocab * 4}, {m->r_next}, {(size_t)i * 4}))
+            return 1;
+    m->r_count = t;
+    return 0;
+}
+}  // namespace
+
+extern "C" {
+
+int ksh_gemma4_decode_round(ksh_gemma4 *m, ksh_kvpool *pool, const int32_t *slots, const uint32_t *tokens, int n, const float *temperature,
+                            const float *min_p, const uint32_t *seed, uint32_t *next_ids)
+{
+    if (!m || !pool || !slots || !tokens || !next_ids) return set_error("ksh_gemma4_decode_round: bad arguments");
+    if (n < 1 || n > kRoundMax) return set_error("ksh_gemma4_decode_round: %d sequences (1 to %d at once)", n, kRoundMax);
+    if (temperature && (!min_p || !seed)) return set_error("ksh_gemma4_decode_round: sampling needs min_p and seed");
+    int max_batch = 0, pool_hd = 0;
+    if (pool_fits(m, pool, &max_batch, &pool_hd)) return 1;
+    for (int i = 0; i < n; i++) {
+        if (slots[i] < 0 || slots[i] >= max_batch) return set_error("bad SlotId");
+        if (ksh_kvpool_occupied(pool, slots[i]) != 1) return set_error("slot not occupied");
+        for (int j = 0; j < i; j++)
+            if (slots[j] == slots[i]) return set_error("ksh_gemma4_decode_round: slot %d is named twice", slots[i]);
+        if (ksh_kvpool_seq_len(pool, slots[i]) >= m->c.max_seq) return set_error("max_seq exceeded");   // gemma_prim.rs:882-884
+        if (tokens[i] >= (uint32_t)m->c.vocab) return set_error("token id %u is outside the vocabulary", tokens[i]);
+    }
+    if (forward_decode_round4(m, pool, slots, tokens, n)) return 1;
+    float ids[kRoundMax];
+    if (ksh_buffer_read(m->ctx, m->r_next, 0, ids, (size_t)n * 4, 1)) return 1;
+    for (int i = 0; i < n; i++) {
+        next_ids[i] = (uint32_t)ids[i];
+        if (temperature && temperature[i] >= 1e-6f) {   // decode_token_sampled's other branch (gemma_prim.rs:1614-1635)
+            std::vector<float> &logits = m->host_logits;
+            logits.resize((size_t)m->c.vocab);
+            if (ksh_buffer_read(m->ctx, m->r_logits, (size_t)i * m->c.vocab * 4, logits.data(), logits.size() * 4, 0) ||
+                ksh_sample_softcap_min_p(logits.data(), logits.size(), m->c.softcap, temperature[i], min_p[i], seed[i], &next_ids[i]))
+                return 1;
+        }
+    }
+    return 0;
+}
+
+ksh_buf *ksh_gemma4_round_logits(ksh_gemma4 *m) { return m ? m->r_logits : nullptr; }
+
+}  // extern "C"
+
+extern "C" {
 
 // GemmaPrimModel::bind_slot (gemma_prim.rs:1277-1292): the model's K / V caches become the slot's and its position the
 // slot's sequence length.  pool == NULL goes back to the model's own caches at position `slot` (0 after a reset).

@@ -111,7 +111,7 @@ __global__ __launch_bounds__(64) void per_head_qkv_q40_kernel(
     const float *q, const float *__restrict__ qw, const float *__restrict__ rope,
     const float *__restrict__ k, const float *__restrict__ kw, const float *__restrict__ v,
     float *q_out, uint8_t *k_out, uint8_t *v_out, int n_q, int n_kv, float eps, const float *meta,
-    int max_seq)
+    int max_seq, const float *slot_ids, size_t slot_stride)
 {
     constexpr int HALF = HD / 2, PER = HD / 64;   // elements per lane
     const int lane = threadIdx.x;
@@ -122,7 +122,17 @@ __global__ __launch_bounds__(64) void per_head_qkv_q40_kernel(
     k += (size_t)tok * n_kv * HD;
     v += (size_t)tok * n_kv * HD;
     q_out += (size_t)tok * n_q * HD;
-    if (meta) {
+    if (slot_ids) {
+        // tokens of different sequences (one decode step for several KV slots): token i has its own record
+        // meta[4 i .. ] with its position in [3], and appends to slot slot_ids[i] of caches laid out
+        // [slot][max_seq, n_kv, hd]
+        const size_t pos = (size_t)min(max((int)meta[4 * tok + 3], 0), max_seq - 1);
+        const size_t slot_bytes = slot_stride ? slot_stride : (size_t)max_seq * n_kv * (HD / 32) * 18;
+        const size_t slot = (size_t)max((int)slot_ids[tok], 0);
+        rope += pos * HD;
+        k_out += slot * slot_bytes + pos * (size_t)n_kv * (HD / 32) * 18;
+        v_out += slot * slot_bytes + pos * (size_t)n_kv * (HD / 32) * 18;
+    } else if (meta) {
         // position kept on the device (meta[3]): the rope input is the whole
         // table and the K/V outputs are the cache bases, so that one captured
         // graph serves every token
@@ -376,7 +386,8 @@ int launch_per_head(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
                        (const float *)a.in[1], (const float *)a.in[2], (const float *)a.in[3],               \
                        (const float *)a.in[4], (const float *)a.in[5], (float *)a.out[0], (uint8_t *)a.out[1], \
                        (uint8_t *)a.out[2], n_q, n_kv, k.desc.params[0],                                      \
-                       k.desc.dims[3] ? (const float *)a.in[6] : nullptr, (int)k.desc.dims[3])
+                       k.desc.dims[3] ? (const float *)a.in[6] : nullptr, (int)k.desc.dims[3],                \
+                       k.desc.dims[5] ? (const float *)a.in[7] : nullptr, (size_t)k.desc.dims[6])
     switch (hd) {
     case 128: KSH_PH(128); break;
     case 256: KSH_PH(256); break;
@@ -539,16 +550,25 @@ int bind_per_head_qkv_q40(ksh_kernel &k)
     const int64_t n_tok = k.desc.dims[4] ? k.desc.dims[4] : 1;
     if (n_tok < 0 || n_tok > 65535) return set_error("rmsnorm_per_head_qkv_q40: n_tok=%lld", (long long)n_tok);
     const size_t rows = max_seq ? (size_t)max_seq : (size_t)n_tok;
-    k.info.n_inputs = max_seq ? 7 : 6;
+    // dims[5] = KV slots when the tokens belong to different sequences: meta is then f32[n_tok][4] (token i's position
+    // in [4 i + 3]), an 8th input f32[n_tok] names each token's slot, and the outputs are caches of dims[5] slots
+    const int64_t n_slots = k.desc.dims[5];
+    if (n_slots < 0 || n_slots > 4096 || (n_slots && !max_seq)) return set_error("rmsnorm_per_head_qkv_q40: slots=%lld", (long long)n_slots);
+    k.info.n_inputs = n_slots ? 8 : max_seq ? 7 : 6;
     k.info.n_outputs = 3;
-    const size_t kvb = (size_t)n_kv * (hd / 32) * 18 * rows;
-    const size_t ib[7] = {(size_t)n_q * hd * 4 * n_tok, (size_t)hd * 4, (size_t)hd * 4 * rows, (size_t)n_kv * hd * 4 * n_tok, (size_t)hd * 4,
-                          (size_t)n_kv * hd * 4 * n_tok, 16};
+    // dims[6] = bytes from one slot of the caches to the next (0: max_seq rows)
+    const size_t one = (size_t)n_kv * (hd / 32) * 18 * rows;
+    const int64_t slot_stride = k.desc.dims[6];
+    if (slot_stride < 0 || (slot_stride && (!n_slots || (size_t)slot_stride < one || slot_stride % 2)))
+        return set_error("rmsnorm_per_head_qkv_q40: slot stride %lld", (long long)slot_stride);
+    const size_t kvb = n_slots ? (size_t)(n_slots - 1) * (slot_stride ? (size_t)slot_stride : one) + one : one;
+    const size_t ib[8] = {(size_t)n_q * hd * 4 * n_tok, (size_t)hd * 4, (size_t)hd * 4 * rows, (size_t)n_kv * hd * 4 * n_tok, (size_t)hd * 4,
+                          (size_t)n_kv * hd * 4 * n_tok, n_slots ? (size_t)16 * n_tok : 16, (size_t)4 * n_tok};
     for (int i = 0; i < k.info.n_inputs; i++) { k.in_bytes[i] = ib[i]; k.in_align[i] = 4; }
     k.out_bytes[0] = (size_t)n_q * hd * 4 * n_tok; k.out_align[0] = 4;
     k.out_bytes[1] = k.out_bytes[2] = kvb; k.out_align[1] = k.out_align[2] = 2;
     set_launch(k, (uint32_t)(n_q + n_kv), (uint32_t)n_tok, 1, 64, 0);
-    set_name(k, "rmsnorm_per_head_qkv_q40_hd%d%s", (int)hd, n_tok > 1 ? "_batch" : "");
+    set_name(k, "rmsnorm_per_head_qkv_q40_hd%d%s", (int)hd, n_slots ? "_slots" : n_tok > 1 ? "_batch" : "");
     k.launch = launch_per_head;
     return 0;
 }

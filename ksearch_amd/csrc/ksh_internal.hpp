@@ -39,6 +39,7 @@ struct ksh_buf {
     void *ptr = nullptr;
     size_t bytes = 0;
     std::atomic<int> rc{1};
+    ksh_buf *parent = nullptr;   // a view: ptr lies inside the parent's allocation, which the view keeps alive
 };
 
 struct ksh_kernel {
@@ -60,6 +61,8 @@ struct ksh_kernel {
 namespace ksh {
 // what entry points outside the runtime's translation unit need of a context
 hipStream_t ctx_stream(ksh_ctx *ctx);
+// a buffer object over bytes [off, off + bytes) of `parent` (retained until the view is released); nullptr + error when out of range
+ksh_buf *buffer_view(ksh_buf *parent, size_t off, size_t bytes);
 void ctx_mark_pending(ksh_ctx *ctx);
 // resolves the device address of the static partial-result array of ksh_softcap_argmax_static for the current
 // device (called when a context is created; the entry point does it itself for a device it has not seen)

@@ -109,6 +109,19 @@ struct ksh_ctx {
 
 namespace ksh {
 hipStream_t ctx_stream(ksh_ctx *ctx) { return ctx->stream; }
+ksh_buf *buffer_view(ksh_buf *parent, size_t off, size_t bytes)
+{
+    if (!parent || off > parent->bytes || bytes > parent->bytes - off) {
+        set_error("buffer_view: range [%zu, %zu) is outside the buffer", off, off + bytes);
+        return nullptr;
+    }
+    ksh_buf *v = new ksh_buf();
+    v->ptr = (char *)parent->ptr + off;
+    v->bytes = bytes;
+    v->parent = parent;
+    ksh_buffer_retain(parent);
+    return v;
+}
 void ctx_mark_pending(ksh_ctx *ctx) { ctx->pending = true; }
 }  // namespace ksh
 
@@ -199,7 +212,10 @@ void ksh_buffer_retain(ksh_buf *buf)
 void ksh_buffer_release(ksh_buf *buf)
 {
     if (buf && buf->rc.fetch_sub(1) == 1) {
-        (void)hipFree(buf->ptr);
+        if (buf->parent)
+            ksh_buffer_release(buf->parent);
+        else
+            (void)hipFree(buf->ptr);
         delete buf;
     }
 }

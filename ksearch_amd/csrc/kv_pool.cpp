@@ -17,11 +17,17 @@ struct ksh_kvpool {
     int max_batch = 0, max_seq = 0, n_kv_layers = 0, hd = 0, n_kv = 0;
     std::vector<char> occupied;
     std::vector<int> seq_len;
-    std::vector<ksh_buf *> k, v;   // [slot][layer]
+    // One allocation per layer and cache, [slot][max_seq * n_kv * (hd / 32) * 18]: a slot's cache is a view into it
+    // (what a model is bound to), and a pass over several slots' tokens addresses all of them from one base.
+    std::vector<ksh_buf *> layer_k, layer_v;   // [layer]
+    std::vector<ksh_buf *> k, v;               // [slot][layer] views
+    size_t slot_bytes = 0;
     ~ksh_kvpool()
     {
         for (ksh_buf *b : k) ksh_buffer_release(b);
         for (ksh_buf *b : v) ksh_buffer_release(b);
+        for (ksh_buf *b : layer_k) ksh_buffer_release(b);
+        for (ksh_buf *b : layer_v) ksh_buffer_release(b);
     }
 };
 
@@ -47,13 +53,21 @@ int ksh_kvpool_create(ksh_ctx *ctx, int max_batch, int max_seq, int n_kv_layers,
     p->occupied.assign((size_t)max_batch, 0);
     p->seq_len.assign((size_t)max_batch, 0);
     const size_t bytes = (size_t)max_seq * n_kv * (hd / 32) * 18;   // q40_nbytes, crates/ksearch_ir/src/lib.rs:52-59
-    for (int i = 0; i < max_batch * n_kv_layers; i++) {
+    p->slot_bytes = bytes;
+    for (int l = 0; l < n_kv_layers; l++) {
         ksh_buf *kb = nullptr, *vb = nullptr;
-        if (ksh_buffer_alloc(ctx, bytes, nullptr, &kb)) return 1;
-        p->k.push_back(kb);
-        if (ksh_buffer_alloc(ctx, bytes, nullptr, &vb)) return 1;
-        p->v.push_back(vb);
+        if (ksh_buffer_alloc(ctx, bytes * max_batch, nullptr, &kb)) return 1;
+        p->layer_k.push_back(kb);
+        if (ksh_buffer_alloc(ctx, bytes * max_batch, nullptr, &vb)) return 1;
+        p->layer_v.push_back(vb);
     }
+    for (int s = 0; s < max_batch; s++)
+        for (int l = 0; l < n_kv_layers; l++) {
+            ksh_buf *kb = buffer_view(p->layer_k[(size_t)l], (size_t)s * bytes, bytes), *vb = buffer_view(p->layer_v[(size_t)l], (size_t)s * bytes, bytes);
+            if (kb) p->k.push_back(kb);
+            if (vb) p->v.push_back(vb);
+            if (!kb || !vb) return 1;
+        }
     *out = p.release();
     return 0;
 }
@@ -131,6 +145,9 @@ ksh_buf *ksh_kvpool_v(const ksh_kvpool *p, int slot, int layer)
 {
     return bad_slot(p, slot) || layer < 0 || layer >= p->n_kv_layers ? nullptr : p->v[(size_t)slot * p->n_kv_layers + layer];
 }
+
+ksh_buf *ksh_kvpool_layer_k(const ksh_kvpool *p, int layer) { return !p || layer < 0 || layer >= p->n_kv_layers ? nullptr : p->layer_k[(size_t)layer]; }
+ksh_buf *ksh_kvpool_layer_v(const ksh_kvpool *p, int layer) { return !p || layer < 0 || layer >= p->n_kv_layers ? nullptr : p->layer_v[(size_t)layer]; }
 
 int ksh_kvpool_dims(const ksh_kvpool *p, int *max_batch, int *max_seq, int *n_kv_layers, int *hd, int *n_kv)
 {

@@ -29,7 +29,7 @@ int done(const char *what)
 template <int HD>
 __global__ __launch_bounds__(64) void per_head_kernel(const float *x, const float *__restrict__ w,
                                                       const float *__restrict__ rope, const float *__restrict__ meta,
-                                                      float *y, float eps, int max_seq, int heads_per_token)
+                                                      float *y, float eps, int max_seq, int heads_per_token, int per_token_meta)
 {
     constexpr int HALF = HD / 2, PER = HD / 64;
     const int lane = threadIdx.x;
@@ -37,7 +37,8 @@ __global__ __launch_bounds__(64) void per_head_kernel(const float *x, const floa
     // heads_per_token > 0 (rmsnorm_per_head_rope_batch, gemma_prim.rs:1411-1424): the heads of a chunk of consecutive
     // positions, token after token; token i takes the rope row of (first position + i)
     const int tok = heads_per_token > 0 ? blockIdx.x / heads_per_token : 0;
-    if (meta) rope += (size_t)min(max((int)meta[3] + tok, 0), max_seq - 1) * HD;
+    // per_token_meta: the tokens belong to different sequences, token i's position is meta[4 i + 3]
+    if (meta) rope += (size_t)min(max(per_token_meta ? (int)meta[4 * tok + 3] : (int)meta[3] + tok, 0), max_seq - 1) * HD;
     float xv[PER], nv[PER];
     float ss = 0.f;
 #pragma unroll
@@ -185,7 +186,7 @@ int launch_per_head(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
     const float *meta = mode == 2 ? (const float *)a.in[3] : nullptr;
 #define KSH_PH(HD)                                                                                                  \
     hipLaunchKernelGGL((per_head_kernel<HD>), dim3(n_heads), dim3(64), 0, st, (const float *)a.in[0],               \
-                       (const float *)a.in[1], rope, meta, (float *)a.out[0], k.desc.params[0], (int)k.desc.dims[3], (int)k.desc.dims[4])
+                       (const float *)a.in[1], rope, meta, (float *)a.out[0], k.desc.params[0], (int)k.desc.dims[3], (int)k.desc.dims[4], (int)k.desc.dims[5])
     switch (hd) {
     case 64: KSH_PH(64); break;
     case 128: KSH_PH(128); break;
@@ -239,7 +240,9 @@ int bind_ple_ops(ksh_kernel &k)
         k.in_bytes[0] = k.out_bytes[0] = (size_t)n_heads * hd * 4;
         k.in_bytes[1] = (size_t)hd * 4;
         k.in_bytes[2] = (size_t)hd * 4 * (mode == 2 ? (size_t)max_seq : 1);
-        k.in_bytes[3] = 16;
+        // dims[5] = 1: one meta record per token (tokens of different sequences; needs heads per token)
+        if (d[5] < 0 || d[5] > 1 || (d[5] && !d[4])) return set_error("rmsnorm_per_head: dims[5]=%lld (per-token positions need heads per token)", (long long)d[5]);
+        k.in_bytes[3] = d[5] ? (size_t)16 * (n_heads / d[4]) : 16;
         for (int i = 0; i < 4; i++) k.in_align[i] = 4;
         k.out_align[0] = 4;
         set_launch(k, (uint32_t)n_heads, 1, 1, 64, 0);

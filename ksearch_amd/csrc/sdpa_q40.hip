@@ -397,11 +397,22 @@ int bind_sdpa(ksh_kernel &k)
             if (nwg < 1) nwg = 1;
         }
         if (nwg < 0 || nwg > 4096) return set_error("sdpa_slots: nwg=%lld", (long long)nwg);
-        k.info.n_inputs = 4;
+        // dims[6] = slots in the K / V pools when the launch's entries are a subset of them in any order (one decode
+        // step for several sequences): a 5th input f32[n_slots] names each entry's slot
+        const int64_t pool_slots = d[6];
+        if (pool_slots < 0 || pool_slots > 65535) return set_error("sdpa_slots: pool slots=%lld", (long long)pool_slots);
+        // dims[7] = bytes from one slot of the pools to the next (0: max_t rows; a pool sized for wider heads has more)
+        const int64_t slot_stride = d[7];
+        if (slot_stride < 0 || (slot_stride && (!pool_slots || (size_t)slot_stride < kvb || slot_stride % 2)))
+            return set_error("sdpa_slots: slot stride %lld", (long long)slot_stride);
+        if (pool_slots && !lanes) return set_error("sdpa_slots: entries that name their pool slot are built for the register form only (hd 128 / 256 / 512, up to 8 q heads per kv head)");
+        k.info.n_inputs = pool_slots ? 5 : 4;
         k.info.n_outputs = 2;
         k.in_bytes[0] = (size_t)n_slots * n_q * hd * 4;
-        k.in_bytes[1] = k.in_bytes[2] = kvb * (size_t)n_slots;
+        k.in_bytes[1] = k.in_bytes[2] = pool_slots ? (size_t)(pool_slots - 1) * (slot_stride ? (size_t)slot_stride : kvb) + kvb : kvb * (size_t)n_slots;
         k.in_bytes[3] = (size_t)n_slots * 16;
+        k.in_bytes[4] = pool_slots ? (size_t)n_slots * 4 : 0;
+        k.in_align[4] = 4;
         k.out_bytes[0] = (size_t)n_slots * n_q * nwg * (hd + 2) * 4;
         k.out_bytes[1] = (size_t)n_slots * n_q * hd * 4;
         k.out_align[1] = 4;

@@ -45,6 +45,8 @@ struct LaneParams {
     const float *q;          // [n_slots][n_q*hd]; fused: the raw q of the QKV GEMV
     const uint8_t *k, *v;    // [n_slots][max_t*n_kv*row_bytes]
     const float *meta;       // [n_slots][meta_stride]: tlen, start, window(, pos)
+    const float *slot_ids;   // nullptr, or [n_slots]: which slot of the K / V pools entry i attends (entries of a decode round)
+    size_t slot_stride;      // bytes from one slot of the pools to the next; 0: max_t * n_kv * row bytes
     float *tmp;              // [n_slots][n_q][nwg][hd+2]
     float *out;              // [n_slots][n_q*hd]
     uint32_t *counters;      // [n_slots*n_kv], zero between launches
@@ -416,9 +418,10 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
         rec_base = (size_t)first + part;   // flat partition index: values [flat][n_q][HD], then (m, l) [flat][n_q][2]
     }
 
-    const size_t slot_bytes = p.kv_shared ? 0 : (size_t)p.max_t * p.n_kv * ROWB;
-    const uint8_t *kbase = p.k + (size_t)slot * slot_bytes + (size_t)kvh * ROWB + 18 * b;
-    const uint8_t *vbase = p.v + (size_t)slot * slot_bytes + (size_t)kvh * ROWB + 18 * b;
+    const size_t slot_bytes = p.kv_shared ? 0 : p.slot_stride ? p.slot_stride : (size_t)p.max_t * p.n_kv * ROWB;
+    const size_t kv_slot = p.slot_ids ? (size_t)max((int)p.slot_ids[slot], 0) : (size_t)slot;
+    const uint8_t *kbase = p.k + kv_slot * slot_bytes + (size_t)kvh * ROWB + 18 * b;
+    const uint8_t *vbase = p.v + kv_slot * slot_bytes + (size_t)kvh * ROWB + 18 * b;
     const size_t row_stride = (size_t)p.n_kv * ROWB;
     const float *qg = p.q + ((size_t)slot * p.n_q + head0) * HD;
 
@@ -533,7 +536,7 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
         __syncthreads();
         if (owner && hg == 0) {
             // the appended row goes to the cache; the owners attend it from LDS
-            const size_t off = (size_t)slot * slot_bytes + ((size_t)pos * p.n_kv + kvh) * ROWB;
+            const size_t off = kv_slot * slot_bytes + ((size_t)pos * p.n_kv + kvh) * ROWB;
             for (int i = tid; i < ROWB; i += NT) {   // (one pass, except 512-wide heads on four waves)
                 if (i < ROWB / 2)
                     reinterpret_cast<uint16_t *>(p.k_w + off)[i] = reinterpret_cast<const uint16_t *>(newrow)[i];
@@ -849,10 +852,11 @@ __global__ __launch_bounds__(kMfmaWaves * 64, 2) void sdpa_mfma_kernel(LaneParam
         p1 = min(p0 + chunk, tlen);
     }
     start = (int)p.meta[(size_t)slot * p.meta_stride + 1];
-    const size_t slot_bytes = p.kv_shared ? 0 : (size_t)p.max_t * p.n_kv * ROWB;
+    const size_t slot_bytes = p.kv_shared ? 0 : p.slot_stride ? p.slot_stride : (size_t)p.max_t * p.n_kv * ROWB;
     const size_t row_stride = (size_t)p.n_kv * ROWB;
-    const uint8_t *kbase = p.k + (size_t)slot * slot_bytes + (size_t)kvh * ROWB;
-    const uint8_t *vbase = p.v + (size_t)slot * slot_bytes + (size_t)kvh * ROWB;
+    const size_t kv_slot = p.slot_ids ? (size_t)max((int)p.slot_ids[slot], 0) : (size_t)slot;
+    const uint8_t *kbase = p.k + kv_slot * slot_bytes + (size_t)kvh * ROWB;
+    const uint8_t *vbase = p.v + kv_slot * slot_bytes + (size_t)kvh * ROWB;
 
     // ---- the first tile's bytes are requested before anything else (they have the longest way to come)
     constexpr int NPC = (PIECES + 63) / 64;
@@ -1193,6 +1197,10 @@ int launch_bound(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
         p.q = (const float *)a.in[0]; p.k = (const uint8_t *)a.in[1]; p.v = (const uint8_t *)a.in[2];
         p.meta = (const float *)a.in[3];
         p.meta_stride = 4;
+        if (k.desc.dims[6]) {   // entries of a decode round: each names its slot of the pools
+            p.slot_ids = (const float *)a.in[4];
+            p.slot_stride = (size_t)k.desc.dims[7];
+        }
         p.tmp = (float *)a.out[0];
         p.out = (float *)a.out[1];
         p.scale = k.desc.params[0];

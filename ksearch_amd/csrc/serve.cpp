@@ -126,31 +126,69 @@ void admit_waiting(ksh_serve *s)
     }
 }
 
-// scheduler.rs:163-241
+// what follows a decoded token (scheduler.rs:196-231)
+void after_token(ksh_serve *s, Active &a, uint32_t next)
+{
+    a.last_token = next;
+    if (next == s->cfg.eos[0] || next == s->cfg.eos[1]) { finish(s, a, KSH_FINISH_STOP); return; }
+    // the reference decodes the piece and looks for its stop strings here; the host's callback stands in
+    if (s->cfg.stop && s->cfg.stop(s->cfg.stop_user, a.id, next)) { finish(s, a, KSH_FINISH_STOP); return; }
+    a.generated.push_back(next);
+    if (repeating_token(a.generated, 24)) { finish(s, a, KSH_FINISH_STOP); return; }
+    if (a.cancelled) { finish(s, a, KSH_FINISH_CANCELLED); return; }   // (the reference: the receiver is gone)
+    push_event(s, a.id, KSH_SERVE_TOKEN, next, 0, 0, 0);
+    if (a.generated.size() >= a.max_tokens) finish(s, a, KSH_FINISH_LENGTH);
+}
+
+// scheduler.rs:163-241.  The reference runs the round's requests one after the other, each a full pass over the
+// weights; from batched_decode decoding requests on they take the step together (ksh_gemma4_decode_round, up to 16
+// at a time), in the order and with the sampler sequence they would have had one by one.
 void decode_round(ksh_serve *s)
 {
+    std::vector<Active *> ready;
     for (Active &a : s->active) {
         if (a.finished || a.prefill) continue;
         if (a.generated.size() >= a.max_tokens) { finish(s, a, KSH_FINISH_LENGTH); continue; }
         if (std::max(ksh_kvpool_seq_len(s->pool, a.slot), 0) >= s->max_seq) { finish(s, a, KSH_FINISH_LENGTH); continue; }
-        uint32_t next = 0;
         a.rng += 0x9E3779B9u;
-        if (ksh_gemma4_bind_slot(s->model, s->pool, a.slot) ||
-            ksh_gemma4_decode_token_sampled(s->model, a.last_token, a.temperature, a.min_p, a.rng, s->cfg.use_graph, &next) ||
-            ksh_kvpool_bump_len_by(s->pool, a.slot, 1, nullptr)) {
-            push_error(s, a.id, ksh_last_error());
-            finish(s, a, KSH_FINISH_ERROR);
-            continue;
+        ready.push_back(&a);
+    }
+    constexpr size_t kMaxRound = 16;
+    for (size_t i0 = 0; i0 < ready.size();) {
+        const size_t left = ready.size() - i0;
+        const size_t n = s->cfg.batched_decode >= 2 && left >= (size_t)s->cfg.batched_decode ? std::min(left, kMaxRound) : 1;
+        if (n == 1) {
+            Active &a = *ready[i0];
+            uint32_t next = 0;
+            if (ksh_gemma4_bind_slot(s->model, s->pool, a.slot) ||
+                ksh_gemma4_decode_token_sampled(s->model, a.last_token, a.temperature, a.min_p, a.rng, s->cfg.use_graph, &next) ||
+                ksh_kvpool_bump_len_by(s->pool, a.slot, 1, nullptr)) {
+                push_error(s, a.id, ksh_last_error());
+                finish(s, a, KSH_FINISH_ERROR);
+            } else {
+                after_token(s, a, next);
+            }
+        } else {
+            int32_t slots[kMaxRound];
+            uint32_t tokens[kMaxRound], seeds[kMaxRound], next[kMaxRound];
+            float temp[kMaxRound], min_p[kMaxRound];
+            for (size_t i = 0; i < n; i++) {
+                const Active &a = *ready[i0 + i];
+                slots[i] = a.slot; tokens[i] = a.last_token; seeds[i] = a.rng; temp[i] = a.temperature; min_p[i] = a.min_p;
+            }
+            const bool failed = ksh_gemma4_decode_round(s->model, s->pool, slots, tokens, (int)n, temp, min_p, seeds, next) != 0;
+            const std::string why = failed ? ksh_last_error() : "";
+            for (size_t i = 0; i < n; i++) {
+                Active &a = *ready[i0 + i];
+                if (failed || ksh_kvpool_bump_len_by(s->pool, a.slot, 1, nullptr)) {
+                    push_error(s, a.id, failed ? why : ksh_last_error());
+                    finish(s, a, KSH_FINISH_ERROR);
+                } else {
+                    after_token(s, a, next[i]);
+                }
+            }
         }
-        a.last_token = next;
-        if (next == s->cfg.eos[0] || next == s->cfg.eos[1]) { finish(s, a, KSH_FINISH_STOP); continue; }
-        // the reference decodes the piece and looks for its stop strings here; the host's callback stands in
-        if (s->cfg.stop && s->cfg.stop(s->cfg.stop_user, a.id, next)) { finish(s, a, KSH_FINISH_STOP); continue; }
-        a.generated.push_back(next);
-        if (repeating_token(a.generated, 24)) { finish(s, a, KSH_FINISH_STOP); continue; }
-        if (a.cancelled) { finish(s, a, KSH_FINISH_CANCELLED); continue; }   // (the reference: the receiver is gone)
-        push_event(s, a.id, KSH_SERVE_TOKEN, next, 0, 0, 0);
-        if (a.generated.size() >= a.max_tokens) finish(s, a, KSH_FINISH_LENGTH);
+        i0 += n;
     }
 }
 
@@ -208,6 +246,7 @@ int ksh_serve_default_cfg(ksh_serve_cfg *cfg)
     cfg->eos[0] = 1;                       // EOS_IDS, scheduler.rs:14
     cfg->eos[1] = 106;
     cfg->use_graph = 1;
+    cfg->batched_decode = 4;   // a joint step costs about four single ones at the real checkpoints' layer layout
     return 0;
 }
 

@@ -125,7 +125,8 @@ SERVE_STOP_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_uint64, C.c_uint32)
 
 class ServeCfg(C.Structure):
     _fields_ = [("slots", C.c_int32), ("prefill_chunk", C.c_int32), ("prefill_tokens_per_tick", C.c_int32),
-                ("eos", C.c_uint32 * 2), ("use_graph", C.c_int32), ("stop", SERVE_STOP_FN), ("stop_user", C.c_void_p)]
+                ("eos", C.c_uint32 * 2), ("use_graph", C.c_int32), ("batched_decode", C.c_int32), ("stop", SERVE_STOP_FN),
+                ("stop_user", C.c_void_p)]
 
 
 class ServeEvent(C.Structure):
@@ -209,10 +210,15 @@ SYMBOLS = {
     "ksh_kvpool_active_batch": (_i, [_vp, C.POINTER(C.c_int), _i]),
     "ksh_kvpool_k": (_vp, [_vp, _i, _i]),
     "ksh_kvpool_v": (_vp, [_vp, _i, _i]),
+    "ksh_kvpool_layer_k": (_vp, [_vp, _i]),
+    "ksh_kvpool_layer_v": (_vp, [_vp, _i]),
     "ksh_kvpool_dims": (_i, [_vp] + [C.POINTER(C.c_int)] * 5),
     "ksh_gemma4_bind_slot": (_i, [_vp, _vp, _i]),
     "ksh_gemma4_decode_token_sampled": (_i, [_vp, C.c_uint32, C.c_float, C.c_float, C.c_uint32, _i, C.POINTER(C.c_uint32)]),
     "ksh_gemma4_prefill_chunk": (_i, [_vp, C.POINTER(C.c_uint32), _i, _i]),
+    "ksh_gemma4_decode_round": (_i, [_vp, _vp, C.POINTER(C.c_int32), C.POINTER(C.c_uint32), _i, C.POINTER(C.c_float), C.POINTER(C.c_float),
+                                     C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]),
+    "ksh_gemma4_round_logits": (_vp, [_vp]),
     "ksh_serve_default_cfg": (_i, [C.POINTER(ServeCfg)]),
     "ksh_serve_create": (_i, [_vp, _vp, C.POINTER(ServeCfg), _vpp]),
     "ksh_serve_destroy": (None, [_vp]),
@@ -981,6 +987,11 @@ class KvPool:
     def v_buf(self, slot: int, layer: int) -> Buffer:
         return Buffer(self.ctx, lib().ksh_kvpool_v(self.h, slot, layer), owned=False)
 
+    def layer_bufs(self, layer: int):
+        """The layer's K and V caches of all slots, [max_batch][max_seq * n_kv * (hd / 32) * 18] each."""
+        return (Buffer(self.ctx, lib().ksh_kvpool_layer_k(self.h, layer), owned=False),
+                Buffer(self.ctx, lib().ksh_kvpool_layer_v(self.h, layer), owned=False))
+
 
 FINISH_REASONS = ("stop", "length", "cancelled", "error")
 
@@ -991,9 +1002,10 @@ class Serve:
     completion_tokens), ("error", request, text)."""
 
     def __init__(self, model, pool, slots: int = 4, prefill_chunk: int = 256, prefill_tokens_per_tick: int = 2048,
-                 eos=(1, 106), use_graph: bool = True, stop=None):
+                 eos=(1, 106), use_graph: bool = True, stop=None, batched_decode: int = 4):
         cfg = ServeCfg()
         _check(lib().ksh_serve_default_cfg(C.byref(cfg)))
+        cfg.batched_decode = int(batched_decode)      # joint decode steps from this many decoding requests on; 0: never
         cfg.slots, cfg.prefill_chunk, cfg.prefill_tokens_per_tick = slots, prefill_chunk, prefill_tokens_per_tick
         cfg.eos[0], cfg.eos[1] = int(eos[0]), int(eos[1])
         cfg.use_graph = int(use_graph)
@@ -1156,6 +1168,28 @@ class Gemma4:
         per layer; `serial` feeds every token through the decode step instead."""
         t = (C.c_uint32 * max(1, len(tokens)))(*[int(x) for x in tokens])
         _check(lib().ksh_gemma4_prefill_chunk(self.h, t, len(tokens), int(bool(use_graph)) | (2 if serial else 0)))
+
+    def decode_round(self, pool, slots, tokens, temperature=None, min_p=None, seeds=None):
+        """One decode step for several sequences as one pass over the weights (the scheduler's decode round,
+        crates/ksearch_cli/src/scheduler.rs:163-231): row i feeds tokens[i] to the sequence in pool slot slots[i].
+        Returns the next ids; the caller bumps the slots' lengths."""
+        n = len(slots)
+        sl = (C.c_int32 * n)(*[int(x) for x in slots])
+        tk = (C.c_uint32 * n)(*[int(x) for x in tokens])
+        out = (C.c_uint32 * n)()
+        if temperature is None:
+            te = mp = sd = None
+        else:
+            te = (C.c_float * n)(*[float(x) for x in temperature])
+            mp = (C.c_float * n)(*[float(x) for x in min_p])
+            sd = (C.c_uint32 * n)(*[int(x) & 0xFFFFFFFF for x in seeds])
+        _check(lib().ksh_gemma4_decode_round(self.h, pool.h, sl, tk, n, te, mp, sd, out))
+        return list(out)
+
+    def round_logits(self, n: int) -> np.ndarray:
+        buf = Buffer(self.ctx, lib().ksh_gemma4_round_logits(self.h), owned=False)
+        v = self.cfg["vocab"]
+        return self.ctx.read_f32(buf, n * v).reshape(n, v)
 
     def bind_slot(self, pool, slot: int):
         """GemmaPrimModel::bind_slot; pool=None goes back to the model's own caches at position `slot`."""

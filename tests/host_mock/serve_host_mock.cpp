@@ -22,10 +22,23 @@ int set_error(const char *fmt, ...)
     g_err = b;
     return 1;
 }
+ksh_buf *buffer_view(ksh_buf *parent, size_t off, size_t bytes)
+{
+    if (!parent || off > parent->bytes || bytes > parent->bytes - off) {
+        set_error("buffer_view: range outside the buffer");
+        return nullptr;
+    }
+    ksh_buf *v = new ksh_buf;
+    v->ptr = (char *)parent->ptr + off;
+    v->bytes = bytes;
+    v->parent = parent;
+    parent->rc++;
+    return v;
+}
 }  // namespace ksh
 
 struct MockCall {
-    int32_t kind;   // 0 bind_slot, 1 prefill_chunk, 2 decode_token_sampled
+    int32_t kind;   // 0 bind_slot, 1 prefill_chunk, 2 decode_token_sampled, 3 one row of decode_round
     int32_t slot, pos, n;
     uint32_t token, seed;
     float temperature, min_p;
@@ -57,7 +70,10 @@ int ksh_buffer_alloc(ksh_ctx *, size_t bytes, const void *init, ksh_buf **out)
 void ksh_buffer_release(ksh_buf *b)
 {
     if (b && --b->rc == 0) {
-        free(b->ptr);
+        if (b->parent)
+            ksh_buffer_release(b->parent);
+        else
+            free(b->ptr);
         delete b;
     }
 }
@@ -121,6 +137,25 @@ int ksh_gemma4_decode_token_sampled(ksh_gemma4 *m, uint32_t token, float tempera
     m->calls.push_back(MockCall{2, m->slot, m->pos, 1, token, seed, temperature, min_p});
     *next = m->mode == 1 ? m->constant : (uint32_t)((31ull * token + 7ull * (unsigned)m->pos + 1) % (unsigned)m->vocab);
     m->pos += 1;
+    return 0;
+}
+
+// one record per row; positions come from the pool, the model's own binding is left alone
+int ksh_gemma4_decode_round(ksh_gemma4 *m, ksh_kvpool *pool, const int32_t *slots, const uint32_t *tokens, int n, const float *temperature,
+                            const float *min_p, const uint32_t *seed, uint32_t *next_ids)
+{
+    if (n < 1 || n > 16) return ksh::set_error("ksh_gemma4_decode_round: %d sequences", n);
+    for (int i = 0; i < n; i++) {
+        const int pos = ksh_kvpool_seq_len(pool, slots[i]);
+        if (pos < 0) return ksh::set_error("bad SlotId");
+        if (pos >= m->max_seq) return ksh::set_error("max_seq exceeded");
+        if (m->mode == 2 && pos == m->fail_pos) return ksh::set_error("mock decode failure at %d", pos);
+    }
+    for (int i = 0; i < n; i++) {
+        const int pos = ksh_kvpool_seq_len(pool, slots[i]);
+        m->calls.push_back(MockCall{3, slots[i], pos, n, tokens[i], seed ? seed[i] : 0, temperature ? temperature[i] : 0.f, min_p ? min_p[i] : 0.f});
+        next_ids[i] = m->mode == 1 ? m->constant : (uint32_t)((31ull * tokens[i] + 7ull * (unsigned)pos + 1) % (unsigned)m->vocab);
+    }
     return 0;
 }
 

@@ -56,7 +56,7 @@ def test_struct_sizes():
     assert C.sizeof(hip.Gemma4Cfg) == 11 * 4 + 6 * 4
     assert C.sizeof(hip.Gemma4Layer) == 11 * 4 + 4 + 16 * 8 + 8          # ints, pad, pointers, scale + tail pad
     assert C.sizeof(hip.Gemma4Globals) == 8 * 8
-    assert C.sizeof(hip.ServeCfg) == 3 * 4 + 8 + 4 + 2 * 8
+    assert C.sizeof(hip.ServeCfg) == 3 * 4 + 8 + 2 * 4 + 4 + 2 * 8          # ints, eos, use_graph + batched_decode, pad, pointers
     assert C.sizeof(hip.ServeEvent) == 8 + 5 * 4 + 4
 
 

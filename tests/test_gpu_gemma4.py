@@ -443,6 +443,7 @@ def real_widths_models(ctx, eng):
 
     w = dict(layers=[{k: host(v) for k, v in lw.items()} for lw in dev["layers"]], globals={k: host(v) for k, v in dev["globals"].items()})
     gpu, cpu = hip.Gemma4(ctx, cfg, dev), oracle.Gemma4(cfg, w)
+    cpu.host_weights = w                # (for a second oracle over the same bytes)
     assert [gpu.kv_source(l) for l in range(n)] == [0, 1, 2, 3, 4, 4, 4, 2, 4]
     return gpu, cpu, cfg, pattern
 
@@ -550,3 +551,155 @@ def test_gemma4_two_sequences_interleaved_through_pool_slots(tiny):
     gpu.reset()
     assert gpu.generate(prompts[0], n_new, use_graph=True)[0] == alone[0]
     pool.close()
+
+
+def slot_rows(ctx, pool, slot, pos, cfg, pattern, owners):
+    """The K / V rows position `pos` left in a pool slot, one per cache-owning layer, padded to the widest."""
+    n = cfg["n_layers"]
+    hd = {l: cfg["hd_swa"] if pattern[l] else cfg["hd_full"] for l in owners}
+    stride = max(cfg["n_kv"] * h // 32 * 18 for h in hd.values())
+    rows = np.zeros((n, 2, stride), np.uint8)
+    for l in owners:
+        row = cfg["n_kv"] * hd[l] // 32 * 18
+        rows[l, 0, :row] = ctx.read_bytes(pool.k_buf(slot, l), row, pos * row)
+        rows[l, 1, :row] = ctx.read_bytes(pool.v_buf(slot, l), row, pos * row)
+    return rows
+
+
+@pytest.mark.parametrize("variant", ["all_q4k", "mixed_q6k_two_kv_heads"])
+def test_gemma4_decode_round_over_pool_slots(ctx, variant):
+    """One decode step for several sequences as one pass over the weights (the scheduler's decode round,
+    crates/ksearch_cli/src/scheduler.rs:163-231, there one step per request).  Three sequences of different lengths in
+    slots 2, 0 and 3 of a four-slot pool (prompts fed through bind_slot + prefill_chunk), then 12 rounds of all three
+    (across the sliding window's edge), one of two of them, and serial steps in between; each sequence has its own
+    oracle, walking the same tokens in lockstep with the rows its slot received: every row's logits within 1e-3, the
+    greedy id the oracle's where its margin allows, appended K / V rows within one code of the oracle's."""
+    cfg = dict(synth.GEMMA4_TINY)
+    q6 = ()
+    if variant != "all_q4k":
+        cfg["n_kv"] = 2
+        q6 = {(1, "wv"), (2, "wdown"), (3, "wq"), (4, "wgate"), (5, "wo"), (6, "wup"), (7, "proj")}
+    w = synth.gemma4_weights(cfg, 651, oracle.quantize_q4k, oracle.quantize_q6k, ffn=FFN, swa_pattern=PATTERN, q6k_tensors=q6, std=0.05)
+    gpu = hip.Gemma4(ctx, cfg, w)
+    n, tol = cfg["n_layers"], 1e-3
+    owners = [l for l in range(n) if gpu.kv_source(l) == l]
+    pool = hip.KvPool(ctx, 4, cfg["max_seq"], len(owners), max(cfg["hd_swa"], cfg["hd_full"]), cfg["n_kv"])
+    for _ in range(4):
+        pool.clear_slot(pool.alloc())
+    pool.free(1)
+    rng = np.random.default_rng(650)
+    slots, pre = [2, 0, 3], [5, 1, 11]
+    cpus = [oracle.Gemma4(cfg, w) for _ in slots]           # one oracle per sequence
+    try:
+        for cpu in cpus:
+            cpu.reset()
+        for s_, n_pre, cpu in zip(slots, pre, cpus):
+            toks = [int(t) for t in rng.integers(0, cfg["vocab"], n_pre)]
+            gpu.bind_slot(pool, s_)
+            gpu.prefill_chunk(toks)
+            pool.bump_len(s_, n_pre)
+            for i, t in enumerate(toks):
+                cpu.forward(t, want_logits=False, adopt_rows=slot_rows(ctx, pool, s_, i, cfg, PATTERN, owners))
+                assert cpu.row_max_step.max() <= 1.0 + 1e-3
+        checked = 0
+
+        def check_rows(active, toks, nxt, logits):
+            nonlocal checked
+            for j, i in enumerate(active):
+                pos = pool.seq_len(slots[i])
+                c_next, c_logits = cpus[i].forward(int(toks[j]), return_logits=True, adopt_rows=slot_rows(ctx, pool, slots[i], pos, cfg, PATTERN, owners))
+                assert cpus[i].row_max_step.max() <= 1.0 + 1e-3, (i, pos)
+                assert_close(logits[j], c_logits, tol, f"sequence {i} at position {pos}")
+                assert nxt[j] == oracle.softcap_argmax(logits[j], cfg["softcap"])
+                top2 = np.sort(c_logits)[-2:]
+                if top2[1] - top2[0] > 2 * tol * max(abs(top2[1]), float(np.sqrt(np.mean(c_logits ** 2)))):
+                    assert nxt[j] == c_next
+                    checked += 1
+                pool.bump_len(slots[i])
+
+        for r in range(12):
+            toks = rng.integers(0, cfg["vocab"], 3)
+            nxt = gpu.decode_round(pool, slots, toks)
+            check_rows([0, 1, 2], toks, nxt, gpu.round_logits(3))
+            if r == 5:
+                # a serial step on one of the slots in between: bind_slot finds the slot's length moved and re-seeks
+                gpu.bind_slot(pool, slots[1])
+                assert gpu.pos == pool.seq_len(slots[1])
+                t = int(rng.integers(0, cfg["vocab"]))
+                g_next = gpu.forward_token(t, want_logits=True, use_graph=True)
+                check_rows([1], [t], [g_next], gpu.logits()[None, :])
+        toks = rng.integers(0, cfg["vocab"], 2)
+        nxt = gpu.decode_round(pool, [slots[2], slots[0]], toks)          # a subset, in another order
+        check_rows([2, 0], toks, nxt, gpu.round_logits(2))
+        nxt = gpu.decode_round(pool, [slots[1]], [7])                      # a round of one
+        check_rows([1], [7], nxt, gpu.round_logits(1))
+        assert checked >= 20
+        # sampled rows: the host sampler's draw on that row's logits
+        toks = rng.integers(0, cfg["vocab"], 3)
+        nxt = gpu.decode_round(pool, slots, toks, temperature=[0.0, 0.8, 1.3], min_p=[0.0, 0.05, 0.0], seeds=[1, 77, 991])
+        lg = gpu.round_logits(3)
+        assert nxt[0] == oracle.softcap_argmax(lg[0], cfg["softcap"])
+        assert nxt[1] == hip.sample_softcap_min_p(lg[1], cfg["softcap"], 0.8, 0.05, 77)
+        assert nxt[2] == hip.sample_softcap_min_p(lg[2], cfg["softcap"], 1.3, 0.0, 991)
+        # errors
+        with pytest.raises(hip.KshError, match="named twice"):
+            gpu.decode_round(pool, [0, 0], [1, 2])
+        with pytest.raises(hip.KshError, match="slot not occupied"):
+            gpu.decode_round(pool, [1, 0], [1, 2])
+        with pytest.raises(hip.KshError, match="bad SlotId"):
+            gpu.decode_round(pool, [9], [1])
+        with pytest.raises(hip.KshError, match="outside the vocabulary"):
+            gpu.decode_round(pool, [0], [cfg["vocab"]])
+        with pytest.raises(hip.KshError, match="1 to 16"):
+            gpu.decode_round(pool, list(range(17)), [1] * 17)
+    finally:
+        for cpu in cpus:
+            cpu.close()
+        gpu.close()
+        pool.close()
+
+
+def test_gemma4_real_widths_decode_round(ctx, eng):
+    """Decode rounds at the real widths (hidden 1536, heads of 256 / 512, window 512, 12288-wide feed-forward): two
+    sequences of 300 and 20 positions in slots 1 and 0 of a pool sized for the 512-wide heads (so the 256-wide layers'
+    caches use half of each slot's stride), six rounds in lockstep with one oracle per sequence.  Bar: 5e-3 for the
+    short sequence, as for the other runs at these widths; 2e-2 for the one that attends 300 rows, where the unscaled
+    scores make the softmax nearly one-hot and a reordering of f32 sums moves single logits by several 1e-3 (the
+    serial step on the same positions: up to 3.5e-3; the rounds: up to 9.6e-3)."""
+    gpu, cpu_a, cfg, pattern = real_widths_models(ctx, eng)
+    n = cfg["n_layers"]
+    owners = [l for l in range(n) if gpu.kv_source(l) == l]
+    pool = hip.KvPool(ctx, 3, cfg["max_seq"], len(owners), 512, cfg["n_kv"])
+    slots, pre = [1, 0], [300, 20]
+    for _ in range(2):
+        pool.clear_slot(pool.alloc())
+    rng = np.random.default_rng(660)
+    # the second sequence's oracle: the same packed bytes, read back from the device like the first's
+    cpu_b = oracle.Gemma4(cfg, cpu_a.host_weights)
+    cpus = [cpu_a, cpu_b]
+    try:
+        for s_, n_pre, cpu in zip(slots, pre, cpus):
+            cpu.reset()
+            toks = [int(t) for t in rng.integers(0, cfg["vocab"], n_pre)]
+            gpu.bind_slot(pool, s_)
+            gpu.prefill_chunk(toks)
+            pool.bump_len(s_, n_pre)
+            for i, t in enumerate(toks):
+                cpu.forward(t, want_logits=False, adopt_rows=slot_rows(ctx, pool, s_, i, cfg, pattern, owners))
+                assert cpu.row_max_step.max() <= 1.0 + 1e-3, (s_, i)
+        for r in range(6):
+            toks = rng.integers(0, cfg["vocab"], 2)
+            nxt = gpu.decode_round(pool, slots, toks)
+            lg = gpu.round_logits(2)
+            for j in range(2):
+                pos = pool.seq_len(slots[j])
+                _, c_logits = cpus[j].forward(int(toks[j]), return_logits=True, adopt_rows=slot_rows(ctx, pool, slots[j], pos, cfg, pattern, owners))
+                assert cpus[j].row_max_step.max() <= 1.0 + 1e-3, (j, pos)
+                assert_close(lg[j], c_logits, 2e-2 if pos >= 64 else 5e-3, f"sequence {j} at position {pos}")
+                assert nxt[j] == oracle.softcap_argmax(lg[j], cfg["softcap"])
+                pool.bump_len(slots[j])
+    finally:
+        cpu_b.close()
+        cpu_a.close()
+        gpu.close()
+        pool.close()

@@ -58,14 +58,16 @@ def split(events):
     return toks, done, errs
 
 
-@pytest.mark.parametrize("use_graph", [True, False])
-def test_three_requests_through_two_slots_equal_the_runs_alone(ctx, model, use_graph):
+@pytest.mark.parametrize("use_graph,batched", [(True, 0), (False, 0), (True, 2)])
+def test_three_requests_through_two_slots_equal_the_runs_alone(ctx, model, use_graph, batched):
+    """batched = 2: whenever both slots decode, their step is one ksh_gemma4_decode_round (one pass over the weights
+    for both); the tokens are still those of the runs alone."""
     m, cfg = model
     prompts = prompts_of(cfg, (5, 9, 3), 700)
     max_new = (10, 6, 8)
     want = [alone(m, p, n) for p, n in zip(prompts, max_new)]
     pool = make_pool(ctx, cfg, 2)
-    sv = hip.Serve(m, pool, slots=2, prefill_chunk=4, prefill_tokens_per_tick=8, eos=NO_EOS, use_graph=use_graph)
+    sv = hip.Serve(m, pool, slots=2, prefill_chunk=4, prefill_tokens_per_tick=8, eos=NO_EOS, use_graph=use_graph, batched_decode=batched)
     ids = [sv.submit(p, n) for p, n in zip(prompts, max_new)]
     events = sv.tick()
     assert sv.pending() == (1, 2) and len(pool.active_batch()) == 2     # the third waits for a slot

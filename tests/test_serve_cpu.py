@@ -58,7 +58,9 @@ class Rig:
         c = ServeCfg()
         assert L.ksh_serve_default_cfg(C.byref(c)) == 0
         assert (c.slots, c.prefill_chunk, c.prefill_tokens_per_tick, tuple(c.eos), c.use_graph) == (4, 256, 2048, (1, 106), 1)
+        assert c.batched_decode == 4
         c.eos[0], c.eos[1] = cfg.pop("eos", NO_EOS)
+        cfg.setdefault("batched_decode", 0)      # the reference's serial rounds unless a test asks for batched ones
         for k, v in cfg.items():
             setattr(c, k, v)
         self._stop = SERVE_STOP_FN(lambda user, req, tok: int(bool(stop(req, tok)))) if stop else SERVE_STOP_FN()
@@ -106,7 +108,7 @@ class Rig:
     def calls(self, clear=True):
         buf = (Call * 4096)()
         n = self.L.mock_model_calls(self.model, buf, 4096)
-        out = [(("bind", "prefill", "decode")[c.kind], c.slot, c.pos, c.n) for c in buf[:n]]
+        out = [(("bind", "prefill", "decode", "round")[c.kind], c.slot, c.pos, c.n) for c in buf[:n]]
         full = list(buf[:n])
         if clear:
             self.L.mock_model_clear_calls(self.model)
@@ -284,3 +286,60 @@ def test_destroy_frees_the_slots_of_running_requests(L):
     assert r.occupied() == 0
     L.ksh_kvpool_destroy(r.pool)
     L.mock_model_destroy(r.model)
+
+
+def test_batched_decode_rounds(L):
+    """batched_decode = 2: two or more decoding requests take their step as one ksh_gemma4_decode_round (one record
+    per row in the mock's log, n = rows of the round), a single one goes through bind_slot + decode_token_sampled as
+    before; tokens, sampler seeds and stop rules are those of the serial rounds.  With the threshold at 3 the last two
+    requests go one by one again."""
+    prompts = [[5, 6, 7], [9, 10], [11, 12, 13, 14]]
+    lens = [6, 3, 5]
+    serial, batched = Rig(L, batched_decode=0), Rig(L, batched_decode=2)
+    logs = {}
+    for name, rig in (("serial", serial), ("batched", batched)):
+        ids = [rig.submit(p, n, temperature=0.7 if i == 1 else 0.0, min_p=0.05, seed=40 + i) for i, (p, n) in enumerate(zip(prompts, lens))]
+        toks, done, errs = split(rig.run())
+        assert not errs
+        for rid, p, n in zip(ids, prompts, lens):
+            assert toks[rid] == expected(p, n) and done[rid][0] == "length"
+        logs[name] = rig.calls()
+        assert rig.occupied() == 0
+    s_calls, s_full = logs["serial"]
+    b_calls, b_full = logs["batched"]
+    assert not any(c[0] == "round" for c in s_calls)
+    rounds = [c for c in b_calls if c[0] == "round"]
+    # 3 tokens by all three requests together, 2 more by the two longer ones, the last by the longest alone
+    assert [c[3] for c in rounds] == [3] * 9 + [2] * 4
+    assert sum(c[0] == "decode" for c in b_calls) == 1
+    # every decoded token saw the same (slot, position, input token, seed, temperature, min_p) as in the serial rounds
+    key = lambda c: (c.slot, c.pos, c.token, c.seed, round(c.temperature, 6), round(c.min_p, 6))
+    assert sorted(key(c) for c in s_full if c.kind == 2) == sorted(key(c) for c in b_full if c.kind in (2, 3))
+    serial.close()
+    batched.close()
+    three = Rig(L, batched_decode=3)
+    ids = [three.submit(p, n) for p, n in zip(prompts, lens)]
+    toks, done, errs = split(three.run())
+    assert not errs and all(toks[r] == expected(p, n) for r, p, n in zip(ids, prompts, lens))
+    calls, _ = three.calls()
+    assert [c[3] for c in calls if c[0] == "round"] == [3] * 9 and sum(c[0] == "decode" for c in calls) == 2 * 2 + 1
+    three.close()
+
+
+def test_batched_decode_more_requests_than_a_round_holds_and_errors(L):
+    """20 decoding requests are two rounds (16 + 4); a failing round sends an error to each of its requests and frees
+    their slots."""
+    rig = Rig(L, pool_slots=20, slots=20, batched_decode=2)
+    ids = [rig.submit([3 + i, 4], 2) for i in range(20)]
+    toks, done, errs = split(rig.run())
+    assert not errs and all(toks[r] == expected([3 + i, 4], 2) for i, r in enumerate(ids))
+    calls, _ = rig.calls()
+    assert sorted({c[3] for c in calls if c[0] == "round"}) == [4, 16]
+    rig.close()
+    rig = Rig(L, mode=2, fail_pos=3, batched_decode=2)
+    a, b = rig.submit([1, 2, 3], 5), rig.submit([4, 5, 6], 5)
+    toks, done, errs = split(rig.run())
+    assert set(errs) == {a, b} and all("mock decode failure" in errs[r] for r in (a, b))
+    assert len(toks[a]) == 1 and len(toks[b]) == 1           # position 2 decoded, position 3 failed
+    assert rig.occupied() == 0
+    rig.close()

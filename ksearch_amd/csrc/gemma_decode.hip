@@ -215,7 +215,7 @@ int encode_token(ksh_gemma *m, bool want_logits, bool short_ctx, int &launches)
     const ksh_gemma_cfg &c = m->c;
     launches = 0;
     ksh_buf *cur = m->x, *other = m->xb;   // the residual stream and its next home
-    if (enc(m, m->k_embed, {m->embd, m->tok}, {cur}, launches)) return 1;
+    // (the token's embedding row is in m->x already: write_token put it there, or the previous step's last launch)
     hipStream_t cst = (hipStream_t)ksh_stream(m->ctx);
     constexpr int kSet = kChainHidden + kChainFfn + kChainHidden;
     if (m->use_chain && (c.n_layers & 1)) {
@@ -288,12 +288,31 @@ int encode_token(ksh_gemma *m, bool want_logits, bool short_ctx, int &launches)
     }
     if (want_logits) {
         // the last layer's rmsnorm_add and the output norm ride in the LM head's prologue
+        // (the final residual stream goes to a buffer of its own: the step's last launch writes the next token's
+        // embedding into m->x)
         if (enc(m, m->k_lm_head, {m->embd_rows ? m->embd_rows : m->embd, m->y, m->output_norm, m->layers[c.n_layers - 1].post_ffw_norm, cur},
-                {m->logits, other}, launches))
+                {m->logits, m->x2}, launches))
             return 1;
-        m->hidden = other;
-        if (enc(m, m->k_argmax, {m->logits}, {m->tok}, launches)) return 1;
-        launches += 1;   // two passes
+        m->hidden = m->x2;
+        // argmax (first pass), then one launch for its second pass, the position update and the next embedding row
+        DecodeTail t{};
+        t.tok = (float *)ksh_buffer_device_ptr(m->tok);
+        t.history = (float *)ksh_buffer_device_ptr(m->history);
+        t.max_hist = c.max_seq;
+        t.meta = (float *)ksh_buffer_device_ptr(m->meta);
+        t.rope = (const float *)ksh_buffer_device_ptr(m->rope);
+        t.rope_cur = (float *)ksh_buffer_device_ptr(m->rope_cur);
+        t.hd = c.hd;
+        t.embd = (const uint8_t *)ksh_buffer_device_ptr(m->embd);
+        t.dtype = KSH_Q6K;
+        t.n_rows = c.vocab;
+        t.n = c.hidden;
+        t.scale = std::sqrt((float)c.hidden);   // gemma_prim.rs:683
+        t.x_out = (float *)ksh_buffer_device_ptr(m->x);
+        if (launch_decode_tail(*m->k_argmax, (const float *)ksh_buffer_device_ptr(m->logits), t, (hipStream_t)ksh_stream(m->ctx))) return 1;
+        ctx_mark_pending(m->ctx);
+        launches += 2;
+        return 0;
     }
     hipStream_t st = (hipStream_t)ksh_stream(m->ctx);
     hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(64), 0, st, (float *)ksh_buffer_device_ptr(m->meta),
@@ -434,7 +453,10 @@ int write_token(ksh_gemma *m, uint32_t token)
     hipLaunchKernelGGL(set_token_kernel, dim3(1), dim3(64), 0, (hipStream_t)ksh_stream(m->ctx),
                        (float *)ksh_buffer_device_ptr(m->tok), (float)token);
     const hipError_t e = hipGetLastError();
-    return e == hipSuccess ? 0 : hip_fail(e, "set_token launch");
+    if (e != hipSuccess) return hip_fail(e, "set_token launch");
+    // its embedding row, where the decode step expects it (a step that produced its own next token has done this itself)
+    int n = 0;
+    return enc(m, m->k_embed, {m->embd, m->tok}, {m->x}, n);
 }
 
 }  // namespace

@@ -353,6 +353,43 @@ __global__ __launch_bounds__(kArgThreads) void softcap_argmax_final_kernel(const
     if (threadIdx.x == 0) out[0] = (float)(bi == 0xFFFFFFFFu ? 0u : bi);
 }
 
+// The end of a decode step as one launch behind the argmax's first pass: fold the partial maxima (the token id), then
+// what were two more launches and the next step's first -- remember the id, advance the position / attended length /
+// current rope row (gemma_prim.rs:1236-1275), and gather the new token's embedding row into the residual stream
+// (copy_scale_indexed, gemma_prim.rs:683), so that the next step starts with its first GEMV.
+__global__ __launch_bounds__(kArgThreads) void decode_tail_kernel(DecodeTail t)
+{
+    __shared__ float sv[4];
+    __shared__ uint32_t si[4];
+    __shared__ uint32_t s_id;
+    float bv = -INFINITY;
+    uint32_t bi = 0xFFFFFFFFu;
+    for (int i = threadIdx.x; i < t.nparts; i += kArgThreads) argmax_fold(bv, bi, t.pv[i], t.pi[i]);
+    argmax_block(bv, bi, sv, si);
+    const int pos = (int)t.meta[3];
+    if (threadIdx.x == 0) {
+        const uint32_t id = bi == 0xFFFFFFFFu ? 0u : bi;
+        s_id = id;
+        t.tok[0] = (float)id;   // the reference carries the index as f32 (exact below 2^24), lower.rs:6126
+        if (t.history && pos < t.max_hist) t.history[pos] = (float)id;
+    }
+    __syncthreads();   // the id is known; every thread has read the position before thread 0 moves it
+    if (pos + 1 < t.max_hist)
+        for (int i = threadIdx.x; i < t.hd; i += kArgThreads) t.rope_cur[i] = t.rope[(size_t)(pos + 1) * t.hd + i];
+    if (threadIdx.x == 0) {
+        t.meta[3] = (float)(pos + 1);
+        t.meta[0] = (float)(pos + 2);   // the next token attends rows [0, pos+1]
+    }
+    int64_t id = (int64_t)s_id;
+    id = id >= t.n_rows ? t.n_rows - 1 : id;    // never read outside the table
+    for (int i = threadIdx.x; i < t.n; i += kArgThreads) {
+        float v;
+        if (t.dtype == KSH_Q6K) v = deq_q6k_at(t.embd + (size_t)id * (size_t)(t.n / 256) * 210 + (size_t)(i >> 8) * 210, i & 255);
+        else v = deq_q4k_at(t.embd + (size_t)id * (size_t)(t.n / 256) * 144 + (size_t)(i >> 8) * 144, i & 255);
+        t.x_out[i] = t.scale * v;
+    }
+}
+
 int done(const char *what)
 {
     const hipError_t e = hipGetLastError();
@@ -454,6 +491,20 @@ constexpr int kMaxDevices = 64;
 void *g_scratch_ptr[kMaxDevices];      // per device: every GPU holds its own copy of the array
 
 }  // namespace
+
+// the soft-capped argmax's first pass over `logits` with the handle's partial-result buffer, then decode_tail_kernel
+int launch_decode_tail(const ksh_kernel &k_argmax, const float *logits, DecodeTail t, hipStream_t st)
+{
+    const int n = (int)k_argmax.desc.dims[0];
+    const int parts = min(kArgParts, (n + kArgThreads - 1) / kArgThreads);
+    float *pv = (float *)k_argmax.scratch;
+    uint32_t *pi = (uint32_t *)(pv + kArgParts);
+    if (t.dtype != KSH_Q6K && t.dtype != KSH_Q4K) return set_error("decode tail: embedding dtype %d", t.dtype);
+    hipLaunchKernelGGL(softcap_argmax_part_kernel, dim3(parts), dim3(kArgThreads), 0, st, logits, n, k_argmax.desc.params[0], pv, pi);
+    t.pv = pv; t.pi = pi; t.nparts = parts;
+    hipLaunchKernelGGL(decode_tail_kernel, dim3(1), dim3(kArgThreads), 0, st, t);
+    return done("decode tail launch");
+}
 
 int argmax_static_setup()
 {

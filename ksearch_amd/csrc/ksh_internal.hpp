@@ -67,6 +67,14 @@ void ctx_mark_pending(ksh_ctx *ctx);
 // resolves the device address of the static partial-result array of ksh_softcap_argmax_static for the current
 // device (called when a context is created; the entry point does it itself for a device it has not seen)
 int argmax_static_setup();
+// the end of a decode step (glue.hip): argmax over the logits, position update, the next token's embedding row
+struct DecodeTail {
+    const float *pv; const uint32_t *pi; int nparts;       // filled in by launch_decode_tail
+    float *tok, *history; int max_hist;
+    float *meta; const float *rope; float *rope_cur; int hd;
+    const uint8_t *embd; int dtype; int64_t n_rows; int n; float scale; float *x_out;
+};
+int launch_decode_tail(const ksh_kernel &k_argmax, const float *logits, DecodeTail t, hipStream_t st);
 }  // namespace ksh
 
 // a pool's identity for whoever caches things per pool (HIP graphs captured over its buffers): unlike its address,

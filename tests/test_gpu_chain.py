@@ -62,8 +62,8 @@ def test_decode_chain_matches_the_oracle_and_the_separate_launches(ctx, monkeypa
             top2 = np.sort(c_logits)[-2:]
             if top2[1] - top2[0] > 2e-3 * max(abs(top2[1]), float(np.sqrt(np.mean(c_logits ** 2)))):
                 assert g_next == c_next, i
-        # one launch per layer instead of four: embed, first QKV, (attention, chain) per layer, LM head, argmax x 2, advance
-        assert gpu.launches_per_token == 2 + 2 * n_layers + 4 + (n_layers & 1)
+        # one launch per layer instead of four: first QKV, (attention, chain) per layer, LM head, argmax + tail
+        assert gpu.launches_per_token == 2 * n_layers + 4 + (n_layers & 1)
         # generate: prompt as a batched chunk (not the chain's business), then the chain token by token from a graph
         gpu.reset()
         a, _, _ = gpu.generate(toks[:9], 12, use_graph=True)

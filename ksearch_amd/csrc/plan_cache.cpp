@@ -53,11 +53,13 @@ static int sdpa_candidates(const ksh_kernel_desc &d, ksh_sched *out, int cap)
                 out[n++] = s;
             }
         // the matrix-core form of the row phase (several slots, heads of 256)
-        if (d.kind == KSH_SDPA_SLOTS && d.dims[2] == 256 && groups <= 8 && d.dims[4] <= 16 && n < cap) {
-            ksh_sched s{};
-            s.tg = 256; s.vec = 2; s.unroll = 1; s.nsg = 4; s.k_split = ks; s.lds_tile = 32;
-            out[n++] = s;
-        }
+        if (d.kind == KSH_SDPA_SLOTS && d.dims[2] == 256 && groups <= 8 && d.dims[4] <= 16)
+            for (uint32_t tile : {32u, 16u}) {                // rows per wave tile: four waves of 32 or eight of 16
+                if (n >= cap) return n;
+                ksh_sched s{};
+                s.tg = 64ull * (128 / tile); s.vec = 2; s.unroll = 1; s.nsg = 128 / tile; s.k_split = ks; s.lds_tile = tile;
+                out[n++] = s;
+            }
     }
     return n;
 }

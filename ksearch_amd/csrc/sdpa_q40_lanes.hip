@@ -282,17 +282,37 @@ __device__ __forceinline__ void norm_rope_regs(const float (&xv)[HD / 64], const
 // Every workgroup derives the same table from the slots' lengths.  Slot s's partitions are the consecutive
 // flat indices from the sum of its predecessors' counts, and its records sit in that order.
 // round > 1: the rows per partition are rounded up to a multiple of it (the matrix-core form works in tiles of rows).
-__device__ __forceinline__ int dealt_rows(const float *meta, int stride, int n_slots, int nwg, int round = 1)
+//
+// A whole wave works the deal out at once: lane s holds slot s's length (one load per lane, all in flight together,
+// where a loop over the slots would wait for one length after the other), the division by the partition size runs
+// in all lanes, and only the running count of partitions is a loop over lanes.  `f` is the flat partition index of
+// the caller (wave-uniform); slot < 0 says that the deal has fewer partitions than that.  With `of_slot` >= 0 the
+// answer is that slot's range of partitions instead (first, nparts).  Up to 64 slots (host-checked: 16).
+struct Deal {
+    int slot, part, nparts, first, tlen, start, c;
+};
+__device__ __forceinline__ Deal deal_wave(const float *meta, int stride, int n_slots, int nwg, int round, int f, int of_slot = -1)
 {
+    const int lane = threadIdx.x & 63, ls = min(lane, n_slots - 1);
+    const int len = (int)meta[(size_t)ls * stride], st = (int)meta[(size_t)ls * stride + 1];
     int T = 0;
-    for (int s = 0; s < n_slots; s++) T += (int)meta[(size_t)s * stride];
-    const int spare = max(1, nwg * n_slots - n_slots);   // host-checked: nwg >= 2
-    const int c = max(1, (T + spare - 1) / spare);
-    return (c + round - 1) / round * round;
-}
-__device__ __forceinline__ int dealt_parts(const float *meta, int stride, int s, int c)
-{
-    return max(1, ((int)meta[(size_t)s * stride] + c - 1) / c);
+    for (int s = 0; s < n_slots; s++) T += __builtin_amdgcn_readlane(len, s);
+    const int spare = max(1, nwg * n_slots - n_slots);
+    int c = max(1, (T + spare - 1) / spare);
+    c = (c + round - 1) / round * round;
+    const int n = max(1, (len + c - 1) / c);
+    Deal d{-1, 0, 0, 0, 0, 0, c};
+    int first = 0;
+    for (int s = 0; s < n_slots; s++) {
+        const int ns = __builtin_amdgcn_readlane(n, s);
+        if (of_slot >= 0 ? s == of_slot : (d.slot < 0 && f < first + ns)) { d.slot = s; d.part = f - first; d.nparts = ns; d.first = first; }
+        first += ns;
+    }
+    if (d.slot >= 0) {
+        d.tlen = __builtin_amdgcn_readlane(len, d.slot);
+        d.start = __builtin_amdgcn_readlane(st, d.slot);
+    }
+    return d;
 }
 
 // The merge of a balanced launch's partials, as a second launch: with a hundred partitions to a long slot a
@@ -312,10 +332,8 @@ __global__ __launch_bounds__(256) void sdpa_dealt_merge_kernel(const float *tmp,
     __shared__ __attribute__((aligned(16))) float part4[16][64];
     const int head = blockIdx.x / (HD / 64), dq = blockIdx.x % (HD / 64), slot = blockIdx.y, S = gridDim.y;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = tid >> 4, j = tid & 15;
-    const int c = dealt_rows(meta, meta_stride, S, nwg, round);
-    int first = 0;
-    for (int s = 0; s < slot; s++) first += dealt_parts(meta, meta_stride, s, c);
-    const int n = dealt_parts(meta, meta_stride, slot, c);
+    const Deal deal = deal_wave(meta, meta_stride, S, nwg, round, 0, slot);
+    const int first = deal.first, n = deal.nparts;
     const size_t P = (size_t)nwg * S;
     const float *ov = tmp + ((size_t)first * n_q + head) * HD + dq * 64 + 4 * j;   // + i * n_q * HD
     const float *ml = tmp + P * n_q * HD + ((size_t)first * n_q + head) * 2;      // + i * n_q * 2
@@ -405,17 +423,10 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
     // partial records: rec(head, part) = tmp + rec_base + head * rec_hs + part * rec_ps
     size_t rec_base = (size_t)slot * p.n_q * p.nwg * (HD + 2), rec_hs = (size_t)p.nwg * (HD + 2), rec_ps = HD + 2;
     if (p.balance) {
-        const int S = gridDim.z, f = blockIdx.z * p.nwg + blockIdx.x;
-        const int c = dealt_rows(p.meta, p.meta_stride, S, p.nwg);
-        int first = 0;
-        slot = -1;
-        for (int s = 0; s < S; s++) {
-            const int n = dealt_parts(p.meta, p.meta_stride, s, c);
-            if (f < first + n) { slot = s; part = f - first; nparts = n; break; }
-            first += n;
-        }
-        if (slot < 0) return;   // left over
-        rec_base = (size_t)first + part;   // flat partition index: values [flat][n_q][HD], then (m, l) [flat][n_q][2]
+        const Deal d = deal_wave(p.meta, p.meta_stride, (int)gridDim.z, p.nwg, 1, blockIdx.z * p.nwg + blockIdx.x);
+        if (d.slot < 0) return;   // left over
+        slot = d.slot; part = d.part; nparts = d.nparts;
+        rec_base = (size_t)d.first + part;   // flat partition index: values [flat][n_q][HD], then (m, l) [flat][n_q][2]
     }
 
     const size_t slot_bytes = p.kv_shared ? 0 : p.slot_stride ? p.slot_stride : (size_t)p.max_t * p.n_kv * ROWB;
@@ -784,7 +795,12 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
 // vector-ALU form, so the same merge kernels follow.
 typedef _Float16 h8v __attribute__((ext_vector_type(8)));
 typedef float f4v __attribute__((ext_vector_type(4)));
-constexpr int kMfmaWaves = 4, kMfmaTile = 32, kMfmaRound = kMfmaWaves * kMfmaTile;
+typedef _Float16 h4v __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+// A workgroup takes rounds of 128 rows: four waves with tiles of 32 rows (the P.V product is a full 16x16x32), or eight
+// waves with tiles of 16 (16x16x16: half the work per wave and two waves per SIMD, for launches whose partitions are a
+// round or two and whose time is therefore one wave's chain of dependent steps).
+constexpr int kMfmaRound = 128;
 
 __device__ __forceinline__ float xor16_max(float x)
 {
@@ -798,9 +814,9 @@ __device__ __forceinline__ float xor32_max(float x)
 }
 
 // 8 nibbles of a dword as f16 (16 + n), in the order (n0, n4), (n1, n5), (n2, n6), (n3, n7)
-__device__ __forceinline__ h8v nibbles_f16(uint32_t d)
+// (M = 0x03C003C0 and G = 0x4C004C00 come in registers: the and-or is then one instruction, which takes no literals)
+__device__ __forceinline__ h8v nibbles_f16(uint32_t d, uint32_t M, uint32_t G)
 {
-    constexpr uint32_t M = 0x03C003C0u, G = 0x4C004C00u;
     const u32x4_t o = {((d << 6) & M) | G, ((d << 2) & M) | G, ((d >> 2) & M) | G, ((d >> 6) & M) | G};
     return __builtin_bit_cast(h8v, o);
 }
@@ -813,15 +829,21 @@ __device__ __forceinline__ int mfma_k_elem(int s, int kq)
     return 4 * kq + byte + ((s >> 1) & 1) * 16;      //    nibble: lo lo hi hi lo lo hi hi
 }
 
-template <int HD>
-__global__ __launch_bounds__(kMfmaWaves * 64, 2) void sdpa_mfma_kernel(LaneParams p)
+template <int HD, int TR>
+__global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_mfma_kernel(LaneParams p)
 {
-    constexpr int NW = kMfmaWaves, NT = NW * 64, NB = HD / 32, ROWB = NB * 18, TR = kMfmaTile, TILEB = TR * ROWB;
+    static_assert(TR == 16 || TR == 32, "tile rows");
+    constexpr int NW = kMfmaRound / TR, NT = NW * 64, NB = HD / 32, ROWB = NB * 18, TILEB = TR * ROWB;
     constexpr int STRIP = 2 * TILEB + 2 * TR * NB * 4;           // K bytes, V bytes, K scales, V scales
     constexpr int PIECES = TR * ROWB / 16;                       // 128-bit pieces of a tile
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int col = lane & 15, q4 = lane >> 4, head = col & 7, is_lo = col >> 3;
+    const uint32_t odd_mask = 0u - (uint32_t)(q4 & 1);     // all ones in the lane groups whose accumulator rows are heads 4..7
+    uint32_t nib_mask = 0x03C003C0u, nib_one = 0x4C004C00u;  // a nibble's place in an f16 mantissa; 16.0 twice
+    asm volatile("" : "+v"(nib_mask), "+v"(nib_one));
+    // the two parts of x = p * dv: hi lanes keep x cut to 11 bits, lo lanes what the cut left over
+    const uint32_t keep = is_lo ? 0xFFFFFFFFu : 0xFFFFE000u, drop = is_lo ? 0xFFFFE000u : 0u;
     uint8_t *strip = lds_raw + (size_t)wave * STRIP;
     uint8_t *kraw = strip, *vraw = strip + TILEB;
     float *ksc = reinterpret_cast<float *>(strip + 2 * TILEB), *vsc = ksc + TR * NB;
@@ -831,34 +853,27 @@ __global__ __launch_bounds__(kMfmaWaves * 64, 2) void sdpa_mfma_kernel(LaneParam
     size_t rec_base = 0;
     int p0, p1, start;
     if (p.balance) {
-        const int S = gridDim.z, f = blockIdx.z * p.nwg + blockIdx.x;
-        const int c = dealt_rows(p.meta, p.meta_stride, S, p.nwg, kMfmaRound);
-        int first = 0;
-        slot = -1;
-        for (int s = 0; s < S; s++) {
-            const int n = dealt_parts(p.meta, p.meta_stride, s, c);
-            if (f < first + n) { slot = s; part = f - first; nparts = n; break; }
-            first += n;
-        }
-        if (slot < 0) return;   // left over
-        rec_base = (size_t)first + part;
-        const int tlen = (int)p.meta[(size_t)slot * p.meta_stride];
-        p0 = part * c;
-        p1 = min(p0 + c, tlen);
+        const Deal d = deal_wave(p.meta, p.meta_stride, (int)gridDim.z, p.nwg, kMfmaRound, blockIdx.z * p.nwg + blockIdx.x);
+        if (d.slot < 0) return;   // left over
+        slot = d.slot; part = d.part; nparts = d.nparts;
+        rec_base = (size_t)d.first + part;
+        p0 = part * d.c;
+        p1 = min(p0 + d.c, d.tlen);
+        start = d.start;
     } else {
         const int tlen = (int)p.meta[(size_t)slot * p.meta_stride];
         const int chunk = ((tlen + nparts - 1) / nparts + TR - 1) / TR * TR;
         p0 = min(part * chunk, tlen);
         p1 = min(p0 + chunk, tlen);
+        start = (int)p.meta[(size_t)slot * p.meta_stride + 1];
     }
-    start = (int)p.meta[(size_t)slot * p.meta_stride + 1];
     const size_t slot_bytes = p.kv_shared ? 0 : p.slot_stride ? p.slot_stride : (size_t)p.max_t * p.n_kv * ROWB;
     const size_t row_stride = (size_t)p.n_kv * ROWB;
     const size_t kv_slot = p.slot_ids ? (size_t)max((int)p.slot_ids[slot], 0) : (size_t)slot;
     const uint8_t *kbase = p.k + kv_slot * slot_bytes + (size_t)kvh * ROWB;
     const uint8_t *vbase = p.v + kv_slot * slot_bytes + (size_t)kvh * ROWB;
 
-    // ---- the first tile's bytes are requested before anything else (they have the longest way to come)
+    // ---- a tile's bytes as whole 128-bit pieces, into registers (the first tile's are requested right behind q)
     constexpr int NPC = (PIECES + 63) / 64;
     u32x4_t kpre[NPC], vpre[NPC];
     auto fetch_tile = [&](int it) __attribute__((always_inline)) {
@@ -876,10 +891,13 @@ __global__ __launch_bounds__(kMfmaWaves * 64, 2) void sdpa_mfma_kernel(LaneParam
             }
         }
     };
-    fetch_tile(0);
 
     // ---- q: the B operands of the score products and 24 * sum_b(q), fixed for the launch.  Wave w prepares blocks
-    // w, w + NW, ... and the workgroup shares them through LDS (behind the strips).
+    // w, w + NW, ... and the workgroup shares them through LDS (behind the strips).  q is asked for before the tile:
+    // loads come back in the order they went out, q is the short way (it was just written) and its preparation
+    // then runs while the tile is on its way.
+    static_assert(NB % NW == 0, "the q blocks divide among the waves");
+    constexpr int QPW = NB / NW;
     h8v qop[NB];
     float qs24[NB];
     {
@@ -887,9 +905,18 @@ __global__ __launch_bounds__(kMfmaWaves * 64, 2) void sdpa_mfma_kernel(LaneParam
         float *qsum_share = reinterpret_cast<float *>(qshare + NB * 64);            // [NB][64]
         const float *qh = p.q + ((size_t)slot * p.n_q + head0 + min(head, groups - 1)) * HD;
         const bool have = head < groups;
-        for (int b = wave; b < NB; b += NW) {
-            const float4 lo4 = *reinterpret_cast<const float4 *>(qh + 32 * b + 4 * q4);        // elements 4kq .. 4kq+3
-            const float4 hi4 = *reinterpret_cast<const float4 *>(qh + 32 * b + 16 + 4 * q4);   // 16+4kq .. 16+4kq+3
+        float4 qlo[QPW], qhi[QPW];
+#pragma unroll
+        for (int u = 0; u < QPW; u++) {
+            const int b = wave + NW * u;
+            qlo[u] = *reinterpret_cast<const float4 *>(qh + 32 * b + 4 * q4);        // elements 4kq .. 4kq+3
+            qhi[u] = *reinterpret_cast<const float4 *>(qh + 32 * b + 16 + 4 * q4);   // 16+4kq .. 16+4kq+3
+        }
+        fetch_tile(0);
+#pragma unroll
+        for (int u = 0; u < QPW; u++) {
+            const int b = wave + NW * u;
+            const float4 lo4 = qlo[u], hi4 = qhi[u];
             const float x[8] = {lo4.x, lo4.z, hi4.x, hi4.z, lo4.y, lo4.w, hi4.y, hi4.w};       // slot order (mfma_k_elem)
             h8v op;
             float sum = 0.f;
@@ -954,9 +981,10 @@ __global__ __launch_bounds__(kMfmaWaves * 64, 2) void sdpa_mfma_kernel(LaneParam
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         if (nvalid > 0) {
             // ---- scores of the tile's two 16-row halves: lane (col, q4) ends up with rows 4*q4 + r of each
-            float sv[8];
+            constexpr int NS = TR / 4;                       // scores (rows) per lane
+            float sv[NS];
 #pragma unroll
-            for (int t = 0; t < 2; t++) {
+            for (int t = 0; t < TR / 16; t++) {
                 float acc[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int b = 0; b < NB; b++) {
@@ -966,7 +994,7 @@ __global__ __launch_bounds__(kMfmaWaves * 64, 2) void sdpa_mfma_kernel(LaneParam
                     const uint8_t *src = kraw + (16 * t + col) * ROWB + 18 * b + 2 + 4 * q4;
                     const uint32_t d = (uint32_t)*reinterpret_cast<const uint16_t *>(src) |
                                        ((uint32_t)*reinterpret_cast<const uint16_t *>(src + 2) << 16);
-                    const f4v c = __builtin_amdgcn_mfma_f32_16x16x32_f16(nibbles_f16(d), qop[b], f4v{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                    const f4v c = __builtin_amdgcn_mfma_f32_16x16x32_f16(nibbles_f16(d, nib_mask, nib_one), qop[b], f4v{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
 #pragma unroll
                     for (int r = 0; r < 4; r++) acc[r] = fmaf(dk[r], c[r] - qs24[b], acc[r]);
                 }
@@ -979,13 +1007,13 @@ __global__ __launch_bounds__(kMfmaWaves * 64, 2) void sdpa_mfma_kernel(LaneParam
             // ---- online softmax over the tile (per column; the maximum across the wave's four lane groups)
             float mt = sv[0];
 #pragma unroll
-            for (int i = 1; i < 8; i++) mt = fmaxf(mt, sv[i]);
+            for (int i = 1; i < NS; i++) mt = fmaxf(mt, sv[i]);
             mt = xor32_max(xor16_max(mt));
             const float m_new = fmaxf(m_run, mt);
             const float alpha = __expf(m_run - m_new);
-            float pr[8], ls = 0.f;
+            float pr[NS], ls = 0.f;
 #pragma unroll
-            for (int i = 0; i < 8; i++) {
+            for (int i = 0; i < NS; i++) {
                 const int row = 16 * (i >> 2) + 4 * q4 + (i & 3);
                 pr[i] = row < nvalid ? __expf(sv[i] - m_new) : 0.f;
                 ls += pr[i];
@@ -1000,9 +1028,10 @@ __global__ __launch_bounds__(kMfmaWaves * 64, 2) void sdpa_mfma_kernel(LaneParam
 #pragma unroll
             for (int h = 0; h < 8; h++) rescale = rescale || ah[h] != 1.0f;
             if (rescale) {
+                // (a bitwise select between the two scalars: an indexed pick would put the eight factors in memory)
                 float ar[4];
 #pragma unroll
-                for (int r = 0; r < 4; r++) ar[r] = (q4 & 1) ? ah[4 + r] : ah[r];
+                for (int r = 0; r < 4; r++) ar[r] = as_f32((as_u32(ah[r]) & ~odd_mask) | (as_u32(ah[4 + r]) & odd_mask));
 #pragma unroll
                 for (int c = 0; c < 2 * NB; c++)
 #pragma unroll
@@ -1014,31 +1043,43 @@ __global__ __launch_bounds__(kMfmaWaves * 64, 2) void sdpa_mfma_kernel(LaneParam
             // 16*(s/4) + 4*q4 + s%4, the rows its own scores belong to
 #pragma unroll
             for (int b = 0; b < NB; b++) {
-                h8v pa;
-                uint32_t vlo[4], vhi[4];
-                const float4 d0 = *reinterpret_cast<const float4 *>(vsc + b * TR + 4 * q4);        // rows 4*q4 .. +3
-                const float4 d1 = *reinterpret_cast<const float4 *>(vsc + b * TR + 16 + 4 * q4);   // rows 16 + 4*q4 .. +3
-                const float dv[8] = {d0.x, d0.y, d0.z, d0.w, d1.x, d1.y, d1.z, d1.w};
+                uint32_t pa[NS / 2], vlo[NS / 2], vhi[NS / 2];
+                float dv[NS];
+#pragma unroll
+                for (int t = 0; t < TR / 16; t++) {
+                    const float4 d4 = *reinterpret_cast<const float4 *>(vsc + b * TR + 16 * t + 4 * q4);   // rows 16t + 4*q4 .. +3
+                    dv[4 * t] = d4.x; dv[4 * t + 1] = d4.y; dv[4 * t + 2] = d4.z; dv[4 * t + 3] = d4.w;
+                }
                 float tsum = 0.f;
 #pragma unroll
-                for (int i = 0; i < 8; i++) {
-                    const float x = pr[i] * dv[i];
-                    const _Float16 hi = (_Float16)x;
-                    const _Float16 lo = (_Float16)(x - (float)hi);
-                    pa[i] = is_lo ? lo : hi;
-                    tsum += x;
+                for (int i = 0; i < NS; i += 2) {
+                    // (the conversion is exact for the hi part and cuts the lo part to 11 of its 13 bits)
+                    const float x0 = pr[i] * dv[i], x1 = pr[i + 1] * dv[i + 1];
+                    const float y0 = as_f32(as_u32(x0) & keep) - as_f32(as_u32(x0) & drop);
+                    const float y1 = as_f32(as_u32(x1) & keep) - as_f32(as_u32(x1) & drop);
+                    pa[i / 2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(y0, y1));
+                    tsum += x0 + x1;
                 }
                 Tl[b] += tsum;                                  // sum(P') of the lane's own rows and column, for the code offset
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
+                for (int i = 0; i < NS / 2; i++) {
                     const int ra = 16 * ((2 * i) >> 2) + 4 * q4 + ((2 * i) & 3), rb = ra + 1;
                     const uint32_t t2 = (uint32_t)vraw[ra * ROWB + 18 * b + 2 + col] | ((uint32_t)vraw[rb * ROWB + 18 * b + 2 + col] << 16);
-                    vlo[i] = ((t2 << 6) & 0x03C003C0u) | 0x4C004C00u;
-                    vhi[i] = ((t2 << 2) & 0x03C003C0u) | 0x4C004C00u;
+                    vlo[i] = ((t2 << 6) & nib_mask) | nib_one;
+                    vhi[i] = ((t2 << 2) & nib_mask) | nib_one;
                 }
-                const u32x4_t lo4 = {vlo[0], vlo[1], vlo[2], vlo[3]}, hi4 = {vhi[0], vhi[1], vhi[2], vhi[3]};
-                O[2 * b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, __builtin_bit_cast(h8v, lo4), O[2 * b], 0, 0, 0);
-                O[2 * b + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, __builtin_bit_cast(h8v, hi4), O[2 * b + 1], 0, 0, 0);
+                if constexpr (TR == 32) {
+                    const h8v pa8 = __builtin_bit_cast(h8v, u32x4_t{pa[0], pa[1], pa[2], pa[3]});
+                    const u32x4_t lo4 = {vlo[0], vlo[1], vlo[2], vlo[3]}, hi4 = {vhi[0], vhi[1], vhi[2], vhi[3]};
+                    O[2 * b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa8, __builtin_bit_cast(h8v, lo4), O[2 * b], 0, 0, 0);
+                    O[2 * b + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa8, __builtin_bit_cast(h8v, hi4), O[2 * b + 1], 0, 0, 0);
+                } else {
+                    // 16 rows: k = 4 * q4 + i is the row itself in both operands
+                    const h4v pa4 = __builtin_bit_cast(h4v, u32x2_t{pa[0], pa[1]});
+                    const u32x2_t lo2 = {vlo[0], vlo[1]}, hi2 = {vhi[0], vhi[1]};
+                    O[2 * b] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa4, __builtin_bit_cast(h4v, lo2), O[2 * b], 0, 0, 0);
+                    O[2 * b + 1] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa4, __builtin_bit_cast(h4v, hi2), O[2 * b + 1], 0, 0, 0);
+                }
             }
         }
     }
@@ -1047,44 +1088,42 @@ __global__ __launch_bounds__(kMfmaWaves * 64, 2) void sdpa_mfma_kernel(LaneParam
     __syncthreads();
     float *ow = reinterpret_cast<float *>(lds_raw);            // [NW][8][HD]
     float *mlw = ow + NW * 8 * HD;                             // [NW][8][2]
-    float *tw = mlw + NW * 8 * 2;                              // [NW][8 heads][NB]: 24 * sum(P') per head and block
     const float l_tot = xor32_sum(xor16_sum(l_run));
-    {
-        // the lanes of a column (four lane groups) and its hi / lo twin (their P' were the two parts of one value)
-        // together hold sum(P'): to a table the accumulator layout can be read from
+    // sum(P') of head h and block b: the four lane groups of column h hold its parts.  The accumulator layout wants
+    // it by row (head 4 * (q4 & 1) + r): read from lane h as a scalar, picked bitwise like the rescale factors.
+    float t24[4][NB];
 #pragma unroll
-        for (int b = 0; b < NB; b++) {
-            const float tcol = xor32_sum(xor16_sum(Tl[b]));
-            if (lane < 8) tw[((size_t)wave * 8 + lane) * NB + b] = 24.f * tcol;
+    for (int b = 0; b < NB; b++) {
+        const uint32_t tcol = as_u32(24.f * xor32_sum(xor16_sum(Tl[b])));
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const uint32_t t_lo = (uint32_t)__builtin_amdgcn_readlane((int)tcol, r), t_hi = (uint32_t)__builtin_amdgcn_readlane((int)tcol, 4 + r);
+            t24[r][b] = as_f32((t_lo & ~odd_mask) | (t_hi & odd_mask));
         }
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     }
     {
-        // hi rows are stored, lo rows added on top: the same wave's LDS operations, in order
-        float *dst[4];
+        // A head's hi rows sit in the lower 32 lanes and its lo rows in the upper 32 (lane ^ 32).  One half-wave swap
+        // per block brings both parts of the block's even 16 columns to the lower lanes and both parts of its odd 16
+        // columns to the upper lanes: swap(a, b) returns {a.lower | b.lower, a.upper | b.upper} by (lower, upper)
+        // lanes.  (The offset 24 * sum(P') of the whole value -- hi and lo part -- is taken off the hi part.)
+        const int odd = q4 >> 1;
 #pragma unroll
-        for (int r = 0; r < 4; r++) dst[r] = ow + ((size_t)wave * 8 + 4 * (q4 & 1) + r) * HD + col;
-        // (the offset 24 * sum(P') of the whole value -- hi and lo part -- is taken off the hi rows)
-        if (q4 < 2) {
+        for (int r = 0; r < 4; r++) {
+            float *dst = ow + ((size_t)wave * 8 + 4 * (q4 & 1) + r) * HD + col + 16 * odd;
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const float *t24 = tw + ((size_t)wave * 8 + 4 * (q4 & 1) + r) * NB;
-#pragma unroll
-                for (int c = 0; c < 2 * NB; c++) dst[r][16 * c] = O[c][r] - t24[c >> 1];
+            for (int b = 0; b < NB; b++) {
+                const auto sw = __builtin_amdgcn_permlane32_swap(as_u32(O[2 * b][r]), as_u32(O[2 * b + 1][r]), false, false);
+                dst[32 * b] = (as_f32(sw[0]) - t24[r][b]) + as_f32(sw[1]);
             }
-        }
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-        if (q4 >= 2) {
-#pragma unroll
-            for (int r = 0; r < 4; r++)
-#pragma unroll
-                for (int c = 0; c < 2 * NB; c++) dst[r][16 * c] += O[c][r];
         }
     }
     if (lane < 8) { mlw[(wave * 8 + lane) * 2] = m_run; mlw[(wave * 8 + lane) * 2 + 1] = l_tot; }
     __syncthreads();
-    for (int o = tid; o < groups * HD; o += NT) {
-        const int h = o / HD, d = o % HD, hq = head0 + h;
+    static_assert(NT % HD == 0 || HD % NT == 0, "whole heads per pass, or whole passes per head");
+#pragma unroll
+    for (int o = tid; o < 8 * HD; o += NT) {
+        const int h = o / HD, d = o % HD, hq = head0 + h;      // (h is the same for a whole wave)
+        if (h >= groups) break;
         float M = -1.0e30f;
 #pragma unroll
         for (int w = 0; w < NW; w++) M = fmaxf(M, mlw[(w * 8 + h) * 2]);
@@ -1108,13 +1147,14 @@ __global__ __launch_bounds__(kMfmaWaves * 64, 2) void sdpa_mfma_kernel(LaneParam
     }
 }
 
-template <int HD>
+template <int HD, int TR>
 constexpr size_t mfma_lds_bytes()
 {
-    constexpr size_t strip = 2 * (size_t)kMfmaTile * (HD / 32 * 18) + 2 * (size_t)kMfmaTile * (HD / 32) * 4;
+    constexpr size_t waves = kMfmaRound / TR;
+    constexpr size_t strip = 2 * (size_t)TR * (HD / 32 * 18) + 2 * (size_t)TR * (HD / 32) * 4;
     constexpr size_t qshare = (size_t)(HD / 32) * 64 * (16 + 4);                 // the shared q operands and sums
-    constexpr size_t fold = (size_t)kMfmaWaves * 8 * HD * 4 + (size_t)kMfmaWaves * 8 * 2 * 4 + (size_t)kMfmaWaves * 8 * (HD / 32) * 4;
-    return strip * kMfmaWaves + qshare > fold ? strip * kMfmaWaves + qshare : fold;
+    constexpr size_t fold = waves * 8 * HD * 4 + waves * 8 * 2 * 4;
+    return strip * waves + qshare > fold ? strip * waves + qshare : fold;
 }
 
 template <int HD, int GP, int NW>
@@ -1174,7 +1214,7 @@ int launch_bound(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
     LaneParams p = base_params(k);
     const int hd = (int)k.desc.dims[2], nw = (k.variant >> 16) & 0xFF;
     p.nwg = k.variant & 0xFFFF;
-    const bool mfma = nw == 0xFF;          // the matrix-core form of the row phase (bind_sdpa_lanes)
+    const bool mfma = nw >= 0xFE;          // the matrix-core form of the row phase (bind_sdpa_lanes): 0xFF tiles of 32 rows, 0xFE of 16
     if (mfma) { p.hsplit = 1; p.groups = p.n_q / p.n_kv; }
     int n_slots = 1;
     switch (k.desc.kind) {
@@ -1209,7 +1249,10 @@ int launch_bound(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
             p.balance = 1;
             p.mode = kModePart;
             if (mfma) {
-                hipLaunchKernelGGL(sdpa_mfma_kernel<256>, dim3(p.nwg, p.n_kv, n_slots), dim3(kMfmaWaves * 64), mfma_lds_bytes<256>(), st, p);
+                if (nw == 0xFF)
+                    hipLaunchKernelGGL((sdpa_mfma_kernel<256, 32>), dim3(p.nwg, p.n_kv, n_slots), dim3(kMfmaRound / 32 * 64), (mfma_lds_bytes<256, 32>()), st, p);
+                else
+                    hipLaunchKernelGGL((sdpa_mfma_kernel<256, 16>), dim3(p.nwg, p.n_kv, n_slots), dim3(kMfmaRound / 16 * 64), (mfma_lds_bytes<256, 16>()), st, p);
                 const hipError_t e0 = hipGetLastError();
                 if (e0 != hipSuccess) return hip_fail(e0, "sdpa (matrix-core form) launch");
             } else if (launch_lanes(p, hd, nw, n_slots, st)) {
@@ -1293,23 +1336,30 @@ int bind_sdpa_lanes(ksh_kernel &k, int nwg, int n_slots)
     const int n_q = (int)d[0], n_kv = (int)d[1], hd = (int)d[2];
     // sched.vec = 2: the matrix-core form of the row phase -- several slots' (or one slot's) split-KV partials for
     // heads of 256 and up to 8 q heads per kv head, merged by a second launch
-    // It is the default where the launch can hold 2^17 rows or more (several long sequences: there it runs at 1.7x
-    // the vector form's rate); below that the two forms tie and the vector form stays (vec = 3 asks for it by name).
+    // It is the default wherever it fits (from one slot of a few thousand rows to sixteen long ones it takes 0.5 to
+    // 1.0 of the vector form's time); vec = 3 asks for the vector form by name.
     const bool mfma_fits = k.desc.kind == KSH_SDPA_SLOTS && hd == 256 && n_q / n_kv <= 8 && n_slots <= 16 && nwg >= 2 && nwg <= 64;
-    if (k.desc.sched.vec == 2 || (k.desc.sched.vec == 0 && mfma_fits && (int64_t)n_slots * d[3] >= (1 << 17))) {
+    if (k.desc.sched.vec == 2 || (k.desc.sched.vec == 0 && mfma_fits)) {
         if (!mfma_fits)
             return set_error("sdpa: the matrix-core form (vec=2) takes KSH_SDPA_SLOTS with hd 256, up to 8 q heads per kv head, "
                              "up to 16 slots and 2..64 partitions");
+        // sched.lds_tile: rows per wave tile, 32 (four waves) or 16 (eight waves).  0 takes 16 where the grid is at
+        // most one workgroup per compute unit (eight-wave workgroups do not share one, so a larger grid would run in
+        // two turns; within one turn the shorter chain per wave is worth about a microsecond)
+        const int tile = k.desc.sched.lds_tile ? (int)k.desc.sched.lds_tile : (int64_t)nwg * n_kv * n_slots <= 256 ? 16 : 32;
+        if (tile != 16 && tile != 32) return set_error("sdpa: the matrix-core form takes tiles of 16 or 32 rows (lds_tile=%d)", tile);
+        const int waves = kMfmaRound / tile;
         k.scratch_bytes = 16;
-        set_launch(k, (uint32_t)nwg, (uint32_t)n_kv, (uint32_t)n_slots, kMfmaWaves * 64, (uint32_t)mfma_lds_bytes<256>());
+        set_launch(k, (uint32_t)nwg, (uint32_t)n_kv, (uint32_t)n_slots, waves * 64,
+                   (uint32_t)(tile == 32 ? mfma_lds_bytes<256, 32>() : mfma_lds_bytes<256, 16>()));
         k.info.sched = k.desc.sched;
         k.info.sched.vec = 2;
-        k.info.sched.tg = kMfmaWaves * 64;
-        k.info.sched.nsg = kMfmaWaves;
+        k.info.sched.tg = waves * 64;
+        k.info.sched.nsg = waves;
         k.info.sched.k_split = (uint32_t)nwg;
-        k.info.sched.lds_tile = kMfmaTile;
+        k.info.sched.lds_tile = tile;
         k.info.sched.unroll = 1;
-        k.variant = nwg | (0xFF << 16) | (1 << 24);
+        k.variant = nwg | ((tile == 32 ? 0xFF : 0xFE) << 16) | (1 << 24);
         k.launch = launch_bound;
         return 0;
     }

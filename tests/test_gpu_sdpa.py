@@ -91,8 +91,13 @@ def test_sdpa_needle(ctx, eng):
                          f"needle tlen={tlen} scale={scale}")
 
 
+# the two forms of the row phase for heads of 256: the library's choice (matrix cores) and the vector form by name
+FORMS = [pytest.param(None, id="default"), pytest.param(dict(vec=3), id="vector_form")]
+
+
+@pytest.mark.parametrize("sched", FORMS)
 @pytest.mark.parametrize("nwg", [0, 16, 64])
-def test_sdpa_slots_batch_equals_serial(ctx, eng, nwg):
+def test_sdpa_slots_batch_equals_serial(ctx, eng, nwg, sched):
     # cfg3 at reduced context, then at full size below
     n_slots, n_q, n_kv, hd, max_t = 4, 8, 1, 256, 2048
     lens, k, v, q = synth.cfg3_q40_attention(n_slots, n_q, n_kv, hd, max_t, lo=100, seed=330)
@@ -101,33 +106,35 @@ def test_sdpa_slots_batch_equals_serial(ctx, eng, nwg):
     meta = np.zeros((n_slots, 4), dtype=np.float32)
     meta[:, 0] = lens
     bm = ctx.buffer_f32(meta)
-    kk = ctx.compile(hip.make_desc(hip.Kind.SDPA_SLOTS, (n_q, n_kv, hd, max_t, n_slots, nwg), (DType.Q40, DType.F32), (0.0625,)))
+    kk = ctx.compile(hip.make_desc(hip.Kind.SDPA_SLOTS, (n_q, n_kv, hd, max_t, n_slots, nwg), (DType.Q40, DType.F32), (0.0625,), sched))
+    assert ("regs" if sched else "mfma") in kk.name
     real_nwg = kk.info.sched.k_split
     tmp = ctx.buffer_empty_f32(n_slots * n_q * real_nwg * (hd + 2))
     out = ctx.buffer_empty_f32(n_slots * n_q * hd)
-    eng.sdpa_slots(ctx, n_q, n_kv, hd, max_t, n_slots, bq, bk, bv, bm, tmp, out, 0.0625, nwg)
+    eng.sdpa_slots(ctx, n_q, n_kv, hd, max_t, n_slots, bq, bk, bv, bm, tmp, out, 0.0625, nwg, sched)
     got = ctx.read_f32(out, n_slots * n_q * hd).reshape(n_slots, -1)
     for s in range(n_slots):
         want = oracle.sdpa_hybrid(q[s], k[s], v[s], n_q, n_kv, hd, int(lens[s]), 0, 0.0625)
         assert_close(got[s], want, TOL, f"slot {s} len {lens[s]}")
 
 
-def test_sdpa_cfg3_full_size(ctx, eng):
+@pytest.mark.parametrize("sched", FORMS)
+def test_sdpa_cfg3_full_size(ctx, eng, sched):
     n_slots, n_q, n_kv, hd, max_t = 4, 8, 1, 256, 16384
     lens, k, v, q = synth.cfg3_q40_attention()
     bq, bk, bv = ctx.buffer_f32(q), ctx.buffer_bytes(k), ctx.buffer_bytes(v)
     meta = np.zeros((n_slots, 4), dtype=np.float32)
     meta[:, 0] = lens
-    kk = ctx.compile(hip.make_desc(hip.Kind.SDPA_SLOTS, (n_q, n_kv, hd, max_t, n_slots, 0), (DType.Q40, DType.F32), (0.0625,)))
+    kk = ctx.compile(hip.make_desc(hip.Kind.SDPA_SLOTS, (n_q, n_kv, hd, max_t, n_slots, 0), (DType.Q40, DType.F32), (0.0625,), sched))
     tmp = ctx.buffer_empty_f32(n_slots * n_q * kk.info.sched.k_split * (hd + 2))
     out = ctx.buffer_empty_f32(n_slots * n_q * hd)
-    eng.sdpa_slots(ctx, n_q, n_kv, hd, max_t, n_slots, bq, bk, bv, ctx.buffer_f32(meta), tmp, out, 0.0625, 0)
+    eng.sdpa_slots(ctx, n_q, n_kv, hd, max_t, n_slots, bq, bk, bv, ctx.buffer_f32(meta), tmp, out, 0.0625, 0, sched)
     got = ctx.read_f32(out, n_slots * n_q * hd).reshape(n_slots, -1)
     for s in range(n_slots):
         assert_close(got[s], oracle.sdpa_hybrid(q[s], k[s], v[s], n_q, n_kv, hd, int(lens[s]), 0, 0.0625), TOL, f"slot {s}")
     # softmax weights sum to one: with V == const c every output equals c (size-independent property)
     vc = np.tile(np.concatenate([np.array([0.5], dtype=np.float16).view(np.uint8), np.full(16, 0xBB, np.uint8)]), k.size // 18)
-    eng.sdpa_slots(ctx, n_q, n_kv, hd, max_t, n_slots, bq, bk, ctx.buffer_bytes(vc), ctx.buffer_f32(meta), tmp, out, 0.0625, 0)
+    eng.sdpa_slots(ctx, n_q, n_kv, hd, max_t, n_slots, bq, bk, ctx.buffer_bytes(vc), ctx.buffer_f32(meta), tmp, out, 0.0625, 0, sched)
     assert np.allclose(ctx.read_f32(out, n_slots * n_q * hd), 1.5, rtol=1e-5)
 
 
@@ -138,7 +145,8 @@ def test_sdpa_cfg3_full_size(ctx, eng):
     (17, 4, None),                      # one more: every slot keeps its own nwg partitions
     (2, 16, [2048, 2048]),              # equal lengths
 ])
-def test_sdpa_slots_partitions_dealt_by_length(ctx, eng, n_slots, nwg, lens):
+@pytest.mark.parametrize("sched", FORMS)
+def test_sdpa_slots_partitions_dealt_by_length(ctx, eng, n_slots, nwg, lens, sched):
     """A launch's nwg * n_slots partitions are shared out by slot length (up to 16 slots); every slot's result is
     still the oracle's attention over its own rows, on two launches in a row (the arrival counters return to zero)."""
     n_q, n_kv, hd, max_t = 8, 1, 256, 2048
@@ -150,7 +158,7 @@ def test_sdpa_slots_partitions_dealt_by_length(ctx, eng, n_slots, nwg, lens):
     tmp = ctx.buffer_empty_f32(n_slots * n_q * nwg * (hd + 2))
     out = ctx.buffer_empty_f32(n_slots * n_q * hd)
     for rep in range(2):
-        eng.sdpa_slots(ctx, n_q, n_kv, hd, max_t, n_slots, bq, bk, bv, bm, tmp, out, 0.0625, nwg)
+        eng.sdpa_slots(ctx, n_q, n_kv, hd, max_t, n_slots, bq, bk, bv, bm, tmp, out, 0.0625, nwg, sched)
         got = ctx.read_f32(out, n_slots * n_q * hd).reshape(n_slots, -1)
         for s in range(n_slots):
             want = oracle.sdpa(q[s], k[s], v[s], n_q, n_kv, hd, lens[s], 0, 0.0625, f64=True)
@@ -386,10 +394,12 @@ def test_beam_search_attention_kinds(ctx, tmp_path, monkeypatch):
     (4, 1, [900, 64], 1024, 4, 100),                   # four q heads, a window that starts at row 100
     (8, 1, [16384, 1024], 16384, 64, 0),               # the longest sequence beside a short one
 ])
-def test_sdpa_slots_matrix_core_form(ctx, n_q, n_kv, lens, max_t, nwg, start):
+@pytest.mark.parametrize("tile", [32, 16])
+def test_sdpa_slots_matrix_core_form(ctx, n_q, n_kv, lens, max_t, nwg, start, tile):
     """The matrix-core form of the row phase (schedule vec = 2: f16 MFMA on exact integer codes, q and p*dv split
-    hi | lo) against the serial oracle per slot, 1e-3 relative; and against the float64 brute force, where it is
-    held to 1e-4 (the products are exact, only f32 accumulation and exp remain)."""
+    hi | lo; four waves with tiles of 32 rows or eight with tiles of 16) against the serial oracle per slot, 1e-3
+    relative; and against the float64 brute force, where it is held to 1e-4 (the products are exact, only f32
+    accumulation and exp remain)."""
     hd, n_slots = 256, len(lens)
     _, kk, vv, q = synth.cfg3_q40_attention(n_slots=n_slots, n_q=n_q, n_kv=n_kv, hd=hd, max_t=max_t, lo=1, seed=1303)
     meta = np.zeros((n_slots, 4), np.float32)
@@ -398,8 +408,8 @@ def test_sdpa_slots_matrix_core_form(ctx, n_q, n_kv, lens, max_t, nwg, start):
     lens = [min(t, max_t - start) for t in lens]
     meta[:, 0] = lens
     scale = 1.0 / 16.0
-    k = ctx.compile(hip.make_desc(hip.Kind.SDPA_SLOTS, (n_q, n_kv, hd, max_t, n_slots, nwg), (DType.Q40, DType.F32), (scale,), dict(vec=2)))
-    assert "mfma" in k.name
+    k = ctx.compile(hip.make_desc(hip.Kind.SDPA_SLOTS, (n_q, n_kv, hd, max_t, n_slots, nwg), (DType.Q40, DType.F32), (scale,), dict(vec=2, lds_tile=tile)))
+    assert "mfma" in k.name and k.info.sched.lds_tile == tile and k.info.sched.nsg == 128 // tile
     parts = k.info.sched.k_split
     tmp, out = ctx.buffer_empty_f32(n_slots * n_q * parts * (hd + 2)), ctx.buffer_empty_f32(n_slots * n_q * hd)
     ins = [ctx.buffer_f32(q), ctx.buffer_bytes(kk.reshape(-1)), ctx.buffer_bytes(vv.reshape(-1)), ctx.buffer_f32(meta)]

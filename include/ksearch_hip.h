@@ -215,7 +215,8 @@ typedef struct {
     uint64_t tg;       /* threads per workgroup (64 * waves) */
     uint32_t vec;      /* inner-product variant.  GEMV: 1 = byte converts + f32 FMA, 3 = int8 dot over 3 digit planes.
                         * Attention: 1 = LDS-tile form, 3 = register (vector-ALU) form, 2 = matrix-core form of the
-                        * row phase (KSH_SDPA_SLOTS, heads of 256, up to 8 q heads per kv head, up to 16 slots) */
+                        * row phase (KSH_SDPA_SLOTS, heads of 256, up to 8 q heads per kv head, up to 16 slots: the
+                        * default there; lds_tile = 32 | 16 picks four waves with tiles of 32 rows or eight with 16) */
     uint32_t unroll;   /* superblocks in flight per lane */
     uint32_t nsg;      /* waves per workgroup */
     uint32_t nr0;      /* rows per wave */

@@ -338,22 +338,32 @@ __global__ __launch_bounds__(256) void sdpa_dealt_merge_kernel(const float *tmp,
     const float *ov = tmp + ((size_t)first * n_q + head) * HD + dq * 64 + 4 * j;   // + i * n_q * HD
     const float *ml = tmp + P * n_q * HD + ((size_t)first * n_q + head) * 2;      // + i * n_q * 2
     const size_t ops = (size_t)n_q * HD, mps = (size_t)n_q * 2;
-    // first batch of values, requested before the weights exist
+    // a thread's (m, l) pairs first (loads come back in the order they went out, and the weights are made of these),
+    // read once and kept in registers across the barrier; then the first batch of values, requested before the
+    // weights exist
+    float2 p2[kMaxParts / 256];
+#pragma unroll
+    for (int u = 0; u < kMaxParts / 256; u++) p2[u] = ldg_f2(ml + (size_t)min(tid + 256 * u, n - 1) * mps, 0);
     float4 v[QB];
 #pragma unroll
     for (int u = 0; u < QB; u++) v[u] = ldg_f4(ov + (size_t)min(g + 16 * u, n - 1) * ops, 0);
     float m = -1.0e30f;
-    for (int i = tid; i < n; i += 256) m = fmaxf(m, ml[i * mps]);
+#pragma unroll
+    for (int u = 0; u < kMaxParts / 256; u++)
+        if (tid + 256 * u < n) m = fmaxf(m, p2[u].x);
     m = wave_max(m);
     if (lane == 0) red[wave] = m;
     __syncthreads();
     const float M = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
     float ls = 0.f;
-    for (int i = tid; i < n; i += 256) {
-        const float2 p2 = ldg_f2(ml + i * mps, 0);
-        const float wt = __expf(p2.x - M);
-        w[i] = wt;
-        ls = fmaf(wt, p2.y, ls);
+#pragma unroll
+    for (int u = 0; u < kMaxParts / 256; u++) {
+        const int i = tid + 256 * u;
+        if (i < n) {
+            const float wt = __expf(p2[u].x - M);
+            w[i] = wt;
+            ls = fmaf(wt, p2[u].y, ls);
+        }
     }
     ls = wave_sum(ls);
     if (lane == 0) red[4 + wave] = ls;

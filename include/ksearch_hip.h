@@ -205,6 +205,22 @@ enum ksh_kind {
      * dims: n_q, n_kv, hd, max_t, n_tok, nwg (0 = default; sched.k_split sets it too).
      * in: q[n_tok, n_q*hd], K, V, meta   out: tmp f32[n_tok*n_q*nwg*(hd+2)], o[n_tok, n_q*hd] */
     KSH_SDPA_BATCH = 29,
+    /* The activations of a decode round (up to 16 rows, one per decoding sequence), prepared once for every GEMM
+     * that reads them.  No counterpart in the reference, whose round is one decode step per request
+     * (crates/ksearch_cli/src/scheduler.rs:163-231).  The operand holds x = hi + 2^-11 lo as f16 fragments of the
+     * matrix instruction (a token's hi and lo part in one tile) and the per-sub-block sums of x.
+     * dims: cols (a multiple of 256), batch (1..16).  in: x f32[batch, cols]
+     * out: xp, 64 * cols + 2048 * (cols / 256) bytes, 16-byte aligned */
+    KSH_ROUND_PREP = 30,
+    /* Up to three Q4_K matrices of one width against one prepared operand, in one launch (q | k | v share their
+     * input), or a gate | up pair stored as gelu(gate) * up (Eng::matvec_batch, crates/ksearch_kernels/src/lib.rs:
+     * 1414-1444, is the reference's batched GEMV for up to 8 rows; fused forms: none there).  Exact integer codes on
+     * the matrix cores, the GEMV's accuracy.
+     * dims: rows0, cols, batch (1..16), rows1, rows2 (0: absent), pair (1: gate | up of rows0 rows each)
+     * dtypes: Q4K.   in: W0, xp (KSH_ROUND_PREP) [, W1 [, W2]]
+     * out: y0 f32[batch, rows0] [, y1 f32[batch, rows1] [, y2 f32[batch, rows2]]]; pair: y0 alone.
+     * Rows longer than 2048 columns are split over workgroups and added by a second launch (one matrix then). */
+    KSH_MATVEC_ROUND = 31,
     KSH_KIND_COUNT
 };
 

@@ -136,7 +136,11 @@ struct ksh_gemma4 {
             *c_ple_tok = nullptr, *c_ple_tmp = nullptr, *c_ple_ctx = nullptr, *c_ple_u = nullptr;
     // decode rounds over several KV slots (allocated at the first round): the per-token table (ids, slots, attended
     // ranges of the two layer kinds), the logits of every token of the round, the greedy ids
-    ksh_buf *r_tab = nullptr, *r_logits = nullptr, *r_next = nullptr;
+    ksh_buf *r_tab = nullptr, *r_logits = nullptr, *r_next = nullptr, *r_xp = nullptr;   // (r_xp: a round's prepared GEMM operand)
+    // a round of t sequences is one graph per t, tied to the pool whose buffers it was captured over
+    ksh_graph *round_graphs[17] = {};
+    bool round_bound[17] = {};     // a width's kernels are bound (a first round launched kernel by kernel)
+    ksh_kvpool *round_pool = nullptr;
     int r_count = 0;
 };
 
@@ -737,6 +741,7 @@ void ksh_gemma4_destroy(ksh_gemma4 *m)
     ksh_graph_destroy(m->own_graphs.body);
     ksh_graph_destroy(m->own_graphs.full);
     for (auto &g : m->slot_graphs) { ksh_graph_destroy(g.body); ksh_graph_destroy(g.full); }
+    for (ksh_graph *g : m->round_graphs) ksh_graph_destroy(g);
     delete m;
 }
 
@@ -907,14 +912,26 @@ int pool_fits(const ksh_gemma4 *m, const ksh_kvpool *pool, int *max_batch, int *
     return 0;
 }
 
+int encode_round4(ksh_gemma4 *m, ksh_kvpool *pool, int t, int max_batch, int pool_hd);
+
+void drop_round_graphs(ksh_gemma4 *m)
+{
+    for (ksh_graph *&g : m->round_graphs) { ksh_graph_destroy(g); g = nullptr; }
+    for (bool &b : m->round_bound) b = false;
+    m->round_pool = nullptr;
+}
+
 int forward_decode_round4(ksh_gemma4 *m, ksh_kvpool *pool, const int32_t *slots, const uint32_t *tokens, int t)
 {
     const ksh_gemma4_cfg &c = m->c;
     int max_batch = 0, pool_hd = 0;
     if (pool_fits(m, pool, &max_batch, &pool_hd)) return 1;
     if (chunk_buffers4(m)) return 1;
+    int64_t widest = std::max<int64_t>(c.hidden, c.ple_dim);
+    for (int l = 0; l < c.n_layers; l++) widest = std::max<int64_t>(widest, std::max<int64_t>(m->layers[l].ffn, m->plan[l].qd));
+    widest = (widest + 255) / 256 * 256;
     if (!m->r_tab && (alloc(m, (size_t)kRoundStride * 10 * 4, &m->r_tab) || alloc(m, (size_t)kRoundMax * c.vocab * 4, &m->r_logits) ||
-                      alloc(m, (size_t)kRoundMax * 4, &m->r_next)))
+                      alloc(m, (size_t)kRoundMax * 4, &m->r_next) || alloc(m, (size_t)(64 * widest + 2048 * (widest / 256)), &m->r_xp)))
         return 1;
     float tab[kRoundStride * 10] = {};
     for (int i = 0; i < t; i++) {
@@ -928,6 +945,35 @@ int forward_decode_round4(ksh_gemma4 *m, ksh_kvpool *pool, const int32_t *slots,
     }
     if (ksh_synchronize(m->ctx)) return 1;   // the table may still be read by the previous round
     if (ksh_buffer_write(m->ctx, m->r_tab, 0, tab, sizeof(tab), 1)) return 1;
+    m->r_count = t;
+    // The launches of a round depend on its width alone (tokens, slots and positions are in the table): one graph per
+    // width, captured at its second round (the first binds the width's kernels, which allocates, and a capture must
+    // not).  KSEARCH_ROUND_GRAPH=0 launches every round kernel by kernel.
+    static const bool use_graph = [] { const char *e = std::getenv("KSEARCH_ROUND_GRAPH"); return !(e && e[0] == '0'); }();
+    if (!use_graph) return encode_round4(m, pool, t, max_batch, pool_hd);
+    if (m->round_pool != pool) { drop_round_graphs(m); m->round_pool = pool; }
+    ksh_graph *&g = m->round_graphs[t];
+    if (!g && !m->round_bound[t]) {
+        m->round_bound[t] = true;
+        return encode_round4(m, pool, t, max_batch, pool_hd);
+    }
+    if (!g) {
+        if (ksh_graph_begin(m->ctx)) return 1;
+        if (encode_round4(m, pool, t, max_batch, pool_hd)) {
+            ksh_graph *dead = nullptr;
+            ksh_graph_end(m->ctx, &dead);
+            ksh_graph_destroy(dead);
+            return 1;
+        }
+        if (ksh_graph_end(m->ctx, &g)) return 1;
+    }
+    return ksh_graph_launch(m->ctx, g);
+}
+
+// every launch of a round of t sequences, behind the table's upload
+int encode_round4(ksh_gemma4 *m, ksh_kvpool *pool, int t, int max_batch, int pool_hd)
+{
+    const ksh_gemma4_cfg &c = m->c;
     const size_t o_ids = 0, o_slots = (size_t)kRoundStride * 4, o_full = (size_t)2 * kRoundStride * 4, o_swa = (size_t)6 * kRoundStride * 4;
     const int64_t h = c.hidden, tp = 32, pt = (int64_t)c.n_layers * c.ple_dim;
     const size_t slot_stride = (size_t)c.max_seq * c.n_kv * (pool_hd / 32) * 18;
@@ -958,6 +1004,17 @@ int forward_decode_round4(ksh_gemma4 *m, ksh_kvpool *pool, const int32_t *slots,
             if (run(kk, {w, x}, {0, (size_t)i * cols * 4}, {y}, {(size_t)i * rows * 4})) return 1;
         return 0;
     };
+    // Q4_K matrices of a round share one prepared operand per distinct input (KSH_ROUND_PREP) and go several to a
+    // launch where they read the same rows (q | k | v; gate | up with the GELU in the epilogue)
+    auto prep = [&](int64_t cols, ksh_buf *x) -> int {
+        ksh_kernel *kk = nullptr;
+        return get(m, KSH_ROUND_PREP, {cols, t}, {KSH_F32}, {}, &kk) || enc(m, kk, {x}, {m->r_xp}, n);
+    };
+    auto mm1 = [&](int dt, int64_t rows, int64_t cols, ksh_buf *w, ksh_buf *x, ksh_buf *y) -> int {
+        ksh_kernel *kk = nullptr;
+        if (dt != KSH_Q4K) return mm(dt, rows, cols, w, x, y);
+        return prep(cols, x) || get(m, KSH_MATVEC_ROUND, {rows, cols, t, 0, 0, 0}, {KSH_Q4K}, {}, &kk) || enc(m, kk, {w, m->r_xp}, {y}, n);
+    };
     if (get(m, KSH_COPY_SCALE_INDEXED, {h, c.vocab, t}, {m->g.dt_embd}, {std::sqrt((float)c.hidden)}, &k) ||
         run(k, {m->g.token_embd, m->r_tab}, {0, o_ids}, {m->c_x}, {0}))
         return 1;
@@ -965,7 +1022,7 @@ int forward_decode_round4(ksh_gemma4 *m, ksh_kvpool *pool, const int32_t *slots,
         ksh_kernel *kg = nullptr, *kn = nullptr, *kmix = nullptr;
         if (get(m, KSH_COPY_SCALE_INDEXED, {pt, c.vocab, t}, {m->g.dt_ple}, {std::sqrt((float)c.ple_dim)}, &kg) ||
             run(kg, {m->g.ple_embd, m->r_tab}, {0, o_ids}, {m->c_ple_tok}, {0}) ||
-            mm(m->g.dt_ple_proj, pt, h, m->g.ple_model_proj, m->c_x, m->c_ple_tmp) ||
+            mm1(m->g.dt_ple_proj, pt, h, m->g.ple_model_proj, m->c_x, m->c_ple_tmp) ||
             get(m, KSH_RMSNORM_PER_HEAD, {(int64_t)t * c.n_layers, c.ple_dim, 0}, {}, {c.eps}, &kn) ||
             enc(m, kn, {m->c_ple_tmp, m->g.ple_proj_norm}, {m->c_ple_ctx}, n) ||
             get(m, KSH_ADD_SCALE, {(int64_t)t * pt}, {}, {0.70710678118654752440f}, &kmix) ||
@@ -984,10 +1041,21 @@ int forward_decode_round4(ksh_gemma4 *m, ksh_kvpool *pool, const int32_t *slots,
         ksh_kernel *k_head = nullptr, *k_sdpa = nullptr, *k_gelu = nullptr;
         if (!sdpa_lanes_supports(c.n_q, c.n_kv, P.hd))
             return set_error("ksh_gemma4_decode_round: attention over several slots is built for heads of 128 / 256 / 512 with up to 8 q heads per kv head");
-        if (enc(m, k_norm, {m->c_x, L.attn_norm}, {m->c_x2}, n) || mm(L.dt_q, P.qd, h, L.wq, m->c_x2, m->c_q)) return 1;
+        if (enc(m, k_norm, {m->c_x, L.attn_norm}, {m->c_x2}, n)) return 1;
+        const bool qkv_q4k = L.dt_q == KSH_Q4K && (!P.owns || (L.dt_k == KSH_Q4K && L.dt_v == KSH_Q4K));
+        if (qkv_q4k) {
+            ksh_kernel *kq = nullptr;
+            if (prep(h, m->c_x2)) return 1;
+            if (P.owns ? (get(m, KSH_MATVEC_ROUND, {P.qd, h, t, P.kvd, P.kvd, 0}, {KSH_Q4K}, {}, &kq) ||
+                          enc(m, kq, {L.wq, m->r_xp, L.wk, L.wv}, {m->c_q, m->c_k, m->c_v}, n))
+                       : (get(m, KSH_MATVEC_ROUND, {P.qd, h, t, 0, 0, 0}, {KSH_Q4K}, {}, &kq) || enc(m, kq, {L.wq, m->r_xp}, {m->c_q}, n)))
+                return 1;
+        } else if (mm(L.dt_q, P.qd, h, L.wq, m->c_x2, m->c_q) ||
+                   (P.owns && (mm(L.dt_k, P.kvd, h, L.wk, m->c_x2, m->c_k) || mm(L.dt_v, P.kvd, h, L.wv, m->c_x2, m->c_v)))) {
+            return 1;
+        }
         if (P.owns) {
-            if (mm(L.dt_k, P.kvd, h, L.wk, m->c_x2, m->c_k) || mm(L.dt_v, P.kvd, h, L.wv, m->c_x2, m->c_v) ||
-                get(m, KSH_RMSNORM_PER_HEAD_QKV_Q40, {c.n_q, c.n_kv, P.hd, c.max_seq, t, max_batch, (int64_t)slot_stride}, {}, {c.eps}, &k_head) ||
+            if (get(m, KSH_RMSNORM_PER_HEAD_QKV_Q40, {c.n_q, c.n_kv, P.hd, c.max_seq, t, max_batch, (int64_t)slot_stride}, {}, {c.eps}, &k_head) ||
                 run(k_head, {m->c_q, L.q_norm, rope_tab, m->c_k, L.k_norm, m->c_v, m->r_tab, m->r_tab}, {0, 0, 0, 0, 0, 0, o_meta, o_slots},
                     {m->c_q, kc, vc}, {0, 0, 0}))
                 return 1;
@@ -999,18 +1067,26 @@ int forward_decode_round4(ksh_gemma4 *m, ksh_kvpool *pool, const int32_t *slots,
         if (get(m, KSH_SDPA_SLOTS, {c.n_q, c.n_kv, P.hd, c.max_seq, t, kRoundPartitions, max_batch, (int64_t)slot_stride}, {KSH_Q40, KSH_F32},
                 {c.attn_scale}, &k_sdpa) ||
             run(k_sdpa, {m->c_q, kc, vc, m->r_tab, m->r_tab}, {0, 0, 0, o_meta, o_slots}, {m->c_tmp, m->c_o}, {0, 0}) ||
-            mm(L.dt_o, h, P.qd, L.wo, m->c_o, m->c_y) ||
-            enc(m, k_add_then, {m->c_y, L.post_attn_norm, m->c_x, L.ffn_norm}, {m->c_x, m->c_x2}, n) ||
-            mm(L.dt_gate, L.ffn, h, L.wgate, m->c_x2, m->c_g) || mm(L.dt_up, L.ffn, h, L.wup, m->c_x2, m->c_u) ||
-            get(m, KSH_GELU_MUL, {(int64_t)t * L.ffn}, {}, {}, &k_gelu) || enc(m, k_gelu, {m->c_g, m->c_u}, {m->c_ff}, n) ||
-            mm(L.dt_down, h, L.ffn, L.wdown, m->c_ff, m->c_y) || enc(m, k_add, {m->c_y, L.post_ffw_norm, m->c_x}, {m->c_x}, n))
+            mm1(L.dt_o, h, P.qd, L.wo, m->c_o, m->c_y) ||
+            enc(m, k_add_then, {m->c_y, L.post_attn_norm, m->c_x, L.ffn_norm}, {m->c_x, m->c_x2}, n))
+            return 1;
+        if (L.dt_gate == KSH_Q4K && L.dt_up == KSH_Q4K) {
+            ksh_kernel *k_gu = nullptr;
+            if (prep(h, m->c_x2) || get(m, KSH_MATVEC_ROUND, {L.ffn, h, t, 0, 0, 1}, {KSH_Q4K}, {}, &k_gu) ||
+                enc(m, k_gu, {L.wgate, m->r_xp, L.wup}, {m->c_ff}, n))
+                return 1;
+        } else if (mm(L.dt_gate, L.ffn, h, L.wgate, m->c_x2, m->c_g) || mm(L.dt_up, L.ffn, h, L.wup, m->c_x2, m->c_u) ||
+                   get(m, KSH_GELU_MUL, {(int64_t)t * L.ffn}, {}, {}, &k_gelu) || enc(m, k_gelu, {m->c_g, m->c_u}, {m->c_ff}, n)) {
+            return 1;
+        }
+        if (mm1(L.dt_down, h, L.ffn, L.wdown, m->c_ff, m->c_y) || enc(m, k_add, {m->c_y, L.post_ffw_norm, m->c_x}, {m->c_x}, n))
             return 1;
         if (c.ple_dim > 0) {
             ksh_kernel *k_gs = nullptr, *k_as = nullptr;
-            if (mm(L.dt_inp_gate, c.ple_dim, h, L.inp_gate, m->c_x, m->c_ple_u) ||
+            if (mm1(L.dt_inp_gate, c.ple_dim, h, L.inp_gate, m->c_x, m->c_ple_u) ||
                 get(m, KSH_GELU_MUL, {(int64_t)t * c.ple_dim, c.ple_dim, pt}, {}, {}, &k_gs) ||
                 enc_off(m, k_gs, {m->c_ple_u, m->c_ple_ctx}, {0, (size_t)l * c.ple_dim * 4}, {m->c_ple_u}, n) ||
-                mm(L.dt_proj, h, c.ple_dim, L.proj, m->c_ple_u, m->c_y) ||
+                mm1(L.dt_proj, h, c.ple_dim, L.proj, m->c_ple_u, m->c_y) ||
                 get(m, KSH_RMSNORM, {h, 1, 1, t}, {}, {c.eps, L.layer_scale}, &k_as) ||
                 enc(m, k_as, {m->c_y, L.post_norm, m->c_x}, {m->c_x}, n))
                 return 1;
@@ -1022,7 +1098,6 @@ int forward_decode_round4(ksh_gemma4 *m, ksh_kvpool *pool, const int32_t *slots,
         if (run(m->k_lm_head[0], {lm_w, m->c_x, m->g.output_norm}, {0, (size_t)i * h * 4, 0}, {m->r_logits}, {(size_t)i * c.vocab * 4}) ||
             run(m->k_argmax, {m->r_logits}, {(size_t)i * c.vocab * 4}, {m->r_next}, {(size_t)i * 4}))
             return 1;
-    m->r_count = t;
     return 0;
 }
 }  // namespace

@@ -122,6 +122,8 @@ int bind_matvec_q4k_family(ksh_kernel &k);
 int bind_matvec_qkv(ksh_kernel &k);
 int bind_matvec_gate_up_gelu(ksh_kernel &k);
 int bind_matvec_batch(ksh_kernel &k);
+int bind_round_prep(ksh_kernel &k);
+int bind_matvec_round(ksh_kernel &k);
 int bind_dequant(ksh_kernel &k);
 int bind_repack_rows(ksh_kernel &k);
 int bind_quantize_k(ksh_kernel &k);

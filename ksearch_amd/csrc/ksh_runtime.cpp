@@ -75,6 +75,8 @@ static int bind(ksh_kernel &k)
     case KSH_ADD_SCALE:
     case KSH_MATVEC_GELU_MUL: return bind_ple_ops(k);
     case KSH_READ_FLOOR: return bind_read_floor(k);
+    case KSH_ROUND_PREP: return bind_round_prep(k);
+    case KSH_MATVEC_ROUND: return bind_matvec_round(k);
     }
     return set_error("unknown kernel kind %d", k.desc.kind);
 }

@@ -33,6 +33,7 @@
 
 #include "ksh_device.hpp"
 #include "ksh_internal.hpp"
+#include "q4k_lane.hpp"
 
 namespace ksh {
 namespace {
@@ -618,6 +619,244 @@ __global__ __launch_bounds__(512) void q4k_mm_skinny_kernel(MmParams p, const _F
     }
 }
 
+// ---- decode rounds (up to 16 tokens) --------------------------------------------------------------------------
+// A round of decoding slots is at most 16 rows, and several GEMMs read the same rows (q | k | v, gate | up).  Two
+// kinds serve it (neither has a counterpart in the reference, whose round is one decode step per request):
+//   KSH_ROUND_PREP    x f32[batch, cols] -> a prepared operand: the fragments of the 32 x 32 x 16 matrix instruction
+//                     with x = hi + 2^-11 lo in ONE tile -- rows 0..15 the tokens' hi parts, rows 16..31 their lo
+//                     parts -- so that one instruction per weight slice serves both parts, and the sums of x per
+//                     sub-block for the bias / min product, hi and lo.  Written once per distinct input.
+//   KSH_MATVEC_ROUND  up to three Q4_K matrices of the same width against one prepared operand in one launch, or a
+//                     gate | up pair whose workgroups hold the same 32 rows of both and store gelu(gate) * up.
+// A workgroup owns 32 weight rows of one matrix and 8 superblocks of columns, one per wave: every load of the
+// workgroup (80 bytes of weights and 288 of activations per lane) goes out before anything is used, so the launch is
+// one memory round trip where the small-batch form above walks a wave's superblocks one round trip at a time.  Rows
+// longer than 2048 columns split over blockIdx.y; the slices' sums go to a scratch buffer and a second launch adds
+// them in a fixed order.  Conversion, scales and the bias / min product are those of the forms above.
+constexpr int kRoundTokens = 16;
+
+__host__ __device__ inline size_t round_xf_halves(int cols) { return (size_t)32 * cols; }
+__host__ __device__ inline size_t round_sx_halves(int cols) { return (size_t)kRoundTokens * (cols / 256) * 32; }
+
+// one thread per 8 elements of the 16 token rows (rows past the batch are written as zeros)
+__global__ __launch_bounds__(256) void mm_round_prep_kernel(const float *__restrict__ X, _Float16 *__restrict__ Xp, int batch, int cols)
+{
+    const int idx = blockIdx.x * 256 + threadIdx.x;
+    const int k8 = cols / 8;
+    if (idx >= kRoundTokens * k8) return;   // (whole quads: cols is a multiple of 32)
+    const int t = idx / k8, j = idx - t * k8;
+    f32x4_t in0 = {0.f, 0.f, 0.f, 0.f}, in1 = in0;
+    if (t < batch) {
+        in0 = reinterpret_cast<const f32x4_t *>(X)[2 * ((size_t)t * k8 + j)];
+        in1 = reinterpret_cast<const f32x4_t *>(X)[2 * ((size_t)t * k8 + j) + 1];
+    }
+    const float f[8] = {in0.x, in0.y, in0.z, in0.w, in1.x, in1.y, in1.z, in1.w};
+    h8 oh, ol;
+    float fh[8], fl[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const _Float16 hi = (_Float16)f[i];
+        const _Float16 lo = (_Float16)((f[i] - (float)hi) * 2048.0f);   // kept 2^11 up, in the normal range wherever hi is
+        oh[kperm(i)] = hi;
+        ol[kperm(i)] = lo;
+        fh[i] = (float)hi;
+        fl[i] = (float)lo;
+    }
+    float sh = ((fh[0] + fh[1]) + (fh[2] + fh[3])) + ((fh[4] + fh[5]) + (fh[6] + fh[7]));
+    float sl = ((fl[0] + fl[1]) + (fl[2] + fl[3])) + ((fl[4] + fl[5]) + (fl[6] + fl[7]));
+    sh += dpp_f32<0xB1>(sh);
+    sh += dpp_f32<0x4E>(sh);
+    sl += dpp_f32<0xB1>(sl);
+    sl += dpp_f32<0x4E>(sl);
+    // fragment of 16 columns: lane = row + 32 * ((k / 8) % 2); row t is the token's hi part, row 16 + t its lo part
+    const size_t frag = (size_t)(j >> 1) * 64 + t + 32 * (j & 1);
+    reinterpret_cast<h8 *>(Xp)[frag] = oh;
+    reinterpret_cast<h8 *>(Xp)[frag + 16] = ol;
+    if ((threadIdx.x & 3) == 0) {
+        const int s = j / 4, jj = s % 8;
+        _Float16 *sx = Xp + round_xf_halves(cols) + ((size_t)t * (cols / 256) + s / 8) * 32;
+        const float sums[2] = {sh, sl};
+#pragma unroll
+        for (int part = 0; part < 2; part++) {
+            _Float16 *dst = sx + part * round_sx_halves(cols);
+            const _Float16 hi = (_Float16)sums[part];
+            const _Float16 lo = (_Float16)(sums[part] - (float)hi);
+            dst[jj] = hi;
+            dst[8 + jj] = hi;
+            dst[16 + jj] = lo;
+            dst[24 + jj] = (_Float16)0.f;
+        }
+    }
+}
+
+struct RoundParams {
+    const uint8_t *W0, *W1, *W2;
+    float *Y0, *Y1, *Y2;
+    int rows0, rows1, rows2, tiles0, tiles1;
+    int cols, batch;
+    const _Float16 *Xp;
+    float *part;                 // [slices][batch][rows0] when the columns are split
+};
+
+// NM = 2: the gate | up pair (W0, W1 of rows0 rows each; gelu(W0 x) * (W1 x) to Y0)
+template <int NM>
+__global__ __launch_bounds__(512) void q4k_mm_round_kernel(RoundParams p)
+{
+    extern __shared__ __attribute__((aligned(16))) float red[];   // [8][NM][16][64]
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 31, h = lane >> 5;
+    // the workgroup's matrix: a choice between arguments already fetched, not an indexed read of them
+    int tile = blockIdx.x;
+    const bool in1 = NM == 1 && tile >= p.tiles0, in2 = in1 && tile - p.tiles0 >= p.tiles1;
+    if (in1) tile -= p.tiles0;
+    if (in2) tile -= p.tiles1;
+    const uint8_t *W = in2 ? p.W2 : in1 ? p.W1 : p.W0;
+    float *Y = in2 ? p.Y2 : in1 ? p.Y1 : p.Y0;
+    const int rows = in2 ? p.rows2 : in1 ? p.rows1 : p.rows0;
+    const int r0 = tile * 32, nsb = p.cols / 256;
+    const int sb = blockIdx.y * 8 + wave;
+    const bool active = sb < nsb;                        // (wave-uniform: a row of 1536 columns leaves two waves idle)
+    const int sbc = min(sb, nsb - 1);
+    const size_t woff = (size_t)min(r0 + n, rows - 1) * nsb * 144 + (size_t)sbc * 144;
+
+    // ---- every load of the wave, up front
+    u32x4_t hdr[NM];
+    u32x2_t q[NM][4][2];
+#pragma unroll
+    for (int m = 0; m < NM; m++) {
+        const uint8_t *blk = (m ? p.W1 : W) + woff;
+        hdr[m] = *reinterpret_cast<const u32x4_t *>(blk);
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            q[m][g][0] = *reinterpret_cast<const u32x2_t *>(blk + 16 + 32 * g + 8 * h);
+            q[m][g][1] = *reinterpret_cast<const u32x2_t *>(blk + 16 + 32 * g + 16 + 8 * h);
+        }
+    }
+    const h8 *xa = reinterpret_cast<const h8 *>(p.Xp) + (size_t)sbc * 16 * 64 + lane;
+    h8 a[16];
+#pragma unroll
+    for (int j = 0; j < 16; j++) a[j] = xa[(size_t)j * 64];
+    // sums of x: rows 0..15 the tokens' hi parts, rows 16..31 their lo parts
+    const _Float16 *sx = p.Xp + round_xf_halves(p.cols) + (n >= 16 ? round_sx_halves(p.cols) : 0) + ((size_t)(n & 15) * nsb + sbc) * 32 + 8 * h;
+    const h8 a2[2] = {*reinterpret_cast<const h8 *>(sx), *reinterpret_cast<const h8 *>(sx + 16)};
+
+    const f16v kZero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int m = 0; m < NM; m++) {
+        f16v C = kZero16;
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const uint4 s = q4k_group_scales(hdr[m].y, hdr[m].z, hdr[m].w, g);   // sc_lo, mn_lo, sc_hi, mn_hi
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                // slice j: bytes (j & 1 ? 16 + 8h : 8h) .. +7, low nibbles for j < 2, high nibbles after
+                const u32x2_t qq = q[m][g][j & 1];
+                const uint32_t sc = j < 2 ? s.x : s.z;
+                uint32_t o[4];
+#pragma unroll
+                for (int i = 0; i < 2; i++) {
+                    const uint32_t d = j < 2 ? qq[i] : qq[i] >> 4;
+                    o[2 * i] = pair_f16(d & 0x000F000Fu, sc);
+                    o[2 * i + 1] = pair_f16((d >> 8) & 0x000F000Fu, sc);
+                }
+                const u32x4_t ov = {o[0], o[1], o[2], o[3]};
+                C = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[4 * g + j], __builtin_bit_cast(h8, ov), C, 0, 0, 0);
+            }
+        }
+        // bias + mins of the superblock: the row's eight coefficients -(dmin*m_j + 1024*d) as f16 hi | lo, against the
+        // sums of x (hi[8] hi[8] lo[8] 0[8] per row and superblock): hi*hi + hi*lo + lo*hi
+        const float d = half_bits_to_f32(hdr[m].x & 0xFFFFu), dmin = half_bits_to_f32(hdr[m].x >> 16);
+        _Float16 chi[8], clo[8];
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const uint4 s = q4k_group_scales(hdr[m].y, hdr[m].z, hdr[m].w, g);
+            const float c0 = -(dmin * (float)s.y + 1024.f * d), c1 = -(dmin * (float)s.w + 1024.f * d);
+            chi[2 * g] = (_Float16)c0; chi[2 * g + 1] = (_Float16)c1;
+            clo[2 * g] = (_Float16)(c0 - (float)chi[2 * g]); clo[2 * g + 1] = (_Float16)(c1 - (float)chi[2 * g + 1]);
+        }
+        h8 b2[2];
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            b2[0][i] = h ? clo[i] : chi[i];                 // columns 0..7: hi, 8..15: lo
+            b2[1][i] = h ? (_Float16)0.f : chi[i];          // columns 16..23: hi, 24..31: zero
+        }
+        f16v F = __builtin_amdgcn_mfma_f32_32x32x16_f16(a2[0], b2[0], kZero16, 0, 0, 0);
+        F = __builtin_amdgcn_mfma_f32_32x32x16_f16(a2[1], b2[1], F, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 16; i++) red[((wave * NM + m) * 16 + i) * 64 + lane] = active ? fmaf(d, C[i], F[i]) : 0.f;
+    }
+    __syncthreads();
+    // accumulator i of lane (n, h) is row 8*(i/4) + 4*h + i%4 of the tile: i < 8 a token's hi part, i + 8 its lo part.
+    // One output per thread: the eight waves' shares in a fixed order.
+    const int i = tid >> 6, t = 8 * (i >> 2) + 4 * h + (i & 3), r = r0 + n;
+    float v[NM];
+#pragma unroll
+    for (int m = 0; m < NM; m++) {
+        float hi = 0.f, lo = 0.f;
+#pragma unroll
+        for (int w = 0; w < 8; w++) {
+            hi += red[((w * NM + m) * 16 + i) * 64 + lane];
+            lo += red[((w * NM + m) * 16 + i + 8) * 64 + lane];
+        }
+        v[m] = fmaf(1.0f / 2048.0f, lo, hi);
+    }
+    if (t < p.batch && r < rows) {
+        const float y = NM == 2 ? gelu_mul_f32(v[0], v[NM - 1]) : v[0];
+        if (gridDim.y == 1) Y[(size_t)t * rows + r] = y;
+        else p.part[((size_t)blockIdx.y * p.batch + t) * rows + r] = y;
+    }
+}
+
+// y[i] = the slices' partial sums of element i, slice after slice
+__global__ __launch_bounds__(256) void mm_round_fold_kernel(const float *__restrict__ part, float *__restrict__ y, int n, int slices)
+{
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    float s = part[i];
+    for (int k = 1; k < slices; k++) s += part[(size_t)k * n + i];
+    y[i] = s;
+}
+
+int launch_round_prep(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
+{
+    const int cols = (int)k.desc.dims[0], batch = (int)k.desc.dims[1];
+    const int n = kRoundTokens * (cols / 8);
+    hipLaunchKernelGGL(mm_round_prep_kernel, dim3((n + 255) / 256), dim3(256), 0, st, (const float *)a.in[0], (_Float16 *)a.out[0], batch, cols);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : hip_fail(e, "round_prep launch");
+}
+
+int launch_matvec_round(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
+{
+    const int64_t *d = k.desc.dims;
+    const bool pair = d[5] != 0;
+    const int n_mat = pair ? 2 : d[4] ? 3 : d[3] ? 2 : 1;
+    RoundParams p{};
+    p.W0 = (const uint8_t *)a.in[0];
+    p.Xp = (const _Float16 *)a.in[1];
+    p.W1 = n_mat > 1 ? (const uint8_t *)a.in[2] : p.W0;
+    p.W2 = n_mat > 2 ? (const uint8_t *)a.in[3] : p.W0;
+    p.Y0 = (float *)a.out[0];
+    p.Y1 = (!pair && n_mat > 1) ? (float *)a.out[1] : p.Y0;
+    p.Y2 = n_mat > 2 ? (float *)a.out[2] : p.Y0;
+    p.rows0 = (int)d[0]; p.rows1 = pair ? (int)d[0] : (int)d[3]; p.rows2 = (int)d[4];
+    p.tiles0 = (p.rows0 + 31) / 32; p.tiles1 = pair ? 0 : (p.rows1 + 31) / 32;
+    p.cols = (int)d[1]; p.batch = (int)d[2];
+    p.part = (float *)k.scratch;
+    const dim3 grid(k.info.grid[0], k.info.grid[1]);
+    if (pair) hipLaunchKernelGGL(q4k_mm_round_kernel<2>, grid, dim3(512), k.info.lds_bytes, st, p);
+    else hipLaunchKernelGGL(q4k_mm_round_kernel<1>, grid, dim3(512), k.info.lds_bytes, st, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return hip_fail(e, "matvec_round launch");
+    if (grid.y > 1) {
+        const int n = p.batch * p.rows0;
+        hipLaunchKernelGGL(mm_round_fold_kernel, dim3((n + 255) / 256), dim3(256), 0, st, (const float *)k.scratch, p.Y0, n, (int)grid.y);
+        e = hipGetLastError();
+        if (e != hipSuccess) return hip_fail(e, "matvec_round fold launch");
+    }
+    return 0;
+}
+
 constexpr int kSkinnyMaxBatch = 64;
 
 int launch_mul_mm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
@@ -698,6 +937,52 @@ int bind_matvec_batch(ksh_kernel &k)
     k.info.sched.tg = kThreadsMM; k.info.sched.nsg = kThreadsMM / 64; k.info.sched.nr0 = BN; k.info.sched.k_split = 1; k.info.sched.lds_tile = KS;
     set_name(k, "mul_mm_%s_%dx%dx%d%s", q6 ? "q6k" : "q4k", BM, BN, KS, f32x ? "_f32x" : "");
     k.launch = launch_mul_mm;
+    return 0;
+}
+
+int bind_round_prep(ksh_kernel &k)
+{
+    const int64_t cols = k.desc.dims[0], batch = k.desc.dims[1];
+    if (cols <= 0 || cols % 256 || cols > (1 << 16)) return set_error("round_prep: cols=%lld is not a positive multiple of 256 up to 65536", (long long)cols);
+    if (batch < 1 || batch > kRoundTokens) return set_error("round_prep: %lld rows (1 to %d)", (long long)batch, kRoundTokens);
+    k.info.n_inputs = 1;
+    k.info.n_outputs = 1;
+    k.in_bytes[0] = (size_t)batch * cols * 4; k.in_align[0] = 16;
+    k.out_bytes[0] = (round_xf_halves((int)cols) + 2 * round_sx_halves((int)cols)) * 2; k.out_align[0] = 16;
+    set_launch(k, (uint32_t)((kRoundTokens * (cols / 8) + 255) / 256), 1, 1, 256, 0);
+    set_name(k, "round_prep_f32x");
+    k.launch = launch_round_prep;
+    return 0;
+}
+
+int bind_matvec_round(ksh_kernel &k)
+{
+    const int64_t *d = k.desc.dims;
+    const int64_t rows0 = d[0], cols = d[1], batch = d[2], rows1 = d[3], rows2 = d[4];
+    const bool pair = d[5] != 0;
+    if (k.desc.dtypes[0] != KSH_Q4K) return set_error("matvec_round: weight dtype %d is not built (Q4_K is)", k.desc.dtypes[0]);
+    if (cols <= 0 || cols % 256 || cols > (1 << 16)) return set_error("matvec_round: cols=%lld is not a positive multiple of 256 up to 65536", (long long)cols);
+    if (batch < 1 || batch > kRoundTokens) return set_error("matvec_round: %lld rows (1 to %d)", (long long)batch, kRoundTokens);
+    if (rows0 <= 0 || rows1 < 0 || rows2 < 0 || (rows2 && !rows1) || rows0 + rows1 + rows2 > (1 << 24))
+        return set_error("matvec_round: rows %lld / %lld / %lld", (long long)rows0, (long long)rows1, (long long)rows2);
+    if (pair && (rows1 || rows2)) return set_error("matvec_round: a gate | up pair names one row count (both matrices have it)");
+    const int slices = (int)((cols / 256 + 7) / 8);
+    if (slices > 1 && (pair || rows1)) return set_error("matvec_round: rows longer than 2048 columns take one matrix per launch");
+    const int n_mat = pair ? 2 : rows2 ? 3 : rows1 ? 2 : 1;
+    const int64_t rows[3] = {rows0, pair ? rows0 : rows1, rows2};
+    k.info.n_inputs = 1 + n_mat;
+    k.info.n_outputs = pair ? 1 : n_mat;
+    k.in_bytes[0] = (size_t)rows0 * (cols / 256) * 144; k.in_align[0] = 16;
+    k.in_bytes[1] = (round_xf_halves((int)cols) + 2 * round_sx_halves((int)cols)) * 2; k.in_align[1] = 16;
+    for (int i = 1; i < n_mat; i++) { k.in_bytes[1 + i] = (size_t)rows[i] * (cols / 256) * 144; k.in_align[1 + i] = 16; }
+    for (int i = 0; i < k.info.n_outputs; i++) { k.out_bytes[i] = (size_t)batch * rows[i] * 4; k.out_align[i] = 4; }
+    k.scratch_bytes = slices > 1 ? (size_t)slices * batch * rows0 * 4 : 0;
+    const int64_t tiles = pair ? (rows0 + 31) / 32 : (rows0 + 31) / 32 + (rows1 + 31) / 32 + (rows2 + 31) / 32;
+    set_launch(k, (uint32_t)tiles, (uint32_t)slices, 1, 512, (uint32_t)(8 * (pair ? 2 : 1) * 16 * 64 * 4));
+    k.info.sched = k.desc.sched;
+    k.info.sched.tg = 512; k.info.sched.nsg = 8; k.info.sched.nr0 = 32; k.info.sched.k_split = (uint32_t)slices; k.info.sched.lds_tile = 16;
+    set_name(k, "matvec_round_q4k_%s%s", pair ? "gate_up_gelu" : n_mat == 3 ? "x3" : n_mat == 2 ? "x2" : "x1", slices > 1 ? "_ksplit" : "");
+    k.launch = launch_matvec_round;
     return 0;
 }
 

@@ -64,6 +64,8 @@ class Kind(enum.IntEnum):           # enum ksh_kind
     MATVEC_GELU_MUL = 27
     READ_FLOOR = 28
     SDPA_BATCH = 29
+    ROUND_PREP = 30
+    MATVEC_ROUND = 31
 
 
 class Sched(C.Structure):           # ksh_sched: OptSchedule retargeted to gfx950

@@ -1,0 +1,101 @@
+"""The decode round's GEMMs (KSH_ROUND_PREP + KSH_MATVEC_ROUND: up to 16 f32 rows against Q4_K matrices on the matrix
+cores, several matrices or a gate | up pair per launch) vs the CPU oracle's dequant + sequential f32 dot per row,
+1e-3 relative; against the float64 product where the claim is the GEMV's accuracy; one-hot rows recover the
+dequantized columns."""
+import numpy as np
+import pytest
+
+import oracle
+from ksearch_amd import hip, synth
+from ksearch_amd.hip import DType, Kind
+from tests.gpu_util import assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = hip.Context()
+    yield c
+    c.close()
+
+
+def prepared(ctx, x, batch, cols):
+    kp = ctx.compile(hip.make_desc(Kind.ROUND_PREP, (cols, batch), (DType.F32,)))
+    xp = ctx.buffer_empty_bytes(64 * cols + 2048 * (cols // 256))
+    ctx.encode_multi(kp, [ctx.buffer_f32(x.reshape(-1))], [xp])
+    return xp
+
+
+def round_mm(ctx, ws, rows, cols, x, batch, pair=False):
+    xp = prepared(ctx, x, batch, cols)
+    r = list(rows) + [0] * (3 - len(rows))
+    k = ctx.compile(hip.make_desc(Kind.MATVEC_ROUND, (r[0], cols, batch, 0 if pair else r[1], r[2], int(pair)), (DType.Q4K,)))
+    bw = [ctx.buffer_bytes(w) for w in ws]
+    outs = [ctx.buffer_empty_f32(batch * rows[0])] if pair else [ctx.buffer_empty_f32(batch * n) for n in rows]
+    ctx.encode_multi(k, [bw[0], xp] + bw[1:], outs)
+    ctx.synchronize()
+    return k, [ctx.read_f32(o, batch * n).reshape(batch, n) for o, n in zip(outs, rows)]
+
+
+@pytest.mark.parametrize("rows,cols,batch", [
+    ((2048,), 1536, 16),            # q of the real checkpoints' layout
+    ((2048, 256, 256), 1536, 16),   # q | k | v in one launch
+    ((2048, 256), 2048, 5),         # two matrices, every wave busy
+    ((100,), 256, 1),               # one row of input, a ragged tile, one superblock
+    ((1536,), 6144, 16),            # down: columns split over three workgroups per tile
+    ((1536,), 12288, 7),            # the double-wide feed-forward: six slices
+    ((33, 1, 31), 512, 3),          # tiles that end inside a matrix
+])
+def test_matvec_round_vs_oracle(ctx, rows, cols, batch):
+    ws = [synth.q4k_blocks(n * cols // 256, seed=900 + i + n) for i, n in enumerate(rows)]
+    x = synth.normal_f32(batch * cols, 901).reshape(batch, cols)
+    k, got = round_mm(ctx, ws, rows, cols, x, batch)
+    assert ("ksplit" in k.name) == (cols > 2048)
+    for w, n, g in zip(ws, rows, got):
+        want = oracle.matmul(oracle.Q4K, w, n, cols, x, batch)
+        assert_close(g, want, 1e-3, f"round {n}x{cols} b{batch}")
+        for t in (0, batch - 1):   # the GEMV's accuracy: f32 activations keep 22 bits
+            w64 = oracle.matvec_f64(oracle.Q4K, w, n, cols, x[t])
+            err = np.max(np.abs(g[t] - w64) / np.maximum(np.abs(w64), np.sqrt(np.mean(w64 ** 2))))
+            assert err < 2e-5, err
+
+
+@pytest.mark.parametrize("rows,cols,batch", [(6144, 1536, 16), (12288, 1536, 3), (96, 2048, 9)])
+def test_matvec_round_gate_up_gelu(ctx, rows, cols, batch):
+    wg, wu = synth.q4k_blocks(rows * cols // 256, seed=910), synth.q4k_blocks(rows * cols // 256, seed=911)
+    x = synth.normal_f32(batch * cols, 912).reshape(batch, cols) * 0.25
+    k, (got,) = round_mm(ctx, [wg, wu], (rows,), cols, x, batch, pair=True)
+    assert "gate_up_gelu" in k.name
+    g, u = oracle.matmul(oracle.Q4K, wg, rows, cols, x, batch), oracle.matmul(oracle.Q4K, wu, rows, cols, x, batch)
+    assert_close(got, oracle.gelu_mul(g.reshape(-1), u.reshape(-1)).reshape(batch, rows), 1e-3, f"gate|up {rows}x{cols} b{batch}")
+
+
+def test_matvec_round_unit_rows_recover_weights(ctx):
+    # X = one-hot rows: Y[t] is column k_t of the dequantized matrix (pins the K order and the hi | lo tile end to end)
+    rows, cols = 64, 4096
+    w = synth.q4k_blocks(rows * cols // 256, seed=920)
+    wd = oracle.dequant(oracle.Q4K, w, rows * cols).reshape(rows, cols)
+    ks = [0, 1, 2, 3, 15, 16, 31, 32, 33, 63, 64, 255, 256, 2047, 2048, 4095]
+    x = np.zeros((len(ks), cols), dtype=np.float32)
+    for t, kk in enumerate(ks):
+        x[t, kk] = 1.0 + 2.0 ** -13      # a value whose lo part is not zero
+    _, (got,) = round_mm(ctx, [w], (rows,), cols, x, len(ks))
+    for t, kk in enumerate(ks):
+        want = wd[:, kk].astype(np.float64) * (1.0 + 2.0 ** -13)
+        assert np.allclose(got[t], want, rtol=1e-5, atol=1e-5 * np.abs(wd).max()), kk
+
+
+def test_matvec_round_errors(ctx):
+    with pytest.raises(hip.KshError, match="1 to 16"):
+        ctx.compile(hip.make_desc(Kind.ROUND_PREP, (1536, 17), (DType.F32,)))
+    with pytest.raises(hip.KshError, match="1 to 16"):
+        ctx.compile(hip.make_desc(Kind.MATVEC_ROUND, (64, 1536, 0, 0, 0, 0), (DType.Q4K,)))
+    with pytest.raises(hip.KshError, match="multiple of 256"):
+        ctx.compile(hip.make_desc(Kind.MATVEC_ROUND, (64, 100, 4, 0, 0, 0), (DType.Q4K,)))
+    with pytest.raises(hip.KshError, match="not built"):
+        ctx.compile(hip.make_desc(Kind.MATVEC_ROUND, (64, 1536, 4, 0, 0, 0), (DType.Q6K,)))
+    with pytest.raises(hip.KshError, match="one matrix per launch"):
+        ctx.compile(hip.make_desc(Kind.MATVEC_ROUND, (64, 4096, 4, 64, 0, 0), (DType.Q4K,)))
+    with pytest.raises(hip.KshError, match="one row count"):
+        ctx.compile(hip.make_desc(Kind.MATVEC_ROUND, (64, 1536, 4, 64, 0, 1), (DType.Q4K,)))

@@ -1094,8 +1094,18 @@ int encode_round4(ksh_gemma4 *m, ksh_kvpool *pool, int t, int max_batch, int poo
     }
     // logits and the greedy id of every row: the output norm rides in the LM head's prologue, as in the decode step
     ksh_buf *lm_w = m->embd_rows ? m->embd_rows : m->g.token_embd;
+    // the LM head once for all rows where the table is kept row-grouped (the matrix cores on exact codes, the int8
+    // scales applied in f32); row by row through the GEMV otherwise
+    const bool lm_batched = m->embd_rows && h % 256 == 0 && h <= 2048;
+    if (lm_batched) {
+        ksh_kernel *k_lm = nullptr;
+        if (enc(m, k_norm, {m->c_x, m->g.output_norm}, {m->c_x2}, n) || prep(h, m->c_x2) ||
+            get(m, KSH_MATVEC_ROUND, {c.vocab, h, t, 0, 0, 0}, {KSH_Q6K_ROWS}, {}, &k_lm) || enc(m, k_lm, {lm_w, m->r_xp}, {m->r_logits}, n))
+            return 1;
+    }
     for (int i = 0; i < t; i++)
-        if (run(m->k_lm_head[0], {lm_w, m->c_x, m->g.output_norm}, {0, (size_t)i * h * 4, 0}, {m->r_logits}, {(size_t)i * c.vocab * 4}) ||
+        if ((!lm_batched &&
+             run(m->k_lm_head[0], {lm_w, m->c_x, m->g.output_norm}, {0, (size_t)i * h * 4, 0}, {m->r_logits}, {(size_t)i * c.vocab * 4})) ||
             run(m->k_argmax, {m->r_logits}, {(size_t)i * c.vocab * 4}, {m->r_next}, {(size_t)i * 4}))
             return 1;
     return 0;

@@ -817,6 +817,109 @@ __global__ __launch_bounds__(256) void mm_round_fold_kernel(const float *__restr
     y[i] = s;
 }
 
+// The same round against a Q6_K matrix with row-grouped fields (KSH_Q6K_ROWS: the LM head as the decode loops keep it;
+// rows of up to 2048 columns).  The B operand is the 6-bit code minus 32 as an exact f16 integer (the code OR-ed into
+// the mantissa of 1024.0, minus 1056 with one packed subtraction per two weights); Q6_K has one int8 scale per 16
+// columns, which is the K depth of the matrix instruction, so the scale is applied in f32 to the instruction's
+// result: nothing is rounded (folded into the f16 operand as the 128 x 128 tile does it, sc * q above 2048 loses
+// its last bit).  A workgroup keeps the activations of the whole row in registers -- wave w the 16 fragments of
+// superblock w -- and walks tiles of 32 weight rows, the next tile's bytes in flight under the current one; the waves'
+// shares of a tile meet in LDS (two buffers, one barrier per tile).
+constexpr int kQ6rRowAlign = 16;
+__host__ __device__ inline size_t round_q6r_row_bytes(int bpr) { return ((size_t)bpr * 210 + kQ6rRowAlign - 1) / kQ6rRowAlign * kQ6rRowAlign; }
+
+struct Round6Params {
+    const uint8_t *W;
+    float *Y;
+    int rows, cols, batch, tiles, tiles_per_wg;
+    const _Float16 *Xp;
+};
+
+struct Q6Tile {
+    u32x2_t ql[2][2][2];   // [half][quadrant parity][low / high 16 positions]: bytes 8h .. 8h+7 of them
+    u32x2_t qh[2][2];      // [half][low / high 16 positions]
+    u32x4_t sc;            // the superblock's 16 int8 scales
+    uint32_t d;
+};
+
+__global__ __launch_bounds__(512) void q6r_mm_round_kernel(Round6Params p)
+{
+    extern __shared__ __attribute__((aligned(16))) float red[];   // [2][8 waves][8][64]
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 31, h = lane >> 5;
+    const int bpr = p.cols / 256;
+    const bool active = wave < bpr;                       // (wave-uniform: a row of 1536 columns leaves two waves idle)
+    const int sbc = min(wave, bpr - 1);
+    const size_t row_bytes = round_q6r_row_bytes(bpr);
+    const h8 *xa = reinterpret_cast<const h8 *>(p.Xp) + (size_t)sbc * 16 * 64 + lane;
+    h8 a[16];
+#pragma unroll
+    for (int j = 0; j < 16; j++) a[j] = xa[(size_t)j * 64];
+    auto load_tile = [&](Q6Tile &dst, int tile) {
+        const uint8_t *rp = p.W + (size_t)min(tile * 32 + n, p.rows - 1) * row_bytes;
+#pragma unroll
+        for (int ip = 0; ip < 2; ip++)
+#pragma unroll
+            for (int lh = 0; lh < 2; lh++) {
+#pragma unroll
+                for (int par = 0; par < 2; par++)
+                    dst.ql[ip][par][lh] = *reinterpret_cast<const u32x2_t *>(rp + (size_t)sbc * 128 + 64 * ip + 32 * par + 16 * lh + 8 * h);
+                dst.qh[ip][lh] = *reinterpret_cast<const u32x2_t *>(rp + (size_t)bpr * 128 + (size_t)sbc * 64 + 32 * ip + 16 * lh + 8 * h);
+            }
+        dst.sc = *reinterpret_cast<const u32x4_t *>(rp + (size_t)bpr * 192 + (size_t)sbc * 16);
+        dst.d = *reinterpret_cast<const uint16_t *>(rp + (size_t)bpr * 208 + (size_t)sbc * 2);
+    };
+    const int tile0 = blockIdx.x * p.tiles_per_wg, tile1 = min(tile0 + p.tiles_per_wg, p.tiles);
+    if (tile0 >= tile1) return;
+    uint32_t byte_mask = 0x00FF00FFu, bias = 0x64006400u;   // in registers: the and-or is then one instruction
+    asm volatile("" : "+v"(byte_mask), "+v"(bias));
+    const h8 k1056 = {(_Float16)1056.f, (_Float16)1056.f, (_Float16)1056.f, (_Float16)1056.f,
+                      (_Float16)1056.f, (_Float16)1056.f, (_Float16)1056.f, (_Float16)1056.f};
+    const f16v kZero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    Q6Tile cur, nxt;
+    load_tile(cur, tile0);
+    int buf = 0;
+    for (int tile = tile0; tile < tile1; tile++) {
+        load_tile(nxt, min(tile + 1, tile1 - 1));
+        f16v G = kZero16;
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            // group j: half ip, quadrant q, positions 16 lh .. +15; element 16 j of the superblock onwards
+            const int ip = j >> 3, q = (j >> 1) & 3, lh = j & 1;
+            const u32x2_t ql2 = cur.ql[ip][q & 1][lh], qh2 = cur.qh[ip][lh];
+            uint32_t o[4];
+#pragma unroll
+            for (int dw = 0; dw < 2; dw++) {
+                const uint32_t lo4 = (ql2[dw] >> (4 * (q >> 1))) & 0x0F0F0F0Fu, hi2 = (qh2[dw] >> (2 * q)) & 0x03030303u;
+                const uint32_t code = lo4 | (hi2 << 4);
+                o[2 * dw] = (code & byte_mask) | bias;              // codes of bytes 0 and 2 as 1024 + c
+                o[2 * dw + 1] = ((code >> 8) & byte_mask) | bias;   // bytes 1 and 3: the order the fragments keep
+            }
+            const u32x4_t ov = {o[0], o[1], o[2], o[3]};
+            const h8 b = __builtin_bit_cast(h8, ov) - k1056;
+            const f16v C = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[j], b, kZero16, 0, 0, 0);
+            const float sc = (float)(int)(int8_t)(cur.sc[j >> 2] >> (8 * (j & 3)));
+#pragma unroll
+            for (int i = 0; i < 16; i++) G[i] = fmaf(sc, C[i], G[i]);
+        }
+        // accumulator i of lane (n, h) is row 8*(i/4) + 4*h + i%4 of the tile: i < 8 a token's hi part, i + 8 its lo part
+        const float d = active ? half_bits_to_f32(cur.d) : 0.f;
+        float *mine = red + (size_t)(buf * 8 + wave) * 8 * 64 + lane;
+#pragma unroll
+        for (int i = 0; i < 8; i++) mine[i * 64] = d * fmaf(1.0f / 2048.0f, G[i + 8], G[i]);
+        __syncthreads();
+        {
+            const int i = wave, t = 8 * (i >> 2) + 4 * h + (i & 3), r = tile * 32 + n;
+            float sum = 0.f;
+#pragma unroll
+            for (int w = 0; w < 8; w++) sum += red[(size_t)((buf * 8 + w) * 8 + i) * 64 + lane];
+            if (t < p.batch && r < p.rows) p.Y[(size_t)t * p.rows + r] = sum;
+        }
+        buf ^= 1;
+        cur = nxt;
+    }
+}
+
 int launch_round_prep(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
 {
     const int cols = (int)k.desc.dims[0], batch = (int)k.desc.dims[1];
@@ -829,6 +932,18 @@ int launch_round_prep(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
 int launch_matvec_round(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
 {
     const int64_t *d = k.desc.dims;
+    if (k.desc.dtypes[0] == KSH_Q6K_ROWS) {
+        Round6Params p6{};
+        p6.W = (const uint8_t *)a.in[0];
+        p6.Xp = (const _Float16 *)a.in[1];
+        p6.Y = (float *)a.out[0];
+        p6.rows = (int)d[0]; p6.cols = (int)d[1]; p6.batch = (int)d[2];
+        p6.tiles = (p6.rows + 31) / 32;
+        p6.tiles_per_wg = (p6.tiles + (int)k.info.grid[0] - 1) / (int)k.info.grid[0];
+        hipLaunchKernelGGL(q6r_mm_round_kernel, dim3(k.info.grid[0]), dim3(512), k.info.lds_bytes, st, p6);
+        const hipError_t e6 = hipGetLastError();
+        return e6 == hipSuccess ? 0 : hip_fail(e6, "matvec_round (Q6_K rows) launch");
+    }
     const bool pair = d[5] != 0;
     const int n_mat = pair ? 2 : d[4] ? 3 : d[3] ? 2 : 1;
     RoundParams p{};
@@ -960,9 +1075,28 @@ int bind_matvec_round(ksh_kernel &k)
     const int64_t *d = k.desc.dims;
     const int64_t rows0 = d[0], cols = d[1], batch = d[2], rows1 = d[3], rows2 = d[4];
     const bool pair = d[5] != 0;
-    if (k.desc.dtypes[0] != KSH_Q4K) return set_error("matvec_round: weight dtype %d is not built (Q4_K is)", k.desc.dtypes[0]);
+    const bool q6r = k.desc.dtypes[0] == KSH_Q6K_ROWS;
+    if (k.desc.dtypes[0] != KSH_Q4K && !q6r) return set_error("matvec_round: weight dtype %d is not built (Q4_K and row-grouped Q6_K are)", k.desc.dtypes[0]);
     if (cols <= 0 || cols % 256 || cols > (1 << 16)) return set_error("matvec_round: cols=%lld is not a positive multiple of 256 up to 65536", (long long)cols);
     if (batch < 1 || batch > kRoundTokens) return set_error("matvec_round: %lld rows (1 to %d)", (long long)batch, kRoundTokens);
+    if (q6r) {
+        if (rows1 || rows2 || pair) return set_error("matvec_round: row-grouped Q6_K takes one matrix per launch");
+        if (cols > 2048) return set_error("matvec_round: row-grouped Q6_K rows of up to 2048 columns (cols=%lld)", (long long)cols);
+        if (rows0 <= 0 || rows0 > (1 << 24)) return set_error("matvec_round: rows %lld", (long long)rows0);
+        k.info.n_inputs = 2;
+        k.info.n_outputs = 1;
+        k.in_bytes[0] = (size_t)rows0 * round_q6r_row_bytes((int)(cols / 256)); k.in_align[0] = 16;
+        k.in_bytes[1] = (round_xf_halves((int)cols) + 2 * round_sx_halves((int)cols)) * 2; k.in_align[1] = 16;
+        k.out_bytes[0] = (size_t)batch * rows0 * 4; k.out_align[0] = 4;
+        // one workgroup per compute unit (its registers hold the activations of a whole row), tiles shared out evenly
+        const int64_t tiles = (rows0 + 31) / 32, per = (tiles + 255) / 256;
+        set_launch(k, (uint32_t)((tiles + per - 1) / per), 1, 1, 512, (uint32_t)(2 * 8 * 8 * 64 * 4));
+        k.info.sched = k.desc.sched;
+        k.info.sched.tg = 512; k.info.sched.nsg = 8; k.info.sched.nr0 = 32; k.info.sched.k_split = 1; k.info.sched.lds_tile = 16;
+        set_name(k, "matvec_round_q6krows");
+        k.launch = launch_matvec_round;
+        return 0;
+    }
     if (rows0 <= 0 || rows1 < 0 || rows2 < 0 || (rows2 && !rows1) || rows0 + rows1 + rows2 > (1 << 24))
         return set_error("matvec_round: rows %lld / %lld / %lld", (long long)rows0, (long long)rows1, (long long)rows2);
     if (pair && (rows1 || rows2)) return set_error("matvec_round: a gate | up pair names one row count (both matrices have it)");

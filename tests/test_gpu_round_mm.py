@@ -8,7 +8,7 @@ import pytest
 import oracle
 from ksearch_amd import hip, synth
 from ksearch_amd.hip import DType, Kind
-from tests.gpu_util import assert_close
+from tests.gpu_util import assert_close, q6k_rows
 
 pytestmark = pytest.mark.gpu
 
@@ -86,6 +86,49 @@ def test_matvec_round_unit_rows_recover_weights(ctx):
         assert np.allclose(got[t], want, rtol=1e-5, atol=1e-5 * np.abs(wd).max()), kk
 
 
+def q6k_blocks_full_scales(n_blocks, seed):
+    """Q6_K blocks whose int8 scales use the whole range (sc * q up to 127 * 32: what an f16 operand would round)."""
+    w = synth.q6k_blocks(n_blocks, seed=seed).reshape(n_blocks, 210).copy()
+    w[:, 192:208] = np.random.default_rng(seed + 1).integers(-128, 128, (n_blocks, 16)).astype(np.int8).view(np.uint8)
+    return w.reshape(-1)
+
+
+@pytest.mark.parametrize("rows,cols,batch,full", [(8192, 1536, 16, False), (4096, 2048, 7, True), (100, 1536, 1, True), (20000, 2048, 16, False)])
+def test_matvec_round_q6k_rows(ctx, rows, cols, batch, full):
+    """The LM head of a round: row-grouped Q6_K, the scale applied in f32 to the matrix instruction's result, so the
+    GEMV's accuracy also holds where |sc * q| passes 2048."""
+    nb = rows * cols // 256
+    w = q6k_blocks_full_scales(nb, 930) if full else synth.q6k_blocks(nb, seed=930)
+    x = synth.normal_f32(batch * cols, 931).reshape(batch, cols)
+    xp = prepared(ctx, x, batch, cols)
+    k = ctx.compile(hip.make_desc(Kind.MATVEC_ROUND, (rows, cols, batch, 0, 0, 0), (DType.Q6K_ROWS,)))
+    y = ctx.buffer_empty_f32(batch * rows)
+    ctx.encode_multi(k, [ctx.buffer_bytes(q6k_rows(w, rows, cols)), xp], [y])
+    got = ctx.read_f32(y, batch * rows).reshape(batch, rows)
+    assert_close(got, oracle.matmul(oracle.Q6K, w, rows, cols, x, batch), 1e-3, f"round q6k rows {rows}x{cols} b{batch}")
+    for t in (0, batch - 1):
+        w64 = oracle.matvec_f64(oracle.Q6K, w, rows, cols, x[t])
+        err = np.max(np.abs(got[t] - w64) / np.maximum(np.abs(w64), np.sqrt(np.mean(w64 ** 2))))
+        assert err < 2e-5, err
+
+
+def test_matvec_round_q6k_rows_unit_rows_recover_weights(ctx):
+    rows, cols = 64, 2048
+    w = q6k_blocks_full_scales(rows * cols // 256, 940)
+    wd = oracle.dequant(oracle.Q6K, w, rows * cols).reshape(rows, cols)
+    ks = [0, 1, 7, 8, 15, 16, 31, 32, 63, 64, 127, 128, 255, 256, 1000, 2047]
+    x = np.zeros((len(ks), cols), dtype=np.float32)
+    for t, kk in enumerate(ks):
+        x[t, kk] = 1.0
+    xp = prepared(ctx, x, len(ks), cols)
+    k = ctx.compile(hip.make_desc(Kind.MATVEC_ROUND, (rows, cols, len(ks), 0, 0, 0), (DType.Q6K_ROWS,)))
+    y = ctx.buffer_empty_f32(len(ks) * rows)
+    ctx.encode_multi(k, [ctx.buffer_bytes(q6k_rows(w, rows, cols)), xp], [y])
+    got = ctx.read_f32(y, len(ks) * rows).reshape(len(ks), rows)
+    for t, kk in enumerate(ks):
+        assert np.array_equal(got[t], wd[:, kk]), kk      # d * sc * (q - 32): exact in f32
+
+
 def test_matvec_round_errors(ctx):
     with pytest.raises(hip.KshError, match="1 to 16"):
         ctx.compile(hip.make_desc(Kind.ROUND_PREP, (1536, 17), (DType.F32,)))
@@ -95,6 +138,8 @@ def test_matvec_round_errors(ctx):
         ctx.compile(hip.make_desc(Kind.MATVEC_ROUND, (64, 100, 4, 0, 0, 0), (DType.Q4K,)))
     with pytest.raises(hip.KshError, match="not built"):
         ctx.compile(hip.make_desc(Kind.MATVEC_ROUND, (64, 1536, 4, 0, 0, 0), (DType.Q6K,)))
+    with pytest.raises(hip.KshError, match="up to 2048 columns"):
+        ctx.compile(hip.make_desc(Kind.MATVEC_ROUND, (64, 4096, 4, 0, 0, 0), (DType.Q6K_ROWS,)))
     with pytest.raises(hip.KshError, match="one matrix per launch"):
         ctx.compile(hip.make_desc(Kind.MATVEC_ROUND, (64, 4096, 4, 64, 0, 0), (DType.Q4K,)))
     with pytest.raises(hip.KshError, match="one row count"):

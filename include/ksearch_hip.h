@@ -209,8 +209,13 @@ enum ksh_kind {
      * that reads them.  No counterpart in the reference, whose round is one decode step per request
      * (crates/ksearch_cli/src/scheduler.rs:163-231).  The operand holds x = hi + 2^-11 lo as f16 fragments of the
      * matrix instruction (a token's hi and lo part in one tile) and the per-sub-block sums of x.
-     * dims: cols (a multiple of 256), batch (1..16).  in: x f32[batch, cols]
-     * out: xp, 64 * cols + 2048 * (cols / 256) bytes, 16-byte aligned */
+     * dims: cols (a multiple of 256), batch (1..16), mode.  params: eps (modes 1, 2)
+     *   mode 0: in: x f32[batch, cols]                         out: xp
+     *   mode 1: the rows' RMSNorm on the way (rmsnorm_rows, crates/ksearch_kernels/src/lib.rs:1478):
+     *           in: x, w f32[cols]                              out: xp of (x * inv) * w
+     *   mode 2: rmsnorm_add_then_rmsnorm on rows: in: y, w_post, res, w_norm   out: xp, x_new f32[batch, cols]
+     *           with x_new = res + (y * inv) * w_post (may be res) and xp of (x_new * inv2) * w_norm
+     * xp: 64 * cols + 2048 * (cols / 256) bytes, 16-byte aligned */
     KSH_ROUND_PREP = 30,
     /* Up to three Q4_K matrices of one width against one prepared operand, in one launch (q | k | v share their
      * input), or a gate | up pair stored as gelu(gate) * up (Eng::matvec_batch, crates/ksearch_kernels/src/lib.rs:

@@ -1010,6 +1010,11 @@ int encode_round4(ksh_gemma4 *m, ksh_kvpool *pool, int t, int max_batch, int poo
         ksh_kernel *kk = nullptr;
         return get(m, KSH_ROUND_PREP, {cols, t}, {KSH_F32}, {}, &kk) || enc(m, kk, {x}, {m->r_xp}, n);
     };
+    // (a norm whose only readers are such GEMMs writes the operand itself)
+    auto prep_norm = [&](int64_t cols, ksh_buf *x, ksh_buf *w) -> int {
+        ksh_kernel *kk = nullptr;
+        return get(m, KSH_ROUND_PREP, {cols, t, 1}, {KSH_F32}, {c.eps}, &kk) || enc(m, kk, {x, w}, {m->r_xp}, n);
+    };
     auto mm1 = [&](int dt, int64_t rows, int64_t cols, ksh_buf *w, ksh_buf *x, ksh_buf *y) -> int {
         ksh_kernel *kk = nullptr;
         if (dt != KSH_Q4K) return mm(dt, rows, cols, w, x, y);
@@ -1041,11 +1046,11 @@ int encode_round4(ksh_gemma4 *m, ksh_kvpool *pool, int t, int max_batch, int poo
         ksh_kernel *k_head = nullptr, *k_sdpa = nullptr, *k_gelu = nullptr;
         if (!sdpa_lanes_supports(c.n_q, c.n_kv, P.hd))
             return set_error("ksh_gemma4_decode_round: attention over several slots is built for heads of 128 / 256 / 512 with up to 8 q heads per kv head");
-        if (enc(m, k_norm, {m->c_x, L.attn_norm}, {m->c_x2}, n)) return 1;
         const bool qkv_q4k = L.dt_q == KSH_Q4K && (!P.owns || (L.dt_k == KSH_Q4K && L.dt_v == KSH_Q4K));
+        if (!qkv_q4k && enc(m, k_norm, {m->c_x, L.attn_norm}, {m->c_x2}, n)) return 1;
         if (qkv_q4k) {
             ksh_kernel *kq = nullptr;
-            if (prep(h, m->c_x2)) return 1;
+            if (prep_norm(h, m->c_x, L.attn_norm)) return 1;
             if (P.owns ? (get(m, KSH_MATVEC_ROUND, {P.qd, h, t, P.kvd, P.kvd, 0}, {KSH_Q4K}, {}, &kq) ||
                           enc(m, kq, {L.wq, m->r_xp, L.wk, L.wv}, {m->c_q, m->c_k, m->c_v}, n))
                        : (get(m, KSH_MATVEC_ROUND, {P.qd, h, t, 0, 0, 0}, {KSH_Q4K}, {}, &kq) || enc(m, kq, {L.wq, m->r_xp}, {m->c_q}, n)))
@@ -1067,12 +1072,15 @@ int encode_round4(ksh_gemma4 *m, ksh_kvpool *pool, int t, int max_batch, int poo
         if (get(m, KSH_SDPA_SLOTS, {c.n_q, c.n_kv, P.hd, c.max_seq, t, kRoundPartitions, max_batch, (int64_t)slot_stride}, {KSH_Q40, KSH_F32},
                 {c.attn_scale}, &k_sdpa) ||
             run(k_sdpa, {m->c_q, kc, vc, m->r_tab, m->r_tab}, {0, 0, 0, o_meta, o_slots}, {m->c_tmp, m->c_o}, {0, 0}) ||
-            mm1(L.dt_o, h, P.qd, L.wo, m->c_o, m->c_y) ||
-            enc(m, k_add_then, {m->c_y, L.post_attn_norm, m->c_x, L.ffn_norm}, {m->c_x, m->c_x2}, n))
+            mm1(L.dt_o, h, P.qd, L.wo, m->c_o, m->c_y))
             return 1;
-        if (L.dt_gate == KSH_Q4K && L.dt_up == KSH_Q4K) {
-            ksh_kernel *k_gu = nullptr;
-            if (prep(h, m->c_x2) || get(m, KSH_MATVEC_ROUND, {L.ffn, h, t, 0, 0, 1}, {KSH_Q4K}, {}, &k_gu) ||
+        const bool gu_q4k = L.dt_gate == KSH_Q4K && L.dt_up == KSH_Q4K && h <= 8192;
+        if (!gu_q4k && enc(m, k_add_then, {m->c_y, L.post_attn_norm, m->c_x, L.ffn_norm}, {m->c_x, m->c_x2}, n)) return 1;
+        if (gu_q4k) {
+            ksh_kernel *k_gu = nullptr, *k_pn = nullptr;
+            if (get(m, KSH_ROUND_PREP, {h, t, 2}, {KSH_F32}, {c.eps}, &k_pn) ||
+                enc(m, k_pn, {m->c_y, L.post_attn_norm, m->c_x, L.ffn_norm}, {m->r_xp, m->c_x}, n) ||
+                get(m, KSH_MATVEC_ROUND, {L.ffn, h, t, 0, 0, 1}, {KSH_Q4K}, {}, &k_gu) ||
                 enc(m, k_gu, {L.wgate, m->r_xp, L.wup}, {m->c_ff}, n))
                 return 1;
         } else if (mm(L.dt_gate, L.ffn, h, L.wgate, m->c_x2, m->c_g) || mm(L.dt_up, L.ffn, h, L.wup, m->c_x2, m->c_u) ||
@@ -1099,7 +1107,7 @@ int encode_round4(ksh_gemma4 *m, ksh_kvpool *pool, int t, int max_batch, int poo
     const bool lm_batched = m->embd_rows && h % 256 == 0 && h <= 2048;
     if (lm_batched) {
         ksh_kernel *k_lm = nullptr;
-        if (enc(m, k_norm, {m->c_x, m->g.output_norm}, {m->c_x2}, n) || prep(h, m->c_x2) ||
+        if (prep_norm(h, m->c_x, m->g.output_norm) ||
             get(m, KSH_MATVEC_ROUND, {c.vocab, h, t, 0, 0, 0}, {KSH_Q6K_ROWS}, {}, &k_lm) || enc(m, k_lm, {lm_w, m->r_xp}, {m->r_logits}, n))
             return 1;
     }

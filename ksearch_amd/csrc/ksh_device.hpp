@@ -92,6 +92,16 @@ __device__ __forceinline__ float row16_sum(float v)
 }
 
 // sum over the whole wave64, result wave-uniform
+// A value about to be split into hi = f16(x) and lo = f16(x - hi): pinned to a register first.  Where x is a product
+// (or sum) the compiler sees, it folds the conversion of hi into a mixed-precision fma that rounds the exact product
+// once in one use and converts the rounded f32 in another; at a rounding tie the two differ by an f16 ulp and the
+// parts then belong to different values.
+__device__ __forceinline__ float pinned(float x)
+{
+    asm volatile("" : "+v"(x));
+    return x;
+}
+
 __device__ __forceinline__ float wave_sum(float v)
 {
     v = row16_sum(v);

@@ -80,6 +80,7 @@ __global__ __launch_bounds__(256) void mm_prep_x_kernel(const uint16_t *__restri
     reinterpret_cast<h8 *>(Xf)[((size_t)(t >> 5) * (cols / 16) + (j >> 1)) * 64 + (t & 31) + 32 * (j & 1)] = o;
     if ((threadIdx.x & 3) == 0) {
         const int s = j / 4;
+        sum = pinned(sum);
         const _Float16 hi = (_Float16)sum;
         const _Float16 lo = (_Float16)(sum - (float)hi);
         _Float16 *a2 = SxA + ((size_t)t * (cols / 256) + s / 8) * 32;
@@ -130,8 +131,9 @@ __global__ __launch_bounds__(256) void mm_prep_x_f32_kernel(const float *__restr
         _Float16 *dst[2] = {SxA_hi + o, SxA_lo + o};
 #pragma unroll
         for (int part = 0; part < 2; part++) {
-            const _Float16 hi = (_Float16)sums[part];
-            const _Float16 lo = (_Float16)(sums[part] - (float)hi);
+            const float sum = pinned(sums[part]);
+            const _Float16 hi = (_Float16)sum;
+            const _Float16 lo = (_Float16)(sum - (float)hi);
             dst[part][jj] = hi;
             dst[part][8 + jj] = hi;
             dst[part][16 + jj] = lo;
@@ -337,7 +339,7 @@ __global__ __launch_bounds__(kThreadsMM) void q_mul_mm_kernel(MmParams p)
 #pragma unroll
                 for (int gg = 0; gg < 2; gg++) {
                     const uint4 s = q4k_group_scales(w.hdr.y, w.hdr.z, w.hdr.w, 2 * lh + gg);
-                    const float c0 = -(dmin * (float)s.y + 1024.f * d), c1 = -(dmin * (float)s.w + 1024.f * d);
+                    const float c0 = pinned(-(dmin * (float)s.y + 1024.f * d)), c1 = pinned(-(dmin * (float)s.w + 1024.f * d));
                     const _Float16 h0 = (_Float16)c0, h1 = (_Float16)c1;
                     const _Float16 l0 = (_Float16)(c0 - (float)h0), l1 = (_Float16)(c1 - (float)h1);
                     hi2[gg] = (uint32_t)__builtin_bit_cast(uint16_t, h0) | ((uint32_t)__builtin_bit_cast(uint16_t, h1) << 16);
@@ -573,7 +575,7 @@ __global__ __launch_bounds__(512) void q4k_mm_skinny_kernel(MmParams p, const _F
 #pragma unroll
         for (int g = 0; g < 4; g++) {
             const uint4 s = q4k_group_scales(hdr.y, hdr.z, hdr.w, g);
-            const float c0 = -(dmin * (float)s.y + 1024.f * d), c1 = -(dmin * (float)s.w + 1024.f * d);
+            const float c0 = pinned(-(dmin * (float)s.y + 1024.f * d)), c1 = pinned(-(dmin * (float)s.w + 1024.f * d));
             chi[2 * g] = (_Float16)c0; chi[2 * g + 1] = (_Float16)c1;
             clo[2 * g] = (_Float16)(c0 - (float)chi[2 * g]); clo[2 * g + 1] = (_Float16)(c1 - (float)chi[2 * g + 1]);
         }
@@ -638,19 +640,10 @@ constexpr int kRoundTokens = 16;
 __host__ __device__ inline size_t round_xf_halves(int cols) { return (size_t)32 * cols; }
 __host__ __device__ inline size_t round_sx_halves(int cols) { return (size_t)kRoundTokens * (cols / 256) * 32; }
 
-// one thread per 8 elements of the 16 token rows (rows past the batch are written as zeros)
-__global__ __launch_bounds__(256) void mm_round_prep_kernel(const float *__restrict__ X, _Float16 *__restrict__ Xp, int batch, int cols)
+// what one thread does with 8 consecutive elements (8 j .. 8 j + 7) of token row t; whole quads call it together
+// (the four threads of a sub-block add their sums up over the quad)
+__device__ __forceinline__ void round_prep_write(const float (&f)[8], int t, int j, int cols, _Float16 *__restrict__ Xp)
 {
-    const int idx = blockIdx.x * 256 + threadIdx.x;
-    const int k8 = cols / 8;
-    if (idx >= kRoundTokens * k8) return;   // (whole quads: cols is a multiple of 32)
-    const int t = idx / k8, j = idx - t * k8;
-    f32x4_t in0 = {0.f, 0.f, 0.f, 0.f}, in1 = in0;
-    if (t < batch) {
-        in0 = reinterpret_cast<const f32x4_t *>(X)[2 * ((size_t)t * k8 + j)];
-        in1 = reinterpret_cast<const f32x4_t *>(X)[2 * ((size_t)t * k8 + j) + 1];
-    }
-    const float f[8] = {in0.x, in0.y, in0.z, in0.w, in1.x, in1.y, in1.z, in1.w};
     h8 oh, ol;
     float fh[8], fl[8];
 #pragma unroll
@@ -679,13 +672,85 @@ __global__ __launch_bounds__(256) void mm_round_prep_kernel(const float *__restr
 #pragma unroll
         for (int part = 0; part < 2; part++) {
             _Float16 *dst = sx + part * round_sx_halves(cols);
-            const _Float16 hi = (_Float16)sums[part];
-            const _Float16 lo = (_Float16)(sums[part] - (float)hi);
+            const float sum = pinned(sums[part]);
+            const _Float16 hi = (_Float16)sum;
+            const _Float16 lo = (_Float16)(sum - (float)hi);
             dst[jj] = hi;
             dst[8 + jj] = hi;
             dst[16 + jj] = lo;
             dst[24 + jj] = (_Float16)0.f;
         }
+    }
+}
+
+// one thread per 8 elements of the 16 token rows (rows past the batch are written as zeros)
+__global__ __launch_bounds__(256) void mm_round_prep_kernel(const float *__restrict__ X, _Float16 *__restrict__ Xp, int batch, int cols)
+{
+    const int idx = blockIdx.x * 256 + threadIdx.x;
+    const int k8 = cols / 8;
+    if (idx >= kRoundTokens * k8) return;   // (whole quads: cols is a multiple of 32)
+    const int t = idx / k8, j = idx - t * k8;
+    f32x4_t in0 = {0.f, 0.f, 0.f, 0.f}, in1 = in0;
+    if (t < batch) {
+        in0 = reinterpret_cast<const f32x4_t *>(X)[2 * ((size_t)t * k8 + j)];
+        in1 = reinterpret_cast<const f32x4_t *>(X)[2 * ((size_t)t * k8 + j) + 1];
+    }
+    const float f[8] = {in0.x, in0.y, in0.z, in0.w, in1.x, in1.y, in1.z, in1.w};
+    round_prep_write(f, t, j, cols, Xp);
+}
+
+// The rows forms of the norms (rmsnorm_rows, rmsnorm_add_then_rmsnorm rows: crates/ksearch_kernels/src/lib.rs:1478-1560)
+// with the prepared operand as their output: one workgroup per token row, the same sums in the same order as the
+// kernels that write f32 rows (explicitly rounded products and sums: nothing is contracted).
+//   MODE 1:  v = (x * inv) * w                                                     -> xp
+//   MODE 2:  x_new = res + (y * inv) * w_post;  v = (x_new * inv2) * w_norm        -> xp, x_new (may be res)
+__device__ __forceinline__ float round_block_sum(float v, float *red)
+{
+    v = wave_sum(v);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    __syncthreads();                       // (red may still be read from the previous sum)
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    return (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+template <int MODE>
+__global__ __launch_bounds__(256) void mm_round_prep_norm_kernel(const float *__restrict__ x, const float *__restrict__ w_first, const float *res,
+                                                                 const float *__restrict__ w_norm, float *x_new, _Float16 *__restrict__ Xp,
+                                                                 int batch, int cols, float eps)
+{
+    __shared__ float red[4];
+    extern __shared__ float mid[];      // MODE 2: the row between the two norms
+    const int t = blockIdx.x, k8 = cols / 8;
+    if (t >= batch) {
+        const float zero[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        for (int j = threadIdx.x; j < k8; j += 256) round_prep_write(zero, t, j, cols, Xp);
+        return;
+    }
+    x += (size_t)t * cols;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < cols; i += 256) ss = __fadd_rn(ss, __fmul_rn(x[i], x[i]));
+    ss = round_block_sum(ss, red);
+    float inv = 1.0f / sqrtf(__fadd_rn(ss / (float)cols, eps));
+    if (MODE == 2) {
+        res += (size_t)t * cols;
+        x_new += (size_t)t * cols;
+        float ss2 = 0.f;
+        for (int i = threadIdx.x; i < cols; i += 256) {
+            const float v = __fadd_rn(res[i], __fmul_rn(__fmul_rn(x[i], inv), w_first[i]));
+            mid[i] = v;
+            x_new[i] = v;
+            ss2 = __fadd_rn(ss2, __fmul_rn(v, v));
+        }
+        ss2 = round_block_sum(ss2, red);
+        inv = 1.0f / sqrtf(__fadd_rn(ss2 / (float)cols, eps));
+    }
+    const float *src = MODE == 2 ? mid : x, *w = MODE == 2 ? w_norm : w_first;
+    for (int j = threadIdx.x; j < k8; j += 256) {
+        float f[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) f[i] = pinned(__fmul_rn(__fmul_rn(src[8 * j + i], inv), w[8 * j + i]));
+        round_prep_write(f, t, j, cols, Xp);
     }
 }
 
@@ -770,7 +835,7 @@ __global__ __launch_bounds__(512) void q4k_mm_round_kernel(RoundParams p)
 #pragma unroll
         for (int g = 0; g < 4; g++) {
             const uint4 s = q4k_group_scales(hdr[m].y, hdr[m].z, hdr[m].w, g);
-            const float c0 = -(dmin * (float)s.y + 1024.f * d), c1 = -(dmin * (float)s.w + 1024.f * d);
+            const float c0 = pinned(-(dmin * (float)s.y + 1024.f * d)), c1 = pinned(-(dmin * (float)s.w + 1024.f * d));
             chi[2 * g] = (_Float16)c0; chi[2 * g + 1] = (_Float16)c1;
             clo[2 * g] = (_Float16)(c0 - (float)chi[2 * g]); clo[2 * g + 1] = (_Float16)(c1 - (float)chi[2 * g + 1]);
         }
@@ -922,9 +987,16 @@ __global__ __launch_bounds__(512) void q6r_mm_round_kernel(Round6Params p)
 
 int launch_round_prep(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
 {
-    const int cols = (int)k.desc.dims[0], batch = (int)k.desc.dims[1];
+    const int cols = (int)k.desc.dims[0], batch = (int)k.desc.dims[1], mode = (int)k.desc.dims[2];
     const int n = kRoundTokens * (cols / 8);
-    hipLaunchKernelGGL(mm_round_prep_kernel, dim3((n + 255) / 256), dim3(256), 0, st, (const float *)a.in[0], (_Float16 *)a.out[0], batch, cols);
+    if (mode == 1)
+        hipLaunchKernelGGL(mm_round_prep_norm_kernel<1>, dim3(kRoundTokens), dim3(256), 0, st, (const float *)a.in[0], (const float *)a.in[1], nullptr, nullptr,
+                           nullptr, (_Float16 *)a.out[0], batch, cols, k.desc.params[0]);
+    else if (mode == 2)
+        hipLaunchKernelGGL(mm_round_prep_norm_kernel<2>, dim3(kRoundTokens), dim3(256), (size_t)cols * 4, st, (const float *)a.in[0], (const float *)a.in[1],
+                           (const float *)a.in[2], (const float *)a.in[3], (float *)a.out[1], (_Float16 *)a.out[0], batch, cols, k.desc.params[0]);
+    else
+        hipLaunchKernelGGL(mm_round_prep_kernel, dim3((n + 255) / 256), dim3(256), 0, st, (const float *)a.in[0], (_Float16 *)a.out[0], batch, cols);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : hip_fail(e, "round_prep launch");
 }
@@ -1057,15 +1129,24 @@ int bind_matvec_batch(ksh_kernel &k)
 
 int bind_round_prep(ksh_kernel &k)
 {
-    const int64_t cols = k.desc.dims[0], batch = k.desc.dims[1];
+    const int64_t cols = k.desc.dims[0], batch = k.desc.dims[1], mode = k.desc.dims[2];
     if (cols <= 0 || cols % 256 || cols > (1 << 16)) return set_error("round_prep: cols=%lld is not a positive multiple of 256 up to 65536", (long long)cols);
     if (batch < 1 || batch > kRoundTokens) return set_error("round_prep: %lld rows (1 to %d)", (long long)batch, kRoundTokens);
-    k.info.n_inputs = 1;
-    k.info.n_outputs = 1;
+    if (mode < 0 || mode > 2) return set_error("round_prep: mode %lld (0 plain, 1 rmsnorm, 2 add then rmsnorm)", (long long)mode);
+    if (mode == 2 && cols > 8192) return set_error("round_prep: the add-then-norm form keeps a row in LDS (cols=%lld, up to 8192)", (long long)cols);
+    k.info.n_inputs = mode == 2 ? 4 : mode == 1 ? 2 : 1;
+    k.info.n_outputs = mode == 2 ? 2 : 1;
     k.in_bytes[0] = (size_t)batch * cols * 4; k.in_align[0] = 16;
+    if (mode) { k.in_bytes[1] = (size_t)cols * 4; k.in_align[1] = 4; }
+    if (mode == 2) {
+        k.in_bytes[2] = (size_t)batch * cols * 4; k.in_align[2] = 4;
+        k.in_bytes[3] = (size_t)cols * 4; k.in_align[3] = 4;
+        k.out_bytes[1] = (size_t)batch * cols * 4; k.out_align[1] = 4;
+    }
     k.out_bytes[0] = (round_xf_halves((int)cols) + 2 * round_sx_halves((int)cols)) * 2; k.out_align[0] = 16;
-    set_launch(k, (uint32_t)((kRoundTokens * (cols / 8) + 255) / 256), 1, 1, 256, 0);
-    set_name(k, "round_prep_f32x");
+    if (mode) set_launch(k, kRoundTokens, 1, 1, 256, mode == 2 ? (uint32_t)cols * 4 : 0);
+    else set_launch(k, (uint32_t)((kRoundTokens * (cols / 8) + 255) / 256), 1, 1, 256, 0);
+    set_name(k, mode == 2 ? "round_prep_add_then_rmsnorm" : mode == 1 ? "round_prep_rmsnorm" : "round_prep_f32x");
     k.launch = launch_round_prep;
     return 0;
 }

@@ -86,6 +86,59 @@ def test_matvec_round_unit_rows_recover_weights(ctx):
         assert np.allclose(got[t], want, rtol=1e-5, atol=1e-5 * np.abs(wd).max()), kk
 
 
+def xp_values(ctx, xp, cols):
+    """A prepared operand back as numbers: x[16, cols] = hi + 2^-11 lo from the fragments (lane = row + 32 * ((k / 8) % 2)
+    per 16 columns, rows 0..15 hi parts and 16..31 lo parts, k stored in the order (0, 2, 1, 3) within every 4), and the
+    per-sub-block sums [16, cols / 32] (hi + lo of the f16 pairs, hi part + 2^-11 lo part)."""
+    nsb = cols // 256
+    raw = ctx.read_bytes(xp, 64 * cols + 2048 * nsb).view(np.float16).astype(np.float64)
+    frag = raw[:32 * cols].reshape(cols // 16, 2, 32, 8)        # [slice][k half][row][position]
+    perm = [0, 2, 1, 3, 4, 6, 5, 7]                              # position kperm(i) holds k = i
+    x = np.empty((32, cols))
+    for i in range(8):
+        x[:, i::16] = frag[:, 0, :, perm[i]].T
+        x[:, 8 + i::16] = frag[:, 1, :, perm[i]].T
+    sums = raw[32 * cols:].reshape(2, 16, nsb, 32)
+    parts = sums[..., 0:8] + sums[..., 16:24]                   # [part][token][superblock][sub-block]
+    return x[:16] + x[16:] / 2048.0, (parts[0] + parts[1] / 2048.0).reshape(16, -1)
+
+
+@pytest.mark.parametrize("cols,batch", [(1536, 16), (256, 3), (8192, 5)])
+def test_round_prep_norm_forms_equal_norm_then_prep(ctx, cols, batch):
+    """Modes 1 and 2 of KSH_ROUND_PREP prepare what the rows norms would have written as f32 rows (to the last bit or
+    two of f32: the operand keeps 22 bits), mode 2's x_new is the add-then-norm kernel's, and the operand of mode 0
+    holds its input to 2^-21."""
+    rng = np.random.default_rng(950 + cols)
+    x, res = synth.normal_f32(batch * cols, 951), synth.normal_f32(batch * cols, 952)
+    w1, w2 = (1.0 + 0.1 * rng.standard_normal(cols)).astype(np.float32), (1.0 + 0.1 * rng.standard_normal(cols)).astype(np.float32)
+    eps = 1e-6
+    n_xp = 64 * cols + 2048 * (cols // 256)
+    bx, br, bw1, bw2 = ctx.buffer_f32(x), ctx.buffer_f32(res), ctx.buffer_f32(w1), ctx.buffer_f32(w2)
+    got = ctx.buffer_empty_bytes(n_xp)
+
+    def check(want_rows, what, tol=2.0 ** -20, floor=2.0 ** -10):
+        vals, sums = xp_values(ctx, got, cols)
+        want = np.zeros((16, cols))
+        want[:batch] = want_rows.astype(np.float64).reshape(batch, cols)
+        err = np.abs(vals - want) / np.maximum(np.abs(want), floor * np.abs(want).max())
+        assert err.max() < tol, (what, err.max(), np.unravel_index(err.argmax(), err.shape))
+        assert np.allclose(sums.reshape(16, -1), want.reshape(16, -1, 32).sum(axis=2), rtol=0, atol=2e-3 * np.abs(want).max()), what
+
+    ctx.encode_multi(ctx.compile(hip.make_desc(Kind.ROUND_PREP, (cols, batch), (DType.F32,))), [bx], [got])
+    check(x, "mode 0")
+    y = ctx.buffer_empty_f32(batch * cols)
+    ctx.encode_multi(ctx.compile(hip.make_desc(Kind.RMSNORM, (cols, 0, 0, batch), (), (eps,))), [bx, bw1], [y])
+    ctx.encode_multi(ctx.compile(hip.make_desc(Kind.ROUND_PREP, (cols, batch, 1), (DType.F32,), (eps,))), [bx, bw1], [got])
+    check(ctx.read_f32(y, batch * cols), "mode 1")
+    xn_want, x2 = ctx.buffer_empty_f32(batch * cols), ctx.buffer_empty_f32(batch * cols)
+    ctx.encode_multi(ctx.compile(hip.make_desc(Kind.RMSNORM_ADD_THEN_RMSNORM, (cols, batch), (), (eps,))), [bx, bw1, br, bw2], [xn_want, x2])
+    xn_got = ctx.buffer_empty_f32(batch * cols)
+    ctx.encode_multi(ctx.compile(hip.make_desc(Kind.ROUND_PREP, (cols, batch, 2), (DType.F32,), (eps,))), [bx, bw1, br, bw2], [got, xn_got])
+    assert np.allclose(ctx.read_f32(xn_got, batch * cols), ctx.read_f32(xn_want, batch * cols), rtol=1e-6, atol=1e-6)   # (a sum that may cancel)
+    # (x_new is a sum that may cancel: the two kernels' last bits of it differ, and the second norm carries that along)
+    check(ctx.read_f32(x2, batch * cols), "mode 2", tol=1e-5, floor=0.1)
+
+
 def q6k_blocks_full_scales(n_blocks, seed):
     """Q6_K blocks whose int8 scales use the whole range (sc * q up to 127 * 32: what an f16 operand would round)."""
     w = synth.q6k_blocks(n_blocks, seed=seed).reshape(n_blocks, 210).copy()

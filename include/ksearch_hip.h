@@ -117,7 +117,8 @@ enum ksh_kind {
     /* CopySlice.  dims: n.  in: src   out: dst */
     KSH_COPY_SLICE = 15,
     /* SoftcapArgmax: argmax_i cap*tanh(x_i/cap), lowest index wins ties, index
-     * stored as f32.  dims: n.  params[0] = cap.  in: x   out: idx f32[1] */
+     * stored as f32.  dims: n, rows (0 or 1: one vector; more: the rows of a decode round, one index each).
+     * params[0] = cap.  in: x f32[rows, n]   out: idx f32[rows] */
     KSH_SOFTCAP_ARGMAX = 16,
     /* Dequantize packed blocks to f32 (the CPU-side dequant_type_to_f32,
      * crates/ksearch_gguf/src/gguf_impl.rs:472-476, as a device kernel).

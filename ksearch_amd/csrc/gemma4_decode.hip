@@ -1111,11 +1111,10 @@ int encode_round4(ksh_gemma4 *m, ksh_kvpool *pool, int t, int max_batch, int poo
             get(m, KSH_MATVEC_ROUND, {c.vocab, h, t, 0, 0, 0}, {KSH_Q6K_ROWS}, {}, &k_lm) || enc(m, k_lm, {lm_w, m->r_xp}, {m->r_logits}, n))
             return 1;
     }
-    for (int i = 0; i < t; i++)
-        if ((!lm_batched &&
-             run(m->k_lm_head[0], {lm_w, m->c_x, m->g.output_norm}, {0, (size_t)i * h * 4, 0}, {m->r_logits}, {(size_t)i * c.vocab * 4})) ||
-            run(m->k_argmax, {m->r_logits}, {(size_t)i * c.vocab * 4}, {m->r_next}, {(size_t)i * 4}))
-            return 1;
+    for (int i = 0; i < t && !lm_batched; i++)
+        if (run(m->k_lm_head[0], {lm_w, m->c_x, m->g.output_norm}, {0, (size_t)i * h * 4, 0}, {m->r_logits}, {(size_t)i * c.vocab * 4})) return 1;
+    ksh_kernel *k_arg = nullptr;
+    if (get(m, KSH_SOFTCAP_ARGMAX, {c.vocab, t}, {}, {c.softcap}, &k_arg) || enc(m, k_arg, {m->r_logits}, {m->r_next}, n)) return 1;
     return 0;
 }
 }  // namespace

@@ -332,6 +332,10 @@ __global__ __launch_bounds__(kArgThreads) void softcap_argmax_part_kernel(const 
     __shared__ uint32_t si[4];
     float bv = -INFINITY;
     uint32_t bi = 0xFFFFFFFFu;
+    // several rows of n values (blockIdx.y): each with its own partial results, gridDim.x of them
+    x += (size_t)blockIdx.y * n;
+    pv += (size_t)blockIdx.y * gridDim.x;
+    pi += (size_t)blockIdx.y * gridDim.x;
     for (int i = blockIdx.x * kArgThreads + threadIdx.x; i < n; i += gridDim.x * kArgThreads) {
         const float y = cap > 0.0f ? cap * tanhf(x[i] / cap) : x[i];
         argmax_fold(bv, bi, y, (uint32_t)i);
@@ -347,10 +351,12 @@ __global__ __launch_bounds__(kArgThreads) void softcap_argmax_final_kernel(const
     __shared__ uint32_t si[4];
     float bv = -INFINITY;
     uint32_t bi = 0xFFFFFFFFu;
+    pv += (size_t)blockIdx.x * nparts;     // one workgroup per row
+    pi += (size_t)blockIdx.x * nparts;
     for (int i = threadIdx.x; i < nparts; i += kArgThreads) argmax_fold(bv, bi, pv[i], pi[i]);
     argmax_block(bv, bi, sv, si);
     // the reference carries the index as f32 (exact below 2^24), lower.rs:6126
-    if (threadIdx.x == 0) out[0] = (float)(bi == 0xFFFFFFFFu ? 0u : bi);
+    if (threadIdx.x == 0) out[blockIdx.x] = (float)(bi == 0xFFFFFFFFu ? 0u : bi);
 }
 
 // The end of a decode step as one launch behind the argmax's first pass: fold the partial maxima (the token id), then
@@ -471,14 +477,14 @@ constexpr int kArgParts = 256;
 
 int launch_softcap_argmax(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
 {
-    // k.scratch holds kArgParts (value, index) pairs
-    const int n = (int)k.desc.dims[0];
+    // k.scratch holds kArgParts (value, index) pairs per row: all values, then all indices
+    const int n = (int)k.desc.dims[0], rows = (int)max((int64_t)1, k.desc.dims[1]);
     const int parts = min(kArgParts, (n + kArgThreads - 1) / kArgThreads);
     float *pv = (float *)k.scratch;
-    uint32_t *pi = (uint32_t *)(pv + kArgParts);
-    hipLaunchKernelGGL(softcap_argmax_part_kernel, dim3(parts), dim3(kArgThreads), 0, st, (const float *)a.in[0], n,
+    uint32_t *pi = (uint32_t *)(pv + (size_t)kArgParts * rows);
+    hipLaunchKernelGGL(softcap_argmax_part_kernel, dim3(parts, rows), dim3(kArgThreads), 0, st, (const float *)a.in[0], n,
                        k.desc.params[0], pv, pi);
-    hipLaunchKernelGGL(softcap_argmax_final_kernel, dim3(1), dim3(kArgThreads), 0, st, pv, pi, parts,
+    hipLaunchKernelGGL(softcap_argmax_final_kernel, dim3(rows), dim3(kArgThreads), 0, st, pv, pi, parts,
                        (float *)a.out[0]);
     return done("softcap_argmax launch");
 }
@@ -692,13 +698,14 @@ int bind_glue(ksh_kernel &k)
 
 int bind_softcap_argmax(ksh_kernel &k)
 {
-    const int64_t n = k.desc.dims[0];
+    const int64_t n = k.desc.dims[0], rows = std::max<int64_t>(1, k.desc.dims[1]);
     if (n <= 0 || n >= (1 << 24)) return set_error("softcap_argmax: n=%lld (the f32 index is exact below 2^24 only)", (long long)n);
+    if (k.desc.dims[1] < 0 || rows > 4096) return set_error("softcap_argmax: %lld rows (up to 4096)", (long long)k.desc.dims[1]);
     k.info.n_inputs = 1;
     k.info.n_outputs = 1;
-    k.in_bytes[0] = (size_t)n * 4; k.in_align[0] = 4;
-    k.out_bytes[0] = 4; k.out_align[0] = 4;
-    k.scratch_bytes = (size_t)kArgParts * 8;
+    k.in_bytes[0] = (size_t)rows * n * 4; k.in_align[0] = 4;
+    k.out_bytes[0] = (size_t)rows * 4; k.out_align[0] = 4;
+    k.scratch_bytes = (size_t)kArgParts * 8 * rows;
     set_launch(k, (uint32_t)min((int64_t)kArgParts, (n + kArgThreads - 1) / kArgThreads), 1, 1, kArgThreads, 32);
     set_name(k, "softcap_argmax");
     k.launch = launch_softcap_argmax;

@@ -182,6 +182,21 @@ def test_matvec_round_q6k_rows_unit_rows_recover_weights(ctx):
         assert np.array_equal(got[t], wd[:, kk]), kk      # d * sc * (q - 32): exact in f32
 
 
+@pytest.mark.parametrize("n,rows", [(1000, 5), (262144, 16), (7, 2)])
+def test_softcap_argmax_rows(ctx, n, rows):
+    """The argmax of every row of a round in one launch pair: per row the single-vector kernel's index (lowest index
+    wins ties, soft cap applied before comparing)."""
+    x = synth.normal_f32(rows * n, 960).reshape(rows, n) * 8.0
+    x[0, n // 2] = x[0, n - 1] = 1e9          # a tie after the cap: the lower index
+    x[rows - 1, :] = -3.0                     # all equal: index 0
+    k = ctx.compile(hip.make_desc(Kind.SOFTCAP_ARGMAX, (n, rows), (), (30.0,)))
+    out = ctx.buffer_empty_f32(rows)
+    ctx.encode_multi(k, [ctx.buffer_f32(x.reshape(-1))], [out])
+    got = ctx.read_f32(out, rows).astype(np.int64)
+    assert list(got) == [oracle.softcap_argmax(x[r], 30.0) for r in range(rows)]
+    assert got[0] == n // 2 and got[rows - 1] == 0
+
+
 def test_matvec_round_errors(ctx):
     with pytest.raises(hip.KshError, match="1 to 16"):
         ctx.compile(hip.make_desc(Kind.ROUND_PREP, (1536, 17), (DType.F32,)))

@@ -136,7 +136,7 @@ struct ksh_gemma4 {
             *c_ple_tok = nullptr, *c_ple_tmp = nullptr, *c_ple_ctx = nullptr, *c_ple_u = nullptr;
     // decode rounds over several KV slots (allocated at the first round): the per-token table (ids, slots, attended
     // ranges of the two layer kinds), the logits of every token of the round, the greedy ids
-    ksh_buf *r_tab = nullptr, *r_logits = nullptr, *r_next = nullptr, *r_xp = nullptr;   // (r_xp: a round's prepared GEMM operand)
+    ksh_buf *r_tab = nullptr, *r_logits = nullptr, *r_next = nullptr, *r_xp = nullptr, *r_xp2 = nullptr;   // (r_xp, r_xp2: a round's prepared GEMM operands)
     // a round of t sequences is one graph per t, tied to the pool whose buffers it was captured over
     ksh_graph *round_graphs[17] = {};
     bool round_bound[17] = {};     // a width's kernels are bound (a first round launched kernel by kernel)
@@ -931,7 +931,8 @@ int forward_decode_round4(ksh_gemma4 *m, ksh_kvpool *pool, const int32_t *slots,
     for (int l = 0; l < c.n_layers; l++) widest = std::max<int64_t>(widest, std::max<int64_t>(m->layers[l].ffn, m->plan[l].qd));
     widest = (widest + 255) / 256 * 256;
     if (!m->r_tab && (alloc(m, (size_t)kRoundStride * 10 * 4, &m->r_tab) || alloc(m, (size_t)kRoundMax * c.vocab * 4, &m->r_logits) ||
-                      alloc(m, (size_t)kRoundMax * 4, &m->r_next) || alloc(m, (size_t)(64 * widest + 2048 * (widest / 256)), &m->r_xp)))
+                      alloc(m, (size_t)kRoundMax * 4, &m->r_next) || alloc(m, (size_t)(64 * widest + 2048 * (widest / 256)), &m->r_xp) ||
+                      alloc(m, (size_t)(64 * widest + 2048 * (widest / 256)), &m->r_xp2)))
         return 1;
     float tab[kRoundStride * 10] = {};
     for (int i = 0; i < t; i++) {
@@ -1075,21 +1076,40 @@ int encode_round4(ksh_gemma4 *m, ksh_kvpool *pool, int t, int max_batch, int poo
             mm1(L.dt_o, h, P.qd, L.wo, m->c_o, m->c_y))
             return 1;
         const bool gu_q4k = L.dt_gate == KSH_Q4K && L.dt_up == KSH_Q4K && h <= 8192;
+        bool down_done = false;
         if (!gu_q4k && enc(m, k_add_then, {m->c_y, L.post_attn_norm, m->c_x, L.ffn_norm}, {m->c_x, m->c_x2}, n)) return 1;
         if (gu_q4k) {
             ksh_kernel *k_gu = nullptr, *k_pn = nullptr;
             if (get(m, KSH_ROUND_PREP, {h, t, 2}, {KSH_F32}, {c.eps}, &k_pn) ||
-                enc(m, k_pn, {m->c_y, L.post_attn_norm, m->c_x, L.ffn_norm}, {m->r_xp, m->c_x}, n) ||
-                get(m, KSH_MATVEC_ROUND, {L.ffn, h, t, 0, 0, 1}, {KSH_Q4K}, {}, &k_gu) ||
-                enc(m, k_gu, {L.wgate, m->r_xp, L.wup}, {m->c_ff}, n))
+                enc(m, k_pn, {m->c_y, L.post_attn_norm, m->c_x, L.ffn_norm}, {m->r_xp, m->c_x}, n))
                 return 1;
+            // gelu(gate) * up leaves as the prepared operand of the down projection where that one takes it
+            const bool chain = L.dt_down == KSH_Q4K && L.ffn % 256 == 0 && h <= 2048;
+            if (get(m, KSH_MATVEC_ROUND, {L.ffn, h, t, 0, 0, 1, chain ? 1 : 0}, {KSH_Q4K}, {}, &k_gu) ||
+                enc(m, k_gu, {L.wgate, m->r_xp, L.wup}, {chain ? m->r_xp2 : m->c_ff}, n))
+                return 1;
+            if (chain) {
+                ksh_kernel *k_dn = nullptr;
+                if (get(m, KSH_MATVEC_ROUND, {h, L.ffn, t, 0, 0, 0}, {KSH_Q4K}, {}, &k_dn) || enc(m, k_dn, {L.wdown, m->r_xp2}, {m->c_y}, n) ||
+                    enc(m, k_add, {m->c_y, L.post_ffw_norm, m->c_x}, {m->c_x}, n))
+                    return 1;
+                down_done = true;
+            }
         } else if (mm(L.dt_gate, L.ffn, h, L.wgate, m->c_x2, m->c_g) || mm(L.dt_up, L.ffn, h, L.wup, m->c_x2, m->c_u) ||
                    get(m, KSH_GELU_MUL, {(int64_t)t * L.ffn}, {}, {}, &k_gelu) || enc(m, k_gelu, {m->c_g, m->c_u}, {m->c_ff}, n)) {
             return 1;
         }
-        if (mm1(L.dt_down, h, L.ffn, L.wdown, m->c_ff, m->c_y) || enc(m, k_add, {m->c_y, L.post_ffw_norm, m->c_x}, {m->c_x}, n))
+        if (!down_done && (mm1(L.dt_down, h, L.ffn, L.wdown, m->c_ff, m->c_y) || enc(m, k_add, {m->c_y, L.post_ffw_norm, m->c_x}, {m->c_x}, n)))
             return 1;
-        if (c.ple_dim > 0) {
+        if (c.ple_dim > 0 && L.dt_inp_gate == KSH_Q4K && L.dt_proj == KSH_Q4K && c.ple_dim % 256 == 0 && h <= 2048) {
+            // the per-layer embedding: gelu(gate x) * context leaves as the projection's prepared operand
+            ksh_kernel *k_pg = nullptr, *k_pp = nullptr, *k_as = nullptr;
+            if (prep(h, m->c_x) || get(m, KSH_MATVEC_ROUND, {c.ple_dim, h, t, 0, 0, 0, 1, pt}, {KSH_Q4K}, {}, &k_pg) ||
+                enc_off(m, k_pg, {L.inp_gate, m->r_xp, m->c_ple_ctx}, {0, 0, (size_t)l * c.ple_dim * 4}, {m->r_xp2}, n) ||
+                get(m, KSH_MATVEC_ROUND, {h, c.ple_dim, t, 0, 0, 0}, {KSH_Q4K}, {}, &k_pp) || enc(m, k_pp, {L.proj, m->r_xp2}, {m->c_y}, n) ||
+                get(m, KSH_RMSNORM, {h, 1, 1, t}, {}, {c.eps, L.layer_scale}, &k_as) || enc(m, k_as, {m->c_y, L.post_norm, m->c_x}, {m->c_x}, n))
+                return 1;
+        } else if (c.ple_dim > 0) {
             ksh_kernel *k_gs = nullptr, *k_as = nullptr;
             if (mm1(L.dt_inp_gate, c.ple_dim, h, L.inp_gate, m->c_x, m->c_ple_u) ||
                 get(m, KSH_GELU_MUL, {(int64_t)t * c.ple_dim, c.ple_dim, pt}, {}, {}, &k_gs) ||

@@ -642,9 +642,9 @@ __host__ __device__ inline size_t round_sx_halves(int cols) { return (size_t)kRo
 
 // what one thread does with 8 consecutive elements (8 j .. 8 j + 7) of token row t; whole quads call it together
 // (the four threads of a sub-block add their sums up over the quad)
-__device__ __forceinline__ void round_prep_write(const float (&f)[8], int t, int j, int cols, _Float16 *__restrict__ Xp)
+// 8 consecutive values as the hi and lo halves of a fragment lane, and the sums of the two parts
+__device__ __forceinline__ void round_split8(const float (&f)[8], h8 &oh, h8 &ol, float &sh, float &sl)
 {
-    h8 oh, ol;
     float fh[8], fl[8];
 #pragma unroll
     for (int i = 0; i < 8; i++) {
@@ -655,8 +655,35 @@ __device__ __forceinline__ void round_prep_write(const float (&f)[8], int t, int
         fh[i] = (float)hi;
         fl[i] = (float)lo;
     }
-    float sh = ((fh[0] + fh[1]) + (fh[2] + fh[3])) + ((fh[4] + fh[5]) + (fh[6] + fh[7]));
-    float sl = ((fl[0] + fl[1]) + (fl[2] + fl[3])) + ((fl[4] + fl[5]) + (fl[6] + fl[7]));
+    sh = ((fh[0] + fh[1]) + (fh[2] + fh[3])) + ((fh[4] + fh[5]) + (fh[6] + fh[7]));
+    sl = ((fl[0] + fl[1]) + (fl[2] + fl[3])) + ((fl[4] + fl[5]) + (fl[6] + fl[7]));
+}
+
+// the sums of a sub-block's hi and lo parts as the bias / min product reads them: hi[8] hi[8] lo[8] 0[8] per row and
+// superblock, entry jj of each
+__device__ __forceinline__ void round_store_sums(_Float16 *__restrict__ Xp, int cols, int t, int sub_block, float sh, float sl)
+{
+    const int jj = sub_block % 8;
+    _Float16 *sx = Xp + round_xf_halves(cols) + ((size_t)t * (cols / 256) + sub_block / 8) * 32;
+    const float sums[2] = {sh, sl};
+#pragma unroll
+    for (int part = 0; part < 2; part++) {
+        _Float16 *dst = sx + part * round_sx_halves(cols);
+        const float sum = pinned(sums[part]);
+        const _Float16 hi = (_Float16)sum;
+        const _Float16 lo = (_Float16)(sum - (float)hi);
+        dst[jj] = hi;
+        dst[8 + jj] = hi;
+        dst[16 + jj] = lo;
+        dst[24 + jj] = (_Float16)0.f;
+    }
+}
+
+__device__ __forceinline__ void round_prep_write(const float (&f)[8], int t, int j, int cols, _Float16 *__restrict__ Xp)
+{
+    h8 oh, ol;
+    float sh, sl;
+    round_split8(f, oh, ol, sh, sl);
     sh += dpp_f32<0xB1>(sh);
     sh += dpp_f32<0x4E>(sh);
     sl += dpp_f32<0xB1>(sl);
@@ -665,22 +692,7 @@ __device__ __forceinline__ void round_prep_write(const float (&f)[8], int t, int
     const size_t frag = (size_t)(j >> 1) * 64 + t + 32 * (j & 1);
     reinterpret_cast<h8 *>(Xp)[frag] = oh;
     reinterpret_cast<h8 *>(Xp)[frag + 16] = ol;
-    if ((threadIdx.x & 3) == 0) {
-        const int s = j / 4, jj = s % 8;
-        _Float16 *sx = Xp + round_xf_halves(cols) + ((size_t)t * (cols / 256) + s / 8) * 32;
-        const float sums[2] = {sh, sl};
-#pragma unroll
-        for (int part = 0; part < 2; part++) {
-            _Float16 *dst = sx + part * round_sx_halves(cols);
-            const float sum = pinned(sums[part]);
-            const _Float16 hi = (_Float16)sum;
-            const _Float16 lo = (_Float16)(sum - (float)hi);
-            dst[jj] = hi;
-            dst[8 + jj] = hi;
-            dst[16 + jj] = lo;
-            dst[24 + jj] = (_Float16)0.f;
-        }
-    }
+    if ((threadIdx.x & 3) == 0) round_store_sums(Xp, cols, t, j / 4, sh, sl);
 }
 
 // one thread per 8 elements of the 16 token rows (rows past the batch are written as zeros)
@@ -761,13 +773,16 @@ struct RoundParams {
     int cols, batch;
     const _Float16 *Xp;
     float *part;                 // [slices][batch][rows0] when the columns are split
+    const float *mul;            // NM = 1: y = gelu(W0 x) * mul[t * mul_stride + r] (the per-layer-embedding gate)
+    int mul_stride;
+    _Float16 *emit;              // not null: the result goes out as the prepared operand of the next GEMM (rows0 columns)
 };
 
 // NM = 2: the gate | up pair (W0, W1 of rows0 rows each; gelu(W0 x) * (W1 x) to Y0)
 template <int NM>
 __global__ __launch_bounds__(512) void q4k_mm_round_kernel(RoundParams p)
 {
-    extern __shared__ __attribute__((aligned(16))) float red[];   // [8][NM][16][64]
+    extern __shared__ __attribute__((aligned(16))) float red[];   // [8][NM][8][64]
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 31, h = lane >> 5;
     // the workgroup's matrix: a choice between arguments already fetched, not an indexed read of them
@@ -847,28 +862,60 @@ __global__ __launch_bounds__(512) void q4k_mm_round_kernel(RoundParams p)
         }
         f16v F = __builtin_amdgcn_mfma_f32_32x32x16_f16(a2[0], b2[0], kZero16, 0, 0, 0);
         F = __builtin_amdgcn_mfma_f32_32x32x16_f16(a2[1], b2[1], F, 0, 0, 0);
+        // accumulator i of lane (n, h) is row 8*(i/4) + 4*h + i%4 of the tile: i < 8 a token's hi part, i + 8 its lo part
 #pragma unroll
-        for (int i = 0; i < 16; i++) red[((wave * NM + m) * 16 + i) * 64 + lane] = active ? fmaf(d, C[i], F[i]) : 0.f;
+        for (int i = 0; i < 8; i++)
+            red[((wave * NM + m) * 8 + i) * 64 + lane] = active ? fmaf(1.0f / 2048.0f, fmaf(d, C[i + 8], F[i + 8]), fmaf(d, C[i], F[i])) : 0.f;
     }
     __syncthreads();
-    // accumulator i of lane (n, h) is row 8*(i/4) + 4*h + i%4 of the tile: i < 8 a token's hi part, i + 8 its lo part.
-    // One output per thread: the eight waves' shares in a fixed order.
+    // one output per thread: the eight waves' shares in a fixed order
     const int i = tid >> 6, t = 8 * (i >> 2) + 4 * h + (i & 3), r = r0 + n;
     float v[NM];
 #pragma unroll
     for (int m = 0; m < NM; m++) {
-        float hi = 0.f, lo = 0.f;
+        v[m] = 0.f;
 #pragma unroll
-        for (int w = 0; w < 8; w++) {
-            hi += red[((w * NM + m) * 16 + i) * 64 + lane];
-            lo += red[((w * NM + m) * 16 + i + 8) * 64 + lane];
-        }
-        v[m] = fmaf(1.0f / 2048.0f, lo, hi);
+        for (int w = 0; w < 8; w++) v[m] += red[((w * NM + m) * 8 + i) * 64 + lane];
     }
-    if (t < p.batch && r < rows) {
-        const float y = NM == 2 ? gelu_mul_f32(v[0], v[NM - 1]) : v[0];
-        if (gridDim.y == 1) Y[(size_t)t * rows + r] = y;
-        else p.part[((size_t)blockIdx.y * p.batch + t) * rows + r] = y;
+    const bool mine = t < p.batch && r < rows;
+    float y = NM == 2 ? gelu_mul_f32(v[0], v[NM - 1]) : v[0];
+    if (NM == 1 && p.mul) y = gelu_mul_f32(y, p.mul[(size_t)min(t, p.batch - 1) * p.mul_stride + min(r, rows - 1)]);
+    if (!p.emit) {
+        if (mine) {
+            if (gridDim.y == 1) Y[(size_t)t * rows + r] = y;
+            else p.part[((size_t)blockIdx.y * p.batch + t) * rows + r] = y;
+        }
+        return;
+    }
+    // The tile's 16 x 32 results are 32 columns of the next GEMM's input: two fragments' worth of every token row and
+    // exactly one sub-block of sums, so the workgroup writes its share of the prepared operand itself (rows0 is a
+    // multiple of 256 and the columns are not split: host-checked).  Rows past the batch are written as zeros.
+    float *T = red + 8 * NM * 8 * 64;             // [16][33]
+    T[t * 33 + n] = mine ? y : 0.f;
+    __syncthreads();
+    if (tid < 64) {
+        const int tt = tid & 15, ks = (tid >> 4) & 1, kh = tid >> 5;
+        float f[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) f[e] = T[tt * 33 + 16 * ks + 8 * kh + e];
+        h8 oh, ol;
+        float sh, sl;
+        round_split8(f, oh, ol, sh, sl);
+        const size_t frag = (size_t)(r0 / 16 + ks) * 64 + tt + 32 * kh;
+        reinterpret_cast<h8 *>(p.emit)[frag] = oh;
+        reinterpret_cast<h8 *>(p.emit)[frag + 16] = ol;
+    } else if (tid < 80) {
+        const int tt = tid - 64;
+        float sh4[4], sl4[4];
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            float f[8];
+#pragma unroll
+            for (int e = 0; e < 8; e++) f[e] = T[tt * 33 + 8 * g + e];
+            h8 oh, ol;
+            round_split8(f, oh, ol, sh4[g], sl4[g]);
+        }
+        round_store_sums(p.emit, rows, tt, r0 / 32, (sh4[0] + sh4[1]) + (sh4[2] + sh4[3]), (sl4[0] + sl4[1]) + (sl4[2] + sl4[3]));
     }
 }
 
@@ -1030,6 +1077,8 @@ int launch_matvec_round(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st
     p.tiles0 = (p.rows0 + 31) / 32; p.tiles1 = pair ? 0 : (p.rows1 + 31) / 32;
     p.cols = (int)d[1]; p.batch = (int)d[2];
     p.part = (float *)k.scratch;
+    if (d[7]) { p.mul = (const float *)a.in[2]; p.mul_stride = (int)d[7]; }
+    if (d[6]) { p.emit = (_Float16 *)a.out[0]; p.Y0 = p.Y1 = p.Y2 = nullptr; }
     const dim3 grid(k.info.grid[0], k.info.grid[1]);
     if (pair) hipLaunchKernelGGL(q4k_mm_round_kernel<2>, grid, dim3(512), k.info.lds_bytes, st, p);
     else hipLaunchKernelGGL(q4k_mm_round_kernel<1>, grid, dim3(512), k.info.lds_bytes, st, p);
@@ -1183,6 +1232,11 @@ int bind_matvec_round(ksh_kernel &k)
     if (pair && (rows1 || rows2)) return set_error("matvec_round: a gate | up pair names one row count (both matrices have it)");
     const int slices = (int)((cols / 256 + 7) / 8);
     if (slices > 1 && (pair || rows1)) return set_error("matvec_round: rows longer than 2048 columns take one matrix per launch");
+    const bool emit = d[6] != 0;
+    const int64_t mul_stride = d[7];
+    if (mul_stride && (pair || rows1 || mul_stride < rows0)) return set_error("matvec_round: the gate multiplier takes one matrix and a row stride of at least its rows");
+    if (emit && (rows1 || slices > 1 || rows0 % 256))
+        return set_error("matvec_round: the result as a prepared operand takes one matrix (or a pair) of up to 2048 columns whose rows are a multiple of 256");
     const int n_mat = pair ? 2 : rows2 ? 3 : rows1 ? 2 : 1;
     const int64_t rows[3] = {rows0, pair ? rows0 : rows1, rows2};
     k.info.n_inputs = 1 + n_mat;
@@ -1190,13 +1244,16 @@ int bind_matvec_round(ksh_kernel &k)
     k.in_bytes[0] = (size_t)rows0 * (cols / 256) * 144; k.in_align[0] = 16;
     k.in_bytes[1] = (round_xf_halves((int)cols) + 2 * round_sx_halves((int)cols)) * 2; k.in_align[1] = 16;
     for (int i = 1; i < n_mat; i++) { k.in_bytes[1 + i] = (size_t)rows[i] * (cols / 256) * 144; k.in_align[1 + i] = 16; }
+    if (mul_stride) { k.info.n_inputs = 3; k.in_bytes[2] = ((size_t)(batch - 1) * mul_stride + rows0) * 4; k.in_align[2] = 4; }
     for (int i = 0; i < k.info.n_outputs; i++) { k.out_bytes[i] = (size_t)batch * rows[i] * 4; k.out_align[i] = 4; }
+    if (emit) { k.out_bytes[0] = (round_xf_halves((int)rows0) + 2 * round_sx_halves((int)rows0)) * 2; k.out_align[0] = 16; }
     k.scratch_bytes = slices > 1 ? (size_t)slices * batch * rows0 * 4 : 0;
     const int64_t tiles = pair ? (rows0 + 31) / 32 : (rows0 + 31) / 32 + (rows1 + 31) / 32 + (rows2 + 31) / 32;
-    set_launch(k, (uint32_t)tiles, (uint32_t)slices, 1, 512, (uint32_t)(8 * (pair ? 2 : 1) * 16 * 64 * 4));
+    set_launch(k, (uint32_t)tiles, (uint32_t)slices, 1, 512, (uint32_t)(8 * (pair ? 2 : 1) * 8 * 64 * 4 + (emit ? 16 * 33 * 4 : 0)));
     k.info.sched = k.desc.sched;
     k.info.sched.tg = 512; k.info.sched.nsg = 8; k.info.sched.nr0 = 32; k.info.sched.k_split = (uint32_t)slices; k.info.sched.lds_tile = 16;
-    set_name(k, "matvec_round_q4k_%s%s", pair ? "gate_up_gelu" : n_mat == 3 ? "x3" : n_mat == 2 ? "x2" : "x1", slices > 1 ? "_ksplit" : "");
+    set_name(k, "matvec_round_q4k_%s%s%s", pair ? "gate_up_gelu" : mul_stride ? "gelu_mul" : n_mat == 3 ? "x3" : n_mat == 2 ? "x2" : "x1",
+             slices > 1 ? "_ksplit" : "", emit ? "_prepared" : "");
     k.launch = launch_matvec_round;
     return 0;
 }

@@ -71,6 +71,39 @@ def test_matvec_round_gate_up_gelu(ctx, rows, cols, batch):
     assert_close(got, oracle.gelu_mul(g.reshape(-1), u.reshape(-1)).reshape(batch, rows), 1e-3, f"gate|up {rows}x{cols} b{batch}")
 
 
+@pytest.mark.parametrize("batch", [16, 3])
+def test_matvec_round_result_as_prepared_operand(ctx, batch):
+    """dims[6] = 1: a launch's result leaves as the next GEMM's prepared operand (here gate | up -> down, and the
+    per-layer-embedding gate with its multiplier -> projection); the values it holds are the f32 results' to 2^-20."""
+    rows, cols = 512, 1536
+    wg, wu = synth.q4k_blocks(rows * cols // 256, seed=970), synth.q4k_blocks(rows * cols // 256, seed=971)
+    x = synth.normal_f32(batch * cols, 972).reshape(batch, cols) * 0.25
+    _, (plain,) = round_mm(ctx, [wg, wu], (rows,), cols, x, batch, pair=True)
+    xp = prepared(ctx, x, batch, cols)
+    out = ctx.buffer_empty_bytes(64 * rows + 2048 * (rows // 256))
+    k = ctx.compile(hip.make_desc(Kind.MATVEC_ROUND, (rows, cols, batch, 0, 0, 1, 1), (DType.Q4K,)))
+    assert k.name.endswith("_prepared")
+    ctx.encode_multi(k, [ctx.buffer_bytes(wg), xp, ctx.buffer_bytes(wu)], [out])
+    vals, sums = xp_values(ctx, out, rows)
+    want = np.zeros((16, rows))
+    want[:batch] = plain
+    assert np.max(np.abs(vals - want) / np.maximum(np.abs(want), 2.0 ** -10 * np.abs(want).max())) < 2.0 ** -20
+    assert np.allclose(sums, want.reshape(16, -1, 32).sum(axis=2), rtol=0, atol=2e-3 * np.abs(want).max())
+    # the gate with its multiplier: gelu(W x) * ctx[t, r], ctx rows `stride` apart
+    stride = 3 * rows
+    ctxv = synth.normal_f32(batch * stride, 973).reshape(batch, stride)
+    k2 = ctx.compile(hip.make_desc(Kind.MATVEC_ROUND, (rows, cols, batch, 0, 0, 0, 0, stride), (DType.Q4K,)))
+    y = ctx.buffer_empty_f32(batch * rows)
+    ctx.encode_offsets_multi(k2, [ctx.buffer_bytes(wg), xp, ctx.buffer_f32(ctxv.reshape(-1))], [0, 0, rows * 4], [y], [0])
+    g = oracle.matmul(oracle.Q4K, wg, rows, cols, x, batch)
+    want2 = oracle.gelu_mul(g.reshape(-1), ctxv[:, rows:2 * rows].reshape(-1)).reshape(batch, rows)
+    assert_close(ctx.read_f32(y, batch * rows).reshape(batch, rows), want2, 1e-3, "gelu(W x) * ctx")
+    k3 = ctx.compile(hip.make_desc(Kind.MATVEC_ROUND, (rows, cols, batch, 0, 0, 0, 1, stride), (DType.Q4K,)))
+    ctx.encode_offsets_multi(k3, [ctx.buffer_bytes(wg), xp, ctx.buffer_f32(ctxv.reshape(-1))], [0, 0, rows * 4], [out], [0])
+    vals, _ = xp_values(ctx, out, rows)
+    assert np.allclose(vals[:batch], ctx.read_f32(y, batch * rows).reshape(batch, rows), rtol=2.0 ** -19, atol=1e-6)
+
+
 def test_matvec_round_unit_rows_recover_weights(ctx):
     # X = one-hot rows: Y[t] is column k_t of the dequantized matrix (pins the K order and the hi | lo tile end to end)
     rows, cols = 64, 4096
@@ -210,5 +243,7 @@ def test_matvec_round_errors(ctx):
         ctx.compile(hip.make_desc(Kind.MATVEC_ROUND, (64, 4096, 4, 0, 0, 0), (DType.Q6K_ROWS,)))
     with pytest.raises(hip.KshError, match="one matrix per launch"):
         ctx.compile(hip.make_desc(Kind.MATVEC_ROUND, (64, 4096, 4, 64, 0, 0), (DType.Q4K,)))
+    with pytest.raises(hip.KshError, match="multiple of 256"):
+        ctx.compile(hip.make_desc(Kind.MATVEC_ROUND, (96, 1536, 4, 0, 0, 0, 1), (DType.Q4K,)))
     with pytest.raises(hip.KshError, match="one row count"):
         ctx.compile(hip.make_desc(Kind.MATVEC_ROUND, (64, 1536, 4, 64, 0, 1), (DType.Q4K,)))

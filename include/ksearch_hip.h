@@ -215,7 +215,9 @@ enum ksh_kind {
      *   mode 1: the rows' RMSNorm on the way (rmsnorm_rows, crates/ksearch_kernels/src/lib.rs:1478):
      *           in: x, w f32[cols]                              out: xp of (x * inv) * w
      *   mode 2: rmsnorm_add_then_rmsnorm on rows: in: y, w_post, res, w_norm   out: xp, x_new f32[batch, cols]
-     *           with x_new = res + (y * inv) * w_post (may be res) and xp of (x_new * inv2) * w_norm
+     *           with x_new = res + (y * inv) * w_post (may be res) and xp of (x_new * inv2) * w_norm; params[1] != 0:
+     *           x_new = params[1] * (res + ...) (rmsnorm_add_scale_rows, :1520-1560, in front of the next norm)
+     *   mode 3: rmsnorm_add on rows: in: y, w, res   out: xp of x_new, x_new = res + (y * inv) * w
      * xp: 64 * cols + 2048 * (cols / 256) bytes, 16-byte aligned */
     KSH_ROUND_PREP = 30,
     /* Up to three Q4_K matrices of one width against one prepared operand, in one launch (q | k | v share their

@@ -1038,6 +1038,29 @@ int encode_round4(ksh_gemma4 *m, ksh_kvpool *pool, int t, int max_batch, int poo
     if (get(m, KSH_RMSNORM, {h, 0, 0, t}, {}, {c.eps}, &k_norm) || get(m, KSH_RMSNORM, {h, 1, 0, t}, {}, {c.eps}, &k_add) ||
         get(m, KSH_RMSNORM_ADD_THEN_RMSNORM, {h, t}, {}, {c.eps}, &k_add_then))
         return 1;
+    ksh_buf *lm_w = m->embd_rows ? m->embd_rows : m->g.token_embd;
+    // the LM head once for all rows where the table is kept row-grouped (the matrix cores on exact codes, the int8
+    // scales applied in f32); row by row through the GEMV otherwise
+    const bool lm_batched = m->embd_rows && h % 256 == 0 && h <= 2048;
+    // a layer whose q | k | v read the prepared operand of the normed residual stream
+    auto qkv_prepared = [&](int l) {
+        const ksh_gemma4_layer &L = m->layers[l];
+        return L.dt_q == KSH_Q4K && (!m->plan[l].owns || (L.dt_k == KSH_Q4K && L.dt_v == KSH_Q4K));
+    };
+    // The norm that closes a layer also writes the operand the next layer's q | k | v (or the LM head) start from, where
+    // those take one: x_new = [scale *] (res + norm(y) * w), xp = norm(x_new) * w_next (KSH_ROUND_PREP mode 2).
+    bool xp_ready = false;
+    auto close_layer = [&](int l, ksh_buf *w, float scale, ksh_kernel *k_plain) -> int {
+        const bool last = l + 1 == c.n_layers;
+        const bool fuse = h <= 8192 && (last ? lm_batched : qkv_prepared(l + 1));
+        if (!fuse) return enc(m, k_plain, {m->c_y, w, m->c_x}, {m->c_x}, n);
+        ksh_kernel *kk = nullptr;
+        if (get(m, KSH_ROUND_PREP, {h, t, 2}, {KSH_F32}, {c.eps, scale}, &kk) ||
+            enc(m, kk, {m->c_y, w, m->c_x, last ? m->g.output_norm : m->layers[l + 1].attn_norm}, {m->r_xp, m->c_x}, n))
+            return 1;
+        xp_ready = true;
+        return 0;
+    };
     for (int l = 0; l < c.n_layers; l++) {
         const ksh_gemma4_layer &L = m->layers[l];
         const LayerPlan &P = m->plan[l];
@@ -1047,11 +1070,12 @@ int encode_round4(ksh_gemma4 *m, ksh_kvpool *pool, int t, int max_batch, int poo
         ksh_kernel *k_head = nullptr, *k_sdpa = nullptr, *k_gelu = nullptr;
         if (!sdpa_lanes_supports(c.n_q, c.n_kv, P.hd))
             return set_error("ksh_gemma4_decode_round: attention over several slots is built for heads of 128 / 256 / 512 with up to 8 q heads per kv head");
-        const bool qkv_q4k = L.dt_q == KSH_Q4K && (!P.owns || (L.dt_k == KSH_Q4K && L.dt_v == KSH_Q4K));
+        const bool qkv_q4k = qkv_prepared(l);
         if (!qkv_q4k && enc(m, k_norm, {m->c_x, L.attn_norm}, {m->c_x2}, n)) return 1;
         if (qkv_q4k) {
             ksh_kernel *kq = nullptr;
-            if (prep_norm(h, m->c_x, L.attn_norm)) return 1;
+            if (!xp_ready && prep_norm(h, m->c_x, L.attn_norm)) return 1;   // (ready: the previous layer's last norm wrote it)
+            xp_ready = false;
             if (P.owns ? (get(m, KSH_MATVEC_ROUND, {P.qd, h, t, P.kvd, P.kvd, 0}, {KSH_Q4K}, {}, &kq) ||
                           enc(m, kq, {L.wq, m->r_xp, L.wk, L.wv}, {m->c_q, m->c_k, m->c_v}, n))
                        : (get(m, KSH_MATVEC_ROUND, {P.qd, h, t, 0, 0, 0}, {KSH_Q4K}, {}, &kq) || enc(m, kq, {L.wq, m->r_xp}, {m->c_q}, n)))
@@ -1090,44 +1114,46 @@ int encode_round4(ksh_gemma4 *m, ksh_kvpool *pool, int t, int max_batch, int poo
                 return 1;
             if (chain) {
                 ksh_kernel *k_dn = nullptr;
-                if (get(m, KSH_MATVEC_ROUND, {h, L.ffn, t, 0, 0, 0}, {KSH_Q4K}, {}, &k_dn) || enc(m, k_dn, {L.wdown, m->r_xp2}, {m->c_y}, n) ||
-                    enc(m, k_add, {m->c_y, L.post_ffw_norm, m->c_x}, {m->c_x}, n))
-                    return 1;
+                if (get(m, KSH_MATVEC_ROUND, {h, L.ffn, t, 0, 0, 0}, {KSH_Q4K}, {}, &k_dn) || enc(m, k_dn, {L.wdown, m->r_xp2}, {m->c_y}, n)) return 1;
                 down_done = true;
             }
         } else if (mm(L.dt_gate, L.ffn, h, L.wgate, m->c_x2, m->c_g) || mm(L.dt_up, L.ffn, h, L.wup, m->c_x2, m->c_u) ||
                    get(m, KSH_GELU_MUL, {(int64_t)t * L.ffn}, {}, {}, &k_gelu) || enc(m, k_gelu, {m->c_g, m->c_u}, {m->c_ff}, n)) {
             return 1;
         }
-        if (!down_done && (mm1(L.dt_down, h, L.ffn, L.wdown, m->c_ff, m->c_y) || enc(m, k_add, {m->c_y, L.post_ffw_norm, m->c_x}, {m->c_x}, n)))
-            return 1;
-        if (c.ple_dim > 0 && L.dt_inp_gate == KSH_Q4K && L.dt_proj == KSH_Q4K && c.ple_dim % 256 == 0 && h <= 2048) {
-            // the per-layer embedding: gelu(gate x) * context leaves as the projection's prepared operand
-            ksh_kernel *k_pg = nullptr, *k_pp = nullptr, *k_as = nullptr;
-            if (prep(h, m->c_x) || get(m, KSH_MATVEC_ROUND, {c.ple_dim, h, t, 0, 0, 0, 1, pt}, {KSH_Q4K}, {}, &k_pg) ||
+        if (!down_done && mm1(L.dt_down, h, L.ffn, L.wdown, m->c_ff, m->c_y)) return 1;
+        // the feed-forward block's closing norm + add
+        const bool ple_q4k = c.ple_dim > 0 && L.dt_inp_gate == KSH_Q4K && L.dt_proj == KSH_Q4K && c.ple_dim % 256 == 0 && h <= 2048;
+        if (c.ple_dim == 0) {
+            if (close_layer(l, L.post_ffw_norm, 0.f, k_add)) return 1;
+        } else if (ple_q4k) {
+            // ... which also prepares the new residual stream for the per-layer-embedding gate (mode 3); the gate's
+            // gelu(W x) * context leaves as the projection's prepared operand
+            ksh_kernel *k_pa = nullptr, *k_pg = nullptr, *k_pp = nullptr, *k_as = nullptr;
+            if (get(m, KSH_ROUND_PREP, {h, t, 3}, {KSH_F32}, {c.eps}, &k_pa) ||
+                enc(m, k_pa, {m->c_y, L.post_ffw_norm, m->c_x}, {m->r_xp, m->c_x}, n) ||
+                get(m, KSH_MATVEC_ROUND, {c.ple_dim, h, t, 0, 0, 0, 1, pt}, {KSH_Q4K}, {}, &k_pg) ||
                 enc_off(m, k_pg, {L.inp_gate, m->r_xp, m->c_ple_ctx}, {0, 0, (size_t)l * c.ple_dim * 4}, {m->r_xp2}, n) ||
                 get(m, KSH_MATVEC_ROUND, {h, c.ple_dim, t, 0, 0, 0}, {KSH_Q4K}, {}, &k_pp) || enc(m, k_pp, {L.proj, m->r_xp2}, {m->c_y}, n) ||
-                get(m, KSH_RMSNORM, {h, 1, 1, t}, {}, {c.eps, L.layer_scale}, &k_as) || enc(m, k_as, {m->c_y, L.post_norm, m->c_x}, {m->c_x}, n))
+                get(m, KSH_RMSNORM, {h, 1, 1, t}, {}, {c.eps, L.layer_scale}, &k_as))
                 return 1;
-        } else if (c.ple_dim > 0) {
+            if (L.layer_scale != 0.f ? close_layer(l, L.post_norm, L.layer_scale, k_as) : enc(m, k_as, {m->c_y, L.post_norm, m->c_x}, {m->c_x}, n)) return 1;
+        } else {
             ksh_kernel *k_gs = nullptr, *k_as = nullptr;
-            if (mm1(L.dt_inp_gate, c.ple_dim, h, L.inp_gate, m->c_x, m->c_ple_u) ||
+            if (enc(m, k_add, {m->c_y, L.post_ffw_norm, m->c_x}, {m->c_x}, n) ||
+                mm1(L.dt_inp_gate, c.ple_dim, h, L.inp_gate, m->c_x, m->c_ple_u) ||
                 get(m, KSH_GELU_MUL, {(int64_t)t * c.ple_dim, c.ple_dim, pt}, {}, {}, &k_gs) ||
                 enc_off(m, k_gs, {m->c_ple_u, m->c_ple_ctx}, {0, (size_t)l * c.ple_dim * 4}, {m->c_ple_u}, n) ||
                 mm1(L.dt_proj, h, c.ple_dim, L.proj, m->c_ple_u, m->c_y) ||
-                get(m, KSH_RMSNORM, {h, 1, 1, t}, {}, {c.eps, L.layer_scale}, &k_as) ||
-                enc(m, k_as, {m->c_y, L.post_norm, m->c_x}, {m->c_x}, n))
+                get(m, KSH_RMSNORM, {h, 1, 1, t}, {}, {c.eps, L.layer_scale}, &k_as))
                 return 1;
+            if (L.layer_scale != 0.f ? close_layer(l, L.post_norm, L.layer_scale, k_as) : enc(m, k_as, {m->c_y, L.post_norm, m->c_x}, {m->c_x}, n)) return 1;
         }
     }
     // logits and the greedy id of every row: the output norm rides in the LM head's prologue, as in the decode step
-    ksh_buf *lm_w = m->embd_rows ? m->embd_rows : m->g.token_embd;
-    // the LM head once for all rows where the table is kept row-grouped (the matrix cores on exact codes, the int8
-    // scales applied in f32); row by row through the GEMV otherwise
-    const bool lm_batched = m->embd_rows && h % 256 == 0 && h <= 2048;
     if (lm_batched) {
         ksh_kernel *k_lm = nullptr;
-        if (prep_norm(h, m->c_x, m->g.output_norm) ||
+        if ((!xp_ready && prep_norm(h, m->c_x, m->g.output_norm)) ||
             get(m, KSH_MATVEC_ROUND, {c.vocab, h, t, 0, 0, 0}, {KSH_Q6K_ROWS}, {}, &k_lm) || enc(m, k_lm, {lm_w, m->r_xp}, {m->r_logits}, n))
             return 1;
     }

@@ -715,7 +715,8 @@ __global__ __launch_bounds__(256) void mm_round_prep_kernel(const float *__restr
 // with the prepared operand as their output: one workgroup per token row, the same sums in the same order as the
 // kernels that write f32 rows (explicitly rounded products and sums: nothing is contracted).
 //   MODE 1:  v = (x * inv) * w                                                     -> xp
-//   MODE 2:  x_new = res + (y * inv) * w_post;  v = (x_new * inv2) * w_norm        -> xp, x_new (may be res)
+//   MODE 2:  x_new = [scale *] (res + (y * inv) * w_post);  v = (x_new * inv2) * w_norm   -> xp, x_new (may be res)
+//   MODE 3:  x_new = res + (y * inv) * w_post;  v = x_new                          -> xp, x_new (may be res)
 __device__ __forceinline__ float round_block_sum(float v, float *red)
 {
     v = wave_sum(v);
@@ -729,7 +730,7 @@ __device__ __forceinline__ float round_block_sum(float v, float *red)
 template <int MODE>
 __global__ __launch_bounds__(256) void mm_round_prep_norm_kernel(const float *__restrict__ x, const float *__restrict__ w_first, const float *res,
                                                                  const float *__restrict__ w_norm, float *x_new, _Float16 *__restrict__ Xp,
-                                                                 int batch, int cols, float eps)
+                                                                 int batch, int cols, float eps, float scale)
 {
     __shared__ float red[4];
     extern __shared__ float mid[];      // MODE 2: the row between the two norms
@@ -744,24 +745,29 @@ __global__ __launch_bounds__(256) void mm_round_prep_norm_kernel(const float *__
     for (int i = threadIdx.x; i < cols; i += 256) ss = __fadd_rn(ss, __fmul_rn(x[i], x[i]));
     ss = round_block_sum(ss, red);
     float inv = 1.0f / sqrtf(__fadd_rn(ss / (float)cols, eps));
-    if (MODE == 2) {
+    if (MODE >= 2) {
         res += (size_t)t * cols;
         x_new += (size_t)t * cols;
         float ss2 = 0.f;
         for (int i = threadIdx.x; i < cols; i += 256) {
-            const float v = __fadd_rn(res[i], __fmul_rn(__fmul_rn(x[i], inv), w_first[i]));
+            float v = __fadd_rn(__fmul_rn(__fmul_rn(x[i], inv), w_first[i]), res[i]);
+            if (scale != 0.f) v = __fmul_rn(scale, v);
             mid[i] = v;
             x_new[i] = v;
             ss2 = __fadd_rn(ss2, __fmul_rn(v, v));
         }
-        ss2 = round_block_sum(ss2, red);
-        inv = 1.0f / sqrtf(__fadd_rn(ss2 / (float)cols, eps));
+        if (MODE == 2) {
+            ss2 = round_block_sum(ss2, red);
+            inv = 1.0f / sqrtf(__fadd_rn(ss2 / (float)cols, eps));
+        } else {
+            __syncthreads();   // the row is read across threads below
+        }
     }
-    const float *src = MODE == 2 ? mid : x, *w = MODE == 2 ? w_norm : w_first;
+    const float *src = MODE >= 2 ? mid : x, *w = MODE == 2 ? w_norm : w_first;
     for (int j = threadIdx.x; j < k8; j += 256) {
         float f[8];
 #pragma unroll
-        for (int i = 0; i < 8; i++) f[i] = pinned(__fmul_rn(__fmul_rn(src[8 * j + i], inv), w[8 * j + i]));
+        for (int i = 0; i < 8; i++) f[i] = MODE == 3 ? src[8 * j + i] : pinned(__fmul_rn(__fmul_rn(src[8 * j + i], inv), w[8 * j + i]));
         round_prep_write(f, t, j, cols, Xp);
     }
 }
@@ -1038,10 +1044,14 @@ int launch_round_prep(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
     const int n = kRoundTokens * (cols / 8);
     if (mode == 1)
         hipLaunchKernelGGL(mm_round_prep_norm_kernel<1>, dim3(kRoundTokens), dim3(256), 0, st, (const float *)a.in[0], (const float *)a.in[1], nullptr, nullptr,
-                           nullptr, (_Float16 *)a.out[0], batch, cols, k.desc.params[0]);
+                           nullptr, (_Float16 *)a.out[0], batch, cols, k.desc.params[0], 0.f);
     else if (mode == 2)
         hipLaunchKernelGGL(mm_round_prep_norm_kernel<2>, dim3(kRoundTokens), dim3(256), (size_t)cols * 4, st, (const float *)a.in[0], (const float *)a.in[1],
-                           (const float *)a.in[2], (const float *)a.in[3], (float *)a.out[1], (_Float16 *)a.out[0], batch, cols, k.desc.params[0]);
+                           (const float *)a.in[2], (const float *)a.in[3], (float *)a.out[1], (_Float16 *)a.out[0], batch, cols, k.desc.params[0],
+                           k.desc.params[1]);
+    else if (mode == 3)
+        hipLaunchKernelGGL(mm_round_prep_norm_kernel<3>, dim3(kRoundTokens), dim3(256), (size_t)cols * 4, st, (const float *)a.in[0], (const float *)a.in[1],
+                           (const float *)a.in[2], nullptr, (float *)a.out[1], (_Float16 *)a.out[0], batch, cols, k.desc.params[0], 0.f);
     else
         hipLaunchKernelGGL(mm_round_prep_kernel, dim3((n + 255) / 256), dim3(256), 0, st, (const float *)a.in[0], (_Float16 *)a.out[0], batch, cols);
     const hipError_t e = hipGetLastError();
@@ -1181,21 +1191,21 @@ int bind_round_prep(ksh_kernel &k)
     const int64_t cols = k.desc.dims[0], batch = k.desc.dims[1], mode = k.desc.dims[2];
     if (cols <= 0 || cols % 256 || cols > (1 << 16)) return set_error("round_prep: cols=%lld is not a positive multiple of 256 up to 65536", (long long)cols);
     if (batch < 1 || batch > kRoundTokens) return set_error("round_prep: %lld rows (1 to %d)", (long long)batch, kRoundTokens);
-    if (mode < 0 || mode > 2) return set_error("round_prep: mode %lld (0 plain, 1 rmsnorm, 2 add then rmsnorm)", (long long)mode);
-    if (mode == 2 && cols > 8192) return set_error("round_prep: the add-then-norm form keeps a row in LDS (cols=%lld, up to 8192)", (long long)cols);
-    k.info.n_inputs = mode == 2 ? 4 : mode == 1 ? 2 : 1;
-    k.info.n_outputs = mode == 2 ? 2 : 1;
+    if (mode < 0 || mode > 3) return set_error("round_prep: mode %lld (0 plain, 1 rmsnorm, 2 add then rmsnorm, 3 rmsnorm add)", (long long)mode);
+    if (mode >= 2 && cols > 8192) return set_error("round_prep: the add-then-norm form keeps a row in LDS (cols=%lld, up to 8192)", (long long)cols);
+    k.info.n_inputs = mode == 2 ? 4 : mode == 3 ? 3 : mode == 1 ? 2 : 1;
+    k.info.n_outputs = mode >= 2 ? 2 : 1;
     k.in_bytes[0] = (size_t)batch * cols * 4; k.in_align[0] = 16;
     if (mode) { k.in_bytes[1] = (size_t)cols * 4; k.in_align[1] = 4; }
-    if (mode == 2) {
+    if (mode >= 2) {
         k.in_bytes[2] = (size_t)batch * cols * 4; k.in_align[2] = 4;
-        k.in_bytes[3] = (size_t)cols * 4; k.in_align[3] = 4;
+        if (mode == 2) { k.in_bytes[3] = (size_t)cols * 4; k.in_align[3] = 4; }
         k.out_bytes[1] = (size_t)batch * cols * 4; k.out_align[1] = 4;
     }
     k.out_bytes[0] = (round_xf_halves((int)cols) + 2 * round_sx_halves((int)cols)) * 2; k.out_align[0] = 16;
-    if (mode) set_launch(k, kRoundTokens, 1, 1, 256, mode == 2 ? (uint32_t)cols * 4 : 0);
+    if (mode) set_launch(k, kRoundTokens, 1, 1, 256, mode >= 2 ? (uint32_t)cols * 4 : 0);
     else set_launch(k, (uint32_t)((kRoundTokens * (cols / 8) + 255) / 256), 1, 1, 256, 0);
-    set_name(k, mode == 2 ? "round_prep_add_then_rmsnorm" : mode == 1 ? "round_prep_rmsnorm" : "round_prep_f32x");
+    set_name(k, mode == 3 ? "round_prep_rmsnorm_add" : mode == 2 ? "round_prep_add_then_rmsnorm" : mode == 1 ? "round_prep_rmsnorm" : "round_prep_f32x");
     k.launch = launch_round_prep;
     return 0;
 }

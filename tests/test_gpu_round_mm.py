@@ -170,6 +170,18 @@ def test_round_prep_norm_forms_equal_norm_then_prep(ctx, cols, batch):
     assert np.allclose(ctx.read_f32(xn_got, batch * cols), ctx.read_f32(xn_want, batch * cols), rtol=1e-6, atol=1e-6)   # (a sum that may cancel)
     # (x_new is a sum that may cancel: the two kernels' last bits of it differ, and the second norm carries that along)
     check(ctx.read_f32(x2, batch * cols), "mode 2", tol=1e-5, floor=0.1)
+    # mode 2 with a scale on x_new (rmsnorm_add_scale rows, then the next norm), mode 3 (rmsnorm_add rows, prepared as it is)
+    scale = 0.375
+    xs = ctx.buffer_empty_f32(batch * cols)
+    ctx.encode_multi(ctx.compile(hip.make_desc(Kind.RMSNORM, (cols, 1, 1, batch), (), (eps, scale))), [bx, bw1, br], [xs])
+    ctx.encode_multi(ctx.compile(hip.make_desc(Kind.RMSNORM, (cols, 0, 0, batch), (), (eps,))), [xs, bw2], [x2])
+    ctx.encode_multi(ctx.compile(hip.make_desc(Kind.ROUND_PREP, (cols, batch, 2), (DType.F32,), (eps, scale))), [bx, bw1, br, bw2], [got, xn_got])
+    assert np.allclose(ctx.read_f32(xn_got, batch * cols), ctx.read_f32(xs, batch * cols), rtol=1e-6, atol=1e-6)
+    check(ctx.read_f32(x2, batch * cols), "mode 2 with a scale", tol=1e-5, floor=0.1)
+    ctx.encode_multi(ctx.compile(hip.make_desc(Kind.RMSNORM, (cols, 1, 0, batch), (), (eps,))), [bx, bw1, br], [xs])
+    ctx.encode_multi(ctx.compile(hip.make_desc(Kind.ROUND_PREP, (cols, batch, 3), (DType.F32,), (eps,))), [bx, bw1, br], [got, xn_got])
+    assert np.allclose(ctx.read_f32(xn_got, batch * cols), ctx.read_f32(xs, batch * cols), rtol=1e-6, atol=1e-6)
+    check(ctx.read_f32(xn_got, batch * cols), "mode 3")
 
 
 def q6k_blocks_full_scales(n_blocks, seed):

@@ -277,7 +277,7 @@ def bench_decode_gemma4_layout(ctx, eng, use_graph=True):
     # for comparison); one host read-back per round
     pool = hip.KvPool(ctx, 16, cfg["max_seq"], n - shared, 512, 1)
     served = {}
-    for n_req, batched in ((2, 0), (2, 2), (4, 0), (4, 2), (8, 2), (16, 2)):
+    for n_req, batched in ((2, 0), (2, 2), (3, 2), (4, 0), (4, 2), (8, 2), (16, 2)):
         sv = hip.Serve(model, pool, slots=n_req, eos=(0xFFFFFFFF, 0xFFFFFFFE), use_graph=use_graph, batched_decode=batched)
         best = 1e9
         for rep in range(2):

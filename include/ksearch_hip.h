@@ -540,7 +540,7 @@ typedef struct {
     int32_t prefill_tokens_per_tick;   /* 2048 */
     uint32_t eos[2];                   /* EOS_IDS (scheduler.rs:14): 1, 106 */
     int32_t use_graph;                 /* replay the model's HIP graphs (1) or launch eagerly (0) */
-    int32_t batched_decode;            /* from this many decoding requests on (>= 2; default 4) they take their step as one
+    int32_t batched_decode;            /* from this many decoding requests on (>= 2; default 3) they take their step as one
                                         * ksh_gemma4_decode_round (the weights are read once per round); 0: always one
                                         * by one, as the reference does */
     ksh_serve_stop_fn stop;            /* may be NULL */

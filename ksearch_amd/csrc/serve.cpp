@@ -246,7 +246,7 @@ int ksh_serve_default_cfg(ksh_serve_cfg *cfg)
     cfg->eos[0] = 1;                       // EOS_IDS, scheduler.rs:14
     cfg->eos[1] = 106;
     cfg->use_graph = 1;
-    cfg->batched_decode = 4;   // a joint step costs about four single ones at the real checkpoints' layer layout
+    cfg->batched_decode = 3;   // a joint step costs about two and a half single ones at the real checkpoints' layer layout
     return 0;
 }
 

@@ -1004,7 +1004,7 @@ class Serve:
     completion_tokens), ("error", request, text)."""
 
     def __init__(self, model, pool, slots: int = 4, prefill_chunk: int = 256, prefill_tokens_per_tick: int = 2048,
-                 eos=(1, 106), use_graph: bool = True, stop=None, batched_decode: int = 4):
+                 eos=(1, 106), use_graph: bool = True, stop=None, batched_decode: int = 3):
         cfg = ServeCfg()
         _check(lib().ksh_serve_default_cfg(C.byref(cfg)))
         cfg.batched_decode = int(batched_decode)      # joint decode steps from this many decoding requests on; 0: never

@@ -58,7 +58,7 @@ class Rig:
         c = ServeCfg()
         assert L.ksh_serve_default_cfg(C.byref(c)) == 0
         assert (c.slots, c.prefill_chunk, c.prefill_tokens_per_tick, tuple(c.eos), c.use_graph) == (4, 256, 2048, (1, 106), 1)
-        assert c.batched_decode == 4
+        assert c.batched_decode == 3
         c.eos[0], c.eos[1] = cfg.pop("eos", NO_EOS)
         cfg.setdefault("batched_decode", 0)      # the reference's serial rounds unless a test asks for batched ones
         for k, v in cfg.items():

@@ -772,6 +772,66 @@ __global__ __launch_bounds__(256) void mm_round_prep_norm_kernel(const float *__
     }
 }
 
+// The same for rows of up to 2048 columns (the widths of the models this serves): thread j owns elements 8 j .. 8 j + 7
+// from the first load to the fragment it writes, every input is requested up front, and the row never passes through
+// LDS -- the launch is one round trip and two block sums where the form above is three dependent passes.  (The sums
+// of squares are taken in a different order than the kernels that write f32 rows: equal to the last bit or two.)
+template <int MODE>
+__global__ __launch_bounds__(256) void mm_round_prep_norm8_kernel(const float *__restrict__ x, const float *__restrict__ w_first, const float *res,
+                                                                  const float *__restrict__ w_norm, float *x_new, _Float16 *__restrict__ Xp,
+                                                                  int batch, int cols, float eps, float scale)
+{
+    __shared__ float red[4];
+    const int t = blockIdx.x, k8 = cols / 8, j = threadIdx.x;
+    const bool has = j < k8;                  // (whole quads: cols is a multiple of 32)
+    if (t >= batch) {
+        const float zero[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        if (has) round_prep_write(zero, t, j, cols, Xp);
+        return;
+    }
+    const f32x4_t z4 = {0.f, 0.f, 0.f, 0.f};
+    const size_t e = (size_t)t * cols + 8 * (size_t)min(j, k8 - 1), ew = 8 * (size_t)min(j, k8 - 1);
+    auto ld8 = [&](const float *p, size_t off, float (&o)[8]) {
+        const f32x4_t a = has ? *reinterpret_cast<const f32x4_t *>(p + off) : z4, b = has ? *reinterpret_cast<const f32x4_t *>(p + off + 4) : z4;
+        o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w; o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+    };
+    float y[8], w1[8], r[8], w2[8];
+    ld8(x, e, y);
+    ld8(w_first, ew, w1);
+    if (MODE >= 2) ld8(res, e, r);
+    if (MODE == 2) ld8(w_norm, ew, w2);
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; i++) ss = __fadd_rn(ss, __fmul_rn(y[i], y[i]));
+    ss = round_block_sum(ss, red);
+    float inv = 1.0f / sqrtf(__fadd_rn(ss / (float)cols, eps));
+    float f[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) f[i] = __fmul_rn(__fmul_rn(y[i], inv), w1[i]);
+    if (MODE >= 2) {
+        float ss2 = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            f[i] = __fadd_rn(f[i], r[i]);
+            if (scale != 0.f) f[i] = __fmul_rn(scale, f[i]);
+            ss2 = __fadd_rn(ss2, __fmul_rn(f[i], f[i]));
+        }
+        if (has) {
+            *reinterpret_cast<f32x4_t *>(x_new + e) = f32x4_t{f[0], f[1], f[2], f[3]};
+            *reinterpret_cast<f32x4_t *>(x_new + e + 4) = f32x4_t{f[4], f[5], f[6], f[7]};
+        }
+        if (MODE == 2) {
+            ss2 = round_block_sum(ss2, red);
+            inv = 1.0f / sqrtf(__fadd_rn(ss2 / (float)cols, eps));
+#pragma unroll
+            for (int i = 0; i < 8; i++) f[i] = __fmul_rn(__fmul_rn(f[i], inv), w2[i]);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; i++) f[i] = pinned(f[i]);
+    if (has) round_prep_write(f, t, j, cols, Xp);
+}
+
 struct RoundParams {
     const uint8_t *W0, *W1, *W2;
     float *Y0, *Y1, *Y2;
@@ -1042,16 +1102,25 @@ int launch_round_prep(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
 {
     const int cols = (int)k.desc.dims[0], batch = (int)k.desc.dims[1], mode = (int)k.desc.dims[2];
     const int n = kRoundTokens * (cols / 8);
-    if (mode == 1)
-        hipLaunchKernelGGL(mm_round_prep_norm_kernel<1>, dim3(kRoundTokens), dim3(256), 0, st, (const float *)a.in[0], (const float *)a.in[1], nullptr, nullptr,
-                           nullptr, (_Float16 *)a.out[0], batch, cols, k.desc.params[0], 0.f);
-    else if (mode == 2)
-        hipLaunchKernelGGL(mm_round_prep_norm_kernel<2>, dim3(kRoundTokens), dim3(256), (size_t)cols * 4, st, (const float *)a.in[0], (const float *)a.in[1],
-                           (const float *)a.in[2], (const float *)a.in[3], (float *)a.out[1], (_Float16 *)a.out[0], batch, cols, k.desc.params[0],
-                           k.desc.params[1]);
-    else if (mode == 3)
-        hipLaunchKernelGGL(mm_round_prep_norm_kernel<3>, dim3(kRoundTokens), dim3(256), (size_t)cols * 4, st, (const float *)a.in[0], (const float *)a.in[1],
-                           (const float *)a.in[2], nullptr, (float *)a.out[1], (_Float16 *)a.out[0], batch, cols, k.desc.params[0], 0.f);
+    const float *in1 = mode ? (const float *)a.in[1] : nullptr, *in2 = mode >= 2 ? (const float *)a.in[2] : nullptr,
+                *in3 = mode == 2 ? (const float *)a.in[3] : nullptr;
+    float *x_new = mode >= 2 ? (float *)a.out[1] : nullptr;
+    const float scale = mode == 2 ? k.desc.params[1] : 0.f;
+#define KSH_PN(KERNEL, M, LDS) \
+    hipLaunchKernelGGL(KERNEL<M>, dim3(kRoundTokens), dim3(256), LDS, st, (const float *)a.in[0], in1, in2, in3, x_new, (_Float16 *)a.out[0], batch, cols, \
+                       k.desc.params[0], scale)
+    if (mode && cols <= 2048) {
+        if (mode == 1) KSH_PN(mm_round_prep_norm8_kernel, 1, 0);
+        else if (mode == 2) KSH_PN(mm_round_prep_norm8_kernel, 2, 0);
+        else KSH_PN(mm_round_prep_norm8_kernel, 3, 0);
+    } else if (mode == 1) {
+        KSH_PN(mm_round_prep_norm_kernel, 1, 0);
+    } else if (mode == 2) {
+        KSH_PN(mm_round_prep_norm_kernel, 2, (size_t)cols * 4);
+    } else if (mode == 3) {
+        KSH_PN(mm_round_prep_norm_kernel, 3, (size_t)cols * 4);
+    }
+#undef KSH_PN
     else
         hipLaunchKernelGGL(mm_round_prep_kernel, dim3((n + 255) / 256), dim3(256), 0, st, (const float *)a.in[0], (_Float16 *)a.out[0], batch, cols);
     const hipError_t e = hipGetLastError();
@@ -1196,11 +1265,12 @@ int bind_round_prep(ksh_kernel &k)
     k.info.n_inputs = mode == 2 ? 4 : mode == 3 ? 3 : mode == 1 ? 2 : 1;
     k.info.n_outputs = mode >= 2 ? 2 : 1;
     k.in_bytes[0] = (size_t)batch * cols * 4; k.in_align[0] = 16;
-    if (mode) { k.in_bytes[1] = (size_t)cols * 4; k.in_align[1] = 4; }
+    // (128-bit loads and stores of every operand)
+    if (mode) { k.in_bytes[1] = (size_t)cols * 4; k.in_align[1] = 16; }
     if (mode >= 2) {
-        k.in_bytes[2] = (size_t)batch * cols * 4; k.in_align[2] = 4;
-        if (mode == 2) { k.in_bytes[3] = (size_t)cols * 4; k.in_align[3] = 4; }
-        k.out_bytes[1] = (size_t)batch * cols * 4; k.out_align[1] = 4;
+        k.in_bytes[2] = (size_t)batch * cols * 4; k.in_align[2] = 16;
+        if (mode == 2) { k.in_bytes[3] = (size_t)cols * 4; k.in_align[3] = 16; }
+        k.out_bytes[1] = (size_t)batch * cols * 4; k.out_align[1] = 16;
     }
     k.out_bytes[0] = (round_xf_halves((int)cols) + 2 * round_sx_halves((int)cols)) * 2; k.out_align[0] = 16;
     if (mode) set_launch(k, kRoundTokens, 1, 1, 256, mode >= 2 ? (uint32_t)cols * 4 : 0);

@@ -1100,6 +1100,11 @@ int encode_round4(ksh_gemma4 *m, ksh_kvpool *pool, int t, int max_batch, int poo
             mm1(L.dt_o, h, P.qd, L.wo, m->c_o, m->c_y))
             return 1;
         const bool gu_q4k = L.dt_gate == KSH_Q4K && L.dt_up == KSH_Q4K && h <= 8192;
+        const bool ple_q4k = c.ple_dim > 0 && L.dt_inp_gate == KSH_Q4K && L.dt_proj == KSH_Q4K && c.ple_dim % 256 == 0 && h <= 2048;
+        // a down projection whose columns are split leaves its slices' partial sums (in c_g) to the closing norm where
+        // that norm is the kind that adds them up
+        const int down_slices = (int)((L.ffn / 256 + 7) / 8);
+        const bool down_unfolded = L.dt_down == KSH_Q4K && ple_q4k && down_slices > 1;
         bool down_done = false;
         if (!gu_q4k && enc(m, k_add_then, {m->c_y, L.post_attn_norm, m->c_x, L.ffn_norm}, {m->c_x, m->c_x2}, n)) return 1;
         if (gu_q4k) {
@@ -1114,24 +1119,31 @@ int encode_round4(ksh_gemma4 *m, ksh_kvpool *pool, int t, int max_batch, int poo
                 return 1;
             if (chain) {
                 ksh_kernel *k_dn = nullptr;
-                if (get(m, KSH_MATVEC_ROUND, {h, L.ffn, t, 0, 0, 0}, {KSH_Q4K}, {}, &k_dn) || enc(m, k_dn, {L.wdown, m->r_xp2}, {m->c_y}, n)) return 1;
+                if (get(m, KSH_MATVEC_ROUND, {h, L.ffn, t, 0, 0, 0, down_unfolded ? 2 : 0}, {KSH_Q4K}, {}, &k_dn) ||
+                    enc(m, k_dn, {L.wdown, m->r_xp2}, {down_unfolded ? m->c_g : m->c_y}, n))
+                    return 1;
                 down_done = true;
             }
         } else if (mm(L.dt_gate, L.ffn, h, L.wgate, m->c_x2, m->c_g) || mm(L.dt_up, L.ffn, h, L.wup, m->c_x2, m->c_u) ||
                    get(m, KSH_GELU_MUL, {(int64_t)t * L.ffn}, {}, {}, &k_gelu) || enc(m, k_gelu, {m->c_g, m->c_u}, {m->c_ff}, n)) {
             return 1;
         }
+        if (!down_done && down_unfolded) {
+            ksh_kernel *k_dn = nullptr;
+            if (prep(L.ffn, m->c_ff) || get(m, KSH_MATVEC_ROUND, {h, L.ffn, t, 0, 0, 0, 2}, {KSH_Q4K}, {}, &k_dn) || enc(m, k_dn, {L.wdown, m->r_xp}, {m->c_g}, n))
+                return 1;
+            down_done = true;
+        }
         if (!down_done && mm1(L.dt_down, h, L.ffn, L.wdown, m->c_ff, m->c_y)) return 1;
         // the feed-forward block's closing norm + add
-        const bool ple_q4k = c.ple_dim > 0 && L.dt_inp_gate == KSH_Q4K && L.dt_proj == KSH_Q4K && c.ple_dim % 256 == 0 && h <= 2048;
         if (c.ple_dim == 0) {
             if (close_layer(l, L.post_ffw_norm, 0.f, k_add)) return 1;
         } else if (ple_q4k) {
             // ... which also prepares the new residual stream for the per-layer-embedding gate (mode 3); the gate's
             // gelu(W x) * context leaves as the projection's prepared operand
             ksh_kernel *k_pa = nullptr, *k_pg = nullptr, *k_pp = nullptr, *k_as = nullptr;
-            if (get(m, KSH_ROUND_PREP, {h, t, 3}, {KSH_F32}, {c.eps}, &k_pa) ||
-                enc(m, k_pa, {m->c_y, L.post_ffw_norm, m->c_x}, {m->r_xp, m->c_x}, n) ||
+            if (get(m, KSH_ROUND_PREP, {h, t, 3, down_unfolded ? down_slices : 0}, {KSH_F32}, {c.eps}, &k_pa) ||
+                enc(m, k_pa, {down_unfolded ? m->c_g : m->c_y, L.post_ffw_norm, m->c_x}, {m->r_xp, m->c_x}, n) ||
                 get(m, KSH_MATVEC_ROUND, {c.ple_dim, h, t, 0, 0, 0, 1, pt}, {KSH_Q4K}, {}, &k_pg) ||
                 enc_off(m, k_pg, {L.inp_gate, m->r_xp, m->c_ple_ctx}, {0, 0, (size_t)l * c.ple_dim * 4}, {m->r_xp2}, n) ||
                 get(m, KSH_MATVEC_ROUND, {h, c.ple_dim, t, 0, 0, 0}, {KSH_Q4K}, {}, &k_pp) || enc(m, k_pp, {L.proj, m->r_xp2}, {m->c_y}, n) ||

@@ -779,7 +779,7 @@ __global__ __launch_bounds__(256) void mm_round_prep_norm_kernel(const float *__
 template <int MODE>
 __global__ __launch_bounds__(256) void mm_round_prep_norm8_kernel(const float *__restrict__ x, const float *__restrict__ w_first, const float *res,
                                                                   const float *__restrict__ w_norm, float *x_new, _Float16 *__restrict__ Xp,
-                                                                  int batch, int cols, float eps, float scale)
+                                                                  int batch, int cols, float eps, float scale, int slices)
 {
     __shared__ float red[4];
     const int t = blockIdx.x, k8 = cols / 8, j = threadIdx.x;
@@ -797,6 +797,14 @@ __global__ __launch_bounds__(256) void mm_round_prep_norm8_kernel(const float *_
     };
     float y[8], w1[8], r[8], w2[8];
     ld8(x, e, y);
+    // x as the column slices' partial sums of a split GEMM ([slices][batch][cols]): added here, slice after slice, in
+    // the order the GEMM's own second launch adds them
+    for (int sl = 1; sl < slices; sl++) {
+        float ys[8];
+        ld8(x, (size_t)sl * batch * cols + e, ys);
+#pragma unroll
+        for (int i = 0; i < 8; i++) y[i] = __fadd_rn(y[i], ys[i]);
+    }
     ld8(w_first, ew, w1);
     if (MODE >= 2) ld8(res, e, r);
     if (MODE == 2) ld8(w_norm, ew, w2);
@@ -1106,13 +1114,17 @@ int launch_round_prep(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
                 *in3 = mode == 2 ? (const float *)a.in[3] : nullptr;
     float *x_new = mode >= 2 ? (float *)a.out[1] : nullptr;
     const float scale = mode == 2 ? k.desc.params[1] : 0.f;
+    const int slices = (int)std::max<int64_t>(1, k.desc.dims[3]);
 #define KSH_PN(KERNEL, M, LDS) \
     hipLaunchKernelGGL(KERNEL<M>, dim3(kRoundTokens), dim3(256), LDS, st, (const float *)a.in[0], in1, in2, in3, x_new, (_Float16 *)a.out[0], batch, cols, \
                        k.desc.params[0], scale)
+#define KSH_PN8(M) \
+    hipLaunchKernelGGL(mm_round_prep_norm8_kernel<M>, dim3(kRoundTokens), dim3(256), 0, st, (const float *)a.in[0], in1, in2, in3, x_new, \
+                       (_Float16 *)a.out[0], batch, cols, k.desc.params[0], scale, slices)
     if (mode && cols <= 2048) {
-        if (mode == 1) KSH_PN(mm_round_prep_norm8_kernel, 1, 0);
-        else if (mode == 2) KSH_PN(mm_round_prep_norm8_kernel, 2, 0);
-        else KSH_PN(mm_round_prep_norm8_kernel, 3, 0);
+        if (mode == 1) KSH_PN8(1);
+        else if (mode == 2) KSH_PN8(2);
+        else KSH_PN8(3);
     } else if (mode == 1) {
         KSH_PN(mm_round_prep_norm_kernel, 1, 0);
     } else if (mode == 2) {
@@ -1121,6 +1133,7 @@ int launch_round_prep(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
         KSH_PN(mm_round_prep_norm_kernel, 3, (size_t)cols * 4);
     }
 #undef KSH_PN
+#undef KSH_PN8
     else
         hipLaunchKernelGGL(mm_round_prep_kernel, dim3((n + 255) / 256), dim3(256), 0, st, (const float *)a.in[0], (_Float16 *)a.out[0], batch, cols);
     const hipError_t e = hipGetLastError();
@@ -1157,13 +1170,14 @@ int launch_matvec_round(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st
     p.cols = (int)d[1]; p.batch = (int)d[2];
     p.part = (float *)k.scratch;
     if (d[7]) { p.mul = (const float *)a.in[2]; p.mul_stride = (int)d[7]; }
-    if (d[6]) { p.emit = (_Float16 *)a.out[0]; p.Y0 = p.Y1 = p.Y2 = nullptr; }
+    if (d[6] == 1) { p.emit = (_Float16 *)a.out[0]; p.Y0 = p.Y1 = p.Y2 = nullptr; }
+    if (d[6] == 2) p.part = (float *)a.out[0];     // the slices' partial sums are the result
     const dim3 grid(k.info.grid[0], k.info.grid[1]);
     if (pair) hipLaunchKernelGGL(q4k_mm_round_kernel<2>, grid, dim3(512), k.info.lds_bytes, st, p);
     else hipLaunchKernelGGL(q4k_mm_round_kernel<1>, grid, dim3(512), k.info.lds_bytes, st, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return hip_fail(e, "matvec_round launch");
-    if (grid.y > 1) {
+    if (grid.y > 1 && d[6] != 2) {
         const int n = p.batch * p.rows0;
         hipLaunchKernelGGL(mm_round_fold_kernel, dim3((n + 255) / 256), dim3(256), 0, st, (const float *)k.scratch, p.Y0, n, (int)grid.y);
         e = hipGetLastError();
@@ -1262,9 +1276,12 @@ int bind_round_prep(ksh_kernel &k)
     if (batch < 1 || batch > kRoundTokens) return set_error("round_prep: %lld rows (1 to %d)", (long long)batch, kRoundTokens);
     if (mode < 0 || mode > 3) return set_error("round_prep: mode %lld (0 plain, 1 rmsnorm, 2 add then rmsnorm, 3 rmsnorm add)", (long long)mode);
     if (mode >= 2 && cols > 8192) return set_error("round_prep: the add-then-norm form keeps a row in LDS (cols=%lld, up to 8192)", (long long)cols);
+    const int64_t slices = std::max<int64_t>(1, k.desc.dims[3]);
+    if (k.desc.dims[3] < 0 || slices > 64 || (slices > 1 && (!mode || cols > 2048)))
+        return set_error("round_prep: an input in %lld column slices takes a norm (mode 1 to 3) and rows of up to 2048 columns", (long long)k.desc.dims[3]);
     k.info.n_inputs = mode == 2 ? 4 : mode == 3 ? 3 : mode == 1 ? 2 : 1;
     k.info.n_outputs = mode >= 2 ? 2 : 1;
-    k.in_bytes[0] = (size_t)batch * cols * 4; k.in_align[0] = 16;
+    k.in_bytes[0] = (size_t)slices * batch * cols * 4; k.in_align[0] = 16;
     // (128-bit loads and stores of every operand)
     if (mode) { k.in_bytes[1] = (size_t)cols * 4; k.in_align[1] = 16; }
     if (mode >= 2) {
@@ -1312,7 +1329,8 @@ int bind_matvec_round(ksh_kernel &k)
     if (pair && (rows1 || rows2)) return set_error("matvec_round: a gate | up pair names one row count (both matrices have it)");
     const int slices = (int)((cols / 256 + 7) / 8);
     if (slices > 1 && (pair || rows1)) return set_error("matvec_round: rows longer than 2048 columns take one matrix per launch");
-    const bool emit = d[6] != 0;
+    const bool emit = d[6] == 1, unfolded = d[6] == 2;
+    if (d[6] < 0 || d[6] > 2) return set_error("matvec_round: result form %lld (0 rows, 1 prepared operand, 2 the column slices' partial sums)", (long long)d[6]);
     const int64_t mul_stride = d[7];
     if (mul_stride && (pair || rows1 || mul_stride < rows0)) return set_error("matvec_round: the gate multiplier takes one matrix and a row stride of at least its rows");
     if (emit && (rows1 || slices > 1 || rows0 % 256))
@@ -1327,7 +1345,9 @@ int bind_matvec_round(ksh_kernel &k)
     if (mul_stride) { k.info.n_inputs = 3; k.in_bytes[2] = ((size_t)(batch - 1) * mul_stride + rows0) * 4; k.in_align[2] = 4; }
     for (int i = 0; i < k.info.n_outputs; i++) { k.out_bytes[i] = (size_t)batch * rows[i] * 4; k.out_align[i] = 4; }
     if (emit) { k.out_bytes[0] = (round_xf_halves((int)rows0) + 2 * round_sx_halves((int)rows0)) * 2; k.out_align[0] = 16; }
-    k.scratch_bytes = slices > 1 ? (size_t)slices * batch * rows0 * 4 : 0;
+    if (unfolded && (rows1 || pair)) return set_error("matvec_round: partial sums as the result take one matrix");
+    k.scratch_bytes = slices > 1 && !unfolded ? (size_t)slices * batch * rows0 * 4 : 0;
+    if (unfolded) k.out_bytes[0] = (size_t)slices * batch * rows0 * 4;
     const int64_t tiles = pair ? (rows0 + 31) / 32 : (rows0 + 31) / 32 + (rows1 + 31) / 32 + (rows2 + 31) / 32;
     set_launch(k, (uint32_t)tiles, (uint32_t)slices, 1, 512, (uint32_t)(8 * (pair ? 2 : 1) * 8 * 64 * 4 + (emit ? 16 * 33 * 4 : 0)));
     k.info.sched = k.desc.sched;

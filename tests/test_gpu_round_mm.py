@@ -104,6 +104,32 @@ def test_matvec_round_result_as_prepared_operand(ctx, batch):
     assert np.allclose(vals[:batch], ctx.read_f32(y, batch * rows).reshape(batch, rows), rtol=2.0 ** -19, atol=1e-6)
 
 
+def test_matvec_round_partial_sums_into_the_closing_norm(ctx):
+    """dims[6] = 2 leaves a split GEMM's column slices unadded, and KSH_ROUND_PREP with dims[3] = slices adds them
+    on its way into the norm: the same x_new and operand as the folded GEMM followed by the plain norm kinds."""
+    rows, cols, batch, eps = 1536, 6144, 9, 1e-6
+    w = synth.q4k_blocks(rows * cols // 256, seed=980)
+    x = synth.normal_f32(batch * cols, 981).reshape(batch, cols) * 0.1
+    res, wn = synth.normal_f32(batch * rows, 982), (1.0 + 0.05 * synth.normal_f32(rows, 983)).astype(np.float32)
+    _, (y,) = round_mm(ctx, [w], (rows,), cols, x, batch)
+    xp = prepared(ctx, x, batch, cols)
+    k = ctx.compile(hip.make_desc(Kind.MATVEC_ROUND, (rows, cols, batch, 0, 0, 0, 2), (DType.Q4K,)))
+    slices = k.info.sched.k_split
+    assert slices == 3
+    parts = ctx.buffer_empty_f32(slices * batch * rows)
+    ctx.encode_multi(k, [ctx.buffer_bytes(w), xp], [parts])
+    p = ctx.read_f32(parts, slices * batch * rows).reshape(slices, batch, rows)
+    assert np.array_equal((p[0] + p[1] + p[2]).view(np.uint32), y.view(np.uint32))      # slice after slice, as the fold adds them
+    n_xp = 64 * rows + 2048 * (rows // 256)
+    got, want = ctx.buffer_empty_bytes(n_xp), ctx.buffer_empty_bytes(n_xp)
+    xn_got, xn_want = ctx.buffer_empty_f32(batch * rows), ctx.buffer_empty_f32(batch * rows)
+    bres, bwn = ctx.buffer_f32(res), ctx.buffer_f32(wn)
+    ctx.encode_multi(ctx.compile(hip.make_desc(Kind.ROUND_PREP, (rows, batch, 3, slices), (DType.F32,), (eps,))), [parts, bwn, bres], [got, xn_got])
+    ctx.encode_multi(ctx.compile(hip.make_desc(Kind.ROUND_PREP, (rows, batch, 3), (DType.F32,), (eps,))), [ctx.buffer_f32(y.reshape(-1)), bwn, bres], [want, xn_want])
+    assert np.array_equal(ctx.read_f32(xn_got, batch * rows).view(np.uint32), ctx.read_f32(xn_want, batch * rows).view(np.uint32))
+    assert np.array_equal(ctx.read_bytes(got, n_xp), ctx.read_bytes(want, n_xp))
+
+
 def test_matvec_round_unit_rows_recover_weights(ctx):
     # X = one-hot rows: Y[t] is column k_t of the dequantized matrix (pins the K order and the hi | lo tile end to end)
     rows, cols = 64, 4096

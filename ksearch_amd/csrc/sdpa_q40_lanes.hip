@@ -932,7 +932,7 @@ __global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_m
             float sum = 0.f;
 #pragma unroll
             for (int s2 = 0; s2 < 8; s2++) {
-                const float xs = have ? x[s2] * p.scale : 0.f;
+                const float xs = pinned(have ? x[s2] * p.scale : 0.f);   // (a product on its way into a hi | lo split)
                 const _Float16 hi = (_Float16)xs;
                 const _Float16 lo = (_Float16)(xs - (float)hi);
                 const _Float16 v = is_lo ? lo : hi;

@@ -84,7 +84,9 @@ enum ksh_kind {
      * in: q[n_slots,n_q*hd], Kpool, Vpool, meta   out: tmp, o[n_slots,n_q*hd]
      * dims[6] = pool slots > 0: the launch's n_slots entries are a subset, in any order, of pools that hold dims[6]
      * slots (one decode step for several sequences); a 5th input f32[n_slots] names each entry's pool slot, and
-     * dims[7] is the byte distance between slots of the pools (0: max_t rows). */
+     * dims[7] is the byte distance between slots of the pools (0: max_t rows).
+     * params[1] != 0: the second output is the prepared operand of a decode round's GEMM over the n_q * hd columns
+     * (as KSH_ROUND_PREP writes it, row = entry) instead of f32 rows; 2 to 16 slots, 2 to 64 partitions. */
     KSH_SDPA_SLOTS = 8,
     /* QuantizeQ40: pack n f32 values (n%32==0) to Q4_0.  dims: n.  in: src  out: dst */
     KSH_QUANTIZE_Q40 = 9,

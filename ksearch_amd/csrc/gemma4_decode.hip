@@ -1094,11 +1094,18 @@ int encode_round4(ksh_gemma4 *m, ksh_kvpool *pool, int t, int max_batch, int poo
                 run(k_head, {m->c_q, L.q_norm, rope_tab, m->r_tab}, {0, 0, 0, o_meta}, {m->c_q}, {0}))
                 return 1;
         }
+        // the attention's merge writes the o projection's prepared operand itself where that projection takes one
+        const bool o_chain = t >= 2 && L.dt_o == KSH_Q4K && P.qd % 256 == 0;
         if (get(m, KSH_SDPA_SLOTS, {c.n_q, c.n_kv, P.hd, c.max_seq, t, kRoundPartitions, max_batch, (int64_t)slot_stride}, {KSH_Q40, KSH_F32},
-                {c.attn_scale}, &k_sdpa) ||
-            run(k_sdpa, {m->c_q, kc, vc, m->r_tab, m->r_tab}, {0, 0, 0, o_meta, o_slots}, {m->c_tmp, m->c_o}, {0, 0}) ||
-            mm1(L.dt_o, h, P.qd, L.wo, m->c_o, m->c_y))
+                {c.attn_scale, o_chain ? 1.0f : 0.0f}, &k_sdpa) ||
+            run(k_sdpa, {m->c_q, kc, vc, m->r_tab, m->r_tab}, {0, 0, 0, o_meta, o_slots}, {m->c_tmp, o_chain ? m->r_xp : m->c_o}, {0, 0}))
             return 1;
+        if (o_chain) {
+            ksh_kernel *k_o = nullptr;
+            if (get(m, KSH_MATVEC_ROUND, {h, P.qd, t, 0, 0, 0}, {KSH_Q4K}, {}, &k_o) || enc(m, k_o, {L.wo, m->r_xp}, {m->c_y}, n)) return 1;
+        } else if (mm1(L.dt_o, h, P.qd, L.wo, m->c_o, m->c_y)) {
+            return 1;
+        }
         const bool gu_q4k = L.dt_gate == KSH_Q4K && L.dt_up == KSH_Q4K && h <= 8192;
         const bool ple_q4k = c.ple_dim > 0 && L.dt_inp_gate == KSH_Q4K && L.dt_proj == KSH_Q4K && c.ple_dim % 256 == 0 && h <= 2048;
         // a down projection whose columns are split leaves its slices' partial sums (in c_g) to the closing norm where

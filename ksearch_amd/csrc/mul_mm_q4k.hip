@@ -34,11 +34,11 @@
 #include "ksh_device.hpp"
 #include "ksh_internal.hpp"
 #include "q4k_lane.hpp"
+#include "round_operand.hpp"
 
 namespace ksh {
 namespace {
 
-typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef float f16v __attribute__((ext_vector_type(16)));
 typedef _Float16 h2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
@@ -46,10 +46,6 @@ typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 constexpr int BM = 128, BN = 128, KS = 64;
 constexpr int PITCH = KS + 8;      // halves per LDS row of the main tiles (144 B: conflict-free 16 B reads)
 constexpr int PITCH2 = 32 + 8;     // halves per LDS row of the min-term tiles
-
-// within every 4 consecutive k the stored order is (0, 2, 1, 3): that is the
-// order the paired nibble extraction produces, applied to X as well
-__device__ __forceinline__ int kperm(int i) { return (i & ~3) | ((i & 1) << 1) | ((i >> 1) & 1); }
 
 // X bf16 -> f16 (permuted) in the order the matrix instruction wants its A operand, plus the min-term
 // operand per (token, superblock): 32 halves = Sx_hi[8] | Sx_hi[8] | Sx_lo[8] | 0[8].
@@ -635,50 +631,9 @@ __global__ __launch_bounds__(512) void q4k_mm_skinny_kernel(MmParams p, const _F
 // one memory round trip where the small-batch form above walks a wave's superblocks one round trip at a time.  Rows
 // longer than 2048 columns split over blockIdx.y; the slices' sums go to a scratch buffer and a second launch adds
 // them in a fixed order.  Conversion, scales and the bias / min product are those of the forms above.
-constexpr int kRoundTokens = 16;
-
-__host__ __device__ inline size_t round_xf_halves(int cols) { return (size_t)32 * cols; }
-__host__ __device__ inline size_t round_sx_halves(int cols) { return (size_t)kRoundTokens * (cols / 256) * 32; }
 
 // what one thread does with 8 consecutive elements (8 j .. 8 j + 7) of token row t; whole quads call it together
 // (the four threads of a sub-block add their sums up over the quad)
-// 8 consecutive values as the hi and lo halves of a fragment lane, and the sums of the two parts
-__device__ __forceinline__ void round_split8(const float (&f)[8], h8 &oh, h8 &ol, float &sh, float &sl)
-{
-    float fh[8], fl[8];
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-        const _Float16 hi = (_Float16)f[i];
-        const _Float16 lo = (_Float16)((f[i] - (float)hi) * 2048.0f);   // kept 2^11 up, in the normal range wherever hi is
-        oh[kperm(i)] = hi;
-        ol[kperm(i)] = lo;
-        fh[i] = (float)hi;
-        fl[i] = (float)lo;
-    }
-    sh = ((fh[0] + fh[1]) + (fh[2] + fh[3])) + ((fh[4] + fh[5]) + (fh[6] + fh[7]));
-    sl = ((fl[0] + fl[1]) + (fl[2] + fl[3])) + ((fl[4] + fl[5]) + (fl[6] + fl[7]));
-}
-
-// the sums of a sub-block's hi and lo parts as the bias / min product reads them: hi[8] hi[8] lo[8] 0[8] per row and
-// superblock, entry jj of each
-__device__ __forceinline__ void round_store_sums(_Float16 *__restrict__ Xp, int cols, int t, int sub_block, float sh, float sl)
-{
-    const int jj = sub_block % 8;
-    _Float16 *sx = Xp + round_xf_halves(cols) + ((size_t)t * (cols / 256) + sub_block / 8) * 32;
-    const float sums[2] = {sh, sl};
-#pragma unroll
-    for (int part = 0; part < 2; part++) {
-        _Float16 *dst = sx + part * round_sx_halves(cols);
-        const float sum = pinned(sums[part]);
-        const _Float16 hi = (_Float16)sum;
-        const _Float16 lo = (_Float16)(sum - (float)hi);
-        dst[jj] = hi;
-        dst[8 + jj] = hi;
-        dst[16 + jj] = lo;
-        dst[24 + jj] = (_Float16)0.f;
-    }
-}
-
 __device__ __forceinline__ void round_prep_write(const float (&f)[8], int t, int j, int cols, _Float16 *__restrict__ Xp)
 {
     h8 oh, ol;

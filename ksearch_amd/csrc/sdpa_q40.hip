@@ -416,6 +416,15 @@ int bind_sdpa(ksh_kernel &k)
         k.out_bytes[0] = (size_t)n_slots * n_q * nwg * (hd + 2) * 4;
         k.out_bytes[1] = (size_t)n_slots * n_q * hd * 4;
         k.out_align[1] = 4;
+        if (k.desc.params[1] != 0.f) {
+            // params[1] != 0: out[1] is the prepared operand of a decode round's GEMM (KSH_MATVEC_ROUND) over the n_q * hd
+            // columns, row = slot
+            const int64_t cols = n_q * hd;
+            if (!lanes || n_slots < 2 || n_slots > 16 || nwg < 2 || nwg > 64 || cols % 256)
+                return set_error("sdpa_slots: the result as a prepared operand takes 2 to 16 slots, 2 to 64 partitions and n_q * hd a multiple of 256");
+            k.out_bytes[1] = (size_t)(64 * cols + 2048 * (cols / 256));
+            k.out_align[1] = 16;
+        }
         set_launch(k, (uint32_t)nwg, (uint32_t)n_kv, (uint32_t)n_slots, kThreads, lds);
         set_name(k, "sdpa_slots_hd%d_nwg%d", (int)hd, (int)nwg);
         k.variant = (int)nwg;

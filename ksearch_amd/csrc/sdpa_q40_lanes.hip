@@ -32,6 +32,7 @@
 //     through LDS, writes one partial per partition, and the last partition
 //     to arrive (a device-scope counter) folds the partials into the output.
 #include "ksh_device.hpp"
+#include "round_operand.hpp"
 #include "q40_pack.hpp"
 #include "ksh_internal.hpp"
 
@@ -321,9 +322,11 @@ __device__ __forceinline__ Deal deal_wave(const float *meta, int stride, int n_s
 // g, g + 16, ..., so that a slot's whole set of records is requested in one go, while the weights
 // exp(m_i - M) are still being worked out.  grid = (n_q * HD / 64, n_slots), 256 threads.
 // Records of a balanced launch: values [flat][n_q][HD], then (m, l) [flat][n_q][2].
+// xp != nullptr: the result leaves as the prepared operand of a decode round's GEMM (row = slot, n_q * HD columns) instead
+// of f32 rows: a workgroup's 64 dimensions are eight fragment lanes and two sub-blocks of sums of its row.
 template <int HD>
 __global__ __launch_bounds__(256) void sdpa_dealt_merge_kernel(const float *tmp, const float *meta, int meta_stride, int nwg,
-                                                                int n_q, float *out, int round)
+                                                                int n_q, float *out, int round, _Float16 *xp)
 {
     constexpr int kMaxParts = 16 * 64;   // host-checked: nwg * n_slots
     constexpr int QB = 8;                // partitions per thread in flight
@@ -391,7 +394,33 @@ __global__ __launch_bounds__(256) void sdpa_dealt_merge_kernel(const float *tmp,
         float sum = 0.f;
 #pragma unroll
         for (int q = 0; q < 16; q++) sum += part4[q][tid];
-        out[((size_t)slot * n_q + head) * HD + dq * 64 + tid] = sum / L;
+        const float y = sum / L;
+        if (!xp) {
+            out[((size_t)slot * n_q + head) * HD + dq * 64 + tid] = y;
+        } else {
+            // (one wave: its LDS operations complete in order; the fences keep the compiler from moving them)
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            part4[0][tid] = y;
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            const int cols = n_q * HD, c0 = head * HD + dq * 64 + 8 * (tid & 7);
+            float f[8];
+#pragma unroll
+            for (int e = 0; e < 8; e++) f[e] = part4[0][8 * (tid & 7) + e];
+            h8 oh, ol;
+            float sh, sl;
+            round_split8(f, oh, ol, sh, sl);
+            sh += dpp_f32<0xB1>(sh);      // the four lanes of a sub-block
+            sh += dpp_f32<0x4E>(sh);
+            sl += dpp_f32<0xB1>(sl);
+            sl += dpp_f32<0x4E>(sl);
+            if (tid < 8) {
+                const int j = c0 / 8;
+                const size_t frag = (size_t)(j >> 1) * 64 + slot + 32 * (j & 1);
+                reinterpret_cast<h8 *>(xp)[frag] = oh;
+                reinterpret_cast<h8 *>(xp)[frag + 16] = ol;
+                if ((tid & 3) == 0) round_store_sums(xp, cols, slot, c0 / 32, sh, sl);
+            }
+        }
     }
 }
 
@@ -1255,7 +1284,10 @@ int launch_bound(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
         p.out = (float *)a.out[1];
         p.scale = k.desc.params[0];
         p.mode = kModeMerge;
+        if (k.desc.params[1] != 0.f && !(balanced_slots(n_slots, p.nwg) || mfma))
+            return set_error("sdpa_slots: the result as a prepared operand needs the launch whose partitions are dealt by length (2 to 16 slots, 2 to 64 partitions)");
         if (balanced_slots(n_slots, p.nwg) || mfma) {
+            _Float16 *xp = k.desc.params[1] != 0.f ? (_Float16 *)a.out[1] : nullptr;
             p.balance = 1;
             p.mode = kModePart;
             if (mfma) {
@@ -1269,11 +1301,11 @@ int launch_bound(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
                 return 1;
             }
             if (hd == 512)
-                hipLaunchKernelGGL(sdpa_dealt_merge_kernel<512>, dim3(p.n_q * 8, n_slots), dim3(256), 0, st, p.tmp, p.meta, p.meta_stride, p.nwg, p.n_q, p.out, mfma ? kMfmaRound : 1);
+                hipLaunchKernelGGL(sdpa_dealt_merge_kernel<512>, dim3(p.n_q * 8, n_slots), dim3(256), 0, st, p.tmp, p.meta, p.meta_stride, p.nwg, p.n_q, p.out, mfma ? kMfmaRound : 1, xp);
             else if (hd == 256)
-                hipLaunchKernelGGL(sdpa_dealt_merge_kernel<256>, dim3(p.n_q * 4, n_slots), dim3(256), 0, st, p.tmp, p.meta, p.meta_stride, p.nwg, p.n_q, p.out, mfma ? kMfmaRound : 1);
+                hipLaunchKernelGGL(sdpa_dealt_merge_kernel<256>, dim3(p.n_q * 4, n_slots), dim3(256), 0, st, p.tmp, p.meta, p.meta_stride, p.nwg, p.n_q, p.out, mfma ? kMfmaRound : 1, xp);
             else
-                hipLaunchKernelGGL(sdpa_dealt_merge_kernel<128>, dim3(p.n_q * 2, n_slots), dim3(256), 0, st, p.tmp, p.meta, p.meta_stride, p.nwg, p.n_q, p.out, mfma ? kMfmaRound : 1);
+                hipLaunchKernelGGL(sdpa_dealt_merge_kernel<128>, dim3(p.n_q * 2, n_slots), dim3(256), 0, st, p.tmp, p.meta, p.meta_stride, p.nwg, p.n_q, p.out, mfma ? kMfmaRound : 1, xp);
             const hipError_t e = hipGetLastError();
             return e == hipSuccess ? 0 : hip_fail(e, "sdpa merge launch");
         }

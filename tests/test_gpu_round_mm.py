@@ -130,6 +130,31 @@ def test_matvec_round_partial_sums_into_the_closing_norm(ctx):
     assert np.array_equal(ctx.read_bytes(got, n_xp), ctx.read_bytes(want, n_xp))
 
 
+@pytest.mark.parametrize("hd,sched", [(256, None), (256, dict(vec=3)), (512, None)])
+def test_sdpa_slots_result_as_prepared_operand(ctx, hd, sched):
+    """KSH_SDPA_SLOTS with params[1] = 1: the merge writes the prepared operand of the o projection; its values are the
+    f32 rows' of the plain launch to 2^-20."""
+    n_slots, n_q, n_kv, max_t, nwg = 5, 8, 1, 1024, 8
+    lens, kk, vv, q = synth.cfg3_q40_attention(n_slots, n_q, n_kv, hd, max_t, lo=1, seed=990)
+    meta = np.zeros((n_slots, 4), np.float32)
+    meta[:, 0] = lens
+    ins = [ctx.buffer_f32(q), ctx.buffer_bytes(kk.reshape(-1)), ctx.buffer_bytes(vv.reshape(-1)), ctx.buffer_f32(meta)]
+    cols = n_q * hd
+    outs = {}
+    for flag in (0.0, 1.0):
+        k = ctx.compile(hip.make_desc(Kind.SDPA_SLOTS, (n_q, n_kv, hd, max_t, n_slots, nwg), (DType.Q40, DType.F32), (0.0625, flag), sched))
+        tmp = ctx.buffer_empty_f32(n_slots * n_q * k.info.sched.k_split * (hd + 2))
+        out = ctx.buffer_empty_bytes(64 * cols + 2048 * (cols // 256)) if flag else ctx.buffer_empty_f32(n_slots * cols)
+        ctx.encode_multi(k, ins, [tmp, out])
+        outs[flag] = out
+    want = np.zeros((16, cols))
+    want[:n_slots] = ctx.read_f32(outs[0.0], n_slots * cols).reshape(n_slots, cols)
+    vals, sums = xp_values(ctx, outs[1.0], cols)
+    err = np.abs(vals[:n_slots] - want[:n_slots]) / np.maximum(np.abs(want[:n_slots]), 2.0 ** -10 * np.abs(want).max())
+    assert err.max() < 2.0 ** -20, err.max()
+    assert np.allclose(sums[:n_slots], want[:n_slots].reshape(n_slots, -1, 32).sum(axis=2), rtol=0, atol=2e-3 * np.abs(want).max())
+
+
 def test_matvec_round_unit_rows_recover_weights(ctx):
     # X = one-hot rows: Y[t] is column k_t of the dequantized matrix (pins the K order and the hi | lo tile end to end)
     rows, cols = 64, 4096

@@ -53,7 +53,9 @@ static int sdpa_candidates(const ksh_kernel_desc &d, ksh_sched *out, int cap)
                 out[n++] = s;
             }
         // the matrix-core form of the row phase (several slots, heads of 256)
-        if (d.kind == KSH_SDPA_SLOTS && d.dims[2] == 256 && groups <= 8 && d.dims[4] <= 16)
+        const int64_t parts = ks ? ks : nwg_dim;
+        if (d.dims[2] == 256 && groups <= 8 &&
+            ((d.kind == KSH_SDPA_SLOTS && d.dims[4] <= 16) || (d.kind == KSH_SDPA_BATCH && d.dims[4] <= 64 && parts >= 2 && parts * d.dims[4] <= 1024)))
             for (uint32_t tile : {32u, 16u}) {                // rows per wave tile: four waves of 32 or eight of 16
                 if (n >= cap) return n;
                 ksh_sched s{};

@@ -1256,6 +1256,29 @@ int launch_bound(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
     const bool mfma = nw >= 0xFE;          // the matrix-core form of the row phase (bind_sdpa_lanes): 0xFF tiles of 32 rows, 0xFE of 16
     if (mfma) { p.hsplit = 1; p.groups = p.n_q / p.n_kv; }
     int n_slots = 1;
+    // the row phase whose partitions are dealt to the slots by length (register or matrix-core form), then the merge launch
+    auto launch_dealt = [&](_Float16 *xp) -> int {
+        p.balance = 1;
+        p.mode = kModePart;
+        if (mfma) {
+            if (nw == 0xFF)
+                hipLaunchKernelGGL((sdpa_mfma_kernel<256, 32>), dim3(p.nwg, p.n_kv, n_slots), dim3(kMfmaRound / 32 * 64), (mfma_lds_bytes<256, 32>()), st, p);
+            else
+                hipLaunchKernelGGL((sdpa_mfma_kernel<256, 16>), dim3(p.nwg, p.n_kv, n_slots), dim3(kMfmaRound / 16 * 64), (mfma_lds_bytes<256, 16>()), st, p);
+            const hipError_t e0 = hipGetLastError();
+            if (e0 != hipSuccess) return hip_fail(e0, "sdpa (matrix-core form) launch");
+        } else if (launch_lanes(p, hd, nw, n_slots, st)) {
+            return 1;
+        }
+        if (hd == 512)
+            hipLaunchKernelGGL(sdpa_dealt_merge_kernel<512>, dim3(p.n_q * 8, n_slots), dim3(256), 0, st, p.tmp, p.meta, p.meta_stride, p.nwg, p.n_q, p.out, mfma ? kMfmaRound : 1, xp);
+        else if (hd == 256)
+            hipLaunchKernelGGL(sdpa_dealt_merge_kernel<256>, dim3(p.n_q * 4, n_slots), dim3(256), 0, st, p.tmp, p.meta, p.meta_stride, p.nwg, p.n_q, p.out, mfma ? kMfmaRound : 1, xp);
+        else
+            hipLaunchKernelGGL(sdpa_dealt_merge_kernel<128>, dim3(p.n_q * 2, n_slots), dim3(256), 0, st, p.tmp, p.meta, p.meta_stride, p.nwg, p.n_q, p.out, mfma ? kMfmaRound : 1, xp);
+        const hipError_t e = hipGetLastError();
+        return e == hipSuccess ? 0 : hip_fail(e, "sdpa merge launch");
+    };
     switch (k.desc.kind) {
     case KSH_SDPA_NAIVE:
         p.q = (const float *)a.in[0]; p.k = (const uint8_t *)a.in[1]; p.v = (const uint8_t *)a.in[2];
@@ -1286,29 +1309,7 @@ int launch_bound(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
         p.mode = kModeMerge;
         if (k.desc.params[1] != 0.f && !(balanced_slots(n_slots, p.nwg) || mfma))
             return set_error("sdpa_slots: the result as a prepared operand needs the launch whose partitions are dealt by length (2 to 16 slots, 2 to 64 partitions)");
-        if (balanced_slots(n_slots, p.nwg) || mfma) {
-            _Float16 *xp = k.desc.params[1] != 0.f ? (_Float16 *)a.out[1] : nullptr;
-            p.balance = 1;
-            p.mode = kModePart;
-            if (mfma) {
-                if (nw == 0xFF)
-                    hipLaunchKernelGGL((sdpa_mfma_kernel<256, 32>), dim3(p.nwg, p.n_kv, n_slots), dim3(kMfmaRound / 32 * 64), (mfma_lds_bytes<256, 32>()), st, p);
-                else
-                    hipLaunchKernelGGL((sdpa_mfma_kernel<256, 16>), dim3(p.nwg, p.n_kv, n_slots), dim3(kMfmaRound / 16 * 64), (mfma_lds_bytes<256, 16>()), st, p);
-                const hipError_t e0 = hipGetLastError();
-                if (e0 != hipSuccess) return hip_fail(e0, "sdpa (matrix-core form) launch");
-            } else if (launch_lanes(p, hd, nw, n_slots, st)) {
-                return 1;
-            }
-            if (hd == 512)
-                hipLaunchKernelGGL(sdpa_dealt_merge_kernel<512>, dim3(p.n_q * 8, n_slots), dim3(256), 0, st, p.tmp, p.meta, p.meta_stride, p.nwg, p.n_q, p.out, mfma ? kMfmaRound : 1, xp);
-            else if (hd == 256)
-                hipLaunchKernelGGL(sdpa_dealt_merge_kernel<256>, dim3(p.n_q * 4, n_slots), dim3(256), 0, st, p.tmp, p.meta, p.meta_stride, p.nwg, p.n_q, p.out, mfma ? kMfmaRound : 1, xp);
-            else
-                hipLaunchKernelGGL(sdpa_dealt_merge_kernel<128>, dim3(p.n_q * 2, n_slots), dim3(256), 0, st, p.tmp, p.meta, p.meta_stride, p.nwg, p.n_q, p.out, mfma ? kMfmaRound : 1, xp);
-            const hipError_t e = hipGetLastError();
-            return e == hipSuccess ? 0 : hip_fail(e, "sdpa merge launch");
-        }
+        if (balanced_slots(n_slots, p.nwg) || mfma) return launch_dealt(k.desc.params[1] != 0.f ? (_Float16 *)a.out[1] : nullptr);
         break;
     case KSH_SDPA_BATCH: {
         // in: q, K, V, meta{tlen of token 0, -, window}   out: tmp, o.  The per-token records are written by a small
@@ -1324,6 +1325,7 @@ int launch_bound(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
         p.scale = k.desc.params[0];
         p.mode = kModeMerge;
         p.kv_shared = 1;
+        if (mfma) return launch_dealt(nullptr);    // every token a slot of its own over the shared cache
         break;
     }
     case KSH_ATTEND_DECODE: {
@@ -1380,18 +1382,23 @@ int bind_sdpa_lanes(ksh_kernel &k, int nwg, int n_slots)
     // heads of 256 and up to 8 q heads per kv head, merged by a second launch
     // It is the default wherever it fits (from one slot of a few thousand rows to sixteen long ones it takes 0.5 to
     // 1.0 of the vector form's time); vec = 3 asks for the vector form by name.
-    const bool mfma_fits = k.desc.kind == KSH_SDPA_SLOTS && hd == 256 && n_q / n_kv <= 8 && n_slots <= 16 && nwg >= 2 && nwg <= 64;
-    if (k.desc.sched.vec == 2 || (k.desc.sched.vec == 0 && mfma_fits)) {
+    // (a chunk of up to 64 prompt tokens over one cache is 64 slots that share it: a schedule of KSH_SDPA_BATCH, not its
+    // default -- timed alone it takes 0.65 to 0.8 of the register form's time, inside a prompt chunk's pass its second
+    // launch costs more than that saves at 63 tokens)
+    const bool batch_fits = k.desc.kind == KSH_SDPA_BATCH && hd == 256 && n_q / n_kv <= 8 && n_slots <= 64 && nwg >= 2 && nwg * n_slots <= 1024;
+    const bool mfma_fits = (k.desc.kind == KSH_SDPA_SLOTS && hd == 256 && n_q / n_kv <= 8 && n_slots <= 16 && nwg >= 2 && nwg <= 64) || batch_fits;
+    if (k.desc.sched.vec == 2 || (k.desc.sched.vec == 0 && mfma_fits && !batch_fits)) {
         if (!mfma_fits)
-            return set_error("sdpa: the matrix-core form (vec=2) takes KSH_SDPA_SLOTS with hd 256, up to 8 q heads per kv head, "
-                             "up to 16 slots and 2..64 partitions");
+            return set_error("sdpa: the matrix-core form (vec=2) takes hd 256 and up to 8 q heads per kv head: KSH_SDPA_SLOTS with up to 16 slots "
+                             "and 2..64 partitions, KSH_SDPA_BATCH with up to 64 tokens and 2 .. 1024 / tokens partitions");
         // sched.lds_tile: rows per wave tile, 32 (four waves) or 16 (eight waves).  0 takes 16 where the grid is at
         // most one workgroup per compute unit (eight-wave workgroups do not share one, so a larger grid would run in
         // two turns; within one turn the shorter chain per wave is worth about a microsecond)
         const int tile = k.desc.sched.lds_tile ? (int)k.desc.sched.lds_tile : (int64_t)nwg * n_kv * n_slots <= 256 ? 16 : 32;
         if (tile != 16 && tile != 32) return set_error("sdpa: the matrix-core form takes tiles of 16 or 32 rows (lds_tile=%d)", tile);
         const int waves = kMfmaRound / tile;
-        k.scratch_bytes = 16;
+        // (the batch kind keeps its per-token records in the scratch, behind room for the register form's counters)
+        k.scratch_bytes = batch_fits ? (((size_t)n_slots * n_kv * 4 + 15) & ~(size_t)15) + (size_t)n_slots * 16 : 16;
         set_launch(k, (uint32_t)nwg, (uint32_t)n_kv, (uint32_t)n_slots, waves * 64,
                    (uint32_t)(tile == 32 ? mfma_lds_bytes<256, 32>() : mfma_lds_bytes<256, 16>()));
         k.info.sched = k.desc.sched;

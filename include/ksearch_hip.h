@@ -394,7 +394,7 @@ int ksh_gemma_reset(ksh_gemma *m);
  * replays a captured HIP graph.  next_id may be NULL (no host read-back). */
 int ksh_gemma_forward_token(ksh_gemma *m, uint32_t token, int use_graph, uint32_t *next_id);
 /* prefill_chunk (crates/ksearch_gemma/src/gemma_prim.rs:1305-1607): n tokens at the model's current position, no
- * logits; chunks of up to 256 tokens run as one batched pass per layer (row norms, MFMA GEMMs over f32 activations,
+ * logits; chunks of up to 1024 tokens run as one batched pass per layer (row norms, MFMA GEMMs over f32 activations,
  * batched per-head norm + RoPE + Q4_0 append, causal attention over the cache), a single token as a decode step. */
 int ksh_gemma_prefill_chunk(ksh_gemma *m, const uint32_t *tokens, int n);
 /* generate_timed (:1658-1768): all prompt tokens but the last through prefill_chunk (use_graph & 2: token by token
@@ -508,7 +508,7 @@ int ksh_sample_softcap_min_p(const float *logits, size_t n, float cap, float tem
 int ksh_gemma4_decode_token_sampled(ksh_gemma4 *m, uint32_t token, float temperature, float min_p, uint32_t seed,
                                     int use_graph, uint32_t *next_id);
 /* GemmaPrimModel::prefill_chunk (gemma_prim.rs:1305-1607): n tokens without logits, then one synchronisation.
- * Chunks of up to 256 tokens run as one batched pass per layer (forward_prefill_chunk), a chunk of one token as a
+ * Chunks of up to 1024 tokens run as one batched pass per layer (forward_prefill_chunk), a chunk of one token as a
  * decode step.  use_graph & 1: decode steps replay the captured graph; use_graph & 2: every token goes through the
  * decode step (no batching).  ksh_gemma4_generate / _generate_until feed the prompt through this with the same flags. */
 int ksh_gemma4_prefill_chunk(ksh_gemma4 *m, const uint32_t *tokens, int n, int use_graph);

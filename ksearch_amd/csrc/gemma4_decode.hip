@@ -365,7 +365,7 @@ int write_token(ksh_gemma4 *m, uint32_t token)
 
 // gemma_prim.rs:33-56: per position cos[0..hd/2) || sin[0..hd/2); pairs past `angles` are the identity
 // prefill_chunk's chunk length (gemma_prim.rs:16)
-constexpr int kChunk4 = 256;
+constexpr int kChunk4 = 1024;
 constexpr int kChunkPartitions4 = 8;
 
 int chunk_buffers4(ksh_gemma4 *m)

@@ -377,7 +377,7 @@ int run_token(ksh_gemma *m, bool want_logits, bool use_graph)
 }
 
 // prefill_chunk's chunk length (gemma_prim.rs:16)
-constexpr int kChunk = 256;
+constexpr int kChunk = 1024;
 constexpr int kChunkPartitions = 8;   // partitions per token of the batched attention (its tmp buffer is sized for this)
 
 int chunk_buffers(ksh_gemma *m)

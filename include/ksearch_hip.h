@@ -205,7 +205,8 @@ enum ksh_kind {
     /* sdpa_hybrid_kv_batch (crates/ksearch_kernels/src/lib.rs:1592-1623, lower.rs:4961-4983): causal attention of
      * n_tok consecutive prompt tokens over one Q4_0 cache that already holds their rows.  meta = f32{tlen of token
      * 0, -, window}: token i attends tlen_i = min(tlen0 + i, window) rows from start_i = tlen0 + i - tlen_i.
-     * dims: n_q, n_kv, hd, max_t, n_tok, nwg (0 = default; sched.k_split sets it too).
+     * dims: n_q, n_kv, hd, max_t, n_tok, nwg (0 = default; sched.k_split sets it too).  Heads of 256 in chunks of
+     * more than 16 tokens run on the matrix cores and are fastest with one partition per token (nwg = 1).
      * in: q[n_tok, n_q*hd], K, V, meta   out: tmp f32[n_tok*n_q*nwg*(hd+2)], o[n_tok, n_q*hd] */
     KSH_SDPA_BATCH = 29,
     /* The activations of a decode round (up to 16 rows, one per decoding sequence), prepared once for every GEMM
@@ -241,8 +242,10 @@ typedef struct {
     uint64_t tg;       /* threads per workgroup (64 * waves) */
     uint32_t vec;      /* inner-product variant.  GEMV: 1 = byte converts + f32 FMA, 3 = int8 dot over 3 digit planes.
                         * Attention: 1 = LDS-tile form, 3 = register (vector-ALU) form, 2 = matrix-core form of the
-                        * row phase (KSH_SDPA_SLOTS, heads of 256, up to 8 q heads per kv head, up to 16 slots: the
-                        * default there; lds_tile = 32 | 16 picks four waves with tiles of 32 rows or eight with 16) */
+                        * row phase (heads of 256, up to 8 q heads per kv head.  KSH_SDPA_SLOTS with up to 16 slots:
+                        * the default there; lds_tile = 32 | 16 picks four waves with tiles of 32 rows or eight with
+                        * 16.  KSH_SDPA_BATCH: the default from 17 tokens on, every token's partitions workgroups of
+                        * their own; vec = 2 with up to 64 tokens deals the partitions to the tokens by length) */
     uint32_t unroll;   /* superblocks in flight per lane */
     uint32_t nsg;      /* waves per workgroup */
     uint32_t nr0;      /* rows per wave */

@@ -412,7 +412,8 @@ int forward_prefill_chunk(ksh_gemma *m, const uint32_t *tokens, int t)
         get(m, KSH_MATVEC_BATCH, {qd, c.hidden, tp}, {KSH_Q4K, KSH_F32, KSH_F32}, {}, &k_mm_q) ||
         get(m, KSH_MATVEC_BATCH, {kvd, c.hidden, tp}, {KSH_Q4K, KSH_F32, KSH_F32}, {}, &k_mm_kv) ||
         get(m, KSH_RMSNORM_PER_HEAD_QKV_Q40, {c.n_q, c.n_kv, c.hd, c.max_seq, t}, {}, {c.eps}, &k_head) ||
-        get(m, KSH_SDPA_BATCH, {c.n_q, c.n_kv, c.hd, c.max_seq, t, m->c_nwg}, {KSH_Q40, KSH_F32}, {c.attn_scale}, &k_sdpa) ||
+        // (chunks of more than 16 tokens take the attention's matrix-core form, which wants one partition per token)
+        get(m, KSH_SDPA_BATCH, {c.n_q, c.n_kv, c.hd, c.max_seq, t, t > 16 && c.hd == 256 && c.n_q / c.n_kv <= 8 ? 1 : m->c_nwg}, {KSH_Q40, KSH_F32}, {c.attn_scale}, &k_sdpa) ||
         get(m, KSH_MATVEC_BATCH, {c.hidden, qd, tp}, {KSH_Q4K, KSH_F32, KSH_F32}, {}, &k_mm_o) ||
         get(m, KSH_RMSNORM_ADD_THEN_RMSNORM, {c.hidden, t}, {}, {c.eps}, &k_add_then) ||
         get(m, KSH_MATVEC_BATCH, {c.ffn, c.hidden, tp}, {KSH_Q4K, KSH_F32, KSH_F32}, {}, &k_mm_ff) ||

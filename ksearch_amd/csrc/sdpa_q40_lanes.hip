@@ -1186,6 +1186,25 @@ __global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_m
     }
 }
 
+// Merge of split-KV partials kept as records (m, l, o[HD]) per (token, head, partition) -- the layout and the rule
+// of SdpaMwgReduce (crates/ksearch_codegen/src/lower.rs:5897-6087) -- for the launch that gives every token of a long
+// prompt chunk its own workgroups.  grid = (n_q, n_tok), HD threads.
+template <int HD>
+__global__ __launch_bounds__(HD) void sdpa_records_merge_kernel(const float *__restrict__ tmp, float *__restrict__ out, int n_q, int nwg)
+{
+    const int h = blockIdx.x, tok = blockIdx.y, d = threadIdx.x;
+    const float *rec = tmp + ((size_t)tok * n_q + h) * nwg * (HD + 2);
+    float M = -1.0e30f;
+    for (int q = 0; q < nwg; q++) M = fmaxf(M, rec[(size_t)q * (HD + 2)]);
+    float L = 0.f, a = 0.f;
+    for (int q = 0; q < nwg; q++) {
+        const float w = __expf(rec[(size_t)q * (HD + 2)] - M);
+        L = fmaf(w, rec[(size_t)q * (HD + 2) + 1], L);
+        a = fmaf(w, rec[(size_t)q * (HD + 2) + 2 + d], a);
+    }
+    out[((size_t)tok * n_q + h) * HD + d] = a / L;
+}
+
 template <int HD, int TR>
 constexpr size_t mfma_lds_bytes()
 {
@@ -1253,7 +1272,9 @@ int launch_bound(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
     LaneParams p = base_params(k);
     const int hd = (int)k.desc.dims[2], nw = (k.variant >> 16) & 0xFF;
     p.nwg = k.variant & 0xFFFF;
-    const bool mfma = nw >= 0xFE;          // the matrix-core form of the row phase (bind_sdpa_lanes): 0xFF tiles of 32 rows, 0xFE of 16
+    // the matrix-core form of the row phase (bind_sdpa_lanes): 0xFF tiles of 32 rows, 0xFE of 16; 0xFD: tiles of 32
+    // rows with every slot's partitions its own workgroups (a long prompt chunk: more tokens than the deal takes)
+    const bool mfma = nw >= 0xFD, own_parts = nw == 0xFD;
     if (mfma) { p.hsplit = 1; p.groups = p.n_q / p.n_kv; }
     int n_slots = 1;
     // the row phase whose partitions are dealt to the slots by length (register or matrix-core form), then the merge launch
@@ -1325,6 +1346,16 @@ int launch_bound(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
         p.scale = k.desc.params[0];
         p.mode = kModeMerge;
         p.kv_shared = 1;
+        if (own_parts) {
+            p.balance = 0;
+            p.mode = kModePart;
+            hipLaunchKernelGGL((sdpa_mfma_kernel<256, 32>), dim3(p.nwg, p.n_kv, n_slots), dim3(kMfmaRound / 32 * 64), (mfma_lds_bytes<256, 32>()), st, p);
+            const hipError_t e0 = hipGetLastError();
+            if (e0 != hipSuccess) return hip_fail(e0, "sdpa_batch (matrix-core form) launch");
+            hipLaunchKernelGGL(sdpa_records_merge_kernel<256>, dim3(p.n_q, n_slots), dim3(256), 0, st, p.tmp, p.out, p.n_q, p.nwg);
+            const hipError_t e1 = hipGetLastError();
+            return e1 == hipSuccess ? 0 : hip_fail(e1, "sdpa_batch merge launch");
+        }
         if (mfma) return launch_dealt(nullptr);    // every token a slot of its own over the shared cache
         break;
     }
@@ -1387,6 +1418,27 @@ int bind_sdpa_lanes(ksh_kernel &k, int nwg, int n_slots)
     // launch costs more than that saves at 63 tokens)
     const bool batch_fits = k.desc.kind == KSH_SDPA_BATCH && hd == 256 && n_q / n_kv <= 8 && n_slots <= 64 && nwg >= 2 && nwg * n_slots <= 1024;
     const bool mfma_fits = (k.desc.kind == KSH_SDPA_SLOTS && hd == 256 && n_q / n_kv <= 8 && n_slots <= 16 && nwg >= 2 && nwg <= 64) || batch_fits;
+    // A chunk of more than 16 tokens: every token's partitions are workgroups of their own (grid = partitions x kv
+    // heads x tokens), records in the reference's layout, merged by a second launch.  Its tokens attend dozens to
+    // thousands of rows each, where the register form's ~200 vector instructions per row and wave are the whole
+    // cost (1024 tokens from an empty cache: 78 us against 422): the default there; vec = 3 asks for the register
+    // form, vec = 2 with up to 64 tokens for the form that deals the partitions by length.
+    const bool long_batch = k.desc.kind == KSH_SDPA_BATCH && hd == 256 && n_q / n_kv <= 8 && n_slots > 16;
+    if (long_batch && ((k.desc.sched.vec == 2 && !batch_fits) || k.desc.sched.vec == 0)) {
+        if (k.desc.sched.lds_tile && k.desc.sched.lds_tile != 32) return set_error("sdpa_batch: the matrix-core form of a long chunk takes tiles of 32 rows (lds_tile=%u)", k.desc.sched.lds_tile);
+        k.scratch_bytes = (((size_t)n_slots * n_kv * 4 + 15) & ~(size_t)15) + (size_t)n_slots * 16;
+        set_launch(k, (uint32_t)nwg, (uint32_t)n_kv, (uint32_t)n_slots, kMfmaRound / 32 * 64, (uint32_t)mfma_lds_bytes<256, 32>());
+        k.info.sched = k.desc.sched;
+        k.info.sched.vec = 2;
+        k.info.sched.tg = kMfmaRound / 32 * 64;
+        k.info.sched.nsg = kMfmaRound / 32;
+        k.info.sched.k_split = (uint32_t)nwg;
+        k.info.sched.lds_tile = 32;
+        k.info.sched.unroll = 1;
+        k.variant = nwg | (0xFD << 16) | (1 << 24);
+        k.launch = launch_bound;
+        return 0;
+    }
     if (k.desc.sched.vec == 2 || (k.desc.sched.vec == 0 && mfma_fits && !batch_fits)) {
         if (!mfma_fits)
             return set_error("sdpa: the matrix-core form (vec=2) takes hd 256 and up to 8 q heads per kv head: KSH_SDPA_SLOTS with up to 16 slots "

@@ -144,6 +144,12 @@ struct MmParams {
     float *Y;
     int rows, cols, batch;
     float accum;                // 0: store; else add `accum` times the result to Y (the second pass of f32 activations)
+    // Small grids (few tokens x few weight rows): blockIdx.z = part * ksplit + slice.  A workgroup then takes the
+    // superblocks of its K slice only, part 1 reads the low parts of f32 activations, and every z stores its own
+    // batch x rows partial sums behind Y_parts for the fold (ksplit = 0: one launch per part, full K, results in Y).
+    int ksplit;
+    const _Float16 *Xf_lo, *SxA_lo;
+    float *Y_parts;
 };
 
 __device__ __forceinline__ uint32_t pair_f16(uint32_t masked, uint32_t sc)
@@ -192,7 +198,16 @@ __global__ __launch_bounds__(kThreadsMM) void q_mul_mm_kernel(MmParams p)
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int t0 = blockIdx.x * BM, r0 = blockIdx.y * BN;
-    const int nsb = p.cols / 256, nsteps = nsb * 4;
+    const int nsb_row = p.cols / 256;                            // superblocks per weight row
+    int nsb = nsb_row, sb0 = 0;                                  // this workgroup's share of them
+    if (p.ksplit) {
+        const int part = blockIdx.z / p.ksplit, slice = blockIdx.z % p.ksplit;
+        nsb = nsb_row / p.ksplit;
+        sb0 = slice * nsb;
+        if (part) { p.Xf = p.Xf_lo; p.SxA = p.SxA_lo; }
+        p.Y = p.Y_parts + (size_t)blockIdx.z * p.batch * p.rows;
+    }
+    const int nsteps = nsb * 4;
 
     if (Q6 && wave >= 4) {
         // ------------------------------------------------------------------ loaders, Q6_K
@@ -200,8 +215,8 @@ __global__ __launch_bounds__(kThreadsMM) void q_mul_mm_kernel(MmParams p)
         // of a superblock = ql bytes 64h + 32lh .. +31 (nibble `part`), qh bytes 32h .. +31 (bit pair
         // 4*part + 2*lh), scales 8h + 4*part + 2*lh and the next one.  Blocks are 2-byte aligned.
         const int lt = tid - 256, lrow = lt >> 1, lh = lt & 1;
-        const size_t row_bytes = (size_t)nsb * 210;
-        const uint8_t *wrow = p.W + (size_t)min(r0 + lrow, p.rows - 1) * row_bytes;
+        const size_t row_bytes = (size_t)nsb_row * 210;
+        const uint8_t *wrow = p.W + (size_t)min(r0 + lrow, p.rows - 1) * row_bytes + (size_t)sb0 * 210;
         struct Sb6Regs {
             u32x2_t ql[8];    // [4h + i]: ql bytes 64h + 32lh + 8i .. +7
             u32x2_t qh[8];    // all 64 qh bytes
@@ -280,9 +295,9 @@ __global__ __launch_bounds__(kThreadsMM) void q_mul_mm_kernel(MmParams p)
     if (!Q6 && wave >= 4) {
         // ------------------------------------------------------------------ loaders
         const int lt = tid - 256, lrow = lt >> 1, lh = lt & 1;   // two threads per tile row
-        const size_t row_bytes = (size_t)nsb * 144;
-        const uint8_t *wrow = p.W + (size_t)min(r0 + lrow, p.rows - 1) * row_bytes;
-        const _Float16 *sxrow = p.SxA + (size_t)min(t0 + lrow, p.batch - 1) * nsb * 32;
+        const size_t row_bytes = (size_t)nsb_row * 144;
+        const uint8_t *wrow = p.W + (size_t)min(r0 + lrow, p.rows - 1) * row_bytes + (size_t)sb0 * 144;
+        const _Float16 *sxrow = p.SxA + ((size_t)min(t0 + lrow, p.batch - 1) * nsb_row + sb0) * 32;
 
         auto fetch_sb = [&](int sb, SbRegs &r) __attribute__((always_inline)) {
             const u32x4_t *w = reinterpret_cast<const u32x4_t *>(wrow + (size_t)sb * 144);
@@ -395,7 +410,7 @@ __global__ __launch_bounds__(kThreadsMM) void q_mul_mm_kernel(MmParams p)
     const h8 *xa[2];
 #pragma unroll
     for (int mt = 0; mt < 2; mt++)
-        xa[mt] = reinterpret_cast<const h8 *>(p.Xf) + (size_t)min((t0 + wm * 64 + mt * 32) / 32, ntt - 1) * (p.cols / 16) * 64 + lane;
+        xa[mt] = reinterpret_cast<const h8 *>(p.Xf) + ((size_t)min((t0 + wm * 64 + mt * 32) / 32, ntt - 1) * (p.cols / 16) + (size_t)sb0 * 16) * 64 + lane;
     struct ARegs { h8 a[2][KS / 16]; };
     auto fetch_a = [&](int step, ARegs &r) __attribute__((always_inline)) {
 #pragma unroll
@@ -958,6 +973,22 @@ __global__ __launch_bounds__(256) void mm_round_fold_kernel(const float *__restr
     y[i] = s;
 }
 
+// y[i] = the K slices' partial sums of element i, slice after slice; the slices of the low parts of f32 activations
+// (parts = 2) come in scaled
+__global__ __launch_bounds__(256) void mm_parts_fold_kernel(const float *__restrict__ part, float *__restrict__ y, int n, int slices, int parts, float lo_scale)
+{
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    float s = part[i];
+    for (int k = 1; k < slices; k++) s += part[(size_t)k * n + i];
+    if (parts == 2) {
+        float l = part[(size_t)slices * n + i];
+        for (int k = 1; k < slices; k++) l += part[(size_t)(slices + k) * n + i];
+        s = fmaf(lo_scale, l, s);
+    }
+    y[i] = s;
+}
+
 // The same round against a Q6_K matrix with row-grouped fields (KSH_Q6K_ROWS: the LM head as the decode loops keep it;
 // rows of up to 2048 columns).  The B operand is the 6-bit code minus 32 as an exact f16 integer (the code OR-ed into
 // the mantissa of 1024.0, minus 1056 with one packed subtraction per two weights); Q6_K has one int8 scale per 16
@@ -1172,6 +1203,23 @@ int launch_mul_mm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
         return e2 == hipSuccess ? 0 : hip_fail(e2, "mul_mm (small batch) launch");
     }
     const dim3 grid((batch + BM - 1) / BM, (rows + BN - 1) / BN);
+    p.ksplit = 0; p.Xf_lo = Xf_lo; p.SxA_lo = SxA_lo; p.Y_parts = nullptr;
+    if (k.variant >= 2) {
+        // few tiles: K slices and both parts of f32 activations as blockIdx.z of one launch, then the fold
+        const int ks = k.variant >> 1, parts = f32x ? 2 : 1;
+        p.Xf = Xf; p.SxA = SxA; p.accum = 0.f;
+        p.ksplit = ks;
+        p.Y_parts = (float *)((f32x ? SxA_lo : SxA) + sx_halves);     // behind the prepared activations
+        const dim3 gz(grid.x, grid.y, ks * parts);
+        if (k.desc.dtypes[0] == KSH_Q6K) hipLaunchKernelGGL(q_mul_mm_kernel<true>, gz, dim3(kThreadsMM), kLdsBytes, st, p);
+        else hipLaunchKernelGGL(q_mul_mm_kernel<false>, gz, dim3(kThreadsMM), kLdsBytes, st, p);
+        hipError_t e3 = hipGetLastError();
+        if (e3 != hipSuccess) return hip_fail(e3, "mul_mm (K slices) launch");
+        const int n2 = batch * rows;
+        hipLaunchKernelGGL(mm_parts_fold_kernel, dim3((n2 + 255) / 256), dim3(256), 0, st, (const float *)p.Y_parts, (float *)a.out[0], n2, ks, parts, 1.0f / 2048.0f);
+        e3 = hipGetLastError();
+        return e3 == hipSuccess ? 0 : hip_fail(e3, "mul_mm fold launch");
+    }
     for (int pass = 0; pass < (f32x ? 2 : 1); pass++) {
         p.Xf = pass ? Xf_lo : Xf;
         p.SxA = pass ? SxA_lo : SxA;
@@ -1216,10 +1264,25 @@ int bind_matvec_batch(ksh_kernel &k)
         k.launch = launch_mul_mm;
         return 0;
     }
-    set_launch(k, (uint32_t)((batch + BM - 1) / BM), (uint32_t)((rows + BN - 1) / BN), 1, kThreadsMM,
+    // Few tiles (a prompt of a few hundred tokens, or a narrow matrix): the superblocks of a row are split into K
+    // slices and, for f32 activations, the hi and the lo part become workgroups of the same launch, until the grid is
+    // about one workgroup per compute unit; every slice stores its partial sums and a second launch adds them in a
+    // fixed order.  sched.k_split names the slice count (a divisor of cols / 256; 1 = none).
+    const int64_t tiles = ((batch + BM - 1) / BM) * ((rows + BN - 1) / BN), nsb = cols / 256, parts = f32x ? 2 : 1;
+    int64_t ks = 1;
+    if (k.desc.sched.k_split) {
+        ks = k.desc.sched.k_split;
+        if (nsb % ks) return set_error("matvec_batch: k_split=%lld does not divide the %lld superblocks of a row", (long long)ks, (long long)nsb);
+    } else {
+        while (tiles * parts * ks < 256 && nsb % (ks * 2) == 0) ks *= 2;
+    }
+    const bool z_form = ks > 1 || (parts == 2 && tiles < 128 && !k.desc.sched.k_split);
+    k.variant = z_form ? (int)(ks << 1) : 0;
+    if (z_form) k.scratch_bytes += (size_t)parts * ks * batch * rows * 4;
+    set_launch(k, (uint32_t)((batch + BM - 1) / BM), (uint32_t)((rows + BN - 1) / BN), z_form ? (uint32_t)(ks * parts) : 1, kThreadsMM,
                (uint32_t)kLdsBytes);
-    k.info.sched.tg = kThreadsMM; k.info.sched.nsg = kThreadsMM / 64; k.info.sched.nr0 = BN; k.info.sched.k_split = 1; k.info.sched.lds_tile = KS;
-    set_name(k, "mul_mm_%s_%dx%dx%d%s", q6 ? "q6k" : "q4k", BM, BN, KS, f32x ? "_f32x" : "");
+    k.info.sched.tg = kThreadsMM; k.info.sched.nsg = kThreadsMM / 64; k.info.sched.nr0 = BN; k.info.sched.k_split = (uint32_t)ks; k.info.sched.lds_tile = KS;
+    set_name(k, "mul_mm_%s_%dx%dx%d%s%s", q6 ? "q6k" : "q4k", BM, BN, KS, f32x ? "_f32x" : "", z_form ? "_kz" : "");
     k.launch = launch_mul_mm;
     return 0;
 }
@@ -1326,6 +1389,14 @@ int mul_mm_candidates(const ksh_kernel_desc &d, ksh_sched *out, int cap)
     if (n < cap && d.dtypes[0] == KSH_Q4K && d.dims[2] <= kSkinnyMaxBatch) {
         ksh_sched s{};
         s.tg = 512; s.nsg = 8; s.nr0 = 32; s.lds_tile = 16; s.unroll = 1; s.vec = 0; s.k_split = 8;
+        out[n++] = s;
+    }
+    // the 128 x 128 tile over K slices, where whole rows leave the grid short of one workgroup per compute unit
+    const int64_t tiles = ((d.dims[2] + BM - 1) / BM) * ((d.dims[0] + BN - 1) / BN) * (d.dtypes[1] == KSH_F32 ? 2 : 1), nsb = d.dims[1] / 256;
+    for (uint32_t ks : {2u, 4u, 8u, 16u}) {
+        if (n >= cap || nsb % ks || tiles * (ks / 2) >= 256) continue;
+        ksh_sched s{};
+        s.tg = kThreadsMM; s.nsg = kThreadsMM / 64; s.nr0 = BN; s.lds_tile = KS; s.unroll = 1; s.vec = 0; s.k_split = ks;
         out[n++] = s;
     }
     return n;

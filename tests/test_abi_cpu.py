@@ -113,3 +113,9 @@ def test_plan_kinds_and_candidates():
     assert len({tuple(s.as_dict().items()) for s in c}) == len(c)
     assert all(s.tg == 64 * s.nsg for s in c)
     assert hip.beam_candidates(hip.make_desc(hip.Kind.RMSNORM, (2048,))) == []
+    # the prefill GEMM: whole rows, the small-batch form up to 64 tokens, K slices where the tiles are few
+    mm = lambda batch, rows, cols, xdt: [(s.nr0, s.k_split) for s in hip.beam_candidates(
+        hip.make_desc(hip.Kind.MATVEC_BATCH, (rows, cols, batch), (hip.DType.Q4K, xdt, hip.DType.F32)))]
+    assert mm(512, 8192, 2048, hip.DType.BF16) == [(128, 1)]
+    assert mm(256, 2048, 2048, hip.DType.F32) == [(128, 1), (128, 2), (128, 4)]
+    assert mm(40, 2048, 1536, hip.DType.F32) == [(128, 1), (32, 8), (128, 2)]

@@ -7,7 +7,7 @@ import pytest
 import oracle
 from ksearch_amd import hip, synth
 from ksearch_amd.hip import DType
-from tests.gpu_util import assert_close
+from tests.gpu_util import assert_close, rel_err
 from tests.test_oracle_ops import check_mul_mm_inputs
 
 pytestmark = pytest.mark.gpu
@@ -132,8 +132,57 @@ def test_mul_mm_q6k_cfg2_shape(ctx, eng):
     xf, xb = xf.reshape(tokens, cols), xb.reshape(tokens, cols)
     got, want = run(ctx, eng, w, rows, cols, xf, xb, tokens, q6=True)
     assert_close(got, want, 1e-3, "q6k 512x8192x2048")
-    got2, _ = run(ctx, eng, w, rows, cols, 2 * xf[:128], synth.bf16_round((2 * xf[:128]).reshape(-1))[1].reshape(128, cols), 128, q6=True)
-    assert np.array_equal(got2, 2 * got[:128])
+    # linearity: twice the activations, twice the result, bit for bit.  128 tokens alone are 64 tiles, which the
+    # library splits into K slices (another summation order: equal to f32 rounding); with the split switched off
+    # (k_split = 1) the 128-token launch adds in the 512-token launch's order.
+    xb2 = synth.bf16_round((2 * xf[:128]).reshape(-1))[1].reshape(128, cols)
+    got2, _ = run(ctx, eng, w, rows, cols, 2 * xf[:128], xb2, 128, q6=True)
+    assert_close(got2, 2 * got[:128], 2e-6, "K slices against the whole row")
+    k1 = ctx.compile(hip.make_desc(hip.Kind.MATVEC_BATCH, (rows, cols, 128), (DType.Q6K, DType.BF16, DType.F32), (), dict(k_split=1)))
+    assert "_kz" not in k1.name and k1.info.sched.k_split == 1
+    y1 = ctx.buffer_empty_f32(128 * rows)
+    ctx.encode_multi(k1, [ctx.buffer_bytes(w), ctx.buffer_bytes(xb2)], [y1])
+    ctx.synchronize()
+    assert np.array_equal(ctx.read_f32(y1, 128 * rows).reshape(128, rows), 2 * got[:128])
+
+
+@pytest.mark.parametrize("wdt,xdt,batch,rows,cols,ks", [(DType.Q4K, DType.BF16, 200, 300, 1536, None), (DType.Q4K, DType.F32, 130, 256, 2048, 4),
+                                                         (DType.Q6K, DType.F32, 70, 200, 1024, None), (DType.Q4K, DType.F32, 300, 2048, 512, None),
+                                                         (DType.Q4K, DType.BF16, 256, 384, 8192, 8), (DType.Q4K, DType.F32, 65, 128, 256, None)])
+def test_mul_mm_k_slices(ctx, wdt, xdt, batch, rows, cols, ks):
+    """Few tiles: a row's superblocks go to K slices (and the hi and lo parts of f32 activations to workgroups of the
+    same launch), every slice stores its partial sums and a fold adds them in a fixed order.  Against the float64
+    product at the accuracy of the whole-row launch (bf16 activations: 1e-3 against the oracle's f32 loop; f32
+    activations: 2e-5), twice for bit-reproducibility, ragged tiles in both directions."""
+    nb = rows * cols // 256
+    w = synth.q4k_blocks(nb, 650) if wdt == DType.Q4K else synth.q6k_blocks(nb, 650)
+    x = synth.normal_f32(batch * cols, 651).reshape(batch, cols)
+    if xdt == DType.BF16:
+        xf, xb = synth.bf16_round(x.reshape(-1))
+        x, xin = xf.reshape(batch, cols), ctx.buffer_bytes(xb)
+    else:
+        xin = ctx.buffer_f32(x)
+    k = ctx.compile(hip.make_desc(hip.Kind.MATVEC_BATCH, (rows, cols, batch), (wdt, xdt, DType.F32), (), dict(k_split=ks) if ks else None))
+    parts = 2 if xdt == DType.F32 else 1
+    assert "_kz" in k.name and k.grid[2] == k.info.sched.k_split * parts, (k.name, k.info.sched.k_split)
+    assert (cols // 256) % k.info.sched.k_split == 0 and (ks is None or k.info.sched.k_split == ks)
+    by, bw = ctx.buffer_empty_f32(batch * rows), ctx.buffer_bytes(w)
+    runs = []
+    for _ in range(2):
+        ctx.encode_multi(k, [bw, xin], [by])
+        ctx.synchronize()
+        runs.append(ctx.read_f32(by, batch * rows).reshape(batch, rows))
+    assert np.array_equal(runs[0], runs[1])
+    odt = oracle.Q4K if wdt == DType.Q4K else oracle.Q6K
+    worst = 0.0
+    for t in range(0, batch, 7):
+        worst = max(worst, float(rel_err(runs[0][t], oracle.matvec_f64(odt, w, rows, cols, x[t])).max()))
+    assert worst <= 2e-5, worst
+
+
+def test_mul_mm_k_slices_must_divide_the_row(ctx):
+    with pytest.raises(hip.KshError, match="does not divide"):
+        ctx.compile(hip.make_desc(hip.Kind.MATVEC_BATCH, (256, 2048, 100), (DType.Q4K, DType.BF16, DType.F32), (), dict(k_split=3)))
 
 
 def test_mul_mm_cfg2_full_size(ctx, eng):
@@ -142,8 +191,18 @@ def test_mul_mm_cfg2_full_size(ctx, eng):
     got, want = run(ctx, eng, w, rows, cols, xf, xb, tokens)
     assert_close(got, want, 1e-3, "cfg2")
     # linearity in X (size-independent property): W(2x) = 2 W(x) exactly in binary floating point
-    got2, _ = run(ctx, eng, w, rows, cols, 2 * xf[:128], synth.bf16_round((2 * xf[:128]).reshape(-1))[1].reshape(128, cols), 128)
-    assert np.array_equal(got2, 2 * got[:128])
+    # (on the first 128 tokens, none of whose values is small enough to lose bits as an f16 subnormal.  128 tokens alone
+    # are 64 tiles, which the library would split into K slices -- the same sums in another order -- so the exact
+    # check asks for whole rows, k_split = 1, and the default launch is held to f32 rounding.)
+    xb2 = synth.bf16_round((2 * xf[:128]).reshape(-1))[1].reshape(128, cols)
+    k1 = ctx.compile(hip.make_desc(hip.Kind.MATVEC_BATCH, (rows, cols, 128), (DType.Q4K, DType.BF16, DType.F32), (), dict(k_split=1)))
+    assert "_kz" not in k1.name
+    y1 = ctx.buffer_empty_f32(128 * rows)
+    ctx.encode_multi(k1, [ctx.buffer_bytes(w), ctx.buffer_bytes(xb2)], [y1])
+    ctx.synchronize()
+    assert np.array_equal(ctx.read_f32(y1, 128 * rows).reshape(128, rows), 2 * got[:128])
+    got3, _ = run(ctx, eng, w, rows, cols, xf[:128], xb[:128], 128)
+    assert_close(got3, got[:128], 2e-6, "K slices against the whole row")
 
 
 def test_mul_mm_errors(ctx):

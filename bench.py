@@ -234,10 +234,12 @@ def bench_decode(ctx, eng, use_graph=True):
     per_tok = cfg["n_layers"] * layer + cfg["vocab"] * h // 256 * 210
     # a long prompt: 1024 tokens are one chunk of the batched pass
     long_prompt = [int(t) for t in np.random.default_rng(4002).integers(0, cfg["vocab"], 1025)]
-    long_ms = []
+    long_ms, mid_ms = [], []
     for _ in range(2):
         m.reset()
         long_ms.append(m.generate(long_prompt, 1, use_graph=use_graph)[1])
+        m.reset()
+        mid_ms.append(m.generate(long_prompt[:257], 1, use_graph=use_graph)[1])
     m.reset()
     out = dict(tok_per_s=round(256 / dec_ms * 1e3, 1), ms_per_token=round(dec_ms / 256, 4),
                launches_per_token=m.launches_per_token, weight_gbps=round(per_tok * 256 / (dec_ms * 1e-3) / 1e9, 1),
@@ -245,6 +247,7 @@ def bench_decode(ctx, eng, use_graph=True):
                prompt_tokens=64, new_tokens=256, graph=bool(use_graph),
                prefill_ms=round(pre_ms, 3), prefill_tok_per_s=round(63 / pre_ms * 1e3, 1),
                prefill_ms_token_by_token=round(serial_pre_ms, 3),
+               prefill_256_tokens_ms=round(min(mid_ms), 2), prefill_256_tok_per_s=round(256 / min(mid_ms) * 1e3, 1),
                prefill_1024_tokens_ms=round(min(long_ms), 2), prefill_1024_tok_per_s=round(1024 / min(long_ms) * 1e3, 1))
     m.close()
     return out

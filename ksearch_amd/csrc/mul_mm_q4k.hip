@@ -1276,7 +1276,8 @@ int bind_matvec_batch(ksh_kernel &k)
     } else {
         while (tiles * parts * ks < 256 && nsb % (ks * 2) == 0) ks *= 2;
     }
-    const bool z_form = ks > 1 || (parts == 2 && tiles < 128 && !k.desc.sched.k_split);
+    // (f32 activations with fewer tiles than compute units: both parts in one launch even without a K split)
+    const bool z_form = ks > 1 || (parts == 2 && tiles < 256 && !k.desc.sched.k_split);
     k.variant = z_form ? (int)(ks << 1) : 0;
     if (z_form) k.scratch_bytes += (size_t)parts * ks * batch * rows * 4;
     set_launch(k, (uint32_t)((batch + BM - 1) / BM), (uint32_t)((rows + BN - 1) / BN), z_form ? (uint32_t)(ks * parts) : 1, kThreadsMM,

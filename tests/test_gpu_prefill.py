@@ -194,7 +194,7 @@ def lockstep_prompt(ctx, gpu, cpu, cfg, toks, first_pos=0):
 @pytest.mark.parametrize("n_prompt", [2, 31, 64, 300])
 def test_prefill_chunk_matches_oracle_in_lockstep(ctx, small_model, n_prompt):
     """prefill_chunk(N tokens) leaves the KV rows of N decode steps (up to one-code flips) and the next decode step
-    gives the oracle's logits; 300 tokens take a chunk of 256 and one of 44, and cross the attention's 128-row switch."""
+    gives the oracle's logits; 300 tokens cross the oracle's 128-row switch to split-KV attention."""
     gpu, cpu = small_model
     toks = np.random.default_rng(740 + n_prompt).integers(0, SMALL["vocab"], n_prompt + 3)
     gpu.reset()
@@ -213,6 +213,31 @@ def test_prefill_chunk_matches_oracle_in_lockstep(ctx, small_model, n_prompt):
         top2 = np.sort(c_logits)[-2:]
         if top2[1] - top2[0] > 2e-3 * max(abs(top2[1]), float(np.sqrt(np.mean(c_logits ** 2)))):
             assert g_next == c_next
+
+
+def test_prefill_long_prompt_takes_two_chunks(ctx):
+    """1100 prompt tokens are a chunk of 1024 and one of 76 (heads of 256: both chunks' attention on the matrix cores,
+    the second over the first one's rows; GEMMs over K slices at 1024 and at 76 rows): every K / V row within one code
+    step of the oracle's, which walks the positions one by one, and the decode steps behind the prompt at 1e-3."""
+    cfg = dict(n_layers=2, hidden=512, ffn=1024, n_q=4, n_kv=1, hd=256, vocab=4096, max_seq=1200,
+               eps=1e-6, softcap=30.0, rope_theta=10000.0, attn_scale=1.0 / 16.0)
+    w = synth.gemma_weights(cfg, 760, oracle.quantize_q4k, synth.chunked(oracle.quantize_q6k), std=0.05)
+    gpu, cpu = hip.Gemma(ctx, cfg, w), oracle.Gemma(cfg, w)
+    n_prompt = 1100
+    toks = np.random.default_rng(761).integers(0, cfg["vocab"], n_prompt + 2)
+    gpu.prefill_chunk(toks[:n_prompt])
+    assert gpu.pos == n_prompt
+    lockstep_prompt(ctx, gpu, cpu, cfg, toks[:n_prompt])
+    row = cfg["hd"] // 32 * 18
+    bufs = [[hip.Buffer(ctx, hip.lib().ksh_gemma_kv(gpu.h, l, w_), owned=False) for w_ in (0, 1)] for l in range(cfg["n_layers"])]
+    for i in range(n_prompt, n_prompt + 2):
+        gpu.forward_token(int(toks[i]), use_graph=bool(i & 1))
+        rows = np.stack([np.stack([ctx.read_bytes(bufs[l][w_], row, i * row) for w_ in (0, 1)]) for l in range(cfg["n_layers"])])
+        _, c_logits = cpu.forward(int(toks[i]), return_logits=True, adopt_rows=rows)
+        assert cpu.row_max_step.max() <= 1.0 + 1e-3
+        assert_close(gpu.logits(), c_logits, 1e-3, f"logits at position {i}")
+    gpu.close()
+    cpu.close()
 
 
 def test_prefill_in_two_calls_and_serial_prefill_agree(ctx, small_model):

@@ -253,6 +253,26 @@ def bench_decode(ctx, eng, use_graph=True):
     return out
 
 
+def bench_prompt_pass(ctx, eng):
+    """Prompt passes of cfg4's model alone (eager launches, for kernel traces): prompts of 256, 1024 and 4000 tokens
+    from an empty cache, each timed on its second run."""
+    from ksearch_amd import hip, synth
+
+    cfg = synth.GEMMA_E2B_SYNTH
+    q4k, q6k = hip.device_quantizers(ctx, eng)
+    m = hip.Gemma(ctx, cfg, synth.gemma_weights(cfg, 4000, q4k, q6k))
+    rng = np.random.default_rng(4002)
+    out = {}
+    for n in (256, 1024, 4000):
+        prompt = [int(t) for t in rng.integers(0, cfg["vocab"], n + 1)]
+        for _ in range(2):
+            m.reset()
+            ms = m.generate(prompt, 1, use_graph=False)[1]
+        out[f"prompt_{n}"] = dict(ms=round(ms, 2), tok_per_s=round(n / ms * 1e3, 1))
+    m.close()
+    return out
+
+
 def bench_decode_gemma4_layout(ctx, eng, use_graph=True):
     """Greedy decode at the layer layout of the real Gemma-4 E2B checkpoints (synthetic weights): 35 layers of
     hidden 1536, four sliding-window layers (head dim 256, window 512) per full-attention layer (head dim 512),
@@ -352,7 +372,7 @@ def main() -> int:
     ap.add_argument("--attn-form", choices=["default", "lanes", "mfma"], default="default",
                     help="cfg3: the split-KV row phase as the register (lanes) or the matrix-core (mfma) kernel instead of "
                          "the library's choice for the shape")
-    ap.add_argument("--only", choices=["cfg1", "cfg2", "cfg3", "cfg4", "gemma4", "copy", "floor"],
+    ap.add_argument("--only", choices=["cfg1", "cfg2", "cfg3", "cfg4", "gemma4", "prefill", "copy", "floor"],
                     help="run one secondary workload and print its record (for profiling runs); 'copy' is a plain "
                          "64 MiB device copy, the known-size kernel that calibrates the FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
@@ -381,6 +401,7 @@ def main() -> int:
         else:
             r = {"cfg2": lambda: bench_prefill(ctx), "cfg3": lambda: bench_attention(ctx, ev, sched={"lanes": dict(vec=3), "mfma": dict(vec=2)}.get(args.attn_form)),
                  "cfg4": lambda: bench_decode(ctx, eng, not args.eager),
+                 "prefill": lambda: bench_prompt_pass(ctx, eng),
                  "gemma4": lambda: bench_decode_gemma4_layout(ctx, eng, not args.eager)}[args.only]()
         ctx.close()
         print(json.dumps({args.only: r}))

@@ -1255,7 +1255,10 @@ int bind_matvec_batch(ksh_kernel &k)
     if (want && want != 32 && want != BN) return set_error("matvec_batch: unsupported schedule nr0=%u (32 or %d)", want, BN);
     const bool can_skinny = !q6 && batch <= kSkinnyMaxBatch;
     if (want == 32 && !can_skinny) return set_error("matvec_batch: the small-batch form takes Q4_K weights and up to %d tokens", kSkinnyMaxBatch);
-    k.variant = (want == 32 || (want == 0 && can_skinny)) ? 1 : 0;
+    // (long rows of a short matrix leave the small-batch form 64 workgroups with four superblocks per wave: from 33
+    // tokens on the tile over K slices is faster there -- 2048 x 8192 at 63 tokens: 27.5 us against 41.0)
+    const bool long_rows = batch > 32 && rows <= 2048 && cols >= 8192;
+    k.variant = (want == 32 || (want == 0 && can_skinny && !long_rows)) ? 1 : 0;
     k.info.sched = k.desc.sched;
     if (k.variant == 1) {
         set_launch(k, (uint32_t)((rows + 31) / 32), 1, 1, 512, (uint32_t)(8 * (batch <= 32 ? 1 : 2) * 16 * 64 * 4));
@@ -1274,7 +1277,7 @@ int bind_matvec_batch(ksh_kernel &k)
         ks = k.desc.sched.k_split;
         if (nsb % ks) return set_error("matvec_batch: k_split=%lld does not divide the %lld superblocks of a row", (long long)ks, (long long)nsb);
     } else {
-        while (tiles * parts * ks < 256 && nsb % (ks * 2) == 0) ks *= 2;
+        while (tiles * parts * ks < 256 && nsb % (ks * 2) == 0 && nsb / (ks * 2) >= 2) ks *= 2;   // (a slice of one superblock is all prologue)
     }
     // (f32 activations with fewer tiles than compute units: both parts in one launch even without a K split)
     const bool z_form = ks > 1 || (parts == 2 && tiles < 256 && !k.desc.sched.k_split);

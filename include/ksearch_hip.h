@@ -59,7 +59,12 @@ enum ksh_kind {
      * dtypes[0] = Q4K | Q6K (GGUF byte order, blocks at 2-byte alignment),
      * dtypes[1] = BF16 (X) or F32 (X is then taken as hi + lo f16 parts, 22 bits, in two passes: the form the
      * decode loops' prompt chunks use), output F32 token-major.
-     * in: W, X   out: Y[batch, rows] */
+     * in: W, X   out: Y[batch, rows]
+     * dims[3], dims[4] (0 = none): rows of a second and a third matrix of the same dtype over the same X, taken in
+     * the same launch (q | k | v of a prompt chunk: one preparation of X, one grid).  in: W, X, W1[, W2]
+     * out: Y, Y1[batch, rows1][, Y2[batch, rows2]].
+     * sched.nr0 = 32 | 128 picks the small-batch form (Q4_K, up to 64 tokens, one matrix) or the 128 x 128 tile;
+     * sched.k_split = the tile's K slices (a divisor of cols / 256; 1 = whole rows; 0 = enough to fill the chip). */
     KSH_MATVEC_BATCH = 2,
     /* MatvecQkv: three GEMVs sharing x.  dims: q_rows, kv_rows, cols.
      * in: Wq, Wk, Wv, x   out: q, k, v */

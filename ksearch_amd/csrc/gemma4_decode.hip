@@ -410,6 +410,19 @@ int forward_prefill_chunk4(ksh_gemma4 *m, const uint32_t *tokens, int t)
         ksh_kernel *kk = nullptr;
         return get(m, KSH_MATVEC_BATCH, {rows, cols, tp}, {dt, KSH_F32, KSH_F32}, {}, &kk) || enc(m, kk, {w, x}, {y}, n);
     };
+    // beyond the small-batch form's 64 tokens, matrices of one dtype over the same rows (q | k | v, gate | up) are one
+    // launch of the 128 x 128 tile over one preparation of the rows
+    auto mm2 = [&](int dt, int64_t rows, int64_t cols, ksh_buf *w0, ksh_buf *w1, ksh_buf *x, ksh_buf *y0, ksh_buf *y1) {
+        ksh_kernel *kk = nullptr;
+        return get(m, KSH_MATVEC_BATCH, {rows, cols, tp, rows}, {dt, KSH_F32, KSH_F32}, {}, &kk) || enc(m, kk, {w0, x, w1}, {y0, y1}, n);
+    };
+    auto mm3 = [&](int dt, int64_t rows0, int64_t rows12, int64_t cols, ksh_buf *w0, ksh_buf *w1, ksh_buf *w2, ksh_buf *x, ksh_buf *y0, ksh_buf *y1,
+                   ksh_buf *y2) {
+        ksh_kernel *kk = nullptr;
+        return get(m, KSH_MATVEC_BATCH, {rows0, cols, tp, rows12, rows12}, {dt, KSH_F32, KSH_F32}, {}, &kk) ||
+               enc(m, kk, {w0, x, w1, w2}, {y0, y1, y2}, n);
+    };
+    const bool merged = tp > 32;
     if (get(m, KSH_COPY_SCALE_INDEXED, {h, c.vocab, t}, {m->g.dt_embd}, {std::sqrt((float)c.hidden)}, &k) ||
         enc(m, k, {m->g.token_embd, m->c_tok}, {m->c_x}, n))
         return 1;
@@ -434,9 +447,11 @@ int forward_prefill_chunk4(ksh_gemma4 *m, const uint32_t *tokens, int t)
         ksh_buf *rope_tab = P.swa ? m->rope_swa : m->rope_full;
         ksh_buf *kc = m->kv_k[P.src], *vc = m->kv_v[P.src];
         ksh_kernel *k_head = nullptr, *k_sdpa = nullptr, *k_gelu = nullptr;
-        if (enc(m, k_norm, {m->c_x, L.attn_norm}, {m->c_x2}, n) || mm(L.dt_q, P.qd, h, L.wq, m->c_x2, m->c_q)) return 1;
+        const bool qkv_merged = merged && P.owns && L.dt_q == L.dt_k && L.dt_q == L.dt_v;
+        if (enc(m, k_norm, {m->c_x, L.attn_norm}, {m->c_x2}, n)) return 1;
+        if (qkv_merged ? mm3(L.dt_q, P.qd, P.kvd, h, L.wq, L.wk, L.wv, m->c_x2, m->c_q, m->c_k, m->c_v) : mm(L.dt_q, P.qd, h, L.wq, m->c_x2, m->c_q)) return 1;
         if (P.owns) {
-            if (mm(L.dt_k, P.kvd, h, L.wk, m->c_x2, m->c_k) || mm(L.dt_v, P.kvd, h, L.wv, m->c_x2, m->c_v) ||
+            if ((!qkv_merged && (mm(L.dt_k, P.kvd, h, L.wk, m->c_x2, m->c_k) || mm(L.dt_v, P.kvd, h, L.wv, m->c_x2, m->c_v))) ||
                 get(m, KSH_RMSNORM_PER_HEAD_QKV_Q40, {c.n_q, c.n_kv, P.hd, c.max_seq, t}, {}, {c.eps}, &k_head) ||
                 enc(m, k_head, {m->c_q, L.q_norm, rope_tab, m->c_k, L.k_norm, m->c_v, m->meta_full}, {m->c_q, kc, vc}, n))
                 return 1;
@@ -450,7 +465,8 @@ int forward_prefill_chunk4(ksh_gemma4 *m, const uint32_t *tokens, int t)
             enc(m, k_sdpa, {m->c_q, kc, vc, P.swa ? m->c_meta_swa : m->c_meta_full}, {m->c_tmp, m->c_o}, n) ||
             mm(L.dt_o, h, P.qd, L.wo, m->c_o, m->c_y) ||
             enc(m, k_add_then, {m->c_y, L.post_attn_norm, m->c_x, L.ffn_norm}, {m->c_x, m->c_x2}, n) ||
-            mm(L.dt_gate, L.ffn, h, L.wgate, m->c_x2, m->c_g) || mm(L.dt_up, L.ffn, h, L.wup, m->c_x2, m->c_u) ||
+            (merged && L.dt_gate == L.dt_up ? mm2(L.dt_gate, L.ffn, h, L.wgate, L.wup, m->c_x2, m->c_g, m->c_u)
+                                            : (mm(L.dt_gate, L.ffn, h, L.wgate, m->c_x2, m->c_g) || mm(L.dt_up, L.ffn, h, L.wup, m->c_x2, m->c_u))) ||
             get(m, KSH_GELU_MUL, {(int64_t)t * L.ffn}, {}, {}, &k_gelu) || enc(m, k_gelu, {m->c_g, m->c_u}, {m->c_ff}, n) ||
             mm(L.dt_down, h, L.ffn, L.wdown, m->c_ff, m->c_y) || enc(m, k_add, {m->c_y, L.post_ffw_norm, m->c_x}, {m->c_x}, n))
             return 1;

@@ -406,6 +406,12 @@ int forward_prefill_chunk(ksh_gemma *m, const uint32_t *tokens, int t)
     if (ksh_synchronize(m->ctx)) return 1;                                   // c_tok may still be read by the previous chunk
     if (ksh_buffer_write(m->ctx, m->c_tok, 0, ids, (size_t)t * 4, 1)) return 1;
     ksh_kernel *k_embed, *k_norm, *k_mm_q, *k_mm_kv, *k_head, *k_sdpa, *k_mm_o, *k_add_then, *k_mm_ff, *k_gelu, *k_mm_down, *k_add;
+    // beyond the small-batch form's 64 tokens q | k | v are one launch of the 128 x 128 tile over one preparation of x
+    // (and gate | up likewise)
+    ksh_kernel *k_mm_qkv = nullptr, *k_mm_gu = nullptr;
+    if (tp > 32 && (get(m, KSH_MATVEC_BATCH, {qd, c.hidden, tp, kvd, kvd}, {KSH_Q4K, KSH_F32, KSH_F32}, {}, &k_mm_qkv) ||
+                    get(m, KSH_MATVEC_BATCH, {c.ffn, c.hidden, tp, c.ffn}, {KSH_Q4K, KSH_F32, KSH_F32}, {}, &k_mm_gu)))
+        return 1;
     const float embed_scale = std::sqrt((float)c.hidden);
     if (get(m, KSH_COPY_SCALE_INDEXED, {c.hidden, c.vocab, t}, {KSH_Q6K}, {embed_scale}, &k_embed) ||
         get(m, KSH_RMSNORM, {c.hidden, 0, 0, t}, {}, {c.eps}, &k_norm) ||
@@ -430,13 +436,15 @@ int forward_prefill_chunk(ksh_gemma *m, const uint32_t *tokens, int t)
     for (int l = 0; l < c.n_layers; l++) {
         const ksh_gemma_layer &L = m->layers[l];
         if (enc(m, k_norm, {m->c_x, L.attn_norm}, {m->c_x2}, n) ||
-            enc(m, k_mm_q, {L.wq, m->c_x2}, {m->c_q}, n) || enc(m, k_mm_kv, {L.wk, m->c_x2}, {m->c_k}, n) ||
-            enc(m, k_mm_kv, {L.wv, m->c_x2}, {m->c_v}, n) ||
+            (k_mm_qkv ? enc(m, k_mm_qkv, {L.wq, m->c_x2, L.wk, L.wv}, {m->c_q, m->c_k, m->c_v}, n)
+                      : (enc(m, k_mm_q, {L.wq, m->c_x2}, {m->c_q}, n) || enc(m, k_mm_kv, {L.wk, m->c_x2}, {m->c_k}, n) ||
+                         enc(m, k_mm_kv, {L.wv, m->c_x2}, {m->c_v}, n))) ||
             enc(m, k_head, {m->c_q, L.q_norm, m->rope, m->c_k, L.k_norm, m->c_v, m->meta}, {m->c_q, m->kv_k[l], m->kv_v[l]}, n) ||
             enc(m, k_sdpa, {m->c_q, m->kv_k[l], m->kv_v[l], m->c_meta}, {m->c_tmp, m->c_o}, n) ||
             enc(m, k_mm_o, {L.wo, m->c_o}, {m->c_y}, n) ||
             enc(m, k_add_then, {m->c_y, L.post_attn_norm, m->c_x, L.ffn_norm}, {m->c_x, m->c_x2}, n) ||
-            enc(m, k_mm_ff, {L.wgate, m->c_x2}, {m->c_g}, n) || enc(m, k_mm_ff, {L.wup, m->c_x2}, {m->c_u}, n) ||
+            (k_mm_gu ? enc(m, k_mm_gu, {L.wgate, m->c_x2, L.wup}, {m->c_g, m->c_u}, n)
+                     : (enc(m, k_mm_ff, {L.wgate, m->c_x2}, {m->c_g}, n) || enc(m, k_mm_ff, {L.wup, m->c_x2}, {m->c_u}, n))) ||
             enc(m, k_gelu, {m->c_g, m->c_u}, {m->c_ff}, n) || enc(m, k_mm_down, {L.wdown, m->c_ff}, {m->c_y}, n) ||
             enc(m, k_add, {m->c_y, L.post_ffw_norm, m->c_x}, {m->c_x}, n))
             return 1;

@@ -150,6 +150,11 @@ struct MmParams {
     int ksplit;
     const _Float16 *Xf_lo, *SxA_lo;
     float *Y_parts;
+    // Up to three matrices that share the activations (q | k | v of a prompt chunk) in one launch of the 128 x 128
+    // tile: blockIdx.y counts the row tiles of W, then of W1, then of W2, each with its own result.
+    const uint8_t *W1, *W2;
+    float *Y1, *Y2;
+    int rows1, rows2;
 };
 
 __device__ __forceinline__ uint32_t pair_f16(uint32_t masked, uint32_t sc)
@@ -197,15 +202,25 @@ __global__ __launch_bounds__(kThreadsMM) void q_mul_mm_kernel(MmParams p)
     auto dsc_stage = [&](int i) { return reinterpret_cast<float *>(lds + 2 * kLdsMain + 2 * kLdsMin) + (i & 1) * BN; };
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int t0 = blockIdx.x * BM, r0 = blockIdx.y * BN;
+    // which matrix this row tile belongs to (the copy of the arguments is this workgroup's own)
+    int by = blockIdx.y, ycol = 0;
+    const int rows_all = p.rows + p.rows1 + p.rows2;
+    if (p.rows1) {
+        const int ty0 = (p.rows + BN - 1) / BN, ty1 = (p.rows1 + BN - 1) / BN;
+        if (by >= ty0 + ty1) { by -= ty0 + ty1; ycol = p.rows + p.rows1; p.W = p.W2; p.Y = p.Y2; p.rows = p.rows2; }
+        else if (by >= ty0) { by -= ty0; ycol = p.rows; p.W = p.W1; p.Y = p.Y1; p.rows = p.rows1; }
+    }
+    const int t0 = blockIdx.x * BM, r0 = by * BN;
     const int nsb_row = p.cols / 256;                            // superblocks per weight row
     int nsb = nsb_row, sb0 = 0;                                  // this workgroup's share of them
+    size_t ystride = (size_t)p.rows;
     if (p.ksplit) {
         const int part = blockIdx.z / p.ksplit, slice = blockIdx.z % p.ksplit;
         nsb = nsb_row / p.ksplit;
         sb0 = slice * nsb;
         if (part) { p.Xf = p.Xf_lo; p.SxA = p.SxA_lo; }
-        p.Y = p.Y_parts + (size_t)blockIdx.z * p.batch * p.rows;
+        p.Y = p.Y_parts + (size_t)blockIdx.z * p.batch * rows_all + ycol;   // partial sums: all matrices' columns side by side
+        ystride = (size_t)rows_all;
     }
     const int nsteps = nsb * 4;
 
@@ -491,7 +506,7 @@ __global__ __launch_bounds__(kThreadsMM) void q_mul_mm_kernel(MmParams p)
             for (int i = 0; i < 16; i++) {
                 const int t = t0 + wm * 64 + mt * 32 + 8 * (i / 4) + 4 * (lane >> 5) + (i & 3);
                 if (t < p.batch && r < p.rows) {
-                    float *y = &p.Y[(size_t)t * p.rows + r];
+                    float *y = &p.Y[(size_t)t * ystride + r];
                     *y = p.accum != 0.f ? fmaf(p.accum, F[mt][nt][i], *y) : F[mt][nt][i];
                 }
             }
@@ -974,9 +989,12 @@ __global__ __launch_bounds__(256) void mm_round_fold_kernel(const float *__restr
 }
 
 // y[i] = the K slices' partial sums of element i, slice after slice; the slices of the low parts of f32 activations
-// (parts = 2) come in scaled
-__global__ __launch_bounds__(256) void mm_parts_fold_kernel(const float *__restrict__ part, float *__restrict__ y, int n, int slices, int parts, float lo_scale)
+// (parts = 2) come in scaled.  The partial sums hold the columns of up to three matrices side by side (rows0 | rows1 |
+// rows2 per token), each with a result buffer of its own.
+__global__ __launch_bounds__(256) void mm_parts_fold_kernel(const float *__restrict__ part, float *__restrict__ y0, float *__restrict__ y1, float *__restrict__ y2,
+                                                             int batch, int rows0, int rows1, int rows2, int slices, int parts, float lo_scale)
 {
+    const int rows_all = rows0 + rows1 + rows2, n = batch * rows_all;
     const int i = blockIdx.x * 256 + threadIdx.x;
     if (i >= n) return;
     float s = part[i];
@@ -986,7 +1004,11 @@ __global__ __launch_bounds__(256) void mm_parts_fold_kernel(const float *__restr
         for (int k = 1; k < slices; k++) l += part[(size_t)(slices + k) * n + i];
         s = fmaf(lo_scale, l, s);
     }
-    y[i] = s;
+    if (!rows1) { y0[i] = s; return; }
+    const int t = i / rows_all, c = i - t * rows_all;
+    if (c < rows0) y0[(size_t)t * rows0 + c] = s;
+    else if (c < rows0 + rows1) y1[(size_t)t * rows1 + c - rows0] = s;
+    else y2[(size_t)t * rows2 + c - rows0 - rows1] = s;
 }
 
 // The same round against a Q6_K matrix with row-grouped fields (KSH_Q6K_ROWS: the LM head as the decode loops keep it;
@@ -1189,6 +1211,10 @@ int launch_mul_mm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
     p.W = (const uint8_t *)a.in[0];
     p.Y = (float *)a.out[0];
     p.rows = rows; p.cols = cols; p.batch = batch;
+    const int rows1 = (int)k.desc.dims[3], rows2 = (int)k.desc.dims[4];
+    p.rows1 = rows1; p.rows2 = rows2;
+    p.W1 = rows1 ? (const uint8_t *)a.in[2] : p.W; p.W2 = rows2 ? (const uint8_t *)a.in[3] : p.W;
+    p.Y1 = rows1 ? (float *)a.out[1] : p.Y; p.Y2 = rows2 ? (float *)a.out[2] : p.Y;
     if (k.variant == 1) {
         // the small-batch form: one launch, the low parts riding along
         p.Xf = Xf; p.SxA = SxA; p.accum = 0.f;
@@ -1202,7 +1228,7 @@ int launch_mul_mm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
         const hipError_t e2 = hipGetLastError();
         return e2 == hipSuccess ? 0 : hip_fail(e2, "mul_mm (small batch) launch");
     }
-    const dim3 grid((batch + BM - 1) / BM, (rows + BN - 1) / BN);
+    const dim3 grid((batch + BM - 1) / BM, (rows + BN - 1) / BN + (rows1 + BN - 1) / BN + (rows2 + BN - 1) / BN);
     p.ksplit = 0; p.Xf_lo = Xf_lo; p.SxA_lo = SxA_lo; p.Y_parts = nullptr;
     if (k.variant >= 2) {
         // few tiles: K slices and both parts of f32 activations as blockIdx.z of one launch, then the fold
@@ -1215,8 +1241,9 @@ int launch_mul_mm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
         else hipLaunchKernelGGL(q_mul_mm_kernel<false>, gz, dim3(kThreadsMM), kLdsBytes, st, p);
         hipError_t e3 = hipGetLastError();
         if (e3 != hipSuccess) return hip_fail(e3, "mul_mm (K slices) launch");
-        const int n2 = batch * rows;
-        hipLaunchKernelGGL(mm_parts_fold_kernel, dim3((n2 + 255) / 256), dim3(256), 0, st, (const float *)p.Y_parts, (float *)a.out[0], n2, ks, parts, 1.0f / 2048.0f);
+        const int n2 = batch * (rows + rows1 + rows2);
+        hipLaunchKernelGGL(mm_parts_fold_kernel, dim3((n2 + 255) / 256), dim3(256), 0, st, (const float *)p.Y_parts, p.Y, p.Y1, p.Y2, batch, rows, rows1, rows2,
+                           ks, parts, 1.0f / 2048.0f);
         e3 = hipGetLastError();
         return e3 == hipSuccess ? 0 : hip_fail(e3, "mul_mm fold launch");
     }
@@ -1242,18 +1269,26 @@ int bind_matvec_batch(ksh_kernel &k)
     if (k.desc.dtypes[1] != KSH_BF16 && !f32x) return set_error("matvec_batch: activation dtype %d is not built (BF16 and F32 are)", k.desc.dtypes[1]);
     if (rows <= 0 || batch <= 0 || rows > (1 << 24) || batch > (1 << 20)) return set_error("matvec_batch: rows=%lld batch=%lld", (long long)rows, (long long)batch);
     if (cols <= 0 || cols % 256 || cols > (1 << 20)) return set_error("matvec_batch: cols=%lld is not a positive multiple of 256", (long long)cols);
-    k.info.n_inputs = 2;
-    k.info.n_outputs = 1;
-    k.in_bytes[0] = (size_t)rows * (cols / 256) * (q6 ? 210 : 144); k.in_align[0] = q6 ? 2 : 16;
+    // dims[3], dims[4]: the rows of a second and a third matrix over the same activations (q | k | v of a prompt
+    // chunk), taken by the 128 x 128 tile in the same launch
+    const int64_t rows1 = k.desc.dims[3], rows2 = k.desc.dims[4], rows_all = rows + rows1 + rows2;
+    if (rows1 < 0 || rows2 < 0 || (rows2 && !rows1) || rows_all > (1 << 24)) return set_error("matvec_batch: rows of the further matrices %lld, %lld", (long long)rows1, (long long)rows2);
+    const int n_mat = 1 + (rows1 > 0) + (rows2 > 0);
+    k.info.n_inputs = 1 + n_mat;
+    k.info.n_outputs = n_mat;
+    const size_t row_bytes = (size_t)(cols / 256) * (q6 ? 210 : 144);
+    k.in_bytes[0] = (size_t)rows * row_bytes; k.in_align[0] = q6 ? 2 : 16;
     k.in_bytes[1] = (size_t)batch * cols * (f32x ? 4 : 2); k.in_align[1] = 16;
     k.out_bytes[0] = (size_t)batch * rows * 4; k.out_align[0] = 4;
+    if (rows1) { k.in_bytes[2] = (size_t)rows1 * row_bytes; k.in_align[2] = k.in_align[0]; k.out_bytes[1] = (size_t)batch * rows1 * 4; k.out_align[1] = 4; }
+    if (rows2) { k.in_bytes[3] = (size_t)rows2 * row_bytes; k.in_align[3] = k.in_align[0]; k.out_bytes[2] = (size_t)batch * rows2 * 4; k.out_align[2] = 4; }
     // f16 copy of X plus the min-term operand (32 halves per token and superblock)
     k.scratch_bytes = ((size_t)((batch + 31) / 32 * 32) * cols * 2 + (size_t)batch * (cols / 256) * 64) * (f32x ? 2 : 1);
     // schedule: nr0 = weight rows per workgroup.  32 = the small-batch form (Q4_K, up to 64 tokens: the default
     // there), 128 = the 128 x 128 tile.
     const uint32_t want = k.desc.sched.nr0;
     if (want && want != 32 && want != BN) return set_error("matvec_batch: unsupported schedule nr0=%u (32 or %d)", want, BN);
-    const bool can_skinny = !q6 && batch <= kSkinnyMaxBatch;
+    const bool can_skinny = !q6 && batch <= kSkinnyMaxBatch && n_mat == 1;
     if (want == 32 && !can_skinny) return set_error("matvec_batch: the small-batch form takes Q4_K weights and up to %d tokens", kSkinnyMaxBatch);
     // (long rows of a short matrix leave the small-batch form 64 workgroups with four superblocks per wave: from 33
     // tokens on the tile over K slices is faster there -- 2048 x 8192 at 63 tokens: 27.5 us against 41.0)
@@ -1271,7 +1306,8 @@ int bind_matvec_batch(ksh_kernel &k)
     // slices and, for f32 activations, the hi and the lo part become workgroups of the same launch, until the grid is
     // about one workgroup per compute unit; every slice stores its partial sums and a second launch adds them in a
     // fixed order.  sched.k_split names the slice count (a divisor of cols / 256; 1 = none).
-    const int64_t tiles = ((batch + BM - 1) / BM) * ((rows + BN - 1) / BN), nsb = cols / 256, parts = f32x ? 2 : 1;
+    const int64_t row_tiles = (rows + BN - 1) / BN + (rows1 + BN - 1) / BN + (rows2 + BN - 1) / BN;
+    const int64_t tiles = ((batch + BM - 1) / BM) * row_tiles, nsb = cols / 256, parts = f32x ? 2 : 1;
     int64_t ks = 1;
     if (k.desc.sched.k_split) {
         ks = k.desc.sched.k_split;
@@ -1282,11 +1318,11 @@ int bind_matvec_batch(ksh_kernel &k)
     // (f32 activations with fewer tiles than compute units: both parts in one launch even without a K split)
     const bool z_form = ks > 1 || (parts == 2 && tiles < 256 && !k.desc.sched.k_split);
     k.variant = z_form ? (int)(ks << 1) : 0;
-    if (z_form) k.scratch_bytes += (size_t)parts * ks * batch * rows * 4;
-    set_launch(k, (uint32_t)((batch + BM - 1) / BM), (uint32_t)((rows + BN - 1) / BN), z_form ? (uint32_t)(ks * parts) : 1, kThreadsMM,
+    if (z_form) k.scratch_bytes += (size_t)parts * ks * batch * rows_all * 4;
+    set_launch(k, (uint32_t)((batch + BM - 1) / BM), (uint32_t)row_tiles, z_form ? (uint32_t)(ks * parts) : 1, kThreadsMM,
                (uint32_t)kLdsBytes);
     k.info.sched.tg = kThreadsMM; k.info.sched.nsg = kThreadsMM / 64; k.info.sched.nr0 = BN; k.info.sched.k_split = (uint32_t)ks; k.info.sched.lds_tile = KS;
-    set_name(k, "mul_mm_%s_%dx%dx%d%s%s", q6 ? "q6k" : "q4k", BM, BN, KS, f32x ? "_f32x" : "", z_form ? "_kz" : "");
+    set_name(k, "mul_mm_%s_%dx%dx%d%s%s%s", q6 ? "q6k" : "q4k", BM, BN, KS, f32x ? "_f32x" : "", z_form ? "_kz" : "", n_mat == 3 ? "_x3" : n_mat == 2 ? "_x2" : "");
     k.launch = launch_mul_mm;
     return 0;
 }
@@ -1390,13 +1426,14 @@ int mul_mm_candidates(const ksh_kernel_desc &d, ksh_sched *out, int cap)
         s.tg = kThreadsMM; s.nsg = kThreadsMM / 64; s.nr0 = BN; s.lds_tile = KS; s.unroll = 1; s.vec = 0; s.k_split = 1;
         out[n++] = s;
     }
-    if (n < cap && d.dtypes[0] == KSH_Q4K && d.dims[2] <= kSkinnyMaxBatch) {
+    if (n < cap && d.dtypes[0] == KSH_Q4K && d.dims[2] <= kSkinnyMaxBatch && !d.dims[3]) {
         ksh_sched s{};
         s.tg = 512; s.nsg = 8; s.nr0 = 32; s.lds_tile = 16; s.unroll = 1; s.vec = 0; s.k_split = 8;
         out[n++] = s;
     }
     // the 128 x 128 tile over K slices, where whole rows leave the grid short of one workgroup per compute unit
-    const int64_t tiles = ((d.dims[2] + BM - 1) / BM) * ((d.dims[0] + BN - 1) / BN) * (d.dtypes[1] == KSH_F32 ? 2 : 1), nsb = d.dims[1] / 256;
+    const int64_t tiles = ((d.dims[2] + BM - 1) / BM) * ((d.dims[0] + BN - 1) / BN + (d.dims[3] + BN - 1) / BN + (d.dims[4] + BN - 1) / BN) * (d.dtypes[1] == KSH_F32 ? 2 : 1),
+                  nsb = d.dims[1] / 256;
     for (uint32_t ks : {2u, 4u, 8u, 16u}) {
         if (n >= cap || nsb % ks || tiles * (ks / 2) >= 256) continue;
         ksh_sched s{};

@@ -180,6 +180,37 @@ def test_mul_mm_k_slices(ctx, wdt, xdt, batch, rows, cols, ks):
     assert worst <= 2e-5, worst
 
 
+@pytest.mark.parametrize("xdt,batch,rows3,cols", [(DType.F32, 200, (384, 128, 128), 1024), (DType.BF16, 300, (2048, 256, 256), 512),
+                                                  (DType.F32, 2048, (2048, 256, 256), 256), (DType.F32, 130, (200, 100, 0), 2048)])
+def test_mul_mm_matrices_sharing_the_activations(ctx, xdt, batch, rows3, cols):
+    """Up to three matrices over the same activations in one launch of the tile (q | k | v of a prompt chunk): every
+    result against the float64 product and against the matrix's own launch, with K slices (few tiles) and as whole
+    rows in two passes (2048 tokens), ragged row tiles, two matrices."""
+    ws = [synth.q4k_blocks(r * cols // 256, 660 + i) for i, r in enumerate(rows3) if r]
+    x = synth.normal_f32(batch * cols, 663).reshape(batch, cols)
+    if xdt == DType.BF16:
+        xf, xb = synth.bf16_round(x.reshape(-1))
+        x, xin = xf.reshape(batch, cols), ctx.buffer_bytes(xb)
+    else:
+        xin = ctx.buffer_f32(x)
+    k = ctx.compile(hip.make_desc(hip.Kind.MATVEC_BATCH, (rows3[0], cols, batch, rows3[1], rows3[2]), (DType.Q4K, xdt, DType.F32)))
+    assert k.name.endswith("_x%d" % len(ws)), k.name
+    assert ("_kz" in k.name) == (xdt == DType.F32 and batch < 2048), k.name      # (512 columns of bf16: two superblocks, no slices)
+    bws = [ctx.buffer_bytes(w) for w in ws]
+    outs = [ctx.buffer_empty_f32(batch * r) for r in rows3 if r]
+    ctx.encode_multi(k, [bws[0], xin] + bws[1:], outs)
+    ctx.synchronize()
+    for i, (w, r) in enumerate(zip(ws, [r for r in rows3 if r])):
+        got = ctx.read_f32(outs[i], batch * r).reshape(batch, r)
+        worst = max(float(rel_err(got[t], oracle.matvec_f64(oracle.Q4K, w, r, cols, x[t])).max()) for t in range(0, batch, 37))
+        assert worst <= 2e-5, (i, worst)
+        k1 = ctx.compile(hip.make_desc(hip.Kind.MATVEC_BATCH, (r, cols, batch), (DType.Q4K, xdt, DType.F32), (), dict(nr0=128)))
+        y1 = ctx.buffer_empty_f32(batch * r)
+        ctx.encode_multi(k1, [bws[i], xin], [y1])
+        ctx.synchronize()
+        assert_close(got, ctx.read_f32(y1, batch * r).reshape(batch, r), 2e-6, f"matrix {i} against its own launch")
+
+
 def test_mul_mm_k_slices_must_divide_the_row(ctx):
     with pytest.raises(hip.KshError, match="does not divide"):
         ctx.compile(hip.make_desc(hip.Kind.MATVEC_BATCH, (256, 2048, 100), (DType.Q4K, DType.BF16, DType.F32), (), dict(k_split=3)))

@@ -460,8 +460,8 @@ int forward_prefill_chunk4(ksh_gemma4 *m, const uint32_t *tokens, int t)
                 enc(m, k_head, {m->c_q, L.q_norm, rope_tab, m->meta_full}, {m->c_q}, n))
                 return 1;
         }
-        // (heads of 256 in chunks of more than 16 tokens take the attention's matrix-core form: one partition per token)
-        if (get(m, KSH_SDPA_BATCH, {c.n_q, c.n_kv, P.hd, c.max_seq, t, t > 16 && P.hd == 256 && c.n_q / c.n_kv <= 8 ? 1 : kChunkPartitions4}, {KSH_Q40, KSH_F32}, {c.attn_scale}, &k_sdpa) ||
+        // (heads of 256 or 512 in chunks of more than 16 tokens take the attention's matrix-core form: one partition per token)
+        if (get(m, KSH_SDPA_BATCH, {c.n_q, c.n_kv, P.hd, c.max_seq, t, t > 16 && (P.hd == 256 || P.hd == 512) && c.n_q / c.n_kv <= 8 ? 1 : kChunkPartitions4}, {KSH_Q40, KSH_F32}, {c.attn_scale}, &k_sdpa) ||
             enc(m, k_sdpa, {m->c_q, kc, vc, P.swa ? m->c_meta_swa : m->c_meta_full}, {m->c_tmp, m->c_o}, n) ||
             mm(L.dt_o, h, P.qd, L.wo, m->c_o, m->c_y) ||
             enc(m, k_add_then, {m->c_y, L.post_attn_norm, m->c_x, L.ffn_norm}, {m->c_x, m->c_x2}, n) ||

@@ -868,13 +868,18 @@ __device__ __forceinline__ int mfma_k_elem(int s, int kq)
     return 4 * kq + byte + ((s >> 1) & 1) * 16;      //    nibble: lo lo hi hi lo lo hi hi
 }
 
-template <int HD, int TR>
+// HDV < HD (heads of 512 as two halves of 256): the workgroups of blockIdx.y = 2 * kvh + half both work out the scores
+// and the softmax over all HD dimensions (the same numbers twice) and each takes P.V for its HDV dimensions of V,
+// whose accumulators are what limits the head size a wave can hold.
+template <int HD, int TR, int HDV = HD>
 __global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_mfma_kernel(LaneParams p)
 {
     static_assert(TR == 16 || TR == 32, "tile rows");
+    static_assert(HD % HDV == 0 && (HDV == HD || TR == 32), "V halves come with tiles of 32 rows");
     constexpr int NW = kMfmaRound / TR, NT = NW * 64, NB = HD / 32, ROWB = NB * 18, TILEB = TR * ROWB;
-    constexpr int STRIP = 2 * TILEB + 2 * TR * NB * 4;           // K bytes, V bytes, K scales, V scales
-    constexpr int PIECES = TR * ROWB / 16;                       // 128-bit pieces of a tile
+    constexpr int NBV = HDV / 32, ROWBV = NBV * 18, TILEBV = TR * ROWBV;   // this workgroup's share of a V row
+    constexpr int STRIP = TILEB + TILEBV + TR * NB * 4 + TR * NBV * 4;     // K bytes, V bytes, K scales, V scales
+    constexpr int PIECES = TR * ROWB / 16, PIECESV = TR * ROWBV / 16;      // 128-bit pieces of a tile
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int col = lane & 15, q4 = lane >> 4, head = col & 7, is_lo = col >> 3;
@@ -885,10 +890,10 @@ __global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_m
     const uint32_t keep = is_lo ? 0xFFFFFFFFu : 0xFFFFE000u, drop = is_lo ? 0xFFFFE000u : 0u;
     uint8_t *strip = lds_raw + (size_t)wave * STRIP;
     uint8_t *kraw = strip, *vraw = strip + TILEB;
-    float *ksc = reinterpret_cast<float *>(strip + 2 * TILEB), *vsc = ksc + TR * NB;
+    float *ksc = reinterpret_cast<float *>(strip + TILEB + TILEBV), *vsc = ksc + TR * NB;
 
     int part = blockIdx.x, slot = blockIdx.z, nparts = p.nwg;
-    const int kvh = blockIdx.y, groups = p.groups, head0 = kvh * groups;
+    const int kvh = blockIdx.y / (HD / HDV), vhalf = blockIdx.y % (HD / HDV), groups = p.groups, head0 = kvh * groups;
     size_t rec_base = 0;
     int p0, p1, start;
     if (p.balance) {
@@ -910,11 +915,11 @@ __global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_m
     const size_t row_stride = (size_t)p.n_kv * ROWB;
     const size_t kv_slot = p.slot_ids ? (size_t)max((int)p.slot_ids[slot], 0) : (size_t)slot;
     const uint8_t *kbase = p.k + kv_slot * slot_bytes + (size_t)kvh * ROWB;
-    const uint8_t *vbase = p.v + kv_slot * slot_bytes + (size_t)kvh * ROWB;
+    const uint8_t *vbase = p.v + kv_slot * slot_bytes + (size_t)kvh * ROWB + (size_t)vhalf * ROWBV;
 
     // ---- a tile's bytes as whole 128-bit pieces, into registers (the first tile's are requested right behind q)
-    constexpr int NPC = (PIECES + 63) / 64;
-    u32x4_t kpre[NPC], vpre[NPC];
+    constexpr int NPC = (PIECES + 63) / 64, NPCV = (PIECESV + 63) / 64;
+    u32x4_t kpre[NPC], vpre[NPCV];
     auto fetch_tile = [&](int it) __attribute__((always_inline)) {
         const int row0 = p0 + (it * NW + wave) * TR;
         const int nvalid = max(0, min(TR, p1 - row0));
@@ -922,11 +927,20 @@ __global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_m
         for (int u = 0; u < NPC; u++) {
             const int idx = lane + 64 * u, row = idx / (ROWB / 16), pc = idx % (ROWB / 16);
             kpre[u] = u32x4_t{0u, 0u, 0u, 0u};
-            vpre[u] = u32x4_t{0u, 0u, 0u, 0u};
+            if (HDV == HD) vpre[u] = u32x4_t{0u, 0u, 0u, 0u};
             if (idx < PIECES && row < nvalid) {
                 const size_t off = (size_t)(start + row0 + row) * row_stride + (size_t)pc * 16;
                 kpre[u] = *reinterpret_cast<const u32x4_t *>(kbase + off);
-                vpre[u] = *reinterpret_cast<const u32x4_t *>(vbase + off);
+                if (HDV == HD) vpre[u] = *reinterpret_cast<const u32x4_t *>(vbase + off);
+            }
+        }
+        if (HDV != HD) {
+#pragma unroll
+            for (int u = 0; u < NPCV; u++) {
+                const int idx = lane + 64 * u, row = idx / (ROWBV / 16), pc = idx % (ROWBV / 16);
+                vpre[u] = u32x4_t{0u, 0u, 0u, 0u};
+                if (idx < PIECESV && row < nvalid)
+                    vpre[u] = *reinterpret_cast<const u32x4_t *>(vbase + (size_t)(start + row0 + row) * row_stride + (size_t)pc * 16);
             }
         }
     };
@@ -940,8 +954,9 @@ __global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_m
     h8v qop[NB];
     float qs24[NB];
     {
-        h8v *qshare = reinterpret_cast<h8v *>(lds_raw + (size_t)NW * STRIP);       // [NB][64] operands
-        float *qsum_share = reinterpret_cast<float *>(qshare + NB * 64);            // [NB][64]
+        // (heads of 512: the shared operands lie over the strips, which nothing has written yet, so that two workgroups fit a compute unit)
+        h8v *qshare = reinterpret_cast<h8v *>(lds_raw + (HDV == HD ? (size_t)NW * STRIP : 0));       // [NB][64] operands
+        float *qsum_share = HDV == HD ? reinterpret_cast<float *>(qshare + NB * 64) : reinterpret_cast<float *>(lds_raw + (size_t)NW * STRIP);   // [NB][64]
         const float *qh = p.q + ((size_t)slot * p.n_q + head0 + min(head, groups - 1)) * HD;
         const bool have = head < groups;
         float4 qlo[QPW], qhi[QPW];
@@ -951,7 +966,7 @@ __global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_m
             qlo[u] = *reinterpret_cast<const float4 *>(qh + 32 * b + 4 * q4);        // elements 4kq .. 4kq+3
             qhi[u] = *reinterpret_cast<const float4 *>(qh + 32 * b + 16 + 4 * q4);   // 16+4kq .. 16+4kq+3
         }
-        fetch_tile(0);
+        if (HDV == HD) fetch_tile(0);      // (heads of 512 have no registers to hold a tile across the q preparation)
 #pragma unroll
         for (int u = 0; u < QPW; u++) {
             const int b = wave + NW * u;
@@ -976,16 +991,17 @@ __global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_m
 #pragma unroll
         for (int b = 0; b < NB; b++) {
             qop[b] = qshare[b * 64 + lane];
-            qs24[b] = qsum_share[b * 64 + lane];
+            if (HDV == HD) qs24[b] = qsum_share[b * 64 + lane];     // (heads of 512 read theirs from LDS block by block: sixteen registers less)
         }
+        if (HDV != HD) __syncthreads();      // every wave has its copy before a strip is written
     }
 
-    f4v O[2 * NB];
-    float Tl[NB];
+    f4v O[2 * NBV];
+    float Tl[NBV];
 #pragma unroll
-    for (int c = 0; c < 2 * NB; c++) O[c] = f4v{0.f, 0.f, 0.f, 0.f};
+    for (int c = 0; c < 2 * NBV; c++) O[c] = f4v{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int b = 0; b < NB; b++) Tl[b] = 0.f;
+    for (int b = 0; b < NBV; b++) Tl[b] = 0.f;
     float m_run = -1.0e30f, l_run = 0.f;
 
     const int ntiles = (p1 - p0 + TR - 1) / TR;
@@ -997,14 +1013,21 @@ __global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_m
         // no workgroup barrier in this loop, only fences that keep the compiler from moving accesses across them.
         // (Later tiles are requested here, not a tile ahead: forty registers less make room for a second wave per
         // SIMD, which covers the wait better than the look-ahead did.)
-        if (it > 0) fetch_tile(it);
+        if (it > 0 || HDV != HD) fetch_tile(it);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
 #pragma unroll
         for (int u = 0; u < NPC; u++) {
             const int idx = lane + 64 * u;
             if (idx < PIECES) {
                 *reinterpret_cast<u32x4_t *>(kraw + idx * 16) = kpre[u];
-                *reinterpret_cast<u32x4_t *>(vraw + idx * 16) = vpre[u];
+                if (HDV == HD) *reinterpret_cast<u32x4_t *>(vraw + idx * 16) = vpre[u];
+            }
+        }
+        if (HDV != HD) {
+#pragma unroll
+            for (int u = 0; u < NPCV; u++) {
+                const int idx = lane + 64 * u;
+                if (idx < PIECESV) *reinterpret_cast<u32x4_t *>(vraw + idx * 16) = vpre[u];
             }
         }
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
@@ -1013,9 +1036,19 @@ __global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_m
         for (int u = 0; u < TR * NB / 64; u++) {
             const int idx = lane + 64 * u, b = idx / TR, row = idx % TR;      // tables are [block][row]
             const uint32_t kb = *reinterpret_cast<const uint16_t *>(kraw + row * ROWB + 18 * b);
-            const uint32_t vb = *reinterpret_cast<const uint16_t *>(vraw + row * ROWB + 18 * b);
             ksc[idx] = row < nvalid ? half_bits_to_f32(kb) : 0.f;
-            vsc[idx] = row < nvalid ? half_bits_to_f32(vb) : 0.f;
+            if (HDV == HD) {
+                const uint32_t vb = *reinterpret_cast<const uint16_t *>(vraw + row * ROWBV + 18 * b);
+                vsc[idx] = row < nvalid ? half_bits_to_f32(vb) : 0.f;
+            }
+        }
+        if (HDV != HD) {
+#pragma unroll
+            for (int u = 0; u < TR * NBV / 64; u++) {
+                const int idx = lane + 64 * u, b = idx / TR, row = idx % TR;
+                const uint32_t vb = *reinterpret_cast<const uint16_t *>(vraw + row * ROWBV + 18 * b);
+                vsc[idx] = row < nvalid ? half_bits_to_f32(vb) : 0.f;
+            }
         }
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         if (nvalid > 0) {
@@ -1034,8 +1067,9 @@ __global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_m
                     const uint32_t d = (uint32_t)*reinterpret_cast<const uint16_t *>(src) |
                                        ((uint32_t)*reinterpret_cast<const uint16_t *>(src + 2) << 16);
                     const f4v c = __builtin_amdgcn_mfma_f32_16x16x32_f16(nibbles_f16(d, nib_mask, nib_one), qop[b], f4v{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                    const float q24 = HDV == HD ? qs24[b] : reinterpret_cast<const float *>(lds_raw + (size_t)NW * STRIP)[b * 64 + lane];
 #pragma unroll
-                    for (int r = 0; r < 4; r++) acc[r] = fmaf(dk[r], c[r] - qs24[b], acc[r]);
+                    for (int r = 0; r < 4; r++) acc[r] = fmaf(dk[r], c[r] - q24, acc[r]);
                 }
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
@@ -1072,16 +1106,16 @@ __global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_m
 #pragma unroll
                 for (int r = 0; r < 4; r++) ar[r] = as_f32((as_u32(ah[r]) & ~odd_mask) | (as_u32(ah[4 + r]) & odd_mask));
 #pragma unroll
-                for (int c = 0; c < 2 * NB; c++)
+                for (int c = 0; c < 2 * NBV; c++)
 #pragma unroll
                     for (int r = 0; r < 4; r++) O[c][r] *= ar[r];
             }
 #pragma unroll
-            for (int b = 0; b < NB; b++) Tl[b] *= alpha;       // (a lane's own column: its own factor)
+            for (int b = 0; b < NBV; b++) Tl[b] *= alpha;       // (a lane's own column: its own factor)
             // ---- P.V per block: P' = p * dv (hi | lo), V codes gathered bytewise: slot s of the lane <-> row
             // 16*(s/4) + 4*q4 + s%4, the rows its own scores belong to
 #pragma unroll
-            for (int b = 0; b < NB; b++) {
+            for (int b = 0; b < NBV; b++) {
                 uint32_t pa[NS / 2], vlo[NS / 2], vhi[NS / 2];
                 float dv[NS];
 #pragma unroll
@@ -1103,7 +1137,7 @@ __global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_m
 #pragma unroll
                 for (int i = 0; i < NS / 2; i++) {
                     const int ra = 16 * ((2 * i) >> 2) + 4 * q4 + ((2 * i) & 3), rb = ra + 1;
-                    const uint32_t t2 = (uint32_t)vraw[ra * ROWB + 18 * b + 2 + col] | ((uint32_t)vraw[rb * ROWB + 18 * b + 2 + col] << 16);
+                    const uint32_t t2 = (uint32_t)vraw[ra * ROWBV + 18 * b + 2 + col] | ((uint32_t)vraw[rb * ROWBV + 18 * b + 2 + col] << 16);
                     vlo[i] = ((t2 << 6) & nib_mask) | nib_one;
                     vhi[i] = ((t2 << 2) & nib_mask) | nib_one;
                 }
@@ -1125,14 +1159,14 @@ __global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_m
 
     // ---- fold: every wave's state to LDS (hi rows first, lo rows added), then one record per head
     __syncthreads();
-    float *ow = reinterpret_cast<float *>(lds_raw);            // [NW][8][HD]
-    float *mlw = ow + NW * 8 * HD;                             // [NW][8][2]
+    float *ow = reinterpret_cast<float *>(lds_raw);            // [NW][8][HDV]
+    float *mlw = ow + NW * 8 * HDV;                            // [NW][8][2]
     const float l_tot = xor32_sum(xor16_sum(l_run));
     // sum(P') of head h and block b: the four lane groups of column h hold its parts.  The accumulator layout wants
     // it by row (head 4 * (q4 & 1) + r): read from lane h as a scalar, picked bitwise like the rescale factors.
-    float t24[4][NB];
+    float t24[4][NBV];
 #pragma unroll
-    for (int b = 0; b < NB; b++) {
+    for (int b = 0; b < NBV; b++) {
         const uint32_t tcol = as_u32(24.f * xor32_sum(xor16_sum(Tl[b])));
 #pragma unroll
         for (int r = 0; r < 4; r++) {
@@ -1148,9 +1182,9 @@ __global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_m
         const int odd = q4 >> 1;
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-            float *dst = ow + ((size_t)wave * 8 + 4 * (q4 & 1) + r) * HD + col + 16 * odd;
+            float *dst = ow + ((size_t)wave * 8 + 4 * (q4 & 1) + r) * HDV + col + 16 * odd;
 #pragma unroll
-            for (int b = 0; b < NB; b++) {
+            for (int b = 0; b < NBV; b++) {
                 const auto sw = __builtin_amdgcn_permlane32_swap(as_u32(O[2 * b][r]), as_u32(O[2 * b + 1][r]), false, false);
                 dst[32 * b] = (as_f32(sw[0]) - t24[r][b]) + as_f32(sw[1]);
             }
@@ -1158,10 +1192,10 @@ __global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_m
     }
     if (lane < 8) { mlw[(wave * 8 + lane) * 2] = m_run; mlw[(wave * 8 + lane) * 2 + 1] = l_tot; }
     __syncthreads();
-    static_assert(NT % HD == 0 || HD % NT == 0, "whole heads per pass, or whole passes per head");
+    static_assert(NT % HDV == 0 || HDV % NT == 0, "whole heads per pass, or whole passes per head");
 #pragma unroll
-    for (int o = tid; o < 8 * HD; o += NT) {
-        const int h = o / HD, d = o % HD, hq = head0 + h;      // (h is the same for a whole wave)
+    for (int o = tid; o < 8 * HDV; o += NT) {
+        const int h = o / HDV, d = o % HDV, hq = head0 + h;      // (h is the same for a whole wave)
         if (h >= groups) break;
         float M = -1.0e30f;
 #pragma unroll
@@ -1171,17 +1205,17 @@ __global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_m
         for (int w = 0; w < NW; w++) {
             const float wt = __expf(mlw[(w * 8 + h) * 2] - M);
             L = fmaf(wt, mlw[(w * 8 + h) * 2 + 1], L);
-            a = fmaf(wt, ow[((size_t)w * 8 + h) * HD + d], a);
+            a = fmaf(wt, ow[((size_t)w * 8 + h) * HDV + d], a);
         }
         if (p.balance) {
             const size_t r = rec_base * p.n_q + hq;
             float *ml = p.tmp + (size_t)gridDim.z * p.nwg * p.n_q * HD;
-            p.tmp[r * HD + d] = a;
-            if (d == 0) { ml[2 * r] = M; ml[2 * r + 1] = L; }
+            p.tmp[r * HD + vhalf * HDV + d] = a;
+            if (d == 0 && vhalf == 0) { ml[2 * r] = M; ml[2 * r + 1] = L; }
         } else {
             float *rec = p.tmp + (size_t)slot * p.n_q * p.nwg * (HD + 2) + (size_t)hq * p.nwg * (HD + 2) + (size_t)part * (HD + 2);
-            rec[2 + d] = a;
-            if (d == 0) { rec[0] = M; rec[1] = L; }
+            rec[2 + vhalf * HDV + d] = a;
+            if (d == 0 && vhalf == 0) { rec[0] = M; rec[1] = L; }
         }
     }
 }
@@ -1205,14 +1239,16 @@ __global__ __launch_bounds__(HD) void sdpa_records_merge_kernel(const float *__r
     out[((size_t)tok * n_q + h) * HD + d] = a / L;
 }
 
-template <int HD, int TR>
+template <int HD, int TR, int HDV = HD>
 constexpr size_t mfma_lds_bytes()
 {
     constexpr size_t waves = kMfmaRound / TR;
-    constexpr size_t strip = 2 * (size_t)TR * (HD / 32 * 18) + 2 * (size_t)TR * (HD / 32) * 4;
+    constexpr size_t strip = (size_t)TR * (HD / 32 * 18) + (size_t)TR * (HDV / 32 * 18) + (size_t)TR * (HD / 32) * 4 + (size_t)TR * (HDV / 32) * 4;
     constexpr size_t qshare = (size_t)(HD / 32) * 64 * (16 + 4);                 // the shared q operands and sums
-    constexpr size_t fold = waves * 8 * HD * 4 + waves * 8 * 2 * 4;
-    return strip * waves + qshare > fold ? strip * waves + qshare : fold;
+    constexpr size_t fold = waves * 8 * HDV * 4 + waves * 8 * 2 * 4;
+    constexpr size_t qsum = (size_t)(HD / 32) * 64 * 4;
+    constexpr size_t front = HDV == HD ? strip * waves + qshare : strip * waves + qsum;   // (HDV < HD: the operands lie over the strips, the sums behind them)
+    return front > fold ? front : fold;
 }
 
 template <int HD, int GP, int NW>
@@ -1349,10 +1385,14 @@ int launch_bound(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
         if (own_parts) {
             p.balance = 0;
             p.mode = kModePart;
-            hipLaunchKernelGGL((sdpa_mfma_kernel<256, 32>), dim3(p.nwg, p.n_kv, n_slots), dim3(kMfmaRound / 32 * 64), (mfma_lds_bytes<256, 32>()), st, p);
+            if (hd == 512)   // two workgroups per kv head, each with half of the V dimensions
+                hipLaunchKernelGGL((sdpa_mfma_kernel<512, 32, 256>), dim3(p.nwg, p.n_kv * 2, n_slots), dim3(kMfmaRound / 32 * 64), (mfma_lds_bytes<512, 32, 256>()), st, p);
+            else
+                hipLaunchKernelGGL((sdpa_mfma_kernel<256, 32>), dim3(p.nwg, p.n_kv, n_slots), dim3(kMfmaRound / 32 * 64), (mfma_lds_bytes<256, 32>()), st, p);
             const hipError_t e0 = hipGetLastError();
             if (e0 != hipSuccess) return hip_fail(e0, "sdpa_batch (matrix-core form) launch");
-            hipLaunchKernelGGL(sdpa_records_merge_kernel<256>, dim3(p.n_q, n_slots), dim3(256), 0, st, p.tmp, p.out, p.n_q, p.nwg);
+            if (hd == 512) hipLaunchKernelGGL(sdpa_records_merge_kernel<512>, dim3(p.n_q, n_slots), dim3(512), 0, st, p.tmp, p.out, p.n_q, p.nwg);
+            else hipLaunchKernelGGL(sdpa_records_merge_kernel<256>, dim3(p.n_q, n_slots), dim3(256), 0, st, p.tmp, p.out, p.n_q, p.nwg);
             const hipError_t e1 = hipGetLastError();
             return e1 == hipSuccess ? 0 : hip_fail(e1, "sdpa_batch merge launch");
         }
@@ -1421,13 +1461,15 @@ int bind_sdpa_lanes(ksh_kernel &k, int nwg, int n_slots)
     // A chunk of more than 16 tokens: every token's partitions are workgroups of their own (grid = partitions x kv
     // heads x tokens), records in the reference's layout, merged by a second launch.  Its tokens attend dozens to
     // thousands of rows each, where the register form's ~200 vector instructions per row and wave are the whole
-    // cost (1024 tokens from an empty cache: 78 us against 422): the default there; vec = 3 asks for the register
-    // form, vec = 2 with up to 64 tokens for the form that deals the partitions by length.
-    const bool long_batch = k.desc.kind == KSH_SDPA_BATCH && hd == 256 && n_q / n_kv <= 8 && n_slots > 16;
+    // cost (1024 tokens from an empty cache: 78 us against 422; heads of 512: 226 against 778): the default there;
+    // vec = 3 asks for the register form, vec = 2 with up to 64 tokens for the form that deals the partitions by length.
+    const bool long_batch = k.desc.kind == KSH_SDPA_BATCH && (hd == 256 || hd == 512) && n_q / n_kv <= 8 && n_slots > 16;
     if (long_batch && ((k.desc.sched.vec == 2 && !batch_fits) || k.desc.sched.vec == 0)) {
         if (k.desc.sched.lds_tile && k.desc.sched.lds_tile != 32) return set_error("sdpa_batch: the matrix-core form of a long chunk takes tiles of 32 rows (lds_tile=%u)", k.desc.sched.lds_tile);
         k.scratch_bytes = (((size_t)n_slots * n_kv * 4 + 15) & ~(size_t)15) + (size_t)n_slots * 16;
-        set_launch(k, (uint32_t)nwg, (uint32_t)n_kv, (uint32_t)n_slots, kMfmaRound / 32 * 64, (uint32_t)mfma_lds_bytes<256, 32>());
+        // (heads of 512: two workgroups per kv head, each with all of the scores and half of the V dimensions)
+        set_launch(k, (uint32_t)nwg, (uint32_t)(hd == 512 ? 2 * n_kv : n_kv), (uint32_t)n_slots, kMfmaRound / 32 * 64,
+                   (uint32_t)(hd == 512 ? mfma_lds_bytes<512, 32, 256>() : mfma_lds_bytes<256, 32>()));
         k.info.sched = k.desc.sched;
         k.info.sched.vec = 2;
         k.info.sched.tg = kMfmaRound / 32 * 64;

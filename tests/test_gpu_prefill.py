@@ -99,14 +99,14 @@ def test_per_head_qkv_q40_batch(ctx, hd, n_q, n_kv):
 
 @pytest.mark.parametrize("hd,n_q,n_kv,sched", [(256, 8, 1, None), (128, 4, 1, None), (256, 4, 2, None), (64, 4, 2, None),
                                                (256, 8, 1, dict(vec=1)), (256, 8, 1, dict(vec=2)), (256, 4, 2, dict(vec=2)),
-                                               (256, 8, 1, dict(vec=3)), (256, 8, 1, dict(k_split=1))])
+                                               (256, 8, 1, dict(vec=3)), (256, 8, 1, dict(k_split=1)), (512, 8, 1, None), (512, 4, 2, dict(k_split=2))])
 @pytest.mark.parametrize("t,pos0,window", [(5, 0, 1 << 20), (33, 100, 1 << 20), (40, 150, 64), (130, 3, 1 << 20), (17, 290, 1 << 20)])
 def test_sdpa_batch_equals_the_serial_oracle(ctx, hd, n_q, n_kv, sched, t, pos0, window):
     """Token i of the chunk attends rows [start_i, pos0 + i] of the one cache: the same numbers as the single-token
     oracle attention with that range -- register form (vec=3; the default up to 16 tokens), tile form (vec=1 or other
-    head sizes), matrix-core forms (heads of 256: the default from 17 tokens on, one or several partitions per token
-    in workgroups of their own; vec=2 with up to 64 tokens deals the partitions by length), with and without a
-    sliding window."""
+    head sizes), matrix-core forms (heads of 256 and 512: the default from 17 tokens on, one or several partitions per
+    token in workgroups of their own, heads of 512 as two workgroups with half of the V dimensions each; vec=2 with
+    up to 64 tokens of 256-wide heads deals the partitions by length), with and without a sliding window."""
     max_t = 320
     row = n_kv * hd // 32 * 18
     kk, vv = synth.q40_blocks(max_t * n_kv * hd // 32, 710), synth.q40_blocks(max_t * n_kv * hd // 32, 711)
@@ -114,7 +114,7 @@ def test_sdpa_batch_equals_the_serial_oracle(ctx, hd, n_q, n_kv, sched, t, pos0,
     scale = 1.0 / np.sqrt(hd)
     k = ctx.compile(hip.make_desc(Kind.SDPA_BATCH, (n_q, n_kv, hd, max_t, t, 0), (DType.Q40, DType.F32), (scale,), sched))
     vec = (sched or {}).get("vec", 0)
-    assert ("mfma" in k.name) == (vec == 2 or (vec == 0 and hd == 256 and t > 16)), k.name
+    assert ("mfma" in k.name) == (vec == 2 or (vec == 0 and hd in (256, 512) and t > 16)), k.name
     nwg = k.info.sched.k_split
     if sched and sched.get("k_split"):
         assert nwg == sched["k_split"]

@@ -441,6 +441,9 @@ int bind_sdpa(ksh_kernel &k)
         int64_t nwg = d[5];
         if (n_tok <= 0 || n_tok > 4096) return set_error("sdpa_batch: n_tok=%lld", (long long)n_tok);
         if (nwg == 0 && k.desc.sched.k_split) nwg = k.desc.sched.k_split;
+        if (nwg == 0 && (hd == 256 || hd == 512) && n_q / n_kv <= 8 && n_tok > 16 && k.desc.sched.vec != 1 && k.desc.sched.vec != 3) {
+            nwg = 1;   // the matrix-core form of a chunk (one workgroup per token) is fastest with one partition per token
+        }
         if (nwg == 0) {
             // ~4 workgroups per compute unit over all tokens, at least 64 rows per partition, at most 16 partitions
             nwg = (1024 + n_tok * n_kv - 1) / (n_tok * n_kv);

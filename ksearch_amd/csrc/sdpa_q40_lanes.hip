@@ -905,11 +905,19 @@ __global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_m
         p1 = min(p0 + d.c, d.tlen);
         start = d.start;
     } else {
-        const int tlen = (int)p.meta[(size_t)slot * p.meta_stride];
+        int tlen;
+        if (p.kv_shared) {
+            // token `slot` of a prompt chunk (crates/ksearch_codegen/src/lower.rs:4961-4983): meta = {rows attended by token 0, -, window}
+            const int abs_t = (int)p.meta[0] + slot;
+            tlen = min(abs_t, (int)p.meta[2]);
+            start = abs_t - tlen;
+        } else {
+            tlen = (int)p.meta[(size_t)slot * p.meta_stride];
+            start = (int)p.meta[(size_t)slot * p.meta_stride + 1];
+        }
         const int chunk = ((tlen + nparts - 1) / nparts + TR - 1) / TR * TR;
         p0 = min(part * chunk, tlen);
         p1 = min(p0 + chunk, tlen);
-        start = (int)p.meta[(size_t)slot * p.meta_stride + 1];
     }
     const size_t slot_bytes = p.kv_shared ? 0 : p.slot_stride ? p.slot_stride : (size_t)p.max_t * p.n_kv * ROWB;
     const size_t row_stride = (size_t)p.n_kv * ROWB;
@@ -1212,6 +1220,8 @@ __global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_m
             float *ml = p.tmp + (size_t)gridDim.z * p.nwg * p.n_q * HD;
             p.tmp[r * HD + vhalf * HDV + d] = a;
             if (d == 0 && vhalf == 0) { ml[2 * r] = M; ml[2 * r + 1] = L; }
+        } else if (p.nwg == 1 && p.out) {
+            p.out[((size_t)slot * p.n_q + hq) * HD + vhalf * HDV + d] = a / L;      // one partition: nothing left to merge
         } else {
             float *rec = p.tmp + (size_t)slot * p.n_q * p.nwg * (HD + 2) + (size_t)hq * p.nwg * (HD + 2) + (size_t)part * (HD + 2);
             rec[2 + vhalf * HDV + d] = a;
@@ -1373,7 +1383,8 @@ int launch_bound(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
         // kernel into the handle's scratch (behind the counters); K and V are shared by all tokens.
         n_slots = (int)k.desc.dims[4];
         float *tok_meta = (float *)((uint8_t *)k.scratch + (((size_t)n_slots * p.n_kv * p.hsplit * 4 + 15) & ~(size_t)15));
-        hipLaunchKernelGGL(sdpa_batch_meta_kernel, dim3((n_slots + 255) / 256), dim3(256), 0, st, (const float *)a.in[3], tok_meta, n_slots);
+        // (the form with a workgroup per token works its token's record out itself)
+        if (!own_parts) hipLaunchKernelGGL(sdpa_batch_meta_kernel, dim3((n_slots + 255) / 256), dim3(256), 0, st, (const float *)a.in[3], tok_meta, n_slots);
         p.q = (const float *)a.in[0]; p.k = (const uint8_t *)a.in[1]; p.v = (const uint8_t *)a.in[2];
         p.meta = tok_meta;
         p.meta_stride = 4;
@@ -1383,6 +1394,7 @@ int launch_bound(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
         p.mode = kModeMerge;
         p.kv_shared = 1;
         if (own_parts) {
+            p.meta = (const float *)a.in[3];
             p.balance = 0;
             p.mode = kModePart;
             if (hd == 512)   // two workgroups per kv head, each with half of the V dimensions
@@ -1391,6 +1403,7 @@ int launch_bound(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
                 hipLaunchKernelGGL((sdpa_mfma_kernel<256, 32>), dim3(p.nwg, p.n_kv, n_slots), dim3(kMfmaRound / 32 * 64), (mfma_lds_bytes<256, 32>()), st, p);
             const hipError_t e0 = hipGetLastError();
             if (e0 != hipSuccess) return hip_fail(e0, "sdpa_batch (matrix-core form) launch");
+            if (p.nwg == 1) return 0;      // (the row launch has stored the finished heads)
             if (hd == 512) hipLaunchKernelGGL(sdpa_records_merge_kernel<512>, dim3(p.n_q, n_slots), dim3(512), 0, st, p.tmp, p.out, p.n_q, p.nwg);
             else hipLaunchKernelGGL(sdpa_records_merge_kernel<256>, dim3(p.n_q, n_slots), dim3(256), 0, st, p.tmp, p.out, p.n_q, p.nwg);
             const hipError_t e1 = hipGetLastError();

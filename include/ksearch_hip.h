@@ -63,6 +63,12 @@ enum ksh_kind {
      * dims[3], dims[4] (0 = none): rows of a second and a third matrix of the same dtype over the same X, taken in
      * the same launch (q | k | v of a prompt chunk: one preparation of X, one grid).  in: W, X, W1[, W2]
      * out: Y, Y1[batch, rows1][, Y2[batch, rows2]].
+     * dims[5] (F32 activations): the producer of the rows, run inside the preparation of X (params[0] = eps) --
+     *   1: X := rmsnorm(X, w)  (in: ..., w[cols]);  2: x_new := res + rmsnorm(X, w_post), X := rmsnorm(x_new, w_norm)
+     *   (in: ..., w_post[cols], res[batch, cols], w_norm[cols]; out: ..., x_new[batch, cols], which may be res);
+     *   3: X := gelu(X) * up  (in: ..., up[batch, cols]).  The norms take rows of a multiple of 512 up to 8192 columns.
+     *   These are the rows forms of RmsNormMatvec* / MatvecGateUpGelu's prologues (crates/ksearch_kernels/src/lib.rs:
+     *   1478-1560, gemma_prim.rs:1516-1538) folded into the GEMM that reads their result.
      * sched.nr0 = 32 | 128 picks the small-batch form (Q4_K, up to 64 tokens, one matrix) or the 128 x 128 tile;
      * sched.k_split = the tile's K slices (a divisor of cols / 256; 1 = whole rows; 0 = enough to fill the chip). */
     KSH_MATVEC_BATCH = 2,

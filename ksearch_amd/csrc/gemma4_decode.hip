@@ -423,6 +423,13 @@ int forward_prefill_chunk4(ksh_gemma4 *m, const uint32_t *tokens, int t)
                enc(m, kk, {w0, x, w1, w2}, {y0, y1, y2}, n);
     };
     const bool merged = tp > 32;
+    // ... with the rows' producers inside the GEMMs' preparations (dims[5]: the attention norm in q | k | v's,
+    // add-then-norm in gate | up's, gelu(gate) * up in the down projection's)
+    const bool inside = merged && h % 512 == 0 && h <= 8192;
+    auto mm_pro = [&](int dt, std::initializer_list<int64_t> dims, std::initializer_list<ksh_buf *> ins, std::initializer_list<ksh_buf *> outs) {
+        ksh_kernel *kk = nullptr;
+        return get(m, KSH_MATVEC_BATCH, dims, {dt, KSH_F32, KSH_F32}, {c.eps}, &kk) || enc(m, kk, ins, outs, n);
+    };
     if (get(m, KSH_COPY_SCALE_INDEXED, {h, c.vocab, t}, {m->g.dt_embd}, {std::sqrt((float)c.hidden)}, &k) ||
         enc(m, k, {m->g.token_embd, m->c_tok}, {m->c_x}, n))
         return 1;
@@ -448,8 +455,15 @@ int forward_prefill_chunk4(ksh_gemma4 *m, const uint32_t *tokens, int t)
         ksh_buf *kc = m->kv_k[P.src], *vc = m->kv_v[P.src];
         ksh_kernel *k_head = nullptr, *k_sdpa = nullptr, *k_gelu = nullptr;
         const bool qkv_merged = merged && P.owns && L.dt_q == L.dt_k && L.dt_q == L.dt_v;
-        if (enc(m, k_norm, {m->c_x, L.attn_norm}, {m->c_x2}, n)) return 1;
-        if (qkv_merged ? mm3(L.dt_q, P.qd, P.kvd, h, L.wq, L.wk, L.wv, m->c_x2, m->c_q, m->c_k, m->c_v) : mm(L.dt_q, P.qd, h, L.wq, m->c_x2, m->c_q)) return 1;
+        const bool q_inside = inside && (qkv_merged || !P.owns);
+        if (q_inside) {
+            if (qkv_merged ? mm_pro(L.dt_q, {P.qd, h, tp, P.kvd, P.kvd, 1}, {L.wq, m->c_x, L.wk, L.wv, L.attn_norm}, {m->c_q, m->c_k, m->c_v})
+                           : mm_pro(L.dt_q, {P.qd, h, tp, 0, 0, 1}, {L.wq, m->c_x, L.attn_norm}, {m->c_q}))
+                return 1;
+        } else {
+            if (enc(m, k_norm, {m->c_x, L.attn_norm}, {m->c_x2}, n)) return 1;
+            if (qkv_merged ? mm3(L.dt_q, P.qd, P.kvd, h, L.wq, L.wk, L.wv, m->c_x2, m->c_q, m->c_k, m->c_v) : mm(L.dt_q, P.qd, h, L.wq, m->c_x2, m->c_q)) return 1;
+        }
         if (P.owns) {
             if ((!qkv_merged && (mm(L.dt_k, P.kvd, h, L.wk, m->c_x2, m->c_k) || mm(L.dt_v, P.kvd, h, L.wv, m->c_x2, m->c_v))) ||
                 get(m, KSH_RMSNORM_PER_HEAD_QKV_Q40, {c.n_q, c.n_kv, P.hd, c.max_seq, t}, {}, {c.eps}, &k_head) ||
@@ -464,11 +478,15 @@ int forward_prefill_chunk4(ksh_gemma4 *m, const uint32_t *tokens, int t)
         if (get(m, KSH_SDPA_BATCH, {c.n_q, c.n_kv, P.hd, c.max_seq, t, t > 16 && (P.hd == 256 || P.hd == 512) && c.n_q / c.n_kv <= 8 ? 1 : kChunkPartitions4}, {KSH_Q40, KSH_F32}, {c.attn_scale}, &k_sdpa) ||
             enc(m, k_sdpa, {m->c_q, kc, vc, P.swa ? m->c_meta_swa : m->c_meta_full}, {m->c_tmp, m->c_o}, n) ||
             mm(L.dt_o, h, P.qd, L.wo, m->c_o, m->c_y) ||
-            enc(m, k_add_then, {m->c_y, L.post_attn_norm, m->c_x, L.ffn_norm}, {m->c_x, m->c_x2}, n) ||
-            (merged && L.dt_gate == L.dt_up ? mm2(L.dt_gate, L.ffn, h, L.wgate, L.wup, m->c_x2, m->c_g, m->c_u)
-                                            : (mm(L.dt_gate, L.ffn, h, L.wgate, m->c_x2, m->c_g) || mm(L.dt_up, L.ffn, h, L.wup, m->c_x2, m->c_u))) ||
-            get(m, KSH_GELU_MUL, {(int64_t)t * L.ffn}, {}, {}, &k_gelu) || enc(m, k_gelu, {m->c_g, m->c_u}, {m->c_ff}, n) ||
-            mm(L.dt_down, h, L.ffn, L.wdown, m->c_ff, m->c_y) || enc(m, k_add, {m->c_y, L.post_ffw_norm, m->c_x}, {m->c_x}, n))
+            (inside && L.dt_gate == L.dt_up
+                 ? mm_pro(L.dt_gate, {L.ffn, h, tp, L.ffn, 0, 2}, {L.wgate, m->c_y, L.wup, L.post_attn_norm, m->c_x, L.ffn_norm}, {m->c_g, m->c_u, m->c_x})
+                 : (enc(m, k_add_then, {m->c_y, L.post_attn_norm, m->c_x, L.ffn_norm}, {m->c_x, m->c_x2}, n) ||
+                    (merged && L.dt_gate == L.dt_up ? mm2(L.dt_gate, L.ffn, h, L.wgate, L.wup, m->c_x2, m->c_g, m->c_u)
+                                                    : (mm(L.dt_gate, L.ffn, h, L.wgate, m->c_x2, m->c_g) || mm(L.dt_up, L.ffn, h, L.wup, m->c_x2, m->c_u))))) ||
+            (inside ? mm_pro(L.dt_down, {h, L.ffn, tp, 0, 0, 3}, {L.wdown, m->c_g, m->c_u}, {m->c_y})
+                    : (get(m, KSH_GELU_MUL, {(int64_t)t * L.ffn}, {}, {}, &k_gelu) || enc(m, k_gelu, {m->c_g, m->c_u}, {m->c_ff}, n) ||
+                       mm(L.dt_down, h, L.ffn, L.wdown, m->c_ff, m->c_y))) ||
+            enc(m, k_add, {m->c_y, L.post_ffw_norm, m->c_x}, {m->c_x}, n))
             return 1;
         if (c.ple_dim > 0) {
             // gemma_prim.rs:1558-1600: u = gelu(Wg x) * ctx_l; x = (x + rms(Wp u) * post_norm) * layer_scale

@@ -408,10 +408,15 @@ int forward_prefill_chunk(ksh_gemma *m, const uint32_t *tokens, int t)
     ksh_kernel *k_embed, *k_norm, *k_mm_q, *k_mm_kv, *k_head, *k_sdpa, *k_mm_o, *k_add_then, *k_mm_ff, *k_gelu, *k_mm_down, *k_add;
     // beyond the small-batch form's 64 tokens q | k | v are one launch of the 128 x 128 tile over one preparation of x
     // (and gate | up likewise)
-    ksh_kernel *k_mm_qkv = nullptr, *k_mm_gu = nullptr;
-    if (tp > 32 && (get(m, KSH_MATVEC_BATCH, {qd, c.hidden, tp, kvd, kvd}, {KSH_Q4K, KSH_F32, KSH_F32}, {}, &k_mm_qkv) ||
-                    get(m, KSH_MATVEC_BATCH, {c.ffn, c.hidden, tp, c.ffn}, {KSH_Q4K, KSH_F32, KSH_F32}, {}, &k_mm_gu)))
+    // with the rows' producers inside the GEMMs' preparations: the attention norm in q | k | v's, add-then-norm in
+    // gate | up's (which also stores the new residual rows), gelu(gate) * up in the down projection's
+    ksh_kernel *k_mm_qkv = nullptr, *k_mm_gu = nullptr, *k_mm_down_g = nullptr;
+    const bool norms_inside = c.hidden % 512 == 0 && c.hidden <= 8192 && c.ffn <= 8192;
+    if (tp > 32 && (get(m, KSH_MATVEC_BATCH, {qd, c.hidden, tp, kvd, kvd, norms_inside ? 1 : 0}, {KSH_Q4K, KSH_F32, KSH_F32}, {c.eps}, &k_mm_qkv) ||
+                    get(m, KSH_MATVEC_BATCH, {c.ffn, c.hidden, tp, c.ffn, 0, norms_inside ? 2 : 0}, {KSH_Q4K, KSH_F32, KSH_F32}, {c.eps}, &k_mm_gu) ||
+                    (norms_inside && get(m, KSH_MATVEC_BATCH, {c.hidden, c.ffn, tp, 0, 0, 3}, {KSH_Q4K, KSH_F32, KSH_F32}, {c.eps}, &k_mm_down_g))))
         return 1;
+    const bool fused = k_mm_qkv && norms_inside;
     const float embed_scale = std::sqrt((float)c.hidden);
     if (get(m, KSH_COPY_SCALE_INDEXED, {c.hidden, c.vocab, t}, {KSH_Q6K}, {embed_scale}, &k_embed) ||
         get(m, KSH_RMSNORM, {c.hidden, 0, 0, t}, {}, {c.eps}, &k_norm) ||
@@ -435,17 +440,19 @@ int forward_prefill_chunk(ksh_gemma *m, const uint32_t *tokens, int t)
     if (enc(m, k_embed, {m->embd, m->c_tok}, {m->c_x}, n)) return 1;
     for (int l = 0; l < c.n_layers; l++) {
         const ksh_gemma_layer &L = m->layers[l];
-        if (enc(m, k_norm, {m->c_x, L.attn_norm}, {m->c_x2}, n) ||
-            (k_mm_qkv ? enc(m, k_mm_qkv, {L.wq, m->c_x2, L.wk, L.wv}, {m->c_q, m->c_k, m->c_v}, n)
+        if ((fused ? enc(m, k_mm_qkv, {L.wq, m->c_x, L.wk, L.wv, L.attn_norm}, {m->c_q, m->c_k, m->c_v}, n) : enc(m, k_norm, {m->c_x, L.attn_norm}, {m->c_x2}, n)) ||
+            (fused ? 0 : k_mm_qkv ? enc(m, k_mm_qkv, {L.wq, m->c_x2, L.wk, L.wv}, {m->c_q, m->c_k, m->c_v}, n)
                       : (enc(m, k_mm_q, {L.wq, m->c_x2}, {m->c_q}, n) || enc(m, k_mm_kv, {L.wk, m->c_x2}, {m->c_k}, n) ||
                          enc(m, k_mm_kv, {L.wv, m->c_x2}, {m->c_v}, n))) ||
             enc(m, k_head, {m->c_q, L.q_norm, m->rope, m->c_k, L.k_norm, m->c_v, m->meta}, {m->c_q, m->kv_k[l], m->kv_v[l]}, n) ||
             enc(m, k_sdpa, {m->c_q, m->kv_k[l], m->kv_v[l], m->c_meta}, {m->c_tmp, m->c_o}, n) ||
             enc(m, k_mm_o, {L.wo, m->c_o}, {m->c_y}, n) ||
-            enc(m, k_add_then, {m->c_y, L.post_attn_norm, m->c_x, L.ffn_norm}, {m->c_x, m->c_x2}, n) ||
-            (k_mm_gu ? enc(m, k_mm_gu, {L.wgate, m->c_x2, L.wup}, {m->c_g, m->c_u}, n)
-                     : (enc(m, k_mm_ff, {L.wgate, m->c_x2}, {m->c_g}, n) || enc(m, k_mm_ff, {L.wup, m->c_x2}, {m->c_u}, n))) ||
-            enc(m, k_gelu, {m->c_g, m->c_u}, {m->c_ff}, n) || enc(m, k_mm_down, {L.wdown, m->c_ff}, {m->c_y}, n) ||
+            (fused ? enc(m, k_mm_gu, {L.wgate, m->c_y, L.wup, L.post_attn_norm, m->c_x, L.ffn_norm}, {m->c_g, m->c_u, m->c_x}, n)
+                   : (enc(m, k_add_then, {m->c_y, L.post_attn_norm, m->c_x, L.ffn_norm}, {m->c_x, m->c_x2}, n) ||
+                      (k_mm_gu ? enc(m, k_mm_gu, {L.wgate, m->c_x2, L.wup}, {m->c_g, m->c_u}, n)
+                               : (enc(m, k_mm_ff, {L.wgate, m->c_x2}, {m->c_g}, n) || enc(m, k_mm_ff, {L.wup, m->c_x2}, {m->c_u}, n))))) ||
+            (fused ? enc(m, k_mm_down_g, {L.wdown, m->c_g, m->c_u}, {m->c_y}, n)
+                   : (enc(m, k_gelu, {m->c_g, m->c_u}, {m->c_ff}, n) || enc(m, k_mm_down, {L.wdown, m->c_ff}, {m->c_y}, n))) ||
             enc(m, k_add, {m->c_y, L.post_ffw_norm, m->c_x}, {m->c_x}, n))
             return 1;
     }

@@ -138,6 +138,109 @@ __global__ __launch_bounds__(256) void mm_prep_x_f32_kernel(const float *__restr
     }
 }
 
+// The same preparation with the producer of the rows folded in (f32 activations), one workgroup per row, cols / 8
+// threads with 8 consecutive elements each:
+//   MODE 1  x = rmsnorm(X, w)                                  (rmsnorm_rows, crates/ksearch_kernels/src/lib.rs:1478-1500)
+//   MODE 2  x_new = res + rmsnorm(X, w_post), stored; x = rmsnorm(x_new, w_norm)   (rmsnorm_add_then_rmsnorm_rows)
+//   MODE 3  x = gelu(X) * up                                   (gelu_mul on rows, gemma_prim.rs:1516-1538)
+// in the operation order of the kernels that do these alone (every product and sum rounded by itself).
+template <int MODE>
+__global__ __launch_bounds__(1024) void mm_prep_rows_kernel(const float *__restrict__ X, const float *__restrict__ P0, const float *P1,
+                                                             const float *__restrict__ P2, float *x_out, _Float16 *__restrict__ Xf_hi,
+                                                             _Float16 *__restrict__ Xf_lo, _Float16 *__restrict__ SxA_hi,
+                                                             _Float16 *__restrict__ SxA_lo, int cols, float eps)
+{
+    __shared__ float red[2][16];
+    const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    // (the norms run with cols / 8 threads, one trip; gelu * up of longer rows takes several)
+    for (int j = threadIdx.x; j < cols / 8; j += blockDim.x) {
+    const size_t e0 = (size_t)t * cols + 8 * (size_t)j;
+    auto ld8 = [](const float *p, float (&v)[8]) __attribute__((always_inline)) {
+        const f32x4_t a = reinterpret_cast<const f32x4_t *>(p)[0], b = reinterpret_cast<const f32x4_t *>(p)[1];
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    };
+    auto row_sum = [&](float v, int which) __attribute__((always_inline)) {
+        v = wave_sum(v);
+        if (lane == 0) red[which][wave] = v;
+        __syncthreads();
+        float s = 0.f;
+        for (int i = 0; i < nw; i++) s += red[which][i];
+        return s;
+    };
+    float f[8];
+    ld8(X + e0, f);
+    if (MODE == 1 || MODE == 2) {
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) ss += f[i] * f[i];
+        const float inv = 1.0f / sqrtf(row_sum(ss, 0) / (float)cols + eps);
+        float w[8];
+        ld8(P0 + 8 * j, w);
+#pragma unroll
+        for (int i = 0; i < 8; i++) f[i] = __fmul_rn(__fmul_rn(f[i], inv), w[i]);
+        if (MODE == 2) {
+            float r[8], wn[8];
+            ld8(P1 + e0, r);
+            float ss2 = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                f[i] = __fadd_rn(r[i], f[i]);
+                ss2 += f[i] * f[i];
+            }
+            reinterpret_cast<f32x4_t *>(x_out + e0)[0] = f32x4_t{f[0], f[1], f[2], f[3]};
+            reinterpret_cast<f32x4_t *>(x_out + e0)[1] = f32x4_t{f[4], f[5], f[6], f[7]};
+            const float inv2 = 1.0f / sqrtf(row_sum(ss2, 1) / (float)cols + eps);
+            ld8(P2 + 8 * j, wn);
+#pragma unroll
+            for (int i = 0; i < 8; i++) f[i] = __fmul_rn(__fmul_rn(f[i], inv2), wn[i]);
+        }
+    }
+    if (MODE == 3) {
+        float u[8];
+        ld8(P0 + e0, u);
+#pragma unroll
+        for (int i = 0; i < 8; i++) f[i] = gelu_mul_f32(f[i], u[i]);
+    }
+    h8 oh, ol;
+    float fh[8], fl[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const float x = pinned(f[i]);
+        const _Float16 hi = (_Float16)x;
+        const _Float16 lo = (_Float16)((x - (float)hi) * 2048.0f);
+        oh[kperm(i)] = hi;
+        ol[kperm(i)] = lo;
+        fh[i] = (float)hi;
+        fl[i] = (float)lo;
+    }
+    float sh = ((fh[0] + fh[1]) + (fh[2] + fh[3])) + ((fh[4] + fh[5]) + (fh[6] + fh[7]));
+    float sl = ((fl[0] + fl[1]) + (fl[2] + fl[3])) + ((fl[4] + fl[5]) + (fl[6] + fl[7]));
+    sh += dpp_f32<0xB1>(sh);
+    sh += dpp_f32<0x4E>(sh);
+    sl += dpp_f32<0xB1>(sl);
+    sl += dpp_f32<0x4E>(sl);
+    const size_t frag = ((size_t)(t >> 5) * (cols / 16) + (j >> 1)) * 64 + (t & 31) + 32 * (j & 1);
+    reinterpret_cast<h8 *>(Xf_hi)[frag] = oh;
+    reinterpret_cast<h8 *>(Xf_lo)[frag] = ol;
+    if ((threadIdx.x & 3) == 0) {
+        const int s = j / 4, jj = s % 8;
+        const size_t o = ((size_t)t * (cols / 256) + s / 8) * 32;
+        const float sums[2] = {sh, sl};
+        _Float16 *dst[2] = {SxA_hi + o, SxA_lo + o};
+#pragma unroll
+        for (int part = 0; part < 2; part++) {
+            const float sum = pinned(sums[part]);
+            const _Float16 hi = (_Float16)sum;
+            const _Float16 lo = (_Float16)(sum - (float)hi);
+            dst[part][jj] = hi;
+            dst[part][8 + jj] = hi;
+            dst[part][16 + jj] = lo;
+            dst[part][24 + jj] = (_Float16)0.f;
+        }
+    }
+    }
+}
+
 struct MmParams {
     const uint8_t *W;
     const _Float16 *Xf, *SxA;   // fragment-ordered f16 activations (mm_prep_x_kernel), sums of x
@@ -1205,7 +1308,20 @@ int launch_mul_mm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
     _Float16 *SxA = Xf + xf_halves;
     _Float16 *Xf_lo = SxA + sx_halves, *SxA_lo = Xf_lo + xf_halves;     // f32 activations only
     const int n = batch * (cols / 8);
-    if (f32x) hipLaunchKernelGGL(mm_prep_x_f32_kernel, dim3((n + 255) / 256), dim3(256), 0, st, (const float *)a.in[1], Xf, Xf_lo, SxA, SxA_lo, batch, cols);
+    const int n_mat0 = 1 + (k.desc.dims[3] > 0) + (k.desc.dims[4] > 0), prologue = (int)k.desc.dims[5];
+    if (prologue) {
+        // the rows' producer runs inside the preparation: in = W, X, [W1, W2,] then the prologue's operands
+        const float *X = (const float *)a.in[1], *q0 = (const float *)a.in[1 + n_mat0];
+        const dim3 pg((unsigned)batch), pb((unsigned)std::min(cols / 8, 1024));
+        const float eps = k.desc.params[0];
+        if (prologue == 1)
+            hipLaunchKernelGGL(mm_prep_rows_kernel<1>, pg, pb, 0, st, X, q0, nullptr, nullptr, nullptr, Xf, Xf_lo, SxA, SxA_lo, cols, eps);
+        else if (prologue == 2)
+            hipLaunchKernelGGL(mm_prep_rows_kernel<2>, pg, pb, 0, st, X, q0, (const float *)a.in[2 + n_mat0], (const float *)a.in[3 + n_mat0], (float *)a.out[n_mat0],
+                               Xf, Xf_lo, SxA, SxA_lo, cols, eps);
+        else
+            hipLaunchKernelGGL(mm_prep_rows_kernel<3>, pg, pb, 0, st, X, q0, nullptr, nullptr, nullptr, Xf, Xf_lo, SxA, SxA_lo, cols, eps);
+    } else if (f32x) hipLaunchKernelGGL(mm_prep_x_f32_kernel, dim3((n + 255) / 256), dim3(256), 0, st, (const float *)a.in[1], Xf, Xf_lo, SxA, SxA_lo, batch, cols);
     else hipLaunchKernelGGL(mm_prep_x_kernel, dim3((n + 255) / 256), dim3(256), 0, st, (const uint16_t *)a.in[1], Xf, SxA, batch, cols);
     MmParams p;
     p.W = (const uint8_t *)a.in[0];
@@ -1282,6 +1398,23 @@ int bind_matvec_batch(ksh_kernel &k)
     k.out_bytes[0] = (size_t)batch * rows * 4; k.out_align[0] = 4;
     if (rows1) { k.in_bytes[2] = (size_t)rows1 * row_bytes; k.in_align[2] = k.in_align[0]; k.out_bytes[1] = (size_t)batch * rows1 * 4; k.out_align[1] = 4; }
     if (rows2) { k.in_bytes[3] = (size_t)rows2 * row_bytes; k.in_align[3] = k.in_align[0]; k.out_bytes[2] = (size_t)batch * rows2 * 4; k.out_align[2] = 4; }
+    // dims[5]: the producer of the rows, run inside the preparation of f32 activations (params[0] = eps):
+    //   1 rmsnorm(X, w)                 in: ..., w[cols]
+    //   2 add then norm                 in: ..., w_post[cols], res[batch, cols], w_norm[cols]   out: ..., x_new[batch, cols] (may be res)
+    //   3 gelu(X) * up                  in: ..., up[batch, cols]
+    const int64_t prologue = k.desc.dims[5];
+    if (prologue < 0 || prologue > 3) return set_error("matvec_batch: prologue %lld (0 none, 1 rmsnorm, 2 add then norm, 3 gelu * up)", (long long)prologue);
+    if (prologue) {
+        if (!f32x) return set_error("matvec_batch: a prologue takes F32 activations");
+        if (prologue != 3 && (cols > 8192 || cols % 512)) return set_error("matvec_batch: a norm prologue takes rows of a multiple of 512 up to 8192 columns, got %lld", (long long)cols);
+        int ni = 1 + n_mat;
+        const size_t vec = (size_t)cols * 4, mat = (size_t)batch * cols * 4;
+        auto add_in = [&](size_t bytes) { k.in_bytes[ni] = bytes; k.in_align[ni] = 16; ni++; };
+        if (prologue == 1) add_in(vec);
+        if (prologue == 2) { add_in(vec); add_in(mat); add_in(vec); k.out_bytes[n_mat] = mat; k.out_align[n_mat] = 16; k.info.n_outputs = n_mat + 1; }
+        if (prologue == 3) add_in(mat);
+        k.info.n_inputs = ni;
+    }
     // f16 copy of X plus the min-term operand (32 halves per token and superblock)
     k.scratch_bytes = ((size_t)((batch + 31) / 32 * 32) * cols * 2 + (size_t)batch * (cols / 256) * 64) * (f32x ? 2 : 1);
     // schedule: nr0 = weight rows per workgroup.  32 = the small-batch form (Q4_K, up to 64 tokens: the default
@@ -1322,7 +1455,8 @@ int bind_matvec_batch(ksh_kernel &k)
     set_launch(k, (uint32_t)((batch + BM - 1) / BM), (uint32_t)row_tiles, z_form ? (uint32_t)(ks * parts) : 1, kThreadsMM,
                (uint32_t)kLdsBytes);
     k.info.sched.tg = kThreadsMM; k.info.sched.nsg = kThreadsMM / 64; k.info.sched.nr0 = BN; k.info.sched.k_split = (uint32_t)ks; k.info.sched.lds_tile = KS;
-    set_name(k, "mul_mm_%s_%dx%dx%d%s%s%s", q6 ? "q6k" : "q4k", BM, BN, KS, f32x ? "_f32x" : "", z_form ? "_kz" : "", n_mat == 3 ? "_x3" : n_mat == 2 ? "_x2" : "");
+    set_name(k, "mul_mm_%s_%dx%dx%d%s%s%s%s", q6 ? "q6k" : "q4k", BM, BN, KS, f32x ? "_f32x" : "", z_form ? "_kz" : "", n_mat == 3 ? "_x3" : n_mat == 2 ? "_x2" : "",
+             prologue == 1 ? "_rms" : prologue == 2 ? "_addrms" : prologue == 3 ? "_gelu" : "");
     k.launch = launch_mul_mm;
     return 0;
 }

@@ -211,6 +211,46 @@ def test_mul_mm_matrices_sharing_the_activations(ctx, xdt, batch, rows3, cols):
         assert_close(got, ctx.read_f32(y1, batch * r).reshape(batch, r), 2e-6, f"matrix {i} against its own launch")
 
 
+@pytest.mark.parametrize("mode,batch,rows3,cols", [(1, 200, (384, 128, 128), 1536), (2, 96, (512, 512, 0), 2048), (3, 130, (256, 0, 0), 8192),
+                                                   (1, 40, (300, 0, 0), 512), (2, 1056, (256, 0, 0), 512), (3, 70, (128, 0, 0), 12288)])
+def test_mul_mm_with_the_rows_producer_inside(ctx, mode, batch, rows3, cols):
+    """dims[5]: the producer of the rows runs inside the GEMM's preparation -- 1: rmsnorm(X, w); 2: x_new = res +
+    rmsnorm(X, w_post) (stored, in place over res) and then rmsnorm(x_new, w_norm); 3: gelu(X) * up.  The rows the
+    GEMM sees are the oracle's ops' results, the products against float64 at 2e-5; one to three
+    matrices, K slices and whole rows, the small-batch form (40 tokens).  (x_new itself at 1e-5: its row sums are added
+    in another order than the oracle's.)"""
+    eps = 1e-6
+    ws = [synth.q4k_blocks(r * cols // 256, 670 + i) for i, r in enumerate(rows3) if r]
+    x = synth.normal_f32(batch * cols, 673).reshape(batch, cols)
+    x[1] *= 40.0
+    w0, w1 = 1.0 + 0.2 * synth.normal_f32(cols, 674), 1.0 + 0.2 * synth.normal_f32(cols, 675)
+    res = synth.normal_f32(batch * cols, 676).reshape(batch, cols)
+    up = synth.normal_f32(batch * cols, 677).reshape(batch, cols)
+    bws = [ctx.buffer_bytes(w) for w in ws]
+    ins, outs = [bws[0], ctx.buffer_f32(x)] + bws[1:], [ctx.buffer_empty_f32(batch * r) for r in rows3 if r]
+    if mode == 1:
+        ins.append(ctx.buffer_f32(w0))
+        rows_in = np.stack([oracle.rmsnorm(x[t], w0, eps) for t in range(batch)])
+    elif mode == 2:
+        bres = ctx.buffer_f32(res)
+        ins += [ctx.buffer_f32(w0), bres, ctx.buffer_f32(w1)]
+        outs.append(bres)                                     # the new residual rows replace the old ones
+        pairs = [oracle.rmsnorm_add_then_rmsnorm(x[t], w0, res[t], w1, eps) for t in range(batch)]
+        x_new, rows_in = np.stack([p[0] for p in pairs]), np.stack([p[1] for p in pairs])
+    else:
+        ins.append(ctx.buffer_f32(up))
+        rows_in = np.stack([oracle.gelu_mul(x[t], up[t]) for t in range(batch)])
+    k = ctx.compile(hip.make_desc(hip.Kind.MATVEC_BATCH, (rows3[0], cols, batch, rows3[1], rows3[2], mode), (DType.Q4K, DType.F32, DType.F32), (eps,)))
+    ctx.encode_multi(k, ins, outs)
+    ctx.synchronize()
+    if mode == 2:
+        assert_close(ctx.read_f32(bres, batch * cols).reshape(batch, cols), x_new, 1e-5, "new residual rows")
+    for i, (w, r) in enumerate(zip(ws, [r for r in rows3 if r])):
+        got = ctx.read_f32(outs[i], batch * r).reshape(batch, r)
+        worst = max(float(rel_err(got[t], oracle.matvec_f64(oracle.Q4K, w, r, cols, rows_in[t])).max()) for t in range(0, batch, 13))
+        assert worst <= 2e-5, (k.name, i, worst)
+
+
 def test_mul_mm_k_slices_must_divide_the_row(ctx):
     with pytest.raises(hip.KshError, match="does not divide"):
         ctx.compile(hip.make_desc(hip.Kind.MATVEC_BATCH, (256, 2048, 100), (DType.Q4K, DType.BF16, DType.F32), (), dict(k_split=3)))

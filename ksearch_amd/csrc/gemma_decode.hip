@@ -417,6 +417,10 @@ int forward_prefill_chunk(ksh_gemma *m, const uint32_t *tokens, int t)
                     (norms_inside && get(m, KSH_MATVEC_BATCH, {c.hidden, c.ffn, tp, 0, 0, 3}, {KSH_Q4K, KSH_F32, KSH_F32}, {c.eps}, &k_mm_down_g))))
         return 1;
     const bool fused = k_mm_qkv && norms_inside;
+    // ... and a layer's closing norm + add with the next layer's attention norm are one add-then-norm, in that
+    // layer's q | k | v preparation (the residual rows it stores are the closed layer's)
+    ksh_kernel *k_mm_qkv_close = nullptr;
+    if (fused && c.n_layers > 1 && get(m, KSH_MATVEC_BATCH, {qd, c.hidden, tp, kvd, kvd, 2}, {KSH_Q4K, KSH_F32, KSH_F32}, {c.eps}, &k_mm_qkv_close)) return 1;
     const float embed_scale = std::sqrt((float)c.hidden);
     if (get(m, KSH_COPY_SCALE_INDEXED, {c.hidden, c.vocab, t}, {KSH_Q6K}, {embed_scale}, &k_embed) ||
         get(m, KSH_RMSNORM, {c.hidden, 0, 0, t}, {}, {c.eps}, &k_norm) ||
@@ -440,7 +444,9 @@ int forward_prefill_chunk(ksh_gemma *m, const uint32_t *tokens, int t)
     if (enc(m, k_embed, {m->embd, m->c_tok}, {m->c_x}, n)) return 1;
     for (int l = 0; l < c.n_layers; l++) {
         const ksh_gemma_layer &L = m->layers[l];
-        if ((fused ? enc(m, k_mm_qkv, {L.wq, m->c_x, L.wk, L.wv, L.attn_norm}, {m->c_q, m->c_k, m->c_v}, n) : enc(m, k_norm, {m->c_x, L.attn_norm}, {m->c_x2}, n)) ||
+        if ((fused ? (l > 0 ? enc(m, k_mm_qkv_close, {L.wq, m->c_y, L.wk, L.wv, m->layers[l - 1].post_ffw_norm, m->c_x, L.attn_norm}, {m->c_q, m->c_k, m->c_v, m->c_x}, n)
+                            : enc(m, k_mm_qkv, {L.wq, m->c_x, L.wk, L.wv, L.attn_norm}, {m->c_q, m->c_k, m->c_v}, n))
+                   : enc(m, k_norm, {m->c_x, L.attn_norm}, {m->c_x2}, n)) ||
             (fused ? 0 : k_mm_qkv ? enc(m, k_mm_qkv, {L.wq, m->c_x2, L.wk, L.wv}, {m->c_q, m->c_k, m->c_v}, n)
                       : (enc(m, k_mm_q, {L.wq, m->c_x2}, {m->c_q}, n) || enc(m, k_mm_kv, {L.wk, m->c_x2}, {m->c_k}, n) ||
                          enc(m, k_mm_kv, {L.wv, m->c_x2}, {m->c_v}, n))) ||
@@ -453,7 +459,7 @@ int forward_prefill_chunk(ksh_gemma *m, const uint32_t *tokens, int t)
                                : (enc(m, k_mm_ff, {L.wgate, m->c_x2}, {m->c_g}, n) || enc(m, k_mm_ff, {L.wup, m->c_x2}, {m->c_u}, n))))) ||
             (fused ? enc(m, k_mm_down_g, {L.wdown, m->c_g, m->c_u}, {m->c_y}, n)
                    : (enc(m, k_gelu, {m->c_g, m->c_u}, {m->c_ff}, n) || enc(m, k_mm_down, {L.wdown, m->c_ff}, {m->c_y}, n))) ||
-            enc(m, k_add, {m->c_y, L.post_ffw_norm, m->c_x}, {m->c_x}, n))
+            ((!fused || l == c.n_layers - 1) && enc(m, k_add, {m->c_y, L.post_ffw_norm, m->c_x}, {m->c_x}, n)))
             return 1;
     }
     hipLaunchKernelGGL(chunk_end_kernel, dim3(1), dim3(64), 0, st, (float *)ksh_buffer_device_ptr(m->meta), t, c.max_seq,

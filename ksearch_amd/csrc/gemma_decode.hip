@@ -124,7 +124,8 @@ struct ksh_gemma {
     std::vector<float> rope0;   // row 0 of the rope table, for reset
     // prompt chunks (allocated at the first chunk): [kChunk, .] activations of the batched layer pass
     ksh_buf *c_tok = nullptr, *c_x = nullptr, *c_x2 = nullptr, *c_y = nullptr, *c_q = nullptr, *c_k = nullptr, *c_v = nullptr, *c_o = nullptr,
-            *c_g = nullptr, *c_u = nullptr, *c_ff = nullptr, *c_tmp = nullptr, *c_meta = nullptr;
+            *c_g = nullptr, *c_u = nullptr, *c_ff = nullptr, *c_tmp = nullptr, *c_meta = nullptr,
+            *c_po = nullptr, *c_pg = nullptr, *c_pd = nullptr;   // unfolded partial sums of the o, gate | up and down projections
     int c_nwg = 0;
     // the decode chain (decode_chain.hip): o-projection, feed-forward and the next layer's QKV as one launch per layer
     bool use_chain = false;
@@ -378,6 +379,7 @@ int run_token(ksh_gemma *m, bool want_logits, bool use_graph)
 
 // prefill_chunk's chunk length (gemma_prim.rs:16)
 constexpr int kChunk = 1024;
+constexpr int kPartsRows = 4;          // room for the unfolded partial sums of a hidden-wide projection: this many chunks of rows
 constexpr int kChunkPartitions = 8;   // partitions per token of the batched attention (its tmp buffer is sized for this)
 
 int chunk_buffers(ksh_gemma *m)
@@ -390,7 +392,8 @@ int chunk_buffers(ksh_gemma *m)
            alloc(m, T * c.hidden * 4, &m->c_y) || alloc(m, T * qd * 4, &m->c_q) || alloc(m, T * kvd * 4, &m->c_k) ||
            alloc(m, T * kvd * 4, &m->c_v) || alloc(m, T * qd * 4, &m->c_o) || alloc(m, T * c.ffn * 4, &m->c_g) ||
            alloc(m, T * c.ffn * 4, &m->c_u) || alloc(m, T * c.ffn * 4, &m->c_ff) ||
-           alloc(m, T * c.n_q * m->c_nwg * (c.hd + 2) * 4, &m->c_tmp) || alloc(m, 16, &m->c_meta);
+           alloc(m, T * c.n_q * m->c_nwg * (c.hd + 2) * 4, &m->c_tmp) || alloc(m, 16, &m->c_meta) ||
+           alloc(m, kPartsRows * T * c.hidden * 4, &m->c_po) || alloc(m, 2 * T * 2 * c.ffn * 4, &m->c_pg) || alloc(m, kPartsRows * T * c.hidden * 4, &m->c_pd);
 }
 
 // forward_prefill_chunk (gemma_prim.rs:1317-1607) for 2 <= t <= kChunk tokens already validated: the layer as
@@ -417,6 +420,22 @@ int forward_prefill_chunk(ksh_gemma *m, const uint32_t *tokens, int t)
                     (norms_inside && get(m, KSH_MATVEC_BATCH, {c.hidden, c.ffn, tp, 0, 0, 3}, {KSH_Q4K, KSH_F32, KSH_F32}, {c.eps}, &k_mm_down_g))))
         return 1;
     const bool fused = k_mm_qkv && norms_inside;
+    // ... and the o, gate | up and down projections leave their K slices' partial sums unfolded for the preparation
+    // that reads them (dims[6], dims[7]): no fold launches but q | k | v's, whose reader is not a GEMM
+    ksh_kernel *u_o = nullptr, *u_gu = nullptr, *u_down = nullptr, *u_down_last = nullptr, *u_qkv = nullptr;
+    bool travel = false;
+    if (fused && c.n_layers > 1) {
+        const size_t T = kChunk;
+        auto parts_of = [](ksh_kernel *kk) { return (int64_t)(kk->info.sched.k_split | 2u << 8); };
+        if (get(m, KSH_MATVEC_BATCH, {c.hidden, qd, tp, 0, 0, 0, 1}, {KSH_Q4K, KSH_F32, KSH_F32}, {c.eps}, &u_o) ||
+            get(m, KSH_MATVEC_BATCH, {c.ffn, c.hidden, tp, c.ffn, 0, 2, 1, parts_of(u_o)}, {KSH_Q4K, KSH_F32, KSH_F32}, {c.eps}, &u_gu) ||
+            get(m, KSH_MATVEC_BATCH, {c.hidden, c.ffn, tp, 0, 0, 3, 1, parts_of(u_gu)}, {KSH_Q4K, KSH_F32, KSH_F32}, {c.eps}, &u_down) ||
+            get(m, KSH_MATVEC_BATCH, {c.hidden, c.ffn, tp, 0, 0, 3, 0, parts_of(u_gu)}, {KSH_Q4K, KSH_F32, KSH_F32}, {c.eps}, &u_down_last) ||
+            get(m, KSH_MATVEC_BATCH, {qd, c.hidden, tp, kvd, kvd, 2, 0, parts_of(u_down)}, {KSH_Q4K, KSH_F32, KSH_F32}, {c.eps}, &u_qkv))
+            return 1;
+        travel = u_o->out_bytes[0] <= kPartsRows * T * c.hidden * 4 && u_gu->out_bytes[0] <= 2 * T * 2 * c.ffn * 4 &&
+                 u_down->out_bytes[0] <= kPartsRows * T * c.hidden * 4;
+    }
     // ... and a layer's closing norm + add with the next layer's attention norm are one add-then-norm, in that
     // layer's q | k | v preparation (the residual rows it stores are the closed layer's)
     ksh_kernel *k_mm_qkv_close = nullptr;
@@ -444,6 +463,19 @@ int forward_prefill_chunk(ksh_gemma *m, const uint32_t *tokens, int t)
     if (enc(m, k_embed, {m->embd, m->c_tok}, {m->c_x}, n)) return 1;
     for (int l = 0; l < c.n_layers; l++) {
         const ksh_gemma_layer &L = m->layers[l];
+        if (travel) {
+            const bool last = l == c.n_layers - 1;
+            if ((l > 0 ? enc(m, u_qkv, {L.wq, m->c_pd, L.wk, L.wv, m->layers[l - 1].post_ffw_norm, m->c_x, L.attn_norm}, {m->c_q, m->c_k, m->c_v, m->c_x}, n)
+                       : enc(m, k_mm_qkv, {L.wq, m->c_x, L.wk, L.wv, L.attn_norm}, {m->c_q, m->c_k, m->c_v}, n)) ||
+                enc(m, k_head, {m->c_q, L.q_norm, m->rope, m->c_k, L.k_norm, m->c_v, m->meta}, {m->c_q, m->kv_k[l], m->kv_v[l]}, n) ||
+                enc(m, k_sdpa, {m->c_q, m->kv_k[l], m->kv_v[l], m->c_meta}, {m->c_tmp, m->c_o}, n) ||
+                enc(m, u_o, {L.wo, m->c_o}, {m->c_po}, n) ||
+                enc(m, u_gu, {L.wgate, m->c_po, L.wup, L.post_attn_norm, m->c_x, L.ffn_norm}, {m->c_pg, m->c_x}, n) ||
+                (last ? (enc(m, u_down_last, {L.wdown, m->c_pg}, {m->c_y}, n) || enc(m, k_add, {m->c_y, L.post_ffw_norm, m->c_x}, {m->c_x}, n))
+                      : enc(m, u_down, {L.wdown, m->c_pg}, {m->c_pd}, n)))
+                return 1;
+            continue;
+        }
         if ((fused ? (l > 0 ? enc(m, k_mm_qkv_close, {L.wq, m->c_y, L.wk, L.wv, m->layers[l - 1].post_ffw_norm, m->c_x, L.attn_norm}, {m->c_q, m->c_k, m->c_v, m->c_x}, n)
                             : enc(m, k_mm_qkv, {L.wq, m->c_x, L.wk, L.wv, L.attn_norm}, {m->c_q, m->c_k, m->c_v}, n))
                    : enc(m, k_norm, {m->c_x, L.attn_norm}, {m->c_x2}, n)) ||

@@ -148,8 +148,11 @@ template <int MODE>
 __global__ __launch_bounds__(1024) void mm_prep_rows_kernel(const float *__restrict__ X, const float *__restrict__ P0, const float *P1,
                                                              const float *__restrict__ P2, float *x_out, _Float16 *__restrict__ Xf_hi,
                                                              _Float16 *__restrict__ Xf_lo, _Float16 *__restrict__ SxA_hi,
-                                                             _Float16 *__restrict__ SxA_lo, int cols, float eps)
+                                                             _Float16 *__restrict__ SxA_lo, int cols, float eps, int x_slices, int x_parts)
 {
+    // x_slices != 0: X is the unfolded partial sums of the GEMM that produced it, [part * x_slices + slice][row][stride]
+    // with stride = cols (MODE 3: 2 * cols, gate | up side by side, and `up` is read from there); the slices are added
+    // here in the fold's order, the second part (the low parts of that GEMM's activations) scaled by 2^-11
     __shared__ float red[2][16];
     const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
     // (the norms run with cols / 8 threads, one trip; gelu * up of longer rows takes several)
@@ -167,8 +170,32 @@ __global__ __launch_bounds__(1024) void mm_prep_rows_kernel(const float *__restr
         for (int i = 0; i < nw; i++) s += red[which][i];
         return s;
     };
+    const size_t x_stride = MODE == 3 ? 2 * (size_t)cols : (size_t)cols, x_plane = (size_t)gridDim.x * x_stride;
+    auto ldx = [&](size_t col0, float (&v)[8]) __attribute__((always_inline)) {
+        const float *src = X + (size_t)t * x_stride + col0 + 8 * (size_t)j;
+        ld8(src, v);
+        for (int k = 1; k < x_slices; k++) {
+            float a[8];
+            ld8(src + (size_t)k * x_plane, a);
+#pragma unroll
+            for (int i = 0; i < 8; i++) v[i] += a[i];
+        }
+        if (x_parts == 2) {
+            float l[8];
+            ld8(src + (size_t)x_slices * x_plane, l);
+            for (int k = 1; k < x_slices; k++) {
+                float a[8];
+                ld8(src + (size_t)(x_slices + k) * x_plane, a);
+#pragma unroll
+                for (int i = 0; i < 8; i++) l[i] += a[i];
+            }
+#pragma unroll
+            for (int i = 0; i < 8; i++) v[i] = fmaf(1.0f / 2048.0f, l[i], v[i]);
+        }
+    };
     float f[8];
-    ld8(X + e0, f);
+    if (x_slices) ldx(0, f);
+    else ld8(X + e0, f);
     if (MODE == 1 || MODE == 2) {
         float ss = 0.f;
 #pragma unroll
@@ -197,7 +224,8 @@ __global__ __launch_bounds__(1024) void mm_prep_rows_kernel(const float *__restr
     }
     if (MODE == 3) {
         float u[8];
-        ld8(P0 + e0, u);
+        if (x_slices) ldx((size_t)cols, u);
+        else ld8(P0 + e0, u);
 #pragma unroll
         for (int i = 0; i < 8; i++) f[i] = gelu_mul_f32(f[i], u[i]);
     }
@@ -1311,16 +1339,18 @@ int launch_mul_mm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
     const int n_mat0 = 1 + (k.desc.dims[3] > 0) + (k.desc.dims[4] > 0), prologue = (int)k.desc.dims[5];
     if (prologue) {
         // the rows' producer runs inside the preparation: in = W, X, [W1, W2,] then the prologue's operands
+        const int xs = (int)(k.desc.dims[7] & 0xFF), xp = (int)(k.desc.dims[7] >> 8);
+        const int n_out0 = k.desc.dims[6] ? 1 : n_mat0;                    // (unfolded partial sums are one buffer)
         const float *X = (const float *)a.in[1], *q0 = (const float *)a.in[1 + n_mat0];
         const dim3 pg((unsigned)batch), pb((unsigned)std::min(cols / 8, 1024));
         const float eps = k.desc.params[0];
         if (prologue == 1)
-            hipLaunchKernelGGL(mm_prep_rows_kernel<1>, pg, pb, 0, st, X, q0, nullptr, nullptr, nullptr, Xf, Xf_lo, SxA, SxA_lo, cols, eps);
+            hipLaunchKernelGGL(mm_prep_rows_kernel<1>, pg, pb, 0, st, X, q0, nullptr, nullptr, nullptr, Xf, Xf_lo, SxA, SxA_lo, cols, eps, xs, xp);
         else if (prologue == 2)
-            hipLaunchKernelGGL(mm_prep_rows_kernel<2>, pg, pb, 0, st, X, q0, (const float *)a.in[2 + n_mat0], (const float *)a.in[3 + n_mat0], (float *)a.out[n_mat0],
-                               Xf, Xf_lo, SxA, SxA_lo, cols, eps);
+            hipLaunchKernelGGL(mm_prep_rows_kernel<2>, pg, pb, 0, st, X, q0, (const float *)a.in[2 + n_mat0], (const float *)a.in[3 + n_mat0], (float *)a.out[n_out0],
+                               Xf, Xf_lo, SxA, SxA_lo, cols, eps, xs, xp);
         else
-            hipLaunchKernelGGL(mm_prep_rows_kernel<3>, pg, pb, 0, st, X, q0, nullptr, nullptr, nullptr, Xf, Xf_lo, SxA, SxA_lo, cols, eps);
+            hipLaunchKernelGGL(mm_prep_rows_kernel<3>, pg, pb, 0, st, X, xs ? X : q0, nullptr, nullptr, nullptr, Xf, Xf_lo, SxA, SxA_lo, cols, eps, xs, xp);
     } else if (f32x) hipLaunchKernelGGL(mm_prep_x_f32_kernel, dim3((n + 255) / 256), dim3(256), 0, st, (const float *)a.in[1], Xf, Xf_lo, SxA, SxA_lo, batch, cols);
     else hipLaunchKernelGGL(mm_prep_x_kernel, dim3((n + 255) / 256), dim3(256), 0, st, (const uint16_t *)a.in[1], Xf, SxA, batch, cols);
     MmParams p;
@@ -1330,7 +1360,8 @@ int launch_mul_mm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
     const int rows1 = (int)k.desc.dims[3], rows2 = (int)k.desc.dims[4];
     p.rows1 = rows1; p.rows2 = rows2;
     p.W1 = rows1 ? (const uint8_t *)a.in[2] : p.W; p.W2 = rows2 ? (const uint8_t *)a.in[3] : p.W;
-    p.Y1 = rows1 ? (float *)a.out[1] : p.Y; p.Y2 = rows2 ? (float *)a.out[2] : p.Y;
+    const bool unfolded_out = k.desc.dims[6] != 0;
+    p.Y1 = rows1 && !unfolded_out ? (float *)a.out[1] : p.Y; p.Y2 = rows2 && !unfolded_out ? (float *)a.out[2] : p.Y;
     if (k.variant == 1) {
         // the small-batch form: one launch, the low parts riding along
         p.Xf = Xf; p.SxA = SxA; p.accum = 0.f;
@@ -1351,12 +1382,14 @@ int launch_mul_mm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
         const int ks = k.variant >> 1, parts = f32x ? 2 : 1;
         p.Xf = Xf; p.SxA = SxA; p.accum = 0.f;
         p.ksplit = ks;
-        p.Y_parts = (float *)((f32x ? SxA_lo : SxA) + sx_halves);     // behind the prepared activations
+        const bool unfolded = k.desc.dims[6] != 0;                    // the partial sums are the result: the reader adds them
+        p.Y_parts = unfolded ? (float *)a.out[0] : (float *)((f32x ? SxA_lo : SxA) + sx_halves);     // (else behind the prepared activations)
         const dim3 gz(grid.x, grid.y, ks * parts);
         if (k.desc.dtypes[0] == KSH_Q6K) hipLaunchKernelGGL(q_mul_mm_kernel<true>, gz, dim3(kThreadsMM), kLdsBytes, st, p);
         else hipLaunchKernelGGL(q_mul_mm_kernel<false>, gz, dim3(kThreadsMM), kLdsBytes, st, p);
         hipError_t e3 = hipGetLastError();
         if (e3 != hipSuccess) return hip_fail(e3, "mul_mm (K slices) launch");
+        if (unfolded) return 0;
         const int n2 = batch * (rows + rows1 + rows2);
         hipLaunchKernelGGL(mm_parts_fold_kernel, dim3((n2 + 255) / 256), dim3(256), 0, st, (const float *)p.Y_parts, p.Y, p.Y1, p.Y2, batch, rows, rows1, rows2,
                            ks, parts, 1.0f / 2048.0f);
@@ -1404,6 +1437,14 @@ int bind_matvec_batch(ksh_kernel &k)
     //   3 gelu(X) * up                  in: ..., up[batch, cols]
     const int64_t prologue = k.desc.dims[5];
     if (prologue < 0 || prologue > 3) return set_error("matvec_batch: prologue %lld (0 none, 1 rmsnorm, 2 add then norm, 3 gelu * up)", (long long)prologue);
+    // dims[6] = 1: the K slices' partial sums are the result, unfolded: out[0] = f32[parts * slices][batch][all rows]
+    // (parts = 2 for F32 activations; the matrices' columns side by side), for a reader that adds them itself --
+    // dims[7] = slices | parts << 8 of the GEMM whose unfolded result this one's X is (prologues 1 to 3; prologue 3
+    // then reads gate | up from that one buffer and takes no `up` operand)
+    const int64_t unfolded = k.desc.dims[6], x_slices = k.desc.dims[7] & 0xFF, x_parts = k.desc.dims[7] >> 8;
+    if (unfolded < 0 || unfolded > 1) return set_error("matvec_batch: dims[6]=%lld (0, or 1 for unfolded partial sums)", (long long)unfolded);
+    if (k.desc.dims[7] && (!prologue || x_slices < 1 || x_slices > 64 || x_parts < 1 || x_parts > 2))
+        return set_error("matvec_batch: X as unfolded partial sums (dims[7]=%lld) takes a prologue, 1 to 64 slices and 1 or 2 parts", (long long)k.desc.dims[7]);
     if (prologue) {
         if (!f32x) return set_error("matvec_batch: a prologue takes F32 activations");
         if (prologue != 3 && (cols > 8192 || cols % 512)) return set_error("matvec_batch: a norm prologue takes rows of a multiple of 512 up to 8192 columns, got %lld", (long long)cols);
@@ -1412,8 +1453,9 @@ int bind_matvec_batch(ksh_kernel &k)
         auto add_in = [&](size_t bytes) { k.in_bytes[ni] = bytes; k.in_align[ni] = 16; ni++; };
         if (prologue == 1) add_in(vec);
         if (prologue == 2) { add_in(vec); add_in(mat); add_in(vec); k.out_bytes[n_mat] = mat; k.out_align[n_mat] = 16; k.info.n_outputs = n_mat + 1; }
-        if (prologue == 3) add_in(mat);
+        if (prologue == 3 && !x_slices) add_in(mat);
         k.info.n_inputs = ni;
+        if (x_slices) k.in_bytes[1] = (size_t)x_slices * x_parts * mat * (prologue == 3 ? 2 : 1);
     }
     // f16 copy of X plus the min-term operand (32 halves per token and superblock)
     k.scratch_bytes = ((size_t)((batch + 31) / 32 * 32) * cols * 2 + (size_t)batch * (cols / 256) * 64) * (f32x ? 2 : 1);
@@ -1421,7 +1463,7 @@ int bind_matvec_batch(ksh_kernel &k)
     // there), 128 = the 128 x 128 tile.
     const uint32_t want = k.desc.sched.nr0;
     if (want && want != 32 && want != BN) return set_error("matvec_batch: unsupported schedule nr0=%u (32 or %d)", want, BN);
-    const bool can_skinny = !q6 && batch <= kSkinnyMaxBatch && n_mat == 1;
+    const bool can_skinny = !q6 && batch <= kSkinnyMaxBatch && n_mat == 1 && !unfolded;
     if (want == 32 && !can_skinny) return set_error("matvec_batch: the small-batch form takes Q4_K weights and up to %d tokens", kSkinnyMaxBatch);
     // (long rows of a short matrix leave the small-batch form 64 workgroups with four superblocks per wave: from 33
     // tokens on the tile over K slices is faster there -- 2048 x 8192 at 63 tokens: 27.5 us against 41.0)
@@ -1449,14 +1491,21 @@ int bind_matvec_batch(ksh_kernel &k)
         while (tiles * parts * ks < 256 && nsb % (ks * 2) == 0 && nsb / (ks * 2) >= 2) ks *= 2;   // (a slice of one superblock is all prologue)
     }
     // (f32 activations with fewer tiles than compute units: both parts in one launch even without a K split)
-    const bool z_form = ks > 1 || (parts == 2 && tiles < 256 && !k.desc.sched.k_split);
+    const bool z_form = unfolded || ks > 1 || (parts == 2 && tiles < 256 && !k.desc.sched.k_split);
     k.variant = z_form ? (int)(ks << 1) : 0;
-    if (z_form) k.scratch_bytes += (size_t)parts * ks * batch * rows_all * 4;
+    if (z_form && !unfolded) k.scratch_bytes += (size_t)parts * ks * batch * rows_all * 4;
+    if (unfolded) {
+        const int keep = prologue == 2 ? 1 : 0;                       // (the add-then-norm prologue's x_new stays an output)
+        if (keep) { k.out_bytes[1] = k.out_bytes[n_mat]; k.out_align[1] = 16; }
+        k.out_bytes[0] = (size_t)parts * ks * batch * rows_all * 4; k.out_align[0] = 16;
+        k.info.n_outputs = 1 + keep;
+    }
     set_launch(k, (uint32_t)((batch + BM - 1) / BM), (uint32_t)row_tiles, z_form ? (uint32_t)(ks * parts) : 1, kThreadsMM,
                (uint32_t)kLdsBytes);
     k.info.sched.tg = kThreadsMM; k.info.sched.nsg = kThreadsMM / 64; k.info.sched.nr0 = BN; k.info.sched.k_split = (uint32_t)ks; k.info.sched.lds_tile = KS;
     set_name(k, "mul_mm_%s_%dx%dx%d%s%s%s%s", q6 ? "q6k" : "q4k", BM, BN, KS, f32x ? "_f32x" : "", z_form ? "_kz" : "", n_mat == 3 ? "_x3" : n_mat == 2 ? "_x2" : "",
              prologue == 1 ? "_rms" : prologue == 2 ? "_addrms" : prologue == 3 ? "_gelu" : "");
+    if (unfolded) { char nm[64]; snprintf(nm, sizeof(nm), "%s", k.info.name); set_name(k, "%s_unfolded", nm); }
     k.launch = launch_mul_mm;
     return 0;
 }

@@ -251,6 +251,49 @@ def test_mul_mm_with_the_rows_producer_inside(ctx, mode, batch, rows3, cols):
         assert worst <= 2e-5, (k.name, i, worst)
 
 
+@pytest.mark.parametrize("batch", [96, 300])
+def test_mul_mm_unfolded_results_feed_the_next_preparation(ctx, batch):
+    """dims[6] = 1 leaves a GEMM's K slices (and the two parts of its f32 activations) as partial sums for a reader
+    that adds them itself; dims[7] tells the next GEMM's prologue that its X is such a buffer.  The chain o-projection
+    -> add-then-norm -> gate | up -> gelu * up -> down gives the very numbers of the same chain with every result
+    folded by its own launch."""
+    eps, hidden, ffn = 1e-6, 512, 1024
+    wo, wg, wu, wd = (synth.q4k_blocks(r * c // 256, 680 + i) for i, (r, c) in enumerate(((hidden, hidden), (ffn, hidden), (ffn, hidden), (hidden, ffn))))
+    bo, bg, bu, bd = (ctx.buffer_bytes(w) for w in (wo, wg, wu, wd))
+    a = ctx.buffer_f32(synth.normal_f32(batch * hidden, 684))
+    # (a small second norm weight keeps gelu(gate) * up of these synthetic weights inside the f16 range of the hi parts)
+    w_post, w_norm = ctx.buffer_f32(1.0 + 0.2 * synth.normal_f32(hidden, 685)), ctx.buffer_f32(0.01 * (1.0 + 0.2 * synth.normal_f32(hidden, 686)))
+    res0 = synth.normal_f32(batch * hidden, 687)
+    f32 = (DType.Q4K, DType.F32, DType.F32)
+    desc = lambda dims: hip.make_desc(hip.Kind.MATVEC_BATCH, dims, f32, (eps,))
+
+    def run(kernel, ins, outs):
+        ctx.encode_multi(kernel, ins, outs)
+        ctx.synchronize()
+
+    # folded: every GEMM finishes its own result
+    y, g, u, out_a = (ctx.buffer_empty_f32(batch * n) for n in (hidden, ffn, ffn, hidden))
+    res_a = ctx.buffer_f32(res0)
+    run(ctx.compile(desc((hidden, hidden, batch))), [bo, a], [y])
+    run(ctx.compile(desc((ffn, hidden, batch, ffn, 0, 2))), [bg, y, bu, w_post, res_a, w_norm], [g, u, res_a])
+    run(ctx.compile(desc((hidden, ffn, batch, 0, 0, 3))), [bd, g, u], [out_a])
+    # unfolded: the partial sums travel
+    ko = ctx.compile(desc((hidden, hidden, batch, 0, 0, 0, 1)))
+    zo = ko.grid[2]
+    assert ko.name.endswith("_unfolded") and zo == 2 * ko.info.sched.k_split
+    po = ctx.buffer_empty_f32(zo * batch * hidden)
+    run(ko, [bo, a], [po])
+    kg = ctx.compile(desc((ffn, hidden, batch, ffn, 0, 2, 1, ko.info.sched.k_split | 2 << 8)))
+    zg = kg.grid[2]
+    pg, res_b = ctx.buffer_empty_f32(zg * batch * 2 * ffn), ctx.buffer_f32(res0)
+    run(kg, [bg, po, bu, w_post, res_b, w_norm], [pg, res_b])
+    out_b = ctx.buffer_empty_f32(batch * hidden)
+    run(ctx.compile(desc((hidden, ffn, batch, 0, 0, 3, 0, kg.info.sched.k_split | 2 << 8))), [bd, pg], [out_b])
+    assert np.array_equal(ctx.read_f32(res_a, batch * hidden), ctx.read_f32(res_b, batch * hidden))
+    assert np.array_equal(ctx.read_f32(out_a, batch * hidden), ctx.read_f32(out_b, batch * hidden))
+    assert np.isfinite(ctx.read_f32(out_a, batch * hidden)).all() and np.abs(ctx.read_f32(out_a, batch * hidden)).max() > 0
+
+
 def test_mul_mm_k_slices_must_divide_the_row(ctx):
     with pytest.raises(hip.KshError, match="does not divide"):
         ctx.compile(hip.make_desc(hip.Kind.MATVEC_BATCH, (256, 2048, 100), (DType.Q4K, DType.BF16, DType.F32), (), dict(k_split=3)))

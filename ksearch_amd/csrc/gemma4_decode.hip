@@ -133,6 +133,7 @@ struct ksh_gemma4 {
     // prompt chunks (allocated at the first chunk): [kChunk, .] activations of the batched layer pass
     ksh_buf *c_tok = nullptr, *c_x = nullptr, *c_x2 = nullptr, *c_y = nullptr, *c_q = nullptr, *c_k = nullptr, *c_v = nullptr, *c_o = nullptr,
             *c_g = nullptr, *c_u = nullptr, *c_ff = nullptr, *c_tmp = nullptr, *c_meta_full = nullptr, *c_meta_swa = nullptr,
+            *c_po = nullptr, *c_pg = nullptr,   // unfolded partial sums of the o and the gate | up projection of a chunk
             *c_ple_tok = nullptr, *c_ple_tmp = nullptr, *c_ple_ctx = nullptr, *c_ple_u = nullptr;
     // decode rounds over several KV slots (allocated at the first round): the per-token table (ids, slots, attended
     // ranges of the two layer kinds), the logits of every token of the round, the greedy ids
@@ -367,6 +368,7 @@ int write_token(ksh_gemma4 *m, uint32_t token)
 // prefill_chunk's chunk length (gemma_prim.rs:16)
 constexpr int kChunk4 = 1024;
 constexpr int kChunkPartitions4 = 8;
+constexpr int kPartsRows4 = 4;      // room for the unfolded partial sums of a hidden-wide projection: this many chunks of rows
 
 int chunk_buffers4(ksh_gemma4 *m)
 {
@@ -380,7 +382,8 @@ int chunk_buffers4(ksh_gemma4 *m)
         alloc(m, T * c.hidden * 4, &m->c_y) || alloc(m, T * qd * 4, &m->c_q) || alloc(m, T * kvd * 4, &m->c_k) ||
         alloc(m, T * kvd * 4, &m->c_v) || alloc(m, T * qd * 4, &m->c_o) || alloc(m, T * max_ff * 4, &m->c_g) ||
         alloc(m, T * max_ff * 4, &m->c_u) || alloc(m, T * max_ff * 4, &m->c_ff) ||
-        alloc(m, T * c.n_q * kChunkPartitions4 * (max_hd + 2) * 4, &m->c_tmp) || alloc(m, 16, &m->c_meta_full) || alloc(m, 16, &m->c_meta_swa))
+        alloc(m, T * c.n_q * kChunkPartitions4 * (max_hd + 2) * 4, &m->c_tmp) || alloc(m, 16, &m->c_meta_full) || alloc(m, 16, &m->c_meta_swa) ||
+        alloc(m, kPartsRows4 * T * c.hidden * 4, &m->c_po) || alloc(m, 2 * T * 2 * max_ff * 4, &m->c_pg))
         return 1;
     if (c.ple_dim > 0 && (alloc(m, T * pt * 4, &m->c_ple_tok) || alloc(m, T * pt * 4, &m->c_ple_tmp) || alloc(m, T * pt * 4, &m->c_ple_ctx) ||
                           alloc(m, T * c.ple_dim * 4, &m->c_ple_u)))
@@ -476,7 +479,25 @@ int forward_prefill_chunk4(ksh_gemma4 *m, const uint32_t *tokens, int t)
         }
         // (heads of 256 or 512 in chunks of more than 16 tokens take the attention's matrix-core form: one partition per token)
         if (get(m, KSH_SDPA_BATCH, {c.n_q, c.n_kv, P.hd, c.max_seq, t, t > 16 && (P.hd == 256 || P.hd == 512) && c.n_q / c.n_kv <= 8 ? 1 : kChunkPartitions4}, {KSH_Q40, KSH_F32}, {c.attn_scale}, &k_sdpa) ||
-            enc(m, k_sdpa, {m->c_q, kc, vc, P.swa ? m->c_meta_swa : m->c_meta_full}, {m->c_tmp, m->c_o}, n) ||
+            enc(m, k_sdpa, {m->c_q, kc, vc, P.swa ? m->c_meta_swa : m->c_meta_full}, {m->c_tmp, m->c_o}, n))
+            return 1;
+        // With the producers inside, the o and the gate | up projection leave their K slices' partial sums unfolded
+        // for the preparation that reads them (dims[6], dims[7]); the down projection folds (a plain norm reads it).
+        ksh_kernel *u_o = nullptr, *u_gu = nullptr;
+        bool travel = false;
+        if (inside && L.dt_gate == L.dt_up) {
+            const size_t T = kChunk4;
+            if (get(m, KSH_MATVEC_BATCH, {h, P.qd, tp, 0, 0, 0, 1}, {L.dt_o, KSH_F32, KSH_F32}, {c.eps}, &u_o) ||
+                get(m, KSH_MATVEC_BATCH, {L.ffn, h, tp, L.ffn, 0, 2, 1, (int64_t)(u_o->info.sched.k_split | 2u << 8)}, {L.dt_gate, KSH_F32, KSH_F32}, {c.eps}, &u_gu))
+                return 1;
+            travel = u_o->out_bytes[0] <= kPartsRows4 * T * c.hidden * 4 && u_gu->out_bytes[0] <= ksh_buffer_size(m->c_pg);
+        }
+        if (travel) {
+            if (enc(m, u_o, {L.wo, m->c_o}, {m->c_po}, n) ||
+                enc(m, u_gu, {L.wgate, m->c_po, L.wup, L.post_attn_norm, m->c_x, L.ffn_norm}, {m->c_pg, m->c_x}, n) ||
+                mm_pro(L.dt_down, {h, L.ffn, tp, 0, 0, 3, 0, (int64_t)(u_gu->info.sched.k_split | 2u << 8)}, {L.wdown, m->c_pg}, {m->c_y}))
+                return 1;
+        } else if (
             mm(L.dt_o, h, P.qd, L.wo, m->c_o, m->c_y) ||
             (inside && L.dt_gate == L.dt_up
                  ? mm_pro(L.dt_gate, {L.ffn, h, tp, L.ffn, 0, 2}, {L.wgate, m->c_y, L.wup, L.post_attn_norm, m->c_x, L.ffn_norm}, {m->c_g, m->c_u, m->c_x})
@@ -485,9 +506,9 @@ int forward_prefill_chunk4(ksh_gemma4 *m, const uint32_t *tokens, int t)
                                                     : (mm(L.dt_gate, L.ffn, h, L.wgate, m->c_x2, m->c_g) || mm(L.dt_up, L.ffn, h, L.wup, m->c_x2, m->c_u))))) ||
             (inside ? mm_pro(L.dt_down, {h, L.ffn, tp, 0, 0, 3}, {L.wdown, m->c_g, m->c_u}, {m->c_y})
                     : (get(m, KSH_GELU_MUL, {(int64_t)t * L.ffn}, {}, {}, &k_gelu) || enc(m, k_gelu, {m->c_g, m->c_u}, {m->c_ff}, n) ||
-                       mm(L.dt_down, h, L.ffn, L.wdown, m->c_ff, m->c_y))) ||
-            enc(m, k_add, {m->c_y, L.post_ffw_norm, m->c_x}, {m->c_x}, n))
+                       mm(L.dt_down, h, L.ffn, L.wdown, m->c_ff, m->c_y))))
             return 1;
+        if (enc(m, k_add, {m->c_y, L.post_ffw_norm, m->c_x}, {m->c_x}, n)) return 1;
         if (c.ple_dim > 0) {
             // gemma_prim.rs:1558-1600: u = gelu(Wg x) * ctx_l; x = (x + rms(Wp u) * post_norm) * layer_scale
             ksh_kernel *k_gs = nullptr, *k_as = nullptr;

@@ -306,6 +306,7 @@ constexpr int kThreadsMM = 512;
 constexpr int kLdsMain = BN * PITCH;             // halves per main stage (the dequantized weight tile)
 constexpr int kLdsMin = (BM + BN) * PITCH2;      // halves per min-term stage
 constexpr size_t kLdsBytes = 2 * (size_t)(kLdsMain + kLdsMin) * 2 + 2 * BN * 4;
+constexpr size_t kLdsBytes64 = 2 * (size_t)(kLdsMain + (64 + BN) * PITCH2) * 2 + 2 * BN * 4;   // the 64-token tile
 
 // Eight waves in two roles, one of each per SIMD.  Waves 0..3 only multiply:
 // each owns a 64 x 64 piece of the tile (2 x 2 MFMA tiles, one LDS operand
@@ -324,13 +325,17 @@ constexpr size_t kLdsBytes = 2 * (size_t)(kLdsMain + kLdsMin) * 2 + 2 * BN * 4;
 // sc_j * q is exact in f16 up to 2048; beyond that (needs |sc_j| > 64) it rounds to the nearest even integer, a
 // relative 2^-11 at most and on those weights only (the reference's tile rounds every weight to half, the same
 // bound).  There is no min term, so the short second product is skipped; d is applied per superblock as for Q4_K.
-template <bool Q6>
-__global__ __launch_bounds__(kThreadsMM) void q_mul_mm_kernel(MmParams p)
+// TM = tokens per workgroup.  128: each multiplying wave owns 64 x 64.  64: each owns 32 x 64 with half the
+// accumulators, the kernel fits 128 registers and 70 KB of LDS, and two workgroups share a compute unit, so that one's
+// barriers and first loads fall into the other's products (the weights are converted once per 64 tokens then).
+template <bool Q6, int TM>
+__global__ __launch_bounds__(kThreadsMM, TM == 64 ? 2 : 1) void q_mul_mm_kernel(MmParams p)
 {
+    constexpr int MT = TM / 64, kLdsMinT = (TM + BN) * PITCH2;
     extern __shared__ __attribute__((aligned(16))) _Float16 lds[];
     auto main_stage = [&](int i) { return lds + (i & 1) * kLdsMain; };
-    auto min_stage = [&](int i) { return lds + 2 * kLdsMain + (i & 1) * kLdsMin; };
-    auto dsc_stage = [&](int i) { return reinterpret_cast<float *>(lds + 2 * kLdsMain + 2 * kLdsMin) + (i & 1) * BN; };
+    auto min_stage = [&](int i) { return lds + 2 * kLdsMain + (i & 1) * kLdsMinT; };
+    auto dsc_stage = [&](int i) { return reinterpret_cast<float *>(lds + 2 * kLdsMain + 2 * kLdsMinT) + (i & 1) * BN; };
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     // which matrix this row tile belongs to (the copy of the arguments is this workgroup's own)
@@ -341,7 +346,7 @@ __global__ __launch_bounds__(kThreadsMM) void q_mul_mm_kernel(MmParams p)
         if (by >= ty0 + ty1) { by -= ty0 + ty1; ycol = p.rows + p.rows1; p.W = p.W2; p.Y = p.Y2; p.rows = p.rows2; }
         else if (by >= ty0) { by -= ty0; ycol = p.rows; p.W = p.W1; p.Y = p.Y1; p.rows = p.rows1; }
     }
-    const int t0 = blockIdx.x * BM, r0 = by * BN;
+    const int t0 = blockIdx.x * TM, r0 = by * BN;
     const int nsb_row = p.cols / 256;                            // superblocks per weight row
     int nsb = nsb_row, sb0 = 0;                                  // this workgroup's share of them
     size_t ystride = (size_t)p.rows;
@@ -489,7 +494,7 @@ __global__ __launch_bounds__(kThreadsMM) void q_mul_mm_kernel(MmParams p)
             }
             if (G == 0) {
                 // bias + mins of this superblock, for the short second product after its fourth step
-                _Float16 *A2s = min_stage(sb), *B2s = A2s + BM * PITCH2;
+                _Float16 *A2s = min_stage(sb), *B2s = A2s + TM * PITCH2;
                 const float d = half_bits_to_f32(w.hdr.x & 0xFFFFu), dmin = half_bits_to_f32(w.hdr.x >> 16);
                 // this thread covers sub-blocks 4*lh .. 4*lh+3 of its row: groups 2*lh, 2*lh+1
                 uint32_t hi2[2], lo2[2];
@@ -509,9 +514,11 @@ __global__ __launch_bounds__(kThreadsMM) void q_mul_mm_kernel(MmParams p)
                 b2[4] = make_uint2(hi2[0], hi2[1]);
                 b2[6] = make_uint2(0u, 0u);
                 if (lh == 0) dsc_stage(sb)[lrow] = d;
-                u32x4_t *dst = reinterpret_cast<u32x4_t *>(&A2s[lrow * PITCH2 + 16 * lh]);
-                dst[0] = w.sx0;
-                dst[1] = w.sx1;
+                if (lrow < TM) {
+                    u32x4_t *dst = reinterpret_cast<u32x4_t *>(&A2s[lrow * PITCH2 + 16 * lh]);
+                    dst[0] = w.sx0;
+                    dst[1] = w.sx1;
+                }
             }
         };
 
@@ -541,9 +548,9 @@ __global__ __launch_bounds__(kThreadsMM) void q_mul_mm_kernel(MmParams p)
 
     // ---------------------------------------------------------------------- multipliers
     const int wm = wave >> 1, wn = wave & 1;
-    f16v F[2][2], Cp[2][2];
+    f16v F[MT][2], Cp[MT][2];
 #pragma unroll
-    for (int a = 0; a < 2; a++)
+    for (int a = 0; a < MT; a++)
 #pragma unroll
         for (int b = 0; b < 2; b++)
 #pragma unroll
@@ -553,14 +560,14 @@ __global__ __launch_bounds__(kThreadsMM) void q_mul_mm_kernel(MmParams p)
     // A operands straight from memory: fragment (token tile, k / 16) is 64 lanes x 16 bytes, 1 KB apart along k.
     // Two register sets, each refilled for two steps ahead as soon as its own step's instructions are issued.
     const int ntt = (p.batch + 31) / 32;
-    const h8 *xa[2];
+    const h8 *xa[MT];
 #pragma unroll
-    for (int mt = 0; mt < 2; mt++)
-        xa[mt] = reinterpret_cast<const h8 *>(p.Xf) + ((size_t)min((t0 + wm * 64 + mt * 32) / 32, ntt - 1) * (p.cols / 16) + (size_t)sb0 * 16) * 64 + lane;
-    struct ARegs { h8 a[2][KS / 16]; };
+    for (int mt = 0; mt < MT; mt++)
+        xa[mt] = reinterpret_cast<const h8 *>(p.Xf) + ((size_t)min((t0 + (wm * MT + mt) * 32) / 32, ntt - 1) * (p.cols / 16) + (size_t)sb0 * 16) * 64 + lane;
+    struct ARegs { h8 a[MT][KS / 16]; };
     auto fetch_a = [&](int step, ARegs &r) __attribute__((always_inline)) {
 #pragma unroll
-        for (int mt = 0; mt < 2; mt++)
+        for (int mt = 0; mt < MT; mt++)
 #pragma unroll
             for (int ks = 0; ks < KS / 16; ks++) r.a[mt][ks] = xa[mt][(size_t)(step * (KS / 16) + ks) * 64];
     };
@@ -580,30 +587,30 @@ __global__ __launch_bounds__(kThreadsMM) void q_mul_mm_kernel(MmParams p)
             for (int nt = 0; nt < 2; nt++)
                 b[nt] = *reinterpret_cast<const h8 *>(&Bs[(wn * 64 + nt * 32 + lm) * PITCH + 16 * ks + lk]);
 #pragma unroll
-            for (int mt = 0; mt < 2; mt++)
+            for (int mt = 0; mt < MT; mt++)
 #pragma unroll
                 for (int nt = 0; nt < 2; nt++)
                     // a superblock's first product starts from the constant zero: no pass over the accumulators to clear them
                     Cp[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A.a[mt][ks], b[nt], (g == 0 && ks == 0) ? kZero16 : Cp[mt][nt], 0, 0, 0);
             // this k slice's fragments are spent: ask for the ones of two steps ahead right away
 #pragma unroll
-            for (int mt = 0; mt < 2; mt++) A.a[mt][ks] = xa[mt][(size_t)(min(step + 2, nsteps - 1) * (KS / 16) + ks) * 64];
+            for (int mt = 0; mt < MT; mt++) A.a[mt][ks] = xa[mt][(size_t)(min(step + 2, nsteps - 1) * (KS / 16) + ks) * 64];
         }
         if (g == 3) {
             // ---- end of the superblock: bias + mins through the short second product, then the row scale
-            const _Float16 *A2s = min_stage(sb), *B2s = A2s + BM * PITCH2;
+            const _Float16 *A2s = min_stage(sb), *B2s = A2s + TM * PITCH2;
             const float *dsc = dsc_stage(sb);
 #pragma unroll
             for (int ks = 0; ks < (Q6 ? 0 : 2); ks++) {
-                h8 a[2], b[2];
+                h8 a[MT], b[2];
 #pragma unroll
-                for (int mt = 0; mt < 2; mt++)
-                    a[mt] = *reinterpret_cast<const h8 *>(&A2s[(wm * 64 + mt * 32 + lm) * PITCH2 + 16 * ks + lk]);
+                for (int mt = 0; mt < MT; mt++)
+                    a[mt] = *reinterpret_cast<const h8 *>(&A2s[((wm * MT + mt) * 32 + lm) * PITCH2 + 16 * ks + lk]);
 #pragma unroll
                 for (int nt = 0; nt < 2; nt++)
                     b[nt] = *reinterpret_cast<const h8 *>(&B2s[(wn * 64 + nt * 32 + lm) * PITCH2 + 16 * ks + lk]);
 #pragma unroll
-                for (int mt = 0; mt < 2; mt++)
+                for (int mt = 0; mt < MT; mt++)
 #pragma unroll
                     for (int nt = 0; nt < 2; nt++)
                         F[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mt], b[nt], F[mt][nt], 0, 0, 0);
@@ -612,7 +619,7 @@ __global__ __launch_bounds__(kThreadsMM) void q_mul_mm_kernel(MmParams p)
             for (int nt = 0; nt < 2; nt++) {
                 const float dn = dsc[wn * 64 + nt * 32 + lm];
 #pragma unroll
-                for (int mt = 0; mt < 2; mt++)
+                for (int mt = 0; mt < MT; mt++)
 #pragma unroll
                     for (int i = 0; i < 16; i++)
                         F[mt][nt][i] = fmaf(dn, Cp[mt][nt][i], F[mt][nt][i]);
@@ -629,13 +636,13 @@ __global__ __launch_bounds__(kThreadsMM) void q_mul_mm_kernel(MmParams p)
 
     // accumulator layout of the 32x32 tile: column = lane % 32, row = 8*(i/4) + 4*(lane/32) + i%4
 #pragma unroll
-    for (int mt = 0; mt < 2; mt++)
+    for (int mt = 0; mt < MT; mt++)
 #pragma unroll
         for (int nt = 0; nt < 2; nt++) {
             const int r = r0 + wn * 64 + nt * 32 + lm;
 #pragma unroll
             for (int i = 0; i < 16; i++) {
-                const int t = t0 + wm * 64 + mt * 32 + 8 * (i / 4) + 4 * (lane >> 5) + (i & 3);
+                const int t = t0 + (wm * MT + mt) * 32 + 8 * (i / 4) + 4 * (lane >> 5) + (i & 3);
                 if (t < p.batch && r < p.rows) {
                     float *y = &p.Y[(size_t)t * ystride + r];
                     *y = p.accum != 0.f ? fmaf(p.accum, F[mt][nt][i], *y) : F[mt][nt][i];
@@ -1375,7 +1382,12 @@ int launch_mul_mm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
         const hipError_t e2 = hipGetLastError();
         return e2 == hipSuccess ? 0 : hip_fail(e2, "mul_mm (small batch) launch");
     }
-    const dim3 grid((batch + BM - 1) / BM, (rows + BN - 1) / BN + (rows1 + BN - 1) / BN + (rows2 + BN - 1) / BN);
+    // up to 64 tokens: the 64-token tile (the other half of a 128-token tile would be empty rows).  Beyond that the
+    // 128-token tile: two 64-token workgroups per compute unit convert every weight twice as often, and the
+    // conversions, not the products, are what a step waits for (cfg2: 40.3 us against 33.7, a 1024-token prompt
+    // pass 17.4 ms against 15.8).
+    const int tm = (batch <= 64 && k.desc.dtypes[0] != KSH_Q6K) ? 64 : 128;
+    const dim3 grid((batch + tm - 1) / tm, (rows + BN - 1) / BN + (rows1 + BN - 1) / BN + (rows2 + BN - 1) / BN);
     p.ksplit = 0; p.Xf_lo = Xf_lo; p.SxA_lo = SxA_lo; p.Y_parts = nullptr;
     if (k.variant >= 2) {
         // few tiles: K slices and both parts of f32 activations as blockIdx.z of one launch, then the fold
@@ -1385,8 +1397,9 @@ int launch_mul_mm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
         const bool unfolded = k.desc.dims[6] != 0;                    // the partial sums are the result: the reader adds them
         p.Y_parts = unfolded ? (float *)a.out[0] : (float *)((f32x ? SxA_lo : SxA) + sx_halves);     // (else behind the prepared activations)
         const dim3 gz(grid.x, grid.y, ks * parts);
-        if (k.desc.dtypes[0] == KSH_Q6K) hipLaunchKernelGGL(q_mul_mm_kernel<true>, gz, dim3(kThreadsMM), kLdsBytes, st, p);
-        else hipLaunchKernelGGL(q_mul_mm_kernel<false>, gz, dim3(kThreadsMM), kLdsBytes, st, p);
+        if (k.desc.dtypes[0] == KSH_Q6K) hipLaunchKernelGGL((q_mul_mm_kernel<true, 128>), gz, dim3(kThreadsMM), kLdsBytes, st, p);
+        else if (tm == 64) hipLaunchKernelGGL((q_mul_mm_kernel<false, 64>), gz, dim3(kThreadsMM), kLdsBytes64, st, p);
+        else hipLaunchKernelGGL((q_mul_mm_kernel<false, 128>), gz, dim3(kThreadsMM), kLdsBytes, st, p);
         hipError_t e3 = hipGetLastError();
         if (e3 != hipSuccess) return hip_fail(e3, "mul_mm (K slices) launch");
         if (unfolded) return 0;
@@ -1400,8 +1413,9 @@ int launch_mul_mm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
         p.Xf = pass ? Xf_lo : Xf;
         p.SxA = pass ? SxA_lo : SxA;
         p.accum = pass ? 1.0f / 2048.0f : 0.f;
-        if (k.desc.dtypes[0] == KSH_Q6K) hipLaunchKernelGGL(q_mul_mm_kernel<true>, grid, dim3(kThreadsMM), kLdsBytes, st, p);
-        else hipLaunchKernelGGL(q_mul_mm_kernel<false>, grid, dim3(kThreadsMM), kLdsBytes, st, p);
+        if (k.desc.dtypes[0] == KSH_Q6K) hipLaunchKernelGGL((q_mul_mm_kernel<true, 128>), grid, dim3(kThreadsMM), kLdsBytes, st, p);
+        else if (tm == 64) hipLaunchKernelGGL((q_mul_mm_kernel<false, 64>), grid, dim3(kThreadsMM), kLdsBytes64, st, p);
+        else hipLaunchKernelGGL((q_mul_mm_kernel<false, 128>), grid, dim3(kThreadsMM), kLdsBytes, st, p);
     }
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : hip_fail(e, "mul_mm launch");

@@ -413,8 +413,8 @@ int forward_prefill_chunk4(ksh_gemma4 *m, const uint32_t *tokens, int t)
         ksh_kernel *kk = nullptr;
         return get(m, KSH_MATVEC_BATCH, {rows, cols, tp}, {dt, KSH_F32, KSH_F32}, {}, &kk) || enc(m, kk, {w, x}, {y}, n);
     };
-    // beyond the small-batch form's 64 tokens, matrices of one dtype over the same rows (q | k | v, gate | up) are one
-    // launch of the 128 x 128 tile over one preparation of the rows
+    // matrices of one dtype over the same rows (q | k | v, gate | up) are one launch of the tile over one preparation
+    // of the rows
     auto mm2 = [&](int dt, int64_t rows, int64_t cols, ksh_buf *w0, ksh_buf *w1, ksh_buf *x, ksh_buf *y0, ksh_buf *y1) {
         ksh_kernel *kk = nullptr;
         return get(m, KSH_MATVEC_BATCH, {rows, cols, tp, rows}, {dt, KSH_F32, KSH_F32}, {}, &kk) || enc(m, kk, {w0, x, w1}, {y0, y1}, n);
@@ -425,7 +425,7 @@ int forward_prefill_chunk4(ksh_gemma4 *m, const uint32_t *tokens, int t)
         return get(m, KSH_MATVEC_BATCH, {rows0, cols, tp, rows12, rows12}, {dt, KSH_F32, KSH_F32}, {}, &kk) ||
                enc(m, kk, {w0, x, w1, w2}, {y0, y1, y2}, n);
     };
-    const bool merged = tp > 32;
+    const bool merged = true;
     // ... with the rows' producers inside the GEMMs' preparations (dims[5]: the attention norm in q | k | v's,
     // add-then-norm in gate | up's, gelu(gate) * up in the down projection's)
     const bool inside = merged && h % 512 == 0 && h <= 8192;

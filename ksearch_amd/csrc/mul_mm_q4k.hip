@@ -293,12 +293,12 @@ __device__ __forceinline__ uint32_t pair_f16(uint32_t masked, uint32_t sc)
     return __umul24(masked, sc) + 0x64006400u;
 }
 
-// what a loader thread (two per tile row) holds per superblock: the 64 quant bytes of TWO of its four
-// 64-column groups (so that a weight row's cache lines are fetched once, not once per step), the header and
-// half of the token's sums of x
+// what a loader thread (two per tile row) holds per superblock: of each of the four 64-column groups the 16 quant
+// bytes it converts (all requested when the superblock opens, so that a weight row's cache lines are fetched once,
+// not once per step), the header and half of the token's sums of x
 // (native vector types: with HIP's uint4 class the copies become memcpys that keep these sets in scratch memory)
 struct SbRegs {
-    u32x4_t q[4];      // quant bytes of groups 2*lh and 2*lh+1, 32 each
+    u32x4_t q[4];      // of each of the four 64-column groups, the 16 quant bytes this thread converts
     u32x4_t hdr, sx0, sx1;
 };
 
@@ -454,27 +454,19 @@ __global__ __launch_bounds__(kThreadsMM, TM == 64 ? 2 : 1) void q_mul_mm_kernel(
             const u32x4_t *w = reinterpret_cast<const u32x4_t *>(wrow + (size_t)sb * 144);
             r.hdr = w[0];
 #pragma unroll
-            for (int i = 0; i < 4; i++) r.q[i] = w[1 + 4 * lh + i];
+            for (int i = 0; i < 4; i++) r.q[i] = w[1 + 2 * i + lh];     // the 16 bytes of group i that this thread converts
             const u32x4_t *sx = reinterpret_cast<const u32x4_t *>(sxrow + sb * 32 + 16 * lh);
             r.sx0 = sx[0];
             r.sx1 = sx[1];
         };
-        // G = the step's group: its 32 quant bytes sit in lane G/2 of every pair, registers q[2*(G%2)] and
-        // q[2*(G%2)+1]; this thread converts bytes 16*lh .. 16*lh+15 of them
+        // G = the step's group: this thread converts bytes 16*lh .. 16*lh+15 of its 32 quant bytes
         auto stage = [&](int step, auto gtag, const SbRegs &w) __attribute__((always_inline)) {
             constexpr int G = decltype(gtag)::value;
             const int sb = step >> 2;
             _Float16 *Bs = main_stage(step);
             {
-                constexpr int kSrc = (G >> 1) ? 0xF5 : 0xA0;   // quad_perm [1,1,3,3] : [0,0,2,2]
-                const u32x4_t c0 = w.q[2 * (G & 1)], c1 = w.q[2 * (G & 1) + 1];
-                uint32_t q[4];
-#pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    const uint32_t b0 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)c0[j], kSrc, 0xF, 0xF, true);
-                    const uint32_t b1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)c1[j], kSrc, 0xF, 0xF, true);
-                    q[j] = lh ? b1 : b0;
-                }
+                const u32x4_t c = w.q[G];
+                const uint32_t q[4] = {c[0], c[1], c[2], c[3]};
                 const uint4 s = q4k_group_scales(w.hdr.y, w.hdr.z, w.hdr.w, G);   // sc_lo, mn_lo, sc_hi, mn_hi
                 uint32_t lo[8], hi[8];
 #pragma unroll

@@ -57,8 +57,9 @@ enum ksh_kind {
     KSH_MATVEC = 1,
     /* MatvecBatch: Y[t,r] = sum_c W[r,c] X[t,c].  dims: rows, cols, batch.
      * dtypes[0] = Q4K | Q6K (GGUF byte order, blocks at 2-byte alignment),
-     * dtypes[1] = BF16 (X) or F32 (X is then taken as hi + lo f16 parts, 22 bits, in two passes: the form the
-     * decode loops' prompt chunks use), output F32 token-major.
+     * dtypes[1] = BF16 (X) or F32 (X is then taken as hi + lo f16 parts, 22 bits: two passes, two sets of workgroups,
+     * or -- Q4_K with a grid of at least 256 tiles -- one workgroup walking both; the form the decode loops' prompt
+     * chunks use), output F32 token-major.
      * in: W, X   out: Y[batch, rows]
      * dims[3], dims[4] (0 = none): rows of a second and a third matrix of the same dtype over the same X, taken in
      * the same launch (q | k | v of a prompt chunk: one preparation of X, one grid).  in: W, X, W1[, W2]

@@ -286,11 +286,15 @@ struct MmParams {
     const uint8_t *W1, *W2;
     float *Y1, *Y2;
     int rows1, rows2;
+    // both = 1 (Q4_K, f32 activations, a grid that fills the chip by itself): a workgroup walks its superblocks twice,
+    // first against the hi parts of the activations, then against the lo parts with the weights' operands scaled by
+    // 2^-11 (an exponent shift: exact), into the same accumulators -- one launch, one result, no second pass over Y
+    int both;
 };
 
-__device__ __forceinline__ uint32_t pair_f16(uint32_t masked, uint32_t sc)
+__device__ __forceinline__ uint32_t pair_f16(uint32_t masked, uint32_t sc, uint32_t base = 0x64006400u)
 {
-    return __umul24(masked, sc) + 0x64006400u;
+    return __umul24(masked, sc) + base;     // base: half 1024.0 twice (0x38003800: half 0.5 = 1024 * 2^-11)
 }
 
 // what a loader thread (two per tile row) holds per superblock: of each of the four 64-column groups the 16 quant
@@ -358,7 +362,8 @@ __global__ __launch_bounds__(kThreadsMM, TM == 64 ? 2 : 1) void q_mul_mm_kernel(
         p.Y = p.Y_parts + (size_t)blockIdx.z * p.batch * rows_all + ycol;   // partial sums: all matrices' columns side by side
         ystride = (size_t)rows_all;
     }
-    const int nsteps = nsb * 4;
+    const int nv = p.both ? 2 * nsb : nsb;                      // superblock visits: [hi parts of x | lo parts of x]
+    const int nsteps = nv * 4;
 
     if (Q6 && wave >= 4) {
         // ------------------------------------------------------------------ loaders, Q6_K
@@ -448,9 +453,13 @@ __global__ __launch_bounds__(kThreadsMM, TM == 64 ? 2 : 1) void q_mul_mm_kernel(
         const int lt = tid - 256, lrow = lt >> 1, lh = lt & 1;   // two threads per tile row
         const size_t row_bytes = (size_t)nsb_row * 144;
         const uint8_t *wrow = p.W + (size_t)min(r0 + lrow, p.rows - 1) * row_bytes + (size_t)sb0 * 144;
-        const _Float16 *sxrow = p.SxA + ((size_t)min(t0 + lrow, p.batch - 1) * nsb_row + sb0) * 32;
+        const size_t sx_off = ((size_t)min(t0 + lrow, p.batch - 1) * nsb_row + sb0) * 32;
+        const _Float16 *sxrow_hi = p.SxA + sx_off, *sxrow_lo = p.SxA_lo + sx_off;
 
-        auto fetch_sb = [&](int sb, SbRegs &r) __attribute__((always_inline)) {
+        auto fetch_sb = [&](int v, SbRegs &r) __attribute__((always_inline)) {
+            const bool second = v >= nsb;                        // (only with p.both)
+            const int sb = second ? v - nsb : v;
+            const _Float16 *sxrow = second ? sxrow_lo : sxrow_hi;
             const u32x4_t *w = reinterpret_cast<const u32x4_t *>(wrow + (size_t)sb * 144);
             r.hdr = w[0];
 #pragma unroll
@@ -463,6 +472,8 @@ __global__ __launch_bounds__(kThreadsMM, TM == 64 ? 2 : 1) void q_mul_mm_kernel(
         auto stage = [&](int step, auto gtag, const SbRegs &w) __attribute__((always_inline)) {
             constexpr int G = decltype(gtag)::value;
             const int sb = step >> 2;
+            const bool second = sb >= nsb;                       // the lo parts' visit: operands 2^-11 down
+            const uint32_t base = second ? 0x38003800u : 0x64006400u;
             _Float16 *Bs = main_stage(step);
             {
                 const u32x4_t c = w.q[G];
@@ -472,10 +483,10 @@ __global__ __launch_bounds__(kThreadsMM, TM == 64 ? 2 : 1) void q_mul_mm_kernel(
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     const uint32_t t4 = q[i] >> 4;
-                    lo[2 * i] = pair_f16(q[i] & 0x000F000Fu, s.x);
-                    lo[2 * i + 1] = pair_f16((q[i] >> 8) & 0x000F000Fu, s.x);
-                    hi[2 * i] = pair_f16(t4 & 0x000F000Fu, s.z);
-                    hi[2 * i + 1] = pair_f16((t4 >> 8) & 0x000F000Fu, s.z);
+                    lo[2 * i] = pair_f16(q[i] & 0x000F000Fu, s.x, base);
+                    lo[2 * i + 1] = pair_f16((q[i] >> 8) & 0x000F000Fu, s.x, base);
+                    hi[2 * i] = pair_f16(t4 & 0x000F000Fu, s.z, base);
+                    hi[2 * i + 1] = pair_f16((t4 >> 8) & 0x000F000Fu, s.z, base);
                 }
                 uint4 *dlo = reinterpret_cast<uint4 *>(&Bs[lrow * PITCH + 16 * lh]);
                 uint4 *dhi = reinterpret_cast<uint4 *>(&Bs[lrow * PITCH + 32 + 16 * lh]);
@@ -493,7 +504,8 @@ __global__ __launch_bounds__(kThreadsMM, TM == 64 ? 2 : 1) void q_mul_mm_kernel(
 #pragma unroll
                 for (int gg = 0; gg < 2; gg++) {
                     const uint4 s = q4k_group_scales(w.hdr.y, w.hdr.z, w.hdr.w, 2 * lh + gg);
-                    const float c0 = pinned(-(dmin * (float)s.y + 1024.f * d)), c1 = pinned(-(dmin * (float)s.w + 1024.f * d));
+                    const float down = second ? 1.0f / 2048.0f : 1.0f;
+                    const float c0 = pinned(-(dmin * (float)s.y + 1024.f * d) * down), c1 = pinned(-(dmin * (float)s.w + 1024.f * d) * down);
                     const _Float16 h0 = (_Float16)c0, h1 = (_Float16)c1;
                     const _Float16 l0 = (_Float16)(c0 - (float)h0), l1 = (_Float16)(c1 - (float)h1);
                     hi2[gg] = (uint32_t)__builtin_bit_cast(uint16_t, h0) | ((uint32_t)__builtin_bit_cast(uint16_t, h1) << 16);
@@ -522,14 +534,14 @@ __global__ __launch_bounds__(kThreadsMM, TM == 64 ? 2 : 1) void q_mul_mm_kernel(
         auto step_body = [&](int sb, auto gtag) __attribute__((always_inline)) {
             constexpr int g = decltype(gtag)::value;
             const int step = 4 * sb + g;
-            if (g == 0) fetch_sb(min(sb + 1, nsb - 1), wnext);
+            if (g == 0) fetch_sb(min(sb + 1, nv - 1), wnext);
             if (step + 1 < nsteps) {
                 if (g == 3) wcur = wnext;
                 stage(step + 1, std::integral_constant<int, (g + 1) & 3>{}, wcur);
             }
             __syncthreads();
         };
-        for (int sb = 0; sb < nsb; sb++) {
+        for (int sb = 0; sb < nv; sb++) {
             step_body(sb, std::integral_constant<int, 0>{});
             step_body(sb, std::integral_constant<int, 1>{});
             step_body(sb, std::integral_constant<int, 2>{});
@@ -556,12 +568,17 @@ __global__ __launch_bounds__(kThreadsMM, TM == 64 ? 2 : 1) void q_mul_mm_kernel(
 #pragma unroll
     for (int mt = 0; mt < MT; mt++)
         xa[mt] = reinterpret_cast<const h8 *>(p.Xf) + ((size_t)min((t0 + (wm * MT + mt) * 32) / 32, ntt - 1) * (p.cols / 16) + (size_t)sb0 * 16) * 64 + lane;
+    // (with p.both the steps of the second visit read the lo parts' fragments)
+    const ptrdiff_t lo_delta = p.both ? (reinterpret_cast<const h8 *>(p.Xf_lo) - reinterpret_cast<const h8 *>(p.Xf)) - (ptrdiff_t)nsb * 16 * 64 : 0;
+    auto afrag = [&](int mt, int step, int ks) __attribute__((always_inline)) {
+        return xa[mt][(ptrdiff_t)(step * (KS / 16) + ks) * 64 + (step >= 4 * nsb ? lo_delta : 0)];
+    };
     struct ARegs { h8 a[MT][KS / 16]; };
     auto fetch_a = [&](int step, ARegs &r) __attribute__((always_inline)) {
 #pragma unroll
         for (int mt = 0; mt < MT; mt++)
 #pragma unroll
-            for (int ks = 0; ks < KS / 16; ks++) r.a[mt][ks] = xa[mt][(size_t)(step * (KS / 16) + ks) * 64];
+            for (int ks = 0; ks < KS / 16; ks++) r.a[mt][ks] = afrag(mt, step, ks);
     };
     ARegs a0, a1;
     fetch_a(0, a0);
@@ -586,7 +603,7 @@ __global__ __launch_bounds__(kThreadsMM, TM == 64 ? 2 : 1) void q_mul_mm_kernel(
                     Cp[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A.a[mt][ks], b[nt], (g == 0 && ks == 0) ? kZero16 : Cp[mt][nt], 0, 0, 0);
             // this k slice's fragments are spent: ask for the ones of two steps ahead right away
 #pragma unroll
-            for (int mt = 0; mt < MT; mt++) A.a[mt][ks] = xa[mt][(size_t)(min(step + 2, nsteps - 1) * (KS / 16) + ks) * 64];
+            for (int mt = 0; mt < MT; mt++) A.a[mt][ks] = afrag(mt, min(step + 2, nsteps - 1), ks);
         }
         if (g == 3) {
             // ---- end of the superblock: bias + mins through the short second product, then the row scale
@@ -619,7 +636,7 @@ __global__ __launch_bounds__(kThreadsMM, TM == 64 ? 2 : 1) void q_mul_mm_kernel(
         }
         __syncthreads();
     };
-    for (int sb = 0; sb < nsb; sb++) {
+    for (int sb = 0; sb < nv; sb++) {
         mul_step(sb, std::integral_constant<int, 0>{}, a0);
         mul_step(sb, std::integral_constant<int, 1>{}, a1);
         mul_step(sb, std::integral_constant<int, 2>{}, a0);
@@ -1326,6 +1343,14 @@ int launch_matvec_round(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st
 
 constexpr int kSkinnyMaxBatch = 64;
 
+// Q4_K weights, f32 activations and at least one tile per compute unit: a workgroup takes the hi and the lo parts of
+// the activations one after the other (MmParams::both) instead of leaving them to two launches or two sets of workgroups
+bool mm_both_parts(const ksh_kernel_desc &d)
+{
+    const int64_t row_tiles = (d.dims[0] + BN - 1) / BN + (d.dims[3] + BN - 1) / BN + (d.dims[4] + BN - 1) / BN;
+    return d.dtypes[0] == KSH_Q4K && d.dtypes[1] == KSH_F32 && ((d.dims[2] + BM - 1) / BM) * row_tiles >= 256;
+}
+
 int launch_mul_mm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
 {
     const int rows = (int)k.desc.dims[0], cols = (int)k.desc.dims[1], batch = (int)k.desc.dims[2];
@@ -1381,9 +1406,10 @@ int launch_mul_mm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
     const int tm = (batch <= 64 && k.desc.dtypes[0] != KSH_Q6K) ? 64 : 128;
     const dim3 grid((batch + tm - 1) / tm, (rows + BN - 1) / BN + (rows1 + BN - 1) / BN + (rows2 + BN - 1) / BN);
     p.ksplit = 0; p.Xf_lo = Xf_lo; p.SxA_lo = SxA_lo; p.Y_parts = nullptr;
+    p.both = mm_both_parts(k.desc) ? 1 : 0;
     if (k.variant >= 2) {
         // few tiles: K slices and both parts of f32 activations as blockIdx.z of one launch, then the fold
-        const int ks = k.variant >> 1, parts = f32x ? 2 : 1;
+        const int ks = k.variant >> 1, parts = f32x && !p.both ? 2 : 1;
         p.Xf = Xf; p.SxA = SxA; p.accum = 0.f;
         p.ksplit = ks;
         const bool unfolded = k.desc.dims[6] != 0;                    // the partial sums are the result: the reader adds them
@@ -1401,7 +1427,7 @@ int launch_mul_mm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
         e3 = hipGetLastError();
         return e3 == hipSuccess ? 0 : hip_fail(e3, "mul_mm fold launch");
     }
-    for (int pass = 0; pass < (f32x ? 2 : 1); pass++) {
+    for (int pass = 0; pass < (f32x && !p.both ? 2 : 1); pass++) {
         p.Xf = pass ? Xf_lo : Xf;
         p.SxA = pass ? SxA_lo : SxA;
         p.accum = pass ? 1.0f / 2048.0f : 0.f;
@@ -1488,7 +1514,7 @@ int bind_matvec_batch(ksh_kernel &k)
     // about one workgroup per compute unit; every slice stores its partial sums and a second launch adds them in a
     // fixed order.  sched.k_split names the slice count (a divisor of cols / 256; 1 = none).
     const int64_t row_tiles = (rows + BN - 1) / BN + (rows1 + BN - 1) / BN + (rows2 + BN - 1) / BN;
-    const int64_t tiles = ((batch + BM - 1) / BM) * row_tiles, nsb = cols / 256, parts = f32x ? 2 : 1;
+    const int64_t tiles = ((batch + BM - 1) / BM) * row_tiles, nsb = cols / 256, parts = f32x && !mm_both_parts(k.desc) ? 2 : 1;
     int64_t ks = 1;
     if (k.desc.sched.k_split) {
         ks = k.desc.sched.k_split;

@@ -219,9 +219,11 @@ def test_prefill_chunk_matches_oracle_in_lockstep(ctx, small_model, n_prompt):
 
 def test_prefill_long_prompt_takes_two_chunks(ctx):
     """1100 prompt tokens are a chunk of 1024 and one of 76 (heads of 256: both chunks' attention on the matrix cores,
-    the second over the first one's rows; GEMMs over K slices at 1024 and at 76 rows): every K / V row within one code
-    step of the oracle's, which walks the positions one by one, and the decode steps behind the prompt at 1e-3."""
-    cfg = dict(n_layers=2, hidden=512, ffn=1024, n_q=4, n_kv=1, hd=256, vocab=4096, max_seq=1200,
+    the second over the first one's rows; GEMMs over K slices at 1024 and at 76 rows, gate | up at 1024 rows with
+    256 tiles: both parts of the activations walked by one workgroup; partial sums travelling between the GEMMs):
+    every K / V row within one code step of the oracle's, which walks the positions one by one, and the decode steps
+    behind the prompt at 1e-3."""
+    cfg = dict(n_layers=2, hidden=512, ffn=2048, n_q=4, n_kv=1, hd=256, vocab=4096, max_seq=1200,
                eps=1e-6, softcap=30.0, rope_theta=10000.0, attn_scale=1.0 / 16.0)
     w = synth.gemma_weights(cfg, 760, oracle.quantize_q4k, synth.chunked(oracle.quantize_q6k), std=0.05)
     gpu, cpu = hip.Gemma(ctx, cfg, w), oracle.Gemma(cfg, w)

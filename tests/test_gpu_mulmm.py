@@ -294,23 +294,28 @@ def test_mul_mm_unfolded_results_feed_the_next_preparation(ctx, batch):
     assert np.isfinite(ctx.read_f32(out_a, batch * hidden)).all() and np.abs(ctx.read_f32(out_a, batch * hidden)).max() > 0
 
 
-@pytest.mark.parametrize("unfolded", [0, 1])
-def test_mul_mm_f32_both_parts_in_one_workgroup(ctx, unfolded):
+@pytest.mark.parametrize("unfolded,k_split", [(0, 0), (1, 0), (0, 2), (1, 4)])
+def test_mul_mm_f32_both_parts_in_one_workgroup(ctx, unfolded, k_split):
     """Q4_K weights, f32 activations and at least 256 tiles: a workgroup walks its superblocks against the hi parts
     and then against the lo parts (weights' operands 2^-11 down, exactly) into the same accumulators -- one launch, one
-    result (or one set of partial sums).  1024 tokens x 4096 rows x 1024 columns against float64, a row of small and a
-    row of large activations among them."""
+    result (or one set of partial sums; with K slices asked for, one per slice).  1024 tokens x 4096 rows x 1024
+    columns against float64, a row of small and a row of large activations among them."""
     batch, rows, cols = 1024, 4096, 1024
     w = synth.q4k_blocks(rows * cols // 256, 690)
     x = synth.normal_f32(batch * cols, 691).reshape(batch, cols)
     x[3] *= 1e-3
     x[4] *= 300.0
-    k = ctx.compile(hip.make_desc(hip.Kind.MATVEC_BATCH, (rows, cols, batch, 0, 0, 0, unfolded), (DType.Q4K, DType.F32, DType.F32)))
-    assert k.grid[2] == 1 and ("_kz" in k.name) == bool(unfolded), (k.name, k.grid)
-    y = ctx.buffer_empty_f32(batch * rows)
+    k = ctx.compile(hip.make_desc(hip.Kind.MATVEC_BATCH, (rows, cols, batch, 0, 0, 0, unfolded), (DType.Q4K, DType.F32, DType.F32), (),
+                                  dict(k_split=k_split) if k_split else None))
+    nz = max(1, k_split)
+    assert k.grid[2] == nz and ("_kz" in k.name) == bool(unfolded or k_split), (k.name, k.grid)
+    y = ctx.buffer_empty_f32(nz * batch * rows if unfolded else batch * rows)
     ctx.encode_multi(k, [ctx.buffer_bytes(w), ctx.buffer_f32(x)], [y])
     ctx.synchronize()
-    got = ctx.read_f32(y, batch * rows).reshape(batch, rows)
+    if unfolded:
+        got = ctx.read_f32(y, nz * batch * rows).reshape(nz, batch, rows).astype(np.float64).sum(axis=0)
+    else:
+        got = ctx.read_f32(y, batch * rows).reshape(batch, rows)
     worst = max(float(rel_err(got[t], oracle.matvec_f64(oracle.Q4K, w, rows, cols, x[t])).max()) for t in (0, 3, 4, 5, 511, 1023))
     assert worst <= 2e-5, worst
 

@@ -139,25 +139,32 @@ __global__ __launch_bounds__(256) void mm_prep_x_f32_kernel(const float *__restr
 }
 
 // The same preparation with the producer of the rows folded in (f32 activations), one workgroup per row, cols / 8
-// threads with 8 consecutive elements each:
+// threads (1024 at most) with 8 consecutive elements each per trip:
+//   MODE 0  x = X
 //   MODE 1  x = rmsnorm(X, w)                                  (rmsnorm_rows, crates/ksearch_kernels/src/lib.rs:1478-1500)
 //   MODE 2  x_new = res + rmsnorm(X, w_post), stored; x = rmsnorm(x_new, w_norm)   (rmsnorm_add_then_rmsnorm_rows)
 //   MODE 3  x = gelu(X) * up                                   (gelu_mul on rows, gemma_prim.rs:1516-1538)
 // in the operation order of the kernels that do these alone (every product and sum rounded by itself).
+//
+// inv_s = nullptr: the two parts as above (lo kept 2^11 up, each part with its own sums), for the small-batch form.
+// inv_s != nullptr (the tile): the row is first scaled by the power of two s that puts its largest magnitude into
+// [2^9, 2^10) -- exact, and any f32 row fits f16 then, sums of 32 elements included -- and x s = hi + lo with BOTH
+// parts at that scale, so that one accumulator takes hi * w and lo * w of the same converted weight.  lo is a
+// subnormal f16 for elements below 2^-13 of the row's largest; what that costs is below 2^-35 of the largest.  The
+// sums of a sub-block are those of hi + lo, split in two halves as for bf16 rows; 1 / s goes to inv_s[row] for the
+// tile's last step.
 template <int MODE>
 __global__ __launch_bounds__(1024) void mm_prep_rows_kernel(const float *__restrict__ X, const float *__restrict__ P0, const float *P1,
                                                              const float *__restrict__ P2, float *x_out, _Float16 *__restrict__ Xf_hi,
                                                              _Float16 *__restrict__ Xf_lo, _Float16 *__restrict__ SxA_hi,
-                                                             _Float16 *__restrict__ SxA_lo, int cols, float eps, int x_slices, int x_parts)
+                                                             _Float16 *__restrict__ SxA_lo, int cols, float eps, int x_slices, int x_parts,
+                                                             float *__restrict__ inv_s)
 {
     // x_slices != 0: X is the unfolded partial sums of the GEMM that produced it, [part * x_slices + slice][row][stride]
     // with stride = cols (MODE 3: 2 * cols, gate | up side by side, and `up` is read from there); the slices are added
     // here in the fold's order, the second part (the low parts of that GEMM's activations) scaled by 2^-11
-    __shared__ float red[2][16];
+    __shared__ float red[3][16];
     const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
-    // (the norms run with cols / 8 threads, one trip; gelu * up of longer rows takes several)
-    for (int j = threadIdx.x; j < cols / 8; j += blockDim.x) {
-    const size_t e0 = (size_t)t * cols + 8 * (size_t)j;
     auto ld8 = [](const float *p, float (&v)[8]) __attribute__((always_inline)) {
         const f32x4_t a = reinterpret_cast<const f32x4_t *>(p)[0], b = reinterpret_cast<const f32x4_t *>(p)[1];
         v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
@@ -171,7 +178,7 @@ __global__ __launch_bounds__(1024) void mm_prep_rows_kernel(const float *__restr
         return s;
     };
     const size_t x_stride = MODE == 3 ? 2 * (size_t)cols : (size_t)cols, x_plane = (size_t)gridDim.x * x_stride;
-    auto ldx = [&](size_t col0, float (&v)[8]) __attribute__((always_inline)) {
+    auto ldx = [&](int j, size_t col0, float (&v)[8]) __attribute__((always_inline)) {
         const float *src = X + (size_t)t * x_stride + col0 + 8 * (size_t)j;
         ld8(src, v);
         for (int k = 1; k < x_slices; k++) {
@@ -193,79 +200,114 @@ __global__ __launch_bounds__(1024) void mm_prep_rows_kernel(const float *__restr
             for (int i = 0; i < 8; i++) v[i] = fmaf(1.0f / 2048.0f, l[i], v[i]);
         }
     };
-    float f[8];
-    if (x_slices) ldx(0, f);
-    else ld8(X + e0, f);
-    if (MODE == 1 || MODE == 2) {
-        float ss = 0.f;
+    // the row's elements 8j .. 8j+7 (the norms run with cols / 8 threads, one trip; plain rows and gelu * up of longer
+    // rows take several)
+    auto produce = [&](int j, float (&f)[8]) __attribute__((always_inline)) {
+        const size_t e0 = (size_t)t * cols + 8 * (size_t)j;
+        if (x_slices) ldx(j, 0, f);
+        else ld8(X + e0, f);
+        if (MODE == 1 || MODE == 2) {
+            float ss = 0.f;
 #pragma unroll
-        for (int i = 0; i < 8; i++) ss += f[i] * f[i];
-        const float inv = 1.0f / sqrtf(row_sum(ss, 0) / (float)cols + eps);
-        float w[8];
-        ld8(P0 + 8 * j, w);
+            for (int i = 0; i < 8; i++) ss += f[i] * f[i];
+            const float inv = 1.0f / sqrtf(row_sum(ss, 0) / (float)cols + eps);
+            float w[8];
+            ld8(P0 + 8 * j, w);
 #pragma unroll
-        for (int i = 0; i < 8; i++) f[i] = __fmul_rn(__fmul_rn(f[i], inv), w[i]);
-        if (MODE == 2) {
-            float r[8], wn[8];
-            ld8(P1 + e0, r);
-            float ss2 = 0.f;
+            for (int i = 0; i < 8; i++) f[i] = __fmul_rn(__fmul_rn(f[i], inv), w[i]);
+            if (MODE == 2) {
+                float r[8], wn[8];
+                ld8(P1 + e0, r);
+                float ss2 = 0.f;
 #pragma unroll
-            for (int i = 0; i < 8; i++) {
-                f[i] = __fadd_rn(r[i], f[i]);
-                ss2 += f[i] * f[i];
+                for (int i = 0; i < 8; i++) {
+                    f[i] = __fadd_rn(r[i], f[i]);
+                    ss2 += f[i] * f[i];
+                }
+                reinterpret_cast<f32x4_t *>(x_out + e0)[0] = f32x4_t{f[0], f[1], f[2], f[3]};
+                reinterpret_cast<f32x4_t *>(x_out + e0)[1] = f32x4_t{f[4], f[5], f[6], f[7]};
+                const float inv2 = 1.0f / sqrtf(row_sum(ss2, 1) / (float)cols + eps);
+                ld8(P2 + 8 * j, wn);
+#pragma unroll
+                for (int i = 0; i < 8; i++) f[i] = __fmul_rn(__fmul_rn(f[i], inv2), wn[i]);
             }
-            reinterpret_cast<f32x4_t *>(x_out + e0)[0] = f32x4_t{f[0], f[1], f[2], f[3]};
-            reinterpret_cast<f32x4_t *>(x_out + e0)[1] = f32x4_t{f[4], f[5], f[6], f[7]};
-            const float inv2 = 1.0f / sqrtf(row_sum(ss2, 1) / (float)cols + eps);
-            ld8(P2 + 8 * j, wn);
-#pragma unroll
-            for (int i = 0; i < 8; i++) f[i] = __fmul_rn(__fmul_rn(f[i], inv2), wn[i]);
         }
-    }
-    if (MODE == 3) {
-        float u[8];
-        if (x_slices) ldx((size_t)cols, u);
-        else ld8(P0 + e0, u);
+        if (MODE == 3) {
+            float u[8];
+            if (x_slices) ldx(j, (size_t)cols, u);
+            else ld8(P0 + e0, u);
 #pragma unroll
-        for (int i = 0; i < 8; i++) f[i] = gelu_mul_f32(f[i], u[i]);
-    }
-    h8 oh, ol;
-    float fh[8], fl[8];
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-        const float x = pinned(f[i]);
-        const _Float16 hi = (_Float16)x;
-        const _Float16 lo = (_Float16)((x - (float)hi) * 2048.0f);
-        oh[kperm(i)] = hi;
-        ol[kperm(i)] = lo;
-        fh[i] = (float)hi;
-        fl[i] = (float)lo;
-    }
-    float sh = ((fh[0] + fh[1]) + (fh[2] + fh[3])) + ((fh[4] + fh[5]) + (fh[6] + fh[7]));
-    float sl = ((fl[0] + fl[1]) + (fl[2] + fl[3])) + ((fl[4] + fl[5]) + (fl[6] + fl[7]));
-    sh += dpp_f32<0xB1>(sh);
-    sh += dpp_f32<0x4E>(sh);
-    sl += dpp_f32<0xB1>(sl);
-    sl += dpp_f32<0x4E>(sl);
-    const size_t frag = ((size_t)(t >> 5) * (cols / 16) + (j >> 1)) * 64 + (t & 31) + 32 * (j & 1);
-    reinterpret_cast<h8 *>(Xf_hi)[frag] = oh;
-    reinterpret_cast<h8 *>(Xf_lo)[frag] = ol;
-    if ((threadIdx.x & 3) == 0) {
-        const int s = j / 4, jj = s % 8;
-        const size_t o = ((size_t)t * (cols / 256) + s / 8) * 32;
-        const float sums[2] = {sh, sl};
-        _Float16 *dst[2] = {SxA_hi + o, SxA_lo + o};
-#pragma unroll
-        for (int part = 0; part < 2; part++) {
-            const float sum = pinned(sums[part]);
-            const _Float16 hi = (_Float16)sum;
-            const _Float16 lo = (_Float16)(sum - (float)hi);
-            dst[part][jj] = hi;
-            dst[part][8 + jj] = hi;
-            dst[part][16 + jj] = lo;
-            dst[part][24 + jj] = (_Float16)0.f;
+            for (int i = 0; i < 8; i++) f[i] = gelu_mul_f32(f[i], u[i]);
         }
+    };
+    const int octets = cols / 8;
+    const bool one_trip = octets <= (int)blockDim.x;
+    float kept[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    float s = 1.0f;
+    if (inv_s) {
+        // the row's largest magnitude (rows of one trip keep their elements; longer ones are produced again below)
+        float m = 0.f;
+        for (int j = threadIdx.x; j < octets; j += blockDim.x) {
+            produce(j, kept);
+#pragma unroll
+            for (int i = 0; i < 8; i++) m = fmaxf(m, fabsf(kept[i]));
+        }
+        m = wave_max(m);
+        if (lane == 0) red[2][wave] = m;
+        __syncthreads();
+        for (int i = 0; i < nw; i++) m = fmaxf(m, red[2][i]);
+        // s = 2^(9 - floor(log2 m)); rows of zeros (and anything below 2^-112) take 2^121, infinities and NaNs 2^-118
+        const uint32_t e = (uint32_t)max((int)((as_u32(m) >> 23) & 0xFFu), 15);
+        s = as_f32((263u - e) << 23);
+        if (threadIdx.x == 0) inv_s[t] = as_f32((e - 9u) << 23);
     }
+    for (int j = threadIdx.x; j < octets; j += blockDim.x) {
+        float f[8];
+        if (inv_s && one_trip) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) f[i] = kept[i];
+        } else {
+            produce(j, f);
+        }
+        h8 oh, ol;
+        float fh[8], fl[8];
+        const float lo_up = inv_s ? 1.0f : 2048.0f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const float x = pinned(f[i]) * s;
+            const _Float16 hi = (_Float16)x;
+            const _Float16 lo = (_Float16)((x - (float)hi) * lo_up);
+            oh[kperm(i)] = hi;
+            ol[kperm(i)] = lo;
+            fh[i] = (float)hi;
+            fl[i] = (float)lo;
+        }
+        float sh = ((fh[0] + fh[1]) + (fh[2] + fh[3])) + ((fh[4] + fh[5]) + (fh[6] + fh[7]));
+        float sl = ((fl[0] + fl[1]) + (fl[2] + fl[3])) + ((fl[4] + fl[5]) + (fl[6] + fl[7]));
+        sh += dpp_f32<0xB1>(sh);
+        sh += dpp_f32<0x4E>(sh);
+        sl += dpp_f32<0xB1>(sl);
+        sl += dpp_f32<0x4E>(sl);
+        const size_t frag = ((size_t)(t >> 5) * (cols / 16) + (j >> 1)) * 64 + (t & 31) + 32 * (j & 1);
+        reinterpret_cast<h8 *>(Xf_hi)[frag] = oh;
+        reinterpret_cast<h8 *>(Xf_lo)[frag] = ol;
+        if ((threadIdx.x & 3) == 0) {
+            const int sbk = j / 4, jj = sbk % 8;
+            const size_t o = ((size_t)t * (cols / 256) + sbk / 8) * 32;
+            const float sums[2] = {inv_s ? sh + sl : sh, sl};
+            _Float16 *dst[2] = {SxA_hi + o, SxA_lo + o};
+#pragma unroll
+            for (int part = 0; part < 2; part++) {
+                if (part && inv_s) break;       // (one set of sums; the other operand's place holds inv_s)
+                const float sum = pinned(sums[part]);
+                const _Float16 hi = (_Float16)sum;
+                const _Float16 lo = (_Float16)(sum - (float)hi);
+                dst[part][jj] = hi;
+                dst[part][8 + jj] = hi;
+                dst[part][16 + jj] = lo;
+                dst[part][24 + jj] = (_Float16)0.f;
+            }
+        }
     }
 }
 
@@ -274,27 +316,24 @@ struct MmParams {
     const _Float16 *Xf, *SxA;   // fragment-ordered f16 activations (mm_prep_x_kernel), sums of x
     float *Y;
     int rows, cols, batch;
-    float accum;                // 0: store; else add `accum` times the result to Y (the second pass of f32 activations)
-    // Small grids (few tokens x few weight rows): blockIdx.z = part * ksplit + slice.  A workgroup then takes the
-    // superblocks of its K slice only, part 1 reads the low parts of f32 activations, and every z stores its own
-    // batch x rows partial sums behind Y_parts for the fold (ksplit = 0: one launch per part, full K, results in Y).
+    // Small grids (few tokens x few weight rows): blockIdx.z = K slice.  A workgroup then takes the superblocks of
+    // its slice only and every z stores its own batch x rows partial sums behind Y_parts for the fold (ksplit = 0:
+    // full K, results in Y).
     int ksplit;
-    const _Float16 *Xf_lo, *SxA_lo;
     float *Y_parts;
     // Up to three matrices that share the activations (q | k | v of a prompt chunk) in one launch of the 128 x 128
     // tile: blockIdx.y counts the row tiles of W, then of W1, then of W2, each with its own result.
     const uint8_t *W1, *W2;
     float *Y1, *Y2;
     int rows1, rows2;
-    // both = 1 (Q4_K, f32 activations, a grid that fills the chip by itself): a workgroup walks its superblocks twice,
-    // first against the hi parts of the activations, then against the lo parts with the weights' operands scaled by
-    // 2^-11 (an exponent shift: exact), into the same accumulators -- one launch, one result, no second pass over Y
-    int both;
+    // f32 activations (the kernel's LO form): the lo parts' fragments and 1 / s per token row (see mm_prep_rows_kernel)
+    const _Float16 *Xf_lo;
+    const float *inv_s;
 };
 
-__device__ __forceinline__ uint32_t pair_f16(uint32_t masked, uint32_t sc, uint32_t base = 0x64006400u)
+__device__ __forceinline__ uint32_t pair_f16(uint32_t masked, uint32_t sc)
 {
-    return __umul24(masked, sc) + base;     // base: half 1024.0 twice (0x38003800: half 0.5 = 1024 * 2^-11)
+    return __umul24(masked, sc) + 0x64006400u;     // half 1024.0 twice
 }
 
 // what a loader thread (two per tile row) holds per superblock: of each of the four 64-column groups the 16 quant
@@ -332,7 +371,10 @@ constexpr size_t kLdsBytes64 = 2 * (size_t)(kLdsMain + (64 + BN) * PITCH2) * 2 +
 // TM = tokens per workgroup.  128: each multiplying wave owns 64 x 64.  64: each owns 32 x 64 with half the
 // accumulators, the kernel fits 128 registers and 70 KB of LDS, and two workgroups share a compute unit, so that one's
 // barriers and first loads fall into the other's products (the weights are converted once per 64 tokens then).
-template <bool Q6, int TM>
+// LO = true: f32 activations as two f16 parts at the row's own scale.  Every converted weight meets the hi and the lo
+// fragment of a token tile in the same accumulator (twice the matrix instructions per conversion, and the
+// conversions are what a step waits for), and the finished sums are multiplied by 1 / s of their token.
+template <bool Q6, int TM, bool LO>
 __global__ __launch_bounds__(kThreadsMM, TM == 64 ? 2 : 1) void q_mul_mm_kernel(MmParams p)
 {
     constexpr int MT = TM / 64, kLdsMinT = (TM + BN) * PITCH2;
@@ -355,15 +397,13 @@ __global__ __launch_bounds__(kThreadsMM, TM == 64 ? 2 : 1) void q_mul_mm_kernel(
     int nsb = nsb_row, sb0 = 0;                                  // this workgroup's share of them
     size_t ystride = (size_t)p.rows;
     if (p.ksplit) {
-        const int part = blockIdx.z / p.ksplit, slice = blockIdx.z % p.ksplit;
+        const int slice = blockIdx.z;
         nsb = nsb_row / p.ksplit;
         sb0 = slice * nsb;
-        if (part) { p.Xf = p.Xf_lo; p.SxA = p.SxA_lo; }
         p.Y = p.Y_parts + (size_t)blockIdx.z * p.batch * rows_all + ycol;   // partial sums: all matrices' columns side by side
         ystride = (size_t)rows_all;
     }
-    const int nv = p.both ? 2 * nsb : nsb;                      // superblock visits: [hi parts of x | lo parts of x]
-    const int nsteps = nv * 4;
+    const int nsteps = nsb * 4;
 
     if (Q6 && wave >= 4) {
         // ------------------------------------------------------------------ loaders, Q6_K
@@ -454,12 +494,9 @@ __global__ __launch_bounds__(kThreadsMM, TM == 64 ? 2 : 1) void q_mul_mm_kernel(
         const size_t row_bytes = (size_t)nsb_row * 144;
         const uint8_t *wrow = p.W + (size_t)min(r0 + lrow, p.rows - 1) * row_bytes + (size_t)sb0 * 144;
         const size_t sx_off = ((size_t)min(t0 + lrow, p.batch - 1) * nsb_row + sb0) * 32;
-        const _Float16 *sxrow_hi = p.SxA + sx_off, *sxrow_lo = p.SxA_lo + sx_off;
+        const _Float16 *sxrow = p.SxA + sx_off;
 
-        auto fetch_sb = [&](int v, SbRegs &r) __attribute__((always_inline)) {
-            const bool second = v >= nsb;                        // (only with p.both)
-            const int sb = second ? v - nsb : v;
-            const _Float16 *sxrow = second ? sxrow_lo : sxrow_hi;
+        auto fetch_sb = [&](int sb, SbRegs &r) __attribute__((always_inline)) {
             const u32x4_t *w = reinterpret_cast<const u32x4_t *>(wrow + (size_t)sb * 144);
             r.hdr = w[0];
 #pragma unroll
@@ -472,8 +509,6 @@ __global__ __launch_bounds__(kThreadsMM, TM == 64 ? 2 : 1) void q_mul_mm_kernel(
         auto stage = [&](int step, auto gtag, const SbRegs &w) __attribute__((always_inline)) {
             constexpr int G = decltype(gtag)::value;
             const int sb = step >> 2;
-            const bool second = sb >= nsb;                       // the lo parts' visit: operands 2^-11 down
-            const uint32_t base = second ? 0x38003800u : 0x64006400u;
             _Float16 *Bs = main_stage(step);
             {
                 const u32x4_t c = w.q[G];
@@ -483,10 +518,10 @@ __global__ __launch_bounds__(kThreadsMM, TM == 64 ? 2 : 1) void q_mul_mm_kernel(
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     const uint32_t t4 = q[i] >> 4;
-                    lo[2 * i] = pair_f16(q[i] & 0x000F000Fu, s.x, base);
-                    lo[2 * i + 1] = pair_f16((q[i] >> 8) & 0x000F000Fu, s.x, base);
-                    hi[2 * i] = pair_f16(t4 & 0x000F000Fu, s.z, base);
-                    hi[2 * i + 1] = pair_f16((t4 >> 8) & 0x000F000Fu, s.z, base);
+                    lo[2 * i] = pair_f16(q[i] & 0x000F000Fu, s.x);
+                    lo[2 * i + 1] = pair_f16((q[i] >> 8) & 0x000F000Fu, s.x);
+                    hi[2 * i] = pair_f16(t4 & 0x000F000Fu, s.z);
+                    hi[2 * i + 1] = pair_f16((t4 >> 8) & 0x000F000Fu, s.z);
                 }
                 uint4 *dlo = reinterpret_cast<uint4 *>(&Bs[lrow * PITCH + 16 * lh]);
                 uint4 *dhi = reinterpret_cast<uint4 *>(&Bs[lrow * PITCH + 32 + 16 * lh]);
@@ -504,8 +539,7 @@ __global__ __launch_bounds__(kThreadsMM, TM == 64 ? 2 : 1) void q_mul_mm_kernel(
 #pragma unroll
                 for (int gg = 0; gg < 2; gg++) {
                     const uint4 s = q4k_group_scales(w.hdr.y, w.hdr.z, w.hdr.w, 2 * lh + gg);
-                    const float down = second ? 1.0f / 2048.0f : 1.0f;
-                    const float c0 = pinned(-(dmin * (float)s.y + 1024.f * d) * down), c1 = pinned(-(dmin * (float)s.w + 1024.f * d) * down);
+                    const float c0 = pinned(-(dmin * (float)s.y + 1024.f * d)), c1 = pinned(-(dmin * (float)s.w + 1024.f * d));
                     const _Float16 h0 = (_Float16)c0, h1 = (_Float16)c1;
                     const _Float16 l0 = (_Float16)(c0 - (float)h0), l1 = (_Float16)(c1 - (float)h1);
                     hi2[gg] = (uint32_t)__builtin_bit_cast(uint16_t, h0) | ((uint32_t)__builtin_bit_cast(uint16_t, h1) << 16);
@@ -534,14 +568,14 @@ __global__ __launch_bounds__(kThreadsMM, TM == 64 ? 2 : 1) void q_mul_mm_kernel(
         auto step_body = [&](int sb, auto gtag) __attribute__((always_inline)) {
             constexpr int g = decltype(gtag)::value;
             const int step = 4 * sb + g;
-            if (g == 0) fetch_sb(min(sb + 1, nv - 1), wnext);
+            if (g == 0) fetch_sb(min(sb + 1, nsb - 1), wnext);
             if (step + 1 < nsteps) {
                 if (g == 3) wcur = wnext;
                 stage(step + 1, std::integral_constant<int, (g + 1) & 3>{}, wcur);
             }
             __syncthreads();
         };
-        for (int sb = 0; sb < nv; sb++) {
+        for (int sb = 0; sb < nsb; sb++) {
             step_body(sb, std::integral_constant<int, 0>{});
             step_body(sb, std::integral_constant<int, 1>{});
             step_body(sb, std::integral_constant<int, 2>{});
@@ -562,27 +596,34 @@ __global__ __launch_bounds__(kThreadsMM, TM == 64 ? 2 : 1) void q_mul_mm_kernel(
     const int lm = lane & 31, lk = (lane >> 5) * 8;
     const f16v kZero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     // A operands straight from memory: fragment (token tile, k / 16) is 64 lanes x 16 bytes, 1 KB apart along k.
-    // Two register sets, each refilled for two steps ahead as soon as its own step's instructions are issued.
+    // Two register sets, each refilled for two steps ahead as soon as its own step's instructions are issued (LO: one
+    // set of hi and lo fragments, refilled for the next step -- a step is long against the way to the cache).
     const int ntt = (p.batch + 31) / 32;
     const h8 *xa[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; mt++)
         xa[mt] = reinterpret_cast<const h8 *>(p.Xf) + ((size_t)min((t0 + (wm * MT + mt) * 32) / 32, ntt - 1) * (p.cols / 16) + (size_t)sb0 * 16) * 64 + lane;
-    // (with p.both the steps of the second visit read the lo parts' fragments)
-    const ptrdiff_t lo_delta = p.both ? (reinterpret_cast<const h8 *>(p.Xf_lo) - reinterpret_cast<const h8 *>(p.Xf)) - (ptrdiff_t)nsb * 16 * 64 : 0;
+    const ptrdiff_t lo_delta = LO ? reinterpret_cast<const h8 *>(p.Xf_lo) - reinterpret_cast<const h8 *>(p.Xf) : 0;
     auto afrag = [&](int mt, int step, int ks) __attribute__((always_inline)) {
-        return xa[mt][(ptrdiff_t)(step * (KS / 16) + ks) * 64 + (step >= 4 * nsb ? lo_delta : 0)];
+        return xa[mt][(ptrdiff_t)(step * (KS / 16) + ks) * 64];
     };
-    struct ARegs { h8 a[MT][KS / 16]; };
+    auto afrag_lo = [&](int mt, int step, int ks) __attribute__((always_inline)) {
+        return xa[mt][(ptrdiff_t)(step * (KS / 16) + ks) * 64 + lo_delta];
+    };
+    constexpr int AHEAD = LO ? 1 : 2;
+    struct ARegs { h8 a[MT][KS / 16], al[LO ? MT : 1][KS / 16]; };
     auto fetch_a = [&](int step, ARegs &r) __attribute__((always_inline)) {
 #pragma unroll
         for (int mt = 0; mt < MT; mt++)
 #pragma unroll
-            for (int ks = 0; ks < KS / 16; ks++) r.a[mt][ks] = afrag(mt, step, ks);
+            for (int ks = 0; ks < KS / 16; ks++) {
+                r.a[mt][ks] = afrag(mt, step, ks);
+                if (LO) r.al[mt][ks] = afrag_lo(mt, step, ks);
+            }
     };
     ARegs a0, a1;
     fetch_a(0, a0);
-    fetch_a(min(1, nsteps - 1), a1);
+    if (!LO) fetch_a(min(1, nsteps - 1), a1);
     __syncthreads();   // stage 0 is written
 
     auto mul_step = [&](int sb, auto gtag, ARegs &A) __attribute__((always_inline)) {
@@ -601,9 +642,19 @@ __global__ __launch_bounds__(kThreadsMM, TM == 64 ? 2 : 1) void q_mul_mm_kernel(
                 for (int nt = 0; nt < 2; nt++)
                     // a superblock's first product starts from the constant zero: no pass over the accumulators to clear them
                     Cp[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A.a[mt][ks], b[nt], (g == 0 && ks == 0) ? kZero16 : Cp[mt][nt], 0, 0, 0);
-            // this k slice's fragments are spent: ask for the ones of two steps ahead right away
+            if (LO) {
 #pragma unroll
-            for (int mt = 0; mt < MT; mt++) A.a[mt][ks] = afrag(mt, min(step + 2, nsteps - 1), ks);
+                for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+                    for (int nt = 0; nt < 2; nt++)
+                        Cp[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A.al[mt][ks], b[nt], Cp[mt][nt], 0, 0, 0);
+            }
+            // this k slice's fragments are spent: ask for the ones of AHEAD steps on right away
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++) {
+                A.a[mt][ks] = afrag(mt, min(step + AHEAD, nsteps - 1), ks);
+                if (LO) A.al[mt][ks] = afrag_lo(mt, min(step + AHEAD, nsteps - 1), ks);
+            }
         }
         if (g == 3) {
             // ---- end of the superblock: bias + mins through the short second product, then the row scale
@@ -636,11 +687,11 @@ __global__ __launch_bounds__(kThreadsMM, TM == 64 ? 2 : 1) void q_mul_mm_kernel(
         }
         __syncthreads();
     };
-    for (int sb = 0; sb < nv; sb++) {
+    for (int sb = 0; sb < nsb; sb++) {
         mul_step(sb, std::integral_constant<int, 0>{}, a0);
-        mul_step(sb, std::integral_constant<int, 1>{}, a1);
+        mul_step(sb, std::integral_constant<int, 1>{}, LO ? a0 : a1);
         mul_step(sb, std::integral_constant<int, 2>{}, a0);
-        mul_step(sb, std::integral_constant<int, 3>{}, a1);
+        mul_step(sb, std::integral_constant<int, 3>{}, LO ? a0 : a1);
     }
 
     // accumulator layout of the 32x32 tile: column = lane % 32, row = 8*(i/4) + 4*(lane/32) + i%4
@@ -652,10 +703,7 @@ __global__ __launch_bounds__(kThreadsMM, TM == 64 ? 2 : 1) void q_mul_mm_kernel(
 #pragma unroll
             for (int i = 0; i < 16; i++) {
                 const int t = t0 + (wm * MT + mt) * 32 + 8 * (i / 4) + 4 * (lane >> 5) + (i & 3);
-                if (t < p.batch && r < p.rows) {
-                    float *y = &p.Y[(size_t)t * ystride + r];
-                    *y = p.accum != 0.f ? fmaf(p.accum, F[mt][nt][i], *y) : F[mt][nt][i];
-                }
+                if (t < p.batch && r < p.rows) p.Y[(size_t)t * ystride + r] = LO ? F[mt][nt][i] * p.inv_s[t] : F[mt][nt][i];
             }
         }
 }
@@ -1343,14 +1391,6 @@ int launch_matvec_round(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st
 
 constexpr int kSkinnyMaxBatch = 64;
 
-// Q4_K weights, f32 activations and at least one tile per compute unit: a workgroup takes the hi and the lo parts of
-// the activations one after the other (MmParams::both) instead of leaving them to two launches or two sets of workgroups
-bool mm_both_parts(const ksh_kernel_desc &d)
-{
-    const int64_t row_tiles = (d.dims[0] + BN - 1) / BN + (d.dims[3] + BN - 1) / BN + (d.dims[4] + BN - 1) / BN;
-    return d.dtypes[0] == KSH_Q4K && d.dtypes[1] == KSH_F32 && ((d.dims[2] + BM - 1) / BM) * row_tiles >= 256;
-}
-
 int launch_mul_mm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
 {
     const int rows = (int)k.desc.dims[0], cols = (int)k.desc.dims[1], batch = (int)k.desc.dims[2];
@@ -1361,21 +1401,27 @@ int launch_mul_mm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
     _Float16 *Xf_lo = SxA + sx_halves, *SxA_lo = Xf_lo + xf_halves;     // f32 activations only
     const int n = batch * (cols / 8);
     const int n_mat0 = 1 + (k.desc.dims[3] > 0) + (k.desc.dims[4] > 0), prologue = (int)k.desc.dims[5];
+    // f32 activations of the tile: both parts at the row's own scale, 1 / s per row where the small-batch form keeps
+    // the sums of the lo parts (which the tile does not use)
+    const bool tile = k.variant != 1;
+    float *inv_s = f32x && tile ? reinterpret_cast<float *>(SxA_lo) : nullptr;
+    const dim3 pg((unsigned)batch), pb((unsigned)std::min((cols / 8 + 63) / 64 * 64, 1024));     // whole waves: the row-wide reductions read every lane
     if (prologue) {
         // the rows' producer runs inside the preparation: in = W, X, [W1, W2,] then the prologue's operands
         const int xs = (int)(k.desc.dims[7] & 0xFF), xp = (int)(k.desc.dims[7] >> 8);
         const int n_out0 = k.desc.dims[6] ? 1 : n_mat0;                    // (unfolded partial sums are one buffer)
         const float *X = (const float *)a.in[1], *q0 = (const float *)a.in[1 + n_mat0];
-        const dim3 pg((unsigned)batch), pb((unsigned)std::min(cols / 8, 1024));
         const float eps = k.desc.params[0];
         if (prologue == 1)
-            hipLaunchKernelGGL(mm_prep_rows_kernel<1>, pg, pb, 0, st, X, q0, nullptr, nullptr, nullptr, Xf, Xf_lo, SxA, SxA_lo, cols, eps, xs, xp);
+            hipLaunchKernelGGL(mm_prep_rows_kernel<1>, pg, pb, 0, st, X, q0, nullptr, nullptr, nullptr, Xf, Xf_lo, SxA, SxA_lo, cols, eps, xs, xp, inv_s);
         else if (prologue == 2)
             hipLaunchKernelGGL(mm_prep_rows_kernel<2>, pg, pb, 0, st, X, q0, (const float *)a.in[2 + n_mat0], (const float *)a.in[3 + n_mat0], (float *)a.out[n_out0],
-                               Xf, Xf_lo, SxA, SxA_lo, cols, eps, xs, xp);
+                               Xf, Xf_lo, SxA, SxA_lo, cols, eps, xs, xp, inv_s);
         else
-            hipLaunchKernelGGL(mm_prep_rows_kernel<3>, pg, pb, 0, st, X, xs ? X : q0, nullptr, nullptr, nullptr, Xf, Xf_lo, SxA, SxA_lo, cols, eps, xs, xp);
-    } else if (f32x) hipLaunchKernelGGL(mm_prep_x_f32_kernel, dim3((n + 255) / 256), dim3(256), 0, st, (const float *)a.in[1], Xf, Xf_lo, SxA, SxA_lo, batch, cols);
+            hipLaunchKernelGGL(mm_prep_rows_kernel<3>, pg, pb, 0, st, X, xs ? X : q0, nullptr, nullptr, nullptr, Xf, Xf_lo, SxA, SxA_lo, cols, eps, xs, xp, inv_s);
+    } else if (f32x && tile)
+        hipLaunchKernelGGL(mm_prep_rows_kernel<0>, pg, pb, 0, st, (const float *)a.in[1], nullptr, nullptr, nullptr, nullptr, Xf, Xf_lo, SxA, SxA_lo, cols, 0.f, 0, 0, inv_s);
+    else if (f32x) hipLaunchKernelGGL(mm_prep_x_f32_kernel, dim3((n + 255) / 256), dim3(256), 0, st, (const float *)a.in[1], Xf, Xf_lo, SxA, SxA_lo, batch, cols);
     else hipLaunchKernelGGL(mm_prep_x_kernel, dim3((n + 255) / 256), dim3(256), 0, st, (const uint16_t *)a.in[1], Xf, SxA, batch, cols);
     MmParams p;
     p.W = (const uint8_t *)a.in[0];
@@ -1388,7 +1434,7 @@ int launch_mul_mm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
     p.Y1 = rows1 && !unfolded_out ? (float *)a.out[1] : p.Y; p.Y2 = rows2 && !unfolded_out ? (float *)a.out[2] : p.Y;
     if (k.variant == 1) {
         // the small-batch form: one launch, the low parts riding along
-        p.Xf = Xf; p.SxA = SxA; p.accum = 0.f;
+        p.Xf = Xf; p.SxA = SxA;
         const dim3 sg((rows + 31) / 32);
         const int mt = batch <= 32 ? 1 : 2;
         const size_t lds = (size_t)8 * mt * 16 * 64 * 4;
@@ -1405,36 +1451,37 @@ int launch_mul_mm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
     // pass 17.4 ms against 15.8).
     const int tm = (batch <= 64 && k.desc.dtypes[0] != KSH_Q6K) ? 64 : 128;
     const dim3 grid((batch + tm - 1) / tm, (rows + BN - 1) / BN + (rows1 + BN - 1) / BN + (rows2 + BN - 1) / BN);
-    p.ksplit = 0; p.Xf_lo = Xf_lo; p.SxA_lo = SxA_lo; p.Y_parts = nullptr;
-    p.both = mm_both_parts(k.desc) ? 1 : 0;
+    p.Xf = Xf; p.SxA = SxA; p.Xf_lo = Xf_lo; p.inv_s = inv_s;
+    p.ksplit = 0; p.Y_parts = nullptr;
+    const bool q6 = k.desc.dtypes[0] == KSH_Q6K;
+    auto launch_tile = [&](dim3 g) {
+#define KSH_TILE(Q6, TM, LDS) \
+    do { \
+        if (f32x) hipLaunchKernelGGL((q_mul_mm_kernel<Q6, TM, true>), g, dim3(kThreadsMM), LDS, st, p); \
+        else hipLaunchKernelGGL((q_mul_mm_kernel<Q6, TM, false>), g, dim3(kThreadsMM), LDS, st, p); \
+    } while (0)
+        if (q6) KSH_TILE(true, 128, kLdsBytes);
+        else if (tm == 64) KSH_TILE(false, 64, kLdsBytes64);
+        else KSH_TILE(false, 128, kLdsBytes);
+#undef KSH_TILE
+    };
     if (k.variant >= 2) {
-        // few tiles: K slices and both parts of f32 activations as blockIdx.z of one launch, then the fold
-        const int ks = k.variant >> 1, parts = f32x && !p.both ? 2 : 1;
-        p.Xf = Xf; p.SxA = SxA; p.accum = 0.f;
+        // few tiles: K slices as blockIdx.z of one launch, then the fold
+        const int ks = k.variant >> 1;
         p.ksplit = ks;
         const bool unfolded = k.desc.dims[6] != 0;                    // the partial sums are the result: the reader adds them
         p.Y_parts = unfolded ? (float *)a.out[0] : (float *)((f32x ? SxA_lo : SxA) + sx_halves);     // (else behind the prepared activations)
-        const dim3 gz(grid.x, grid.y, ks * parts);
-        if (k.desc.dtypes[0] == KSH_Q6K) hipLaunchKernelGGL((q_mul_mm_kernel<true, 128>), gz, dim3(kThreadsMM), kLdsBytes, st, p);
-        else if (tm == 64) hipLaunchKernelGGL((q_mul_mm_kernel<false, 64>), gz, dim3(kThreadsMM), kLdsBytes64, st, p);
-        else hipLaunchKernelGGL((q_mul_mm_kernel<false, 128>), gz, dim3(kThreadsMM), kLdsBytes, st, p);
+        launch_tile(dim3(grid.x, grid.y, ks));
         hipError_t e3 = hipGetLastError();
         if (e3 != hipSuccess) return hip_fail(e3, "mul_mm (K slices) launch");
         if (unfolded) return 0;
         const int n2 = batch * (rows + rows1 + rows2);
         hipLaunchKernelGGL(mm_parts_fold_kernel, dim3((n2 + 255) / 256), dim3(256), 0, st, (const float *)p.Y_parts, p.Y, p.Y1, p.Y2, batch, rows, rows1, rows2,
-                           ks, parts, 1.0f / 2048.0f);
+                           ks, 1, 1.0f / 2048.0f);
         e3 = hipGetLastError();
         return e3 == hipSuccess ? 0 : hip_fail(e3, "mul_mm fold launch");
     }
-    for (int pass = 0; pass < (f32x && !p.both ? 2 : 1); pass++) {
-        p.Xf = pass ? Xf_lo : Xf;
-        p.SxA = pass ? SxA_lo : SxA;
-        p.accum = pass ? 1.0f / 2048.0f : 0.f;
-        if (k.desc.dtypes[0] == KSH_Q6K) hipLaunchKernelGGL((q_mul_mm_kernel<true, 128>), grid, dim3(kThreadsMM), kLdsBytes, st, p);
-        else if (tm == 64) hipLaunchKernelGGL((q_mul_mm_kernel<false, 64>), grid, dim3(kThreadsMM), kLdsBytes64, st, p);
-        else hipLaunchKernelGGL((q_mul_mm_kernel<false, 128>), grid, dim3(kThreadsMM), kLdsBytes, st, p);
-    }
+    launch_tile(grid);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : hip_fail(e, "mul_mm launch");
 }
@@ -1469,10 +1516,11 @@ int bind_matvec_batch(ksh_kernel &k)
     //   3 gelu(X) * up                  in: ..., up[batch, cols]
     const int64_t prologue = k.desc.dims[5];
     if (prologue < 0 || prologue > 3) return set_error("matvec_batch: prologue %lld (0 none, 1 rmsnorm, 2 add then norm, 3 gelu * up)", (long long)prologue);
-    // dims[6] = 1: the K slices' partial sums are the result, unfolded: out[0] = f32[parts * slices][batch][all rows]
-    // (parts = 2 for F32 activations; the matrices' columns side by side), for a reader that adds them itself --
+    // dims[6] = 1: the K slices' partial sums are the result, unfolded: out[0] = f32[slices][batch][all rows] (the
+    // matrices' columns side by side; slices = grid[2] of the bound kernel), for a reader that adds them itself --
     // dims[7] = slices | parts << 8 of the GEMM whose unfolded result this one's X is (prologues 1 to 3; prologue 3
-    // then reads gate | up from that one buffer and takes no `up` operand)
+    // then reads gate | up from that one buffer and takes no `up` operand).  parts = grid[2] / k_split of that GEMM:
+    // 1 for this library's tile; 2 reads a second set of planes as 2^-11 times the sums of the activations' low parts.
     const int64_t unfolded = k.desc.dims[6], x_slices = k.desc.dims[7] & 0xFF, x_parts = k.desc.dims[7] >> 8;
     if (unfolded < 0 || unfolded > 1) return set_error("matvec_batch: dims[6]=%lld (0, or 1 for unfolded partial sums)", (long long)unfolded);
     if (k.desc.dims[7] && (!prologue || x_slices < 1 || x_slices > 64 || x_parts < 1 || x_parts > 2))
@@ -1514,25 +1562,24 @@ int bind_matvec_batch(ksh_kernel &k)
     // about one workgroup per compute unit; every slice stores its partial sums and a second launch adds them in a
     // fixed order.  sched.k_split names the slice count (a divisor of cols / 256; 1 = none).
     const int64_t row_tiles = (rows + BN - 1) / BN + (rows1 + BN - 1) / BN + (rows2 + BN - 1) / BN;
-    const int64_t tiles = ((batch + BM - 1) / BM) * row_tiles, nsb = cols / 256, parts = f32x && !mm_both_parts(k.desc) ? 2 : 1;
+    const int64_t tiles = ((batch + BM - 1) / BM) * row_tiles, nsb = cols / 256;
     int64_t ks = 1;
     if (k.desc.sched.k_split) {
         ks = k.desc.sched.k_split;
         if (nsb % ks) return set_error("matvec_batch: k_split=%lld does not divide the %lld superblocks of a row", (long long)ks, (long long)nsb);
     } else {
-        while (tiles * parts * ks < 256 && nsb % (ks * 2) == 0 && nsb / (ks * 2) >= 2) ks *= 2;   // (a slice of one superblock is all prologue)
+        while (tiles * ks < 256 && nsb % (ks * 2) == 0 && nsb / (ks * 2) >= 2) ks *= 2;   // (a slice of one superblock is all prologue)
     }
-    // (f32 activations with fewer tiles than compute units: both parts in one launch even without a K split)
-    const bool z_form = unfolded || ks > 1 || (parts == 2 && tiles < 256 && !k.desc.sched.k_split);
+    const bool z_form = unfolded || ks > 1;
     k.variant = z_form ? (int)(ks << 1) : 0;
-    if (z_form && !unfolded) k.scratch_bytes += (size_t)parts * ks * batch * rows_all * 4;
+    if (z_form && !unfolded) k.scratch_bytes += (size_t)ks * batch * rows_all * 4;
     if (unfolded) {
         const int keep = prologue == 2 ? 1 : 0;                       // (the add-then-norm prologue's x_new stays an output)
         if (keep) { k.out_bytes[1] = k.out_bytes[n_mat]; k.out_align[1] = 16; }
-        k.out_bytes[0] = (size_t)parts * ks * batch * rows_all * 4; k.out_align[0] = 16;
+        k.out_bytes[0] = (size_t)ks * batch * rows_all * 4; k.out_align[0] = 16;
         k.info.n_outputs = 1 + keep;
     }
-    set_launch(k, (uint32_t)((batch + BM - 1) / BM), (uint32_t)row_tiles, z_form ? (uint32_t)(ks * parts) : 1, kThreadsMM,
+    set_launch(k, (uint32_t)((batch + BM - 1) / BM), (uint32_t)row_tiles, z_form ? (uint32_t)ks : 1, kThreadsMM,
                (uint32_t)kLdsBytes);
     k.info.sched.tg = kThreadsMM; k.info.sched.nsg = kThreadsMM / 64; k.info.sched.nr0 = BN; k.info.sched.k_split = (uint32_t)ks; k.info.sched.lds_tile = KS;
     set_name(k, "mul_mm_%s_%dx%dx%d%s%s%s%s", q6 ? "q6k" : "q4k", BM, BN, KS, f32x ? "_f32x" : "", z_form ? "_kz" : "", n_mat == 3 ? "_x3" : n_mat == 2 ? "_x2" : "",

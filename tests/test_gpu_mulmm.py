@@ -150,8 +150,8 @@ def test_mul_mm_q6k_cfg2_shape(ctx, eng):
                                                          (DType.Q6K, DType.F32, 70, 200, 1024, None), (DType.Q4K, DType.F32, 300, 2048, 512, None),
                                                          (DType.Q4K, DType.BF16, 256, 384, 8192, 8), (DType.Q4K, DType.F32, 65, 128, 256, None)])
 def test_mul_mm_k_slices(ctx, wdt, xdt, batch, rows, cols, ks):
-    """Few tiles: a row's superblocks go to K slices (and the hi and lo parts of f32 activations to workgroups of the
-    same launch), every slice stores its partial sums and a fold adds them in a fixed order.  Against the float64
+    """Few tiles: a row's superblocks go to K slices (rows of at least four superblocks), every slice stores its
+    partial sums and a fold adds them in a fixed order.  Against the float64
     product at the accuracy of the whole-row launch (bf16 activations: 1e-3 against the oracle's f32 loop; f32
     activations: 2e-5), twice for bit-reproducibility, ragged tiles in both directions."""
     nb = rows * cols // 256
@@ -163,8 +163,7 @@ def test_mul_mm_k_slices(ctx, wdt, xdt, batch, rows, cols, ks):
     else:
         xin = ctx.buffer_f32(x)
     k = ctx.compile(hip.make_desc(hip.Kind.MATVEC_BATCH, (rows, cols, batch), (wdt, xdt, DType.F32), (), dict(k_split=ks) if ks else None))
-    parts = 2 if xdt == DType.F32 else 1
-    assert "_kz" in k.name and k.grid[2] == k.info.sched.k_split * parts, (k.name, k.info.sched.k_split)
+    assert ("_kz" in k.name) == (k.info.sched.k_split > 1) == (cols >= 1024) and k.grid[2] == k.info.sched.k_split, (k.name, k.info.sched.k_split)
     assert (cols // 256) % k.info.sched.k_split == 0 and (ks is None or k.info.sched.k_split == ks)
     by, bw = ctx.buffer_empty_f32(batch * rows), ctx.buffer_bytes(w)
     runs = []
@@ -195,7 +194,7 @@ def test_mul_mm_matrices_sharing_the_activations(ctx, xdt, batch, rows3, cols):
         xin = ctx.buffer_f32(x)
     k = ctx.compile(hip.make_desc(hip.Kind.MATVEC_BATCH, (rows3[0], cols, batch, rows3[1], rows3[2]), (DType.Q4K, xdt, DType.F32)))
     assert k.name.endswith("_x%d" % len(ws)), k.name
-    assert ("_kz" in k.name) == (xdt == DType.F32 and batch < 2048), k.name      # (512 columns of bf16: two superblocks, no slices)
+    assert ("_kz" in k.name) == (cols >= 1024), k.name      # (rows of one or two superblocks: no slices)
     bws = [ctx.buffer_bytes(w) for w in ws]
     outs = [ctx.buffer_empty_f32(batch * r) for r in rows3 if r]
     ctx.encode_multi(k, [bws[0], xin] + bws[1:], outs)
@@ -253,7 +252,7 @@ def test_mul_mm_with_the_rows_producer_inside(ctx, mode, batch, rows3, cols):
 
 @pytest.mark.parametrize("batch", [96, 300])
 def test_mul_mm_unfolded_results_feed_the_next_preparation(ctx, batch):
-    """dims[6] = 1 leaves a GEMM's K slices (and the two parts of its f32 activations) as partial sums for a reader
+    """dims[6] = 1 leaves a GEMM's K slices as partial sums for a reader
     that adds them itself; dims[7] tells the next GEMM's prologue that its X is such a buffer.  The chain o-projection
     -> add-then-norm -> gate | up -> gelu * up -> down gives the very numbers of the same chain with every result
     folded by its own launch."""
@@ -280,15 +279,15 @@ def test_mul_mm_unfolded_results_feed_the_next_preparation(ctx, batch):
     # unfolded: the partial sums travel
     ko = ctx.compile(desc((hidden, hidden, batch, 0, 0, 0, 1)))
     zo = ko.grid[2]
-    assert ko.name.endswith("_unfolded") and zo == 2 * ko.info.sched.k_split
+    assert ko.name.endswith("_unfolded") and zo == ko.info.sched.k_split
     po = ctx.buffer_empty_f32(zo * batch * hidden)
     run(ko, [bo, a], [po])
-    kg = ctx.compile(desc((ffn, hidden, batch, ffn, 0, 2, 1, ko.info.sched.k_split | 2 << 8)))
+    kg = ctx.compile(desc((ffn, hidden, batch, ffn, 0, 2, 1, ko.info.sched.k_split | (zo // ko.info.sched.k_split) << 8)))
     zg = kg.grid[2]
     pg, res_b = ctx.buffer_empty_f32(zg * batch * 2 * ffn), ctx.buffer_f32(res0)
     run(kg, [bg, po, bu, w_post, res_b, w_norm], [pg, res_b])
     out_b = ctx.buffer_empty_f32(batch * hidden)
-    run(ctx.compile(desc((hidden, ffn, batch, 0, 0, 3, 0, kg.info.sched.k_split | 2 << 8))), [bd, pg], [out_b])
+    run(ctx.compile(desc((hidden, ffn, batch, 0, 0, 3, 0, kg.info.sched.k_split | (zg // kg.info.sched.k_split) << 8))), [bd, pg], [out_b])
     assert np.array_equal(ctx.read_f32(res_a, batch * hidden), ctx.read_f32(res_b, batch * hidden))
     assert np.array_equal(ctx.read_f32(out_a, batch * hidden), ctx.read_f32(out_b, batch * hidden))
     assert np.isfinite(ctx.read_f32(out_a, batch * hidden)).all() and np.abs(ctx.read_f32(out_a, batch * hidden)).max() > 0
@@ -296,15 +295,20 @@ def test_mul_mm_unfolded_results_feed_the_next_preparation(ctx, batch):
 
 @pytest.mark.parametrize("unfolded,k_split", [(0, 0), (1, 0), (0, 2), (1, 4)])
 def test_mul_mm_f32_both_parts_in_one_workgroup(ctx, unfolded, k_split):
-    """Q4_K weights, f32 activations and at least 256 tiles: a workgroup walks its superblocks against the hi parts
-    and then against the lo parts (weights' operands 2^-11 down, exactly) into the same accumulators -- one launch, one
-    result (or one set of partial sums; with K slices asked for, one per slice).  1024 tokens x 4096 rows x 1024
-    columns against float64, a row of small and a row of large activations among them."""
+    """f32 activations on the tile: each row is scaled by its own power of two and split into two f16 parts at that
+    scale, and every converted weight meets both parts in the same accumulator -- one launch, one result (or one set
+    of partial sums; with K slices asked for, one per slice).  1024 tokens x 4096 rows x 1024 columns against
+    float64; among the rows a small one, a large one, one far beyond the f16 range, one of zeros and one whose
+    largest element is 10^7 times the others."""
     batch, rows, cols = 1024, 4096, 1024
     w = synth.q4k_blocks(rows * cols // 256, 690)
     x = synth.normal_f32(batch * cols, 691).reshape(batch, cols)
     x[3] *= 1e-3
     x[4] *= 300.0
+    x[6] *= 1e12
+    x[7] = 0.0
+    x[8] *= 1e-3
+    x[8, 5] = 1e4
     k = ctx.compile(hip.make_desc(hip.Kind.MATVEC_BATCH, (rows, cols, batch, 0, 0, 0, unfolded), (DType.Q4K, DType.F32, DType.F32), (),
                                   dict(k_split=k_split) if k_split else None))
     nz = max(1, k_split)
@@ -316,8 +320,9 @@ def test_mul_mm_f32_both_parts_in_one_workgroup(ctx, unfolded, k_split):
         got = ctx.read_f32(y, nz * batch * rows).reshape(nz, batch, rows).astype(np.float64).sum(axis=0)
     else:
         got = ctx.read_f32(y, batch * rows).reshape(batch, rows)
-    worst = max(float(rel_err(got[t], oracle.matvec_f64(oracle.Q4K, w, rows, cols, x[t])).max()) for t in (0, 3, 4, 5, 511, 1023))
+    worst = max(float(rel_err(got[t], oracle.matvec_f64(oracle.Q4K, w, rows, cols, x[t])).max()) for t in (0, 3, 4, 5, 6, 8, 511, 1023))
     assert worst <= 2e-5, worst
+    assert not got[7].any()
 
 
 def test_mul_mm_k_slices_must_divide_the_row(ctx):

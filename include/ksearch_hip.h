@@ -73,10 +73,9 @@ enum ksh_kind {
      * dims[6] = 1: the tile's K slices stay unfolded -- out[0] is then f32[slices][batch][rows + rows1 + rows2]
      *   (slices = info.grid[2] = info.sched.k_split, the matrices' columns side by side) for a reader that adds them
      *   itself; out[1] = x_new with prologue 2.
-     * dims[7] = slices | parts << 8 of the GEMM whose unfolded result this one's X is (with a prologue; prologue 3
-     *   then reads gate | up from that one buffer and takes no `up` operand; parts = info.grid[2] / k_split of that
-     *   GEMM, 1 for this library's tile).  The sums are added in the fold's order, so a chain of GEMMs gives the same
-     *   numbers with and without its folds.
+     * dims[7] = the slices (info.grid[2]) of the GEMM whose unfolded result this one's X is (with a prologue;
+     *   prologue 3 then reads gate | up from that one buffer and takes no `up` operand).  The sums are added in the
+     *   fold's order, so a chain of GEMMs gives the same numbers with and without its folds.
      * F32 activations travel as hi + lo f16 parts.  The tile scales every row by its own power of two first (any
      * finite f32 row fits); the small-batch form does not: there |x| must stay below 65504.
      * sched.nr0 = 32 | 128 picks the small-batch form (Q4_K, up to 64 tokens, one matrix) or the 128 x 128 tile;

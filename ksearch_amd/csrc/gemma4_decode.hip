@@ -488,14 +488,14 @@ int forward_prefill_chunk4(ksh_gemma4 *m, const uint32_t *tokens, int t)
         if (inside && L.dt_gate == L.dt_up) {
             const size_t T = kChunk4;
             if (get(m, KSH_MATVEC_BATCH, {h, P.qd, tp, 0, 0, 0, 1}, {L.dt_o, KSH_F32, KSH_F32}, {c.eps}, &u_o) ||
-                get(m, KSH_MATVEC_BATCH, {L.ffn, h, tp, L.ffn, 0, 2, 1, (int64_t)(u_o->info.sched.k_split | (u_o->info.grid[2] / u_o->info.sched.k_split) << 8)}, {L.dt_gate, KSH_F32, KSH_F32}, {c.eps}, &u_gu))
+                get(m, KSH_MATVEC_BATCH, {L.ffn, h, tp, L.ffn, 0, 2, 1, (int64_t)u_o->info.grid[2]}, {L.dt_gate, KSH_F32, KSH_F32}, {c.eps}, &u_gu))
                 return 1;
             travel = u_o->out_bytes[0] <= kPartsRows4 * T * c.hidden * 4 && u_gu->out_bytes[0] <= ksh_buffer_size(m->c_pg);
         }
         if (travel) {
             if (enc(m, u_o, {L.wo, m->c_o}, {m->c_po}, n) ||
                 enc(m, u_gu, {L.wgate, m->c_po, L.wup, L.post_attn_norm, m->c_x, L.ffn_norm}, {m->c_pg, m->c_x}, n) ||
-                mm_pro(L.dt_down, {h, L.ffn, tp, 0, 0, 3, 0, (int64_t)(u_gu->info.sched.k_split | (u_gu->info.grid[2] / u_gu->info.sched.k_split) << 8)}, {L.wdown, m->c_pg}, {m->c_y}))
+                mm_pro(L.dt_down, {h, L.ffn, tp, 0, 0, 3, 0, (int64_t)u_gu->info.grid[2]}, {L.wdown, m->c_pg}, {m->c_y}))
                 return 1;
         } else if (
             mm(L.dt_o, h, P.qd, L.wo, m->c_o, m->c_y) ||

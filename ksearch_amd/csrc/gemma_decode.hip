@@ -427,7 +427,7 @@ int forward_prefill_chunk(ksh_gemma *m, const uint32_t *tokens, int t)
     bool travel = false;
     if (fused && c.n_layers > 1) {
         const size_t T = kChunk;
-        auto parts_of = [](ksh_kernel *kk) { return (int64_t)(kk->info.sched.k_split | (kk->info.grid[2] / kk->info.sched.k_split) << 8); };
+        auto parts_of = [](ksh_kernel *kk) { return (int64_t)kk->info.grid[2]; };      // the planes of its unfolded result
         if (get(m, KSH_MATVEC_BATCH, {c.hidden, qd, tp, 0, 0, 0, 1}, {KSH_Q4K, KSH_F32, KSH_F32}, {c.eps}, &u_o) ||
             get(m, KSH_MATVEC_BATCH, {c.ffn, c.hidden, tp, c.ffn, 0, 2, 1, parts_of(u_o)}, {KSH_Q4K, KSH_F32, KSH_F32}, {c.eps}, &u_gu) ||
             get(m, KSH_MATVEC_BATCH, {c.hidden, c.ffn, tp, 0, 0, 3, 1, parts_of(u_gu)}, {KSH_Q4K, KSH_F32, KSH_F32}, {c.eps}, &u_down) ||

@@ -157,12 +157,12 @@ template <int MODE>
 __global__ __launch_bounds__(1024) void mm_prep_rows_kernel(const float *__restrict__ X, const float *__restrict__ P0, const float *P1,
                                                              const float *__restrict__ P2, float *x_out, _Float16 *__restrict__ Xf_hi,
                                                              _Float16 *__restrict__ Xf_lo, _Float16 *__restrict__ SxA_hi,
-                                                             _Float16 *__restrict__ SxA_lo, int cols, float eps, int x_slices, int x_parts,
+                                                             _Float16 *__restrict__ SxA_lo, int cols, float eps, int x_slices,
                                                              float *__restrict__ inv_s)
 {
-    // x_slices != 0: X is the unfolded partial sums of the GEMM that produced it, [part * x_slices + slice][row][stride]
-    // with stride = cols (MODE 3: 2 * cols, gate | up side by side, and `up` is read from there); the slices are added
-    // here in the fold's order, the second part (the low parts of that GEMM's activations) scaled by 2^-11
+    // x_slices != 0: X is the unfolded partial sums of the GEMM that produced it, [slice][row][stride] with stride =
+    // cols (MODE 3: 2 * cols, gate | up side by side, and `up` is read from there); the slices are added here in the
+    // fold's order
     __shared__ float red[3][16];
     const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
     auto ld8 = [](const float *p, float (&v)[8]) __attribute__((always_inline)) {
@@ -186,18 +186,6 @@ __global__ __launch_bounds__(1024) void mm_prep_rows_kernel(const float *__restr
             ld8(src + (size_t)k * x_plane, a);
 #pragma unroll
             for (int i = 0; i < 8; i++) v[i] += a[i];
-        }
-        if (x_parts == 2) {
-            float l[8];
-            ld8(src + (size_t)x_slices * x_plane, l);
-            for (int k = 1; k < x_slices; k++) {
-                float a[8];
-                ld8(src + (size_t)(x_slices + k) * x_plane, a);
-#pragma unroll
-                for (int i = 0; i < 8; i++) l[i] += a[i];
-            }
-#pragma unroll
-            for (int i = 0; i < 8; i++) v[i] = fmaf(1.0f / 2048.0f, l[i], v[i]);
         }
     };
     // the row's elements 8j .. 8j+7 (the norms run with cols / 8 threads, one trip; plain rows and gelu * up of longer
@@ -1187,18 +1175,13 @@ __global__ __launch_bounds__(256) void mm_round_fold_kernel(const float *__restr
 // (parts = 2) come in scaled.  The partial sums hold the columns of up to three matrices side by side (rows0 | rows1 |
 // rows2 per token), each with a result buffer of its own.
 __global__ __launch_bounds__(256) void mm_parts_fold_kernel(const float *__restrict__ part, float *__restrict__ y0, float *__restrict__ y1, float *__restrict__ y2,
-                                                             int batch, int rows0, int rows1, int rows2, int slices, int parts, float lo_scale)
+                                                             int batch, int rows0, int rows1, int rows2, int slices)
 {
     const int rows_all = rows0 + rows1 + rows2, n = batch * rows_all;
     const int i = blockIdx.x * 256 + threadIdx.x;
     if (i >= n) return;
     float s = part[i];
     for (int k = 1; k < slices; k++) s += part[(size_t)k * n + i];
-    if (parts == 2) {
-        float l = part[(size_t)slices * n + i];
-        for (int k = 1; k < slices; k++) l += part[(size_t)(slices + k) * n + i];
-        s = fmaf(lo_scale, l, s);
-    }
     if (!rows1) { y0[i] = s; return; }
     const int t = i / rows_all, c = i - t * rows_all;
     if (c < rows0) y0[(size_t)t * rows0 + c] = s;
@@ -1391,6 +1374,21 @@ int launch_matvec_round(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st
 
 constexpr int kSkinnyMaxBatch = 64;
 
+// Tokens per workgroup of the tile.  64 (Q4_K): up to 64 tokens (the other half of a 128-token tile would be empty
+// rows), and wherever the 128-token tiles and their K slices are fewer than the compute units (bf16 activations) or
+// than twice the compute units (f32 activations, whose tile runs two products per converted weight) -- two
+// workgroups share a compute unit then, and twice as many of them fill the chip.  Beyond that the 128-token tile
+// (bf16, cfg2: 33.7 us against 40.3 with 64-token tiles; f32, prompts of 256 / 1024 / 4000 tokens through cfg4's
+// model: 5.05 / 14.1 / 67.7 ms with this rule, 5.07 / 14.25 / 68.0 with 64-token tiles throughout, 5.3 / 14.9 / 72.7
+// with 128-token tiles from 65 tokens on).
+int mm_tile_tokens(const ksh_kernel_desc &d, int64_t ks)
+{
+    if (d.dtypes[0] == KSH_Q6K) return 128;
+    const int64_t row_tiles = (d.dims[0] + BN - 1) / BN + (d.dims[3] + BN - 1) / BN + (d.dims[4] + BN - 1) / BN;
+    const int64_t fill = d.dtypes[1] == KSH_F32 ? 512 : 256;
+    return d.dims[2] <= 64 || ((d.dims[2] + BM - 1) / BM) * row_tiles * ks < fill ? 64 : 128;
+}
+
 int launch_mul_mm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
 {
     const int rows = (int)k.desc.dims[0], cols = (int)k.desc.dims[1], batch = (int)k.desc.dims[2];
@@ -1408,19 +1406,19 @@ int launch_mul_mm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
     const dim3 pg((unsigned)batch), pb((unsigned)std::min((cols / 8 + 63) / 64 * 64, 1024));     // whole waves: the row-wide reductions read every lane
     if (prologue) {
         // the rows' producer runs inside the preparation: in = W, X, [W1, W2,] then the prologue's operands
-        const int xs = (int)(k.desc.dims[7] & 0xFF), xp = (int)(k.desc.dims[7] >> 8);
+        const int xs = (int)k.desc.dims[7];
         const int n_out0 = k.desc.dims[6] ? 1 : n_mat0;                    // (unfolded partial sums are one buffer)
         const float *X = (const float *)a.in[1], *q0 = (const float *)a.in[1 + n_mat0];
         const float eps = k.desc.params[0];
         if (prologue == 1)
-            hipLaunchKernelGGL(mm_prep_rows_kernel<1>, pg, pb, 0, st, X, q0, nullptr, nullptr, nullptr, Xf, Xf_lo, SxA, SxA_lo, cols, eps, xs, xp, inv_s);
+            hipLaunchKernelGGL(mm_prep_rows_kernel<1>, pg, pb, 0, st, X, q0, nullptr, nullptr, nullptr, Xf, Xf_lo, SxA, SxA_lo, cols, eps, xs, inv_s);
         else if (prologue == 2)
             hipLaunchKernelGGL(mm_prep_rows_kernel<2>, pg, pb, 0, st, X, q0, (const float *)a.in[2 + n_mat0], (const float *)a.in[3 + n_mat0], (float *)a.out[n_out0],
-                               Xf, Xf_lo, SxA, SxA_lo, cols, eps, xs, xp, inv_s);
+                               Xf, Xf_lo, SxA, SxA_lo, cols, eps, xs, inv_s);
         else
-            hipLaunchKernelGGL(mm_prep_rows_kernel<3>, pg, pb, 0, st, X, xs ? X : q0, nullptr, nullptr, nullptr, Xf, Xf_lo, SxA, SxA_lo, cols, eps, xs, xp, inv_s);
+            hipLaunchKernelGGL(mm_prep_rows_kernel<3>, pg, pb, 0, st, X, xs ? X : q0, nullptr, nullptr, nullptr, Xf, Xf_lo, SxA, SxA_lo, cols, eps, xs, inv_s);
     } else if (f32x && tile)
-        hipLaunchKernelGGL(mm_prep_rows_kernel<0>, pg, pb, 0, st, (const float *)a.in[1], nullptr, nullptr, nullptr, nullptr, Xf, Xf_lo, SxA, SxA_lo, cols, 0.f, 0, 0, inv_s);
+        hipLaunchKernelGGL(mm_prep_rows_kernel<0>, pg, pb, 0, st, (const float *)a.in[1], nullptr, nullptr, nullptr, nullptr, Xf, Xf_lo, SxA, SxA_lo, cols, 0.f, 0, inv_s);
     else if (f32x) hipLaunchKernelGGL(mm_prep_x_f32_kernel, dim3((n + 255) / 256), dim3(256), 0, st, (const float *)a.in[1], Xf, Xf_lo, SxA, SxA_lo, batch, cols);
     else hipLaunchKernelGGL(mm_prep_x_kernel, dim3((n + 255) / 256), dim3(256), 0, st, (const uint16_t *)a.in[1], Xf, SxA, batch, cols);
     MmParams p;
@@ -1445,11 +1443,7 @@ int launch_mul_mm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
         const hipError_t e2 = hipGetLastError();
         return e2 == hipSuccess ? 0 : hip_fail(e2, "mul_mm (small batch) launch");
     }
-    // up to 64 tokens: the 64-token tile (the other half of a 128-token tile would be empty rows).  Beyond that the
-    // 128-token tile: two 64-token workgroups per compute unit convert every weight twice as often, and the
-    // conversions, not the products, are what a step waits for (cfg2: 40.3 us against 33.7, a 1024-token prompt
-    // pass 17.4 ms against 15.8).
-    const int tm = (batch <= 64 && k.desc.dtypes[0] != KSH_Q6K) ? 64 : 128;
+    const int tm = mm_tile_tokens(k.desc, k.variant >= 2 ? k.variant >> 1 : 1);
     const dim3 grid((batch + tm - 1) / tm, (rows + BN - 1) / BN + (rows1 + BN - 1) / BN + (rows2 + BN - 1) / BN);
     p.Xf = Xf; p.SxA = SxA; p.Xf_lo = Xf_lo; p.inv_s = inv_s;
     p.ksplit = 0; p.Y_parts = nullptr;
@@ -1477,7 +1471,7 @@ int launch_mul_mm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
         if (unfolded) return 0;
         const int n2 = batch * (rows + rows1 + rows2);
         hipLaunchKernelGGL(mm_parts_fold_kernel, dim3((n2 + 255) / 256), dim3(256), 0, st, (const float *)p.Y_parts, p.Y, p.Y1, p.Y2, batch, rows, rows1, rows2,
-                           ks, 1, 1.0f / 2048.0f);
+                           ks);
         e3 = hipGetLastError();
         return e3 == hipSuccess ? 0 : hip_fail(e3, "mul_mm fold launch");
     }
@@ -1518,13 +1512,12 @@ int bind_matvec_batch(ksh_kernel &k)
     if (prologue < 0 || prologue > 3) return set_error("matvec_batch: prologue %lld (0 none, 1 rmsnorm, 2 add then norm, 3 gelu * up)", (long long)prologue);
     // dims[6] = 1: the K slices' partial sums are the result, unfolded: out[0] = f32[slices][batch][all rows] (the
     // matrices' columns side by side; slices = grid[2] of the bound kernel), for a reader that adds them itself --
-    // dims[7] = slices | parts << 8 of the GEMM whose unfolded result this one's X is (prologues 1 to 3; prologue 3
-    // then reads gate | up from that one buffer and takes no `up` operand).  parts = grid[2] / k_split of that GEMM:
-    // 1 for this library's tile; 2 reads a second set of planes as 2^-11 times the sums of the activations' low parts.
-    const int64_t unfolded = k.desc.dims[6], x_slices = k.desc.dims[7] & 0xFF, x_parts = k.desc.dims[7] >> 8;
+    // dims[7] = the slices (grid[2]) of the GEMM whose unfolded result this one's X is (prologues 1 to 3; prologue 3
+    // then reads gate | up from that one buffer and takes no `up` operand)
+    const int64_t unfolded = k.desc.dims[6], x_slices = k.desc.dims[7];
     if (unfolded < 0 || unfolded > 1) return set_error("matvec_batch: dims[6]=%lld (0, or 1 for unfolded partial sums)", (long long)unfolded);
-    if (k.desc.dims[7] && (!prologue || x_slices < 1 || x_slices > 64 || x_parts < 1 || x_parts > 2))
-        return set_error("matvec_batch: X as unfolded partial sums (dims[7]=%lld) takes a prologue, 1 to 64 slices and 1 or 2 parts", (long long)k.desc.dims[7]);
+    if (x_slices && (!prologue || x_slices < 1 || x_slices > 64))
+        return set_error("matvec_batch: X as unfolded partial sums (dims[7]=%lld) takes a prologue and 1 to 64 slices", (long long)k.desc.dims[7]);
     if (prologue) {
         if (!f32x) return set_error("matvec_batch: a prologue takes F32 activations");
         if (prologue != 3 && (cols > 8192 || cols % 512)) return set_error("matvec_batch: a norm prologue takes rows of a multiple of 512 up to 8192 columns, got %lld", (long long)cols);
@@ -1535,7 +1528,7 @@ int bind_matvec_batch(ksh_kernel &k)
         if (prologue == 2) { add_in(vec); add_in(mat); add_in(vec); k.out_bytes[n_mat] = mat; k.out_align[n_mat] = 16; k.info.n_outputs = n_mat + 1; }
         if (prologue == 3 && !x_slices) add_in(mat);
         k.info.n_inputs = ni;
-        if (x_slices) k.in_bytes[1] = (size_t)x_slices * x_parts * mat * (prologue == 3 ? 2 : 1);
+        if (x_slices) k.in_bytes[1] = (size_t)x_slices * mat * (prologue == 3 ? 2 : 1);
     }
     // f16 copy of X plus the min-term operand (32 halves per token and superblock)
     k.scratch_bytes = ((size_t)((batch + 31) / 32 * 32) * cols * 2 + (size_t)batch * (cols / 256) * 64) * (f32x ? 2 : 1);
@@ -1579,8 +1572,9 @@ int bind_matvec_batch(ksh_kernel &k)
         k.out_bytes[0] = (size_t)ks * batch * rows_all * 4; k.out_align[0] = 16;
         k.info.n_outputs = 1 + keep;
     }
-    set_launch(k, (uint32_t)((batch + BM - 1) / BM), (uint32_t)row_tiles, z_form ? (uint32_t)ks : 1, kThreadsMM,
-               (uint32_t)kLdsBytes);
+    const int tm = mm_tile_tokens(k.desc, ks);
+    set_launch(k, (uint32_t)((batch + tm - 1) / tm), (uint32_t)row_tiles, z_form ? (uint32_t)ks : 1, kThreadsMM,
+               (uint32_t)(tm == 64 ? kLdsBytes64 : kLdsBytes));
     k.info.sched.tg = kThreadsMM; k.info.sched.nsg = kThreadsMM / 64; k.info.sched.nr0 = BN; k.info.sched.k_split = (uint32_t)ks; k.info.sched.lds_tile = KS;
     set_name(k, "mul_mm_%s_%dx%dx%d%s%s%s%s", q6 ? "q6k" : "q4k", BM, BN, KS, f32x ? "_f32x" : "", z_form ? "_kz" : "", n_mat == 3 ? "_x3" : n_mat == 2 ? "_x2" : "",
              prologue == 1 ? "_rms" : prologue == 2 ? "_addrms" : prologue == 3 ? "_gelu" : "");

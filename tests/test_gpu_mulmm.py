@@ -282,12 +282,12 @@ def test_mul_mm_unfolded_results_feed_the_next_preparation(ctx, batch):
     assert ko.name.endswith("_unfolded") and zo == ko.info.sched.k_split
     po = ctx.buffer_empty_f32(zo * batch * hidden)
     run(ko, [bo, a], [po])
-    kg = ctx.compile(desc((ffn, hidden, batch, ffn, 0, 2, 1, ko.info.sched.k_split | (zo // ko.info.sched.k_split) << 8)))
+    kg = ctx.compile(desc((ffn, hidden, batch, ffn, 0, 2, 1, zo)))
     zg = kg.grid[2]
     pg, res_b = ctx.buffer_empty_f32(zg * batch * 2 * ffn), ctx.buffer_f32(res0)
     run(kg, [bg, po, bu, w_post, res_b, w_norm], [pg, res_b])
     out_b = ctx.buffer_empty_f32(batch * hidden)
-    run(ctx.compile(desc((hidden, ffn, batch, 0, 0, 3, 0, kg.info.sched.k_split | (zg // kg.info.sched.k_split) << 8))), [bd, pg], [out_b])
+    run(ctx.compile(desc((hidden, ffn, batch, 0, 0, 3, 0, zg))), [bd, pg], [out_b])
     assert np.array_equal(ctx.read_f32(res_a, batch * hidden), ctx.read_f32(res_b, batch * hidden))
     assert np.array_equal(ctx.read_f32(out_a, batch * hidden), ctx.read_f32(out_b, batch * hidden))
     assert np.isfinite(ctx.read_f32(out_a, batch * hidden)).all() and np.abs(ctx.read_f32(out_a, batch * hidden)).max() > 0

@@ -220,7 +220,7 @@ def test_prefill_chunk_matches_oracle_in_lockstep(ctx, small_model, n_prompt):
 def test_prefill_long_prompt_takes_two_chunks(ctx):
     """1100 prompt tokens are a chunk of 1024 and one of 76 (heads of 256: both chunks' attention on the matrix cores,
     the second over the first one's rows; GEMMs over K slices at 1024 and at 76 rows, gate | up at 1024 rows with
-    256 tiles: both parts of the activations walked by one workgroup; partial sums travelling between the GEMMs):
+    256 tiles of 128 tokens, so of 64 tokens each; partial sums travelling between the GEMMs):
     every K / V row within one code step of the oracle's, which walks the positions one by one, and the decode steps
     behind the prompt at 1e-3."""
     cfg = dict(n_layers=2, hidden=512, ffn=2048, n_q=4, n_kv=1, hd=256, vocab=4096, max_seq=1200,

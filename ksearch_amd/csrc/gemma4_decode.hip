@@ -142,6 +142,8 @@ struct ksh_gemma4 {
     ksh_graph *round_graphs[17] = {};
     bool round_bound[17] = {};     // a width's kernels are bound (a first round launched kernel by kernel)
     ksh_kvpool *round_pool = nullptr;
+    uint64_t round_pool_uid = 0;   // a new pool can come up at a destroyed pool's address: the graphs are tied to the pool's uid as well
+    bool round_graph = true;       // KSEARCH_ROUND_GRAPH, read when the model is created
     int r_count = 0;
 };
 
@@ -732,6 +734,7 @@ int ksh_gemma4_create(ksh_ctx *ctx, const ksh_gemma4_cfg *cfg, const ksh_gemma4_
     m->g = *globals;
     m->layers.assign(layers, layers + c.n_layers);
     m->plan.resize(c.n_layers);
+    if (const char *e = std::getenv("KSEARCH_ROUND_GRAPH")) m->round_graph = e[0] != '0';
     const int max_hd = std::max(c.hd_swa, c.hd_full);
     int max_ff = 0;
     for (const ksh_gemma4_layer &L : m->layers) max_ff = std::max(max_ff, (int)L.ffn);
@@ -975,6 +978,7 @@ void drop_round_graphs(ksh_gemma4 *m)
     for (ksh_graph *&g : m->round_graphs) { ksh_graph_destroy(g); g = nullptr; }
     for (bool &b : m->round_bound) b = false;
     m->round_pool = nullptr;
+    m->round_pool_uid = 0;
 }
 
 int forward_decode_round4(ksh_gemma4 *m, ksh_kvpool *pool, const int32_t *slots, const uint32_t *tokens, int t)
@@ -1005,14 +1009,20 @@ int forward_decode_round4(ksh_gemma4 *m, ksh_kvpool *pool, const int32_t *slots,
     m->r_count = t;
     // The launches of a round depend on its width alone (tokens, slots and positions are in the table): one graph per
     // width, captured at its second round (the first binds the width's kernels, which allocates, and a capture must
-    // not).  KSEARCH_ROUND_GRAPH=0 launches every round kernel by kernel.
-    static const bool use_graph = [] { const char *e = std::getenv("KSEARCH_ROUND_GRAPH"); return !(e && e[0] == '0'); }();
-    if (!use_graph) return encode_round4(m, pool, t, max_batch, pool_hd);
-    if (m->round_pool != pool) { drop_round_graphs(m); m->round_pool = pool; }
+    // not).  KSEARCH_ROUND_GRAPH=0 (read when the model is created) launches every round kernel by kernel.
+    if (!m->round_graph) return encode_round4(m, pool, t, max_batch, pool_hd);
+    // the graphs hold the pool's device addresses: another pool, or a new pool at a destroyed one's address, drops them
+    if (m->round_pool != pool || m->round_pool_uid != ksh_kvpool_uid(pool)) {
+        drop_round_graphs(m);
+        m->round_pool = pool;
+        m->round_pool_uid = ksh_kvpool_uid(pool);
+    }
     ksh_graph *&g = m->round_graphs[t];
     if (!g && !m->round_bound[t]) {
+        // bound only once every kernel of the width has been looked up: a capture must find nothing left to allocate
+        if (encode_round4(m, pool, t, max_batch, pool_hd)) return 1;
         m->round_bound[t] = true;
-        return encode_round4(m, pool, t, max_batch, pool_hd);
+        return 0;
     }
     if (!g) {
         if (ksh_graph_begin(m->ctx)) return 1;

@@ -35,7 +35,6 @@
 #include <functional>
 #include <vector>
 
-#include "decode_chain.hpp"
 #include "ksh_device.hpp"
 #include "ksh_internal.hpp"
 
@@ -127,10 +126,6 @@ struct ksh_gemma {
             *c_g = nullptr, *c_u = nullptr, *c_ff = nullptr, *c_tmp = nullptr, *c_meta = nullptr,
             *c_po = nullptr, *c_pg = nullptr, *c_pd = nullptr;   // unfolded partial sums of the o, gate | up and down projections
     int c_nwg = 0;
-    // the decode chain (decode_chain.hip): o-projection, feed-forward and the next layer's QKV as one launch per layer
-    bool use_chain = false;
-    int chain_spin_limit = 1 << 18;   // polls per wait before it gives up (KSEARCH_CHAIN_SPIN_LIMIT: tests of the time-out path)
-    ksh_buf *chain_vec = nullptr, *chain_err = nullptr;   // two sets of hand-over vectors {o, ff, y}; the time-out flag
 };
 
 namespace {
@@ -206,7 +201,6 @@ void warm_plan(ksh_gemma *m, int kind, std::initializer_list<int64_t> dims, std:
 // o-projection folds them in its prologue: 0.8 us per layer less at 320 positions, 1.5 us more at 1500,
 // where 16 partitions and the merge inside the attention launch win.
 // (KSEARCH_SHORT_CONTEXT overrides the limit when the model is built; 0 switches the short form off.)
-constexpr bool kChainDefault = false;
 constexpr int kShortContext = 640;
 constexpr int kShortPartitions = 8;
 
@@ -217,18 +211,9 @@ int encode_token(ksh_gemma *m, bool want_logits, bool short_ctx, int &launches)
     launches = 0;
     ksh_buf *cur = m->x, *other = m->xb;   // the residual stream and its next home
     // (the token's embedding row is in m->x already: write_token put it there, or the previous step's last launch)
-    hipStream_t cst = (hipStream_t)ksh_stream(m->ctx);
-    constexpr int kSet = kChainHidden + kChainFfn + kChainHidden;
-    if (m->use_chain && (c.n_layers & 1)) {
-        // an odd number of chain launches per token: the sets do not alternate across the token boundary
-        if (decode_chain_fill((uint32_t *)ksh_buffer_device_ptr(m->chain_vec), 2 * kSet, cst)) return 1;
-        launches += 1;
-    }
     for (int l = 0; l < c.n_layers; l++) {
         const ksh_gemma_layer &L = m->layers[l];
-        if (m->use_chain && l > 0) {
-            // q, k, v came out of the previous layer's chain launch
-        } else if (l == 0) {
+        if (l == 0) {
             if (enc(m, m->k_qkv_first, {L.wq, L.wk, L.wv, cur, L.attn_norm}, {m->tq, m->tk, m->tv}, launches)) return 1;
         } else {
             // closes layer l-1 (x += rmsnorm(down, post_ffw_norm), gemma_prim.rs:1150-1160) and opens layer l
@@ -251,35 +236,6 @@ int encode_token(ksh_gemma *m, bool want_logits, bool short_ctx, int &launches)
                 return 1;
             if (enc(m, m->k_sdpa, {m->tq, m->kv_k[l], m->kv_v[l], m->meta}, {m->attn_tmp, m->to}, launches)) return 1;
             if (m->sdpa_launches == 2) launches += 1;   // partials, then the merge
-        }
-        if (m->use_chain) {
-            const bool last = l == c.n_layers - 1;
-            const ksh_gemma_layer &N = m->layers[last ? l : l + 1];
-            auto f = [](ksh_buf *b) { return (float *)ksh_buffer_device_ptr(b); };
-            auto q = [](ksh_buf *b) { return (const uint8_t *)ksh_buffer_device_ptr(b); };
-            uint32_t *sets = (uint32_t *)ksh_buffer_device_ptr(m->chain_vec);
-            uint32_t *mine = sets + (size_t)(l & 1) * kSet, *theirs = sets + (size_t)((l + 1) & 1) * kSet;
-            ChainParams p{};
-            p.wo = q(L.wo);
-            p.attn = short_ctx ? f(m->attn_tmp) : f(m->to);
-            p.attn_parts = short_ctx ? kShortPartitions : 0;
-            p.hd_log2 = __builtin_ctz((unsigned)c.hd);
-            p.wgate = q(L.wgate); p.wup = q(L.wup); p.wdown = q(L.wdown);
-            p.post_attn_norm = f(L.post_attn_norm); p.ffn_norm = f(L.ffn_norm);
-            p.x = f(cur);
-            p.wq = q(N.wq); p.wk = q(N.wk); p.wv = q(N.wv);
-            p.post_ffw_norm = f(L.post_ffw_norm); p.attn_norm_next = f(N.attn_norm);
-            p.q_out = f(m->tq); p.k_out = f(m->tk); p.v_out = f(m->tv);
-            p.y_out = f(m->y);
-            p.last = last;
-            p.eps = c.eps;
-            p.o = mine; p.ff = mine + kChainHidden; p.y = mine + kChainHidden + kChainFfn;
-            p.o_other = theirs; p.ff_other = theirs + kChainHidden; p.y_other = theirs + kChainHidden + kChainFfn;
-            p.err = (int *)ksh_buffer_device_ptr(m->chain_err);
-            p.spin_limit = m->chain_spin_limit;
-            if (decode_chain_launch(p, cst)) return 1;
-            launches += 1;
-            continue;
         }
         if (short_ctx ? enc(m, m->k_oproj_merge, {L.wo, m->attn_tmp}, {m->y}, launches) : enc(m, m->k_oproj, {L.wo, m->to}, {m->y}, launches))
             return 1;
@@ -324,29 +280,6 @@ int encode_token(ksh_gemma *m, bool want_logits, bool short_ctx, int &launches)
     if (e != hipSuccess) return hip_fail(e, "advance launch");
     launches += 1;
     return 0;
-}
-
-// the hand-over vectors back to "nothing written", the time-out flag down
-int chain_clear(ksh_gemma *m)
-{
-    if (!m->use_chain) return 0;
-    constexpr int kSet = kChainHidden + kChainFfn + kChainHidden;
-    const int zero = 0;
-    if (decode_chain_fill((uint32_t *)ksh_buffer_device_ptr(m->chain_vec), 2 * kSet, (hipStream_t)ksh_stream(m->ctx))) return 1;
-    return ksh_buffer_write(m->ctx, m->chain_err, 0, &zero, 4, 1);
-}
-
-// after a synchronisation: did a hand-over wait of the decode chain run out?  (Then the tokens since the last check
-// are garbage.)
-int chain_check(ksh_gemma *m)
-{
-    if (!m->use_chain) return 0;
-    int err = 0;
-    if (ksh_buffer_read(m->ctx, m->chain_err, 0, &err, 4, 1)) return 1;
-    if (!err) return 0;
-    (void)chain_clear(m);
-    return set_error("decode chain: a hand-over wait ran out (its 256 workgroups must all be resident: is the GPU shared?); "
-                     "KSEARCH_DECODE_CHAIN=0 runs the layer as separate launches");
 }
 
 int run_token(ksh_gemma *m, bool want_logits, bool use_graph)
@@ -654,18 +587,6 @@ int ksh_gemma_create(ksh_ctx *ctx, const ksh_gemma_cfg *cfg, const ksh_gemma_lay
             get(g, KSH_SDPA_SLOTS, {c.n_q, c.n_kv, c.hd, c.max_seq, 1, g->nwg}, {KSH_Q40, KSH_F32}, {c.attn_scale}, &g->k_sdpa))
             return 1;
     }
-    // The decode chain: o-projection, feed-forward and the next layer's QKV of a layer as one launch whose phases hand
-    // their vectors over through memory.  Built for these widths; KSEARCH_DECODE_CHAIN=0 / 1 switches it off / on.
-    {
-        const bool fits = c.hidden == kChainHidden && c.ffn == kChainFfn && qd == 2048 && kvd == 256 && (c.hd & (c.hd - 1)) == 0 &&
-                          decode_chain_fits_device();
-        const char *e = getenv("KSEARCH_DECODE_CHAIN");
-        g->use_chain = fits && (e ? atoi(e) != 0 : kChainDefault);
-        if (e && atoi(e) != 0 && !fits) return set_error("KSEARCH_DECODE_CHAIN: the chain is built for hidden 2048, ffn 8192, 2048 + 256 + 256 q / k / v rows on a device that holds its 256 workgroups at once");
-        if (const char *sl = getenv("KSEARCH_CHAIN_SPIN_LIMIT")) g->chain_spin_limit = std::max(0, atoi(sl));
-        if (g->use_chain && (alloc(g, (size_t)2 * (kChainHidden + kChainFfn + kChainHidden) * 4, &g->chain_vec) || alloc(g, 16, &g->chain_err)))
-            return 1;
-    }
     if (ksh_gemma_reset(g)) return 1;
     *out = m.release();
     return 0;
@@ -689,7 +610,6 @@ int ksh_gemma_reset(ksh_gemma *m)
     const float meta[4] = {1.f, 0.f, 0.f, 0.f};   // tlen, start, window, pos
     if (ksh_buffer_write(m->ctx, m->meta, 0, meta, 16, 1)) return 1;
     if (ksh_buffer_write(m->ctx, m->rope_cur, 0, m->rope0.data(), m->rope0.size() * 4, 1)) return 1;
-    if (chain_clear(m)) return 1;
     m->pos = 0;
     return 0;
 }
@@ -704,7 +624,6 @@ int ksh_gemma_forward_token(ksh_gemma *m, uint32_t token, int use_graph, uint32_
         float f = 0.f;
         if (ksh_buffer_read(m->ctx, m->tok, 0, &f, 4, 1)) return 1;
         *next_id = (uint32_t)f;
-        if (chain_check(m)) return 1;
     }
     return 0;
 }
@@ -761,7 +680,7 @@ int ksh_gemma_generate(ksh_gemma *m, const uint32_t *prompt, int n_prompt, int n
         if (ksh_buffer_read(m->ctx, m->history, (size_t)first * 4, ids.data(), (size_t)n_new * 4, 1)) return 1;
         for (int i = 0; i < n_new; i++) out_ids[i] = (uint32_t)ids[i];
     }
-    return chain_check(m);
+    return 0;
 }
 
 ksh_buf *ksh_gemma_logits(ksh_gemma *m) { return m ? m->logits : nullptr; }

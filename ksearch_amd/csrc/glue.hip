@@ -12,6 +12,8 @@
 // Built with -ffp-contract=off so that `u*cos - v*sin` and `(x*inv)*w + res`
 // round exactly like the unfused expressions they restate; the Q4_0 codes that
 // come out of the pack are integer functions of those values.
+#include <atomic>
+
 #include "ksh_device.hpp"
 #include "q40_pack.hpp"
 #include "ksh_internal.hpp"
@@ -494,7 +496,7 @@ int launch_softcap_argmax(const ksh_kernel &k, const LaunchArgs &a, hipStream_t 
 // kernels get the per-device address that call returns.
 static __device__ __align__(256) unsigned char scratch[kArgParts * 8];
 constexpr int kMaxDevices = 64;
-void *g_scratch_ptr[kMaxDevices];      // per device: every GPU holds its own copy of the array
+std::atomic<void *> g_scratch_ptr[kMaxDevices];   // per device: every GPU holds its own copy of the array (set once, by whichever thread comes first)
 
 }  // namespace
 
@@ -517,11 +519,11 @@ int argmax_static_setup()
     int dev = -1;
     KSH_HIP(hipGetDevice(&dev));
     if (dev < 0 || dev >= kMaxDevices) return set_error("softcap_argmax_static: device ordinal %d", dev);
-    if (g_scratch_ptr[dev]) return 0;
+    if (g_scratch_ptr[dev].load(std::memory_order_acquire)) return 0;
     void *p = nullptr;
     KSH_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
     if (!p) return set_error("softcap_argmax_static: the partial-result array has no device address");
-    g_scratch_ptr[dev] = p;
+    g_scratch_ptr[dev].store(p, std::memory_order_release);   // (two threads racing here store the same address)
     return 0;
 }
 
@@ -541,11 +543,11 @@ extern "C" int ksh_softcap_argmax_static(ksh_ctx *ctx, ksh_buf *x, uint64_t x_of
     if (out_off % 4 || out_off > out->bytes || 4 > out->bytes - out_off)
         return set_error("ksh_softcap_argmax_static: out needs 4 bytes from 4-byte-aligned offset %llu, buffer has %zu",
                          (unsigned long long)out_off, out->bytes);
-    int dev = -1;
-    KSH_HIP(hipGetDevice(&dev));
+    // the array of the device the context's stream runs on, whatever device the calling thread has current
+    const int dev = ctx_device(ctx);
     if (dev < 0 || dev >= kMaxDevices) return set_error("ksh_softcap_argmax_static: device ordinal %d", dev);
-    if (!g_scratch_ptr[dev] && argmax_static_setup()) return 1;
-    float *pv = (float *)g_scratch_ptr[dev];
+    float *pv = (float *)g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!pv) return set_error("ksh_softcap_argmax_static: the context's device %d has no resolved array (ksh_ctx_create resolves it)", dev);
     uint32_t *pi = (uint32_t *)(pv + kArgParts);
     const int parts = (int)min((int64_t)kArgParts, (n + kArgThreads - 1) / kArgThreads);
     hipStream_t st = ctx_stream(ctx);

@@ -61,11 +61,13 @@ struct ksh_kernel {
 namespace ksh {
 // what entry points outside the runtime's translation unit need of a context
 hipStream_t ctx_stream(ksh_ctx *ctx);
+int ctx_device(ksh_ctx *ctx);   // the ordinal of the device the context's stream belongs to
 // a buffer object over bytes [off, off + bytes) of `parent` (retained until the view is released); nullptr + error when out of range
 ksh_buf *buffer_view(ksh_buf *parent, size_t off, size_t bytes);
 void ctx_mark_pending(ksh_ctx *ctx);
 // resolves the device address of the static partial-result array of ksh_softcap_argmax_static for the current
-// device (called when a context is created; the entry point does it itself for a device it has not seen)
+// device (called when a context is created, with the context's device current; the entry point then uses the
+// address kept for the context's device)
 int argmax_static_setup();
 // the end of a decode step (glue.hip): argmax over the logits, position update, the next token's embedding row
 struct DecodeTail {

@@ -111,6 +111,7 @@ struct ksh_ctx {
 
 namespace ksh {
 hipStream_t ctx_stream(ksh_ctx *ctx) { return ctx->stream; }
+int ctx_device(ksh_ctx *ctx) { return ctx->device; }
 ksh_buf *buffer_view(ksh_buf *parent, size_t off, size_t bytes)
 {
     if (!parent || off > parent->bytes || bytes > parent->bytes - off) {

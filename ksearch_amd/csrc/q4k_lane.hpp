@@ -1,6 +1,6 @@
 // What one lane of the Q4_K GEMV kernels does with one (row, superblock, 64-element group): the three 16-byte loads,
 // the group's activations as registers (padded f32, or three int8 digit planes), and the f32 contribution to y[row].
-// Shared by the GEMV family (matvec_q4k.hip) and the decode chain (decode_chain.hip).
+// Shared by the kernels of the GEMV family (matvec_q4k.hip).
 //
 // Arithmetic per (row, superblock, group), all f32:
 //   acc += d*sc_lo * sum(n_lo*x) + d*sc_hi * sum(n_hi*x) - dmin*(m_lo*Sx_lo + m_hi*Sx_hi)

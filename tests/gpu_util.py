@@ -12,6 +12,16 @@ def rel_err(got, want):
     return np.abs(got - want) / np.maximum(np.abs(want), max(floor, 1e-30))
 
 
+def plain_rel_err(got, want):
+    """|got-want| / |want| with no floor, over the elements at least as large as the vector's rms (where a plain
+    relative error is meaningful in f32): the figure the floored bar is reported beside."""
+    got = np.asarray(got, dtype=np.float64).ravel()
+    want = np.asarray(want, dtype=np.float64).ravel()
+    big = np.abs(want) >= np.sqrt(np.mean(want ** 2)) if want.size else np.zeros(0, bool)
+    big &= want != 0
+    return np.abs(got[big] - want[big]) / np.abs(want[big])
+
+
 def assert_close(got, want, tol, what=""):
     e = rel_err(got, want)
     i = int(np.argmax(e)) if e.size else 0

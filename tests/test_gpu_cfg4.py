@@ -19,7 +19,7 @@ import pytest
 
 import oracle
 from ksearch_amd import hip, synth
-from tests.gpu_util import rel_err
+from tests.gpu_util import plain_rel_err, rel_err
 
 pytestmark = pytest.mark.gpu
 HERE = os.path.dirname(os.path.abspath(__file__))
@@ -77,14 +77,18 @@ def test_cfg4_lockstep_with_the_oracle(model):
     n_pre = len(prompt) - 1
     m.prefill_chunk(prompt[:n_pre])
     flipped, t0 = 0, time.time()
+    first_flip = None           # the first position whose K / V row the device packed differently from the oracle (by one code)
     for i in range(n_pre):
         rows = device_rows(ctx, bufs, i, row)
         cpu.forward(prompt[i], want_logits=False, adopt_rows=rows, threads=16)
         assert cpu.row_max_step.max() <= 1.0 + 1e-3, f"prompt position {i}: {cpu.row_max_step.max()} codes, layer {np.argmax(cpu.row_max_step.max(1))}"
         flipped += int(cpu.row_diff_bytes.sum())
+        if first_flip is None and cpu.row_diff_bytes.sum() > 0:
+            first_flip = i
     seq = [prompt[-1]] + generated[:-1]
     expect_next = generated
-    worst, argmax_checked, near_ties = 0.0, 0, 0
+    worst, worst_plain, argmax_checked, near_ties = 0.0, 0.0, 0, 0
+    margins = []                # the oracle's top-2 margin per decode step, relative to the logit scale
     for j, tok in enumerate(seq):
         i = n_pre + j
         g_next = m.forward_token(tok, use_graph=True)
@@ -94,15 +98,22 @@ def test_cfg4_lockstep_with_the_oracle(model):
         # K / V rows: the device's are the oracle's up to one code of a value on a rounding boundary
         assert cpu.row_max_step.max() <= 1.0 + 1e-3, f"step {i}: {cpu.row_max_step.max()} codes, layer {np.argmax(cpu.row_max_step.max(1))}"
         flipped += int(cpu.row_diff_bytes.sum())
-        # logits: all 262144, every step
+        if first_flip is None and cpu.row_diff_bytes.sum() > 0:
+            first_flip = i
+        # logits: all 262144, every step; the bar is stated on |d| / max(|want|, rms(want)), and the plain |d| / |want|
+        # over the elements of at least rms size is held to it as well
         err = float(rel_err(g_logits, c_logits).max())
         worst = max(worst, err)
         assert err <= 1e-3, f"step {i}: logits off by {err:.2e}"
+        err_plain = float(plain_rel_err(g_logits, c_logits).max())
+        worst_plain = max(worst_plain, err_plain)
+        assert err_plain <= 1e-3, f"step {i}: logits of rms size and above off by {err_plain:.2e} of themselves"
         assert g_next == oracle.softcap_argmax(g_logits, cfg["softcap"]), i
         assert g_next == expect_next[j], f"step {i}: the replay left the free run"
         # greedy token: the oracle's, unless its two best are closer than the numeric tolerance
         top2 = np.partition(c_logits, -2)[-2:]
         scale = max(abs(float(top2[1])), float(np.sqrt(np.mean(c_logits.astype(np.float64) ** 2))))
+        margins.append(float(top2[1] - top2[0]) / scale)
         if top2[1] - top2[0] > 2e-3 * scale:
             argmax_checked += 1
             assert g_next == c_next, f"step {i}: margin {top2[1] - top2[0]:.3e}"
@@ -110,7 +121,16 @@ def test_cfg4_lockstep_with_the_oracle(model):
             near_ties += 1
             assert c_logits[c_next] - c_logits[g_next] <= 2e-3 * scale, i
     n = n_pre + len(seq)
-    print(f"cfg4 lockstep: {n_pre} prompt positions prefilled as one chunk + {len(seq)} decode steps, worst logit error {worst:.2e}, {argmax_checked} greedy tokens equal the oracle's, "
+    # Where the free run leaves the oracle's own free run (the fixture), something must explain it: a K / V row that
+    # the device packed one code away from the oracle's at or before the position that produced the token (from then
+    # on the two runs attend different caches), or an oracle margin at that step below the numeric tolerance.
+    if n_same < N_NEW:
+        at = n_pre + n_same     # the position whose step produced the first differing token
+        explained = (first_flip is not None and first_flip <= at) or margins[n_same] < 2e-3
+        print(f"cfg4 free run leaves the fixture at decode step {n_same} (position {at}); first one-code K / V flip at position {first_flip}; "
+              f"oracle margin there {margins[n_same]:.2e}")
+        assert explained, f"free run differs at step {n_same} with no K / V flip up to position {at} and a margin of {margins[n_same]:.2e}"
+    print(f"cfg4 lockstep: {n_pre} prompt positions prefilled as one chunk + {len(seq)} decode steps, worst logit error {worst:.2e} (floored), {worst_plain:.2e} (plain, elements >= rms), {argmax_checked} greedy tokens equal the oracle's, "
           f"{near_ties} near-ties, {flipped} of {n * n_layers * 2 * row} KV bytes differ by one code ({time.time() - t0:.0f}s)")
     assert flipped <= 0.02 * n * n_layers * 2 * row
     assert argmax_checked >= 0.9 * len(seq)

@@ -664,6 +664,59 @@ def test_gemma4_decode_round_over_pool_slots(ctx, variant):
         pool.close()
 
 
+def test_gemma4_decode_round_after_the_pool_is_replaced(ctx):
+    """The per-width round graphs hold the pool's device addresses.  A pool that is destroyed and replaced (the host
+    object of the new one may well come up at the old one's address, its layers elsewhere) must get graphs of its own:
+    two rounds on the first pool (the second captures the width's graph), the pool closed, a larger one opened, then
+    three rounds on it in lockstep with one oracle per sequence."""
+    cfg = dict(synth.GEMMA4_TINY)
+    w = synth.gemma4_weights(cfg, 652, oracle.quantize_q4k, oracle.quantize_q6k, ffn=FFN, swa_pattern=PATTERN, std=0.05)
+    gpu = hip.Gemma4(ctx, cfg, w)
+    n, tol = cfg["n_layers"], 1e-3
+    owners = [l for l in range(n) if gpu.kv_source(l) == l]
+    rng = np.random.default_rng(653)
+    cpus = []
+    pool = None
+    try:
+        for n_slots in (2, 5):
+            pool = hip.KvPool(ctx, n_slots, cfg["max_seq"], len(owners), max(cfg["hd_swa"], cfg["hd_full"]), cfg["n_kv"])
+            slots = [pool.alloc() for _ in range(n_slots)][-2:]
+            for s_ in slots:
+                pool.clear_slot(s_)
+            cpus = [oracle.Gemma4(cfg, w) for _ in slots]
+            for s_, n_pre, cpu in zip(slots, (3, 6), cpus):
+                cpu.reset()
+                toks = [int(t) for t in rng.integers(0, cfg["vocab"], n_pre)]
+                gpu.bind_slot(pool, s_)
+                gpu.prefill_chunk(toks)
+                pool.bump_len(s_, n_pre)
+                for i, t in enumerate(toks):
+                    cpu.forward(t, want_logits=False, adopt_rows=slot_rows(ctx, pool, s_, i, cfg, PATTERN, owners))
+            for r in range(3):
+                toks = rng.integers(0, cfg["vocab"], 2)
+                gpu.decode_round(pool, slots, toks)
+                logits = gpu.round_logits(2)
+                for j, s_ in enumerate(slots):
+                    pos = pool.seq_len(s_)
+                    _, c_logits = cpus[j].forward(int(toks[j]), return_logits=True, adopt_rows=slot_rows(ctx, pool, s_, pos, cfg, PATTERN, owners))
+                    assert cpus[j].row_max_step.max() <= 1.0 + 1e-3, (n_slots, r, j)
+                    assert_close(logits[j], c_logits, tol, f"pool of {n_slots}, round {r}, sequence {j}")
+                    pool.bump_len(s_)
+            for cpu in cpus:
+                cpu.close()
+            cpus = []
+            gpu.bind_slot(None, 0)
+            pool.close()
+            pool = None
+            junk = ctx.buffer_empty_f32(300_000)   # moves the next pool's layers off the old ones' addresses
+    finally:
+        for cpu in cpus:
+            cpu.close()
+        gpu.close()
+        if pool is not None:
+            pool.close()
+
+
 def test_gemma4_real_widths_decode_round(ctx, eng):
     """Decode rounds at the real widths (hidden 1536, heads of 256 / 512, window 512, 12288-wide feed-forward): two
     sequences of 300 and 20 positions in slots 1 and 0 of a pool sized for the 512-wide heads (so the 256-wide layers'

@@ -9,7 +9,8 @@ timed launches cycle through `--copies` distinct copies of the weight matrix
 (64 x 9.4 MB = 604 MB, more than the 256 MB last-level cache plus L2), so every
 launch streams its weights from HBM; inputs are resident in HBM before the
 timed region.  The launches are captured in one HIP graph and timed with HIP
-events recorded on the stream the graph runs on.
+events recorded on the stream the graph runs on; the figure is the median of
+five replays of that graph, each of exactly K launches.
 
 value            algorithmic GB/s = (W + x + y bytes) * K / elapsed
 roofline         the same figure against MI355X's 8 TB/s HBM peak
@@ -65,10 +66,13 @@ class HipEvents:
         return float(ms.value)
 
 
-def timed_graph(ctx, ev, encode_one, n_launches: int, warmup: int) -> float:
+def timed_graph(ctx, ev, encode_one, n_launches: int, warmup: int, replays: int = 1) -> float:
     """Captures `n_launches` calls of encode_one(i) into a graph, runs `warmup`
     launches eagerly first and (when there is a warm-up at all) one untimed replay,
-    then times one replay.  Returns ms for that replay."""
+    then times `replays` replays, each of exactly `n_launches` launches between a
+    synchronisation and an event pair of its own, and returns the median replay's ms
+    (a short graph's time is its launches plus the ~10 us it takes to get the graph
+    going, and that part jitters from replay to replay)."""
     for i in range(warmup):
         encode_one(i)
     ctx.synchronize()
@@ -78,16 +82,18 @@ def timed_graph(ctx, ev, encode_one, n_launches: int, warmup: int) -> float:
     g = ctx.graph_end()
     if warmup:
         ctx.graph_launch(g)      # the first replay of a new executable graph also uploads it: part of the warm-up
-    ctx.synchronize()
-    ev.start(ctx.stream)
-    ctx.graph_launch(g)
-    ms = ev.stop_ms(ctx.stream)
+    times = []
+    for _ in range(max(1, replays)):
+        ctx.synchronize()
+        ev.start(ctx.stream)
+        ctx.graph_launch(g)
+        times.append(ev.stop_ms(ctx.stream))
     ctx.synchronize()
     ctx.graph_destroy(g)
-    return ms
+    return float(np.median(times))
 
 
-def bench_matvec(ctx, eng, ev, dtype, rows, cols, w_host, x_host, copies, steps, warmup, sched=None):
+def bench_matvec(ctx, eng, ev, dtype, rows, cols, w_host, x_host, copies, steps, warmup, sched=None, replays=1):
     from ksearch_amd import hip
 
     wbytes = w_host.size
@@ -98,7 +104,7 @@ def bench_matvec(ctx, eng, ev, dtype, rows, cols, w_host, x_host, copies, steps,
     def one(i):
         ctx.encode_offsets_multi(k, [big, bx], [(i % copies) * wbytes, 0], [by], [0])
 
-    ms = timed_graph(ctx, ev, one, steps, warmup)
+    ms = timed_graph(ctx, ev, one, steps, warmup, replays)
     alg = wbytes + cols * 4 + rows * 4
     big.release()
     return dict(kernel=k.name, us_per_launch=ms * 1e3 / steps, gbps=alg * steps / (ms * 1e-3) / 1e9,
@@ -328,6 +334,88 @@ def bench_decode_gemma4_layout(ctx, eng, use_graph=True):
     return r
 
 
+def bench_timeline(ctx, eng, tokens=24):
+    """Where a decode step's launches spend their time, from inside: the timeline build of the library
+    (ksearch_amd/lib/libksearch_hip_stamps.so: the same sources with -DKSH_STAMPS) has lane 0 of every wave write the
+    chip-wide 100 MHz counter between its phases.  cfg4's model decodes `tokens` tokens from position 64 through the
+    captured graph; after each token the records of the last launch of every shape are read -- the last layer's
+    QKV, attention step, o-projection, gate || up, down, and the LM head, which follow one another, so their records
+    share one time axis.  Per launch: when its waves enter, and the median / slowest wave at each phase boundary,
+    in microseconds from the launch's first wave; `gap_before_us` is the time from the previous launch's last
+    acknowledged store to this launch's first wave.  The timestamps themselves cost a little (one counter read and
+    one store per phase and wave): the timeline build decodes ~3 % slower than the product build."""
+    from ksearch_amd import hip, synth
+
+    L = hip.lib()
+    S, W, T = 8, 4096, 8          # slots per record, records per tag, tags (ksh_device.hpp)
+    readers = {}
+    for name in ("ksh_stamps_matvec_q4k", "ksh_stamps_sdpa_lanes", "ksh_stamps_matvec_q6k"):
+        fn = getattr(L, name)
+        fn.restype, fn.argtypes = C.c_int, [C.POINTER(C.c_ulonglong), C.c_size_t]
+        readers[name] = fn
+
+    def read(name):
+        buf = (C.c_ulonglong * (T * W * S))()
+        assert readers[name](buf, T * W * S) == 0
+        return np.frombuffer(buf, dtype=np.uint64).reshape(T, W, S).astype(np.int64)
+
+    cfg = synth.GEMMA_E2B_SYNTH
+    q4k, q6k = hip.device_quantizers(ctx, eng)
+    m = hip.Gemma(ctx, cfg, synth.gemma_weights(cfg, 4000, q4k, q6k))
+    prompt = [int(t) for t in np.random.default_rng(4001).integers(0, cfg["vocab"], 64)]
+    out, _, _ = m.generate(prompt, 4, use_graph=True)
+    tok = out[-1]
+    for r in readers:
+        read(r)                    # clears what the warm-up left
+    # (kernel, reader, tag, names of the phase boundaries 1..6)
+    gemv = ["loads issued", "vector staged", "barrier passed", "products done", "stores issued", "stores acknowledged"]
+    launches = [
+        ("qkv (add + norm prologue, 2.9 MB)", "ksh_stamps_matvec_q4k", 4, gemv),
+        ("attention step (norm, rope, append, <= 8 partitions)", "ksh_stamps_sdpa_lanes", 1,
+         ["front loads issued", "length and position in", "q and new row ready", "rows done", "row groups folded", "records acknowledged"]),
+        ("o-projection (merges the partitions, 2.4 MB)", "ksh_stamps_matvec_q4k", 6, gemv),
+        ("gate || up + GELU (add + norm prologue, 18.9 MB)", "ksh_stamps_matvec_q4k", 5, gemv),
+        ("down (9.4 MB)", "ksh_stamps_matvec_q4k", 0, gemv),
+        ("LM head (add + norm prologue, 440 MB; every 4th workgroup)", "ksh_stamps_matvec_q6k", 0,
+         ["loads issued", "vector staged", "barrier passed", "first row done", "last row stored", "stores acknowledged"]),
+    ]
+    acc = {name: [] for name, *_ in launches}
+    for _ in range(tokens):
+        tok = m.forward_token(tok, use_graph=True)
+        bufs = {r: read(r) for r in readers}
+        prev_end = None
+        for name, reader, tag, phases in launches:
+            a = bufs[reader][tag]
+            a = a[a[:, 0] > 0]
+            if not len(a):
+                raise SystemExit(f"bench.py: the timeline build left no records for {name!r}")
+            t0 = a[:, 0].min()
+            row = dict(waves=len(a), gap=None if prev_end is None else (t0 - prev_end) * 0.01,
+                       entry_p50=(np.median(a[:, 0]) - t0) * 0.01, entry_max=(a[:, 0].max() - t0) * 0.01)
+            for i in range(1, 7):
+                v = a[:, i][a[:, i] > 0]
+                row[f"p50_{i}"] = (np.median(v) - t0) * 0.01 if len(v) else None
+                row[f"max_{i}"] = (v.max() - t0) * 0.01 if len(v) else None
+            prev_end = max(int(a[:, i][a[:, i] > 0].max()) for i in range(1, 7) if (a[:, i] > 0).any())
+            row["span"] = (prev_end - t0) * 0.01
+            acc[name].append(row)
+    m.close()
+    res = {"tokens": tokens, "unit": "us from the launch's first wave; median over the tokens of (p50 over waves | slowest wave)"}
+    for name, reader, tag, phases in launches:
+        rows = acc[name]
+
+        def med(k):
+            v = [r[k] for r in rows if r[k] is not None]
+            return round(float(np.median(v)), 2) if v else None
+
+        rec = {"waves": rows[0]["waves"], "gap_before_us": med("gap"), "entry_p50": med("entry_p50"), "entry_last": med("entry_max"),
+               "first_wave_to_last_ack_us": med("span")}
+        for i, ph in enumerate(phases, 1):
+            rec[ph] = [med(f"p50_{i}"), med(f"max_{i}")]
+        res[name] = rec
+    return res
+
+
 def cpu_baseline_matvec(w, x, rows, cols, budget_s=1.5):
     """The CPU checker (oracle/) timed on this machine: all cores, then one."""
     import oracle
@@ -372,7 +460,7 @@ def main() -> int:
     ap.add_argument("--attn-form", choices=["default", "lanes", "mfma"], default="default",
                     help="cfg3: the split-KV row phase as the register (lanes) or the matrix-core (mfma) kernel instead of "
                          "the library's choice for the shape")
-    ap.add_argument("--only", choices=["cfg1", "cfg2", "cfg3", "cfg4", "gemma4", "prefill", "copy", "floor"],
+    ap.add_argument("--only", choices=["cfg1", "cfg2", "cfg3", "cfg4", "gemma4", "prefill", "copy", "floor", "timeline"],
                     help="run one secondary workload and print its record (for profiling runs); 'copy' is a plain "
                          "64 MiB device copy, the known-size kernel that calibrates the FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
@@ -384,6 +472,24 @@ def main() -> int:
     from ksearch_amd import hip, synth
     from ksearch_amd.hip import DType
 
+    if args.only == "timeline":
+        # the timeline build of the library (phase timestamps compiled in); nothing else in this script uses it
+        from ksearch_amd import _build
+
+        hip.LIB_PATH = _build.STAMPS_LIB_PATH
+        os.environ["KSEARCH_SKIP_BEAM"] = "1"      # the library's default schedules
+        ctx, eng = hip.Context(), hip.Eng()
+        r = bench_timeline(ctx, eng)
+        ctx.close()
+        print(json.dumps({"timeline": r}))
+        for name, rec in r.items():
+            if isinstance(rec, dict):
+                print(f"{name}: waves {rec['waves']}, gap before {rec['gap_before_us']}, entries p50 {rec['entry_p50']} last {rec['entry_last']}, "
+                      f"first wave -> last ack {rec['first_wave_to_last_ack_us']}", file=sys.stderr)
+                for k, v in rec.items():
+                    if isinstance(v, list):
+                        print(f"    {k:28s} p50 {v[0]}   slowest {v[1]}", file=sys.stderr)
+        return 0
     ctx, eng, ev = hip.Context(), hip.Eng(), HipEvents()
     if args.only == "copy":
         n = 16 << 20
@@ -408,7 +514,7 @@ def main() -> int:
         return 0
     rows = cols = 4096
     w, x = synth.cfg0_q4k_matvec()
-    head = bench_matvec(ctx, eng, ev, DType.Q4K, rows, cols, w, x, args.copies, args.steps, args.warmup)
+    head = bench_matvec(ctx, eng, ev, DType.Q4K, rows, cols, w, x, args.copies, args.steps, args.warmup, replays=5)
     traffic = measured_traffic(head["kernel"])      # before the minutes of secondary workloads, not after
 
     also = {}

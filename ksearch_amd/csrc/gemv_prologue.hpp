@@ -171,9 +171,14 @@ struct StageRegs {
 // kMerge: whether the kernel is built with the kMergeParts source at all (the Q4_K kernels' prologue instances are)
 // KMAX: a compile-time bound on the float4 per thread (kernels built for a fixed row length): what lies past it
 // takes no registers, which is what decides the occupancy of the long-running LM head.
-template <int NT, bool kMerge = false, int KMAX = kStageX>
-__device__ __forceinline__ void stage_fetch(const Prologue &pr, int cols, StageRegs &s)
+// KIND: the prologue kind when the kernel is built for one (-1: read from the descriptor at run time).  With it and a
+// row length known at compile time the front of the kernel is a straight run of loads with constant offsets; with
+// neither it is a chain of compare-and-branch pairs, one per possible float4, in front of the first weight load.
+template <int NT, bool kMerge = false, int KMAX = kStageX, int KIND = -1>
+__device__ __forceinline__ void stage_fetch(const Prologue &pr_in, int cols, StageRegs &s)
 {
+    Prologue pr = pr_in;
+    if (KIND >= 0) pr.kind = KIND;
     constexpr int KX = KMAX < kStageX ? KMAX : kStageX, KP = KMAX < kStageP ? KMAX : kStageP;
     // n4 is a multiple of 64, so "this float4 exists" is a per-wave fact: keep it
     // in scalar registers and the loads stay unpredicated
@@ -218,9 +223,11 @@ __device__ __forceinline__ void stage_fetch(const Prologue &pr, int cols, StageR
 
 // Every thread must call this (it contains barriers); the LDS image is complete
 // after the caller's next __syncthreads().
-template <int XF, int NT, bool kMerge = false, int KMAX = kStageX>
-__device__ __forceinline__ void stage_finish(const Prologue &pr, uint8_t *lds, int cols, StageRegs &s)
+template <int XF, int NT, bool kMerge = false, int KMAX = kStageX, int KIND = -1>
+__device__ __forceinline__ void stage_finish(const Prologue &pr_in, uint8_t *lds, int cols, StageRegs &s)
 {
+    Prologue pr = pr_in;
+    if (KIND >= 0) pr.kind = KIND;
     constexpr int KX = KMAX < kStageX ? KMAX : kStageX, KP = KMAX < kStageP ? KMAX : kStageP;
     const int wbase = __builtin_amdgcn_readfirstlane(threadIdx.x & ~63), tid = wbase + (threadIdx.x & 63), n4 = cols / 4;
     float *red = reinterpret_cast<float *>(lds + xs_image_bytes<XF>(cols));

@@ -9,6 +9,58 @@
 
 namespace ksh {
 
+// Phase timestamps, compiled in only with -DKSH_STAMPS (the timeline build of the library; the product build has
+// none).  A wave reads the chip-wide 100 MHz real-time counter at its phase boundaries into registers
+// (KSH_STAMP(slot)) and writes the lot when it is done (KSH_STAMP_FLUSH: waits for the wave's own memory operations
+// to be acknowledged, takes the last slot, stores the record) -- a store in the middle of the kernel would be a
+// second kind of memory operation in flight, and the exact counts the kernels wait on would turn into waits for
+// everything.  Records are indexed by (tag, wave in the launch), a tag per kernel shape, so the buffer holds the
+// last launch of each shape; the counter is the same for every wave of the chip, so records of different kernels
+// share one time axis.  Each translation unit that stamps defines the buffer with KSH_STAMP_BUFFER and an
+// extern "C" reader with KSH_STAMP_READER(name).
+constexpr int kStampSlots = 8, kStampWaves = 4096, kStampTags = 8;
+#ifdef KSH_STAMPS
+#define KSH_STAMP_BUFFER static __device__ unsigned long long g_stamps[ksh::kStampTags * ksh::kStampWaves * ksh::kStampSlots];
+#define KSH_STAMP_BEGIN unsigned long long ksh_st_[ksh::kStampSlots] = {}; ksh_st_[0] = wall_clock64();
+#define KSH_STAMP(slot)                                                                                                   \
+    do {                                                                                                                  \
+        __builtin_amdgcn_sched_barrier(0); /* nothing is scheduled across the reading of the counter */                   \
+        ksh_st_[slot] = wall_clock64();                                                                                   \
+        __builtin_amdgcn_sched_barrier(0);                                                                                \
+    } while (0)
+// pins "value v is in its register" in front of the next timestamp (a load's result is otherwise waited for wherever
+// the compiler first needs it)
+#define KSH_STAMP_USE(v) asm volatile("" ::"v"(v))
+#define KSH_STAMP_FLUSH(tag, wave_in_launch, last_slot)                                                                   \
+    do {                                                                                                                  \
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                                                  \
+        ksh_st_[last_slot] = wall_clock64();                                                                              \
+        if ((threadIdx.x & 63) == 0 && (int)(wave_in_launch) < ksh::kStampWaves) {                                         \
+            unsigned long long *rec_ = g_stamps + ((size_t)(tag) * ksh::kStampWaves + (size_t)(wave_in_launch)) * ksh::kStampSlots; \
+            for (int i_ = 0; i_ < ksh::kStampSlots; i_++) rec_[i_] = ksh_st_[i_];                                          \
+        }                                                                                                                 \
+    } while (0)
+// copies the records out (and clears them): dst holds n counters, n <= tags * waves * slots
+#define KSH_STAMP_READER(name)                                                                                            \
+    extern "C" int name(unsigned long long *dst, size_t n)                                                                \
+    {                                                                                                                     \
+        const size_t all = (size_t)ksh::kStampTags * ksh::kStampWaves * ksh::kStampSlots;                                  \
+        if (!dst || n > all) return 1;                                                                                    \
+        if (hipDeviceSynchronize() != hipSuccess) return 1;                                                               \
+        if (hipMemcpyFromSymbol(dst, HIP_SYMBOL(g_stamps), n * 8, 0, hipMemcpyDeviceToHost) != hipSuccess) return 1;       \
+        void *p = nullptr;                                                                                                \
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_stamps)) != hipSuccess) return 1;                                        \
+        return hipMemset(p, 0, all * 8) != hipSuccess;                                                                    \
+    }
+#else
+#define KSH_STAMP_BUFFER
+#define KSH_STAMP_BEGIN
+#define KSH_STAMP(slot) do {} while (0)
+#define KSH_STAMP_USE(v) do {} while (0)
+#define KSH_STAMP_FLUSH(tag, wave_in_launch, last_slot) do {} while (0)
+#define KSH_STAMP_READER(name)
+#endif
+
 // Loads and stores that say "global memory" themselves.  A pointer that went
 // through an opaque statement (or a select the compiler cannot see through) is
 // otherwise accessed with flat instructions, which count against the LDS
@@ -42,6 +94,17 @@ __device__ __forceinline__ void stg_f4(float *p, size_t i, float4 v)
 __device__ __forceinline__ void stg_f32(float *p, size_t i, float v) { ((KSH_GLOBAL float *)p)[i] = v; }
 
 constexpr int kWave = 64;
+
+// A zero the compiler cannot see through, in a vector register.  Added to the index of a load whose address is the
+// same in every lane, it keeps the load a vector load.  Left alone such a load becomes a scalar load, and scalar
+// loads return out of order: the first wait for ANY of them -- the kernel arguments included -- then waits for all,
+// which puts a memory round trip for a small record in front of everything issued behind that wait.
+__device__ __forceinline__ int opaque_zero_v()
+{
+    int z = 0;
+    asm volatile("" : "+v"(z));
+    return z;
+}
 
 __device__ __forceinline__ float as_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
 __device__ __forceinline__ uint32_t as_u32(float f) { return __builtin_bit_cast(uint32_t, f); }

@@ -34,8 +34,16 @@
 #include "ksh_internal.hpp"
 #include "q4k_lane.hpp"
 
+KSH_STAMP_BUFFER
+KSH_STAMP_READER(ksh_stamps_matvec_q4k)
+
 namespace ksh {
 namespace {
+
+// timeline build: one record set per decode-step shape -- tag = prologue kind * 2 + (two matrices per wave)
+// slots: 0 entry, 1 every load issued, 2 vector staged, 3 barrier passed, 4 inner products done, 5 stores issued, 6 stores acknowledged,
+//        7 (half-wave form) the vector's loads issued, in front of the barrier that holds the weight loads back
+#define KSH_GEMV_TAG(p, NM) ((p).pro.kind * 2 + ((NM) - 1))
 
 // One launch covers up to three weight matrices that share the input vector.
 //   mode 0: the matrices are independent row ranges (plain GEMV: one; QKV:
@@ -130,15 +138,20 @@ __device__ __forceinline__ WaveTask wave_task(const MatvecParams &p, int wv, int
 // first HBM round trip overlaps the prologue.
 // MERGE: built with the partition-merging prologue (kept out of every other instance: a longer program in front
 // of the first weight load costs 0.1 us at 4096 x 4096)
-template <int R, int NW, int NM, int XF, bool MULTI, bool MERGE>
+// CB: superblocks per row when the instance is built for one row length (0: p.bpr); KIND: its prologue kind (-1:
+// p.pro.kind).  The instances with both (the plain GEMV over 4096 and 8192 columns) reach their weight loads in a
+// fraction of the instructions the general form needs.
+template <int R, int NW, int NM, int XF, bool MULTI, bool MERGE, int CB = 0, int KIND = -1>
 __global__ __launch_bounds__(NW * 64) void q4k_gemv_kernel(MatvecParams p_in)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t xs[];
     const MatvecParams p = fetch_params(p_in);
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    KSH_STAMP_BEGIN
     const int g = lane & 3, bl = lane >> 2;
-    const int bpr = p.bpr, cols = bpr * 256;
+    const int bpr = CB ? CB : p.bpr, cols = bpr * 256;
     const size_t row_bytes = (size_t)bpr * kQ4kBytes;
+    constexpr int KMAX = CB ? (CB * 64 + NW * 64 - 1) / (NW * 64) : kStageX;   // float4 of the vector per thread
     const WaveTask t = wave_task(p, blockIdx.x * NW + wave, R);
 
     const uint8_t *rowp[NM][R];
@@ -158,13 +171,21 @@ __global__ __launch_bounds__(NW * 64) void q4k_gemv_kernel(MatvecParams p_in)
     Q4kLane cur[NM][R], nxt[MULTI ? NM : 1][MULTI ? R : 1];
     StageRegs sr;
     constexpr int RPRE = R;   // (splitting the issue as the half-wave form does costs 0.5 us at 4096 x 4096)
-    stage_fetch<NW * 64, MERGE>(p.pro, cols, sr);
+    stage_fetch<NW * 64, MERGE, KMAX, KIND>(p.pro, cols, sr);
+    // The short front reaches its weight loads a few dozen instructions behind the vector's, and loads of different
+    // waves share one in-order path per compute unit: without this barrier a wave's vector loads queue behind another
+    // wave's HBM-cold weights (vector staged in the slowest wave at 2.3 us instead of 1.7).  The general form's long
+    // front keeps the two apart by itself.
+    if (CB) __syncthreads();
 #pragma unroll
     for (int m = 0; m < NM; m++)
 #pragma unroll
         for (int r = 0; r < RPRE; r++) cur[m][r] = q4k_load(rowp[m][r] + (size_t)min(bl, bpr - 1) * kQ4kBytes, g);
-    stage_finish<XF, NW * 64, MERGE>(p.pro, xs, cols, sr);
+    KSH_STAMP(1);
+    stage_finish<XF, NW * 64, MERGE, KMAX, KIND>(p.pro, xs, cols, sr);
+    KSH_STAMP(2);
     __syncthreads();
+    KSH_STAMP(3);
     if (!t.active) return;
 #pragma unroll
     for (int m = 0; m < NM; m++)
@@ -204,14 +225,25 @@ __global__ __launch_bounds__(NW * 64) void q4k_gemv_kernel(MatvecParams p_in)
         }
     }
 
+    KSH_STAMP_USE(acc[NM - 1][R - 1]);
+    KSH_STAMP(4);
+    // every row is reduced before the first is stored: a store in front of a later row's wait makes that wait one for
+    // the store's acknowledgement as well (loads and stores retire in order)
+    float res[R];
 #pragma unroll
     for (int r = 0; r < R; r++) {
         float s[NM];
 #pragma unroll
         for (int m = 0; m < NM; m++) s[m] = wave_sum(acc[m][r]);
-        const int row = t.row0 + r;
-        if (lane == 0 && row < t.rows) stg_f32(t.y, row, (NM == 2) ? gelu_mul_f32(s[0], s[NM - 1]) : s[0]);
+        res[r] = (NM == 2) ? gelu_mul_f32(s[0], s[NM - 1]) : s[0];
     }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int row = t.row0 + r;
+        if (lane == 0 && row < t.rows) stg_f32(t.y, row, res[r]);
+    }
+    KSH_STAMP(5);
+    KSH_STAMP_FLUSH(KSH_GEMV_TAG(p, NM), blockIdx.x * NW + wave, 6);
 }
 
 // Half-wave form for rows of at most 8 superblocks (BPR = 8: 2048 columns, no lane idles; BPR = 6: 1536 columns,
@@ -223,6 +255,7 @@ __global__ __launch_bounds__(NW * 64) void q4k_gemv_half_kernel(MatvecParams p_i
     extern __shared__ __attribute__((aligned(16))) uint8_t xs[];
     const MatvecParams p = fetch_params(p_in);
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    KSH_STAMP_BEGIN
     const int g = lane & 3, slot = (lane >> 2) & 7, hw = lane >> 5;
     constexpr int bpr = BPR;
     const int bl = BPR == 8 ? slot : min(slot, BPR - 1);
@@ -237,6 +270,7 @@ __global__ __launch_bounds__(NW * 64) void q4k_gemv_half_kernel(MatvecParams p_i
     // With a normalising prologue every wave's vector loads are queued before any wave's weight loads: behind
     // another wave's HBM-cold weights in the compute unit's memory pipeline they came back up to 1.3 us late, and
     // the prologue's reduction waits for the slowest wave.
+    KSH_STAMP(7);
     if (p.pro.kind != kPlain) __syncthreads();
     auto load_r = [&](int r) {
         const size_t off = (size_t)min(row0 + r, t.rows - 1) * row_bytes + (size_t)bl * kQ4kBytes;
@@ -250,8 +284,11 @@ __global__ __launch_bounds__(NW * 64) void q4k_gemv_half_kernel(MatvecParams p_i
     // and stream in while the first is being multiplied (gate || up, 2048 ->
     // 8192 with the add-then-norm prologue: 8.1 -> 7.1 us).
     load_r(0);
+    KSH_STAMP(1);
     stage_finish<XF, NW * 64, MERGE>(p.pro, xs, bpr * 256, sr);
+    KSH_STAMP(2);
     __syncthreads();
+    KSH_STAMP(3);
     if (!t.active) return;
 #pragma unroll
     for (int r = 1; r < R; r++) load_r(r);
@@ -259,6 +296,8 @@ __global__ __launch_bounds__(NW * 64) void q4k_gemv_half_kernel(MatvecParams p_i
     XGroup<XF> X;
     X.load(xs, bpr * 256, bl, g);
 
+    // (every row is multiplied and reduced before the first is stored, as in the full-wave form)
+    float res[R];
 #pragma unroll
     for (int r = 0; r < R; r++) {
         float s[NM];
@@ -268,9 +307,17 @@ __global__ __launch_bounds__(NW * 64) void q4k_gemv_half_kernel(MatvecParams p_i
             const float2 hs = wave_half_sums(mine ? v : 0.f);
             s[m] = hw ? hs.y : hs.x;
         }
-        const int row = row0 + r;
-        if ((lane & 31) == 0 && row < t.rows) stg_f32(t.y, row, (NM == 2) ? gelu_mul_f32(s[0], s[NM - 1]) : s[0]);
+        res[r] = (NM == 2) ? gelu_mul_f32(s[0], s[NM - 1]) : s[0];
     }
+    KSH_STAMP_USE(res[R - 1]);
+    KSH_STAMP(4);
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int row = row0 + r;
+        if ((lane & 31) == 0 && row < t.rows) stg_f32(t.y, row, res[r]);
+    }
+    KSH_STAMP(5);
+    KSH_STAMP_FLUSH(KSH_GEMV_TAG(p, NM), blockIdx.x * NW + wave, 6);
 }
 
 struct Q4kGeom {
@@ -290,6 +337,10 @@ void launch_pro(bool half, const MatvecParams &p, unsigned grid, size_t lds, hip
         hipLaunchKernelGGL((q4k_gemv_half_kernel<R, NW, NM, XF, MERGE, 8>), dim3(grid), dim3(NW * 64), lds, st, p);
     else if (half)
         hipLaunchKernelGGL((q4k_gemv_half_kernel<R, NW, NM, XF, MERGE, 6>), dim3(grid), dim3(NW * 64), lds, st, p);
+    // the plain GEMV over 4096 columns, built for that row length (4.25 against 4.35 us at 4096 x 4096; the same for 8192
+    // columns -- the down projection -- was slower inside the decode loop, 1111 against 1123 tok/s, and is not built)
+    else if (NM == 1 && !MERGE && NW == 8 && R <= 2 && p.pro.kind == kPlain && p.bpr == 16)
+        hipLaunchKernelGGL((q4k_gemv_kernel<(R <= 2 ? R : 1), 8, 1, XF, false, false, 16, kPlain>), dim3(grid), dim3(NW * 64), lds, st, p);
     else if (p.bpr > 16)
         hipLaunchKernelGGL((q4k_gemv_kernel<R, NW, NM, XF, true, MERGE>), dim3(grid), dim3(NW * 64), lds, st, p);
     else

@@ -31,6 +31,9 @@
 #include "gemv_prologue.hpp"
 #include "ksh_internal.hpp"
 
+KSH_STAMP_BUFFER
+KSH_STAMP_READER(ksh_stamps_matvec_q6k)
+
 namespace ksh {
 namespace {
 
@@ -277,6 +280,11 @@ __global__ __launch_bounds__(NW * 64) void q6r_gemv_kernel(Q6kParams p)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t xs[];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    // timeline build (tag 0): slots 0 entry, 1 loads issued, 2 vector staged, 3 barrier passed, 4 first row done, 5 last row stored, 6 acknowledged
+    // (every fourth workgroup leaves records: 2048 workgroups of 8 waves are more than the buffer holds)
+    const int sw = (blockIdx.x & 3) ? kStampWaves : (int)(blockIdx.x >> 2) * NW + wave;
+    (void)sw;
+    KSH_STAMP_BEGIN
     const int bl = lane >> 3;
     const int cols = p.bpr * 256;
     const size_t row_bytes = q6r_row_bytes(p.bpr);
@@ -296,8 +304,11 @@ __global__ __launch_bounds__(NW * 64) void q6r_gemv_kernel(Q6kParams p)
     StageRegs sr;
     stage_fetch<NW * 64, false, KMAX>(p.pro, cols, sr);
     load_rows(cur, min(w0, p.rows - 1));
+    KSH_STAMP(1);
     stage_finish<kXQ6, NW * 64, false, KMAX>(p.pro, xs, cols, sr);
+    KSH_STAMP(2);
     __syncthreads();
+    KSH_STAMP(3);
     if (w0 >= w1) return;
 
     XQ6r X[STEPS];
@@ -314,11 +325,14 @@ __global__ __launch_bounds__(NW * 64) void q6r_gemv_kernel(Q6kParams p)
             acc = wave_sum(acc);
             if (lane == 0 && row0 + r < w1) p.y[row0 + r] = acc;
         }
+        if (row0 == w0) KSH_STAMP(4);
 #pragma unroll
         for (int s = 0; s < STEPS; s++)
 #pragma unroll
             for (int r = 0; r < R; r++) cur[s][r] = nxt[s][r];
     }
+    KSH_STAMP(5);
+    KSH_STAMP_FLUSH(0, sw, 6);
 }
 
 struct Q6kGeom {

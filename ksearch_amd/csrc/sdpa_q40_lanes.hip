@@ -36,8 +36,16 @@
 #include "q40_pack.hpp"
 #include "ksh_internal.hpp"
 
+KSH_STAMP_BUFFER
+KSH_STAMP_READER(ksh_stamps_sdpa_lanes)
+
 namespace ksh {
 namespace {
+
+// timeline build, register-form kernel: tag 0 plain attention, 1 the fused decode step
+// slots: 0 entry, 1 every load of the front issued, 2 length and position in, 3 q (and the new row) ready,
+//        4 rows done, 5 row groups folded, 6 records stored (acknowledged)
+#define KSH_LANES_WAVE ((((int)blockIdx.z * (int)gridDim.y + (int)blockIdx.y) * (int)gridDim.x + (int)blockIdx.x) * NW + wave)
 
 enum { kModeDirect = 0, kModePart = 1, kModeMerge = 2, kModeSplitPart = 3 };   // SplitPart: values and (m, l) pairs in separate arrays, no merge
 constexpr int kRT = 4;   // row steps per softmax update
@@ -63,6 +71,19 @@ struct LaneParams {
     int no_append; // fused: the step's K / V row is in the cache already (a layer that reuses another layer's cache): q is normed and
                    // roped as usual, nothing is appended, every attended row comes from the cache
 };
+
+// Kernel arguments are fetched with scalar loads where they are first used; left alone the compiler spreads them
+// over the kernel's front (four groups here), and a wave pays one scalar-cache round trip after another before its
+// first vector load.  An empty statement at the top that reads every field makes them a few wide loads issued
+// together and one wait.  (The fields are only read, not passed through the statement: a pointer that comes out of
+// an opaque statement is no longer known to point to global memory and would be accessed with flat instructions.)
+__device__ __forceinline__ void touch_lane_params(const LaneParams &p)
+{
+    asm volatile("" ::"s"(p.q), "s"(p.k), "s"(p.v), "s"(p.meta), "s"(p.slot_ids), "s"(p.slot_stride), "s"(p.tmp), "s"(p.out), "s"(p.counters));
+    asm volatile("" ::"s"(p.qw), "s"(p.kw), "s"(p.rope), "s"(p.k_raw), "s"(p.v_raw), "s"(p.k_w), "s"(p.v_w));
+    asm volatile("" ::"s"(p.eps), "s"(p.scale), "s"(p.n_q), "s"(p.n_kv), "s"(p.max_t), "s"(p.nwg), "s"(p.meta_stride), "s"(p.mode), "s"(p.fused),
+                 "s"(p.groups), "s"(p.hsplit), "s"(p.balance), "s"(p.rope_row), "s"(p.kv_shared), "s"(p.no_append));
+}
 
 __device__ __forceinline__ uint32_t ld32_a2(const uint8_t *p)
 {
@@ -442,6 +463,7 @@ __global__ void sdpa_batch_meta_kernel(const float *meta, float *tok_meta, int n
 template <int HD, int GP, int NW>
 __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
 {
+    touch_lane_params(p);
     constexpr int LPR = HD / 8, RPS = 64 / LPR, HPL = GP / 4, NSLOT = NW * RPS, NT = NW * 64;
     constexpr int SLOTF = GP * HD + 2 * GP;   // floats of one row group's state
     constexpr int ROWB = HD / 32 * 18;
@@ -454,6 +476,7 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
     __shared__ int last_flag;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    KSH_STAMP_BEGIN
     const int j = lane % LPR, sub = lane / LPR, b = j >> 2, w = j & 3, c = w;
     int part = blockIdx.x, slot = blockIdx.z, nparts = p.nwg;
     const int kvh = blockIdx.y / p.hsplit, hg = blockIdx.y % p.hsplit;
@@ -502,8 +525,12 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
     // Vector loads return in the order they were issued: the length and position first, then what the fused
     // prologue needs (raw q / k / v of this workgroup's head tasks, the norm weights, the position's rope row
     // when it is given directly), then the rows.
-    const float *meta = p.meta + (size_t)slot * p.meta_stride;
-    const float meta_tlen = meta[0], meta_start = meta[1], meta_pos = dealt ? meta[3] : 0.f;
+    // The record is read with vector loads (opaque_zero_v) and without a branch around the position (the other kinds'
+    // record may end after three floats, so they read its first again): as scalar loads, or behind a branch, the
+    // values -- which end up in scalar registers -- were waited for right here, two memory round trips one after the
+    // other in front of every other load of the launch.
+    const float *meta = p.meta + (size_t)slot * p.meta_stride + opaque_zero_v();
+    const float meta_tlen = meta[0], meta_start = meta[1], meta_pos = meta[dealt ? 3 : 0];
     // head tasks: q heads 0..groups-1, then K and V (used by the owner only); a wave takes tasks wave, wave+NW, ...
     constexpr int PER = HD / 64, MAXT = GP / NW + 1;
     float xv[MAXT][PER], wq[PER], wk[PER], cs[PER / 2], sn[PER / 2];
@@ -531,7 +558,11 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
 #pragma unroll
         for (int t = 0; t < kRT; t++) cur[t] = load_row_at(0, min(dealt_row(0, t), p.max_t - 1));   // as if start == 0
     }
+    KSH_STAMP(1);
+    __builtin_amdgcn_sched_barrier(0);   // the record's first use stays behind the front's last load
     const int tlen = (int)meta_tlen, start = (int)meta_start;
+    KSH_STAMP_USE(tlen);
+    KSH_STAMP(2);
     const int chunk = (tlen + nparts - 1) / nparts;
     const int p0 = part * chunk;
     int p1 = min(p0 + chunk, tlen);
@@ -555,7 +586,7 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
     // ---- q into registers (and, fused, the new K/V row into the cache) -------
     float qv[GP][8], Sq[GP];
     if (p.fused) {
-        const int pos = min(max((int)meta_pos, 0), p.max_t - 1);
+        const int pos = dealt ? min(max((int)meta_pos, 0), p.max_t - 1) : 0;
         const int ntask = groups + (owner ? 2 : 0);
         if (!p.rope_row) {
             const float *rope = p.rope + (size_t)pos * HD;
@@ -614,6 +645,8 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
 #pragma unroll
     for (int h = 0; h < GP; h++)
         Sq[h] = ((qv[h][0] + qv[h][1]) + (qv[h][2] + qv[h][3])) + ((qv[h][4] + qv[h][5]) + (qv[h][6] + qv[h][7]));
+    KSH_STAMP_USE(Sq[0]);
+    KSH_STAMP(3);
 
     State<GP> st;
 #pragma unroll
@@ -666,6 +699,8 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
         process_rows<HD, GP, 1>(r, valid, live, qv, Sq, st, c);
     }
 
+    KSH_STAMP_USE(st.O[0][0]);
+    KSH_STAMP(4);
     // ---- fold the row groups of this workgroup ------------------------------
     {
         float *my = slots + (wave * RPS + sub) * SLOTF;
@@ -724,6 +759,7 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
             }
             accw[ob] = a; Mh[ob] = M; Lh[ob] = L;
         }
+        KSH_STAMP(5);
 #pragma unroll
         for (int ob = 0; ob < OBW; ob++) {
             const int o = tid + ob * NT;
@@ -748,6 +784,7 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
             }
         }
     }
+    KSH_STAMP_FLUSH(p.fused ? 1 : 0, KSH_LANES_WAVE, 6);
     if (p.mode != kModeMerge) return;
 
     // ---- the last partition to arrive folds the partials (lower.rs:5897-6087) -

@@ -131,6 +131,21 @@ def bench_floor(ctx, eng, ev, copies, steps, warmup):
 
         us = min(timed_graph(ctx, ev, one, steps, warmup) for _ in range(5)) * 1e3 / steps
         out[name] = dict(kernel=k.name, us_per_launch=round(us, 3), tbps=round(wbytes / us / 1e6, 2) if mode else None)
+    # what an empty launch costs in other shapes: workgroups x threads, with and without the LDS reservation, and with an
+    # argument block of the GEMV's size
+    shapes = {}
+    for wgs in (256, 512, 1024):
+        for thr in (64, 128, 256, 512):
+            row = []
+            for no_lds, big_args in ((0, 0), (1, 0), (0, 1)):
+                k = ctx.compile(hip.make_desc(hip.Kind.READ_FLOOR, (rows, cols, 0, wgs, thr, no_lds, big_args), (hip.DType.Q4K,)))
+
+                def one(i, k=k):
+                    ctx.encode_offsets_multi(k, [big], [(i % copies) * wbytes], [sink], [0])
+
+                row.append(round(min(timed_graph(ctx, ev, one, steps, warmup) for _ in range(3)) * 1e3 / steps, 3))
+            shapes[f"{wgs}x{thr}"] = dict(us_with_lds=row[0], us_without_lds=row[1], us_with_gemv_sized_arguments=row[2])
+    out["empty_launch_by_shape"] = shapes
     big.release()
     g = min((bench_matvec(ctx, eng, ev, hip.DType.Q4K, rows, cols, w, x, copies, steps, warmup) for _ in range(5)),
             key=lambda r: r["us_per_launch"])

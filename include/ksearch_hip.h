@@ -50,7 +50,15 @@ enum ksh_dtype {
 
 /* The KernelKind variants on the hot path (crates/ksearch_ir/src/kernel.rs:399-744).
  * Inputs/outputs are listed in binding order; "act" = activation dtype
- * (dtypes[1], F32 unless stated). */
+ * (dtypes[1], F32 unless stated).
+ * dtypes[1] = KSH_F16: the reference's buffer types (x_dtype, crates/ksearch_codegen/src/lower.rs:1134-1140;
+ * buffer_empty_f16, crates/ksearch_gemma/src/gemma_prim.rs:229-252): every binding that is an activation vector, a
+ * norm weight or the logits is half, f32 inside the kernels, results rounded to nearest even; packed weights and
+ * caches, the rope table, meta records, token ids, split-KV partials and the argmax index keep their types.  Taken
+ * by the kinds Eng calls (KSH_MATVEC .. KSH_GATE_UP_GELU and their RMSNORM_ forms, the RMSNORM and SDPA kinds,
+ * KSH_ATTEND_DECODE, KSH_ATTN_MERGE_MATVEC, KSH_COPY_SCALE_INDEXED, KSH_GELU_MUL, KSH_ADD_SCALE,
+ * KSH_MATVEC_GELU_MUL, KSH_COPY_SLICE, KSH_SOFTCAP_ARGMAX, and the plain KSH_MATVEC_BATCH, whose Y is half with
+ * dtypes[2] = KSH_F16). */
 enum ksh_kind {
     /* Matvec{rows,cols,weight_dtype}: y = W x.  dims: rows, cols.
      * dtypes[0] = Q4K | Q6K.  in: W, x   out: y[rows] */
@@ -220,7 +228,9 @@ enum ksh_kind {
      * workgroup size and LDS reservation of the default GEMV schedule (2 rows per wave, 8 waves), doing nothing
      * (mode 0), issuing exactly the GEMV's weight loads and nothing else (mode 1), or reading the same bytes with
      * flat 128-bit loads (mode 2).  dims: rows, cols (<= 4096), mode.  dtypes: Q4K.  in: W   out: sink f32[1]
-     * (never written for real weights) */
+     * (never written for real weights).  The empty launch takes other shapes: dims[3] workgroups, dims[4] threads per
+     * workgroup (a multiple of 64 up to 512), dims[5] = 1 no LDS reservation, dims[6] = 1 an argument block of the
+     * GEMV's size (0 everywhere: the GEMV's own launch shape and four scalar arguments). */
     KSH_READ_FLOOR = 28,
     /* sdpa_hybrid_kv_batch (crates/ksearch_kernels/src/lib.rs:1592-1623, lower.rs:4961-4983): causal attention of
      * n_tok consecutive prompt tokens over one Q4_0 cache that already holds their rows.  meta = f32{tlen of token

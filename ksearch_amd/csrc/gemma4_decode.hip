@@ -21,6 +21,7 @@
 
 #include "ksh_device.hpp"
 #include "ksh_internal.hpp"
+#include "section_timer.hpp"
 
 namespace {
 
@@ -144,6 +145,7 @@ struct ksh_gemma4 {
     ksh_kvpool *round_pool = nullptr;
     uint64_t round_pool_uid = 0;   // a new pool can come up at a destroyed pool's address: the graphs are tied to the pool's uid as well
     bool round_graph = true;       // KSEARCH_ROUND_GRAPH, read when the model is created
+    ksh::SectionTimer prof;        // KSEARCH_PROFILE (read when the model is created): per-section times of every decode step
     int r_count = 0;
 };
 
@@ -237,6 +239,7 @@ int encode_token(ksh_gemma4 *m, bool want_logits, int &launches)
     launches = 0;
     Stream s{m->x, m->xb};
     if (enc(m, m->k_embed, {m->g.token_embd, m->tok}, {s.cur}, launches)) return 1;
+    m->prof.mark(SectionTimer::kEmbed);
     if (c.ple_dim > 0) {
         // ple_from_idx + ple_prepass (gemma_prim.rs:712-728, 845-878)
         if (enc(m, m->k_ple_gather, {m->g.ple_embd, m->tok}, {m->ple_tok}, launches) ||
@@ -244,6 +247,7 @@ int encode_token(ksh_gemma4 *m, bool want_logits, int &launches)
             enc(m, m->k_ple_norm, {m->ple_tmp, m->g.ple_proj_norm}, {m->ple_ctx}, launches) ||
             enc(m, m->k_ple_mix, {m->ple_ctx, m->ple_tok}, {m->ple_ctx}, launches))
             return 1;
+        m->prof.mark(SectionTimer::kPrepass);
     }
     for (int l = 0; l < c.n_layers; l++) {
         const ksh_gemma4_layer &L = m->layers[l];
@@ -280,6 +284,7 @@ int encode_token(ksh_gemma4 *m, bool want_logits, int &launches)
             if (enc(m, P.sdpa, {m->tq, kc, vc, meta}, {m->attn_tmp, m->to}, launches)) return 1;
         }
         if (enc(m, P.oproj, {L.wo, parts ? m->attn_tmp : m->to}, {m->y}, launches)) return 1;
+        m->prof.mark(SectionTimer::kAttn);
         // -- feed-forward on norm(x + rms(o)*post_attn_norm)
         s.y = m->y;
         s.w = L.post_attn_norm;
@@ -294,6 +299,7 @@ int encode_token(ksh_gemma4 *m, bool want_logits, int &launches)
                 return 1;
         }
         if (enc(m, P.down, {L.wdown, m->ff}, {m->y}, launches)) return 1;
+        m->prof.mark(SectionTimer::kMlp);
         s.y = m->y;
         s.w = L.post_ffw_norm;
         if (c.ple_dim > 0) {
@@ -305,6 +311,7 @@ int encode_token(ksh_gemma4 *m, bool want_logits, int &launches)
                 return 1;
             std::swap(s.cur, s.other);
             if (enc(m, P.ple_proj, {L.proj, m->ple_u}, {m->y}, launches)) return 1;
+            m->prof.mark(SectionTimer::kPle);
             s.y = m->y;
             s.w = L.post_norm;
         }
@@ -328,6 +335,7 @@ int encode_token(ksh_gemma4 *m, bool want_logits, int &launches)
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return hip_fail(e, "advance launch");
     launches += 1;
+    m->prof.mark(SectionTimer::kLogits);
     return 0;
 }
 
@@ -335,7 +343,12 @@ int run_token(ksh_gemma4 *m, bool want_logits, bool use_graph)
 {
     if (m->pos >= m->c.max_seq) return set_error("max_seq exceeded");   // gemma_prim.rs:882-884
     int n = 0;
-    if (!use_graph) {
+    if (m->prof.on) {
+        // gemma_prim.rs:885: with KSEARCH_PROFILE every step is timed section by section (launched kernel by kernel)
+        m->prof.begin((hipStream_t)ksh_stream(m->ctx));
+        if (encode_token(m, want_logits, n)) return 1;
+        m->prof.report(want_logits ? "decode" : "prefill", m->pos);
+    } else if (!use_graph) {
         if (encode_token(m, want_logits, n)) return 1;
     } else {
         ksh_graph *&g = want_logits ? m->g_full : m->g_body;
@@ -353,7 +366,7 @@ int run_token(ksh_gemma4 *m, bool want_logits, bool use_graph)
         }
         if (ksh_graph_launch(m->ctx, g)) return 1;
     }
-    if (want_logits && !use_graph) m->launches_full = n;
+    if (want_logits && (!use_graph || m->prof.on)) m->launches_full = n;
     m->pos += 1;
     return 0;
 }
@@ -735,6 +748,7 @@ int ksh_gemma4_create(ksh_ctx *ctx, const ksh_gemma4_cfg *cfg, const ksh_gemma4_
     m->layers.assign(layers, layers + c.n_layers);
     m->plan.resize(c.n_layers);
     if (const char *e = std::getenv("KSEARCH_ROUND_GRAPH")) m->round_graph = e[0] != '0';
+    m->prof.on = std::getenv("KSEARCH_PROFILE") != nullptr;
     const int max_hd = std::max(c.hd_swa, c.hd_full);
     int max_ff = 0;
     for (const ksh_gemma4_layer &L : m->layers) max_ff = std::max(max_ff, (int)L.ffn);

@@ -37,6 +37,7 @@
 
 #include "ksh_device.hpp"
 #include "ksh_internal.hpp"
+#include "section_timer.hpp"
 
 namespace {
 
@@ -126,6 +127,7 @@ struct ksh_gemma {
             *c_g = nullptr, *c_u = nullptr, *c_ff = nullptr, *c_tmp = nullptr, *c_meta = nullptr,
             *c_po = nullptr, *c_pg = nullptr, *c_pd = nullptr;   // unfolded partial sums of the o, gate | up and down projections
     int c_nwg = 0;
+    ksh::SectionTimer prof;   // KSEARCH_PROFILE (read when the model is created): per-section times of every decode step
 };
 
 namespace {
@@ -239,9 +241,11 @@ int encode_token(ksh_gemma *m, bool want_logits, bool short_ctx, int &launches)
         }
         if (short_ctx ? enc(m, m->k_oproj_merge, {L.wo, m->attn_tmp}, {m->y}, launches) : enc(m, m->k_oproj, {L.wo, m->to}, {m->y}, launches))
             return 1;
+        m->prof.mark(SectionTimer::kAttn);
         if (enc(m, m->k_gate_up, {L.wgate, L.wup, m->y, L.ffn_norm, L.post_attn_norm, cur}, {m->ff, other}, launches)) return 1;
         std::swap(cur, other);
         if (enc(m, m->k_down, {L.wdown, m->ff}, {m->y}, launches)) return 1;
+        m->prof.mark(SectionTimer::kMlp);
     }
     if (want_logits) {
         // the last layer's rmsnorm_add and the output norm ride in the LM head's prologue
@@ -269,6 +273,7 @@ int encode_token(ksh_gemma *m, bool want_logits, bool short_ctx, int &launches)
         if (launch_decode_tail(*m->k_argmax, (const float *)ksh_buffer_device_ptr(m->logits), t, (hipStream_t)ksh_stream(m->ctx))) return 1;
         ctx_mark_pending(m->ctx);
         launches += 2;
+        m->prof.mark(SectionTimer::kLogits);
         return 0;
     }
     hipStream_t st = (hipStream_t)ksh_stream(m->ctx);
@@ -279,6 +284,7 @@ int encode_token(ksh_gemma *m, bool want_logits, bool short_ctx, int &launches)
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return hip_fail(e, "advance launch");
     launches += 1;
+    m->prof.mark(SectionTimer::kLogits);
     return 0;
 }
 
@@ -287,7 +293,12 @@ int run_token(ksh_gemma *m, bool want_logits, bool use_graph)
     if (m->pos >= m->c.max_seq) return set_error("max_seq exceeded");   // gemma_prim.rs:882-884
     int n = 0;
     const bool short_ctx = m->k_attend_parts && m->pos < m->short_context;
-    if (!use_graph) {
+    if (m->prof.on) {
+        // gemma_prim.rs:885: with KSEARCH_PROFILE every step is timed section by section (launched kernel by kernel)
+        m->prof.begin((hipStream_t)ksh_stream(m->ctx));
+        if (encode_token(m, want_logits, short_ctx, n)) return 1;
+        m->prof.report(want_logits ? "decode" : "prefill", m->pos);
+    } else if (!use_graph) {
         if (encode_token(m, want_logits, short_ctx, n)) return 1;
     } else {
         ksh_graph *&g = want_logits ? m->g_full[short_ctx] : m->g_body[short_ctx];
@@ -305,7 +316,7 @@ int run_token(ksh_gemma *m, bool want_logits, bool use_graph)
         }
         if (ksh_graph_launch(m->ctx, g)) return 1;
     }
-    if (want_logits && !use_graph) m->launches_full = n;
+    if (want_logits && (!use_graph || m->prof.on)) m->launches_full = n;
     m->pos += 1;
     return 0;
 }
@@ -587,6 +598,7 @@ int ksh_gemma_create(ksh_ctx *ctx, const ksh_gemma_cfg *cfg, const ksh_gemma_lay
             get(g, KSH_SDPA_SLOTS, {c.n_q, c.n_kv, c.hd, c.max_seq, 1, g->nwg}, {KSH_Q40, KSH_F32}, {c.attn_scale}, &g->k_sdpa))
             return 1;
     }
+    g->prof.on = getenv("KSEARCH_PROFILE") != nullptr;
     if (ksh_gemma_reset(g)) return 1;
     *out = m.release();
     return 0;

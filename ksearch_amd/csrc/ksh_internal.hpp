@@ -56,6 +56,11 @@ struct ksh_kernel {
     size_t scratch_bytes = 0;
     void *scratch = nullptr;
     int (*launch)(const ksh_kernel &, const ksh::LaunchArgs &, hipStream_t) = nullptr;
+    // a handle with half activations at the boundary (half_boundary.hip): the f32 handle it wraps, which bindings are
+    // half, and where their f32 staging lies in `scratch`
+    const ksh_kernel *inner = nullptr;
+    uint32_t half_in = 0, half_out = 0;
+    size_t stage_in[ksh::kMaxIn] = {}, stage_out[ksh::kMaxOut] = {};
 };
 
 namespace ksh {
@@ -65,6 +70,9 @@ int ctx_device(ksh_ctx *ctx);   // the ordinal of the device the context's strea
 // a buffer object over bytes [off, off + bytes) of `parent` (retained until the view is released); nullptr + error when out of range
 ksh_buf *buffer_view(ksh_buf *parent, size_t off, size_t bytes);
 void ctx_mark_pending(ksh_ctx *ctx);
+// half activations at the boundary: whether the kind takes them, and the wrapping of its bound f32 handle
+bool half_boundary_kind(const ksh_kernel_desc &d);
+int bind_half_boundary(ksh_kernel &k, const ksh_kernel &inner);
 // resolves the device address of the static partial-result array of ksh_softcap_argmax_static for the current
 // device (called when a context is created, with the context's device current; the entry point then uses the
 // address kept for the context's device)

@@ -293,6 +293,25 @@ int ksh_kernel_get(ksh_ctx *ctx, const ksh_kernel_desc *desc, ksh_kernel **out)
         *out = it->second.get();
         return 0;
     }
+    if (key.dtypes[1] == KSH_F16 && half_boundary_kind(key)) {
+        // half activations at the boundary: the f32 handle of the same descriptor, wrapped (half_boundary.hip)
+        ksh_kernel_desc f32 = *desc;
+        f32.dtypes[1] = KSH_F32;
+        if (key.kind == KSH_MATVEC_BATCH && f32.dtypes[2] == KSH_F16) f32.dtypes[2] = KSH_F32;
+        ksh_kernel *inner = nullptr;
+        if (ksh_kernel_get(ctx, &f32, &inner)) return 1;
+        auto k = std::make_unique<ksh_kernel>();
+        k->desc = key;
+        if (bind_half_boundary(*k, *inner)) return 1;
+        if (k->scratch_bytes) {
+            KSH_HIP(hipMalloc(&k->scratch, k->scratch_bytes));
+            KSH_HIP(hipMemset(k->scratch, 0, k->scratch_bytes));
+            KSH_HIP(hipStreamSynchronize(nullptr));
+        }
+        *out = k.get();
+        ctx->kernels[key] = std::move(k);
+        return 0;
+    }
     ksh_sched planned{};
     bool have_plan = false;
     // tg = all ones asks for the library's default schedule whatever the plan cache holds (the schedule search times

@@ -52,14 +52,30 @@ __global__ __launch_bounds__(kNW * 64) void read_floor_kernel(const uint8_t *__r
     if (acc == 0x12345678u) sink[0] = 1.0f;      // keeps the loads alive; random weights never take this branch
 }
 
+// the empty launch again with an argument block of the GEMV's size (19 pointers and integers: 136 bytes)
+struct PaddedArgs {
+    const uint8_t *p[9];
+    float *sink;
+    int v[14];
+};
+__global__ __launch_bounds__(kNW * 64) void read_floor_empty_args_kernel(PaddedArgs a)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t xs[];
+    if (threadIdx.x == 0xFFFF) a.sink[0] = (float)xs[0] + (float)a.v[13];
+}
+
 int launch_read_floor(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
 {
     const int rows = (int)k.desc.dims[0], bpr = (int)(k.desc.dims[1] / 256), mode = (int)k.desc.dims[2];
-    const dim3 grid(k.info.grid[0]), block(kNW * 64);
+    const dim3 grid(k.info.grid[0]), block(k.info.block[0]);
     const size_t lds = k.info.lds_bytes;
     const uint8_t *W = (const uint8_t *)a.in[0];
     float *sink = (float *)a.out[0];
-    if (mode == 0) hipLaunchKernelGGL(read_floor_kernel<0>, grid, block, lds, st, W, rows, bpr, sink);
+    if (mode == 0 && k.desc.dims[6]) {
+        PaddedArgs pa{};
+        pa.p[0] = W; pa.sink = sink; pa.v[0] = rows; pa.v[1] = bpr;
+        hipLaunchKernelGGL(read_floor_empty_args_kernel, grid, block, lds, st, pa);
+    } else if (mode == 0) hipLaunchKernelGGL(read_floor_kernel<0>, grid, block, lds, st, W, rows, bpr, sink);
     else if (mode == 1) hipLaunchKernelGGL(read_floor_kernel<1>, grid, block, lds, st, W, rows, bpr, sink);
     else hipLaunchKernelGGL(read_floor_kernel<2>, grid, block, lds, st, W, rows, bpr, sink);
     const hipError_t e = hipGetLastError();
@@ -80,9 +96,21 @@ int bind_read_floor(ksh_kernel &k)
     k.info.n_outputs = 1;
     k.in_bytes[0] = (size_t)rows * (cols / 256) * kBlk; k.in_align[0] = 16;
     k.out_bytes[0] = 4; k.out_align[0] = 4;
-    const uint32_t grid = (uint32_t)((rows + kR * kNW - 1) / (kR * kNW));
+    uint32_t grid = (uint32_t)((rows + kR * kNW - 1) / (kR * kNW)), threads = kNW * 64;
     // LDS as the GEMV's int8 digit-plane image of the vector: 208 bytes per 64 columns + 16 per group + 128
-    set_launch(k, grid, 1, 1, kNW * 64, (uint32_t)((cols / 64) * 224 + 128));
+    uint32_t lds = (uint32_t)((cols / 64) * 224 + 128);
+    // the empty launch in other shapes: dims[3] workgroups, dims[4] threads per workgroup (a multiple of 64 up to 512),
+    // dims[5] = 1 without the LDS reservation, dims[6] = 1 with an argument block of the GEMV's size
+    if (mode == 0) {
+        const int64_t g = k.desc.dims[3], t = k.desc.dims[4];
+        if (g < 0 || g > (1 << 20) || t < 0 || t > kNW * 64 || t % 64) return set_error("read_floor: %lld workgroups of %lld threads", (long long)g, (long long)t);
+        if (g) grid = (uint32_t)g;
+        if (t) threads = (uint32_t)t;
+        if (k.desc.dims[5]) lds = 0;
+    } else if (k.desc.dims[3] || k.desc.dims[4] || k.desc.dims[5] || k.desc.dims[6]) {
+        return set_error("read_floor: the launch shape is a parameter of the empty launch (mode 0) only");
+    }
+    set_launch(k, grid, 1, 1, threads, lds);
     set_name(k, "read_floor_q4k_%s", mode == 0 ? "empty" : mode == 1 ? "lanes" : "flat");
     k.launch = launch_read_floor;
     return 0;

@@ -139,6 +139,31 @@ def test_generate_graph_equals_eager_and_oracle(small_model):
     assert n_same >= 8
 
 
+def test_profile_mode_prints_sections_and_changes_nothing(ctx, capfd, monkeypatch):
+    """KSEARCH_PROFILE (gemma_prim.rs:885, 1260-1273): every step prints one line with its per-section times; the
+    tokens are those of the unprofiled model."""
+    w = synth.gemma_weights(SMALL, 500, oracle.quantize_q4k, synth.chunked(oracle.quantize_q6k), std=0.05)
+    prompt = [int(t) for t in np.random.default_rng(505).integers(0, SMALL["vocab"], 5)]
+    plain = hip.Gemma(ctx, SMALL, w)
+    want, _, _ = plain.generate(prompt, 6, use_graph=True)
+    plain.close()
+    monkeypatch.setenv("KSEARCH_PROFILE", "1")
+    prof = hip.Gemma(ctx, SMALL, w)
+    monkeypatch.delenv("KSEARCH_PROFILE")
+    capfd.readouterr()
+    got, _, _ = prof.generate(prompt, 6, use_graph=True, serial_prefill=True)
+    prof.close()
+    err = capfd.readouterr().err
+    assert got == want
+    lines = [l for l in err.splitlines() if l.startswith("[profile]")]
+    assert len([l for l in lines if " decode " in l]) == 6 and len([l for l in lines if " prefill " in l]) == len(prompt) - 1
+    fields = dict(f.split("=") for f in lines[-1].split()[2:])
+    assert set(fields) == {"pos", "embed", "prepass", "attn", "mlp", "ple", "logits+sync", "total"}
+    ms = {k: float(v[:-2]) for k, v in fields.items() if k != "pos"}
+    assert ms["attn"] > 0 and ms["mlp"] > 0 and ms["logits+sync"] > 0
+    assert abs(ms["total"] - sum(v for k, v in ms.items() if k != "total")) < 1e-2
+
+
 def test_generate_refuses_past_max_seq(small_model):
     gpu, _, _ = small_model
     gpu.reset()

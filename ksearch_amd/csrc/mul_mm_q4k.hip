@@ -51,31 +51,47 @@ constexpr int PITCH2 = 32 + 8;     // halves per LDS row of the min-term tiles
 // operand per (token, superblock): 32 halves = Sx_hi[8] | Sx_hi[8] | Sx_lo[8] | 0[8].
 // Xf[token / 32][k / 16][lane][8] with lane = token % 32 + 32 * ((k / 8) % 2): one 32 x 16 fragment is 1 KB,
 // lane after lane, so that a multiplying wave fetches it with a single 128-bit load per lane and the
-// activations never pass through LDS.  One thread per 8 elements; the four threads of a sub-block add their
-// sums up over the quad.
+// activations never pass through LDS.
+// A wave takes 32 tokens x one 32-column sub-block: lane (token % 32, h) converts the 8-element runs h and 2 + h
+// of the sub-block and is lane token % 32 + 32 h of the sub-block's two fragments, so both leave as whole
+// kilobytes, lane after lane (with a thread per run in row order, the eight 16-byte pieces of a 128-byte line of
+// Xf came from eight workgroups: 5.7 us for 2 MB).  The four waves of a workgroup take neighbouring sub-blocks, so
+// that together they read whole lines of X.  The sub-block's sum is (run 0 + run 1) + (run 2 + run 3), the two
+// halves of the wave trading their runs' sums.
 __global__ __launch_bounds__(256) void mm_prep_x_kernel(const uint16_t *__restrict__ X, _Float16 *__restrict__ Xf,
                                                         _Float16 *__restrict__ SxA, int batch, int cols)
 {
-    const int idx = blockIdx.x * 256 + threadIdx.x;
-    if (idx >= batch * (cols / 8)) return;   // (whole quads: cols is a multiple of 32)
-    const u32x4_t in = reinterpret_cast<const u32x4_t *>(X)[idx];
-    const uint32_t w[4] = {in.x, in.y, in.z, in.w};
-    float f[8];
+    const int lane = threadIdx.x & 63, wave = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int nsub = cols / 32, tb = wave / nsub, s = wave - tb * nsub;
+    const int t = tb * 32 + (lane & 31), h = lane >> 5;
+    if (tb * 32 >= batch) return;
+    const bool live = t < batch;
+    const u32x4_t *row = reinterpret_cast<const u32x4_t *>(X + (size_t)min(t, batch - 1) * cols);   // (rows past the batch: read a real row, store nothing)
+    float c[2];
+    h8 o[2];
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        f[2 * i] = as_f32(w[i] << 16);
-        f[2 * i + 1] = as_f32(w[i] & 0xFFFF0000u);
+    for (int r = 0; r < 2; r++) {
+        const u32x4_t in = row[4 * s + 2 * r + h];
+        const uint32_t w[4] = {in.x, in.y, in.z, in.w};
+        float f[8];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            f[2 * i] = as_f32(w[i] << 16);
+            f[2 * i + 1] = as_f32(w[i] & 0xFFFF0000u);
+        }
+        c[r] = ((f[0] + f[1]) + (f[2] + f[3])) + ((f[4] + f[5]) + (f[6] + f[7]));
+#pragma unroll
+        for (int i = 0; i < 8; i++) o[r][kperm(i)] = (_Float16)f[i];
     }
-    float sum = ((f[0] + f[1]) + (f[2] + f[3])) + ((f[4] + f[5]) + (f[6] + f[7]));
-    sum += dpp_f32<0xB1>(sum);   // quad neighbours: 1 0 3 2, then 2 3 0 1
-    sum += dpp_f32<0x4E>(sum);
-    h8 o;
-#pragma unroll
-    for (int i = 0; i < 8; i++) o[kperm(i)] = (_Float16)f[i];
-    const int k8 = cols / 8, t = idx / k8, j = idx - t * k8;
-    reinterpret_cast<h8 *>(Xf)[((size_t)(t >> 5) * (cols / 16) + (j >> 1)) * 64 + (t & 31) + 32 * (j & 1)] = o;
-    if ((threadIdx.x & 3) == 0) {
-        const int s = j / 4;
+    // the other half's runs: (run 0 + run 1) and (run 2 + run 3), the same in both halves
+    const auto x0 = __builtin_amdgcn_permlane32_swap(as_u32(c[0]), as_u32(c[0]), false, false);
+    const auto x1 = __builtin_amdgcn_permlane32_swap(as_u32(c[1]), as_u32(c[1]), false, false);
+    float sum = (as_f32(x0[0]) + as_f32(x0[1])) + (as_f32(x1[0]) + as_f32(x1[1]));
+    if (!live) return;
+    h8 *frag = reinterpret_cast<h8 *>(Xf) + ((size_t)tb * (cols / 16) + 2 * s) * 64 + lane;
+    frag[0] = o[0];
+    frag[64] = o[1];
+    if (h == 0) {
         sum = pinned(sum);
         const _Float16 hi = (_Float16)sum;
         const _Float16 lo = (_Float16)(sum - (float)hi);
@@ -1420,7 +1436,7 @@ int launch_mul_mm(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
     } else if (f32x && tile)
         hipLaunchKernelGGL(mm_prep_rows_kernel<0>, pg, pb, 0, st, (const float *)a.in[1], nullptr, nullptr, nullptr, nullptr, Xf, Xf_lo, SxA, SxA_lo, cols, 0.f, 0, inv_s);
     else if (f32x) hipLaunchKernelGGL(mm_prep_x_f32_kernel, dim3((n + 255) / 256), dim3(256), 0, st, (const float *)a.in[1], Xf, Xf_lo, SxA, SxA_lo, batch, cols);
-    else hipLaunchKernelGGL(mm_prep_x_kernel, dim3((n + 255) / 256), dim3(256), 0, st, (const uint16_t *)a.in[1], Xf, SxA, batch, cols);
+    else hipLaunchKernelGGL(mm_prep_x_kernel, dim3(((batch + 31) / 32 * (cols / 32) + 3) / 4), dim3(256), 0, st, (const uint16_t *)a.in[1], Xf, SxA, batch, cols);
     MmParams p;
     p.W = (const uint8_t *)a.in[0];
     p.Y = (float *)a.out[0];

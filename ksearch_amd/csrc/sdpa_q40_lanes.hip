@@ -460,10 +460,20 @@ __global__ void sdpa_batch_meta_kernel(const float *meta, float *tok_meta, int n
 }
 
 // grid = (nwg, n_kv, n_slots)
-template <int HD, int GP, int NW>
-__global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
+// FUSED: the decode step's form (p.fused), a kernel of its own: with the choice made at compile time the front of
+// either form is one run of loads without the other form's branches in it, and the wait for the record in front of
+// the rows counts exactly the loads behind it.
+template <int HD, int GP, int NW, bool FUSED>
+__global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p_in)
 {
-    touch_lane_params(p);
+    touch_lane_params(p_in);
+    LaneParams p = p_in;
+    p.fused = FUSED;
+    if (FUSED) {   // one sequence, its own cache, partitions of equal size: what the other kinds' fields would select is not compiled in
+        p.balance = 0;
+        p.slot_ids = nullptr;
+        p.kv_shared = 0;
+    }
     constexpr int LPR = HD / 8, RPS = 64 / LPR, HPL = GP / 4, NSLOT = NW * RPS, NT = NW * 64;
     constexpr int SLOTF = GP * HD + 2 * GP;   // floats of one row group's state
     constexpr int ROWB = HD / 32 * 18;
@@ -478,8 +488,8 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p)
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     KSH_STAMP_BEGIN
     const int j = lane % LPR, sub = lane / LPR, b = j >> 2, w = j & 3, c = w;
-    int part = blockIdx.x, slot = blockIdx.z, nparts = p.nwg;
-    const int kvh = blockIdx.y / p.hsplit, hg = blockIdx.y % p.hsplit;
+    int part = blockIdx.x, slot = FUSED ? 0 : blockIdx.z, nparts = p.nwg;
+    const int kvh = p.n_kv == 1 ? 0 : blockIdx.y / p.hsplit, hg = blockIdx.y - kvh * p.hsplit;   // (one kv head: no division in the front)
     const int groups = p.groups;
     const int head0 = (kvh * p.hsplit + hg) * groups;   // first q head of this workgroup
     // partial records: rec(head, part) = tmp + rec_base + head * rec_hs + part * rec_ps
@@ -913,6 +923,7 @@ __global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_m
 {
     static_assert(TR == 16 || TR == 32, "tile rows");
     static_assert(HD % HDV == 0 && (HDV == HD || TR == 32), "V halves come with tiles of 32 rows");
+    touch_lane_params(p);   // every kernel argument in one round trip
     constexpr int NW = kMfmaRound / TR, NT = NW * 64, NB = HD / 32, ROWB = NB * 18, TILEB = TR * ROWB;
     constexpr int NBV = HDV / 32, ROWBV = NBV * 18, TILEBV = TR * ROWBV;   // this workgroup's share of a V row
     constexpr int STRIP = TILEB + TILEBV + TR * NB * 4 + TR * NBV * 4;     // K bytes, V bytes, K scales, V scales
@@ -1309,7 +1320,8 @@ template <int HD, int GP, int NW>
 int launch_inst(const LaneParams &p, int n_slots, hipStream_t st)
 {
     const size_t lds = lanes_lds_bytes<HD, GP, NW>();
-    hipLaunchKernelGGL((sdpa_lanes_kernel<HD, GP, NW>), dim3(p.nwg, p.n_kv * p.hsplit, n_slots), dim3(NW * 64), lds, st, p);
+    if (p.fused) hipLaunchKernelGGL((sdpa_lanes_kernel<HD, GP, NW, true>), dim3(p.nwg, p.n_kv * p.hsplit, n_slots), dim3(NW * 64), lds, st, p);
+    else hipLaunchKernelGGL((sdpa_lanes_kernel<HD, GP, NW, false>), dim3(p.nwg, p.n_kv * p.hsplit, n_slots), dim3(NW * 64), lds, st, p);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : hip_fail(e, "sdpa (register form) launch");
 }

@@ -188,14 +188,21 @@ __device__ __forceinline__ void stage_fetch(const Prologue &pr_in, int cols, Sta
         // eight partitions' values and (m, l) pairs; partitions past nwg re-read the
         // last one, so that the number of loads is fixed
         if (wbase < n4) {
-            const int e = tid * 4, h = e >> pr.hd_log2, d = e - (h << pr.hd_log2);
-            const float *o = pr.x + (((size_t)h * pr.nwg) << pr.hd_log2) + d;
-            const float *ml = pr.w_norm + (size_t)h * pr.nwg * 2;
+            // byte offsets in 32 bits against the two base pointers (the buffers are a few hundred KB): one add per load
+            // where 64-bit addresses cost a shift and an add-with-carry pair each, in front of the first weight load
+            const uint32_t e = (uint32_t)tid * 4, h = e >> pr.hd_log2, d = e - (h << pr.hd_log2);
+            const uint32_t o0 = (((h * (uint32_t)pr.nwg) << pr.hd_log2) + d) * 4, ml0 = h * (uint32_t)pr.nwg * 8;
+            const KSH_GLOBAL char *ob = (const KSH_GLOBAL char *)pr.x, *mb = (const KSH_GLOBAL char *)pr.w_norm;
+            typedef float f32x2_t __attribute__((ext_vector_type(2)));
 #pragma unroll
-            for (int q = 0; q < kMergeMaxParts; q++) s.x[q] = ldg_f4(o + ((size_t)min(q, pr.nwg - 1) << pr.hd_log2), 0);
+            for (int q = 0; q < kMergeMaxParts; q++) {
+                const f32x4_t v = *(const KSH_GLOBAL f32x4_t *)(ob + (o0 + (((uint32_t)min(q, pr.nwg - 1) << pr.hd_log2) * 4)));
+                s.x[q] = make_float4(v.x, v.y, v.z, v.w);
+            }
 #pragma unroll
             for (int q = 0; q < kMergeMaxParts / 2; q++) {
-                const float2 a = ldg_f2(ml, min(2 * q, pr.nwg - 1)), b = ldg_f2(ml, min(2 * q + 1, pr.nwg - 1));
+                const f32x2_t a = *(const KSH_GLOBAL f32x2_t *)(mb + (ml0 + (uint32_t)min(2 * q, pr.nwg - 1) * 8));
+                const f32x2_t b = *(const KSH_GLOBAL f32x2_t *)(mb + (ml0 + (uint32_t)min(2 * q + 1, pr.nwg - 1) * 8));
                 s.wn[q] = make_float4(a.x, a.y, b.x, b.y);
             }
         }

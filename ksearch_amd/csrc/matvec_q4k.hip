@@ -109,9 +109,22 @@ __device__ __forceinline__ T sel3(bool in1, bool in2, T a0, T a1, T a2)
 // index must live in scalar registers (readfirstlane): the matrix is then
 // picked with scalar loads of the kernel arguments instead of a per-lane
 // gather from them, which would put a memory round trip in front of every load.
+template <int NM>
 __device__ __forceinline__ WaveTask wave_task(const MatvecParams &p, int wv, int rpw)
 {
     WaveTask t;
+    // one matrix, or a gate | up pair whose waves all own rows of both: nothing to choose between (a scalar branch
+    // instead of thirty selects in front of the first weight load)
+    if (NM == 2 || (p.waves1 == 0 && p.waves2 == 0)) {
+        t.W0 = p.W0;
+        t.W1 = p.W1;
+        t.y = p.y0;
+        t.rows = p.rows0;
+        t.row0 = wv * rpw;
+        t.active = t.row0 < t.rows;
+        if (!t.active) t.row0 = 0;
+        return t;
+    }
     // selects between already-fetched arguments rather than indexing them
     const bool in1 = p.mode == 0 && wv >= p.waves0;
     const bool in2 = in1 && wv - p.waves0 >= p.waves1;
@@ -152,7 +165,7 @@ __global__ __launch_bounds__(NW * 64) void q4k_gemv_kernel(MatvecParams p_in)
     const int bpr = CB ? CB : p.bpr, cols = bpr * 256;
     const size_t row_bytes = (size_t)bpr * kQ4kBytes;
     constexpr int KMAX = CB ? (CB * 64 + NW * 64 - 1) / (NW * 64) : kStageX;   // float4 of the vector per thread
-    const WaveTask t = wave_task(p, blockIdx.x * NW + wave, R);
+    const WaveTask t = wave_task<NM>(p, blockIdx.x * NW + wave, R);
 
     const uint8_t *rowp[NM][R];
 #pragma unroll
@@ -261,17 +274,20 @@ __global__ __launch_bounds__(NW * 64) void q4k_gemv_half_kernel(MatvecParams p_i
     const int bl = BPR == 8 ? slot : min(slot, BPR - 1);
     const bool mine = BPR == 8 || slot < BPR;
     constexpr size_t row_bytes = (size_t)bpr * kQ4kBytes;
-    WaveTask t = wave_task(p, blockIdx.x * NW + wave, 2 * R);
+    WaveTask t = wave_task<NM>(p, blockIdx.x * NW + wave, 2 * R);
     const int row0 = t.row0 + hw * R;
 
     Q4kLane L[NM][R];
     StageRegs sr;
-    stage_fetch<NW * 64, MERGE>(p.pro, bpr * 256, sr);
+    // (the instances that merge attention partitions are launched for that prologue alone: the other kinds' loads
+    // and arithmetic are not compiled into them)
+    constexpr int KIND = MERGE ? kMergeParts : -1;
+    stage_fetch<NW * 64, MERGE, kStageX, KIND>(p.pro, bpr * 256, sr);
     // With a normalising prologue every wave's vector loads are queued before any wave's weight loads: behind
     // another wave's HBM-cold weights in the compute unit's memory pipeline they came back up to 1.3 us late, and
     // the prologue's reduction waits for the slowest wave.
     KSH_STAMP(7);
-    if (p.pro.kind != kPlain) __syncthreads();
+    if (MERGE || p.pro.kind != kPlain) __syncthreads();
     auto load_r = [&](int r) {
         const size_t off = (size_t)min(row0 + r, t.rows - 1) * row_bytes + (size_t)bl * kQ4kBytes;
         L[0][r] = q4k_load(t.W0 + off, g);
@@ -285,7 +301,7 @@ __global__ __launch_bounds__(NW * 64) void q4k_gemv_half_kernel(MatvecParams p_i
     // 8192 with the add-then-norm prologue: 8.1 -> 7.1 us).
     load_r(0);
     KSH_STAMP(1);
-    stage_finish<XF, NW * 64, MERGE>(p.pro, xs, bpr * 256, sr);
+    stage_finish<XF, NW * 64, MERGE, kStageX, KIND>(p.pro, xs, bpr * 256, sr);
     KSH_STAMP(2);
     __syncthreads();
     KSH_STAMP(3);

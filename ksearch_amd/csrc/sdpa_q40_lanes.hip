@@ -918,12 +918,16 @@ __device__ __forceinline__ int mfma_k_elem(int s, int kq)
 // HDV < HD (heads of 512 as two halves of 256): the workgroups of blockIdx.y = 2 * kvh + half both work out the scores
 // and the softmax over all HD dimensions (the same numbers twice) and each takes P.V for its HDV dimensions of V,
 // whose accumulators are what limits the head size a wave can hold.
-template <int HD, int TR, int HDV = HD>
-__global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_mfma_kernel(LaneParams p)
+// BAL: the launch whose partitions are dealt to the slots by length (p.balance), known when the kernel is built: either
+// form's front then holds its own way to its rows only.
+template <int HD, int TR, int HDV = HD, bool BAL = false>
+__global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_mfma_kernel(LaneParams p_in)
 {
+    LaneParams p = p_in;
+    p.balance = BAL;
     static_assert(TR == 16 || TR == 32, "tile rows");
     static_assert(HD % HDV == 0 && (HDV == HD || TR == 32), "V halves come with tiles of 32 rows");
-    touch_lane_params(p);   // every kernel argument in one round trip
+    touch_lane_params(p_in);   // every kernel argument in one round trip
     constexpr int NW = kMfmaRound / TR, NT = NW * 64, NB = HD / 32, ROWB = NB * 18, TILEB = TR * ROWB;
     constexpr int NBV = HDV / 32, ROWBV = NBV * 18, TILEBV = TR * ROWBV;   // this workgroup's share of a V row
     constexpr int STRIP = TILEB + TILEBV + TR * NB * 4 + TR * NBV * 4;     // K bytes, V bytes, K scales, V scales
@@ -1378,9 +1382,9 @@ int launch_bound(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
         p.mode = kModePart;
         if (mfma) {
             if (nw == 0xFF)
-                hipLaunchKernelGGL((sdpa_mfma_kernel<256, 32>), dim3(p.nwg, p.n_kv, n_slots), dim3(kMfmaRound / 32 * 64), (mfma_lds_bytes<256, 32>()), st, p);
+                hipLaunchKernelGGL((sdpa_mfma_kernel<256, 32, 256, true>), dim3(p.nwg, p.n_kv, n_slots), dim3(kMfmaRound / 32 * 64), (mfma_lds_bytes<256, 32>()), st, p);
             else
-                hipLaunchKernelGGL((sdpa_mfma_kernel<256, 16>), dim3(p.nwg, p.n_kv, n_slots), dim3(kMfmaRound / 16 * 64), (mfma_lds_bytes<256, 16>()), st, p);
+                hipLaunchKernelGGL((sdpa_mfma_kernel<256, 16, 256, true>), dim3(p.nwg, p.n_kv, n_slots), dim3(kMfmaRound / 16 * 64), (mfma_lds_bytes<256, 16>()), st, p);
             const hipError_t e0 = hipGetLastError();
             if (e0 != hipSuccess) return hip_fail(e0, "sdpa (matrix-core form) launch");
         } else if (launch_lanes(p, hd, nw, n_slots, st)) {

@@ -358,7 +358,7 @@ def bench_timeline(ctx, eng, tokens=24):
     share one time axis.  Per launch: when its waves enter, and the median / slowest wave at each phase boundary,
     in microseconds from the launch's first wave; `gap_before_us` is the time from the previous launch's last
     acknowledged store to this launch's first wave.  The timestamps themselves cost a little (one counter read and
-    one store per phase and wave): the timeline build decodes ~3 % slower than the product build."""
+    one store per wave): the timeline build decodes a few per cent slower than the product build."""
     from ksearch_amd import hip, synth
 
     L = hip.lib()
@@ -450,10 +450,10 @@ def cpu_baseline_matvec(w, x, rows, cols, budget_s=1.5):
 
 
 # HBM bytes per launch of the headline kernel, from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
-# profiles/q4k_gemv_cfg0_cold.txt (2.00 x 4765.1 KiB fetched + 16.0 KiB written).  Counters cannot be read from
+# profiles/q4k_gemv_cfg0_cold.txt (2.00 x 4705.5 KiB fetched + 16.0 KiB written).  Counters cannot be read from
 # inside this script, so the figure is carried here for the kernel it was taken on; a headline kernel that is not in
 # the table is an error (the counters have to be taken again for it), never a silent null.
-MEASURED_TRAFFIC_BYTES = {"matvec_q4k_r2_w8_v3": 9775309}
+MEASURED_TRAFFIC_BYTES = {"matvec_q4k_r2_w8_v3": 9653248}
 
 
 def measured_traffic(kernel: str) -> int:

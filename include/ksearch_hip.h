@@ -270,7 +270,9 @@ enum ksh_kind {
  * means "library default, whatever the plan cache holds". */
 typedef struct {
     uint64_t tg;       /* threads per workgroup (64 * waves) */
-    uint32_t vec;      /* inner-product variant.  GEMV: 1 = byte converts + f32 FMA, 3 = int8 dot over 3 digit planes.
+    uint32_t vec;      /* inner-product variant.  GEMV: 1 = byte converts + f32 FMA, 3 = int8 dot over 3 digit planes,
+                        * 2 (Q4_K kinds, by request only: the schedule search never offers it) = int8 dot over 2 digit
+                        * planes, the activations to 2^-16 of their 32-element sub-block's largest magnitude.
                         * Attention: 1 = LDS-tile form, 3 = register (vector-ALU) form, 2 = matrix-core form of the
                         * row phase (heads of 256, up to 8 q heads per kv head.  KSH_SDPA_SLOTS with up to 16 slots:
                         * the default there; lds_tile = 32 | 16 picks four waves with tiles of 32 rows or eight with

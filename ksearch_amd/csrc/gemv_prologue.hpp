@@ -19,6 +19,11 @@
 //         followed by s[] and the exact f32 sub-block sums Sx[].  |x - s X| <= s/2, i.e.
 //         2^-21 of the sub-block's largest magnitude: below f32 summation noise of a
 //         2048-term dot, so the integer dot products (exact) keep f32-class accuracy.
+//   I8x2  the same with s = amax/32767 and two digits, X = 256 m + l with m a signed and l an unsigned byte (the
+//         nibbles are non-negative, so l meets them in the unsigned dot instruction), M[64] L[64] + 16 bytes of
+//         padding per 64 elements (lane stride 36 dwords): |x - s X| <= 2^-16 of the sub-block's largest magnitude
+//         -- finer than the half-precision activations of the reference -- for a third fewer integer dot
+//         instructions per weight.
 #pragma once
 
 #include "ksh_device.hpp"
@@ -27,7 +32,7 @@ namespace ksh {
 
 enum { kPlain = 0, kRms = 1, kAddThenRms = 2, kMergeParts = 3 };
 constexpr int kMergeMaxParts = 8;
-enum { kXF32 = 0, kXI8 = 3, kXQ6 = 6 };
+enum { kXF32 = 0, kXI2 = 2, kXI8 = 3, kXQ6 = 6 };
 
 struct Prologue {
     const float *x;        // kPlain/kRms: the vector; kAddThenRms: y; kMergeParts: o[heads][nwg][hd]
@@ -42,6 +47,7 @@ struct Prologue {
 
 __host__ __device__ constexpr int xs_f32_floats(int cols) { return cols + (cols >> 6) * 4; }
 __host__ __device__ constexpr int xs_i8_bytes(int cols) { return (cols >> 6) * 208 + (cols >> 5) * 8; }
+__host__ __device__ constexpr int xs_i2_bytes(int cols) { return (cols >> 6) * 144 + (cols >> 5) * 8; }
 __device__ __forceinline__ int xs_f32_index(int e) { return e + ((e >> 6) << 2); }
 
 // Q6 planes: per 128 elements H[128] M[128] L[128], then for each run of 8
@@ -52,7 +58,7 @@ __host__ __device__ constexpr int xs_q6_bytes(int cols) { return (cols >> 7) * k
 template <int XF>
 __host__ __device__ constexpr size_t xs_image_bytes(int cols)
 {
-    return XF == kXI8 ? (size_t)xs_i8_bytes(cols) : XF == kXQ6 ? (size_t)xs_q6_bytes(cols) : (size_t)xs_f32_floats(cols) * 4;
+    return XF == kXI8 ? (size_t)xs_i8_bytes(cols) : XF == kXI2 ? (size_t)xs_i2_bytes(cols) : XF == kXQ6 ? (size_t)xs_q6_bytes(cols) : (size_t)xs_f32_floats(cols) * 4;
 }
 template <int XF>
 __host__ __device__ constexpr size_t xs_bytes(int cols)
@@ -130,6 +136,26 @@ __device__ __forceinline__ void store_x4(uint8_t *lds, int cols, int i, float4 v
     }
     const float amax = oct_max(fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
     const float sum = oct_sum((v.x + v.y) + (v.z + v.w));
+    if (XF == kXI2) {
+        const float inv = amax > 0.f ? 32767.0f / amax : 0.f;
+        const float xs4[4] = {v.x, v.y, v.z, v.w};
+        int m[4], l[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int X = (int)rintf(xs4[k] * inv);
+            l[k] = X & 255;
+            m[k] = X >> 8;
+        }
+        uint8_t *chunk = lds + (i >> 4) * 144 + (i & 15) * 4;
+        *reinterpret_cast<uint32_t *>(chunk) = pack4_i8(m[0], m[1], m[2], m[3]);
+        *reinterpret_cast<uint32_t *>(chunk + 64) = pack4_i8(l[0], l[1], l[2], l[3]);
+        if ((threadIdx.x & 7) == 0) {
+            float *sc = reinterpret_cast<float *>(lds + (cols >> 6) * 144);
+            sc[2 * (i >> 3)] = amax * (1.0f / 32767.0f);
+            sc[2 * (i >> 3) + 1] = sum;
+        }
+        return;
+    }
     const float inv = amax > 0.f ? 1048575.0f / amax : 0.f;
     const float s = amax * (1.0f / 1048575.0f);
     const float xs4[4] = {v.x, v.y, v.z, v.w};

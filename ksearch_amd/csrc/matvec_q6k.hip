@@ -347,7 +347,7 @@ Q6kGeom pick_geom6(const ksh_sched &s, int rows)
     // rows a wave walks: long enough to amortise the x staging, short enough
     // to leave >= 8 workgroups per CU
     int rpw = s.unroll ? (int)s.unroll * G.R : 16;
-    while (rpw > G.R && rows / (rpw * G.NW) < 2048) rpw >>= 1;
+    if (!s.unroll) while (rpw > G.R && rows / (rpw * G.NW) < 2048) rpw >>= 1;   // (an explicit count is taken as given)
     if (rpw < G.R) rpw = G.R;
     G.rpw = rpw;
     return G;

@@ -629,17 +629,38 @@ __global__ __launch_bounds__(kThreadsMM, TM == 64 ? 2 : 1) void q_mul_mm_kernel(
     fetch_a(0, a0);
     if (!LO) fetch_a(min(1, nsteps - 1), a1);
     __syncthreads();   // stage 0 is written
-
     auto mul_step = [&](int sb, auto gtag, ARegs &A) __attribute__((always_inline)) {
         constexpr int g = decltype(gtag)::value;
         const int step = 4 * sb + g;
         const _Float16 *Bs = main_stage(step);
+        // B operands a k slice ahead (bf16 / f16 activations on the 128-token tile): left to itself the compiler reads a
+        // slice's two operands into the registers the previous slice's products have just released, so every slice
+        // begins with an LDS round trip in front of its four matrix instructions (cfg2: 32.5 -> 31.1 us per pair).  With
+        // f32 activations a slice has eight products and the prompt passes do not gain (256 tokens: 5.1 -> 5.3 ms).
+        constexpr bool BPIPE = !LO && TM == 128;
+        h8 bb[2][2];
+        if (BPIPE) {
+#pragma unroll
+            for (int nt = 0; nt < 2; nt++)
+                bb[0][nt] = *reinterpret_cast<const h8 *>(&Bs[(wn * 64 + nt * 32 + lm) * PITCH + lk]);
+        }
 #pragma unroll
         for (int ks = 0; ks < KS / 16; ks++) {
             h8 b[2];
+            if (BPIPE) {
+                if (ks + 1 < KS / 16) {
 #pragma unroll
-            for (int nt = 0; nt < 2; nt++)
-                b[nt] = *reinterpret_cast<const h8 *>(&Bs[(wn * 64 + nt * 32 + lm) * PITCH + 16 * ks + lk]);
+                    for (int nt = 0; nt < 2; nt++)
+                        bb[(ks + 1) & 1][nt] = *reinterpret_cast<const h8 *>(&Bs[(wn * 64 + nt * 32 + lm) * PITCH + 16 * (ks + 1) + lk]);
+                }
+                __builtin_amdgcn_sched_barrier(0);   // (the requests stay in front of this slice's products)
+                b[0] = bb[ks & 1][0];
+                b[1] = bb[ks & 1][1];
+            } else {
+#pragma unroll
+                for (int nt = 0; nt < 2; nt++)
+                    b[nt] = *reinterpret_cast<const h8 *>(&Bs[(wn * 64 + nt * 32 + lm) * PITCH + 16 * ks + lk]);
+            }
 #pragma unroll
             for (int mt = 0; mt < MT; mt++)
 #pragma unroll
@@ -659,6 +680,7 @@ __global__ __launch_bounds__(kThreadsMM, TM == 64 ? 2 : 1) void q_mul_mm_kernel(
                 A.a[mt][ks] = afrag(mt, min(step + AHEAD, nsteps - 1), ks);
                 if (LO) A.al[mt][ks] = afrag_lo(mt, min(step + AHEAD, nsteps - 1), ks);
             }
+            if (BPIPE) __builtin_amdgcn_sched_barrier(0);
         }
         if (g == 3) {
             // ---- end of the superblock: bias + mins through the short second product, then the row scale

@@ -108,6 +108,41 @@ struct XGroup<kXI8> {
     }
 };
 
+template <>
+struct XGroup<kXI2> {
+    uint32_t M[16], Lo[16];   // two digit planes (signed high bytes, unsigned low bytes): dwords 0..7 low sub-block, 8..15 high sub-block
+    float s_lo, s_hi, sx_lo, sx_hi;
+    __device__ __forceinline__ void load(const uint8_t *lds, int cols, int b, int g)
+    {
+        const int c = b * 4 + g;
+        const uint4 *p = reinterpret_cast<const uint4 *>(lds + c * 144);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint4 m = p[i], l = p[4 + i];
+            M[4 * i] = m.x; M[4 * i + 1] = m.y; M[4 * i + 2] = m.z; M[4 * i + 3] = m.w;
+            Lo[4 * i] = l.x; Lo[4 * i + 1] = l.y; Lo[4 * i + 2] = l.z; Lo[4 * i + 3] = l.w;
+        }
+        const float4 sc = *reinterpret_cast<const float4 *>(lds + (cols >> 6) * 144 + c * 16);
+        s_lo = sc.x; sx_lo = sc.y; s_hi = sc.z; sx_hi = sc.w;
+    }
+    __device__ __forceinline__ void dot(const Q4kLane &L, float &lo, float &hi) const
+    {
+        int ml = 0, ll = 0, mh = 0, lh = 0;
+        const uint32_t q[8] = {L.qa.x, L.qa.y, L.qa.z, L.qa.w, L.qb.x, L.qb.y, L.qb.z, L.qb.w};
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const int a = (int)(q[k] & 0x0F0F0F0Fu), c = (int)((q[k] >> 4) & 0x0F0F0F0Fu);
+            ml = __builtin_amdgcn_sdot4(a, (int)M[k], ml, false);
+            ll = (int)__builtin_amdgcn_udot4((uint32_t)a, Lo[k], (uint32_t)ll, false);
+            mh = __builtin_amdgcn_sdot4(c, (int)M[8 + k], mh, false);
+            lh = (int)__builtin_amdgcn_udot4((uint32_t)c, Lo[8 + k], (uint32_t)lh, false);
+        }
+        // |256 ml + ll| <= 32 * 15 * 32767 < 2^24: the conversion is exact
+        lo = s_lo * (float)((ml << 8) + ll);
+        hi = s_hi * (float)((mh << 8) + lh);
+    }
+};
+
 // one (row, superblock, group): the f32 contribution to y[row]
 template <int XF>
 __device__ __forceinline__ float q4k_group_dot(const Q4kLane &L, int g, const XGroup<XF> &X)

@@ -90,6 +90,27 @@ def test_matvec_q4k_cfg0_full_size(ctx, eng, sched):
     assert_close(got, oracle.matvec_f64(oracle.Q4K, w, rows, cols, x), 1e-5, "cfg0 vs f64")
 
 
+@pytest.mark.parametrize("rows,cols,nsg,nr0", [(4096, 4096, 8, 2), (2048, 2048, 8, 1), (2048, 1536, 8, 2), (512, 8192, 4, 1)])
+def test_matvec_q4k_two_digit_planes(ctx, eng, rows, cols, nsg, nr0):
+    # vec = 2: the activations as two int8 digits, 2^-16 of the sub-block's largest magnitude.  By request only (the
+    # schedule search does not list it); held to the 1e-3 bar against the oracle and to 1e-4 of the f64 truth on
+    # normal inputs, and bit-exact on unit vectors (one digit pair per sub-block is then exact)
+    sched = dict(tg=64 * nsg, vec=2, unroll=1, nsg=nsg, nr0=nr0, k_split=1, lds_tile=0)
+    w = synth.q4k_blocks(rows * cols // 256, seed=rows + cols)
+    x = synth.normal_f32(cols, seed=11)
+    bw, bx, by = ctx.buffer_bytes(w), ctx.buffer_f32(x), ctx.buffer_empty_f32(rows)
+    eng.matvec_wd(ctx, rows, cols, DType.Q4K, bw, bx, by, sched)
+    got = ctx.read_f32(by, rows)
+    assert_close(got, oracle.matvec(oracle.Q4K, w, rows, cols, x), TOL, f"two planes {rows}x{cols}")
+    assert_close(got, oracle.matvec_f64(oracle.Q4K, w, rows, cols, x), 1e-4, "two planes vs f64")
+    wd = oracle.dequant(oracle.Q4K, w, rows * cols).reshape(rows, cols)
+    for j in (0, 31, 32, cols - 1):
+        e = np.zeros(cols, dtype=np.float32)
+        e[j] = 1.0
+        eng.matvec_wd(ctx, rows, cols, DType.Q4K, bw, ctx.buffer_f32(e), by, sched)
+        assert np.allclose(ctx.read_f32(by, rows), wd[:, j], rtol=1e-6, atol=1e-9), j
+
+
 def test_matvec_q4k_unit_vectors_recover_weights(ctx, eng):
     # y = W e_j is column j of the dequantized matrix: pins the lane -> element map
     rows, cols = 8, 4096

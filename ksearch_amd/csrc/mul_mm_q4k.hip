@@ -635,9 +635,10 @@ __global__ __launch_bounds__(kThreadsMM, TM == 64 ? 2 : 1) void q_mul_mm_kernel(
         const _Float16 *Bs = main_stage(step);
         // B operands a k slice ahead (bf16 / f16 activations on the 128-token tile): left to itself the compiler reads a
         // slice's two operands into the registers the previous slice's products have just released, so every slice
-        // begins with an LDS round trip in front of its four matrix instructions (cfg2: 32.5 -> 31.1 us per pair).  With
-        // f32 activations a slice has eight products and the prompt passes do not gain (256 tokens: 5.1 -> 5.3 ms).
-        constexpr bool BPIPE = !LO && TM == 128;
+        // begins with an LDS round trip in front of its four matrix instructions (cfg2: 32.5 -> 31.1 us per pair; with
+        // f32 activations a slice has eight products to hide it behind: prompts of 1024 / 4000 tokens 14.1 / 67.6 ->
+        // 14.0 / 67.1 ms).  The 64-token tile loses by it (a 256-token prompt 5.1 -> 5.3 ms) and keeps the plain order.
+        constexpr bool BPIPE = TM == 128;
         h8 bb[2][2];
         if (BPIPE) {
 #pragma unroll

@@ -77,12 +77,14 @@ def test_cfg4_lockstep_with_the_oracle(model):
     n_pre = len(prompt) - 1
     m.prefill_chunk(prompt[:n_pre])
     flipped, t0 = 0, time.time()
+    flipped_by_layer = np.zeros(n_layers, dtype=np.int64)
     first_flip = None           # the first position whose K / V row the device packed differently from the oracle (by one code)
     for i in range(n_pre):
         rows = device_rows(ctx, bufs, i, row)
         cpu.forward(prompt[i], want_logits=False, adopt_rows=rows, threads=16)
         assert cpu.row_max_step.max() <= 1.0 + 1e-3, f"prompt position {i}: {cpu.row_max_step.max()} codes, layer {np.argmax(cpu.row_max_step.max(1))}"
         flipped += int(cpu.row_diff_bytes.sum())
+        flipped_by_layer += cpu.row_diff_bytes.reshape(n_layers, -1).sum(1).astype(np.int64)
         if first_flip is None and cpu.row_diff_bytes.sum() > 0:
             first_flip = i
     seq = [prompt[-1]] + generated[:-1]
@@ -98,6 +100,7 @@ def test_cfg4_lockstep_with_the_oracle(model):
         # K / V rows: the device's are the oracle's up to one code of a value on a rounding boundary
         assert cpu.row_max_step.max() <= 1.0 + 1e-3, f"step {i}: {cpu.row_max_step.max()} codes, layer {np.argmax(cpu.row_max_step.max(1))}"
         flipped += int(cpu.row_diff_bytes.sum())
+        flipped_by_layer += cpu.row_diff_bytes.reshape(n_layers, -1).sum(1).astype(np.int64)
         if first_flip is None and cpu.row_diff_bytes.sum() > 0:
             first_flip = i
         # logits: all 262144, every step; the bar is stated on |d| / max(|want|, rms(want)), and the plain |d| / |want|
@@ -132,7 +135,10 @@ def test_cfg4_lockstep_with_the_oracle(model):
         assert explained, f"free run differs at step {n_same} with no K / V flip up to position {at} and a margin of {margins[n_same]:.2e}"
     print(f"cfg4 lockstep: {n_pre} prompt positions prefilled as one chunk + {len(seq)} decode steps, worst logit error {worst:.2e} (floored), {worst_plain:.2e} (plain, elements >= rms), {argmax_checked} greedy tokens equal the oracle's, "
           f"{near_ties} near-ties, {flipped} of {n * n_layers * 2 * row} KV bytes differ by one code ({time.time() - t0:.0f}s)")
-    assert flipped <= 0.02 * n * n_layers * 2 * row
+    print("cfg4 lockstep: bytes that differ by one code, per layer: " + " ".join(str(int(v)) for v in flipped_by_layer))
+    # measured: 350 - 533 of 2,756,160 bytes (1.3e-4 - 1.9e-4), at most 24 in any layer; the bounds leave a factor of five and more
+    assert flipped <= 1e-3 * n * n_layers * 2 * row
+    assert flipped_by_layer.max() <= 4e-3 * n * 2 * row
     assert argmax_checked >= 0.9 * len(seq)
 
 

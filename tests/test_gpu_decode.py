@@ -105,7 +105,9 @@ def test_forward_token_matches_oracle_teacher_forced(small_model):
         if top2[1] - top2[0] > 2e-3 * max(abs(top2[1]), float(np.sqrt(np.mean(c_logits ** 2)))):
             assert g_next == c_next, f"step {i}: margin {top2[1] - top2[0]}"
             agree += 1
-    assert agree >= 30 and flipped <= 0.02 * 40 * SMALL["n_layers"] * 2 * row and gpu.pos == cpu.pos == len(toks)
+    print(f"small model, 40 teacher-forced steps: {flipped} of {40 * SMALL['n_layers'] * 2 * row} KV bytes differ by one code")
+    # (measured: 1 - 2 of 17,280 bytes; the bound is 34)
+    assert agree >= 30 and flipped <= 0.002 * 40 * SMALL["n_layers"] * 2 * row and gpu.pos == cpu.pos == len(toks)
     with pytest.raises(hip.KshError, match="outside the vocabulary"):
         gpu.forward_token(SMALL["vocab"])
 

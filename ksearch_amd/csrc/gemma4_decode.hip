@@ -121,11 +121,12 @@ struct ksh_gemma4 {
     ksh_kernel *k_embed = nullptr, *k_ple_gather = nullptr, *k_ple_proj = nullptr, *k_ple_norm = nullptr, *k_ple_mix = nullptr,
                *k_lm_head[2] = {nullptr, nullptr}, *k_argmax = nullptr;
     ksh_graph *g_body = nullptr, *g_full = nullptr;   // the graphs of the caches in use (own or a pool slot's)
+    ksh_graph *g_span = nullptr;                      // kSpan decode steps with logits as one graph (generate's loop)
     std::vector<float> rope0_full, rope0_swa;
     int pos = 0, launches_full = 0;
     // serving: the model's own caches, and the graphs captured for each slot of the pool it was last bound to
     std::vector<ksh_buf *> own_k, own_v;
-    struct SlotGraphs { ksh_graph *body = nullptr, *full = nullptr; };
+    struct SlotGraphs { ksh_graph *body = nullptr, *full = nullptr, *span = nullptr; };
     ksh_kvpool *pool = nullptr;
     uint64_t pool_uid = 0;   // (a new pool can be allocated where a destroyed one lay: the address alone does not identify it)
     std::vector<SlotGraphs> slot_graphs;
@@ -368,6 +369,34 @@ int run_token(ksh_gemma4 *m, bool want_logits, bool use_graph)
     }
     if (want_logits && (!use_graph || m->prof.on)) m->launches_full = n;
     m->pos += 1;
+    return 0;
+}
+
+// Several decode steps as one graph launch: positions, attended ranges, rope rows and the token live on the device
+// and are advanced by the step's last kernel, so a token's graph repeated kSpan times is kSpan tokens (what it saves
+// is the time between two graph launches, ~6 us each).
+constexpr int kSpan = 8;
+
+int run_span(ksh_gemma4 *m)
+{
+    ksh_graph *&g = m->g_span;
+    if (!g) {
+        int n = 0;
+        if (ksh_synchronize(m->ctx)) return 1;
+        if (ksh_graph_begin(m->ctx)) return 1;
+        for (int i = 0; i < kSpan; i++) {
+            if (encode_token(m, true, n)) {
+                ksh_graph *dead = nullptr;
+                ksh_graph_end(m->ctx, &dead);
+                ksh_graph_destroy(dead);
+                return 1;
+            }
+        }
+        if (ksh_graph_end(m->ctx, &g)) return 1;
+        m->launches_full = n;   // (the count of one step: every step starts its own)
+    }
+    if (ksh_graph_launch(m->ctx, g)) return 1;
+    m->pos += kSpan;
     return 0;
 }
 
@@ -720,7 +749,8 @@ void stash_graphs(ksh_gemma4 *m)
     ksh_gemma4::SlotGraphs &g = m->bound_slot >= 0 ? m->slot_graphs[(size_t)m->bound_slot] : m->own_graphs;
     g.body = m->g_body;
     g.full = m->g_full;
-    m->g_body = m->g_full = nullptr;
+    g.span = m->g_span;
+    m->g_body = m->g_full = m->g_span = nullptr;
 }
 
 }  // namespace
@@ -813,7 +843,8 @@ void ksh_gemma4_destroy(ksh_gemma4 *m)
     stash_graphs(m);
     ksh_graph_destroy(m->own_graphs.body);
     ksh_graph_destroy(m->own_graphs.full);
-    for (auto &g : m->slot_graphs) { ksh_graph_destroy(g.body); ksh_graph_destroy(g.full); }
+    ksh_graph_destroy(m->own_graphs.span);
+    for (auto &g : m->slot_graphs) { ksh_graph_destroy(g.body); ksh_graph_destroy(g.full); ksh_graph_destroy(g.span); }
     for (ksh_graph *g : m->round_graphs) ksh_graph_destroy(g);
     delete m;
 }
@@ -861,8 +892,15 @@ int ksh_gemma4_generate(ksh_gemma4 *m, const uint32_t *prompt, int n_prompt, int
     if (ksh_synchronize(m->ctx)) return 1;
     const auto t1 = clk::now();
     const int first = m->pos;
-    for (int i = 0; i < n_new; i++)
-        if (run_token(m, true, (use_graph & 1) != 0)) return 1;
+    for (int i = 0; i < n_new;) {
+        if ((use_graph & 1) && n_new - i >= kSpan && !m->prof.on && m->pos + kSpan <= m->c.max_seq) {
+            if (run_span(m)) return 1;
+            i += kSpan;
+        } else {
+            if (run_token(m, true, (use_graph & 1) != 0)) return 1;
+            i += 1;
+        }
+    }
     if (ksh_synchronize(m->ctx)) return 1;
     const auto t2 = clk::now();
     if (prefill_ms) *prefill_ms = std::chrono::duration<double, std::milli>(t1 - t0).count();
@@ -1331,7 +1369,7 @@ int ksh_gemma4_bind_slot(ksh_gemma4 *m, ksh_kvpool *pool, int slot)
     if (pool && !same_pool) {
         // graphs captured over another pool's buffers are of no use any more
         if (ksh_synchronize(m->ctx)) return 1;
-        for (auto &g : m->slot_graphs) { ksh_graph_destroy(g.body); ksh_graph_destroy(g.full); }
+        for (auto &g : m->slot_graphs) { ksh_graph_destroy(g.body); ksh_graph_destroy(g.full); ksh_graph_destroy(g.span); }
         int max_batch = 0;
         ksh_kvpool_dims(pool, &max_batch, nullptr, nullptr, nullptr, nullptr);
         m->slot_graphs.assign((size_t)max_batch, ksh_gemma4::SlotGraphs{});
@@ -1347,6 +1385,7 @@ int ksh_gemma4_bind_slot(ksh_gemma4 *m, ksh_kvpool *pool, int slot)
     const ksh_gemma4::SlotGraphs &g = pool ? m->slot_graphs[(size_t)slot] : m->own_graphs;
     m->g_body = g.body;
     m->g_full = g.full;
+    m->g_span = g.span;
     m->pos = pos;
     // the device-side position, attended ranges and rope rows, ordered behind whatever is still running
     const int at = std::min(pos, c.max_seq - 1);

@@ -116,6 +116,7 @@ struct ksh_gemma {
                *k_oproj = nullptr, *k_add_then = nullptr, *k_gate_up = nullptr, *k_down = nullptr,
                *k_lm_head = nullptr, *k_argmax = nullptr;
     ksh_graph *g_body[2] = {nullptr, nullptr}, *g_full[2] = {nullptr, nullptr};   // [1]: the short-context form
+    ksh_graph *g_span[2] = {nullptr, nullptr};   // kSpan decode steps with logits in one graph (generate's loop)
     int pos = 0;
     int launches_full = 0;
     int nwg = 16;
@@ -319,6 +320,42 @@ int run_token(ksh_gemma *m, bool want_logits, bool use_graph)
     if (want_logits && (!use_graph || m->prof.on)) m->launches_full = n;
     m->pos += 1;
     return 0;
+}
+
+// Several decode steps as one graph launch.  Position, attended length, rope row and the token itself live on the
+// device and are advanced by the step's last kernel, so a token's graph repeated kSpan times is kSpan tokens; the
+// generate loop uses it while the whole span stays on one form of the attention step.
+constexpr int kSpan = 8;
+
+int run_span(ksh_gemma *m)
+{
+    const bool short_ctx = m->k_attend_parts && m->pos < m->short_context;
+    ksh_graph *&g = m->g_span[short_ctx];
+    if (!g) {
+        int n = 0;
+        if (ksh_synchronize(m->ctx)) return 1;
+        if (ksh_graph_begin(m->ctx)) return 1;
+        for (int i = 0; i < kSpan; i++) {
+            if (encode_token(m, true, short_ctx, n)) {
+                ksh_graph *dead = nullptr;
+                ksh_graph_end(m->ctx, &dead);
+                ksh_graph_destroy(dead);
+                return 1;
+            }
+        }
+        if (ksh_graph_end(m->ctx, &g)) return 1;
+        m->launches_full = n;   // (the count of one step: every step starts its own)
+    }
+    if (ksh_graph_launch(m->ctx, g)) return 1;
+    m->pos += kSpan;
+    return 0;
+}
+
+bool span_fits(const ksh_gemma *m, int remaining)
+{
+    if (remaining < kSpan || m->prof.on || m->pos + kSpan > m->c.max_seq) return false;
+    if (!m->k_attend_parts) return true;
+    return (m->pos < m->short_context) == (m->pos + kSpan - 1 < m->short_context);
 }
 
 // prefill_chunk's chunk length (gemma_prim.rs:16)
@@ -611,6 +648,7 @@ void ksh_gemma_destroy(ksh_gemma *m)
     for (int i = 0; i < 2; i++) {
         ksh_graph_destroy(m->g_body[i]);
         ksh_graph_destroy(m->g_full[i]);
+        ksh_graph_destroy(m->g_span[i]);
     }
     delete m;
 }
@@ -681,8 +719,15 @@ int ksh_gemma_generate(ksh_gemma *m, const uint32_t *prompt, int n_prompt, int n
     if (ksh_synchronize(m->ctx)) return 1;
     const auto t1 = clk::now();
     const int first = m->pos;
-    for (int i = 0; i < n_new; i++)
-        if (run_token(m, true, graph)) return 1;
+    for (int i = 0; i < n_new;) {
+        if (graph && span_fits(m, n_new - i)) {
+            if (run_span(m)) return 1;
+            i += kSpan;
+        } else {
+            if (run_token(m, true, graph)) return 1;
+            i += 1;
+        }
+    }
     if (ksh_synchronize(m->ctx)) return 1;
     const auto t2 = clk::now();
     if (prefill_ms) *prefill_ms = std::chrono::duration<double, std::milli>(t1 - t0).count();

@@ -28,6 +28,37 @@ def test_library_exports_every_declared_symbol():
     assert sorted(hip.SYMBOLS) == names
 
 
+def _header_prototypes():
+    """name -> number of parameters, from the header's declarations"""
+    text = open(os.path.join(ROOT, "include", "ksearch_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    out = {}
+    for name, params in re.findall(r"(?m)^\s*(?:const\s+)?\w+(?:\s+const)?[\s\*]+(ksh_\w+)\s*\(([^;{)]*)\)\s*;", text):
+        params = params.strip()
+        out[name] = 0 if params in ("", "void") else params.count(",") + 1
+    return out
+
+
+def test_rust_listing_in_the_integration_notes_covers_the_header():
+    """The binding a maintainer would add declares every function of the header with the
+    header's number of parameters, and every structure the header defines by value."""
+    protos = _header_prototypes()
+    assert sorted(protos) == header_symbols()
+    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    rust = text[text.index("## 2. FFI declarations"):text.index("## 3.")]
+    declared = {}
+    for name, params in re.findall(r"pub fn (ksh_\w+)\(([^;]*?)\)\s*(?:->[^;]*)?;", rust, flags=re.S):
+        params = params.strip()
+        declared[name] = 0 if not params else len(re.findall(r"\b\w+\s*:", params))
+    assert sorted(declared) == sorted(protos), sorted(set(protos) ^ set(declared))
+    for name, n in protos.items():
+        assert declared[name] == n, f"{name}: {declared[name]} parameters in the Rust listing, {n} in the header"
+    header = open(os.path.join(ROOT, "include", "ksearch_hip.h")).read()
+    for c_name in re.findall(r"\}\s*(ksh_\w+)\s*;", header):
+        rust_name = "".join(w.capitalize() for w in c_name.split("_"))
+        assert f"pub struct {rust_name} " in rust, f"{c_name} has no {rust_name} in the Rust listing"
+
+
 def test_enums_match_header():
     text = open(os.path.join(ROOT, "include", "ksearch_hip.h")).read()
     for m in re.finditer(r"\b(KSH_[A-Z0-9_]+)\s*=\s*(\d+)", text):

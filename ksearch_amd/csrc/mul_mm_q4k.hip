@@ -23,8 +23,8 @@
 // values lose at most 2^-25 absolutely).
 //
 // Tiling: a workgroup owns 128 tokens x 128 weight rows; each of its four
-// multiplying waves owns 64 x 64 as 2 x 2 v_mfma_f32_32x32x16_f16 tiles (four
-// more waves load and convert).  M = tokens, N = weight
+// multiplying waves owns 32 tokens x 128 rows as 1 x 4 v_mfma_f32_32x32x16_f16
+// tiles (four more waves load and convert).  M = tokens, N = weight
 // rows, so a lane's accumulator column is one weight row (one d per lane) and
 // stores are contiguous along Y's row index.  K advances 64 columns (one
 // 64-element group: 32 quant bytes per row) per step through a double-buffered
@@ -356,8 +356,8 @@ constexpr size_t kLdsBytes = 2 * (size_t)(kLdsMain + kLdsMin) * 2 + 2 * BN * 4;
 constexpr size_t kLdsBytes64 = 2 * (size_t)(kLdsMain + (64 + BN) * PITCH2) * 2 + 2 * BN * 4;   // the 64-token tile
 
 // Eight waves in two roles, one of each per SIMD.  Waves 0..3 only multiply:
-// each owns a 64 x 64 piece of the tile (2 x 2 MFMA tiles, one LDS operand
-// read per matrix instruction) and works on LDS stage s&1.  Waves 4..7 only
+// each owns 32 tokens x 128 columns of the 128-token tile (1 x 4 MFMA tiles; of
+// the 64-token tile 32 x 64) and works on LDS stage s&1.  Waves 4..7 only
 // load and convert: during the same step they request the activations of step
 // s+4 (and, when a superblock opens, the next superblock's weights) and write
 // step s+1 into stage (s+1)&1.  One barrier per K step joins them, so the
@@ -372,7 +372,7 @@ constexpr size_t kLdsBytes64 = 2 * (size_t)(kLdsMain + (64 + BN) * PITCH2) * 2 +
 // sc_j * q is exact in f16 up to 2048; beyond that (needs |sc_j| > 64) it rounds to the nearest even integer, a
 // relative 2^-11 at most and on those weights only (the reference's tile rounds every weight to half, the same
 // bound).  There is no min term, so the short second product is skipped; d is applied per superblock as for Q4_K.
-// TM = tokens per workgroup.  128: each multiplying wave owns 64 x 64.  64: each owns 32 x 64 with half the
+// TM = tokens per workgroup.  128: each multiplying wave owns 32 x 128.  64: each owns 32 x 64 with half the
 // accumulators, the kernel fits 128 registers and 70 KB of LDS, and two workgroups share a compute unit, so that one's
 // barriers and first loads fall into the other's products (the weights are converted once per 64 tokens then).
 // LO = true: f32 activations as two f16 parts at the row's own scale.  Every converted weight meets the hi and the lo
@@ -589,12 +589,18 @@ __global__ __launch_bounds__(kThreadsMM, TM == 64 ? 2 : 1) void q_mul_mm_kernel(
     }
 
     // ---------------------------------------------------------------------- multipliers
-    const int wm = wave >> 1, wn = wave & 1;
-    f16v F[MT][2], Cp[MT][2];
+    // WIDE (the 128-token tiles): a multiplying wave owns 32 tokens x all 128 columns instead of 64 x 64 -- one A fragment
+    // per k slice serves four products, so the activations cross the vector-memory path once per workgroup instead of
+    // twice (that path was busy for two thirds of the kernel), and all four waves read every B operand from LDS (twice
+    // the LDS reads, which the operands requested a slice ahead hide): cfg2 31.5 -> 30.5 us per pair.
+    constexpr bool WIDE = TM == 128;
+    constexpr int MW = WIDE ? 1 : MT, NW_ = WIDE ? 4 : 2, NSPAN = WIDE ? 0 : 64;
+    const int wm = WIDE ? wave : wave >> 1, wn = WIDE ? 0 : wave & 1;
+    f16v F[MW][NW_], Cp[MW][NW_];
 #pragma unroll
-    for (int a = 0; a < MT; a++)
+    for (int a = 0; a < MW; a++)
 #pragma unroll
-        for (int b = 0; b < 2; b++)
+        for (int b = 0; b < NW_; b++)
 #pragma unroll
             for (int i = 0; i < 16; i++) { F[a][b][i] = 0.f; Cp[a][b][i] = 0.f; }
     const int lm = lane & 31, lk = (lane >> 5) * 8;
@@ -603,10 +609,10 @@ __global__ __launch_bounds__(kThreadsMM, TM == 64 ? 2 : 1) void q_mul_mm_kernel(
     // Two register sets, each refilled for two steps ahead as soon as its own step's instructions are issued (LO: one
     // set of hi and lo fragments, refilled for the next step -- a step is long against the way to the cache).
     const int ntt = (p.batch + 31) / 32;
-    const h8 *xa[MT];
+    const h8 *xa[MW];
 #pragma unroll
-    for (int mt = 0; mt < MT; mt++)
-        xa[mt] = reinterpret_cast<const h8 *>(p.Xf) + ((size_t)min((t0 + (wm * MT + mt) * 32) / 32, ntt - 1) * (p.cols / 16) + (size_t)sb0 * 16) * 64 + lane;
+    for (int mt = 0; mt < MW; mt++)
+        xa[mt] = reinterpret_cast<const h8 *>(p.Xf) + ((size_t)min((t0 + (wm * MW + mt) * 32) / 32, ntt - 1) * (p.cols / 16) + (size_t)sb0 * 16) * 64 + lane;
     const ptrdiff_t lo_delta = LO ? reinterpret_cast<const h8 *>(p.Xf_lo) - reinterpret_cast<const h8 *>(p.Xf) : 0;
     auto afrag = [&](int mt, int step, int ks) __attribute__((always_inline)) {
         return xa[mt][(ptrdiff_t)(step * (KS / 16) + ks) * 64];
@@ -615,10 +621,10 @@ __global__ __launch_bounds__(kThreadsMM, TM == 64 ? 2 : 1) void q_mul_mm_kernel(
         return xa[mt][(ptrdiff_t)(step * (KS / 16) + ks) * 64 + lo_delta];
     };
     constexpr int AHEAD = LO ? 1 : 2;
-    struct ARegs { h8 a[MT][KS / 16], al[LO ? MT : 1][KS / 16]; };
+    struct ARegs { h8 a[MW][KS / 16], al[LO ? MW : 1][KS / 16]; };
     auto fetch_a = [&](int step, ARegs &r) __attribute__((always_inline)) {
 #pragma unroll
-        for (int mt = 0; mt < MT; mt++)
+        for (int mt = 0; mt < MW; mt++)
 #pragma unroll
             for (int ks = 0; ks < KS / 16; ks++) {
                 r.a[mt][ks] = afrag(mt, step, ks);
@@ -639,45 +645,45 @@ __global__ __launch_bounds__(kThreadsMM, TM == 64 ? 2 : 1) void q_mul_mm_kernel(
         // f32 activations a slice has eight products to hide it behind: prompts of 1024 / 4000 tokens 14.1 / 67.6 ->
         // 14.0 / 67.1 ms).  The 64-token tile loses by it (a 256-token prompt 5.1 -> 5.3 ms) and keeps the plain order.
         constexpr bool BPIPE = TM == 128;
-        h8 bb[2][2];
+        h8 bb[2][NW_];
         if (BPIPE) {
 #pragma unroll
-            for (int nt = 0; nt < 2; nt++)
-                bb[0][nt] = *reinterpret_cast<const h8 *>(&Bs[(wn * 64 + nt * 32 + lm) * PITCH + lk]);
+            for (int nt = 0; nt < NW_; nt++)
+                bb[0][nt] = *reinterpret_cast<const h8 *>(&Bs[(wn * NSPAN + nt * 32 + lm) * PITCH + lk]);
         }
 #pragma unroll
         for (int ks = 0; ks < KS / 16; ks++) {
-            h8 b[2];
+            h8 b[NW_];
             if (BPIPE) {
                 if (ks + 1 < KS / 16) {
 #pragma unroll
-                    for (int nt = 0; nt < 2; nt++)
-                        bb[(ks + 1) & 1][nt] = *reinterpret_cast<const h8 *>(&Bs[(wn * 64 + nt * 32 + lm) * PITCH + 16 * (ks + 1) + lk]);
+                    for (int nt = 0; nt < NW_; nt++)
+                        bb[(ks + 1) & 1][nt] = *reinterpret_cast<const h8 *>(&Bs[(wn * NSPAN + nt * 32 + lm) * PITCH + 16 * (ks + 1) + lk]);
                 }
                 __builtin_amdgcn_sched_barrier(0);   // (the requests stay in front of this slice's products)
-                b[0] = bb[ks & 1][0];
-                b[1] = bb[ks & 1][1];
+#pragma unroll
+                for (int nt = 0; nt < NW_; nt++) b[nt] = bb[ks & 1][nt];
             } else {
 #pragma unroll
-                for (int nt = 0; nt < 2; nt++)
-                    b[nt] = *reinterpret_cast<const h8 *>(&Bs[(wn * 64 + nt * 32 + lm) * PITCH + 16 * ks + lk]);
+                for (int nt = 0; nt < NW_; nt++)
+                    b[nt] = *reinterpret_cast<const h8 *>(&Bs[(wn * NSPAN + nt * 32 + lm) * PITCH + 16 * ks + lk]);
             }
 #pragma unroll
-            for (int mt = 0; mt < MT; mt++)
+            for (int mt = 0; mt < MW; mt++)
 #pragma unroll
-                for (int nt = 0; nt < 2; nt++)
+                for (int nt = 0; nt < NW_; nt++)
                     // a superblock's first product starts from the constant zero: no pass over the accumulators to clear them
                     Cp[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A.a[mt][ks], b[nt], (g == 0 && ks == 0) ? kZero16 : Cp[mt][nt], 0, 0, 0);
             if (LO) {
 #pragma unroll
-                for (int mt = 0; mt < MT; mt++)
+                for (int mt = 0; mt < MW; mt++)
 #pragma unroll
-                    for (int nt = 0; nt < 2; nt++)
+                    for (int nt = 0; nt < NW_; nt++)
                         Cp[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A.al[mt][ks], b[nt], Cp[mt][nt], 0, 0, 0);
             }
             // this k slice's fragments are spent: ask for the ones of AHEAD steps on right away
 #pragma unroll
-            for (int mt = 0; mt < MT; mt++) {
+            for (int mt = 0; mt < MW; mt++) {
                 A.a[mt][ks] = afrag(mt, min(step + AHEAD, nsteps - 1), ks);
                 if (LO) A.al[mt][ks] = afrag_lo(mt, min(step + AHEAD, nsteps - 1), ks);
             }
@@ -689,24 +695,24 @@ __global__ __launch_bounds__(kThreadsMM, TM == 64 ? 2 : 1) void q_mul_mm_kernel(
             const float *dsc = dsc_stage(sb);
 #pragma unroll
             for (int ks = 0; ks < (Q6 ? 0 : 2); ks++) {
-                h8 a[MT], b[2];
+                h8 a[MW], b[NW_];
 #pragma unroll
-                for (int mt = 0; mt < MT; mt++)
-                    a[mt] = *reinterpret_cast<const h8 *>(&A2s[((wm * MT + mt) * 32 + lm) * PITCH2 + 16 * ks + lk]);
+                for (int mt = 0; mt < MW; mt++)
+                    a[mt] = *reinterpret_cast<const h8 *>(&A2s[((wm * MW + mt) * 32 + lm) * PITCH2 + 16 * ks + lk]);
 #pragma unroll
-                for (int nt = 0; nt < 2; nt++)
-                    b[nt] = *reinterpret_cast<const h8 *>(&B2s[(wn * 64 + nt * 32 + lm) * PITCH2 + 16 * ks + lk]);
+                for (int nt = 0; nt < NW_; nt++)
+                    b[nt] = *reinterpret_cast<const h8 *>(&B2s[(wn * NSPAN + nt * 32 + lm) * PITCH2 + 16 * ks + lk]);
 #pragma unroll
-                for (int mt = 0; mt < MT; mt++)
+                for (int mt = 0; mt < MW; mt++)
 #pragma unroll
-                    for (int nt = 0; nt < 2; nt++)
+                    for (int nt = 0; nt < NW_; nt++)
                         F[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mt], b[nt], F[mt][nt], 0, 0, 0);
             }
 #pragma unroll
-            for (int nt = 0; nt < 2; nt++) {
-                const float dn = dsc[wn * 64 + nt * 32 + lm];
+            for (int nt = 0; nt < NW_; nt++) {
+                const float dn = dsc[wn * NSPAN + nt * 32 + lm];
 #pragma unroll
-                for (int mt = 0; mt < MT; mt++)
+                for (int mt = 0; mt < MW; mt++)
 #pragma unroll
                     for (int i = 0; i < 16; i++)
                         F[mt][nt][i] = fmaf(dn, Cp[mt][nt][i], F[mt][nt][i]);
@@ -723,13 +729,13 @@ __global__ __launch_bounds__(kThreadsMM, TM == 64 ? 2 : 1) void q_mul_mm_kernel(
 
     // accumulator layout of the 32x32 tile: column = lane % 32, row = 8*(i/4) + 4*(lane/32) + i%4
 #pragma unroll
-    for (int mt = 0; mt < MT; mt++)
+    for (int mt = 0; mt < MW; mt++)
 #pragma unroll
-        for (int nt = 0; nt < 2; nt++) {
-            const int r = r0 + wn * 64 + nt * 32 + lm;
+        for (int nt = 0; nt < NW_; nt++) {
+            const int r = r0 + wn * NSPAN + nt * 32 + lm;
 #pragma unroll
             for (int i = 0; i < 16; i++) {
-                const int t = t0 + (wm * MT + mt) * 32 + 8 * (i / 4) + 4 * (lane >> 5) + (i & 3);
+                const int t = t0 + (wm * MW + mt) * 32 + 8 * (i / 4) + 4 * (lane >> 5) + (i & 3);
                 if (t < p.batch && r < p.rows) p.Y[(size_t)t * ystride + r] = LO ? F[mt][nt][i] * p.inv_s[t] : F[mt][nt][i];
             }
         }

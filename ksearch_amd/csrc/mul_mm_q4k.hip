@@ -1600,13 +1600,15 @@ int bind_matvec_batch(ksh_kernel &k)
     // about one workgroup per compute unit; every slice stores its partial sums and a second launch adds them in a
     // fixed order.  sched.k_split names the slice count (a divisor of cols / 256; 1 = none).
     const int64_t row_tiles = (rows + BN - 1) / BN + (rows1 + BN - 1) / BN + (rows2 + BN - 1) / BN;
-    const int64_t tiles = ((batch + BM - 1) / BM) * row_tiles, nsb = cols / 256;
+    const int64_t nsb = cols / 256;
     int64_t ks = 1;
     if (k.desc.sched.k_split) {
         ks = k.desc.sched.k_split;
         if (nsb % ks) return set_error("matvec_batch: k_split=%lld does not divide the %lld superblocks of a row", (long long)ks, (long long)nsb);
     } else {
-        while (tiles * ks < 256 && nsb % (ks * 2) == 0 && nsb / (ks * 2) >= 2) ks *= 2;   // (a slice of one superblock is all prologue)
+        // (a slice of one superblock is all prologue; the workgroups are counted with the token tile they will have)
+        auto workgroups = [&](int64_t s) { const int64_t tm_s = mm_tile_tokens(k.desc, s); return ((batch + tm_s - 1) / tm_s) * row_tiles * s; };
+        while (nsb % (ks * 2) == 0 && nsb / (ks * 2) >= 2 && workgroups(ks * 2) <= 256) ks *= 2;
     }
     const bool z_form = unfolded || ks > 1;
     k.variant = z_form ? (int)(ks << 1) : 0;

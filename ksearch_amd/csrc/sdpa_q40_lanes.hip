@@ -920,12 +920,18 @@ __device__ __forceinline__ int mfma_k_elem(int s, int kq)
 // whose accumulators are what limits the head size a wave can hold.
 // BAL: the launch whose partitions are dealt to the slots by length (p.balance), known when the kernel is built: either
 // form's front then holds its own way to its rows only.
-template <int HD, int TR, int HDV = HD, bool BAL = false>
+// PVX (eight waves with tiles of 16 rows, heads of 256): the waves share P.V by V block instead of by rows.  Every wave
+// still takes the scores of its own 16 rows, the round's maximum and the probabilities meet in LDS (two barriers), and
+// wave w then multiplies all 128 rows of the round into the 32 dimensions of block w -- its accumulators are final for
+// the workgroup, so the eight-way fold of whole states through LDS and the pass that merges them fall away (they took
+// a quarter of the launch) and every wave stores its own slice of the record.
+template <int HD, int TR, int HDV = HD, bool BAL = false, bool PVX = false>
 __global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_mfma_kernel(LaneParams p_in)
 {
     LaneParams p = p_in;
     p.balance = BAL;
     static_assert(TR == 16 || TR == 32, "tile rows");
+    static_assert(!PVX || (TR == 16 && HDV == HD && HD / 32 == kMfmaRound / TR), "a V block per wave");
     static_assert(HD % HDV == 0 && (HDV == HD || TR == 32), "V halves come with tiles of 32 rows");
     touch_lane_params(p_in);   // every kernel argument in one round trip
     constexpr int NW = kMfmaRound / TR, NT = NW * 64, NB = HD / 32, ROWB = NB * 18, TILEB = TR * ROWB;
@@ -1056,13 +1062,17 @@ __global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_m
         if (HDV != HD) __syncthreads();      // every wave has its copy before a strip is written
     }
 
-    f4v O[2 * NBV];
-    float Tl[NBV];
+    constexpr int NACC = PVX ? 1 : NBV;                     // V blocks a wave accumulates
+    f4v O[2 * NACC];
+    float Tl[NACC];
 #pragma unroll
-    for (int c = 0; c < 2 * NBV; c++) O[c] = f4v{0.f, 0.f, 0.f, 0.f};
+    for (int c = 0; c < 2 * NACC; c++) O[c] = f4v{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int b = 0; b < NBV; b++) Tl[b] = 0.f;
+    for (int b = 0; b < NACC; b++) Tl[b] = 0.f;
     float m_run = -1.0e30f, l_run = 0.f;
+    // PVX: what the waves exchange per round, behind the shared q operands
+    float *Psh = reinterpret_cast<float *>(lds_raw + (size_t)NW * STRIP + (size_t)NB * 64 * (16 + 4));   // [8 heads][128 rows]
+    float *mxs = Psh + 8 * kMfmaRound, *lws = mxs + NW * 8;                                               // [wave][head] each
 
     const int ntiles = (p1 - p0 + TR - 1) / TR;
     const int nsteps = (ntiles + NW - 1) / NW;               // the same for every wave: the barriers below are uniform
@@ -1111,6 +1121,98 @@ __global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_m
             }
         }
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        if constexpr (PVX) {
+            // ---- scores of the wave's 16 rows (as below): lane (col, q4) ends up with rows 4*q4 + r
+            float sv[4] = {-1.0e30f, -1.0e30f, -1.0e30f, -1.0e30f};
+            if (nvalid > 0) {
+                float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int b = 0; b < NB; b++) {
+                    const float4 dk4 = *reinterpret_cast<const float4 *>(ksc + b * TR + 4 * q4);
+                    const float dk[4] = {dk4.x, dk4.y, dk4.z, dk4.w};
+                    const uint8_t *src = kraw + col * ROWB + 18 * b + 2 + 4 * q4;
+                    const uint32_t d = (uint32_t)*reinterpret_cast<const uint16_t *>(src) |
+                                       ((uint32_t)*reinterpret_cast<const uint16_t *>(src + 2) << 16);
+                    const f4v c = __builtin_amdgcn_mfma_f32_16x16x32_f16(nibbles_f16(d, nib_mask, nib_one), qop[b], f4v{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+#pragma unroll
+                    for (int r = 0; r < 4; r++) acc[r] = fmaf(dk[r], c[r] - qs24[b], acc[r]);
+                }
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const float tot = acc[r] + dpp_f32<0x128>(acc[r]);        // hi + lo column (row_ror:8)
+                    sv[r] = (4 * q4 + r) < nvalid ? tot : -1.0e30f;
+                }
+            }
+            // ---- probabilities against the wave's own maximum; maxima, sums and probabilities meet in LDS behind one
+            // barrier (which also makes every wave's V bytes and scale tables visible to the others), and a tile's factor
+            // exp(m_tile - m) rides on its V scales in the product below
+            float mt = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
+            mt = xor32_max(xor16_max(mt));
+            float pr[4], ls = 0.f;
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                pr[r] = (4 * q4 + r) < nvalid ? __expf(sv[r] - mt) : 0.f;
+                ls += pr[r];
+            }
+            ls = xor32_sum(xor16_sum(ls));                     // the wave's 16 rows of this column's head
+            if (!is_lo) *reinterpret_cast<float4 *>(Psh + head * kMfmaRound + TR * wave + 4 * q4) = make_float4(pr[0], pr[1], pr[2], pr[3]);
+            if (lane < 8) { mxs[wave * 8 + lane] = mt; lws[wave * 8 + lane] = ls; }
+            __syncthreads();
+            float mw[NW], mr = -1.0e30f;
+#pragma unroll
+            for (int w = 0; w < NW; w++) { mw[w] = mxs[w * 8 + head]; mr = fmaxf(mr, mw[w]); }
+            const float m_new = fmaxf(m_run, mr);
+            const float alpha = __expf(m_run - m_new);
+            float fw[NW], lr = 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; w++) {
+                fw[w] = __expf(mw[w] - m_new);
+                lr = fmaf(fw[w], lws[w * 8 + head], lr);
+            }
+            l_run = fmaf(l_run, alpha, lr);
+            m_run = m_new;
+            if (it > 0) {
+                // (the first round's factor multiplies zeros)
+                float ah[8], ar[4];
+#pragma unroll
+                for (int h = 0; h < 8; h++) ah[h] = as_f32((uint32_t)__builtin_amdgcn_readlane((int)as_u32(alpha), h));
+#pragma unroll
+                for (int r = 0; r < 4; r++) ar[r] = as_f32((as_u32(ah[r]) & ~odd_mask) | (as_u32(ah[4 + r]) & odd_mask));
+#pragma unroll
+                for (int c = 0; c < 2; c++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) O[c][r] *= ar[r];
+                Tl[0] *= alpha;
+            }
+            // ---- P.V of block `wave` over the round's eight tiles: tile j lies in wave j's strip
+            float tsum = 0.f;
+#pragma unroll
+            for (int j = 0; j < NW; j++) {
+                const uint8_t *vj = lds_raw + (size_t)j * STRIP + TILEB;
+                const float *vscj = reinterpret_cast<const float *>(lds_raw + (size_t)j * STRIP + TILEB + TILEBV) + TR * NB;
+                const float4 p4 = *reinterpret_cast<const float4 *>(Psh + head * kMfmaRound + TR * j + 4 * q4);
+                const float4 d4 = *reinterpret_cast<const float4 *>(vscj + wave * TR + 4 * q4);
+                const float x[4] = {p4.x * (d4.x * fw[j]), p4.y * (d4.y * fw[j]), p4.z * (d4.z * fw[j]), p4.w * (d4.w * fw[j])};
+                uint32_t pa[2], vlo[2], vhi[2];
+#pragma unroll
+                for (int i = 0; i < 2; i++) {
+                    const float y0 = as_f32(as_u32(x[2 * i]) & keep) - as_f32(as_u32(x[2 * i]) & drop);
+                    const float y1 = as_f32(as_u32(x[2 * i + 1]) & keep) - as_f32(as_u32(x[2 * i + 1]) & drop);
+                    pa[i] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(y0, y1));
+                    tsum += x[2 * i] + x[2 * i + 1];
+                    const int ra = 4 * q4 + 2 * i;
+                    const uint32_t t2 = (uint32_t)vj[ra * ROWBV + 18 * wave + 2 + col] | ((uint32_t)vj[(ra + 1) * ROWBV + 18 * wave + 2 + col] << 16);
+                    vlo[i] = ((t2 << 6) & nib_mask) | nib_one;
+                    vhi[i] = ((t2 << 2) & nib_mask) | nib_one;
+                }
+                const h4v pa4 = __builtin_bit_cast(h4v, u32x2_t{pa[0], pa[1]});
+                const u32x2_t lo2 = {vlo[0], vlo[1]}, hi2 = {vhi[0], vhi[1]};
+                O[0] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa4, __builtin_bit_cast(h4v, lo2), O[0], 0, 0, 0);
+                O[1] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa4, __builtin_bit_cast(h4v, hi2), O[1], 0, 0, 0);
+            }
+            Tl[0] += tsum;
+            if (it + 1 < nsteps) __syncthreads();      // the strips and the exchange are written again
+        } else
         if (nvalid > 0) {
             // ---- scores of the tile's two 16-row halves: lane (col, q4) ends up with rows 4*q4 + r of each
             constexpr int NS = TR / 4;                       // scores (rows) per lane
@@ -1217,6 +1319,42 @@ __global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_m
         }
     }
 
+    if constexpr (PVX) {
+        // ---- every wave stores the 32 dimensions of its block for all heads; wave 0 adds (m, l)
+        const uint32_t tcol = as_u32(24.f * xor32_sum(xor16_sum(Tl[0])));
+        const int odd = q4 >> 1, d = 32 * wave + col + 16 * odd;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const uint32_t t_lo = (uint32_t)__builtin_amdgcn_readlane((int)tcol, r), t_hi = (uint32_t)__builtin_amdgcn_readlane((int)tcol, 4 + r);
+            const float t24 = as_f32((t_lo & ~odd_mask) | (t_hi & odd_mask));
+            const uint32_t l_lo = (uint32_t)__builtin_amdgcn_readlane((int)as_u32(l_run), r), l_hi = (uint32_t)__builtin_amdgcn_readlane((int)as_u32(l_run), 4 + r);
+            const float L = as_f32((l_lo & ~odd_mask) | (l_hi & odd_mask));
+            const auto sw = __builtin_amdgcn_permlane32_swap(as_u32(O[0][r]), as_u32(O[1][r]), false, false);
+            const float a = (as_f32(sw[0]) - t24) + as_f32(sw[1]);
+            const int h = 4 * (q4 & 1) + r, hq = head0 + h;
+            if (h >= groups) continue;
+            if (p.balance) {
+                p.tmp[(rec_base * p.n_q + hq) * HD + d] = a;
+            } else if (p.nwg == 1 && p.out) {
+                p.out[((size_t)slot * p.n_q + hq) * HD + d] = a / L;
+            } else {
+                p.tmp[(size_t)slot * p.n_q * p.nwg * (HD + 2) + (size_t)hq * p.nwg * (HD + 2) + (size_t)part * (HD + 2) + 2 + d] = a;
+            }
+        }
+        if (wave == 0 && lane < 8 && lane < groups) {
+            const int hq = head0 + lane;
+            if (p.balance) {
+                float *ml = p.tmp + (size_t)gridDim.z * p.nwg * p.n_q * HD;
+                ml[2 * (rec_base * p.n_q + hq)] = m_run;
+                ml[2 * (rec_base * p.n_q + hq) + 1] = l_run;
+            } else if (!(p.nwg == 1 && p.out)) {
+                float *rec = p.tmp + (size_t)slot * p.n_q * p.nwg * (HD + 2) + (size_t)hq * p.nwg * (HD + 2) + (size_t)part * (HD + 2);
+                rec[0] = m_run;
+                rec[1] = l_run;
+            }
+        }
+        return;
+    }
     // ---- fold: every wave's state to LDS (hi rows first, lo rows added), then one record per head
     __syncthreads();
     float *ow = reinterpret_cast<float *>(lds_raw);            // [NW][8][HDV]
@@ -1301,7 +1439,7 @@ __global__ __launch_bounds__(HD) void sdpa_records_merge_kernel(const float *__r
     out[((size_t)tok * n_q + h) * HD + d] = a / L;
 }
 
-template <int HD, int TR, int HDV = HD>
+template <int HD, int TR, int HDV = HD, bool PVX = false>
 constexpr size_t mfma_lds_bytes()
 {
     constexpr size_t waves = kMfmaRound / TR;
@@ -1310,6 +1448,7 @@ constexpr size_t mfma_lds_bytes()
     constexpr size_t fold = waves * 8 * HDV * 4 + waves * 8 * 2 * 4;
     constexpr size_t qsum = (size_t)(HD / 32) * 64 * 4;
     constexpr size_t front = HDV == HD ? strip * waves + qshare : strip * waves + qsum;   // (HDV < HD: the operands lie over the strips, the sums behind them)
+    if (PVX) return front + (8 * kMfmaRound + 2 * waves * 8) * 4;                         // + the probabilities, maxima and sums the waves exchange; no fold
     return front > fold ? front : fold;
 }
 
@@ -1384,7 +1523,7 @@ int launch_bound(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
             if (nw == 0xFF)
                 hipLaunchKernelGGL((sdpa_mfma_kernel<256, 32, 256, true>), dim3(p.nwg, p.n_kv, n_slots), dim3(kMfmaRound / 32 * 64), (mfma_lds_bytes<256, 32>()), st, p);
             else
-                hipLaunchKernelGGL((sdpa_mfma_kernel<256, 16, 256, true>), dim3(p.nwg, p.n_kv, n_slots), dim3(kMfmaRound / 16 * 64), (mfma_lds_bytes<256, 16>()), st, p);
+                hipLaunchKernelGGL((sdpa_mfma_kernel<256, 16, 256, true, true>), dim3(p.nwg, p.n_kv, n_slots), dim3(kMfmaRound / 16 * 64), (mfma_lds_bytes<256, 16, 256, true>()), st, p);
             const hipError_t e0 = hipGetLastError();
             if (e0 != hipSuccess) return hip_fail(e0, "sdpa (matrix-core form) launch");
         } else if (launch_lanes(p, hd, nw, n_slots, st)) {
@@ -1560,7 +1699,7 @@ int bind_sdpa_lanes(ksh_kernel &k, int nwg, int n_slots)
         // (the batch kind keeps its per-token records in the scratch, behind room for the register form's counters)
         k.scratch_bytes = batch_fits ? (((size_t)n_slots * n_kv * 4 + 15) & ~(size_t)15) + (size_t)n_slots * 16 : 16;
         set_launch(k, (uint32_t)nwg, (uint32_t)n_kv, (uint32_t)n_slots, waves * 64,
-                   (uint32_t)(tile == 32 ? mfma_lds_bytes<256, 32>() : mfma_lds_bytes<256, 16>()));
+                   (uint32_t)(tile == 32 ? mfma_lds_bytes<256, 32>() : mfma_lds_bytes<256, 16, 256, true>()));
         k.info.sched = k.desc.sched;
         k.info.sched.vec = 2;
         k.info.sched.tg = waves * 64;

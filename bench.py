@@ -428,6 +428,37 @@ def bench_timeline(ctx, eng, tokens=24):
         for i, ph in enumerate(phases, 1):
             rec[ph] = [med(f"p50_{i}"), med(f"max_{i}")]
         res[name] = rec
+
+    # cfg3's row kernel (the matrix-core form whose waves share P.V by V block), hot: the same statistics over twelve launches
+    n_slots, n_q, n_kv, hd, max_t = 4, 8, 1, 256, 16384
+    lens, kk, vv, q = synth.cfg3_q40_attention()
+    meta = np.zeros((n_slots, 4), dtype=np.float32)
+    meta[:, 0] = lens
+    k = ctx.compile(hip.make_desc(hip.Kind.SDPA_SLOTS, (n_q, n_kv, hd, max_t, n_slots, 0), (hip.DType.Q40, hip.DType.F32), (1.0 / 16.0,)))
+    nwg = k.info.sched.k_split
+    ins = [ctx.buffer_f32(q), ctx.buffer_bytes(kk), ctx.buffer_bytes(vv), ctx.buffer_f32(meta)]
+    outs = [ctx.buffer_empty_f32(n_slots * n_q * nwg * (hd + 2)), ctx.buffer_empty_f32(n_slots * n_q * hd)]
+    ctx.run(k, ins, outs, iters=3)
+    read("ksh_stamps_sdpa_lanes")
+    phases = ["the deal is known", "q operands shared", "tile and scale tables in LDS", "probabilities written", "products done", "stores acknowledged"]
+    rows = []
+    for _ in range(12):
+        ctx.run(k, ins, outs, iters=1)
+        a = read("ksh_stamps_sdpa_lanes")[2]
+        a = a[a[:, 6] > 0]
+        if not len(a):
+            raise SystemExit("bench.py: the timeline build left no records for cfg3's row kernel")
+        t0 = a[:, 0].min()
+        row = dict(waves=len(a), entry_p50=(np.median(a[:, 0]) - t0) * 0.01, entry_max=(a[:, 0].max() - t0) * 0.01)
+        for i in range(1, 7):
+            row[f"p50_{i}"], row[f"max_{i}"] = (np.median(a[:, i]) - t0) * 0.01, (a[:, i].max() - t0) * 0.01
+        rows.append(row)
+    rec = {"waves": rows[0]["waves"], "kernel": k.name, "gap_before_us": None,
+           "entry_p50": round(float(np.median([r["entry_p50"] for r in rows])), 2), "entry_last": round(float(np.median([r["entry_max"] for r in rows])), 2),
+           "first_wave_to_last_ack_us": round(float(np.median([r["max_6"] for r in rows])), 2)}
+    for i, ph in enumerate(phases, 1):
+        rec[ph] = [round(float(np.median([r[f"p50_{i}"] for r in rows])), 2), round(float(np.median([r[f"max_{i}"] for r in rows])), 2)]
+    res["cfg3 attention, row kernel (waves with rows)"] = rec
     return res
 
 

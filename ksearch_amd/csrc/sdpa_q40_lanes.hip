@@ -42,7 +42,9 @@ KSH_STAMP_READER(ksh_stamps_sdpa_lanes)
 namespace ksh {
 namespace {
 
-// timeline build, register-form kernel: tag 0 plain attention, 1 the fused decode step
+// timeline build, register-form kernel: tag 0 plain attention, 1 the fused decode step; tag 2 the matrix-core row phase in
+// its V-block form (slots: 1 the deal is known, 2 q operands shared, 3 tile and scale tables in LDS, 4 probabilities
+// written, 5 products done, 6 stores acknowledged)
 // slots: 0 entry, 1 every load of the front issued, 2 length and position in, 3 q (and the new row) ready,
 //        4 rows done, 5 row groups folded, 6 records stored (acknowledged)
 #define KSH_LANES_WAVE ((((int)blockIdx.z * (int)gridDim.y + (int)blockIdx.y) * (int)gridDim.x + (int)blockIdx.x) * NW + wave)
@@ -934,6 +936,7 @@ __global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_m
     static_assert(!PVX || (TR == 16 && HDV == HD && HD / 32 == kMfmaRound / TR), "a V block per wave");
     static_assert(HD % HDV == 0 && (HDV == HD || TR == 32), "V halves come with tiles of 32 rows");
     touch_lane_params(p_in);   // every kernel argument in one round trip
+    KSH_STAMP_BEGIN
     constexpr int NW = kMfmaRound / TR, NT = NW * 64, NB = HD / 32, ROWB = NB * 18, TILEB = TR * ROWB;
     constexpr int NBV = HDV / 32, ROWBV = NBV * 18, TILEBV = TR * ROWBV;   // this workgroup's share of a V row
     constexpr int STRIP = TILEB + TILEBV + TR * NB * 4 + TR * NBV * 4;     // K bytes, V bytes, K scales, V scales
@@ -962,6 +965,7 @@ __global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_m
         p0 = part * d.c;
         p1 = min(p0 + d.c, d.tlen);
         start = d.start;
+        if (PVX) { KSH_STAMP_USE(start); KSH_STAMP(1); }
     } else {
         int tlen;
         if (p.kv_shared) {
@@ -1060,6 +1064,7 @@ __global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_m
             if (HDV == HD) qs24[b] = qsum_share[b * 64 + lane];     // (heads of 512 read theirs from LDS block by block: sixteen registers less)
         }
         if (HDV != HD) __syncthreads();      // every wave has its copy before a strip is written
+        if (PVX) { KSH_STAMP_USE(qs24[NB - 1]); KSH_STAMP(2); }
     }
 
     constexpr int NACC = PVX ? 1 : NBV;                     // V blocks a wave accumulates
@@ -1122,6 +1127,7 @@ __global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_m
         }
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         if constexpr (PVX) {
+            if (it == 0) KSH_STAMP(3);
             // ---- scores of the wave's 16 rows (as below): lane (col, q4) ends up with rows 4*q4 + r
             float sv[4] = {-1.0e30f, -1.0e30f, -1.0e30f, -1.0e30f};
             if (nvalid > 0) {
@@ -1157,6 +1163,7 @@ __global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_m
             ls = xor32_sum(xor16_sum(ls));                     // the wave's 16 rows of this column's head
             if (!is_lo) *reinterpret_cast<float4 *>(Psh + head * kMfmaRound + TR * wave + 4 * q4) = make_float4(pr[0], pr[1], pr[2], pr[3]);
             if (lane < 8) { mxs[wave * 8 + lane] = mt; lws[wave * 8 + lane] = ls; }
+            if (it == 0) KSH_STAMP(4);
             __syncthreads();
             float mw[NW], mr = -1.0e30f;
 #pragma unroll
@@ -1211,6 +1218,7 @@ __global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_m
                 O[1] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa4, __builtin_bit_cast(h4v, hi2), O[1], 0, 0, 0);
             }
             Tl[0] += tsum;
+            if (it + 1 == nsteps) { KSH_STAMP_USE(O[1][3]); KSH_STAMP(5); }
             if (it + 1 < nsteps) __syncthreads();      // the strips and the exchange are written again
         } else
         if (nvalid > 0) {
@@ -1353,6 +1361,7 @@ __global__ __launch_bounds__(kMfmaRound / TR * 64, TR == 32 ? 2 : 1) void sdpa_m
                 rec[1] = l_run;
             }
         }
+        KSH_STAMP_FLUSH(2, ((int)blockIdx.z * (int)gridDim.x + (int)blockIdx.x) * NW + wave, 6);
         return;
     }
     // ---- fold: every wave's state to LDS (hi rows first, lo rows added), then one record per head

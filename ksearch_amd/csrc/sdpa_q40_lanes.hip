@@ -1531,8 +1531,12 @@ int launch_bound(const ksh_kernel &k, const LaunchArgs &a, hipStream_t st)
         if (mfma) {
             if (nw == 0xFF)
                 hipLaunchKernelGGL((sdpa_mfma_kernel<256, 32, 256, true>), dim3(p.nwg, p.n_kv, n_slots), dim3(kMfmaRound / 32 * 64), (mfma_lds_bytes<256, 32>()), st, p);
-            else
+            else if ((size_t)p.max_t <= (size_t)3 * kMfmaRound * (p.nwg - 1))
+                // partitions of at most three rounds even when every slot is full: the waves share P.V by V block (two
+                // barriers a round, no fold: a round costs ~0.7 us more than in the barrier-free loop, the fold ~2.2 us once)
                 hipLaunchKernelGGL((sdpa_mfma_kernel<256, 16, 256, true, true>), dim3(p.nwg, p.n_kv, n_slots), dim3(kMfmaRound / 16 * 64), (mfma_lds_bytes<256, 16, 256, true>()), st, p);
+            else
+                hipLaunchKernelGGL((sdpa_mfma_kernel<256, 16, 256, true>), dim3(p.nwg, p.n_kv, n_slots), dim3(kMfmaRound / 16 * 64), (mfma_lds_bytes<256, 16>()), st, p);
             const hipError_t e0 = hipGetLastError();
             if (e0 != hipSuccess) return hip_fail(e0, "sdpa (matrix-core form) launch");
         } else if (launch_lanes(p, hd, nw, n_slots, st)) {
@@ -1708,7 +1712,7 @@ int bind_sdpa_lanes(ksh_kernel &k, int nwg, int n_slots)
         // (the batch kind keeps its per-token records in the scratch, behind room for the register form's counters)
         k.scratch_bytes = batch_fits ? (((size_t)n_slots * n_kv * 4 + 15) & ~(size_t)15) + (size_t)n_slots * 16 : 16;
         set_launch(k, (uint32_t)nwg, (uint32_t)n_kv, (uint32_t)n_slots, waves * 64,
-                   (uint32_t)(tile == 32 ? mfma_lds_bytes<256, 32>() : mfma_lds_bytes<256, 16, 256, true>()));
+                   (uint32_t)(tile == 32 ? mfma_lds_bytes<256, 32>() : mfma_lds_bytes<256, 16>()));
         k.info.sched = k.desc.sched;
         k.info.sched.vec = 2;
         k.info.sched.tg = waves * 64;

@@ -118,9 +118,11 @@ struct RowRegs {
     uint32_t kd, ks, vd, vs;
 };
 
+// (GP = 1: a workgroup with a single q head -- the decode step's unmerged form with the heads spread over the
+// workgroups -- where the instances for four heads would carry three heads of zeros through every row)
 template <int GP>
 struct State {
-    float m[GP / 4], l[GP / 4];
+    float m[(GP + 3) / 4], l[(GP + 3) / 4];
     float O[GP][8], S[GP];
 };
 
@@ -133,37 +135,51 @@ __device__ __forceinline__ int head_of(int c, int i)
 
 // per-lane partial dots of GP heads -> finished dots of GP/4 heads, in every lane of the row group
 template <int HD, int GP>
-__device__ __forceinline__ void reduce_heads(const float (&v)[GP], int c, float (&out)[GP / 4])
+__device__ __forceinline__ void reduce_heads(const float (&v)[GP], int c, float (&out)[(GP + 3) / 4])
 {
-    const bool b0 = c & 1, b1 = c & 2;
-    float a[GP / 2];
-#pragma unroll
-    for (int i = 0; i < GP / 2; i++) {
-        const float keep = b0 ? v[i + GP / 2] : v[i], send = b0 ? v[i] : v[i + GP / 2];
-        a[i] = keep + dpp_f32<0xB1>(send);   // quad_perm [1,0,3,2]
-    }
-#pragma unroll
-    for (int i = 0; i < GP / 4; i++) {
-        const float keep = b1 ? a[i + GP / 4] : a[i], send = b1 ? a[i] : a[i + GP / 4];
-        float x = keep + dpp_f32<0x4E>(send);   // quad_perm [2,3,0,1]
-        x += dpp_f32<0x124>(x);                 // row_ror:4
-        x += dpp_f32<0x128>(x);                 // row_ror:8
+    if constexpr (GP == 1) {
+        float x = v[0] + dpp_f32<0xB1>(v[0]);   // the quad's four dwords of the block ...
+        x += dpp_f32<0x4E>(x);
+        x += dpp_f32<0x124>(x);                 // ... and the row group's blocks
+        x += dpp_f32<0x128>(x);
         if (HD >= 256) x = xor16_sum(x);
         if (HD == 512) x = xor32_sum(x);
-        out[i] = x;
+        out[0] = x;
+    } else {
+        const bool b0 = c & 1, b1 = c & 2;
+        float a[GP / 2];
+#pragma unroll
+        for (int i = 0; i < GP / 2; i++) {
+            const float keep = b0 ? v[i + GP / 2] : v[i], send = b0 ? v[i] : v[i + GP / 2];
+            a[i] = keep + dpp_f32<0xB1>(send);   // quad_perm [1,0,3,2]
+        }
+#pragma unroll
+        for (int i = 0; i < GP / 4; i++) {
+            const float keep = b1 ? a[i + GP / 4] : a[i], send = b1 ? a[i] : a[i + GP / 4];
+            float x = keep + dpp_f32<0x4E>(send);   // quad_perm [2,3,0,1]
+            x += dpp_f32<0x124>(x);                 // row_ror:4
+            x += dpp_f32<0x128>(x);                 // row_ror:8
+            if (HD >= 256) x = xor16_sum(x);
+            if (HD == 512) x = xor32_sum(x);
+            out[i] = x;
+        }
     }
 }
 
 // one lane's GP/4 values -> all GP, through the quad
 template <int GP>
-__device__ __forceinline__ void quad_gather(const float (&x)[GP / 4], float (&all)[GP])
+__device__ __forceinline__ void quad_gather(const float (&x)[(GP + 3) / 4], float (&all)[GP])
 {
+    if constexpr (GP == 1) {
+        all[0] = x[0];
+    } else {
 #pragma unroll
-    for (int i = 0; i < GP / 4; i++) {
-        all[i] = dpp_f32<0x00>(x[i]);
-        all[GP / 2 + i] = dpp_f32<0x55>(x[i]);
-        all[GP / 4 + i] = dpp_f32<0xAA>(x[i]);
-        all[GP / 2 + GP / 4 + i] = dpp_f32<0xFF>(x[i]);
+        for (int i = 0; i < GP / 4; i++) {
+            all[i] = dpp_f32<0x00>(x[i]);
+            all[GP / 2 + i] = dpp_f32<0x55>(x[i]);
+            all[GP / 4 + i] = dpp_f32<0xAA>(x[i]);
+            all[GP / 2 + GP / 4 + i] = dpp_f32<0xFF>(x[i]);
+        }
     }
 }
 
@@ -180,7 +196,7 @@ __device__ __forceinline__ void process_rows(const RowRegs (&r)[NR], const bool 
                                              const float (&qv)[GP][8], const float (&Sq)[GP], State<GP> &st, int c)
 {
     // valid: this lane's row exists; live: some row of this wave's step exists (wave-uniform: dead steps are skipped)
-    constexpr int HPL = GP / 4;
+    constexpr int HPL = (GP + 3) / 4;
     float s[NR][HPL];
 #pragma unroll
     for (int t = 0; t < NR; t++) {
@@ -476,8 +492,9 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p_in)
         p.slot_ids = nullptr;
         p.kv_shared = 0;
     }
-    constexpr int LPR = HD / 8, RPS = 64 / LPR, HPL = GP / 4, NSLOT = NW * RPS, NT = NW * 64;
-    constexpr int SLOTF = GP * HD + 2 * GP;   // floats of one row group's state
+    constexpr int LPR = HD / 8, RPS = 64 / LPR, HPL = (GP + 3) / 4, NSLOT = NW * RPS, NT = NW * 64;
+    constexpr int MLF = (2 * GP + 3) / 4 * 4;  // the (m, l) pairs in front of a row group's values, padded so that those stay 16-byte aligned
+    constexpr int SLOTF = GP * HD + MLF;      // floats of one row group's state
     constexpr int ROWB = HD / 32 * 18;
     extern __shared__ __attribute__((aligned(16))) float smem[];
     float *qs = smem;                            // [GP][HD]            fused prologue only
@@ -728,7 +745,7 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p_in)
         for (int h = 0; h < GP; h++) {
             if (h >= groups) break;   // heads past the workgroup's share carry nothing
             const float o8 = 8.f * st.S[h];
-            float *o = my + 2 * GP + h * HD + 32 * b + 4 * w;
+            float *o = my + MLF + h * HD + 32 * b + 4 * w;
             *reinterpret_cast<float4 *>(o) = make_float4(st.O[h][0] - o8, st.O[h][1] - o8, st.O[h][2] - o8, st.O[h][3] - o8);
             *reinterpret_cast<float4 *>(o + 16) = make_float4(st.O[h][4] - o8, st.O[h][5] - o8, st.O[h][6] - o8, st.O[h][7] - o8);
         }
@@ -740,7 +757,7 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p_in)
         // Fully unrolled: one wave per SIMD has nothing to hide an LDS round trip behind, so all reads go out first.
         // (With four outputs per thread -- eight heads -- that is four times the exponentials: there a wave per head
         // publishes the weights and a second barrier follows, 1 us less at 4 slots x 64 partitions.)
-        constexpr int OBW = GP * HD / NT;
+        constexpr int OBW = GP * HD >= NT ? GP * HD / NT : 1;
         constexpr bool kOwnWeights = OBW <= 2;
         float accw[OBW], Mh[OBW], Lh[OBW];
         if (!kOwnWeights) {
@@ -761,11 +778,11 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p_in)
                 for (int s = 0; s < NSLOT; s++) {
                     const float wt = __expf(mv[s] - M);
                     L = fmaf(wt, slots[s * SLOTF + 2 * h + 1], L);
-                    a = fmaf(wt, slots[s * SLOTF + 2 * GP + h * HD + d], a);
+                    a = fmaf(wt, slots[s * SLOTF + MLF + h * HD + d], a);
                 }
             } else {
 #pragma unroll
-                for (int s = 0; s < NSLOT; s++) a = fmaf(wts[h * NSLOT + s], slots[s * SLOTF + 2 * GP + h * HD + d], a);
+                for (int s = 0; s < NSLOT; s++) a = fmaf(wts[h * NSLOT + s], slots[s * SLOTF + MLF + h * HD + d], a);
                 M = mlh[2 * h];
                 L = mlh[2 * h + 1];
             }
@@ -813,7 +830,7 @@ __global__ __launch_bounds__(NW * 64) void sdpa_lanes_kernel(LaneParams p_in)
     // The records come from the memory side (about a microsecond away), so all of
     // a thread's loads -- its output elements' values from up to QB partitions,
     // then its share of the (m, l) pairs -- are issued before anything is used.
-    constexpr int QB = 16, OB = GP * HD / NT;   // partitions in flight x output elements per thread
+    constexpr int QB = 16, OB = GP * HD >= NT ? GP * HD / NT : 1;   // partitions in flight x output elements per thread
     const int nwgp = (nparts + QB - 1) / QB * QB;
     float *w2 = slots;                          // [groups][nwgp] weights, zero past nparts
     float *mq = slots + groups * nwgp;          // [groups][nparts][2]
@@ -1465,7 +1482,7 @@ template <int HD, int GP, int NW>
 constexpr size_t lanes_lds_bytes()
 {
     constexpr int NSLOT = NW * (64 / (HD / 8));
-    return ((size_t)GP * HD + (size_t)NSLOT * (GP * HD + 2 * GP) + (size_t)GP * NSLOT + 2 * GP) * 4 + 2 * (HD / 32 * 18) + 16;
+    return ((size_t)GP * HD + (size_t)NSLOT * (GP * HD + (2 * GP + 3) / 4 * 4) + (size_t)GP * NSLOT + 2 * GP) * 4 + 2 * (HD / 32 * 18) + 16;
 }
 
 template <int HD, int GP, int NW>
@@ -1480,6 +1497,13 @@ int launch_inst(const LaneParams &p, int n_slots, hipStream_t st)
 
 int launch_lanes(const LaneParams &p, int hd, int nw, int n_slots, hipStream_t st)
 {
+    // the decode step's unmerged partitions with one q head per workgroup: its own instance (heads of 256)
+    if (p.fused && p.mode == kModeSplitPart && p.groups == 1 && hd == 256 && (nw == 4 || nw == 8)) {
+        if (nw == 8) hipLaunchKernelGGL((sdpa_lanes_kernel<256, 1, 8, true>), dim3(p.nwg, p.n_kv * p.hsplit, n_slots), dim3(512), (lanes_lds_bytes<256, 1, 8>()), st, p);
+        else hipLaunchKernelGGL((sdpa_lanes_kernel<256, 1, 4, true>), dim3(p.nwg, p.n_kv * p.hsplit, n_slots), dim3(256), (lanes_lds_bytes<256, 1, 4>()), st, p);
+        const hipError_t e = hipGetLastError();
+        return e == hipSuccess ? 0 : hip_fail(e, "sdpa (register form, one head) launch");
+    }
     const int gp = p.groups <= 4 ? 4 : 8;
 #define KSH_CASE(H, G, W) \
     if (hd == H && gp == G && nw == W) return launch_inst<H, G, W>(p, n_slots, st);
@@ -1490,11 +1514,11 @@ int launch_lanes(const LaneParams &p, int hd, int nw, int n_slots, hipStream_t s
     return set_error("sdpa (register form): no instance for hd=%d groups=%d nsg=%d", hd, p.groups, nw);
 }
 
-size_t lanes_lds(int hd, int groups, int nw)
+size_t lanes_lds(int hd, int groups, int nw, bool one_head = false)
 {
-    const int gp = groups <= 4 ? 4 : 8;
+    const int gp = one_head ? 1 : groups <= 4 ? 4 : 8;
     const int nslot = nw * (64 / (hd / 8));
-    return ((size_t)gp * hd + (size_t)nslot * (gp * hd + 2 * gp) + (size_t)gp * nslot + 2 * gp) * 4 + 2 * (hd / 32 * 18) + 16;
+    return ((size_t)gp * hd + (size_t)nslot * (gp * hd + (2 * gp + 3) / 4 * 4) + (size_t)gp * nslot + 2 * gp) * 4 + 2 * (hd / 32 * 18) + 16;
 }
 
 LaneParams base_params(const ksh_kernel &k)
@@ -1740,7 +1764,7 @@ int bind_sdpa_lanes(ksh_kernel &k, int nwg, int n_slots)
     if (hsplit < 1 || hsplit > 255 || total_groups % hsplit) return set_error("sdpa: unsupported schedule unroll=%d (must divide %d)", hsplit, total_groups);
     if (hd == 512 && total_groups / hsplit > 4) return set_error("sdpa: heads of 512 take at most four q heads per workgroup (unroll=%d leaves %d)", hsplit, total_groups / hsplit);
     const int wg_groups = total_groups / hsplit;
-    const size_t lds = lanes_lds(hd, wg_groups, nw);
+    const size_t lds = lanes_lds(hd, wg_groups, nw, k.desc.kind == KSH_ATTEND_DECODE && k.desc.dims[5] != 0 && wg_groups == 1 && hd == 256);   // (launch_lanes' one-head instance)
     const bool merges = k.desc.kind == KSH_SDPA_SLOTS || k.desc.kind == KSH_SDPA_BATCH || (k.desc.kind == KSH_ATTEND_DECODE && !k.desc.dims[5]);
     if (merges && !(k.desc.kind == KSH_SDPA_SLOTS && balanced_slots(n_slots, nwg)) &&   // (those merge in a launch of their own)
         (size_t)wg_groups * (nwg + 16) * 3 * 4 > (size_t)nw * (64 / (hd / 8)) * ((wg_groups <= 4 ? 4 : 8) * hd) * 4)

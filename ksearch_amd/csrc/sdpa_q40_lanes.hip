@@ -145,6 +145,17 @@ __device__ __forceinline__ void reduce_heads(const float (&v)[GP], int c, float 
         if (HD >= 256) x = xor16_sum(x);
         if (HD == 512) x = xor32_sum(x);
         out[0] = x;
+    } else if constexpr (GP == 2) {
+        // lanes with c & 1 = 0 end up with head 0, the others with head 1
+        const bool b0 = c & 1;
+        const float keep = b0 ? v[1] : v[0], send = b0 ? v[0] : v[1];
+        float x = keep + dpp_f32<0xB1>(send);   // quad_perm [1,0,3,2]
+        x += dpp_f32<0x4E>(x);                  // quad_perm [2,3,0,1]
+        x += dpp_f32<0x124>(x);
+        x += dpp_f32<0x128>(x);
+        if (HD >= 256) x = xor16_sum(x);
+        if (HD == 512) x = xor32_sum(x);
+        out[0] = x;
     } else {
         const bool b0 = c & 1, b1 = c & 2;
         float a[GP / 2];
@@ -172,6 +183,9 @@ __device__ __forceinline__ void quad_gather(const float (&x)[(GP + 3) / 4], floa
 {
     if constexpr (GP == 1) {
         all[0] = x[0];
+    } else if constexpr (GP == 2) {
+        all[0] = dpp_f32<0x00>(x[0]);
+        all[1] = dpp_f32<0x55>(x[0]);
     } else {
 #pragma unroll
         for (int i = 0; i < GP / 4; i++) {
@@ -1495,14 +1509,24 @@ int launch_inst(const LaneParams &p, int n_slots, hipStream_t st)
     return e == hipSuccess ? 0 : hip_fail(e, "sdpa (register form) launch");
 }
 
+// which launches take the instances for one or two q heads per workgroup: the fused decode step at heads of 256 -- one
+// head where its partitions stay unmerged, two in either form
+bool lanes_few_heads(int fused, int mode, int groups, int hd)
+{
+    return fused && hd == 256 && ((groups == 1 && mode == kModeSplitPart) || groups == 2);
+}
+
 int launch_lanes(const LaneParams &p, int hd, int nw, int n_slots, hipStream_t st)
 {
-    // the decode step's unmerged partitions with one q head per workgroup: its own instance (heads of 256)
-    if (p.fused && p.mode == kModeSplitPart && p.groups == 1 && hd == 256 && (nw == 4 || nw == 8)) {
-        if (nw == 8) hipLaunchKernelGGL((sdpa_lanes_kernel<256, 1, 8, true>), dim3(p.nwg, p.n_kv * p.hsplit, n_slots), dim3(512), (lanes_lds_bytes<256, 1, 8>()), st, p);
-        else hipLaunchKernelGGL((sdpa_lanes_kernel<256, 1, 4, true>), dim3(p.nwg, p.n_kv * p.hsplit, n_slots), dim3(256), (lanes_lds_bytes<256, 1, 4>()), st, p);
+    // the decode step with one or two q heads per workgroup (heads of 256): instances of their own
+    if (lanes_few_heads(p.fused, p.mode, p.groups, hd) && (nw == 4 || nw == 8)) {
+        const dim3 grid(p.nwg, p.n_kv * p.hsplit, n_slots);
+        if (p.groups == 1 && nw == 8) hipLaunchKernelGGL((sdpa_lanes_kernel<256, 1, 8, true>), grid, dim3(512), (lanes_lds_bytes<256, 1, 8>()), st, p);
+        else if (p.groups == 1) hipLaunchKernelGGL((sdpa_lanes_kernel<256, 1, 4, true>), grid, dim3(256), (lanes_lds_bytes<256, 1, 4>()), st, p);
+        else if (nw == 8) hipLaunchKernelGGL((sdpa_lanes_kernel<256, 2, 8, true>), grid, dim3(512), (lanes_lds_bytes<256, 2, 8>()), st, p);
+        else hipLaunchKernelGGL((sdpa_lanes_kernel<256, 2, 4, true>), grid, dim3(256), (lanes_lds_bytes<256, 2, 4>()), st, p);
         const hipError_t e = hipGetLastError();
-        return e == hipSuccess ? 0 : hip_fail(e, "sdpa (register form, one head) launch");
+        return e == hipSuccess ? 0 : hip_fail(e, "sdpa (register form, one or two heads) launch");
     }
     const int gp = p.groups <= 4 ? 4 : 8;
 #define KSH_CASE(H, G, W) \
@@ -1514,9 +1538,9 @@ int launch_lanes(const LaneParams &p, int hd, int nw, int n_slots, hipStream_t s
     return set_error("sdpa (register form): no instance for hd=%d groups=%d nsg=%d", hd, p.groups, nw);
 }
 
-size_t lanes_lds(int hd, int groups, int nw, bool one_head = false)
+size_t lanes_lds(int hd, int groups, int nw, bool few_heads = false)
 {
-    const int gp = one_head ? 1 : groups <= 4 ? 4 : 8;
+    const int gp = few_heads ? groups : groups <= 4 ? 4 : 8;
     const int nslot = nw * (64 / (hd / 8));
     return ((size_t)gp * hd + (size_t)nslot * (gp * hd + (2 * gp + 3) / 4 * 4) + (size_t)gp * nslot + 2 * gp) * 4 + 2 * (hd / 32 * 18) + 16;
 }
@@ -1764,7 +1788,7 @@ int bind_sdpa_lanes(ksh_kernel &k, int nwg, int n_slots)
     if (hsplit < 1 || hsplit > 255 || total_groups % hsplit) return set_error("sdpa: unsupported schedule unroll=%d (must divide %d)", hsplit, total_groups);
     if (hd == 512 && total_groups / hsplit > 4) return set_error("sdpa: heads of 512 take at most four q heads per workgroup (unroll=%d leaves %d)", hsplit, total_groups / hsplit);
     const int wg_groups = total_groups / hsplit;
-    const size_t lds = lanes_lds(hd, wg_groups, nw, k.desc.kind == KSH_ATTEND_DECODE && k.desc.dims[5] != 0 && wg_groups == 1 && hd == 256);   // (launch_lanes' one-head instance)
+    const size_t lds = lanes_lds(hd, wg_groups, nw, k.desc.kind == KSH_ATTEND_DECODE && lanes_few_heads(1, k.desc.dims[5] ? kModeSplitPart : kModeMerge, wg_groups, hd));
     const bool merges = k.desc.kind == KSH_SDPA_SLOTS || k.desc.kind == KSH_SDPA_BATCH || (k.desc.kind == KSH_ATTEND_DECODE && !k.desc.dims[5]);
     if (merges && !(k.desc.kind == KSH_SDPA_SLOTS && balanced_slots(n_slots, nwg)) &&   // (those merge in a launch of their own)
         (size_t)wg_groups * (nwg + 16) * 3 * 4 > (size_t)nw * (64 / (hd / 8)) * ((wg_groups <= 4 ? 4 : 8) * hd) * 4)

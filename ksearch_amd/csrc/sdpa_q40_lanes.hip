@@ -1509,11 +1509,11 @@ int launch_inst(const LaneParams &p, int n_slots, hipStream_t st)
     return e == hipSuccess ? 0 : hip_fail(e, "sdpa (register form) launch");
 }
 
-// which launches take the instances for one or two q heads per workgroup: the fused decode step at heads of 256 -- one
-// head where its partitions stay unmerged, two in either form
+// which launches take the instances for one or two q heads per workgroup: the fused decode step -- at heads of 256 one
+// head where its partitions stay unmerged and two in either form, at heads of 512 two
 bool lanes_few_heads(int fused, int mode, int groups, int hd)
 {
-    return fused && hd == 256 && ((groups == 1 && mode == kModeSplitPart) || groups == 2);
+    return fused && ((hd == 256 && ((groups == 1 && mode == kModeSplitPart) || groups == 2)) || (hd == 512 && groups == 2));
 }
 
 int launch_lanes(const LaneParams &p, int hd, int nw, int n_slots, hipStream_t st)
@@ -1521,7 +1521,9 @@ int launch_lanes(const LaneParams &p, int hd, int nw, int n_slots, hipStream_t s
     // the decode step with one or two q heads per workgroup (heads of 256): instances of their own
     if (lanes_few_heads(p.fused, p.mode, p.groups, hd) && (nw == 4 || nw == 8)) {
         const dim3 grid(p.nwg, p.n_kv * p.hsplit, n_slots);
-        if (p.groups == 1 && nw == 8) hipLaunchKernelGGL((sdpa_lanes_kernel<256, 1, 8, true>), grid, dim3(512), (lanes_lds_bytes<256, 1, 8>()), st, p);
+        if (hd == 512 && nw == 8) hipLaunchKernelGGL((sdpa_lanes_kernel<512, 2, 8, true>), grid, dim3(512), (lanes_lds_bytes<512, 2, 8>()), st, p);
+        else if (hd == 512) hipLaunchKernelGGL((sdpa_lanes_kernel<512, 2, 4, true>), grid, dim3(256), (lanes_lds_bytes<512, 2, 4>()), st, p);
+        else if (p.groups == 1 && nw == 8) hipLaunchKernelGGL((sdpa_lanes_kernel<256, 1, 8, true>), grid, dim3(512), (lanes_lds_bytes<256, 1, 8>()), st, p);
         else if (p.groups == 1) hipLaunchKernelGGL((sdpa_lanes_kernel<256, 1, 4, true>), grid, dim3(256), (lanes_lds_bytes<256, 1, 4>()), st, p);
         else if (nw == 8) hipLaunchKernelGGL((sdpa_lanes_kernel<256, 2, 8, true>), grid, dim3(512), (lanes_lds_bytes<256, 2, 8>()), st, p);
         else hipLaunchKernelGGL((sdpa_lanes_kernel<256, 2, 4, true>), grid, dim3(256), (lanes_lds_bytes<256, 2, 4>()), st, p);

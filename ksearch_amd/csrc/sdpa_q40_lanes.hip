@@ -1509,11 +1509,12 @@ int launch_inst(const LaneParams &p, int n_slots, hipStream_t st)
     return e == hipSuccess ? 0 : hip_fail(e, "sdpa (register form) launch");
 }
 
-// which launches take the instances for one or two q heads per workgroup: the fused decode step -- at heads of 256 one
-// head where its partitions stay unmerged and two in either form, at heads of 512 two
+// which launches take the instances for one or two q heads per workgroup: the fused decode step at heads of 256 (one or
+// two) and 512 (two)
 bool lanes_few_heads(int fused, int mode, int groups, int hd)
 {
-    return fused && ((hd == 256 && ((groups == 1 && mode == kModeSplitPart) || groups == 2)) || (hd == 512 && groups == 2));
+    (void)mode;
+    return fused && ((hd == 256 && groups <= 2) || (hd == 512 && groups == 2));
 }
 
 int launch_lanes(const LaneParams &p, int hd, int nw, int n_slots, hipStream_t st)

@@ -271,6 +271,54 @@ def test_attend_decode_reading_another_layers_cache(ctx, eng, n_q, n_kv, hd, max
     assert np.array_equal(ctx.read_bytes(kc, max_seq * row), k) and np.array_equal(ctx.read_bytes(vc, max_seq * row), v)
 
 
+@pytest.mark.parametrize("n_q,n_kv,hd,max_seq,pos,nwg,start", [
+    (8, 1, 256, 1024, 300, 8, 0),
+    (8, 1, 256, 1024, 700, 16, 150),    # a window that has begun to slide
+    (8, 1, 512, 1024, 300, 8, 0),       # 512-wide heads: at most four per workgroup
+    (8, 2, 256, 512, 200, 4, 0),        # two kv heads of four q heads each
+])
+@pytest.mark.parametrize("parts", [False, True])
+def test_attend_decode_every_head_split(ctx, eng, n_q, n_kv, hd, max_seq, pos, nwg, start, parts):
+    """The decode step under every split of a kv head's q heads over workgroups (sched.unroll) and both workgroup sizes:
+    eight, four, two heads per workgroup or one (the last two have kernel instances of their own at heads of 256 / 512),
+    merged in the launch or left as partitions; each against the oracle's attention over the device's cache."""
+    eps, scale = 1e-6, 1.0 / float(np.sqrt(hd))
+    row = n_kv * hd // 32 * 18
+    k, v = kv(max_seq, n_kv, hd, 740 + pos)
+    k[pos * row:] = 0
+    v[pos * row:] = 0
+    q, kr, vr = (synth.normal_f32(r * hd, 750 + i) for i, r in enumerate((n_q, n_kv, n_kv)))
+    qw, kw = 1.0 + 0.2 * synth.normal_f32(hd, 753), 1.0 + 0.2 * synth.normal_f32(hd, 754)
+    rope = oracle.rope_table(max_seq, hd, 10000.0)
+    tlen = pos + 1 - start
+    meta = ctx.buffer_f32([tlen, start, tlen if start else 0, pos])
+    groups, ran = n_q // n_kv, 0
+    for unroll in (1, 2, 4, 8):
+        if groups % unroll or (hd == 512 and groups // unroll > 4):
+            continue
+        for nsg in (4, 8):
+            kk = ctx.compile(hip.make_desc(hip.Kind.ATTEND_DECODE, (n_q, n_kv, hd, max_seq, nwg, int(parts), 1), (DType.Q40, DType.F32), (eps, scale),
+                                           dict(vec=3, unroll=unroll, nsg=nsg)))
+            assert kk.info.sched.unroll == unroll and kk.info.sched.nsg == nsg
+            kc, vc, tmp, out = ctx.buffer_bytes(k), ctx.buffer_bytes(v), ctx.buffer_empty_f32(n_q * nwg * (hd + 2)), ctx.buffer_empty_f32(n_q * hd)
+            ins = [ctx.buffer_f32(a) for a in (q, qw, rope[pos], kr, kw, vr)] + [meta]
+            for rep in range(2):                 # twice: the arrival counter of the merging form must come back to zero
+                ctx.encode_multi(kk, ins, [kc, vc, tmp] if parts else [kc, vc, tmp, out])
+            if parts:
+                t = ctx.read_f32(tmp, n_q * nwg * (hd + 2))
+                o, ml = t[:n_q * nwg * hd].reshape(n_q, nwg, hd).astype(np.float64), t[n_q * nwg * hd:].reshape(n_q, nwg, 2).astype(np.float64)
+                wt = np.exp(ml[:, :, 0] - ml[:, :, 0].max(1, keepdims=True))
+                got = ((wt[:, :, None] * o).sum(1) / (wt * ml[:, :, 1]).sum(1)[:, None]).reshape(-1)
+            else:
+                got = ctx.read_f32(out, n_q * hd)
+            gk, gv = ctx.read_bytes(kc, max_seq * row), ctx.read_bytes(vc, max_seq * row)
+            wq = oracle.rmsnorm_per_head_qkv_q40(q, qw, rope[pos], kr, kw, vr, n_q, n_kv, hd, eps)[0]
+            want = oracle.sdpa(wq, gk, gv, n_q, n_kv, hd, tlen, start, scale, f64=True)
+            assert_close(got, want, TOL, f"unroll {unroll}, {nsg} waves")
+            ran += 1
+    assert ran >= 4
+
+
 @pytest.mark.parametrize("n_q,n_kv,hd,max_seq,pos,nwg,rows", [
     (8, 1, 256, 4096, 0, 8, 2048),      # one row: seven partitions are empty
     (8, 1, 256, 4096, 5, 8, 2048),      # fewer rows than partitions

@@ -1791,6 +1791,9 @@ int bind_sdpa_lanes(ksh_kernel &k, int nwg, int n_slots)
     if (hsplit < 1 || hsplit > 255 || total_groups % hsplit) return set_error("sdpa: unsupported schedule unroll=%d (must divide %d)", hsplit, total_groups);
     if (hd == 512 && total_groups / hsplit > 4) return set_error("sdpa: heads of 512 take at most four q heads per workgroup (unroll=%d leaves %d)", hsplit, total_groups / hsplit);
     const int wg_groups = total_groups / hsplit;
+    // the unmerged decode step with one head per workgroup: four waves (eight row groups to fold instead of sixteen; in
+    // cfg4's loop 1207-1210 against 1194-1197 tok/s with eight, per launch 4.1 against 4.7 us at 64 rows, equal at 300 - 600)
+    if (!k.desc.sched.nsg && k.desc.kind == KSH_ATTEND_DECODE && k.desc.dims[5] != 0 && wg_groups == 1 && hd == 256) nw = 4;
     const size_t lds = lanes_lds(hd, wg_groups, nw, k.desc.kind == KSH_ATTEND_DECODE && lanes_few_heads(1, k.desc.dims[5] ? kModeSplitPart : kModeMerge, wg_groups, hd));
     const bool merges = k.desc.kind == KSH_SDPA_SLOTS || k.desc.kind == KSH_SDPA_BATCH || (k.desc.kind == KSH_ATTEND_DECODE && !k.desc.dims[5]);
     if (merges && !(k.desc.kind == KSH_SDPA_SLOTS && balanced_slots(n_slots, nwg)) &&   // (those merge in a launch of their own)

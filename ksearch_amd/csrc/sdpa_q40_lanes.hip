@@ -1509,12 +1509,11 @@ int launch_inst(const LaneParams &p, int n_slots, hipStream_t st)
     return e == hipSuccess ? 0 : hip_fail(e, "sdpa (register form) launch");
 }
 
-// which launches take the instances for one or two q heads per workgroup: the fused decode step at heads of 256 (one or
-// two) and 512 (two)
+// which launches take the instances for one or two q heads per workgroup: the fused decode step at heads of 256 and 512
 bool lanes_few_heads(int fused, int mode, int groups, int hd)
 {
     (void)mode;
-    return fused && ((hd == 256 && groups <= 2) || (hd == 512 && groups == 2));
+    return fused && (hd == 256 || hd == 512) && groups <= 2;
 }
 
 int launch_lanes(const LaneParams &p, int hd, int nw, int n_slots, hipStream_t st)
@@ -1522,7 +1521,9 @@ int launch_lanes(const LaneParams &p, int hd, int nw, int n_slots, hipStream_t s
     // the decode step with one or two q heads per workgroup (heads of 256): instances of their own
     if (lanes_few_heads(p.fused, p.mode, p.groups, hd) && (nw == 4 || nw == 8)) {
         const dim3 grid(p.nwg, p.n_kv * p.hsplit, n_slots);
-        if (hd == 512 && nw == 8) hipLaunchKernelGGL((sdpa_lanes_kernel<512, 2, 8, true>), grid, dim3(512), (lanes_lds_bytes<512, 2, 8>()), st, p);
+        if (hd == 512 && p.groups == 1 && nw == 8) hipLaunchKernelGGL((sdpa_lanes_kernel<512, 1, 8, true>), grid, dim3(512), (lanes_lds_bytes<512, 1, 8>()), st, p);
+        else if (hd == 512 && p.groups == 1) hipLaunchKernelGGL((sdpa_lanes_kernel<512, 1, 4, true>), grid, dim3(256), (lanes_lds_bytes<512, 1, 4>()), st, p);
+        else if (hd == 512 && nw == 8) hipLaunchKernelGGL((sdpa_lanes_kernel<512, 2, 8, true>), grid, dim3(512), (lanes_lds_bytes<512, 2, 8>()), st, p);
         else if (hd == 512) hipLaunchKernelGGL((sdpa_lanes_kernel<512, 2, 4, true>), grid, dim3(256), (lanes_lds_bytes<512, 2, 4>()), st, p);
         else if (p.groups == 1 && nw == 8) hipLaunchKernelGGL((sdpa_lanes_kernel<256, 1, 8, true>), grid, dim3(512), (lanes_lds_bytes<256, 1, 8>()), st, p);
         else if (p.groups == 1) hipLaunchKernelGGL((sdpa_lanes_kernel<256, 1, 4, true>), grid, dim3(256), (lanes_lds_bytes<256, 1, 4>()), st, p);
@@ -1782,10 +1783,12 @@ int bind_sdpa_lanes(ksh_kernel &k, int nwg, int n_slots)
     // sched.unroll: workgroups per kv head, each with a share of its q heads (rows are then unpacked once per
     // share, but a decode step's latency is in the per-row work and the merge, both of which shrink with it)
     const int total_groups = n_q / n_kv;
-    // (defaults from timing the decode shape: two heads per workgroup where the launch merges, one where it does not)
+    // (defaults from timing the decode shape: two heads per workgroup where the launch merges, one where it does not;
+    // heads of 512, merging, 16 partitions, eight waves: one head per workgroup 8.3 / 9.6 / 15.2 us at 320 / 1000 / 3000
+    // rows against 8.9 / 10.9 / 17.3 with two)
     int hsplit = k.desc.sched.unroll ? (int)k.desc.sched.unroll
                  : k.desc.kind != KSH_ATTEND_DECODE || total_groups < 4 ? 1
-                 : k.desc.dims[5] ? total_groups : (total_groups % 2 == 0 ? total_groups / 2 : 1);
+                 : k.desc.dims[5] || hd == 512 ? total_groups : (total_groups % 2 == 0 ? total_groups / 2 : 1);
     // heads of 512: at most four per workgroup (the fold's LDS)
     if (hd == 512 && !k.desc.sched.unroll && total_groups / hsplit > 4 && total_groups % 4 == 0) hsplit = total_groups / 4;
     if (hsplit < 1 || hsplit > 255 || total_groups % hsplit) return set_error("sdpa: unsupported schedule unroll=%d (must divide %d)", hsplit, total_groups);
@@ -1794,6 +1797,8 @@ int bind_sdpa_lanes(ksh_kernel &k, int nwg, int n_slots)
     // the unmerged decode step with one head per workgroup: four waves (eight row groups to fold instead of sixteen; in
     // cfg4's loop 1207-1210 against 1194-1197 tok/s with eight, per launch 4.1 against 4.7 us at 64 rows, equal at 300 - 600)
     if (!k.desc.sched.nsg && k.desc.kind == KSH_ATTEND_DECODE && k.desc.dims[5] != 0 && wg_groups == 1 && hd == 256) nw = 4;
+    // heads of 512, one per workgroup, merging: eight waves at every partition length (16 row groups of 32 lanes)
+    if (!k.desc.sched.nsg && k.desc.kind == KSH_ATTEND_DECODE && k.desc.dims[5] == 0 && wg_groups == 1 && hd == 512) nw = 8;
     const size_t lds = lanes_lds(hd, wg_groups, nw, k.desc.kind == KSH_ATTEND_DECODE && lanes_few_heads(1, k.desc.dims[5] ? kModeSplitPart : kModeMerge, wg_groups, hd));
     const bool merges = k.desc.kind == KSH_SDPA_SLOTS || k.desc.kind == KSH_SDPA_BATCH || (k.desc.kind == KSH_ATTEND_DECODE && !k.desc.dims[5]);
     if (merges && !(k.desc.kind == KSH_SDPA_SLOTS && balanced_slots(n_slots, nwg)) &&   // (those merge in a launch of their own)

@@ -337,34 +337,73 @@ __device__ __forceinline__ void norm_rope_regs(const float (&xv)[HD / 64], const
 // flat indices from the sum of its predecessors' counts, and its records sit in that order.
 // round > 1: the rows per partition are rounded up to a multiple of it (the matrix-core form works in tiles of rows).
 //
-// A whole wave works the deal out at once: lane s holds slot s's length (one load per lane, all in flight together,
-// where a loop over the slots would wait for one length after the other), the division by the partition size runs
-// in all lanes, and only the running count of partitions is a loop over lanes.  `f` is the flat partition index of
-// the caller (wave-uniform); slot < 0 says that the deal has fewer partitions than that.  With `of_slot` >= 0 the
-// answer is that slot's range of partitions instead (first, nparts).  Up to 64 slots (host-checked: 16).
+// A whole wave works the deal out at once, as one short chain of vector instructions (a launch of this kind is a chain
+// of dependent steps: the first form of this routine -- two loops over the slots with a lane read each, three integer
+// divisions, uniform values moving between the vector and the scalar unit -- was 0.8 us of the merge launch and as much
+// of the row launch): lane s of every 16-lane row holds slot s's length (one load per lane, all in flight together), the
+// total is a row sum that every lane ends up with, the two divisions go through a reciprocal with an exact fix-up and no
+// branch, the running count of partitions is a prefix sum over the row (row shifts), the owner of a flat index is the
+// number of slots whose running count does not exceed it, and only the answer is read out of the lanes.
+// `f` is the flat partition index of the caller (wave-uniform); slot < 0 says that the deal has fewer partitions than
+// that.  With `of_slot` >= 0 the answer is that slot's range of partitions instead (first, nparts).  Up to 64 slots
+// (more than 16: one slot per lane of the wave, and the rows' totals cross through lane reads); `round` is a power of
+// two; lengths and their total below 2^22.
 struct Deal {
     int slot, part, nparts, first, tlen, start, c;
 };
+// ceil(a / b) with rb ~ 1 / b (one ulp): the truncated product is off by one at most, either way, and the remainder
+// against it says which
+__device__ __forceinline__ uint32_t ceil_div_rcp(uint32_t a, uint32_t b, float rb)
+{
+    const uint32_t q = (uint32_t)((float)a * rb);
+    const int32_t t = (int32_t)(a - q * b);      // in (-b, 2b)
+    return q + (t > 0 ? 1u : 0u) + (t > (int32_t)b ? 1u : 0u);
+}
+template <int SHR>
+__device__ __forceinline__ int row_shr_i32(int v)   // lane i of a 16-lane row reads lane i - SHR of it, 0 below the row's start
+{
+    return __builtin_amdgcn_update_dpp(0, v, 0x110 + SHR, 0xF, 0xF, true);
+}
 __device__ __forceinline__ Deal deal_wave(const float *meta, int stride, int n_slots, int nwg, int round, int f, int of_slot = -1)
 {
-    const int lane = threadIdx.x & 63, ls = min(lane, n_slots - 1);
-    const int len = (int)meta[(size_t)ls * stride], st = (int)meta[(size_t)ls * stride + 1];
-    int T = 0;
-    for (int s = 0; s < n_slots; s++) T += __builtin_amdgcn_readlane(len, s);
-    const int spare = max(1, nwg * n_slots - n_slots);
-    int c = max(1, (T + spare - 1) / spare);
-    c = (c + round - 1) / round * round;
-    const int n = max(1, (len + c - 1) / c);
-    Deal d{-1, 0, 0, 0, 0, 0, c};
-    int first = 0;
-    for (int s = 0; s < n_slots; s++) {
-        const int ns = __builtin_amdgcn_readlane(n, s);
-        if (of_slot >= 0 ? s == of_slot : (d.slot < 0 && f < first + ns)) { d.slot = s; d.part = f - first; d.nparts = ns; d.first = first; }
-        first += ns;
+    const int lane = threadIdx.x & 63;
+    const bool wide = n_slots > 16;
+    const int sl = wide ? lane : (lane & 15), ls = min(sl, n_slots - 1);
+    const bool live = sl < n_slots;
+    const float lenf = meta[(size_t)ls * stride];
+    const int st = (int)meta[(size_t)ls * stride + 1];
+    const uint32_t spare = (uint32_t)max(1, nwg * n_slots - n_slots);
+    const float rspare = __builtin_amdgcn_rcpf((float)spare);
+    const uint32_t len = live ? (uint32_t)lenf : 0u;
+    float Tf = row16_sum(live ? lenf : 0.f);      // (integers below 2^24: exact in f32)
+    if (wide) {
+        const float a = as_f32((uint32_t)__builtin_amdgcn_readlane((int)as_u32(Tf), 0)), b = as_f32((uint32_t)__builtin_amdgcn_readlane((int)as_u32(Tf), 16));
+        const float c = as_f32((uint32_t)__builtin_amdgcn_readlane((int)as_u32(Tf), 32)), d = as_f32((uint32_t)__builtin_amdgcn_readlane((int)as_u32(Tf), 48));
+        Tf = (a + b) + (c + d);
     }
-    if (d.slot >= 0) {
-        d.tlen = __builtin_amdgcn_readlane(len, d.slot);
-        d.start = __builtin_amdgcn_readlane(st, d.slot);
+    uint32_t c = max(1u, ceil_div_rcp((uint32_t)Tf, spare, rspare));
+    c = (c + (uint32_t)round - 1u) & ~((uint32_t)round - 1u);
+    const int n = live ? (int)max(1u, ceil_div_rcp(len, c, __builtin_amdgcn_rcpf((float)c))) : 0;
+    // partitions up to and with each lane's slot
+    int incl = n;
+    incl += row_shr_i32<1>(incl);
+    incl += row_shr_i32<2>(incl);
+    incl += row_shr_i32<4>(incl);
+    incl += row_shr_i32<8>(incl);
+    if (wide) {
+        const int t0 = __builtin_amdgcn_readlane(incl, 15), t1 = __builtin_amdgcn_readlane(incl, 31), t2 = __builtin_amdgcn_readlane(incl, 47);
+        incl += lane >= 48 ? t0 + t1 + t2 : lane >= 32 ? t0 + t1 : lane >= 16 ? t0 : 0;
+    }
+    const int excl = incl - n;
+    const int slot = of_slot >= 0 ? of_slot : (int)__builtin_popcountll(__builtin_amdgcn_ballot_w64(live && (wide || lane < 16) && incl <= f));
+    Deal d{-1, 0, 0, 0, 0, 0, __builtin_amdgcn_readfirstlane((int)c)};
+    if (slot < n_slots) {
+        d.slot = slot;
+        d.first = __builtin_amdgcn_readlane(excl, slot);
+        d.nparts = __builtin_amdgcn_readlane(n, slot);
+        d.part = f - d.first;
+        d.tlen = __builtin_amdgcn_readlane((int)len, slot);
+        d.start = __builtin_amdgcn_readlane(st, slot);
     }
     return d;
 }
